@@ -1,0 +1,446 @@
+"""CPU oracle for the weight-quantized linear path -- TEST INFRASTRUCTURE ONLY.
+
+numpy + ctypes front-end of ``libtppx_oracle.so`` (``oracle/tppx_oracle.c``).
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this module; the product package never does.
+
+bf16 tensors are carried as ``numpy.uint16`` bit patterns.
+
+The layout helpers restate the reference's ``view``/``permute`` chains
+(``src/tpp_pytorch_extension/utils/blocked_layout.py:28-80``,
+``src/csrc/qtypes.cpp:783-932``) with numpy ``reshape``/``transpose`` so that
+they can be compared, byte for byte, with the closed-form index maps coded in
+C (``orc_remap_quantize_*``).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libtppx_oracle.so")
+_REF_PATH = os.path.join(_HERE, "_ref", "libmxref.so")
+
+POST_NONE, POST_SILU, POST_MUL, POST_ADD_SCALE, POST_ADD2_SCALE, POST_GELU, POST_RELU = range(7)
+MODE_IDEAL, MODE_FAITHFUL, MODE_F64 = range(3)
+
+_c_i64 = ctypes.c_int64
+_c_p = ctypes.c_void_p
+
+
+def build(force=False):
+    """Compile the C restatement (and the reference shim when the reference
+    tree is present)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libtppx_oracle.so"])
+    if os.path.isdir("/root/reference/src/csrc"):
+        subprocess.check_call(["make", "-C", _HERE, "ref"])
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                "oracle library not built: run `make -C oracle` (or __graft_entry__.build())"
+            )
+        L = ctypes.CDLL(_LIB_PATH)
+        L.orc_mx_scale_byte.argtypes = [ctypes.c_float]
+        L.orc_mx_scale_byte.restype = ctypes.c_int
+        L.orc_mx_quant_scale.argtypes = [ctypes.c_int]
+        L.orc_mx_quant_scale.restype = ctypes.c_float
+        L.orc_mx_dequant_scale.argtypes = [ctypes.c_int]
+        L.orc_mx_dequant_scale.restype = ctypes.c_float
+        L.orc_e2m1_encode.argtypes = [ctypes.c_float]
+        L.orc_e2m1_encode.restype = ctypes.c_int
+        L.orc_e2m1_decode.argtypes = [ctypes.c_int]
+        L.orc_e2m1_decode.restype = ctypes.c_float
+        L.orc_num_threads.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def ref_lib():
+    """The shim around the reference's own mxfp_quant.h, or None when it was
+    not built (it only builds where the reference tree is mounted)."""
+    if not os.path.exists(_REF_PATH):
+        return None
+    R = ctypes.CDLL(_REF_PATH)
+    R.ref_mx_shared_scale.argtypes = [ctypes.c_float]
+    R.ref_mx_shared_scale.restype = ctypes.c_float
+    R.ref_e2m1_round.argtypes = [ctypes.c_float]
+    R.ref_e2m1_round.restype = ctypes.c_float
+    return R
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(_c_p)
+
+
+def _c(a, dt):
+    return np.ascontiguousarray(a, dtype=dt)
+
+
+# ----------------------------------------------------------------------------
+# bf16 helpers
+# ----------------------------------------------------------------------------
+def f32_to_bf16(a):
+    a = _c(a, np.float32)
+    out = np.empty(a.shape, np.uint16)
+    lib().orc_f32_to_bf16(_p(a), _p(out), _c_i64(a.size))
+    return out
+
+
+def bf16_to_f32(a):
+    a = _c(a, np.uint16)
+    return (a.astype(np.uint32) << 16).view(np.float32)
+
+
+def bf16_round(a):
+    """fp32 -> nearest bf16 -> fp32."""
+    return bf16_to_f32(f32_to_bf16(a))
+
+
+# ----------------------------------------------------------------------------
+# element math (scalar)
+# ----------------------------------------------------------------------------
+def mx_scale_byte(amax):
+    return lib().orc_mx_scale_byte(float(amax))
+
+
+def mx_quant_scale(x):
+    return lib().orc_mx_quant_scale(int(x))
+
+
+def mx_dequant_scale(x):
+    return lib().orc_mx_dequant_scale(int(x))
+
+
+def e2m1_encode(v):
+    return lib().orc_e2m1_encode(float(v))
+
+
+def e2m1_decode(c):
+    return lib().orc_e2m1_decode(int(c))
+
+
+E2M1_TABLE = np.array(
+    [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0],
+    np.float32,
+)
+
+
+# ----------------------------------------------------------------------------
+# blocked layout  (blocked_layout.py:28-80 ; llm_common.py:468-490 ; nn.py:27-44)
+# ----------------------------------------------------------------------------
+def block_weight(W, bk=16, bc=64, vnni=2):
+    """W[N,K] -> [N/bk, K/bc, bc/vnni, bk, vnni] (vnni > 1) or
+    [N/bk, K/bc, bc, bk] (vnni == 1): view + permute(0,2,3,1[,4])."""
+    N, K = W.shape
+    assert N % bk == 0 and K % bc == 0
+    if vnni == 1:
+        return np.ascontiguousarray(W.reshape(N // bk, bk, K // bc, bc).transpose(0, 2, 3, 1))
+    assert bc % vnni == 0
+    return np.ascontiguousarray(
+        W.reshape(N // bk, bk, K // bc, bc // vnni, vnni).transpose(0, 2, 3, 1, 4)
+    )
+
+
+def unblock_weight(Wb):
+    if Wb.ndim == 4:
+        n1, c1, c2, k2 = Wb.shape
+        return np.ascontiguousarray(Wb.transpose(0, 3, 1, 2)).reshape(n1 * k2, c1 * c2)
+    n1, c1, c2, k2, c3 = Wb.shape
+    return np.ascontiguousarray(Wb.transpose(0, 3, 1, 2, 4)).reshape(n1 * k2, c1 * c2 * c3)
+
+
+def remap_mxfp4(t):
+    """The re-layout half of remap_and_quantize_mxfp4 (qtypes.cpp:783-839,
+    default USE_MXFP4_INT8=0): bring a blocked weight to [N/32,K/.,.,32,2]."""
+    want = 32
+    if t.ndim == 5:
+        K1, C1, C2, K2, C3 = t.shape
+        if K2 < want and want % K2 == 0:
+            r = want // K2
+            if K1 % r:
+                raise ValueError("Shape not compatible for MXFP4")
+            t = t.reshape(K1 // r, r, C1, C2, K2, C3).transpose(0, 2, 3, 1, 4, 5)
+            t = np.ascontiguousarray(t).reshape(K1 // r, C1, C2, r * K2, C3)
+        elif K2 > want and K2 % want == 0:
+            r = K2 // want
+            t = t.reshape(K1, C1, C2, r, want, C3).transpose(0, 3, 1, 2, 4, 5)
+            t = np.ascontiguousarray(t).reshape(K1 * r, C1, C2, want, C3)
+    elif t.ndim == 4:
+        K1, C1, C2, K2 = t.shape
+        if C2 % 2:
+            raise ValueError("Shape not compatible for VNNI2")
+        if K2 < want and want % K2 == 0:
+            r = want // K2
+            if K1 % r:
+                raise ValueError("Shape not compatible for MXFP4")
+            t = t.reshape(K1 // r, r, C1, C2 // 2, 2, K2).transpose(0, 2, 3, 1, 5, 4)
+            t = np.ascontiguousarray(t).reshape(K1 // r, C1, C2 // 2, r * K2, 2)
+        elif K2 > want and K2 % want == 0:
+            r = K2 // want
+            t = t.reshape(K1, C1, C2 // 2, 2, r, want).transpose(0, 4, 1, 2, 5, 3)
+            t = np.ascontiguousarray(t).reshape(K1 * r, C1, C2 // 2, want, 2)
+        else:
+            t = t.reshape(K1, C1, C2 // 2, 2, K2).transpose(0, 1, 2, 4, 3)
+            t = np.ascontiguousarray(t)
+    else:
+        raise ValueError("expected a 4-D or 5-D blocked weight")
+    return np.ascontiguousarray(t)
+
+
+def qint8_block_size(K, env_block=256):
+    """Block-size choice of remap_and_quantize_qint8 (qtypes.cpp:878-889)."""
+    if K % env_block == 0:
+        return env_block
+    q = 4096
+    while q >= 64:
+        if env_block > q and K % q == 0:
+            return q
+        q //= 2
+    return None
+
+
+def remap_qint8(t, env_block=256):
+    """The re-layout half of remap_and_quantize_qint8 (qtypes.cpp:866-924):
+    -> ([N/bk, K/QBS, QBS/4, bk, 4], QBS)."""
+    if t.ndim == 5:
+        K1, C1, C2, K2, C3 = t.shape
+        C = C1 * C2 * C3
+        qbs = qint8_block_size(C, env_block)
+        if qbs is not None:
+            C2, C1 = qbs // C3, C // qbs
+        if C3 != 4:
+            r = 4 // C3
+            if C2 % r:
+                raise ValueError("Shape not compatible for VNNI4")
+            t = t.reshape(K1, C1, C2 // r, r, K2, C3).transpose(0, 1, 2, 4, 3, 5)
+            t = np.ascontiguousarray(t).reshape(K1, C1, C2 // r, K2, r * C3)
+        else:
+            t = t.reshape(K1, C1, C2, K2, C3)
+        return np.ascontiguousarray(t), C2 * C3
+    if t.ndim == 4:
+        K1, C1, C2, K2 = t.shape
+        C = C1 * C2
+        qbs = qint8_block_size(C, env_block)
+        if qbs is not None:
+            C2, C1 = qbs, C // qbs
+        if C2 % 4:
+            raise ValueError("Shape not compatible for VNNI4")
+        t = t.reshape(K1, C1, C2 // 4, 4, K2).transpose(0, 1, 2, 4, 3)
+        return np.ascontiguousarray(t), C2
+    raise ValueError("expected a 4-D or 5-D blocked weight")
+
+
+def _per_block_geometry(shape, block_size, axis, is_vnni, pack):
+    """(pre, bs, post, vnni, scale_shape) of PerBlockQuantizer (qtypes.h:30-68)."""
+    sizes = list(shape)
+    if axis < 0:
+        axis += len(sizes)
+    if is_vnni:
+        vnni = sizes.pop()
+    else:
+        assert axis == len(sizes) - 1, "Invalid axis"
+        assert sizes[axis] % pack == 0
+        vnni = pack
+        sizes[axis] //= pack
+    assert block_size % vnni == 0
+    bsi = block_size // vnni
+    assert len(sizes) > axis and sizes[axis] % bsi == 0
+    sizes[axis] //= bsi
+    pre = int(np.prod(sizes[: axis + 1], dtype=np.int64))
+    post = int(np.prod(sizes[axis + 1 :], dtype=np.int64))
+    return pre, bsi, post, vnni, sizes
+
+
+def quantize_mxfp4(t, block_size=32, axis=2, is_vnni=True):
+    """quantize_mxfp4 (qtypes.cpp:602-611) on an fp32 array.
+    Returns (packed uint8 with last dim halved, E8M0 scale bytes)."""
+    t = _c(t, np.float32)
+    pre, bs, post, vnni, ssz = _per_block_geometry(t.shape, block_size, axis, is_vnni, 2)
+    out = np.empty(t.shape[:-1] + (t.shape[-1] // 2,), np.uint8)
+    sc = np.empty(ssz, np.uint8)
+    lib().orc_mxfp4_quantize_generic(
+        _p(t), _c_i64(pre), _c_i64(bs), _c_i64(post), _c_i64(vnni), _p(out), _p(sc)
+    )
+    return out, sc
+
+
+def dequantize_mxfp4(q, sc, block_size=32, axis=2, is_vnni=True):
+    q = _c(q, np.uint8)
+    sc = _c(sc, np.uint8)
+    shape = q.shape[:-1] + (q.shape[-1] * 2,)
+    pre, bs, post, vnni, _ = _per_block_geometry(shape, block_size, axis, is_vnni, 2)
+    out = np.empty(shape, np.float32)
+    lib().orc_mxfp4_dequantize_generic(
+        _p(q), _p(sc), _c_i64(pre), _c_i64(bs), _c_i64(post), _c_i64(vnni), _p(out)
+    )
+    return out
+
+
+def quantize_int8sym(t, block_size, axis, is_vnni):
+    """quantize_int8sym (qtypes.cpp:613-624) on an fp32 array."""
+    t = _c(t, np.float32)
+    pre, bs, post, vnni, ssz = _per_block_geometry(t.shape, block_size, axis, is_vnni, 1)
+    out = np.empty(t.shape, np.int8)
+    sc = np.empty(ssz, np.float32)
+    lib().orc_int8_quantize_generic(
+        _p(t), _c_i64(pre), _c_i64(bs), _c_i64(post), _c_i64(vnni), _p(out), _p(sc)
+    )
+    return out, sc
+
+
+def dequantize_int8sym(q, sc, block_size, axis, is_vnni):
+    q = _c(q, np.int8)
+    sc = _c(sc, np.float32)
+    pre, bs, post, vnni, _ = _per_block_geometry(q.shape, block_size, axis, is_vnni, 1)
+    out = np.empty(q.shape, np.float32)
+    lib().orc_int8_dequantize_generic(
+        _p(q), _p(sc), _c_i64(pre), _c_i64(bs), _c_i64(post), _c_i64(vnni), _p(out)
+    )
+    return out
+
+
+def remap_and_quantize_mxfp4_blocked(Wb):
+    """Full reference entry point on a blocked fp32 array (view/permute chain
+    + generic quantiser).  -> (qdata [N/32,K/64,32,32] u8, scales [N/32,K/64,2,32] u8)"""
+    t = remap_mxfp4(_c(Wb, np.float32))
+    q, sc = quantize_mxfp4(t, 32, 2, True)
+    return q.reshape(q.shape[:-1]), sc
+
+
+def remap_and_quantize_qint8_blocked(Wb, env_block=256):
+    """-> (q [N/bk,K/QBS,QBS/4,bk,4] i8, scales [N/bk,K/QBS,1,bk] f32, QBS)"""
+    t, qbs = remap_qint8(_c(Wb, np.float32), env_block)
+    q, sc = quantize_int8sym(t, qbs, 2, True)
+    return q, sc, qbs
+
+
+# closed-form (plain W[N,K]) versions coded in C -----------------------------
+def remap_quantize_mxfp4(W):
+    W = _c(W, np.float32)
+    N, K = W.shape
+    assert N % 32 == 0 and K % 64 == 0
+    q = np.empty((N // 32, K // 64, 32, 32), np.uint8)
+    sc = np.empty((N // 32, K // 64, 2, 32), np.uint8)
+    lib().orc_remap_quantize_mxfp4(_p(W), _c_i64(N), _c_i64(K), _p(q), _p(sc))
+    return q, sc
+
+
+def dequantize_mxfp4_plain(q, sc):
+    q = _c(q, np.uint8)
+    sc = _c(sc, np.uint8)
+    N, K = q.shape[0] * 32, q.shape[1] * 64
+    W = np.empty((N, K), np.float32)
+    lib().orc_dequantize_mxfp4(_p(q), _p(sc), _c_i64(N), _c_i64(K), _p(W))
+    return W
+
+
+def remap_quantize_qint8(W, qbs=None, env_block=256):
+    W = _c(W, np.float32)
+    N, K = W.shape
+    if qbs is None:
+        qbs = qint8_block_size(K, env_block)
+    assert N % 16 == 0 and K % qbs == 0 and qbs % 64 == 0
+    q = np.empty((N // 16, K // qbs, qbs // 4, 16, 4), np.int8)
+    sc = np.empty((N // 16, K // qbs, 1, 16), np.float32)
+    lib().orc_remap_quantize_qint8(_p(W), _c_i64(N), _c_i64(K), _c_i64(qbs), _p(q), _p(sc))
+    return q, sc, qbs
+
+
+def dequantize_qint8_plain(q, sc):
+    q = _c(q, np.int8)
+    sc = _c(sc, np.float32)
+    n1, nb, a, bk, v = q.shape
+    assert bk == 16 and v == 4
+    qbs = a * 4
+    N, K = n1 * 16, nb * qbs
+    W = np.empty((N, K), np.float32)
+    lib().orc_dequantize_qint8(_p(q), _p(sc), _c_i64(N), _c_i64(K), _c_i64(qbs), _p(W))
+    return W
+
+
+def quant_act_int8(x_bf16, qbs):
+    x = _c(x_bf16, np.uint16)
+    M, K = x.shape
+    xq = np.empty((M, K), np.int8)
+    sa = np.empty((M, K // qbs), np.float32)
+    lib().orc_quant_act_int8(_p(x), _c_i64(M), _c_i64(K), _c_i64(qbs), _p(xq), _p(sa))
+    return xq, sa
+
+
+def qint8_block_sums(xq, q):
+    xq = _c(xq, np.int8)
+    q = _c(q, np.int8)
+    M, K = xq.shape
+    n1, nb, a, bk, v = q.shape
+    N, qbs = n1 * 16, a * 4
+    acc = np.empty((M, N, nb), np.int32)
+    lib().orc_qint8_block_sums(_p(xq), _c_i64(M), _c_i64(K), _p(q), _c_i64(N), _c_i64(qbs), _p(acc))
+    return acc
+
+
+# ----------------------------------------------------------------------------
+# post-ops and linears
+# ----------------------------------------------------------------------------
+def post_op(y_bf16, post, in1=None, in2=None, scale=1.0):
+    y = _c(y_bf16, np.uint16).copy()
+    in1 = None if in1 is None else _c(in1, np.uint16)
+    in2 = None if in2 is None else _c(in2, np.uint16)
+    lib().orc_post_op(_p(y), _c_i64(y.size), ctypes.c_int(post), _p(in1), _p(in2), ctypes.c_float(scale))
+    return y
+
+
+def linear_mxfp4(x_bf16, q, sc, bias=None, post=POST_NONE, post_in=None, post_in2=None,
+                 post_scale=1.0, mode=MODE_IDEAL):
+    x = _c(x_bf16, np.uint16)
+    q = _c(q, np.uint8)
+    sc = _c(sc, np.uint8)
+    M, K = x.shape
+    N = q.shape[0] * 32
+    assert q.shape[1] * 64 == K
+    bias = None if bias is None else _c(bias, np.uint16)
+    post_in = None if post_in is None else _c(post_in, np.uint16)
+    post_in2 = None if post_in2 is None else _c(post_in2, np.uint16)
+    y = np.empty((M, N), np.uint16)
+    lib().orc_linear_mxfp4(
+        _p(x), _c_i64(M), _c_i64(K), _p(q), _p(sc), _c_i64(N), _p(bias), ctypes.c_int(post),
+        _p(post_in), _p(post_in2), ctypes.c_float(post_scale), ctypes.c_int(mode), _p(y),
+    )
+    return y
+
+
+def linear_qint8(x_bf16, q, sw, bias=None, post=POST_NONE, post_in=None, post_in2=None,
+                 post_scale=1.0, mode=MODE_IDEAL):
+    x = _c(x_bf16, np.uint16)
+    q = _c(q, np.int8)
+    sw = _c(sw, np.float32)
+    M, K = x.shape
+    n1, nb, a, bk, v = q.shape
+    N, qbs = n1 * 16, a * 4
+    assert nb * qbs == K
+    bias = None if bias is None else _c(bias, np.uint16)
+    post_in = None if post_in is None else _c(post_in, np.uint16)
+    post_in2 = None if post_in2 is None else _c(post_in2, np.uint16)
+    y = np.empty((M, N), np.uint16)
+    lib().orc_linear_qint8(
+        _p(x), _c_i64(M), _c_i64(K), _p(q), _p(sw), _c_i64(N), _c_i64(qbs), _p(bias),
+        ctypes.c_int(post), _p(post_in), _p(post_in2), ctypes.c_float(post_scale),
+        ctypes.c_int(mode), _p(y),
+    )
+    return y
+
+
+def num_threads():
+    return lib().orc_num_threads()
+
+
+def set_num_threads(n):
+    lib().orc_set_num_threads(ctypes.c_int(int(n)))
