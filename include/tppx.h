@@ -1,0 +1,194 @@
+/*
+ * tppx -- C ABI of the MI355X (gfx950) weight-quantized linear path.
+ *
+ * This is the drop-in boundary for the reference's quantized-linear path
+ * (MXFP4 weight-only and QINT8 W8A8 linears with fused bias / SiLU / mul /
+ * residual-add epilogues, fused QKV, and the quantize / remap helpers).
+ *
+ * Conventions
+ *   - Every function returns 0 on success or a negative TPPX_E* code; nothing
+ *     throws and nothing terminates the process (the reference's TPP_ASSERT
+ *     printf+exit(1), src/csrc/utils.h:34-41, becomes an error code).
+ *     tppx_last_error() returns a thread-local message for the last failure.
+ *   - All data pointers are DEVICE pointers, 16-byte aligned, owned by the
+ *     caller.  The library allocates no device memory.
+ *   - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
+ *     default stream) and the call returns without synchronising.
+ *   - Arguments are validated before any HIP call, so the error paths can be
+ *     exercised on a machine without a GPU.
+ *   - bf16 = bfloat16 bit patterns; M = rows of the activation (tokens),
+ *     K = in-features, N = out-features.
+ *
+ * Weight formats
+ *   "reference layout" (what the quantize entry points emit, byte-identical to
+ *   the reference's QTensor storage):
+ *     MXFP4  qdata  u8 [N/32][K/64][32][32]  byte[nk][nc][c2][k2] holds
+ *                      W[nk*32+k2][nc*64+2*c2] (low nibble) and [..+1] (high)
+ *            scales u8 [N/32][K/64][2][32]   E8M0 of W[nk*32+k2][nc*64+h*32..+31]
+ *     QINT8  q      i8 [N/16][K/QBS][QBS/4][16][4]  = W[n1*16+k2][b*QBS+a*4+v]
+ *            scales f32[N/16][K/QBS][16]
+ *   "native layout" (what the linear entry points consume; produced once by
+ *   tppx_prepack_*; one 1 KiB tile = one wave-wide 128-bit load = one MFMA
+ *   operand):
+ *     MXFP4  qdata  u8 [N/16][K/128][4 g][16 n][16 B]  the 16 B are the 32
+ *                      E2M1 codes of W[nt*16+n][kt*128+g*32 .. +31], even K in
+ *                      the low nibble
+ *            scales u8 [N/16][K/128][4 g][16 n]
+ *     QINT8  q      i8 [N/16][K/64][4 g][16 n][16 B]   W[nt*16+n][kt*64+g*16..+15]
+ *            scales: the reference array is used unchanged.
+ */
+#ifndef TPPX_H
+#define TPPX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TPPX_VERSION 100
+
+#define TPPX_OK 0
+#define TPPX_EINVAL (-1)       /* null / misaligned pointer, bad enum value   */
+#define TPPX_ESHAPE (-2)       /* a shape constraint of the path is violated  */
+#define TPPX_EUNSUPPORTED (-3) /* legal in the reference, not built here      */
+#define TPPX_EHIP (-4)         /* the HIP runtime reported an error           */
+
+/* Post-ops, applied to the bf16-rounded GEMM(+bias) tile exactly where the
+ * reference applies them (src/csrc/fused_gemm.h:1343-1488). */
+#define TPPX_POST_NONE 0       /* NullPostOp      fused_gemm.h:1343 */
+#define TPPX_POST_SILU 1       /* SiluPostOp      fused_gemm.h:1369 */
+#define TPPX_POST_MUL 2        /* MulPostOp       fused_gemm.h:1409 */
+#define TPPX_POST_ADD_SCALE 3  /* AddScalePostOp  fused_gemm.h:1434 */
+#define TPPX_POST_ADD2_SCALE 4 /* Add2ScalePostOp fused_gemm.h:1460 */
+#define TPPX_POST_GELU 5       /* GeluPostOp      fused_gemm.h:1349 */
+#define TPPX_POST_RELU 6       /* ReluPostOp      fused_gemm.h:1389 */
+
+/* Element type of a floating-point weight handed to the quantizers. */
+#define TPPX_DT_F32 0
+#define TPPX_DT_BF16 1
+
+/* flags for the linear entry points */
+#define TPPX_FLAG_NONE 0
+#define TPPX_FLAG_FORCE_SKINNY 1 /* always take the decode (streaming) kernel */
+#define TPPX_FLAG_FORCE_TILED 2  /* always take the prefill (LDS-tiled) kernel */
+#define TPPX_FLAG_ACT_FP8 4      /* MXFP4 prefill: round activations to MXFP8
+                                    (E4M3 + E8M0/32) and use the scaled
+                                    f8f6f4 MFMA -- NOT the reference numerics */
+
+typedef void* tppx_stream_t;
+
+int tppx_version(void);
+const char* tppx_last_error(void);
+
+/* ---- quantize / remap -------------------------------------------------- */
+
+/* Replaces qtype.remap_and_quantize_mxfp4 (src/csrc/qtypes.cpp:783-864; bound
+ * at qtypes.cpp:1089).  `w` is a blocked weight whose element (n,k) lives at
+ *   ((n/bk)*(K/bc) + k/bc)*bk*bc + ((k%bc)/vnni)*bk*vnni + (n%bk)*vnni + k%vnni
+ * (bk=1, bc=K, vnni=1 describes a plain row-major [N][K]); the 5-D bf16
+ * tensors of the reference are bk=16, bc=64, vnni=2, the 4-D fp32 ones
+ * vnni=1.  Needs N%32==0, K%64==0.  Output: reference layout. */
+int tppx_quantize_mxfp4(const void* w, int w_dtype, int64_t N, int64_t K,
+                        int64_t bk, int64_t bc, int64_t vnni, void* qdata,
+                        void* scales, tppx_stream_t stream);
+
+/* Replaces qtype.remap_and_quantize_qint8 (src/csrc/qtypes.cpp:866-932; bound
+ * at qtypes.cpp:1091).  qbs is the K block the caller derived with the
+ * reference rule (256 if it divides K, else the largest smaller power of two
+ * >= 64 that does).  Needs N%16==0, K%qbs==0, qbs%64==0. */
+int tppx_quantize_qint8(const void* w, int w_dtype, int64_t N, int64_t K,
+                        int64_t bk, int64_t bc, int64_t vnni, int64_t qbs,
+                        void* q, void* scales, tppx_stream_t stream);
+
+/* Replaces at::Tensor::dequantize() of the two custom quantizers
+ * (PerBlockMxFPQuantizer / PerBlockAffineQuantizer::dequantize,
+ * src/csrc/qtypes.cpp:438-473,521-577).  Output fp32 in the blocked shape of
+ * the quantized tensor: [N/32][K/64][32][32][2] resp. [N/16][K/QBS][QBS/4][16][4]. */
+int tppx_dequantize_mxfp4(const void* qdata, const void* scales, int64_t N,
+                          int64_t K, void* out_f32, tppx_stream_t stream);
+int tppx_dequantize_qint8(const void* q, const void* scales, int64_t N,
+                          int64_t K, int64_t qbs, void* out_f32,
+                          tppx_stream_t stream);
+
+/* Reference layout -> native layout.  Plays the role of the reference's cached
+ * first-token weight remap (wt_tensor_for_first_token,
+ * src/csrc/llm/fused_llm_infer.cpp:366-420): a one-time re-layout kept next to
+ * the weight.  MXFP4 needs K%128==0. */
+int tppx_prepack_mxfp4(const void* qdata_ref, const void* scales_ref, int64_t N,
+                       int64_t K, void* qdata_nat, void* scales_nat,
+                       tppx_stream_t stream);
+int tppx_prepack_qint8(const void* q_ref, int64_t N, int64_t K, int64_t qbs,
+                       void* q_nat, tppx_stream_t stream);
+
+/* Replaces quantize_int8sym(t_in, block_size, -1, false) on the activation
+ * (src/csrc/fused_gemm.h:1249 -> src/csrc/qtypes.cpp:613-624): x bf16 [M][K]
+ * -> xq i8 [M][K], sa f32 [M][K/qbs]. */
+int tppx_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs,
+                        void* xq, void* sa, tppx_stream_t stream);
+
+/* ---- linears ----------------------------------------------------------- */
+
+/* Replaces call_gemm_with_post_op -> TppBlockedLinearW<bf16,uint8_t,bf16>
+ * (MXFP4 branch, src/csrc/fused_gemm.h:785-1073,1510-1522) i.e.
+ * torch.ops.tpp_llm.fc_plain (src/csrc/llm/fused_llm_infer.cpp:1514,1589) and
+ * the post-op GEMMs of the decoder layer (fused_llm_infer.cpp:1261-1273).
+ *   y[M][N] = post( bf16( bias[n] + sum_k x[m][k]*deq(W)[n][k] ) )
+ * x bf16 [M][K]; qw/sw native layout; bias bf16 [N] or NULL; post_in /
+ * post_in2 bf16 [M][N] as the post-op needs; y bf16 [M][N]. */
+int tppx_linear_mxfp4(const void* x, const void* qw, const void* sw,
+                      const void* bias, const void* post_in,
+                      const void* post_in2, void* y, int64_t M, int64_t N,
+                      int64_t K, int post_op, float post_scale, int flags,
+                      tppx_stream_t stream);
+
+/* Replaces TppBlockedQInt8LinearW<bf16,uint8_t,bf16>
+ * (src/csrc/fused_gemm.h:1076-1341,1530-1534): activations are quantized into
+ * the caller's scratch xq (i8 [M][K]) / sa (f32 [M][K/qbs]) and then
+ *   y = post( bf16( bias + sum_b float(sum_{k in b} xq*wq) * sa[m][b]*sw[n][b] ) ) */
+int tppx_linear_qint8(const void* x, void* xq, void* sa, const void* qw,
+                      const void* sw, const void* bias, const void* post_in,
+                      const void* post_in2, void* y, int64_t M, int64_t N,
+                      int64_t K, int64_t qbs, int post_op, float post_scale,
+                      int flags, tppx_stream_t stream);
+
+/* One GEMM of a fused group sharing the activation. */
+typedef struct tppx_seg {
+  const void* qw;       /* native weight */
+  const void* sw;       /* its scales    */
+  const void* bias;     /* bf16 [N] or NULL */
+  const void* post_in;  /* bf16 [M][N] or NULL */
+  const void* post_in2; /* bf16 [M][N] or NULL */
+  void* y;              /* bf16 [M][N] */
+  int64_t N;
+  int32_t post_op;
+  float post_scale;
+} tppx_seg;
+
+/* Replaces fused_qkv_gemm -> TppBlockedLinearW::fused_gemm /
+ * TppBlockedQInt8LinearW::fused_gemm (src/csrc/llm/fused_llm_infer.cpp:423-505,
+ * src/csrc/fused_gemm.h:1001-1064,1273-1332): up to 4 GEMMs over one
+ * activation in one launch, each with its own output tensor and post-op. */
+int tppx_multi_linear_mxfp4(const void* x, const tppx_seg* segs, int n_segs,
+                            int64_t M, int64_t K, int flags,
+                            tppx_stream_t stream);
+int tppx_multi_linear_qint8(const void* x, void* xq, void* sa,
+                            const tppx_seg* segs, int n_segs, int64_t M,
+                            int64_t K, int64_t qbs, int flags,
+                            tppx_stream_t stream);
+
+/* Replaces the gate/up pair of the Llama MLP
+ * (src/csrc/llm/fused_llm_infer.cpp:1271-1272: i_gemm(SiluPostOp) then
+ * i_gemm(MulPostOp)) in one launch with the same bf16 rounding points:
+ *   g = silu(bf16(x Wg^T + bg));  y = bf16( g * bf16(x Wu^T + bu) ) */
+int tppx_swiglu_mxfp4(const void* x, const void* qw_gate, const void* sw_gate,
+                      const void* bias_gate, const void* qw_up,
+                      const void* sw_up, const void* bias_up, void* y,
+                      int64_t M, int64_t N, int64_t K, int flags,
+                      tppx_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TPPX_H */

@@ -1,0 +1,161 @@
+"""Parity of the HIP linears against the CPU oracle (ideal mode: fp32
+accumulate, one bf16 rounding, reference rounding points in the post-ops).
+
+Stated tolerance: every output within 1 bf16 ulp of the oracle (2 ulp where a
+sigmoid is involved, because libm's and the GPU's expf differ in the last
+bit), relative L2 error <= 4e-3; against the reference's own bf16 re-rounding
+schedule (faithful mode) rel-L2 <= 2^-9 * sqrt(#K-groups) for QINT8.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from util import t2bits, randn_bf16, block_bf16, assert_close_bf16, err_stats
+
+pytestmark = pytest.mark.gpu
+
+POSTS = {"none": O.POST_NONE, "silu": O.POST_SILU, "mul": O.POST_MUL, "add": O.POST_ADD_SCALE,
+         "add2": O.POST_ADD2_SCALE, "gelu": O.POST_GELU, "relu": O.POST_RELU}
+
+
+def _ops():
+    import tpp_pytorch_extension  # noqa: F401
+    from tpp_pytorch_extension import _ops
+    return _ops
+
+
+def _make(fmt, N, K, seed):
+    ops = _ops()
+    W = randn_bf16((N, K), 0.02, seed)
+    Wb = block_bf16(W).cuda()
+    if fmt == "mxfp4":
+        qw = ops.remap_and_quantize_mxfp4(Wb)
+        q_or, s_or = O.remap_quantize_mxfp4(W.float().numpy())
+    else:
+        qw = ops.remap_and_quantize_qint8(Wb)
+        q_or, s_or, _ = O.remap_quantize_qint8(W.float().numpy())
+    # the quantized bytes must be identical before the GEMM is compared
+    assert np.array_equal(qw.qdata.cpu().numpy(), q_or), "quantized values differ from the oracle"
+    assert np.array_equal(qw.scales.cpu().numpy().reshape(s_or.shape), s_or), "scales differ from the oracle"
+    return qw, q_or, s_or
+
+
+def _run(fmt, M, N, K, post, with_bias, seed, ulps=1):
+    ops = _ops()
+    qw, q_or, s_or = _make(fmt, N, K, seed)
+    x = randn_bf16((M, K), 1.0, seed + 1)
+    bias = randn_bf16((N,), 0.01, seed + 2) if with_bias else None
+    in1 = randn_bf16((M, N), 1.0, seed + 3)
+    in2 = randn_bf16((M, N), 1.0, seed + 4)
+    scale = 0.5 if post in ("add", "add2") else 1.0
+    y = ops.linear(x.cuda(), qw, None if bias is None else bias.cuda(), POSTS[post],
+                   in1.cuda(), in2.cuda(), scale)
+    torch.cuda.synchronize()
+    lin = O.linear_mxfp4 if fmt == "mxfp4" else O.linear_qint8
+    ref = lin(t2bits(x), q_or, s_or, None if bias is None else t2bits(bias), POSTS[post],
+              t2bits(in1), t2bits(in2), scale, O.MODE_IDEAL)
+    s = assert_close_bf16(t2bits(y), ref, ulps=ulps, what=f"{fmt} M={M} N={N} K={K} post={post}")
+    return y, ref, s, (qw, q_or, s_or, x, bias, in1, in2, scale)
+
+
+@pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 64])
+def test_fc_plain_small(fmt, M):
+    _run(fmt, M, 256, 512, "none", True, 100 + M)
+
+
+@pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])
+@pytest.mark.parametrize("post", ["silu", "mul", "add", "add2", "gelu", "relu"])
+def test_post_ops(fmt, post):
+    _run(fmt, 5, 128, 768, post, post != "mul", 200, ulps=2 if post in ("silu", "gelu") else 1)
+
+
+@pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])
+def test_no_bias_ragged_k(fmt):
+    # K = 11008 = 86*128 = 43*256: an odd number of K units, waves get uneven ranges
+    _run(fmt, 8, 64, 11008, "none", False, 300)
+
+
+def test_cfg1_mxfp4_fc_plain():
+    """BASELINE config 1: M=16, K=N=4096, MXFP4, bias."""
+    _run("mxfp4", 16, 4096, 4096, "none", True, 1235)
+
+
+@pytest.mark.parametrize("M", [1, 8, 32, 64])
+def test_cfg2_qint8_fc_add(M):
+    """BASELINE config 2 (down-projection shape scaled in N to keep the CPU oracle fast)."""
+    y, ref, s, ctx = _run("qint8", M, 512, 11008, "add", False, 1236 + M)
+    qw, q_or, s_or, x, bias, in1, in2, scale = ctx
+    faithful = O.linear_qint8(t2bits(x), q_or, s_or, None, O.POST_ADD_SCALE, t2bits(in1), None, scale,
+                              O.MODE_FAITHFUL)
+    st = err_stats(t2bits(y), faithful)
+    groups = 11008 // (256 if M == 64 else 64)
+    assert st["rel_l2"] <= 2.0 ** -9 * np.sqrt(groups), st["rel_l2"]
+
+
+def test_qint8_block_64_and_128():
+    ops = _ops()
+    for K in (192, 384):  # -> QBS 64 and 128 by the reference's rule
+        W = randn_bf16((64, K), 0.02, 7)
+        qw = ops.remap_and_quantize_qint8(block_bf16(W).cuda())
+        q_or, s_or, qbs = O.remap_quantize_qint8(W.float().numpy())
+        assert qw.block_size == qbs
+        assert np.array_equal(qw.qdata.cpu().numpy(), q_or)
+        x = randn_bf16((4, K), 1.0, 8)
+        y = ops.fc_plain(x.cuda(), qw, torch.Tensor())
+        ref = O.linear_qint8(t2bits(x), q_or, s_or)
+        assert_close_bf16(t2bits(y), ref, what=f"qbs={qbs}")
+
+
+@pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])
+def test_qkv_gemm_equals_separate(fmt):
+    ops = _ops()
+    K, M = 1024, 7
+    ws = [_make(fmt, n, K, 40 + i)[0] for i, n in enumerate((512, 128, 128))]
+    bs = [randn_bf16((n,), 0.01, 50 + i).cuda() for i, n in enumerate((512, 128, 128))]
+    x = randn_bf16((2, M, K), 1.0, 60).cuda()
+    outs = torch.ops.tpp_llm.qkv_gemm(x, ws, bs)
+    for w, b, o in zip(ws, bs, outs):
+        sep = torch.ops.tpp_llm.fc_plain(x, w, b, -1, [])
+        assert o.shape == sep.shape == (2, M, w.weight_nk()[0])
+        assert torch.equal(o, sep)
+
+
+def test_swiglu_fused_equals_composition():
+    ops = _ops()
+    K, N, M = 512, 1024, 9
+    wg, wu = _make("mxfp4", N, K, 70)[0], _make("mxfp4", N, K, 71)[0]
+    wd = _make("mxfp4", K, N, 72)[0]
+    x = randn_bf16((M, K), 1.0, 73).cuda()
+    fused = ops.swiglu_gate_up(x, wg, wu)
+    g = ops.fc_silu(x, wg, None)
+    u = ops.fc_mul(x, wu, None, g)
+    assert torch.equal(fused, u)
+    out = torch.ops.tpp_llm.swiglu_mlp(x, wg, wu, wd, x, 1.0)
+    assert torch.equal(out, ops.fc_add(u, wd, None, x, 1.0))
+
+
+def test_module_api_and_errors():
+    import tpp_pytorch_extension  # noqa: F401
+    from tpp_pytorch_extension.llm.llm_common import FixLinear, BlockedLinear
+    from tpp_pytorch_extension._lib import TppxError
+
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(256, 128, bias=True)
+    W, b = lin.weight.data.clone(), lin.bias.data.clone()
+    FixLinear(lin, 16, 64, torch.bfloat16, weight_dtype="mxfp4")
+    assert isinstance(lin, BlockedLinear) and lin.weight.is_quantized
+    assert lin.weight.dtype == torch.quint4x2 and lin.weight.size(-1) == 2
+    x = torch.randn(3, 5, 256).cuda()
+    y = lin(x)  # fp32 input is cast to bf16 by the module, as in the reference
+    q_or, s_or = O.remap_quantize_mxfp4(W.to(torch.bfloat16).float().numpy())
+    ref = O.linear_mxfp4(t2bits(x.to(torch.bfloat16).view(15, 256)), q_or, s_or, t2bits(b.to(torch.bfloat16)))
+    assert y.shape == (3, 5, 128) and y.dtype == torch.bfloat16
+    assert_close_bf16(t2bits(y).reshape(15, 128), ref, what="BlockedLinear")
+    with pytest.raises(TppxError):
+        torch.ops.tpp_llm.fc_plain(x.to(torch.bfloat16)[..., :128].contiguous(), lin.weight, torch.Tensor(), -1, [])
+    with pytest.raises(TppxError):
+        torch.ops.tpp_llm.fc_plain(x, lin.weight, torch.Tensor(), -1, [])  # fp32 activations
+    e = torch.ops.tpp_llm.fc_plain(torch.empty(0, 256, dtype=torch.bfloat16).cuda(), lin.weight, torch.Tensor(), -1, [])
+    assert e.shape == (0, 128)

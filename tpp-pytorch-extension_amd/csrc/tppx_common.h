@@ -1,0 +1,86 @@
+// Shared host/device helpers of the gfx950 quantized-linear library.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tppx.h"
+
+namespace tppx {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(16))) int i32x16;
+
+// ---- error plumbing (host) ------------------------------------------------
+int set_error(int code, const char* fmt, ...);
+int check_hip(hipError_t e, const char* what);
+
+#define TPPX_REQUIRE(cond, code, ...)          \
+  do {                                         \
+    if (!(cond))                               \
+      return ::tppx::set_error(code, __VA_ARGS__); \
+  } while (0)
+
+static inline bool aligned16(const void* p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+// ---- bf16 <-> fp32 (device) -----------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) {
+  return __uint_as_float(h << 16);
+}
+
+// round to nearest even, NaN kept quiet (same rule as the CPU side)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u)
+    return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+__device__ __forceinline__ float round_bf16(float f) {
+  return bf16_bits_to_f32(f32_to_bf16_bits(f));
+}
+
+// ---- post-ops on the bf16-rounded GEMM result -------------------------------
+// `v` is bias + dot product in fp32.  The value is rounded to bf16 first and
+// every post-op re-rounds where the CPU path stores its bf16 tile.
+__device__ __forceinline__ uint32_t apply_post_bits(float v, int post,
+                                                    uint32_t in1, uint32_t in2,
+                                                    float scale) {
+  uint32_t yb = f32_to_bf16_bits(v);
+  float y = bf16_bits_to_f32(yb);
+  switch (post) {
+    case TPPX_POST_SILU: {
+      float s = round_bf16(1.0f / (1.0f + expf(-y)));
+      return f32_to_bf16_bits(y * s);
+    }
+    case TPPX_POST_MUL:
+      return f32_to_bf16_bits(bf16_bits_to_f32(in1) * y);
+    case TPPX_POST_ADD_SCALE:
+      return f32_to_bf16_bits(fmaf(bf16_bits_to_f32(in1), scale, y));
+    case TPPX_POST_ADD2_SCALE: {
+      float t = round_bf16(y + bf16_bits_to_f32(in1));
+      return f32_to_bf16_bits(fmaf(bf16_bits_to_f32(in2), scale, t));
+    }
+    case TPPX_POST_GELU:
+      return f32_to_bf16_bits(0.5f * y * (1.0f + erff(y * 0.70710678118654752f)));
+    case TPPX_POST_RELU:
+      return (yb & 0x8000u) ? 0u : yb;
+    default:
+      return yb;
+  }
+}
+
+// E8M0 byte -> fp32 factor used when de-quantising (byte shifted into the
+// exponent field; 0 gives 0.0, 255 gives +Inf).
+__device__ __forceinline__ float e8m0_to_f32(uint32_t x) {
+  return __uint_as_float((x & 0xffu) << 23);
+}
+
+} // namespace tppx

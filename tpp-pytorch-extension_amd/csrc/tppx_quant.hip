@@ -1,0 +1,395 @@
+// Quantize / de-quantize / re-layout kernels (HBM-bound byte work, one-time per
+// weight except for the activation quantizer which runs on every QINT8 call).
+#include "tppx_common.h"
+
+namespace tppx {
+
+// offset of element (n,k) of a blocked weight (see tppx_quantize_mxfp4 in tppx.h)
+__device__ __forceinline__ int64_t blocked_off(int64_t n, int64_t k, int64_t K,
+                                               int64_t bk, int64_t bc,
+                                               int64_t vnni) {
+  int64_t kb = k % bc;
+  return ((n / bk) * (K / bc) + k / bc) * bk * bc + (kb / vnni) * bk * vnni +
+      (n % bk) * vnni + kb % vnni;
+}
+
+template <typename T>
+__device__ __forceinline__ float load_as_f32(const T* p, int64_t i);
+template <>
+__device__ __forceinline__ float load_as_f32<float>(const float* p, int64_t i) {
+  return p[i];
+}
+template <>
+__device__ __forceinline__ float load_as_f32<uint16_t>(const uint16_t* p,
+                                                      int64_t i) {
+  return bf16_bits_to_f32(p[i]);
+}
+
+// E2M1 code of an already scaled value: nearest, ties to even mantissa,
+// saturating at 6, +-0 -> 0, NaN -> 0.
+__device__ __forceinline__ uint32_t e2m1_encode(float v) {
+  if (v != v)
+    return 0;
+  float a = fabsf(v);
+  uint32_t c = a <= 0.25f ? 0u
+      : a < 0.75f         ? 1u
+      : a <= 1.25f        ? 2u
+      : a < 1.75f         ? 3u
+      : a <= 2.5f         ? 4u
+      : a < 3.5f          ? 5u
+      : a <= 5.0f         ? 6u
+                          : 7u;
+  if (c != 0 && (__float_as_uint(v) >> 31))
+    c |= 8u;
+  return c;
+}
+
+// One thread per MX block (one output channel x 32 consecutive K).
+// Threads are ordered with the channel-in-32 index fastest so that the byte
+// and scale stores of a wave fall into contiguous 32-byte runs.
+template <typename T>
+__global__ void __launch_bounds__(256)
+quantize_mxfp4_kernel(const T* __restrict__ w, int64_t N, int64_t K, int64_t bk,
+                      int64_t bc, int64_t vnni, uint8_t* __restrict__ qdata,
+                      uint8_t* __restrict__ scales) {
+  int64_t nblk = (N / 32) * (K / 64) * 2 * 32;
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= nblk)
+    return;
+  int64_t k2 = t & 31;
+  int64_t h = (t >> 5) & 1;
+  int64_t rest = t >> 6;
+  int64_t Nc = K / 64;
+  int64_t nc = rest % Nc, nk = rest / Nc;
+  int64_t n = nk * 32 + k2, k0 = nc * 64 + h * 32;
+  float v[32];
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 32; j++) {
+    v[j] = load_as_f32<T>(w, blocked_off(n, k0 + j, K, bk, bc, vnni));
+    float a = fabsf(v[j]);
+    amax = a > amax ? a : amax;
+  }
+  int e = (int)((__float_as_uint(amax) >> 23) & 0xffu);
+  bool flush = (e == 0);
+  int x = (e == 255) ? 255 : (e - 2 < 0 ? 0 : e - 2);
+  scales[((nk * Nc + nc) * 2 + h) * 32 + k2] = (uint8_t)x;
+  // division by the power-of-two scale is an exact exponent shift; x == 0
+  // stands for 2^-127, x == 255 for NaN (all codes 0)
+  int sh = 127 - x;
+#pragma unroll
+  for (int p = 0; p < 16; p++) {
+    uint32_t c0 = 0, c1 = 0;
+    if (!flush && x != 255) {
+      c0 = e2m1_encode(ldexpf(v[2 * p], sh));
+      c1 = e2m1_encode(ldexpf(v[2 * p + 1], sh));
+    }
+    qdata[((nk * Nc + nc) * 32 + (h * 16 + p)) * 32 + k2] =
+        (uint8_t)(c0 | (c1 << 4));
+  }
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1)
+    v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+__device__ __forceinline__ float int8_scale_of(float amax) {
+  return (float)((double)amax / 127.0);
+}
+__device__ __forceinline__ float int8_inv_scale(float s) {
+  return s != 0.0f ? __frcp_rn(s) : 0.0f;
+}
+__device__ __forceinline__ int int8_q(float v, float inv) {
+  float r = rintf(__fmul_rn(v, inv));
+  r = fminf(fmaxf(r, -127.0f), 127.0f);
+  return (int)r;
+}
+
+// One wave per (output channel, K block of qbs).
+template <typename T>
+__global__ void __launch_bounds__(256)
+quantize_qint8_kernel(const T* __restrict__ w, int64_t N, int64_t K, int64_t bk,
+                      int64_t bc, int64_t vnni, int64_t qbs,
+                      int8_t* __restrict__ q, float* __restrict__ scales) {
+  int64_t nb = K / qbs;
+  int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  int lane = threadIdx.x & 63;
+  if (wave >= N * nb)
+    return;
+  // channel-in-16 fastest so neighbouring waves write neighbouring rows
+  int64_t k2 = wave & 15;
+  int64_t rest = wave >> 4;
+  int64_t b = rest % nb, n1 = rest / nb;
+  int64_t n = n1 * 16 + k2;
+  float amax = 0.0f;
+  for (int64_t j = lane; j < qbs; j += 64) {
+    float a = fabsf(load_as_f32<T>(w, blocked_off(n, b * qbs + j, K, bk, bc, vnni)));
+    amax = a > amax ? a : amax;
+  }
+  amax = wave_max(amax);
+  float s = int8_scale_of(amax);
+  float inv = int8_inv_scale(s);
+  if (lane == 0)
+    scales[(n1 * nb + b) * 16 + k2] = s;
+  for (int64_t j = lane; j < qbs; j += 64) {
+    float v = load_as_f32<T>(w, blocked_off(n, b * qbs + j, K, bk, bc, vnni));
+    q[(((n1 * nb + b) * (qbs / 4) + (j >> 2)) * 16 + k2) * 4 + (j & 3)] =
+        (int8_t)int8_q(v, inv);
+  }
+}
+
+__constant__ float c_e2m1_tbl[16] = {0.0f,  0.5f,  1.0f,  1.5f, 2.0f,  3.0f,
+                                     4.0f,  6.0f,  -0.0f, -0.5f, -1.0f, -1.5f,
+                                     -2.0f, -3.0f, -4.0f, -6.0f};
+
+// one thread per packed byte; out is [N/32][K/64][32][32][2] fp32
+__global__ void __launch_bounds__(256)
+dequantize_mxfp4_kernel(const uint8_t* __restrict__ qdata,
+                        const uint8_t* __restrict__ scales, int64_t nbytes,
+                        float* __restrict__ out) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= nbytes)
+    return;
+  int64_t k2 = t & 31, c2 = (t >> 5) & 31, tile = t >> 10;
+  uint32_t b = qdata[t];
+  float s = e8m0_to_f32(scales[(tile * 2 + (c2 >> 4)) * 32 + k2]);
+  float2 r;
+  r.x = c_e2m1_tbl[b & 0xf] * s;
+  r.y = c_e2m1_tbl[b >> 4] * s;
+  reinterpret_cast<float2*>(out)[t] = r;
+}
+
+// one thread per 4 int8; out [N/16][K/QBS][QBS/4][16][4] fp32
+__global__ void __launch_bounds__(256)
+dequantize_qint8_kernel(const int8_t* __restrict__ q,
+                        const float* __restrict__ scales, int64_t ngroups,
+                        int64_t qbs, float* __restrict__ out) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= ngroups)
+    return;
+  int64_t k2 = t & 15;
+  int64_t blk = (t >> 4) / (qbs / 4); // (n1*nb + b)
+  float s = scales[blk * 16 + k2];
+  uint32_t v = reinterpret_cast<const uint32_t*>(q)[t];
+  float4 r;
+  r.x = (float)(int8_t)(v & 0xff) * s;
+  r.y = (float)(int8_t)((v >> 8) & 0xff) * s;
+  r.z = (float)(int8_t)((v >> 16) & 0xff) * s;
+  r.w = (float)(int8_t)(v >> 24) * s;
+  reinterpret_cast<float4*>(out)[t] = r;
+}
+
+// one thread per native 16-byte chunk (nt, kt, g, n)
+__global__ void __launch_bounds__(256)
+prepack_mxfp4_kernel(const uint8_t* __restrict__ qref,
+                     const uint8_t* __restrict__ sref, int64_t N, int64_t K,
+                     uint8_t* __restrict__ qnat, uint8_t* __restrict__ snat) {
+  int64_t nchunks = N * (K / 32);
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= nchunks)
+    return;
+  int64_t n16 = t & 15, g = (t >> 4) & 3, rest = t >> 6;
+  int64_t KT = K / 128, Nc = K / 64;
+  int64_t kt = rest % KT, nt = rest / KT;
+  int64_t n = nt * 16 + n16, k0 = kt * 128 + g * 32;
+  int64_t nk = n >> 5, k2 = n & 31, nc = k0 >> 6, c2b = (k0 & 63) >> 1;
+  const uint8_t* src = qref + ((nk * Nc + nc) * 32 + c2b) * 32 + k2;
+  uint32_t wd[4];
+#pragma unroll
+  for (int d = 0; d < 4; d++) {
+    uint32_t v = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      v |= (uint32_t)src[(d * 4 + i) * 32] << (8 * i);
+    wd[d] = v;
+  }
+  reinterpret_cast<uint4*>(qnat)[t] = make_uint4(wd[0], wd[1], wd[2], wd[3]);
+  snat[t] = sref[((nk * Nc + nc) * 2 + ((k0 & 63) >> 5)) * 32 + k2];
+}
+
+__global__ void __launch_bounds__(256)
+prepack_qint8_kernel(const int8_t* __restrict__ qref, int64_t N, int64_t K,
+                     int64_t qbs, int8_t* __restrict__ qnat) {
+  int64_t nchunks = N * (K / 16);
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= nchunks)
+    return;
+  int64_t n16 = t & 15, g = (t >> 4) & 3, rest = t >> 6;
+  int64_t KT = K / 64, nb = K / qbs;
+  int64_t kt = rest % KT, nt = rest / KT;
+  int64_t k0 = kt * 64 + g * 16;
+  int64_t b = k0 / qbs, a0 = (k0 % qbs) >> 2;
+  const uint32_t* src = reinterpret_cast<const uint32_t*>(qref) +
+      ((nt * nb + b) * (qbs / 4) + a0) * 16 + n16;
+  reinterpret_cast<uint4*>(qnat)[t] =
+      make_uint4(src[0], src[16], src[32], src[48]);
+}
+
+// Activation quantizer: one wave per (row, K block).  Each lane owns
+// consecutive pairs so loads and stores stay contiguous.
+__global__ void __launch_bounds__(256)
+quant_act_int8_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
+                      int64_t qbs, int8_t* __restrict__ xq,
+                      float* __restrict__ sa) {
+  int64_t nb = K / qbs;
+  int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  int lane = threadIdx.x & 63;
+  if (wave >= M * nb)
+    return;
+  int64_t m = wave / nb, b = wave % nb;
+  const uint16_t* p = x + m * K + b * qbs;
+  int8_t* o = xq + m * K + b * qbs;
+  if (qbs == 256) {
+    // 4 consecutive bf16 per lane
+    uint2 raw = reinterpret_cast<const uint2*>(p)[lane];
+    float v0 = bf16_bits_to_f32(raw.x & 0xffffu), v1 = bf16_bits_to_f32(raw.x >> 16);
+    float v2 = bf16_bits_to_f32(raw.y & 0xffffu), v3 = bf16_bits_to_f32(raw.y >> 16);
+    float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
+    amax = wave_max(amax);
+    float s = int8_scale_of(amax);
+    float inv = int8_inv_scale(s);
+    if (lane == 0)
+      sa[m * nb + b] = s;
+    uint32_t packed = (uint32_t)(int8_q(v0, inv) & 0xff) |
+        ((uint32_t)(int8_q(v1, inv) & 0xff) << 8) |
+        ((uint32_t)(int8_q(v2, inv) & 0xff) << 16) |
+        ((uint32_t)(int8_q(v3, inv) & 0xff) << 24);
+    reinterpret_cast<uint32_t*>(o)[lane] = packed;
+  } else {
+    float amax = 0.0f;
+    for (int64_t j = lane; j < qbs; j += 64)
+      amax = fmaxf(amax, fabsf(bf16_bits_to_f32(p[j])));
+    amax = wave_max(amax);
+    float s = int8_scale_of(amax);
+    float inv = int8_inv_scale(s);
+    if (lane == 0)
+      sa[m * nb + b] = s;
+    for (int64_t j = lane; j < qbs; j += 64)
+      o[j] = (int8_t)int8_q(bf16_bits_to_f32(p[j]), inv);
+  }
+}
+
+static inline unsigned grid_for(int64_t n, int block) {
+  return (unsigned)((n + block - 1) / block);
+}
+
+} // namespace tppx
+
+using namespace tppx;
+
+extern "C" int tppx_quantize_mxfp4(const void* w, int w_dtype, int64_t N,
+                                   int64_t K, int64_t bk, int64_t bc,
+                                   int64_t vnni, void* qdata, void* scales,
+                                   tppx_stream_t stream) {
+  TPPX_REQUIRE(w && qdata && scales, TPPX_EINVAL, "tppx_quantize_mxfp4: null pointer");
+  TPPX_REQUIRE(w_dtype == TPPX_DT_F32 || w_dtype == TPPX_DT_BF16, TPPX_EINVAL,
+               "tppx_quantize_mxfp4: unknown weight dtype %d", w_dtype);
+  TPPX_REQUIRE(N > 0 && K > 0 && N % 32 == 0 && K % 64 == 0, TPPX_ESHAPE,
+               "tppx_quantize_mxfp4: shape not compatible for MXFP4 (N=%ld must be a multiple of 32, K=%ld of 64)",
+               (long)N, (long)K);
+  TPPX_REQUIRE(bk > 0 && bc > 0 && vnni > 0 && N % bk == 0 && K % bc == 0 && bc % vnni == 0,
+               TPPX_ESHAPE, "tppx_quantize_mxfp4: blocking (bk=%ld, bc=%ld, vnni=%ld) does not divide [%ld,%ld]",
+               (long)bk, (long)bc, (long)vnni, (long)N, (long)K);
+  int64_t nblk = N * (K / 32);
+  hipStream_t s = (hipStream_t)stream;
+  if (w_dtype == TPPX_DT_F32)
+    quantize_mxfp4_kernel<float><<<grid_for(nblk, 256), 256, 0, s>>>(
+        (const float*)w, N, K, bk, bc, vnni, (uint8_t*)qdata, (uint8_t*)scales);
+  else
+    quantize_mxfp4_kernel<uint16_t><<<grid_for(nblk, 256), 256, 0, s>>>(
+        (const uint16_t*)w, N, K, bk, bc, vnni, (uint8_t*)qdata, (uint8_t*)scales);
+  return check_hip(hipGetLastError(), "tppx_quantize_mxfp4");
+}
+
+extern "C" int tppx_quantize_qint8(const void* w, int w_dtype, int64_t N,
+                                   int64_t K, int64_t bk, int64_t bc,
+                                   int64_t vnni, int64_t qbs, void* q,
+                                   void* scales, tppx_stream_t stream) {
+  TPPX_REQUIRE(w && q && scales, TPPX_EINVAL, "tppx_quantize_qint8: null pointer");
+  TPPX_REQUIRE(w_dtype == TPPX_DT_F32 || w_dtype == TPPX_DT_BF16, TPPX_EINVAL,
+               "tppx_quantize_qint8: unknown weight dtype %d", w_dtype);
+  TPPX_REQUIRE(N > 0 && K > 0 && N % 16 == 0 && K % 64 == 0, TPPX_ESHAPE,
+               "tppx_quantize_qint8: N=%ld must be a multiple of 16 and K=%ld of 64", (long)N, (long)K);
+  TPPX_REQUIRE(qbs > 0 && qbs % 64 == 0 && K % qbs == 0, TPPX_ESHAPE,
+               "tppx_quantize_qint8: block size %ld must be a multiple of 64 dividing K=%ld", (long)qbs, (long)K);
+  TPPX_REQUIRE(bk > 0 && bc > 0 && vnni > 0 && N % bk == 0 && K % bc == 0 && bc % vnni == 0,
+               TPPX_ESHAPE, "tppx_quantize_qint8: blocking (bk=%ld, bc=%ld, vnni=%ld) does not divide [%ld,%ld]",
+               (long)bk, (long)bc, (long)vnni, (long)N, (long)K);
+  int64_t nthreads = N * (K / qbs) * 64;
+  hipStream_t s = (hipStream_t)stream;
+  if (w_dtype == TPPX_DT_F32)
+    quantize_qint8_kernel<float><<<grid_for(nthreads, 256), 256, 0, s>>>(
+        (const float*)w, N, K, bk, bc, vnni, qbs, (int8_t*)q, (float*)scales);
+  else
+    quantize_qint8_kernel<uint16_t><<<grid_for(nthreads, 256), 256, 0, s>>>(
+        (const uint16_t*)w, N, K, bk, bc, vnni, qbs, (int8_t*)q, (float*)scales);
+  return check_hip(hipGetLastError(), "tppx_quantize_qint8");
+}
+
+extern "C" int tppx_dequantize_mxfp4(const void* qdata, const void* scales,
+                                     int64_t N, int64_t K, void* out_f32,
+                                     tppx_stream_t stream) {
+  TPPX_REQUIRE(qdata && scales && out_f32, TPPX_EINVAL, "tppx_dequantize_mxfp4: null pointer");
+  TPPX_REQUIRE(N > 0 && K > 0 && N % 32 == 0 && K % 64 == 0, TPPX_ESHAPE,
+               "tppx_dequantize_mxfp4: N=%ld must be a multiple of 32 and K=%ld of 64", (long)N, (long)K);
+  int64_t nbytes = N * K / 2;
+  dequantize_mxfp4_kernel<<<grid_for(nbytes, 256), 256, 0, (hipStream_t)stream>>>(
+      (const uint8_t*)qdata, (const uint8_t*)scales, nbytes, (float*)out_f32);
+  return check_hip(hipGetLastError(), "tppx_dequantize_mxfp4");
+}
+
+extern "C" int tppx_dequantize_qint8(const void* q, const void* scales,
+                                     int64_t N, int64_t K, int64_t qbs,
+                                     void* out_f32, tppx_stream_t stream) {
+  TPPX_REQUIRE(q && scales && out_f32, TPPX_EINVAL, "tppx_dequantize_qint8: null pointer");
+  TPPX_REQUIRE(N > 0 && K > 0 && N % 16 == 0 && qbs > 0 && qbs % 4 == 0 && K % qbs == 0,
+               TPPX_ESHAPE, "tppx_dequantize_qint8: bad shape N=%ld K=%ld qbs=%ld", (long)N, (long)K, (long)qbs);
+  int64_t ngroups = N * K / 4;
+  dequantize_qint8_kernel<<<grid_for(ngroups, 256), 256, 0, (hipStream_t)stream>>>(
+      (const int8_t*)q, (const float*)scales, ngroups, qbs, (float*)out_f32);
+  return check_hip(hipGetLastError(), "tppx_dequantize_qint8");
+}
+
+extern "C" int tppx_prepack_mxfp4(const void* qdata_ref, const void* scales_ref,
+                                  int64_t N, int64_t K, void* qdata_nat,
+                                  void* scales_nat, tppx_stream_t stream) {
+  TPPX_REQUIRE(qdata_ref && scales_ref && qdata_nat && scales_nat, TPPX_EINVAL,
+               "tppx_prepack_mxfp4: null pointer");
+  TPPX_REQUIRE(aligned16(qdata_nat), TPPX_EINVAL, "tppx_prepack_mxfp4: output not 16-byte aligned");
+  TPPX_REQUIRE(N > 0 && K > 0 && N % 32 == 0 && K % 128 == 0, TPPX_ESHAPE,
+               "tppx_prepack_mxfp4: N=%ld must be a multiple of 32 and K=%ld of 128", (long)N, (long)K);
+  int64_t nchunks = N * (K / 32);
+  prepack_mxfp4_kernel<<<grid_for(nchunks, 256), 256, 0, (hipStream_t)stream>>>(
+      (const uint8_t*)qdata_ref, (const uint8_t*)scales_ref, N, K,
+      (uint8_t*)qdata_nat, (uint8_t*)scales_nat);
+  return check_hip(hipGetLastError(), "tppx_prepack_mxfp4");
+}
+
+extern "C" int tppx_prepack_qint8(const void* q_ref, int64_t N, int64_t K,
+                                  int64_t qbs, void* q_nat,
+                                  tppx_stream_t stream) {
+  TPPX_REQUIRE(q_ref && q_nat, TPPX_EINVAL, "tppx_prepack_qint8: null pointer");
+  TPPX_REQUIRE(aligned16(q_nat) && aligned16(q_ref), TPPX_EINVAL, "tppx_prepack_qint8: pointer not 16-byte aligned");
+  TPPX_REQUIRE(N > 0 && K > 0 && N % 16 == 0 && qbs > 0 && qbs % 64 == 0 && K % qbs == 0,
+               TPPX_ESHAPE, "tppx_prepack_qint8: bad shape N=%ld K=%ld qbs=%ld", (long)N, (long)K, (long)qbs);
+  int64_t nchunks = N * (K / 16);
+  prepack_qint8_kernel<<<grid_for(nchunks, 256), 256, 0, (hipStream_t)stream>>>(
+      (const int8_t*)q_ref, N, K, qbs, (int8_t*)q_nat);
+  return check_hip(hipGetLastError(), "tppx_prepack_qint8");
+}
+
+extern "C" int tppx_quant_act_int8(const void* x, int64_t M, int64_t K,
+                                   int64_t qbs, void* xq, void* sa,
+                                   tppx_stream_t stream) {
+  TPPX_REQUIRE(x && xq && sa, TPPX_EINVAL, "tppx_quant_act_int8: null pointer");
+  TPPX_REQUIRE(aligned16(x) && aligned16(xq), TPPX_EINVAL, "tppx_quant_act_int8: pointer not 16-byte aligned");
+  TPPX_REQUIRE(M > 0 && K > 0 && qbs > 0 && qbs % 64 == 0 && K % qbs == 0, TPPX_ESHAPE,
+               "tppx_quant_act_int8: bad shape M=%ld K=%ld qbs=%ld", (long)M, (long)K, (long)qbs);
+  int64_t nthreads = M * (K / qbs) * 64;
+  quant_act_int8_kernel<<<grid_for(nthreads, 256), 256, 0, (hipStream_t)stream>>>(
+      (const uint16_t*)x, M, K, qbs, (int8_t*)xq, (float*)sa);
+  return check_hip(hipGetLastError(), "tppx_quant_act_int8");
+}

@@ -1,0 +1,106 @@
+"""ctypes binding of libtppx_hip.so (the C ABI declared in include/tppx.h).
+
+The HIP library is the only compute backend of this package: if it is missing
+the import of any op fails loudly; there is no CPU or eager fallback.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtppx_hip.so")
+
+OK, EINVAL, ESHAPE, EUNSUPPORTED, EHIP = 0, -1, -2, -3, -4
+POST_NONE, POST_SILU, POST_MUL, POST_ADD_SCALE, POST_ADD2_SCALE, POST_GELU, POST_RELU = range(7)
+DT_F32, DT_BF16 = 0, 1
+FLAG_NONE, FLAG_FORCE_SKINNY, FLAG_FORCE_TILED, FLAG_ACT_FP8 = 0, 1, 2, 4
+
+
+class TppxError(RuntimeError):
+    """Raised where the reference would TPP_ASSERT (printf + exit) or TORCH_CHECK."""
+
+    def __init__(self, code, msg):
+        super().__init__(f"tppx error {code}: {msg}")
+        self.code = code
+
+
+class Seg(ctypes.Structure):
+    _fields_ = [
+        ("qw", ctypes.c_void_p),
+        ("sw", ctypes.c_void_p),
+        ("bias", ctypes.c_void_p),
+        ("post_in", ctypes.c_void_p),
+        ("post_in2", ctypes.c_void_p),
+        ("y", ctypes.c_void_p),
+        ("N", ctypes.c_int64),
+        ("post_op", ctypes.c_int32),
+        ("post_scale", ctypes.c_float),
+    ]
+
+
+_vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+
+# name -> argtypes; every entry point declared in include/tppx.h
+SIGNATURES = {
+    "tppx_version": [],
+    "tppx_last_error": [],
+    "tppx_quantize_mxfp4": [_vp, _i32, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp],
+    "tppx_quantize_qint8": [_vp, _i32, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp],
+    "tppx_dequantize_mxfp4": [_vp, _vp, _i64, _i64, _vp, _vp],
+    "tppx_dequantize_qint8": [_vp, _vp, _i64, _i64, _i64, _vp, _vp],
+    "tppx_prepack_mxfp4": [_vp, _vp, _i64, _i64, _vp, _vp, _vp],
+    "tppx_prepack_qint8": [_vp, _i64, _i64, _i64, _vp, _vp],
+    "tppx_quant_act_int8": [_vp, _i64, _i64, _i64, _vp, _vp, _vp],
+    "tppx_linear_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _f32, _i32, _vp],
+    "tppx_linear_qint8": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _f32, _i32, _vp],
+    "tppx_multi_linear_mxfp4": [_vp, ctypes.POINTER(Seg), _i32, _i64, _i64, _i32, _vp],
+    "tppx_multi_linear_qint8": [_vp, _vp, _vp, ctypes.POINTER(Seg), _i32, _i64, _i64, _i64, _i32, _vp],
+    "tppx_swiglu_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
+}
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: the HIP extension has not been built "
+                "(run __graft_entry__.build() or `make -C tpp-pytorch-extension_amd/csrc`). "
+                "This package has no fallback path."
+            )
+        L = ctypes.CDLL(LIB_PATH)
+        for name, argtypes in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.argtypes = argtypes
+            fn.restype = ctypes.c_int
+        L.tppx_last_error.restype = ctypes.c_char_p
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != OK:
+        raise TppxError(rc, lib().tppx_last_error().decode())
+
+
+def ptr(t):
+    """Device pointer of a tensor, or NULL for None / an empty tensor."""
+    if t is None or t.numel() == 0:
+        return None
+    return t.data_ptr()
+
+
+def stream_of(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def require_gpu(t, what):
+    if not t.is_cuda:
+        raise TppxError(
+            EINVAL,
+            f"{what} must live on the GPU (got device {t.device}); the quantized-linear "
+            "path runs only as HIP kernels and has no CPU fallback",
+        )

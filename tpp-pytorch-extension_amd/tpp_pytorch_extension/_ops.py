@@ -1,0 +1,461 @@
+"""Operator layer: the reference's ``torch.ops.tpp_llm`` entry point plus the
+post-op variants the decoder layer uses, and the ``_C._qtype`` helper set.
+
+Every function here validates, allocates the output with torch and enqueues
+HIP kernels through the C ABI on the current stream.  Nothing computes on the
+host.
+"""
+import ctypes
+import os
+
+import torch
+
+from . import _lib
+from ._lib import (POST_NONE, POST_SILU, POST_MUL, POST_ADD_SCALE, POST_ADD2_SCALE, POST_GELU,
+                   POST_RELU, TppxError)
+from ._qtensor import QTensor, QSCHEME_MXFP, QSCHEME_AFFINE
+
+# QINT8_BLOCK_SIZE is read once at import like the reference's file-static
+# (src/csrc/qtypes.cpp:28).
+QINT8_BLOCK_SIZE = int(os.environ.get("QINT8_BLOCK_SIZE", "256"))
+
+
+# ----------------------------------------------------------------------------
+# quantize / remap helpers  (reference: pybind submodule _qtype, qtypes.cpp:1075-1093)
+# ----------------------------------------------------------------------------
+def _blocked_geometry(t):
+    """(N, K, bk, bc, vnni) of a blocked weight [N/bk, K/bc, bc/v, bk, v] or [N/bk, K/bc, bc, bk]."""
+    if t.dim() == 5:
+        n1, c1, c2, k2, c3 = t.shape
+        return n1 * k2, c1 * c2 * c3, k2, c2 * c3, c3
+    if t.dim() == 4:
+        n1, c1, c2, k2 = t.shape
+        return n1 * k2, c1 * c2, k2, c2, 1
+    if t.dim() == 2:
+        return t.shape[0], t.shape[1], 1, t.shape[1], 1
+    raise TppxError(_lib.ESHAPE, f"expected a 4-D or 5-D blocked weight, got shape {tuple(t.shape)}")
+
+
+def _float_weight_on_gpu(t):
+    if isinstance(t, QTensor):
+        raise TppxError(_lib.EINVAL, "weight is already quantized")
+    t = t.detach()
+    if t.dtype == torch.bfloat16:
+        dt = _lib.DT_BF16
+    elif t.dtype == torch.float32:
+        dt = _lib.DT_F32
+    else:
+        raise TppxError(_lib.EUNSUPPORTED, f"Unknown dtype for quantization: {t.dtype}")
+    if not t.is_cuda:
+        if not torch.cuda.is_available():
+            _lib.require_gpu(t, "weight to quantize")
+        t = t.cuda()
+    return t.contiguous(), dt
+
+
+def remap_and_quantize_mxfp4(t):
+    """Reference: remap_and_quantize_mxfp4 (src/csrc/qtypes.cpp:783-864).
+    Blocked bf16 5-D / fp32 4-D weight -> quint4x2 tensor [N/32, K/64, 32, 32, 2]."""
+    L = _lib.lib()
+    t, dt = _float_weight_on_gpu(t)
+    N, K, bk, bc, vnni = _blocked_geometry(t)
+    if t.dim() == 4 and bc % 2:
+        raise TppxError(_lib.ESHAPE, "Shape not compatible for VNNI2")
+    if bk < 32 and (32 % bk or (N // bk) % (32 // bk)):
+        raise TppxError(_lib.ESHAPE, "Shape not compatible for MXFP4")
+    if bc != 64:
+        raise TppxError(_lib.EUNSUPPORTED, f"MXFP4 weights are built for input-channel blocks of 64 (got {bc})")
+    if N % 32 or K % 64:
+        raise TppxError(_lib.ESHAPE, "Shape not compatible for MXFP4")
+    q = torch.empty((N // 32, K // 64, 32, 32), dtype=torch.uint8, device=t.device)
+    sc = torch.empty((N // 32, K // 64, 2, 32), dtype=torch.uint8, device=t.device)
+    _lib.check(L.tppx_quantize_mxfp4(t.data_ptr(), dt, N, K, bk, bc, vnni, q.data_ptr(), sc.data_ptr(),
+                                     _lib.stream_of(t)))
+    return QTensor(q, sc, (N // 32, K // 64, 32, 32, 2), torch.quint4x2, QSCHEME_MXFP, 32, 2, True, 2)
+
+
+def qint8_block_size_for(K):
+    """Block-size rule of remap_and_quantize_qint8 (qtypes.cpp:878-889)."""
+    if K % QINT8_BLOCK_SIZE == 0:
+        return QINT8_BLOCK_SIZE
+    q = 4096
+    while q >= 64:
+        if QINT8_BLOCK_SIZE > q and K % q == 0:
+            return q
+        q //= 2
+    raise TppxError(_lib.ESHAPE, f"no QINT8 block size divides K={K}")
+
+
+def remap_and_quantize_qint8(t):
+    """Reference: remap_and_quantize_qint8 (src/csrc/qtypes.cpp:866-932).
+    -> qint8 tensor [N/16, K/QBS, QBS/4, 16, 4] with fp32 scales [N/16, K/QBS, 1, 16]."""
+    L = _lib.lib()
+    t, dt = _float_weight_on_gpu(t)
+    N, K, bk, bc, vnni = _blocked_geometry(t)
+    if bk != 16:
+        raise TppxError(_lib.EUNSUPPORTED, f"QINT8 weights are built for output-channel blocks of 16 (got {bk})")
+    if 4 % vnni:
+        raise TppxError(_lib.ESHAPE, "Shape not compatible for VNNI4")
+    qbs = qint8_block_size_for(K)
+    q = torch.empty((N // 16, K // qbs, qbs // 4, 16, 4), dtype=torch.int8, device=t.device)
+    sc = torch.empty((N // 16, K // qbs, 1, 16), dtype=torch.float32, device=t.device)
+    _lib.check(L.tppx_quantize_qint8(t.data_ptr(), dt, N, K, bk, bc, vnni, qbs, q.data_ptr(),
+                                     sc.data_ptr(), _lib.stream_of(t)))
+    return QTensor(q, sc, tuple(q.shape), torch.qint8, QSCHEME_AFFINE, qbs, 2, True, 1)
+
+
+def quantize_mxfp4(t, block_size, axis, is_vnni):
+    """Reference: quantize_mxfp4 (qtypes.cpp:602-611).  Built for the layout
+    remap_and_quantize_mxfp4 feeds it: [N/32, K/64, 32, 32, 2], block 32, axis 2, VNNI."""
+    if axis < 0:
+        axis += t.dim()
+    if not (t.dim() == 5 and tuple(t.shape[2:]) == (32, 32, 2) and block_size == 32 and axis == 2 and is_vnni):
+        raise TppxError(
+            _lib.EUNSUPPORTED,
+            "quantize_mxfp4 is built for blocked weights [N/32, K/64, 32, 32, 2] with block_size=32, axis=2, is_vnni=True",
+        )
+    return remap_and_quantize_mxfp4(t)
+
+
+def quantize_mxfp(t, block_size, axis, is_vnni, dtype):
+    """Reference: quantize_mxfp (qtypes.cpp:592-600); only the E2M1 element type is built."""
+    if dtype != torch.quint4x2:
+        raise TppxError(_lib.EUNSUPPORTED, f"MX element type {dtype} is not built (only quint4x2 / E2M1)")
+    return quantize_mxfp4(t, block_size, axis, is_vnni)
+
+
+def quantize_int8sym(t, block_size, axis, is_vnni):
+    """Reference: quantize_int8sym (qtypes.cpp:613-624).  Two layouts are built:
+    the VNNI4 weight [N/16, K/QBS, QBS/4, 16, 4] (axis 2) and row-major
+    activations [..., K] quantized along the last axis (is_vnni False)."""
+    L = _lib.lib()
+    if axis < 0:
+        axis += t.dim()
+    if is_vnni:
+        if not (t.dim() == 5 and tuple(t.shape[3:]) == (16, 4) and axis == 2 and t.shape[2] * 4 == block_size):
+            raise TppxError(
+                _lib.EUNSUPPORTED,
+                "quantize_int8sym(is_vnni=True) is built for weights [N/16, K/QBS, QBS/4, 16, 4] with axis=2",
+            )
+        t, dt = _float_weight_on_gpu(t)
+        N, K = t.shape[0] * 16, t.shape[1] * block_size
+        q = torch.empty(tuple(t.shape), dtype=torch.int8, device=t.device)
+        sc = torch.empty((t.shape[0], t.shape[1], 1, 16), dtype=torch.float32, device=t.device)
+        # the input is already [N/16][K/QBS][QBS/4][16][4]: bk=16, bc=QBS, vnni=4
+        _lib.check(L.tppx_quantize_qint8(t.data_ptr(), dt, N, K, 16, block_size, 4, block_size,
+                                         q.data_ptr(), sc.data_ptr(), _lib.stream_of(t)))
+        return QTensor(q, sc, tuple(q.shape), torch.qint8, QSCHEME_AFFINE, block_size, 2, True, 1)
+    if axis != t.dim() - 1:
+        raise TppxError(_lib.EINVAL, f"Invalid axis {axis}")
+    _lib.require_gpu(t, "activation to quantize")
+    if t.dtype != torch.bfloat16:
+        raise TppxError(_lib.EUNSUPPORTED, f"activation quantization is built for bfloat16 (got {t.dtype})")
+    K = t.shape[-1]
+    if K % block_size:
+        raise TppxError(_lib.ESHAPE, "Axis size must be multiple of block_size")
+    t = t.contiguous()
+    M = t.numel() // K
+    xq = torch.empty(tuple(t.shape), dtype=torch.int8, device=t.device)
+    sa = torch.empty(tuple(t.shape[:-1]) + (K // block_size,), dtype=torch.float32, device=t.device)
+    _lib.check(L.tppx_quant_act_int8(t.data_ptr(), M, K, block_size, xq.data_ptr(), sa.data_ptr(),
+                                     _lib.stream_of(t)))
+    return QTensor(xq, sa, tuple(t.shape), torch.qint8, QSCHEME_AFFINE, block_size, axis, False, 1)
+
+
+def create_qtensor_int8sym(val, scales, block_size, axis, is_vnni):
+    """Reference: create_qtensor_int8sym (qtypes.cpp:654-668): wrap caller-supplied int8 values + fp32 scales."""
+    if val.dtype != torch.int8 or scales.dtype != torch.float32:
+        raise TppxError(_lib.EINVAL, "create_qtensor_int8sym expects int8 values and float32 scales")
+    if axis < 0:
+        axis += val.dim()
+    return QTensor(val.contiguous(), scales.contiguous(), tuple(val.shape), torch.qint8, QSCHEME_AFFINE,
+                   block_size, axis, is_vnni, 1)
+
+
+def _unbuilt(name):
+    def f(*a, **k):
+        raise TppxError(_lib.EUNSUPPORTED, f"{name} is outside the MXFP4 / QINT8 path built here")
+    f.__name__ = name
+    return f
+
+
+quantize_int4sym = _unbuilt("quantize_int4sym")
+create_qtensor_int2sym = _unbuilt("create_qtensor_int2sym")
+remap_and_quantize_qint2_intlv = _unbuilt("remap_and_quantize_qint2_intlv")
+
+
+def _as_q(t):
+    if not isinstance(t, QTensor):
+        raise TppxError(_lib.EINVAL, "expected a per-block quantized tensor")
+    return t
+
+
+def q_per_block_scales(t):
+    return _as_q(t).scales
+
+
+def q_per_block_pack_size(t):
+    return _as_q(t).pack_size
+
+
+def q_per_block_block_size(t):
+    return _as_q(t).block_size
+
+
+def q_per_block_axis(t):
+    return _as_q(t).axis
+
+
+def q_per_block_qval(t):
+    """Packed storage in the reference layout: int8 values for qint8, the
+    packed uint8 bytes [N/32, K/64, 32, 32] for quint4x2."""
+    return _as_q(t).qdata
+
+
+def fix_vnni(t):
+    """Reference: fix_vnni (qtypes.cpp:740-781): pure re-layout of an unquantized blocked weight."""
+    dims = t.dim()
+    if dims < 4:
+        raise TppxError(_lib.ESHAPE, f"Invalid shape, dims = {dims}")
+    K1, C1, C2, K2 = t.shape[:4]
+    C3 = t.shape[4] if dims == 5 else 1
+    if t.dtype == torch.bfloat16:
+        if C3 == 2:
+            return t
+        if C3 == 4:
+            return (t.view(K1, C1, C2, K2, 2, 2).permute(0, 1, 2, 4, 3, 5).contiguous()
+                    .view(K1, C1, C2 * 2, K2, 2))
+        if C3 == 1:
+            if C2 % 2:
+                raise TppxError(_lib.ESHAPE, f"Shape incompatible for VNNI2 layout, C2 = {C2}")
+            return t.view(K1, C1, C2 // 2, 2, K2).permute(0, 1, 2, 4, 3).contiguous()
+        raise TppxError(_lib.ESHAPE, "Shape incompatible for VNNI2 layout")
+    if t.dtype == torch.float32:
+        if C3 == 1 and dims == 4:
+            return t
+        if C3 == 1:
+            return t.view(K1, C1, C2, K2)
+        return t.permute(0, 1, 2, 4, 3).contiguous().view(K1, C1, C2 * C3, K2)
+    raise TppxError(_lib.EUNSUPPORTED, "Unknown dtype for FIX_VNNI layout")
+
+
+# ----------------------------------------------------------------------------
+# linears
+# ----------------------------------------------------------------------------
+def _prep_input(input, weight):
+    if not isinstance(weight, QTensor):
+        raise TppxError(
+            _lib.EUNSUPPORTED,
+            "only MXFP4 / QINT8 quantized weights are built on this path "
+            "(quantize the weight with remap_and_quantize_mxfp4 / remap_and_quantize_qint8)",
+        )
+    if not weight.is_weight():
+        raise TppxError(_lib.EUNSUPPORTED, f"Unsupported qscheme / layout for a linear weight: {weight!r}")
+    _lib.require_gpu(weight.qdata, "weight")
+    if isinstance(input, QTensor):
+        raise TppxError(_lib.EUNSUPPORTED, "pre-quantized activations are not built; pass bfloat16")
+    _lib.require_gpu(input, "input")
+    if input.dtype != torch.bfloat16:
+        raise TppxError(_lib.EUNSUPPORTED,
+                        f"quantized weights take bfloat16 activations (got {input.dtype})")
+    N, K = weight.weight_nk()
+    if input.shape[-1] != K:
+        raise TppxError(_lib.ESHAPE, f"input has {input.shape[-1]} features, weight expects {K}")
+    x = input.contiguous()
+    M = x.numel() // K
+    return x, M, N, K
+
+
+def _prep_bias(bias, N, dev):
+    if bias is None or bias.numel() == 0:
+        return None
+    if bias.numel() != N:
+        raise TppxError(_lib.ESHAPE, f"bias has {bias.numel()} elements, expected {N}")
+    if bias.dtype != torch.bfloat16 or bias.device != dev:
+        bias = bias.to(device=dev, dtype=torch.bfloat16)
+    return bias.contiguous()
+
+
+def _prep_post(t, M, N, name, dev):
+    if t is None:
+        return None
+    if t.numel() != M * N or t.shape[-1] != N:
+        raise TppxError(_lib.ESHAPE, f"{name} must have the output's shape [..., {N}] with {M} rows, got {tuple(t.shape)}")
+    if t.dtype != torch.bfloat16 or t.device != dev:
+        raise TppxError(_lib.EINVAL, f"{name} must be a bfloat16 tensor on {dev}")
+    return t.contiguous()
+
+
+def _qint8_scratch(x, M, K, qbs):
+    xq = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    sa = torch.empty((M, K // qbs), dtype=torch.float32, device=x.device)
+    return xq, sa
+
+
+def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0, flags=0):
+    """One quantized GEMM with a fused post-op
+    (call_gemm_with_post_op, src/csrc/fused_gemm.h:1510-1597)."""
+    L = _lib.lib()
+    x, M, N, K = _prep_input(input, weight)
+    out_shape = tuple(input.shape[:-1]) + (N,)
+    y = torch.empty(out_shape, dtype=torch.bfloat16, device=x.device)
+    if M == 0:
+        return y
+    bias = _prep_bias(bias, N, x.device)
+    post_in = _prep_post(post_in, M, N, "post-op input", x.device)
+    post_in2 = _prep_post(post_in2, M, N, "second post-op input", x.device)
+    qn, sn = weight.native()
+    st = _lib.stream_of(x)
+    if weight._qscheme == QSCHEME_MXFP:
+        _lib.check(L.tppx_linear_mxfp4(x.data_ptr(), qn.data_ptr(), sn.data_ptr(), _lib.ptr(bias),
+                                       _lib.ptr(post_in), _lib.ptr(post_in2), y.data_ptr(), M, N, K,
+                                       post, post_scale, flags, st))
+    else:
+        qbs = weight.block_size
+        xq, sa = _qint8_scratch(x, M, K, qbs)
+        _lib.check(L.tppx_linear_qint8(x.data_ptr(), xq.data_ptr(), sa.data_ptr(), qn.data_ptr(),
+                                       sn.data_ptr(), _lib.ptr(bias), _lib.ptr(post_in),
+                                       _lib.ptr(post_in2), y.data_ptr(), M, N, K, qbs, post,
+                                       post_scale, flags, st))
+    return y
+
+
+def fc_plain(input, weight, bias, parallel_dim=-1, split_sizes=()):
+    """torch.ops.tpp_llm.fc_plain (fc_plain_wrap, src/csrc/llm/fused_llm_infer.cpp:1514-1566)."""
+    if parallel_dim not in (-1, None):
+        raise TppxError(_lib.EUNSUPPORTED,
+                        "tensor-parallel fc_plain (parallel_dim 0/1) needs a process group; this build runs one GPU")
+    return linear(input, weight, bias, POST_NONE)
+
+
+def fc_add(input, weight, bias, residual, scale=1.0):
+    """GEMM + AddScalePostOp(residual, scale) (fused_llm_infer.cpp:1261,1273)."""
+    return linear(input, weight, bias, POST_ADD_SCALE, residual, None, scale)
+
+
+def fc_add2(input, weight, bias, residual1, residual2, scale=1.0):
+    """GEMM + Add2ScalePostOp (src/csrc/fused_gemm.h:1460)."""
+    return linear(input, weight, bias, POST_ADD2_SCALE, residual1, residual2, scale)
+
+
+def fc_silu(input, weight, bias):
+    """GEMM + SiluPostOp (fused_llm_infer.cpp:1271)."""
+    return linear(input, weight, bias, POST_SILU)
+
+
+def fc_gelu(input, weight, bias):
+    return linear(input, weight, bias, POST_GELU)
+
+
+def fc_relu(input, weight, bias):
+    return linear(input, weight, bias, POST_RELU)
+
+
+def fc_mul(input, weight, bias, mul_in):
+    """GEMM + MulPostOp(mul_in) (fused_llm_infer.cpp:1272)."""
+    return linear(input, weight, bias, POST_MUL, mul_in)
+
+
+def qkv_gemm(input, weights, biases):
+    """fused_qkv_gemm (src/csrc/llm/fused_llm_infer.cpp:423-505): several GEMMs
+    over one activation in one launch; a 4th GEMM gets GELU (GPT-J fc_in)."""
+    L = _lib.lib()
+    weights = list(weights)
+    biases = list(biases) if biases is not None else []
+    n = len(weights)
+    if n < 1 or n > 4:
+        raise TppxError(_lib.EINVAL, f"qkv_gemm takes 1..4 weights, got {n}")
+    while len(biases) < n:
+        biases.append(None)
+    x, M, N0, K = _prep_input(input, weights[0])
+    scheme = weights[0]._qscheme
+    segs = (_lib.Seg * n)()
+    outs, keep = [], []
+    for i, w in enumerate(weights):
+        xi, Mi, Ni, Ki = _prep_input(input, w)
+        if w._qscheme != scheme or Ki != K or w.block_size != weights[0].block_size:
+            raise TppxError(_lib.ESHAPE, "Fused QKV weight block mismatch")
+        y = torch.empty(tuple(input.shape[:-1]) + (Ni,), dtype=torch.bfloat16, device=x.device)
+        b = _prep_bias(biases[i], Ni, x.device)
+        qn, sn = w.native()
+        keep.append((b, qn, sn))
+        segs[i].qw = qn.data_ptr()
+        segs[i].sw = sn.data_ptr()
+        segs[i].bias = _lib.ptr(b)
+        segs[i].post_in = None
+        segs[i].post_in2 = None
+        segs[i].y = y.data_ptr()
+        segs[i].N = Ni
+        segs[i].post_op = POST_GELU if (n == 4 and i == 3) else POST_NONE
+        segs[i].post_scale = 1.0
+        outs.append(y)
+    if M == 0:
+        return outs
+    st = _lib.stream_of(x)
+    if scheme == QSCHEME_MXFP:
+        _lib.check(L.tppx_multi_linear_mxfp4(x.data_ptr(), segs, n, M, K, 0, st))
+    else:
+        qbs = weights[0].block_size
+        xq, sa = _qint8_scratch(x, M, K, qbs)
+        _lib.check(L.tppx_multi_linear_qint8(x.data_ptr(), xq.data_ptr(), sa.data_ptr(), segs, n, M, K,
+                                             qbs, 0, st))
+    return outs
+
+
+def swiglu_gate_up(input, w_gate, w_up, b_gate=None, b_up=None):
+    """silu(x Wg^T) * (x Wu^T) in one launch with the reference's bf16 rounding
+    points (fused_llm_infer.cpp:1271-1272)."""
+    L = _lib.lib()
+    x, M, N, K = _prep_input(input, w_gate)
+    x2, M2, N2, K2 = _prep_input(input, w_up)
+    if N2 != N or w_gate._qscheme != w_up._qscheme:
+        raise TppxError(_lib.ESHAPE, "gate and up projections must have the same shape and format")
+    if w_gate._qscheme != QSCHEME_MXFP:
+        g = fc_silu(input, w_gate, b_gate)
+        return fc_mul(input, w_up, b_up, g)
+    y = torch.empty(tuple(input.shape[:-1]) + (N,), dtype=torch.bfloat16, device=x.device)
+    if M == 0:
+        return y
+    bg = _prep_bias(b_gate, N, x.device)
+    bu = _prep_bias(b_up, N, x.device)
+    qg, sg = w_gate.native()
+    qu, su = w_up.native()
+    _lib.check(L.tppx_swiglu_mxfp4(x.data_ptr(), qg.data_ptr(), sg.data_ptr(), _lib.ptr(bg), qu.data_ptr(),
+                                   su.data_ptr(), _lib.ptr(bu), y.data_ptr(), M, N, K, 0, _lib.stream_of(x)))
+    return y
+
+
+def swiglu_mlp(input, w_gate, w_up, w_down, residual, scale=1.0):
+    """The Llama MLP block (fused_llm_infer.cpp:1271-1273):
+    down( silu(gate(x)) * up(x) ) + residual*scale."""
+    inter = swiglu_gate_up(input, w_gate, w_up)
+    return fc_add(inter, w_down, None, residual, scale)
+
+
+# ----------------------------------------------------------------------------
+# torch.library registration (namespace tpp_llm, like TORCH_LIBRARY(tpp_llm, m),
+# fused_llm_infer.cpp:1588-1611)
+# ----------------------------------------------------------------------------
+_libdef = torch.library.Library("tpp_llm", "DEF")
+_libdef.define("fc_plain(Tensor input, Tensor weight, Tensor bias, int parallel_dim, int[] split_sizes) -> Tensor")
+_libdef.define("fc_add(Tensor input, Tensor weight, Tensor bias, Tensor residual, float scale=1.0) -> Tensor")
+_libdef.define("fc_silu(Tensor input, Tensor weight, Tensor bias) -> Tensor")
+_libdef.define("fc_mul(Tensor input, Tensor weight, Tensor bias, Tensor mul_in) -> Tensor")
+_libdef.define("qkv_gemm(Tensor input, Tensor[] weights, Tensor[] biases) -> Tensor[]")
+_libdef.define("swiglu_mlp(Tensor input, Tensor w_gate, Tensor w_up, Tensor w_down, Tensor residual, float scale=1.0) -> Tensor")
+
+_IMPLS = {
+    "fc_plain": fc_plain,
+    "fc_add": fc_add,
+    "fc_silu": fc_silu,
+    "fc_mul": fc_mul,
+    "qkv_gemm": qkv_gemm,
+    "swiglu_mlp": swiglu_mlp,
+}
+for _name, _fn in _IMPLS.items():
+    # plain (non-subclass) tensors land here: the weight is then not quantized,
+    # which this build rejects with a clear error inside the implementation
+    _libdef.impl(_name, _fn, "CompositeExplicitAutograd")
+
+# QTensor.__torch_dispatch__ routes the ops here
+DISPATCH = {getattr(torch.ops.tpp_llm, n).default: f for n, f in _IMPLS.items()}

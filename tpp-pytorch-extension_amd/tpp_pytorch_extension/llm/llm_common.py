@@ -1,0 +1,115 @@
+"""LLM-side module API of the quantized linear.
+
+Reference: ``src/tpp_pytorch_extension/llm/llm_common.py`` -- ``fc_plain``
+(:379), ``BlockedLinear`` (:383-434) and ``FixLinear`` (:437-515).  The
+generation wrapper, KV cache and tensor-parallel sharding of that file are
+outside the path built here.
+"""
+import torch
+
+from ..utils.blocked_layout import BlockedParameter, BlockedModule
+from ..utils.xsmm import get_vnni_blocking
+from .._C import _fused_llm_infer as fused_llm_cpp  # noqa: F401
+from .._C import _qtype as qtype
+
+USE_LOW_PREC_PARAMS = True
+global_layer_dtype = torch.float32
+
+
+def block(model):
+    for m in model.modules():
+        if hasattr(m, "maybe_block_params"):
+            m.maybe_block_params()
+
+
+def fc_plain(input, weight, bias=torch.Tensor(), parallel_dim=-1, split_sizes=[]):
+    return torch.ops.tpp_llm.fc_plain(input, weight, bias, parallel_dim, split_sizes)
+
+
+class BlockedLinear(BlockedModule, torch.nn.Linear):
+    def maybe_block_params(self):
+        if hasattr(self.weight, "block"):
+            self.weight.block()
+        if self.bias is not None and hasattr(self.bias, "block"):
+            self.bias.block()
+
+    def parallelize(self, dim, rank, size, block_size=1):
+        if size <= 1:
+            return
+        raise NotImplementedError("tensor-parallel sharding is not part of the single-GPU path")
+
+    def _io_dtype(self):
+        return torch.bfloat16 if self.weight.is_quantized else self.weight.dtype
+
+    def forward(self, input):
+        self.maybe_block_params()
+        bias = self.bias if self.bias is not None else torch.Tensor().to(self._io_dtype())
+        input = input.to(self._io_dtype())
+        parallel_dim = self.parallel_dim if self.model_parallel else -1
+        split_sizes = self.split_sizes if hasattr(self, "split_sizes") else []
+        return fc_plain(input, self.weight, bias, parallel_dim, split_sizes)
+
+    # post-op variants used by the decoder layer
+    # (src/csrc/llm/fused_llm_infer.cpp:1261-1273)
+    def forward_add(self, input, residual, scale=1.0):
+        bias = self.bias if self.bias is not None else torch.Tensor()
+        return torch.ops.tpp_llm.fc_add(input.to(self._io_dtype()), self.weight, bias, residual, scale)
+
+    def forward_silu(self, input):
+        bias = self.bias if self.bias is not None else torch.Tensor()
+        return torch.ops.tpp_llm.fc_silu(input.to(self._io_dtype()), self.weight, bias)
+
+    def forward_mul(self, input, mul_in):
+        bias = self.bias if self.bias is not None else torch.Tensor()
+        return torch.ops.tpp_llm.fc_mul(input.to(self._io_dtype()), self.weight, bias, mul_in)
+
+
+def _resolve_weight_dtype(weight_dtype, layer_dtype):
+    if weight_dtype is None:
+        return layer_dtype
+    if isinstance(weight_dtype, str):
+        if weight_dtype in ("mxfp4", "qint8", "qint2"):
+            return weight_dtype
+        try:
+            return getattr(torch, weight_dtype)
+        except AttributeError:
+            raise ValueError(f"Unknown weight_dtype {weight_dtype}")
+    if not isinstance(weight_dtype, torch.dtype):
+        raise ValueError(f"weight_dtype must be either str or torch.dtype but is {type(weight_dtype)}")
+    return weight_dtype
+
+
+def FixLinear(self, bk=None, bc=None, layer_dtype=global_layer_dtype, parallel_dim=None, block_size=1,
+              weight_dtype=None):
+    """Turn an nn.Linear into a BlockedLinear: block the weight ([bk, bc] tiles,
+    VNNI-packed for low precision) and quantize it when weight_dtype names a
+    quantized format."""
+    if not isinstance(self, torch.nn.Linear) or isinstance(self, BlockedLinear):
+        return
+    self.__class__ = BlockedLinear
+    self.model_parallel = False
+    if parallel_dim is not None:
+        self.parallelize(parallel_dim, 0, 1, block_size=block_size)
+    weight_dtype = _resolve_weight_dtype(weight_dtype, layer_dtype)
+
+    self.weight = BlockedParameter(self.weight.data)
+    if layer_dtype != torch.float32 and USE_LOW_PREC_PARAMS:
+        v = get_vnni_blocking(layer_dtype)
+        self.weight.set_blocking_param(([bk, [bc // v, v]], [0, 2, 3, 1, 4], layer_dtype))
+    else:
+        self.weight.set_blocking_param(([bk, bc], [0, 2, 3, 1]))
+    if self.bias is not None:
+        self.bias = BlockedParameter(self.bias.data)
+        self.bias.set_blocking_param((None, None, layer_dtype))
+    block(self)
+    with torch.no_grad():
+        if weight_dtype == "mxfp4":
+            self.weight = torch.nn.Parameter(qtype.remap_and_quantize_mxfp4(self.weight), requires_grad=False)
+        elif weight_dtype == "qint8":
+            self.weight = torch.nn.Parameter(qtype.remap_and_quantize_qint8(self.weight), requires_grad=False)
+        elif weight_dtype == "qint2":
+            self.weight = torch.nn.Parameter(qtype.remap_and_quantize_qint2_intlv(self.weight), requires_grad=False)
+        else:
+            self.weight = torch.nn.Parameter(self.weight.data.to(weight_dtype), requires_grad=False)
+        if self.bias is not None and isinstance(weight_dtype, str):
+            self.bias = torch.nn.Parameter(self.bias.data.to(torch.bfloat16), requires_grad=False)
