@@ -1,0 +1,312 @@
+#!/usr/bin/env python3
+"""Benchmark of the weight-quantized linear path on one MI355X.
+
+Default workload (the configuration the metric is quoted on): QINT8 W8A8
+`fc_add` at the Llama-7B MLP shapes -- up-projection 4096 -> 11008 and
+down-projection 11008 -> 4096 -- for M in {1, 8, 32, 64}; one "step" is one
+pass over those 8 fused linears.  Inputs are resident in HBM before the timed
+region; weights cycle through a pool larger than the 256 MB Infinity Cache so
+that every launch streams its weight from HBM.
+
+Prints ONE JSON line: whole-job HBM throughput (algorithmic bytes / wall time),
+the roofline of the dominant kernel (timed with events on the launch stream)
+and the CPU restatement of the reference path timed on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "tpp-pytorch-extension_amd"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
+PEAKS_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "fp4": 10100.0}
+
+
+def algorithmic_bytes(fmt, M, N, K, qbs=256, bias=False, post_in=True):
+    """weights + scales + X + bias + post-op input + Y (bf16 activations)."""
+    if fmt == "qint8":
+        w = N * K + 4 * N * (K // qbs)
+    else:
+        w = N * K // 2 + N * K // 32
+    return w + 2 * M * K + (2 * N if bias else 0) + (2 * M * N if post_in else 0) + 2 * M * N
+
+
+def make_inputs(torch, shapes, Ms, seed):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    W = {name: (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16) for name, (N, K) in shapes.items()}
+    X = {(name, M): torch.randn((M, K), generator=g).to(torch.bfloat16)
+         for name, (N, K) in shapes.items() for M in Ms}
+    R = {(name, M): torch.randn((M, N), generator=g).to(torch.bfloat16)
+         for name, (N, K) in shapes.items() for M in Ms}
+    return W, X, R
+
+
+def block_bf16(W):
+    N, K = W.shape
+    return W.view(N // 16, 16, K // 64, 32, 2).permute(0, 2, 3, 1, 4).contiguous()
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--fmt", default="qint8", choices=["qint8", "mxfp4"])
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--pool", type=int, default=2, help="number of distinct weight sets cycled through")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus must be 1 (every box has one GPU and the "
+              "path has no collectives)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import tpp_pytorch_extension  # noqa: F401
+    from tpp_pytorch_extension import _ops
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    fmt = args.fmt
+    shapes = {"up": (11008, 4096), "down": (4096, 11008)}
+    Ms = [1, 8, 32, 64]
+    qbs = 256
+    W, X, R = make_inputs(torch, shapes, Ms, 1236)
+    quant = _ops.remap_and_quantize_qint8 if fmt == "qint8" else _ops.remap_and_quantize_mxfp4
+
+    # pool of weight sets: every (set, shape, M) gets its own copy so a step
+    # touches len(Ms) * (45+45) MB = 360 MB of distinct weight bytes (QINT8)
+    pool = []
+    for s in range(max(1, args.pool)):
+        ws = {}
+        for name in shapes:
+            base = quant(block_bf16(W[name]).to(dev))
+            base.native()
+            for M in Ms:
+                q = base._clone_with(base.qdata, base.scales)
+                q._native = tuple(t.clone() for t in base._native)
+                ws[(name, M)] = q
+        pool.append(ws)
+    Xd = {k: v.to(dev) for k, v in X.items()}
+    Rd = {k: v.to(dev) for k, v in R.items()}
+    empty = torch.empty(0, dtype=torch.bfloat16, device=dev)
+
+    def step(ws):
+        outs = []
+        for M in Ms:
+            for name in ("up", "down"):
+                outs.append(torch.ops.tpp_llm.fc_add(Xd[(name, M)], ws[(name, M)], empty, Rd[(name, M)], 1.0))
+        return outs
+
+    bytes_per_step = sum(algorithmic_bytes(fmt, M, N, K, qbs) for (N, K) in shapes.values() for M in Ms)
+    flops_per_step = sum(2 * M * N * K for (N, K) in shapes.values() for M in Ms)
+
+    graphs = None
+    if not args.no_graph:
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for ws in pool:
+                    step(ws)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graphs = []
+            for ws in pool:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    keep = step(ws)
+                graphs.append((g, keep))
+        except Exception as e:  # graph capture unavailable: time eager launches
+            print(f"bench.py: graph capture failed ({e!r}); timing eager launches", file=sys.stderr)
+            graphs = None
+
+    def run_step(i):
+        if graphs is not None:
+            graphs[i % len(graphs)][0].replay()
+        else:
+            step(pool[i % len(pool)])
+
+    for i in range(args.warmup):
+        run_step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        run_step(i)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value_tbs = bytes_per_step / (ms_per_step * 1e-3) / 1e12
+
+    # ---- roofline leg: the GEMM kernel alone, events on the launch stream ----
+    roof = roofline_leg(torch, _ops, fmt, pool, Xd, Rd, Ms, shapes, qbs, args)
+
+    # ---- CPU baseline: the oracle (port of the reference recipe) -------------
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(fmt, W, X, R, Ms, shapes, qbs, bytes_per_step)
+
+    out = {
+        "metric": "quant-GEMM HBM TB/s (decode)",
+        "value": round(value_tbs, 4),
+        "unit": "TB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8" if fmt == "qint8" else "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": ("cfg2: QINT8 W8A8 (QBS=256) fc_add" if fmt == "qint8" else "MXFP4 fc_add")
+            + ", Llama-7B MLP up 4096->11008 + down 11008->4096, M in {1,8,32,64}; one step = these 8 fused linears",
+            "launch": "hipGraph replay of one step" if graphs is not None else "eager launches",
+            "weight_pool_MB": round(len(pool) * len(Ms) * sum(algorithmic_bytes(fmt, 0, N, K, qbs, post_in=False)
+                                                              for (N, K) in shapes.values()) / 1e6, 1),
+            "bytes_per_step": bytes_per_step,
+            "tflops": round(flops_per_step / (ms_per_step * 1e-3) / 1e12, 2),
+        },
+        "roofline": roof,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+def roofline_leg(torch, _ops, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
+    """Launch only the dominant GEMM kernel (activations pre-quantized for
+    QINT8) for every (shape, M) of the step, many times, between two events on
+    the launch stream; achieved = algorithmic bytes / mean launch duration."""
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    launches = []
+    keep = []
+    for ws in pool:
+        for M in Ms:
+            for name, (N, K) in shapes.items():
+                w = ws[(name, M)]
+                qn, sn = w.native()
+                x = Xd[(name, M)]
+                r = Rd[(name, M)]
+                y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+                if fmt == "qint8":
+                    xq = torch.empty((M, K), dtype=torch.int8, device=dev)
+                    sa = torch.empty((M, K // qbs), dtype=torch.float32, device=dev)
+                    _lib.check(L.tppx_quant_act_int8(x.data_ptr(), M, K, qbs, xq.data_ptr(), sa.data_ptr(),
+                                                     _lib.stream_of(x)))
+                    keep += [xq, sa, y]
+                    launches.append(("q", (None, xq.data_ptr(), sa.data_ptr(), qn.data_ptr(), sn.data_ptr(), None,
+                                           r.data_ptr(), None, y.data_ptr(), M, N, K, qbs, 3, 1.0, 0), M, N, K))
+                else:
+                    keep += [y]
+                    launches.append(("m", (x.data_ptr(), qn.data_ptr(), sn.data_ptr(), None, r.data_ptr(), None,
+                                           y.data_ptr(), M, N, K, 3, 1.0, 0), M, N, K))
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def fire():
+        for kind, a, M, N, K in launches:
+            if kind == "q":
+                _lib.check(L.tppx_linear_qint8(*a, stream))
+            else:
+                _lib.check(L.tppx_linear_mxfp4(*a, stream))
+
+    g = None
+    if not args.no_graph:
+        try:
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                stream = torch.cuda.current_stream().cuda_stream
+                fire()
+            stream = torch.cuda.current_stream().cuda_stream
+        except Exception:
+            g = None
+            stream = torch.cuda.current_stream().cuda_stream
+    reps = max(4, args.steps // max(1, len(pool)))
+    for _ in range(3):
+        g.replay() if g is not None else fire()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        g.replay() if g is not None else fire()
+    e1.record()
+    torch.cuda.synchronize()
+    total_ms = e0.elapsed_time(e1)
+    n_launch = reps * len(launches)
+    total_bytes = reps * sum(algorithmic_bytes(fmt, M, N, K, qbs) for _, _, M, N, K in launches)
+    avg_us = total_ms * 1e3 / n_launch
+    achieved = total_bytes / (total_ms * 1e-3) / 1e9
+    return {
+        "bound": "hbm",
+        "kernel": "skinny_qint8_kernel" if fmt == "qint8" else "skinny_mxfp4_kernel",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "avg_launch_us": round(avg_us, 3),
+        "bytes_per_launch": total_bytes // n_launch,
+        "launches_timed": n_launch,
+    }
+
+
+def cpu_baseline(fmt, W, X, R, Ms, shapes, qbs, bytes_per_step):
+    """The oracle's restatement of the reference CPU path on the host cores,
+    one step's worth of linears on the same seeded inputs, repeated while the
+    total stays within ~10 s."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numpy as np
+    import torch
+    import oracle as O
+
+    def bits(t):
+        return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+    cores = len(os.sched_getaffinity(0))
+    cores = min(cores, O.num_threads()) if O.num_threads() > 0 else cores
+    O.set_num_threads(cores)
+    qw = {}
+    for name in shapes:
+        Wf = W[name].float().numpy()
+        qw[name] = O.remap_quantize_qint8(Wf)[:2] if fmt == "qint8" else O.remap_quantize_mxfp4(Wf)
+    lin = O.linear_qint8 if fmt == "qint8" else O.linear_mxfp4
+    xs = {k: bits(v) for k, v in X.items()}
+    rs = {k: bits(v) for k, v in R.items()}
+
+    def one_step():
+        for M in Ms:
+            for name in shapes:
+                q, s = qw[name]
+                lin(xs[(name, M)], q, s, None, O.POST_ADD_SCALE, rs[(name, M)], None, 1.0, O.MODE_FAITHFUL)
+
+    one_step()  # warm-up
+    n, t0 = 0, time.perf_counter()
+    while True:
+        one_step()
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt > 10.0 or n >= 10:
+            break
+    sec = dt / n
+    return {
+        "value": round(bytes_per_step / sec / 1e12, 5),
+        "unit": "TB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{n} passes over the same 8-linear step (C/OpenMP restatement of the reference recipe, "
+                  f"faithful bf16 re-rounding; not the libxsmm JIT), {round(sec * 1e3, 1)} ms per step",
+    }
+
+
+if __name__ == "__main__":
+    main()

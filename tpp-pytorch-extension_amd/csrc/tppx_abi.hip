@@ -108,11 +108,13 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
 
 static int run_qint8(const char* who, const void* x, void* xq, void* sa, const tppx_seg* segs,
                      int n_segs, int64_t M, int64_t K, int64_t qbs, int flags, hipStream_t stream) {
-  int rc = check_common(who, x, M, K, n_segs, flags);
+  // x == NULL: xq / sa already hold quantized activations (the reference's
+  // pre-quantized input case, src/csrc/fused_gemm.h:1244-1246)
+  int rc = check_common(who, x ? x : xq, M, K, n_segs, flags);
   if (rc)
     return rc;
   TPPX_REQUIRE(segs, TPPX_EINVAL, "%s: null segment table", who);
-  TPPX_REQUIRE(xq && sa, TPPX_EINVAL, "%s: null activation-quantization scratch", who);
+  TPPX_REQUIRE(xq && sa, TPPX_EINVAL, "%s: null activation-quantization buffers", who);
   TPPX_REQUIRE(aligned16(xq), TPPX_EINVAL, "%s: scratch pointer not 16-byte aligned", who);
   TPPX_REQUIRE(K > 0 && K % 64 == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of 64", who, (long)K);
   TPPX_REQUIRE(qbs > 0 && qbs % 64 == 0 && K % qbs == 0, TPPX_ESHAPE, "%s: block size mismatch (qbs=%ld, K=%ld)", who, (long)qbs, (long)K);
@@ -136,9 +138,11 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
   p.K = (int)K;
   p.qbs = (int)qbs;
   p.kunits = (int)(K / qbs);
-  rc = tppx_quant_act_int8(x, M, K, qbs, xq, sa, stream);
-  if (rc)
-    return rc;
+  if (x) {
+    rc = tppx_quant_act_int8(x, M, K, qbs, xq, sa, stream);
+    if (rc)
+      return rc;
+  }
   SkinnyPlan pl = plan_skinny(M, tiles, p.kunits, all_even, false);
   p.units_per_wave = pl.units_per_wave;
   return check_hip(launch_skinny_qint8(p, pl, stream), who);
