@@ -204,7 +204,9 @@ def roofline_leg(torch, _ops, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
                     _lib.check(L.tppx_quant_act_int8(x.data_ptr(), M, K, qbs, xq.data_ptr(), sa.data_ptr(),
                                                      _lib.stream_of(x)))
                     keep += [xq, sa, y]
-                    launches.append(("q", (None, xq.data_ptr(), sa.data_ptr(), qn.data_ptr(), sn.data_ptr(), None,
+                    # M <= 16: the kernel quantises the bf16 activations itself (single launch)
+                    xin = x.data_ptr() if M <= 16 else None
+                    launches.append(("q", (xin, xq.data_ptr(), sa.data_ptr(), qn.data_ptr(), sn.data_ptr(), None,
                                            r.data_ptr(), None, y.data_ptr(), M, N, K, qbs, 3, 1.0, 0), M, N, K))
                 else:
                     keep += [y]
@@ -213,12 +215,14 @@ def roofline_leg(torch, _ops, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
     torch.cuda.synchronize()
     stream = torch.cuda.current_stream().cuda_stream
 
+    ws = _lib.workspace(torch.empty(1, device=dev))
+
     def fire():
         for kind, a, M, N, K in launches:
             if kind == "q":
-                _lib.check(L.tppx_linear_qint8(*a, stream))
+                _lib.check(L.tppx_linear_qint8(*a, ws.data_ptr(), ws.numel(), stream))
             else:
-                _lib.check(L.tppx_linear_mxfp4(*a, stream))
+                _lib.check(L.tppx_linear_mxfp4(*a, ws.data_ptr(), ws.numel(), stream))
 
     g = None
     if not args.no_graph:
@@ -248,7 +252,7 @@ def roofline_leg(torch, _ops, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
     achieved = total_bytes / (total_ms * 1e-3) / 1e9
     return {
         "bound": "hbm",
-        "kernel": "skinny_qint8_kernel" if fmt == "qint8" else "skinny_mxfp4_kernel",
+        "kernel": "decode_qint8_kernel" if fmt == "qint8" else "decode_mxfp4_kernel",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",

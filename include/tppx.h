@@ -130,6 +130,14 @@ int tppx_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs,
 
 /* ---- linears ----------------------------------------------------------- */
 
+/* Workspace (`ws`, `ws_bytes`) of the linear entry points: optional device
+ * scratch, 256-byte aligned, that lets decode-shape launches with more than 16
+ * rows split K across workgroups (fp32 partial tiles, summed by a second small
+ * launch).  It needs no initialisation and carries no state between calls.
+ * Launches that share a workspace must be ordered on one stream.  With
+ * ws == NULL (or too small) the kernels simply do not split K.  32 MiB covers
+ * every decode shape up to M=64, N=32768. */
+
 /* Replaces call_gemm_with_post_op -> TppBlockedLinearW<bf16,uint8_t,bf16>
  * (MXFP4 branch, src/csrc/fused_gemm.h:785-1073,1510-1522) i.e.
  * torch.ops.tpp_llm.fc_plain (src/csrc/llm/fused_llm_infer.cpp:1514,1589) and
@@ -141,7 +149,7 @@ int tppx_linear_mxfp4(const void* x, const void* qw, const void* sw,
                       const void* bias, const void* post_in,
                       const void* post_in2, void* y, int64_t M, int64_t N,
                       int64_t K, int post_op, float post_scale, int flags,
-                      tppx_stream_t stream);
+                      void* ws, int64_t ws_bytes, tppx_stream_t stream);
 
 /* Replaces TppBlockedQInt8LinearW<bf16,uint8_t,bf16>
  * (src/csrc/fused_gemm.h:1076-1341,1530-1534): activations are quantized into
@@ -153,7 +161,8 @@ int tppx_linear_qint8(const void* x, void* xq, void* sa, const void* qw,
                       const void* sw, const void* bias, const void* post_in,
                       const void* post_in2, void* y, int64_t M, int64_t N,
                       int64_t K, int64_t qbs, int post_op, float post_scale,
-                      int flags, tppx_stream_t stream);
+                      int flags, void* ws, int64_t ws_bytes,
+                      tppx_stream_t stream);
 
 /* One GEMM of a fused group sharing the activation. */
 typedef struct tppx_seg {
@@ -173,12 +182,12 @@ typedef struct tppx_seg {
  * src/csrc/fused_gemm.h:1001-1064,1273-1332): up to 4 GEMMs over one
  * activation in one launch, each with its own output tensor and post-op. */
 int tppx_multi_linear_mxfp4(const void* x, const tppx_seg* segs, int n_segs,
-                            int64_t M, int64_t K, int flags,
-                            tppx_stream_t stream);
+                            int64_t M, int64_t K, int flags, void* ws,
+                            int64_t ws_bytes, tppx_stream_t stream);
 int tppx_multi_linear_qint8(const void* x, void* xq, void* sa,
                             const tppx_seg* segs, int n_segs, int64_t M,
-                            int64_t K, int64_t qbs, int flags,
-                            tppx_stream_t stream);
+                            int64_t K, int64_t qbs, int flags, void* ws,
+                            int64_t ws_bytes, tppx_stream_t stream);
 
 /* Replaces the gate/up pair of the Llama MLP
  * (src/csrc/llm/fused_llm_infer.cpp:1271-1272: i_gemm(SiluPostOp) then
@@ -187,8 +196,8 @@ int tppx_multi_linear_qint8(const void* x, void* xq, void* sa,
 int tppx_swiglu_mxfp4(const void* x, const void* qw_gate, const void* sw_gate,
                       const void* bias_gate, const void* qw_up,
                       const void* sw_up, const void* bias_up, void* y,
-                      int64_t M, int64_t N, int64_t K, int flags,
-                      tppx_stream_t stream);
+                      int64_t M, int64_t N, int64_t K, int flags, void* ws,
+                      int64_t ws_bytes, tppx_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -36,7 +36,7 @@ static bool valid_post(int post) {
 }
 
 // Checks one segment and fills the device descriptor.
-static int fill_seg(const char* who, const tppx_seg& s, SkinnySeg& d, int n_mult) {
+static int fill_seg(const char* who, const tppx_seg& s, DecodeSeg& d, int n_mult) {
   TPPX_REQUIRE(s.qw && s.sw && s.y, TPPX_EINVAL, "%s: null weight/scale/output pointer", who);
   TPPX_REQUIRE(aligned16(s.qw) && aligned16(s.y), TPPX_EINVAL, "%s: weight/output pointer not 16-byte aligned", who);
   TPPX_REQUIRE(valid_post(s.post_op), TPPX_EINVAL, "%s: unknown post-op id %d", who, s.post_op);
@@ -53,12 +53,14 @@ static int fill_seg(const char* who, const tppx_seg& s, SkinnySeg& d, int n_mult
   d.post_in2 = need2 ? (const uint16_t*)s.post_in2 : nullptr;
   d.y = (uint16_t*)s.y;
   d.N = (int)s.N;
+  d.tiles = (int)(s.N / 16);
   d.post_op = s.post_op;
   d.post_scale = s.post_scale;
   return TPPX_OK;
 }
 
-static int check_common(const char* who, const void* x, int64_t M, int64_t K, int n_segs, int flags) {
+static int check_common(const char* who, const void* x, int64_t M, int64_t K, int n_segs, int flags,
+                        const void* ws, int64_t ws_bytes) {
   TPPX_REQUIRE(x, TPPX_EINVAL, "%s: null activation pointer", who);
   TPPX_REQUIRE(aligned16(x), TPPX_EINVAL, "%s: activation pointer not 16-byte aligned", who);
   TPPX_REQUIRE(M > 0, TPPX_ESHAPE, "%s: M=%ld must be positive", who, (long)M);
@@ -66,51 +68,94 @@ static int check_common(const char* who, const void* x, int64_t M, int64_t K, in
   TPPX_REQUIRE(n_segs >= 1 && n_segs <= TPPX_MAX_SEGS, TPPX_EINVAL, "%s: number of fused GEMMs %d not in 1..%d", who, n_segs, TPPX_MAX_SEGS);
   TPPX_REQUIRE((flags & ~(TPPX_FLAG_FORCE_SKINNY | TPPX_FLAG_FORCE_TILED | TPPX_FLAG_ACT_FP8)) == 0, TPPX_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
   TPPX_REQUIRE(!((flags & TPPX_FLAG_FORCE_SKINNY) && (flags & TPPX_FLAG_FORCE_TILED)), TPPX_EINVAL, "%s: contradictory kernel-family flags", who);
+  TPPX_REQUIRE(ws_bytes >= 0 && (ws_bytes == 0 || ws), TPPX_EINVAL, "%s: workspace size %ld given with a null workspace", who, (long)ws_bytes);
+  TPPX_REQUIRE(ws == nullptr || (reinterpret_cast<uintptr_t>(ws) & 255u) == 0, TPPX_EINVAL, "%s: workspace not 256-byte aligned", who);
   return TPPX_OK;
 }
 
+// Fills segments, group/tile offsets; returns total tiles through *tiles.
+static void set_groups(DecodeParams& p, int tiles_per_group, bool dual) {
+  int groups = 0;
+  for (int i = 0; i < p.n_seg; i++) {
+    p.seg[i].grp0 = groups;
+    groups += (p.seg[i].tiles + tiles_per_group - 1) / tiles_per_group;
+  }
+  if (dual) {
+    p.seg[1].grp0 = 0;
+    groups = (p.seg[0].tiles + tiles_per_group - 1) / tiles_per_group;
+  }
+  p.groups = groups;
+}
+
+static int fill_all(const char* who, const tppx_seg* segs, int n_segs, int n_mult, bool dual,
+                    DecodeParams& p) {
+  int tiles = 0, groups = 0;
+  for (int i = 0; i < n_segs; i++) {
+    int rc = fill_seg(who, segs[i], p.seg[i], n_mult);
+    if (rc)
+      return rc;
+    p.seg[i].tile0 = tiles;
+    p.seg[i].grp0 = groups;
+    tiles += p.seg[i].tiles;
+    groups += (p.seg[i].tiles + 7) / 8;
+  }
+  if (dual) {
+    TPPX_REQUIRE(n_segs == 2 && segs[0].N == segs[1].N, TPPX_ESHAPE, "%s: gate and up projections must have equal N", who);
+    p.seg[1].tile0 = 0;
+    p.seg[1].grp0 = 0;
+    tiles = p.seg[0].tiles;
+    groups = (tiles + 7) / 8;
+  }
+  p.n_seg = n_segs;
+  p.total_tiles = tiles;
+  p.groups = groups;
+  return TPPX_OK;
+}
+
+static void bind_workspace(DecodeParams& p, const DecodePlan& pl, void* ws) {
+  p.S = pl.S;
+  p.cht = pl.cht;
+  p.part = (float*)ws;
+}
+
 static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n_segs,
-                     int64_t M, int64_t K, int flags, bool dual, hipStream_t stream) {
-  int rc = check_common(who, x, M, K, n_segs, flags);
+                     int64_t M, int64_t K, int flags, bool dual, void* ws, int64_t ws_bytes,
+                     hipStream_t stream) {
+  int rc = check_common(who, x, M, K, n_segs, flags, ws, ws_bytes);
   if (rc)
     return rc;
   TPPX_REQUIRE(segs, TPPX_EINVAL, "%s: null segment table", who);
   TPPX_REQUIRE(K > 0 && K % 64 == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of 64", who, (long)K);
   TPPX_REQUIRE(K % 128 == 0, TPPX_EUNSUPPORTED, "%s: K=%ld is not a multiple of 128 (native MXFP4 tiles span 128 input channels)", who, (long)K);
-  SkinnyParams p;
-  memset(&p, 0, sizeof(p));
-  int tiles = 0;
-  bool all_even = true;
-  for (int i = 0; i < n_segs; i++) {
-    rc = fill_seg(who, segs[i], p.seg[i], 32);
-    if (rc)
-      return rc;
-    p.seg[i].tile0 = tiles;
-    int t = (int)(segs[i].N / 16);
-    all_even = all_even && (t % 2 == 0);
-    tiles += t;
-  }
-  if (dual) {
-    TPPX_REQUIRE(n_segs == 2 && segs[0].N == segs[1].N, TPPX_ESHAPE, "%s: gate and up projections must have equal N", who);
-    tiles = (int)(segs[0].N / 16);
-    p.seg[1].tile0 = 0;
-  }
   TPPX_REQUIRE(!(flags & TPPX_FLAG_ACT_FP8), TPPX_EUNSUPPORTED, "%s: the FP8-activation path is not available", who);
-  p.n_seg = n_segs;
+  DecodeParams p;
+  memset(&p, 0, sizeof(p));
+  rc = fill_all(who, segs, n_segs, 32, dual, p);
+  if (rc)
+    return rc;
   p.x = x;
   p.M = (int)M;
   p.K = (int)K;
-  p.kunits = (int)(K / 128);
-  SkinnyPlan pl = plan_skinny(M, tiles, p.kunits, all_even, dual);
-  p.units_per_wave = pl.units_per_wave;
-  return check_hip(launch_skinny_mxfp4(p, pl, dual, stream), who);
+  p.units = (int)(K / 128);
+  p.tpb = 1;
+  p.S = 1;
+  if (M <= 16 && env_int("TPPX_MXFP4_SPLITK", 0) == 0) {
+    // GEMV class: K reduction inside the workgroup
+    SkinnyPlan sp = plan_skinny(0, M, p.total_tiles, p.units, dual);
+    set_groups(p, dual ? 1 : sp.ntw, dual);
+    return check_hip(launch_skinny_mxfp4(p, sp, dual, stream), who);
+  }
+  DecodePlan pl = plan_decode(0, M, p.groups, p.total_tiles, p.units, 1, dual, (size_t)ws_bytes);
+  bind_workspace(p, pl, ws);
+  return check_hip(launch_decode_mxfp4(p, pl, dual, stream), who);
 }
 
 static int run_qint8(const char* who, const void* x, void* xq, void* sa, const tppx_seg* segs,
-                     int n_segs, int64_t M, int64_t K, int64_t qbs, int flags, hipStream_t stream) {
+                     int n_segs, int64_t M, int64_t K, int64_t qbs, int flags, void* ws,
+                     int64_t ws_bytes, hipStream_t stream) {
   // x == NULL: xq / sa already hold quantized activations (the reference's
   // pre-quantized input case, src/csrc/fused_gemm.h:1244-1246)
-  int rc = check_common(who, x ? x : xq, M, K, n_segs, flags);
+  int rc = check_common(who, x ? x : xq, M, K, n_segs, flags, ws, ws_bytes);
   if (rc)
     return rc;
   TPPX_REQUIRE(segs, TPPX_EINVAL, "%s: null segment table", who);
@@ -118,34 +163,41 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
   TPPX_REQUIRE(aligned16(xq), TPPX_EINVAL, "%s: scratch pointer not 16-byte aligned", who);
   TPPX_REQUIRE(K > 0 && K % 64 == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of 64", who, (long)K);
   TPPX_REQUIRE(qbs > 0 && qbs % 64 == 0 && K % qbs == 0, TPPX_ESHAPE, "%s: block size mismatch (qbs=%ld, K=%ld)", who, (long)qbs, (long)K);
-  SkinnyParams p;
+  DecodeParams p;
   memset(&p, 0, sizeof(p));
-  int tiles = 0;
-  bool all_even = true;
-  for (int i = 0; i < n_segs; i++) {
-    rc = fill_seg(who, segs[i], p.seg[i], 16);
-    if (rc)
-      return rc;
-    p.seg[i].tile0 = tiles;
-    int t = (int)(segs[i].N / 16);
-    all_even = all_even && (t % 2 == 0);
-    tiles += t;
-  }
-  p.n_seg = n_segs;
+  rc = fill_all(who, segs, n_segs, 16, false, p);
+  if (rc)
+    return rc;
+  p.x = x;
   p.xq = xq;
   p.sa = (const float*)sa;
   p.M = (int)M;
   p.K = (int)K;
-  p.qbs = (int)qbs;
-  p.kunits = (int)(K / qbs);
-  if (x) {
+  p.units = (int)(K / qbs);
+  p.tpb = (int)(qbs / 64);
+  const int force = env_int("TPPX_QINT8_SPLITK", -1);
+  if (force == 1 || (force != 0 && M > 16)) {
+    // more than one MFMA row group: activations shared through LDS, K split
+    // across workgroups
+    DecodePlan pl = plan_decode(1, M, p.groups, p.total_tiles, p.units, p.tpb, false, (size_t)ws_bytes);
+    bind_workspace(p, pl, ws);
+    if (x && !pl.fused_quant) {
+      rc = tppx_quant_act_int8(x, M, K, qbs, xq, sa, stream);
+      if (rc)
+        return rc;
+    }
+    return check_hip(launch_decode_qint8(p, pl, stream), who);
+  }
+  p.S = 1;
+  SkinnyPlan sp = plan_skinny(1, M, p.total_tiles, p.units, false);
+  sp.fused_quant = sp.fused_quant && x != nullptr && qbs == 256;
+  if (x && !sp.fused_quant) {
     rc = tppx_quant_act_int8(x, M, K, qbs, xq, sa, stream);
     if (rc)
       return rc;
   }
-  SkinnyPlan pl = plan_skinny(M, tiles, p.kunits, all_even, false);
-  p.units_per_wave = pl.units_per_wave;
-  return check_hip(launch_skinny_qint8(p, pl, stream), who);
+  set_groups(p, sp.ntw, false);
+  return check_hip(launch_skinny_qint8(p, sp, stream), who);
 }
 
 } // namespace tppx
@@ -164,27 +216,28 @@ extern "C" int tppx_linear_mxfp4(const void* x, const void* qw, const void* sw,
                                  const void* bias, const void* post_in,
                                  const void* post_in2, void* y, int64_t M,
                                  int64_t N, int64_t K, int post_op,
-                                 float post_scale, int flags,
-                                 tppx_stream_t stream) {
+                                 float post_scale, int flags, void* ws,
+                                 int64_t ws_bytes, tppx_stream_t stream) {
   tppx_seg s = {qw, sw, bias, post_in, post_in2, y, N, post_op, post_scale};
-  return run_mxfp4("tppx_linear_mxfp4", x, &s, 1, M, K, flags, false, (hipStream_t)stream);
+  return run_mxfp4("tppx_linear_mxfp4", x, &s, 1, M, K, flags, false, ws, ws_bytes, (hipStream_t)stream);
 }
 
 extern "C" int tppx_multi_linear_mxfp4(const void* x, const tppx_seg* segs,
                                        int n_segs, int64_t M, int64_t K,
-                                       int flags, tppx_stream_t stream) {
-  return run_mxfp4("tppx_multi_linear_mxfp4", x, segs, n_segs, M, K, flags, false, (hipStream_t)stream);
+                                       int flags, void* ws, int64_t ws_bytes,
+                                       tppx_stream_t stream) {
+  return run_mxfp4("tppx_multi_linear_mxfp4", x, segs, n_segs, M, K, flags, false, ws, ws_bytes, (hipStream_t)stream);
 }
 
 extern "C" int tppx_swiglu_mxfp4(const void* x, const void* qw_gate,
                                  const void* sw_gate, const void* bias_gate,
                                  const void* qw_up, const void* sw_up,
                                  const void* bias_up, void* y, int64_t M,
-                                 int64_t N, int64_t K, int flags,
-                                 tppx_stream_t stream) {
+                                 int64_t N, int64_t K, int flags, void* ws,
+                                 int64_t ws_bytes, tppx_stream_t stream) {
   tppx_seg s[2] = {{qw_gate, sw_gate, bias_gate, nullptr, nullptr, y, N, TPPX_POST_NONE, 1.0f},
                    {qw_up, sw_up, bias_up, nullptr, nullptr, y, N, TPPX_POST_NONE, 1.0f}};
-  return run_mxfp4("tppx_swiglu_mxfp4", x, s, 2, M, K, flags, true, (hipStream_t)stream);
+  return run_mxfp4("tppx_swiglu_mxfp4", x, s, 2, M, K, flags, true, ws, ws_bytes, (hipStream_t)stream);
 }
 
 extern "C" int tppx_linear_qint8(const void* x, void* xq, void* sa,
@@ -192,15 +245,16 @@ extern "C" int tppx_linear_qint8(const void* x, void* xq, void* sa,
                                  const void* bias, const void* post_in,
                                  const void* post_in2, void* y, int64_t M,
                                  int64_t N, int64_t K, int64_t qbs, int post_op,
-                                 float post_scale, int flags,
-                                 tppx_stream_t stream) {
+                                 float post_scale, int flags, void* ws,
+                                 int64_t ws_bytes, tppx_stream_t stream) {
   tppx_seg s = {qw, sw, bias, post_in, post_in2, y, N, post_op, post_scale};
-  return run_qint8("tppx_linear_qint8", x, xq, sa, &s, 1, M, K, qbs, flags, (hipStream_t)stream);
+  return run_qint8("tppx_linear_qint8", x, xq, sa, &s, 1, M, K, qbs, flags, ws, ws_bytes, (hipStream_t)stream);
 }
 
 extern "C" int tppx_multi_linear_qint8(const void* x, void* xq, void* sa,
                                        const tppx_seg* segs, int n_segs,
                                        int64_t M, int64_t K, int64_t qbs,
-                                       int flags, tppx_stream_t stream) {
-  return run_qint8("tppx_multi_linear_qint8", x, xq, sa, segs, n_segs, M, K, qbs, flags, (hipStream_t)stream);
+                                       int flags, void* ws, int64_t ws_bytes,
+                                       tppx_stream_t stream) {
+  return run_qint8("tppx_multi_linear_qint8", x, xq, sa, segs, n_segs, M, K, qbs, flags, ws, ws_bytes, (hipStream_t)stream);
 }

@@ -1,6 +1,7 @@
 // Host-side launch descriptors shared by the C-ABI layer and the kernel files.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <stddef.h>
 #include <stdint.h>
 
 #define TPPX_MAX_SEGS 4
@@ -8,7 +9,7 @@
 namespace tppx {
 
 // One GEMM of a (possibly fused) group; device pointers.
-struct SkinnySeg {
+struct DecodeSeg {
   const void* qw;           // native weight tiles
   const void* sw;           // scales (u8 native for MXFP4, f32 reference for QINT8)
   const uint16_t* bias;     // bf16 [N] or null
@@ -16,31 +17,50 @@ struct SkinnySeg {
   const uint16_t* post_in2; // bf16 [M][N] or null
   uint16_t* y;              // bf16 [M][N]
   int N;
-  int tile0;                // first 16-channel tile of this GEMM in the fused tile space
+  int tiles;                // N / 16
+  int tile0;                // first tile of this GEMM in the fused tile space
+  int grp0;                 // first workgroup group (8 tiles each) of this GEMM
   int post_op;
   float post_scale;
 };
 
-struct SkinnyParams {
-  SkinnySeg seg[TPPX_MAX_SEGS];
+struct DecodeParams {
+  DecodeSeg seg[TPPX_MAX_SEGS];
   int n_seg;
-  const void* x;   // bf16 [M][K]            (MXFP4)
-  const void* xq;  // int8 [M][K]            (QINT8)
-  const float* sa; // f32  [M][K/qbs]        (QINT8)
+  int groups;      // sum over segments of ceil(tiles / 8)
+  int total_tiles; // sum of tiles (one segment's tiles for the dual gate/up kernel)
+  const void* x;   // bf16 [M][K]
+  const void* xq;  // int8 [M][K]     (QINT8, unless quantised in-kernel)
+  const float* sa; // f32  [M][K/qbs] (QINT8, unless quantised in-kernel)
   int M, K;
-  int kunits;         // K/128 (MXFP4) or K/qbs (QINT8)
-  int units_per_wave; // contiguous K units handled by one wave
-  int qbs;
+  int units; // K/128 (MXFP4 tiles) or K/qbs (QINT8 blocks)
+  int tpb;   // native tiles per unit (1 for MXFP4, qbs/64 for QINT8)
+  int S;     // K splits across workgroups
+  int cht;   // tiles of activations staged in LDS at a time
+  float* part;   // [S][grid_y][total_tiles][acc][MG][64] x f32x4 partial tiles (S > 1)
 };
 
+struct DecodePlan {
+  int mg, S, cht, grid_x, grid_y;
+  bool fused_quant;
+  size_t lds_bytes, counter_bytes;
+};
+
+// in-workgroup K split ("skinny") launch shape
 struct SkinnyPlan {
-  int mg, nt, waves, units_per_wave, grid_x, grid_y;
+  int mg, ntw, waves, max_units, grid_y;
+  bool fused_quant; // QINT8, M <= 4: activations quantised inside the GEMM kernel
 };
 
 int env_int(const char* name, int dflt);
 
-SkinnyPlan plan_skinny(int64_t M, int total_tiles, int kunits, bool all_even, bool dual);
-hipError_t launch_skinny_mxfp4(const SkinnyParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream);
-hipError_t launch_skinny_qint8(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t stream);
+SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual);
+hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream);
+hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream);
+
+DecodePlan plan_decode(int fmt, int64_t M, int groups, int total_tiles, int units, int tpb, bool dual,
+                       size_t ws_bytes);
+hipError_t launch_decode_mxfp4(const DecodeParams& p, const DecodePlan& pl, bool dual, hipStream_t stream);
+hipError_t launch_decode_qint8(const DecodeParams& p, const DecodePlan& pl, hipStream_t stream);
 
 } // namespace tppx

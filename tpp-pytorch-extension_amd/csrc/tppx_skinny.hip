@@ -1,14 +1,17 @@
-// Decode-shape ("skinny", M <= 64 per block row) weight-streaming kernels.
+// Decode-shape kernels with the K reduction kept inside the workgroup.
 //
-// Work decomposition: one workgroup owns NT consecutive 16-channel weight
-// tiles and all of K; its waves split K into contiguous ranges, stream their
-// 1 KiB native tiles straight from HBM into registers with one 128-bit load
-// per lane (PF loads in flight per wave), feed them to the 16x16 MFMA with the
-// activation rows as the other operand, and the per-wave fp32 partial tiles
-// are summed through LDS in a fixed order (deterministic results) before the
-// fused epilogue (bias, bf16 rounding, post-op) stores bf16.
+// One workgroup owns NTW consecutive 16-channel weight tiles and ALL of K; its
+// W (<= 16) waves split K into contiguous ranges.  A wave streams the native
+// 1 KiB tiles of its range for its NTW channel tiles straight from HBM into
+// registers (one 128-bit load per lane and tile, PF k-tiles in flight, the
+// first PF issued before anything else) together with the matching activation
+// operand (L2 resident), feeds the 16x16 MFMA, and at the end the W partial
+// tiles are summed through LDS in a fixed order (deterministic) and the fused
+// epilogue runs with post-op inputs that were fetched at kernel start.
+// No global atomics, no second pass: the tail after the last weight byte
+// arrives is one LDS round trip.
 //
-// MFMA operand convention used throughout (A = activations, B = weights):
+// MFMA operand convention (A = activations, B = weights):
 //   lane l supplies row/col (l & 15) and K group (l >> 4);
 //   result register r of lane l is D[m = (l >> 4) * 4 + r][n = l & 15].
 #include "tppx_common.h"
@@ -16,7 +19,7 @@
 
 namespace tppx {
 
-__device__ __forceinline__ bf16x8 cvt_fp4x8(uint32_t codes, float scale) {
+__device__ __forceinline__ bf16x8 sk_cvt_fp4x8(uint32_t codes, float scale) {
   bf16x2 c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 0);
   bf16x2 c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 1);
   bf16x2 c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 2);
@@ -27,388 +30,536 @@ __device__ __forceinline__ bf16x8 cvt_fp4x8(uint32_t codes, float scale) {
   return w;
 }
 
-__device__ __forceinline__ int find_seg(const SkinnyParams& p, int tile) {
+__device__ __forceinline__ int sk_find_seg(const DecodeParams& p, int grp) {
   int s = 0;
 #pragma unroll
   for (int i = 1; i < TPPX_MAX_SEGS; i++)
-    if (i < p.n_seg && tile >= p.seg[i].tile0)
+    if (i < p.n_seg && grp >= p.seg[i].grp0)
       s = i;
   return s;
 }
 
-// Sum the per-wave partial tiles through LDS and run the epilogue.
-// red layout: [wave][(nt*MG + mg)*256 + r*64 + lane]
-template <int MG, int NT, bool DUAL>
-__device__ __forceinline__ void reduce_and_store(const SkinnyParams& p,
-                                                 f32x4 (&acc)[NT][MG],
-                                                 int seg_id, int local_tile,
-                                                 int m0, float* red) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int W = blockDim.x >> 6;
-  constexpr int ELEMS = NT * MG * 256;
-  {
-    float* mine = red + wave * ELEMS;
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++)
-#pragma unroll
-      for (int mg = 0; mg < MG; mg++)
-#pragma unroll
-        for (int r = 0; r < 4; r++)
-          mine[(nt * MG + mg) * 256 + r * 64 + lane] = acc[nt][mg][r];
-    __syncthreads();
-  }
-  constexpr int OUT_ELEMS = DUAL ? ELEMS / 2 : ELEMS;
-  for (int e = threadIdx.x; e < OUT_ELEMS; e += blockDim.x) {
-    const int l = e & 63, r = (e >> 6) & 3, mg = (e >> 8) % MG;
-    const int nt = (e >> 8) / MG;
-    float v = 0.0f, v2 = 0.0f;
-    for (int w = 0; w < W; w++)
-      v += red[w * ELEMS + e];
-    if (DUAL)
-      for (int w = 0; w < W; w++)
-        v2 += red[w * ELEMS + e + ELEMS / 2];
-    const int m = m0 + mg * 16 + (l >> 4) * 4 + r;
-    if (m >= p.M)
-      continue;
-    if (DUAL) {
-      const SkinnySeg& g = p.seg[0];
-      const SkinnySeg& u = p.seg[1];
-      const int n = (local_tile + nt) * 16 + (l & 15);
-      if (g.bias)
-        v += bf16_bits_to_f32(g.bias[n]);
-      if (u.bias)
-        v2 += bf16_bits_to_f32(u.bias[n]);
-      uint32_t gact = apply_post_bits(v, TPPX_POST_SILU, 0, 0, 1.0f);
-      uint32_t out = apply_post_bits(v2, TPPX_POST_MUL, gact, 0, 1.0f);
-      g.y[(int64_t)m * g.N + n] = (uint16_t)out;
-    } else {
-      const SkinnySeg& sg = p.seg[seg_id];
-      const int n = (local_tile + nt) * 16 + (l & 15);
-      const int64_t o = (int64_t)m * sg.N + n;
-      if (sg.bias)
-        v += bf16_bits_to_f32(sg.bias[n]);
-      uint32_t in1 = sg.post_in ? sg.post_in[o] : 0u;
-      uint32_t in2 = sg.post_in2 ? sg.post_in2[o] : 0u;
-      sg.y[o] = (uint16_t)apply_post_bits(v, sg.post_op, in1, in2, sg.post_scale);
-    }
-  }
-}
+// LDS reduction over the waves of the workgroup + fused epilogue.
+// red layout: [wave][(a*MG + mg)*256 + r*64 + lane]; every thread finishes
+// EPT = NACC_OUT*MG*256 / blockDim outputs whose post-op inputs it fetched
+// before the main loop.
+template <int MG, int NACC, bool DUAL, int MINW>
+struct SkEpilogue {
+  static constexpr int ELEMS = NACC * MG * 256;
+  static constexpr int OUT = DUAL ? ELEMS / 2 : ELEMS;
+  // outputs per thread; the launcher never uses fewer than MINW waves
+  static constexpr int MAXE = (OUT + MINW * 64 - 1) / (MINW * 64);
+  int64_t off[MAXE];
+  uint32_t in1[MAXE], in2[MAXE];
+  float bias[MAXE], bias2[MAXE];
+  bool ok[MAXE];
 
-// ---------------------------------------------------------------------------
-// MXFP4 weight-only: bf16 activations x (E2M1 * 2^e -> bf16, exact) weights,
-// v_mfma_f32_16x16x32_bf16, fp32 accumulation over all of K.
-// One native tile = 16 channels x 128 K = 4 MFMAs (one MX block per lane).
-// ---------------------------------------------------------------------------
-template <int MG, int NT, int PF, bool DUAL>
-__global__ void __launch_bounds__(512)
-skinny_mxfp4_kernel(const SkinnyParams p) {
-  extern __shared__ float red[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int KT = p.kunits;
-  constexpr int NTG = DUAL ? NT / 2 : NT; // distinct channel tiles per group
-  const int tile = blockIdx.x * NTG;
-  const int seg_id = DUAL ? 0 : find_seg(p, tile);
-  const int local_tile = tile - p.seg[seg_id].tile0;
-  const int m0 = blockIdx.y * (16 * MG);
-  const int kbeg = wave * p.units_per_wave;
-  const int kend = min(kbeg + p.units_per_wave, KT);
-
-  const i32x4* wq[NT];
-  const uint8_t* ws[NT];
+  __device__ __forceinline__ void prefetch(const DecodeParams& p, const DecodeSeg& sg, int ltile0, int m0) {
 #pragma unroll
-  for (int nt = 0; nt < NT; nt++) {
-    const SkinnySeg& sg = DUAL ? p.seg[nt / NTG] : p.seg[seg_id];
-    const int64_t lt = local_tile + (DUAL ? nt % NTG : nt);
-    wq[nt] = reinterpret_cast<const i32x4*>(sg.qw) + lt * KT * 64 + lane;
-    ws[nt] = reinterpret_cast<const uint8_t*>(sg.sw) + lt * KT * 64 + lane;
-  }
-  const uint16_t* xrow[MG];
-#pragma unroll
-  for (int mg = 0; mg < MG; mg++) {
-    int m = min(m0 + mg * 16 + (lane & 15), p.M - 1);
-    xrow[mg] = reinterpret_cast<const uint16_t*>(p.x) + (int64_t)m * p.K + (lane >> 4) * 32;
-  }
-
-  f32x4 acc[NT][MG];
-#pragma unroll
-  for (int nt = 0; nt < NT; nt++)
-#pragma unroll
-    for (int mg = 0; mg < MG; mg++)
-      acc[nt][mg] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  i32x4 wreg[PF][NT];
-  uint32_t sreg[PF][NT];
-  bf16x8 xreg[PF][MG][4];
-
-  auto load_stage = [&](int st, int kt) {
-    kt = min(kt, kend - 1); // clamped: redundant but always in bounds
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)kt * 64);
-      sreg[st][nt] = ws[nt][(int64_t)kt * 64];
-    }
-#pragma unroll
-    for (int mg = 0; mg < MG; mg++)
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        xreg[st][mg][j] = *reinterpret_cast<const bf16x8*>(xrow[mg] + kt * 128 + j * 8);
-  };
-  auto compute_stage = [&](int st) {
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      const float s = e8m0_to_f32(sreg[st][nt]);
-      const uint32_t cw[4] = {(uint32_t)wreg[st][nt][0], (uint32_t)wreg[st][nt][1], (uint32_t)wreg[st][nt][2], (uint32_t)wreg[st][nt][3]};
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        bf16x8 wb = cvt_fp4x8(cw[j], s);
-#pragma unroll
-        for (int mg = 0; mg < MG; mg++)
-          acc[nt][mg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              xreg[st][mg][j], wb, acc[nt][mg], 0, 0, 0);
-      }
-    }
-  };
-
-  if (kbeg < kend) {
-#pragma unroll
-    for (int i = 0; i < PF; i++)
-      load_stage(i, kbeg + i);
-    for (int kt = kbeg; kt < kend; kt += PF) {
-#pragma unroll
-      for (int i = 0; i < PF; i++) {
-        if (kt + i < kend) {
-          compute_stage(i);
-          if (kt + i + PF < kend)
-            load_stage(i, kt + i + PF);
+    for (int i = 0; i < MAXE; i++) {
+      const int e = threadIdx.x + i * blockDim.x;
+      ok[i] = false;
+      in1[i] = in2[i] = 0;
+      bias[i] = bias2[i] = 0.f;
+      off[i] = 0;
+      if (e < OUT) {
+        const int l = e & 63, r = (e >> 6) & 3, mg = (e >> 8) % MG, a = (e >> 8) / MG;
+        const int m = m0 + mg * 16 + (l >> 4) * 4 + r;
+        const int n = (ltile0 + a) * 16 + (l & 15);
+        ok[i] = m < p.M && (ltile0 + a) < sg.tiles;
+        if (ok[i]) {
+          off[i] = (int64_t)m * sg.N + n;
+          if (sg.bias)
+            bias[i] = bf16_bits_to_f32(sg.bias[n]);
+          if (DUAL && p.seg[1].bias)
+            bias2[i] = bf16_bits_to_f32(p.seg[1].bias[n]);
+          if (sg.post_in)
+            in1[i] = sg.post_in[off[i]];
+          if (sg.post_in2)
+            in2[i] = sg.post_in2[off[i]];
         }
       }
     }
   }
-  reduce_and_store<MG, NT, DUAL>(p, acc, seg_id, local_tile, m0, red);
-}
 
-// ---------------------------------------------------------------------------
-// QINT8 (W8A8): int8 activations x int8 weights, v_mfma_i32_16x16x64_i8 with
-// exact int32 sums per K block of qbs, then fp32 scale-and-accumulate
-//   f = fma(float(acc), sa[m][b] * sw[n][b], f).
-// One native tile = 16 channels x 64 K = 1 MFMA; a unit of work is one block
-// of qbs/64 tiles.
-// ---------------------------------------------------------------------------
-template <int MG, int NT, int PF>
-__global__ void __launch_bounds__(512)
-skinny_qint8_kernel(const SkinnyParams p) {
-  extern __shared__ float red[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int NB = p.kunits;       // K blocks of qbs
-  const int TPB = p.qbs >> 6;    // tiles per block
-  const int KT = NB * TPB;
-  const int tile = blockIdx.x * NT;
-  const int seg_id = find_seg(p, tile);
-  const SkinnySeg& sg = p.seg[seg_id];
-  const int local_tile = tile - sg.tile0;
-  const int m0 = blockIdx.y * (16 * MG);
-  const int bbeg = wave * p.units_per_wave;
-  const int bend = min(bbeg + p.units_per_wave, NB);
-  const int kbeg = bbeg * TPB, kend = bend * TPB;
-
-  const i32x4* wq[NT];
-  const float* ws[NT];
+  __device__ __forceinline__ void finish(const DecodeSeg& sg, f32x4 (&acc)[NACC][MG], float* red) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int W = blockDim.x >> 6;
+    float* mine = red + wave * ELEMS;
 #pragma unroll
-  for (int nt = 0; nt < NT; nt++) {
-    const int64_t lt = local_tile + nt;
+    for (int a = 0; a < NACC; a++)
+#pragma unroll
+      for (int mg = 0; mg < MG; mg++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          mine[(a * MG + mg) * 256 + r * 64 + lane] = acc[a][mg][r];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < MAXE; i++) {
+      const int e = threadIdx.x + i * blockDim.x;
+      if (e < OUT) {
+        float v = 0.f, v2 = 0.f;
+        for (int w = 0; w < W; w++)
+          v += red[w * ELEMS + e];
+        if (DUAL)
+          for (int w = 0; w < W; w++)
+            v2 += red[w * ELEMS + e + ELEMS / 2];
+        if (ok[i]) {
+          uint32_t out;
+          if (DUAL) {
+            uint32_t gact = apply_post_bits(v + bias[i], TPPX_POST_SILU, 0, 0, 1.0f);
+            out = apply_post_bits(v2 + bias2[i], TPPX_POST_MUL, gact, 0, 1.0f);
+          } else {
+            out = apply_post_bits(v + bias[i], sg.post_op, in1[i], in2[i], sg.post_scale);
+          }
+          sg.y[off[i]] = (uint16_t)out;
+        }
+      }
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------
+// QINT8 (W8A8), activations already quantised (int8 [M][K] + f32 [M][K/qbs]).
+// ---------------------------------------------------------------------------
+template <int MG, int NTW, int PF, int MAXW, int MINW>
+__global__ void __launch_bounds__(MAXW * 64)
+skinny_qint8_kernel(const DecodeParams p) {
+  extern __shared__ __align__(16) float sk_lds[];
+  constexpr int MPAD = MG * 16;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int W = blockDim.x >> 6;
+  const int grp = blockIdx.x;
+  const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
+  const int ltile0 = (grp - sg.grp0) * NTW;
+  const int m0 = blockIdx.y * MPAD;
+  const int NB = p.units, TPB = p.tpb, KT = NB * TPB;
+  const int u0 = (int)(((int64_t)wave * NB) / W), u1 = (int)(((int64_t)(wave + 1) * NB) / W);
+  const int t0 = u0 * TPB, t1 = u1 * TPB;
+
+  const i32x4* wq[NTW];
+  const float* ws[NTW];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++) {
+    const int64_t lt = min(ltile0 + nt, sg.tiles - 1); // ragged last group: duplicate, not stored
     wq[nt] = reinterpret_cast<const i32x4*>(sg.qw) + lt * KT * 64 + lane;
     ws[nt] = reinterpret_cast<const float*>(sg.sw) + lt * NB * 16 + (lane & 15);
   }
   const int8_t* xrow[MG];
-  const float* sarow[MG][4];
 #pragma unroll
   for (int mg = 0; mg < MG; mg++) {
-    int m = min(m0 + mg * 16 + (lane & 15), p.M - 1);
+    const int m = min(m0 + mg * 16 + (lane & 15), p.M - 1);
     xrow[mg] = reinterpret_cast<const int8_t*>(p.xq) + (int64_t)m * p.K + (lane >> 4) * 16;
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-      int mr = min(m0 + mg * 16 + (lane >> 4) * 4 + r, p.M - 1);
-      sarow[mg][r] = p.sa + (int64_t)mr * NB;
-    }
   }
 
-  f32x4 facc[NT][MG];
-  i32x4 iacc[NT][MG];
+  // Loads return in issue order: the small L2-resident ones (activation
+  // scales, post-op inputs) go out BEFORE the weight ring so that waiting for
+  // them does not wait for HBM.
+  SkEpilogue<MG, NTW, false, MINW> ep;
+  ep.prefetch(p, sg, ltile0, m0);
+  // activation scales of this wave's K blocks, transposed in LDS: [u - u0][MPAD]
+  float* red = sk_lds;
+  float* sa_s = sk_lds + (size_t)W * NTW * MG * 256 + (size_t)wave * p.cht * MPAD;
+  for (int i = lane; i < (u1 - u0) * MPAD; i += 64) {
+    const int ul = i / MPAD, mr = i - ul * MPAD;
+    sa_s[i] = p.sa[(int64_t)min(m0 + mr, p.M - 1) * NB + u0 + ul];
+  }
+
+  i32x4 wreg[PF][NTW], xreg[PF][MG];
+  auto load_stage = [&](int st, int t) {
+    t = min(t, t1 - 1);
 #pragma unroll
-  for (int nt = 0; nt < NT; nt++)
+    for (int nt = 0; nt < NTW; nt++)
+      wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64);
+#pragma unroll
+    for (int mg = 0; mg < MG; mg++)
+      xreg[st][mg] = *reinterpret_cast<const i32x4*>(xrow[mg] + t * 64);
+  };
+  if (t0 < t1) {
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+      load_stage(i, t0 + i);
+  }
+
+  f32x4 facc[NTW][MG];
+  i32x4 iacc[NTW][MG];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++)
 #pragma unroll
     for (int mg = 0; mg < MG; mg++) {
       facc[nt][mg] = f32x4{0.f, 0.f, 0.f, 0.f};
       iacc[nt][mg] = i32x4{0, 0, 0, 0};
     }
 
-  i32x4 wreg[PF][NT];
-  i32x4 xreg[PF][MG];
-
-  auto load_stage = [&](int st, int kt) {
-    kt = min(kt, kend - 1);
+  for (int t = t0; t < t1; t += PF) {
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++)
-      wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)kt * 64);
+    for (int i = 0; i < PF; i++) {
+      const int tt = t + i;
+      if (tt < t1) {
 #pragma unroll
-    for (int mg = 0; mg < MG; mg++)
-      xreg[st][mg] = *reinterpret_cast<const i32x4*>(xrow[mg] + kt * 64);
-  };
-  auto compute_stage = [&](int st, int kt) {
+        for (int nt = 0; nt < NTW; nt++)
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++)
+          for (int mg = 0; mg < MG; mg++)
+            iacc[nt][mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xreg[i][mg], wreg[i][nt], iacc[nt][mg], 0, 0, 0);
+        if (tt + PF < t1)
+          load_stage(i, tt + PF);
+        if ((tt + 1) % TPB == 0) { // K block complete: scale and fold into fp32
+          const int b = tt / TPB;
 #pragma unroll
-      for (int mg = 0; mg < MG; mg++)
-        iacc[nt][mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-            xreg[st][mg], wreg[st][nt], iacc[nt][mg], 0, 0, 0);
-    if ((kt + 1) % TPB == 0) { // block complete: scale and fold into fp32
-      const int b = kt / TPB;
+          for (int mg = 0; mg < MG; mg++) {
+            const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + (b - u0) * MPAD + mg * 16 + (lane >> 4) * 4);
 #pragma unroll
-      for (int nt = 0; nt < NT; nt++) {
-        const float swv = ws[nt][b * 16];
+            for (int nt = 0; nt < NTW; nt++) {
+              const float swv = ws[nt][b * 16];
 #pragma unroll
-        for (int mg = 0; mg < MG; mg++)
-#pragma unroll
-          for (int r = 0; r < 4; r++) {
-            const float s = sarow[mg][r][b] * swv;
-            facc[nt][mg][r] = fmaf((float)iacc[nt][mg][r], s, facc[nt][mg][r]);
-            iacc[nt][mg][r] = 0;
+              for (int r = 0; r < 4; r++) {
+                facc[nt][mg][r] = fmaf((float)iacc[nt][mg][r], sav[r] * swv, facc[nt][mg][r]);
+                iacc[nt][mg][r] = 0;
+              }
+            }
           }
-      }
-    }
-  };
-
-  if (kbeg < kend) {
-#pragma unroll
-    for (int i = 0; i < PF; i++)
-      load_stage(i, kbeg + i);
-    for (int kt = kbeg; kt < kend; kt += PF) {
-#pragma unroll
-      for (int i = 0; i < PF; i++) {
-        if (kt + i < kend) {
-          compute_stage(i, kt + i);
-          if (kt + i + PF < kend)
-            load_stage(i, kt + i + PF);
         }
       }
     }
   }
-  reduce_and_store<MG, NT, false>(p, facc, seg_id, local_tile, m0, red);
+  ep.finish(sg, facc, red);
 }
 
 // ---------------------------------------------------------------------------
-// launchers
+// QINT8 with the activation quantisation fused in, for M <= 4 (qbs == 256).
+// Every wave quantises the rows of its own K range (one (row, block) item =
+// 64 lanes x 4 values, DPP max reduction) into a wave-private LDS region that
+// keeps only the M valid rows of each operand tile, then reads its MFMA
+// operand from there (lanes of the padded rows re-read row M-1), so the main
+// loop issues weight loads only and the whole ring is in flight from the
+// first instruction.
 // ---------------------------------------------------------------------------
-template <int MG, int NT, int PF, bool DUAL>
-static hipError_t launch_mxfp4_t(const SkinnyParams& p, dim3 grid, int waves,
-                                 hipStream_t stream) {
-  size_t lds = (size_t)waves * NT * MG * 256 * sizeof(float);
-  auto kern = skinny_mxfp4_kernel<MG, NT, PF, DUAL>;
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess)
-      return e;
-  }
-  kern<<<grid, dim3(64 * waves), lds, stream>>>(p);
-  return hipGetLastError();
+template <int CTRL>
+__device__ __forceinline__ float sk_dpp_max(float v) {
+  int o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true);
+  return fmaxf(v, __int_as_float(o));
+}
+__device__ __forceinline__ float sk_wave_max(float v) {
+  v = sk_dpp_max<0xB1>(v);  // quad_perm [1,0,3,2]
+  v = sk_dpp_max<0x4E>(v);  // quad_perm [2,3,0,1]
+  v = sk_dpp_max<0x141>(v); // row_half_mirror
+  v = sk_dpp_max<0x140>(v); // row_mirror
+  float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+__device__ __forceinline__ int sk_int8_rne(float v, float inv) {
+  float r = rintf(__fmul_rn(v, inv));
+  return (int)fminf(fmaxf(r, -127.0f), 127.0f);
 }
 
-template <int MG, int NT, int PF>
-static hipError_t launch_qint8_t(const SkinnyParams& p, dim3 grid, int waves,
-                                 hipStream_t stream) {
-  size_t lds = (size_t)waves * NT * MG * 256 * sizeof(float);
-  auto kern = skinny_qint8_kernel<MG, NT, PF>;
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess)
-      return e;
+template <int NTW, int PF, int MAXW, int MINW>
+__global__ void __launch_bounds__(MAXW * 64)
+skinny_qint8_fq_kernel(const DecodeParams p) {
+  extern __shared__ __align__(16) float sk_lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int W = blockDim.x >> 6;
+  const int grp = blockIdx.x;
+  const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
+  const int ltile0 = (grp - sg.grp0) * NTW;
+  const int M = p.M; // <= 4, one block row
+  const int NB = p.units, KT = NB * 4;
+  const int u0 = (int)(((int64_t)wave * NB) / W), u1 = (int)(((int64_t)(wave + 1) * NB) / W);
+  const int t0 = u0 * 4, t1 = u1 * 4;
+
+  const i32x4* wq[NTW];
+  const float* ws[NTW];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++) {
+    const int64_t lt = min(ltile0 + nt, sg.tiles - 1);
+    wq[nt] = reinterpret_cast<const i32x4*>(sg.qw) + lt * KT * 64 + lane;
+    ws[nt] = reinterpret_cast<const float*>(sg.sw) + lt * NB * 16 + (lane & 15);
   }
-  kern<<<grid, dim3(64 * waves), lds, stream>>>(p);
-  return hipGetLastError();
+  // Loads return in issue order, so everything small and L2-resident that the
+  // wave needs early (its activation rows, the post-op inputs) is requested
+  // BEFORE the weight ring: waiting for it then does not wait for HBM.
+  // One (row, block) item = 256 values = 16 lanes x 16 values, so a wave
+  // quantises four items per pass and the max reduction stays inside a DPP row.
+  constexpr int XP = 3; // passes: M <= 4 rows x <= 3 blocks per wave = 12 items
+  const uint16_t* xb = reinterpret_cast<const uint16_t*>(p.x);
+  const int nitems = M * (u1 - u0);
+  uint4 raw[XP][2];
+#pragma unroll
+  for (int ps = 0; ps < XP; ps++) {
+    const int it = min(ps * 4 + (lane >> 4), max(nitems - 1, 0));
+    const int ul = it / M, mr = it - ul * M;
+    const uint4* src = reinterpret_cast<const uint4*>(xb + (int64_t)mr * p.K + (int64_t)(u0 + ul) * 256 + (lane & 15) * 16);
+    raw[ps][0] = src[0];
+    raw[ps][1] = src[1];
+  }
+  SkEpilogue<1, NTW, false, MINW> ep;
+  ep.prefetch(p, sg, ltile0, 0);
+
+  i32x4 wreg[PF][NTW];
+  auto load_stage = [&](int st, int t) {
+    t = min(t, t1 - 1);
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++)
+      wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64);
+  };
+  if (t0 < t1) {
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+      load_stage(i, t0 + i);
+  }
+
+  // wave-private LDS: xq [tile][g][M rows][16 B], then sa [unit][4]
+  float* red = sk_lds;
+  uint8_t* mine = reinterpret_cast<uint8_t*>(sk_lds + (size_t)W * NTW * 256) + (size_t)wave * p.cht * (4 * 256 + 16);
+  uint32_t* xq_s = reinterpret_cast<uint32_t*>(mine);
+  float* sa_s = reinterpret_cast<float*>(mine + (size_t)p.cht * 4 * 256);
+#pragma unroll
+  for (int ps = 0; ps < XP; ps++) {
+    if (ps * 4 < nitems) { // wave-uniform
+      const int it = ps * 4 + (lane >> 4);
+      const int itc = min(it, nitems - 1);
+      const int ul = itc / M, mr = itc - ul * M;
+      const uint32_t wd[8] = {raw[ps][0].x, raw[ps][0].y, raw[ps][0].z, raw[ps][0].w,
+                              raw[ps][1].x, raw[ps][1].y, raw[ps][1].z, raw[ps][1].w};
+      float v[16];
+      float amax = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        v[2 * j] = bf16_bits_to_f32(wd[j] & 0xffffu);
+        v[2 * j + 1] = bf16_bits_to_f32(wd[j] >> 16);
+        amax = fmaxf(amax, fmaxf(fabsf(v[2 * j]), fabsf(v[2 * j + 1])));
+      }
+      amax = sk_dpp_max<0xB1>(amax);  // quad_perm [1,0,3,2]
+      amax = sk_dpp_max<0x4E>(amax);  // quad_perm [2,3,0,1]
+      amax = sk_dpp_max<0x141>(amax); // row_half_mirror
+      amax = sk_dpp_max<0x140>(amax); // row_mirror: every lane of the row holds the max
+      // == float(double(amax) / 127.0): amax is a bf16 value, so the
+      // quotient cannot sit on a double-rounding boundary
+      const float sc = __fdiv_rn(amax, 127.0f);
+      const float inv = sc != 0.0f ? __frcp_rn(sc) : 0.0f;
+      uint32_t pk[4];
+#pragma unroll
+      for (int d = 0; d < 4; d++)
+        pk[d] = (uint32_t)(sk_int8_rne(v[4 * d], inv) & 0xff) | ((uint32_t)(sk_int8_rne(v[4 * d + 1], inv) & 0xff) << 8) |
+            ((uint32_t)(sk_int8_rne(v[4 * d + 2], inv) & 0xff) << 16) | ((uint32_t)(sk_int8_rne(v[4 * d + 3], inv) & 0xff) << 24);
+      if (it < nitems) {
+        // values k = (lane&15)*16.. of the block: tile (lane&15)/4, K group (lane&15)%4
+        const int tl = ul * 4 + ((lane & 15) >> 2), g = lane & 3;
+        reinterpret_cast<uint4*>(xq_s)[(tl * 4 + g) * M + mr] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        if ((lane & 15) == 0)
+          sa_s[ul * 4 + mr] = sc;
+      }
+    }
+  }
+  const int xoff = ((lane >> 4) * M + min(lane & 15, M - 1)) * 4; // dword offset inside a tile
+
+  f32x4 facc[NTW][1];
+  i32x4 iacc[NTW];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++) {
+    facc[nt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+    iacc[nt] = i32x4{0, 0, 0, 0};
+  }
+  for (int t = t0; t < t1; t += PF) {
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      const int tt = t + i;
+      if (tt < t1) {
+        const i32x4 xa = *reinterpret_cast<const i32x4*>(xq_s + (tt - t0) * 16 * M + xoff);
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++)
+          iacc[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa, wreg[i][nt], iacc[nt], 0, 0, 0);
+        if (tt + PF < t1)
+          load_stage(i, tt + PF);
+        if ((tt & 3) == 3) { // K block complete
+          const int b = tt >> 2;
+          // result rows (lane>>4)*4 + r: only the first lane group holds valid rows (M <= 4)
+          const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + (b - u0) * 4);
+#pragma unroll
+          for (int nt = 0; nt < NTW; nt++) {
+            const float swv = ws[nt][b * 16];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              facc[nt][0][r] = fmaf((float)iacc[nt][r], sav[r] * swv, facc[nt][0][r]);
+              iacc[nt][r] = 0;
+            }
+          }
+        }
+      }
+    }
+  }
+  ep.finish(sg, facc, red);
 }
 
-// Pick (MG, NT, waves) for a problem.  total_tiles = sum of N/16 over the
-// segments; kunits = K/128 (MXFP4) or K/qbs (QINT8).
-SkinnyPlan plan_skinny(int64_t M, int total_tiles, int kunits, bool all_even,
-                       bool dual) {
+// ---------------------------------------------------------------------------
+// MXFP4 weight-only, M <= 16 per block row (one MFMA row group).
+// DUAL: NTW = 2 accumulators = the gate tile and the up tile of one channel
+// tile; epilogue silu(gate) * up.
+// ---------------------------------------------------------------------------
+template <int NTW, int PF, int MAXW, int MINW, bool DUAL>
+__global__ void __launch_bounds__(MAXW * 64)
+skinny_mxfp4_kernel(const DecodeParams p) {
+  extern __shared__ __align__(16) float sk_lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int W = blockDim.x >> 6;
+  const int grp = blockIdx.x;
+  const int seg_id = DUAL ? 0 : sk_find_seg(p, grp);
+  const DecodeSeg& sg = p.seg[seg_id];
+  const int ltile0 = (grp - sg.grp0) * (DUAL ? 1 : NTW);
+  const int m0 = blockIdx.y * 16;
+  const int KT = p.units;
+  const int t0 = (int)(((int64_t)wave * KT) / W), t1 = (int)(((int64_t)(wave + 1) * KT) / W);
+
+  const i32x4* wq[NTW];
+  const uint8_t* wsc[NTW];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++) {
+    const DecodeSeg& ss = p.seg[DUAL ? nt : seg_id];
+    const int64_t lt = DUAL ? ltile0 : min(ltile0 + nt, sg.tiles - 1);
+    wq[nt] = reinterpret_cast<const i32x4*>(ss.qw) + lt * KT * 64 + lane;
+    wsc[nt] = reinterpret_cast<const uint8_t*>(ss.sw) + lt * KT * 64 + lane;
+  }
+  const int mrow = min(m0 + (lane & 15), p.M - 1);
+  const uint16_t* xrow = reinterpret_cast<const uint16_t*>(p.x) + (int64_t)mrow * p.K + (lane >> 4) * 32;
+
+  i32x4 wreg[PF][NTW];
+  uint32_t sreg[PF][NTW];
+  bf16x8 xreg[PF][4];
+  auto load_stage = [&](int st, int t) {
+    t = min(t, t1 - 1);
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++) {
+      wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64);
+      sreg[st][nt] = wsc[nt][(int64_t)t * 64];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      xreg[st][j] = *reinterpret_cast<const bf16x8*>(xrow + t * 128 + j * 8);
+  };
+  if (t0 < t1) {
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+      load_stage(i, t0 + i);
+  }
+
+  SkEpilogue<1, NTW, DUAL, MINW> ep;
+  ep.prefetch(p, sg, ltile0, m0);
+
+  f32x4 acc[NTW][1];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++)
+    acc[nt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int t = t0; t < t1; t += PF) {
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      const int tt = t + i;
+      if (tt < t1) {
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++) {
+          const float sc = e8m0_to_f32(sreg[i][nt]);
+#pragma unroll
+          for (int j = 0; j < 4; j++)
+            acc[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                xreg[i][j], sk_cvt_fp4x8((uint32_t)wreg[i][nt][j], sc), acc[nt][0], 0, 0, 0);
+        }
+        if (tt + PF < t1)
+          load_stage(i, tt + PF);
+      }
+    }
+  }
+  ep.finish(sg, acc, sk_lds);
+}
+
+// ---------------------------------------------------------------------------
+// planning and launch
+// ---------------------------------------------------------------------------
+SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual) {
   SkinnyPlan pl;
-  int mrows = (int)(M < 64 ? M : 64);
-  pl.mg = mrows <= 16 ? 1 : (mrows <= 32 ? 2 : 4);
+  const int mrows = (int)(M < 64 ? M : 64);
+  pl.mg = fmt == 0 ? 1 : (mrows <= 16 ? 1 : (mrows <= 32 ? 2 : 4));
   pl.grid_y = (int)((M + 16 * pl.mg - 1) / (16 * pl.mg));
-  pl.nt = 1;
-  // Two channel tiles per wave halve the activation-operand traffic once the
-  // activation block is as large as the weight tile it meets.
-  if (!dual && all_even && pl.mg >= 2 && total_tiles >= 1024)
-    pl.nt = 2;
-  int env_nt = env_int("TPPX_SKINNY_NT", 0);
-  if (!dual && env_nt == 1)
-    pl.nt = 1;
-  if (!dual && env_nt == 2 && all_even)
-    pl.nt = 2;
+  // two channel tiles per wave once there are plenty of tiles: halves the
+  // activation-operand traffic per weight byte
+  pl.ntw = (!dual && total_tiles >= 512) ? 2 : 1;
+  int env_ntw = env_int("TPPX_SKINNY_NTW", 0);
+  if (!dual && (env_ntw == 1 || env_ntw == 2))
+    pl.ntw = env_ntw;
   if (dual)
-    pl.nt = 2;
-  int groups = dual ? total_tiles : total_tiles / pl.nt;
-  // aim for ~16 waves per CU over 256 CUs, at least 2 K units per wave
-  int target_waves = 256 * 16;
-  int w = (target_waves + groups * pl.grid_y - 1) / (groups * pl.grid_y);
-  if (w > 8)
-    w = 8;
-  if (w > kunits / 2)
-    w = kunits / 2;
-  if (w < 1)
-    w = 1;
-  int env_w = env_int("TPPX_SKINNY_WAVES", 0);
-  if (env_w > 0)
-    w = env_w > 8 ? 8 : env_w;
-  if (w > kunits)
-    w = kunits;
-  pl.units_per_wave = (kunits + w - 1) / w;
-  pl.waves = (kunits + pl.units_per_wave - 1) / pl.units_per_wave;
-  pl.grid_x = groups;
+    pl.ntw = 2;
+  // Wave-count window of the kernel instantiation that will run (register
+  // budget: 16 waves leave 128 VGPRs per lane, 8 leave 256; the epilogue's
+  // outputs-per-thread bound sets the minimum).  Waves beyond the number of K
+  // units simply get an empty range.
+  int max_w, min_w;
+  if (fmt == 1) {
+    max_w = pl.mg == 4 ? 8 : 16;
+    min_w = (pl.mg == 4 || (pl.mg == 2 && pl.ntw == 2)) ? 8 : 4;
+  } else {
+    max_w = pl.ntw == 2 ? 8 : 16;
+    min_w = 4;
+  }
+  // few tiles: one 16-wave workgroup per CU keeps the whole weight in flight
+  int w = env_int("TPPX_SKINNY_WAVES", (total_tiles / pl.ntw <= 320) ? 16 : 8);
+  if (w > units)
+    w = units;
+  if (w > max_w)
+    w = max_w;
+  if (w < min_w)
+    w = min_w;
+  pl.waves = w;
+  pl.fused_quant = (fmt == 1 && M <= 4 && env_int("TPPX_SKINNY_FUSEDQ", 1) != 0);
+  pl.max_units = (units + w - 1) / w;
   return pl;
 }
 
-hipError_t launch_skinny_mxfp4(const SkinnyParams& p, const SkinnyPlan& pl,
-                               bool dual, hipStream_t stream) {
-  dim3 grid(pl.grid_x, pl.grid_y);
-  if (dual) {
-    switch (pl.mg) {
-      case 1: return launch_mxfp4_t<1, 2, 4, true>(p, grid, pl.waves, stream);
-      case 2: return launch_mxfp4_t<2, 2, 2, true>(p, grid, pl.waves, stream);
-      default: return launch_mxfp4_t<4, 2, 1, true>(p, grid, pl.waves, stream);
-    }
+template <typename K>
+static hipError_t sk_launch(K kern, const DecodeParams& p, dim3 grid, int waves, size_t lds, hipStream_t stream) {
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess)
+      return e;
   }
-  if (pl.nt == 2) {
+  kern<<<grid, dim3(64 * waves), lds, stream>>>(p);
+  return hipGetLastError();
+}
+
+// groups are counted per segment by the caller with the same ntw
+hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream) {
+  p.cht = pl.max_units; // per-wave slots of activation scales in LDS
+  dim3 grid(p.groups, pl.grid_y);
+  if (pl.fused_quant) {
+    size_t lds = (size_t)pl.waves * pl.ntw * 256 * sizeof(float) + (size_t)pl.waves * pl.max_units * (4 * 256 + 16);
+    if (pl.ntw == 2)
+      return sk_launch(skinny_qint8_fq_kernel<2, 8, 16, 4>, p, grid, pl.waves, lds, stream);
+    return sk_launch(skinny_qint8_fq_kernel<1, 12, 16, 4>, p, grid, pl.waves, lds, stream);
+  }
+  size_t lds = ((size_t)pl.waves * pl.ntw * pl.mg * 256 + (size_t)pl.waves * pl.max_units * pl.mg * 16) * sizeof(float);
+  if (pl.ntw == 2) {
     switch (pl.mg) {
-      case 1: return launch_mxfp4_t<1, 2, 4, false>(p, grid, pl.waves, stream);
-      case 2: return launch_mxfp4_t<2, 2, 2, false>(p, grid, pl.waves, stream);
-      default: return launch_mxfp4_t<4, 2, 1, false>(p, grid, pl.waves, stream);
+      case 1: return sk_launch(skinny_qint8_kernel<1, 2, 4, 16, 4>, p, grid, pl.waves, lds, stream);
+      case 2: return sk_launch(skinny_qint8_kernel<2, 2, 3, 16, 8>, p, grid, pl.waves, lds, stream);
+      default: return sk_launch(skinny_qint8_kernel<4, 2, 4, 8, 8>, p, grid, pl.waves, lds, stream);
     }
   }
   switch (pl.mg) {
-    case 1: return launch_mxfp4_t<1, 1, 4, false>(p, grid, pl.waves, stream);
-    case 2: return launch_mxfp4_t<2, 1, 2, false>(p, grid, pl.waves, stream);
-    default: return launch_mxfp4_t<4, 1, 1, false>(p, grid, pl.waves, stream);
+    case 1: return sk_launch(skinny_qint8_kernel<1, 1, 8, 16, 4>, p, grid, pl.waves, lds, stream);
+    case 2: return sk_launch(skinny_qint8_kernel<2, 1, 6, 16, 4>, p, grid, pl.waves, lds, stream);
+    default: return sk_launch(skinny_qint8_kernel<4, 1, 6, 8, 8>, p, grid, pl.waves, lds, stream);
   }
 }
 
-hipError_t launch_skinny_qint8(const SkinnyParams& p, const SkinnyPlan& pl,
-                               hipStream_t stream) {
-  dim3 grid(pl.grid_x, pl.grid_y);
-  if (pl.nt == 2) {
-    switch (pl.mg) {
-      case 1: return launch_qint8_t<1, 2, 4>(p, grid, pl.waves, stream);
-      case 2: return launch_qint8_t<2, 2, 4>(p, grid, pl.waves, stream);
-      default: return launch_qint8_t<4, 2, 4>(p, grid, pl.waves, stream);
-    }
-  }
-  switch (pl.mg) {
-    case 1: return launch_qint8_t<1, 1, 4>(p, grid, pl.waves, stream);
-    case 2: return launch_qint8_t<2, 1, 4>(p, grid, pl.waves, stream);
-    default: return launch_qint8_t<4, 1, 4>(p, grid, pl.waves, stream);
-  }
+hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream) {
+  dim3 grid(p.groups, pl.grid_y);
+  size_t lds = (size_t)pl.waves * pl.ntw * 256 * sizeof(float);
+  if (dual)
+    return sk_launch(skinny_mxfp4_kernel<2, 6, 8, 4, true>, p, grid, pl.waves, lds, stream);
+  if (pl.ntw == 2)
+    return sk_launch(skinny_mxfp4_kernel<2, 6, 8, 4, false>, p, grid, pl.waves, lds, stream);
+  return sk_launch(skinny_mxfp4_kernel<1, 4, 16, 4, false>, p, grid, pl.waves, lds, stream);
 }
 
 } // namespace tppx

@@ -52,11 +52,12 @@ SIGNATURES = {
     "tppx_prepack_mxfp4": [_vp, _vp, _i64, _i64, _vp, _vp, _vp],
     "tppx_prepack_qint8": [_vp, _i64, _i64, _i64, _vp, _vp],
     "tppx_quant_act_int8": [_vp, _i64, _i64, _i64, _vp, _vp, _vp],
-    "tppx_linear_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _f32, _i32, _vp],
-    "tppx_linear_qint8": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _f32, _i32, _vp],
-    "tppx_multi_linear_mxfp4": [_vp, ctypes.POINTER(Seg), _i32, _i64, _i64, _i32, _vp],
-    "tppx_multi_linear_qint8": [_vp, _vp, _vp, ctypes.POINTER(Seg), _i32, _i64, _i64, _i64, _i32, _vp],
-    "tppx_swiglu_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
+    "tppx_linear_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _f32, _i32, _vp, _i64, _vp],
+    "tppx_linear_qint8": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _f32, _i32,
+                          _vp, _i64, _vp],
+    "tppx_multi_linear_mxfp4": [_vp, ctypes.POINTER(Seg), _i32, _i64, _i64, _i32, _vp, _i64, _vp],
+    "tppx_multi_linear_qint8": [_vp, _vp, _vp, ctypes.POINTER(Seg), _i32, _i64, _i64, _i64, _i32, _vp, _i64, _vp],
+    "tppx_swiglu_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp],
 }
 
 _lib = None
@@ -95,6 +96,26 @@ def ptr(t):
 
 def stream_of(t):
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+WORKSPACE_BYTES = 32 << 20
+_workspaces = {}
+
+
+def workspace(t):
+    """Zero-initialised split-K scratch of `t`'s device (see include/tppx.h).
+    One buffer per device: ops that use it must be ordered with respect to
+    each other (same stream, or streams ordered by events / graph replay),
+    which is how the single-caller reference behaves as well."""
+    key = t.device.index
+    ws = _workspaces.get(key)
+    if ws is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise TppxError(EINVAL, "first call on this device happens inside graph capture: run the op once "
+                                    "eagerly before capturing so that its workspace exists")
+        ws = torch.zeros(WORKSPACE_BYTES, dtype=torch.uint8, device=t.device)
+        _workspaces[key] = ws
+    return ws
 
 
 def require_gpu(t, what):

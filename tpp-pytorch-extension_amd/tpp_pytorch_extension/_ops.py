@@ -306,17 +306,18 @@ def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None
     post_in2 = _prep_post(post_in2, M, N, "second post-op input", x.device)
     qn, sn = weight.native()
     st = _lib.stream_of(x)
+    ws = _lib.workspace(x)
     if weight._qscheme == QSCHEME_MXFP:
         _lib.check(L.tppx_linear_mxfp4(x.data_ptr(), qn.data_ptr(), sn.data_ptr(), _lib.ptr(bias),
                                        _lib.ptr(post_in), _lib.ptr(post_in2), y.data_ptr(), M, N, K,
-                                       post, post_scale, flags, st))
+                                       post, post_scale, flags, ws.data_ptr(), ws.numel(), st))
     else:
         qbs = weight.block_size
         xq, sa = _qint8_scratch(x, M, K, qbs)
         _lib.check(L.tppx_linear_qint8(x.data_ptr(), xq.data_ptr(), sa.data_ptr(), qn.data_ptr(),
                                        sn.data_ptr(), _lib.ptr(bias), _lib.ptr(post_in),
                                        _lib.ptr(post_in2), y.data_ptr(), M, N, K, qbs, post,
-                                       post_scale, flags, st))
+                                       post_scale, flags, ws.data_ptr(), ws.numel(), st))
     return y
 
 
@@ -392,13 +393,14 @@ def qkv_gemm(input, weights, biases):
     if M == 0:
         return outs
     st = _lib.stream_of(x)
+    ws = _lib.workspace(x)
     if scheme == QSCHEME_MXFP:
-        _lib.check(L.tppx_multi_linear_mxfp4(x.data_ptr(), segs, n, M, K, 0, st))
+        _lib.check(L.tppx_multi_linear_mxfp4(x.data_ptr(), segs, n, M, K, 0, ws.data_ptr(), ws.numel(), st))
     else:
         qbs = weights[0].block_size
         xq, sa = _qint8_scratch(x, M, K, qbs)
         _lib.check(L.tppx_multi_linear_qint8(x.data_ptr(), xq.data_ptr(), sa.data_ptr(), segs, n, M, K,
-                                             qbs, 0, st))
+                                             qbs, 0, ws.data_ptr(), ws.numel(), st))
     return outs
 
 
@@ -420,8 +422,10 @@ def swiglu_gate_up(input, w_gate, w_up, b_gate=None, b_up=None):
     bu = _prep_bias(b_up, N, x.device)
     qg, sg = w_gate.native()
     qu, su = w_up.native()
+    ws = _lib.workspace(x)
     _lib.check(L.tppx_swiglu_mxfp4(x.data_ptr(), qg.data_ptr(), sg.data_ptr(), _lib.ptr(bg), qu.data_ptr(),
-                                   su.data_ptr(), _lib.ptr(bu), y.data_ptr(), M, N, K, 0, _lib.stream_of(x)))
+                                   su.data_ptr(), _lib.ptr(bu), y.data_ptr(), M, N, K, 0, ws.data_ptr(),
+                                   ws.numel(), _lib.stream_of(x)))
     return y
 
 
