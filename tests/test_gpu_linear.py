@@ -159,3 +159,38 @@ def test_module_api_and_errors():
         torch.ops.tpp_llm.fc_plain(x, lin.weight, torch.Tensor(), -1, [])  # fp32 activations
     e = torch.ops.tpp_llm.fc_plain(torch.empty(0, 256, dtype=torch.bfloat16).cuda(), lin.weight, torch.Tensor(), -1, [])
     assert e.shape == (0, 128)
+
+
+@pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])
+@pytest.mark.parametrize("M", [65, 200, 256])
+def test_prefill_tiled_small(fmt, M):
+    """More than 64 rows takes the LDS-tiled kernels; N = 384 leaves the last
+    128-wide block half empty, M = 65 / 200 leave the last row block ragged."""
+    _run(fmt, M, 384, 1024, "add", True, 500 + M)
+
+
+@pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])
+def test_prefill_tiled_m2048(fmt):
+    """Prefill row count of BASELINE config 4 (M = 2048) on a layer slice the
+    CPU oracle finishes in seconds; also compared with the reference's chunked
+    bf16 re-rounding schedule (K = 8192 > 4096 -> two chunks for MXFP4)."""
+    y, ref, s, ctx = _run(fmt, 2048, 256, 8192, "none", True, 600)
+    qw, q_or, s_or, x, bias, in1, in2, scale = ctx
+    lin = O.linear_mxfp4 if fmt == "mxfp4" else O.linear_qint8
+    faithful = lin(t2bits(x), q_or, s_or, t2bits(bias), O.POST_NONE, None, None, 1.0, O.MODE_FAITHFUL)
+    st = err_stats(t2bits(y), faithful)
+    bound = 2.0 ** -9 * np.sqrt(2 if fmt == "mxfp4" else 8192 // 256)
+    assert st["rel_l2"] <= bound, st["rel_l2"]
+
+
+def test_prefill_qkv_and_swiglu_equal_composition():
+    ops = _ops()
+    K, M = 1024, 130
+    ws = [_make("mxfp4", n, K, 80 + i)[0] for i, n in enumerate((256, 128, 128))]
+    x = randn_bf16((M, K), 1.0, 90).cuda()
+    outs = torch.ops.tpp_llm.qkv_gemm(x, ws, [torch.Tensor()] * 3)
+    for w, o in zip(ws, outs):
+        assert torch.equal(o, ops.fc_plain(x, w, None))
+    wg, wu = _make("mxfp4", 512, K, 91)[0], _make("mxfp4", 512, K, 92)[0]
+    fused = ops.swiglu_gate_up(x, wg, wu)
+    assert torch.equal(fused, ops.fc_mul(x, wu, None, ops.fc_silu(x, wg, None)))

@@ -118,6 +118,38 @@ static void bind_workspace(DecodeParams& p, const DecodePlan& pl, void* ws) {
   p.part = (float*)ws;
 }
 
+static const int64_t TILED_MIN_M = 65; // more rows than the decode kernels cover in one block row
+
+static bool want_tiled(int64_t M, int flags) {
+  if (flags & TPPX_FLAG_FORCE_SKINNY)
+    return false;
+  if (flags & TPPX_FLAG_FORCE_TILED)
+    return true;
+  return M >= env_int("TPPX_TILED_MIN_M", (int)TILED_MIN_M);
+}
+
+static TiledParams tiled_from_seg(const DecodeParams& p, int i) {
+  TiledParams t;
+  memset(&t, 0, sizeof(t));
+  const DecodeSeg& s = p.seg[i];
+  t.x = p.x;
+  t.xq = p.xq;
+  t.sa = p.sa;
+  t.qw = s.qw;
+  t.sw = s.sw;
+  t.bias = s.bias;
+  t.post_in = s.post_in;
+  t.post_in2 = s.post_in2;
+  t.y = s.y;
+  t.M = p.M;
+  t.N = s.N;
+  t.K = p.K;
+  t.tiles = s.tiles;
+  t.post_op = s.post_op;
+  t.post_scale = s.post_scale;
+  return t;
+}
+
 static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n_segs,
                      int64_t M, int64_t K, int flags, bool dual, void* ws, int64_t ws_bytes,
                      hipStream_t stream) {
@@ -139,6 +171,21 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
   p.units = (int)(K / 128);
   p.tpb = 1;
   p.S = 1;
+  if (want_tiled(M, flags)) {
+    // prefill shapes: one LDS-tiled launch per GEMM of the group; the fused
+    // gate/up pair becomes silu(gate) followed by up * gate (same rounding)
+    for (int i = 0; i < n_segs; i++) {
+      TiledParams t = tiled_from_seg(p, i);
+      if (dual) {
+        t.post_op = i == 0 ? TPPX_POST_SILU : TPPX_POST_MUL;
+        t.post_in = i == 0 ? nullptr : (const uint16_t*)segs[0].y;
+      }
+      rc = check_hip(launch_tiled_mxfp4(t, stream), who);
+      if (rc)
+        return rc;
+    }
+    return TPPX_OK;
+  }
   if (M <= 16 && env_int("TPPX_MXFP4_SPLITK", 0) == 0) {
     // GEMV class: K reduction inside the workgroup
     SkinnyPlan sp = plan_skinny(0, M, p.total_tiles, p.units, dual);
@@ -175,6 +222,21 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
   p.K = (int)K;
   p.units = (int)(K / qbs);
   p.tpb = (int)(qbs / 64);
+  if (want_tiled(M, flags) && qbs % 128 == 0) {
+    if (x) {
+      rc = tppx_quant_act_int8(x, M, K, qbs, xq, sa, stream);
+      if (rc)
+        return rc;
+    }
+    for (int i = 0; i < n_segs; i++) {
+      TiledParams t = tiled_from_seg(p, i);
+      t.qbs = (int)qbs;
+      rc = check_hip(launch_tiled_qint8(t, stream), who);
+      if (rc)
+        return rc;
+    }
+    return TPPX_OK;
+  }
   const int force = env_int("TPPX_QINT8_SPLITK", -1);
   if (force == 1 || (force != 0 && M > 16)) {
     // more than one MFMA row group: activations shared through LDS, K split

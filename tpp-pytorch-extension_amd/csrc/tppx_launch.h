@@ -52,6 +52,27 @@ struct SkinnyPlan {
   bool fused_quant; // QINT8, M <= 4: activations quantised inside the GEMM kernel
 };
 
+// one GEMM on the LDS-tiled (prefill) kernels
+struct TiledParams {
+  const void* x;   // bf16 [M][K]           (MXFP4)
+  const void* xq;  // int8 [M][K]           (QINT8)
+  const float* sa; // f32  [M][K/qbs]       (QINT8)
+  const void* qw;
+  const void* sw;
+  const uint16_t* bias;
+  const uint16_t* post_in;
+  const uint16_t* post_in2;
+  uint16_t* y;
+  int M, N, K;
+  int tiles; // N / 16
+  int qbs;
+  int post_op;
+  float post_scale;
+};
+
+hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream);
+hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream);
+
 int env_int(const char* name, int dflt);
 
 SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual);

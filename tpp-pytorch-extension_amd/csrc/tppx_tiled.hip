@@ -1,2 +1,332 @@
-// placeholder until the LDS-tiled prefill kernels land
+// Prefill-shape (large M) LDS-tiled MFMA kernels.
+//
+// Workgroup tile 128 (M) x 128 (N), 4 waves in a 2 x 2 grid, each wave 64 x 64
+// = 4 x 4 MFMA tiles of 16 x 16.  Per K step of 128 input channels:
+//   A (activations): global -> registers -> LDS, stored in MFMA operand order
+//     so that a wave-wide ds_read_b128 is lane-contiguous (conflict free); two
+//     LDS buffers, the global loads of step k+1 are in flight while step k is
+//     multiplied.
+//   B (weights): the native 1 KiB tiles ARE the MFMA operand layout, so every
+//     wave loads its four channel tiles straight from global/L2 into registers
+//     (one 128-bit load per lane and tile, next step prefetched) - no LDS, no
+//     re-layout.  MXFP4 codes are expanded to bf16 in registers with the
+//     hardware E8M0-scaled convert (exact) and multiplied with
+//     v_mfma_f32_16x16x32_bf16; QINT8 uses v_mfma_i32_16x16x64_i8 with exact
+//     int32 sums per K block and an fp32 scale-and-accumulate.
+// Workgroup ids are remapped so that the workgroups of one XCD (ids equal
+// mod 8) walk consecutive M blocks of the same N block: the weight tiles of
+// that N block stay in the XCD's L2.
+//
+// MFMA operand convention (A = activations, B = weights):
+//   lane l supplies row/col (l & 15) and K group (l >> 4);
+//   result register r of lane l is D[m = (l >> 4) * 4 + r][n = l & 15].
 #include "tppx_common.h"
+#include "tppx_launch.h"
+
+namespace tppx {
+
+__device__ __forceinline__ bf16x8 tl_cvt_fp4x8(uint32_t codes, float scale) {
+  bf16x2 c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 0);
+  bf16x2 c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 1);
+  bf16x2 c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 2);
+  bf16x2 c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 3);
+  bf16x8 w;
+  w[0] = c0[0]; w[1] = c0[1]; w[2] = c1[0]; w[3] = c1[1];
+  w[4] = c2[0]; w[5] = c2[1]; w[6] = c3[0]; w[7] = c3[1];
+  return w;
+}
+
+// XCD-aware tile order: returns (bm, bn) of this workgroup.
+__device__ __forceinline__ void tile_of_block(int MB, int NB, int& bm, int& bn) {
+  int id = blockIdx.x;
+  const int T = MB * NB;
+  if ((T & 7) == 0) {
+    const int per = T >> 3;
+    id = (id & 7) * per + (id >> 3);
+  }
+  bm = id % MB;
+  bn = id / MB;
+}
+
+template <typename Acc>
+__device__ __forceinline__ void tiled_epilogue(const TiledParams& p, Acc& acc, int m_base, int tile_base) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int nt = 0; nt < 4; nt++) {
+    const int tile = tile_base + nt;
+    if (tile >= p.tiles)
+      continue;
+    const int n = tile * 16 + (lane & 15);
+    const float b = p.bias ? bf16_bits_to_f32(p.bias[n]) : 0.0f;
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int m = m_base + mt * 16 + (lane >> 4) * 4 + r;
+        if (m < p.M) {
+          const int64_t o = (int64_t)m * p.N + n;
+          uint32_t in1 = p.post_in ? p.post_in[o] : 0u;
+          uint32_t in2 = p.post_in2 ? p.post_in2[o] : 0u;
+          p.y[o] = (uint16_t)apply_post_bits(acc[mt][nt][r] + b, p.post_op, in1, in2, p.post_scale);
+        }
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// MXFP4, bf16 activations (exact reference numerics, fp32 accumulation over K)
+// LDS A layout per buffer: [mt 8][j 4][lane 64] x 16 B  (32 KiB)
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+tiled_mxfp4_kernel(const TiledParams p) {
+  extern __shared__ __align__(16) uint8_t tl_lds[];
+  bf16x8* As = reinterpret_cast<bf16x8*>(tl_lds); // 2 buffers x 2048 slots
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int MB = (p.M + 127) >> 7, NB = (p.tiles + 7) >> 3;
+  int bm, bn;
+  tile_of_block(MB, NB, bm, bn);
+  const int KT = p.K >> 7; // K steps of 128 = native tiles along K
+  const int m_wg = bm * 128;
+  const int tile_base = bn * 8 + wn * 4;
+
+  const i32x4* wq[4];
+  const uint8_t* wsc[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; nt++) {
+    const int64_t t = min(tile_base + nt, p.tiles - 1);
+    wq[nt] = reinterpret_cast<const i32x4*>(p.qw) + t * KT * 64 + lane;
+    wsc[nt] = reinterpret_cast<const uint8_t*>(p.sw) + t * KT * 64 + lane;
+  }
+  // A staging: thread handles LDS slots tid + 256*q  ->  (r16, g, j = wave, mt = q)
+  const uint16_t* xb = reinterpret_cast<const uint16_t*>(p.x);
+  const uint16_t* arow[8];
+#pragma unroll
+  for (int q = 0; q < 8; q++) {
+    const int m = min(m_wg + q * 16 + (tid & 15), p.M - 1);
+    arow[q] = xb + (int64_t)m * p.K + ((tid >> 4) & 3) * 32 + wave * 8;
+  }
+
+  bf16x8 areg[8];
+  i32x4 breg[4];
+  uint32_t bsc[4];
+  auto load_a = [&](int ks) {
+#pragma unroll
+    for (int q = 0; q < 8; q++)
+      areg[q] = *reinterpret_cast<const bf16x8*>(arow[q] + ks * 128);
+  };
+  auto load_b = [&](int ks) {
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+      breg[nt] = wq[nt][(int64_t)ks * 64];
+      bsc[nt] = wsc[nt][(int64_t)ks * 64];
+    }
+  };
+  auto store_a = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < 8; q++)
+      As[buf * 2048 + q * 256 + tid] = areg[q];
+  };
+
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++)
+      acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  load_a(0);
+  load_b(0);
+  store_a(0);
+  __syncthreads();
+  for (int ks = 0; ks < KT; ks++) {
+    const int buf = ks & 1;
+    i32x4 bcur[4];
+    float sc[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+      bcur[nt] = breg[nt];
+      sc[nt] = e8m0_to_f32(bsc[nt]);
+    }
+    if (ks + 1 < KT) {
+      load_a(ks + 1);
+      load_b(ks + 1);
+    }
+    const bf16x8* Ab = As + buf * 2048 + (wm * 4) * 256 + lane;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      bf16x8 a[4], b[4];
+#pragma unroll
+      for (int mt = 0; mt < 4; mt++)
+        a[mt] = Ab[mt * 256 + j * 64];
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+        b[nt] = tl_cvt_fp4x8((uint32_t)bcur[nt][j], sc[nt]);
+#pragma unroll
+      for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[mt], b[nt], acc[mt][nt], 0, 0, 0);
+    }
+    if (ks + 1 < KT)
+      store_a(buf ^ 1);
+    __syncthreads();
+  }
+  tiled_epilogue(p, acc, m_wg + wm * 64, tile_base);
+}
+
+// ---------------------------------------------------------------------------
+// QINT8 (W8A8): activations pre-quantised (int8 [M][K], f32 [M][K/qbs]).
+// K step = 128 = two native tiles; LDS A layout per buffer:
+// [mt 8][t 2][lane 64] x 16 B (16 KiB) + the activation scales of the step's
+// K block for the 128 rows.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+tiled_qint8_kernel(const TiledParams p) {
+  extern __shared__ __align__(16) uint8_t tl_lds[];
+  i32x4* As = reinterpret_cast<i32x4*>(tl_lds);                 // 2 x 1024 slots
+  float* sa_s = reinterpret_cast<float*>(tl_lds + 2 * 1024 * 16); // 2 x 128
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int MB = (p.M + 127) >> 7, NB = (p.tiles + 7) >> 3;
+  int bm, bn;
+  tile_of_block(MB, NB, bm, bn);
+  const int KS = p.K >> 7;        // K steps of 128
+  const int KT = p.K >> 6;        // native tiles along K
+  const int SPB = p.qbs >> 7;     // steps per K block (qbs is a multiple of 128 here)
+  const int NBK = p.K / p.qbs;
+  const int m_wg = bm * 128;
+  const int tile_base = bn * 8 + wn * 4;
+
+  const i32x4* wq[4];
+  const float* wsc[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; nt++) {
+    const int64_t t = min(tile_base + nt, p.tiles - 1);
+    wq[nt] = reinterpret_cast<const i32x4*>(p.qw) + t * KT * 64 + lane;
+    wsc[nt] = reinterpret_cast<const float*>(p.sw) + t * NBK * 16 + (lane & 15);
+  }
+  // A staging: slots tid + 256*q -> (r16, g, t = wave & 1, mt = 2*q + (wave >> 1))
+  const int8_t* xq = reinterpret_cast<const int8_t*>(p.xq);
+  const int8_t* arow[4];
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    const int mt = q * 2 + (wave >> 1);
+    const int m = min(m_wg + mt * 16 + (tid & 15), p.M - 1);
+    arow[q] = xq + (int64_t)m * p.K + (wave & 1) * 64 + ((tid >> 4) & 3) * 16;
+  }
+  const int sa_row = min(m_wg + (tid & 127), p.M - 1);
+
+  i32x4 areg[4], breg[2][4];
+  float sareg = 0.f;
+  auto load_a = [&](int ks) {
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+      areg[q] = *reinterpret_cast<const i32x4*>(arow[q] + ks * 128);
+    if (ks % SPB == 0 && tid < 128)
+      sareg = p.sa[(int64_t)sa_row * NBK + ks / SPB];
+  };
+  auto load_b = [&](int ks) {
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+        breg[t][nt] = wq[nt][(int64_t)(ks * 2 + t) * 64];
+  };
+  auto store_a = [&](int ks, int buf) {
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+      As[buf * 1024 + q * 256 + tid] = areg[q];
+    if (ks % SPB == 0 && tid < 128)
+      sa_s[((ks / SPB) & 1) * 128 + tid] = sareg;
+  };
+
+  f32x4 facc[4][4];
+  i32x4 iacc[4][4];
+#pragma unroll
+  for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+      facc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      iacc[mt][nt] = i32x4{0, 0, 0, 0};
+    }
+
+  load_a(0);
+  load_b(0);
+  store_a(0, 0);
+  __syncthreads();
+  for (int ks = 0; ks < KS; ks++) {
+    const int buf = ks & 1;
+    i32x4 bcur[2][4];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+        bcur[t][nt] = breg[t][nt];
+    if (ks + 1 < KS) {
+      load_a(ks + 1);
+      load_b(ks + 1);
+    }
+    // slot = (mt*2 + t)*64 + lane with mt = wm*4 + i
+    const i32x4* Ab = As + buf * 1024 + (wm * 4) * 128 + lane;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      i32x4 a[4];
+#pragma unroll
+      for (int mt = 0; mt < 4; mt++)
+        a[mt] = Ab[mt * 128 + t * 64];
+#pragma unroll
+      for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+          iacc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[mt], bcur[t][nt], iacc[mt][nt], 0, 0, 0);
+    }
+    if ((ks + 1) % SPB == 0) { // K block complete: scale and fold into fp32
+      const int b = ks / SPB;
+      const float* sab = sa_s + (b & 1) * 128 + wm * 64 + (lane >> 4) * 4;
+      float swv[4];
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+        swv[nt] = wsc[nt][b * 16];
+#pragma unroll
+      for (int mt = 0; mt < 4; mt++) {
+        const f32x4 sav = *reinterpret_cast<const f32x4*>(sab + mt * 16);
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            facc[mt][nt][r] = fmaf((float)iacc[mt][nt][r], sav[r] * swv[nt], facc[mt][nt][r]);
+            iacc[mt][nt][r] = 0;
+          }
+      }
+    }
+    if (ks + 1 < KS)
+      store_a(ks + 1, buf ^ 1);
+    __syncthreads();
+  }
+  tiled_epilogue(p, facc, m_wg + wm * 64, tile_base);
+}
+
+hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream) {
+  const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
+  const size_t lds = 2 * 2048 * 16;
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_mxfp4_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess)
+      return e;
+    attr_done = true;
+  }
+  tiled_mxfp4_kernel<<<dim3(MB * NB), dim3(256), lds, stream>>>(p);
+  return hipGetLastError();
+}
+
+hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream) {
+  const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
+  const size_t lds = 2 * 1024 * 16 + 2 * 128 * sizeof(float);
+  tiled_qint8_kernel<<<dim3(MB * NB), dim3(256), lds, stream>>>(p);
+  return hipGetLastError();
+}
+
+} // namespace tppx
