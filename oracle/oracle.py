@@ -128,6 +128,20 @@ def e2m1_decode(c):
     return lib().orc_e2m1_decode(int(c))
 
 
+def e2m1_encode_array(v):
+    v = _c(v, np.float32)
+    out = np.empty(v.shape, np.int32)
+    lib().orc_e2m1_encode_n(_p(v), _p(out), _c_i64(v.size))
+    return out.astype(np.int64)
+
+
+def mx_quant_scale_of_amax_array(a):
+    a = _c(a, np.float32)
+    out = np.empty(a.shape, np.float32)
+    lib().orc_mx_quant_scale_of_amax_n(_p(a), _p(out), _c_i64(a.size))
+    return out
+
+
 E2M1_TABLE = np.array(
     [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0],
     np.float32,

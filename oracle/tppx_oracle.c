@@ -121,10 +121,20 @@ ORC_API float orc_e2m1_decode(int code) {
  * Follows quantize_elemwise(v, 3, 2, 6.0, rd_even, true, true)
  * (mxfp_quant.h:240-300) plus the value->code chain of MxFP4Quant::quantize
  * (qtypes.cpp:87-131; "scaled_out == 0.0" catches -0 before the -0.0 branch;
- * a NaN matches no branch and leaves code 0). */
+ * a NaN matches no branch and leaves code 0, see below). */
 ORC_API int orc_e2m1_encode(float v) {
-  if (v != v)
+  if (v != v) {
+    /* A NaN whose mantissa rounds to zero at 2 bits turns into Inf inside
+     * quantize_elemwise and saturates to +-6; every other NaN matches no
+     * branch of the value->code chain and leaves 0.  (Only a signalling NaN
+     * can get here with such a mantissa, and the division by the block scale
+     * that precedes this step quiets it, so the quantiser itself always
+     * yields 0 for a NaN element.) */
+    uint32_t u = f32_bits(v);
+    if ((u & 0x7fffffu) <= 0x200000u)
+      return 7 | (int)((u >> 31) << 3);
     return 0;
+  }
   float a = fabsf(v);
   int c;
   if (a <= 0.25f)
@@ -146,6 +156,16 @@ ORC_API int orc_e2m1_encode(float v) {
   if (c != 0 && (f32_bits(v) >> 31))
     c |= 8;
   return c;
+}
+
+/* array forms (bit patterns reach the scalar functions unchanged) */
+ORC_API void orc_e2m1_encode_n(const float* v, int32_t* codes, int64_t n) {
+  for (int64_t i = 0; i < n; i++)
+    codes[i] = orc_e2m1_encode(v[i]);
+}
+ORC_API void orc_mx_quant_scale_of_amax_n(const float* amax, float* scale, int64_t n) {
+  for (int64_t i = 0; i < n; i++)
+    scale[i] = orc_mx_quant_scale(orc_mx_scale_byte(amax[i]));
 }
 
 /* Quantise one MX block given its amax: returns the scale byte, fills codes.

@@ -1,0 +1,186 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every
+entry point include/tppx.h declares, arguments are validated before any HIP
+call (error codes, never a crash or exit), and the Python drop-in layer
+(blocked layouts, module classes, helper names) behaves like the reference's.
+"""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _lib():
+    import tpp_pytorch_extension  # noqa: F401
+    from tpp_pytorch_extension import _lib
+    return _lib
+
+
+def test_header_symbols_are_exported_and_bound():
+    L = _lib()
+    hdr = open(os.path.join(ROOT, "include", "tppx.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    declared = set(re.findall(r"\b(tppx_[a-z0-9_]+)\s*\(", hdr))
+    assert len(declared) >= 14
+    lib = L.lib()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in tppx.h but not exported"
+    assert declared == set(L.SIGNATURES), "ctypes signatures and tppx.h disagree"
+    assert lib.tppx_version() == 100
+
+
+def test_seg_struct_matches_header_layout():
+    L = _lib()
+    # 6 pointers, int64, int32, float
+    assert ctypes.sizeof(L.Seg) == 6 * 8 + 8 + 4 + 4
+    assert L.Seg.N.offset == 48 and L.Seg.post_op.offset == 56 and L.Seg.post_scale.offset == 60
+
+
+def test_argument_validation_without_gpu():
+    L = _lib()
+    lib = L.lib()
+    A = 1 << 20  # a fake, 16-byte aligned "device pointer": validation must reject before touching it
+
+    def err():
+        return lib.tppx_last_error().decode()
+
+    # null pointers
+    assert lib.tppx_linear_mxfp4(None, A, A, None, None, None, A, 1, 32, 128, 0, 1.0, 0, None, 0, None) == L.EINVAL
+    assert "null" in err()
+    assert lib.tppx_linear_qint8(A, None, A, A, A, None, None, None, A, 1, 16, 256, 256, 0, 1.0, 0, None, 0, None) == L.EINVAL
+    # misaligned
+    assert lib.tppx_linear_mxfp4(A + 2, A, A, None, None, None, A, 1, 32, 128, 0, 1.0, 0, None, 0, None) == L.EINVAL
+    assert "aligned" in err()
+    # shapes: M = 0, K not a multiple of 64, N not a multiple of 32 / 16, block size mismatch
+    assert lib.tppx_linear_mxfp4(A, A, A, None, None, None, A, 0, 32, 128, 0, 1.0, 0, None, 0, None) == L.ESHAPE
+    assert lib.tppx_linear_mxfp4(A, A, A, None, None, None, A, 1, 32, 100, 0, 1.0, 0, None, 0, None) == L.ESHAPE
+    assert lib.tppx_linear_mxfp4(A, A, A, None, None, None, A, 1, 48, 128, 0, 1.0, 0, None, 0, None) == L.ESHAPE
+    assert lib.tppx_linear_mxfp4(A, A, A, None, None, None, A, 1, 32, 192, 0, 1.0, 0, None, 0, None) == L.EUNSUPPORTED
+    assert lib.tppx_linear_qint8(A, A, A, A, A, None, None, None, A, 1, 24, 256, 256, 0, 1.0, 0, None, 0, None) == L.ESHAPE
+    assert lib.tppx_linear_qint8(A, A, A, A, A, None, None, None, A, 1, 16, 256, 192, 0, 1.0, 0, None, 0, None) == L.ESHAPE
+    assert "block size" in err()
+    # post-op id and its inputs
+    assert lib.tppx_linear_mxfp4(A, A, A, None, None, None, A, 1, 32, 128, 9, 1.0, 0, None, 0, None) == L.EINVAL
+    assert lib.tppx_linear_mxfp4(A, A, A, None, None, None, A, 1, 32, 128, L.POST_MUL, 1.0, 0, None, 0, None) == L.EINVAL
+    assert "post_in" in err()
+    assert lib.tppx_linear_mxfp4(A, A, A, None, A, None, A, 1, 32, 128, L.POST_ADD2_SCALE, 1.0, 0, None, 0, None) == L.EINVAL
+    # flags and workspace
+    assert lib.tppx_linear_mxfp4(A, A, A, None, None, None, A, 1, 32, 128, 0, 1.0, 64, None, 0, None) == L.EINVAL
+    assert lib.tppx_linear_mxfp4(A, A, A, None, None, None, A, 1, 32, 128, 0, 1.0, 3, None, 0, None) == L.EINVAL
+    assert lib.tppx_linear_mxfp4(A, A, A, None, None, None, A, 1, 32, 128, 0, 1.0, 0, None, 4096, None) == L.EINVAL
+    # fused groups
+    segs = (L.Seg * 5)()
+    assert lib.tppx_multi_linear_mxfp4(A, segs, 5, 1, 128, 0, None, 0, None) == L.EINVAL
+    assert lib.tppx_multi_linear_mxfp4(A, segs, 0, 1, 128, 0, None, 0, None) == L.EINVAL
+    # quantizers
+    assert lib.tppx_quantize_mxfp4(A, 0, 48, 128, 16, 64, 2, A, A, None) == L.ESHAPE
+    assert lib.tppx_quantize_mxfp4(A, 7, 64, 128, 16, 64, 2, A, A, None) == L.EINVAL
+    assert lib.tppx_quantize_qint8(A, 1, 64, 128, 16, 64, 2, 96, A, A, None) == L.ESHAPE
+    assert lib.tppx_quant_act_int8(A, 1, 100, 256, A, A, None) == L.ESHAPE
+    assert lib.tppx_prepack_mxfp4(A, A, 64, 192, A, A, None) == L.ESHAPE
+    assert lib.tppx_dequantize_qint8(None, A, 16, 256, 256, A, None) == L.EINVAL
+
+
+def test_python_layer_fails_loudly_without_gpu():
+    L = _lib()
+    from tpp_pytorch_extension._C import _qtype
+    if torch.cuda.is_available():
+        pytest.skip("checks the no-GPU behaviour")
+    w = torch.randn(64, 128).to(torch.bfloat16).view(4, 16, 2, 32, 2).permute(0, 2, 3, 1, 4).contiguous()
+    with pytest.raises(L.TppxError):
+        _qtype.remap_and_quantize_mxfp4(w)
+    with pytest.raises(L.TppxError):
+        torch.ops.tpp_llm.fc_plain(torch.randn(2, 128), torch.randn(64, 128), torch.Tensor(), -1, [])
+
+
+def test_reference_names_are_importable():
+    import tpp_pytorch_extension as tpx
+    from tpp_pytorch_extension import qtypes, nn
+    from tpp_pytorch_extension._C import _qtype, _fused_llm_infer
+    from tpp_pytorch_extension.llm import llm_common
+    from tpp_pytorch_extension.utils import blocked_layout
+    for n in ("quantize_mxfp", "quantize_mxfp4", "quantize_int8sym", "quantize_int4sym", "create_qtensor_int8sym",
+              "create_qtensor_int2sym", "q_per_block_scales", "q_per_block_pack_size", "q_per_block_block_size",
+              "q_per_block_axis", "remap_and_quantize_mxfp4", "remap_and_quantize_qint8",
+              "remap_and_quantize_qint2_intlv", "fix_vnni"):
+        assert callable(getattr(_qtype, n)), n
+    for n in ("get_qval", "get_scales", "get_axis", "get_block_size", "q_per_block_qval"):
+        assert callable(getattr(qtypes, n)), n
+    assert callable(_fused_llm_infer.fc_plain) and callable(nn.fc_plain) and callable(llm_common.fc_plain)
+    for n in ("BlockedLinear", "FixLinear"):
+        assert hasattr(llm_common, n)
+    for n in ("TppLinear", "BlockedWeight", "FixLinear", "OptimizeForLinear"):
+        assert hasattr(nn, n)
+    for n in ("BlockingManager", "BlockedParameter", "BlockedModule"):
+        assert hasattr(blocked_layout, n)
+    assert tpx.get_vnni_blocking(torch.bfloat16) == 2 and tpx.get_vnni_blocking(torch.float32) == 1
+    for op in ("fc_plain", "fc_add", "fc_silu", "fc_mul", "qkv_gemm", "swiglu_mlp"):
+        assert hasattr(torch.ops.tpp_llm, op)
+
+
+def test_blocking_manager_matches_index_formula():
+    from tpp_pytorch_extension.utils.blocked_layout import BlockingManager
+    from tpp_pytorch_extension.nn import BlockedWeight
+    N, K = 48, 128
+    W = torch.arange(N * K, dtype=torch.float32).view(N, K)
+    bm = BlockingManager(W.shape, blocking_factors=[16, [32, 2]], permute=[0, 2, 3, 1, 4])
+    Wb = bm.block(W)
+    assert list(Wb.shape) == [3, 2, 32, 16, 2] == bm.blocked_shape
+    for (n1, c1, c2, k2, c3) in [(0, 0, 0, 0, 0), (2, 1, 31, 15, 1), (1, 0, 7, 3, 1)]:
+        assert Wb[n1, c1, c2, k2, c3] == W[n1 * 16 + k2, c1 * 64 + c2 * 2 + c3]
+    assert torch.equal(bm.unblock(Wb), W)
+    assert torch.equal(BlockedWeight(W, 16, 64, torch.bfloat16), Wb.to(torch.bfloat16))
+    assert torch.equal(BlockedWeight(W, 16, 64, torch.float32), W.view(3, 16, 2, 64).permute(0, 2, 3, 1))
+    with pytest.raises(AssertionError):
+        BlockingManager((50, 128), blocking_factors=[16, 64], permute=[0, 2, 3, 1])
+
+
+def test_blocked_module_state_dict_round_trip():
+    """BlockedModule saves BlockedParameters in the plain layout and re-blocks
+    them on load (reference: blocked_layout.py:309-364)."""
+    from tpp_pytorch_extension.utils.blocked_layout import BlockedModule, BlockedParameter
+
+    class Mod(BlockedModule):
+        def __init__(self):
+            super().__init__()
+            self.w = BlockedParameter(torch.arange(64 * 128, dtype=torch.float32).view(64, 128))
+            self.w.set_blocking_param(([16, 64], [0, 2, 3, 1]))
+
+    m = Mod()
+    plain = m.w.data.clone()
+    m.w.block()
+    assert list(m.w.shape) == [4, 2, 64, 16] and m.w.is_blocked()
+    sd = m.state_dict()
+    assert list(sd["w"].shape) == [64, 128] and torch.equal(sd["w"], plain)
+    assert m.w.is_blocked()
+    m2 = Mod()
+    m2.w.block()
+    m2.load_state_dict({"w": plain * 2})
+    assert m2.w.is_blocked() and list(m2.w.shape) == [4, 2, 64, 16]
+    m2.w.unblock()
+    assert torch.equal(m2.w.data, plain * 2)
+
+
+def test_fix_linear_unquantized_keeps_blocked_weight():
+    from tpp_pytorch_extension.llm.llm_common import FixLinear, BlockedLinear
+    torch.manual_seed(1)
+    lin = torch.nn.Linear(128, 64, bias=True)
+    W = lin.weight.data.clone()
+    FixLinear(lin, 16, 64, torch.float32)
+    assert isinstance(lin, BlockedLinear) and list(lin.weight.shape) == [4, 2, 64, 16]
+    assert torch.equal(lin.weight.data, W.view(4, 16, 2, 64).permute(0, 2, 3, 1))
+    with pytest.raises(ValueError):
+        FixLinear(torch.nn.Linear(64, 64), 16, 64, torch.bfloat16, weight_dtype="nf4")
+
+
+def test_fix_vnni_and_block_size_rule():
+    from tpp_pytorch_extension import _ops
+    t = torch.arange(2 * 2 * 8 * 4 * 4, dtype=torch.float32).view(2, 2, 8, 4, 4).to(torch.bfloat16)
+    v2 = _ops.fix_vnni(t)
+    assert list(v2.shape) == [2, 2, 16, 4, 2]
+    assert v2[1, 0, 5, 2, 1] == t[1, 0, 2, 2, 3]  # c2'=5 -> c2=2, half 1 -> c3 = 2 + 1
+    assert _ops.qint8_block_size_for(4096) == 256 and _ops.qint8_block_size_for(11008) == 256
+    assert _ops.qint8_block_size_for(192) == 64 and _ops.qint8_block_size_for(384) == 128

@@ -1,0 +1,267 @@
+"""Pins the CPU oracle (oracle/tppx_oracle.c) before anything is compared with it.
+
+Evidence used, per function:
+  * MX element / scale math: golden vectors written from the reference's own
+    src/csrc/mxfp_quant.h (tests/golden/mxfp4_golden.npz), the live shim
+    around that header where it was built, OCP-MX known answers, and an
+    independent nearest / ties-to-even table search over all bf16 patterns.
+  * INT8: invariants (|w - q*s| <= s/2, the block maximum maps to +-127, an
+    all-zero block has scale 0) and an fp64 restatement.
+  * Layouts: the closed-form index maps coded in C against the view/permute
+    chain restated with numpy, and against a brute-force loop on a tiny case.
+  * Linears: fp64 matmul over the exactly de-quantized weight; exact int32
+    block sums; agreement of the faithful and ideal modes where the reference
+    rounds only once.
+  * Post-ops: torch CPU ops with the same bf16 rounding points.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from util import bits2f, t2bits, randn_bf16
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mxfp4_golden.npz")
+GRID = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], np.float64)
+
+
+def _encode_all(vals):
+    return O.e2m1_encode_array(vals)
+
+
+def _ref_value_to_code(ref):
+    """The value -> code chain of the reference (qtypes.cpp:99-131): +-0 -> 0,
+    a NaN matches nothing and leaves 0."""
+    codes = np.zeros(ref.shape, np.int64)
+    for i, r in enumerate(ref):
+        if r != r or r == 0.0:
+            continue
+        idx = int(np.where(GRID == abs(float(r)))[0][0])
+        codes[i] = idx | (8 if r < 0 else 0)
+    return codes
+
+
+def test_e2m1_against_golden_all_bf16():
+    g = np.load(GOLD)
+    vals = (np.arange(65536, dtype=np.uint32) << 16).view(np.float32)
+    want = _ref_value_to_code(g["e2m1_bf16_out"].view(np.float32))
+    got = _encode_all(vals)
+    assert np.array_equal(got, want)
+
+
+def test_e2m1_against_golden_ties_and_random_fp32():
+    g = np.load(GOLD)
+    vals = g["tie_in"].view(np.float32)
+    want = _ref_value_to_code(g["tie_out"].view(np.float32))
+    assert np.array_equal(_encode_all(vals), want)
+
+
+def test_scale_against_golden():
+    g = np.load(GOLD)
+    a = (np.arange(32768, dtype=np.uint32) << 16).view(np.float32)
+    assert np.array_equal(O.mx_quant_scale_of_amax_array(a).view(np.uint32), g["scale_bf16_out"])
+    a = g["scale_in"].view(np.float32)
+    assert np.array_equal(O.mx_quant_scale_of_amax_array(a).view(np.uint32), g["scale_out"])
+
+
+def test_against_live_reference_shim():
+    R = O.ref_lib()
+    if R is None:
+        pytest.skip("oracle/_ref not built (reference tree not mounted)")
+    rng = np.random.default_rng(3)
+    for v in (rng.standard_normal(3000) * 4).astype(np.float32):
+        r = R.ref_e2m1_round(float(v))
+        want = 0.0 if (r != r) else r
+        assert O.e2m1_decode(O.e2m1_encode(float(v))) == want
+    for v in np.abs(rng.standard_normal(3000)).astype(np.float32) * np.float32(2.0) ** rng.integers(-130, 127, 3000):
+        v = np.float32(v)
+        a = np.float32(R.ref_mx_shared_scale(float(v))).view(np.uint32)
+        b = np.float32(O.mx_quant_scale(O.mx_scale_byte(float(v)))).view(np.uint32)
+        assert a == b
+
+
+def test_ocp_mx_known_answers():
+    # value/scale -> E2M1 value (ties to even mantissa, saturation at 6)
+    for v, want in [(1.25, 1.0), (1.75, 2.0), (2.5, 2.0), (3.5, 4.0), (5.0, 4.0), (0.25, 0.0), (0.75, 1.0),
+                    (7.0, 6.0), (6.5, 6.0), (-5.0, -4.0), (0.2499, 0.0), (0.2501, 0.5), (100.0, 6.0),
+                    (-0.08, 0.0)]:
+        assert O.e2m1_decode(O.e2m1_encode(v)) == want, v
+    assert O.e2m1_encode(-0.08) == 0  # never the negative-zero code
+    assert O.e2m1_encode(-0.0) == 0
+    # block maximum -> E8M0 byte: floor(log2 max) - 2 + 127
+    for a, want in [(1.0, 125), (0.078, 121), (6.0, 127), (7.9, 127), (0.0, 0), (1e-40, 0), (3e38, 252)]:
+        assert O.mx_scale_byte(a) == want, a
+    assert O.mx_dequant_scale(0) == 0.0 and O.mx_dequant_scale(127) == 1.0
+
+
+def test_e2m1_independent_table_search():
+    """Nearest grid point, ties to the even code, computed in fp64 without the
+    oracle's threshold chain."""
+    vals = (np.arange(65536, dtype=np.uint32) << 16).view(np.float32)
+    finite = np.isfinite(vals)
+    a = np.minimum(np.abs(vals[finite].astype(np.float64)), 8.0)  # everything from 8 up saturates
+    grid9 = np.append(GRID, 8.0)  # 8 = first value beyond the format; rounds there, then saturates
+    d = np.abs(a[:, None] - grid9[None, :])
+    best = d.min(axis=1)
+    cand = d == best[:, None]
+    idx = np.empty(a.shape, np.int64)
+    for i in range(a.size):
+        c = np.flatnonzero(cand[i])
+        idx[i] = c[0] if len(c) == 1 else [k for k in c if k % 2 == 0][0]
+    idx = np.minimum(idx, 7)
+    want = np.where((idx > 0) & (np.signbit(vals[finite])), idx | 8, idx)
+    assert np.array_equal(_encode_all(vals[finite]), want)
+
+
+def test_int8_invariants():
+    rng = np.random.default_rng(5)
+    t = (rng.standard_normal((6, 4, 64, 16, 4)) * 0.02).astype(np.float32)
+    t[0, 0] = 0.0  # an all-zero block
+    q, s = O.quantize_int8sym(t, 256, 2, True)
+    assert s.shape == (6, 4, 1, 16) and q.shape == t.shape
+    assert np.all(s[0, 0] == 0.0) and np.all(q[0, 0] == 0)
+    sb = np.broadcast_to(s[:, :, :, :, None], (6, 4, 1, 16, 1))
+    assert np.all(np.abs(t - q * sb) <= sb * 0.5 * (1 + 1e-6) + 1e-12)
+    amax = np.abs(t).max(axis=(2, 4))
+    assert np.array_equal(s[:, :, 0, :], (amax.astype(np.float64) / 127.0).astype(np.float32))
+    assert np.array_equal(np.abs(q).max(axis=(2, 4))[1:], np.full((5, 4, 16), 127))
+    d = O.dequantize_int8sym(q, s, 256, 2, True)
+    assert np.array_equal(d, q.astype(np.float32) * sb)
+
+
+def test_act_quant_matches_generic_quantizer():
+    x = randn_bf16((5, 768), 1.0, 11)
+    xq, sa = O.quant_act_int8(t2bits(x), 256)
+    q2, s2 = O.quantize_int8sym(x.float().numpy(), 256, -1, False)
+    assert np.array_equal(xq, q2) and np.array_equal(sa, s2)
+
+
+@pytest.mark.parametrize("shape", [(64, 128), (96, 320)])
+def test_layout_closed_form_equals_view_permute_chain(shape):
+    N, K = shape
+    rng = np.random.default_rng(N)
+    W = O.bf16_round((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+    for vnni in (2, 1):  # 5-D bf16-style and 4-D fp32-style blocked inputs
+        Wb = O.block_weight(W, 16, 64, vnni)
+        assert np.array_equal(O.unblock_weight(Wb), W)
+        q1, s1 = O.remap_and_quantize_mxfp4_blocked(Wb)
+        q2, s2 = O.remap_quantize_mxfp4(W)
+        assert np.array_equal(q1, q2) and np.array_equal(s1, s2)
+        qa, sa, qbs = O.remap_and_quantize_qint8_blocked(Wb)
+        qb, sb, qbs2 = O.remap_quantize_qint8(W)
+        assert qbs == qbs2 and np.array_equal(qa, qb) and np.array_equal(sa, sb)
+    # a 64-wide output block (K2 > 32) is split instead of paired
+    q3, s3 = O.remap_and_quantize_mxfp4_blocked(O.block_weight(W[:64], 64, 64, 2))
+    q4, s4 = O.remap_quantize_mxfp4(W[:64])
+    assert np.array_equal(q3, q4) and np.array_equal(s3, s4)
+
+
+def test_layout_brute_force_index_formula():
+    N, K = 32, 64
+    W = np.arange(N * K, dtype=np.float32).reshape(N, K) % 13 - 6.0
+    q, s = O.remap_quantize_mxfp4(W)
+    Wd = O.dequantize_mxfp4_plain(q, s)
+    t5 = O.dequantize_mxfp4(q.reshape(1, 1, 32, 32, 1), s)  # generic blocked-shape dequantizer
+    for n in range(N):
+        for k in range(K):
+            b = int(q[0, 0, k // 2, n])
+            code = (b >> 4) if (k & 1) else (b & 15)
+            x = int(s[0, 0, k // 32, n])
+            assert Wd[n, k] == O.E2M1_TABLE[code] * O.mx_dequant_scale(x)
+            assert t5[0, 0, k // 2, n, k & 1] == Wd[n, k]
+    qi, si, qbs = O.remap_quantize_qint8(W)
+    assert qbs == 64
+    Wi = O.dequantize_qint8_plain(qi, si)
+    for n in range(N):
+        for k in range(K):
+            assert Wi[n, k] == np.float32(qi[n // 16, 0, k // 4, n % 16, k % 4]) * si[n // 16, 0, 0, n % 16]
+
+
+def test_qint8_block_size_rule():
+    assert O.qint8_block_size(4096) == 256 and O.qint8_block_size(11008) == 256
+    assert O.qint8_block_size(192) == 64 and O.qint8_block_size(384) == 128
+    assert O.qint8_block_size(4096, 4096) == 4096
+
+
+def test_mx_roundtrip_error_bound():
+    rng = np.random.default_rng(9)
+    W = (rng.standard_normal((64, 256)) * 0.02).astype(np.float32)
+    q, s = O.remap_quantize_mxfp4(W)
+    Wd = O.dequantize_mxfp4_plain(q, s)
+    scale = np.array([[O.mx_dequant_scale(int(s[n // 32, k // 64, (k % 64) // 32, n % 32])) for k in range(256)]
+                      for n in range(64)], np.float32)
+    # the block maximum lies in [4, 8) scale units: rounding costs at most half
+    # the largest step (1.0) and saturation at 6 at most 2.0
+    assert np.all(np.abs(W - Wd) <= scale * 2.0 + 1e-12)
+    assert np.all(np.abs(W - Wd)[np.abs(W) <= 6 * scale] <= scale[np.abs(W) <= 6 * scale] * 1.0 + 1e-12)
+
+
+@pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])
+def test_linear_reduces_to_fp64_matmul(fmt):
+    M, N, K = 7, 96, 512
+    W = randn_bf16((N, K), 0.02, 21).float().numpy()
+    x = randn_bf16((M, K), 1.0, 22)
+    bias = randn_bf16((N,), 0.01, 23)
+    xb, bb = t2bits(x), t2bits(bias)
+    if fmt == "mxfp4":
+        q, s = O.remap_quantize_mxfp4(W)
+        Wd = O.dequantize_mxfp4_plain(q, s).astype(np.float64)
+        want = x.float().numpy().astype(np.float64) @ Wd.T + bits2f(bb)
+        y = O.linear_mxfp4(xb, q, s, bb)
+        y64 = O.linear_mxfp4(xb, q, s, bb, mode=O.MODE_F64)
+        assert np.array_equal(y, O.linear_mxfp4(xb, q, s, bb, mode=O.MODE_FAITHFUL))  # one chunk when M/64 <= 4
+    else:
+        q, s, qbs = O.remap_quantize_qint8(W)
+        xq, sa = O.quant_act_int8(xb, qbs)
+        acc = O.qint8_block_sums(xq, q)
+        Wq = np.round(O.dequantize_qint8_plain(q, np.ones_like(s))).astype(np.int64)
+        want_acc = np.einsum("mbk,nbk->mnb", xq.astype(np.int64).reshape(M, K // qbs, qbs), Wq.reshape(N, K // qbs, qbs))
+        assert np.array_equal(acc, want_acc)  # exact int32 block sums
+        sw = s.reshape(N // 16, K // qbs, 16).transpose(0, 2, 1).reshape(N, K // qbs)
+        want = (acc.astype(np.float64) * sa[:, None, :].astype(np.float64) * sw[None].astype(np.float64)).sum(-1) + bits2f(bb)
+        y = O.linear_qint8(xb, q, s, bb)
+        y64 = O.linear_qint8(xb, q, s, bb, mode=O.MODE_F64)
+    want_bf16 = O.f32_to_bf16(want.astype(np.float32))
+    # fp64 mode is the exact sum rounded once (up to the double->float->bf16 double rounding)
+    assert np.mean(y64 != want_bf16) < 2e-3
+    # fp32 accumulation stays within one bf16 ulp of the exact result
+    d = np.abs(bits2f(y).astype(np.float64) - want)
+    assert np.all(d <= 2.0 ** -7 * np.abs(want) + 2.0 ** -8 * np.sqrt(np.mean(want * want)))
+
+
+def test_faithful_chunking_differs_only_within_tolerance():
+    M, N, K = 384, 32, 8192  # M/64 > 4 -> the reference re-rounds every 4096 input channels
+    W = randn_bf16((N, K), 0.02, 31).float().numpy()
+    x = t2bits(randn_bf16((M, K), 1.0, 32))
+    q, s = O.remap_quantize_mxfp4(W)
+    a = bits2f(O.linear_mxfp4(x, q, s, mode=O.MODE_IDEAL)).astype(np.float64)
+    b = bits2f(O.linear_mxfp4(x, q, s, mode=O.MODE_FAITHFUL)).astype(np.float64)
+    assert np.any(a != b)
+    assert np.sqrt(((a - b) ** 2).sum() / (a ** 2).sum()) < 2.0 ** -9 * np.sqrt(2)
+
+
+def test_post_ops_against_torch_rounding_points():
+    y = randn_bf16((4096,), 2.0, 41)
+    in1 = randn_bf16((4096,), 1.0, 42)
+    in2 = randn_bf16((4096,), 1.0, 43)
+    bf = torch.bfloat16
+    yf, a, b = y.float(), in1.float(), in2.float()
+    cases = {
+        O.POST_MUL: (a * yf).to(bf),
+        O.POST_ADD_SCALE: (yf + a * 0.5).to(bf),
+        O.POST_ADD2_SCALE: ((yf + a).to(bf).float() + b * 0.5).to(bf),
+        O.POST_RELU: torch.clamp_min(y, 0),
+    }
+    for post, want in cases.items():
+        got = O.post_op(t2bits(y), post, t2bits(in1), t2bits(in2), 0.5)
+        assert np.array_equal(got, t2bits(want)), post
+    # transcendental post-ops: libm vs torch may differ in the last fp32 bit
+    silu = (yf * torch.sigmoid(yf).to(bf).float()).to(bf)
+    gelu = torch.nn.functional.gelu(yf).to(bf)
+    for post, want in ((O.POST_SILU, silu), (O.POST_GELU, gelu)):
+        got = bits2f(O.post_op(t2bits(y), post)).astype(np.float64)
+        w = want.float().numpy().astype(np.float64)
+        assert np.all(np.abs(got - w) <= 2.0 ** -7 * np.abs(w) + 1e-30)
+        assert np.mean(got != w) < 0.01
