@@ -238,7 +238,7 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
     return TPPX_OK;
   }
   const int force = env_int("TPPX_QINT8_SPLITK", -1);
-  if (force == 1 || (force != 0 && M > 16)) {
+  if (p.tpb == 4 && (force == 1 || (force != 0 && M > 16))) {
     // more than one MFMA row group: activations shared through LDS, K split
     // across workgroups
     DecodePlan pl = plan_decode(1, M, p.groups, p.total_tiles, p.units, p.tpb, false, (size_t)ws_bytes);

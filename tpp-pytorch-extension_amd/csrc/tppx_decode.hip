@@ -248,31 +248,47 @@ decode_qint8_kernel(const DecodeParams p) {
     __syncthreads();
     // ---- stream the weights of this chunk ----
     if (active) {
-      for (int t = tc; t < tce; t += PF) {
+      // multiply ring slot i with tile tt; `last` = tt closes a K block
+      auto consume = [&](int i, int tt, bool last, bool fast) {
+        const int tl = tt - tc;
+#pragma unroll
+        for (int mg = 0; mg < MG; mg++)
+          iacc[mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xs[(tl * MG + mg) * 64 + lane], wreg[i], iacc[mg], 0, 0, 0);
+        if (last) { // scale and fold into fp32
+          const int ul = (fast ? (tt >> 2) : tt / TPB) - uc;
+          const float swv = sw_s[(ul * 8 + wave) * 16 + (lane & 15)];
+#pragma unroll
+          for (int mg = 0; mg < MG; mg++) {
+            const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + ul * MPAD + mg * 16 + (lane >> 4) * 4);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              facc[0][mg][r] = fmaf((float)iacc[mg][r], sav[r] * swv, facc[0][mg][r]);
+              iacc[mg][r] = 0;
+            }
+          }
+        }
+      };
+      int t = tc;
+      if (TPB == 4) {
+        // Full groups whose reloads are all real tiles: no branch and no load
+        // other than the ring inside, so the wait counts stay exact and PF
+        // tiles are really in flight (a branch in the body drains the ring).
+        for (; t + PF <= tce && t + 2 * PF <= t1; t += PF) {
+#pragma unroll
+          for (int i = 0; i < PF; i++) {
+            consume(i, t + i, (i & 3) == 3, true);
+            load_w(i, t + i + PF);
+          }
+        }
+      }
+      for (; t < tce; t += PF) {
 #pragma unroll
         for (int i = 0; i < PF; i++) {
           const int tt = t + i;
           if (tt < tce) {
-            const int tl = tt - tc;
-#pragma unroll
-            for (int mg = 0; mg < MG; mg++)
-              iacc[mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xs[(tl * MG + mg) * 64 + lane], wreg[i],
-                                                               iacc[mg], 0, 0, 0);
+            consume(i, tt, (tt + 1) % TPB == 0, false);
             if (tt + PF < t1)
               load_w(i, tt + PF);
-            if ((tt + 1) % TPB == 0) { // K block complete: scale and fold into fp32
-              const int ul = tt / TPB - uc;
-              const float swv = sw_s[(ul * 8 + wave) * 16 + (lane & 15)];
-#pragma unroll
-              for (int mg = 0; mg < MG; mg++) {
-                const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + ul * MPAD + mg * 16 + (lane >> 4) * 4);
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                  facc[0][mg][r] = fmaf((float)iacc[mg][r], sav[r] * swv, facc[0][mg][r]);
-                  iacc[mg][r] = 0;
-                }
-              }
-            }
           }
         }
       }
@@ -371,30 +387,43 @@ decode_mxfp4_kernel(const DecodeParams p) {
     }
     __syncthreads();
     if (active) {
-      for (int t = tc; t < tce; t += PF) {
+      auto consume = [&](int i, int tt) {
+        const int tl = tt - tc;
+        float sc[NW];
+#pragma unroll
+        for (int s = 0; s < NW; s++)
+          sc[s] = e8m0_to_f32(sreg[i][s]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          bf16x8 wb[NW];
+#pragma unroll
+          for (int s = 0; s < NW; s++)
+            wb[s] = cvt_fp4x8((uint32_t)wreg[i][s][j], sc[s]);
+#pragma unroll
+          for (int mg = 0; mg < MG; mg++) {
+            const bf16x8 xa = xs[((tl * MG + mg) * 4 + j) * 64 + lane];
+#pragma unroll
+            for (int s = 0; s < NW; s++)
+              acc[s][mg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, wb[s], acc[s][mg], 0, 0, 0);
+          }
+        }
+      };
+      int t = tc;
+      // Full groups whose reloads are all real tiles run without a branch in
+      // the body, so the ring keeps PF tiles in flight with exact wait counts.
+      for (; t + PF <= tce && t + 2 * PF <= t1; t += PF) {
+#pragma unroll
+        for (int i = 0; i < PF; i++) {
+          consume(i, t + i);
+          load_w(i, t + i + PF);
+        }
+      }
+      for (; t < tce; t += PF) {
 #pragma unroll
         for (int i = 0; i < PF; i++) {
           const int tt = t + i;
           if (tt < tce) {
-            const int tl = tt - tc;
-            float sc[NW];
-#pragma unroll
-            for (int s = 0; s < NW; s++)
-              sc[s] = e8m0_to_f32(sreg[i][s]);
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-              bf16x8 wb[NW];
-#pragma unroll
-              for (int s = 0; s < NW; s++)
-                wb[s] = cvt_fp4x8((uint32_t)wreg[i][s][j], sc[s]);
-#pragma unroll
-              for (int mg = 0; mg < MG; mg++) {
-                const bf16x8 xa = xs[((tl * MG + mg) * 4 + j) * 64 + lane];
-#pragma unroll
-                for (int s = 0; s < NW; s++)
-                  acc[s][mg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, wb[s], acc[s][mg], 0, 0, 0);
-              }
-            }
+            consume(i, tt);
             if (tt + PF < t1)
               load_w(i, tt + PF);
           }

@@ -134,6 +134,7 @@ skinny_qint8_kernel(const DecodeParams p) {
   const int ltile0 = (grp - sg.grp0) * NTW;
   const int m0 = blockIdx.y * MPAD;
   const int NB = p.units, TPB = p.tpb, KT = NB * TPB;
+  const bool TPB4 = (TPB == 4) && (PF % 4 == 0); // 256-wide K blocks: the default
   const int u0 = (int)(((int64_t)wave * NB) / W), u1 = (int)(((int64_t)(wave + 1) * NB) / W);
   const int t0 = u0 * TPB, t1 = u1 * TPB;
 
@@ -165,12 +166,21 @@ skinny_qint8_kernel(const DecodeParams p) {
     sa_s[i] = p.sa[(int64_t)min(m0 + mr, p.M - 1) * NB + u0 + ul];
   }
 
+  // Ring of PF stages; a stage = the weight tiles, their block scale and the
+  // activation operand of one k-tile.  The main loop has NO branch and NO load
+  // other than the ring itself, so the compiler's wait counts stay exact and
+  // PF stages are really in flight (a load that must be waited for out of
+  // order, or a branch inside the loop, drains the whole ring).
   i32x4 wreg[PF][NTW], xreg[PF][MG];
-  auto load_stage = [&](int st, int t) {
-    t = min(t, t1 - 1);
+  float sreg[PF][NTW];
+  auto load_stage = [&](int st, int t, bool fast) {
+    t = min(t, t1 - 1); // past the end: re-read the last tile (never consumed)
+    const int b = fast ? (t >> 2) : t / TPB;
 #pragma unroll
-    for (int nt = 0; nt < NTW; nt++)
+    for (int nt = 0; nt < NTW; nt++) {
       wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64);
+      sreg[st][nt] = ws[nt][b * 16];
+    }
 #pragma unroll
     for (int mg = 0; mg < MG; mg++)
       xreg[st][mg] = *reinterpret_cast<const i32x4*>(xrow[mg] + t * 64);
@@ -178,7 +188,7 @@ skinny_qint8_kernel(const DecodeParams p) {
   if (t0 < t1) {
 #pragma unroll
     for (int i = 0; i < PF; i++)
-      load_stage(i, t0 + i);
+      load_stage(i, t0 + i, false);
   }
 
   f32x4 facc[NTW][MG];
@@ -191,34 +201,52 @@ skinny_qint8_kernel(const DecodeParams p) {
       iacc[nt][mg] = i32x4{0, 0, 0, 0};
     }
 
-  for (int t = t0; t < t1; t += PF) {
+  // multiply stage i (tile tt); `last` = tt closes a K block: fold into fp32
+  auto consume = [&](int i, int tt, bool last, bool fast) {
+    float swv[NTW];
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++) {
+      swv[nt] = sreg[i][nt];
+#pragma unroll
+      for (int mg = 0; mg < MG; mg++)
+        iacc[nt][mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xreg[i][mg], wreg[i][nt], iacc[nt][mg], 0, 0, 0);
+    }
+    if (last) {
+      const int b = fast ? (tt >> 2) : tt / TPB;
+#pragma unroll
+      for (int mg = 0; mg < MG; mg++) {
+        const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + (b - u0) * MPAD + mg * 16 + (lane >> 4) * 4);
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            facc[nt][mg][r] = fmaf((float)iacc[nt][mg][r], sav[r] * swv[nt], facc[nt][mg][r]);
+            iacc[nt][mg][r] = 0;
+          }
+      }
+    }
+  };
+
+  int t = t0;
+  if (TPB4) {
+    // full groups of PF tiles: static block boundaries (PF and t0 are multiples of 4)
+    for (; t + 2 * PF <= t1; t += PF) { // every reload of these groups is a real tile
+#pragma unroll
+      for (int i = 0; i < PF; i++) {
+        consume(i, t + i, (i & 3) == 3, true);
+        load_stage(i, t + i + PF, true);
+      }
+    }
+  }
+  // remaining tiles (and every tile when the K block is not 256 wide)
+  for (; t < t1; t += PF) {
 #pragma unroll
     for (int i = 0; i < PF; i++) {
       const int tt = t + i;
       if (tt < t1) {
-#pragma unroll
-        for (int nt = 0; nt < NTW; nt++)
-#pragma unroll
-          for (int mg = 0; mg < MG; mg++)
-            iacc[nt][mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xreg[i][mg], wreg[i][nt], iacc[nt][mg], 0, 0, 0);
+        consume(i, tt, (tt + 1) % TPB == 0, false);
         if (tt + PF < t1)
-          load_stage(i, tt + PF);
-        if ((tt + 1) % TPB == 0) { // K block complete: scale and fold into fp32
-          const int b = tt / TPB;
-#pragma unroll
-          for (int mg = 0; mg < MG; mg++) {
-            const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + (b - u0) * MPAD + mg * 16 + (lane >> 4) * 4);
-#pragma unroll
-            for (int nt = 0; nt < NTW; nt++) {
-              const float swv = ws[nt][b * 16];
-#pragma unroll
-              for (int r = 0; r < 4; r++) {
-                facc[nt][mg][r] = fmaf((float)iacc[nt][mg][r], sav[r] * swv, facc[nt][mg][r]);
-                iacc[nt][mg][r] = 0;
-              }
-            }
-          }
-        }
+          load_stage(i, tt + PF, false);
       }
     }
   }
@@ -297,12 +325,16 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
   SkEpilogue<1, NTW, false, MINW> ep;
   ep.prefetch(p, sg, ltile0, 0);
 
+  // ring stage = weight tiles + their block scale (see skinny_qint8_kernel)
   i32x4 wreg[PF][NTW];
+  float sreg[PF][NTW];
   auto load_stage = [&](int st, int t) {
     t = min(t, t1 - 1);
 #pragma unroll
-    for (int nt = 0; nt < NTW; nt++)
+    for (int nt = 0; nt < NTW; nt++) {
       wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64);
+      sreg[st][nt] = ws[nt][(t >> 2) * 16];
+    }
   };
   if (t0 < t1) {
 #pragma unroll
@@ -362,31 +394,42 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
     facc[nt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
     iacc[nt] = i32x4{0, 0, 0, 0};
   }
-  for (int t = t0; t < t1; t += PF) {
+  auto consume = [&](int i, int tt, bool last) {
+    const i32x4 xa = *reinterpret_cast<const i32x4*>(xq_s + (tt - t0) * 16 * M + xoff);
+    float swv[NTW];
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++) {
+      swv[nt] = sreg[i][nt];
+      iacc[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa, wreg[i][nt], iacc[nt], 0, 0, 0);
+    }
+    if (last) { // K block complete
+      // result rows (lane>>4)*4 + r: only the first lane group holds valid rows (M <= 4)
+      const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + ((tt >> 2) - u0) * 4);
+#pragma unroll
+      for (int nt = 0; nt < NTW; nt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          facc[nt][0][r] = fmaf((float)iacc[nt][r], sav[r] * swv[nt], facc[nt][0][r]);
+          iacc[nt][r] = 0;
+        }
+    }
+  };
+  int t = t0;
+  for (; t + 2 * PF <= t1; t += PF) { // every reload of these groups is a real tile // branch-free full groups (PF is a multiple of 4)
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      consume(i, t + i, (i & 3) == 3);
+      load_stage(i, t + i + PF);
+    }
+  }
+  for (; t < t1; t += PF) {
 #pragma unroll
     for (int i = 0; i < PF; i++) {
       const int tt = t + i;
       if (tt < t1) {
-        const i32x4 xa = *reinterpret_cast<const i32x4*>(xq_s + (tt - t0) * 16 * M + xoff);
-#pragma unroll
-        for (int nt = 0; nt < NTW; nt++)
-          iacc[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa, wreg[i][nt], iacc[nt], 0, 0, 0);
+        consume(i, tt, (i & 3) == 3);
         if (tt + PF < t1)
           load_stage(i, tt + PF);
-        if ((tt & 3) == 3) { // K block complete
-          const int b = tt >> 2;
-          // result rows (lane>>4)*4 + r: only the first lane group holds valid rows (M <= 4)
-          const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + (b - u0) * 4);
-#pragma unroll
-          for (int nt = 0; nt < NTW; nt++) {
-            const float swv = ws[nt][b * 16];
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-              facc[nt][0][r] = fmaf((float)iacc[nt][r], sav[r] * swv, facc[nt][0][r]);
-              iacc[nt][r] = 0;
-            }
-          }
-        }
       }
     }
   }
@@ -452,19 +495,30 @@ skinny_mxfp4_kernel(const DecodeParams p) {
   for (int nt = 0; nt < NTW; nt++)
     acc[nt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int t = t0; t < t1; t += PF) {
+  auto consume = [&](int i) {
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++) {
+      const float sc = e8m0_to_f32(sreg[i][nt]);
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        acc[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            xreg[i][j], sk_cvt_fp4x8((uint32_t)wreg[i][nt][j], sc), acc[nt][0], 0, 0, 0);
+    }
+  };
+  int t = t0;
+  for (; t + 2 * PF <= t1; t += PF) { // every reload of these groups is a real tile // branch-free full groups: exact wait counts, PF stages in flight
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      consume(i);
+      load_stage(i, t + i + PF); // clamped past the end (re-reads the last tile, never consumed)
+    }
+  }
+  for (; t < t1; t += PF) {
 #pragma unroll
     for (int i = 0; i < PF; i++) {
       const int tt = t + i;
       if (tt < t1) {
-#pragma unroll
-        for (int nt = 0; nt < NTW; nt++) {
-          const float sc = e8m0_to_f32(sreg[i][nt]);
-#pragma unroll
-          for (int j = 0; j < 4; j++)
-            acc[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                xreg[i][j], sk_cvt_fp4x8((uint32_t)wreg[i][nt][j], sc), acc[nt][0], 0, 0, 0);
-        }
+        consume(i);
         if (tt + PF < t1)
           load_stage(i, tt + PF);
       }
@@ -495,7 +549,7 @@ SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual
   // units simply get an empty range.
   int max_w, min_w;
   if (fmt == 1) {
-    max_w = pl.mg == 4 ? 8 : 16;
+    max_w = (pl.mg == 4 || (pl.mg == 2 && pl.ntw == 2)) ? 8 : 16;
     min_w = (pl.mg == 4 || (pl.mg == 2 && pl.ntw == 2)) ? 8 : 4;
   } else {
     max_w = pl.ntw == 2 ? 8 : 16;
@@ -534,21 +588,21 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
   if (pl.fused_quant) {
     size_t lds = (size_t)pl.waves * pl.ntw * 256 * sizeof(float) + (size_t)pl.waves * pl.max_units * (4 * 256 + 16);
     if (pl.ntw == 2)
-      return sk_launch(skinny_qint8_fq_kernel<2, 8, 16, 4>, p, grid, pl.waves, lds, stream);
+      return sk_launch(skinny_qint8_fq_kernel<2, 4, 16, 4>, p, grid, pl.waves, lds, stream);
     return sk_launch(skinny_qint8_fq_kernel<1, 12, 16, 4>, p, grid, pl.waves, lds, stream);
   }
   size_t lds = ((size_t)pl.waves * pl.ntw * pl.mg * 256 + (size_t)pl.waves * pl.max_units * pl.mg * 16) * sizeof(float);
   if (pl.ntw == 2) {
     switch (pl.mg) {
       case 1: return sk_launch(skinny_qint8_kernel<1, 2, 4, 16, 4>, p, grid, pl.waves, lds, stream);
-      case 2: return sk_launch(skinny_qint8_kernel<2, 2, 3, 16, 8>, p, grid, pl.waves, lds, stream);
+      case 2: return sk_launch(skinny_qint8_kernel<2, 2, 8, 8, 8>, p, grid, pl.waves, lds, stream);
       default: return sk_launch(skinny_qint8_kernel<4, 2, 4, 8, 8>, p, grid, pl.waves, lds, stream);
     }
   }
   switch (pl.mg) {
-    case 1: return sk_launch(skinny_qint8_kernel<1, 1, 8, 16, 4>, p, grid, pl.waves, lds, stream);
-    case 2: return sk_launch(skinny_qint8_kernel<2, 1, 6, 16, 4>, p, grid, pl.waves, lds, stream);
-    default: return sk_launch(skinny_qint8_kernel<4, 1, 6, 8, 8>, p, grid, pl.waves, lds, stream);
+    case 1: return sk_launch(skinny_qint8_kernel<1, 1, 4, 16, 4>, p, grid, pl.waves, lds, stream);
+    case 2: return sk_launch(skinny_qint8_kernel<2, 1, 4, 16, 4>, p, grid, pl.waves, lds, stream);
+    default: return sk_launch(skinny_qint8_kernel<4, 1, 8, 8, 8>, p, grid, pl.waves, lds, stream);
   }
 }
 
