@@ -153,10 +153,13 @@ int tppx_linear_mxfp4(const void* x, const void* qw, const void* sw,
 
 /* Replaces TppBlockedQInt8LinearW<bf16,uint8_t,bf16>
  * (src/csrc/fused_gemm.h:1076-1341,1530-1534): activations are quantized into
- * the caller's scratch xq (i8 [M][K]) / sa (f32 [M][K/qbs]) and then
+ * the caller's scratch xq (room for roundup(M,64)*K bytes) / sa (room for
+ * roundup(M,64)*(K/qbs) floats) and then
  *   y = post( bf16( bias + sum_b float(sum_{k in b} xq*wq) * sa[m][b]*sw[n][b] ) )
- * x == NULL means xq / sa already hold the quantized activations (the
- * reference accepts a pre-quantized qint8 input, fused_gemm.h:1244-1246). */
+ * x == NULL means xq (i8 [M][K] row-major) / sa already hold the quantized
+ * activations (the reference accepts a pre-quantized qint8 input,
+ * fused_gemm.h:1244-1246).  With x != NULL the layout written into xq is
+ * private to the library (the GEMM reads it in MFMA operand order). */
 int tppx_linear_qint8(const void* x, void* xq, void* sa, const void* qw,
                       const void* sw, const void* bias, const void* post_in,
                       const void* post_in2, void* y, int64_t M, int64_t N,

@@ -238,7 +238,7 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
     return TPPX_OK;
   }
   const int force = env_int("TPPX_QINT8_SPLITK", -1);
-  if (p.tpb == 4 && (force == 1 || (force != 0 && M > 16))) {
+  if (p.tpb == 4 && M > 4 && force == 1) {
     // more than one MFMA row group: activations shared through LDS, K split
     // across workgroups
     DecodePlan pl = plan_decode(1, M, p.groups, p.total_tiles, p.units, p.tpb, false, (size_t)ws_bytes);
@@ -254,7 +254,10 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
   SkinnyPlan sp = plan_skinny(1, M, p.total_tiles, p.units, false);
   sp.fused_quant = sp.fused_quant && x != nullptr && qbs == 256;
   if (x && !sp.fused_quant) {
-    rc = tppx_quant_act_int8(x, M, K, qbs, xq, sa, stream);
+    // quantise straight into MFMA operand order: the GEMM then reads one
+    // contiguous 1 KiB per operand instead of 16 rows x 64 B
+    p.mt = sp.grid_y * sp.mg;
+    rc = check_hip(launch_quant_act_int8(x, M, K, qbs, xq, sa, p.mt, stream), who);
     if (rc)
       return rc;
   }

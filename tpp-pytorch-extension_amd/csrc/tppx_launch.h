@@ -30,9 +30,10 @@ struct DecodeParams {
   int groups;      // sum over segments of ceil(tiles / 8)
   int total_tiles; // sum of tiles (one segment's tiles for the dual gate/up kernel)
   const void* x;   // bf16 [M][K]
-  const void* xq;  // int8 [M][K]     (QINT8, unless quantised in-kernel)
+  const void* xq;  // int8 [M][K], or MFMA operand order when mt > 0 (QINT8, unless quantised in-kernel)
   const float* sa; // f32  [M][K/qbs] (QINT8, unless quantised in-kernel)
   int M, K;
+  int mt;    // > 0: xq is [K/64][mt][4 g][16 m][16 B] (operand tiles of 16 rows x 64 K); 0: row-major
   int units; // K/128 (MXFP4 tiles) or K/qbs (QINT8 blocks)
   int tpb;   // native tiles per unit (1 for MXFP4, qbs/64 for QINT8)
   int S;     // K splits across workgroups
@@ -74,6 +75,10 @@ hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream);
 hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream);
 
 int env_int(const char* name, int dflt);
+
+// dynamic activation quantisation; mt > 0 writes xq in MFMA operand order (see DecodeParams::mt)
+hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs, void* xq, void* sa, int mt,
+                                 hipStream_t stream);
 
 SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual);
 hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream);

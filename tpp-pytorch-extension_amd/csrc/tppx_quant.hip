@@ -233,7 +233,7 @@ prepack_qint8_kernel(const int8_t* __restrict__ qref, int64_t N, int64_t K,
 __global__ void __launch_bounds__(256)
 quant_act_int8_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
                       int64_t qbs, int8_t* __restrict__ xq,
-                      float* __restrict__ sa) {
+                      float* __restrict__ sa, int mt) {
   int64_t nb = K / qbs;
   int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
   int lane = threadIdx.x & 63;
@@ -252,12 +252,19 @@ quant_act_int8_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
     float s = int8_scale_of(amax);
     float inv = int8_inv_scale(s);
     if (lane == 0)
-      sa[m * nb + b] = s;
+      sa[mt > 0 ? b * (int64_t)mt * 16 + m : m * nb + b] = s;
     uint32_t packed = (uint32_t)(int8_q(v0, inv) & 0xff) |
         ((uint32_t)(int8_q(v1, inv) & 0xff) << 8) |
         ((uint32_t)(int8_q(v2, inv) & 0xff) << 16) |
         ((uint32_t)(int8_q(v3, inv) & 0xff) << 24);
-    reinterpret_cast<uint32_t*>(o)[lane] = packed;
+    if (mt > 0) {
+      // operand order: tile (k/64, m/16), lane slot (k%64)/16*16 + m%16, 16 B each
+      const int64_t t = b * 4 + (lane >> 4);
+      const int64_t slot = ((t * mt + (m >> 4)) * 64 + ((lane & 15) >> 2) * 16 + (m & 15));
+      reinterpret_cast<uint32_t*>(xq)[slot * 4 + (lane & 3)] = packed;
+    } else {
+      reinterpret_cast<uint32_t*>(o)[lane] = packed;
+    }
   } else {
     float amax = 0.0f;
     for (int64_t j = lane; j < qbs; j += 64)
@@ -266,14 +273,29 @@ quant_act_int8_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
     float s = int8_scale_of(amax);
     float inv = int8_inv_scale(s);
     if (lane == 0)
-      sa[m * nb + b] = s;
-    for (int64_t j = lane; j < qbs; j += 64)
-      o[j] = (int8_t)int8_q(bf16_bits_to_f32(p[j]), inv);
+      sa[mt > 0 ? b * (int64_t)mt * 16 + m : m * nb + b] = s;
+    for (int64_t j = lane; j < qbs; j += 64) {
+      const int8_t q = (int8_t)int8_q(bf16_bits_to_f32(p[j]), inv);
+      if (mt > 0) {
+        const int64_t k = b * qbs + j;
+        xq[(((k >> 6) * mt + (m >> 4)) * 64 + ((k & 63) >> 4) * 16 + (m & 15)) * 16 + (k & 15)] = q;
+      } else {
+        o[j] = q;
+      }
+    }
   }
 }
 
 static inline unsigned grid_for(int64_t n, int block) {
   return (unsigned)((n + block - 1) / block);
+}
+
+hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs, void* xq, void* sa, int mt,
+                                 hipStream_t stream) {
+  int64_t nthreads = M * (K / qbs) * 64;
+  quant_act_int8_kernel<<<grid_for(nthreads, 256), 256, 0, stream>>>((const uint16_t*)x, M, K, qbs, (int8_t*)xq,
+                                                                    (float*)sa, mt);
+  return hipGetLastError();
 }
 
 } // namespace tppx
@@ -388,8 +410,5 @@ extern "C" int tppx_quant_act_int8(const void* x, int64_t M, int64_t K,
   TPPX_REQUIRE(aligned16(x) && aligned16(xq), TPPX_EINVAL, "tppx_quant_act_int8: pointer not 16-byte aligned");
   TPPX_REQUIRE(M > 0 && K > 0 && qbs > 0 && qbs % 64 == 0 && K % qbs == 0, TPPX_ESHAPE,
                "tppx_quant_act_int8: bad shape M=%ld K=%ld qbs=%ld", (long)M, (long)K, (long)qbs);
-  int64_t nthreads = M * (K / qbs) * 64;
-  quant_act_int8_kernel<<<grid_for(nthreads, 256), 256, 0, (hipStream_t)stream>>>(
-      (const uint16_t*)x, M, K, qbs, (int8_t*)xq, (float*)sa);
-  return check_hip(hipGetLastError(), "tppx_quant_act_int8");
+  return check_hip(launch_quant_act_int8(x, M, K, qbs, xq, sa, 0, (hipStream_t)stream), "tppx_quant_act_int8");
 }

@@ -122,7 +122,7 @@ struct SkEpilogue {
 // ---------------------------------------------------------------------------
 // QINT8 (W8A8), activations already quantised (int8 [M][K] + f32 [M][K/qbs]).
 // ---------------------------------------------------------------------------
-template <int MG, int NTW, int PF, int MAXW, int MINW>
+template <int MG, int NTW, int PF, int MAXW, int MINW, bool XOP>
 __global__ void __launch_bounds__(MAXW * 64)
 skinny_qint8_kernel(const DecodeParams p) {
   extern __shared__ __align__(16) float sk_lds[];
@@ -134,7 +134,8 @@ skinny_qint8_kernel(const DecodeParams p) {
   const int ltile0 = (grp - sg.grp0) * NTW;
   const int m0 = blockIdx.y * MPAD;
   const int NB = p.units, TPB = p.tpb, KT = NB * TPB;
-  const bool TPB4 = (TPB == 4) && (PF % 4 == 0); // 256-wide K blocks: the default
+  const bool TPB4 = TPB == 4; // 256-wide K blocks: the default
+  constexpr int UN = (PF % 4 == 0) ? PF : (PF % 2 == 0 ? 2 * PF : 4 * PF); // lcm(PF, 4) tiles per unrolled trip
   const int u0 = (int)(((int64_t)wave * NB) / W), u1 = (int)(((int64_t)(wave + 1) * NB) / W);
   const int t0 = u0 * TPB, t1 = u1 * TPB;
 
@@ -146,7 +147,11 @@ skinny_qint8_kernel(const DecodeParams p) {
     wq[nt] = reinterpret_cast<const i32x4*>(sg.qw) + lt * KT * 64 + lane;
     ws[nt] = reinterpret_cast<const float*>(sg.sw) + lt * NB * 16 + (lane & 15);
   }
+  // XOP: activations in operand order, one contiguous 1 KiB read per (k-tile,
+  // row tile); otherwise row-major rows, 16 rows x 64 B per read.
   const int8_t* xrow[MG];
+  const i32x4* xop = reinterpret_cast<const i32x4*>(p.xq) + (int64_t)blockIdx.y * MG * 64 + lane;
+  const int xstride = p.mt * 64;
 #pragma unroll
   for (int mg = 0; mg < MG; mg++) {
     const int m = min(m0 + mg * 16 + (lane & 15), p.M - 1);
@@ -161,9 +166,20 @@ skinny_qint8_kernel(const DecodeParams p) {
   // activation scales of this wave's K blocks, transposed in LDS: [u - u0][MPAD]
   float* red = sk_lds;
   float* sa_s = sk_lds + (size_t)W * NTW * MG * 256 + (size_t)wave * p.cht * MPAD;
-  for (int i = lane; i < (u1 - u0) * MPAD; i += 64) {
+  const int nsa = (u1 - u0) * MPAD;
+  const int mtp = p.mt * 16;
+  constexpr int SAB = 2 * MG; // loads per batch: 8 K blocks of this wave
+  auto load_sa = [&](int i) {
+    i = min(i, nsa - 1);
     const int ul = i / MPAD, mr = i - ul * MPAD;
-    sa_s[i] = p.sa[(int64_t)min(m0 + mr, p.M - 1) * NB + u0 + ul];
+    // XOP: scales transposed by the quantisation kernel, [K/qbs][mt*16]
+    return XOP ? p.sa[(int64_t)(u0 + ul) * mtp + m0 + mr] : p.sa[(int64_t)min(m0 + mr, p.M - 1) * NB + u0 + ul];
+  };
+  float sa0[SAB];
+  if (t0 < t1) {
+#pragma unroll
+    for (int j = 0; j < SAB; j++)
+      sa0[j] = load_sa(j * 64 + lane);
   }
 
   // Ring of PF stages; a stage = the weight tiles, their block scale and the
@@ -183,12 +199,27 @@ skinny_qint8_kernel(const DecodeParams p) {
     }
 #pragma unroll
     for (int mg = 0; mg < MG; mg++)
-      xreg[st][mg] = *reinterpret_cast<const i32x4*>(xrow[mg] + t * 64);
+      xreg[st][mg] = XOP ? xop[(int64_t)t * xstride + mg * 64] : *reinterpret_cast<const i32x4*>(xrow[mg] + t * 64);
   };
   if (t0 < t1) {
 #pragma unroll
     for (int i = 0; i < PF; i++)
       load_stage(i, t0 + i, false);
+    // the scales were requested first, so they are here long before the ring
+#pragma unroll
+    for (int j = 0; j < SAB; j++)
+      if (j * 64 + lane < nsa)
+        sa_s[j * 64 + lane] = sa0[j];
+    for (int i0 = SAB * 64; i0 < nsa; i0 += SAB * 64) { // more than 8 K blocks per wave: rare
+      float v[SAB];
+#pragma unroll
+      for (int j = 0; j < SAB; j++)
+        v[j] = load_sa(i0 + j * 64 + lane);
+#pragma unroll
+      for (int j = 0; j < SAB; j++)
+        if (i0 + j * 64 + lane < nsa)
+          sa_s[i0 + j * 64 + lane] = v[j];
+    }
   }
 
   f32x4 facc[NTW][MG];
@@ -229,20 +260,23 @@ skinny_qint8_kernel(const DecodeParams p) {
 
   int t = t0;
   if (TPB4) {
-    // full groups of PF tiles: static block boundaries (PF and t0 are multiples of 4)
-    for (; t + 2 * PF <= t1; t += PF) { // every reload of these groups is a real tile
+    // full trips of UN tiles: static ring slots and block boundaries (t0 is a
+    // multiple of 4), every reload a real tile
+    for (; t + UN + PF <= t1; t += UN) {
 #pragma unroll
-      for (int i = 0; i < PF; i++) {
-        consume(i, t + i, (i & 3) == 3, true);
-        load_stage(i, t + i + PF, true);
+      for (int i = 0; i < UN; i++) {
+        consume(i % PF, t + i, (i & 3) == 3, true);
+        load_stage(i % PF, t + i + PF, true);
+        __builtin_amdgcn_sched_barrier(0); // keep the reload right behind its stage: the ring stays PF deep
       }
     }
   }
-  // remaining tiles (and every tile when the K block is not 256 wide)
-  for (; t < t1; t += PF) {
+  // remaining tiles (and every tile when the K block is not 256 wide); the
+  // ring slot of tile tt is (tt - t0) % PF
+  for (int tb = t; tb < t1; tb += PF) {
 #pragma unroll
     for (int i = 0; i < PF; i++) {
-      const int tt = t + i;
+      const int tt = tb + i;
       if (tt < t1) {
         consume(i, tt, (tt + 1) % TPB == 0, false);
         if (tt + PF < t1)
@@ -420,6 +454,7 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
     for (int i = 0; i < PF; i++) {
       consume(i, t + i, (i & 3) == 3);
       load_stage(i, t + i + PF);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
   for (; t < t1; t += PF) {
@@ -511,6 +546,7 @@ skinny_mxfp4_kernel(const DecodeParams p) {
     for (int i = 0; i < PF; i++) {
       consume(i);
       load_stage(i, t + i + PF); // clamped past the end (re-reads the last tile, never consumed)
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
   for (; t < t1; t += PF) {
@@ -543,14 +579,18 @@ SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual
     pl.ntw = env_ntw;
   if (dual)
     pl.ntw = 2;
+  // more than 16 rows: these kernels run one workgroup per CU, so prefer a grid
+  // of at most 256 workgroups (a second, partly filled round costs a full one)
+  if (fmt == 1 && pl.mg > 1 && env_ntw == 0 && total_tiles > 512 && total_tiles <= 768)
+    pl.ntw = 3;
   // Wave-count window of the kernel instantiation that will run (register
   // budget: 16 waves leave 128 VGPRs per lane, 8 leave 256; the epilogue's
   // outputs-per-thread bound sets the minimum).  Waves beyond the number of K
   // units simply get an empty range.
   int max_w, min_w;
   if (fmt == 1) {
-    max_w = (pl.mg == 4 || (pl.mg == 2 && pl.ntw == 2)) ? 8 : 16;
-    min_w = (pl.mg == 4 || (pl.mg == 2 && pl.ntw == 2)) ? 8 : 4;
+    max_w = (pl.mg == 4 || (pl.mg == 2 && pl.ntw >= 2)) ? 8 : 16;
+    min_w = (pl.mg == 4 || (pl.mg == 2 && pl.ntw >= 2)) ? 8 : 4;
   } else {
     max_w = pl.ntw == 2 ? 8 : 16;
     min_w = 4;
@@ -592,18 +632,27 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
     return sk_launch(skinny_qint8_fq_kernel<1, 12, 16, 4>, p, grid, pl.waves, lds, stream);
   }
   size_t lds = ((size_t)pl.waves * pl.ntw * pl.mg * 256 + (size_t)pl.waves * pl.max_units * pl.mg * 16) * sizeof(float);
+#define SKQ(MG, NTW, PF, MAXW, MINW)                                                                   \
+  return p.mt > 0 ? sk_launch(skinny_qint8_kernel<MG, NTW, PF, MAXW, MINW, true>, p, grid, pl.waves, lds, stream) \
+                  : sk_launch(skinny_qint8_kernel<MG, NTW, PF, MAXW, MINW, false>, p, grid, pl.waves, lds, stream)
+  if (pl.ntw == 3) {
+    if (pl.mg == 2)
+      SKQ(2, 3, 4, 8, 8);
+    SKQ(4, 3, 3, 8, 8);
+  }
   if (pl.ntw == 2) {
     switch (pl.mg) {
-      case 1: return sk_launch(skinny_qint8_kernel<1, 2, 4, 16, 4>, p, grid, pl.waves, lds, stream);
-      case 2: return sk_launch(skinny_qint8_kernel<2, 2, 8, 8, 8>, p, grid, pl.waves, lds, stream);
-      default: return sk_launch(skinny_qint8_kernel<4, 2, 4, 8, 8>, p, grid, pl.waves, lds, stream);
+      case 1: SKQ(1, 2, 4, 16, 4);
+      case 2: SKQ(2, 2, 8, 8, 8);
+      default: SKQ(4, 2, 4, 8, 8);
     }
   }
   switch (pl.mg) {
-    case 1: return sk_launch(skinny_qint8_kernel<1, 1, 4, 16, 4>, p, grid, pl.waves, lds, stream);
-    case 2: return sk_launch(skinny_qint8_kernel<2, 1, 4, 16, 4>, p, grid, pl.waves, lds, stream);
-    default: return sk_launch(skinny_qint8_kernel<4, 1, 8, 8, 8>, p, grid, pl.waves, lds, stream);
+    case 1: SKQ(1, 1, 4, 16, 4);
+    case 2: SKQ(2, 1, 4, 16, 4);
+    default: SKQ(4, 1, 8, 8, 8);
   }
+#undef SKQ
 }
 
 hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream) {

@@ -287,8 +287,9 @@ def _prep_post(t, M, N, name, dev):
 
 
 def _qint8_scratch(x, M, K, qbs):
-    xq = torch.empty((M, K), dtype=torch.int8, device=x.device)
-    sa = torch.empty((M, K // qbs), dtype=torch.float32, device=x.device)
+    # the library may lay the quantized rows out in 64-row operand tiles
+    xq = torch.empty(((M + 63) // 64 * 64, K), dtype=torch.int8, device=x.device)
+    sa = torch.empty(((M + 63) // 64 * 64, K // qbs), dtype=torch.float32, device=x.device)
     return xq, sa
 
 
