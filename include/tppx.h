@@ -76,6 +76,10 @@ extern "C" {
 #define TPPX_FLAG_ACT_FP8 4      /* MXFP4 prefill: round activations to MXFP8
                                     (E4M3 + E8M0/32) and use the scaled
                                     f8f6f4 MFMA -- NOT the reference numerics */
+#define TPPX_FLAG_XQ_REUSE 8     /* QINT8, x != NULL: xq / sa still hold this
+                                    very x as an earlier call with the same
+                                    M, K, qbs, flags left it (several GEMMs on
+                                    one input): skip the re-quantization */
 
 typedef void* tppx_stream_t;
 
@@ -201,6 +205,19 @@ int tppx_swiglu_mxfp4(const void* x, const void* qw_gate, const void* sw_gate,
                       const void* sw_up, const void* bias_up, void* y,
                       int64_t M, int64_t N, int64_t K, int flags, void* ws,
                       int64_t ws_bytes, tppx_stream_t stream);
+
+/* ---- launch plans ------------------------------------------------------- */
+
+/* No counterpart in the reference.  Writes into buf, one line per kernel, what
+ * tppx_linear_mxfp4 / tppx_linear_qint8 would enqueue for this shape
+ * ("<kernel name as a profiler prints it> grid=XxYxZ block=B lds=L"), and
+ * launches nothing: for benchmarks and profilers that must name the kernel they
+ * time.  x_given = 0 describes the pre-quantized (x == NULL) case. */
+int tppx_plan_linear_mxfp4(int64_t M, int64_t N, int64_t K, int flags,
+                           int64_t ws_bytes, char* buf, int64_t buf_len);
+int tppx_plan_linear_qint8(int64_t M, int64_t N, int64_t K, int64_t qbs,
+                           int x_given, int flags, int64_t ws_bytes, char* buf,
+                           int64_t buf_len);
 
 #ifdef __cplusplus
 }

@@ -5,6 +5,9 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <cxxabi.h>
+#include <string>
+
 #include "tppx_common.h"
 #include "tppx_launch.h"
 
@@ -24,6 +27,33 @@ int check_hip(hipError_t e, const char* what) {
   if (e == hipSuccess)
     return TPPX_OK;
   return set_error(TPPX_EHIP, "%s: HIP error %d (%s)", what, (int)e, hipGetErrorString(e));
+}
+
+static thread_local std::string* g_plan = nullptr;
+
+bool plan_recording() {
+  return g_plan != nullptr;
+}
+
+void plan_note(const void* kernel_fn, dim3 grid, dim3 block, size_t lds_bytes) {
+  if (!g_plan)
+    return;
+  // name of the device function as a profiler prints it
+  std::string name = "?";
+  const char* mangled = hipKernelNameRefByPtr(kernel_fn, nullptr);
+  if (mangled && *mangled) {
+    int status = 0;
+    char* dem = abi::__cxa_demangle(mangled, nullptr, nullptr, &status);
+    name = (status == 0 && dem) ? dem : mangled;
+    free(dem);
+    const size_t paren = name.rfind('(');
+    if (paren != std::string::npos)
+      name.resize(paren);
+  }
+  char line[640];
+  snprintf(line, sizeof(line), "%s grid=%ux%ux%u block=%u lds=%zu\n", name.c_str(), grid.x, grid.y, grid.z, block.x,
+           lds_bytes);
+  *g_plan += line;
 }
 
 int env_int(const char* name, int dflt) {
@@ -66,7 +96,7 @@ static int check_common(const char* who, const void* x, int64_t M, int64_t K, in
   TPPX_REQUIRE(M > 0, TPPX_ESHAPE, "%s: M=%ld must be positive", who, (long)M);
   TPPX_REQUIRE(M < (1 << 24) && K < (1 << 24), TPPX_ESHAPE, "%s: M=%ld or K=%ld too large", who, (long)M, (long)K);
   TPPX_REQUIRE(n_segs >= 1 && n_segs <= TPPX_MAX_SEGS, TPPX_EINVAL, "%s: number of fused GEMMs %d not in 1..%d", who, n_segs, TPPX_MAX_SEGS);
-  TPPX_REQUIRE((flags & ~(TPPX_FLAG_FORCE_SKINNY | TPPX_FLAG_FORCE_TILED | TPPX_FLAG_ACT_FP8)) == 0, TPPX_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
+  TPPX_REQUIRE((flags & ~(TPPX_FLAG_FORCE_SKINNY | TPPX_FLAG_FORCE_TILED | TPPX_FLAG_ACT_FP8 | TPPX_FLAG_XQ_REUSE)) == 0, TPPX_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
   TPPX_REQUIRE(!((flags & TPPX_FLAG_FORCE_SKINNY) && (flags & TPPX_FLAG_FORCE_TILED)), TPPX_EINVAL, "%s: contradictory kernel-family flags", who);
   TPPX_REQUIRE(ws_bytes >= 0 && (ws_bytes == 0 || ws), TPPX_EINVAL, "%s: workspace size %ld given with a null workspace", who, (long)ws_bytes);
   TPPX_REQUIRE(ws == nullptr || (reinterpret_cast<uintptr_t>(ws) & 255u) == 0, TPPX_EINVAL, "%s: workspace not 256-byte aligned", who);
@@ -222,9 +252,10 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
   p.K = (int)K;
   p.units = (int)(K / qbs);
   p.tpb = (int)(qbs / 64);
+  const bool reuse = (flags & TPPX_FLAG_XQ_REUSE) != 0; // xq / sa still hold this x, quantized by an earlier call
   if (want_tiled(M, flags) && qbs % 128 == 0) {
-    if (x) {
-      rc = tppx_quant_act_int8(x, M, K, qbs, xq, sa, stream);
+    if (x && !reuse) {
+      rc = check_hip(launch_quant_act_int8(x, M, K, qbs, xq, sa, 0, stream), who);
       if (rc)
         return rc;
     }
@@ -243,8 +274,8 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
     // across workgroups
     DecodePlan pl = plan_decode(1, M, p.groups, p.total_tiles, p.units, p.tpb, false, (size_t)ws_bytes);
     bind_workspace(p, pl, ws);
-    if (x && !pl.fused_quant) {
-      rc = tppx_quant_act_int8(x, M, K, qbs, xq, sa, stream);
+    if (x && !pl.fused_quant && !reuse) {
+      rc = check_hip(launch_quant_act_int8(x, M, K, qbs, xq, sa, 0, stream), who);
       if (rc)
         return rc;
     }
@@ -257,7 +288,7 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
     // quantise straight into MFMA operand order: the GEMM then reads one
     // contiguous 1 KiB per operand instead of 16 rows x 64 B
     p.mt = sp.grid_y * sp.mg;
-    rc = check_hip(launch_quant_act_int8(x, M, K, qbs, xq, sa, p.mt, stream), who);
+    rc = reuse ? TPPX_OK : check_hip(launch_quant_act_int8(x, M, K, qbs, xq, sa, p.mt, stream), who);
     if (rc)
       return rc;
   }
@@ -322,4 +353,36 @@ extern "C" int tppx_multi_linear_qint8(const void* x, void* xq, void* sa,
                                        int flags, void* ws, int64_t ws_bytes,
                                        tppx_stream_t stream) {
   return run_qint8("tppx_multi_linear_qint8", x, xq, sa, segs, n_segs, M, K, qbs, flags, ws, ws_bytes, (hipStream_t)stream);
+}
+
+// ---- launch plans -----------------------------------------------------------
+static int emit_plan(const char* who, int rc, std::string& text, char* buf, int64_t buf_len) {
+  g_plan = nullptr;
+  if (rc)
+    return rc;
+  TPPX_REQUIRE(buf && buf_len > 0, TPPX_EINVAL, "%s: null or empty text buffer", who);
+  snprintf(buf, (size_t)buf_len, "%s", text.c_str());
+  return TPPX_OK;
+}
+
+extern "C" int tppx_plan_linear_mxfp4(int64_t M, int64_t N, int64_t K, int flags, int64_t ws_bytes, char* buf,
+                                      int64_t buf_len) {
+  // placeholder addresses: validated for alignment, never dereferenced
+  void* a = reinterpret_cast<void*>(uintptr_t(1) << 20);
+  std::string text;
+  g_plan = &text;
+  tppx_seg s = {a, a, nullptr, nullptr, nullptr, a, N, TPPX_POST_NONE, 1.0f};
+  int rc = run_mxfp4("tppx_plan_linear_mxfp4", a, &s, 1, M, K, flags, false, ws_bytes > 0 ? a : nullptr, ws_bytes, nullptr);
+  return emit_plan("tppx_plan_linear_mxfp4", rc, text, buf, buf_len);
+}
+
+extern "C" int tppx_plan_linear_qint8(int64_t M, int64_t N, int64_t K, int64_t qbs, int x_given, int flags,
+                                      int64_t ws_bytes, char* buf, int64_t buf_len) {
+  void* a = reinterpret_cast<void*>(uintptr_t(1) << 20);
+  std::string text;
+  g_plan = &text;
+  tppx_seg s = {a, a, nullptr, nullptr, nullptr, a, N, TPPX_POST_NONE, 1.0f};
+  int rc = run_qint8("tppx_plan_linear_qint8", x_given ? a : nullptr, a, a, &s, 1, M, K, qbs, flags,
+                     ws_bytes > 0 ? a : nullptr, ws_bytes, nullptr);
+  return emit_plan("tppx_plan_linear_qint8", rc, text, buf, buf_len);
 }

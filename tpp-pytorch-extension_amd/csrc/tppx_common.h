@@ -25,6 +25,19 @@ int check_hip(hipError_t e, const char* what);
       return ::tppx::set_error(code, __VA_ARGS__); \
   } while (0)
 
+// ---- launch plan recording (host) -------------------------------------------
+// While a plan is being recorded (tppx_plan_linear_*), launch sites describe
+// the kernel they would run and launch nothing.
+bool plan_recording();
+void plan_note(const void* kernel_fn, dim3 grid, dim3 block, size_t lds_bytes);
+#define TPPX_PLAN_ONLY(kern, grid, block, lds)                                  \
+  do {                                                                          \
+    if (::tppx::plan_recording()) {                                             \
+      ::tppx::plan_note(reinterpret_cast<const void*>(kern), grid, block, lds); \
+      return hipSuccess;                                                        \
+    }                                                                           \
+  } while (0)
+
 static inline bool aligned16(const void* p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }

@@ -529,6 +529,7 @@ splitk_finish_kernel(const DecodeParams p) {
 template <int MG, bool DUAL>
 static hipError_t launch_finish(const DecodeParams& p, const DecodePlan& pl, hipStream_t stream) {
   const int64_t waves = (int64_t)p.total_tiles * MG * pl.grid_y;
+  TPPX_PLAN_ONLY((splitk_finish_kernel<MG, DUAL>), dim3((unsigned)((waves + 3) / 4)), dim3(256), 0);
   splitk_finish_kernel<MG, DUAL><<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(p);
   return hipGetLastError();
 }
@@ -602,6 +603,7 @@ DecodePlan plan_decode(int fmt, int64_t M, int groups, int total_tiles, int unit
 
 template <typename K>
 static hipError_t launch_k(K kern, const DecodeParams& p, const DecodePlan& pl, hipStream_t stream) {
+  TPPX_PLAN_ONLY(kern, dim3(pl.grid_x, pl.grid_y), dim3(512), pl.lds_bytes);
   if (pl.lds_bytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds_bytes);

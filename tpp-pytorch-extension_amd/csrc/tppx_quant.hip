@@ -293,6 +293,7 @@ static inline unsigned grid_for(int64_t n, int block) {
 hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs, void* xq, void* sa, int mt,
                                  hipStream_t stream) {
   int64_t nthreads = M * (K / qbs) * 64;
+  TPPX_PLAN_ONLY(quant_act_int8_kernel, dim3(grid_for(nthreads, 256)), dim3(256), 0);
   quant_act_int8_kernel<<<grid_for(nthreads, 256), 256, 0, stream>>>((const uint16_t*)x, M, K, qbs, (int8_t*)xq,
                                                                     (float*)sa, mt);
   return hipGetLastError();

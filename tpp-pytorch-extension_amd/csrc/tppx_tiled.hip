@@ -310,6 +310,7 @@ tiled_qint8_kernel(const TiledParams p) {
 hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream) {
   const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
   const size_t lds = 2 * 2048 * 16;
+  TPPX_PLAN_ONLY(tiled_mxfp4_kernel, dim3(MB * NB), dim3(256), lds);
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_mxfp4_kernel),
@@ -325,6 +326,7 @@ hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream) {
 hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream) {
   const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
   const size_t lds = 2 * 1024 * 16 + 2 * 128 * sizeof(float);
+  TPPX_PLAN_ONLY(tiled_qint8_kernel, dim3(MB * NB), dim3(256), lds);
   tiled_qint8_kernel<<<dim3(MB * NB), dim3(256), lds, stream>>>(p);
   return hipGetLastError();
 }

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libtppx_hip.so")
 OK, EINVAL, ESHAPE, EUNSUPPORTED, EHIP = 0, -1, -2, -3, -4
 POST_NONE, POST_SILU, POST_MUL, POST_ADD_SCALE, POST_ADD2_SCALE, POST_GELU, POST_RELU = range(7)
 DT_F32, DT_BF16 = 0, 1
-FLAG_NONE, FLAG_FORCE_SKINNY, FLAG_FORCE_TILED, FLAG_ACT_FP8 = 0, 1, 2, 4
+FLAG_NONE, FLAG_FORCE_SKINNY, FLAG_FORCE_TILED, FLAG_ACT_FP8, FLAG_XQ_REUSE = 0, 1, 2, 4, 8
 
 
 class TppxError(RuntimeError):
@@ -58,6 +58,8 @@ SIGNATURES = {
     "tppx_multi_linear_mxfp4": [_vp, ctypes.POINTER(Seg), _i32, _i64, _i64, _i32, _vp, _i64, _vp],
     "tppx_multi_linear_qint8": [_vp, _vp, _vp, ctypes.POINTER(Seg), _i32, _i64, _i64, _i64, _i32, _vp, _i64, _vp],
     "tppx_swiglu_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp],
+    "tppx_plan_linear_mxfp4": [_i64, _i64, _i64, _i32, _i64, ctypes.c_char_p, _i64],
+    "tppx_plan_linear_qint8": [_i64, _i64, _i64, _i64, _i32, _i32, _i64, ctypes.c_char_p, _i64],
 }
 
 _lib = None
