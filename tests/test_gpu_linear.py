@@ -194,3 +194,81 @@ def test_prefill_qkv_and_swiglu_equal_composition():
     wg, wu = _make("mxfp4", 512, K, 91)[0], _make("mxfp4", 512, K, 92)[0]
     fused = ops.swiglu_gate_up(x, wg, wu)
     assert torch.equal(fused, ops.fc_mul(x, wu, None, ops.fc_silu(x, wg, None)))
+
+
+_FULL_UP = {}
+
+
+def _full_up():
+    """One Llama-7B up-projection weight (N=11008, K=4096), quantized once."""
+    if not _FULL_UP:
+        _FULL_UP["w"] = _make("qint8", 11008, 4096, 4242)
+    return _FULL_UP["w"]
+
+
+@pytest.mark.parametrize("M", [1, 4, 8, 16, 32, 40, 64])
+def test_cfg2_qint8_up_projection_full_size(M):
+    """The kernel variants that only large N selects (two and three channel
+    tiles per wave, ragged last workgroup: 688 tiles), at BASELINE's real shape."""
+    ops = _ops()
+    qw, q_or, s_or = _full_up()
+    x = randn_bf16((M, 4096), 1.0, 500 + M)
+    r = randn_bf16((M, 11008), 1.0, 600 + M)
+    y = torch.ops.tpp_llm.fc_add(x.cuda(), qw, torch.Tensor(), r.cuda(), 1.0)
+    ref = O.linear_qint8(t2bits(x), q_or, s_or, None, O.POST_ADD_SCALE, t2bits(r), None, 1.0, O.MODE_IDEAL)
+    pre = O.linear_qint8(t2bits(x), q_or, s_or)
+    assert_close_bf16(t2bits(y), ref, what=f"qint8 up-projection M={M}", pre_bits=pre)
+
+
+@pytest.mark.parametrize("M", [3, 24, 64])
+def test_qint8_prequantized_and_reused_activations(M):
+    """x == NULL takes row-major int8 activations + scales (the reference's
+    pre-quantized input); TPPX_FLAG_XQ_REUSE skips the re-quantization when a
+    second GEMM runs on the same input.  Both must give the bits of the plain
+    call, and the activation quantization itself must match the oracle."""
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    N, K, qbs = 512, 1024, 256
+    qw, q_or, s_or = _make("qint8", N, K, 31)
+    qw2, q_or2, s_or2 = _make("qint8", N, K, 32)
+    x = randn_bf16((M, K), 1.0, 33).cuda()
+    st = _lib.stream_of(x)
+    ws = _lib.workspace(x)
+    xq_rm = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    sa_rm = torch.empty((M, K // qbs), dtype=torch.float32, device="cuda")
+    _lib.check(L.tppx_quant_act_int8(x.data_ptr(), M, K, qbs, xq_rm.data_ptr(), sa_rm.data_ptr(), st))
+    xq_or, sa_or = O.quant_act_int8(t2bits(x.cpu()), qbs)
+    assert np.array_equal(xq_rm.cpu().numpy(), xq_or) and np.array_equal(sa_rm.cpu().numpy(), sa_or)
+
+    def call(xptr, xq, sa, w, flags):
+        qn, sn = w.native()
+        y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+        _lib.check(L.tppx_linear_qint8(xptr, xq.data_ptr(), sa.data_ptr(), qn.data_ptr(), sn.data_ptr(), None, None,
+                                       None, y.data_ptr(), M, N, K, qbs, 0, 1.0, flags, ws.data_ptr(), ws.numel(), st))
+        return y
+
+    xq = torch.empty(((M + 63) // 64 * 64, K), dtype=torch.int8, device="cuda")
+    sa = torch.empty(((M + 63) // 64 * 64, K // qbs), dtype=torch.float32, device="cuda")
+    y_plain = call(x.data_ptr(), xq, sa, qw, 0)
+    y2_reuse = call(x.data_ptr(), xq, sa, qw2, _lib.FLAG_XQ_REUSE)
+    y2_plain = call(x.data_ptr(), xq.clone().zero_(), sa.clone().zero_(), qw2, 0)
+    y_pre = call(None, xq_rm, sa_rm, qw, 0)
+    torch.cuda.synchronize()
+    ref = O.linear_qint8(t2bits(x.cpu()), q_or, s_or)
+    assert_close_bf16(t2bits(y_plain), ref, what=f"plain M={M}")
+    assert torch.equal(y_pre, y_plain), "pre-quantized input gives different bits"
+    assert torch.equal(y2_reuse, y2_plain), "reused activation quantization gives different bits"
+
+
+def test_launch_plan_names_the_kernels():
+    import ctypes
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    buf = ctypes.create_string_buffer(2048)
+    _lib.check(L.tppx_plan_linear_qint8(64, 11008, 4096, 256, 1, 0, 1 << 25, buf, len(buf)))
+    lines = buf.value.decode().strip().splitlines()
+    assert len(lines) == 2 and "quant_act_int8_kernel" in lines[0] and "skinny_qint8_kernel<" in lines[1]
+    _lib.check(L.tppx_plan_linear_qint8(1, 11008, 4096, 256, 1, 0, 1 << 25, buf, len(buf)))
+    assert buf.value.decode().count("\n") == 1 and "skinny_qint8_fq_kernel<" in buf.value.decode()
+    _lib.check(L.tppx_plan_linear_mxfp4(2048, 8192, 8192, 0, 0, buf, len(buf)))
+    assert "tiled_mxfp4_kernel" in buf.value.decode()

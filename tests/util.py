@@ -43,14 +43,19 @@ def err_stats(got_bits, ref_bits):
     }
 
 
-def assert_close_bf16(got_bits, ref_bits, ulps=1, rel_l2=4e-3, what=""):
+def assert_close_bf16(got_bits, ref_bits, ulps=1, rel_l2=4e-3, what="", pre_bits=None):
     """Tolerance of the parity tests: every element within `ulps` bf16 ulps of
     the oracle (|d| <= ulps * (2^-7 |ref| + 2^-8 rms(ref)), the second term
-    covering outputs that cancel to near zero) and relative L2 error <= rel_l2."""
+    covering outputs that cancel to near zero) and relative L2 error <= rel_l2.
+    `pre_bits` = the bf16 GEMM(+bias) tile before an additive post-op: one ulp
+    of THAT value is allowed too, since the post-op input can cancel it."""
     s = err_stats(got_bits, ref_bits)
     g = bits2f(got_bits).astype(np.float64)
     r = bits2f(ref_bits).astype(np.float64)
-    bound = ulps * (2.0 ** -7 * np.abs(r) + 2.0 ** -8 * s["rms"])
+    mag = np.abs(r)
+    if pre_bits is not None:
+        mag = np.maximum(mag, np.abs(bits2f(pre_bits).astype(np.float64)))
+    bound = ulps * (2.0 ** -7 * mag + 2.0 ** -8 * s["rms"])
     bad = np.abs(g - r) > bound
     assert not bad.any(), (
         f"{what}: {int(bad.sum())} elements beyond {ulps} ulp; max_abs={s['max_abs']:.4g} "
