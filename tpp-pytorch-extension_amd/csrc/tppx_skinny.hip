@@ -476,8 +476,10 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
 // DUAL: NTW = 2 accumulators = the gate tile and the up tile of one channel
 // tile; epilogue silu(gate) * up.
 // ---------------------------------------------------------------------------
-template <int NTW, int PF, int MAXW, int MINW, bool DUAL>
-__global__ void __launch_bounds__(MAXW * 64)
+// WPE = waves per SIMD the register budget must allow (2 workgroups of 8
+// waves per CU need 4).
+template <int NTW, int PF, int MAXW, int MINW, bool DUAL, int WPE = 1>
+__global__ void __launch_bounds__(MAXW * 64, WPE)
 skinny_mxfp4_kernel(const DecodeParams p) {
   extern __shared__ __align__(16) float sk_lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -639,7 +641,7 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
   if (pl.ntw == 3) {
     if (pl.mg == 2)
       SKQ(2, 3, 4, 8, 8);
-    SKQ(4, 3, 3, 8, 8);
+    SKQ(4, 3, 2, 8, 8);
   }
   if (pl.ntw == 2) {
     switch (pl.mg) {
@@ -660,9 +662,9 @@ hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual,
   dim3 grid(p.groups, pl.grid_y);
   size_t lds = (size_t)pl.waves * pl.ntw * 256 * sizeof(float);
   if (dual)
-    return sk_launch(skinny_mxfp4_kernel<2, 6, 8, 4, true>, p, grid, pl.waves, lds, stream);
+    return sk_launch(skinny_mxfp4_kernel<2, 2, 8, 4, true, 4>, p, grid, pl.waves, lds, stream);
   if (pl.ntw == 2)
-    return sk_launch(skinny_mxfp4_kernel<2, 6, 8, 4, false>, p, grid, pl.waves, lds, stream);
+    return sk_launch(skinny_mxfp4_kernel<2, 2, 8, 4, false, 4>, p, grid, pl.waves, lds, stream);
   return sk_launch(skinny_mxfp4_kernel<1, 4, 16, 4, false>, p, grid, pl.waves, lds, stream);
 }
 
