@@ -307,7 +307,201 @@ tiled_qint8_kernel(const TiledParams p) {
   tiled_epilogue(p, facc, m_wg + wm * 64, tile_base);
 }
 
+// ---------------------------------------------------------------------------
+// Large-M MXFP4 kernel: workgroup tile 256 (M) x 256 (N), 8 waves in a 2 x 4
+// grid (two per SIMD, so one wave's conversions and LDS reads run under the
+// other's MFMAs), each wave 128 x 64 = 8 x 4 MFMA tiles (128 accumulator
+// registers).  Every expanded weight operand feeds 8 MFMAs.
+//   A: rows are read from global memory row-contiguously (a wave instruction
+//      covers 4 rows x 256 B) and written into LDS in MFMA operand order; the
+//      16-byte slot of row m inside its 256-byte group is XOR-ed with the
+//      chunk index so that both the scattered writes and the operand reads
+//      are bank-conflict free.  Two LDS buffers of 64 KiB.
+//   B: native tiles straight from global/L2, next K step prefetched.
+// LDS slot of (row tile mt, step j, K group g, row m) = (mt*4 + j)*64 + g*16 + (m ^ (g*4 + j)).
+// ---------------------------------------------------------------------------
+// Epilogue of a 128 x 64 wave tile through a wave-private LDS region: the
+// fp32 sums of 64 rows at a time are written there (statically indexed, so the
+// accumulators stay in registers), then read back row-contiguously; every
+// lane finishes 8 adjacent channels and writes them with one 16-byte store.
+constexpr int EP_LD = 68; // floats per staged row: 64 + 4 keeps the 4-row lane groups on distinct banks
+__device__ __forceinline__ void big_epilogue(const TiledParams& p, f32x4 (&acc)[8][4], float* stage, int m_base,
+                                             int tile_base) {
+  const int lane = threadIdx.x & 63;
+  const int cx = (lane & 7) * 8; // first of this lane's 8 channels inside the wave tile
+  const int tile = tile_base + (cx >> 4);
+  const bool tile_ok = tile < p.tiles;
+  const int n = min(tile, p.tiles - 1) * 16 + (cx & 15);
+  float bias[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    bias[e] = p.bias ? bf16_bits_to_f32(p.bias[n + e]) : 0.0f;
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          stage[(mt * 16 + (lane >> 4) * 4 + r) * EP_LD + nt * 16 + (lane & 15)] = acc[h * 4 + mt][nt][r];
+    // same wave wrote and reads: no barrier, the compiler orders the LDS accesses
+    for (int it = 0; it < 8; it++) {
+      const int row = it * 8 + (lane >> 3);
+      const int m = m_base + h * 64 + row;
+      const f32x4 v0 = *reinterpret_cast<const f32x4*>(stage + row * EP_LD + cx);
+      const f32x4 v1 = *reinterpret_cast<const f32x4*>(stage + row * EP_LD + cx + 4);
+      if (tile_ok && m < p.M) {
+        const int64_t o = (int64_t)m * p.N + n;
+        uint4 i1 = make_uint4(0, 0, 0, 0), i2 = make_uint4(0, 0, 0, 0);
+        if (p.post_in)
+          i1 = *reinterpret_cast<const uint4*>(p.post_in + o);
+        if (p.post_in2)
+          i2 = *reinterpret_cast<const uint4*>(p.post_in2 + o);
+        const uint32_t w1[4] = {i1.x, i1.y, i1.z, i1.w}, w2[4] = {i2.x, i2.y, i2.z, i2.w};
+        uint32_t out[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float lo = (e < 2 ? v0[2 * e] : v1[2 * e - 4]) + bias[2 * e];
+          const float hi = (e < 2 ? v0[2 * e + 1] : v1[2 * e - 3]) + bias[2 * e + 1];
+          const uint32_t a = apply_post_bits(lo, p.post_op, w1[e] & 0xffffu, w2[e] & 0xffffu, p.post_scale);
+          const uint32_t b = apply_post_bits(hi, p.post_op, w1[e] >> 16, w2[e] >> 16, p.post_scale);
+          out[e] = (a & 0xffffu) | (b << 16);
+        }
+        *reinterpret_cast<uint4*>(p.y + o) = make_uint4(out[0], out[1], out[2], out[3]);
+      }
+    }
+  }
+}
+
+__global__ void __launch_bounds__(512)
+big_mxfp4_kernel(const TiledParams p) {
+  extern __shared__ __align__(16) uint8_t tl_lds[];
+  bf16x8* As = reinterpret_cast<bf16x8*>(tl_lds); // 2 buffers x 4096 slots of 16 B
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int MB = (p.M + 255) >> 8, NB = (p.tiles + 15) >> 4;
+  int bm, bn;
+  tile_of_block(MB, NB, bm, bn);
+  const int KT = p.K >> 7;
+  const int m_wg = bm * 256;
+  const int tile_base = bn * 16 + wn * 4;
+
+  const i32x4* wqb = reinterpret_cast<const i32x4*>(p.qw) + lane;
+  const uint8_t* wsb = reinterpret_cast<const uint8_t*>(p.sw) + lane;
+  int woff[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; nt++)
+    woff[nt] = min(tile_base + nt, p.tiles - 1) * KT * 64;
+
+  // A staging: thread = (16-byte chunk c of a 256-byte row segment, row r0 of a 32-row pass)
+  const int c = tid & 15, r0 = tid >> 4;
+  const uint16_t* xb = reinterpret_cast<const uint16_t*>(p.x) + c * 8;
+  const int wslot = ((r0 >> 4) * 4 + (c & 3)) * 64 + (c >> 2) * 16 + ((r0 & 15) ^ c); // + pass*512
+  int rd[4]; // operand read slot of this lane for step j (+ mt*256)
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+    rd[j] = j * 64 + (lane >> 4) * 16 + ((lane & 15) ^ ((lane >> 4) * 4 + j));
+
+  bf16x8 areg[4]; // half of the next A tile at a time (passes h*4 .. h*4+3)
+  i32x4 breg[4];
+  uint32_t bsc[4];
+  auto load_a = [&](int ks, int h) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int row = min(m_wg + (h * 4 + i) * 32 + r0, p.M - 1);
+      areg[i] = *reinterpret_cast<const bf16x8*>(xb + (int64_t)row * p.K + ks * 128);
+    }
+  };
+  auto load_b = [&](int ks) {
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+      breg[nt] = wqb[woff[nt] + ks * 64];
+      bsc[nt] = wsb[woff[nt] + ks * 64];
+    }
+  };
+  auto store_a = [&](int buf, int h) {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      As[buf * 4096 + (h * 4 + i) * 512 + wslot] = areg[i];
+  };
+
+  f32x4 acc[8][4];
+#pragma unroll
+  for (int mt = 0; mt < 8; mt++)
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++)
+      acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  load_a(0, 0);
+  store_a(0, 0);
+  load_a(0, 1);
+  store_a(0, 1);
+  load_b(0);
+  __syncthreads();
+  for (int ks = 0; ks < KT; ks++) {
+    const int buf = ks & 1;
+    const bool more = ks + 1 < KT;
+    i32x4 bcur[4];
+    float sc[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+      bcur[nt] = breg[nt];
+      sc[nt] = e8m0_to_f32(bsc[nt]);
+    }
+    if (more) {
+      load_b(ks + 1);
+      load_a(ks + 1, 0);
+    }
+    const bf16x8* Ab = As + buf * 4096 + (wm * 8) * 256;
+    // 32 operand reads per K step (q = j*8 + mt), kept two ahead of the MFMAs
+    // that consume them so the LDS latency is covered by 8 MFMAs
+    bf16x8 ar[3], b[4];
+    ar[0] = Ab[0 * 256 + rd[0]];
+    ar[1] = Ab[1 * 256 + rd[0]];
+#pragma unroll
+    for (int q = 0; q < 32; q++) {
+      const int j = q >> 3, mt = q & 7;
+      if (mt == 0) {
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+          b[nt] = tl_cvt_fp4x8((uint32_t)bcur[nt][j], sc[nt]);
+      }
+      if (q + 2 < 32)
+        ar[(q + 2) % 3] = Ab[((q + 2) & 7) * 256 + rd[(q + 2) >> 3]];
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ar[q % 3], b[nt], acc[mt][nt], 0, 0, 0);
+      if (q == 15 && more) { // first half has had two steps of MFMAs to land
+        store_a(buf ^ 1, 0);
+        load_a(ks + 1, 1);
+      }
+    }
+    if (more)
+      store_a(buf ^ 1, 1);
+    __syncthreads();
+  }
+  // every wave has left the main loop (barrier above): LDS is free for the epilogue staging
+  big_epilogue(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * 128, tile_base);
+}
+
 hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream) {
+  if (p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192)) {
+    const int MB = (p.M + 255) / 256, NB = (p.tiles + 15) / 16;
+    const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the two 64 KiB A buffers
+    TPPX_PLAN_ONLY(big_mxfp4_kernel, dim3(MB * NB), dim3(512), lds);
+    static bool big_attr_done = false;
+    if (!big_attr_done) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_mxfp4_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess)
+        return e;
+      big_attr_done = true;
+    }
+    big_mxfp4_kernel<<<dim3(MB * NB), dim3(512), lds, stream>>>(p);
+    return hipGetLastError();
+  }
+
   const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
   const size_t lds = 2 * 2048 * 16;
   TPPX_PLAN_ONLY(tiled_mxfp4_kernel, dim3(MB * NB), dim3(256), lds);
