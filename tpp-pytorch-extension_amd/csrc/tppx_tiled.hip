@@ -20,6 +20,8 @@
 // MFMA operand convention (A = activations, B = weights):
 //   lane l supplies row/col (l & 15) and K group (l >> 4);
 //   result register r of lane l is D[m = (l >> 4) * 4 + r][n = l & 15].
+#include <type_traits>
+
 #include "tppx_common.h"
 #include "tppx_launch.h"
 
@@ -309,15 +311,16 @@ tiled_qint8_kernel(const TiledParams p) {
 
 // ---------------------------------------------------------------------------
 // Large-M MXFP4 kernel: workgroup tile 256 (M) x 256 (N), 8 waves in a 2 x 4
-// grid (two per SIMD, so one wave's conversions and LDS reads run under the
-// other's MFMAs), each wave 128 x 64 = 8 x 4 MFMA tiles (128 accumulator
-// registers).  Every expanded weight operand feeds 8 MFMAs.
+// grid (two per SIMD), each wave 128 x 64 = 8 x 4 MFMA tiles (128 accumulator
+// registers).  Every expanded weight operand feeds 8 MFMAs, every activation
+// operand read from LDS feeds 4 and is requested two MFMA groups ahead.
 //   A: rows are read from global memory row-contiguously (a wave instruction
 //      covers 4 rows x 256 B) and written into LDS in MFMA operand order; the
 //      16-byte slot of row m inside its 256-byte group is XOR-ed with the
 //      chunk index so that both the scattered writes and the operand reads
-//      are bank-conflict free.  Two LDS buffers of 64 KiB.
-//   B: native tiles straight from global/L2, next K step prefetched.
+//      are bank-conflict free.  Two LDS buffers of 64 KiB; the next tile is
+//      fetched a quarter at a time to keep the staging registers few.
+//   B: native tiles straight from global/L2, fetched half a K step ahead.
 // LDS slot of (row tile mt, step j, K group g, row m) = (mt*4 + j)*64 + g*16 + (m ^ (g*4 + j)).
 // ---------------------------------------------------------------------------
 // Epilogue of a 128 x 64 wave tile through a wave-private LDS region: the
@@ -374,6 +377,28 @@ __device__ __forceinline__ void big_epilogue(const TiledParams& p, f32x4 (&acc)[
   }
 }
 
+// LDS operand reads issued by hand, so that they can be kept several MFMA
+// groups ahead of their use: the compiler does not track them, the waits are
+// explicit (LDS operations complete in issue order, so "at most N younger
+// operations outstanding" is enough) and are tied to the destination
+// registers so that nothing using them can move above the wait.
+template <int OFF>
+__device__ __forceinline__ void lds_read_b128_async(i32x4& dst, uint32_t byte_addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(byte_addr), "n"(OFF));
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_keep(i32x4& r) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(r) : "n"(N));
+}
+// compile-time loop: f(std::integral_constant<int, I>) for I in [B, E)
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
 __global__ void __launch_bounds__(512)
 big_mxfp4_kernel(const TiledParams p) {
   extern __shared__ __align__(16) uint8_t tl_lds[];
@@ -387,43 +412,71 @@ big_mxfp4_kernel(const TiledParams p) {
   const int m_wg = bm * 256;
   const int tile_base = bn * 16 + wn * 4;
 
-  const i32x4* wqb = reinterpret_cast<const i32x4*>(p.qw) + lane;
-  const uint8_t* wsb = reinterpret_cast<const uint8_t*>(p.sw) + lane;
-  int woff[4];
+  // Every global address below is a uniform base pointer plus a 32-bit byte
+  // offset per lane (the launcher checks that the operands are smaller than
+  // 4 GiB): one offset register instead of a 64-bit pointer pair per stream.
+  const char* qwb = reinterpret_cast<const char*>(p.qw);
+  const char* swb = reinterpret_cast<const char*>(p.sw);
+  uint32_t woff[4]; // slot index of this lane in tile nt at K step 0
 #pragma unroll
   for (int nt = 0; nt < 4; nt++)
-    woff[nt] = min(tile_base + nt, p.tiles - 1) * KT * 64;
+    woff[nt] = (uint32_t)(min(tile_base + nt, p.tiles - 1) * KT * 64 + lane);
 
   // A staging: thread = (16-byte chunk c of a 256-byte row segment, row r0 of a 32-row pass)
   const int c = tid & 15, r0 = tid >> 4;
-  const uint16_t* xb = reinterpret_cast<const uint16_t*>(p.x) + c * 8;
   const int wslot = ((r0 >> 4) * 4 + (c & 3)) * 64 + (c >> 2) * 16 + ((r0 & 15) ^ c); // + pass*512
-  int rd[4]; // operand read slot of this lane for step j (+ mt*256)
+  uint32_t rdb[4]; // byte offset of this lane's operand slot for step j (+ mt*4096)
 #pragma unroll
   for (int j = 0; j < 4; j++)
-    rd[j] = j * 64 + (lane >> 4) * 16 + ((lane & 15) ^ ((lane >> 4) * 4 + j));
+    rdb[j] = (uint32_t)(j * 64 + (lane >> 4) * 16 + ((lane & 15) ^ ((lane >> 4) * 4 + j))) * 16u;
+  const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>(tl_lds); // LDS byte address of the buffers
+  // rows of this thread: m_wg + pass*32 + r0; past the end of the matrix they
+  // re-read the last row (those outputs are never stored)
+  const bool full = m_wg + 256 <= p.M; // uniform
+  const char* xbase = reinterpret_cast<const char*>(p.x);
+  const uint32_t xoff = (uint32_t)(min(m_wg + r0, p.M - 1) * p.K + c * 8) * 2u;
+  const uint32_t pass_stride = (uint32_t)(32 * p.K) * 2u; // uniform
 
-  bf16x8 areg[4]; // half of the next A tile at a time (passes h*4 .. h*4+3)
-  i32x4 breg[4];
-  uint32_t bsc[4];
+  bf16x8 areg[2]; // a quarter of the next A tile at a time (passes h*2, h*2+1)
   auto load_a = [&](int ks, int h) {
+    if (full) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int row = min(m_wg + (h * 4 + i) * 32 + r0, p.M - 1);
-      areg[i] = *reinterpret_cast<const bf16x8*>(xb + (int64_t)row * p.K + ks * 128);
-    }
-  };
-  auto load_b = [&](int ks) {
+      for (int i = 0; i < 2; i++)
+        areg[i] = *reinterpret_cast<const bf16x8*>(xbase + (size_t)(xoff + (uint32_t)(h * 2 + i) * pass_stride + (uint32_t)ks * 256u));
+    } else {
 #pragma unroll
-    for (int nt = 0; nt < 4; nt++) {
-      breg[nt] = wqb[woff[nt] + ks * 64];
-      bsc[nt] = wsb[woff[nt] + ks * 64];
+      for (int i = 0; i < 2; i++) {
+        const int row = min(m_wg + (h * 2 + i) * 32 + r0, p.M - 1);
+        areg[i] = *reinterpret_cast<const bf16x8*>(xbase + (size_t)((uint32_t)(row * p.K + c * 8 + ks * 128) * 2u));
+      }
     }
   };
   auto store_a = [&](int buf, int h) {
 #pragma unroll
-    for (int i = 0; i < 4; i++)
-      As[buf * 4096 + (h * 4 + i) * 512 + wslot] = areg[i];
+    for (int i = 0; i < 2; i++)
+      As[buf * 4096 + (h * 2 + i) * 512 + wslot] = areg[i];
+  };
+  // B of one K step: 4 tiles x 4 dwords (one per step j) and the scale factors
+  uint32_t bc[4][4];
+  float sc[4];
+  i32x4 bnext[4];
+  uint32_t snext[4];
+  auto load_b = [&](int ks) {
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+      const uint32_t slot = woff[nt] + (uint32_t)ks * 64u;
+      bnext[nt] = *reinterpret_cast<const i32x4*>(qwb + (size_t)(slot * 16u));
+      snext[nt] = *reinterpret_cast<const uint8_t*>(swb + (size_t)slot);
+    }
+  };
+  auto take_b = [&]() {
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        bc[nt][j] = (uint32_t)bnext[nt][j];
+      sc[nt] = e8m0_to_f32(snext[nt]);
+    }
   };
 
   f32x4 acc[8][4];
@@ -433,52 +486,57 @@ big_mxfp4_kernel(const TiledParams p) {
     for (int nt = 0; nt < 4; nt++)
       acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  load_a(0, 0);
-  store_a(0, 0);
-  load_a(0, 1);
-  store_a(0, 1);
+#pragma unroll
+  for (int h = 0; h < 4; h++) {
+    load_a(0, h);
+    store_a(0, h);
+  }
   load_b(0);
   __syncthreads();
   for (int ks = 0; ks < KT; ks++) {
     const int buf = ks & 1;
     const bool more = ks + 1 < KT;
-    i32x4 bcur[4];
-    float sc[4];
-#pragma unroll
-    for (int nt = 0; nt < 4; nt++) {
-      bcur[nt] = breg[nt];
-      sc[nt] = e8m0_to_f32(bsc[nt]);
-    }
-    if (more) {
-      load_b(ks + 1);
+    take_b();
+    if (more)
       load_a(ks + 1, 0);
-    }
-    const bf16x8* Ab = As + buf * 4096 + (wm * 8) * 256;
     // 32 operand reads per K step (q = j*8 + mt), kept two ahead of the MFMAs
     // that consume them so the LDS latency is covered by 8 MFMAs
-    bf16x8 ar[3], b[4];
-    ar[0] = Ab[0 * 256 + rd[0]];
-    ar[1] = Ab[1 * 256 + rd[0]];
-#pragma unroll
-    for (int q = 0; q < 32; q++) {
-      const int j = q >> 3, mt = q & 7;
-      if (mt == 0) {
+    const uint32_t abase = lds0 + (uint32_t)(buf * 4096 + wm * 8 * 256) * 16u;
+    i32x4 ar[3];
+    bf16x8 b[4];
+    lds_read_b128_async<0>(ar[0], abase + rdb[0]);
+    lds_read_b128_async<4096>(ar[1], abase + rdb[0]);
+    static_for<0, 32>([&](auto Q) {
+      constexpr int q = decltype(Q)::value;
+      constexpr int j = q >> 3, mt = q & 7;
+      if constexpr (mt == 0) {
 #pragma unroll
         for (int nt = 0; nt < 4; nt++)
-          b[nt] = tl_cvt_fp4x8((uint32_t)bcur[nt][j], sc[nt]);
+          b[nt] = tl_cvt_fp4x8(bc[nt][j], sc[nt]);
       }
-      if (q + 2 < 32)
-        ar[(q + 2) % 3] = Ab[((q + 2) & 7) * 256 + rd[(q + 2) >> 3]];
+      if constexpr (q + 2 < 32) {
+        lds_read_b128_async<((q + 2) & 7) * 4096>(ar[(q + 2) % 3], abase + rdb[(q + 2) >> 3]);
+        lds_wait_keep<2>(ar[q % 3]);
+      } else if constexpr (q + 1 < 32) {
+        lds_wait_keep<1>(ar[q % 3]);
+      } else {
+        lds_wait_keep<0>(ar[q % 3]);
+      }
+      const bf16x8 a = __builtin_bit_cast(bf16x8, ar[q % 3]);
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
-        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ar[q % 3], b[nt], acc[mt][nt], 0, 0, 0);
-      if (q == 15 && more) { // first half has had two steps of MFMAs to land
-        store_a(buf ^ 1, 0);
-        load_a(ks + 1, 1);
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[nt], acc[mt][nt], 0, 0, 0);
+      if constexpr (mt == 7 && j < 3) {
+        if (more) { // the quarter fetched one step ago has landed: store it, fetch the next
+          store_a(buf ^ 1, j);
+          load_a(ks + 1, j + 1);
+          if (j == 1)
+            load_b(ks + 1); // dwords of steps 0 and 1 of the current B are dead by now
+        }
       }
-    }
+    });
     if (more)
-      store_a(buf ^ 1, 1);
+      store_a(buf ^ 1, 3);
     __syncthreads();
   }
   // every wave has left the main loop (barrier above): LDS is free for the epilogue staging
@@ -486,7 +544,9 @@ big_mxfp4_kernel(const TiledParams p) {
 }
 
 hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream) {
-  if (p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192)) {
+  // the large-M kernel addresses its operands with 32-bit byte offsets
+  const bool fits32 = (int64_t)p.M * p.K * 2 < ((int64_t)1 << 32) && (int64_t)p.tiles * 8 * p.K < ((int64_t)1 << 32);
+  if (p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && fits32) {
     const int MB = (p.M + 255) / 256, NB = (p.tiles + 15) / 16;
     const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the two 64 KiB A buffers
     TPPX_PLAN_ONLY(big_mxfp4_kernel, dim3(MB * NB), dim3(512), lds);
