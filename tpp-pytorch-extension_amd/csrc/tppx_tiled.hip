@@ -422,39 +422,42 @@ big_mxfp4_kernel(const TiledParams p) {
   for (int nt = 0; nt < 4; nt++)
     woff[nt] = (uint32_t)(min(tile_base + nt, p.tiles - 1) * KT * 64 + lane);
 
-  // A staging: thread = (16-byte chunk c of a 256-byte row segment, row r0 of a 32-row pass)
-  const int c = tid & 15, r0 = tid >> 4;
-  const int wslot = ((r0 >> 4) * 4 + (c & 3)) * 64 + (c >> 2) * 16 + ((r0 & 15) ^ c); // + pass*512
-  uint32_t rdb[4]; // byte offset of this lane's operand slot for step j (+ mt*4096)
-#pragma unroll
-  for (int j = 0; j < 4; j++)
-    rdb[j] = (uint32_t)(j * 64 + (lane >> 4) * 16 + ((lane & 15) ^ ((lane >> 4) * 4 + j))) * 16u;
+  // A tile (256 rows x 128 K, 64 KiB): 64 blocks of 4 rows x 256 B go from
+  // global memory straight into LDS, one wave instruction per block (lane =
+  // row r of the block, 16-byte chunk).  The LDS image of an instruction is
+  // lane-linear, so the swizzle is applied on the global side: the lane at
+  // position ch of row m fetches chunk ch ^ (m & 15).  Operand reads of one K
+  // group (16 rows, same chunk) then fall on 16 different bank groups.
+  //   LDS byte address of chunk ck of row m of row tile mt:
+  //     mt*4096 + (m>>2)*1024 + (m&3)*256 + ((ck ^ m) & 15)*16
   const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>(tl_lds); // LDS byte address of the buffers
-  // rows of this thread: m_wg + pass*32 + r0; past the end of the matrix they
-  // re-read the last row (those outputs are never stored)
-  const bool full = m_wg + 256 <= p.M; // uniform
+  uint32_t rdb[4]; // byte offset of this lane's operand for step j (+ mt*4096): chunk ck = g*4 + j
+  {
+    const int m = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      rdb[j] = (uint32_t)((m >> 2) * 1024 + (m & 3) * 256 + (((g * 4 + j) ^ m) & 15) * 16);
+  }
   const char* xbase = reinterpret_cast<const char*>(p.x);
-  const uint32_t xoff = (uint32_t)(min(m_wg + r0, p.M - 1) * p.K + c * 8) * 2u;
-  const uint32_t pass_stride = (uint32_t)(32 * p.K) * 2u; // uniform
-
-  bf16x8 areg[2]; // a quarter of the next A tile at a time (passes h*2, h*2+1)
-  auto load_a = [&](int ks, int h) {
-    if (full) {
+  // this wave's 8 blocks: blk = wave*8 + i -> rows blk*4 + (lane>>4)
+  const int rin = (lane >> 4);          // row inside the block
+  const int ch = lane & 15;             // chunk position of this lane inside the row
+  uint32_t xoff[8];                     // byte offset of this lane's source at K step 0
 #pragma unroll
-      for (int i = 0; i < 2; i++)
-        areg[i] = *reinterpret_cast<const bf16x8*>(xbase + (size_t)(xoff + (uint32_t)(h * 2 + i) * pass_stride + (uint32_t)ks * 256u));
-    } else {
+  for (int i = 0; i < 8; i++) {
+    const int blk = wave * 8 + i;
+    const int m16 = (blk & 3) * 4 + rin;               // row inside its 16-row tile
+    const int row = min(m_wg + blk * 4 + rin, p.M - 1); // past the end: re-read the last row (never stored)
+    xoff[i] = (uint32_t)(row * p.K + ((ch ^ m16) & 15) * 8) * 2u;
+  }
+  auto load_a = [&](int ks, int buf) {
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
-        const int row = min(m_wg + (h * 2 + i) * 32 + r0, p.M - 1);
-        areg[i] = *reinterpret_cast<const bf16x8*>(xbase + (size_t)((uint32_t)(row * p.K + c * 8 + ks * 128) * 2u));
-      }
+    for (int i = 0; i < 8; i++) {
+      const char* src = xbase + (size_t)(xoff[i] + (uint32_t)ks * 256u);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)(tl_lds + buf * 65536 + (wave * 8 + i) * 1024),
+                                       16, 0, 0);
     }
-  };
-  auto store_a = [&](int buf, int h) {
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-      As[buf * 4096 + (h * 2 + i) * 512 + wslot] = areg[i];
   };
   // B of one K step: 4 tiles x 4 dwords (one per step j) and the scale factors
   uint32_t bc[4][4];
@@ -486,11 +489,7 @@ big_mxfp4_kernel(const TiledParams p) {
     for (int nt = 0; nt < 4; nt++)
       acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-#pragma unroll
-  for (int h = 0; h < 4; h++) {
-    load_a(0, h);
-    store_a(0, h);
-  }
+  load_a(0, 0);
   load_b(0);
   __syncthreads();
   for (int ks = 0; ks < KT; ks++) {
@@ -498,10 +497,10 @@ big_mxfp4_kernel(const TiledParams p) {
     const bool more = ks + 1 < KT;
     take_b();
     if (more)
-      load_a(ks + 1, 0);
+      load_a(ks + 1, buf ^ 1); // lands in the other buffer during this step's MFMAs
     // 32 operand reads per K step (q = j*8 + mt), kept two ahead of the MFMAs
     // that consume them so the LDS latency is covered by 8 MFMAs
-    const uint32_t abase = lds0 + (uint32_t)(buf * 4096 + wm * 8 * 256) * 16u;
+    const uint32_t abase = lds0 + (uint32_t)(buf * 65536 + wm * 8 * 4096);
     i32x4 ar[3];
     bf16x8 b[4];
     lds_read_b128_async<0>(ar[0], abase + rdb[0]);
@@ -526,18 +525,12 @@ big_mxfp4_kernel(const TiledParams p) {
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
         acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[nt], acc[mt][nt], 0, 0, 0);
-      if constexpr (mt == 7 && j < 3) {
-        if (more) { // the quarter fetched one step ago has landed: store it, fetch the next
-          store_a(buf ^ 1, j);
-          load_a(ks + 1, j + 1);
-          if (j == 1)
-            load_b(ks + 1); // dwords of steps 0 and 1 of the current B are dead by now
-        }
+      if constexpr (q == 15) {
+        if (more)
+          load_b(ks + 1); // dwords of steps 0 and 1 of the current B are dead by now
       }
     });
-    if (more)
-      store_a(buf ^ 1, 3);
-    __syncthreads();
+    __syncthreads(); // waits for this wave's direct-to-LDS loads, then for everybody's
   }
   // every wave has left the main loop (barrier above): LDS is free for the epilogue staging
   big_epilogue(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * 128, tile_base);
