@@ -403,7 +403,8 @@ __global__ void __launch_bounds__(512)
 big_mxfp4_kernel(const TiledParams p) {
   extern __shared__ __align__(16) uint8_t tl_lds[];
   bf16x8* As = reinterpret_cast<bf16x8*>(tl_lds); // 2 buffers x 4096 slots of 16 B
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform: keeps LDS bases and block indices scalar
   const int wm = wave & 1, wn = wave >> 1;
   const int MB = (p.M + 255) >> 8, NB = (p.tiles + 15) >> 4;
   int bm, bn;
@@ -442,19 +443,24 @@ big_mxfp4_kernel(const TiledParams p) {
   // this wave's 8 blocks: blk = wave*8 + i -> rows blk*4 + (lane>>4)
   const int rin = (lane >> 4);          // row inside the block
   const int ch = lane & 15;             // chunk position of this lane inside the row
-  uint32_t xoff[8];                     // byte offset of this lane's source at K step 0
-#pragma unroll
-  for (int i = 0; i < 8; i++) {
-    const int blk = wave * 8 + i;
-    const int m16 = (blk & 3) * 4 + rin;               // row inside its 16-row tile
-    const int row = min(m_wg + blk * 4 + rin, p.M - 1); // past the end: re-read the last row (never stored)
-    xoff[i] = (uint32_t)(row * p.K + ((ch ^ m16) & 15) * 8) * 2u;
-  }
+  // source byte offset of block i at K step ks:
+  //   row(i) * K * 2 + ((ch ^ m16(i)) & 15) * 16 + ks * 256, row(i) = m_wg + (wave*8 + i)*4 + rin,
+  //   m16(i) = (i & 3)*4 + rin (wave*8 is a multiple of 4)
+  const bool full = m_wg + 256 <= p.M; // uniform
+  const uint32_t xrow0 = (uint32_t)((m_wg + wave * 32 + rin) * p.K) * 2u;
+  const uint32_t blk_stride = (uint32_t)(4 * p.K) * 2u; // uniform
   auto load_a = [&](int ks, int buf) {
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-      const char* src = xbase + (size_t)(xoff[i] + (uint32_t)ks * 256u);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+      const uint32_t sw = (uint32_t)((ch ^ ((i & 3) * 4 + rin)) & 15) * 16u;
+      uint32_t off;
+      if (full) {
+        off = xrow0 + (uint32_t)i * blk_stride + sw + (uint32_t)ks * 256u;
+      } else { // past the end: re-read the last row (never stored)
+        const int row = min(m_wg + (wave * 8 + i) * 4 + rin, p.M - 1);
+        off = (uint32_t)(row * p.K) * 2u + sw + (uint32_t)ks * 256u;
+      }
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xbase + (size_t)off),
                                        (__attribute__((address_space(3))) void*)(tl_lds + buf * 65536 + (wave * 8 + i) * 1024),
                                        16, 0, 0);
     }
