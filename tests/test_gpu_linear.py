@@ -169,6 +169,14 @@ def test_prefill_tiled_small(fmt, M):
     _run(fmt, M, 384, 1024, "add", True, 500 + M)
 
 
+@pytest.mark.parametrize("post", ["none", "silu", "mul", "add2", "gelu"])
+def test_prefill_mxfp4_ragged_blocks_and_post_ops(post):
+    """Large-M MXFP4 kernel (256 x 256 workgroup tiles): two row blocks with a
+    ragged second one, three channel blocks with two tiles in the last, an odd
+    number of K steps, every fused epilogue through the coalesced store path."""
+    _run("mxfp4", 300, 544, 384, post, post != "mul", 700, ulps=2 if post in ("silu", "gelu") else 1)
+
+
 @pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])
 def test_prefill_tiled_m2048(fmt):
     """Prefill row count of BASELINE config 4 (M = 2048) on a layer slice the
@@ -271,4 +279,6 @@ def test_launch_plan_names_the_kernels():
     _lib.check(L.tppx_plan_linear_qint8(1, 11008, 4096, 256, 1, 0, 1 << 25, buf, len(buf)))
     assert buf.value.decode().count("\n") == 1 and "skinny_qint8_fq_kernel<" in buf.value.decode()
     _lib.check(L.tppx_plan_linear_mxfp4(2048, 8192, 8192, 0, 0, buf, len(buf)))
+    assert "big_mxfp4_kernel" in buf.value.decode()
+    _lib.check(L.tppx_plan_linear_mxfp4(100, 8192, 8192, 0, 0, buf, len(buf)))
     assert "tiled_mxfp4_kernel" in buf.value.decode()

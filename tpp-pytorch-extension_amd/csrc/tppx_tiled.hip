@@ -504,13 +504,16 @@ big_mxfp4_kernel(const TiledParams p) {
     take_b();
     if (more)
       load_a(ks + 1, buf ^ 1); // lands in the other buffer during this step's MFMAs
-    // 32 operand reads per K step (q = j*8 + mt), kept two ahead of the MFMAs
-    // that consume them so the LDS latency is covered by 8 MFMAs
+    // 32 operand reads per K step (q = j*8 + mt), kept RD ahead of the MFMAs
+    // that consume them so the LDS latency is covered by 4*RD MFMAs
     const uint32_t abase = lds0 + (uint32_t)(buf * 65536 + wm * 8 * 4096);
-    i32x4 ar[3];
+    constexpr int RD = 3; // operand reads in flight ahead of the MFMAs
+    i32x4 ar[RD + 1];
     bf16x8 b[4];
-    lds_read_b128_async<0>(ar[0], abase + rdb[0]);
-    lds_read_b128_async<4096>(ar[1], abase + rdb[0]);
+    static_for<0, RD>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      lds_read_b128_async<(i & 7) * 4096>(ar[i], abase + rdb[i >> 3]);
+    });
     static_for<0, 32>([&](auto Q) {
       constexpr int q = decltype(Q)::value;
       constexpr int j = q >> 3, mt = q & 7;
@@ -519,15 +522,13 @@ big_mxfp4_kernel(const TiledParams p) {
         for (int nt = 0; nt < 4; nt++)
           b[nt] = tl_cvt_fp4x8(bc[nt][j], sc[nt]);
       }
-      if constexpr (q + 2 < 32) {
-        lds_read_b128_async<((q + 2) & 7) * 4096>(ar[(q + 2) % 3], abase + rdb[(q + 2) >> 3]);
-        lds_wait_keep<2>(ar[q % 3]);
-      } else if constexpr (q + 1 < 32) {
-        lds_wait_keep<1>(ar[q % 3]);
+      if constexpr (q + RD < 32) {
+        lds_read_b128_async<((q + RD) & 7) * 4096>(ar[(q + RD) % (RD + 1)], abase + rdb[(q + RD) >> 3]);
+        lds_wait_keep<RD>(ar[q % (RD + 1)]);
       } else {
-        lds_wait_keep<0>(ar[q % 3]);
+        lds_wait_keep<31 - q>(ar[q % (RD + 1)]);
       }
-      const bf16x8 a = __builtin_bit_cast(bf16x8, ar[q % 3]);
+      const bf16x8 a = __builtin_bit_cast(bf16x8, ar[q % (RD + 1)]);
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
         acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[nt], acc[mt][nt], 0, 0, 0);
