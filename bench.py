@@ -55,6 +55,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--fmt", default="qint8", choices=["qint8", "mxfp4"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill"],
+                    help="decode = the configuration the headline metric is quoted on (default); prefill = the "
+                         "MXFP4 linears of one 70B-shape decoder layer at M = 2048 (TFLOP/s, MFMA roofline)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pool", type=int, default=2, help="number of distinct weight sets cycled through")
@@ -76,6 +79,9 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.workload == "prefill":
+        return run_prefill(torch, _ops, args)
 
     fmt = args.fmt
     shapes = {"up": (11008, 4096), "down": (4096, 11008)}
@@ -189,6 +195,106 @@ def main():
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))
+
+
+def run_prefill(torch, _ops, args):
+    """BASELINE config 4: M = 2048 tokens through the MXFP4 linears of one decoder layer with hidden 8192
+    (fused qkv 8192 -> 8192+1024+1024, o 8192 -> 8192 + residual, gate/up 8192 -> 28672 as silu then mul,
+    down 28672 -> 8192 + residual).  One step = those five op calls (seven GEMMs)."""
+    from tpp_pytorch_extension import _lib
+    dev = torch.device("cuda:0")
+    M, H, I = 2048, 8192, 28672
+    g = torch.Generator(device=dev).manual_seed(1238)
+
+    def mk(N, K):
+        W = (torch.randn((N, K), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        q = _ops.remap_and_quantize_mxfp4(W.view(N // 16, 16, K // 64, 32, 2).permute(0, 2, 3, 1, 4).contiguous())
+        q.native()
+        return q
+
+    wq, wk, wv, wo = mk(H, H), mk(1024, H), mk(1024, H), mk(H, H)
+    wg, wu, wd = mk(I, H), mk(I, H), mk(H, I)
+    x = torch.randn((M, H), generator=g, device=dev).to(torch.bfloat16)
+    res = torch.randn((M, H), generator=g, device=dev).to(torch.bfloat16)
+    empty = torch.empty(0, dtype=torch.bfloat16, device=dev)
+
+    def step():
+        q, k, v = torch.ops.tpp_llm.qkv_gemm(x, [wq, wk, wv], [empty] * 3)
+        h = torch.ops.tpp_llm.fc_add(q, wo, empty, res, 1.0)
+        gate = torch.ops.tpp_llm.fc_silu(h, wg, empty)
+        inter = torch.ops.tpp_llm.fc_mul(h, wu, empty, gate)
+        return torch.ops.tpp_llm.fc_add(inter, wd, empty, h, 1.0), k, v
+
+    gemms = [("qkv", 10240, H), ("o", H, H), ("gate", I, H), ("up", I, H), ("down", H, I)]
+    flops = sum(2.0 * M * N * K for _, N, K in gemms)
+    steps, warmup = max(3, min(args.steps, 20)), max(1, min(args.warmup, 3))
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+
+    # roofline leg: the largest GEMM (down projection) alone, events on the launch stream
+    L = _lib.lib()
+    plan = kernel_plan(L, "mxfp4", M, H, I, 0, 0, 0)
+    inter = torch.randn((M, I), generator=g, device=dev).to(torch.bfloat16)
+    for _ in range(2):
+        torch.ops.tpp_llm.fc_add(inter, wd, empty, res, 1.0)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = 10
+    e0.record()
+    for _ in range(reps):
+        torch.ops.tpp_llm.fc_add(inter, wd, empty, res, 1.0)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / reps
+    fl = 2.0 * M * H * I
+    roof = {"bound": "mfma", "kernel": plan[-1][0] if plan else "?", "call": f"down M={M} N={H} K={I}",
+            "achieved": round(fl / us / 1e6, 1), "peak": PEAKS_TFLOPS["bf16"], "unit": "TFLOP/s",
+            "frac": round(fl / us / 1e6 / PEAKS_TFLOPS["bf16"], 4), "traffic": None,
+            "avg_launch_us": round(us, 1), "flops_per_launch": fl, "launches_timed": reps,
+            "timing": "events on the launch stream around eager launches of this op alone"}
+    cpu = None if args.no_cpu else cpu_baseline_prefill(H)
+    print(json.dumps({
+        "metric": "quant-GEMM TFLOP/s (prefill)", "value": round(flops / (ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "cfg4: MXFP4 linears of one decoder layer (hidden 8192, intermediate 28672, kv 1024) at "
+                               "M = 2048: qkv_gemm, fc_add(o), fc_silu(gate), fc_mul(up), fc_add(down)",
+                   "launch": "eager op calls", "flops_per_step": flops},
+        "roofline": roof, "cpu_baseline": cpu}))
+
+
+def cpu_baseline_prefill(H):
+    """The oracle's MXFP4 linear on a bounded sample: 256 rows through an 8192 x 8192 projection, faithful mode."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numpy as np
+    import oracle as O
+    cores = len(os.sched_getaffinity(0))
+    cores = min(cores, O.num_threads()) if O.num_threads() > 0 else cores
+    O.set_num_threads(cores)
+    rng = np.random.default_rng(7)
+    Ms, N = 256, 2048
+    W = (rng.standard_normal((N, H), dtype=np.float32) * 0.02).astype(np.float32)
+    q, sc = O.remap_quantize_mxfp4(W)
+    xf = rng.standard_normal((Ms, H), dtype=np.float32)
+    xb = (xf.view(np.uint32) >> 16).astype(np.uint16)  # truncation is fine for a timing input
+    O.linear_mxfp4(xb, q, sc, None, O.POST_NONE, None, None, 1.0, O.MODE_FAITHFUL)
+    n, t0 = 0, time.perf_counter()
+    while True:
+        O.linear_mxfp4(xb, q, sc, None, O.POST_NONE, None, None, 1.0, O.MODE_FAITHFUL)
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt > 12.0 or n >= 200:
+            break
+    fl = 2.0 * Ms * N * H
+    return {"value": round(fl * n / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{n} passes of a {Ms} x {N} x {H} MXFP4 linear (C/OpenMP restatement of the reference recipe, "
+                      f"faithful mode; not the libxsmm JIT), {round(dt / n * 1e3, 1)} ms each"}
 
 
 def kernel_plan(L, fmt, M, N, K, qbs, flags, ws_bytes):

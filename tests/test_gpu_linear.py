@@ -204,6 +204,19 @@ def test_prefill_qkv_and_swiglu_equal_composition():
     assert torch.equal(fused, ops.fc_mul(x, wu, None, ops.fc_silu(x, wg, None)))
 
 
+def test_prefill_qkv_one_launch_equals_separate():
+    """With enough rows the fused q/k/v GEMMs share one launch of the large-M
+    kernel (one grid over the channel blocks of all three)."""
+    ops = _ops()
+    K, M = 512, 300
+    ws = [_make("mxfp4", n, K, 180 + i)[0] for i, n in enumerate((544, 128, 256))]
+    x = randn_bf16((M, K), 1.0, 190).cuda()
+    bs = [randn_bf16((n,), 0.01, 195 + i).cuda() for i, n in enumerate((544, 128, 256))]
+    outs = torch.ops.tpp_llm.qkv_gemm(x, ws, bs)
+    for w, b, o in zip(ws, bs, outs):
+        assert torch.equal(o, ops.fc_plain(x, w, b))
+
+
 _FULL_UP = {}
 
 

@@ -204,6 +204,16 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
   if (want_tiled(M, flags)) {
     // prefill shapes: one LDS-tiled launch per GEMM of the group; the fused
     // gate/up pair becomes silu(gate) followed by up * gate (same rounding)
+    if (!dual && n_segs > 1) {
+      TiledParams t[TPPX_MAX_SEGS];
+      bool group = true;
+      for (int i = 0; i < n_segs; i++) {
+        t[i] = tiled_from_seg(p, i);
+        group = group && tiled_mxfp4_takes_groups(t[i]);
+      }
+      if (group) // fused q/k/v: one grid over the channel blocks of all GEMMs
+        return check_hip(launch_tiled_mxfp4_group(t, n_segs, stream), who);
+    }
     for (int i = 0; i < n_segs; i++) {
       TiledParams t = tiled_from_seg(p, i);
       if (dual) {

@@ -72,6 +72,9 @@ struct TiledParams {
 };
 
 hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream);
+// large-M kernel: several GEMMs over one activation in one launch
+bool tiled_mxfp4_takes_groups(const TiledParams& p);
+hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream);
 hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream);
 
 int env_int(const char* name, int dflt);

@@ -20,6 +20,7 @@
 // MFMA operand convention (A = activations, B = weights):
 //   lane l supplies row/col (l & 15) and K group (l >> 4);
 //   result register r of lane l is D[m = (l >> 4) * 4 + r][n = l & 15].
+#include <string.h>
 #include <type_traits>
 
 #include "tppx_common.h"
@@ -399,16 +400,33 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
+// Several GEMMs over one activation (fused q/k/v) share a launch: the channel
+// blocks of all segments form one grid.
+struct BigParams {
+  TiledParams seg[TPPX_MAX_SEGS];
+  int nb0[TPPX_MAX_SEGS + 1]; // first channel block of each segment, then the total
+  int n_seg;
+};
+
 __global__ void __launch_bounds__(512)
-big_mxfp4_kernel(const TiledParams p) {
+big_mxfp4_kernel(const BigParams P) {
   extern __shared__ __align__(16) uint8_t tl_lds[];
-  bf16x8* As = reinterpret_cast<bf16x8*>(tl_lds); // 2 buffers x 4096 slots of 16 B
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform: keeps LDS bases and block indices scalar
   const int wm = wave & 1, wn = wave >> 1;
-  const int MB = (p.M + 255) >> 8, NB = (p.tiles + 15) >> 4;
+  const int MB = (P.seg[0].M + 255) >> 8;
   int bm, bn;
-  tile_of_block(MB, NB, bm, bn);
+  tile_of_block(MB, P.nb0[P.n_seg], bm, bn);
+  // pick this block's GEMM with uniform selects (everything stays in scalar registers)
+  TiledParams p = P.seg[0];
+  int nb_first = 0;
+#pragma unroll
+  for (int i = 1; i < TPPX_MAX_SEGS; i++)
+    if (i < P.n_seg && bn >= P.nb0[i]) {
+      p = P.seg[i];
+      nb_first = P.nb0[i];
+    }
+  bn -= nb_first;
   const int KT = p.K >> 7;
   const int m_wg = bm * 256;
   const int tile_base = bn * 16 + wn * 4;
@@ -543,25 +561,45 @@ big_mxfp4_kernel(const TiledParams p) {
   big_epilogue(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * 128, tile_base);
 }
 
-hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream) {
-  // the large-M kernel addresses its operands with 32-bit byte offsets
-  const bool fits32 = (int64_t)p.M * p.K * 2 < ((int64_t)1 << 32) && (int64_t)p.tiles * 8 * p.K < ((int64_t)1 << 32);
-  if (p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && fits32) {
-    const int MB = (p.M + 255) / 256, NB = (p.tiles + 15) / 16;
-    const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the two 64 KiB A buffers
-    TPPX_PLAN_ONLY(big_mxfp4_kernel, dim3(MB * NB), dim3(512), lds);
-    static bool big_attr_done = false;
-    if (!big_attr_done) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_mxfp4_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess)
-        return e;
-      big_attr_done = true;
-    }
-    big_mxfp4_kernel<<<dim3(MB * NB), dim3(512), lds, stream>>>(p);
-    return hipGetLastError();
-  }
+// the large-M kernel addresses its operands with 32-bit byte offsets
+static bool big_fits(const TiledParams& p) {
+  return (int64_t)p.M * p.K * 2 < ((int64_t)1 << 32) && (int64_t)p.tiles * 8 * p.K < ((int64_t)1 << 32);
+}
 
+bool tiled_mxfp4_takes_groups(const TiledParams& p) {
+  return p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && big_fits(p);
+}
+
+hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream) {
+  BigParams P;
+  memset(&P, 0, sizeof(P));
+  int nb = 0;
+  for (int i = 0; i < n; i++) {
+    P.seg[i] = t[i];
+    P.nb0[i] = nb;
+    nb += (t[i].tiles + 15) / 16;
+  }
+  for (int i = n; i <= TPPX_MAX_SEGS; i++)
+    P.nb0[i] = nb;
+  P.n_seg = n;
+  const int MB = (t[0].M + 255) / 256;
+  const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the two 64 KiB A buffers
+  TPPX_PLAN_ONLY(big_mxfp4_kernel, dim3(MB * nb), dim3(512), lds);
+  static bool big_attr_done = false;
+  if (!big_attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_mxfp4_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess)
+      return e;
+    big_attr_done = true;
+  }
+  big_mxfp4_kernel<<<dim3(MB * nb), dim3(512), lds, stream>>>(P);
+  return hipGetLastError();
+}
+
+hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream) {
+  if (tiled_mxfp4_takes_groups(p))
+    return launch_tiled_mxfp4_group(&p, 1, stream);
   const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
   const size_t lds = 2 * 2048 * 16;
   TPPX_PLAN_ONLY(tiled_mxfp4_kernel, dim3(MB * NB), dim3(256), lds);
