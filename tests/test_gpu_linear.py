@@ -204,6 +204,22 @@ def test_prefill_qkv_and_swiglu_equal_composition():
     assert torch.equal(fused, ops.fc_mul(x, wu, None, ops.fc_silu(x, wg, None)))
 
 
+@pytest.mark.parametrize("M", [2, 12])
+def test_swiglu_full_size_gate_up_equals_composition(M):
+    """Llama-7B gate/up shape (688 channel tiles): the fused kernel takes one
+    (M <= 4) or two channel tiles of each GEMM per workgroup; both must give the
+    bits of silu-then-mul through the single-GEMM kernels, and match the oracle."""
+    ops = _ops()
+    wg, qg, sg_ = _make("mxfp4", 11008, 512, 301)
+    wu, qu, su = _make("mxfp4", 11008, 512, 302)
+    x = randn_bf16((M, 512), 1.0, 303)
+    fused = ops.swiglu_gate_up(x.cuda(), wg, wu)
+    assert torch.equal(fused, ops.fc_mul(x.cuda(), wu, None, ops.fc_silu(x.cuda(), wg, None)))
+    gate = O.linear_mxfp4(t2bits(x), qg, sg_, None, O.POST_SILU)
+    ref = O.linear_mxfp4(t2bits(x), qu, su, None, O.POST_MUL, gate)
+    assert_close_bf16(t2bits(fused), ref, ulps=2, what=f"swiglu gate/up M={M}")
+
+
 def test_prefill_qkv_one_launch_equals_separate():
     """With enough rows the fused q/k/v GEMMs share one launch of the large-M
     kernel (one grid over the channel blocks of all three)."""

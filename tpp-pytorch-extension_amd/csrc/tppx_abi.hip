@@ -229,7 +229,7 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
   if (M <= 16 && env_int("TPPX_MXFP4_SPLITK", 0) == 0) {
     // GEMV class: K reduction inside the workgroup
     SkinnyPlan sp = plan_skinny(0, M, p.total_tiles, p.units, dual);
-    set_groups(p, dual ? 1 : sp.ntw, dual);
+    set_groups(p, sp.ntw, dual);
     return check_hip(launch_skinny_mxfp4(p, sp, dual, stream), who);
   }
   DecodePlan pl = plan_decode(0, M, p.groups, p.total_tiles, p.units, 1, dual, (size_t)ws_bytes);

@@ -473,34 +473,41 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
 
 // ---------------------------------------------------------------------------
 // MXFP4 weight-only, M <= 16 per block row (one MFMA row group).
-// DUAL: NTW = 2 accumulators = the gate tile and the up tile of one channel
-// tile; epilogue silu(gate) * up.
+// NT channel tiles per workgroup; DUAL: the gate AND the up tile of each of
+// them (NACC = 2*NT accumulators, gate tiles first), epilogue silu(gate) * up.
 // ---------------------------------------------------------------------------
 // WPE = waves per SIMD the register budget must allow (2 workgroups of 8
 // waves per CU need 4).
-template <int NTW, int PF, int MAXW, int MINW, bool DUAL, int WPE = 1>
+template <int NT, int PF, int MAXW, int MINW, bool DUAL, int WPE = 1>
 __global__ void __launch_bounds__(MAXW * 64, WPE)
 skinny_mxfp4_kernel(const DecodeParams p) {
+  constexpr int NTW = DUAL ? 2 * NT : NT; // weight tiles per ring stage = accumulators
   extern __shared__ __align__(16) float sk_lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int W = blockDim.x >> 6;
   const int grp = blockIdx.x;
   const int seg_id = DUAL ? 0 : sk_find_seg(p, grp);
   const DecodeSeg& sg = p.seg[seg_id];
-  const int ltile0 = (grp - sg.grp0) * (DUAL ? 1 : NTW);
+  const int ltile0 = (grp - sg.grp0) * NT;
   const int m0 = blockIdx.y * 16;
   const int KT = p.units;
   const int t0 = (int)(((int64_t)wave * KT) / W), t1 = (int)(((int64_t)(wave + 1) * KT) / W);
 
-  const i32x4* wq[NTW];
-  const uint8_t* wsc[NTW];
+  // uniform base pointer per GEMM + one 32-bit slot offset per channel tile
+  // (gate and up tiles share it): no 64-bit pointer pair per stream
+  constexpr int NSEG = DUAL ? 2 : 1;
+  const char* qwb[NSEG];
+  const char* swb[NSEG];
 #pragma unroll
-  for (int nt = 0; nt < NTW; nt++) {
-    const DecodeSeg& ss = p.seg[DUAL ? nt : seg_id];
-    const int64_t lt = DUAL ? ltile0 : min(ltile0 + nt, sg.tiles - 1);
-    wq[nt] = reinterpret_cast<const i32x4*>(ss.qw) + lt * KT * 64 + lane;
-    wsc[nt] = reinterpret_cast<const uint8_t*>(ss.sw) + lt * KT * 64 + lane;
+  for (int sgi = 0; sgi < NSEG; sgi++) {
+    const DecodeSeg& ss = p.seg[DUAL ? sgi : seg_id];
+    qwb[sgi] = reinterpret_cast<const char*>(ss.qw);
+    swb[sgi] = reinterpret_cast<const char*>(ss.sw);
   }
+  uint32_t woff[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; nt++)
+    woff[nt] = (uint32_t)(min(ltile0 + nt, sg.tiles - 1) * KT * 64 + lane); // ragged last group: duplicate, not stored
   const int mrow = min(m0 + (lane & 15), p.M - 1);
   const uint16_t* xrow = reinterpret_cast<const uint16_t*>(p.x) + (int64_t)mrow * p.K + (lane >> 4) * 32;
 
@@ -511,8 +518,9 @@ skinny_mxfp4_kernel(const DecodeParams p) {
     t = min(t, t1 - 1);
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
-      wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64);
-      sreg[st][nt] = wsc[nt][(int64_t)t * 64];
+      const uint32_t slot = woff[nt % NT] + (uint32_t)t * 64u;
+      wreg[st][nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(qwb[nt / NT] + (size_t)(slot * 16u)));
+      sreg[st][nt] = *reinterpret_cast<const uint8_t*>(swb[nt / NT] + (size_t)slot);
     }
 #pragma unroll
     for (int j = 0; j < 4; j++)
@@ -579,8 +587,8 @@ SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual
   int env_ntw = env_int("TPPX_SKINNY_NTW", 0);
   if (!dual && (env_ntw == 1 || env_ntw == 2))
     pl.ntw = env_ntw;
-  if (dual)
-    pl.ntw = 2;
+  if (dual) // channel tiles per workgroup of EACH of the two GEMMs
+    pl.ntw = (total_tiles >= 512 && M > 4 && env_ntw != 1) ? 2 : 1; // few rows: activation traffic is negligible
   // more than 16 rows: these kernels run one workgroup per CU, so prefer a grid
   // of at most 256 workgroups (a second, partly filled round costs a full one)
   if (fmt == 1 && pl.mg > 1 && env_ntw == 0 && total_tiles > 512 && total_tiles <= 768)
@@ -594,7 +602,7 @@ SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual
     max_w = (pl.mg == 4 || (pl.mg == 2 && pl.ntw >= 2)) ? 8 : 16;
     min_w = (pl.mg == 4 || (pl.mg == 2 && pl.ntw >= 2)) ? 8 : 4;
   } else {
-    max_w = pl.ntw == 2 ? 8 : 16;
+    max_w = (dual || pl.ntw == 2) ? 8 : 16;
     min_w = 4;
   }
   // few tiles: one 16-wave workgroup per CU keeps the whole weight in flight
@@ -660,9 +668,12 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
 
 hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream) {
   dim3 grid(p.groups, pl.grid_y);
-  size_t lds = (size_t)pl.waves * pl.ntw * 256 * sizeof(float);
-  if (dual)
-    return sk_launch(skinny_mxfp4_kernel<2, 2, 8, 4, true, 4>, p, grid, pl.waves, lds, stream);
+  size_t lds = (size_t)pl.waves * pl.ntw * (dual ? 2 : 1) * 256 * sizeof(float);
+  if (dual) {
+    if (pl.ntw == 2)
+      return sk_launch(skinny_mxfp4_kernel<2, 2, 8, 4, true, 4>, p, grid, pl.waves, lds, stream);
+    return sk_launch(skinny_mxfp4_kernel<1, 2, 8, 4, true, 4>, p, grid, pl.waves, lds, stream);
+  }
   if (pl.ntw == 2)
     return sk_launch(skinny_mxfp4_kernel<2, 2, 8, 4, false, 4>, p, grid, pl.waves, lds, stream);
   return sk_launch(skinny_mxfp4_kernel<1, 4, 16, 4, false>, p, grid, pl.waves, lds, stream);
