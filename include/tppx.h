@@ -206,6 +206,47 @@ int tppx_swiglu_mxfp4(const void* x, const void* qw_gate, const void* sw_gate,
                       int64_t M, int64_t N, int64_t K, int flags, void* ws,
                       int64_t ws_bytes, tppx_stream_t stream);
 
+/* ---- decode-side operators of the decoder layer -------------------------- */
+
+/* Replaces llama_rms_norm / RMSNormFwdTPP (src/csrc/llm/fused_llm_infer.cpp:309-363,
+ * src/csrc/xsmm_functors.h:4575-4660): y = bf16((x * rsqrt(mean(x^2) + eps)) * gamma),
+ * x, y bf16 [rows][K] (K % 8 == 0), gamma f32 or bf16 [K] (TPPX_DT_*). */
+int tppx_rms_norm(const void* x, const void* gamma, int gamma_dtype, void* y,
+                  int64_t rows, int64_t K, float eps, tppx_stream_t stream);
+
+/* Replaces apply_rotary_pos_emb_llama (src/csrc/llm/fused_llm_infer.cpp:207-253):
+ * in place on t bf16 [B][S][N][H]; emb_pos f32 [2][MP][HR] (cos, sin); pos i64
+ * [B_pos][S] with B_pos 1 or B; positions >= MP are left untouched. */
+int tppx_rotary_llama(void* t, const void* emb_pos, const void* pos, int64_t B,
+                      int64_t S, int64_t N, int64_t H, int64_t MP, int64_t HR,
+                      int64_t B_pos, tppx_stream_t stream);
+
+/* The two rotary calls of LlamaDecoderLayer::_forward (fused_llm_infer.cpp:1252-1253)
+ * and LayerCache::update (src/csrc/llm/attn.h:198-222) in one launch: rotates q
+ * (may be NULL) and k in place and writes the rotated k and v rows into the
+ * cache [B][Nkv][Smax][H] at position *offset_dev + s (offset_dev: device i32,
+ * the cache length before the call, so the call can sit in a replayed graph;
+ * emb_pos == NULL appends without rotation). */
+int tppx_rotary_kv_append_llama(void* q, void* k, const void* v,
+                                const void* emb_pos, const void* pos,
+                                void* kcache, void* vcache,
+                                const void* offset_dev, int64_t B, int64_t S,
+                                int64_t Nq, int64_t Nkv, int64_t H, int64_t MP,
+                                int64_t HR, int64_t B_pos, int64_t Smax,
+                                tppx_stream_t stream);
+
+/* Replaces attn<T> (src/csrc/llm/attn.cpp:781-955) for one query token per
+ * sequence: q bf16 [B][Nq][128], cache bf16 [B][Nkv][Smax][128], additive mask
+ * bf16 [B][mask_ld] or NULL; valid keys = *kv_len_dev (device i32) + kv_len_add
+ * (the counter may still hold the length before this step's append); out bf16
+ * [B][Nq][128].  ws: optional scratch for split-KV partial results. */
+int tppx_attn_decode(const void* q, const void* kcache, const void* vcache,
+                     const void* mask, int64_t mask_ld, const void* kv_len_dev,
+                     int64_t kv_len_add, void* out, int64_t B, int64_t Nq,
+                     int64_t Nkv, int64_t H,
+                     int64_t Smax, void* ws, int64_t ws_bytes,
+                     tppx_stream_t stream);
+
 /* ---- launch plans ------------------------------------------------------- */
 
 /* No counterpart in the reference.  Writes into buf, one line per kernel, what

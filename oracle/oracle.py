@@ -458,3 +458,68 @@ def num_threads():
 
 def set_num_threads(n):
     lib().orc_set_num_threads(ctypes.c_int(int(n)))
+
+
+# ---------------------------------------------------------------------------
+# Decode-side operators of the decoder layer (numpy restatements; float math,
+# compared with a stated tolerance, not bit-exact)
+# ---------------------------------------------------------------------------
+def _bf16_round_f32(a):
+    """fp32 array -> nearest-even bf16, returned as fp32 values."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint32) << 16
+    return r.astype(np.uint32).view(np.float32)
+
+
+def rms_norm(x_bf16, gamma_f32, eps):
+    """RMSNormFwdTPP::ref (src/csrc/xsmm_functors.h:4628-4654) on rows of x: v = mean(x^2);
+    s = 1/sqrt(v + eps); out = bf16((x*s)*gamma), all in fp32.  Returns bf16 bit patterns."""
+    x = bf16_to_f32(_c(x_bf16, np.uint16))
+    g = np.asarray(gamma_f32, np.float32)
+    v = (x.astype(np.float32) ** 2).sum(-1, dtype=np.float32) * np.float32(1.0 / x.shape[-1])
+    s = (np.float32(1.0) / np.sqrt(v + np.float32(eps), dtype=np.float32)).astype(np.float32)
+    out = (x * s[..., None]).astype(np.float32) * g
+    return f32_to_bf16(out.astype(np.float32))
+
+
+def rotary_llama(t_bf16, emb_pos, pos, N, H):
+    """apply_rotary_pos_emb_llama (src/csrc/llm/fused_llm_infer.cpp:207-253): t [B][S][N*H] bf16 bits,
+    emb_pos f32 [2][MP][HR] (cos, sin), pos i64 [B_pos][S]; pairs (h2, HR/2 + h2); positions >= MP untouched."""
+    t = bf16_to_f32(_c(t_bf16, np.uint16)).copy()
+    B, S = t.shape[0], t.shape[1]
+    t = t.reshape(B, S, N, H)
+    MP, HR = emb_pos.shape[1], emb_pos.shape[2]
+    coff = HR // 2
+    for b in range(B):
+        for s in range(S):
+            p = int(pos[0 if pos.shape[0] == 1 else b][s])
+            if p >= MP:
+                continue
+            cos, sin = emb_pos[0][p][:coff].astype(np.float32), emb_pos[1][p][:coff].astype(np.float32)
+            in0, in1 = t[b, s, :, :coff].copy(), t[b, s, :, coff:HR].copy()
+            t[b, s, :, :coff] = _bf16_round_f32(in0 * cos - in1 * sin)
+            t[b, s, :, coff:HR] = _bf16_round_f32(in1 * cos + in0 * sin)
+    return f32_to_bf16(t.reshape(B, S, N * H))
+
+
+def attn_decode(q_bf16, k_bf16, v_bf16, mask_f32=None, round_probs=True):
+    """attn<T> (src/csrc/llm/attn.cpp:781-955) for one query token: q [B][Nq][H], k / v [B][Nkv][L][H] (bf16 bits),
+    additive mask f32 [B][L] or None.  scores = q.k / sqrt(H) + mask (fp32); p = exp(s - max); the probabilities that
+    multiply V are rounded to bf16 (the reference stores them in bf16, attn.cpp:900-905) while the normaliser sums
+    the unrounded ones; output bf16.  Accumulation in fp64 here (the order-independent answer)."""
+    q = bf16_to_f32(_c(q_bf16, np.uint16)).astype(np.float64)
+    k = bf16_to_f32(_c(k_bf16, np.uint16)).astype(np.float64)
+    v = bf16_to_f32(_c(v_bf16, np.uint16)).astype(np.float64)
+    B, Nq, H = q.shape
+    Nkv = k.shape[1]
+    R = Nq // Nkv
+    out = np.empty((B, Nq, H), np.float32)
+    for b in range(B):
+        for n in range(Nq):
+            s = (k[b, n // R] @ q[b, n]) / np.sqrt(np.float64(H))
+            if mask_f32 is not None:
+                s = s + mask_f32[b][: s.shape[0]].astype(np.float64)
+            p = np.exp(s - s.max())
+            pb = _bf16_round_f32(p.astype(np.float32)).astype(np.float64) if round_probs else p
+            out[b, n] = (pb @ v[b, n // R] / p.sum()).astype(np.float32)
+    return f32_to_bf16(out)

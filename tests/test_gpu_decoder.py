@@ -1,0 +1,184 @@
+"""Parity of the decode-side operators (RMSNorm, rotary, KV append, decode
+attention) and of one decoder-layer step against the numpy restatements in
+oracle/ and against plain PyTorch fp32 references.
+
+Stated tolerances (floating-point kernels): RMSNorm and rotary within 1 bf16 ulp
+of the fp32 recipe; attention rel-L2 <= 5e-3 and every element within
+2^-7 * max|out| of the fp64 answer (probabilities rounded to bf16 as the
+reference stores them); a whole layer step rel-L2 <= 2e-2 against the
+composition of the oracle functions.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from util import t2bits, randn_bf16, block_bf16, bits2f, assert_close_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def _llm():
+    import tpp_pytorch_extension  # noqa: F401
+    from tpp_pytorch_extension.llm import fused_llama_infer as F
+    return F
+
+
+@pytest.mark.parametrize("K", [4096, 1000, 8])
+@pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
+def test_rms_norm(K, gdt):
+    F = _llm()
+    x = randn_bf16((7, 3, K), 1.5, 11)
+    g = (torch.randn(K, generator=torch.Generator().manual_seed(12)) * 0.5 + 1.0).to(gdt)
+    y = F.rms_norm(x.cuda(), g.cuda(), 1e-5)
+    ref = O.rms_norm(t2bits(x).reshape(-1, K), g.float().numpy(), 1e-5)
+    assert_close_bf16(t2bits(y).reshape(-1, K), ref, what=f"rms_norm K={K}")
+    # independent torch fp32 statement of the same formula
+    xf = x.float()
+    t = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)) * g.float()
+    assert_close_bf16(t2bits(y).reshape(-1, K), t2bits(t.to(torch.bfloat16)).reshape(-1, K), what="rms_norm vs torch")
+
+
+@pytest.mark.parametrize("HR", [128, 64])
+def test_rotary_llama(HR):
+    F = _llm()
+    B, S, N, H, MP = 2, 5, 6, 128, 64
+    t = randn_bf16((B, S, N * H), 1.0, 21)
+    emb = F.llama_rotary_table(MP, HR, device="cpu")
+    pos = torch.tensor([[3, 9, 63, 64, 0], [1, 2, 3, 4, 70]], dtype=torch.int64)  # 64 and 70 are out of range: untouched
+    got = F.apply_rotary_pos_emb_llama(t.clone().cuda(), emb.cuda(), pos.cuda(), N, H)
+    ref = O.rotary_llama(t2bits(t), emb.numpy(), pos.numpy(), N, H)
+    assert_close_bf16(t2bits(got), ref, what=f"rotary HR={HR}")
+    # untouched positions are bit-identical to the input
+    assert torch.equal(got.cpu()[0, 3], t[0, 3]) and torch.equal(got.cpu()[1, 4], t[1, 4])
+    # broadcast positions ([1][S])
+    got1 = F.apply_rotary_pos_emb_llama(t.clone().cuda(), emb.cuda(), pos[:1].cuda(), N, H)
+    ref1 = O.rotary_llama(t2bits(t), emb.numpy(), pos[:1].numpy(), N, H)
+    assert_close_bf16(t2bits(got1), ref1, what="rotary broadcast positions")
+
+
+def _attn(F, q, kc, vc, L, mask=None, ws=True):
+    from tpp_pytorch_extension import _lib
+    Lb = _lib.lib()
+    B, Nq, H = q.shape
+    Nkv, Smax = kc.shape[1], kc.shape[2]
+    out = torch.empty_like(q)
+    ln = torch.tensor([L - 1], dtype=torch.int32, device="cuda")  # counter before the append, +1 in the call
+    w = _lib.workspace(q)
+    _lib.check(Lb.tppx_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                   None if mask is None else mask.data_ptr(), 0 if mask is None else mask.shape[1],
+                                   ln.data_ptr(), 1, out.data_ptr(), B, Nq, Nkv, H, Smax,
+                                   w.data_ptr() if ws else None, w.numel() if ws else 0, _lib.stream_of(q)))
+    return out
+
+
+@pytest.mark.parametrize("B,Nq,Nkv,L,Smax", [(1, 32, 32, 2048, 2304), (3, 8, 2, 77, 128), (2, 4, 4, 1, 64),
+                                             (16, 32, 32, 300, 512)])
+def test_attn_decode(B, Nq, Nkv, L, Smax):
+    F = _llm()
+    q = randn_bf16((B, Nq, 128), 1.0, 31)
+    k = randn_bf16((B, Nkv, Smax, 128), 1.0, 32)
+    v = randn_bf16((B, Nkv, Smax, 128), 1.0, 33)
+    got = _attn(F, q.cuda(), k.cuda(), v.cuda(), L)
+    ref = O.attn_decode(t2bits(q), t2bits(k[:, :, :L]), t2bits(v[:, :, :L]))
+    g, r = bits2f(t2bits(got)).astype(np.float64), bits2f(ref).astype(np.float64)
+    rel = np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum())
+    assert rel <= 5e-3, rel
+    assert np.abs(g - r).max() <= 2.0 ** -7 * np.abs(r).max()
+    # one workgroup per head (no workspace) gives the same answer within the same bound
+    got1 = _attn(F, q.cuda(), k.cuda(), v.cuda(), L, ws=False)
+    g1 = bits2f(t2bits(got1)).astype(np.float64)
+    assert np.sqrt(((g1 - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3
+    # plain PyTorch fp32 softmax attention
+    kk = k[:, :, :L].float().repeat_interleave(Nq // Nkv, dim=1)
+    vv = v[:, :, :L].float().repeat_interleave(Nq // Nkv, dim=1)
+    s = torch.einsum("bnh,bnlh->bnl", q.float(), kk) / np.sqrt(128.0)
+    t = torch.einsum("bnl,bnlh->bnh", torch.softmax(s, -1), vv).numpy().astype(np.float64)
+    assert np.sqrt(((g - t) ** 2).sum() / (t ** 2).sum()) <= 1e-2
+
+
+def test_attn_decode_mask():
+    F = _llm()
+    B, Nq, L, Smax = 2, 4, 100, 128
+    q = randn_bf16((B, Nq, 128), 1.0, 41)
+    k = randn_bf16((B, Nq, Smax, 128), 1.0, 42)
+    v = randn_bf16((B, Nq, Smax, 128), 1.0, 43)
+    keep = torch.ones(B, L, dtype=torch.int64)
+    keep[0, :17] = 0  # left padding of sequence 0
+    mask = F.TppCache(Smax).align_and_invert_mask(keep.to(torch.bfloat16))
+    assert mask.shape == (B, 128) and float(mask[0, 0]) == -9984.0 and float(mask[0, 17]) == 0.0  # bf16(-10000)
+    got = _attn(F, q.cuda(), k.cuda(), v.cuda(), L, mask=mask.cuda())
+    ref = O.attn_decode(t2bits(q), t2bits(k[:, :, :L]), t2bits(v[:, :, :L]), mask.float().numpy())
+    g, r = bits2f(t2bits(got)).astype(np.float64), bits2f(ref).astype(np.float64)
+    assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3
+
+
+def test_decoder_layer_step_and_cache():
+    """One LlamaDecoderLayer.forward on a small shape against the composition of the oracle functions, plus the
+    cache bookkeeping (append position, rotated keys in the cache, reference method names)."""
+    F = _llm()
+    from tpp_pytorch_extension import _ops
+    hidden, inter, Nq, Nkv, H, MP = 512, 1024, 4, 2, 128, 256
+    B, ctx, cap = 2, 37, 64
+    rng = torch.Generator().manual_seed(5)
+
+    def lin(N, K, seed):
+        W = randn_bf16((N, K), 0.05, seed)
+        return W, _ops.remap_and_quantize_mxfp4(block_bf16(W).cuda()), O.remap_quantize_mxfp4(W.float().numpy())
+
+    Ws = [lin(Nq * H, hidden, 51), lin(Nkv * H, hidden, 52), lin(Nkv * H, hidden, 53), lin(hidden, Nq * H, 54),
+          lin(inter, hidden, 55), lin(inter, hidden, 56), lin(hidden, inter, 57)]
+    g1 = torch.rand(hidden, generator=rng) + 0.5
+    g2 = torch.rand(hidden, generator=rng) + 0.5
+    EP = F.llama_rotary_table(MP, H, device="cpu")
+    layer = F.LlamaDecoderLayer([g1.cuda(), Ws[0][1], Ws[1][1], Ws[2][1], Ws[3][1], g2.cuda(), Ws[4][1], Ws[5][1],
+                                 Ws[6][1], EP.cuda()], 0, 1e-5, H, MP, H)
+    cache = F.TppCache(cap)
+    k0, v0 = randn_bf16((B, Nkv, ctx, H), 1.0, 61), randn_bf16((B, Nkv, ctx, H), 1.0, 62)
+    cache.fill_(0, k0.cuda(), v0.cuda())
+    assert cache.get_seq_length() == ctx and cache.get_capacity() == cap and cache.size() == 1
+    x = randn_bf16((B, 1, hidden), 1.0, 63)
+    pos = torch.full((B, 1), ctx, dtype=torch.int64)
+    out = layer.forward([x.cuda(), None, pos.cuda()], cache, True)[0]
+    cache.advance(1)
+    assert cache.get_seq_length() == ctx + 1
+
+    # oracle composition (fused_llm_infer.cpp:1229-1275)
+    def mm(a_bits, w, post=O.POST_NONE, post_in=None):
+        return O.linear_mxfp4(a_bits, w[2][0], w[2][1], None, post, post_in, None, 1.0, O.MODE_IDEAL)
+
+    xb = t2bits(x).reshape(B, hidden)
+    h = O.rms_norm(xb, g1.numpy(), 1e-5)
+    q, k, v = mm(h, Ws[0]), mm(h, Ws[1]), mm(h, Ws[2])
+    q = O.rotary_llama(q.reshape(B, 1, -1), EP.numpy(), pos.numpy(), Nq, H).reshape(B, Nq, H)
+    k = O.rotary_llama(k.reshape(B, 1, -1), EP.numpy(), pos.numpy(), Nkv, H).reshape(B, Nkv, 1, H)
+    kall = np.concatenate([t2bits(k0), k], axis=2)
+    vall = np.concatenate([t2bits(v0), v.reshape(B, Nkv, 1, H)], axis=2)
+    ctxv = O.attn_decode(q, kall, vall).reshape(B, Nq * H)
+    so = mm(ctxv, Ws[3], O.POST_ADD_SCALE, xb)
+    h2 = O.rms_norm(so, g2.numpy(), 1e-5)
+    gate = mm(h2, Ws[4], O.POST_SILU)
+    inter_v = mm(h2, Ws[5], O.POST_MUL, gate)
+    ref = mm(inter_v, Ws[6], O.POST_ADD_SCALE, so)
+    g, r = bits2f(t2bits(out)).reshape(B, hidden).astype(np.float64), bits2f(ref).astype(np.float64)
+    rel = np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum())
+    assert rel <= 2e-2, rel
+    # the cache got the rotated key and the value at position ctx, earlier positions untouched
+    kc, vc = cache.get(0)
+    assert kc.shape[2] == ctx + 1
+    assert_close_bf16(t2bits(kc[:, :, ctx]), k.reshape(B, Nkv, H), what="cached key")
+    assert_close_bf16(t2bits(vc[:, :, ctx]), v.reshape(B, Nkv, H), what="cached value")
+    assert torch.equal(kc[:, :, :ctx].cpu(), k0)
+    with pytest.raises(Exception):
+        layer.forward([x.repeat(1, 2, 1).cuda(), None, pos.cuda()], cache, True)  # more than one query token
+
+
+def test_greedy_decode_graph_equals_eager():
+    """The replayed decode-step graph produces the tokens of the eager loop (same kernels, same order)."""
+    F = _llm()
+    model = F.LlamaDecoder(hidden=512, inter=1024, n_layers=2, n_heads=4, n_kv_heads=4, vocab=1024,
+                           max_positions=256, seed=3)
+    tok = torch.tensor([5, 77, 300], dtype=torch.int64, device="cuda")
+    a = model.greedy_decode(tok, model.new_cache(3, 40, 64), 8, use_graph=False)
+    b = model.greedy_decode(tok, model.new_cache(3, 40, 64), 8, use_graph=True)
+    assert a.shape == (3, 8) and torch.equal(a, b)

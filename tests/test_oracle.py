@@ -265,3 +265,78 @@ def test_post_ops_against_torch_rounding_points():
         w = want.float().numpy().astype(np.float64)
         assert np.all(np.abs(got - w) <= 2.0 ** -7 * np.abs(w) + 1e-30)
         assert np.mean(got != w) < 0.01
+
+
+# ---------------------------------------------------------------------------
+# decode-side operators: the numpy restatements against independent statements
+# ---------------------------------------------------------------------------
+def test_oracle_rms_norm_against_torch_and_closed_form():
+    import torch
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(5, 384, generator=g) * 2).to(torch.bfloat16)
+    w = torch.rand(384, generator=g) + 0.5
+    got = O.bf16_to_f32(O.rms_norm(x.view(torch.int16).numpy().view(np.uint16), w.numpy(), 1e-6))
+    xf = x.float()
+    ref = ((xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)) * w).to(torch.bfloat16).float().numpy()
+    assert np.abs(got - ref).max() <= 2.0 ** -7 * np.abs(ref).max()
+    assert (got != ref).mean() < 0.02  # at most a last-bit difference from the order of the fp32 operations
+    # closed form: a constant row c with unit weight normalises to sign(c) (eps negligible)
+    c = np.full((1, 64), 3.0, np.float32)
+    one = O.bf16_to_f32(O.rms_norm(O.f32_to_bf16(c), np.ones(64, np.float32), 1e-12))
+    assert np.allclose(one, 1.0, atol=2.0 ** -8)
+
+
+def test_oracle_rotary_is_a_rotation_and_matches_rotate_half():
+    import torch
+    B, S, N, H, MP = 2, 3, 2, 32, 16
+    g = torch.Generator().manual_seed(4)
+    t = torch.randn(B, S, N * H, generator=g).to(torch.bfloat16)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, H, 2).float() / H))
+    fr = torch.outer(torch.arange(MP).float(), inv)
+    emb = torch.stack((torch.cat((fr, fr), -1).cos(), torch.cat((fr, fr), -1).sin()))
+    pos = torch.tensor([[0, 5, 15], [7, 16, 2]])  # 16 is out of range
+    got = O.bf16_to_f32(O.rotary_llama(t.view(torch.int16).numpy().view(np.uint16), emb.numpy(), pos.numpy(), N, H))
+    # the Hugging Face formulation: x*cos + rotate_half(x)*sin with rotate_half(x) = cat(-x2, x1)
+    x = t.float().view(B, S, N, H)
+    p = pos.clamp(max=MP - 1)
+    cos, sin = emb[0][p][:, :, None, :], emb[1][p][:, :, None, :]
+    rh = torch.cat((-x[..., H // 2:], x[..., :H // 2]), -1)
+    ref = (x * cos + rh * sin)
+    ref[1, 1] = x[1, 1]  # position 16 >= MP stays untouched
+    ref = ref.to(torch.bfloat16).float().view(B, S, N * H).numpy()
+    assert np.abs(got - ref).max() <= 2.0 ** -7 * np.abs(ref).max()
+    # position 0 is the identity, and a rotation keeps the norm of every (h2, H/2+h2) pair
+    assert np.array_equal(got[0, 0], t.float().numpy()[0, 0])
+    a = t.float().view(B, S, N, 2, H // 2).numpy()
+    b = got.reshape(B, S, N, 2, H // 2)
+    assert np.allclose((a ** 2).sum(3), (b ** 2).sum(3), rtol=2e-2, atol=1e-3)
+
+
+def test_oracle_attn_decode_against_softmax_and_special_cases():
+    import torch
+    B, Nq, Nkv, L, H = 2, 4, 2, 19, 16
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(B, Nq, H, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Nkv, L, H, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Nkv, L, H, generator=g).to(torch.bfloat16)
+    bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
+    got = O.bf16_to_f32(O.attn_decode(bits(q), bits(k), bits(v), None, round_probs=False))
+    kk, vv = k.double().repeat_interleave(2, 1), v.double().repeat_interleave(2, 1)
+    s = torch.einsum("bnh,bnlh->bnl", q.double(), kk) / np.sqrt(H)
+    ref = torch.einsum("bnl,bnlh->bnh", torch.softmax(s, -1), vv).numpy()
+    assert np.abs(got - ref).max() <= 2.0 ** -8 * np.abs(ref).max() + 1e-6
+    # bf16 probabilities change the answer by well under a percent
+    gotb = O.bf16_to_f32(O.attn_decode(bits(q), bits(k), bits(v)))
+    assert np.sqrt(((gotb - ref) ** 2).sum() / (ref ** 2).sum()) < 5e-3
+    # one key: the output is that key's value; identical values: the output is that value whatever the scores
+    one = O.bf16_to_f32(O.attn_decode(bits(q), bits(k[:, :, :1]), bits(v[:, :, :1])))
+    assert np.array_equal(one, v[:, :, 0].float().repeat_interleave(2, 1).numpy())
+    vc = v[:, :, :1].expand(-1, -1, L, -1)
+    same = O.bf16_to_f32(O.attn_decode(bits(q), bits(k), bits(vc), None, round_probs=False))
+    assert np.abs(same - vc[:, :, 0].float().repeat_interleave(2, 1).numpy()).max() <= 2.0 ** -7 * 4
+    # a -10000 mask entry removes the key
+    m = np.zeros((B, L), np.float32); m[:, 3] = -10000.0
+    masked = O.bf16_to_f32(O.attn_decode(bits(q), bits(k), bits(v), m, round_probs=False))
+    keep = [i for i in range(L) if i != 3]
+    dropped = O.bf16_to_f32(O.attn_decode(bits(q), bits(k[:, :, keep]), bits(v[:, :, keep]), None, round_probs=False))
+    assert np.array_equal(masked, dropped)

@@ -1,0 +1,415 @@
+// Decode-side operators around the quantized linears of a Llama decoder layer:
+// RMSNorm, rotary position embedding, KV-cache append and single-query
+// (decode) attention.  All of them are bandwidth bound: one pass over their
+// inputs with 128-bit coalesced accesses, reductions inside a wave with DPP,
+// fp32 arithmetic, one bf16 rounding where the CPU path stores bf16.
+#include <math.h>
+#include <string.h>
+
+#include "tppx_common.h"
+
+namespace tppx {
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+// sum / max over the 16 lanes of a DPP row; every lane of the row gets the result
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_mov<0xB1>(v);  // quad_perm [1,0,3,2]
+  v += dpp_mov<0x4E>(v);  // quad_perm [2,3,0,1]
+  v += dpp_mov<0x141>(v); // row_half_mirror
+  v += dpp_mov<0x140>(v); // row_mirror
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row16_sum(v);
+  float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return (a + b) + (c + d);
+}
+
+__device__ __forceinline__ void unpack8(const uint4& w, float (&f)[8]) {
+  const uint32_t d[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    f[2 * i] = bf16_bits_to_f32(d[i] & 0xffffu);
+    f[2 * i + 1] = bf16_bits_to_f32(d[i] >> 16);
+  }
+}
+__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
+  uint32_t d[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+    d[i] = f32_to_bf16_bits(f[2 * i]) | (f32_to_bf16_bits(f[2 * i + 1]) << 16);
+  return make_uint4(d[0], d[1], d[2], d[3]);
+}
+
+// ---------------------------------------------------------------------------
+// RMSNorm: y = bf16( (x * rsqrt(mean(x^2) + eps)) * gamma ), fp32 inside.
+// One workgroup of 256 threads per row; K a multiple of 8.
+// ---------------------------------------------------------------------------
+template <bool GAMMA_F32>
+__global__ void __launch_bounds__(256)
+rms_norm_kernel(const uint16_t* __restrict__ x, const void* __restrict__ gamma, uint16_t* __restrict__ y,
+                int K, float eps) {
+  __shared__ float red[4];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const uint4* xr = reinterpret_cast<const uint4*>(x + (int64_t)row * K);
+  uint4* yr = reinterpret_cast<uint4*>(y + (int64_t)row * K);
+  const int nchunk = K >> 3;
+  float ss = 0.f;
+  for (int i = tid; i < nchunk; i += 256) {
+    float f[8];
+    unpack8(xr[i], f);
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      ss = fmaf(f[e], f[e], ss);
+  }
+  ss = wave_sum(ss);
+  if ((tid & 63) == 0)
+    red[tid >> 6] = ss;
+  __syncthreads();
+  const float v = ((red[0] + red[1]) + (red[2] + red[3])) * (1.0f / (float)K);
+  const float s = 1.0f / sqrtf(v + eps);
+  for (int i = tid; i < nchunk; i += 256) {
+    float f[8], g[8];
+    unpack8(xr[i], f); // second read hits L2/L1
+    if (GAMMA_F32) {
+      const float4* gp = reinterpret_cast<const float4*>(gamma) + 2 * i;
+      const float4 g0 = gp[0], g1 = gp[1];
+      g[0] = g0.x; g[1] = g0.y; g[2] = g0.z; g[3] = g0.w;
+      g[4] = g1.x; g[5] = g1.y; g[6] = g1.z; g[7] = g1.w;
+    } else {
+      unpack8(reinterpret_cast<const uint4*>(gamma)[i], g);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      f[e] = (f[e] * s) * g[e];
+    yr[i] = pack8(f);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Llama rotary embedding, in place on t [B][S][N][H] (rotate-half pairs
+// (h2, HR/2 + h2)), cos/sin table f32 [2][MP][HR], positions i64 [B_pos][S].
+// Optionally the rotated key rows and the value rows are also written into
+// the KV cache [B][N][Smax][H] at position offset + s (offset read from device
+// memory), so that one launch covers rotary(q), rotary(k) and the cache append.
+// One thread per (token, head, pair of 8-wide chunks).
+// ---------------------------------------------------------------------------
+struct RotaryParams {
+  uint16_t* q;         // [B][S][Nq][H] or null
+  uint16_t* k;         // [B][S][Nkv][H] or null
+  const uint16_t* v;   // [B][S][Nkv][H] or null (append only)
+  uint16_t* kc;        // [B][Nkv][Smax][H] or null
+  uint16_t* vc;
+  const float* emb;    // [2][MP][HR] or null (append without rotation)
+  const int64_t* pos;  // [B_pos][S]
+  const int32_t* offset; // device scalar: cache length before this append
+  int B, S, Nq, Nkv, H, MP, HR, B_pos, Smax;
+};
+
+__global__ void __launch_bounds__(256)
+rotary_append_kernel(const RotaryParams p) {
+  // work item = (b, s, head in [0, Nq + Nkv + Nkv), chunk c of H/8); the pair partner is fetched by the same thread
+  const int CH = p.H >> 3;
+  const int heads = (p.q ? p.Nq : 0) + (p.k ? p.Nkv : 0) + ((p.v && p.vc) ? p.Nkv : 0);
+  const int64_t total = (int64_t)p.B * p.S * heads * CH;
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= total)
+    return;
+  const int c = (int)(id % CH);
+  int hh = (int)((id / CH) % heads);
+  const int64_t tok = id / ((int64_t)CH * heads);
+  const int s = (int)(tok % p.S), b = (int)(tok / p.S);
+  const int nq = p.q ? p.Nq : 0, nk = p.k ? p.Nkv : 0;
+  const int off = (p.kc || p.vc) ? *p.offset : 0;
+  if (hh >= nq + nk) { // value rows: plain copy into the cache
+    const int n = hh - nq - nk;
+    const uint4 w = reinterpret_cast<const uint4*>(p.v + (((int64_t)b * p.S + s) * p.Nkv + n) * p.H)[c];
+    if (off + s < p.Smax)
+      reinterpret_cast<uint4*>(p.vc + (((int64_t)b * p.Nkv + n) * p.Smax + off + s) * p.H)[c] = w;
+    return;
+  }
+  const bool is_k = hh >= nq;
+  const int n = is_k ? hh - nq : hh;
+  uint16_t* row = is_k ? p.k + (((int64_t)b * p.S + s) * p.Nkv + n) * p.H
+                       : p.q + (((int64_t)b * p.S + s) * p.Nq + n) * p.H;
+  uint4 w = reinterpret_cast<uint4*>(row)[c];
+  const int coff = p.HR >> 1;
+  const int h0 = c * 8;
+  const int64_t pp = p.pos[(int64_t)(p.B_pos == 1 ? 0 : b) * p.S + s];
+  if (p.emb && h0 < p.HR && pp < p.MP) {
+    // this chunk holds first halves (h0 < HR/2) or second halves of rotation pairs
+    const bool first = h0 < coff;
+    const int h2 = first ? h0 : h0 - coff;
+    const uint4 wo = reinterpret_cast<const uint4*>(row)[first ? c + (coff >> 3) : c - (coff >> 3)];
+    float a[8], o[8], r[8];
+    unpack8(w, a);
+    unpack8(wo, o);
+    const float* cs = p.emb + pp * p.HR + h2;
+    const float* sn = p.emb + ((int64_t)p.MP + pp) * p.HR + h2;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      // first half: in0*cos - in1*sin ; second half: in1*cos + in0*sin
+      r[e] = first ? a[e] * cs[e] - o[e] * sn[e] : a[e] * cs[e] + o[e] * sn[e];
+    }
+    w = pack8(r);
+  }
+  // The two threads of a rotation pair sit in the same wave (H/8 is a power of
+  // two <= 64 and work items are numbered chunk-fastest), and this store needs
+  // both loaded chunks, so the wave's loads have returned before it issues.
+  reinterpret_cast<uint4*>(row)[c] = w;
+  if (is_k && p.kc && off + s < p.Smax)
+    reinterpret_cast<uint4*>(p.kc + (((int64_t)b * p.Nkv + n) * p.Smax + off + s) * p.H)[c] = w;
+}
+
+// ---------------------------------------------------------------------------
+// Decode attention (one query token per sequence), head size 128, cache
+// [B][Nkv][Smax][128] bf16.  Grid (B*Nq, splits); 4 waves; a wave instruction
+// reads 4 keys (lane = key l>>4, 16-byte chunk l&15); every 16-lane row keeps
+// its own running (max, sum, 8 output dims per lane) over its keys, merged at
+// the end through LDS.  Scores: fp32 dot * 1/sqrt(H) + mask; probabilities are
+// rounded to bf16 before they multiply V (as the CPU path stores them), sums
+// and the output accumulate in fp32.
+// ---------------------------------------------------------------------------
+struct AttnParams {
+  const uint16_t* q;    // [B][Nq][128]
+  const uint16_t* kc;   // [B][Nkv][Smax][128]
+  const uint16_t* vc;
+  const uint16_t* mask; // bf16 [B][mask_ld] additive, or null
+  const int32_t* kv_len; // device scalar; valid keys = *kv_len + kv_len_add
+  int kv_len_add;
+  uint16_t* out;        // [B][Nq][128]
+  float* part;          // [B*Nq][splits][130]
+  int B, Nq, Nkv, Smax, mask_ld, splits;
+  float scale;
+};
+
+__global__ void __launch_bounds__(256)
+attn_decode_kernel(const AttnParams p) {
+  __shared__ float sm[16], sl[16];
+  __shared__ float sacc[16][128];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 4, c = lane & 15;
+  const int bh = blockIdx.x, b = bh / p.Nq, hq = bh - b * p.Nq;
+  const int hk = hq / (p.Nq / p.Nkv);
+  const int L = max(0, min(*p.kv_len + p.kv_len_add, p.Smax));
+  // this workgroup's keys: [k0, k1), split evenly in multiples of 64
+  const int per = ((L + p.splits - 1) / p.splits + 63) & ~63;
+  const int k0 = blockIdx.y * per, k1 = min(k0 + per, L);
+
+  float qf[8];
+  unpack8(reinterpret_cast<const uint4*>(p.q + (int64_t)bh * 128)[c], qf);
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    qf[e] *= p.scale;
+  const uint4* kb = reinterpret_cast<const uint4*>(p.kc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128) + c;
+  const uint4* vb = reinterpret_cast<const uint4*>(p.vc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128) + c;
+  const uint16_t* mrow = p.mask ? p.mask + (int64_t)b * p.mask_ld : nullptr;
+
+  float m = -3.0e38f, l = 0.f, acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    acc[e] = 0.f;
+  for (int base = k0 + wave * 16; base < k1; base += 64) {
+    uint4 kw[4], vw[4];
+    int key[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      key[u] = base + u * 4 + g;
+      const int kk = min(key[u], L - 1);
+      kw[u] = kb[(int64_t)kk * 16];
+      vw[u] = vb[(int64_t)kk * 16];
+    }
+    float sc[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      float kf[8];
+      unpack8(kw[u], kf);
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        d = fmaf(qf[e], kf[e], d);
+      d = row16_sum(d);
+      if (mrow && key[u] < p.mask_ld && key[u] < k1)
+        d += bf16_bits_to_f32(mrow[key[u]]);
+      sc[u] = key[u] < k1 ? d : -3.0e38f;
+    }
+    const float mn = fmaxf(fmaxf(m, fmaxf(sc[0], sc[1])), fmaxf(sc[2], sc[3]));
+    const float alpha = __expf(m - mn);
+    l *= alpha;
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      acc[e] *= alpha;
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const float pr = key[u] < k1 ? __expf(sc[u] - mn) : 0.f;
+      l += pr;
+      const float pb = round_bf16(pr);
+      float vf[8];
+      unpack8(vw[u], vf);
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        acc[e] = fmaf(pb, vf[e], acc[e]);
+    }
+    m = mn;
+  }
+  // merge the 16 (wave, row) states
+  const int st = wave * 4 + g;
+  if (c == 0) {
+    sm[st] = m;
+    sl[st] = l;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    sacc[st][c * 8 + e] = acc[e];
+  __syncthreads();
+  if (tid < 128) {
+    float M = sm[0];
+#pragma unroll
+    for (int i = 1; i < 16; i++)
+      M = fmaxf(M, sm[i]);
+    float Ls = 0.f, o = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const float w = __expf(sm[i] - M);
+      Ls = fmaf(w, sl[i], Ls);
+      o = fmaf(w, sacc[i][tid], o);
+    }
+    if (p.splits == 1) {
+      p.out[(int64_t)bh * 128 + tid] = (uint16_t)f32_to_bf16_bits(Ls > 0.f ? o / Ls : 0.f);
+    } else {
+      float* dst = p.part + ((int64_t)bh * p.splits + blockIdx.y) * 130;
+      dst[2 + tid] = o;
+      if (tid == 0) {
+        dst[0] = M;
+        dst[1] = Ls;
+      }
+    }
+  }
+}
+
+__global__ void __launch_bounds__(128)
+attn_combine_kernel(const AttnParams p) {
+  const int bh = blockIdx.x, tid = threadIdx.x;
+  const float* src = p.part + (int64_t)bh * p.splits * 130;
+  float M = -3.0e38f;
+  for (int i = 0; i < p.splits; i++)
+    M = fmaxf(M, src[i * 130]);
+  float Ls = 0.f, o = 0.f;
+  for (int i = 0; i < p.splits; i++) {
+    const float w = __expf(src[i * 130] - M);
+    Ls = fmaf(w, src[i * 130 + 1], Ls);
+    o = fmaf(w, src[i * 130 + 2 + tid], o);
+  }
+  p.out[(int64_t)bh * 128 + tid] = (uint16_t)f32_to_bf16_bits(Ls > 0.f ? o / Ls : 0.f);
+}
+
+} // namespace tppx
+
+using namespace tppx;
+
+extern "C" int tppx_rms_norm(const void* x, const void* gamma, int gamma_dtype, void* y, int64_t rows, int64_t K,
+                             float eps, tppx_stream_t stream) {
+  TPPX_REQUIRE(x && gamma && y, TPPX_EINVAL, "tppx_rms_norm: null pointer");
+  TPPX_REQUIRE(aligned16(x) && aligned16(gamma) && aligned16(y), TPPX_EINVAL, "tppx_rms_norm: pointer not 16-byte aligned");
+  TPPX_REQUIRE(gamma_dtype == TPPX_DT_F32 || gamma_dtype == TPPX_DT_BF16, TPPX_EINVAL, "tppx_rms_norm: unknown gamma dtype %d", gamma_dtype);
+  TPPX_REQUIRE(rows > 0 && rows < ((int64_t)1 << 31) && K > 0 && K % 8 == 0 && K < (1 << 24), TPPX_ESHAPE,
+               "tppx_rms_norm: bad shape rows=%ld K=%ld (K must be a multiple of 8)", (long)rows, (long)K);
+  if (gamma_dtype == TPPX_DT_F32)
+    rms_norm_kernel<true><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
+        (const uint16_t*)x, gamma, (uint16_t*)y, (int)K, eps);
+  else
+    rms_norm_kernel<false><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
+        (const uint16_t*)x, gamma, (uint16_t*)y, (int)K, eps);
+  return check_hip(hipGetLastError(), "tppx_rms_norm");
+}
+
+static int rotary_common(const char* who, RotaryParams& p, hipStream_t stream) {
+  TPPX_REQUIRE(p.B > 0 && p.S > 0 && p.H >= 16 && p.H <= 512 && (p.H & (p.H - 1)) == 0, TPPX_ESHAPE,
+               "%s: bad shape B=%d S=%d H=%d (head size must be a power of two in 16..512)", who, p.B, p.S, p.H);
+  if (p.emb)
+    TPPX_REQUIRE(p.HR > 0 && p.HR <= p.H && p.HR % 16 == 0 && p.MP > 0, TPPX_ESHAPE,
+                 "%s: rotary_dim=%d must be a multiple of 16 and <= H=%d", who, p.HR, p.H);
+  TPPX_REQUIRE(p.B_pos == 1 || p.B_pos == p.B, TPPX_ESHAPE, "%s: position_ids shape not compatible", who);
+  const int heads = (p.q ? p.Nq : 0) + (p.k ? p.Nkv : 0) + ((p.v && p.vc) ? p.Nkv : 0);
+  const int64_t total = (int64_t)p.B * p.S * heads * (p.H / 8);
+  TPPX_REQUIRE(total > 0 && total < ((int64_t)1 << 40), TPPX_ESHAPE, "%s: nothing to do", who);
+  rotary_append_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream>>>(p);
+  return check_hip(hipGetLastError(), who);
+}
+
+extern "C" int tppx_rotary_llama(void* t, const void* emb_pos, const void* pos, int64_t B, int64_t S, int64_t N,
+                                 int64_t H, int64_t MP, int64_t HR, int64_t B_pos, tppx_stream_t stream) {
+  TPPX_REQUIRE(t && emb_pos && pos, TPPX_EINVAL, "tppx_rotary_llama: null pointer");
+  TPPX_REQUIRE(aligned16(t), TPPX_EINVAL, "tppx_rotary_llama: pointer not 16-byte aligned");
+  TPPX_REQUIRE(N > 0, TPPX_ESHAPE, "tppx_rotary_llama: N=%ld", (long)N);
+  RotaryParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = (uint16_t*)t;
+  p.emb = (const float*)emb_pos;
+  p.pos = (const int64_t*)pos;
+  p.B = (int)B; p.S = (int)S; p.Nq = (int)N; p.H = (int)H; p.MP = (int)MP; p.HR = (int)HR; p.B_pos = (int)B_pos;
+  return rotary_common("tppx_rotary_llama", p, (hipStream_t)stream);
+}
+
+extern "C" int tppx_rotary_kv_append_llama(void* q, void* k, const void* v, const void* emb_pos, const void* pos,
+                                           void* kcache, void* vcache, const void* offset_dev, int64_t B,
+                                           int64_t S, int64_t Nq, int64_t Nkv, int64_t H, int64_t MP, int64_t HR,
+                                           int64_t B_pos, int64_t Smax, tppx_stream_t stream) {
+  const char* who = "tppx_rotary_kv_append_llama";
+  TPPX_REQUIRE(k && v && kcache && vcache && offset_dev && pos, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(aligned16(k) && aligned16(v) && aligned16(kcache) && aligned16(vcache) && (!q || aligned16(q)),
+               TPPX_EINVAL, "%s: pointer not 16-byte aligned", who);
+  TPPX_REQUIRE(Nkv > 0 && Smax > 0 && (!q || Nq > 0), TPPX_ESHAPE, "%s: bad head counts / capacity", who);
+  RotaryParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = (uint16_t*)q; p.k = (uint16_t*)k; p.v = (const uint16_t*)v;
+  p.kc = (uint16_t*)kcache; p.vc = (uint16_t*)vcache;
+  p.emb = (const float*)emb_pos; p.pos = (const int64_t*)pos; p.offset = (const int32_t*)offset_dev;
+  p.B = (int)B; p.S = (int)S; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.H = (int)H; p.MP = (int)MP; p.HR = (int)HR;
+  p.B_pos = (int)B_pos; p.Smax = (int)Smax;
+  return rotary_common(who, p, (hipStream_t)stream);
+}
+
+extern "C" int tppx_attn_decode(const void* q, const void* kcache, const void* vcache, const void* mask,
+                                int64_t mask_ld, const void* kv_len_dev, int64_t kv_len_add, void* out, int64_t B, int64_t Nq,
+                                int64_t Nkv, int64_t H, int64_t Smax, void* ws, int64_t ws_bytes,
+                                tppx_stream_t stream) {
+  const char* who = "tppx_attn_decode";
+  TPPX_REQUIRE(q && kcache && vcache && kv_len_dev && out, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(aligned16(q) && aligned16(kcache) && aligned16(vcache) && aligned16(out), TPPX_EINVAL,
+               "%s: pointer not 16-byte aligned", who);
+  TPPX_REQUIRE(H == 128, TPPX_EUNSUPPORTED, "%s: head size %ld (only 128 is built)", who, (long)H);
+  TPPX_REQUIRE(B > 0 && Nq > 0 && Nkv > 0 && Nq % Nkv == 0 && Smax > 0 && B * Nq < (1 << 30), TPPX_ESHAPE,
+               "%s: bad shape B=%ld Nq=%ld Nkv=%ld Smax=%ld", who, (long)B, (long)Nq, (long)Nkv, (long)Smax);
+  TPPX_REQUIRE(ws_bytes >= 0 && (ws_bytes == 0 || ws), TPPX_EINVAL, "%s: workspace size given with a null workspace", who);
+  AttnParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = (const uint16_t*)q; p.kc = (const uint16_t*)kcache; p.vc = (const uint16_t*)vcache;
+  p.mask = (const uint16_t*)mask; p.kv_len = (const int32_t*)kv_len_dev; p.kv_len_add = (int)kv_len_add; p.out = (uint16_t*)out;
+  p.B = (int)B; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.Smax = (int)Smax; p.mask_ld = (int)mask_ld;
+  p.scale = 1.0f / sqrtf((float)H);
+  // enough workgroups to cover the chip about twice, at least 256 keys per split
+  int64_t splits = (512 + B * Nq - 1) / (B * Nq);
+  const int64_t max_by_len = (Smax + 255) / 256;
+  if (splits > max_by_len)
+    splits = max_by_len;
+  if (splits > 32)
+    splits = 32;
+  const int64_t need = B * Nq * splits * 130 * (int64_t)sizeof(float);
+  if (splits > 1 && need > ws_bytes)
+    splits = 1; // no room for partial results: one workgroup per head
+  p.splits = (int)splits;
+  p.part = (float*)ws;
+  attn_decode_kernel<<<dim3((unsigned)(B * Nq), (unsigned)splits), dim3(256), 0, (hipStream_t)stream>>>(p);
+  int rc = check_hip(hipGetLastError(), who);
+  if (rc || splits == 1)
+    return rc;
+  attn_combine_kernel<<<dim3((unsigned)(B * Nq)), dim3(128), 0, (hipStream_t)stream>>>(p);
+  return check_hip(hipGetLastError(), who);
+}

@@ -1,0 +1,258 @@
+"""Llama decoder layer on the GPU: the reference's fused decoder block
+(`LlamaDecoderLayer::_forward`, src/csrc/llm/fused_llm_infer.cpp:1195-1286) and
+its KV cache (`TppCache` / `LayerCache`, src/csrc/llm/attn.h:164-404) for the
+decode step (one new token per sequence), built from the quantized linears and
+the decode-side kernels of libtppx_hip.so.
+
+`LlamaDecoderLayer` keeps the constructor and `forward` signature of
+`torch.classes.tpp_llm.LlamaDecoderLayer` (fused_llm_infer.cpp:1084-1110,
+1186-1192, 1603-1606); `TppCache` keeps the reference's method names.  Prompt
+processing (more than one query token per sequence) is not built: the cache is
+filled with `TppCache.fill_` or token by token.
+"""
+import math
+
+import torch
+
+from .. import _lib, _ops
+from .._lib import TppxError
+
+
+# ---------------------------------------------------------------------------
+# operator wrappers
+# ---------------------------------------------------------------------------
+def _bf16_cuda(t, name):
+    if not t.is_cuda or t.dtype != torch.bfloat16:
+        raise TppxError(_lib.EINVAL, f"{name} must be a bfloat16 tensor on the GPU")
+    return t.contiguous()
+
+
+def rms_norm(t_in, t_wt, eps):
+    """llama_rms_norm (fused_llm_infer.cpp:337-363): bf16 in/out, fp32 or bf16 weight."""
+    L = _lib.lib()
+    x = _bf16_cuda(t_in, "input")
+    K = x.shape[-1]
+    if t_wt.dtype not in (torch.float32, torch.bfloat16) or t_wt.numel() != K or not t_wt.is_cuda:
+        raise TppxError(_lib.EINVAL, "llama_rms_norm: weight must be fp32 or bf16 [K] on the GPU")
+    y = torch.empty_like(x)
+    rows = x.numel() // K
+    if rows:
+        _lib.check(L.tppx_rms_norm(x.data_ptr(), t_wt.contiguous().data_ptr(), 0 if t_wt.dtype == torch.float32 else 1,
+                                   y.data_ptr(), rows, K, float(eps), _lib.stream_of(x)))
+    return y
+
+
+def apply_rotary_pos_emb_llama(t_in, t_emb_pos, t_pos, N, H):
+    """In place on t_in [B][S][N*H] (fused_llm_infer.cpp:207-253); t_emb_pos f32 [2][MP][HR]; t_pos i64 [B_pos][S]."""
+    L = _lib.lib()
+    if not t_in.is_cuda or t_in.dtype != torch.bfloat16 or not t_in.is_contiguous():
+        raise TppxError(_lib.EINVAL, "rotary: input must be a contiguous bfloat16 tensor on the GPU")
+    B, S = t_in.shape[0], t_in.shape[1]
+    _lib.check(L.tppx_rotary_llama(t_in.data_ptr(), t_emb_pos.data_ptr(), t_pos.data_ptr(), B, S, N, H,
+                                   t_emb_pos.shape[1], t_emb_pos.shape[2], t_pos.shape[0], _lib.stream_of(t_in)))
+    return t_in
+
+
+class TppCache:
+    """KV cache of all layers (TppCache, src/csrc/llm/attn.h:229-404).  Storage per layer is
+    `[B][Nkv][capacity][H]` bf16 for keys and for values (the reference's blocked
+    `[S1][B][N][32][H]` layouts are internal to its CPU kernels; nothing outside the class sees them).
+    The sequence length lives in a device int32 so that a decode step can be replayed as a graph."""
+
+    block_size = 32  # LayerCache::block_size, used by align_and_invert_mask
+
+    def __init__(self, capacity=0):
+        self.capacity = int(capacity)
+        self.layers = {}          # layer_idx -> (k, v)
+        self.seq_len_dev = None   # int32 [1]: keys in the cache (same for every layer)
+        self._host_len = 0
+
+    # -- reference method names -------------------------------------------------
+    def get_seq_length(self, layer_idx=0):
+        return self._host_len
+
+    def get_capacity(self):
+        return self.capacity
+
+    def size(self):
+        return len(self.layers)
+
+    def get(self, layer_idx):
+        k, v = self.layers[layer_idx]
+        return [k[:, :, :self._host_len], v[:, :, :self._host_len]]
+
+    def crop(self, max_length):
+        if self._host_len > max_length:
+            self._host_len = int(max_length)
+            self.seq_len_dev.fill_(self._host_len)
+
+    def align_and_invert_mask(self, t_mask, pad_value=-10000.0):
+        """attn.h:310-322: [B][S] 0/1 mask -> additive mask padded to a multiple of 32 keys."""
+        B, S = t_mask.shape
+        S_pad = (S + self.block_size - 1) // self.block_size * self.block_size
+        mask_pad = t_mask.new_full((B, S_pad), pad_value)
+        mask_pad[:, :S].masked_fill_(t_mask == 1, 0.0)
+        return mask_pad
+
+    # -- storage ------------------------------------------------------------------
+    def _ensure(self, layer_idx, B, Nkv, H, device):
+        if self.capacity <= 0:
+            raise TppxError(_lib.EINVAL, "TppCache: give the cache a capacity (keys per sequence) before use")
+        if layer_idx not in self.layers:
+            k = torch.zeros((B, Nkv, self.capacity, H), dtype=torch.bfloat16, device=device)
+            self.layers[layer_idx] = (k, torch.zeros_like(k))
+        if self.seq_len_dev is None:
+            self.seq_len_dev = torch.zeros(1, dtype=torch.int32, device=device)
+        return self.layers[layer_idx]
+
+    def fill_(self, layer_idx, keys, values):
+        """Load a context: keys / values bf16 [B][Nkv][S][H] become positions 0..S-1."""
+        B, Nkv, S, H = keys.shape
+        k, v = self._ensure(layer_idx, B, Nkv, H, keys.device)
+        k[:, :, :S].copy_(keys)
+        v[:, :, :S].copy_(values)
+        self._host_len = S
+        self.seq_len_dev.fill_(S)
+        return self
+
+    def advance(self, n=1):
+        """One decode step appended n keys to every layer (host-side bookkeeping + device counter)."""
+        self._host_len += n
+        self.seq_len_dev.add_(n)
+
+
+class LlamaDecoderLayer:
+    """torch.classes.tpp_llm.LlamaDecoderLayer(params, layer_idx, eps, H, max_positions, rotary_dim)
+    with params = [ln_in gamma, Wq, Wk, Wv, Wo, ln_post gamma, Wg, Wu, Wd, embed_positions]
+    (fused_llm_infer.cpp:1096-1110); the linears are quantized tensors of this package."""
+
+    def __init__(self, params, layer_idx, eps, H, max_positions, rotary_dim):
+        (self.t_Gi, self.t_Wq, self.t_Wk, self.t_Wv, self.t_Wp, self.t_Gpa,
+         self.t_Wg, self.t_Wu, self.t_Wd, self.t_EP) = params
+        self.layer_idx, self.eps, self.H = int(layer_idx), float(eps), int(H)
+        self.max_positions, self.rotary_dim = int(max_positions), int(rotary_dim)
+        self.Nq = _ops._as_q(self.t_Wq).weight_nk()[0] // self.H
+        self.Nkv = _ops._as_q(self.t_Wk).weight_nk()[0] // self.H
+
+    def forward(self, inputs, cache, use_cache=True):
+        """inputs = [hidden [B][1][hidden], additive mask [B][keys] or empty, position_ids i64 [B or 1][1]]."""
+        L = _lib.lib()
+        t_HS, t_am, t_pid = inputs[0], inputs[1], inputs[2]
+        B, S, hidden = t_HS.shape
+        if S != 1:
+            raise TppxError(_lib.EUNSUPPORTED, "LlamaDecoderLayer: only the decode step (one token per sequence) is built")
+        st = _lib.stream_of(t_HS)
+        empty = torch.empty(0, dtype=torch.bfloat16, device=t_HS.device)
+        t_res = t_HS
+        h = rms_norm(t_HS, self.t_Gi, self.eps)
+        q, k, v = _ops.qkv_gemm(h, [self.t_Wq, self.t_Wk, self.t_Wv], [empty] * 3)
+        kc, vc = cache._ensure(self.layer_idx, B, self.Nkv, self.H, t_HS.device)
+        # rotary on q and k + append of k, v at position seq_len (device counter), one launch
+        _lib.check(L.tppx_rotary_kv_append_llama(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), self.t_EP.data_ptr(), t_pid.data_ptr(), kc.data_ptr(),
+            vc.data_ptr(), cache.seq_len_dev.data_ptr(), B, 1, self.Nq, self.Nkv, self.H, self.t_EP.shape[1],
+            self.t_EP.shape[2], t_pid.shape[0], cache.capacity, st))
+        # attention over seq_len + 1 keys
+        ctx = torch.empty_like(q)
+        ws = _lib.workspace(t_HS)
+        mask_ptr = t_am.data_ptr() if t_am is not None and t_am.numel() else None
+        mask_ld = t_am.shape[-1] if mask_ptr else 0
+        _lib.check(L.tppx_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
+                                      cache.seq_len_dev.data_ptr(), 1, ctx.data_ptr(), B, self.Nq, self.Nkv, self.H,
+                                      cache.capacity, ws.data_ptr(), ws.numel(), st))
+        t_SO = _ops.fc_add(ctx, self.t_Wp, empty, t_res, 1.0)
+        h = rms_norm(t_SO, self.t_Gpa, self.eps)
+        t_I = _ops.swiglu_gate_up(h, self.t_Wg, self.t_Wu)
+        t_Out = _ops.fc_add(t_I, self.t_Wd, empty, t_SO, 1.0)
+        return [t_Out]
+
+
+def llama_rotary_table(max_positions, head_dim, base=10000.0, device="cuda"):
+    """embed_positions as OptimizeModelForLlama builds it (fused_llama_infer.py:188-201): f32 [2][MP][head_dim]
+    = cos / sin of position * inv_freq, frequencies repeated over the two halves."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    freqs = torch.outer(torch.arange(max_positions, dtype=torch.float32), inv_freq)
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return torch.stack((emb.cos(), emb.sin())).to(device)
+
+
+class LlamaDecoder:
+    """Self-contained Llama-shape decoder for greedy decoding with random-initialised, quantized weights:
+    embedding, `n_layers` LlamaDecoderLayer, final RMSNorm, quantized lm_head, argmax.  One decode step is
+    captured once as a HIP graph (positions, sequence length and the current token live in device memory)
+    and replayed per token."""
+
+    def __init__(self, hidden=4096, inter=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab=32000,
+                 max_positions=4096, eps=1e-5, weight_dtype="mxfp4", seed=0, device="cuda"):
+        self.hidden, self.n_layers, self.vocab = hidden, n_layers, vocab
+        self.H = hidden // n_heads
+        self.eps, self.device = eps, torch.device(device)
+        g = torch.Generator(device=self.device).manual_seed(seed)
+        quant = _ops.remap_and_quantize_mxfp4 if weight_dtype == "mxfp4" else _ops.remap_and_quantize_qint8
+
+        def lin(N, K):
+            W = (torch.randn((N, K), generator=g, device=self.device) * 0.02).to(torch.bfloat16)
+            q = quant(W.view(N // 16, 16, K // 64, 32, 2).permute(0, 2, 3, 1, 4).contiguous())
+            q.native()
+            return q
+
+        self.embed = (torch.randn((vocab, hidden), generator=g, device=self.device) * 0.02).to(torch.bfloat16)
+        self.EP = llama_rotary_table(max_positions, self.H, device=self.device)
+        ones = torch.ones(hidden, dtype=torch.float32, device=self.device)
+        self.layers = []
+        for i in range(n_layers):
+            params = [ones, lin(n_heads * self.H, hidden), lin(n_kv_heads * self.H, hidden), lin(n_kv_heads * self.H, hidden),
+                      lin(hidden, n_heads * self.H), ones, lin(inter, hidden), lin(inter, hidden), lin(hidden, inter), self.EP]
+            self.layers.append(LlamaDecoderLayer(params, i, eps, self.H, max_positions, self.H))
+        self.norm_w = ones
+        self.lm_head = lin(vocab, hidden)
+        self.n_kv_heads = n_kv_heads
+        self._graph = None
+
+    def new_cache(self, B, context, capacity, seed=1):
+        """Cache pre-filled with `context` positions of N(0,1) keys / values in every layer."""
+        cache = TppCache(capacity)
+        g = torch.Generator(device=self.device).manual_seed(seed)
+        for i in range(self.n_layers):
+            shape = (B, self.n_kv_heads, context, self.H)
+            cache.fill_(i, torch.randn(shape, generator=g, device=self.device).to(torch.bfloat16),
+                        torch.randn(shape, generator=g, device=self.device).to(torch.bfloat16))
+        return cache
+
+    def step(self, tokens, pos, cache):
+        """tokens i64 [B] (device), pos i64 [B][1] (device) -> next tokens i64 [B]; appends to the cache storage
+        (the caller advances the counters)."""
+        h = self.embed.index_select(0, tokens).unsqueeze(1)
+        for layer in self.layers:
+            h = layer.forward([h, None, pos], cache)[0]
+        h = rms_norm(h, self.norm_w, self.eps)
+        logits = _ops.fc_plain(h, self.lm_head, None)
+        return logits.view(logits.shape[0], -1).argmax(dim=-1)
+
+    def greedy_decode(self, tokens, cache, n_new, use_graph=True):
+        """Greedy decode of n_new tokens per sequence from the [B] start tokens; returns i64 [B][n_new]."""
+        B = tokens.shape[0]
+        cur = tokens.clone()
+        pos = torch.full((B, 1), cache.get_seq_length(), dtype=torch.int64, device=self.device)
+        out = torch.empty((B, n_new), dtype=torch.int64, device=self.device)
+        if use_graph:
+            nxt = self.step(cur, pos, cache)  # warm-up outside capture (allocations, lazy module loads)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                nxt = self.step(cur, pos, cache)
+                cur.copy_(nxt)
+                pos.add_(1)
+                cache.seq_len_dev.add_(1)
+            for t in range(n_new):
+                graph.replay()
+                out[:, t].copy_(cur)
+                cache._host_len += 1
+        else:
+            for t in range(n_new):
+                nxt = self.step(cur, pos, cache)
+                cur.copy_(nxt)
+                out[:, t].copy_(cur)
+                pos.add_(1)
+                cache.advance(1)
+        return out
