@@ -55,7 +55,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--fmt", default="qint8", choices=["qint8", "mxfp4"])
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill"],
+    ap.add_argument("--batch", type=int, default=1, help="sequences for --workload tokens (1 or 16 in the baseline)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "tokens"],
                     help="decode = the configuration the headline metric is quoted on (default); prefill = the "
                          "MXFP4 linears of one 70B-shape decoder layer at M = 2048 (TFLOP/s, MFMA roofline)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
@@ -82,6 +83,8 @@ def main():
 
     if args.workload == "prefill":
         return run_prefill(torch, _ops, args)
+    if args.workload == "tokens":
+        return run_tokens(torch, args)
 
     fmt = args.fmt
     shapes = {"up": (11008, 4096), "down": (4096, 11008)}
@@ -195,6 +198,44 @@ def main():
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))
+
+
+def run_tokens(torch, args):
+    """BASELINE config 5: 32-layer Llama-2-7B-shape decoder, all linears (and the lm_head) MXFP4, KV cache
+    pre-filled with 2048 positions of N(0,1), greedy decode of 128 new tokens for `--batch` sequences from
+    random token ids; the decode step is one replayed HIP graph."""
+    from tpp_pytorch_extension.llm import fused_llama_infer as F
+    dev = torch.device("cuda:0")
+    B, ctx, new = args.batch, 2048, 128
+    model = F.LlamaDecoder(hidden=4096, inter=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab=32000,
+                           max_positions=4096, weight_dtype="mxfp4", seed=1239)
+    tok = torch.randint(0, 32000, (B,), generator=torch.Generator().manual_seed(5), dtype=torch.int64).to(dev)
+    model.greedy_decode(tok, model.new_cache(B, ctx, ctx + new + 32), 8)  # warm-up run
+    cache = model.new_cache(B, ctx, ctx + new + 32)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = model.greedy_decode(tok, cache, new)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    # the replays alone (capture and warm-up step excluded)
+    cache2 = model.new_cache(B, ctx, ctx + new + 32)
+    steps_t = model.time_decode_steps(tok, cache2, new)
+    ms = steps_t * 1e3 / new
+    lin_bytes = 32 * (3 * 4096 * 4096 + 4096 * 4096 + 3 * 11008 * 4096) * (0.5 + 1.0 / 32) + 32000 * 4096 * (0.5 + 1.0 / 32)
+    kv_bytes = B * 32 * 2 * 32 * (ctx + new / 2) * 128 * 2
+    achieved = (lin_bytes + kv_bytes) / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "7B-shape decode tokens/s", "value": round(B * new / steps_t, 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": new, "warmup": 8, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"cfg5: 32-layer Llama-2-7B-shape decoder, MXFP4 linears and lm_head, bf16 RMSNorm / rotary / "
+                               f"KV cache, context {ctx} of N(0,1), greedy decode of {new} tokens, batch {B}",
+                   "launch": "one HIP graph per decode step, replayed", "batch": B,
+                   "wall_s_including_capture": round(dt, 4), "tokens": int(out.numel())},
+        "roofline": {"bound": "hbm", "kernel": "whole decode step (all kernels of the graph)", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_step": int(lin_bytes + kv_bytes)},
+        "cpu_baseline": None}))
 
 
 def run_prefill(torch, _ops, args):

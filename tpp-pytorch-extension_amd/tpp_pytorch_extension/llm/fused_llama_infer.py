@@ -229,6 +229,28 @@ class LlamaDecoder:
         logits = _ops.fc_plain(h, self.lm_head, None)
         return logits.view(logits.shape[0], -1).argmax(dim=-1)
 
+    def time_decode_steps(self, tokens, cache, n_new):
+        """Seconds spent in n_new replays of the captured decode step (capture excluded)."""
+        import time
+        B = tokens.shape[0]
+        cur = tokens.clone()
+        pos = torch.full((B, 1), cache.get_seq_length(), dtype=torch.int64, device=self.device)
+        self.step(cur, pos, cache)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            nxt = self.step(cur, pos, cache)
+            cur.copy_(nxt)
+            pos.add_(1)
+            cache.seq_len_dev.add_(1)
+        graph.replay()  # one untimed replay
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_new - 1):
+            graph.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * n_new / (n_new - 1)
+
     def greedy_decode(self, tokens, cache, n_new, use_graph=True):
         """Greedy decode of n_new tokens per sequence from the [B] start tokens; returns i64 [B][n_new]."""
         B = tokens.shape[0]
