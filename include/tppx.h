@@ -206,6 +206,25 @@ int tppx_swiglu_mxfp4(const void* x, const void* qw_gate, const void* sw_gate,
                       int64_t M, int64_t N, int64_t K, int flags, void* ws,
                       int64_t ws_bytes, tppx_stream_t stream);
 
+/* llama_rms_norm followed by the GEMMs that consume it, in ONE launch, for
+ * decode steps (M <= 16): the two calls
+ *   t_HS = llama_rms_norm(t_HS, gamma, eps); fused_qkv_gemm(t_HS, {Wq,Wk,Wv}, ...)
+ * (src/csrc/llm/fused_llm_infer.cpp:1231,1247-1251) resp.
+ *   t_HS = llama_rms_norm(t_SO, gamma, eps); i_gemm(Silu)...; i_gemm(Mul)...
+ * (:1269-1272) with the same bf16 rounding of the normalised activations.
+ * gamma f32 [K]; gamma == NULL skips the normalisation (same kernel, plain x).
+ * TPPX_EUNSUPPORTED when M > 16 or K is too large for the LDS staging: run
+ * tppx_rms_norm and the GEMM entry points separately then. */
+int tppx_norm_multi_linear_mxfp4(const void* x, const void* gamma, float eps,
+                                 const tppx_seg* segs, int n_segs, int64_t M,
+                                 int64_t K, int flags, tppx_stream_t stream);
+int tppx_norm_swiglu_mxfp4(const void* x, const void* gamma, float eps,
+                           const void* qw_gate, const void* sw_gate,
+                           const void* bias_gate, const void* qw_up,
+                           const void* sw_up, const void* bias_up, void* y,
+                           int64_t M, int64_t N, int64_t K, int flags,
+                           tppx_stream_t stream);
+
 /* ---- decode-side operators of the decoder layer -------------------------- */
 
 /* Replaces llama_rms_norm / RMSNormFwdTPP (src/csrc/llm/fused_llm_infer.cpp:309-363,

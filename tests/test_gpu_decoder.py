@@ -182,3 +182,40 @@ def test_greedy_decode_graph_equals_eager():
     a = model.greedy_decode(tok, model.new_cache(3, 40, 64), 8, use_graph=False)
     b = model.greedy_decode(tok, model.new_cache(3, 40, 64), 8, use_graph=True)
     assert a.shape == (3, 8) and torch.equal(a, b)
+
+
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("K", [512, 4096])
+def test_rms_norm_fused_into_gemms(M, K, monkeypatch):
+    """llama_rms_norm inside the q/k/v launch and inside the gate/up launch gives the bits of the separate
+    normalisation kernel followed by the plain GEMM launches, except where the row scale differs in its last bit
+    (sum order) and flips a bf16 rounding of a normalised activation: compared with the GEMM tolerance."""
+    F = _llm()
+    from tpp_pytorch_extension import _ops
+    monkeypatch.setattr(_ops, "FUSE_NORM", True)
+    Ns = (1536, 512, 512) if K == 4096 else (12288, 256, 256)   # 768+ channel tiles exercise 3 tiles per workgroup
+    ws = []
+    for i, n in enumerate(Ns):
+        W = randn_bf16((n, K), 0.03, 400 + i)
+        ws.append(_ops.remap_and_quantize_mxfp4(block_bf16(W).cuda()))
+    x = randn_bf16((M, K), 1.3, 410).cuda()
+    gamma = (torch.rand(K, generator=torch.Generator().manual_seed(411)) + 0.5).cuda()
+    fused = _ops.qkv_gemm(x, ws, [None] * 3, norm=(gamma, 1e-5))
+    h = F.rms_norm(x, gamma, 1e-5)
+    sep = _ops.qkv_gemm(h, ws, [None] * 3)
+    for a, b in zip(fused, sep):
+        assert_close_bf16(t2bits(a), t2bits(b), what=f"fused norm qkv M={M} K={K}")
+        assert (a != b).float().mean() < 0.01
+    wg, wu = ws[1], ws[2]
+    fz = _ops.swiglu_gate_up(x, wg, wu, norm=(gamma, 1e-5))
+    sp = _ops.swiglu_gate_up(h, wg, wu)
+    assert_close_bf16(t2bits(fz), t2bits(sp), ulps=2, what=f"fused norm swiglu M={M} K={K}")
+    # without a norm the same entry point is a plain GEMM
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    qn, sn = ws[0].native()
+    y = torch.empty((M, Ns[0]), dtype=torch.bfloat16, device="cuda")
+    seg = (_lib.Seg * 1)()
+    seg[0].qw, seg[0].sw, seg[0].y, seg[0].N, seg[0].post_op, seg[0].post_scale = qn.data_ptr(), sn.data_ptr(), y.data_ptr(), Ns[0], 0, 1.0
+    _lib.check(L.tppx_norm_multi_linear_mxfp4(h.data_ptr(), None, 0.0, seg, 1, M, K, 0, _lib.stream_of(h)))
+    assert_close_bf16(t2bits(y), t2bits(sep[0]), what="LDS-staged plain GEMM")

@@ -117,6 +117,22 @@ static void set_groups(DecodeParams& p, int tiles_per_group, bool dual) {
   p.groups = groups;
 }
 
+// LDS-staged decode kernel (M <= 16): channel tiles per workgroup = the fewest that keep the grid within one round of
+// 256 workgroups (the kernel runs one workgroup per CU).  False when the K slice of a wave does not fit its staging.
+static bool plan_xl(DecodeParams& p, bool dual, int* nt_out) {
+  const int nt_max = dual ? 3 : 4;
+  int nt = 1;
+  for (; nt < nt_max; nt++) {
+    set_groups(p, nt, dual);
+    if (p.groups <= 256)
+      break;
+  }
+  set_groups(p, nt, dual);
+  *nt_out = nt;
+  // staging per wave: 16 rows x 32 chunks of 16 bytes, so at most 2 K tiles per wave and slices of 16 or 32 chunks
+  return p.units <= 32 && (p.units % 16 == 0 || p.units <= 16) && skinny_mxfp4_xl_lds(p.units, nt, dual) <= 160 * 1024;
+}
+
 static int fill_all(const char* who, const tppx_seg* segs, int n_segs, int n_mult, bool dual,
                     DecodeParams& p) {
   int tiles = 0, groups = 0;
@@ -226,6 +242,9 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     }
     return TPPX_OK;
   }
+  int nt_xl = 1;
+  if (M <= 16 && env_int("TPPX_MXFP4_XL", 1) == 1 && plan_xl(p, dual, &nt_xl))
+    return check_hip(launch_skinny_mxfp4_xl(p, nt_xl, dual, stream), who);
   if (M <= 16 && env_int("TPPX_MXFP4_SPLITK", 0) == 0) {
     // GEMV class: K reduction inside the workgroup
     SkinnyPlan sp = plan_skinny(0, M, p.total_tiles, p.units, dual);
@@ -306,9 +325,52 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
   return check_hip(launch_skinny_qint8(p, sp, stream), who);
 }
 
+// LDS-staged MXFP4 decode kernel (M <= 16) with an optional RMSNorm in front
+static int run_mxfp4_xl(const char* who, const void* x, const void* gamma, float eps, const tppx_seg* segs,
+                        int n_segs, int64_t M, int64_t K, int flags, bool dual, hipStream_t stream) {
+  int rc = check_common(who, x, M, K, n_segs, flags, nullptr, 0);
+  if (rc)
+    return rc;
+  TPPX_REQUIRE(segs, TPPX_EINVAL, "%s: null segment table", who);
+  TPPX_REQUIRE(K > 0 && K % 128 == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of 128", who, (long)K);
+  TPPX_REQUIRE(M <= 16, TPPX_EUNSUPPORTED, "%s: more than 16 rows (M=%ld): run the normalisation and the GEMM separately", who, (long)M);
+  TPPX_REQUIRE(gamma == nullptr || aligned16(gamma), TPPX_EINVAL, "%s: gamma not 16-byte aligned", who);
+  DecodeParams p;
+  memset(&p, 0, sizeof(p));
+  rc = fill_all(who, segs, n_segs, 32, dual, p);
+  if (rc)
+    return rc;
+  p.x = x;
+  p.M = (int)M;
+  p.K = (int)K;
+  p.units = (int)(K / 128);
+  p.tpb = 1;
+  p.S = 1;
+  p.norm_gamma = (const float*)gamma;
+  p.norm_eps = eps;
+  int nt = 1;
+  TPPX_REQUIRE(plan_xl(p, dual, &nt), TPPX_EUNSUPPORTED,
+               "%s: K=%ld does not split into 16 slices of 128 or 256 input channels (or fewer than 16 tiles) that fit the LDS staging; run the steps separately", who, (long)K);
+  return check_hip(launch_skinny_mxfp4_xl(p, nt, dual, stream), who);
+}
+
 } // namespace tppx
 
 using namespace tppx;
+
+extern "C" int tppx_norm_multi_linear_mxfp4(const void* x, const void* gamma, float eps, const tppx_seg* segs,
+                                            int n_segs, int64_t M, int64_t K, int flags, tppx_stream_t stream) {
+  return run_mxfp4_xl("tppx_norm_multi_linear_mxfp4", x, gamma, eps, segs, n_segs, M, K, flags, false, (hipStream_t)stream);
+}
+
+extern "C" int tppx_norm_swiglu_mxfp4(const void* x, const void* gamma, float eps, const void* qw_gate,
+                                      const void* sw_gate, const void* bias_gate, const void* qw_up,
+                                      const void* sw_up, const void* bias_up, void* y, int64_t M, int64_t N,
+                                      int64_t K, int flags, tppx_stream_t stream) {
+  tppx_seg s[2] = {{qw_gate, sw_gate, bias_gate, nullptr, nullptr, y, N, TPPX_POST_NONE, 1.0f},
+                   {qw_up, sw_up, bias_up, nullptr, nullptr, y, N, TPPX_POST_NONE, 1.0f}};
+  return run_mxfp4_xl("tppx_norm_swiglu_mxfp4", x, gamma, eps, s, 2, M, K, flags, true, (hipStream_t)stream);
+}
 
 extern "C" int tppx_version(void) {
   return TPPX_VERSION;

@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 #include "tppx.h"
 
@@ -94,6 +95,15 @@ __device__ __forceinline__ uint32_t apply_post_bits(float v, int post,
 // exponent field; 0 gives 0.0, 255 gives +Inf).
 __device__ __forceinline__ float e8m0_to_f32(uint32_t x) {
   return __uint_as_float((x & 0xffu) << 23);
+}
+
+// compile-time loop: f(std::integral_constant<int, I>) for I in [B, E)
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    static_for<B + 1, E>(f);
+  }
 }
 
 } // namespace tppx

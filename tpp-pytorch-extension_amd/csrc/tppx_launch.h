@@ -39,6 +39,8 @@ struct DecodeParams {
   int S;     // K splits across workgroups
   int cht;   // tiles of activations staged in LDS at a time
   float* part;   // [S][grid_y][total_tiles][acc][MG][64] x f32x4 partial tiles (S > 1)
+  const float* norm_gamma; // f32 [K]: RMSNorm fused in front of the GEMM (LDS-staged MXFP4 kernel), or null
+  float norm_eps;
 };
 
 struct DecodePlan {
@@ -86,6 +88,8 @@ hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qb
 SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual);
 hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream);
 hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream);
+size_t skinny_mxfp4_xl_lds(int units, int nt, bool dual);
+hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_t stream);
 
 DecodePlan plan_decode(int fmt, int64_t M, int groups, int total_tiles, int units, int tpb, bool dual,
                        size_t ws_bytes);

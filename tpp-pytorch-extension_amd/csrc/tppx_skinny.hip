@@ -82,10 +82,11 @@ struct SkEpilogue {
     }
   }
 
-  __device__ __forceinline__ void finish(const DecodeSeg& sg, f32x4 (&acc)[NACC][MG], float* red) {
+  // stride = floats between the regions of two waves (>= ELEMS)
+  __device__ __forceinline__ void finish(const DecodeSeg& sg, f32x4 (&acc)[NACC][MG], float* red, int stride = ELEMS) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int W = blockDim.x >> 6;
-    float* mine = red + wave * ELEMS;
+    float* mine = red + wave * stride;
 #pragma unroll
     for (int a = 0; a < NACC; a++)
 #pragma unroll
@@ -100,10 +101,10 @@ struct SkEpilogue {
       if (e < OUT) {
         float v = 0.f, v2 = 0.f;
         for (int w = 0; w < W; w++)
-          v += red[w * ELEMS + e];
+          v += red[w * stride + e];
         if (DUAL)
           for (int w = 0; w < W; w++)
-            v2 += red[w * ELEMS + e + ELEMS / 2];
+            v2 += red[w * stride + e + ELEMS / 2];
         if (ok[i]) {
           uint32_t out;
           if (DUAL) {
@@ -574,6 +575,208 @@ skinny_mxfp4_kernel(const DecodeParams p) {
 }
 
 // ---------------------------------------------------------------------------
+// MXFP4, M <= 16, activations staged in LDS by the wave that consumes them,
+// with an optional transform on the way in:
+//   XMODE 0  x as it is
+//   XMODE 1  RMSNorm: bf16((x * rsqrt(mean_k x^2 + eps)) * gamma[k]) -- the
+//            normalisation kernel in front of the GEMM disappears
+// Sixteen waves split K.  A wave reads its K slice of every row with
+// row-contiguous 16-byte loads (a wave instruction covers whole 256-byte row
+// segments; the operand-shaped reads of the register path touch 16 cache
+// lines per 16 lanes) and writes it to its private LDS region as
+// [chunk][row ^ (chunk & 15)] x 16 B: conflict free on the way in and as MFMA
+// operand reads (lane = row, 4 K groups) on the way out.  The main loop then
+// streams only weights.  RMSNorm needs the whole row: the 16 waves exchange
+// per-(row, K tile) partial sums of squares through LDS and add them in a
+// fixed order.  The reduction scratch of the epilogue reuses the x regions.
+// ---------------------------------------------------------------------------
+template <int NT, int PF, bool DUAL, int XMODE>
+__global__ void __launch_bounds__(1024)
+skinny_mxfp4_xl_kernel(const DecodeParams p) {
+  extern __shared__ __align__(16) float sk_lds[];
+  constexpr int NTW = DUAL ? 2 * NT : NT;
+  constexpr int W = 16;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int grp = blockIdx.x;
+  const int seg_id = DUAL ? 0 : sk_find_seg(p, grp);
+  const DecodeSeg& sg = p.seg[seg_id];
+  const int ltile0 = (grp - sg.grp0) * NT;
+  const int KT = p.units;
+  const int t0 = (wave * KT) / W, t1 = ((wave + 1) * KT) / W;
+  const int cht = p.cht;                       // K tiles per wave, at most
+  const int wstride = max(cht * 1024, NTW * 256); // floats per wave region (x slice, later the reduction scratch)
+  uint4* xs = reinterpret_cast<uint4*>(sk_lds + (size_t)wave * wstride);
+  float* wss = sk_lds + (size_t)W * wstride;   // [wave][row 16][tile cht] partial sums of squares
+
+  constexpr int NSEG = DUAL ? 2 : 1;
+  const char* qwb[NSEG];
+  const char* swb[NSEG];
+#pragma unroll
+  for (int sgi = 0; sgi < NSEG; sgi++) {
+    const DecodeSeg& ss = p.seg[DUAL ? sgi : seg_id];
+    qwb[sgi] = reinterpret_cast<const char*>(ss.qw);
+    swb[sgi] = reinterpret_cast<const char*>(ss.sw);
+  }
+  uint32_t woff[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; nt++)
+    woff[nt] = (uint32_t)(min(ltile0 + nt, sg.tiles - 1) * KT * 64 + lane);
+
+  // ---- activations of this wave's K slice -> LDS ----
+  // Loads return in issue order, so the (L2-resident) activation and gamma
+  // loads go out BEFORE the weight ring and are not held up by HBM latency.
+  constexpr int XNI = 8;                   // (row, chunk) items per lane: 16 rows x 32 chunks / 64 lanes
+  const int nch = (t1 - t0) * 16;          // 16-byte chunks per row in the slice
+  const int items = p.M * nch;             // (row, chunk), chunk fastest: 16 consecutive lanes = one K tile of one row
+  const int nsh = nch > 16 ? 5 : 4;        // the host admits slices of 0, 16 or 32 chunks only
+  const int cmask = (1 << nsh) - 1;
+  const char* xb = reinterpret_cast<const char*>(p.x);
+  const uint32_t xk0 = (uint32_t)t0 * 256u; // byte offset of the slice inside a row
+  i32x4 raw[XNI]; // first-class vectors: copies of the HIP struct type are memcpys, which keep the array in scratch
+  // items past the end repeat the last one (and later store the same value to the same slot): nothing depends on
+  // the lane, so the loads stay batched in front of the weight ring.  Up to 4 rows need the first 2 items only.
+  const bool many = items > 2 * 64;
+  auto load_x = [&](auto IT) {
+    constexpr int it = decltype(IT)::value;
+    const int i = min(it * 64 + lane, max(items - 1, 0));
+    const int row = i >> nsh, ck = i & cmask;
+    raw[it] = *reinterpret_cast<const i32x4*>(xb + (size_t)((uint32_t)(row * p.K) * 2u + xk0 + (uint32_t)ck * 16u));
+  };
+  static_for<0, 2>(load_x);
+  if (many)
+    static_for<2, XNI>(load_x);
+  // the chunk of a lane is the same in every item when the slice is 16 or 32 chunks wide
+  float gm[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};
+  if (XMODE == 1 && nch) {
+    const float4* gp = reinterpret_cast<const float4*>(p.norm_gamma + (size_t)t0 * 128 + (size_t)(lane & cmask) * 8);
+    const float4 g0 = gp[0], g1 = gp[1];
+    gm[0] = g0.x; gm[1] = g0.y; gm[2] = g0.z; gm[3] = g0.w;
+    gm[4] = g1.x; gm[5] = g1.y; gm[6] = g1.z; gm[7] = g1.w;
+  }
+  SkEpilogue<1, NTW, DUAL, 16> ep;
+  ep.prefetch(p, sg, ltile0, 0);
+
+  // weight ring: it has the HBM latency to cover
+  i32x4 wreg[PF][NTW];
+  uint32_t sreg[PF][NTW];
+  auto load_stage = [&](int st, int t) {
+    t = min(t, t1 - 1);
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++) {
+      const uint32_t slot = woff[nt % NT] + (uint32_t)t * 64u;
+      wreg[st][nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(qwb[nt / NT] + (size_t)(slot * 16u)));
+      sreg[st][nt] = *reinterpret_cast<const uint8_t*>(swb[nt / NT] + (size_t)slot);
+    }
+  };
+  if (t0 < t1) {
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+      load_stage(i, t0 + i);
+  }
+
+  float* srow = wss + W * 16 * cht + wave * 16; // this wave's copy of the 16 row scales
+  // raw activations go to their operand slots right away; the norm rescales them in place
+  auto stash_x = [&](auto IT) {
+    constexpr int it = decltype(IT)::value;
+    const int i = it * 64 + lane;
+    const int ic = min(i, max(items - 1, 0));
+    const int row = ic >> nsh, ck = ic & cmask;
+    if (XMODE == 1) {
+      const uint32_t d[4] = {(uint32_t)raw[it][0], (uint32_t)raw[it][1], (uint32_t)raw[it][2], (uint32_t)raw[it][3]};
+      float ssq = 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const float lo = bf16_bits_to_f32(d[e] & 0xffffu), hi = bf16_bits_to_f32(d[e] >> 16);
+        ssq = fmaf(lo, lo, ssq);
+        ssq = fmaf(hi, hi, ssq);
+      }
+      // sum over the 16 lanes of a DPP row = one (row, K tile) pair
+      ssq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ssq), 0xB1, 0xf, 0xf, true));
+      ssq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ssq), 0x4E, 0xf, 0xf, true));
+      ssq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ssq), 0x141, 0xf, 0xf, true));
+      ssq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ssq), 0x140, 0xf, 0xf, true));
+      if (i < items && (lane & 15) == 0)
+        wss[(wave * 16 + row) * cht + (ck >> 4)] = ssq;
+    }
+    *reinterpret_cast<i32x4*>(&xs[ck * 16 + (row ^ (ck & 15))]) = raw[it];
+  };
+  static_for<0, 2>(stash_x);
+  if (many)
+    static_for<2, XNI>(stash_x);
+  if (XMODE == 1) {
+    __syncthreads();
+    // mean of squares of whole rows: waves and tiles in a fixed order; lane r < 16 owns row r
+    if (lane < 16 && lane < p.M) {
+      float tot = 0.f;
+      for (int w2 = 0; w2 < W; w2++) {
+        const int nt2 = ((w2 + 1) * KT) / W - (w2 * KT) / W;
+        for (int tl = 0; tl < nt2; tl++)
+          tot += wss[(w2 * 16 + lane) * cht + tl];
+      }
+      srow[lane] = 1.0f / sqrtf(tot * (1.0f / (float)p.K) + p.norm_eps);
+    }
+    __builtin_amdgcn_wave_barrier(); // the scales are read by the other lanes of this wave
+#pragma unroll 1
+    for (int i = lane; i < items; i += 64) {
+      const int row = i >> nsh, ck = i & cmask;
+      uint4* slot = &xs[ck * 16 + (row ^ (ck & 15))];
+      const uint4 w = *slot;
+      const float sc = srow[row];
+      const uint32_t d[4] = {w.x, w.y, w.z, w.w};
+      uint32_t o[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const float lo = (bf16_bits_to_f32(d[e] & 0xffffu) * sc) * gm[2 * e];
+        const float hi = (bf16_bits_to_f32(d[e] >> 16) * sc) * gm[2 * e + 1];
+        o[e] = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+      }
+      *slot = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+  }
+  // the wave reads only what it wrote itself: program order is enough
+
+  f32x4 acc[NTW][1];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++)
+    acc[nt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // operand slot of this lane for step j inside a K tile: chunk g*4 + j, row m
+  int rdo[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int cj = (lane >> 4) * 4 + j;
+    rdo[j] = cj * 16 + ((lane & 15) ^ cj);
+  }
+  auto consume = [&](int i, int tl) {
+    bf16x8 xa[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      xa[j] = __builtin_bit_cast(bf16x8, xs[tl * 256 + rdo[j]]);
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++) {
+      const float sc = e8m0_to_f32(sreg[i][nt]);
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        acc[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            xa[j], sk_cvt_fp4x8((uint32_t)wreg[i][nt][j], sc), acc[nt][0], 0, 0, 0);
+    }
+  };
+  for (int t = t0; t < t1; t += PF) {
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      const int tt = t + i;
+      if (tt < t1) {
+        consume(i, tt - t0);
+        if (tt + PF < t1)
+          load_stage(i, tt + PF);
+      }
+    }
+  }
+  __syncthreads(); // every wave is done with its x region before it becomes reduction scratch
+  ep.finish(sg, acc, sk_lds, wstride);
+}
+
+// ---------------------------------------------------------------------------
 // planning and launch
 // ---------------------------------------------------------------------------
 SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual) {
@@ -664,6 +867,39 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
     default: SKQ(4, 1, 8, 8, 8);
   }
 #undef SKQ
+}
+
+// x staged in LDS, optional fused RMSNorm; 16 waves; nt = channel tiles per workgroup (of each GEMM when dual)
+size_t skinny_mxfp4_xl_lds(int units, int nt, bool dual) {
+  const int cht = (units + 15) / 16;
+  const int ntw = dual ? 2 * nt : nt;
+  const size_t wstride = (size_t)(cht * 1024 > ntw * 256 ? cht * 1024 : ntw * 256);
+  return (16 * wstride + (size_t)16 * 16 * cht + 16 * 16) * sizeof(float);
+}
+
+hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_t stream) {
+  p.cht = (p.units + 15) / 16;
+  const size_t lds = skinny_mxfp4_xl_lds(p.units, nt, dual);
+  dim3 grid(p.groups, 1);
+  const bool norm = p.norm_gamma != nullptr;
+#define SKXL(NT, DUAL)                                                                                       \
+  return norm ? sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 1>, p, grid, 16, lds, stream)                  \
+              : sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 0>, p, grid, 16, lds, stream)
+  if (dual) {
+    if (nt == 3)
+      SKXL(3, true);
+    if (nt == 2)
+      SKXL(2, true);
+    SKXL(1, true);
+  }
+  if (nt == 4)
+    SKXL(4, false);
+  if (nt == 3)
+    SKXL(3, false);
+  if (nt == 2)
+    SKXL(2, false);
+  SKXL(1, false);
+#undef SKXL
 }
 
 hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream) {

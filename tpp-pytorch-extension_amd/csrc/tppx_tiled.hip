@@ -391,14 +391,6 @@ template <int N>
 __device__ __forceinline__ void lds_wait_keep(i32x4& r) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(r) : "n"(N));
 }
-// compile-time loop: f(std::integral_constant<int, I>) for I in [B, E)
-template <int B, int E, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (B < E) {
-    f(std::integral_constant<int, B>{});
-    static_for<B + 1, E>(f);
-  }
-}
 
 // Several GEMMs over one activation (fused q/k/v) share a launch: the channel
 // blocks of all segments form one grid.

@@ -358,10 +358,48 @@ def fc_mul(input, weight, bias, mul_in):
     return linear(input, weight, bias, POST_MUL, mul_in)
 
 
-def qkv_gemm(input, weights, biases):
-    """fused_qkv_gemm (src/csrc/llm/fused_llm_infer.cpp:423-505): several GEMMs
-    over one activation in one launch; a 4th GEMM gets GELU (GPT-J fc_in)."""
+def rms_norm(t_in, t_wt, eps):
+    """llama_rms_norm (src/csrc/llm/fused_llm_infer.cpp:337-363): bf16 in/out, fp32 or bf16 weight."""
     L = _lib.lib()
+    if not t_in.is_cuda or t_in.dtype != torch.bfloat16:
+        raise TppxError(_lib.EINVAL, "llama_rms_norm: input must be a bfloat16 tensor on the GPU")
+    x = t_in.contiguous()
+    K = x.shape[-1]
+    if t_wt.dtype not in (torch.float32, torch.bfloat16) or t_wt.numel() != K or not t_wt.is_cuda:
+        raise TppxError(_lib.EINVAL, "llama_rms_norm: weight must be fp32 or bf16 [K] on the GPU")
+    y = torch.empty_like(x)
+    rows = x.numel() // K
+    if rows:
+        _lib.check(L.tppx_rms_norm(x.data_ptr(), t_wt.contiguous().data_ptr(), 0 if t_wt.dtype == torch.float32 else 1,
+                                   y.data_ptr(), rows, K, float(eps), _lib.stream_of(x)))
+    return y
+
+
+# RMSNorm inside the GEMM launch (tppx_norm_multi_linear_mxfp4 / tppx_norm_swiglu_mxfp4).  Off by default: on MI355X
+# the fused launch measured slower than the normalisation kernel followed by the plain launch (every workgroup
+# repeats the row reduction behind a barrier, and the extra registers spill); TPPX_FUSE_NORM=1 turns it on.
+FUSE_NORM = os.environ.get("TPPX_FUSE_NORM", "0") == "1"
+
+
+def _norm_fusable(norm, scheme, M, K):
+    """RMSNorm can ride inside the GEMM launch for MXFP4 decode steps (<= 16 rows, the LDS staging fits)."""
+    if norm is None or not FUSE_NORM:
+        return False
+    gamma, _ = norm
+    return (scheme == QSCHEME_MXFP and 0 < M <= 16 and K % 128 == 0 and (K == 4096 or K == 2048 or K <= 2048)
+            and gamma.dtype == torch.float32 and gamma.is_cuda and gamma.is_contiguous())
+
+
+def qkv_gemm(input, weights, biases, norm=None):
+    """fused_qkv_gemm (src/csrc/llm/fused_llm_infer.cpp:423-505): several GEMMs
+    over one activation in one launch; a 4th GEMM gets GELU (GPT-J fc_in).
+    norm = (gamma, eps): llama_rms_norm is applied to the input first (inside
+    the same launch for MXFP4 decode steps, as a separate launch otherwise)."""
+    L = _lib.lib()
+    if norm is not None:
+        xin, Min, _, Kin = _prep_input(input, list(weights)[0])
+        if not _norm_fusable(norm, list(weights)[0]._qscheme, Min, Kin):
+            input, norm = rms_norm(input, norm[0], norm[1]), None
     weights = list(weights)
     biases = list(biases) if biases is not None else []
     n = len(weights)
@@ -395,7 +433,9 @@ def qkv_gemm(input, weights, biases):
         return outs
     st = _lib.stream_of(x)
     ws = _lib.workspace(x)
-    if scheme == QSCHEME_MXFP:
+    if scheme == QSCHEME_MXFP and norm is not None:
+        _lib.check(L.tppx_norm_multi_linear_mxfp4(x.data_ptr(), norm[0].data_ptr(), float(norm[1]), segs, n, M, K, 0, st))
+    elif scheme == QSCHEME_MXFP:
         _lib.check(L.tppx_multi_linear_mxfp4(x.data_ptr(), segs, n, M, K, 0, ws.data_ptr(), ws.numel(), st))
     else:
         qbs = weights[0].block_size
@@ -405,10 +445,15 @@ def qkv_gemm(input, weights, biases):
     return outs
 
 
-def swiglu_gate_up(input, w_gate, w_up, b_gate=None, b_up=None):
+def swiglu_gate_up(input, w_gate, w_up, b_gate=None, b_up=None, norm=None):
     """silu(x Wg^T) * (x Wu^T) in one launch with the reference's bf16 rounding
-    points (fused_llm_infer.cpp:1271-1272)."""
+    points (fused_llm_infer.cpp:1271-1272).  norm = (gamma, eps): llama_rms_norm
+    on the input first (fused_llm_infer.cpp:1269), inside the launch when possible."""
     L = _lib.lib()
+    if norm is not None:
+        _, M0, _, K0 = _prep_input(input, w_gate)
+        if not _norm_fusable(norm, w_gate._qscheme, M0, K0):
+            input, norm = rms_norm(input, norm[0], norm[1]), None
     x, M, N, K = _prep_input(input, w_gate)
     x2, M2, N2, K2 = _prep_input(input, w_up)
     if N2 != N or w_gate._qscheme != w_up._qscheme:
@@ -423,6 +468,11 @@ def swiglu_gate_up(input, w_gate, w_up, b_gate=None, b_up=None):
     bu = _prep_bias(b_up, N, x.device)
     qg, sg = w_gate.native()
     qu, su = w_up.native()
+    if norm is not None:
+        _lib.check(L.tppx_norm_swiglu_mxfp4(x.data_ptr(), norm[0].data_ptr(), float(norm[1]), qg.data_ptr(), sg.data_ptr(),
+                                            _lib.ptr(bg), qu.data_ptr(), su.data_ptr(), _lib.ptr(bu), y.data_ptr(),
+                                            M, N, K, 0, _lib.stream_of(x)))
+        return y
     ws = _lib.workspace(x)
     _lib.check(L.tppx_swiglu_mxfp4(x.data_ptr(), qg.data_ptr(), sg.data_ptr(), _lib.ptr(bg), qu.data_ptr(),
                                    su.data_ptr(), _lib.ptr(bu), y.data_ptr(), M, N, K, 0, ws.data_ptr(),

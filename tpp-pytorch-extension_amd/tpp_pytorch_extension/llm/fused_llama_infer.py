@@ -27,19 +27,7 @@ def _bf16_cuda(t, name):
     return t.contiguous()
 
 
-def rms_norm(t_in, t_wt, eps):
-    """llama_rms_norm (fused_llm_infer.cpp:337-363): bf16 in/out, fp32 or bf16 weight."""
-    L = _lib.lib()
-    x = _bf16_cuda(t_in, "input")
-    K = x.shape[-1]
-    if t_wt.dtype not in (torch.float32, torch.bfloat16) or t_wt.numel() != K or not t_wt.is_cuda:
-        raise TppxError(_lib.EINVAL, "llama_rms_norm: weight must be fp32 or bf16 [K] on the GPU")
-    y = torch.empty_like(x)
-    rows = x.numel() // K
-    if rows:
-        _lib.check(L.tppx_rms_norm(x.data_ptr(), t_wt.contiguous().data_ptr(), 0 if t_wt.dtype == torch.float32 else 1,
-                                   y.data_ptr(), rows, K, float(eps), _lib.stream_of(x)))
-    return y
+rms_norm = _ops.rms_norm  # llama_rms_norm (fused_llm_infer.cpp:337-363)
 
 
 def apply_rotary_pos_emb_llama(t_in, t_emb_pos, t_pos, N, H):
@@ -144,8 +132,8 @@ class LlamaDecoderLayer:
         st = _lib.stream_of(t_HS)
         empty = torch.empty(0, dtype=torch.bfloat16, device=t_HS.device)
         t_res = t_HS
-        h = rms_norm(t_HS, self.t_Gi, self.eps)
-        q, k, v = _ops.qkv_gemm(h, [self.t_Wq, self.t_Wk, self.t_Wv], [empty] * 3)
+        # input RMSNorm + q/k/v GEMMs (one launch for MXFP4 decode steps)
+        q, k, v = _ops.qkv_gemm(t_HS, [self.t_Wq, self.t_Wk, self.t_Wv], [empty] * 3, norm=(self.t_Gi, self.eps))
         kc, vc = cache._ensure(self.layer_idx, B, self.Nkv, self.H, t_HS.device)
         # rotary on q and k + append of k, v at position seq_len (device counter), one launch
         _lib.check(L.tppx_rotary_kv_append_llama(
@@ -161,8 +149,8 @@ class LlamaDecoderLayer:
                                       cache.seq_len_dev.data_ptr(), 1, ctx.data_ptr(), B, self.Nq, self.Nkv, self.H,
                                       cache.capacity, ws.data_ptr(), ws.numel(), st))
         t_SO = _ops.fc_add(ctx, self.t_Wp, empty, t_res, 1.0)
-        h = rms_norm(t_SO, self.t_Gpa, self.eps)
-        t_I = _ops.swiglu_gate_up(h, self.t_Wg, self.t_Wu)
+        # post-attention RMSNorm + gate/up GEMMs + silu*mul
+        t_I = _ops.swiglu_gate_up(t_SO, self.t_Wg, self.t_Wu, norm=(self.t_Gpa, self.eps))
         t_Out = _ops.fc_add(t_I, self.t_Wd, empty, t_SO, 1.0)
         return [t_Out]
 
