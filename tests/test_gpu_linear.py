@@ -257,6 +257,13 @@ def test_cfg2_qint8_up_projection_full_size(M):
     assert_close_bf16(t2bits(y), ref, what=f"qint8 up-projection M={M}", pre_bits=pre)
 
 
+def test_qint8_fused_quant_shared_lds():
+    """16 rows x K=8192 with three channel tiles per workgroup: the quantised activations and the cross-wave
+    reduction do not fit the LDS side by side, so the reduction reuses the activations' region."""
+    y, ref, s, ctx = _run("qint8", 16, 8448, 8192, "add", True, 4242)
+    assert_close_bf16(t2bits(y), ref, what="qint8 M=16 K=8192 N=8448")
+
+
 @pytest.mark.parametrize("M", [3, 24, 64])
 def test_qint8_prequantized_and_reused_activations(M):
     """x == NULL takes row-major int8 activations + scales (the reference's

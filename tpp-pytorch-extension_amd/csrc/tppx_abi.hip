@@ -311,8 +311,7 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
     return check_hip(launch_decode_qint8(p, pl, stream), who);
   }
   p.S = 1;
-  SkinnyPlan sp = plan_skinny(1, M, p.total_tiles, p.units, false);
-  sp.fused_quant = sp.fused_quant && x != nullptr && qbs == 256;
+  SkinnyPlan sp = plan_skinny(1, M, p.total_tiles, p.units, false, x != nullptr && qbs == 256);
   if (x && !sp.fused_quant) {
     // quantise straight into MFMA operand order: the GEMM then reads one
     // contiguous 1 KiB per operand instead of 16 rows x 64 B

@@ -38,6 +38,7 @@ struct DecodeParams {
   int tpb;   // native tiles per unit (1 for MXFP4, qbs/64 for QINT8)
   int S;     // K splits across workgroups
   int cht;   // tiles of activations staged in LDS at a time
+  int lds_overlap; // fused-quantisation QINT8 kernel: the reduction region reuses the LDS of the activations
   float* part;   // [S][grid_y][total_tiles][acc][MG][64] x f32x4 partial tiles (S > 1)
   const float* norm_gamma; // f32 [K]: RMSNorm fused in front of the GEMM (LDS-staged MXFP4 kernel), or null
   float norm_eps;
@@ -52,7 +53,8 @@ struct DecodePlan {
 // in-workgroup K split ("skinny") launch shape
 struct SkinnyPlan {
   int mg, ntw, waves, max_units, grid_y;
-  bool fused_quant; // QINT8, M <= 4: activations quantised inside the GEMM kernel
+  bool fused_quant; // QINT8, M <= 16: activations quantised inside the GEMM kernel
+  bool lds_overlap; // ... and its reduction region reuses the LDS of the quantised activations
 };
 
 // one GEMM on the LDS-tiled (prefill) kernels
@@ -85,7 +87,8 @@ int env_int(const char* name, int dflt);
 hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs, void* xq, void* sa, int mt,
                                  hipStream_t stream);
 
-SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual);
+// can_fuse_quant: QINT8 with bf16 activations at hand and 256-wide blocks (the in-kernel quantisation's case)
+SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual, bool can_fuse_quant = false);
 hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream);
 hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream);
 size_t skinny_mxfp4_xl_lds(int units, int nt, bool dual);

@@ -289,9 +289,9 @@ skinny_qint8_kernel(const DecodeParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// QINT8 with the activation quantisation fused in, for M <= 4 (qbs == 256).
+// QINT8 with the activation quantisation fused in, for M <= 16 (qbs == 256).
 // Every wave quantises the rows of its own K range (one (row, block) item =
-// 64 lanes x 4 values, DPP max reduction) into a wave-private LDS region that
+// 16 lanes x 16 values, DPP max reduction) into a wave-private LDS region that
 // keeps only the M valid rows of each operand tile, then reads its MFMA
 // operand from there (lanes of the padded rows re-read row M-1), so the main
 // loop issues weight loads only and the whole ring is in flight from the
@@ -318,16 +318,31 @@ __device__ __forceinline__ int sk_int8_rne(float v, float inv) {
   return (int)fminf(fmaxf(r, -127.0f), 127.0f);
 }
 
-template <int NTW, int PF, int MAXW, int MINW>
+// Four values * inv, rounded to nearest even, as packed int8.  |v * inv| <= 127 up to rounding (inv = 1 / (amax / 127)
+// or 0), so no clamp is needed; adding 1.5 * 2^23 to the rounded product rounds it to an integer exactly as rintf does
+// and leaves its two's complement in the low mantissa byte.
+__device__ __forceinline__ uint32_t sk_int8x4_rne(float a, float b, float c, float d, float inv) {
+  const float magic = 12582912.0f;
+  // the products must be rounded to f32 before the add (a fused multiply-add rounds once and differs in rare
+  // cases); the empty asm makes each product opaque so that it cannot be contracted into the add
+  float pa = a * inv, pb = b * inv, pc = c * inv, pd = d * inv;
+  asm("" : "+v"(pa), "+v"(pb), "+v"(pc), "+v"(pd));
+  const uint32_t ua = __float_as_uint(pa + magic), ub = __float_as_uint(pb + magic);
+  const uint32_t uc = __float_as_uint(pc + magic), ud = __float_as_uint(pd + magic);
+  // v_perm_b32: selector bytes 0..3 pick from the second operand, 4..7 from the first, 0x0c gives zero
+  return __builtin_amdgcn_perm(ub, ua, 0x0c0c0400u) | __builtin_amdgcn_perm(ud, uc, 0x04000c0cu);
+}
+
+template <int NTW, int PF, int MAXW, int MINW, int XB>
 __global__ void __launch_bounds__(MAXW * 64)
 skinny_qint8_fq_kernel(const DecodeParams p) {
   extern __shared__ __align__(16) float sk_lds[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int W = blockDim.x >> 6;
   const int grp = blockIdx.x;
   const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
   const int ltile0 = (grp - sg.grp0) * NTW;
-  const int M = p.M; // <= 4, one block row
+  const int M = p.M; // <= 16, one block row
   const int NB = p.units, KT = NB * 4;
   const int u0 = (int)(((int64_t)wave * NB) / W), u1 = (int)(((int64_t)(wave + 1) * NB) / W);
   const int t0 = u0 * 4, t1 = u1 * 4;
@@ -344,19 +359,21 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
   // wave needs early (its activation rows, the post-op inputs) is requested
   // BEFORE the weight ring: waiting for it then does not wait for HBM.
   // One (row, block) item = 256 values = 16 lanes x 16 values, so a wave
-  // quantises four items per pass and the max reduction stays inside a DPP row.
-  constexpr int XP = 3; // passes: M <= 4 rows x <= 3 blocks per wave = 12 items
+  // quantises four items per pass and the max reduction stays inside a DPP
+  // row.  Items are numbered row-fastest; XB passes are in flight at a time.
   const uint16_t* xb = reinterpret_cast<const uint16_t*>(p.x);
   const int nitems = M * (u1 - u0);
-  uint4 raw[XP][2];
-#pragma unroll
-  for (int ps = 0; ps < XP; ps++) {
-    const int it = min(ps * 4 + (lane >> 4), max(nitems - 1, 0));
-    const int ul = it / M, mr = it - ul * M;
-    const uint4* src = reinterpret_cast<const uint4*>(xb + (int64_t)mr * p.K + (int64_t)(u0 + ul) * 256 + (lane & 15) * 16);
+  const uint32_t Mu = (uint32_t)M;
+  i32x4 raw[XB][2]; // first-class vectors: copies of the HIP struct type would keep the array in scratch
+  auto load_pass = [&](auto PS, int base) {
+    constexpr int ps = decltype(PS)::value;
+    const uint32_t it = (uint32_t)min((base + ps) * 4 + (lane >> 4), max(nitems - 1, 0));
+    const uint32_t ul = it / Mu, mr = it - ul * Mu;
+    const i32x4* src = reinterpret_cast<const i32x4*>(xb + (int64_t)mr * p.K + (int64_t)(u0 + (int)ul) * 256 + (lane & 15) * 16);
     raw[ps][0] = src[0];
     raw[ps][1] = src[1];
-  }
+  };
+  static_for<0, XB>([&](auto PS) { load_pass(PS, 0); });
   SkEpilogue<1, NTW, false, MINW> ep;
   ep.prefetch(p, sg, ltile0, 0);
 
@@ -377,25 +394,25 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
       load_stage(i, t0 + i);
   }
 
-  // wave-private LDS: xq [tile][g][M rows][16 B], then sa [unit][4]
+  // wave-private LDS: xq [tile][g][M rows][16 B], then sa [unit][16]; the region of the cross-wave reduction
+  // comes first unless both do not fit side by side (they overlap then, with a barrier in between)
   float* red = sk_lds;
-  uint8_t* mine = reinterpret_cast<uint8_t*>(sk_lds + (size_t)W * NTW * 256) + (size_t)wave * p.cht * (4 * 256 + 16);
+  uint8_t* mine = reinterpret_cast<uint8_t*>(sk_lds + (p.lds_overlap ? 0 : (size_t)W * NTW * 256)) + (size_t)wave * p.cht * (256 * M + 64);
   uint32_t* xq_s = reinterpret_cast<uint32_t*>(mine);
-  float* sa_s = reinterpret_cast<float*>(mine + (size_t)p.cht * 4 * 256);
-#pragma unroll
-  for (int ps = 0; ps < XP; ps++) {
-    if (ps * 4 < nitems) { // wave-uniform
-      const int it = ps * 4 + (lane >> 4);
-      const int itc = min(it, nitems - 1);
-      const int ul = itc / M, mr = itc - ul * M;
-      const uint32_t wd[8] = {raw[ps][0].x, raw[ps][0].y, raw[ps][0].z, raw[ps][0].w,
-                              raw[ps][1].x, raw[ps][1].y, raw[ps][1].z, raw[ps][1].w};
+  float* sa_s = reinterpret_cast<float*>(mine + (size_t)p.cht * 256 * M);
+  auto quant_pass = [&](auto PS, int base) {
+    constexpr int ps = decltype(PS)::value;
+    if ((base + ps) * 4 < nitems) { // wave-uniform
+      const int it = (base + ps) * 4 + (lane >> 4);
+      const uint32_t itc = (uint32_t)min(it, nitems - 1);
+      const uint32_t ul = itc / Mu, mr = itc - ul * Mu;
       float v[16];
       float amax = 0.0f;
 #pragma unroll
       for (int j = 0; j < 8; j++) {
-        v[2 * j] = bf16_bits_to_f32(wd[j] & 0xffffu);
-        v[2 * j + 1] = bf16_bits_to_f32(wd[j] >> 16);
+        const uint32_t wd = (uint32_t)raw[ps][j >> 2][j & 3];
+        v[2 * j] = bf16_bits_to_f32(wd & 0xffffu);
+        v[2 * j + 1] = bf16_bits_to_f32(wd >> 16);
         amax = fmaxf(amax, fmaxf(fabsf(v[2 * j]), fabsf(v[2 * j + 1])));
       }
       amax = sk_dpp_max<0xB1>(amax);  // quad_perm [1,0,3,2]
@@ -409,16 +426,20 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
       uint32_t pk[4];
 #pragma unroll
       for (int d = 0; d < 4; d++)
-        pk[d] = (uint32_t)(sk_int8_rne(v[4 * d], inv) & 0xff) | ((uint32_t)(sk_int8_rne(v[4 * d + 1], inv) & 0xff) << 8) |
-            ((uint32_t)(sk_int8_rne(v[4 * d + 2], inv) & 0xff) << 16) | ((uint32_t)(sk_int8_rne(v[4 * d + 3], inv) & 0xff) << 24);
+        pk[d] = sk_int8x4_rne(v[4 * d], v[4 * d + 1], v[4 * d + 2], v[4 * d + 3], inv);
       if (it < nitems) {
         // values k = (lane&15)*16.. of the block: tile (lane&15)/4, K group (lane&15)%4
-        const int tl = ul * 4 + ((lane & 15) >> 2), g = lane & 3;
-        reinterpret_cast<uint4*>(xq_s)[(tl * 4 + g) * M + mr] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        const int tl = (int)ul * 4 + ((lane & 15) >> 2), g = lane & 3;
+        reinterpret_cast<uint4*>(xq_s)[(tl * 4 + g) * M + (int)mr] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
         if ((lane & 15) == 0)
-          sa_s[ul * 4 + mr] = sc;
+          sa_s[ul * 16 + mr] = sc;
       }
     }
+  };
+  static_for<0, XB>([&](auto PS) { quant_pass(PS, 0); });
+  for (int base = XB; base * 4 < nitems; base += XB) { // more than 16 items per wave
+    static_for<0, XB>([&](auto PS) { load_pass(PS, base); });
+    static_for<0, XB>([&](auto PS) { quant_pass(PS, base); });
   }
   const int xoff = ((lane >> 4) * M + min(lane & 15, M - 1)) * 4; // dword offset inside a tile
 
@@ -438,8 +459,8 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
       iacc[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa, wreg[i][nt], iacc[nt], 0, 0, 0);
     }
     if (last) { // K block complete
-      // result rows (lane>>4)*4 + r: only the first lane group holds valid rows (M <= 4)
-      const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + ((tt >> 2) - u0) * 4);
+      // result rows (lane>>4)*4 + r; scales of rows >= M are whatever the LDS held: those rows are not stored
+      const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + ((tt >> 2) - u0) * 16 + (lane >> 4) * 4);
 #pragma unroll
       for (int nt = 0; nt < NTW; nt++)
 #pragma unroll
@@ -450,7 +471,7 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
     }
   };
   int t = t0;
-  for (; t + 2 * PF <= t1; t += PF) { // every reload of these groups is a real tile // branch-free full groups (PF is a multiple of 4)
+  for (; t + 2 * PF <= t1; t += PF) { // branch-free full groups (PF is a multiple of 4): every reload is a real tile
 #pragma unroll
     for (int i = 0; i < PF; i++) {
       consume(i, t + i, (i & 3) == 3);
@@ -469,6 +490,8 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
       }
     }
   }
+  if (p.lds_overlap)
+    __syncthreads(); // the reduction region overlaps the activations other waves may still be reading
   ep.finish(sg, facc, red);
 }
 
@@ -779,7 +802,7 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
 // ---------------------------------------------------------------------------
 // planning and launch
 // ---------------------------------------------------------------------------
-SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual) {
+SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual, bool can_fuse_quant) {
   SkinnyPlan pl;
   const int mrows = (int)(M < 64 ? M : 64);
   pl.mg = fmt == 0 ? 1 : (mrows <= 16 ? 1 : (mrows <= 32 ? 2 : 4));
@@ -817,8 +840,23 @@ SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual
   if (w < min_w)
     w = min_w;
   pl.waves = w;
-  pl.fused_quant = (fmt == 1 && M <= 4 && env_int("TPPX_SKINNY_FUSEDQ", 1) != 0);
   pl.max_units = (units + w - 1) / w;
+  pl.fused_quant = false;
+  pl.lds_overlap = false;
+  if (fmt == 1 && M <= 16 && can_fuse_quant && env_int("TPPX_SKINNY_FUSEDQ", 1) != 0) {
+    // quantisation inside the GEMM kernel: 16 waves, the fewest channel tiles per workgroup that keep the grid
+    // within one round of 256 workgroups, as long as the quantised rows of all waves fit the LDS
+    const int ntw = total_tiles <= 256 ? 1 : (total_tiles <= 512 ? 2 : 3);
+    const int cht = (units + 15) / 16;
+    const size_t xbytes = (size_t)16 * cht * (256 * (size_t)M + 64), rbytes = (size_t)16 * ntw * 1024;
+    if (xbytes <= 160 * 1024 && rbytes <= 160 * 1024) {
+      pl.fused_quant = true;
+      pl.lds_overlap = xbytes + rbytes > 160 * 1024;
+      pl.ntw = ntw;
+      pl.waves = 16;
+      pl.max_units = cht;
+    }
+  }
   return pl;
 }
 
@@ -840,10 +878,14 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
   p.cht = pl.max_units; // per-wave slots of activation scales in LDS
   dim3 grid(p.groups, pl.grid_y);
   if (pl.fused_quant) {
-    size_t lds = (size_t)pl.waves * pl.ntw * 256 * sizeof(float) + (size_t)pl.waves * pl.max_units * (4 * 256 + 16);
+    const size_t xbytes = (size_t)16 * pl.max_units * (256 * (size_t)p.M + 64), rbytes = (size_t)16 * pl.ntw * 1024;
+    const size_t lds = pl.lds_overlap ? (xbytes > rbytes ? xbytes : rbytes) : xbytes + rbytes;
+    p.lds_overlap = pl.lds_overlap ? 1 : 0;
+    if (pl.ntw == 3)
+      return sk_launch(skinny_qint8_fq_kernel<3, 4, 16, 16, 2>, p, grid, 16, lds, stream);
     if (pl.ntw == 2)
-      return sk_launch(skinny_qint8_fq_kernel<2, 4, 16, 4>, p, grid, pl.waves, lds, stream);
-    return sk_launch(skinny_qint8_fq_kernel<1, 12, 16, 4>, p, grid, pl.waves, lds, stream);
+      return sk_launch(skinny_qint8_fq_kernel<2, 4, 16, 16, 4>, p, grid, 16, lds, stream);
+    return sk_launch(skinny_qint8_fq_kernel<1, 8, 16, 16, 4>, p, grid, 16, lds, stream);
   }
   size_t lds = ((size_t)pl.waves * pl.ntw * pl.mg * 256 + (size_t)pl.waves * pl.max_units * pl.mg * 16) * sizeof(float);
 #define SKQ(MG, NTW, PF, MAXW, MINW)                                                                   \
