@@ -51,7 +51,7 @@ struct SkEpilogue {
   static constexpr int MAXE = (OUT + MINW * 64 - 1) / (MINW * 64);
   int64_t off[MAXE];
   uint32_t in1[MAXE], in2[MAXE];
-  float bias[MAXE], bias2[MAXE];
+  uint32_t bias[MAXE], bias2[MAXE]; // bf16 bits, converted at use: a conversion here would wait for the load at once
   bool ok[MAXE];
 
   __device__ __forceinline__ void prefetch(const DecodeParams& p, const DecodeSeg& sg, int ltile0, int m0) {
@@ -60,7 +60,7 @@ struct SkEpilogue {
       const int e = threadIdx.x + i * blockDim.x;
       ok[i] = false;
       in1[i] = in2[i] = 0;
-      bias[i] = bias2[i] = 0.f;
+      bias[i] = bias2[i] = 0;
       off[i] = 0;
       if (e < OUT) {
         const int l = e & 63, r = (e >> 6) & 3, mg = (e >> 8) % MG, a = (e >> 8) / MG;
@@ -70,9 +70,9 @@ struct SkEpilogue {
         if (ok[i]) {
           off[i] = (int64_t)m * sg.N + n;
           if (sg.bias)
-            bias[i] = bf16_bits_to_f32(sg.bias[n]);
+            bias[i] = sg.bias[n];
           if (DUAL && p.seg[1].bias)
-            bias2[i] = bf16_bits_to_f32(p.seg[1].bias[n]);
+            bias2[i] = p.seg[1].bias[n];
           if (sg.post_in)
             in1[i] = sg.post_in[off[i]];
           if (sg.post_in2)
@@ -108,10 +108,10 @@ struct SkEpilogue {
         if (ok[i]) {
           uint32_t out;
           if (DUAL) {
-            uint32_t gact = apply_post_bits(v + bias[i], TPPX_POST_SILU, 0, 0, 1.0f);
-            out = apply_post_bits(v2 + bias2[i], TPPX_POST_MUL, gact, 0, 1.0f);
+            uint32_t gact = apply_post_bits(v + bf16_bits_to_f32(bias[i]), TPPX_POST_SILU, 0, 0, 1.0f);
+            out = apply_post_bits(v2 + bf16_bits_to_f32(bias2[i]), TPPX_POST_MUL, gact, 0, 1.0f);
           } else {
-            out = apply_post_bits(v + bias[i], sg.post_op, in1[i], in2[i], sg.post_scale);
+            out = apply_post_bits(v + bf16_bits_to_f32(bias[i]), sg.post_op, in1[i], in2[i], sg.post_scale);
           }
           sg.y[off[i]] = (uint16_t)out;
         }
@@ -613,7 +613,7 @@ skinny_mxfp4_kernel(const DecodeParams p) {
 // per-(row, K tile) partial sums of squares through LDS and add them in a
 // fixed order.  The reduction scratch of the epilogue reuses the x regions.
 // ---------------------------------------------------------------------------
-template <int NT, int PF, bool DUAL, int XMODE>
+template <int NT, int PF, bool DUAL, int XMODE, int XNI>
 __global__ void __launch_bounds__(1024)
 skinny_mxfp4_xl_kernel(const DecodeParams p) {
   extern __shared__ __align__(16) float sk_lds[];
@@ -647,38 +647,35 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
     woff[nt] = (uint32_t)(min(ltile0 + nt, sg.tiles - 1) * KT * 64 + lane);
 
   // ---- activations of this wave's K slice -> LDS ----
-  // Loads return in issue order, so the (L2-resident) activation and gamma
-  // loads go out BEFORE the weight ring and are not held up by HBM latency.
-  constexpr int XNI = 8;                   // (row, chunk) items per lane: 16 rows x 32 chunks / 64 lanes
+  // Loads return in issue order, so the (L2-resident) activation and gamma loads go out BEFORE the weight ring and
+  // are not held up by HBM latency.  They are issued and waited for by hand ("at most the ring outstanding"): the
+  // compiler's own count is conservative across the branches around here and would wait for the ring as well, which
+  // would put everything up to the main loop behind the first HBM round trip instead of inside it.
   const int nch = (t1 - t0) * 16;          // 16-byte chunks per row in the slice
   const int items = p.M * nch;             // (row, chunk), chunk fastest: 16 consecutive lanes = one K tile of one row
   const int nsh = nch > 16 ? 5 : 4;        // the host admits slices of 0, 16 or 32 chunks only
   const int cmask = (1 << nsh) - 1;
   const char* xb = reinterpret_cast<const char*>(p.x);
   const uint32_t xk0 = (uint32_t)t0 * 256u; // byte offset of the slice inside a row
-  i32x4 raw[XNI]; // first-class vectors: copies of the HIP struct type are memcpys, which keep the array in scratch
-  // items past the end repeat the last one (and later store the same value to the same slot): nothing depends on
-  // the lane, so the loads stay batched in front of the weight ring.  Up to 4 rows need the first 2 items only.
-  const bool many = items > 2 * 64;
-  auto load_x = [&](auto IT) {
+  // XNI (row, chunk) items per lane: 2 cover 4 rows, 8 cover 16.  Items past the end repeat the last one (and later
+  // store the same value to the same slot).  First-class vectors: the HIP struct types would stay in scratch.
+  i32x4 raw[XNI];
+  static_for<0, XNI>([&](auto IT) {
     constexpr int it = decltype(IT)::value;
     const int i = min(it * 64 + lane, max(items - 1, 0));
     const int row = i >> nsh, ck = i & cmask;
-    raw[it] = *reinterpret_cast<const i32x4*>(xb + (size_t)((uint32_t)(row * p.K) * 2u + xk0 + (uint32_t)ck * 16u));
-  };
-  static_for<0, 2>(load_x);
-  if (many)
-    static_for<2, XNI>(load_x);
+    const char* src = xb + (size_t)((uint32_t)(row * p.K) * 2u + xk0 + (uint32_t)ck * 16u);
+    i32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(src) : "memory");
+    raw[it] = v;
+  });
   // the chunk of a lane is the same in every item when the slice is 16 or 32 chunks wide
-  float gm[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};
-  if (XMODE == 1 && nch) {
-    const float4* gp = reinterpret_cast<const float4*>(p.norm_gamma + (size_t)t0 * 128 + (size_t)(lane & cmask) * 8);
-    const float4 g0 = gp[0], g1 = gp[1];
-    gm[0] = g0.x; gm[1] = g0.y; gm[2] = g0.z; gm[3] = g0.w;
-    gm[4] = g1.x; gm[5] = g1.y; gm[6] = g1.z; gm[7] = g1.w;
+  f32x4 gm0 = f32x4{1.f, 1.f, 1.f, 1.f}, gm1 = gm0;
+  if (XMODE == 1) {
+    const float* gp = p.norm_gamma + (size_t)min(t0, KT - 1) * 128 + (size_t)(lane & cmask) * 8;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(gm0) : "v"(gp) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(gm1) : "v"(gp + 4) : "memory");
   }
-  SkEpilogue<1, NTW, DUAL, 16> ep;
-  ep.prefetch(p, sg, ltile0, 0);
 
   // weight ring: it has the HBM latency to cover
   i32x4 wreg[PF][NTW];
@@ -697,20 +694,42 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
     for (int i = 0; i < PF; i++)
       load_stage(i, t0 + i);
   }
+  // a full ring is PF stages of distinct tiles: 2 * NTW loads each.  Shorter slices (the stages would repeat a tile
+  // and the compiler may merge the repeats) simply wait for everything.
+  if (t1 - t0 >= PF)
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PF * NTW * 2) : "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+  // every use of the hand-loaded registers stays behind the wait
+  static_for<0, XNI>([&](auto IT) {
+    i32x4 v = raw[decltype(IT)::value];
+    asm volatile("" : "+v"(v));
+    raw[decltype(IT)::value] = v;
+  });
+  asm volatile("" : "+v"(gm0), "+v"(gm1));
 
+  // the slot arithmetic below starts from an opaque copy of the lane index, so that it is redone here instead of
+  // being carried in registers across the loads above (where registers are scarcest)
+  int lane2 = lane;
+  asm volatile("" : "+v"(lane2));
   float* srow = wss + W * 16 * cht + wave * 16; // this wave's copy of the 16 row scales
+  if (XMODE == 1) {
+    // slots of rows and tiles this wave does not have count as zero
+    if (lane < 16 * cht)
+      wss[wave * 16 * cht + lane] = 0.f;
+  }
   // raw activations go to their operand slots right away; the norm rescales them in place
-  auto stash_x = [&](auto IT) {
+  static_for<0, XNI>([&](auto IT) {
     constexpr int it = decltype(IT)::value;
-    const int i = it * 64 + lane;
+    const int i = it * 64 + lane2;
     const int ic = min(i, max(items - 1, 0));
     const int row = ic >> nsh, ck = ic & cmask;
     if (XMODE == 1) {
-      const uint32_t d[4] = {(uint32_t)raw[it][0], (uint32_t)raw[it][1], (uint32_t)raw[it][2], (uint32_t)raw[it][3]};
       float ssq = 0.f;
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        const float lo = bf16_bits_to_f32(d[e] & 0xffffu), hi = bf16_bits_to_f32(d[e] >> 16);
+        const uint32_t d = (uint32_t)raw[it][e];
+        const float lo = bf16_bits_to_f32(d & 0xffffu), hi = bf16_bits_to_f32(d >> 16);
         ssq = fmaf(lo, lo, ssq);
         ssq = fmaf(hi, hi, ssq);
       }
@@ -719,45 +738,48 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
       ssq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ssq), 0x4E, 0xf, 0xf, true));
       ssq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ssq), 0x141, 0xf, 0xf, true));
       ssq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ssq), 0x140, 0xf, 0xf, true));
-      if (i < items && (lane & 15) == 0)
+      if (i < items && (lane2 & 15) == 0)
         wss[(wave * 16 + row) * cht + (ck >> 4)] = ssq;
     }
     *reinterpret_cast<i32x4*>(&xs[ck * 16 + (row ^ (ck & 15))]) = raw[it];
-  };
-  static_for<0, 2>(stash_x);
-  if (many)
-    static_for<2, XNI>(stash_x);
+  });
   if (XMODE == 1) {
-    __syncthreads();
-    // mean of squares of whole rows: waves and tiles in a fixed order; lane r < 16 owns row r
-    if (lane < 16 && lane < p.M) {
-      float tot = 0.f;
-      for (int w2 = 0; w2 < W; w2++) {
-        const int nt2 = ((w2 + 1) * KT) / W - (w2 * KT) / W;
-        for (int tl = 0; tl < nt2; tl++)
-          tot += wss[(w2 * 16 + lane) * cht + tl];
-      }
+    // LDS only: a full __syncthreads would also wait for the weight ring
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
+    // mean of squares of whole rows in a fixed order: lane (q, r) adds waves 4q..4q+3 of row r, then the quarters
+    const int q = lane >> 4, r = lane & 15;
+    float tot = 0.f;
+#pragma unroll
+    for (int w2 = 0; w2 < 4; w2++)
+      for (int tl = 0; tl < cht; tl++)
+        tot += wss[((q * 4 + w2) * 16 + r) * cht + tl];
+    tot += __shfl_xor(tot, 16);
+    tot += __shfl_xor(tot, 32);
+    if (lane < 16)
       srow[lane] = 1.0f / sqrtf(tot * (1.0f / (float)p.K) + p.norm_eps);
-    }
     __builtin_amdgcn_wave_barrier(); // the scales are read by the other lanes of this wave
 #pragma unroll 1
     for (int i = lane; i < items; i += 64) {
       const int row = i >> nsh, ck = i & cmask;
-      uint4* slot = &xs[ck * 16 + (row ^ (ck & 15))];
-      const uint4 w = *slot;
+      i32x4* slot = reinterpret_cast<i32x4*>(&xs[ck * 16 + (row ^ (ck & 15))]);
+      const i32x4 w = *slot;
       const float sc = srow[row];
-      const uint32_t d[4] = {w.x, w.y, w.z, w.w};
-      uint32_t o[4];
+      i32x4 o;
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        const float lo = (bf16_bits_to_f32(d[e] & 0xffffu) * sc) * gm[2 * e];
-        const float hi = (bf16_bits_to_f32(d[e] >> 16) * sc) * gm[2 * e + 1];
-        o[e] = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+        const uint32_t d = (uint32_t)w[e];
+        const float lo = (bf16_bits_to_f32(d & 0xffffu) * sc) * (e < 2 ? gm0[2 * e] : gm1[2 * e - 4]);
+        const float hi = (bf16_bits_to_f32(d >> 16) * sc) * (e < 2 ? gm0[2 * e + 1] : gm1[2 * e - 3]);
+        o[e] = (int)(f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16));
       }
-      *slot = make_uint4(o[0], o[1], o[2], o[3]);
+      *slot = o;
     }
   }
   // the wave reads only what it wrote itself: program order is enough
+
+  // post-op inputs: requested here so that their registers are not live while the activations are in flight
+  SkEpilogue<1, NTW, DUAL, 16> ep;
+  ep.prefetch(p, sg, ltile0, 0);
 
   f32x4 acc[NTW][1];
 #pragma unroll
@@ -924,9 +946,12 @@ hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_
   const size_t lds = skinny_mxfp4_xl_lds(p.units, nt, dual);
   dim3 grid(p.groups, 1);
   const bool norm = p.norm_gamma != nullptr;
+  const bool few = p.M <= 4; // 4 rows x 32 chunks fit two items per lane
 #define SKXL(NT, DUAL)                                                                                       \
-  return norm ? sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 1>, p, grid, 16, lds, stream)                  \
-              : sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 0>, p, grid, 16, lds, stream)
+  return norm ? (few ? sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 1, 2>, p, grid, 16, lds, stream)        \
+                     : sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 1, 8>, p, grid, 16, lds, stream))       \
+              : (few ? sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 0, 2>, p, grid, 16, lds, stream)        \
+                     : sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 0, 8>, p, grid, 16, lds, stream))
   if (dual) {
     if (nt == 3)
       SKXL(3, true);
