@@ -220,6 +220,34 @@ def test_swiglu_full_size_gate_up_equals_composition(M):
     assert_close_bf16(t2bits(fused), ref, ulps=2, what=f"swiglu gate/up M={M}")
 
 
+@pytest.mark.parametrize("M", [17, 32, 40, 64])
+def test_mxfp4_row_group_kernel_full_size(M):
+    """17..64 rows at the Llama-7B up-projection shape (688 channel tiles: three per workgroup, ragged last group,
+    M = 40: a partly filled row group) with bias and the residual post-op."""
+    y, ref, s, ctx = _run("mxfp4", M, 11008, 1024, "add", True, 7100 + M)
+
+
+@pytest.mark.parametrize("M", [24, 64])
+def test_mxfp4_row_group_kernel_uneven_k_split_and_swiglu(M):
+    """K = 11008 (86 K tiles over 8 waves: 10 or 11 each); q/k/v segments in one launch; the gate/up pair as
+    silu(gate) then up * gate in place: all equal to the single-GEMM calls bit for bit, which match the oracle."""
+    ops = _ops()
+    y, ref, s, ctx = _run("mxfp4", M, 256, 11008, "none", False, 7200 + M)
+    K = 1024
+    ws = [_make("mxfp4", n, K, 7300 + i)[0] for i, n in enumerate((4096, 512, 512))]
+    x = randn_bf16((M, K), 1.0, 7310).cuda()
+    outs = torch.ops.tpp_llm.qkv_gemm(x, ws, [torch.Tensor()] * 3)
+    for w, o in zip(ws, outs):
+        assert torch.equal(o, ops.fc_plain(x, w, None))
+    wg, qg, sg_ = _make("mxfp4", 11008, K, 7320)
+    wu, qu, su = _make("mxfp4", 11008, K, 7321)
+    fused = ops.swiglu_gate_up(x, wg, wu)
+    assert torch.equal(fused, ops.fc_mul(x, wu, None, ops.fc_silu(x, wg, None)))
+    gate = O.linear_mxfp4(t2bits(x.cpu()), qg, sg_, None, O.POST_SILU)
+    ref2 = O.linear_mxfp4(t2bits(x.cpu()), qu, su, None, O.POST_MUL, gate)
+    assert_close_bf16(t2bits(fused), ref2, ulps=2, what=f"swiglu gate/up M={M}")
+
+
 def test_prefill_qkv_one_launch_equals_separate():
     """With enough rows the fused q/k/v GEMMs share one launch of the large-M
     kernel (one grid over the channel blocks of all three)."""

@@ -71,7 +71,7 @@ static int fill_seg(const char* who, const tppx_seg& s, DecodeSeg& d, int n_mult
   TPPX_REQUIRE(aligned16(s.qw) && aligned16(s.y), TPPX_EINVAL, "%s: weight/output pointer not 16-byte aligned", who);
   TPPX_REQUIRE(valid_post(s.post_op), TPPX_EINVAL, "%s: unknown post-op id %d", who, s.post_op);
   TPPX_REQUIRE(s.N > 0 && s.N % n_mult == 0, TPPX_ESHAPE, "%s: N=%ld must be a positive multiple of %d", who, (long)s.N, n_mult);
-  TPPX_REQUIRE(s.N < (1 << 30), TPPX_ESHAPE, "%s: N=%ld too large", who, (long)s.N);
+  TPPX_REQUIRE(s.N <= (1 << 25), TPPX_ESHAPE, "%s: N=%ld too large (at most 2^25 output channels)", who, (long)s.N);
   bool need1 = s.post_op == TPPX_POST_MUL || s.post_op == TPPX_POST_ADD_SCALE || s.post_op == TPPX_POST_ADD2_SCALE;
   bool need2 = s.post_op == TPPX_POST_ADD2_SCALE;
   TPPX_REQUIRE(!need1 || s.post_in, TPPX_EINVAL, "%s: post-op %d needs post_in", who, s.post_op);
@@ -250,6 +250,18 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     SkinnyPlan sp = plan_skinny(0, M, p.total_tiles, p.units, dual);
     set_groups(p, sp.ntw, dual);
     return check_hip(launch_skinny_mxfp4(p, sp, dual, stream), who);
+  }
+  if (env_int("TPPX_MXFP4_SPLITK", 0) == 0) {
+    // 17..64 rows: several MFMA row groups per workgroup, activations streamed through wave-private LDS
+    const int mg = M <= 32 ? 2 : 4;
+    int nt = 1;
+    for (; nt < 3; nt++) {
+      set_groups(p, nt, dual);
+      if (p.groups <= 256)
+        break;
+    }
+    set_groups(p, nt, dual);
+    return check_hip(launch_skinny_mxfp4_mg(p, mg, nt, dual, stream), who);
   }
   DecodePlan pl = plan_decode(0, M, p.groups, p.total_tiles, p.units, 1, dual, (size_t)ws_bytes);
   bind_workspace(p, pl, ws);

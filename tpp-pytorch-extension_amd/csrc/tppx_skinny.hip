@@ -49,26 +49,23 @@ struct SkEpilogue {
   static constexpr int OUT = DUAL ? ELEMS / 2 : ELEMS;
   // outputs per thread; the launcher never uses fewer than MINW waves
   static constexpr int MAXE = (OUT + MINW * 64 - 1) / (MINW * 64);
-  int64_t off[MAXE];
+  int off[MAXE]; // element offset of the output (the launcher checks M * N < 2^31), or -1: nothing to store
   uint32_t in1[MAXE], in2[MAXE];
   uint32_t bias[MAXE], bias2[MAXE]; // bf16 bits, converted at use: a conversion here would wait for the load at once
-  bool ok[MAXE];
 
   __device__ __forceinline__ void prefetch(const DecodeParams& p, const DecodeSeg& sg, int ltile0, int m0) {
 #pragma unroll
     for (int i = 0; i < MAXE; i++) {
       const int e = threadIdx.x + i * blockDim.x;
-      ok[i] = false;
       in1[i] = in2[i] = 0;
       bias[i] = bias2[i] = 0;
-      off[i] = 0;
+      off[i] = -1;
       if (e < OUT) {
         const int l = e & 63, r = (e >> 6) & 3, mg = (e >> 8) % MG, a = (e >> 8) / MG;
         const int m = m0 + mg * 16 + (l >> 4) * 4 + r;
         const int n = (ltile0 + a) * 16 + (l & 15);
-        ok[i] = m < p.M && (ltile0 + a) < sg.tiles;
-        if (ok[i]) {
-          off[i] = (int64_t)m * sg.N + n;
+        if (m < p.M && (ltile0 + a) < sg.tiles) {
+          off[i] = m * sg.N + n;
           if (sg.bias)
             bias[i] = sg.bias[n];
           if (DUAL && p.seg[1].bias)
@@ -80,6 +77,43 @@ struct SkEpilogue {
         }
       }
     }
+  }
+
+  // The same with half the scratch for the gate/up pair: the gate tiles are reduced first, then the up tiles
+  // (same sums in the same order as finish()).  stride >= ELEMS / 2.
+  __device__ __forceinline__ void finish_halves(const DecodeSeg& sg, f32x4 (&acc)[NACC][MG], float* red, int stride = ELEMS / 2) {
+    static_assert(DUAL, "two reduction rounds are for the gate/up pair");
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int W = blockDim.x >> 6;
+    float* mine = red + wave * stride;
+    float v[2][MAXE];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      if (h)
+        __syncthreads(); // everybody has read the gate sums
+#pragma unroll
+      for (int a = 0; a < NACC / 2; a++)
+#pragma unroll
+        for (int mg = 0; mg < MG; mg++)
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+            mine[(a * MG + mg) * 256 + r * 64 + lane] = acc[h * (NACC / 2) + a][mg][r];
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < MAXE; i++) {
+        const int e = threadIdx.x + i * blockDim.x;
+        v[h][i] = 0.f;
+        if (e < OUT)
+          for (int w = 0; w < W; w++)
+            v[h][i] += red[w * stride + e];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < MAXE; i++)
+      if (off[i] >= 0) {
+        const uint32_t gact = apply_post_bits(v[0][i] + bf16_bits_to_f32(bias[i]), TPPX_POST_SILU, 0, 0, 1.0f);
+        sg.y[off[i]] = (uint16_t)apply_post_bits(v[1][i] + bf16_bits_to_f32(bias2[i]), TPPX_POST_MUL, gact, 0, 1.0f);
+      }
   }
 
   // stride = floats between the regions of two waves (>= ELEMS)
@@ -105,7 +139,7 @@ struct SkEpilogue {
         if (DUAL)
           for (int w = 0; w < W; w++)
             v2 += red[w * stride + e + ELEMS / 2];
-        if (ok[i]) {
+        if (off[i] >= 0) {
           uint32_t out;
           if (DUAL) {
             uint32_t gact = apply_post_bits(v + bf16_bits_to_f32(bias[i]), TPPX_POST_SILU, 0, 0, 1.0f);
@@ -824,6 +858,172 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
 // ---------------------------------------------------------------------------
 // planning and launch
 // ---------------------------------------------------------------------------
+// ---------------------------------------------------------------------------
+// MXFP4 weight-only, 17..64 rows: MG row groups of 16 per workgroup.
+// Eight waves split K.  A wave walks its K tiles one at a time: the bf16
+// activations of the tile (MG*16 rows x 256 B, row-contiguous 16-byte loads,
+// requested a tile ahead into registers) are written to the wave's private
+// LDS region in MFMA operand order -- slot (chunk, row) = chunk*MPAD + (row ^
+// chunk), the same conflict-free image the 16-row kernel uses -- and read back
+// as A operands; every dequantised weight operand feeds MG MFMAs.  No barrier
+// before the final cross-wave reduction, no operand-shaped global loads, no
+// second kernel.  The epilogue's reduction scratch reuses the activation
+// regions.
+// ---------------------------------------------------------------------------
+template <int MG, int NT, bool DUAL, int PF>
+__global__ void __launch_bounds__(512)
+skinny_mxfp4_mg_kernel(const DecodeParams p) {
+  extern __shared__ __align__(16) float sk_lds[];
+  constexpr int W = 8, MPAD = MG * 16, XL = MG * 4;
+  constexpr int NTW = DUAL ? 2 * NT : NT; // DUAL: the gate AND the up tile of each channel tile (gate tiles first)
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int grp = blockIdx.x;
+  const int seg_id = DUAL ? 0 : sk_find_seg(p, grp);
+  const DecodeSeg& sg = p.seg[seg_id];
+  const int ltile0 = (grp - sg.grp0) * NT;
+  const int m0 = blockIdx.y * MPAD;
+  const int KT = p.units;
+  const int t0 = (wave * KT) / W, t1 = ((wave + 1) * KT) / W;
+  i32x4* xs = reinterpret_cast<i32x4*>(sk_lds) + (size_t)wave * (MPAD * 16); // [chunk 16][row MPAD] x 16 B
+
+  constexpr int NSEG = DUAL ? 2 : 1;
+  const char* qwb[NSEG];
+  const char* swb[NSEG];
+#pragma unroll
+  for (int sgi = 0; sgi < NSEG; sgi++) {
+    const DecodeSeg& ss = p.seg[DUAL ? sgi : seg_id];
+    qwb[sgi] = reinterpret_cast<const char*>(ss.qw);
+    swb[sgi] = reinterpret_cast<const char*>(ss.sw);
+  }
+  uint32_t woff[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; nt++)
+    woff[nt] = (uint32_t)(min(ltile0 + nt, sg.tiles - 1) * KT * 64 + lane);
+
+  // activation item `it` of this lane: row it*4 + lane/16 of the block row, chunk lane%16 of the tile's 256 bytes;
+  // rows past M re-read row M-1 (their results are not stored)
+  const char* xb = reinterpret_cast<const char*>(p.x);
+  const int r4 = lane >> 4, c16 = lane & 15;
+  // The per-item addresses are cheap to derive and expensive to keep (2 * XL registers): both helpers start from
+  // opaque copies of the lane coordinates so that the compiler rebuilds them at every call instead of hoisting them
+  // out of the K loop.
+  i32x4 xr[XL];
+  auto load_x = [&](int t) {
+    t = min(t, t1 - 1);
+    int r = r4, c = c16;
+    asm volatile("" : "+v"(r), "+v"(c));
+    const uint32_t base = (uint32_t)t * 256u + (uint32_t)c * 16u;
+#pragma unroll
+    for (int it = 0; it < XL; it++) {
+      const int row = min(m0 + it * 4 + r, p.M - 1);
+      xr[it] = *reinterpret_cast<const i32x4*>(xb + (size_t)((uint32_t)(row * p.K) * 2u + base));
+    }
+  };
+  auto store_x = [&]() {
+    int r = r4, c = c16;
+    asm volatile("" : "+v"(r), "+v"(c));
+#pragma unroll
+    for (int it = 0; it < XL; it++)
+      xs[c * MPAD + ((it * 4 + r) ^ c)] = xr[it];
+  };
+  // operand slot of this lane for step j: chunk g*4 + j, row m of row group mg (+ mg*16)
+  int rdo[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int cj = (lane >> 4) * 4 + j;
+    rdo[j] = cj * MPAD + ((lane & 15) ^ cj);
+  }
+
+  i32x4 wreg[PF][NTW];
+  uint32_t sreg[PF][NTW];
+  auto load_stage = [&](int st, int t) {
+    t = min(t, t1 - 1);
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++) {
+      const uint32_t slot = woff[nt % NT] + (uint32_t)t * 64u;
+      wreg[st][nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(qwb[nt / NT] + (size_t)(slot * 16u)));
+      sreg[st][nt] = *reinterpret_cast<const uint8_t*>(swb[nt / NT] + (size_t)slot);
+    }
+  };
+  if (t0 < t1) {
+    load_x(t0); // needed first, requested first
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+      load_stage(i, t0 + i);
+  }
+  // post-op inputs early, except where registers are scarcest (the gate/up pair has none but its biases)
+  constexpr bool LATE_EP = DUAL && MG == 4;
+  SkEpilogue<MG, NTW, DUAL, W> ep;
+  if (!LATE_EP)
+    ep.prefetch(p, sg, ltile0, m0);
+
+  f32x4 acc[NTW][MG];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++)
+#pragma unroll
+    for (int mg = 0; mg < MG; mg++)
+      acc[nt][mg] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // one K tile: activations of the tile into LDS, the next tile's requested, then 4 steps x MG x NT MFMAs
+  auto consume = [&](int i, int tnext) {
+    store_x();
+    load_x(tnext);
+    float sc[NTW];
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++)
+      sc[nt] = e8m0_to_f32(sreg[i][nt]);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      // NT dequantised operands at a time (DUAL: the gate tiles, then the up tiles; the activation operands are
+      // read again, which is cheaper than keeping either set in registers)
+#pragma unroll
+      for (int h = 0; h < NTW / NT; h++) {
+        bf16x8 b[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++)
+          b[nt] = sk_cvt_fp4x8((uint32_t)wreg[i][h * NT + nt][j], sc[h * NT + nt]);
+#pragma unroll
+        for (int mg = 0; mg < MG; mg++) {
+          const bf16x8 a = __builtin_bit_cast(bf16x8, xs[rdo[j] + mg * 16]);
+#pragma unroll
+          for (int nt = 0; nt < NT; nt++)
+            acc[h * NT + nt][mg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[nt], acc[h * NT + nt][mg], 0, 0, 0);
+        }
+        if (MG * NT >= 12)
+          __builtin_amdgcn_sched_barrier(0); // widest variants: keep the operands of one group live at a time
+      }
+    }
+  };
+  int t = t0;
+  for (; t + 2 * PF <= t1; t += PF) { // branch-free full groups: every reload is a real tile, wait counts stay exact
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      consume(i, t + i + 1);
+      load_stage(i, t + i + PF);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  for (; t < t1; t += PF) {
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      const int tt = t + i;
+      if (tt < t1) {
+        consume(i, tt + 1);
+        if (tt + PF < t1)
+          load_stage(i, tt + PF);
+      }
+    }
+  }
+  if (LATE_EP)
+    ep.prefetch(p, sg, ltile0, m0);
+  __syncthreads(); // every wave is done with its activation region before it becomes reduction scratch
+  if constexpr (DUAL)
+    ep.finish_halves(sg, acc, sk_lds);
+  else
+    ep.finish(sg, acc, sk_lds);
+}
+
 SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual, bool can_fuse_quant) {
   SkinnyPlan pl;
   const int mrows = (int)(M < 64 ? M : 64);
@@ -967,6 +1167,46 @@ hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_
     SKXL(2, false);
   SKXL(1, false);
 #undef SKXL
+}
+
+size_t skinny_mxfp4_mg_lds(int mg, int ntw) {
+  const size_t xbytes = (size_t)8 * mg * 16 * 256, rbytes = (size_t)8 * ntw * mg * 1024;
+  return xbytes > rbytes ? xbytes : rbytes;
+}
+
+// mg = 2 (up to 32 rows per block row) or 4; nt = channel tiles per workgroup (1..3; of each GEMM when dual);
+// groups counted by the caller
+hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hipStream_t stream) {
+  dim3 grid(p.groups, (p.M + mg * 16 - 1) / (mg * 16));
+  const size_t lds = skinny_mxfp4_mg_lds(mg, nt); // the gate/up pair is reduced one half at a time
+#define SKMG(MG, NT, DUAL, PF) return sk_launch(skinny_mxfp4_mg_kernel<MG, NT, DUAL, PF>, p, grid, 8, lds, stream)
+  if (dual) {
+    if (mg == 2) {
+      if (nt == 3)
+        SKMG(2, 3, true, 2);
+      if (nt == 2)
+        SKMG(2, 2, true, 2);
+      SKMG(2, 1, true, 2);
+    }
+    if (nt == 3)
+      SKMG(4, 3, true, 1); // 96 accumulators + 64 staging registers: one ring stage
+    if (nt == 2)
+      SKMG(4, 2, true, 2);
+    SKMG(4, 1, true, 2);
+  }
+  if (mg == 2) {
+    if (nt == 3)
+      SKMG(2, 3, false, 2);
+    if (nt == 2)
+      SKMG(2, 2, false, 2);
+    SKMG(2, 1, false, 2);
+  }
+  if (nt == 3)
+    SKMG(4, 3, false, 2);
+  if (nt == 2)
+    SKMG(4, 2, false, 2);
+  SKMG(4, 1, false, 2);
+#undef SKMG
 }
 
 hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream) {
