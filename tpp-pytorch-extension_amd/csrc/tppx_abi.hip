@@ -133,6 +133,22 @@ static bool plan_xl(DecodeParams& p, bool dual, int* nt_out) {
   return p.units <= 32 && (p.units % 16 == 0 || p.units <= 16) && skinny_mxfp4_xl_lds(p.units, nt, dual) <= 160 * 1024;
 }
 
+// K split of the single-kernel decode paths for more than 16 rows: the largest S in {4, 2} (at most max_s) such that
+// S channel tiles per workgroup still give at most 256 workgroups in all, every part keeps 2048 input channels, and
+// the partial tiles fit the workspace; 1 otherwise (also whenever there are enough channel tiles for three per
+// workgroup, where the activations are the smaller stream anyway).
+static int pick_split(const DecodeParams& p, int64_t M, int64_t K, int mg, int max_s, int64_t ws_bytes) {
+  if (env_int("TPPX_SKINNY_SPLITK", 1) == 0 || p.n_seg != 1 || M > 64)
+    return 1;
+  for (int s = max_s; s >= 2; s >>= 1) {
+    const int groups = (p.total_tiles + s - 1) / s;
+    const int64_t need = (int64_t)s * p.total_tiles * mg * 256 * (int64_t)sizeof(float);
+    if (p.total_tiles <= 256 && groups * s <= 256 && K / s >= 2048 && need <= ws_bytes)
+      return s;
+  }
+  return 1;
+}
+
 static int fill_all(const char* who, const tppx_seg* segs, int n_segs, int n_mult, bool dual,
                     DecodeParams& p) {
   int tiles = 0, groups = 0;
@@ -254,14 +270,27 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
   if (env_int("TPPX_MXFP4_SPLITK", 0) == 0) {
     // 17..64 rows: several MFMA row groups per workgroup, activations streamed through wave-private LDS
     const int mg = M <= 32 ? 2 : 4;
-    int nt = 1;
-    for (; nt < 3; nt++) {
-      set_groups(p, nt, dual);
-      if (p.groups <= 256)
-        break;
+    // Few channel tiles and a long K: every workgroup would pull all of the activations (M x K) through its CU.
+    // Split K across S workgroups that own S times the channel tiles each: the same number of workgroups, 1/S of
+    // the activations per CU, fp32 partial tiles through the workspace and a second small kernel.
+    // (measured: 26 -> 22 us for 64 rows at K = 11008 / N = 4096; no gain for 32 rows, and none for QINT8, whose
+    // int8 activations are half the bytes)
+    const int S = (dual || mg != 4) ? 1 : pick_split(p, M, K, mg, 4, ws_bytes);
+    int nt = S;
+    if (S == 1) {
+      for (; nt < 3; nt++) {
+        set_groups(p, nt, dual);
+        if (p.groups <= 256)
+          break;
+      }
     }
     set_groups(p, nt, dual);
-    return check_hip(launch_skinny_mxfp4_mg(p, mg, nt, dual, stream), who);
+    p.S = S;
+    p.part = (float*)ws;
+    rc = check_hip(launch_skinny_mxfp4_mg(p, mg, nt, dual, stream), who);
+    if (rc == TPPX_OK && S > 1)
+      rc = check_hip(launch_splitk_finish(p, mg, 1, stream), who);
+    return rc;
   }
   DecodePlan pl = plan_decode(0, M, p.groups, p.total_tiles, p.units, 1, dual, (size_t)ws_bytes);
   bind_workspace(p, pl, ws);

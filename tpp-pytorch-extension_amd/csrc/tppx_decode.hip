@@ -534,6 +534,17 @@ static hipError_t launch_finish(const DecodeParams& p, const DecodePlan& pl, hip
   return hipGetLastError();
 }
 
+// second pass for the single-kernel paths that split K across workgroups (same partial layout, one GEMM per tile)
+hipError_t launch_splitk_finish(const DecodeParams& p, int mg, int grid_y, hipStream_t stream) {
+  DecodePlan pl = DecodePlan();
+  pl.grid_y = grid_y;
+  switch (mg) {
+    case 1: return launch_finish<1, false>(p, pl, stream);
+    case 2: return launch_finish<2, false>(p, pl, stream);
+    default: return launch_finish<4, false>(p, pl, stream);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // planning and launch
 // ---------------------------------------------------------------------------

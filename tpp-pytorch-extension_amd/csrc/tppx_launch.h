@@ -99,5 +99,6 @@ DecodePlan plan_decode(int fmt, int64_t M, int groups, int total_tiles, int unit
                        size_t ws_bytes);
 hipError_t launch_decode_mxfp4(const DecodeParams& p, const DecodePlan& pl, bool dual, hipStream_t stream);
 hipError_t launch_decode_qint8(const DecodeParams& p, const DecodePlan& pl, hipStream_t stream);
+hipError_t launch_splitk_finish(const DecodeParams& p, int mg, int grid_y, hipStream_t stream);
 
 } // namespace tppx

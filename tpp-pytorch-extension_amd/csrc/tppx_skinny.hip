@@ -116,6 +116,38 @@ struct SkEpilogue {
       }
   }
 
+  // K split across workgroups (blockIdx.z = part): the workgroup's sums go to the workspace as accumulator
+  // fragments, [part][block row][tile][row group][lane] x f32x4, for the second-pass kernel that adds the parts in
+  // a fixed order and runs the epilogue.
+  __device__ __forceinline__ void finish_partial(const DecodeParams& p, const DecodeSeg& sg, f32x4 (&acc)[NACC][MG],
+                                                 float* red, int ltile0, int stride = ELEMS) {
+    static_assert(!DUAL, "the gate/up pair is not split");
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int W = blockDim.x >> 6;
+    float* mine = red + wave * stride;
+#pragma unroll
+    for (int a = 0; a < NACC; a++)
+#pragma unroll
+      for (int mg = 0; mg < MG; mg++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          mine[(a * MG + mg) * 256 + r * 64 + lane] = acc[a][mg][r];
+    __syncthreads();
+    float* part = p.part + ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * p.total_tiles * (MG * 256);
+#pragma unroll
+    for (int i = 0; i < MAXE; i++) {
+      const int e = threadIdx.x + i * blockDim.x;
+      if (e < OUT) {
+        float v = 0.f;
+        for (int w = 0; w < W; w++)
+          v += red[w * stride + e];
+        const int l = e & 63, r = (e >> 6) & 3, mg = (e >> 8) % MG, a = (e >> 8) / MG;
+        if (ltile0 + a < sg.tiles)
+          part[((size_t)(sg.tile0 + ltile0 + a) * MG + mg) * 256 + l * 4 + r] = v;
+      }
+    }
+  }
+
   // stride = floats between the regions of two waves (>= ELEMS)
   __device__ __forceinline__ void finish(const DecodeSeg& sg, f32x4 (&acc)[NACC][MG], float* red, int stride = ELEMS) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -171,7 +203,9 @@ skinny_qint8_kernel(const DecodeParams p) {
   const int NB = p.units, TPB = p.tpb, KT = NB * TPB;
   const bool TPB4 = TPB == 4; // 256-wide K blocks: the default
   constexpr int UN = (PF % 4 == 0) ? PF : (PF % 2 == 0 ? 2 * PF : 4 * PF); // lcm(PF, 4) tiles per unrolled trip
-  const int u0 = (int)(((int64_t)wave * NB) / W), u1 = (int)(((int64_t)(wave + 1) * NB) / W);
+  // K blocks of this workgroup (all of them unless K is split across workgroups), then of this wave
+  const int ub = (int)(((int64_t)blockIdx.z * NB) / p.S), ue = (int)(((int64_t)(blockIdx.z + 1) * NB) / p.S);
+  const int u0 = ub + (int)(((int64_t)wave * (ue - ub)) / W), u1 = ub + (int)(((int64_t)(wave + 1) * (ue - ub)) / W);
   const int t0 = u0 * TPB, t1 = u1 * TPB;
 
   const i32x4* wq[NTW];
@@ -319,7 +353,10 @@ skinny_qint8_kernel(const DecodeParams p) {
       }
     }
   }
-  ep.finish(sg, facc, red);
+  if (p.S > 1)
+    ep.finish_partial(p, sg, facc, red, ltile0);
+  else
+    ep.finish(sg, facc, red);
 }
 
 // ---------------------------------------------------------------------------
@@ -884,7 +921,9 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
   const int ltile0 = (grp - sg.grp0) * NT;
   const int m0 = blockIdx.y * MPAD;
   const int KT = p.units;
-  const int t0 = (wave * KT) / W, t1 = ((wave + 1) * KT) / W;
+  // K tiles of this workgroup (all of them unless K is split across workgroups), then of this wave
+  const int tb = (int)(((int64_t)blockIdx.z * KT) / p.S), te = (int)(((int64_t)(blockIdx.z + 1) * KT) / p.S);
+  const int t0 = tb + (wave * (te - tb)) / W, t1 = tb + ((wave + 1) * (te - tb)) / W;
   i32x4* xs = reinterpret_cast<i32x4*>(sk_lds) + (size_t)wave * (MPAD * 16); // [chunk 16][row MPAD] x 16 B
 
   constexpr int NSEG = DUAL ? 2 : 1;
@@ -1018,10 +1057,14 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
   if (LATE_EP)
     ep.prefetch(p, sg, ltile0, m0);
   __syncthreads(); // every wave is done with its activation region before it becomes reduction scratch
-  if constexpr (DUAL)
+  if constexpr (DUAL) {
     ep.finish_halves(sg, acc, sk_lds);
-  else
-    ep.finish(sg, acc, sk_lds);
+  } else {
+    if (p.S > 1)
+      ep.finish_partial(p, sg, acc, sk_lds, ltile0);
+    else
+      ep.finish(sg, acc, sk_lds);
+  }
 }
 
 SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual, bool can_fuse_quant) {
@@ -1098,7 +1141,7 @@ static hipError_t sk_launch(K kern, const DecodeParams& p, dim3 grid, int waves,
 // groups are counted per segment by the caller with the same ntw
 hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream) {
   p.cht = pl.max_units; // per-wave slots of activation scales in LDS
-  dim3 grid(p.groups, pl.grid_y);
+  dim3 grid(p.groups, pl.grid_y, pl.fused_quant ? 1 : p.S);
   if (pl.fused_quant) {
     const size_t xbytes = (size_t)16 * pl.max_units * (256 * (size_t)p.M + 64), rbytes = (size_t)16 * pl.ntw * 1024;
     const size_t lds = pl.lds_overlap ? (xbytes > rbytes ? xbytes : rbytes) : xbytes + rbytes;
@@ -1128,7 +1171,10 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
   switch (pl.mg) {
     case 1: SKQ(1, 1, 4, 16, 4);
     case 2: SKQ(2, 1, 4, 16, 4);
-    default: SKQ(4, 1, 8, 8, 8);
+    default:
+      if (p.mt > 0)
+        return sk_launch(skinny_qint8_kernel<4, 1, 8, 8, 8, true>, p, grid, pl.waves, lds, stream);
+      return sk_launch(skinny_qint8_kernel<4, 1, 4, 8, 8, false>, p, grid, pl.waves, lds, stream); // row-major rows: shorter ring, no spills
   }
 #undef SKQ
 }
@@ -1177,7 +1223,7 @@ size_t skinny_mxfp4_mg_lds(int mg, int ntw) {
 // mg = 2 (up to 32 rows per block row) or 4; nt = channel tiles per workgroup (1..3; of each GEMM when dual);
 // groups counted by the caller
 hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hipStream_t stream) {
-  dim3 grid(p.groups, (p.M + mg * 16 - 1) / (mg * 16));
+  dim3 grid(p.groups, (p.M + mg * 16 - 1) / (mg * 16), p.S);
   const size_t lds = skinny_mxfp4_mg_lds(mg, nt); // the gate/up pair is reduced one half at a time
 #define SKMG(MG, NT, DUAL, PF) return sk_launch(skinny_mxfp4_mg_kernel<MG, NT, DUAL, PF>, p, grid, 8, lds, stream)
   if (dual) {
@@ -1195,12 +1241,16 @@ hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hi
     SKMG(4, 1, true, 2);
   }
   if (mg == 2) {
+    if (nt == 4)
+      SKMG(2, 4, false, 2);
     if (nt == 3)
       SKMG(2, 3, false, 2);
     if (nt == 2)
       SKMG(2, 2, false, 2);
     SKMG(2, 1, false, 2);
   }
+  if (nt == 4)
+    SKMG(4, 4, false, 1);
   if (nt == 3)
     SKMG(4, 3, false, 2);
   if (nt == 2)
