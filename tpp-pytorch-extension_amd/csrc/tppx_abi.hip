@@ -261,6 +261,18 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
   int nt_xl = 1;
   if (M <= 16 && env_int("TPPX_MXFP4_XL", 1) == 1 && plan_xl(p, dual, &nt_xl))
     return check_hip(launch_skinny_mxfp4_xl(p, nt_xl, dual, stream), who);
+  if (M > 4 && M <= 16 && env_int("TPPX_MXFP4_MG1", 1) == 1) {
+    // K that the LDS-staged kernel above cannot hold: the tile-by-tile kernel with one row group (measured at
+    // K = 11008, N = 4096: 16 rows 14.7 -> 11.7 us; up to 4 rows the register-operand kernel below is faster)
+    int nt = 1;
+    for (; nt < 3; nt++) {
+      set_groups(p, nt, dual);
+      if (p.groups <= 256)
+        break;
+    }
+    set_groups(p, nt, dual);
+    return check_hip(launch_skinny_mxfp4_mg(p, 1, nt, dual, stream), who);
+  }
   if (M <= 16 && env_int("TPPX_MXFP4_SPLITK", 0) == 0) {
     // GEMV class: K reduction inside the workgroup
     SkinnyPlan sp = plan_skinny(0, M, p.total_tiles, p.units, dual);

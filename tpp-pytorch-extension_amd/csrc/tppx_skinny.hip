@@ -907,11 +907,11 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
 // second kernel.  The epilogue's reduction scratch reuses the activation
 // regions.
 // ---------------------------------------------------------------------------
-template <int MG, int NT, bool DUAL, int PF>
-__global__ void __launch_bounds__(512)
+template <int MG, int NT, bool DUAL, int PF, int W = 8>
+__global__ void __launch_bounds__(W * 64)
 skinny_mxfp4_mg_kernel(const DecodeParams p) {
   extern __shared__ __align__(16) float sk_lds[];
-  constexpr int W = 8, MPAD = MG * 16, XL = MG * 4;
+  constexpr int MPAD = MG * 16, XL = MG * 4;
   constexpr int NTW = DUAL ? 2 * NT : NT; // DUAL: the gate AND the up tile of each channel tile (gate tiles first)
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1215,16 +1215,33 @@ hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_
 #undef SKXL
 }
 
-size_t skinny_mxfp4_mg_lds(int mg, int ntw) {
-  const size_t xbytes = (size_t)8 * mg * 16 * 256, rbytes = (size_t)8 * ntw * mg * 1024;
+size_t skinny_mxfp4_mg_lds(int mg, int ntw, int waves) {
+  const size_t xbytes = (size_t)waves * mg * 16 * 256, rbytes = (size_t)waves * ntw * mg * 1024;
   return xbytes > rbytes ? xbytes : rbytes;
 }
 
-// mg = 2 (up to 32 rows per block row) or 4; nt = channel tiles per workgroup (1..3; of each GEMM when dual);
+// mg = 1, 2 or 4 row groups of 16 per block row; nt = channel tiles per workgroup (1..4; of each GEMM when dual);
 // groups counted by the caller
 hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hipStream_t stream) {
   dim3 grid(p.groups, (p.M + mg * 16 - 1) / (mg * 16), p.S);
-  const size_t lds = skinny_mxfp4_mg_lds(mg, nt); // the gate/up pair is reduced one half at a time
+  if (mg == 1) { // up to 16 rows: sixteen waves, deeper weight ring
+    const size_t lds1 = skinny_mxfp4_mg_lds(1, nt, 16);
+#define SKMG1(NT, DUAL, PF) return sk_launch(skinny_mxfp4_mg_kernel<1, NT, DUAL, PF, 16>, p, grid, 16, lds1, stream)
+    if (dual) {
+      if (nt == 3)
+        SKMG1(3, true, 1);
+      if (nt == 2)
+        SKMG1(2, true, 2);
+      SKMG1(1, true, 4);
+    }
+    if (nt == 3)
+      SKMG1(3, false, 4);
+    if (nt == 2)
+      SKMG1(2, false, 4);
+    SKMG1(1, false, 4);
+#undef SKMG1
+  }
+  const size_t lds = skinny_mxfp4_mg_lds(mg, nt, 8); // the gate/up pair is reduced one half at a time
 #define SKMG(MG, NT, DUAL, PF) return sk_launch(skinny_mxfp4_mg_kernel<MG, NT, DUAL, PF>, p, grid, 8, lds, stream)
   if (dual) {
     if (mg == 2) {
