@@ -159,25 +159,19 @@ static int fill_all(const char* who, const tppx_seg* segs, int n_segs, int n_mul
     p.seg[i].tile0 = tiles;
     p.seg[i].grp0 = groups;
     tiles += p.seg[i].tiles;
-    groups += (p.seg[i].tiles + 7) / 8;
+    groups += p.seg[i].tiles; // one tile per workgroup until set_groups() says otherwise
   }
   if (dual) {
     TPPX_REQUIRE(n_segs == 2 && segs[0].N == segs[1].N, TPPX_ESHAPE, "%s: gate and up projections must have equal N", who);
     p.seg[1].tile0 = 0;
     p.seg[1].grp0 = 0;
     tiles = p.seg[0].tiles;
-    groups = (tiles + 7) / 8;
+    groups = tiles;
   }
   p.n_seg = n_segs;
   p.total_tiles = tiles;
   p.groups = groups;
   return TPPX_OK;
-}
-
-static void bind_workspace(DecodeParams& p, const DecodePlan& pl, void* ws) {
-  p.S = pl.S;
-  p.cht = pl.cht;
-  p.part = (float*)ws;
 }
 
 static const int64_t TILED_MIN_M = 65; // more rows than the decode kernels cover in one block row
@@ -273,13 +267,13 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     set_groups(p, nt, dual);
     return check_hip(launch_skinny_mxfp4_mg(p, 1, nt, dual, stream), who);
   }
-  if (M <= 16 && env_int("TPPX_MXFP4_SPLITK", 0) == 0) {
-    // GEMV class: K reduction inside the workgroup
+  if (M <= 16) {
+    // GEMV class: K reduction inside the workgroup, operands straight from global memory
     SkinnyPlan sp = plan_skinny(0, M, p.total_tiles, p.units, dual);
     set_groups(p, sp.ntw, dual);
     return check_hip(launch_skinny_mxfp4(p, sp, dual, stream), who);
   }
-  if (env_int("TPPX_MXFP4_SPLITK", 0) == 0) {
+  {
     // 17..64 rows: several MFMA row groups per workgroup, activations streamed through wave-private LDS
     const int mg = M <= 32 ? 2 : 4;
     // Few channel tiles and a long K: every workgroup would pull all of the activations (M x K) through its CU.
@@ -304,9 +298,6 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
       rc = check_hip(launch_splitk_finish(p, mg, 1, stream), who);
     return rc;
   }
-  DecodePlan pl = plan_decode(0, M, p.groups, p.total_tiles, p.units, 1, dual, (size_t)ws_bytes);
-  bind_workspace(p, pl, ws);
-  return check_hip(launch_decode_mxfp4(p, pl, dual, stream), who);
 }
 
 static int run_qint8(const char* who, const void* x, void* xq, void* sa, const tppx_seg* segs,
@@ -349,19 +340,6 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
         return rc;
     }
     return TPPX_OK;
-  }
-  const int force = env_int("TPPX_QINT8_SPLITK", -1);
-  if (p.tpb == 4 && M > 4 && force == 1) {
-    // more than one MFMA row group: activations shared through LDS, K split
-    // across workgroups
-    DecodePlan pl = plan_decode(1, M, p.groups, p.total_tiles, p.units, p.tpb, false, (size_t)ws_bytes);
-    bind_workspace(p, pl, ws);
-    if (x && !pl.fused_quant && !reuse) {
-      rc = check_hip(launch_quant_act_int8(x, M, K, qbs, xq, sa, 0, stream), who);
-      if (rc)
-        return rc;
-    }
-    return check_hip(launch_decode_qint8(p, pl, stream), who);
   }
   p.S = 1;
   SkinnyPlan sp = plan_skinny(1, M, p.total_tiles, p.units, false, x != nullptr && qbs == 256);

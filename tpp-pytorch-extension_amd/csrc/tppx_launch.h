@@ -19,7 +19,7 @@ struct DecodeSeg {
   int N;
   int tiles;                // N / 16
   int tile0;                // first tile of this GEMM in the fused tile space
-  int grp0;                 // first workgroup group (8 tiles each) of this GEMM
+  int grp0;                 // first workgroup (group of channel tiles) of this GEMM in the launch
   int post_op;
   float post_scale;
 };
@@ -27,7 +27,7 @@ struct DecodeSeg {
 struct DecodeParams {
   DecodeSeg seg[TPPX_MAX_SEGS];
   int n_seg;
-  int groups;      // sum over segments of ceil(tiles / 8)
+  int groups;      // workgroups along x: sum over segments of ceil(tiles / tiles per workgroup)
   int total_tiles; // sum of tiles (one segment's tiles for the dual gate/up kernel)
   const void* x;   // bf16 [M][K]
   const void* xq;  // int8 [M][K], or MFMA operand order when mt > 0 (QINT8, unless quantised in-kernel)
@@ -36,18 +36,12 @@ struct DecodeParams {
   int mt;    // > 0: xq is [K/64][mt][4 g][16 m][16 B] (operand tiles of 16 rows x 64 K); 0: row-major
   int units; // K/128 (MXFP4 tiles) or K/qbs (QINT8 blocks)
   int tpb;   // native tiles per unit (1 for MXFP4, qbs/64 for QINT8)
-  int S;     // K splits across workgroups
+  int S;     // K parts across workgroups (grid z); > 1: partial sums go to `part`, a second kernel finishes
   int cht;   // tiles of activations staged in LDS at a time
   int lds_overlap; // fused-quantisation QINT8 kernel: the reduction region reuses the LDS of the activations
-  float* part;   // [S][grid_y][total_tiles][acc][MG][64] x f32x4 partial tiles (S > 1)
+  float* part;   // [S][block row][total_tiles][MG][64] x f32x4 partial tiles (S > 1)
   const float* norm_gamma; // f32 [K]: RMSNorm fused in front of the GEMM (LDS-staged MXFP4 kernel), or null
   float norm_eps;
-};
-
-struct DecodePlan {
-  int mg, S, cht, grid_x, grid_y;
-  bool fused_quant;
-  size_t lds_bytes, counter_bytes;
 };
 
 // in-workgroup K split ("skinny") launch shape
@@ -95,10 +89,6 @@ size_t skinny_mxfp4_xl_lds(int units, int nt, bool dual);
 hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hipStream_t stream);
 hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_t stream);
 
-DecodePlan plan_decode(int fmt, int64_t M, int groups, int total_tiles, int units, int tpb, bool dual,
-                       size_t ws_bytes);
-hipError_t launch_decode_mxfp4(const DecodeParams& p, const DecodePlan& pl, bool dual, hipStream_t stream);
-hipError_t launch_decode_qint8(const DecodeParams& p, const DecodePlan& pl, hipStream_t stream);
 hipError_t launch_splitk_finish(const DecodeParams& p, int mg, int grid_y, hipStream_t stream);
 
 } // namespace tppx
