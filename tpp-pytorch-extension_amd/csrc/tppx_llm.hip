@@ -7,6 +7,7 @@
 #include <string.h>
 
 #include "tppx_common.h"
+#include "tppx_launch.h"
 
 namespace tppx {
 
@@ -189,6 +190,10 @@ struct AttnParams {
   float scale;
 };
 
+__device__ __forceinline__ uint4 as_uint4(const i32x4& v) {
+  return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
+}
+
 __global__ void __launch_bounds__(256)
 attn_decode_kernel(const AttnParams p) {
   __shared__ float sm[16], sl[16];
@@ -215,21 +220,30 @@ attn_decode_kernel(const AttnParams p) {
 #pragma unroll
   for (int e = 0; e < 8; e++)
     acc[e] = 0.f;
-  for (int base = k0 + wave * 16; base < k1; base += 64) {
-    uint4 kw[4], vw[4];
-    int key[4];
+  constexpr int NU = 4; // keys per DPP row and trip (8 measured no better)
+  // 4 * NU keys per wave and trip (NU per DPP row); the next trip's K and V rows are requested before this trip's
+  // arithmetic so that a wave always has loads in flight (keys past the end re-read the last key, never used)
+  i32x4 kw[NU], vw[NU], kn[NU], vn[NU];
+  auto load_kv = [&](int base, i32x4 (&kd)[NU], i32x4 (&vd)[NU]) {
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
-      key[u] = base + u * 4 + g;
-      const int kk = min(key[u], L - 1);
-      kw[u] = kb[(int64_t)kk * 16];
-      vw[u] = vb[(int64_t)kk * 16];
+    for (int u = 0; u < NU; u++) {
+      const int kk = max(min(base + u * 4 + g, L - 1), 0);
+      kd[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(kb + (int64_t)kk * 16));
+      vd[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(vb + (int64_t)kk * 16));
     }
-    float sc[4];
+  };
+  load_kv(k0 + wave * (4 * NU), kw, vw);
+  for (int base = k0 + wave * (4 * NU); base < k1; base += 16 * NU) {
+    load_kv(base + 16 * NU, kn, vn);
+    int key[NU];
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
+    for (int u = 0; u < NU; u++)
+      key[u] = base + u * 4 + g;
+    float sc[NU];
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
       float kf[8];
-      unpack8(kw[u], kf);
+      unpack8(as_uint4(kw[u]), kf);
       float d = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; e++)
@@ -239,24 +253,32 @@ attn_decode_kernel(const AttnParams p) {
         d += bf16_bits_to_f32(mrow[key[u]]);
       sc[u] = key[u] < k1 ? d : -3.0e38f;
     }
-    const float mn = fmaxf(fmaxf(m, fmaxf(sc[0], sc[1])), fmaxf(sc[2], sc[3]));
+    float mn = m;
+#pragma unroll
+    for (int u = 0; u < NU; u++)
+      mn = fmaxf(mn, sc[u]);
     const float alpha = __expf(m - mn);
     l *= alpha;
 #pragma unroll
     for (int e = 0; e < 8; e++)
       acc[e] *= alpha;
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
+    for (int u = 0; u < NU; u++) {
       const float pr = key[u] < k1 ? __expf(sc[u] - mn) : 0.f;
       l += pr;
       const float pb = round_bf16(pr);
       float vf[8];
-      unpack8(vw[u], vf);
+      unpack8(as_uint4(vw[u]), vf);
 #pragma unroll
       for (int e = 0; e < 8; e++)
         acc[e] = fmaf(pb, vf[e], acc[e]);
     }
     m = mn;
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+      kw[u] = kn[u];
+      vw[u] = vn[u];
+    }
   }
   // merge the 16 (wave, row) states
   const int st = wave * 4 + g;
@@ -395,8 +417,9 @@ extern "C" int tppx_attn_decode(const void* q, const void* kcache, const void* v
   p.B = (int)B; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.Smax = (int)Smax; p.mask_ld = (int)mask_ld;
   p.scale = 1.0f / sqrtf((float)H);
   // enough workgroups to cover the chip about twice, at least 256 keys per split
-  int64_t splits = (512 + B * Nq - 1) / (B * Nq);
-  const int64_t max_by_len = (Smax + 255) / 256;
+  const int64_t target = env_int("TPPX_ATTN_TARGET_WGS", 512), min_keys = env_int("TPPX_ATTN_MIN_KEYS", 256);
+  int64_t splits = (target + B * Nq - 1) / (B * Nq);
+  const int64_t max_by_len = (Smax + min_keys - 1) / min_keys;
   if (splits > max_by_len)
     splits = max_by_len;
   if (splits > 32)
