@@ -1,15 +1,22 @@
-// Decode-shape kernels with the K reduction kept inside the workgroup.
+// Decode-shape kernels (up to 64 rows) with the K reduction kept inside the workgroup.
 //
-// One workgroup owns NTW consecutive 16-channel weight tiles and ALL of K; its
-// W (<= 16) waves split K into contiguous ranges.  A wave streams the native
-// 1 KiB tiles of its range for its NTW channel tiles straight from HBM into
-// registers (one 128-bit load per lane and tile, PF k-tiles in flight, the
-// first PF issued before anything else) together with the matching activation
-// operand (L2 resident), feeds the 16x16 MFMA, and at the end the W partial
-// tiles are summed through LDS in a fixed order (deterministic) and the fused
-// epilogue runs with post-op inputs that were fetched at kernel start.
-// No global atomics, no second pass: the tail after the last weight byte
-// arrives is one LDS round trip.
+// One workgroup owns a few consecutive 16-channel weight tiles and all of K
+// (or one of a few K parts, see finish_partial); its 8 or 16 waves split K
+// into contiguous ranges.  A wave streams the native 1 KiB tiles of its range
+// straight from HBM into registers (one 128-bit load per lane and tile, a ring
+// of PF k-tiles in flight, issued before anything that could wait), feeds the
+// 16x16 MFMA, and at the end the waves' partial tiles are summed through LDS
+// in a fixed order (deterministic) and the fused epilogue runs.  No global
+// atomics.  The kernels differ in how the activation operand gets there:
+//   skinny_qint8_kernel     int8 activations already in MFMA operand order in
+//                           global memory (written by the quantiser), 17..64 rows
+//   skinny_qint8_fq_kernel  bf16 activations quantised by the consuming wave into
+//                           wave-private LDS, up to 16 rows
+//   skinny_mxfp4_kernel     bf16 operands straight from global memory (few rows)
+//   skinny_mxfp4_xl_kernel  the wave's whole K slice staged once in LDS, up to
+//                           16 rows; optional RMSNorm in front
+//   skinny_mxfp4_mg_kernel  activations streamed through LDS one K tile at a
+//                           time, 1, 2 or 4 row groups of 16
 //
 // MFMA operand convention (A = activations, B = weights):
 //   lane l supplies row/col (l & 15) and K group (l >> 4);

@@ -315,14 +315,15 @@ tiled_qint8_kernel(const TiledParams p) {
 // grid (two per SIMD), each wave 128 x 64 = 8 x 4 MFMA tiles (128 accumulator
 // registers).  Every expanded weight operand feeds 8 MFMAs, every activation
 // operand read from LDS feeds 4 and is requested two MFMA groups ahead.
-//   A: rows are read from global memory row-contiguously (a wave instruction
-//      covers 4 rows x 256 B) and written into LDS in MFMA operand order; the
-//      16-byte slot of row m inside its 256-byte group is XOR-ed with the
-//      chunk index so that both the scattered writes and the operand reads
-//      are bank-conflict free.  Two LDS buffers of 64 KiB; the next tile is
-//      fetched a quarter at a time to keep the staging registers few.
+//   A: 4 rows x 256 B per wave instruction go from global memory straight
+//      into LDS (global_load_lds, no staging registers), a whole K step ahead,
+//      two buffers of 64 KiB.  The LDS image of such a load is lane-linear, so
+//      the bank swizzle is applied on the source side: the lane at position c
+//      of row m fetches chunk c ^ (m & 15), and the operand reads of a K group
+//      fall on 16 different bank groups.
 //   B: native tiles straight from global/L2, fetched half a K step ahead.
-// LDS slot of (row tile mt, step j, K group g, row m) = (mt*4 + j)*64 + g*16 + (m ^ (g*4 + j)).
+// LDS byte address of chunk ck of row m of row tile mt:
+//   mt*4096 + (m>>2)*1024 + (m&3)*256 + ((ck ^ m) & 15)*16.
 // ---------------------------------------------------------------------------
 // Epilogue of a 128 x 64 wave tile through a wave-private LDS region: the
 // fp32 sums of 64 rows at a time are written there (statically indexed, so the
