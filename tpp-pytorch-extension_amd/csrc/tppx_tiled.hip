@@ -330,7 +330,8 @@ tiled_qint8_kernel(const TiledParams p) {
 // accumulators stay in registers), then read back row-contiguously; every
 // lane finishes 8 adjacent channels and writes them with one 16-byte store.
 constexpr int EP_LD = 68; // floats per staged row: 64 + 4 keeps the 4-row lane groups on distinct banks
-__device__ __forceinline__ void big_epilogue(const TiledParams& p, f32x4 (&acc)[8][4], float* stage, int m_base,
+template <int MT>
+__device__ __forceinline__ void big_epilogue(const TiledParams& p, f32x4 (&acc)[MT][4], float* stage, int m_base,
                                              int tile_base) {
   const int lane = threadIdx.x & 63;
   const int cx = (lane & 7) * 8; // first of this lane's 8 channels inside the wave tile
@@ -342,7 +343,7 @@ __device__ __forceinline__ void big_epilogue(const TiledParams& p, f32x4 (&acc)[
   for (int e = 0; e < 8; e++)
     bias[e] = p.bias ? bf16_bits_to_f32(p.bias[n + e]) : 0.0f;
 #pragma unroll
-  for (int h = 0; h < 2; h++) {
+  for (int h = 0; h < MT / 4; h++) {
 #pragma unroll
     for (int mt = 0; mt < 4; mt++)
 #pragma unroll
@@ -401,13 +402,18 @@ struct BigParams {
   int n_seg;
 };
 
+// MT = 16-row tiles per wave along M: 8 (workgroup tile 256 x 256) or 4 (128 x 256, for shapes whose 256-row tiles
+// would leave most of the last round of workgroups empty).
+template <int MT>
 __global__ void __launch_bounds__(512)
 big_mxfp4_kernel(const BigParams P) {
+  constexpr int WGM = MT * 32;     // rows per workgroup
+  constexpr int ABUF = WGM * 256;  // bytes of one A buffer (rows x 128 K bf16)
   extern __shared__ __align__(16) uint8_t tl_lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform: keeps LDS bases and block indices scalar
   const int wm = wave & 1, wn = wave >> 1;
-  const int MB = (P.seg[0].M + 255) >> 8;
+  const int MB = (P.seg[0].M + WGM - 1) / WGM;
   int bm, bn;
   tile_of_block(MB, P.nb0[P.n_seg], bm, bn);
   // pick this block's GEMM with uniform selects (everything stays in scalar registers)
@@ -421,7 +427,7 @@ big_mxfp4_kernel(const BigParams P) {
     }
   bn -= nb_first;
   const int KT = p.K >> 7;
-  const int m_wg = bm * 256;
+  const int m_wg = bm * WGM;
   const int tile_base = bn * 16 + wn * 4;
 
   // Every global address below is a uniform base pointer plus a 32-bit byte
@@ -457,22 +463,22 @@ big_mxfp4_kernel(const BigParams P) {
   // source byte offset of block i at K step ks:
   //   row(i) * K * 2 + ((ch ^ m16(i)) & 15) * 16 + ks * 256, row(i) = m_wg + (wave*8 + i)*4 + rin,
   //   m16(i) = (i & 3)*4 + rin (wave*8 is a multiple of 4)
-  const bool full = m_wg + 256 <= p.M; // uniform
-  const uint32_t xrow0 = (uint32_t)((m_wg + wave * 32 + rin) * p.K) * 2u;
+  const bool full = m_wg + WGM <= p.M; // uniform
+  const uint32_t xrow0 = (uint32_t)((m_wg + wave * (MT * 4) + rin) * p.K) * 2u;
   const uint32_t blk_stride = (uint32_t)(4 * p.K) * 2u; // uniform
   auto load_a = [&](int ks, int buf) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int i = 0; i < MT; i++) {
       const uint32_t sw = (uint32_t)((ch ^ ((i & 3) * 4 + rin)) & 15) * 16u;
       uint32_t off;
       if (full) {
         off = xrow0 + (uint32_t)i * blk_stride + sw + (uint32_t)ks * 256u;
       } else { // past the end: re-read the last row (never stored)
-        const int row = min(m_wg + (wave * 8 + i) * 4 + rin, p.M - 1);
+        const int row = min(m_wg + (wave * MT + i) * 4 + rin, p.M - 1);
         off = (uint32_t)(row * p.K) * 2u + sw + (uint32_t)ks * 256u;
       }
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xbase + (size_t)off),
-                                       (__attribute__((address_space(3))) void*)(tl_lds + buf * 65536 + (wave * 8 + i) * 1024),
+                                       (__attribute__((address_space(3))) void*)(tl_lds + buf * ABUF + (wave * MT + i) * 1024),
                                        16, 0, 0);
     }
   };
@@ -499,9 +505,9 @@ big_mxfp4_kernel(const BigParams P) {
     }
   };
 
-  f32x4 acc[8][4];
+  f32x4 acc[MT][4];
 #pragma unroll
-  for (int mt = 0; mt < 8; mt++)
+  for (int mt = 0; mt < MT; mt++)
 #pragma unroll
     for (int nt = 0; nt < 4; nt++)
       acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -515,35 +521,36 @@ big_mxfp4_kernel(const BigParams P) {
     take_b();
     if (more)
       load_a(ks + 1, buf ^ 1); // lands in the other buffer during this step's MFMAs
-    // 32 operand reads per K step (q = j*8 + mt), kept RD ahead of the MFMAs
+    // 4*MT operand reads per K step (q = j*MT + mt), kept RD ahead of the MFMAs
     // that consume them so the LDS latency is covered by 4*RD MFMAs
-    const uint32_t abase = lds0 + (uint32_t)(buf * 65536 + wm * 8 * 4096);
+    const uint32_t abase = lds0 + (uint32_t)(buf * ABUF + wm * MT * 4096);
     constexpr int RD = 3; // operand reads in flight ahead of the MFMAs
+    constexpr int NQ = 4 * MT;
     i32x4 ar[RD + 1];
     bf16x8 b[4];
     static_for<0, RD>([&](auto I) {
       constexpr int i = decltype(I)::value;
-      lds_read_b128_async<(i & 7) * 4096>(ar[i], abase + rdb[i >> 3]);
+      lds_read_b128_async<(i % MT) * 4096>(ar[i], abase + rdb[i / MT]);
     });
-    static_for<0, 32>([&](auto Q) {
+    static_for<0, NQ>([&](auto Q) {
       constexpr int q = decltype(Q)::value;
-      constexpr int j = q >> 3, mt = q & 7;
+      constexpr int j = q / MT, mt = q % MT;
       if constexpr (mt == 0) {
 #pragma unroll
         for (int nt = 0; nt < 4; nt++)
           b[nt] = tl_cvt_fp4x8(bc[nt][j], sc[nt]);
       }
-      if constexpr (q + RD < 32) {
-        lds_read_b128_async<((q + RD) & 7) * 4096>(ar[(q + RD) % (RD + 1)], abase + rdb[(q + RD) >> 3]);
+      if constexpr (q + RD < NQ) {
+        lds_read_b128_async<((q + RD) % MT) * 4096>(ar[(q + RD) % (RD + 1)], abase + rdb[(q + RD) / MT]);
         lds_wait_keep<RD>(ar[q % (RD + 1)]);
       } else {
-        lds_wait_keep<31 - q>(ar[q % (RD + 1)]);
+        lds_wait_keep<NQ - 1 - q>(ar[q % (RD + 1)]);
       }
       const bf16x8 a = __builtin_bit_cast(bf16x8, ar[q % (RD + 1)]);
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
         acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[nt], acc[mt][nt], 0, 0, 0);
-      if constexpr (q == 15) {
+      if constexpr (q == NQ / 2 - 1) {
         if (more)
           load_b(ks + 1); // dwords of steps 0 and 1 of the current B are dead by now
       }
@@ -551,7 +558,7 @@ big_mxfp4_kernel(const BigParams P) {
     __syncthreads(); // waits for this wave's direct-to-LDS loads, then for everybody's
   }
   // every wave has left the main loop (barrier above): LDS is free for the epilogue staging
-  big_epilogue(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * 128, tile_base);
+  big_epilogue<MT>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
 }
 
 // the large-M kernel addresses its operands with 32-bit byte offsets
@@ -575,18 +582,35 @@ hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t str
   for (int i = n; i <= TPPX_MAX_SEGS; i++)
     P.nb0[i] = nb;
   P.n_seg = n;
-  const int MB = (t[0].M + 255) / 256;
-  const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the two 64 KiB A buffers
-  TPPX_PLAN_ONLY(big_mxfp4_kernel, dim3(MB * nb), dim3(512), lds);
+  const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the two A buffers
+  // 256-row tiles unless their last round of workgroups (256 CUs, one workgroup each) would be less than half
+  // full while 128-row tiles fill it better: then every workgroup takes half the rows
+  const int MB8 = (t[0].M + 255) / 256, MB4 = (t[0].M + 127) / 128;
+  auto rounds = [](int wgs) { return (wgs + 255) / 256; };
+  // (measured: a 128-row workgroup needs about 0.57 of the time of a 256-row one)
+  const double cost8 = rounds(MB8 * nb), cost4 = 0.5 * 1.15 * rounds(MB4 * nb);
+  int mt = cost4 < cost8 ? 4 : 8;
+  const int env_mt = env_int("TPPX_TILED_BIG_MT", 0);
+  if (env_mt == 4 || env_mt == 8)
+    mt = env_mt;
   static bool big_attr_done = false;
   if (!big_attr_done) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_mxfp4_kernel),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_mxfp4_kernel<8>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_mxfp4_kernel<4>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess)
       return e;
     big_attr_done = true;
   }
-  big_mxfp4_kernel<<<dim3(MB * nb), dim3(512), lds, stream>>>(P);
+  if (mt == 4) {
+    TPPX_PLAN_ONLY(big_mxfp4_kernel<4>, dim3(MB4 * nb), dim3(512), lds);
+    big_mxfp4_kernel<4><<<dim3(MB4 * nb), dim3(512), lds, stream>>>(P);
+  } else {
+    TPPX_PLAN_ONLY(big_mxfp4_kernel<8>, dim3(MB8 * nb), dim3(512), lds);
+    big_mxfp4_kernel<8><<<dim3(MB8 * nb), dim3(512), lds, stream>>>(P);
+  }
   return hipGetLastError();
 }
 
