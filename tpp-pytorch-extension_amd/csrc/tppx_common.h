@@ -71,7 +71,9 @@ __device__ __forceinline__ uint32_t apply_post_bits(float v, int post,
   float y = bf16_bits_to_f32(yb);
   switch (post) {
     case TPPX_POST_SILU: {
-      float s = round_bf16(1.0f / (1.0f + expf(-y)));
+      // hardware exp2 / reciprocal: their error (about 1e-7 relative) is far below the bf16 rounding that follows,
+      // and the full-precision expf + divide cost as much as 30 MFMA issue slots per output in the prefill epilogue
+      float s = round_bf16(__frcp_rn(1.0f + __expf(-y)));
       return f32_to_bf16_bits(y * s);
     }
     case TPPX_POST_MUL:
