@@ -332,6 +332,40 @@ def test_qint8_prequantized_and_reused_activations(M):
     assert torch.equal(y2_reuse, y2_plain), "reused activation quantization gives different bits"
 
 
+def _shape_sweep():
+    """48 seeded (format, M, N, K, post-op, bias) cases across the kernel selection boundaries: 1..64 rows, channel
+    counts that leave ragged workgroups, K from one native tile to the Llama intermediate size."""
+    import random
+    rnd = random.Random(20240)
+    cases = []
+    for i in range(48):
+        fmt = rnd.choice(["mxfp4", "qint8"])
+        M = rnd.choice([1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 20, 31, 32, 33, 47, 48, 63, 64])
+        N = rnd.choice([32, 64, 96, 160, 512, 1056, 4128, 8224])
+        K = rnd.choice([128, 256, 384, 512, 1024, 2048, 2304, 4096, 5120, 8192, 11008])
+        if fmt == "qint8" and K % 256:
+            K = (K // 256 + 1) * 256
+        cases.append((fmt, M, N, K, rnd.choice(["none", "silu", "mul", "add", "add2", "gelu", "relu"]), rnd.random() < 0.5, 9100 + i))
+    return cases
+
+
+@pytest.mark.parametrize("fmt,M,N,K,post,bias,seed", _shape_sweep())
+def test_shape_sweep(fmt, M, N, K, post, bias, seed):
+    ops = _ops()
+    qw, q_or, s_or = _make(fmt, N, K, seed)
+    x = randn_bf16((M, K), 1.0, seed + 1)
+    b = randn_bf16((N,), 0.01, seed + 2) if bias else None
+    in1, in2 = randn_bf16((M, N), 1.0, seed + 3), randn_bf16((M, N), 1.0, seed + 4)
+    scale = 0.5 if post in ("add", "add2") else 1.0
+    y = ops.linear(x.cuda(), qw, None if b is None else b.cuda(), POSTS[post], in1.cuda(), in2.cuda(), scale)
+    lin = O.linear_mxfp4 if fmt == "mxfp4" else O.linear_qint8
+    bb = None if b is None else t2bits(b)
+    ref = lin(t2bits(x), q_or, s_or, bb, POSTS[post], t2bits(in1), t2bits(in2), scale, O.MODE_IDEAL)
+    pre = lin(t2bits(x), q_or, s_or, bb) if post in ("add", "add2") else None  # the tile a residual can cancel
+    assert_close_bf16(t2bits(y), ref, ulps=2 if post in ("silu", "gelu") else 1,
+                      what=f"{fmt} M={M} N={N} K={K} post={post}", pre_bits=pre)
+
+
 def test_launch_plan_names_the_kernels():
     import ctypes
     from tpp_pytorch_extension import _lib
