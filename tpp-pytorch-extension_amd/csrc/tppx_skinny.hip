@@ -21,6 +21,9 @@
 // MFMA operand convention (A = activations, B = weights):
 //   lane l supplies row/col (l & 15) and K group (l >> 4);
 //   result register r of lane l is D[m = (l >> 4) * 4 + r][n = l & 15].
+#include <mutex>
+#include <unordered_map>
+
 #include "tppx_common.h"
 #include "tppx_launch.h"
 
@@ -1135,11 +1138,20 @@ SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual
 template <typename K>
 static hipError_t sk_launch(K kern, const DecodeParams& p, dim3 grid, int waves, size_t lds, hipStream_t stream) {
   TPPX_PLAN_ONLY(kern, grid, dim3(64 * waves), lds);
+  // raise the dynamic-LDS limit of a kernel once per size instead of on every launch (all kernels here share one
+  // function type, so the record is keyed by the kernel's address)
   if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess)
-      return e;
+    static std::mutex mu;
+    static std::unordered_map<const void*, size_t> allowed;
+    std::lock_guard<std::mutex> lock(mu);
+    size_t& have = allowed[reinterpret_cast<const void*>(kern)];
+    if (lds > have) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess)
+        return e;
+      have = lds;
+    }
   }
   kern<<<grid, dim3(64 * waves), lds, stream>>>(p);
   return hipGetLastError();
