@@ -240,8 +240,9 @@ def run_tokens(torch, args):
 
 def run_prefill(torch, _ops, args):
     """BASELINE config 4: M = 2048 tokens through the MXFP4 linears of one decoder layer with hidden 8192
-    (fused qkv 8192 -> 8192+1024+1024, o 8192 -> 8192 + residual, gate/up 8192 -> 28672 as silu then mul,
-    down 28672 -> 8192 + residual).  One step = those five op calls (seven GEMMs)."""
+    (fused qkv 8192 -> 8192+1024+1024, o 8192 -> 8192 + residual, then the MLP block gate/up 8192 -> 28672 with
+    silu * mul and down 28672 -> 8192 + residual through the package's swiglu_mlp op, whose result is bit-identical
+    to fc_silu, fc_mul, fc_add in sequence).  One step = those three op calls (seven GEMMs)."""
     from tpp_pytorch_extension import _lib
     dev = torch.device("cuda:0")
     M, H, I = 2048, 8192, 28672
@@ -262,9 +263,7 @@ def run_prefill(torch, _ops, args):
     def step():
         q, k, v = torch.ops.tpp_llm.qkv_gemm(x, [wq, wk, wv], [empty] * 3)
         h = torch.ops.tpp_llm.fc_add(q, wo, empty, res, 1.0)
-        gate = torch.ops.tpp_llm.fc_silu(h, wg, empty)
-        inter = torch.ops.tpp_llm.fc_mul(h, wu, empty, gate)
-        return torch.ops.tpp_llm.fc_add(inter, wd, empty, h, 1.0), k, v
+        return torch.ops.tpp_llm.swiglu_mlp(h, wg, wu, wd, h, 1.0), k, v
 
     gemms = [("qkv", 10240, H), ("o", H, H), ("gate", I, H), ("up", I, H), ("down", H, I)]
     flops = sum(2.0 * M * N * K for _, N, K in gemms)
@@ -305,7 +304,7 @@ def run_prefill(torch, _ops, args):
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "cfg4: MXFP4 linears of one decoder layer (hidden 8192, intermediate 28672, kv 1024) at "
-                               "M = 2048: qkv_gemm, fc_add(o), fc_silu(gate), fc_mul(up), fc_add(down)",
+                               "M = 2048: qkv_gemm, fc_add(o), swiglu_mlp(gate, up, down)",
                    "launch": "eager op calls", "flops_per_step": flops},
         "roofline": roof, "cpu_baseline": cpu}))
 

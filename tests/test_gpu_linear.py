@@ -204,6 +204,24 @@ def test_prefill_qkv_and_swiglu_equal_composition():
     assert torch.equal(fused, ops.fc_mul(x, wu, None, ops.fc_silu(x, wg, None)))
 
 
+@pytest.mark.parametrize("bias", [False, True])
+def test_prefill_swiglu_one_grid_equals_composition(bias):
+    """Prefill rows: gate and up run as ONE grid of the large-M kernel (the gate tile parked in the workspace) and an
+    elementwise pass forms silu(gate) * up: the bits of fc_silu followed by fc_mul, ragged last row block included."""
+    ops = _ops()
+    K, M, N = 512, 300, 1056
+    wg, qg, sg_ = _make("mxfp4", N, K, 191)
+    wu, qu, su = _make("mxfp4", N, K, 192)
+    x = randn_bf16((M, K), 1.0, 193).cuda()
+    bg = randn_bf16((N,), 0.05, 194).cuda() if bias else None
+    bu = randn_bf16((N,), 0.05, 195).cuda() if bias else None
+    fused = ops.swiglu_gate_up(x, wg, wu, bg, bu)
+    assert torch.equal(fused, ops.fc_mul(x, wu, bu, ops.fc_silu(x, wg, bg)))
+    gate = O.linear_mxfp4(t2bits(x.cpu()), qg, sg_, None if bg is None else t2bits(bg.cpu()), O.POST_SILU)
+    ref = O.linear_mxfp4(t2bits(x.cpu()), qu, su, None if bu is None else t2bits(bu.cpu()), O.POST_MUL, gate)
+    assert_close_bf16(t2bits(fused), ref, ulps=2, what="prefill swiglu gate/up")
+
+
 @pytest.mark.parametrize("M", [2, 12])
 def test_swiglu_full_size_gate_up_equals_composition(M):
     """Llama-7B gate/up shape (688 channel tiles): the fused kernel takes one

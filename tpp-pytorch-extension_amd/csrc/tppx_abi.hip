@@ -240,6 +240,24 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
       if (group) // fused q/k/v: one grid over the channel blocks of all GEMMs
         return check_hip(launch_tiled_mxfp4_group(t, n_segs, stream), who);
     }
+    if (dual) {
+      // Gate and up as ONE grid when that fills the last round of workgroups better than two launches (28672
+      // channels at 2048 rows: 2 x 3.5 rounds of 256 CUs become 7): the gate GEMM leaves its bf16 tile (bias + dot,
+      // the value the reference applies SiLU to) in the workspace, an elementwise pass then forms
+      // silu(gate) * up with the reference's rounding points.  Needs M * N bf16 of workspace.
+      TiledParams t[2] = {tiled_from_seg(p, 0), tiled_from_seg(p, 1)};
+      const int64_t wgs = ((M + 255) / 256) * ((t[0].tiles + 15) / 16);
+      const bool fewer_rounds = (2 * wgs + 255) / 256 < 2 * ((wgs + 255) / 256);
+      if (fewer_rounds && ws && ws_bytes >= M * (int64_t)t[0].N * 2 && tiled_mxfp4_takes_groups(t[0]) &&
+          env_int("TPPX_TILED_DUAL_GROUP", 1) != 0) {
+        t[0].y = (uint16_t*)ws;
+        t[0].post_op = t[1].post_op = TPPX_POST_NONE;
+        rc = check_hip(launch_tiled_mxfp4_group(t, 2, stream), who);
+        if (rc)
+          return rc;
+        return check_hip(launch_silu_mul((const uint16_t*)ws, (uint16_t*)segs[1].y, M * (int64_t)t[0].N, stream), who);
+      }
+    }
     for (int i = 0; i < n_segs; i++) {
       TiledParams t = tiled_from_seg(p, i);
       if (dual) {

@@ -632,6 +632,34 @@ hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// silu(gate) * up over two bf16 tiles that already hold bias + dot (see the gate/up group launch)
+__global__ void __launch_bounds__(256)
+silu_mul_kernel(const uint16_t* __restrict__ gate, uint16_t* __restrict__ y, int64_t n8) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+    const uint4 g = reinterpret_cast<const uint4*>(gate)[i];
+    const uint4 u = reinterpret_cast<const uint4*>(y)[i];
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const uint32_t a0 = apply_post_bits(bf16_bits_to_f32(gw[e] & 0xffffu), TPPX_POST_SILU, 0, 0, 1.0f);
+      const uint32_t a1 = apply_post_bits(bf16_bits_to_f32(gw[e] >> 16), TPPX_POST_SILU, 0, 0, 1.0f);
+      const uint32_t b0 = apply_post_bits(bf16_bits_to_f32(uw[e] & 0xffffu), TPPX_POST_MUL, a0, 0, 1.0f);
+      const uint32_t b1 = apply_post_bits(bf16_bits_to_f32(uw[e] >> 16), TPPX_POST_MUL, a1, 0, 1.0f);
+      o[e] = (b0 & 0xffffu) | (b1 << 16);
+    }
+    reinterpret_cast<uint4*>(y)[i] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
+hipError_t launch_silu_mul(const uint16_t* gate, uint16_t* y, int64_t n, hipStream_t stream) {
+  const int64_t n8 = n / 8;
+  const unsigned blocks = (unsigned)((n8 + 255) / 256 < 256 * 16 ? (n8 + 255) / 256 : 256 * 16);
+  TPPX_PLAN_ONLY(silu_mul_kernel, dim3(blocks), dim3(256), 0);
+  silu_mul_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(gate, y, n8);
+  return hipGetLastError();
+}
+
 hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream) {
   const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
   const size_t lds = 2 * 1024 * 16 + 2 * 128 * sizeof(float);

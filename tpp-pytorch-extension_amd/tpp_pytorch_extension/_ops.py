@@ -474,6 +474,9 @@ def swiglu_gate_up(input, w_gate, w_up, b_gate=None, b_up=None, norm=None):
                                             M, N, K, 0, _lib.stream_of(x)))
         return y
     ws = _lib.workspace(x)
+    if M > 64 and M * N * 2 > ws.numel():
+        # prefill: room for the gate tile lets the library run gate and up as one grid (fuller last round)
+        ws = torch.empty(M * N * 2, dtype=torch.uint8, device=x.device)
     _lib.check(L.tppx_swiglu_mxfp4(x.data_ptr(), qg.data_ptr(), sg.data_ptr(), _lib.ptr(bg), qu.data_ptr(),
                                    su.data_ptr(), _lib.ptr(bu), y.data_ptr(), M, N, K, 0, ws.data_ptr(),
                                    ws.numel(), _lib.stream_of(x)))
