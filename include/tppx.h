@@ -199,7 +199,10 @@ int tppx_multi_linear_qint8(const void* x, void* xq, void* sa,
 /* Replaces the gate/up pair of the Llama MLP
  * (src/csrc/llm/fused_llm_infer.cpp:1271-1272: i_gemm(SiluPostOp) then
  * i_gemm(MulPostOp)) in one launch with the same bf16 rounding points:
- *   g = silu(bf16(x Wg^T + bg));  y = bf16( g * bf16(x Wu^T + bu) ) */
+ *   g = silu(bf16(x Wg^T + bg));  y = bf16( g * bf16(x Wu^T + bu) )
+ * Prefill shapes (M >= 192): with M * N * 2 bytes of workspace both GEMMs run
+ * as one grid (the gate tile parked in the workspace) followed by an
+ * elementwise pass; without it, as two launches.  Same bits either way. */
 int tppx_swiglu_mxfp4(const void* x, const void* qw_gate, const void* sw_gate,
                       const void* bias_gate, const void* qw_up,
                       const void* sw_up, const void* bias_up, void* y,
