@@ -285,6 +285,17 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     set_groups(p, nt, dual);
     return check_hip(launch_skinny_mxfp4_mg(p, 1, nt, dual, stream), who);
   }
+  if (M <= 4 && !dual && p.units <= 128 && env_int("TPPX_MXFP4_X4", 1) == 1) {
+    // up to 4 rows, K beyond the 16-row LDS image: the same staging with only the 4 rows kept
+    int nt = 1;
+    for (; nt < 3; nt++) {
+      set_groups(p, nt, false);
+      if (p.groups <= 256)
+        break;
+    }
+    set_groups(p, nt, false);
+    return check_hip(launch_skinny_mxfp4_x4(p, nt, stream), who);
+  }
   if (M <= 16) {
     // GEMV class: K reduction inside the workgroup, operands straight from global memory
     SkinnyPlan sp = plan_skinny(0, M, p.total_tiles, p.units, dual);

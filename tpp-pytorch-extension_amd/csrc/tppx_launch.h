@@ -88,6 +88,7 @@ SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual
 hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream);
 hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream);
 size_t skinny_mxfp4_xl_lds(int units, int nt, bool dual);
+hipError_t launch_skinny_mxfp4_x4(DecodeParams& p, int nt, hipStream_t stream);
 hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hipStream_t stream);
 hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_t stream);
 

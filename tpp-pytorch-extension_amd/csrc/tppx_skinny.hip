@@ -906,6 +906,130 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
 // planning and launch
 // ---------------------------------------------------------------------------
 // ---------------------------------------------------------------------------
+// MXFP4 weight-only, up to 4 rows, long K (the Llama down-projection of a
+// batch-1 decode step): the LDS-staged kernel above with only the 4 rows kept
+// -- slot (chunk, row) = chunk*4 + (row ^ (chunk & 3)); the 16 MFMA rows read
+// row m & 3 -- so that K up to 16384 fits (cht KiB per wave instead of 4*cht).
+// Sixteen waves split K; x and the weight ring are requested as there.
+// ---------------------------------------------------------------------------
+template <int NT, int PF>
+__global__ void __launch_bounds__(1024)
+skinny_mxfp4_x4_kernel(const DecodeParams p) {
+  extern __shared__ __align__(16) float sk_lds[];
+  constexpr int W = 16, XNI = 8; // item it of a lane: row it / 2, chunk (it % 2) * 64 + lane: 4 rows x 128 chunks
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int grp = blockIdx.x;
+  const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
+  const int ltile0 = (grp - sg.grp0) * NT;
+  const int KT = p.units;
+  const int t0 = (wave * KT) / W, t1 = ((wave + 1) * KT) / W;
+  const int wstride = max(p.cht * 256, NT * 256); // floats per wave region (x slice, later the reduction scratch)
+  i32x4* xs = reinterpret_cast<i32x4*>(sk_lds + (size_t)wave * wstride);
+  const char* qwb = reinterpret_cast<const char*>(sg.qw);
+  const char* swb = reinterpret_cast<const char*>(sg.sw);
+  uint32_t woff[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; nt++)
+    woff[nt] = (uint32_t)(min(ltile0 + nt, sg.tiles - 1) * KT * 64 + lane);
+
+  // activations first (L2 resident), by hand, so that waiting for them does not wait for the weight ring
+  const int nch = (t1 - t0) * 16;
+  const char* xb = reinterpret_cast<const char*>(p.x);
+  const uint32_t xk0 = (uint32_t)t0 * 256u;
+  i32x4 raw[XNI];
+  static_for<0, XNI>([&](auto IT) {
+    constexpr int it = decltype(IT)::value;
+    const int row = min(it >> 1, p.M - 1), ck = max(min((it & 1) * 64 + lane, nch - 1), 0);
+    const char* src = xb + (size_t)((uint32_t)(row * p.K) * 2u + xk0 + (uint32_t)ck * 16u);
+    i32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(src) : "memory");
+    raw[it] = v;
+  });
+  i32x4 wreg[PF][NT];
+  uint32_t sreg[PF][NT];
+  auto load_stage = [&](int st, int t) {
+    t = min(t, t1 - 1);
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      const uint32_t slot = woff[nt] + (uint32_t)t * 64u;
+      wreg[st][nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(qwb + (size_t)(slot * 16u)));
+      sreg[st][nt] = *reinterpret_cast<const uint8_t*>(swb + (size_t)slot);
+    }
+  };
+  if (t0 < t1) {
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+      load_stage(i, t0 + i);
+  }
+  if (t1 - t0 >= PF) // a full ring: PF stages of distinct tiles, 2 * NT loads each
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PF * NT * 2) : "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+  int lane2 = lane;
+  asm volatile("" : "+v"(lane2));
+  static_for<0, XNI>([&](auto IT) {
+    constexpr int it = decltype(IT)::value;
+    i32x4 v = raw[it];
+    asm volatile("" : "+v"(v)); // the use stays behind the wait
+    const int row = it >> 1, ck = (it & 1) * 64 + lane2;
+    if (row < p.M && ck < nch)
+      xs[ck * 4 + (row ^ (ck & 3))] = v;
+  });
+  // the wave reads only what it wrote itself: program order is enough
+
+  SkEpilogue<1, NT, false, 16> ep;
+  ep.prefetch(p, sg, ltile0, 0);
+  f32x4 acc[NT][1];
+#pragma unroll
+  for (int nt = 0; nt < NT; nt++)
+    acc[nt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // operand slot of this lane for step j inside a K tile: chunk g*4 + j (+ 16 per tile), row m & 3
+  int rdo[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int cj = (lane >> 4) * 4 + j;
+    rdo[j] = cj * 4 + ((lane & 3) ^ (cj & 3));
+  }
+  auto consume = [&](int i, int tl) {
+    bf16x8 xa[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      xa[j] = __builtin_bit_cast(bf16x8, xs[tl * 64 + rdo[j]]);
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      const float sc = e8m0_to_f32(sreg[i][nt]);
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        acc[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            xa[j], sk_cvt_fp4x8((uint32_t)wreg[i][nt][j], sc), acc[nt][0], 0, 0, 0);
+    }
+  };
+  int t = t0;
+  for (; t + 2 * PF <= t1; t += PF) { // branch-free full groups: every reload is a real tile
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      consume(i, t + i - t0);
+      load_stage(i, t + i + PF);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  for (; t < t1; t += PF) {
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      const int tt = t + i;
+      if (tt < t1) {
+        consume(i, tt - t0);
+        if (tt + PF < t1)
+          load_stage(i, tt + PF);
+      }
+    }
+  }
+  __syncthreads(); // every wave is done with its x region before it becomes reduction scratch
+  ep.finish(sg, acc, sk_lds, wstride);
+}
+
+// ---------------------------------------------------------------------------
 // MXFP4 weight-only, 17..64 rows: MG row groups of 16 per workgroup.
 // Eight waves split K.  A wave walks its K tiles one at a time: the bf16
 // activations of the tile (MG*16 rows x 256 B, row-contiguous 16-byte loads,
@@ -1232,6 +1356,19 @@ hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_
     SKXL(2, false);
   SKXL(1, false);
 #undef SKXL
+}
+
+// up to 4 rows, K up to 16384 (8 tiles per wave); nt = channel tiles per workgroup (1..3)
+hipError_t launch_skinny_mxfp4_x4(DecodeParams& p, int nt, hipStream_t stream) {
+  p.cht = (p.units + 15) / 16;
+  const size_t wstride = (size_t)(p.cht * 256 > nt * 256 ? p.cht * 256 : nt * 256);
+  const size_t lds = 16 * wstride * sizeof(float);
+  dim3 grid(p.groups, 1);
+  if (nt == 3)
+    return sk_launch(skinny_mxfp4_x4_kernel<3, 2>, p, grid, 16, lds, stream);
+  if (nt == 2)
+    return sk_launch(skinny_mxfp4_x4_kernel<2, 4>, p, grid, 16, lds, stream);
+  return sk_launch(skinny_mxfp4_x4_kernel<1, 4>, p, grid, 16, lds, stream);
 }
 
 size_t skinny_mxfp4_mg_lds(int mg, int ntw, int waves) {
