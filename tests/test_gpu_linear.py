@@ -223,6 +223,22 @@ def test_prefill_swiglu_one_grid_equals_composition(bias):
 
 
 @pytest.mark.parametrize("M", [2, 12])
+def test_swiglu_long_k_few_rows(M):
+    """Gate/up pair with K = 8192 (beyond the 16-row LDS image): the 4-row staged kernel (M = 2) and the tile-by-tile
+    kernel with one row group (M = 12) with two accumulator sets; bits of silu-then-mul, and the oracle."""
+    ops = _ops()
+    K, N = 8192, 1056
+    wg, qg, sg_ = _make("mxfp4", N, K, 311)
+    wu, qu, su = _make("mxfp4", N, K, 312)
+    x = randn_bf16((M, K), 1.0, 313)
+    fused = ops.swiglu_gate_up(x.cuda(), wg, wu)
+    assert torch.equal(fused, ops.fc_mul(x.cuda(), wu, None, ops.fc_silu(x.cuda(), wg, None)))
+    gate = O.linear_mxfp4(t2bits(x), qg, sg_, None, O.POST_SILU)
+    ref = O.linear_mxfp4(t2bits(x), qu, su, None, O.POST_MUL, gate)
+    assert_close_bf16(t2bits(fused), ref, ulps=2, what=f"swiglu gate/up K=8192 M={M}")
+
+
+@pytest.mark.parametrize("M", [2, 12])
 def test_swiglu_full_size_gate_up_equals_composition(M):
     """Llama-7B gate/up shape (688 channel tiles): the fused kernel takes one
     (M <= 4) or two channel tiles of each GEMM per workgroup; both must give the

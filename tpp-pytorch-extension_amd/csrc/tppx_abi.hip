@@ -273,9 +273,11 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
   int nt_xl = 1;
   if (M <= 16 && env_int("TPPX_MXFP4_XL", 1) == 1 && plan_xl(p, dual, &nt_xl))
     return check_hip(launch_skinny_mxfp4_xl(p, nt_xl, dual, stream), who);
-  if (M > 4 && M <= 16 && env_int("TPPX_MXFP4_MG1", 1) == 1) {
-    // K that the LDS-staged kernel above cannot hold: the tile-by-tile kernel with one row group (measured at
-    // K = 11008, N = 4096: 16 rows 14.7 -> 11.7 us; up to 4 rows the register-operand kernel below is faster)
+  if (M <= 16) {
+    // K that the LDS-staged kernel above cannot hold.  Up to 4 rows (and K up to 16384): the same staging with only
+    // the 4 rows kept; otherwise the tile-by-tile kernel with one row group (measured at K = 11008, N = 4096:
+    // 1 row 8.8 -> 7.7 us, 16 rows 14.7 -> 11.7 us against operands read straight from global memory).
+    const bool x4 = M <= 4 && p.units <= 128;
     int nt = 1;
     for (; nt < 3; nt++) {
       set_groups(p, nt, dual);
@@ -283,24 +285,7 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
         break;
     }
     set_groups(p, nt, dual);
-    return check_hip(launch_skinny_mxfp4_mg(p, 1, nt, dual, stream), who);
-  }
-  if (M <= 4 && !dual && p.units <= 128 && env_int("TPPX_MXFP4_X4", 1) == 1) {
-    // up to 4 rows, K beyond the 16-row LDS image: the same staging with only the 4 rows kept
-    int nt = 1;
-    for (; nt < 3; nt++) {
-      set_groups(p, nt, false);
-      if (p.groups <= 256)
-        break;
-    }
-    set_groups(p, nt, false);
-    return check_hip(launch_skinny_mxfp4_x4(p, nt, stream), who);
-  }
-  if (M <= 16) {
-    // GEMV class: K reduction inside the workgroup, operands straight from global memory
-    SkinnyPlan sp = plan_skinny(0, M, p.total_tiles, p.units, dual);
-    set_groups(p, sp.ntw, dual);
-    return check_hip(launch_skinny_mxfp4(p, sp, dual, stream), who);
+    return check_hip(x4 ? launch_skinny_mxfp4_x4(p, nt, dual, stream) : launch_skinny_mxfp4_mg(p, 1, nt, dual, stream), who);
   }
   {
     // 17..64 rows: several MFMA row groups per workgroup, activations streamed through wave-private LDS
@@ -371,7 +356,7 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
     return TPPX_OK;
   }
   p.S = 1;
-  SkinnyPlan sp = plan_skinny(1, M, p.total_tiles, p.units, false, x != nullptr && qbs == 256);
+  SkinnyPlan sp = plan_skinny(M, p.total_tiles, p.units, x != nullptr && qbs == 256);
   if (x && !sp.fused_quant) {
     // quantise straight into MFMA operand order: the GEMM then reads one
     // contiguous 1 KiB per operand instead of 16 rows x 64 B

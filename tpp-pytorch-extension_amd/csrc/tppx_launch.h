@@ -44,7 +44,7 @@ struct DecodeParams {
   float norm_eps;
 };
 
-// in-workgroup K split ("skinny") launch shape
+// launch shape of the QINT8 decode kernels (K split inside the workgroup)
 struct SkinnyPlan {
   int mg, ntw, waves, max_units, grid_y;
   bool fused_quant; // QINT8, M <= 16: activations quantised inside the GEMM kernel
@@ -83,12 +83,11 @@ int env_int(const char* name, int dflt);
 hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs, void* xq, void* sa, int mt,
                                  hipStream_t stream);
 
-// can_fuse_quant: QINT8 with bf16 activations at hand and 256-wide blocks (the in-kernel quantisation's case)
-SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual, bool can_fuse_quant = false);
+// can_fuse_quant: bf16 activations at hand and 256-wide blocks (the in-kernel quantisation's case)
+SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, bool can_fuse_quant);
 hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream);
-hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream);
 size_t skinny_mxfp4_xl_lds(int units, int nt, bool dual);
-hipError_t launch_skinny_mxfp4_x4(DecodeParams& p, int nt, hipStream_t stream);
+hipError_t launch_skinny_mxfp4_x4(DecodeParams& p, int nt, bool dual, hipStream_t stream);
 hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hipStream_t stream);
 hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_t stream);
 

@@ -12,9 +12,9 @@
 //                           global memory (written by the quantiser), 17..64 rows
 //   skinny_qint8_fq_kernel  bf16 activations quantised by the consuming wave into
 //                           wave-private LDS, up to 16 rows
-//   skinny_mxfp4_kernel     bf16 operands straight from global memory (few rows)
 //   skinny_mxfp4_xl_kernel  the wave's whole K slice staged once in LDS, up to
 //                           16 rows; optional RMSNorm in front
+//   skinny_mxfp4_x4_kernel  the same with only 4 rows kept, for long K
 //   skinny_mxfp4_mg_kernel  activations streamed through LDS one K tile at a
 //                           time, 1, 2 or 4 row groups of 16
 //
@@ -577,108 +577,6 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// MXFP4 weight-only, M <= 16 per block row (one MFMA row group).
-// NT channel tiles per workgroup; DUAL: the gate AND the up tile of each of
-// them (NACC = 2*NT accumulators, gate tiles first), epilogue silu(gate) * up.
-// ---------------------------------------------------------------------------
-// WPE = waves per SIMD the register budget must allow (2 workgroups of 8
-// waves per CU need 4).
-template <int NT, int PF, int MAXW, int MINW, bool DUAL, int WPE = 1>
-__global__ void __launch_bounds__(MAXW * 64, WPE)
-skinny_mxfp4_kernel(const DecodeParams p) {
-  constexpr int NTW = DUAL ? 2 * NT : NT; // weight tiles per ring stage = accumulators
-  extern __shared__ __align__(16) float sk_lds[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int W = blockDim.x >> 6;
-  const int grp = blockIdx.x;
-  const int seg_id = DUAL ? 0 : sk_find_seg(p, grp);
-  const DecodeSeg& sg = p.seg[seg_id];
-  const int ltile0 = (grp - sg.grp0) * NT;
-  const int m0 = blockIdx.y * 16;
-  const int KT = p.units;
-  const int t0 = (int)(((int64_t)wave * KT) / W), t1 = (int)(((int64_t)(wave + 1) * KT) / W);
-
-  // uniform base pointer per GEMM + one 32-bit slot offset per channel tile
-  // (gate and up tiles share it): no 64-bit pointer pair per stream
-  constexpr int NSEG = DUAL ? 2 : 1;
-  const char* qwb[NSEG];
-  const char* swb[NSEG];
-#pragma unroll
-  for (int sgi = 0; sgi < NSEG; sgi++) {
-    const DecodeSeg& ss = p.seg[DUAL ? sgi : seg_id];
-    qwb[sgi] = reinterpret_cast<const char*>(ss.qw);
-    swb[sgi] = reinterpret_cast<const char*>(ss.sw);
-  }
-  uint32_t woff[NT];
-#pragma unroll
-  for (int nt = 0; nt < NT; nt++)
-    woff[nt] = (uint32_t)(min(ltile0 + nt, sg.tiles - 1) * KT * 64 + lane); // ragged last group: duplicate, not stored
-  const int mrow = min(m0 + (lane & 15), p.M - 1);
-  const uint16_t* xrow = reinterpret_cast<const uint16_t*>(p.x) + (int64_t)mrow * p.K + (lane >> 4) * 32;
-
-  i32x4 wreg[PF][NTW];
-  uint32_t sreg[PF][NTW];
-  bf16x8 xreg[PF][4];
-  auto load_stage = [&](int st, int t) {
-    t = min(t, t1 - 1);
-#pragma unroll
-    for (int nt = 0; nt < NTW; nt++) {
-      const uint32_t slot = woff[nt % NT] + (uint32_t)t * 64u;
-      wreg[st][nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(qwb[nt / NT] + (size_t)(slot * 16u)));
-      sreg[st][nt] = *reinterpret_cast<const uint8_t*>(swb[nt / NT] + (size_t)slot);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; j++)
-      xreg[st][j] = *reinterpret_cast<const bf16x8*>(xrow + t * 128 + j * 8);
-  };
-  if (t0 < t1) {
-#pragma unroll
-    for (int i = 0; i < PF; i++)
-      load_stage(i, t0 + i);
-  }
-
-  SkEpilogue<1, NTW, DUAL, MINW> ep;
-  ep.prefetch(p, sg, ltile0, m0);
-
-  f32x4 acc[NTW][1];
-#pragma unroll
-  for (int nt = 0; nt < NTW; nt++)
-    acc[nt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  auto consume = [&](int i) {
-#pragma unroll
-    for (int nt = 0; nt < NTW; nt++) {
-      const float sc = e8m0_to_f32(sreg[i][nt]);
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        acc[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            xreg[i][j], sk_cvt_fp4x8((uint32_t)wreg[i][nt][j], sc), acc[nt][0], 0, 0, 0);
-    }
-  };
-  int t = t0;
-  for (; t + 2 * PF <= t1; t += PF) { // every reload of these groups is a real tile // branch-free full groups: exact wait counts, PF stages in flight
-#pragma unroll
-    for (int i = 0; i < PF; i++) {
-      consume(i);
-      load_stage(i, t + i + PF); // clamped past the end (re-reads the last tile, never consumed)
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  }
-  for (; t < t1; t += PF) {
-#pragma unroll
-    for (int i = 0; i < PF; i++) {
-      const int tt = t + i;
-      if (tt < t1) {
-        consume(i);
-        if (tt + PF < t1)
-          load_stage(i, tt + PF);
-      }
-    }
-  }
-  ep.finish(sg, acc, sk_lds);
-}
-
-// ---------------------------------------------------------------------------
 // MXFP4, M <= 16, activations staged in LDS by the wave that consumes them,
 // with an optional transform on the way in:
 //   XMODE 0  x as it is
@@ -912,22 +810,31 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
 // row m & 3 -- so that K up to 16384 fits (cht KiB per wave instead of 4*cht).
 // Sixteen waves split K; x and the weight ring are requested as there.
 // ---------------------------------------------------------------------------
-template <int NT, int PF>
+template <int NT, int PF, bool DUAL>
 __global__ void __launch_bounds__(1024)
 skinny_mxfp4_x4_kernel(const DecodeParams p) {
   extern __shared__ __align__(16) float sk_lds[];
+  constexpr int NTW = DUAL ? 2 * NT : NT; // DUAL: the gate AND the up tile of each channel tile (gate tiles first)
   constexpr int W = 16, XNI = 8; // item it of a lane: row it / 2, chunk (it % 2) * 64 + lane: 4 rows x 128 chunks
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int grp = blockIdx.x;
-  const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
+  const int seg_id = DUAL ? 0 : sk_find_seg(p, grp);
+  const DecodeSeg& sg = p.seg[seg_id];
   const int ltile0 = (grp - sg.grp0) * NT;
   const int KT = p.units;
   const int t0 = (wave * KT) / W, t1 = ((wave + 1) * KT) / W;
-  const int wstride = max(p.cht * 256, NT * 256); // floats per wave region (x slice, later the reduction scratch)
+  const int wstride = max(p.cht * 256, NTW * 256); // floats per wave region (x slice, later the reduction scratch)
   i32x4* xs = reinterpret_cast<i32x4*>(sk_lds + (size_t)wave * wstride);
-  const char* qwb = reinterpret_cast<const char*>(sg.qw);
-  const char* swb = reinterpret_cast<const char*>(sg.sw);
+  constexpr int NSEG = DUAL ? 2 : 1;
+  const char* qwb[NSEG];
+  const char* swb[NSEG];
+#pragma unroll
+  for (int sgi = 0; sgi < NSEG; sgi++) {
+    const DecodeSeg& ss = p.seg[DUAL ? sgi : seg_id];
+    qwb[sgi] = reinterpret_cast<const char*>(ss.qw);
+    swb[sgi] = reinterpret_cast<const char*>(ss.sw);
+  }
   uint32_t woff[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; nt++)
@@ -946,15 +853,15 @@ skinny_mxfp4_x4_kernel(const DecodeParams p) {
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(src) : "memory");
     raw[it] = v;
   });
-  i32x4 wreg[PF][NT];
-  uint32_t sreg[PF][NT];
+  i32x4 wreg[PF][NTW];
+  uint32_t sreg[PF][NTW];
   auto load_stage = [&](int st, int t) {
     t = min(t, t1 - 1);
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      const uint32_t slot = woff[nt] + (uint32_t)t * 64u;
-      wreg[st][nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(qwb + (size_t)(slot * 16u)));
-      sreg[st][nt] = *reinterpret_cast<const uint8_t*>(swb + (size_t)slot);
+    for (int nt = 0; nt < NTW; nt++) {
+      const uint32_t slot = woff[nt % NT] + (uint32_t)t * 64u;
+      wreg[st][nt] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(qwb[nt / NT] + (size_t)(slot * 16u)));
+      sreg[st][nt] = *reinterpret_cast<const uint8_t*>(swb[nt / NT] + (size_t)slot);
     }
   };
   if (t0 < t1) {
@@ -962,8 +869,8 @@ skinny_mxfp4_x4_kernel(const DecodeParams p) {
     for (int i = 0; i < PF; i++)
       load_stage(i, t0 + i);
   }
-  if (t1 - t0 >= PF) // a full ring: PF stages of distinct tiles, 2 * NT loads each
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PF * NT * 2) : "memory");
+  if (t1 - t0 >= PF) // a full ring: PF stages of distinct tiles, 2 * NTW loads each
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PF * NTW * 2) : "memory");
   else
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
   int lane2 = lane;
@@ -978,11 +885,11 @@ skinny_mxfp4_x4_kernel(const DecodeParams p) {
   });
   // the wave reads only what it wrote itself: program order is enough
 
-  SkEpilogue<1, NT, false, 16> ep;
+  SkEpilogue<1, NTW, DUAL, 16> ep;
   ep.prefetch(p, sg, ltile0, 0);
-  f32x4 acc[NT][1];
+  f32x4 acc[NTW][1];
 #pragma unroll
-  for (int nt = 0; nt < NT; nt++)
+  for (int nt = 0; nt < NTW; nt++)
     acc[nt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
   // operand slot of this lane for step j inside a K tile: chunk g*4 + j (+ 16 per tile), row m & 3
   int rdo[4];
@@ -997,7 +904,7 @@ skinny_mxfp4_x4_kernel(const DecodeParams p) {
     for (int j = 0; j < 4; j++)
       xa[j] = __builtin_bit_cast(bf16x8, xs[tl * 64 + rdo[j]]);
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
+    for (int nt = 0; nt < NTW; nt++) {
       const float sc = e8m0_to_f32(sreg[i][nt]);
 #pragma unroll
       for (int j = 0; j < 4; j++)
@@ -1201,35 +1108,28 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
   }
 }
 
-SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual, bool can_fuse_quant) {
+// launch shape of the QINT8 decode kernels
+SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, bool can_fuse_quant) {
   SkinnyPlan pl;
   const int mrows = (int)(M < 64 ? M : 64);
-  pl.mg = fmt == 0 ? 1 : (mrows <= 16 ? 1 : (mrows <= 32 ? 2 : 4));
+  pl.mg = mrows <= 16 ? 1 : (mrows <= 32 ? 2 : 4);
   pl.grid_y = (int)((M + 16 * pl.mg - 1) / (16 * pl.mg));
   // two channel tiles per wave once there are plenty of tiles: halves the
   // activation-operand traffic per weight byte
-  pl.ntw = (!dual && total_tiles >= 512) ? 2 : 1;
-  int env_ntw = env_int("TPPX_SKINNY_NTW", 0);
-  if (!dual && (env_ntw == 1 || env_ntw == 2))
+  pl.ntw = total_tiles >= 512 ? 2 : 1;
+  const int env_ntw = env_int("TPPX_SKINNY_NTW", 0);
+  if (env_ntw == 1 || env_ntw == 2)
     pl.ntw = env_ntw;
-  if (dual) // channel tiles per workgroup of EACH of the two GEMMs
-    pl.ntw = (total_tiles >= 512 && M > 4 && env_ntw != 1) ? 2 : 1; // few rows: activation traffic is negligible
   // more than 16 rows: these kernels run one workgroup per CU, so prefer a grid
   // of at most 256 workgroups (a second, partly filled round costs a full one)
-  if (fmt == 1 && pl.mg > 1 && env_ntw == 0 && total_tiles > 512 && total_tiles <= 768)
+  if (pl.mg > 1 && env_ntw == 0 && total_tiles > 512 && total_tiles <= 768)
     pl.ntw = 3;
   // Wave-count window of the kernel instantiation that will run (register
   // budget: 16 waves leave 128 VGPRs per lane, 8 leave 256; the epilogue's
   // outputs-per-thread bound sets the minimum).  Waves beyond the number of K
   // units simply get an empty range.
-  int max_w, min_w;
-  if (fmt == 1) {
-    max_w = (pl.mg == 4 || (pl.mg == 2 && pl.ntw >= 2)) ? 8 : 16;
-    min_w = (pl.mg == 4 || (pl.mg == 2 && pl.ntw >= 2)) ? 8 : 4;
-  } else {
-    max_w = (dual || pl.ntw == 2) ? 8 : 16;
-    min_w = 4;
-  }
+  const bool wide = pl.mg == 4 || (pl.mg == 2 && pl.ntw >= 2);
+  const int max_w = wide ? 8 : 16, min_w = wide ? 8 : 4;
   // few tiles: one 16-wave workgroup per CU keeps the whole weight in flight
   int w = env_int("TPPX_SKINNY_WAVES", (total_tiles / pl.ntw <= 320) ? 16 : 8);
   if (w > units)
@@ -1242,7 +1142,7 @@ SkinnyPlan plan_skinny(int fmt, int64_t M, int total_tiles, int units, bool dual
   pl.max_units = (units + w - 1) / w;
   pl.fused_quant = false;
   pl.lds_overlap = false;
-  if (fmt == 1 && M <= 16 && can_fuse_quant && env_int("TPPX_SKINNY_FUSEDQ", 1) != 0) {
+  if (M <= 16 && can_fuse_quant && env_int("TPPX_SKINNY_FUSEDQ", 1) != 0) {
     // quantisation inside the GEMM kernel: 16 waves, the fewest channel tiles per workgroup that keep the grid
     // within one round of 256 workgroups, as long as the quantised rows of all waves fit the LDS
     const int ntw = total_tiles <= 256 ? 1 : (total_tiles <= 512 ? 2 : 3);
@@ -1358,17 +1258,25 @@ hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_
 #undef SKXL
 }
 
-// up to 4 rows, K up to 16384 (8 tiles per wave); nt = channel tiles per workgroup (1..3)
-hipError_t launch_skinny_mxfp4_x4(DecodeParams& p, int nt, hipStream_t stream) {
+// up to 4 rows, K up to 16384 (8 tiles per wave); nt = channel tiles per workgroup (1..3; of each GEMM when dual)
+hipError_t launch_skinny_mxfp4_x4(DecodeParams& p, int nt, bool dual, hipStream_t stream) {
   p.cht = (p.units + 15) / 16;
-  const size_t wstride = (size_t)(p.cht * 256 > nt * 256 ? p.cht * 256 : nt * 256);
+  const int ntw = dual ? 2 * nt : nt;
+  const size_t wstride = (size_t)(p.cht * 256 > ntw * 256 ? p.cht * 256 : ntw * 256);
   const size_t lds = 16 * wstride * sizeof(float);
   dim3 grid(p.groups, 1);
+  if (dual) {
+    if (nt == 3)
+      return sk_launch(skinny_mxfp4_x4_kernel<3, 2, true>, p, grid, 16, lds, stream);
+    if (nt == 2)
+      return sk_launch(skinny_mxfp4_x4_kernel<2, 2, true>, p, grid, 16, lds, stream);
+    return sk_launch(skinny_mxfp4_x4_kernel<1, 4, true>, p, grid, 16, lds, stream);
+  }
   if (nt == 3)
-    return sk_launch(skinny_mxfp4_x4_kernel<3, 2>, p, grid, 16, lds, stream);
+    return sk_launch(skinny_mxfp4_x4_kernel<3, 2, false>, p, grid, 16, lds, stream);
   if (nt == 2)
-    return sk_launch(skinny_mxfp4_x4_kernel<2, 4>, p, grid, 16, lds, stream);
-  return sk_launch(skinny_mxfp4_x4_kernel<1, 4>, p, grid, 16, lds, stream);
+    return sk_launch(skinny_mxfp4_x4_kernel<2, 4, false>, p, grid, 16, lds, stream);
+  return sk_launch(skinny_mxfp4_x4_kernel<1, 4, false>, p, grid, 16, lds, stream);
 }
 
 size_t skinny_mxfp4_mg_lds(int mg, int ntw, int waves) {
@@ -1430,19 +1338,6 @@ hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hi
     SKMG(4, 2, false, 2);
   SKMG(4, 1, false, 2);
 #undef SKMG
-}
-
-hipError_t launch_skinny_mxfp4(DecodeParams& p, const SkinnyPlan& pl, bool dual, hipStream_t stream) {
-  dim3 grid(p.groups, pl.grid_y);
-  size_t lds = (size_t)pl.waves * pl.ntw * (dual ? 2 : 1) * 256 * sizeof(float);
-  if (dual) {
-    if (pl.ntw == 2)
-      return sk_launch(skinny_mxfp4_kernel<2, 2, 8, 4, true, 4>, p, grid, pl.waves, lds, stream);
-    return sk_launch(skinny_mxfp4_kernel<1, 2, 8, 4, true, 4>, p, grid, pl.waves, lds, stream);
-  }
-  if (pl.ntw == 2)
-    return sk_launch(skinny_mxfp4_kernel<2, 2, 8, 4, false, 4>, p, grid, pl.waves, lds, stream);
-  return sk_launch(skinny_mxfp4_kernel<1, 4, 16, 4, false>, p, grid, pl.waves, lds, stream);
 }
 
 } // namespace tppx
