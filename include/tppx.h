@@ -136,11 +136,15 @@ int tppx_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs,
 
 /* Workspace (`ws`, `ws_bytes`) of the linear entry points: optional device
  * scratch, 256-byte aligned, that lets decode-shape launches with more than 16
- * rows split K across workgroups (fp32 partial tiles, summed by a second small
- * launch).  It needs no initialisation and carries no state between calls.
+ * rows split K across workgroups (fp32 partial tiles, summed inside the same
+ * launch by whichever workgroup of a tile finishes last, in a fixed order).
+ * It needs no initialisation and carries no state between calls.
  * Launches that share a workspace must be ordered on one stream.  With
  * ws == NULL (or too small) the kernels simply do not split K.  32 MiB covers
- * every decode shape up to M=64, N=32768. */
+ * every decode shape up to M=64, N=32768.  The arrival counters of such a
+ * launch live in the library (16384 per device, handed out in rotation, at
+ * most 256 per launch), so K-split launches on different streams may overlap
+ * as long as fewer than 64 of them are in flight on one device. */
 
 /* Replaces call_gemm_with_post_op -> TppBlockedLinearW<bf16,uint8_t,bf16>
  * (MXFP4 branch, src/csrc/fused_gemm.h:785-1073,1510-1522) i.e.

@@ -282,6 +282,25 @@ def test_mxfp4_row_group_kernel_uneven_k_split_and_swiglu(M):
     assert_close_bf16(t2bits(fused), ref2, ulps=2, what=f"swiglu gate/up M={M}")
 
 
+@pytest.mark.parametrize("fmt,M,N", [("mxfp4", 40, 4096), ("mxfp4", 64, 4064), ("qint8", 40, 4096), ("qint8", 64, 4080)])
+def test_k_split_across_workgroups(fmt, M, N):
+    """33..64 rows, at most 256 channel tiles and K = 11008: K is split across workgroups (4 parts of 21/22/21/22
+    K tiles for MXFP4, 2 parts of 21/22 blocks for QINT8), the partial sums go through the workspace and the
+    workgroup that finishes last adds them.  N = 4064 (254 tiles) or 4080 (255): a ragged last group; M = 40: a partly filled row
+    group.  Forty launches in a row must give the same bits (the arrival counters return to zero, no launch sees
+    another's partial sums)."""
+    ops = _ops()
+    y, ref, s, ctx = _run(fmt, M, N, 11008, "add", True, 7400 + M)
+    qw, q_or, s_or, x, bias, in1, in2, scale = ctx
+    xs, b, r = x.cuda(), bias.cuda(), in1.cuda()
+    first = torch.ops.tpp_llm.fc_add(xs, qw, b, r, scale)
+    outs = [torch.ops.tpp_llm.fc_add(xs, qw, b, r, scale) for _ in range(40)]
+    torch.cuda.synchronize()
+    assert torch.equal(first, y)
+    for o in outs:
+        assert torch.equal(o, first)
+
+
 def test_prefill_qkv_one_launch_equals_separate():
     """With enough rows the fused q/k/v GEMMs share one launch of the large-M
     kernel (one grid over the channel blocks of all three)."""

@@ -134,16 +134,16 @@ static bool plan_xl(DecodeParams& p, bool dual, int* nt_out) {
 }
 
 // K split of the single-kernel decode paths for more than 16 rows: the largest S in {4, 2} (at most max_s) such that
-// S channel tiles per workgroup still give at most 256 workgroups in all, every part keeps 2048 input channels, and
+// S channel tiles per workgroup still give at most 256 workgroups in all, every part keeps min_k input channels, and
 // the partial tiles fit the workspace; 1 otherwise (also whenever there are enough channel tiles for three per
 // workgroup, where the activations are the smaller stream anyway).
-static int pick_split(const DecodeParams& p, int64_t M, int64_t K, int mg, int max_s, int64_t ws_bytes) {
+static int pick_split(const DecodeParams& p, int64_t M, int64_t K, int mg, int max_s, int64_t min_k, int64_t ws_bytes) {
   if (env_int("TPPX_SKINNY_SPLITK", 1) == 0 || p.n_seg != 1 || M > 64)
     return 1;
   for (int s = max_s; s >= 2; s >>= 1) {
     const int groups = (p.total_tiles + s - 1) / s;
     const int64_t need = (int64_t)s * p.total_tiles * mg * 256 * (int64_t)sizeof(float);
-    if (p.total_tiles <= 256 && groups * s <= 256 && K / s >= 2048 && need <= ws_bytes)
+    if (p.total_tiles <= 256 && groups * s <= 256 && K / s >= min_k && need <= ws_bytes)
       return s;
   }
   return 1;
@@ -292,10 +292,9 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     const int mg = M <= 32 ? 2 : 4;
     // Few channel tiles and a long K: every workgroup would pull all of the activations (M x K) through its CU.
     // Split K across S workgroups that own S times the channel tiles each: the same number of workgroups, 1/S of
-    // the activations per CU, fp32 partial tiles through the workspace and a second small kernel.
-    // (measured: 26 -> 22 us for 64 rows at K = 11008 / N = 4096; no gain for 32 rows, and none for QINT8, whose
-    // int8 activations are half the bytes)
-    const int S = (dual || mg != 4) ? 1 : pick_split(p, M, K, mg, 4, ws_bytes);
+    // the activations per CU, fp32 partial tiles through the workspace, summed by whichever of the S workgroups
+    // finishes last (measured: 26 -> 21 us for 64 rows at K = 11008 / N = 4096; no gain for 32 rows).
+    const int S = (dual || mg != 4) ? 1 : pick_split(p, M, K, mg, 4, 2048, ws_bytes);
     int nt = S;
     if (S == 1) {
       for (; nt < 3; nt++) {
@@ -307,10 +306,7 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     set_groups(p, nt, dual);
     p.S = S;
     p.part = (float*)ws;
-    rc = check_hip(launch_skinny_mxfp4_mg(p, mg, nt, dual, stream), who);
-    if (rc == TPPX_OK && S > 1)
-      rc = check_hip(launch_splitk_finish(p, mg, 1, stream), who);
-    return rc;
+    return check_hip(launch_skinny_mxfp4_mg(p, mg, nt, dual, stream), who);
   }
 }
 
@@ -357,6 +353,16 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
   }
   p.S = 1;
   SkinnyPlan sp = plan_skinny(M, p.total_tiles, p.units, x != nullptr && qbs == 256);
+  // 33..64 rows, few channel tiles and a long K: every workgroup would pull all of the int8 activations (M x K)
+  // through its CU.  Two K parts of two channel tiles each halve that (measured at N = 4096, 64 rows: K = 11008
+  // 20.4 -> 18.5 us, K = 14336 25.1 -> 21.6 us; K = 8192 and shorter lose to the extra pass over the partial sums).
+  if (sp.mg == 4 && !sp.fused_quant && pick_split(p, M, K, sp.mg, 2, 5504, ws_bytes) == 2) {
+    p.S = 2;
+    p.part = (float*)ws;
+    sp.ntw = 2;
+    sp.waves = 8;
+    sp.max_units = (p.units + 7) / 8;
+  }
   if (x && !sp.fused_quant) {
     // quantise straight into MFMA operand order: the GEMM then reads one
     // contiguous 1 KiB per operand instead of 16 rows x 64 B

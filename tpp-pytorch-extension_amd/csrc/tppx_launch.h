@@ -36,10 +36,12 @@ struct DecodeParams {
   int mt;    // > 0: xq is [K/64][mt][4 g][16 m][16 B] (operand tiles of 16 rows x 64 K); 0: row-major
   int units; // K/128 (MXFP4 tiles) or K/qbs (QINT8 blocks)
   int tpb;   // native tiles per unit (1 for MXFP4, qbs/64 for QINT8)
-  int S;     // K parts across workgroups (grid z); > 1: partial sums go to `part`, a second kernel finishes
+  int S;     // K parts across workgroups (grid z, at most 4); > 1: partial sums go to `part`, the workgroup that
+             // arrives last at its ticket adds them and runs the epilogue
+  int ticket0; // first arrival counter of this launch (S > 1), see skinny_split_tickets()
   int cht;   // tiles of activations staged in LDS at a time
   int lds_overlap; // fused-quantisation QINT8 kernel: the reduction region reuses the LDS of the activations
-  float* part;   // [S][block row][total_tiles][MG][64] x f32x4 partial tiles (S > 1)
+  float* part;   // [S][block row][total_tiles][MG][256] fp32 partial tiles (S > 1)
   const float* norm_gamma; // f32 [K]: RMSNorm fused in front of the GEMM (LDS-staged MXFP4 kernel), or null
   float norm_eps;
 };
@@ -91,6 +93,7 @@ hipError_t launch_skinny_mxfp4_x4(DecodeParams& p, int nt, bool dual, hipStream_
 hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hipStream_t stream);
 hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_t stream);
 
-hipError_t launch_splitk_finish(const DecodeParams& p, int mg, int grid_y, hipStream_t stream);
+// window of `n` arrival counters for one K-split launch (first index), or -1 when n exceeds what the library keeps
+int skinny_split_tickets(int n);
 
 } // namespace tppx

@@ -1,13 +1,13 @@
 // Decode-shape kernels (up to 64 rows) with the K reduction kept inside the workgroup.
 //
 // One workgroup owns a few consecutive 16-channel weight tiles and all of K
-// (or one of a few K parts, see finish_partial); its 8 or 16 waves split K
+// (or one of a few K parts, see finish_split); its 8 or 16 waves split K
 // into contiguous ranges.  A wave streams the native 1 KiB tiles of its range
 // straight from HBM into registers (one 128-bit load per lane and tile, a ring
 // of PF k-tiles in flight, issued before anything that could wait), feeds the
 // 16x16 MFMA, and at the end the waves' partial tiles are summed through LDS
-// in a fixed order (deterministic) and the fused epilogue runs.  No global
-// atomics.  The kernels differ in how the activation operand gets there:
+// in a fixed order (deterministic) and the fused epilogue runs.  No atomics
+// on data.  The kernels differ in how the activation operand gets there:
 //   skinny_qint8_kernel     int8 activations already in MFMA operand order in
 //                           global memory (written by the quantiser), 17..64 rows
 //   skinny_qint8_fq_kernel  bf16 activations quantised by the consuming wave into
@@ -48,6 +48,13 @@ __device__ __forceinline__ int sk_find_seg(const DecodeParams& p, int grp) {
       s = i;
   return s;
 }
+
+// Arrival counters of the launches that split K across workgroups: one per (block row, channel group), all zero
+// between launches (the counting instruction wraps to zero on the last arrival).  A launch takes a window of
+// them that the host hands out in rotation, so launches in flight at the same time do not share counters as long
+// as fewer than SK_TICKETS counters are in use at once.
+constexpr int SK_TICKETS = 16384;
+__device__ unsigned int sk_split_tickets[SK_TICKETS];
 
 // LDS reduction over the waves of the workgroup + fused epilogue.
 // red layout: [wave][(a*MG + mg)*256 + r*64 + lane]; every thread finishes
@@ -126,12 +133,13 @@ struct SkEpilogue {
       }
   }
 
-  // K split across workgroups (blockIdx.z = part): the workgroup's sums go to the workspace as accumulator
-  // fragments, [part][block row][tile][row group][lane] x f32x4, for the second-pass kernel that adds the parts in
-  // a fixed order and runs the epilogue.
-  __device__ __forceinline__ void finish_partial(const DecodeParams& p, const DecodeSeg& sg, f32x4 (&acc)[NACC][MG],
-                                                 float* red, int ltile0, int stride = ELEMS) {
+  // K split across workgroups (blockIdx.z = part).  Every workgroup leaves its sums in the workspace,
+  // [part][block row][tile][row group][r * 64 + lane] floats, and takes a ticket; the workgroup that arrives last
+  // adds the parts in part order (the same sums whichever workgroup that is) and runs the epilogue.  Nobody waits.
+  __device__ __forceinline__ void finish_split(const DecodeParams& p, const DecodeSeg& sg, f32x4 (&acc)[NACC][MG],
+                                               float* red, int ltile0, int stride = ELEMS) {
     static_assert(!DUAL, "the gate/up pair is not split");
+    __shared__ int arrived_last;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int W = blockDim.x >> 6;
     float* mine = red + wave * stride;
@@ -143,19 +151,52 @@ struct SkEpilogue {
         for (int r = 0; r < 4; r++)
           mine[(a * MG + mg) * 256 + r * 64 + lane] = acc[a][mg][r];
     __syncthreads();
-    float* part = p.part + ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * p.total_tiles * (MG * 256);
+    const size_t part_stride = (size_t)gridDim.y * p.total_tiles * (MG * 256);
+    float* part = p.part + ((size_t)blockIdx.y * p.total_tiles + sg.tile0 + ltile0) * (MG * 256);
+    float own[MAXE];
 #pragma unroll
     for (int i = 0; i < MAXE; i++) {
       const int e = threadIdx.x + i * blockDim.x;
+      own[i] = 0.f;
       if (e < OUT) {
-        float v = 0.f;
         for (int w = 0; w < W; w++)
-          v += red[w * stride + e];
-        const int l = e & 63, r = (e >> 6) & 3, mg = (e >> 8) % MG, a = (e >> 8) / MG;
-        if (ltile0 + a < sg.tiles)
-          part[((size_t)(sg.tile0 + ltile0 + a) * MG + mg) * 256 + l * 4 + r] = v;
+          own[i] += red[w * stride + e];
+        if (ltile0 + e / (MG * 256) < sg.tiles)
+          __hip_atomic_store(part + blockIdx.z * part_stride + e, own[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
+    // The sums travel as device-scope atomic stores and loads (written through to, and read from, the level all
+    // XCDs share), so no cache write-back or invalidate is needed: a device-wide fence here costs more than the
+    // whole kernel (measured: +8 us with one fencing thread per workgroup, +40 us with all).  Order: the stores are
+    // complete at the barrier (it waits for outstanding memory operations), then the ticket, then the loads.
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const unsigned int last = (unsigned int)p.S - 1;
+      arrived_last = atomicInc(&sk_split_tickets[p.ticket0 + blockIdx.y * gridDim.x + blockIdx.x], last) == last;
+    }
+    __syncthreads();
+    if (!arrived_last)
+      return;
+    float pv[MAXE][4];
+#pragma unroll
+    for (int i = 0; i < MAXE; i++)
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        pv[i][k] = 0.f;
+        if (off[i] >= 0 && k < p.S && k != (int)blockIdx.z)
+          pv[i][k] = __hip_atomic_load(part + k * part_stride + threadIdx.x + i * blockDim.x, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+      }
+#pragma unroll
+    for (int i = 0; i < MAXE; i++)
+      if (off[i] >= 0) {
+        float v = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+          if (k < p.S)
+            v += k == (int)blockIdx.z ? own[i] : pv[i][k];
+        sg.y[off[i]] = (uint16_t)apply_post_bits(v + bf16_bits_to_f32(bias[i]), sg.post_op, in1[i], in2[i], sg.post_scale);
+      }
   }
 
   // stride = floats between the regions of two waves (>= ELEMS)
@@ -364,7 +405,7 @@ skinny_qint8_kernel(const DecodeParams p) {
     }
   }
   if (p.S > 1)
-    ep.finish_partial(p, sg, facc, red, ltile0);
+    ep.finish_split(p, sg, facc, red, ltile0);
   else
     ep.finish(sg, facc, red);
 }
@@ -1102,7 +1143,7 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
     ep.finish_halves(sg, acc, sk_lds);
   } else {
     if (p.S > 1)
-      ep.finish_partial(p, sg, acc, sk_lds, ltile0);
+      ep.finish_split(p, sg, acc, sk_lds, ltile0);
     else
       ep.finish(sg, acc, sk_lds);
   }
@@ -1159,6 +1200,19 @@ SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, bool can_fuse_quan
   return pl;
 }
 
+int skinny_split_tickets(int n) {
+  static std::mutex mu;
+  static int cursor = 0;
+  if (n <= 0 || n > SK_TICKETS)
+    return -1;
+  std::lock_guard<std::mutex> lock(mu);
+  if (cursor + n > SK_TICKETS)
+    cursor = 0;
+  const int first = cursor;
+  cursor += n;
+  return first;
+}
+
 template <typename K>
 static hipError_t sk_launch(K kern, const DecodeParams& p, dim3 grid, int waves, size_t lds, hipStream_t stream) {
   TPPX_PLAN_ONLY(kern, grid, dim3(64 * waves), lds);
@@ -1185,6 +1239,8 @@ static hipError_t sk_launch(K kern, const DecodeParams& p, dim3 grid, int waves,
 hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream) {
   p.cht = pl.max_units; // per-wave slots of activation scales in LDS
   dim3 grid(p.groups, pl.grid_y, pl.fused_quant ? 1 : p.S);
+  if (grid.z > 1 && (p.S > 4 || (p.ticket0 = skinny_split_tickets((int)(grid.x * grid.y))) < 0))
+    return hipErrorInvalidValue;
   if (pl.fused_quant) {
     const size_t xbytes = (size_t)16 * pl.max_units * (256 * (size_t)p.M + 64), rbytes = (size_t)16 * pl.ntw * 1024;
     const size_t lds = pl.lds_overlap ? (xbytes > rbytes ? xbytes : rbytes) : xbytes + rbytes;
@@ -1288,6 +1344,8 @@ size_t skinny_mxfp4_mg_lds(int mg, int ntw, int waves) {
 // groups counted by the caller
 hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hipStream_t stream) {
   dim3 grid(p.groups, (p.M + mg * 16 - 1) / (mg * 16), p.S);
+  if (p.S > 1 && (p.S > 4 || (p.ticket0 = skinny_split_tickets((int)(grid.x * grid.y))) < 0))
+    return hipErrorInvalidValue;
   if (mg == 1) { // up to 16 rows: sixteen waves, deeper weight ring
     const size_t lds1 = skinny_mxfp4_mg_lds(1, nt, 16);
 #define SKMG1(NT, DUAL, PF) return sk_launch(skinny_mxfp4_mg_kernel<1, NT, DUAL, PF, 16>, p, grid, 16, lds1, stream)
