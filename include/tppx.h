@@ -273,6 +273,17 @@ int tppx_attn_decode(const void* q, const void* kcache, const void* vcache,
                      int64_t Smax, void* ws, int64_t ws_bytes,
                      tppx_stream_t stream);
 
+/* The same attn<T> (src/csrc/llm/attn.cpp:781-955, isCausal) for S query tokens
+ * per sequence (prompt processing, or several new tokens on a filled cache):
+ * q / out bf16 [B][S][Nq][128]; the cache already holds the S new keys at
+ * positions past_len .. past_len+S-1 (tppx_rotary_kv_append_llama before this
+ * call); query i sees keys 0 .. past_len+i; additive mask bf16 [B][mask_ld]
+ * over key positions or NULL. */
+int tppx_attn_prefill(const void* q, const void* kcache, const void* vcache,
+                      const void* mask, int64_t mask_ld, int64_t past_len,
+                      void* out, int64_t B, int64_t S, int64_t Nq, int64_t Nkv,
+                      int64_t H, int64_t Smax, tppx_stream_t stream);
+
 /* ---- launch plans ------------------------------------------------------- */
 
 /* No counterpart in the reference.  Writes into buf, one line per kernel, what

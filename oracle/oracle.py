@@ -523,3 +523,30 @@ def attn_decode(q_bf16, k_bf16, v_bf16, mask_f32=None, round_probs=True):
             pb = _bf16_round_f32(p.astype(np.float32)).astype(np.float64) if round_probs else p
             out[b, n] = (pb @ v[b, n // R] / p.sum()).astype(np.float32)
     return f32_to_bf16(out)
+
+
+def attn_prefill(q_bf16, k_bf16, v_bf16, mask_f32=None, round_probs=True):
+    """attn<T> (src/csrc/llm/attn.cpp:781-955) with isCausal for S query tokens: q [B][S][Nq][H], k / v
+    [B][Nkv][L][H] (bf16 bits; the last S keys belong to the S queries, attn.cpp:797 offset = key_len - Sq), additive
+    mask f32 [B][L] or None.  Query i sees keys 0 .. L-S+i (the reference overwrites the later scores with -1e9,
+    attn.cpp:884-900, whose exponential is exactly 0 in fp32); the rest as attn_decode: probabilities rounded to bf16
+    before they multiply V, the normaliser sums the unrounded ones, fp64 accumulation, bf16 output [B][S][Nq][H]."""
+    q = bf16_to_f32(_c(q_bf16, np.uint16)).astype(np.float64)
+    k = bf16_to_f32(_c(k_bf16, np.uint16)).astype(np.float64)
+    v = bf16_to_f32(_c(v_bf16, np.uint16)).astype(np.float64)
+    B, S, Nq, H = q.shape
+    Nkv, L = k.shape[1], k.shape[2]
+    R = Nq // Nkv
+    off = L - S
+    out = np.empty((B, S, Nq, H), np.float32)
+    for b in range(B):
+        for n in range(Nq):
+            sc = (q[b, :, n] @ k[b, n // R].T) / np.sqrt(np.float64(H))  # [S][L]
+            if mask_f32 is not None:
+                sc = sc + mask_f32[b][None, :L].astype(np.float64)
+            for i in range(S):
+                s = sc[i, : off + i + 1]
+                p_ = np.exp(s - s.max())
+                pb = _bf16_round_f32(p_.astype(np.float32)).astype(np.float64) if round_probs else p_
+                out[b, i, n] = (pb @ v[b, n // R][: off + i + 1] / p_.sum()).astype(np.float32)
+    return f32_to_bf16(out)

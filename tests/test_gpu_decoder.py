@@ -113,6 +113,66 @@ def test_attn_decode_mask():
     assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3
 
 
+def _attn_prefill(q, kc, vc, past, mask=None):
+    from tpp_pytorch_extension import _lib
+    Lb = _lib.lib()
+    B, S, Nq, H = q.shape
+    Nkv, Smax = kc.shape[1], kc.shape[2]
+    out = torch.empty_like(q)
+    _lib.check(Lb.tppx_attn_prefill(q.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                    None if mask is None else mask.data_ptr(), 0 if mask is None else mask.shape[1],
+                                    past, out.data_ptr(), B, S, Nq, Nkv, H, Smax, _lib.stream_of(q)))
+    return out
+
+
+@pytest.mark.parametrize("B,S,Nq,Nkv,past,Smax", [(1, 256, 4, 4, 0, 256), (2, 77, 8, 2, 0, 128), (2, 5, 4, 4, 100, 128),
+                                                  (1, 130, 2, 1, 63, 256), (3, 1, 4, 2, 40, 64)])
+def test_attn_prefill(B, S, Nq, Nkv, past, Smax):
+    """Causal attention for S query tokens against the oracle (tolerance as for the single-query kernel: rel-L2
+    5e-3, max-abs 2^-7 of the largest output) and against plain PyTorch fp32 causal softmax attention (1e-2)."""
+    _llm()
+    L = past + S
+    q = randn_bf16((B, S, Nq, 128), 1.0, 51)
+    k = randn_bf16((B, Nkv, Smax, 128), 1.0, 52)
+    v = randn_bf16((B, Nkv, Smax, 128), 1.0, 53)
+    got = _attn_prefill(q.cuda(), k.cuda(), v.cuda(), past)
+    ref = O.attn_prefill(t2bits(q), t2bits(k[:, :, :L]), t2bits(v[:, :, :L]))
+    g, r = bits2f(t2bits(got)).astype(np.float64), bits2f(ref).astype(np.float64)
+    assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3
+    assert np.abs(g - r).max() <= 2.0 ** -7 * np.abs(r).max()
+    kk = k[:, :, :L].float().repeat_interleave(Nq // Nkv, dim=1)
+    vv = v[:, :, :L].float().repeat_interleave(Nq // Nkv, dim=1)
+    s = torch.einsum("bsnh,bnlh->bnsl", q.float(), kk) / np.sqrt(128.0)
+    causal = torch.arange(L)[None, :] > (past + torch.arange(S))[:, None]
+    s = s.masked_fill(causal[None, None], float("-inf"))
+    t = torch.einsum("bnsl,bnlh->bsnh", torch.softmax(s, -1), vv).numpy().astype(np.float64)
+    assert np.sqrt(((g - t) ** 2).sum() / (t ** 2).sum()) <= 1e-2
+    if S == 1:  # one query: the single-query kernel's problem
+        F = _llm()
+        dec = _attn(F, q[:, 0].contiguous().cuda(), k.cuda(), v.cuda(), L)
+        d = bits2f(t2bits(dec)).astype(np.float64).reshape(g.shape)
+        assert np.sqrt(((g - d) ** 2).sum() / (d ** 2).sum()) <= 5e-3
+
+
+def test_attn_prefill_mask_and_errors():
+    F = _llm()
+    from tpp_pytorch_extension._lib import TppxError
+    B, S, Nq, Smax = 2, 70, 4, 128
+    q = randn_bf16((B, S, Nq, 128), 1.0, 61)
+    k = randn_bf16((B, Nq, Smax, 128), 1.0, 62)
+    v = randn_bf16((B, Nq, Smax, 128), 1.0, 63)
+    keep = torch.ones(B, S, dtype=torch.int64)
+    keep[0, :9] = 0  # left padding of sequence 0
+    mask = F.TppCache(Smax).align_and_invert_mask(keep.to(torch.bfloat16))
+    got = _attn_prefill(q.cuda(), k.cuda(), v.cuda(), 0, mask=mask.cuda())
+    ref = O.attn_prefill(t2bits(q), t2bits(k[:, :, :S]), t2bits(v[:, :, :S]), mask.float().numpy())
+    g, r = bits2f(t2bits(got)).astype(np.float64), bits2f(ref).astype(np.float64)
+    # rows of sequence 0 that see only padded keys are the plain average the reference also produces; compare all
+    assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3
+    with pytest.raises(TppxError):
+        _attn_prefill(q.cuda(), k.cuda(), v.cuda(), Smax - S + 1)  # does not fit the cache
+
+
 def test_decoder_layer_step_and_cache():
     """One LlamaDecoderLayer.forward on a small shape against the composition of the oracle functions, plus the
     cache bookkeeping (append position, rotated keys in the cache, reference method names)."""

@@ -340,3 +340,32 @@ def test_oracle_attn_decode_against_softmax_and_special_cases():
     keep = [i for i in range(L) if i != 3]
     dropped = O.bf16_to_f32(O.attn_decode(bits(q), bits(k[:, :, keep]), bits(v[:, :, keep]), None, round_probs=False))
     assert np.array_equal(masked, dropped)
+
+
+def test_oracle_attn_prefill_against_causal_softmax_and_decode():
+    """Pins the multi-query restatement: (i) the textbook causal softmax attention in fp64 (library routine),
+    (ii) row i equals the single-query function on the first off+i+1 keys (bit for bit: same arithmetic),
+    (iii) the first query of an empty-past prompt returns the first value row exactly."""
+    import torch
+    B, S, Nq, Nkv, past, H = 2, 7, 4, 2, 5, 16
+    L = past + S
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn(B, S, Nq, H, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Nkv, L, H, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Nkv, L, H, generator=g).to(torch.bfloat16)
+    bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
+    got = O.bf16_to_f32(O.attn_prefill(bits(q), bits(k), bits(v), None, round_probs=False))
+    kk, vv = k.double().repeat_interleave(2, 1), v.double().repeat_interleave(2, 1)
+    s = torch.einsum("bsnh,bnlh->bnsl", q.double(), kk) / np.sqrt(H)
+    causal = torch.arange(L)[None, :] > (past + torch.arange(S))[:, None]
+    s = s.masked_fill(causal[None, None], float("-inf"))
+    ref = torch.einsum("bnsl,bnlh->bsnh", torch.softmax(s, -1), vv).numpy()
+    assert np.abs(got - ref).max() <= 2.0 ** -8 * np.abs(ref).max() + 1e-6
+    m = np.zeros((B, L), np.float32); m[0, :3] = -10000.0
+    full = O.attn_prefill(bits(q), bits(k), bits(v), m)
+    for i in range(S):
+        n_keys = past + i + 1
+        one = O.attn_decode(bits(q[:, i]), bits(k[:, :, :n_keys]), bits(v[:, :, :n_keys]), m)
+        assert np.array_equal(full[:, i], one), i
+    first = O.bf16_to_f32(O.attn_prefill(bits(q), bits(k[:, :, :S]), bits(v[:, :, :S])))
+    assert np.array_equal(first[:, 0], v[:, :, 0].float().repeat_interleave(2, 1).numpy())

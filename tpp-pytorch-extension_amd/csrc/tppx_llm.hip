@@ -331,6 +331,168 @@ attn_combine_kernel(const AttnParams p) {
   p.out[(int64_t)bh * 128 + tid] = (uint16_t)f32_to_bf16_bits(Ls > 0.f ? o / Ls : 0.f);
 }
 
+// ---------------------------------------------------------------------------
+// Prompt attention: S query tokens per sequence at positions past .. past+S-1
+// over the cache [B][Nkv][Smax][128], causal (query i sees keys 0 .. past+i).
+// Grid (ceil(S/64), B*Nq); 4 waves of 16 queries each share the K and V tiles
+// of 64 keys through LDS.  Both products run on the 16x16x32 bf16 MFMA in
+// transposed form, so that no probability ever changes lanes:
+//   scores^T[key][query] = K tile (rows = keys) x Q^T      (4 MFMAs per 16 keys)
+//   out^T[dim][query]   += V^T tile (rows = dims) x P^T    (2 MFMAs per 16 dims)
+// The score tile's result layout -- lane (g, c) holds keys g*4+r of query c --
+// is, after rounding to bf16, already the second operand of the V product
+// (its 32 K slots filled with the lane's keys of two score tiles; the V^T
+// operand picks the same keys).  V is transposed on its way into LDS.
+// Online softmax per query: fp32 scores * 1/sqrt(H) + mask, running max and
+// sum, probabilities rounded to bf16 before they multiply V, sum and output
+// in fp32 (the same arithmetic as the single-query kernel above).
+// ---------------------------------------------------------------------------
+struct AttnPrefillParams {
+  const uint16_t* q;    // [B][S][Nq][128]
+  const uint16_t* kc;   // [B][Nkv][Smax][128]
+  const uint16_t* vc;
+  const uint16_t* mask; // bf16 [B][mask_ld] additive, or null
+  uint16_t* out;        // [B][S][Nq][128]
+  int B, S, Nq, Nkv, Smax, mask_ld, past;
+  float scale;
+};
+
+constexpr int AP_KP = 136; // LDS row pitch of the K tile, bf16 elements (128 + 8: rows 16-byte aligned, banks spread)
+constexpr int AP_VP = 68;  // LDS row pitch of the V^T tile (64 keys + 4: rows 8-byte aligned)
+
+__global__ void __launch_bounds__(256)
+attn_prefill_kernel(const AttnPrefillParams p) {
+  __shared__ __align__(16) uint16_t ks[64 * AP_KP];
+  __shared__ __align__(16) uint16_t vt[128 * AP_VP];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 4, c = lane & 15;
+  const int bh = blockIdx.y, b = bh / p.Nq, hq = bh - b * p.Nq;
+  const int hk = hq / (p.Nq / p.Nkv);
+  const int q0 = blockIdx.x * 64 + wave * 16;
+  const int qi = min(q0 + c, p.S - 1); // this lane's query (rows past the end repeat the last one, never stored)
+  const int qpos = p.past + qi;        // last key it sees
+  const int last_key = p.past + p.S - 1;
+
+  bf16x8 qreg[4];
+  {
+    const uint16_t* qrow = p.q + (((int64_t)b * p.S + qi) * p.Nq + hq) * 128;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      qreg[j] = *reinterpret_cast<const bf16x8*>(qrow + j * 32 + g * 8);
+  }
+  const uint16_t* kbase = p.kc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128;
+  const uint16_t* vbase = p.vc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128;
+  const uint16_t* mrow = p.mask ? p.mask + (int64_t)b * p.mask_ld : nullptr;
+
+  // staging registers: K rows chunk-fastest (coalesced), V rows key-fastest (so that the transposed 2-byte LDS
+  // writes of a wave fall into consecutive addresses)
+  i32x4 kst[4], vst[4];
+  auto load_tile = [&](int kb) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int idx = tid + i * 256;
+      const int kk = min(kb * 64 + (idx >> 4), last_key);
+      kst[i] = *reinterpret_cast<const i32x4*>(kbase + (int64_t)kk * 128 + (idx & 15) * 8);
+      const int kv = min(kb * 64 + (idx & 63), last_key);
+      vst[i] = *reinterpret_cast<const i32x4*>(vbase + (int64_t)kv * 128 + (idx >> 6) * 8);
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int idx = tid + i * 256;
+      *reinterpret_cast<i32x4*>(ks + (idx >> 4) * AP_KP + (idx & 15) * 8) = kst[i];
+      const int key = idx & 63, ch = idx >> 6;
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        vt[(ch * 8 + e) * AP_VP + key] = (uint16_t)((uint32_t)vst[i][e >> 1] >> ((e & 1) * 16));
+    }
+  };
+
+  float m = -3.0e38f, l = 0.f;
+  f32x4 acc[8];
+#pragma unroll
+  for (int dt = 0; dt < 8; dt++)
+    acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // key tiles up to the one holding the last key of the workgroup's last query (the same for all four waves)
+  const int nkb = (p.past + min((int)blockIdx.x * 64 + 63, p.S - 1)) / 64 + 1;
+  load_tile(0);
+  for (int kb = 0; kb < nkb; kb++) {
+    __syncthreads(); // the previous tile has been read by every wave
+    store_tile();
+    __syncthreads();
+    if (kb + 1 < nkb)
+      load_tile(kb + 1); // in flight during the arithmetic below
+
+    f32x4 sc[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      sc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks + (t * 16 + c) * AP_KP + j * 32 + g * 8);
+        sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[j], sc[t], 0, 0, 0);
+      }
+    }
+    float mx = -3.0e38f;
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int key = kb * 64 + t * 16 + g * 4 + r;
+        float v = sc[t][r] * p.scale;
+        if (mrow && key < p.mask_ld)
+          v += bf16_bits_to_f32(mrow[min(key, p.mask_ld - 1)]);
+        v = key <= qpos ? v : -3.0e38f;
+        sc[t][r] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float mn = fmaxf(m, mx); // finite from the first tile on: key 0 is visible to every query
+    const float alpha = __expf(m - mn);
+    l *= alpha;
+#pragma unroll
+    for (int dt = 0; dt < 8; dt++)
+      acc[dt] *= alpha;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++)
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const int t = 2 * u + (j >> 2), r = j & 3;
+        const int key = kb * 64 + t * 16 + g * 4 + r;
+        const float pr = key <= qpos ? __expf(sc[t][r] - mn) : 0.f;
+        l += pr;
+        pb[u][j] = (__bf16)pr;
+      }
+    m = mn;
+#pragma unroll
+    for (int dt = 0; dt < 8; dt++)
+#pragma unroll
+      for (int u = 0; u < 2; u++) {
+        const uint16_t* vrow = vt + (dt * 16 + c) * AP_VP + u * 32 + g * 4;
+        const uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 16);
+        i32x4 av = {(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
+        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), pb[u], acc[dt], 0, 0, 0);
+      }
+  }
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+  if (q0 + c < p.S) {
+    uint16_t* orow = p.out + (((int64_t)b * p.S + q0 + c) * p.Nq + hq) * 128;
+#pragma unroll
+    for (int dt = 0; dt < 8; dt++) {
+      uint32_t w[2];
+#pragma unroll
+      for (int h = 0; h < 2; h++)
+        w[h] = f32_to_bf16_bits(l > 0.f ? acc[dt][2 * h] / l : 0.f) |
+               (f32_to_bf16_bits(l > 0.f ? acc[dt][2 * h + 1] / l : 0.f) << 16);
+      *reinterpret_cast<uint2*>(orow + dt * 16 + g * 4) = make_uint2(w[0], w[1]);
+    }
+  }
+}
+
 } // namespace tppx
 
 using namespace tppx;
@@ -434,5 +596,31 @@ extern "C" int tppx_attn_decode(const void* q, const void* kcache, const void* v
   if (rc || splits == 1)
     return rc;
   attn_combine_kernel<<<dim3((unsigned)(B * Nq)), dim3(128), 0, (hipStream_t)stream>>>(p);
+  return check_hip(hipGetLastError(), who);
+}
+
+extern "C" int tppx_attn_prefill(const void* q, const void* kcache, const void* vcache, const void* mask,
+                                 int64_t mask_ld, int64_t past_len, void* out, int64_t B, int64_t S, int64_t Nq,
+                                 int64_t Nkv, int64_t H, int64_t Smax, tppx_stream_t stream) {
+  const char* who = "tppx_attn_prefill";
+  TPPX_REQUIRE(q && kcache && vcache && out, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(aligned16(q) && aligned16(kcache) && aligned16(vcache) && aligned16(out), TPPX_EINVAL,
+               "%s: pointer not 16-byte aligned", who);
+  TPPX_REQUIRE(H == 128, TPPX_EUNSUPPORTED, "%s: head size %ld (only 128 is built)", who, (long)H);
+  TPPX_REQUIRE(B > 0 && S > 0 && Nq > 0 && Nkv > 0 && Nq % Nkv == 0 && Smax > 0 && B * Nq < 65536 &&
+                   S < ((int64_t)1 << 24) && Smax < ((int64_t)1 << 30),
+               TPPX_ESHAPE, "%s: bad shape B=%ld S=%ld Nq=%ld Nkv=%ld Smax=%ld", who, (long)B, (long)S, (long)Nq,
+               (long)Nkv, (long)Smax);
+  TPPX_REQUIRE(past_len >= 0 && past_len + S <= Smax, TPPX_ESHAPE,
+               "%s: %ld cached + %ld new keys exceed the cache capacity %ld", who, (long)past_len, (long)S, (long)Smax);
+  TPPX_REQUIRE(!mask || mask_ld > 0, TPPX_EINVAL, "%s: mask given with mask_ld=%ld", who, (long)mask_ld);
+  AttnPrefillParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = (const uint16_t*)q; p.kc = (const uint16_t*)kcache; p.vc = (const uint16_t*)vcache;
+  p.mask = (const uint16_t*)mask; p.out = (uint16_t*)out;
+  p.B = (int)B; p.S = (int)S; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.Smax = (int)Smax; p.mask_ld = (int)mask_ld;
+  p.past = (int)past_len;
+  p.scale = 1.0f / sqrtf((float)H);
+  attn_prefill_kernel<<<dim3((unsigned)((S + 63) / 64), (unsigned)(B * Nq)), dim3(256), 0, (hipStream_t)stream>>>(p);
   return check_hip(hipGetLastError(), who);
 }
