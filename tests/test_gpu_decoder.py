@@ -230,7 +230,88 @@ def test_decoder_layer_step_and_cache():
     assert_close_bf16(t2bits(vc[:, :, ctx]), v.reshape(B, Nkv, H), what="cached value")
     assert torch.equal(kc[:, :, :ctx].cpu(), k0)
     with pytest.raises(Exception):
-        layer.forward([x.repeat(1, 2, 1).cuda(), None, pos.cuda()], cache, True)  # more than one query token
+        layer.forward([x.repeat(1, 2, 1).cuda(), None, pos.cuda()], cache, True)  # two tokens, one position each
+
+
+@pytest.mark.parametrize("past,S", [(0, 70), (37, 9)])
+def test_decoder_layer_prompt(past, S):
+    """LlamaDecoderLayer.forward on S tokens per sequence (prompt processing, with and without cached keys)
+    against the composition of the oracle functions; the S rotated keys and the values land in the cache."""
+    F = _llm()
+    from tpp_pytorch_extension import _ops
+    hidden, inter, Nq, Nkv, H, MP = 512, 1024, 4, 2, 128, 256
+    B, cap = 2, 128
+    rng = torch.Generator().manual_seed(15)
+
+    def lin(N, K, seed):
+        W = randn_bf16((N, K), 0.05, seed)
+        return W, _ops.remap_and_quantize_mxfp4(block_bf16(W).cuda()), O.remap_quantize_mxfp4(W.float().numpy())
+
+    Ws = [lin(Nq * H, hidden, 151), lin(Nkv * H, hidden, 152), lin(Nkv * H, hidden, 153), lin(hidden, Nq * H, 154),
+          lin(inter, hidden, 155), lin(inter, hidden, 156), lin(hidden, inter, 157)]
+    g1 = torch.rand(hidden, generator=rng) + 0.5
+    g2 = torch.rand(hidden, generator=rng) + 0.5
+    EP = F.llama_rotary_table(MP, H, device="cpu")
+    layer = F.LlamaDecoderLayer([g1.cuda(), Ws[0][1], Ws[1][1], Ws[2][1], Ws[3][1], g2.cuda(), Ws[4][1], Ws[5][1],
+                                 Ws[6][1], EP.cuda()], 0, 1e-5, H, MP, H)
+    cache = F.TppCache(cap)
+    k0, v0 = randn_bf16((B, Nkv, past, H), 1.0, 161), randn_bf16((B, Nkv, past, H), 1.0, 162)
+    if past:
+        cache.fill_(0, k0.cuda(), v0.cuda())
+    x = randn_bf16((B, S, hidden), 1.0, 163)
+    pos = torch.arange(past, past + S, dtype=torch.int64).unsqueeze(0)
+    out = layer.forward([x.cuda(), None, pos.cuda()], cache, True)[0]
+    cache.advance(S)
+    assert out.shape == (B, S, hidden) and cache.get_seq_length() == past + S
+
+    def mm(a_bits, w, post=O.POST_NONE, post_in=None):
+        return O.linear_mxfp4(a_bits, w[2][0], w[2][1], None, post, post_in, None, 1.0, O.MODE_IDEAL)
+
+    xb = t2bits(x).reshape(B * S, hidden)
+    h = O.rms_norm(xb, g1.numpy(), 1e-5)
+    q, k, v = mm(h, Ws[0]), mm(h, Ws[1]), mm(h, Ws[2])
+    q = O.rotary_llama(q.reshape(B, S, -1), EP.numpy(), pos.numpy(), Nq, H).reshape(B, S, Nq, H)
+    k = O.rotary_llama(k.reshape(B, S, -1), EP.numpy(), pos.numpy(), Nkv, H).reshape(B, S, Nkv, H).transpose(0, 2, 1, 3)
+    v = v.reshape(B, S, Nkv, H).transpose(0, 2, 1, 3)
+    kall = np.concatenate([t2bits(k0), k], axis=2)
+    vall = np.concatenate([t2bits(v0), v], axis=2)
+    ctxv = O.attn_prefill(q, kall, vall).reshape(B * S, Nq * H)
+    so = mm(ctxv, Ws[3], O.POST_ADD_SCALE, xb)
+    h2 = O.rms_norm(so, g2.numpy(), 1e-5)
+    gate = mm(h2, Ws[4], O.POST_SILU)
+    ref = mm(mm(h2, Ws[5], O.POST_MUL, gate), Ws[6], O.POST_ADD_SCALE, so)
+    g, r = bits2f(t2bits(out)).reshape(B * S, hidden).astype(np.float64), bits2f(ref).astype(np.float64)
+    rel = np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum())
+    assert rel <= 2e-2, rel
+    kc, vc = cache.get(0)
+    assert_close_bf16(t2bits(kc[:, :, past:]), np.ascontiguousarray(k), what="cached keys")
+    assert_close_bf16(t2bits(vc[:, :, past:]), np.ascontiguousarray(v), what="cached values")
+    if past:
+        assert torch.equal(kc[:, :, :past].cpu(), k0)
+
+
+def test_generate_prompt_then_decode():
+    """Prompt in one pass + decode steps: the first generated token equals the one obtained by feeding the prompt
+    token by token through the decode step (same keys in the cache up to rounding, same argmax on this seed), and
+    the graph and eager decode loops agree after a prompt."""
+    F = _llm()
+    model = F.LlamaDecoder(hidden=512, inter=1024, n_layers=2, n_heads=4, n_kv_heads=2, vocab=1024,
+                           max_positions=256, seed=4)
+    prompt = torch.randint(0, 1024, (3, 21), generator=torch.Generator().manual_seed(9)).cuda()
+    a = model.generate(prompt, 6, use_graph=True)
+    b = model.generate(prompt, 6, use_graph=False)
+    assert a.shape == (3, 6) and torch.equal(a, b)
+    # token by token
+    cache = F.TppCache(64)
+    for t in range(prompt.shape[1]):
+        pos = torch.full((3, 1), t, dtype=torch.int64, device="cuda")
+        nxt = model.step(prompt[:, t].contiguous(), pos, cache)
+        cache.advance(1)
+    c2 = F.TppCache(64)
+    model.prefill(prompt, c2)
+    k1, k2 = cache.get(1)[0].float(), c2.get(1)[0].float()
+    assert ((k1 - k2).norm() / k1.norm()).item() <= 2e-2
+    assert torch.equal(nxt, a[:, 0])
 
 
 def test_greedy_decode_graph_equals_eager():

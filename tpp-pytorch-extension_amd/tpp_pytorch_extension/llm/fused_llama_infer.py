@@ -123,12 +123,19 @@ class LlamaDecoderLayer:
         self.Nkv = _ops._as_q(self.t_Wk).weight_nk()[0] // self.H
 
     def forward(self, inputs, cache, use_cache=True):
-        """inputs = [hidden [B][1][hidden], additive mask [B][keys] or empty, position_ids i64 [B or 1][1]]."""
+        """inputs = [hidden [B][S][hidden], additive mask [B][keys] or empty, position_ids i64 [B or 1][S]].
+        S = 1 is the decode step (cache length read from the device counter, so the call can be replayed in a
+        graph); S > 1 processes a prompt or several new tokens causally on top of the cached keys.  The S new keys
+        go to cache positions get_seq_length() .. +S-1; the caller advances the cache once all layers have run."""
         L = _lib.lib()
         t_HS, t_am, t_pid = inputs[0], inputs[1], inputs[2]
         B, S, hidden = t_HS.shape
-        if S != 1:
-            raise TppxError(_lib.EUNSUPPORTED, "LlamaDecoderLayer: only the decode step (one token per sequence) is built")
+        if cache.get_seq_length() + S > cache.capacity:
+            raise TppxError(_lib.ESHAPE, f"LlamaDecoderLayer: {cache.get_seq_length()} cached + {S} new keys exceed "
+                                         f"the cache capacity {cache.capacity}")
+        if t_pid.dim() != 2 or t_pid.shape[1] != S or t_pid.shape[0] not in (1, B) or t_pid.dtype != torch.int64:
+            raise TppxError(_lib.ESHAPE, f"LlamaDecoderLayer: position_ids must be int64 [B or 1][S={S}], got "
+                                         f"{tuple(t_pid.shape)} {t_pid.dtype}")
         st = _lib.stream_of(t_HS)
         empty = torch.empty(0, dtype=torch.bfloat16, device=t_HS.device)
         t_res = t_HS
@@ -138,16 +145,21 @@ class LlamaDecoderLayer:
         # rotary on q and k + append of k, v at position seq_len (device counter), one launch
         _lib.check(L.tppx_rotary_kv_append_llama(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), self.t_EP.data_ptr(), t_pid.data_ptr(), kc.data_ptr(),
-            vc.data_ptr(), cache.seq_len_dev.data_ptr(), B, 1, self.Nq, self.Nkv, self.H, self.t_EP.shape[1],
+            vc.data_ptr(), cache.seq_len_dev.data_ptr(), B, S, self.Nq, self.Nkv, self.H, self.t_EP.shape[1],
             self.t_EP.shape[2], t_pid.shape[0], cache.capacity, st))
-        # attention over seq_len + 1 keys
+        # attention over the cached keys + the new ones
         ctx = torch.empty_like(q)
         ws = _lib.workspace(t_HS)
         mask_ptr = t_am.data_ptr() if t_am is not None and t_am.numel() else None
         mask_ld = t_am.shape[-1] if mask_ptr else 0
-        _lib.check(L.tppx_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
-                                      cache.seq_len_dev.data_ptr(), 1, ctx.data_ptr(), B, self.Nq, self.Nkv, self.H,
-                                      cache.capacity, ws.data_ptr(), ws.numel(), st))
+        if S == 1:
+            _lib.check(L.tppx_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
+                                          cache.seq_len_dev.data_ptr(), 1, ctx.data_ptr(), B, self.Nq, self.Nkv, self.H,
+                                          cache.capacity, ws.data_ptr(), ws.numel(), st))
+        else:
+            _lib.check(L.tppx_attn_prefill(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
+                                           cache.get_seq_length(), ctx.data_ptr(), B, S, self.Nq, self.Nkv, self.H,
+                                           cache.capacity, st))
         t_SO = _ops.fc_add(ctx, self.t_Wp, empty, t_res, 1.0)
         # post-attention RMSNorm + gate/up GEMMs + silu*mul
         t_I = _ops.swiglu_gate_up(t_SO, self.t_Wg, self.t_Wu, norm=(self.t_Gpa, self.eps))
@@ -216,6 +228,31 @@ class LlamaDecoder:
         h = rms_norm(h, self.norm_w, self.eps)
         logits = _ops.fc_plain(h, self.lm_head, None)
         return logits.view(logits.shape[0], -1).argmax(dim=-1)
+
+    def prefill(self, prompt, cache, mask=None):
+        """prompt i64 [B][S] (device) on top of whatever the cache holds -> next tokens i64 [B]; advances the cache
+        by S.  mask: additive bf16 [B][keys] over cache positions (TppCache.align_and_invert_mask) or None."""
+        B, S = prompt.shape
+        past = cache.get_seq_length()
+        pos = torch.arange(past, past + S, dtype=torch.int64, device=self.device).unsqueeze(0)
+        h = self.embed.index_select(0, prompt.reshape(-1)).view(B, S, self.hidden)
+        for layer in self.layers:
+            h = layer.forward([h, mask, pos], cache)[0]
+        cache.advance(S)
+        h = rms_norm(h[:, -1:].contiguous(), self.norm_w, self.eps)  # only the last position feeds the lm_head
+        logits = _ops.fc_plain(h, self.lm_head, None)
+        return logits.view(B, -1).argmax(dim=-1)
+
+    def generate(self, prompt, n_new, capacity=None, use_graph=True):
+        """Greedy generation as run_generation.py drives it: the prompt in one pass, then one token per step.
+        Returns i64 [B][n_new]."""
+        B, S = prompt.shape
+        cache = TppCache(capacity or S + n_new + 32)
+        first = self.prefill(prompt, cache)
+        if n_new == 1:
+            return first.view(B, 1)
+        rest = self.greedy_decode(first, cache, n_new - 1, use_graph=use_graph)
+        return torch.cat([first.view(B, 1), rest], dim=1)
 
     def time_decode_steps(self, tokens, cache, n_new):
         """Seconds spent in n_new replays of the captured decode step (capture excluded)."""
