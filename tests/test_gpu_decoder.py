@@ -360,3 +360,57 @@ def test_rms_norm_fused_into_gemms(M, K, monkeypatch):
     seg[0].qw, seg[0].sw, seg[0].y, seg[0].N, seg[0].post_op, seg[0].post_scale = qn.data_ptr(), sn.data_ptr(), y.data_ptr(), Ns[0], 0, 1.0
     _lib.check(L.tppx_norm_multi_linear_mxfp4(h.data_ptr(), None, 0.0, seg, 1, M, K, 0, _lib.stream_of(h)))
     assert_close_bf16(t2bits(y), t2bits(sep[0]), what="LDS-staged plain GEMM")
+
+
+def test_optimize_model_for_llama_against_transformers():
+    """OptimizeModelForLlama on a random-initialised transformers LlamaForCausalLM (2 layers, GQA 4/2 heads of
+    128): the logits of the prompt pass and of two decode steps against the stock transformers model in fp32 on
+    the CPU holding the *dequantized* MXFP4 weights (exactly representable), i.e. the same function up to the
+    bf16 roundings of the fused path.  Left padding goes through the additive key mask."""
+    transformers = pytest.importorskip("transformers")
+    import copy
+    F = _llm()
+    cfg = transformers.LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4,
+                                   num_key_value_heads=2, vocab_size=1024, max_position_embeddings=256, head_dim=128,
+                                   rms_norm_eps=1e-5, attn_implementation="eager")
+    torch.manual_seed(11)
+    ref_model = transformers.LlamaForCausalLM(cfg).eval()
+    with torch.no_grad():
+        for m in ref_model.modules():
+            if isinstance(m, torch.nn.Linear):  # weights := dequantize(quantize(weights)), as the fused model sees them
+                w = m.weight.data.to(torch.bfloat16).float()
+                q, sc = O.remap_quantize_mxfp4(w.numpy())
+                m.weight.data.copy_(torch.from_numpy(O.dequantize_mxfp4_plain(q, sc)))
+            elif isinstance(m, torch.nn.Embedding):
+                m.weight.data.copy_(m.weight.data.to(torch.bfloat16).float())
+    opt_model = F.OptimizeModelForLlama(copy.deepcopy(ref_model), torch.bfloat16, "cuda", "mxfp4").eval()
+
+    ids = torch.randint(0, 1024, (2, 19), generator=torch.Generator().manual_seed(12))
+    am = torch.ones_like(ids)
+    am[1, :4] = 0  # left padding of sequence 1
+    pos = (am.cumsum(-1) - 1).clamp(min=0)
+
+    def rel(a, b):
+        a, b = a.double(), b.double()
+        return float(((a - b).norm() / b.norm()))
+
+    with torch.no_grad():
+        r = ref_model(input_ids=ids, attention_mask=am, position_ids=pos, use_cache=True)
+        o = opt_model(input_ids=ids.cuda(), attention_mask=am.cuda(), position_ids=pos.cuda(), use_cache=True)
+        assert o.logits.shape == r.logits.shape
+        # padded positions of sequence 1 are arbitrary in both models; compare the real ones
+        assert rel(o.logits[0].float().cpu(), r.logits[0]) <= 3e-2
+        assert rel(o.logits[1, 4:].float().cpu(), r.logits[1, 4:]) <= 3e-2
+        cache_o, cache_r = o.past_key_values, r.past_key_values
+        assert cache_o.get_seq_length() == 19 and len(cache_o) == 2
+        for step in range(2):
+            nxt = r.logits[:, -1].argmax(-1, keepdim=True)
+            am = torch.cat([am, torch.ones(2, 1, dtype=am.dtype)], 1)
+            pos = pos[:, -1:] + 1
+            r = ref_model(input_ids=nxt, attention_mask=am, position_ids=pos, past_key_values=cache_r, use_cache=True)
+            o = opt_model(input_ids=nxt.cuda(), attention_mask=am.cuda(), position_ids=pos.cuda(),
+                          past_key_values=cache_o, use_cache=True)
+            assert rel(o.logits.float().cpu(), r.logits) <= 3e-2
+        assert cache_o.get_seq_length() == 21
+    out = F.generate_greedy(opt_model, ids[:1].cuda(), 5)
+    assert out.shape == (1, 24) and torch.equal(out[:, :19].cpu(), ids[:1])

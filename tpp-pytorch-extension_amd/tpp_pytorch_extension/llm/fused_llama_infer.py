@@ -1,16 +1,21 @@
 """Llama decoder layer on the GPU: the reference's fused decoder block
 (`LlamaDecoderLayer::_forward`, src/csrc/llm/fused_llm_infer.cpp:1195-1286) and
 its KV cache (`TppCache` / `LayerCache`, src/csrc/llm/attn.h:164-404) for the
-decode step (one new token per sequence), built from the quantized linears and
-the decode-side kernels of libtppx_hip.so.
+decode step (one new token per sequence) and for prompt processing, built from
+the quantized linears and the decoder-side kernels of libtppx_hip.so.
 
 `LlamaDecoderLayer` keeps the constructor and `forward` signature of
 `torch.classes.tpp_llm.LlamaDecoderLayer` (fused_llm_infer.cpp:1084-1110,
-1186-1192, 1603-1606); `TppCache` keeps the reference's method names.  Prompt
-processing (more than one query token per sequence) is not built: the cache is
-filled with `TppCache.fill_` or token by token.
+1186-1192, 1603-1606); `TppCache` keeps the reference's method names.
+
+`OptimizeModelForLlama` / `FixLlamaDecoderLayer` / `LlamaModel_forward` are the
+front-end of src/tpp_pytorch_extension/llm/fused_llama_infer.py:104-336 for a
+Hugging Face `LlamaForCausalLM`: every decoder layer is replaced by one
+`LlamaDecoderLayer` call, the model's forward runs on a `TppCache`.
 """
 import math
+import os
+import types
 
 import torch
 
@@ -303,3 +308,140 @@ class LlamaDecoder:
                 pos.add_(1)
                 cache.advance(1)
         return out
+
+
+# ---------------------------------------------------------------------------
+# Hugging Face front-end (src/tpp_pytorch_extension/llm/fused_llama_infer.py:45-336)
+# ---------------------------------------------------------------------------
+class LlamaDecoderLayerModule(torch.nn.Module):
+    """What a transformers LlamaDecoderLayer becomes (fused_llama_infer.py:45-101): the module keeps its
+    sub-modules (quantized in place) and forwards through `cpp_block`, one LlamaDecoderLayer of this file."""
+
+    def forward(self, hidden_states, attention_mask=None, position_ids=None, past_key_values=None, use_cache=False,
+                past_key_value=None, **kwargs):
+        if not hasattr(self, "cpp_block"):
+            raise ValueError("cpp_block is not initialized")
+        if position_ids is None:
+            raise ValueError("position_ids is required")
+        cache = past_key_values if past_key_values is not None else past_key_value
+        if cache is None:
+            raise ValueError("the optimized decoder layer needs a TppCache (past_key_values)")
+        core = cache.get_cpp() if hasattr(cache, "get_cpp") else cache
+        hs = hidden_states.to(torch.bfloat16).contiguous()
+        mask = attention_mask.to(torch.bfloat16).contiguous() if attention_mask is not None else None
+        return self.cpp_block.forward([hs, mask, position_ids.contiguous()], core, use_cache)[0]
+
+
+def FixLlamaDecoderLayer(self, bk=None, bc=None, layer_dtype=torch.bfloat16, weight_dtype="mxfp4",
+                         embed_positions=None):
+    """fused_llama_infer.py:104-173: quantize the seven linears of a transformers LlamaDecoderLayer in place
+    (FixLinear with [bk, bc] blocking) and attach the fused block."""
+    import transformers
+    from .llm_common import FixLinear
+    if not isinstance(self, transformers.models.llama.modeling_llama.LlamaDecoderLayer):
+        return
+    self.__class__ = LlamaDecoderLayerModule
+    self.features_block_size = bc
+    self.layer_dtype = layer_dtype
+    self.model_parallel = False
+    for m in self.modules():
+        if isinstance(m, torch.nn.Linear):
+            if m.bias is not None:
+                raise NotImplementedError("attention_bias / mlp_bias are not supported for Llama")
+            FixLinear(m, bk, bc, layer_dtype, weight_dtype=weight_dtype)
+    if not hasattr(self, "cpp_block"):
+        at, mlp = self.self_attn, self.mlp
+        params = [self.input_layernorm.weight.data.float(), at.q_proj.weight, at.k_proj.weight, at.v_proj.weight,
+                  at.o_proj.weight, self.post_attention_layernorm.weight.data.float(), mlp.gate_proj.weight,
+                  mlp.up_proj.weight, mlp.down_proj.weight, embed_positions]
+        self.cpp_block = LlamaDecoderLayer(params, at.layer_idx, self.input_layernorm.variance_epsilon, at.head_dim,
+                                           embed_positions.shape[1], at.head_dim)
+
+
+def LlamaModel_forward(self, input_ids=None, attention_mask=None, position_ids=None, past_key_values=None,
+                       inputs_embeds=None, use_cache=None, cache_position=None, **kwargs):
+    """fused_llama_infer.py:228-336: embeddings, position ids from the cache length, additive key mask from the
+    0/1 attention mask, the decoder layers on a TppCache, final norm."""
+    from transformers.modeling_outputs import BaseModelOutputWithPast
+    from .llm_common import TppCache as HFTppCache
+    if (input_ids is None) == (inputs_embeds is None):
+        raise ValueError("You cannot specify both input_ids and inputs_embeds at the same time, and must specify either one")
+    if inputs_embeds is None:
+        inputs_embeds = self.embed_tokens(input_ids)
+    if not isinstance(past_key_values, HFTppCache):
+        if past_key_values is None or past_key_values.get_seq_length() == 0:
+            past_key_values = HFTppCache(capacity=self._tpp_kv_capacity)
+        else:
+            raise ValueError("past_key_values must be of TppCache type")
+    past_seen = past_key_values.get_seq_length()
+    S = inputs_embeds.shape[1]
+    if cache_position is None:
+        cache_position = torch.arange(past_seen, past_seen + S, device=inputs_embeds.device)
+    if position_ids is None:
+        position_ids = cache_position.unsqueeze(0)
+    mask = None if attention_mask is None else past_key_values.align_and_invert_mask(attention_mask, inputs_embeds)
+    hidden_states = inputs_embeds.to(torch.bfloat16)
+    for layer in self.layers[: self.config.num_hidden_layers]:
+        hidden_states = layer(hidden_states, attention_mask=mask, position_ids=position_ids,
+                              past_key_values=past_key_values, use_cache=True)
+    past_key_values.get_cpp().advance(S)
+    hidden_states = rms_norm(hidden_states, self._tpp_norm_weight, self._tpp_norm_eps)
+    return BaseModelOutputWithPast(last_hidden_state=hidden_states, past_key_values=past_key_values)
+
+
+def OptimizeModelForLlama(model, dtype=torch.bfloat16, device="cuda", weight_dtype="mxfp4"):
+    """fused_llama_infer.py:176-226 for one GPU: the rotary table from the model's own rotary_emb, every
+    LlamaDecoderLayer fused, every remaining nn.Linear (the lm_head) turned into a BlockedLinear, LlamaModel.forward
+    of this instance replaced.  Differences: the linears must be quantized (weight_dtype "mxfp4" or "qint8"; the
+    reference keeps the lm_head in bf16 unless asked to quantize it) and the KV cache is allocated for
+    TPPX_KV_CAPACITY keys per sequence (default: the model's max_position_embeddings)."""
+    import transformers
+    from .llm_common import FixLinear
+    if weight_dtype not in ("mxfp4", "qint8"):
+        raise TppxError(_lib.EUNSUPPORTED, f"OptimizeModelForLlama: weight_dtype {weight_dtype!r} (only quantized linears are built)")
+    if getattr(model.config, "attention_bias", False):
+        raise NotImplementedError("attention_bias is not supported for Llama yet!")
+    model.config._attn_implementation = "tpp"
+    embed_positions = None
+    for m in model.modules():
+        if isinstance(m, transformers.models.llama.modeling_llama.LlamaPreTrainedModel) and hasattr(m, "rotary_emb"):
+            # before the model is cast: the rotary module's frequencies are still fp32
+            mp = m.rotary_emb.config.max_position_embeddings
+            where = m.rotary_emb.inv_freq.device
+            cs = m.rotary_emb(torch.empty([1], dtype=torch.float, device=where), torch.arange(mp, device=where).unsqueeze(0))
+            embed_positions = torch.cat(cs, dim=0).view([2, mp, -1]).to(torch.float).to(device).contiguous()
+            break
+    if embed_positions is None:
+        raise NotImplementedError("Unable to create embed_positions")
+    model.to(device=device, dtype=dtype)
+    with torch.no_grad():
+        for m in list(model.modules()):
+            if isinstance(m, transformers.models.llama.modeling_llama.LlamaDecoderLayer):
+                FixLlamaDecoderLayer(m, 16, 64, dtype, weight_dtype, embed_positions)
+        for m in list(model.modules()):
+            if isinstance(m, torch.nn.Linear) and m.weight.shape[0] % 32 == 0 and m.weight.shape[1] % 64 == 0:
+                FixLinear(m, 16, 64, dtype, weight_dtype=weight_dtype)  # no-op for the ones fixed above
+    for m in model.modules():
+        if isinstance(m, transformers.models.llama.modeling_llama.LlamaModel):
+            m._tpp_kv_capacity = int(os.environ.get("TPPX_KV_CAPACITY", embed_positions.shape[1]))
+            m._tpp_norm_weight = m.norm.weight.data.float().contiguous()
+            m._tpp_norm_eps = m.norm.variance_epsilon
+            m.forward = types.MethodType(LlamaModel_forward, m)
+    return model
+
+
+def generate_greedy(model, input_ids, max_new_tokens, attention_mask=None):
+    """Greedy loop over an optimized LlamaForCausalLM as run_generation.py drives generate(): the prompt in one
+    forward, then one token per forward on the same TppCache.  Returns i64 [B][S + max_new_tokens]."""
+    ids = input_ids
+    cache = None
+    cur = input_ids
+    for _ in range(max_new_tokens):
+        out = model(input_ids=cur, attention_mask=attention_mask, past_key_values=cache, use_cache=True,
+                    logits_to_keep=1)
+        cache = out.past_key_values
+        cur = out.logits[:, -1].argmax(dim=-1, keepdim=True)
+        ids = torch.cat([ids, cur], dim=1)
+        if attention_mask is not None:
+            attention_mask = torch.cat([attention_mask, attention_mask.new_ones((ids.shape[0], 1))], dim=1)
+    return ids

@@ -1,9 +1,10 @@
 """LLM-side module API of the quantized linear.
 
 Reference: ``src/tpp_pytorch_extension/llm/llm_common.py`` -- ``fc_plain``
-(:379), ``BlockedLinear`` (:383-434) and ``FixLinear`` (:437-515).  The
-generation wrapper, KV cache and tensor-parallel sharding of that file are
-outside the path built here.
+(:379), ``BlockedLinear`` (:383-434), ``FixLinear`` (:437-515) and the
+``TppCache`` wrapper handed around as ``past_key_values`` (:80-182).  The
+generation wrapper and tensor-parallel sharding of that file are outside the
+path built here.
 """
 import torch
 
@@ -113,3 +114,54 @@ def FixLinear(self, bk=None, bc=None, layer_dtype=global_layer_dtype, parallel_d
             self.weight = torch.nn.Parameter(self.weight.data.to(weight_dtype), requires_grad=False)
         if self.bias is not None and isinstance(weight_dtype, str):
             self.bias = torch.nn.Parameter(self.bias.data.to(torch.bfloat16), requires_grad=False)
+
+
+class TppCache:
+    """past_key_values object of the optimized models (llm_common.py:80-182): a thin wrapper around the cache the
+    fused decoder layers append to (`get_cpp()`).  Keys are appended inside the layers, so `update` is not a
+    way in; beam reordering is not built."""
+
+    def __init__(self, capacity=0, **kwargs):
+        from .fused_llama_infer import TppCache as _CoreCache
+        self.tpp_cache = _CoreCache(capacity)
+
+    def __len__(self):
+        return self.tpp_cache.size()
+
+    def __getitem__(self, layer_idx):
+        raise NotImplementedError
+
+    def __iter__(self):
+        raise NotImplementedError
+
+    def update(self, key_states, value_states, layer_idx, cache_kwargs=None):
+        raise NotImplementedError("the fused decoder layer appends keys and values itself")
+
+    def get_seq_length(self, layer_idx=0):
+        return self.tpp_cache.get_seq_length(layer_idx)
+
+    def get_max_length(self):
+        return self.tpp_cache.get_capacity()
+
+    def crop(self, max_length):
+        seq_len = self.get_seq_length()
+        if max_length < 0:
+            max_length = seq_len - abs(max_length)
+        if seq_len > max_length:
+            self.tpp_cache.crop(max_length)
+
+    def align_and_invert_mask(self, mask, inputs_embeds):
+        if mask is None:
+            mask = torch.ones((inputs_embeds.shape[0], inputs_embeds.shape[1]), device=inputs_embeds.device,
+                              dtype=torch.bfloat16)
+        return self.tpp_cache.align_and_invert_mask(mask.to(torch.bfloat16), torch.finfo(torch.bfloat16).min)
+
+    def reorder_cache(self, beam_idx):
+        raise NotImplementedError("beam search is not part of the single-GPU decode path")
+
+    def get_cpp(self):
+        return self.tpp_cache
+
+
+def generate_past_key_values(model, batch_size, seq_len, num_beams=1):
+    return TppCache(capacity=seq_len)
