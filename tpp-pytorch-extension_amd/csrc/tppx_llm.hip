@@ -360,25 +360,33 @@ struct AttnPrefillParams {
 constexpr int AP_KP = 136; // LDS row pitch of the K tile, bf16 elements (128 + 8: rows 16-byte aligned, banks spread)
 constexpr int AP_VP = 68;  // LDS row pitch of the V^T tile (64 keys + 4: rows 8-byte aligned)
 
+// QG = query groups of 16 per wave: every K / V^T operand read from LDS feeds QG MFMAs (with one group the LDS
+// reads, 32 KB per wave and key tile, take twice the cycles of the 32 MFMAs they feed).
+template <int QG>
 __global__ void __launch_bounds__(256)
 attn_prefill_kernel(const AttnPrefillParams p) {
   __shared__ __align__(16) uint16_t ks[64 * AP_KP];
   __shared__ __align__(16) uint16_t vt[128 * AP_VP];
+  constexpr int QB = 64 * QG; // queries per workgroup
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 4, c = lane & 15;
   const int bh = blockIdx.y, b = bh / p.Nq, hq = bh - b * p.Nq;
   const int hk = hq / (p.Nq / p.Nkv);
-  const int q0 = blockIdx.x * 64 + wave * 16;
-  const int qi = min(q0 + c, p.S - 1); // this lane's query (rows past the end repeat the last one, never stored)
-  const int qpos = p.past + qi;        // last key it sees
+  // the last query blocks see the most keys: start them first
+  const int qblk = (int)gridDim.x - 1 - (int)blockIdx.x;
+  const int q0 = qblk * QB + wave * (16 * QG);
   const int last_key = p.past + p.S - 1;
 
-  bf16x8 qreg[4];
-  {
+  int qpos[QG]; // last key this lane's query of group qg sees (rows past the end repeat the last query, never stored)
+  bf16x8 qreg[QG][4];
+#pragma unroll
+  for (int qg = 0; qg < QG; qg++) {
+    const int qi = min(q0 + qg * 16 + c, p.S - 1);
+    qpos[qg] = p.past + qi;
     const uint16_t* qrow = p.q + (((int64_t)b * p.S + qi) * p.Nq + hq) * 128;
 #pragma unroll
     for (int j = 0; j < 4; j++)
-      qreg[j] = *reinterpret_cast<const bf16x8*>(qrow + j * 32 + g * 8);
+      qreg[qg][j] = *reinterpret_cast<const bf16x8*>(qrow + j * 32 + g * 8);
   }
   const uint16_t* kbase = p.kc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128;
   const uint16_t* vbase = p.vc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128;
@@ -409,13 +417,18 @@ attn_prefill_kernel(const AttnPrefillParams p) {
     }
   };
 
-  float m = -3.0e38f, l = 0.f;
-  f32x4 acc[8];
+  float m[QG], l[QG];
+  f32x4 acc[QG][8];
 #pragma unroll
-  for (int dt = 0; dt < 8; dt++)
-    acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int qg = 0; qg < QG; qg++) {
+    m[qg] = -3.0e38f;
+    l[qg] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < 8; dt++)
+      acc[qg][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
   // key tiles up to the one holding the last key of the workgroup's last query (the same for all four waves)
-  const int nkb = (p.past + min((int)blockIdx.x * 64 + 63, p.S - 1)) / 64 + 1;
+  const int nkb = (p.past + min(qblk * QB + QB - 1, p.S - 1)) / 64 + 1;
   load_tile(0);
   for (int kb = 0; kb < nkb; kb++) {
     __syncthreads(); // the previous tile has been read by every wave
@@ -424,71 +437,90 @@ attn_prefill_kernel(const AttnPrefillParams p) {
     if (kb + 1 < nkb)
       load_tile(kb + 1); // in flight during the arithmetic below
 
-    f32x4 sc[4];
+    f32x4 sc[QG][4];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
-      sc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int qg = 0; qg < QG; qg++)
+        sc[qg][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks + (t * 16 + c) * AP_KP + j * 32 + g * 8);
-        sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[j], sc[t], 0, 0, 0);
+#pragma unroll
+        for (int qg = 0; qg < QG; qg++)
+          sc[qg][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[qg][j], sc[qg][t], 0, 0, 0);
       }
     }
-    float mx = -3.0e38f;
+    float mk[16]; // additive mask of this lane's 16 keys
 #pragma unroll
-    for (int t = 0; t < 4; t++)
+    for (int i = 0; i < 16; i++) {
+      const int key = kb * 64 + (i >> 2) * 16 + g * 4 + (i & 3);
+      mk[i] = (mrow && key < p.mask_ld) ? bf16_bits_to_f32(mrow[key]) : 0.f;
+    }
+    bf16x8 pb[QG][2];
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int key = kb * 64 + t * 16 + g * 4 + r;
-        float v = sc[t][r] * p.scale;
-        if (mrow && key < p.mask_ld)
-          v += bf16_bits_to_f32(mrow[min(key, p.mask_ld - 1)]);
-        v = key <= qpos ? v : -3.0e38f;
-        sc[t][r] = v;
-        mx = fmaxf(mx, v);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float mn = fmaxf(m, mx); // finite from the first tile on: key 0 is visible to every query
-    const float alpha = __expf(m - mn);
-    l *= alpha;
+    for (int qg = 0; qg < QG; qg++) {
+      float mx = -3.0e38f;
 #pragma unroll
-    for (int dt = 0; dt < 8; dt++)
-      acc[dt] *= alpha;
-    bf16x8 pb[2];
+      for (int t = 0; t < 4; t++)
 #pragma unroll
-    for (int u = 0; u < 2; u++)
+        for (int r = 0; r < 4; r++) {
+          const int key = kb * 64 + t * 16 + g * 4 + r;
+          const float v = key <= qpos[qg] ? sc[qg][t][r] * p.scale + mk[t * 4 + r] : -3.0e38f;
+          sc[qg][t][r] = v;
+          mx = fmaxf(mx, v);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float mn = fmaxf(m[qg], mx); // finite from the first tile on: key 0 is visible to every query
+      const float alpha = __expf(m[qg] - mn);
+      l[qg] *= alpha;
 #pragma unroll
-      for (int j = 0; j < 8; j++) {
-        const int t = 2 * u + (j >> 2), r = j & 3;
-        const int key = kb * 64 + t * 16 + g * 4 + r;
-        const float pr = key <= qpos ? __expf(sc[t][r] - mn) : 0.f;
-        l += pr;
-        pb[u][j] = (__bf16)pr;
-      }
-    m = mn;
+      for (int dt = 0; dt < 8; dt++)
+        acc[qg][dt] *= alpha;
+#pragma unroll
+      for (int u = 0; u < 2; u++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const int t = 2 * u + (j >> 2), r = j & 3;
+          const int key = kb * 64 + t * 16 + g * 4 + r;
+          const float pr = key <= qpos[qg] ? __expf(sc[qg][t][r] - mn) : 0.f;
+          l[qg] += pr;
+          pb[qg][u][j] = (__bf16)pr;
+        }
+      m[qg] = mn;
+    }
 #pragma unroll
     for (int dt = 0; dt < 8; dt++)
 #pragma unroll
       for (int u = 0; u < 2; u++) {
+        // K slots g*8 .. g*8+7 of the operand = keys u*32 + g*4 .. +3 and u*32 + 16 + g*4 .. +3 of the tile,
+        // the keys pb[.][u] holds in the same slots
         const uint16_t* vrow = vt + (dt * 16 + c) * AP_VP + u * 32 + g * 4;
         const uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 16);
-        i32x4 av = {(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
-        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), pb[u], acc[dt], 0, 0, 0);
+        const i32x4 av = {(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
+#pragma unroll
+        for (int qg = 0; qg < QG; qg++)
+          acc[qg][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), pb[qg][u], acc[qg][dt], 0, 0, 0);
       }
   }
-  l += __shfl_xor(l, 16);
-  l += __shfl_xor(l, 32);
-  if (q0 + c < p.S) {
-    uint16_t* orow = p.out + (((int64_t)b * p.S + q0 + c) * p.Nq + hq) * 128;
 #pragma unroll
-    for (int dt = 0; dt < 8; dt++) {
-      uint32_t w[2];
+  for (int qg = 0; qg < QG; qg++) {
+    float ls = l[qg];
+    ls += __shfl_xor(ls, 16);
+    ls += __shfl_xor(ls, 32);
+    const int qi = q0 + qg * 16 + c;
+    if (qi < p.S) {
+      uint16_t* orow = p.out + (((int64_t)b * p.S + qi) * p.Nq + hq) * 128;
 #pragma unroll
-      for (int h = 0; h < 2; h++)
-        w[h] = f32_to_bf16_bits(l > 0.f ? acc[dt][2 * h] / l : 0.f) |
-               (f32_to_bf16_bits(l > 0.f ? acc[dt][2 * h + 1] / l : 0.f) << 16);
-      *reinterpret_cast<uint2*>(orow + dt * 16 + g * 4) = make_uint2(w[0], w[1]);
+      for (int dt = 0; dt < 8; dt++) {
+        uint32_t w[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+          w[h] = f32_to_bf16_bits(ls > 0.f ? acc[qg][dt][2 * h] / ls : 0.f) |
+                 (f32_to_bf16_bits(ls > 0.f ? acc[qg][dt][2 * h + 1] / ls : 0.f) << 16);
+        *reinterpret_cast<uint2*>(orow + dt * 16 + g * 4) = make_uint2(w[0], w[1]);
+      }
     }
   }
 }
@@ -621,6 +653,8 @@ extern "C" int tppx_attn_prefill(const void* q, const void* kcache, const void* 
   p.B = (int)B; p.S = (int)S; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.Smax = (int)Smax; p.mask_ld = (int)mask_ld;
   p.past = (int)past_len;
   p.scale = 1.0f / sqrtf((float)H);
-  attn_prefill_kernel<<<dim3((unsigned)((S + 63) / 64), (unsigned)(B * Nq)), dim3(256), 0, (hipStream_t)stream>>>(p);
+  // 16 queries per wave: 32 (QG = 2) halve the LDS reads per MFMA but need 248 registers, one wave per SIMD, and
+  // measured slower (S = 2048, 32 heads: 197 us against 172 us)
+  attn_prefill_kernel<1><<<dim3((unsigned)((S + 63) / 64), (unsigned)(B * Nq)), dim3(256), 0, (hipStream_t)stream>>>(p);
   return check_hip(hipGetLastError(), who);
 }
