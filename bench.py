@@ -56,9 +56,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--fmt", default="qint8", choices=["qint8", "mxfp4"])
     ap.add_argument("--batch", type=int, default=1, help="sequences for --workload tokens (1 or 16 in the baseline)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "tokens"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "tokens", "prompt"],
                     help="decode = the configuration the headline metric is quoted on (default); prefill = the "
-                         "MXFP4 linears of one 70B-shape decoder layer at M = 2048 (TFLOP/s, MFMA roofline)")
+                         "MXFP4 linears of one 70B-shape decoder layer at M = 2048 (TFLOP/s, MFMA roofline); tokens = "
+                         "7B-shape greedy decode; prompt = a 2048-token prompt through the same 7B-shape decoder")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pool", type=int, default=2, help="number of distinct weight sets cycled through")
@@ -85,6 +86,8 @@ def main():
         return run_prefill(torch, _ops, args)
     if args.workload == "tokens":
         return run_tokens(torch, args)
+    if args.workload == "prompt":
+        return run_prompt(torch, args)
 
     fmt = args.fmt
     shapes = {"up": (11008, 4096), "down": (4096, 11008)}
@@ -235,6 +238,42 @@ def run_tokens(torch, args):
         "roofline": {"bound": "hbm", "kernel": "whole decode step (all kernels of the graph)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "bytes_per_step": int(lin_bytes + kv_bytes)},
+        "cpu_baseline": None}))
+
+
+def run_prompt(torch, args):
+    """Prompt processing on the 7B-shape decoder of config 5: `--batch` sequences of 2048 random token ids through
+    the 32 layers in one pass (MXFP4 linears on the large-M kernels, causal attention, keys appended to an empty
+    cache), then the lm_head on the last position.  Not a BASELINE configuration; reported as prompt tokens/s."""
+    from tpp_pytorch_extension.llm import fused_llama_infer as F
+    dev = torch.device("cuda:0")
+    B, S = args.batch, 2048
+    model = F.LlamaDecoder(hidden=4096, inter=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab=32000,
+                           max_positions=4096, weight_dtype="mxfp4", seed=1239)
+    prompt = torch.randint(0, 32000, (B, S), generator=torch.Generator().manual_seed(6), dtype=torch.int64).to(dev)
+    steps, warmup = max(2, min(args.steps, 8)), max(1, min(args.warmup, 2))
+    caches = [F.TppCache(S + 32) for _ in range(steps + warmup)]
+    for c in caches[:warmup]:
+        model.prefill(prompt, c)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for c in caches[warmup:]:
+        model.prefill(prompt, c)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    lin_flops = 2.0 * B * S * 32 * (4 * 4096 * 4096 + 3 * 11008 * 4096) + 2.0 * B * 32000 * 4096
+    attn_flops = 32 * 4.0 * B * 32 * 128 * (S * (S + 1) / 2)
+    tf = (lin_flops + attn_flops) / (ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "7B-shape prompt tokens/s", "value": round(B * S / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"32-layer Llama-2-7B-shape decoder, MXFP4 linears, prompt of {S} tokens x batch {B} in "
+                               f"one pass onto an empty KV cache", "launch": "eager op calls", "batch": B},
+        "roofline": {"bound": "mfma", "kernel": "whole prompt pass (GEMMs + causal attention + glue)",
+                     "achieved": round(tf, 1), "peak": PEAKS_TFLOPS["bf16"], "unit": "TFLOP/s",
+                     "frac": round(tf / PEAKS_TFLOPS["bf16"], 4), "traffic": None,
+                     "flops_per_step": lin_flops + attn_flops},
         "cpu_baseline": None}))
 
 

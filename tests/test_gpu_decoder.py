@@ -154,6 +154,23 @@ def test_attn_prefill(B, S, Nq, Nkv, past, Smax):
         assert np.sqrt(((g - d) ** 2).sum() / (d ** 2).sum()) <= 5e-3
 
 
+def test_attn_prefill_full_size_rows_equal_single_query_problem():
+    """The 7B prompt shape (2048 tokens, 32 heads): every sampled query row must solve the single-query problem on
+    the keys it sees -- checked against the oracle's single-query function, which the multi-query restatement is
+    pinned to row by row (the full multi-query oracle would take minutes at this size)."""
+    _llm()
+    B, S, Nq = 1, 2048, 32
+    q = randn_bf16((B, S, Nq, 128), 1.0, 71)
+    k = randn_bf16((B, Nq, S, 128), 1.0, 72)
+    v = randn_bf16((B, Nq, S, 128), 1.0, 73)
+    got = _attn_prefill(q.cuda(), k.cuda(), v.cuda(), 0).cpu()
+    for i in (0, 1, 63, 64, 65, 1023, 1024, 2046, 2047):
+        ref = O.attn_decode(t2bits(q[:, i]), t2bits(k[:, :, :i + 1]), t2bits(v[:, :, :i + 1]))
+        g, r = bits2f(t2bits(got[:, i])).astype(np.float64), bits2f(ref).astype(np.float64)
+        assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3, i
+        assert np.abs(g - r).max() <= 2.0 ** -7 * np.abs(r).max(), i
+
+
 def test_attn_prefill_mask_and_errors():
     F = _llm()
     from tpp_pytorch_extension._lib import TppxError
