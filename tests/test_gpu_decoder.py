@@ -379,11 +379,13 @@ def test_rms_norm_fused_into_gemms(M, K, monkeypatch):
     assert_close_bf16(t2bits(y), t2bits(sep[0]), what="LDS-staged plain GEMM")
 
 
-def test_optimize_model_for_llama_against_transformers():
+@pytest.mark.parametrize("weight_dtype", ["mxfp4", "qint8"])
+def test_optimize_model_for_llama_against_transformers(weight_dtype):
     """OptimizeModelForLlama on a random-initialised transformers LlamaForCausalLM (2 layers, GQA 4/2 heads of
     128): the logits of the prompt pass and of two decode steps against the stock transformers model in fp32 on
-    the CPU holding the *dequantized* MXFP4 weights (exactly representable), i.e. the same function up to the
-    bf16 roundings of the fused path.  Left padding goes through the additive key mask."""
+    the CPU holding the *dequantized* weights (exactly representable), i.e. the same function up to the bf16
+    roundings of the fused path (and, for QINT8, the int8 rounding of the activations: looser bound).  Left
+    padding goes through the additive key mask."""
     transformers = pytest.importorskip("transformers")
     import copy
     F = _llm()
@@ -396,11 +398,16 @@ def test_optimize_model_for_llama_against_transformers():
         for m in ref_model.modules():
             if isinstance(m, torch.nn.Linear):  # weights := dequantize(quantize(weights)), as the fused model sees them
                 w = m.weight.data.to(torch.bfloat16).float()
-                q, sc = O.remap_quantize_mxfp4(w.numpy())
-                m.weight.data.copy_(torch.from_numpy(O.dequantize_mxfp4_plain(q, sc)))
+                if weight_dtype == "mxfp4":
+                    q, sc = O.remap_quantize_mxfp4(w.numpy())
+                    m.weight.data.copy_(torch.from_numpy(O.dequantize_mxfp4_plain(q, sc)))
+                else:
+                    q, sc, _ = O.remap_quantize_qint8(w.numpy())
+                    m.weight.data.copy_(torch.from_numpy(O.dequantize_qint8_plain(q, sc)))
             elif isinstance(m, torch.nn.Embedding):
                 m.weight.data.copy_(m.weight.data.to(torch.bfloat16).float())
-    opt_model = F.OptimizeModelForLlama(copy.deepcopy(ref_model), torch.bfloat16, "cuda", "mxfp4").eval()
+    opt_model = F.OptimizeModelForLlama(copy.deepcopy(ref_model), torch.bfloat16, "cuda", weight_dtype).eval()
+    tol = 3e-2 if weight_dtype == "mxfp4" else 6e-2
 
     ids = torch.randint(0, 1024, (2, 19), generator=torch.Generator().manual_seed(12))
     am = torch.ones_like(ids)
@@ -416,8 +423,8 @@ def test_optimize_model_for_llama_against_transformers():
         o = opt_model(input_ids=ids.cuda(), attention_mask=am.cuda(), position_ids=pos.cuda(), use_cache=True)
         assert o.logits.shape == r.logits.shape
         # padded positions of sequence 1 are arbitrary in both models; compare the real ones
-        assert rel(o.logits[0].float().cpu(), r.logits[0]) <= 3e-2
-        assert rel(o.logits[1, 4:].float().cpu(), r.logits[1, 4:]) <= 3e-2
+        assert rel(o.logits[0].float().cpu(), r.logits[0]) <= tol
+        assert rel(o.logits[1, 4:].float().cpu(), r.logits[1, 4:]) <= tol
         cache_o, cache_r = o.past_key_values, r.past_key_values
         assert cache_o.get_seq_length() == 19 and len(cache_o) == 2
         for step in range(2):
@@ -427,7 +434,7 @@ def test_optimize_model_for_llama_against_transformers():
             r = ref_model(input_ids=nxt, attention_mask=am, position_ids=pos, past_key_values=cache_r, use_cache=True)
             o = opt_model(input_ids=nxt.cuda(), attention_mask=am.cuda(), position_ids=pos.cuda(),
                           past_key_values=cache_o, use_cache=True)
-            assert rel(o.logits.float().cpu(), r.logits) <= 3e-2
+            assert rel(o.logits.float().cpu(), r.logits) <= tol
         assert cache_o.get_seq_length() == 21
     out = F.generate_greedy(opt_model, ids[:1].cuda(), 5)
     assert out.shape == (1, 24) and torch.equal(out[:, :19].cpu(), ids[:1])
