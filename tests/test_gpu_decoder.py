@@ -97,6 +97,22 @@ def test_attn_decode(B, Nq, Nkv, L, Smax):
     assert np.sqrt(((g - t) ** 2).sum() / (t ** 2).sum()) <= 1e-2
 
 
+def test_attn_decode_split_merge_in_launch_equals_second_kernel(monkeypatch):
+    """With a workspace the keys are split over several workgroups per head; the split that arrives last merges
+    them inside the launch.  Twenty launches in a row (the arrival counters must return to zero) give the bits of
+    the two-kernel path (TPPX_ATTN_ONE_LAUNCH=0), which merges in the same order."""
+    F = _llm()
+    B, Nq, Nkv, L, Smax = 2, 8, 4, 1500, 1536
+    q = randn_bf16((B, Nq, 128), 1.0, 81).cuda()
+    k = randn_bf16((B, Nkv, Smax, 128), 1.0, 82).cuda()
+    v = randn_bf16((B, Nkv, Smax, 128), 1.0, 83).cuda()
+    outs = [_attn(F, q, k, v, L) for _ in range(20)]
+    monkeypatch.setenv("TPPX_ATTN_ONE_LAUNCH", "0")
+    two = _attn(F, q, k, v, L)
+    for o in outs:
+        assert torch.equal(o, two)
+
+
 def test_attn_decode_mask():
     F = _llm()
     B, Nq, L, Smax = 2, 4, 100, 128

@@ -6,6 +6,8 @@
 #include <math.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "tppx_common.h"
 #include "tppx_launch.h"
 
@@ -187,8 +189,14 @@ struct AttnParams {
   uint16_t* out;        // [B][Nq][128]
   float* part;          // [B*Nq][splits][130]
   int B, Nq, Nkv, Smax, mask_ld, splits;
+  int ticket0;          // >= 0: first arrival counter of this launch (the last split to arrive merges); < 0: second kernel
   float scale;
 };
+
+// Arrival counters of the split launches, one per (sequence, head): zero between launches (the counting
+// instruction wraps on the last arrival); a launch takes a window handed out in rotation by the host.
+constexpr int ATTN_TICKETS = 16384;
+__device__ unsigned int attn_tickets[ATTN_TICKETS];
 
 __device__ __forceinline__ uint4 as_uint4(const i32x4& v) {
   return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
@@ -304,15 +312,63 @@ attn_decode_kernel(const AttnParams p) {
     }
     if (p.splits == 1) {
       p.out[(int64_t)bh * 128 + tid] = (uint16_t)f32_to_bf16_bits(Ls > 0.f ? o / Ls : 0.f);
-    } else {
+    } else if (p.ticket0 < 0) {
       float* dst = p.part + ((int64_t)bh * p.splits + blockIdx.y) * 130;
       dst[2 + tid] = o;
       if (tid == 0) {
         dst[0] = M;
         dst[1] = Ls;
       }
+    } else {
+      // device-scope atomic stores: written through to the level all XCDs share, no cache write-back needed
+      float* dst = p.part + ((int64_t)bh * p.splits + blockIdx.y) * 130;
+      __hip_atomic_store(dst + 2 + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tid == 0) {
+        __hip_atomic_store(dst, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(dst + 1, Ls, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
   }
+  if (p.splits == 1 || p.ticket0 < 0)
+    return;
+  // The split that arrives last merges all of them, in split order (the same sums whichever split that is).
+  // Order: the stores above are complete at the barrier (it waits for outstanding memory operations), then the
+  // ticket, then the device-scope loads of the other splits' results.  Nobody waits for anybody.
+  __shared__ int arrived_last;
+  __syncthreads();
+  if (tid == 0) {
+    const unsigned int last = (unsigned int)p.splits - 1;
+    arrived_last = atomicInc(&attn_tickets[p.ticket0 + bh], last) == last;
+  }
+  __syncthreads();
+  if (!arrived_last || tid >= 128)
+    return;
+  const float* src = p.part + (int64_t)bh * p.splits * 130;
+  float pm[32], pl[32], po[32]; // every load in flight at once (at most 32 splits)
+#pragma unroll
+  for (int i = 0; i < 32; i++) {
+    pm[i] = -3.0e38f;
+    pl[i] = po[i] = 0.f;
+    if (i < p.splits) {
+      pm[i] = __hip_atomic_load(src + i * 130, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      pl[i] = __hip_atomic_load(src + i * 130 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      po[i] = __hip_atomic_load(src + i * 130 + 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  float M = -3.0e38f;
+#pragma unroll
+  for (int i = 0; i < 32; i++)
+    if (i < p.splits)
+      M = fmaxf(M, pm[i]);
+  float Ls = 0.f, o = 0.f;
+#pragma unroll
+  for (int i = 0; i < 32; i++)
+    if (i < p.splits) {
+      const float w = __expf(pm[i] - M);
+      Ls = fmaf(w, pl[i], Ls);
+      o = fmaf(w, po[i], o);
+    }
+  p.out[(int64_t)bh * 128 + tid] = (uint16_t)f32_to_bf16_bits(Ls > 0.f ? o / Ls : 0.f);
 }
 
 __global__ void __launch_bounds__(128)
@@ -623,9 +679,21 @@ extern "C" int tppx_attn_decode(const void* q, const void* kcache, const void* v
     splits = 1; // no room for partial results: one workgroup per head
   p.splits = (int)splits;
   p.part = (float*)ws;
+  p.ticket0 = -1;
+  if (splits > 1 && B * Nq <= ATTN_TICKETS && env_int("TPPX_ATTN_ONE_LAUNCH", 1) != 0) {
+    // window of B * Nq arrival counters, handed out in rotation so that split launches in flight on different
+    // streams do not share counters
+    static std::mutex mu;
+    static int cursor = 0;
+    std::lock_guard<std::mutex> lock(mu);
+    if (cursor + B * Nq > ATTN_TICKETS)
+      cursor = 0;
+    p.ticket0 = cursor;
+    cursor += (int)(B * Nq);
+  }
   attn_decode_kernel<<<dim3((unsigned)(B * Nq), (unsigned)splits), dim3(256), 0, (hipStream_t)stream>>>(p);
   int rc = check_hip(hipGetLastError(), who);
-  if (rc || splits == 1)
+  if (rc || splits == 1 || p.ticket0 >= 0)
     return rc;
   attn_combine_kernel<<<dim3((unsigned)(B * Nq)), dim3(128), 0, (hipStream_t)stream>>>(p);
   return check_hip(hipGetLastError(), who);
