@@ -232,6 +232,35 @@ int tppx_norm_swiglu_mxfp4(const void* x, const void* gamma, float eps,
                            int64_t M, int64_t N, int64_t K, int flags,
                            tppx_stream_t stream);
 
+/* The same two fusions without a pass over x for the normalisation: the launch
+ * that WROTE x (the residual-add GEMM before the norm: o-projection,
+ * down-projection of the previous layer) leaves, per row, the sums of squares
+ * of its bf16 outputs in row_sumsq, f32 [16][256] ([row][workgroup], every call
+ * overwrites the 256 slots of its M rows); the consuming launch adds a row's
+ * 256 slots, takes 1/sqrt(sum/K + eps) and normalises the activations on
+ * their way into LDS.  M <= 16, MXFP4 decode kernels only (TPPX_EUNSUPPORTED
+ * otherwise: use the entry points above).  The table is plain device memory
+ * owned by the caller; producer and consumer must be ordered on one stream.
+ * No counterpart in the reference (its norm is a separate pass,
+ * fused_llm_infer.cpp:1231,1269); results differ from that pass only through
+ * the summation order of the squares (fp32). */
+int tppx_linear_mxfp4_rowsq(const void* x, const void* qw, const void* sw,
+                            const void* bias, const void* post_in,
+                            const void* post_in2, void* y, int64_t M, int64_t N,
+                            int64_t K, int post_op, float post_scale, int flags,
+                            void* ws, int64_t ws_bytes, void* row_sumsq,
+                            tppx_stream_t stream);
+int tppx_normsq_multi_linear_mxfp4(const void* x, const void* row_sumsq,
+                                   const void* gamma, float eps,
+                                   const tppx_seg* segs, int n_segs, int64_t M,
+                                   int64_t K, int flags, tppx_stream_t stream);
+int tppx_normsq_swiglu_mxfp4(const void* x, const void* row_sumsq,
+                             const void* gamma, float eps, const void* qw_gate,
+                             const void* sw_gate, const void* bias_gate,
+                             const void* qw_up, const void* sw_up,
+                             const void* bias_up, void* y, int64_t M, int64_t N,
+                             int64_t K, int flags, tppx_stream_t stream);
+
 /* ---- decode-side operators of the decoder layer -------------------------- */
 
 /* Replaces llama_rms_norm / RMSNormFwdTPP (src/csrc/llm/fused_llm_infer.cpp:309-363,

@@ -395,6 +395,36 @@ def test_rms_norm_fused_into_gemms(M, K, monkeypatch):
     assert_close_bf16(t2bits(y), t2bits(sep[0]), what="LDS-staged plain GEMM")
 
 
+@pytest.mark.parametrize("M", [1, 3, 16])
+@pytest.mark.parametrize("Kprod,N", [(512, 4096), (11008, 4096), (1024, 2048)])
+def test_rms_norm_from_row_sums(M, Kprod, N):
+    """The residual-add GEMM leaves the row sums of squares of its output in a [16][256] table (every producing
+    kernel: all rows in LDS, 4 rows for a long K, one row group); the table equals the sums computed from the output
+    bits, and the q/k/v and gate/up launches that take their RMSNorm scale from it match the normalisation kernel
+    followed by the plain launches within the GEMM tolerance (the row scale can differ in its last bit)."""
+    F = _llm()
+    from tpp_pytorch_extension import _ops
+    Wp = _ops.remap_and_quantize_mxfp4(block_bf16(randn_bf16((N, Kprod), 0.03, 500)).cuda())
+    xin = randn_bf16((M, Kprod), 1.0, 501).cuda()
+    res = randn_bf16((M, N), 1.0, 502).cuda()
+    tab = torch.full((16, 256), 7.0, dtype=torch.float32, device="cuda")  # stale contents must not survive
+    h = _ops.fc_add(xin, Wp, None, res, 1.0, row_sumsq=tab)
+    assert torch.equal(h, _ops.fc_add(xin, Wp, None, res, 1.0))
+    want = (h.double() ** 2).sum(-1).cpu().numpy()
+    got = tab[:M].double().sum(-1).cpu().numpy()
+    assert np.allclose(got, want, rtol=1e-5), (got, want)
+    gamma = (torch.rand(N, generator=torch.Generator().manual_seed(503)) + 0.5).cuda()
+    ws = [_ops.remap_and_quantize_mxfp4(block_bf16(randn_bf16((n, N), 0.03, 510 + i)).cuda())
+          for i, n in enumerate((1536, 512, 512))]
+    hn = F.rms_norm(h, gamma, 1e-5)
+    fused = _ops.qkv_gemm(h, ws, [None] * 3, norm=(gamma, 1e-5, tab))
+    for a, b in zip(fused, _ops.qkv_gemm(hn, ws, [None] * 3)):
+        assert_close_bf16(t2bits(a), t2bits(b), what=f"norm from row sums, qkv M={M}")
+        assert (a != b).float().mean() < 0.01
+    fz = _ops.swiglu_gate_up(h, ws[1], ws[2], norm=(gamma, 1e-5, tab))
+    assert_close_bf16(t2bits(fz), t2bits(_ops.swiglu_gate_up(hn, ws[1], ws[2])), ulps=2, what=f"norm from row sums, swiglu M={M}")
+
+
 @pytest.mark.parametrize("weight_dtype", ["mxfp4", "qint8"])
 def test_optimize_model_for_llama_against_transformers(weight_dtype):
     """OptimizeModelForLlama on a random-initialised transformers LlamaForCausalLM (2 layers, GQA 4/2 heads of

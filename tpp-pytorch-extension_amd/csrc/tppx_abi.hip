@@ -208,10 +208,13 @@ static TiledParams tiled_from_seg(const DecodeParams& p, int i) {
 
 static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n_segs,
                      int64_t M, int64_t K, int flags, bool dual, void* ws, int64_t ws_bytes,
-                     hipStream_t stream) {
+                     hipStream_t stream, float* row_sumsq = nullptr) {
   int rc = check_common(who, x, M, K, n_segs, flags, ws, ws_bytes);
   if (rc)
     return rc;
+  TPPX_REQUIRE(!row_sumsq || (M <= 16 && n_segs == 1 && !dual && ((uintptr_t)row_sumsq & 15) == 0), TPPX_EUNSUPPORTED,
+               "%s: row sums of squares are produced for one GEMM of at most 16 rows (M=%ld) into a 16-byte aligned table",
+               who, (long)M);
   TPPX_REQUIRE(segs, TPPX_EINVAL, "%s: null segment table", who);
   TPPX_REQUIRE(K > 0 && K % 64 == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of 64", who, (long)K);
   TPPX_REQUIRE(K % 128 == 0, TPPX_EUNSUPPORTED, "%s: K=%ld is not a multiple of 128 (native MXFP4 tiles span 128 input channels)", who, (long)K);
@@ -227,7 +230,9 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
   p.units = (int)(K / 128);
   p.tpb = 1;
   p.S = 1;
+  p.sumsq_out = row_sumsq;
   if (want_tiled(M, flags)) {
+    TPPX_REQUIRE(!row_sumsq, TPPX_EUNSUPPORTED, "%s: row sums of squares are not produced by the large-M kernels", who);
     // prefill shapes: one LDS-tiled launch per GEMM of the group; the fused
     // gate/up pair becomes silu(gate) followed by up * gate (same rounding)
     if (!dual && n_segs > 1) {
@@ -271,8 +276,10 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     return TPPX_OK;
   }
   int nt_xl = 1;
-  if (M <= 16 && env_int("TPPX_MXFP4_XL", 1) == 1 && plan_xl(p, dual, &nt_xl))
+  if (M <= 16 && env_int("TPPX_MXFP4_XL", 1) == 1 && plan_xl(p, dual, &nt_xl)) {
+    TPPX_REQUIRE(!row_sumsq || p.groups <= 256, TPPX_EUNSUPPORTED, "%s: N=%ld needs more than 256 workgroups; the table of row sums has 256 slots", who, (long)segs[0].N);
     return check_hip(launch_skinny_mxfp4_xl(p, nt_xl, dual, stream), who);
+  }
   if (M <= 16) {
     // K that the LDS-staged kernel above cannot hold.  Up to 4 rows (and K up to 16384): the same staging with only
     // the 4 rows kept; otherwise the tile-by-tile kernel with one row group (measured at K = 11008, N = 4096:
@@ -285,6 +292,7 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
         break;
     }
     set_groups(p, nt, dual);
+    TPPX_REQUIRE(!row_sumsq || p.groups <= 256, TPPX_EUNSUPPORTED, "%s: N=%ld needs more than 256 workgroups; the table of row sums has 256 slots", who, (long)segs[0].N);
     return check_hip(x4 ? launch_skinny_mxfp4_x4(p, nt, dual, stream) : launch_skinny_mxfp4_mg(p, 1, nt, dual, stream), who);
   }
   {
@@ -377,7 +385,8 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
 
 // LDS-staged MXFP4 decode kernel (M <= 16) with an optional RMSNorm in front
 static int run_mxfp4_xl(const char* who, const void* x, const void* gamma, float eps, const tppx_seg* segs,
-                        int n_segs, int64_t M, int64_t K, int flags, bool dual, hipStream_t stream) {
+                        int n_segs, int64_t M, int64_t K, int flags, bool dual, hipStream_t stream,
+                        const float* row_sumsq = nullptr) {
   int rc = check_common(who, x, M, K, n_segs, flags, nullptr, 0);
   if (rc)
     return rc;
@@ -398,6 +407,9 @@ static int run_mxfp4_xl(const char* who, const void* x, const void* gamma, float
   p.S = 1;
   p.norm_gamma = (const float*)gamma;
   p.norm_eps = eps;
+  TPPX_REQUIRE(!row_sumsq || (gamma && ((uintptr_t)row_sumsq & 15) == 0), TPPX_EINVAL,
+               "%s: the table of row sums needs gamma and 16-byte alignment", who);
+  p.sumsq_in = row_sumsq;
   int nt = 1;
   TPPX_REQUIRE(plan_xl(p, dual, &nt), TPPX_EUNSUPPORTED,
                "%s: K=%ld does not split into 16 slices of 128 or 256 input channels (or fewer than 16 tiles) that fit the LDS staging; run the steps separately", who, (long)K);
@@ -420,6 +432,35 @@ extern "C" int tppx_norm_swiglu_mxfp4(const void* x, const void* gamma, float ep
   tppx_seg s[2] = {{qw_gate, sw_gate, bias_gate, nullptr, nullptr, y, N, TPPX_POST_NONE, 1.0f},
                    {qw_up, sw_up, bias_up, nullptr, nullptr, y, N, TPPX_POST_NONE, 1.0f}};
   return run_mxfp4_xl("tppx_norm_swiglu_mxfp4", x, gamma, eps, s, 2, M, K, flags, true, (hipStream_t)stream);
+}
+
+extern "C" int tppx_linear_mxfp4_rowsq(const void* x, const void* qw, const void* sw, const void* bias,
+                                       const void* post_in, const void* post_in2, void* y, int64_t M, int64_t N,
+                                       int64_t K, int post_op, float post_scale, int flags, void* ws,
+                                       int64_t ws_bytes, void* row_sumsq, tppx_stream_t stream) {
+  const char* who = "tppx_linear_mxfp4_rowsq";
+  TPPX_REQUIRE(row_sumsq, TPPX_EINVAL, "%s: null table of row sums", who);
+  tppx_seg s = {qw, sw, bias, post_in, post_in2, y, N, post_op, post_scale};
+  return run_mxfp4(who, x, &s, 1, M, K, flags, false, ws, ws_bytes, (hipStream_t)stream, (float*)row_sumsq);
+}
+
+extern "C" int tppx_normsq_multi_linear_mxfp4(const void* x, const void* row_sumsq, const void* gamma, float eps,
+                                              const tppx_seg* segs, int n_segs, int64_t M, int64_t K, int flags,
+                                              tppx_stream_t stream) {
+  const char* who = "tppx_normsq_multi_linear_mxfp4";
+  TPPX_REQUIRE(row_sumsq && gamma, TPPX_EINVAL, "%s: null table of row sums or gamma", who);
+  return run_mxfp4_xl(who, x, gamma, eps, segs, n_segs, M, K, flags, false, (hipStream_t)stream, (const float*)row_sumsq);
+}
+
+extern "C" int tppx_normsq_swiglu_mxfp4(const void* x, const void* row_sumsq, const void* gamma, float eps,
+                                        const void* qw_gate, const void* sw_gate, const void* bias_gate,
+                                        const void* qw_up, const void* sw_up, const void* bias_up, void* y,
+                                        int64_t M, int64_t N, int64_t K, int flags, tppx_stream_t stream) {
+  const char* who = "tppx_normsq_swiglu_mxfp4";
+  TPPX_REQUIRE(row_sumsq && gamma, TPPX_EINVAL, "%s: null table of row sums or gamma", who);
+  tppx_seg s[2] = {{qw_gate, sw_gate, bias_gate, nullptr, nullptr, y, N, TPPX_POST_NONE, 1.0f},
+                   {qw_up, sw_up, bias_up, nullptr, nullptr, y, N, TPPX_POST_NONE, 1.0f}};
+  return run_mxfp4_xl(who, x, gamma, eps, s, 2, M, K, flags, true, (hipStream_t)stream, (const float*)row_sumsq);
 }
 
 extern "C" int tppx_version(void) {

@@ -44,6 +44,11 @@ struct DecodeParams {
   float* part;   // [S][block row][total_tiles][MG][256] fp32 partial tiles (S > 1)
   const float* norm_gamma; // f32 [K]: RMSNorm fused in front of the GEMM (LDS-staged MXFP4 kernel), or null
   float norm_eps;
+  // Row sums of squares handed from the GEMM that writes a tensor to the GEMM that normalises it: f32 [16][256],
+  // entry [row][workgroup] = sum of squares of the bf16 outputs of that row owned by that workgroup (unused
+  // workgroup slots zero).  The consumer adds a row's 256 entries instead of making a pass over the row.
+  float* sumsq_out;      // written by this launch's epilogue (M <= 16, single GEMM), or null
+  const float* sumsq_in; // with norm_gamma: the table the launch that produced x wrote, or null (sum x^2 here)
 };
 
 // launch shape of the QINT8 decode kernels (K split inside the workgroup)

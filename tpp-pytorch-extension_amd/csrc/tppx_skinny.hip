@@ -40,6 +40,14 @@ __device__ __forceinline__ bf16x8 sk_cvt_fp4x8(uint32_t codes, float scale) {
   return w;
 }
 
+// two floats -> two bf16 (round to nearest even) in one dword: the hardware conversion, one instruction per pair
+// (the normalisation in front of a GEMM converts M x K values in EVERY workgroup)
+__device__ __forceinline__ uint32_t sk_pack_bf16(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2;
+  const bf16x2 v = __builtin_convertvector(f32x2{lo, hi}, bf16x2);
+  return __builtin_bit_cast(uint32_t, v);
+}
+
 __device__ __forceinline__ int sk_find_seg(const DecodeParams& p, int grp) {
   int s = 0;
 #pragma unroll
@@ -199,8 +207,12 @@ struct SkEpilogue {
       }
   }
 
-  // stride = floats between the regions of two waves (>= ELEMS)
-  __device__ __forceinline__ void finish(const DecodeSeg& sg, f32x4 (&acc)[NACC][MG], float* red, int stride = ELEMS) {
+  // stride = floats between the regions of two waves (>= ELEMS).  sumsq (MG == 1, not the gate/up pair): also
+  // leave, per row, the sum of squares of this workgroup's rounded outputs in sumsq[row][blockIdx.x] of a
+  // [16][256] table (workgroup 0 zeroes the slots past the grid), added in a fixed order.
+  __device__ __forceinline__ void finish(const DecodeSeg& sg, f32x4 (&acc)[NACC][MG], float* red, int stride = ELEMS,
+                                         float* sumsq = nullptr, int M = 0) {
+    __shared__ float sq_s[16 * NACC];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int W = blockDim.x >> 6;
     float* mine = red + wave * stride;
@@ -222,8 +234,8 @@ struct SkEpilogue {
         if (DUAL)
           for (int w = 0; w < W; w++)
             v2 += red[w * stride + e + ELEMS / 2];
+        uint32_t out = 0;
         if (off[i] >= 0) {
-          uint32_t out;
           if (DUAL) {
             uint32_t gact = apply_post_bits(v + bf16_bits_to_f32(bias[i]), TPPX_POST_SILU, 0, 0, 1.0f);
             out = apply_post_bits(v2 + bf16_bits_to_f32(bias2[i]), TPPX_POST_MUL, gact, 0, 1.0f);
@@ -232,7 +244,34 @@ struct SkEpilogue {
           }
           sg.y[off[i]] = (uint16_t)out;
         }
+        if (!DUAL && MG == 1 && sumsq) { // wave-uniform: e < OUT holds for whole waves
+          const float ov = off[i] >= 0 ? bf16_bits_to_f32(out & 0xffffu) : 0.f;
+          float sq = ov * ov;
+          // the 16 lanes of a DPP row hold the 16 channels of one (row, tile) pair
+          sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0xB1, 0xf, 0xf, true));
+          sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0x4E, 0xf, 0xf, true));
+          sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0x141, 0xf, 0xf, true));
+          sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0x140, 0xf, 0xf, true));
+          if ((e & 15) == 0)
+            sq_s[(((e & 63) >> 4) * 4 + ((e >> 6) & 3)) * NACC + (e >> 8)] = sq; // [row][tile]
+        }
       }
+    }
+    if (!DUAL && MG == 1 && sumsq) {
+      __syncthreads();
+      if (threadIdx.x < 16 && (int)threadIdx.x < M) {
+        float tot = 0.f;
+#pragma unroll
+        for (int a = 0; a < NACC; a++)
+          tot += sq_s[threadIdx.x * NACC + a];
+        sumsq[threadIdx.x * 256 + blockIdx.x] = tot;
+      }
+      if (blockIdx.x == 0)
+        for (int j = (int)gridDim.x + (int)threadIdx.x; j < 256 * min(M, 16); j += (int)blockDim.x) {
+          const int row = j >> 8, part = j & 255; // slots gridDim.x .. 255 of every row (j walks a superset)
+          if (part >= (int)gridDim.x)
+            sumsq[row * 256 + part] = 0.f;
+        }
     }
   }
 };
@@ -691,10 +730,24 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
   });
   // the chunk of a lane is the same in every item when the slice is 16 or 32 chunks wide
   f32x4 gm0 = f32x4{1.f, 1.f, 1.f, 1.f}, gm1 = gm0;
-  if (XMODE == 1) {
+  if (XMODE != 0) {
     const float* gp = p.norm_gamma + (size_t)min(t0, KT - 1) * 128 + (size_t)(lane & cmask) * 8;
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(gm0) : "v"(gp) : "memory");
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(gm1) : "v"(gp + 4) : "memory");
+  }
+  // XMODE 2: the 256 sums of squares per row left by the launch that wrote x, 4 per lane.  Up to 4 rows (XNI == 2):
+  // every wave adds up all rows itself, no exchange; more rows: wave w adds up row w and the waves exchange the
+  // scales through LDS behind a barrier.
+  constexpr int NPQ = XNI == 2 ? 4 : 1;
+  f32x4 pq[NPQ];
+  if (XMODE == 2) {
+    static_for<0, NPQ>([&](auto R) {
+      constexpr int r = decltype(R)::value;
+      const float* sp = p.sumsq_in + (size_t)min(NPQ == 1 ? wave : r, p.M - 1) * 256 + (size_t)lane * 4;
+      f32x4 v;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(sp) : "memory");
+      pq[r] = v;
+    });
   }
 
   // weight ring: it has the HBM latency to cover
@@ -727,6 +780,13 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
     raw[decltype(IT)::value] = v;
   });
   asm volatile("" : "+v"(gm0), "+v"(gm1));
+  if (XMODE == 2) {
+    static_for<0, NPQ>([&](auto R) {
+      f32x4 v = pq[decltype(R)::value];
+      asm volatile("" : "+v"(v));
+      pq[decltype(R)::value] = v;
+    });
+  }
 
   // the slot arithmetic below starts from an opaque copy of the lane index, so that it is redone here instead of
   // being carried in registers across the loads above (where registers are scarcest)
@@ -737,6 +797,38 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
     // slots of rows and tiles this wave does not have count as zero
     if (lane < 16 * cht)
       wss[wave * 16 * cht + lane] = 0.f;
+  }
+  float rscale[NPQ]; // XMODE 2: 1/sqrt(mean square + eps) of row r (XNI == 2) or of row `wave`
+  if (XMODE == 2) {
+    // a row's sum in a fixed order: four entries per lane, a DPP row, the four DPP rows
+    static_for<0, NPQ>([&](auto R) {
+      constexpr int r = decltype(R)::value;
+      float tot = (pq[r][0] + pq[r][1]) + (pq[r][2] + pq[r][3]);
+      tot += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(tot), 0xB1, 0xf, 0xf, true));
+      tot += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(tot), 0x4E, 0xf, 0xf, true));
+      tot += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(tot), 0x141, 0xf, 0xf, true));
+      tot += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(tot), 0x140, 0xf, 0xf, true));
+      const float a0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tot), 0));
+      const float a1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tot), 16));
+      const float a2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tot), 32));
+      const float a3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tot), 48));
+      rscale[r] = 1.0f / sqrtf(((a0 + a1) + (a2 + a3)) * (1.0f / (float)p.K) + p.norm_eps);
+    });
+    if (NPQ == 1) {
+      // waves past M repeat the last row into a slot nobody reads
+      if (lane2 == 0)
+        wss[wave] = rscale[0];
+      // LDS only: a full __syncthreads would also wait for the weight ring
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
+    } else {
+      // through this wave's own LDS slots: selected by row in registers, the compiler turns the selection into an
+      // indexed read of a stack array, a memory load that has to wait for the whole weight ring
+      static_for<0, NPQ>([&](auto R) {
+        if (lane2 == 0)
+          srow[decltype(R)::value] = rscale[decltype(R)::value];
+      });
+      __builtin_amdgcn_wave_barrier();
+    }
   }
   // raw activations go to their operand slots right away; the norm rescales them in place
   static_for<0, XNI>([&](auto IT) {
@@ -761,7 +853,21 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
       if (i < items && (lane2 & 15) == 0)
         wss[(wave * 16 + row) * cht + (ck >> 4)] = ssq;
     }
-    *reinterpret_cast<i32x4*>(&xs[ck * 16 + (row ^ (ck & 15))]) = raw[it];
+    if (XMODE == 2) {
+      // normalised on the way in: (x * scale) * gamma, one rounding
+      const float sc = NPQ == 1 ? wss[row] : srow[row];
+      i32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const uint32_t d = (uint32_t)raw[it][e];
+        const float lo = (bf16_bits_to_f32(d & 0xffffu) * sc) * (e < 2 ? gm0[2 * e] : gm1[2 * e - 4]);
+        const float hi = (bf16_bits_to_f32(d >> 16) * sc) * (e < 2 ? gm0[2 * e + 1] : gm1[2 * e - 3]);
+        o[e] = (int)sk_pack_bf16(lo, hi);
+      }
+      *reinterpret_cast<i32x4*>(&xs[ck * 16 + (row ^ (ck & 15))]) = o;
+    } else {
+      *reinterpret_cast<i32x4*>(&xs[ck * 16 + (row ^ (ck & 15))]) = raw[it];
+    }
   });
   if (XMODE == 1) {
     // LDS only: a full __syncthreads would also wait for the weight ring
@@ -790,12 +896,17 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
         const uint32_t d = (uint32_t)w[e];
         const float lo = (bf16_bits_to_f32(d & 0xffffu) * sc) * (e < 2 ? gm0[2 * e] : gm1[2 * e - 4]);
         const float hi = (bf16_bits_to_f32(d >> 16) * sc) * (e < 2 ? gm0[2 * e + 1] : gm1[2 * e - 3]);
-        o[e] = (int)(f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16));
+        o[e] = (int)sk_pack_bf16(lo, hi);
       }
       *slot = o;
     }
   }
   // the wave reads only what it wrote itself: program order is enough
+
+  // Nothing from below may be scheduled into the staging code above: with the normalisation's long arithmetic
+  // there, the scheduler pulled the first uses of the weight ring's registers (scale conversions of the main loop)
+  // up into it, and the wait for the WHOLE ring that those need landed in front of the staging (+2.4 us).
+  __builtin_amdgcn_sched_barrier(0);
 
   // post-op inputs: requested here so that their registers are not live while the activations are in flight
   SkEpilogue<1, NTW, DUAL, 16> ep;
@@ -838,7 +949,7 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
     }
   }
   __syncthreads(); // every wave is done with its x region before it becomes reduction scratch
-  ep.finish(sg, acc, sk_lds, wstride);
+  ep.finish(sg, acc, sk_lds, wstride, p.sumsq_out, p.M);
 }
 
 // ---------------------------------------------------------------------------
@@ -974,7 +1085,7 @@ skinny_mxfp4_x4_kernel(const DecodeParams p) {
     }
   }
   __syncthreads(); // every wave is done with its x region before it becomes reduction scratch
-  ep.finish(sg, acc, sk_lds, wstride);
+  ep.finish(sg, acc, sk_lds, wstride, p.sumsq_out, p.M);
 }
 
 // ---------------------------------------------------------------------------
@@ -1145,7 +1256,7 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
     if (p.S > 1)
       ep.finish_split(p, sg, acc, sk_lds, ltile0);
     else
-      ep.finish(sg, acc, sk_lds);
+      ep.finish(sg, acc, sk_lds, decltype(ep)::ELEMS, p.sumsq_out, p.M);
   }
 }
 
@@ -1292,11 +1403,14 @@ hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_
   dim3 grid(p.groups, 1);
   const bool norm = p.norm_gamma != nullptr;
   const bool few = p.M <= 4; // 4 rows x 32 chunks fit two items per lane
+  const bool handed = norm && p.sumsq_in != nullptr; // row sums of squares come from the launch that wrote x
 #define SKXL(NT, DUAL)                                                                                       \
-  return norm ? (few ? sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 1, 2>, p, grid, 16, lds, stream)        \
-                     : sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 1, 8>, p, grid, 16, lds, stream))       \
-              : (few ? sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 0, 2>, p, grid, 16, lds, stream)        \
-                     : sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 0, 8>, p, grid, 16, lds, stream))
+  return handed ? (few ? sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 2, 2>, p, grid, 16, lds, stream)      \
+                       : sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 2, 8>, p, grid, 16, lds, stream))     \
+       : norm   ? (few ? sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 1, 2>, p, grid, 16, lds, stream)      \
+                       : sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 1, 8>, p, grid, 16, lds, stream))     \
+                : (few ? sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 0, 2>, p, grid, 16, lds, stream)      \
+                       : sk_launch(skinny_mxfp4_xl_kernel<NT, 2, DUAL, 0, 8>, p, grid, 16, lds, stream))
   if (dual) {
     if (nt == 3)
       SKXL(3, true);

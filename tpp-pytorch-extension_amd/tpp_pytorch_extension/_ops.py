@@ -293,9 +293,12 @@ def _qint8_scratch(x, M, K, qbs):
     return xq, sa
 
 
-def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0, flags=0):
+def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0, flags=0,
+           row_sumsq=None):
     """One quantized GEMM with a fused post-op
-    (call_gemm_with_post_op, src/csrc/fused_gemm.h:1510-1597)."""
+    (call_gemm_with_post_op, src/csrc/fused_gemm.h:1510-1597).
+    row_sumsq: f32 [16][256] table that receives the row sums of squares of the output (see sums_table());
+    only honoured where takes_row_sums() says so."""
     L = _lib.lib()
     x, M, N, K = _prep_input(input, weight)
     out_shape = tuple(input.shape[:-1]) + (N,)
@@ -308,7 +311,14 @@ def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None
     qn, sn = weight.native()
     st = _lib.stream_of(x)
     ws = _lib.workspace(x)
-    if weight._qscheme == QSCHEME_MXFP:
+    if row_sumsq is not None:
+        if not takes_row_sums(weight, M):
+            raise TppxError(_lib.EUNSUPPORTED, "row sums of squares need an MXFP4 weight and at most 16 rows")
+        _lib.check(L.tppx_linear_mxfp4_rowsq(x.data_ptr(), qn.data_ptr(), sn.data_ptr(), _lib.ptr(bias),
+                                             _lib.ptr(post_in), _lib.ptr(post_in2), y.data_ptr(), M, N, K,
+                                             post, post_scale, flags, ws.data_ptr(), ws.numel(),
+                                             row_sumsq.data_ptr(), st))
+    elif weight._qscheme == QSCHEME_MXFP:
         _lib.check(L.tppx_linear_mxfp4(x.data_ptr(), qn.data_ptr(), sn.data_ptr(), _lib.ptr(bias),
                                        _lib.ptr(post_in), _lib.ptr(post_in2), y.data_ptr(), M, N, K,
                                        post, post_scale, flags, ws.data_ptr(), ws.numel(), st))
@@ -330,9 +340,9 @@ def fc_plain(input, weight, bias, parallel_dim=-1, split_sizes=()):
     return linear(input, weight, bias, POST_NONE)
 
 
-def fc_add(input, weight, bias, residual, scale=1.0):
+def fc_add(input, weight, bias, residual, scale=1.0, row_sumsq=None):
     """GEMM + AddScalePostOp(residual, scale) (fused_llm_infer.cpp:1261,1273)."""
-    return linear(input, weight, bias, POST_ADD_SCALE, residual, None, scale)
+    return linear(input, weight, bias, POST_ADD_SCALE, residual, None, scale, row_sumsq=row_sumsq)
 
 
 def fc_add2(input, weight, bias, residual1, residual2, scale=1.0):
@@ -381,13 +391,43 @@ def rms_norm(t_in, t_wt, eps):
 FUSE_NORM = os.environ.get("TPPX_FUSE_NORM", "0") == "1"
 
 
-def _norm_fusable(norm, scheme, M, K):
-    """RMSNorm can ride inside the GEMM launch for MXFP4 decode steps (<= 16 rows, the LDS staging fits)."""
-    if norm is None or not FUSE_NORM:
-        return False
-    gamma, _ = norm
+# RMSNorm scale from row sums of squares that the GEMM which wrote the activations left behind
+# (tppx_linear_mxfp4_rowsq -> tppx_normsq_*): no normalisation launch and no pass over the row.  On by default;
+# TPPX_NORM_FROM_SUMS=0 goes back to the separate normalisation kernel.
+NORM_FROM_SUMS = os.environ.get("TPPX_NORM_FROM_SUMS", "1") == "1"
+
+
+def sums_table(device):
+    """A table for the row sums of squares of one activation tensor: f32 [16][256]."""
+    return torch.zeros((16, 256), dtype=torch.float32, device=device)
+
+
+def takes_row_sums(weight, M):
+    """Can the GEMM with this weight leave row sums of squares of its output (MXFP4 decode kernels, <= 16 rows,
+    at most 256 workgroups of up to three channel tiles: 12288 output channels)?"""
+    w = _as_q(weight)
+    return NORM_FROM_SUMS and w._qscheme == QSCHEME_MXFP and 0 < M <= 16 and w.weight_nk()[0] <= 12288
+
+
+def _norm_fits(norm, scheme, M, K):
+    gamma = norm[0]
     return (scheme == QSCHEME_MXFP and 0 < M <= 16 and K % 128 == 0 and (K == 4096 or K == 2048 or K <= 2048)
             and gamma.dtype == torch.float32 and gamma.is_cuda and gamma.is_contiguous())
+
+
+def _norm_fusable(norm, scheme, M, K):
+    """RMSNorm can ride inside the GEMM launch for MXFP4 decode steps (<= 16 rows, the LDS staging fits): always
+    when the row sums of squares are handed over (norm = (gamma, eps, table)), otherwise only with TPPX_FUSE_NORM."""
+    if norm is None:
+        return False
+    handed = len(norm) > 2 and norm[2] is not None
+    if not (handed and NORM_FROM_SUMS) and not FUSE_NORM:
+        return False
+    return _norm_fits(norm, scheme, M, K)
+
+
+def _norm_table(norm):
+    return norm[2] if (len(norm) > 2 and norm[2] is not None and NORM_FROM_SUMS) else None
 
 
 def qkv_gemm(input, weights, biases, norm=None):
@@ -433,7 +473,10 @@ def qkv_gemm(input, weights, biases, norm=None):
         return outs
     st = _lib.stream_of(x)
     ws = _lib.workspace(x)
-    if scheme == QSCHEME_MXFP and norm is not None:
+    if scheme == QSCHEME_MXFP and norm is not None and _norm_table(norm) is not None:
+        _lib.check(L.tppx_normsq_multi_linear_mxfp4(x.data_ptr(), _norm_table(norm).data_ptr(), norm[0].data_ptr(),
+                                                    float(norm[1]), segs, n, M, K, 0, st))
+    elif scheme == QSCHEME_MXFP and norm is not None:
         _lib.check(L.tppx_norm_multi_linear_mxfp4(x.data_ptr(), norm[0].data_ptr(), float(norm[1]), segs, n, M, K, 0, st))
     elif scheme == QSCHEME_MXFP:
         _lib.check(L.tppx_multi_linear_mxfp4(x.data_ptr(), segs, n, M, K, 0, ws.data_ptr(), ws.numel(), st))
@@ -468,6 +511,12 @@ def swiglu_gate_up(input, w_gate, w_up, b_gate=None, b_up=None, norm=None):
     bu = _prep_bias(b_up, N, x.device)
     qg, sg = w_gate.native()
     qu, su = w_up.native()
+    if norm is not None and _norm_table(norm) is not None:
+        _lib.check(L.tppx_normsq_swiglu_mxfp4(x.data_ptr(), _norm_table(norm).data_ptr(), norm[0].data_ptr(),
+                                              float(norm[1]), qg.data_ptr(), sg.data_ptr(), _lib.ptr(bg),
+                                              qu.data_ptr(), su.data_ptr(), _lib.ptr(bu), y.data_ptr(), M, N, K, 0,
+                                              _lib.stream_of(x)))
+        return y
     if norm is not None:
         _lib.check(L.tppx_norm_swiglu_mxfp4(x.data_ptr(), norm[0].data_ptr(), float(norm[1]), qg.data_ptr(), sg.data_ptr(),
                                             _lib.ptr(bg), qu.data_ptr(), su.data_ptr(), _lib.ptr(bu), y.data_ptr(),

@@ -59,6 +59,10 @@ class TppCache:
         self.layers = {}          # layer_idx -> (k, v)
         self.seq_len_dev = None   # int32 [1]: keys in the cache (same for every layer)
         self._host_len = 0
+        # decode steps: row sums of squares of the residual stream, handed from the GEMM that writes it to the
+        # GEMM behind the next RMSNorm (two tables: after attention, after the MLP) + the tensor the second belongs to
+        self._sums = None
+        self._sums_of = None
 
     # -- reference method names -------------------------------------------------
     def get_seq_length(self, layer_idx=0):
@@ -144,8 +148,17 @@ class LlamaDecoderLayer:
         st = _lib.stream_of(t_HS)
         empty = torch.empty(0, dtype=torch.bfloat16, device=t_HS.device)
         t_res = t_HS
-        # input RMSNorm + q/k/v GEMMs (one launch for MXFP4 decode steps)
-        q, k, v = _ops.qkv_gemm(t_HS, [self.t_Wq, self.t_Wk, self.t_Wv], [empty] * 3, norm=(self.t_Gi, self.eps))
+        # Decode steps on MXFP4 weights: the o- and down-projection launches leave the row sums of squares of the
+        # residual stream, so the RMSNorm behind them is a scale applied while the next GEMM stages its input.
+        M = B * S
+        if cache._sums is None:
+            cache._sums = (_ops.sums_table(t_HS.device), _ops.sums_table(t_HS.device))
+        sums_attn = cache._sums[0] if _ops.takes_row_sums(self.t_Wp, M) else None
+        sums_out = cache._sums[1] if _ops.takes_row_sums(self.t_Wd, M) else None
+        sums_in = cache._sums[1] if cache._sums_of is t_HS else None
+        # input RMSNorm + q/k/v GEMMs
+        q, k, v = _ops.qkv_gemm(t_HS, [self.t_Wq, self.t_Wk, self.t_Wv], [empty] * 3,
+                                norm=(self.t_Gi, self.eps, sums_in))
         kc, vc = cache._ensure(self.layer_idx, B, self.Nkv, self.H, t_HS.device)
         # rotary on q and k + append of k, v at position seq_len (device counter), one launch
         _lib.check(L.tppx_rotary_kv_append_llama(
@@ -165,10 +178,11 @@ class LlamaDecoderLayer:
             _lib.check(L.tppx_attn_prefill(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
                                            cache.get_seq_length(), ctx.data_ptr(), B, S, self.Nq, self.Nkv, self.H,
                                            cache.capacity, st))
-        t_SO = _ops.fc_add(ctx, self.t_Wp, empty, t_res, 1.0)
+        t_SO = _ops.fc_add(ctx, self.t_Wp, empty, t_res, 1.0, row_sumsq=sums_attn)
         # post-attention RMSNorm + gate/up GEMMs + silu*mul
-        t_I = _ops.swiglu_gate_up(t_SO, self.t_Wg, self.t_Wu, norm=(self.t_Gpa, self.eps))
-        t_Out = _ops.fc_add(t_I, self.t_Wd, empty, t_SO, 1.0)
+        t_I = _ops.swiglu_gate_up(t_SO, self.t_Wg, self.t_Wu, norm=(self.t_Gpa, self.eps, sums_attn))
+        t_Out = _ops.fc_add(t_I, self.t_Wd, empty, t_SO, 1.0, row_sumsq=sums_out)
+        cache._sums_of = t_Out if sums_out is not None else None
         return [t_Out]
 
 
