@@ -302,6 +302,22 @@ int tppx_attn_decode(const void* q, const void* kcache, const void* vcache,
                      int64_t Smax, void* ws, int64_t ws_bytes,
                      tppx_stream_t stream);
 
+/* The same with the launch in front of it folded in: tppx_rotary_kv_append_llama
+ * for one token per sequence followed by tppx_attn_decode with kv_len_add = 1
+ * (fused_llm_infer.cpp:1252-1253, attn.h:198-222, attn.cpp:781-955).  q bf16
+ * [B][Nq][128], k / v bf16 [B][Nkv][128] as the q/k/v GEMMs leave them
+ * (unrotated; they stay untouched), emb_pos f32 [2][MP][128] or NULL (append
+ * without rotation), pos i64 [B_pos] with B_pos 1 or B; the rotated key and the
+ * value are written to cache position *kv_len_dev (nothing is written when the
+ * cache is full) and attended to together with the cached keys. */
+int tppx_attn_decode_rotary(const void* q, const void* k, const void* v,
+                            const void* emb_pos, const void* pos, int64_t B_pos,
+                            int64_t MP, int64_t HR, void* kcache, void* vcache,
+                            const void* mask, int64_t mask_ld,
+                            const void* kv_len_dev, void* out, int64_t B,
+                            int64_t Nq, int64_t Nkv, int64_t H, int64_t Smax,
+                            void* ws, int64_t ws_bytes, tppx_stream_t stream);
+
 /* The same attn<T> (src/csrc/llm/attn.cpp:781-955, isCausal) for S query tokens
  * per sequence (prompt processing, or several new tokens on a filled cache):
  * q / out bf16 [B][S][Nq][128]; the cache already holds the S new keys at

@@ -113,6 +113,59 @@ def test_attn_decode_split_merge_in_launch_equals_second_kernel(monkeypatch):
         assert torch.equal(o, two)
 
 
+@pytest.mark.parametrize("B,Nq,Nkv,L0,Smax,B_pos", [(1, 32, 32, 2048, 2304, 1), (3, 8, 2, 300, 512, 3), (2, 4, 4, 0, 64, 1),
+                                                     (16, 32, 32, 77, 128, 16)])
+def test_attn_decode_with_rotary_and_append_in_the_launch(B, Nq, Nkv, L0, Smax, B_pos):
+    """tppx_attn_decode_rotary = tppx_rotary_kv_append_llama + tppx_attn_decode(kv_len_add = 1) in one launch: same
+    attention output (the rotation may contract its multiply-adds differently: bf16 tolerance), the same key / value
+    row appended at position L0, nothing else in the cache touched, q / k / v inputs left as they were."""
+    F = _llm()
+    from tpp_pytorch_extension import _lib
+    Lb = _lib.lib()
+    MP = 4096
+    EP = F.llama_rotary_table(MP, 128)
+    q = randn_bf16((B, 1, Nq * 128), 1.0, 91).cuda()
+    k = randn_bf16((B, 1, Nkv * 128), 1.0, 92).cuda()
+    v = randn_bf16((B, 1, Nkv * 128), 1.0, 93).cuda()
+    kc0 = randn_bf16((B, Nkv, Smax, 128), 1.0, 94).cuda()
+    vc0 = randn_bf16((B, Nkv, Smax, 128), 1.0, 95).cuda()
+    pos = (torch.arange(B_pos, dtype=torch.int64) * 3 + L0).view(B_pos, 1).cuda()
+    ln = torch.tensor([L0], dtype=torch.int32, device="cuda")
+    st = _lib.stream_of(q)
+    w = _lib.workspace(q)
+    # two launches
+    qa, ka, kca, vca = q.clone(), k.clone(), kc0.clone(), vc0.clone()
+    _lib.check(Lb.tppx_rotary_kv_append_llama(qa.data_ptr(), ka.data_ptr(), v.data_ptr(), EP.data_ptr(), pos.data_ptr(),
+                                              kca.data_ptr(), vca.data_ptr(), ln.data_ptr(), B, 1, Nq, Nkv, 128, MP, 128,
+                                              B_pos, Smax, st))
+    outa = torch.empty((B, Nq, 128), dtype=torch.bfloat16, device="cuda")
+    _lib.check(Lb.tppx_attn_decode(qa.data_ptr(), kca.data_ptr(), vca.data_ptr(), None, 0, ln.data_ptr(), 1,
+                                   outa.data_ptr(), B, Nq, Nkv, 128, Smax, w.data_ptr(), w.numel(), st))
+    # one launch
+    qb, kb, vb, kcb, vcb = q.clone(), k.clone(), v.clone(), kc0.clone(), vc0.clone()
+    outb = torch.empty_like(outa)
+    _lib.check(Lb.tppx_attn_decode_rotary(qb.data_ptr(), kb.data_ptr(), vb.data_ptr(), EP.data_ptr(), pos.data_ptr(), B_pos,
+                                          MP, 128, kcb.data_ptr(), vcb.data_ptr(), None, 0, ln.data_ptr(), outb.data_ptr(),
+                                          B, Nq, Nkv, 128, Smax, w.data_ptr(), w.numel(), st))
+    torch.cuda.synchronize()
+    assert torch.equal(qb, q) and torch.equal(kb, k) and torch.equal(vb, v)
+    assert_close_bf16(t2bits(kcb[:, :, L0]), t2bits(kca[:, :, L0]), what="appended key")
+    assert torch.equal(vcb[:, :, L0], vca[:, :, L0])
+    keep = torch.ones(Smax, dtype=torch.bool)
+    keep[L0] = False
+    assert torch.equal(kcb[:, :, keep], kc0[:, :, keep]) and torch.equal(vcb[:, :, keep], vc0[:, :, keep])
+    a, b = outa.double(), outb.double()
+    assert float((a - b).norm() / a.norm()) <= 5e-3
+    assert float((a - b).abs().max()) <= 2.0 ** -7 * float(a.abs().max())
+    # a full cache: nothing is written, the cached keys are attended to
+    full = torch.tensor([Smax], dtype=torch.int32, device="cuda")
+    _lib.check(Lb.tppx_attn_decode_rotary(qb.data_ptr(), kb.data_ptr(), vb.data_ptr(), EP.data_ptr(), pos.data_ptr(), B_pos,
+                                          MP, 128, kcb.data_ptr(), vcb.data_ptr(), None, 0, full.data_ptr(), outb.data_ptr(),
+                                          B, Nq, Nkv, 128, Smax, w.data_ptr(), w.numel(), st))
+    torch.cuda.synchronize()
+    assert torch.equal(kcb[:, :, keep], kc0[:, :, keep]) and torch.isfinite(outb.float()).all()
+
+
 def test_attn_decode_mask():
     F = _llm()
     B, Nq, L, Smax = 2, 4, 100, 128

@@ -191,6 +191,12 @@ struct AttnParams {
   int B, Nq, Nkv, Smax, mask_ld, splits;
   int ticket0;          // >= 0: first arrival counter of this launch (the last split to arrive merges); < 0: second kernel
   float scale;
+  // ROT: the query and the step's new key / value arrive unrotated and not yet in the cache
+  const uint16_t* k_new; // [B][Nkv][128]
+  const uint16_t* v_new; // [B][Nkv][128]
+  const float* emb;      // f32 [2][MP][128] cos / sin
+  const int64_t* pos;    // i64 [B_pos] position of the new token
+  int MP, B_pos;
 };
 
 // Arrival counters of the split launches, one per (sequence, head): zero between launches (the counting
@@ -202,6 +208,11 @@ __device__ __forceinline__ uint4 as_uint4(const i32x4& v) {
   return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
 }
 
+// ROT: the launch also does what the rotary + append launch did before it (fused_llm_infer.cpp:1252-1253 and
+// LayerCache::update, attn.h:198-222): q and the new key arrive unrotated, every workgroup rotates its query, the
+// key / value of the new token (cache position *kv_len) are taken from registers wherever that position is read,
+// and one workgroup per KV head writes them into the cache.  Rotated values are rounded to bf16 first, as stored.
+template <bool ROT>
 __global__ void __launch_bounds__(256)
 attn_decode_kernel(const AttnParams p) {
   __shared__ float sm[16], sl[16];
@@ -210,13 +221,64 @@ attn_decode_kernel(const AttnParams p) {
   const int g = lane >> 4, c = lane & 15;
   const int bh = blockIdx.x, b = bh / p.Nq, hq = bh - b * p.Nq;
   const int hk = hq / (p.Nq / p.Nkv);
-  const int L = max(0, min(*p.kv_len + p.kv_len_add, p.Smax));
+  const int len0 = *p.kv_len;
+  const int L = max(0, min(len0 + p.kv_len_add, p.Smax));
+  const int nk = (ROT && len0 >= 0 && len0 < p.Smax) ? len0 : -1; // cache position of the new token
   // this workgroup's keys: [k0, k1), split evenly in multiples of 64
   const int per = ((L + p.splits - 1) / p.splits + 63) & ~63;
   const int k0 = blockIdx.y * per, k1 = min(k0 + per, L);
 
   float qf[8];
-  unpack8(reinterpret_cast<const uint4*>(p.q + (int64_t)bh * 128)[c], qf);
+  i32x4 knew = {0, 0, 0, 0}, vnew = {0, 0, 0, 0};
+  if (!ROT) {
+    unpack8(reinterpret_cast<const uint4*>(p.q + (int64_t)bh * 128)[c], qf);
+  } else {
+    // chunk c holds first halves (c < 8) or second halves of the rotation pairs (h2, 64 + h2); partner chunk c ^ 8
+    const bool first = c < 8;
+    const int64_t pp = p.pos[p.B_pos == 1 ? 0 : b];
+    const bool rot = p.emb != nullptr && pp < p.MP;
+    float cs[8], sn[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      cs[e] = sn[e] = 0.f;
+    if (rot) {
+      const float* cp = p.emb + pp * 128 + (c & 7) * 8;
+      const float* sp = p.emb + ((int64_t)p.MP + pp) * 128 + (c & 7) * 8;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        cs[e] = cp[e];
+        sn[e] = sp[e];
+      }
+    }
+    auto rotate = [&](const uint16_t* row, float (&r)[8]) -> uint4 {
+      const uint4 w = reinterpret_cast<const uint4*>(row)[c];
+      if (!rot) {
+        unpack8(w, r);
+        return w;
+      }
+      const uint4 wo = reinterpret_cast<const uint4*>(row)[c ^ 8];
+      float a[8], o[8];
+      unpack8(w, a);
+      unpack8(wo, o);
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        r[e] = first ? a[e] * cs[e] - o[e] * sn[e] : a[e] * cs[e] + o[e] * sn[e];
+      const uint4 out = pack8(r);
+      unpack8(out, r); // the rotated row is a bf16 tensor
+      return out;
+    };
+    rotate(p.q + (int64_t)bh * 128, qf);
+    float kr[8];
+    const uint4 kw4 = rotate(p.k_new + ((int64_t)b * p.Nkv + hk) * 128, kr);
+    knew = i32x4{(int)kw4.x, (int)kw4.y, (int)kw4.z, (int)kw4.w};
+    vnew = *reinterpret_cast<const i32x4*>(p.v_new + ((int64_t)b * p.Nkv + hk) * 128 + c * 8);
+    // one workgroup per KV head appends: the first query head of the group, the split that owns the position
+    if (nk >= 0 && hq == hk * (p.Nq / p.Nkv) && nk >= k0 && nk < k1 && tid < 16) {
+      const int64_t o = (((int64_t)b * p.Nkv + hk) * p.Smax + nk) * 128 + c * 8;
+      *reinterpret_cast<i32x4*>(const_cast<uint16_t*>(p.kc) + o) = knew;
+      *reinterpret_cast<i32x4*>(const_cast<uint16_t*>(p.vc) + o) = vnew;
+    }
+  }
 #pragma unroll
   for (int e = 0; e < 8; e++)
     qf[e] *= p.scale;
@@ -238,6 +300,10 @@ attn_decode_kernel(const AttnParams p) {
       const int kk = max(min(base + u * 4 + g, L - 1), 0);
       kd[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(kb + (int64_t)kk * 16));
       vd[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(vb + (int64_t)kk * 16));
+      if (ROT && kk == nk) { // not in the cache yet (or being written by another workgroup right now)
+        kd[u] = knew;
+        vd[u] = vnew;
+      }
     }
   };
   load_kv(k0 + wave * (4 * NU), kw, vw);
@@ -648,24 +714,9 @@ extern "C" int tppx_rotary_kv_append_llama(void* q, void* k, const void* v, cons
   return rotary_common(who, p, (hipStream_t)stream);
 }
 
-extern "C" int tppx_attn_decode(const void* q, const void* kcache, const void* vcache, const void* mask,
-                                int64_t mask_ld, const void* kv_len_dev, int64_t kv_len_add, void* out, int64_t B, int64_t Nq,
-                                int64_t Nkv, int64_t H, int64_t Smax, void* ws, int64_t ws_bytes,
-                                tppx_stream_t stream) {
-  const char* who = "tppx_attn_decode";
-  TPPX_REQUIRE(q && kcache && vcache && kv_len_dev && out, TPPX_EINVAL, "%s: null pointer", who);
-  TPPX_REQUIRE(aligned16(q) && aligned16(kcache) && aligned16(vcache) && aligned16(out), TPPX_EINVAL,
-               "%s: pointer not 16-byte aligned", who);
-  TPPX_REQUIRE(H == 128, TPPX_EUNSUPPORTED, "%s: head size %ld (only 128 is built)", who, (long)H);
-  TPPX_REQUIRE(B > 0 && Nq > 0 && Nkv > 0 && Nq % Nkv == 0 && Smax > 0 && B * Nq < (1 << 30), TPPX_ESHAPE,
-               "%s: bad shape B=%ld Nq=%ld Nkv=%ld Smax=%ld", who, (long)B, (long)Nq, (long)Nkv, (long)Smax);
-  TPPX_REQUIRE(ws_bytes >= 0 && (ws_bytes == 0 || ws), TPPX_EINVAL, "%s: workspace size given with a null workspace", who);
-  AttnParams p;
-  memset(&p, 0, sizeof(p));
-  p.q = (const uint16_t*)q; p.kc = (const uint16_t*)kcache; p.vc = (const uint16_t*)vcache;
-  p.mask = (const uint16_t*)mask; p.kv_len = (const int32_t*)kv_len_dev; p.kv_len_add = (int)kv_len_add; p.out = (uint16_t*)out;
-  p.B = (int)B; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.Smax = (int)Smax; p.mask_ld = (int)mask_ld;
-  p.scale = 1.0f / sqrtf((float)H);
+// shared tail of the two single-query entry points: split planning, counters, launch
+static int attn_decode_launch(const char* who, AttnParams& p, bool rot, int64_t B, int64_t Nq, int64_t Smax, void* ws,
+                              int64_t ws_bytes, hipStream_t stream) {
   // enough workgroups to cover the chip about twice, at least 256 keys per split
   const int64_t target = env_int("TPPX_ATTN_TARGET_WGS", 512), min_keys = env_int("TPPX_ATTN_MIN_KEYS", 256);
   int64_t splits = (target + B * Nq - 1) / (B * Nq);
@@ -691,12 +742,65 @@ extern "C" int tppx_attn_decode(const void* q, const void* kcache, const void* v
     p.ticket0 = cursor;
     cursor += (int)(B * Nq);
   }
-  attn_decode_kernel<<<dim3((unsigned)(B * Nq), (unsigned)splits), dim3(256), 0, (hipStream_t)stream>>>(p);
+  const dim3 grid((unsigned)(B * Nq), (unsigned)splits);
+  if (rot)
+    attn_decode_kernel<true><<<grid, dim3(256), 0, stream>>>(p);
+  else
+    attn_decode_kernel<false><<<grid, dim3(256), 0, stream>>>(p);
   int rc = check_hip(hipGetLastError(), who);
   if (rc || splits == 1 || p.ticket0 >= 0)
     return rc;
-  attn_combine_kernel<<<dim3((unsigned)(B * Nq)), dim3(128), 0, (hipStream_t)stream>>>(p);
+  attn_combine_kernel<<<dim3((unsigned)(B * Nq)), dim3(128), 0, stream>>>(p);
   return check_hip(hipGetLastError(), who);
+}
+
+extern "C" int tppx_attn_decode(const void* q, const void* kcache, const void* vcache, const void* mask,
+                                int64_t mask_ld, const void* kv_len_dev, int64_t kv_len_add, void* out, int64_t B, int64_t Nq,
+                                int64_t Nkv, int64_t H, int64_t Smax, void* ws, int64_t ws_bytes,
+                                tppx_stream_t stream) {
+  const char* who = "tppx_attn_decode";
+  TPPX_REQUIRE(q && kcache && vcache && kv_len_dev && out, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(aligned16(q) && aligned16(kcache) && aligned16(vcache) && aligned16(out), TPPX_EINVAL,
+               "%s: pointer not 16-byte aligned", who);
+  TPPX_REQUIRE(H == 128, TPPX_EUNSUPPORTED, "%s: head size %ld (only 128 is built)", who, (long)H);
+  TPPX_REQUIRE(B > 0 && Nq > 0 && Nkv > 0 && Nq % Nkv == 0 && Smax > 0 && B * Nq < (1 << 30), TPPX_ESHAPE,
+               "%s: bad shape B=%ld Nq=%ld Nkv=%ld Smax=%ld", who, (long)B, (long)Nq, (long)Nkv, (long)Smax);
+  TPPX_REQUIRE(ws_bytes >= 0 && (ws_bytes == 0 || ws), TPPX_EINVAL, "%s: workspace size given with a null workspace", who);
+  AttnParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = (const uint16_t*)q; p.kc = (const uint16_t*)kcache; p.vc = (const uint16_t*)vcache;
+  p.mask = (const uint16_t*)mask; p.kv_len = (const int32_t*)kv_len_dev; p.kv_len_add = (int)kv_len_add; p.out = (uint16_t*)out;
+  p.B = (int)B; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.Smax = (int)Smax; p.mask_ld = (int)mask_ld;
+  p.scale = 1.0f / sqrtf((float)H);
+  return attn_decode_launch(who, p, false, B, Nq, Smax, ws, ws_bytes, (hipStream_t)stream);
+}
+
+extern "C" int tppx_attn_decode_rotary(const void* q, const void* k, const void* v, const void* emb_pos,
+                                       const void* pos, int64_t B_pos, int64_t MP, int64_t HR, void* kcache,
+                                       void* vcache, const void* mask, int64_t mask_ld, const void* kv_len_dev,
+                                       void* out, int64_t B, int64_t Nq, int64_t Nkv, int64_t H, int64_t Smax,
+                                       void* ws, int64_t ws_bytes, tppx_stream_t stream) {
+  const char* who = "tppx_attn_decode_rotary";
+  TPPX_REQUIRE(q && k && v && pos && kcache && vcache && kv_len_dev && out, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(kcache) && aligned16(vcache) && aligned16(out) &&
+                   (!emb_pos || aligned16(emb_pos)),
+               TPPX_EINVAL, "%s: pointer not 16-byte aligned", who);
+  TPPX_REQUIRE(H == 128 && (!emb_pos || HR == 128), TPPX_EUNSUPPORTED,
+               "%s: head size %ld / rotary size %ld (only 128 with a full-width rotation is built)", who, (long)H, (long)HR);
+  TPPX_REQUIRE(B > 0 && Nq > 0 && Nkv > 0 && Nq % Nkv == 0 && Smax > 0 && B * Nq < (1 << 30) && (B_pos == 1 || B_pos == B) &&
+                   (!emb_pos || MP > 0),
+               TPPX_ESHAPE, "%s: bad shape B=%ld Nq=%ld Nkv=%ld Smax=%ld B_pos=%ld MP=%ld", who, (long)B, (long)Nq,
+               (long)Nkv, (long)Smax, (long)B_pos, (long)MP);
+  TPPX_REQUIRE(ws_bytes >= 0 && (ws_bytes == 0 || ws), TPPX_EINVAL, "%s: workspace size given with a null workspace", who);
+  AttnParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = (const uint16_t*)q; p.kc = (const uint16_t*)kcache; p.vc = (const uint16_t*)vcache;
+  p.mask = (const uint16_t*)mask; p.kv_len = (const int32_t*)kv_len_dev; p.kv_len_add = 1; p.out = (uint16_t*)out;
+  p.B = (int)B; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.Smax = (int)Smax; p.mask_ld = (int)mask_ld;
+  p.scale = 1.0f / sqrtf((float)H);
+  p.k_new = (const uint16_t*)k; p.v_new = (const uint16_t*)v; p.emb = (const float*)emb_pos; p.pos = (const int64_t*)pos;
+  p.MP = (int)MP; p.B_pos = (int)B_pos;
+  return attn_decode_launch(who, p, true, B, Nq, Smax, ws, ws_bytes, (hipStream_t)stream);
 }
 
 extern "C" int tppx_attn_prefill(const void* q, const void* kcache, const void* vcache, const void* mask,

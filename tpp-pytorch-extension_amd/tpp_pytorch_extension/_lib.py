@@ -68,6 +68,7 @@ SIGNATURES = {
     "tppx_rotary_kv_append_llama": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                     _i64, _i64, _vp],
     "tppx_attn_decode": [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp],
+    "tppx_attn_decode_rotary": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp],
     "tppx_attn_prefill": [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     "tppx_plan_linear_mxfp4": [_i64, _i64, _i64, _i32, _i64, ctypes.c_char_p, _i64],
     "tppx_plan_linear_qint8": [_i64, _i64, _i64, _i64, _i32, _i32, _i64, ctypes.c_char_p, _i64],

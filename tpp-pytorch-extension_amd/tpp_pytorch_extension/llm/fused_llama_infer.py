@@ -34,6 +34,9 @@ def _bf16_cuda(t, name):
 
 rms_norm = _ops.rms_norm  # llama_rms_norm (fused_llm_infer.cpp:337-363)
 
+# decode steps: rotary embedding + cache append inside the attention launch (TPPX_FUSE_ROTARY=0: separate launch)
+FUSE_ROTARY = os.environ.get("TPPX_FUSE_ROTARY", "1") == "1"
+
 
 def apply_rotary_pos_emb_llama(t_in, t_emb_pos, t_pos, N, H):
     """In place on t_in [B][S][N*H] (fused_llm_infer.cpp:207-253); t_emb_pos f32 [2][MP][HR]; t_pos i64 [B_pos][S]."""
@@ -160,6 +163,18 @@ class LlamaDecoderLayer:
         q, k, v = _ops.qkv_gemm(t_HS, [self.t_Wq, self.t_Wk, self.t_Wv], [empty] * 3,
                                 norm=(self.t_Gi, self.eps, sums_in))
         kc, vc = cache._ensure(self.layer_idx, B, self.Nkv, self.H, t_HS.device)
+        ws = _lib.workspace(t_HS)
+        mask_ptr = t_am.data_ptr() if t_am is not None and t_am.numel() else None
+        mask_ld = t_am.shape[-1] if mask_ptr else 0
+        if S == 1 and FUSE_ROTARY and self.H == 128 and self.t_EP.shape[2] == 128:
+            # decode step: rotary, cache append and attention in one launch
+            ctx = torch.empty_like(q)
+            _lib.check(L.tppx_attn_decode_rotary(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), self.t_EP.data_ptr(), t_pid.data_ptr(), t_pid.shape[0],
+                self.t_EP.shape[1], self.t_EP.shape[2], kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
+                cache.seq_len_dev.data_ptr(), ctx.data_ptr(), B, self.Nq, self.Nkv, self.H, cache.capacity,
+                ws.data_ptr(), ws.numel(), st))
+            return self._after_attention(ctx, t_res, empty, cache, sums_attn, sums_out)
         # rotary on q and k + append of k, v at position seq_len (device counter), one launch
         _lib.check(L.tppx_rotary_kv_append_llama(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), self.t_EP.data_ptr(), t_pid.data_ptr(), kc.data_ptr(),
@@ -167,9 +182,6 @@ class LlamaDecoderLayer:
             self.t_EP.shape[2], t_pid.shape[0], cache.capacity, st))
         # attention over the cached keys + the new ones
         ctx = torch.empty_like(q)
-        ws = _lib.workspace(t_HS)
-        mask_ptr = t_am.data_ptr() if t_am is not None and t_am.numel() else None
-        mask_ld = t_am.shape[-1] if mask_ptr else 0
         if S == 1:
             _lib.check(L.tppx_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
                                           cache.seq_len_dev.data_ptr(), 1, ctx.data_ptr(), B, self.Nq, self.Nkv, self.H,
@@ -178,6 +190,9 @@ class LlamaDecoderLayer:
             _lib.check(L.tppx_attn_prefill(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
                                            cache.get_seq_length(), ctx.data_ptr(), B, S, self.Nq, self.Nkv, self.H,
                                            cache.capacity, st))
+        return self._after_attention(ctx, t_res, empty, cache, sums_attn, sums_out)
+
+    def _after_attention(self, ctx, t_res, empty, cache, sums_attn, sums_out):
         t_SO = _ops.fc_add(ctx, self.t_Wp, empty, t_res, 1.0, row_sumsq=sums_attn)
         # post-attention RMSNorm + gate/up GEMMs + silu*mul
         t_I = _ops.swiglu_gate_up(t_SO, self.t_Wg, self.t_Wu, norm=(self.t_Gpa, self.eps, sums_attn))
