@@ -184,7 +184,7 @@ tiled_mxfp4_kernel(const TiledParams p) {
 // [mt 8][t 2][lane 64] x 16 B (16 KiB) + the activation scales of the step's
 // K block for the 128 rows.
 // ---------------------------------------------------------------------------
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2) // two workgroups per CU: without the bound the compiler spreads into 327 registers, one wave per SIMD
 tiled_qint8_kernel(const TiledParams p) {
   extern __shared__ __align__(16) uint8_t tl_lds[];
   i32x4* As = reinterpret_cast<i32x4*>(tl_lds);                 // 2 x 1024 slots
