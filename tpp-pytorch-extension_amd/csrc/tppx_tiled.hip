@@ -561,6 +561,201 @@ big_mxfp4_kernel(const BigParams P) {
   big_epilogue<MT>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
 }
 
+// ---------------------------------------------------------------------------
+// Large-M QINT8 (W8A8, 256-wide blocks): 128 x 256 workgroup tile, 8 waves
+// (2 x 4), wave tile 64 x 64, K step 256 = one scale block in two halves.
+// What bounds int8 at this size is operand delivery, not the MFMA: weights are
+// 4x the bytes of MXFP4 per MAC, the MFMA runs at twice the bf16 rate, and the
+// two accumulator sets (int32 block sums, fp32 running sums) leave no room for
+// a second set of weight registers.  So BOTH operands go from global memory
+// straight into LDS (no staging registers, nothing for the compiler to wait
+// on before the barrier), each weight tile is fetched once per workgroup
+// instead of once per wave row, and LDS (about twice the bandwidth of the
+// vector memory path) feeds the MFMAs:
+//   A: int8 rows, 256 B per row and K step, the layout, swizzle and operand
+//      reads of the MXFP4 kernel above (the operand of MFMA step j is chunk
+//      j*4 + g of the row); two buffers of 32 KiB, loaded a step ahead.
+//   B: native 1 KiB tiles (16 channels x 64 K, lane-linear = MFMA operand
+//      order), 16 tiles x 2 K tiles = 32 KiB per half step, two buffers,
+//      loaded half a step ahead; a lane reads its own 16 bytes, no conflicts.
+//   int32 block sums (exact) are folded into fp32 at the end of every step
+//   with sa[m] * sw[n]; the activation scales of a step reach the waves
+//   through LDS, requested two steps ahead.
+// LDS: A 2 x 32 KiB | B 2 x 32 KiB | scales 2 KiB (the epilogue staging reuses it).
+// ---------------------------------------------------------------------------
+template <int N>
+__device__ __forceinline__ void lds_wait_keep8(i32x4& r, i32x4 (&b)[4][2]) {
+  asm volatile("s_waitcnt lgkmcnt(%9)"
+               : "+v"(r), "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[1][0]), "+v"(b[1][1]), "+v"(b[2][0]), "+v"(b[2][1]),
+                 "+v"(b[3][0]), "+v"(b[3][1])
+               : "n"(N));
+}
+
+__global__ void __launch_bounds__(512)
+big_qint8_kernel(const TiledParams p) {
+  constexpr int MT = 4, WGM = 128, ABUF = WGM * 256, BBUF = 32 * 1024;
+  extern __shared__ __align__(16) uint8_t tl_lds[];
+  uint8_t* b_lds = tl_lds + 2 * ABUF;
+  float* sa_s = reinterpret_cast<float*>(tl_lds + 2 * ABUF + 2 * BBUF); // [4][128]: scales of steps ks .. ks+2 (mod 4)
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+  const int MB = (p.M + WGM - 1) / WGM, NB = (p.tiles + 15) >> 4;
+  int bm, bn;
+  tile_of_block(MB, NB, bm, bn);
+  const int KS = p.K >> 8;   // K steps = scale blocks
+  const int KT64 = p.K >> 6; // native tiles along K
+  const int m_wg = bm * WGM;
+  const int tile_base = bn * 16 + wn * 4;
+
+  const float* swp = reinterpret_cast<const float*>(p.sw);
+  uint32_t soff[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; nt++)
+    soff[nt] = (uint32_t)(min(tile_base + nt, p.tiles - 1) * KS * 16 + (lane & 15));
+  const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>(tl_lds);
+  uint32_t rdb[4];
+  {
+    const int m = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      rdb[j] = (uint32_t)((m >> 2) * 1024 + (m & 3) * 256 + (((j * 4 + g) ^ m) & 15) * 16);
+  }
+  const char* xbase = reinterpret_cast<const char*>(p.xq);
+  const int rin = lane >> 4, ch = lane & 15;
+  const bool full = m_wg + WGM <= p.M;
+  const uint32_t xrow0 = (uint32_t)((m_wg + wave * (MT * 4) + rin) * p.K);
+  const uint32_t blk_stride = (uint32_t)(4 * p.K);
+  auto load_a = [&](int ks, int buf) {
+#pragma unroll
+    for (int i = 0; i < MT; i++) {
+      const uint32_t sw = (uint32_t)((ch ^ ((i & 3) * 4 + rin)) & 15) * 16u;
+      uint32_t off;
+      if (full) {
+        off = xrow0 + (uint32_t)i * blk_stride + sw + (uint32_t)ks * 256u;
+      } else {
+        const int row = min(m_wg + (wave * MT + i) * 4 + rin, p.M - 1);
+        off = (uint32_t)(row * p.K) + sw + (uint32_t)ks * 256u;
+      }
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xbase + (size_t)off),
+                                       (__attribute__((address_space(3))) void*)(tl_lds + buf * ABUF + (wave * MT + i) * 1024),
+                                       16, 0, 0);
+    }
+  };
+  // B of half step hs (= 2*ks + h): this wave brings tiles 2*wave, 2*wave + 1 of the 16, both K tiles of the half
+  const char* qwb = reinterpret_cast<const char*>(p.qw);
+  uint32_t bsrc[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+    bsrc[i] = (uint32_t)(min(bn * 16 + wave * 2 + i, p.tiles - 1) * KT64 * 64 + lane);
+  auto load_b = [&](int hs, int bb) {
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(qwb + (size_t)((bsrc[i] + (uint32_t)(hs * 2 + kt) * 64u) * 16u)),
+            (__attribute__((address_space(3))) void*)(b_lds + bb * BBUF + ((wave * 2 + i) * 2 + kt) * 1024), 16, 0, 0);
+  };
+  // activation scales: thread t < 128 carries the scale of row t for the step two ahead
+  const float* sarow = p.sa + (int64_t)min(m_wg + (tid & 127), p.M - 1) * KS;
+  float sareg = 0.f;
+  float swv[4], swn[4];
+
+  f32x4 facc[MT][4];
+  i32x4 iacc[MT][4];
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+      facc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      iacc[mt][nt] = i32x4{0, 0, 0, 0};
+    }
+
+  load_a(0, 0);
+  load_b(0, 0);
+#pragma unroll
+  for (int nt = 0; nt < 4; nt++)
+    swn[nt] = swp[soff[nt]];
+  if (tid < 128) {
+    sa_s[tid] = sarow[0];
+    if (KS > 1)
+      sa_s[128 + tid] = sarow[1];
+    sareg = KS > 2 ? sarow[2] : 0.f;
+  }
+  __syncthreads();
+  const uint32_t bwave = lds0 + (uint32_t)(2 * ABUF + wn * 8 * 1024) + (uint32_t)lane * 16u; // this wave's 4 tiles
+  for (int ks = 0; ks < KS; ks++) {
+    const int buf = ks & 1;
+    const bool more = ks + 1 < KS;
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++)
+      swv[nt] = swn[nt];
+    if (tid < 128 && ks + 2 < KS) {
+      sa_s[((ks + 2) & 3) * 128 + tid] = sareg; // loaded two steps ago
+      sareg = ks + 3 < KS ? sarow[ks + 3] : 0.f;
+    }
+    if (more) {
+      load_a(ks + 1, buf ^ 1);
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+        swn[nt] = swp[soff[nt] + (uint32_t)(ks + 1) * 16u];
+    }
+    const uint32_t abase = lds0 + (uint32_t)(buf * ABUF + wm * MT * 4096);
+    static_for<0, 2>([&](auto H) {
+      constexpr int h = decltype(H)::value;
+      // the other B buffer was read in the previous half step (barrier behind it): refill it for the next one
+      if (h == 0 || more)
+        load_b(2 * ks + h + 1, h ^ 1);
+      const uint32_t bbase = bwave + (uint32_t)(h * BBUF);
+      // operand reads of the half step, in order: 8 weight operands, then the activation operands RD ahead of use
+      i32x4 bq[4][2];
+      static_for<0, 8>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+        lds_read_b128_async<((i >> 1) * 2 + (i & 1)) * 1024>(bq[i >> 1][i & 1], bbase);
+      });
+      constexpr int RD = 3, NQ = 2 * MT;
+      i32x4 ar[RD + 1];
+      static_for<0, RD>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+        lds_read_b128_async<(i % MT) * 4096>(ar[i], abase + rdb[h * 2 + i / MT]);
+      });
+      static_for<0, NQ>([&](auto Q) {
+        constexpr int q = decltype(Q)::value;
+        constexpr int j = q / MT, mt = q % MT;
+        if constexpr (q + RD < NQ)
+          lds_read_b128_async<((q + RD) % MT) * 4096>(ar[(q + RD) % (RD + 1)], abase + rdb[h * 2 + (q + RD) / MT]);
+        constexpr int left = q + RD < NQ ? RD : NQ - 1 - q; // younger reads still allowed in flight
+        if constexpr (q == 0)
+          lds_wait_keep8<left>(ar[0], bq); // everything older, the 8 weight operands included, has arrived
+        else
+          lds_wait_keep<left>(ar[q % (RD + 1)]);
+        const i32x4 a = ar[q % (RD + 1)];
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+          iacc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bq[nt][j], iacc[mt][nt], 0, 0, 0);
+      });
+      if constexpr (h == 0)
+        __syncthreads(); // B buffer 0 may be refilled, buffer 1 has landed
+    });
+    // fold the block: facc += int32 sum * (sa[row] * sw[channel])
+    const float* sab = sa_s + (ks & 3) * 128 + wm * 64 + (lane >> 4) * 4;
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+      const f32x4 sav = *reinterpret_cast<const f32x4*>(sab + mt * 16);
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          facc[mt][nt][r] = fmaf((float)iacc[mt][nt][r], sav[r] * swv[nt], facc[mt][nt][r]);
+          iacc[mt][nt][r] = 0;
+        }
+    }
+    __syncthreads();
+  }
+  big_epilogue<MT>(p, facc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
+}
+
 // the large-M kernel addresses its operands with 32-bit byte offsets
 static bool big_fits(const TiledParams& p) {
   return (int64_t)p.M * p.K * 2 < ((int64_t)1 << 32) && (int64_t)p.tiles * 8 * p.K < ((int64_t)1 << 32);
@@ -661,6 +856,23 @@ hipError_t launch_silu_mul(const uint16_t* gate, uint16_t* y, int64_t n, hipStre
 }
 
 hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream) {
+  if (p.qbs == 256 && p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && env_int("TPPX_TILED_BIG_QINT8", 1) != 0 &&
+      (int64_t)p.M * p.K < ((int64_t)1 << 32) && (int64_t)p.tiles * 16 * p.K < ((int64_t)1 << 32)) {
+    const int MB4 = (p.M + 127) / 128, NB16 = (p.tiles + 15) / 16;
+    const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the A and B buffers + the scale slots
+    static_assert(8 * 64 * EP_LD * sizeof(float) >= 2 * 128 * 256 + 2 * 32 * 1024 + 4 * 128 * sizeof(float), "LDS plan");
+    TPPX_PLAN_ONLY(big_qint8_kernel, dim3(MB4 * NB16), dim3(512), lds);
+    static bool attr_done = false;
+    if (!attr_done) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_qint8_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess)
+        return e;
+      attr_done = true;
+    }
+    big_qint8_kernel<<<dim3(MB4 * NB16), dim3(512), lds, stream>>>(p);
+    return hipGetLastError();
+  }
   const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
   const size_t lds = 2 * 1024 * 16 + 2 * 128 * sizeof(float);
   TPPX_PLAN_ONLY(tiled_qint8_kernel, dim3(MB * NB), dim3(256), lds);
