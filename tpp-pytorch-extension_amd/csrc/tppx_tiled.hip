@@ -731,9 +731,10 @@ big_qint8_kernel(const TiledParams p) {
         else
           lds_wait_keep<left>(ar[q % (RD + 1)]);
         const i32x4 a = ar[q % (RD + 1)];
+        constexpr bool first = h == 0 && j == 0; // first MFMA of the block on this row tile: starts from zero
 #pragma unroll
         for (int nt = 0; nt < 4; nt++)
-          iacc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bq[nt][j], iacc[mt][nt], 0, 0, 0);
+          iacc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bq[nt][j], first ? i32x4{0, 0, 0, 0} : iacc[mt][nt], 0, 0, 0);
       });
       if constexpr (h == 0)
         __syncthreads(); // B buffer 0 may be refilled, buffer 1 has landed
@@ -746,10 +747,8 @@ big_qint8_kernel(const TiledParams p) {
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
+        for (int r = 0; r < 4; r++)
           facc[mt][nt][r] = fmaf((float)iacc[mt][nt][r], sav[r] * swv[nt], facc[mt][nt][r]);
-          iacc[mt][nt][r] = 0;
-        }
     }
     __syncthreads();
   }
