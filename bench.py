@@ -60,6 +60,8 @@ def main():
                     help="decode = the configuration the headline metric is quoted on (default); prefill = the "
                          "MXFP4 linears of one 70B-shape decoder layer at M = 2048 (TFLOP/s, MFMA roofline); tokens = "
                          "7B-shape greedy decode; prompt = a 2048-token prompt through the same 7B-shape decoder")
+    ap.add_argument("--prefill-fmt", default="mxfp4", choices=["mxfp4", "qint8"],
+                    help="weight format of --workload prefill (BASELINE config 4 is MXFP4; qint8 = the same layer W8A8)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pool", type=int, default=2, help="number of distinct weight sets cycled through")
@@ -287,9 +289,12 @@ def run_prefill(torch, _ops, args):
     M, H, I = 2048, 8192, 28672
     g = torch.Generator(device=dev).manual_seed(1238)
 
+    pfmt = args.prefill_fmt
+    quant = _ops.remap_and_quantize_mxfp4 if pfmt == "mxfp4" else _ops.remap_and_quantize_qint8
+
     def mk(N, K):
         W = (torch.randn((N, K), generator=g, device=dev) * 0.02).to(torch.bfloat16)
-        q = _ops.remap_and_quantize_mxfp4(W.view(N // 16, 16, K // 64, 32, 2).permute(0, 2, 3, 1, 4).contiguous())
+        q = quant(W.view(N // 16, 16, K // 64, 32, 2).permute(0, 2, 3, 1, 4).contiguous())
         q.native()
         return q
 
@@ -318,7 +323,7 @@ def run_prefill(torch, _ops, args):
 
     # roofline leg: the largest GEMM (down projection) alone, events on the launch stream
     L = _lib.lib()
-    plan = kernel_plan(L, "mxfp4", M, H, I, 0, 0, 0)
+    plan = kernel_plan(L, pfmt, M, H, I, 256, 0, 0)
     inter = torch.randn((M, I), generator=g, device=dev).to(torch.bfloat16)
     for _ in range(2):
         torch.ops.tpp_llm.fc_add(inter, wd, empty, res, 1.0)
@@ -332,17 +337,20 @@ def run_prefill(torch, _ops, args):
     torch.cuda.synchronize()
     us = e0.elapsed_time(e1) * 1e3 / reps
     fl = 2.0 * M * H * I
+    peak = PEAKS_TFLOPS["bf16"] if pfmt == "mxfp4" else PEAKS_TFLOPS["int8"]
     roof = {"bound": "mfma", "kernel": plan[-1][0] if plan else "?", "call": f"down M={M} N={H} K={I}",
-            "achieved": round(fl / us / 1e6, 1), "peak": PEAKS_TFLOPS["bf16"], "unit": "TFLOP/s",
-            "frac": round(fl / us / 1e6 / PEAKS_TFLOPS["bf16"], 4), "traffic": None,
+            "achieved": round(fl / us / 1e6, 1), "peak": peak, "unit": "TFLOP/s" if pfmt == "mxfp4" else "TOP/s",
+            "frac": round(fl / us / 1e6 / peak, 4), "traffic": None,
             "avg_launch_us": round(us, 1), "flops_per_launch": fl, "launches_timed": reps,
             "timing": "events on the launch stream around eager launches of this op alone"}
-    cpu = None if args.no_cpu else cpu_baseline_prefill(H)
+    cpu = None if (args.no_cpu or pfmt != "mxfp4") else cpu_baseline_prefill(H)
     print(json.dumps({
-        "metric": "quant-GEMM TFLOP/s (prefill)", "value": round(flops / (ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+        "metric": "quant-GEMM TFLOP/s (prefill)", "value": round(flops / (ms * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s" if pfmt == "mxfp4" else "TOP/s",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "cfg4: MXFP4 linears of one decoder layer (hidden 8192, intermediate 28672, kv 1024) at "
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if pfmt == "mxfp4" else "int8", "data": "synthetic",
+        "config": {"workload": ("cfg4: MXFP4" if pfmt == "mxfp4" else "cfg4's layer with QINT8 W8A8 (QBS=256)") +
+                               " linears of one decoder layer (hidden 8192, intermediate 28672, kv 1024) at "
                                "M = 2048: qkv_gemm, fc_add(o), swiglu_mlp(gate, up, down)",
                    "launch": "eager op calls", "flops_per_step": flops},
         "roofline": roof, "cpu_baseline": cpu}))

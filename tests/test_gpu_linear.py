@@ -301,6 +301,22 @@ def test_k_split_across_workgroups(fmt, M, N):
         assert torch.equal(o, first)
 
 
+def test_prefill_qint8_qkv_one_launch_equals_separate():
+    """QINT8, enough rows for the large-M kernel: fused q/k/v share one launch (ragged channel blocks: 544, 128 and
+    256 channels) and give the bits of the single-GEMM calls, which match the oracle."""
+    ops = _ops()
+    K, M = 1024, 300
+    made = [_make("qint8", n, K, 280 + i) for i, n in enumerate((544, 128, 256))]
+    ws = [m[0] for m in made]
+    x = randn_bf16((M, K), 1.0, 290)
+    bs = [randn_bf16((n,), 0.01, 295 + i).cuda() for i, n in enumerate((544, 128, 256))]
+    outs = torch.ops.tpp_llm.qkv_gemm(x.cuda(), ws, bs)
+    for (w, q_or, s_or), b, o in zip(made, bs, outs):
+        assert torch.equal(o, ops.fc_plain(x.cuda(), w, b))
+        ref = O.linear_qint8(t2bits(x), q_or, s_or, t2bits(b.cpu()))
+        assert_close_bf16(t2bits(o), ref, what="qint8 fused qkv, large M")
+
+
 def test_prefill_qkv_one_launch_equals_separate():
     """With enough rows the fused q/k/v GEMMs share one launch of the large-M
     kernel (one grid over the channel blocks of all three)."""

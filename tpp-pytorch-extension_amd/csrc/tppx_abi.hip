@@ -350,6 +350,17 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
       if (rc)
         return rc;
     }
+    if (n_segs > 1) { // fused q/k/v: one grid over the channel blocks of all GEMMs when the large-M kernel takes them
+      TiledParams t[TPPX_MAX_SEGS];
+      bool group = true;
+      for (int i = 0; i < n_segs; i++) {
+        t[i] = tiled_from_seg(p, i);
+        t[i].qbs = (int)qbs;
+        group = group && tiled_qint8_takes_groups(t[i]);
+      }
+      if (group)
+        return check_hip(launch_tiled_qint8_group(t, n_segs, stream), who);
+    }
     for (int i = 0; i < n_segs; i++) {
       TiledParams t = tiled_from_seg(p, i);
       t.qbs = (int)qbs;

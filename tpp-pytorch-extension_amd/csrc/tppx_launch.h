@@ -81,6 +81,8 @@ hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream);
 bool tiled_mxfp4_takes_groups(const TiledParams& p);
 hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream);
 hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream);
+bool tiled_qint8_takes_groups(const TiledParams& p);
+hipError_t launch_tiled_qint8_group(const TiledParams* t, int n, hipStream_t stream);
 // y[i] = bf16( silu(gate[i]) * y[i] ) with the rounding points of SiluPostOp followed by MulPostOp; n % 8 == 0
 hipError_t launch_silu_mul(const uint16_t* gate, uint16_t* y, int64_t n, hipStream_t stream);
 

@@ -592,7 +592,7 @@ __device__ __forceinline__ void lds_wait_keep8(i32x4& r, i32x4 (&b)[4][2]) {
 }
 
 __global__ void __launch_bounds__(512)
-big_qint8_kernel(const TiledParams p) {
+big_qint8_kernel(const BigParams P) {
   constexpr int MT = 4, WGM = 128, ABUF = WGM * 256, BBUF = 32 * 1024;
   extern __shared__ __align__(16) uint8_t tl_lds[];
   uint8_t* b_lds = tl_lds + 2 * ABUF;
@@ -600,9 +600,19 @@ big_qint8_kernel(const TiledParams p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 1, wn = wave >> 1;
-  const int MB = (p.M + WGM - 1) / WGM, NB = (p.tiles + 15) >> 4;
+  const int MB = (P.seg[0].M + WGM - 1) / WGM;
   int bm, bn;
-  tile_of_block(MB, NB, bm, bn);
+  tile_of_block(MB, P.nb0[P.n_seg], bm, bn);
+  // several GEMMs over one activation (fused q/k/v) share the launch: pick this block's with uniform selects
+  TiledParams p = P.seg[0];
+  int nb_first = 0;
+#pragma unroll
+  for (int i = 1; i < TPPX_MAX_SEGS; i++)
+    if (i < P.n_seg && bn >= P.nb0[i]) {
+      p = P.seg[i];
+      nb_first = P.nb0[i];
+    }
+  bn -= nb_first;
   const int KS = p.K >> 8;   // K steps = scale blocks
   const int KT64 = p.K >> 6; // native tiles along K
   const int m_wg = bm * WGM;
@@ -854,10 +864,26 @@ hipError_t launch_silu_mul(const uint16_t* gate, uint16_t* y, int64_t n, hipStre
   return hipGetLastError();
 }
 
-hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream) {
-  if (p.qbs == 256 && p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && env_int("TPPX_TILED_BIG_QINT8", 1) != 0 &&
-      (int64_t)p.M * p.K < ((int64_t)1 << 32) && (int64_t)p.tiles * 16 * p.K < ((int64_t)1 << 32)) {
-    const int MB4 = (p.M + 127) / 128, NB16 = (p.tiles + 15) / 16;
+bool tiled_qint8_takes_groups(const TiledParams& p) {
+  return p.qbs == 256 && p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && env_int("TPPX_TILED_BIG_QINT8", 1) != 0 &&
+         (int64_t)p.M * p.K < ((int64_t)1 << 32) && (int64_t)p.tiles * 16 * p.K < ((int64_t)1 << 32);
+}
+
+// n GEMMs over the same quantised activations (same M, K, xq, sa) in one launch of the large-M kernel
+hipError_t launch_tiled_qint8_group(const TiledParams* t, int n, hipStream_t stream) {
+  {
+    BigParams P;
+    memset(&P, 0, sizeof(P));
+    int nb = 0;
+    for (int i = 0; i < n; i++) {
+      P.seg[i] = t[i];
+      P.nb0[i] = nb;
+      nb += (t[i].tiles + 15) / 16;
+    }
+    for (int i = n; i <= TPPX_MAX_SEGS; i++)
+      P.nb0[i] = nb;
+    P.n_seg = n;
+    const int MB4 = (t[0].M + 127) / 128, NB16 = nb;
     const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the A and B buffers + the scale slots
     static_assert(8 * 64 * EP_LD * sizeof(float) >= 2 * 128 * 256 + 2 * 32 * 1024 + 4 * 128 * sizeof(float), "LDS plan");
     TPPX_PLAN_ONLY(big_qint8_kernel, dim3(MB4 * NB16), dim3(512), lds);
@@ -869,9 +895,14 @@ hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream) {
         return e;
       attr_done = true;
     }
-    big_qint8_kernel<<<dim3(MB4 * NB16), dim3(512), lds, stream>>>(p);
+    big_qint8_kernel<<<dim3(MB4 * NB16), dim3(512), lds, stream>>>(P);
     return hipGetLastError();
   }
+}
+
+hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream) {
+  if (tiled_qint8_takes_groups(p))
+    return launch_tiled_qint8_group(&p, 1, stream);
   const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
   const size_t lds = 2 * 1024 * 16 + 2 * 128 * sizeof(float);
   TPPX_PLAN_ONLY(tiled_qint8_kernel, dim3(MB * NB), dim3(256), lds);
