@@ -563,40 +563,45 @@ big_mxfp4_kernel(const BigParams P) {
 
 // ---------------------------------------------------------------------------
 // Large-M QINT8 (W8A8, 256-wide blocks): 128 x 256 workgroup tile, 8 waves
-// (2 x 4), wave tile 64 x 64, K step 256 = one scale block in two halves.
-// What bounds int8 at this size is operand delivery, not the MFMA: weights are
-// 4x the bytes of MXFP4 per MAC, the MFMA runs at twice the bf16 rate, and the
-// two accumulator sets (int32 block sums, fp32 running sums) leave no room for
-// a second set of weight registers.  So BOTH operands go from global memory
-// straight into LDS (no staging registers, nothing for the compiler to wait
-// on before the barrier), each weight tile is fetched once per workgroup
-// instead of once per wave row, and LDS (about twice the bandwidth of the
-// vector memory path) feeds the MFMAs:
-//   A: int8 rows, 256 B per row and K step, the layout, swizzle and operand
-//      reads of the MXFP4 kernel above (the operand of MFMA step j is chunk
-//      j*4 + g of the row); two buffers of 32 KiB, loaded a step ahead.
-//   B: native 1 KiB tiles (16 channels x 64 K, lane-linear = MFMA operand
-//      order), 16 tiles x 2 K tiles = 32 KiB per half step, two buffers,
-//      loaded half a step ahead; a lane reads its own 16 bytes, no conflicts.
-//   int32 block sums (exact) are folded into fp32 at the end of every step
-//   with sa[m] * sw[n]; the activation scales of a step reach the waves
-//   through LDS, requested two steps ahead.
-// LDS: A 2 x 32 KiB | B 2 x 32 KiB | scales 2 KiB (the epilogue staging reuses it).
+// (2 x 4), wave tile 64 x 64, K step 256 = one scale block.
+// What bounds int8 at this size is operand delivery and the fold, not the
+// MFMA: weights are 4x the bytes of MXFP4 per MAC, the MFMA runs at twice the
+// bf16 rate, and every block's int32 sums have to be converted, scaled by
+// sa[m] * sw[n] and added to the fp32 sums (3 vector instructions per output
+// and block, 3/4 of the MFMA time).  So:
+//   * BOTH operands go from global memory straight into LDS (no staging
+//     registers, nothing for the compiler to wait on before the barrier) and
+//     every weight tile is fetched once per workgroup instead of once per wave
+//     row.  A: int8 rows, 256 B per row and step, the layout, swizzle and
+//     operand reads of the MXFP4 kernel above (operand of MFMA step j = chunk
+//     j*4 + g of the row), two buffers.  B: native 1 KiB tiles (lane-linear =
+//     operand order), 16 tiles x 4 K tiles = 64 KiB, ONE buffer: at the start
+//     of a step every wave copies its 16 operands into registers, a barrier
+//     frees the buffer and the next step's tiles stream in during the MFMAs.
+//   * The MFMAs of a step run row tile by row tile (all of K for 16 rows, then
+//     the next 16), into one of two small sets of int32 sums, and the fold of
+//     row tile mt sits between the first and the second MFMA group of row tile
+//     mt + 1: vector and matrix work overlap inside a wave, and the two waves
+//     of a SIMD do not fold at the same moment.  The first MFMA of a row tile
+//     starts from a zero operand.
+//   * Activation scales reach the waves through LDS, requested two steps ahead.
+// LDS: A 2 x 32 KiB | B 64 KiB | scales 2 KiB (the epilogue staging reuses it).
 // ---------------------------------------------------------------------------
 template <int N>
-__device__ __forceinline__ void lds_wait_keep8(i32x4& r, i32x4 (&b)[4][2]) {
-  asm volatile("s_waitcnt lgkmcnt(%9)"
-               : "+v"(r), "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[1][0]), "+v"(b[1][1]), "+v"(b[2][0]), "+v"(b[2][1]),
-                 "+v"(b[3][0]), "+v"(b[3][1])
+__device__ __forceinline__ void lds_wait_keep16(i32x4 (&b)[4][4]) {
+  asm volatile("s_waitcnt lgkmcnt(%16)"
+               : "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[0][2]), "+v"(b[0][3]), "+v"(b[1][0]), "+v"(b[1][1]), "+v"(b[1][2]),
+                 "+v"(b[1][3]), "+v"(b[2][0]), "+v"(b[2][1]), "+v"(b[2][2]), "+v"(b[2][3]), "+v"(b[3][0]), "+v"(b[3][1]),
+                 "+v"(b[3][2]), "+v"(b[3][3])
                : "n"(N));
 }
 
 __global__ void __launch_bounds__(512)
 big_qint8_kernel(const BigParams P) {
-  constexpr int MT = 4, WGM = 128, ABUF = WGM * 256, BBUF = 32 * 1024;
+  constexpr int MT = 4, WGM = 128, ABUF = WGM * 256, BBUF = 64 * 1024;
   extern __shared__ __align__(16) uint8_t tl_lds[];
   uint8_t* b_lds = tl_lds + 2 * ABUF;
-  float* sa_s = reinterpret_cast<float*>(tl_lds + 2 * ABUF + 2 * BBUF); // [4][128]: scales of steps ks .. ks+2 (mod 4)
+  float* sa_s = reinterpret_cast<float*>(tl_lds + 2 * ABUF + BBUF); // [4][128]: scales of steps ks .. ks+2 (mod 4)
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 1, wn = wave >> 1;
@@ -652,20 +657,20 @@ big_qint8_kernel(const BigParams P) {
                                        16, 0, 0);
     }
   };
-  // B of half step hs (= 2*ks + h): this wave brings tiles 2*wave, 2*wave + 1 of the 16, both K tiles of the half
+  // B of step ks: this wave brings tiles 2*wave, 2*wave + 1 of the 16, all four K tiles; LDS slot (tile*4 + kt) KiB
   const char* qwb = reinterpret_cast<const char*>(p.qw);
   uint32_t bsrc[2];
 #pragma unroll
   for (int i = 0; i < 2; i++)
     bsrc[i] = (uint32_t)(min(bn * 16 + wave * 2 + i, p.tiles - 1) * KT64 * 64 + lane);
-  auto load_b = [&](int hs, int bb) {
+  auto load_b = [&](int ks) {
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-      for (int kt = 0; kt < 2; kt++)
+      for (int kt = 0; kt < 4; kt++)
         __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(qwb + (size_t)((bsrc[i] + (uint32_t)(hs * 2 + kt) * 64u) * 16u)),
-            (__attribute__((address_space(3))) void*)(b_lds + bb * BBUF + ((wave * 2 + i) * 2 + kt) * 1024), 16, 0, 0);
+            (const __attribute__((address_space(1))) void*)(qwb + (size_t)((bsrc[i] + (uint32_t)(ks * 4 + kt) * 64u) * 16u)),
+            (__attribute__((address_space(3))) void*)(b_lds + ((wave * 2 + i) * 4 + kt) * 1024), 16, 0, 0);
   };
   // activation scales: thread t < 128 carries the scale of row t for the step two ahead
   const float* sarow = p.sa + (int64_t)min(m_wg + (tid & 127), p.M - 1) * KS;
@@ -673,17 +678,20 @@ big_qint8_kernel(const BigParams P) {
   float swv[4], swn[4];
 
   f32x4 facc[MT][4];
-  i32x4 iacc[MT][4];
+  i32x4 iacc[2][4]; // block sums of the row tile in flight and of the one being folded
 #pragma unroll
   for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-    for (int nt = 0; nt < 4; nt++) {
+    for (int nt = 0; nt < 4; nt++)
       facc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-      iacc[mt][nt] = i32x4{0, 0, 0, 0};
-    }
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++)
+      iacc[i][nt] = i32x4{0, 0, 0, 0};
 
   load_a(0, 0);
-  load_b(0, 0);
+  load_b(0);
 #pragma unroll
   for (int nt = 0; nt < 4; nt++)
     swn[nt] = swp[soff[nt]];
@@ -694,10 +702,16 @@ big_qint8_kernel(const BigParams P) {
     sareg = KS > 2 ? sarow[2] : 0.f;
   }
   __syncthreads();
-  const uint32_t bwave = lds0 + (uint32_t)(2 * ABUF + wn * 8 * 1024) + (uint32_t)lane * 16u; // this wave's 4 tiles
+  const uint32_t bwave = lds0 + (uint32_t)(2 * ABUF + wn * 16 * 1024) + (uint32_t)lane * 16u; // this wave's 4 tiles
   for (int ks = 0; ks < KS; ks++) {
     const int buf = ks & 1;
     const bool more = ks + 1 < KS;
+    // this step's weight operands: LDS -> registers, then the buffer is free for the next step's tiles
+    i32x4 bq[4][4]; // [tile][MFMA step j]
+    static_for<0, 16>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      lds_read_b128_async<i * 1024>(bq[i >> 2][i & 3], bwave);
+    });
 #pragma unroll
     for (int nt = 0; nt < 4; nt++)
       swv[nt] = swn[nt];
@@ -705,61 +719,50 @@ big_qint8_kernel(const BigParams P) {
       sa_s[((ks + 2) & 3) * 128 + tid] = sareg; // loaded two steps ago
       sareg = ks + 3 < KS ? sarow[ks + 3] : 0.f;
     }
+    lds_wait_keep16<0>(bq);
+    __syncthreads();
     if (more) {
+      load_b(ks + 1);
       load_a(ks + 1, buf ^ 1);
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
         swn[nt] = swp[soff[nt] + (uint32_t)(ks + 1) * 16u];
     }
     const uint32_t abase = lds0 + (uint32_t)(buf * ABUF + wm * MT * 4096);
-    static_for<0, 2>([&](auto H) {
-      constexpr int h = decltype(H)::value;
-      // the other B buffer was read in the previous half step (barrier behind it): refill it for the next one
-      if (h == 0 || more)
-        load_b(2 * ks + h + 1, h ^ 1);
-      const uint32_t bbase = bwave + (uint32_t)(h * BBUF);
-      // operand reads of the half step, in order: 8 weight operands, then the activation operands RD ahead of use
-      i32x4 bq[4][2];
-      static_for<0, 8>([&](auto I) {
-        constexpr int i = decltype(I)::value;
-        lds_read_b128_async<((i >> 1) * 2 + (i & 1)) * 1024>(bq[i >> 1][i & 1], bbase);
-      });
-      constexpr int RD = 3, NQ = 2 * MT;
-      i32x4 ar[RD + 1];
-      static_for<0, RD>([&](auto I) {
-        constexpr int i = decltype(I)::value;
-        lds_read_b128_async<(i % MT) * 4096>(ar[i], abase + rdb[h * 2 + i / MT]);
-      });
-      static_for<0, NQ>([&](auto Q) {
-        constexpr int q = decltype(Q)::value;
-        constexpr int j = q / MT, mt = q % MT;
-        if constexpr (q + RD < NQ)
-          lds_read_b128_async<((q + RD) % MT) * 4096>(ar[(q + RD) % (RD + 1)], abase + rdb[h * 2 + (q + RD) / MT]);
-        constexpr int left = q + RD < NQ ? RD : NQ - 1 - q; // younger reads still allowed in flight
-        if constexpr (q == 0)
-          lds_wait_keep8<left>(ar[0], bq); // everything older, the 8 weight operands included, has arrived
-        else
-          lds_wait_keep<left>(ar[q % (RD + 1)]);
-        const i32x4 a = ar[q % (RD + 1)];
-        constexpr bool first = h == 0 && j == 0; // first MFMA of the block on this row tile: starts from zero
-#pragma unroll
-        for (int nt = 0; nt < 4; nt++)
-          iacc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bq[nt][j], first ? i32x4{0, 0, 0, 0} : iacc[mt][nt], 0, 0, 0);
-      });
-      if constexpr (h == 0)
-        __syncthreads(); // B buffer 0 may be refilled, buffer 1 has landed
-    });
-    // fold the block: facc += int32 sum * (sa[row] * sw[channel])
     const float* sab = sa_s + (ks & 3) * 128 + wm * 64 + (lane >> 4) * 4;
-#pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
+    auto fold = [&](auto MTI) { // facc += int32 sum * (sa[row] * sw[channel]) for row tile mt
+      constexpr int mt = decltype(MTI)::value;
       const f32x4 sav = *reinterpret_cast<const f32x4*>(sab + mt * 16);
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
 #pragma unroll
         for (int r = 0; r < 4; r++)
-          facc[mt][nt][r] = fmaf((float)iacc[mt][nt][r], sav[r] * swv[nt], facc[mt][nt][r]);
-    }
+          facc[mt][nt][r] = fmaf((float)iacc[mt & 1][nt][r], sav[r] * swv[nt], facc[mt][nt][r]);
+    };
+    // activation operands in order q = mt*4 + j, RD ahead of their use
+    constexpr int RD = 3, NQ = 4 * MT;
+    i32x4 ar[RD + 1];
+    static_for<0, RD>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      lds_read_b128_async<(i / 4) * 4096>(ar[i], abase + rdb[i % 4]);
+    });
+    static_for<0, NQ>([&](auto Q) {
+      constexpr int q = decltype(Q)::value;
+      constexpr int mt = q / 4, j = q % 4;
+      if constexpr (q + RD < NQ) {
+        lds_read_b128_async<((q + RD) / 4) * 4096>(ar[(q + RD) % (RD + 1)], abase + rdb[(q + RD) % 4]);
+        lds_wait_keep<RD>(ar[q % (RD + 1)]);
+      } else {
+        lds_wait_keep<NQ - 1 - q>(ar[q % (RD + 1)]);
+      }
+      const i32x4 a = ar[q % (RD + 1)];
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+        iacc[mt & 1][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bq[nt][j], j == 0 ? i32x4{0, 0, 0, 0} : iacc[mt & 1][nt], 0, 0, 0);
+      if constexpr (j == 0 && mt > 0)
+        fold(std::integral_constant<int, mt - 1>{}); // the previous row tile, under this row tile's MFMAs
+    });
+    fold(std::integral_constant<int, MT - 1>{});
     __syncthreads();
   }
   big_epilogue<MT>(p, facc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
@@ -885,7 +888,7 @@ hipError_t launch_tiled_qint8_group(const TiledParams* t, int n, hipStream_t str
     P.n_seg = n;
     const int MB4 = (t[0].M + 127) / 128, NB16 = nb;
     const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the A and B buffers + the scale slots
-    static_assert(8 * 64 * EP_LD * sizeof(float) >= 2 * 128 * 256 + 2 * 32 * 1024 + 4 * 128 * sizeof(float), "LDS plan");
+    static_assert(8 * 64 * EP_LD * sizeof(float) >= 2 * 128 * 256 + 64 * 1024 + 4 * 128 * sizeof(float), "LDS plan");
     TPPX_PLAN_ONLY(big_qint8_kernel, dim3(MB4 * NB16), dim3(512), lds);
     static bool attr_done = false;
     if (!attr_done) {
