@@ -514,17 +514,19 @@ attn_prefill_kernel(const AttnPrefillParams p) {
   const uint16_t* vbase = p.vc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128;
   const uint16_t* mrow = p.mask ? p.mask + (int64_t)b * p.mask_ld : nullptr;
 
-  // staging registers: K rows chunk-fastest (coalesced), V rows key-fastest (so that the transposed 2-byte LDS
-  // writes of a wave fall into consecutive addresses)
+  // staging registers: K rows chunk-fastest (coalesced); V: a thread takes one 16-byte chunk (8 dims) of FOUR
+  // consecutive keys, so that the transposed image is written as 8 x 8 bytes (4 keys of one dim, packed with two
+  // byte permutes) instead of 32 two-byte writes
   i32x4 kst[4], vst[4];
+  const int vq = tid & 15, vch = tid >> 4; // key quad, chunk
   auto load_tile = [&](int kb) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int idx = tid + i * 256;
       const int kk = min(kb * 64 + (idx >> 4), last_key);
       kst[i] = *reinterpret_cast<const i32x4*>(kbase + (int64_t)kk * 128 + (idx & 15) * 8);
-      const int kv = min(kb * 64 + (idx & 63), last_key);
-      vst[i] = *reinterpret_cast<const i32x4*>(vbase + (int64_t)kv * 128 + (idx >> 6) * 8);
+      const int kv = min(kb * 64 + vq * 4 + i, last_key);
+      vst[i] = *reinterpret_cast<const i32x4*>(vbase + (int64_t)kv * 128 + vch * 8);
     }
   };
   auto store_tile = [&]() {
@@ -532,10 +534,14 @@ attn_prefill_kernel(const AttnPrefillParams p) {
     for (int i = 0; i < 4; i++) {
       const int idx = tid + i * 256;
       *reinterpret_cast<i32x4*>(ks + (idx >> 4) * AP_KP + (idx & 15) * 8) = kst[i];
-      const int key = idx & 63, ch = idx >> 6;
+    }
 #pragma unroll
-      for (int e = 0; e < 8; e++)
-        vt[(ch * 8 + e) * AP_VP + key] = (uint16_t)((uint32_t)vst[i][e >> 1] >> ((e & 1) * 16));
+    for (int e = 0; e < 8; e++) {
+      // dim vch*8 + e of keys 4*vq .. 4*vq+3: the low (e even) or high (e odd) halves of dword e/2 of the four rows
+      const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+      const uint32_t lo = __builtin_amdgcn_perm((uint32_t)vst[1][e >> 1], (uint32_t)vst[0][e >> 1], sel);
+      const uint32_t hi = __builtin_amdgcn_perm((uint32_t)vst[3][e >> 1], (uint32_t)vst[2][e >> 1], sel);
+      *reinterpret_cast<uint2*>(vt + (vch * 8 + e) * AP_VP + vq * 4) = make_uint2(lo, hi);
     }
   };
 
