@@ -545,6 +545,7 @@ attn_prefill_kernel(const AttnPrefillParams p) {
     }
   };
 
+  const float scale2 = p.scale * 1.44269504f;
   float m[QG], l[QG];
   f32x4 acc[QG][8];
 #pragma unroll
@@ -583,7 +584,7 @@ attn_prefill_kernel(const AttnPrefillParams p) {
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int key = kb * 64 + (i >> 2) * 16 + g * 4 + (i & 3);
-      mk[i] = (mrow && key < p.mask_ld) ? bf16_bits_to_f32(mrow[key]) : 0.f;
+      mk[i] = (mrow && key < p.mask_ld) ? bf16_bits_to_f32(mrow[key]) * 1.44269504f : 0.f; // base-2 domain, see below
     }
     bf16x8 pb[QG][2];
 #pragma unroll
@@ -594,14 +595,16 @@ attn_prefill_kernel(const AttnPrefillParams p) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const int key = kb * 64 + t * 16 + g * 4 + r;
-          const float v = key <= qpos[qg] ? sc[qg][t][r] * p.scale + mk[t * 4 + r] : -3.0e38f;
+          // scores in the base-2 domain (scale * log2 e folded into one multiplier): a probability is one exp2;
+          // keys past the causal edge get -inf, whose exp2 is exactly 0 against the finite running maximum
+          const float v = key <= qpos[qg] ? sc[qg][t][r] * scale2 + mk[t * 4 + r] : -INFINITY;
           sc[qg][t][r] = v;
           mx = fmaxf(mx, v);
         }
       mx = fmaxf(mx, __shfl_xor(mx, 16));
       mx = fmaxf(mx, __shfl_xor(mx, 32));
       const float mn = fmaxf(m[qg], mx); // finite from the first tile on: key 0 is visible to every query
-      const float alpha = __expf(m[qg] - mn);
+      const float alpha = __builtin_amdgcn_exp2f(m[qg] - mn);
       l[qg] *= alpha;
 #pragma unroll
       for (int dt = 0; dt < 8; dt++)
@@ -610,9 +613,7 @@ attn_prefill_kernel(const AttnPrefillParams p) {
       for (int u = 0; u < 2; u++)
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-          const int t = 2 * u + (j >> 2), r = j & 3;
-          const int key = kb * 64 + t * 16 + g * 4 + r;
-          const float pr = key <= qpos[qg] ? __expf(sc[qg][t][r] - mn) : 0.f;
+          const float pr = __builtin_amdgcn_exp2f(sc[qg][2 * u + (j >> 2)][j & 3] - mn);
           l[qg] += pr;
           pb[qg][u][j] = (__bf16)pr;
         }
