@@ -580,11 +580,22 @@ attn_prefill_kernel(const AttnPrefillParams p) {
           sc[qg][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[qg][j], sc[qg][t], 0, 0, 0);
       }
     }
-    float mk[16]; // additive mask of this lane's 16 keys
+    // Scores in the base-2 domain (scale * log2 e folded into one multiplier): a probability is one exp2.  The
+    // additive mask is read only when there is one (wave-uniform branch: no addresses, no predicated loads).
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      const int key = kb * 64 + (i >> 2) * 16 + g * 4 + (i & 3);
-      mk[i] = (mrow && key < p.mask_ld) ? bf16_bits_to_f32(mrow[key]) * 1.44269504f : 0.f; // base-2 domain, see below
+    for (int qg = 0; qg < QG; qg++)
+#pragma unroll
+      for (int t = 0; t < 4; t++)
+        sc[qg][t] *= scale2;
+    if (mrow) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int key = kb * 64 + (i >> 2) * 16 + g * 4 + (i & 3);
+        const float mk = key < p.mask_ld ? bf16_bits_to_f32(mrow[key]) * 1.44269504f : 0.f;
+#pragma unroll
+        for (int qg = 0; qg < QG; qg++)
+          sc[qg][i >> 2][i & 3] += mk;
+      }
     }
     bf16x8 pb[QG][2];
 #pragma unroll
@@ -595,9 +606,8 @@ attn_prefill_kernel(const AttnPrefillParams p) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const int key = kb * 64 + t * 16 + g * 4 + r;
-          // scores in the base-2 domain (scale * log2 e folded into one multiplier): a probability is one exp2;
           // keys past the causal edge get -inf, whose exp2 is exactly 0 against the finite running maximum
-          const float v = key <= qpos[qg] ? sc[qg][t][r] * scale2 + mk[t * 4 + r] : -INFINITY;
+          const float v = key <= qpos[qg] ? sc[qg][t][r] : -INFINITY;
           sc[qg][t][r] = v;
           mx = fmaxf(mx, v);
         }
