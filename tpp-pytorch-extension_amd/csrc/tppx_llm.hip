@@ -598,19 +598,26 @@ attn_prefill_kernel(const AttnPrefillParams p) {
       }
     }
     bf16x8 pb[QG][2];
+    // only the tiles that reach past the position of this wave's first query hide anything (wave-uniform)
+    const bool edge = kb * 64 + 63 > p.past + q0;
 #pragma unroll
     for (int qg = 0; qg < QG; qg++) {
+      if (edge) {
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const int key = kb * 64 + t * 16 + g * 4 + r;
+            // keys past the causal edge get -inf, whose exp2 is exactly 0 against the finite running maximum
+            sc[qg][t][r] = key <= qpos[qg] ? sc[qg][t][r] : -INFINITY;
+          }
+      }
       float mx = -3.0e38f;
 #pragma unroll
       for (int t = 0; t < 4; t++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const int key = kb * 64 + t * 16 + g * 4 + r;
-          // keys past the causal edge get -inf, whose exp2 is exactly 0 against the finite running maximum
-          const float v = key <= qpos[qg] ? sc[qg][t][r] : -INFINITY;
-          sc[qg][t][r] = v;
-          mx = fmaxf(mx, v);
-        }
+        for (int r = 0; r < 4; r++)
+          mx = fmaxf(mx, sc[qg][t][r]);
       mx = fmaxf(mx, __shfl_xor(mx, 16));
       mx = fmaxf(mx, __shfl_xor(mx, 32));
       const float mn = fmaxf(m[qg], mx); // finite from the first tile on: key 0 is visible to every query
