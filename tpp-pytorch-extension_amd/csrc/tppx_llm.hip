@@ -849,8 +849,14 @@ extern "C" int tppx_attn_prefill(const void* q, const void* kcache, const void* 
   p.B = (int)B; p.S = (int)S; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.Smax = (int)Smax; p.mask_ld = (int)mask_ld;
   p.past = (int)past_len;
   p.scale = 1.0f / sqrtf((float)H);
-  // 16 queries per wave: 32 (QG = 2) halve the LDS reads per MFMA but need 248 registers, one wave per SIMD, and
-  // measured slower (S = 2048, 32 heads: 197 us against 172 us)
-  attn_prefill_kernel<1><<<dim3((unsigned)((S + 63) / 64), (unsigned)(B * Nq)), dim3(256), 0, (hipStream_t)stream>>>(p);
+  // 32 queries per wave (QG = 2) halve the LDS reads per MFMA at 226 registers, still two waves per SIMD; they win
+  // when the launch still has two workgroups per CU (S = 2048, 32 heads: 97 us against 117 us; 16 x 128 queries
+  // behind 1024 cached keys: 69 against 96 us) and lose below that (S = 512, 32 heads: 22.5 against 17 us)
+  const long wgs2 = ((S + 127) / 128) * B * Nq;
+  const int qg = env_int("TPPX_ATTN_QG", wgs2 >= 512 ? 2 : 1);
+  if (qg == 2 && S > 64)
+    attn_prefill_kernel<2><<<dim3((unsigned)((S + 127) / 128), (unsigned)(B * Nq)), dim3(256), 0, (hipStream_t)stream>>>(p);
+  else
+    attn_prefill_kernel<1><<<dim3((unsigned)((S + 63) / 64), (unsigned)(B * Nq)), dim3(256), 0, (hipStream_t)stream>>>(p);
   return check_hip(hipGetLastError(), who);
 }
