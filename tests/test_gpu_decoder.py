@@ -196,10 +196,13 @@ def _attn_prefill(q, kc, vc, past, mask=None):
 
 @pytest.mark.parametrize("B,S,Nq,Nkv,past,Smax", [(1, 256, 4, 4, 0, 256), (2, 77, 8, 2, 0, 128), (2, 5, 4, 4, 100, 128),
                                                   (1, 130, 2, 1, 63, 256), (3, 1, 4, 2, 40, 64)])
-def test_attn_prefill(B, S, Nq, Nkv, past, Smax):
+@pytest.mark.parametrize("queries_per_wave", [16, 32])
+def test_attn_prefill(B, S, Nq, Nkv, past, Smax, queries_per_wave, monkeypatch):
     """Causal attention for S query tokens against the oracle (tolerance as for the single-query kernel: rel-L2
-    5e-3, max-abs 2^-7 of the largest output) and against plain PyTorch fp32 causal softmax attention (1e-2)."""
+    5e-3, max-abs 2^-7 of the largest output) and against plain PyTorch fp32 causal softmax attention (1e-2), with
+    both of the kernel's shapes (the library picks by launch size; the knob forces one)."""
     _llm()
+    monkeypatch.setenv("TPPX_ATTN_QG", str(queries_per_wave // 16))
     L = past + S
     q = randn_bf16((B, S, Nq, 128), 1.0, 51)
     k = randn_bf16((B, Nkv, Smax, 128), 1.0, 52)
@@ -240,8 +243,10 @@ def test_attn_prefill_full_size_rows_equal_single_query_problem():
         assert np.abs(g - r).max() <= 2.0 ** -7 * np.abs(r).max(), i
 
 
-def test_attn_prefill_mask_and_errors():
+@pytest.mark.parametrize("queries_per_wave", [16, 32])
+def test_attn_prefill_mask_and_errors(queries_per_wave, monkeypatch):
     F = _llm()
+    monkeypatch.setenv("TPPX_ATTN_QG", str(queries_per_wave // 16))
     from tpp_pytorch_extension._lib import TppxError
     B, S, Nq, Smax = 2, 70, 4, 128
     q = randn_bf16((B, S, Nq, 128), 1.0, 61)
