@@ -542,3 +542,50 @@ def test_optimize_model_for_llama_against_transformers(weight_dtype):
         assert cache_o.get_seq_length() == 21
     out = F.generate_greedy(opt_model, ids[:1].cuda(), 5)
     assert out.shape == (1, 24) and torch.equal(out[:, :19].cpu(), ids[:1])
+
+
+def _tiny_optimized_llama(weight_dtype="mxfp4", seed=21):
+    transformers = pytest.importorskip("transformers")
+    F = _llm()
+    cfg = transformers.LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4,
+                                   num_key_value_heads=2, vocab_size=1024, max_position_embeddings=256, head_dim=128,
+                                   rms_norm_eps=1e-5, attn_implementation="eager")
+    torch.manual_seed(seed)
+    return F, F.OptimizeModelForLlama(transformers.LlamaForCausalLM(cfg).eval(), torch.bfloat16, "cuda", weight_dtype).eval()
+
+
+def test_transformers_generate_on_optimized_model():
+    """run_generation.py:420 calls model.generate(): greedy generate() of the installed transformers on the optimized
+    model (cache created by the patched forward, or a TppCache handed in) returns what the package's own greedy
+    loop returns; beam search runs on the same cache through reorder_cache."""
+    F, opt = _tiny_optimized_llama()
+    from tpp_pytorch_extension.llm.llm_common import TppCache
+    ids = torch.randint(0, 1024, (2, 19), generator=torch.Generator().manual_seed(12)).cuda()
+    am = torch.ones_like(ids)
+    am[1, :4] = 0
+    want = F.generate_greedy(opt, ids, 6, attention_mask=am)
+    got = opt.generate(input_ids=ids, attention_mask=am, max_new_tokens=6, do_sample=False)
+    assert torch.equal(got, want)
+    got = opt.generate(input_ids=ids, attention_mask=am, max_new_tokens=6, do_sample=False,
+                       past_key_values=TppCache(capacity=64))
+    assert torch.equal(got, want)
+    beams = opt.generate(input_ids=ids, attention_mask=am, max_new_tokens=6, do_sample=False, num_beams=3)
+    assert beams.shape == want.shape and torch.equal(beams[:, :19], ids)
+
+
+def test_cache_reorder_moves_sequences():
+    """TppCache.reorder_cache (attn.h:327-366): after reordering with [1, 0] a decode step on swapped tokens gives
+    the swapped logits of the same step on the untouched cache, bit for bit (rows of a decode step do not mix)."""
+    F, opt = _tiny_optimized_llama()
+    ids = torch.randint(0, 1024, (2, 23), generator=torch.Generator().manual_seed(13)).cuda()
+    nxt = torch.tensor([[5], [9]], device="cuda")
+    with torch.no_grad():
+        a = opt(input_ids=ids, use_cache=True)
+        la = opt(input_ids=nxt, past_key_values=a.past_key_values, use_cache=True).logits
+        b = opt(input_ids=ids, use_cache=True)
+        b.past_key_values.reorder_cache(torch.tensor([1, 0], device="cuda"))
+        lb = opt(input_ids=nxt.flip(0), past_key_values=b.past_key_values, use_cache=True).logits
+    assert torch.equal(lb, la.flip(0))
+    from tpp_pytorch_extension._lib import TppxError
+    with pytest.raises(TppxError):
+        b.past_key_values.reorder_cache(torch.tensor([0, 1, 0], device="cuda"))

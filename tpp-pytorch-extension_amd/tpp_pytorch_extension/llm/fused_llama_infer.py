@@ -86,6 +86,18 @@ class TppCache:
             self._host_len = int(max_length)
             self.seq_len_dev.fill_(self._host_len)
 
+    def reorder_cache(self, beam_idx):
+        """attn.h:327-366 (beam search): afterwards sequence b continues the keys and values sequence beam_idx[b]
+        held.  The reference records the indices and gathers inside attention; here the rows move once per step."""
+        beam_idx = beam_idx.to(torch.int64)
+        for i, (k, v) in self.layers.items():
+            if beam_idx.numel() != k.shape[0]:
+                raise TppxError(_lib.ESHAPE, f"TppCache.reorder_cache: {beam_idx.numel()} indices for {k.shape[0]} sequences")
+            n = self._host_len
+            k[:, :, :n].copy_(k[:, :, :n].index_select(0, beam_idx.to(k.device)))
+            v[:, :, :n].copy_(v[:, :, :n].index_select(0, beam_idx.to(v.device)))
+        self._sums_of = None
+
     def align_and_invert_mask(self, t_mask, pad_value=-10000.0):
         """attn.h:310-322: [B][S] 0/1 mask -> additive mask padded to a multiple of 32 keys."""
         B, S = t_mask.shape

@@ -119,7 +119,11 @@ def FixLinear(self, bk=None, bc=None, layer_dtype=global_layer_dtype, parallel_d
 class TppCache:
     """past_key_values object of the optimized models (llm_common.py:80-182): a thin wrapper around the cache the
     fused decoder layers append to (`get_cpp()`).  Keys are appended inside the layers, so `update` is not a
-    way in; beam reordering is not built."""
+    way in."""
+
+    # what transformers' generate() asks of a cache object it did not create
+    is_compileable = False
+    is_sliding = False
 
     def __init__(self, capacity=0, **kwargs):
         from .fused_llama_infer import TppCache as _CoreCache
@@ -157,7 +161,7 @@ class TppCache:
         return self.tpp_cache.align_and_invert_mask(mask.to(torch.bfloat16), torch.finfo(torch.bfloat16).min)
 
     def reorder_cache(self, beam_idx):
-        raise NotImplementedError("beam search is not part of the single-GPU decode path")
+        self.tpp_cache.reorder_cache(beam_idx)
 
     def get_cpp(self):
         return self.tpp_cache
