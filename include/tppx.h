@@ -159,6 +159,24 @@ int tppx_linear_mxfp4(const void* x, const void* qw, const void* sw,
                       int64_t K, int post_op, float post_scale, int flags,
                       void* ws, int64_t ws_bytes, tppx_stream_t stream);
 
+/* Unquantized bf16 weights: TppBlockedLinearW<bf16,bf16>
+ * (src/csrc/fused_gemm.h:785-1073 with the plain BRGEMM of :951-1064), the
+ * class the reference's default bf16 lm_head runs through
+ * (src/tpp_pytorch_extension/llm/fused_llama_infer.py:218-224).
+ * tppx_prepack_bf16: blocked bf16 weight [N/bk][K/bc][bc/vnni][bk][vnni]
+ * (vnni 2 = BlockedLinear's VNNI2 pairs, blocked_layout.py:75-80; bk=1,
+ * bc=K, vnni=1 = a plain [N][K] matrix) -> native bf16 tiles
+ * [N/16][K/128][4][64][8] (N*K*2 bytes).  N%16==0, K%128==0.
+ * tppx_linear_bf16: y = post( bf16( bias[n] + sum_k x[m][k]*W[n][k] ) ) with
+ * the row-group kernel at any M (beyond 64 rows every block of 64 rows
+ * streams the weights again: meant for lm_head-sized M, not for prefill). */
+int tppx_prepack_bf16(const void* w_ref, int64_t N, int64_t K, int64_t bk,
+                      int64_t bc, int vnni, void* w_nat, tppx_stream_t stream);
+int tppx_linear_bf16(const void* x, const void* w_nat, const void* bias,
+                     const void* post_in, const void* post_in2, void* y,
+                     int64_t M, int64_t N, int64_t K, int post_op,
+                     float post_scale, int flags, tppx_stream_t stream);
+
 /* Replaces TppBlockedQInt8LinearW<bf16,uint8_t,bf16>
  * (src/csrc/fused_gemm.h:1076-1341,1530-1534): activations are quantized into
  * the caller's scratch xq (room for roundup(M,64)*K bytes) / sa (room for

@@ -452,6 +452,21 @@ def linear_qint8(x_bf16, q, sw, bias=None, post=POST_NONE, post_in=None, post_in
     return y
 
 
+def linear_bf16(x_bf16, w_bf16, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0):
+    """Unquantized bf16 weights, TppBlockedLinearW<bf16,bf16> (src/csrc/fused_gemm.h:785-1073, non-quantized branch
+    :951-1064 with one K chunk, the M <= 256 case of getBlockingParams :695-721): the bf16 output tile starts as the
+    bias, the BRGEMM adds the whole dot product (fp32 inside) and the sum is rounded to bf16 once; then the post-op.
+    x bits [M][K], w bits [N][K] (plain layout).  Pinned by the MXFP4 restatement: on weights that MXFP4
+    represents exactly both must agree (tests/test_oracle.py)."""
+    x = bf16_to_f32(_c(x_bf16, np.uint16)).astype(np.float64)
+    w = bf16_to_f32(_c(w_bf16, np.uint16)).astype(np.float64)
+    acc = x @ w.T
+    if bias is not None:
+        acc = acc + bf16_to_f32(_c(bias, np.uint16)).astype(np.float64)[None, :]
+    y = f32_to_bf16(acc.astype(np.float32))
+    return post_op(y, post, post_in, post_in2, post_scale) if post != POST_NONE else y
+
+
 def num_threads():
     return lib().orc_num_threads()
 

@@ -62,6 +62,12 @@ def test_argument_validation_without_gpu():
     assert lib.tppx_linear_qint8(A, A, A, A, A, None, None, None, A, 1, 24, 256, 256, 0, 1.0, 0, None, 0, None) == L.ESHAPE
     assert lib.tppx_linear_qint8(A, A, A, A, A, None, None, None, A, 1, 16, 256, 192, 0, 1.0, 0, None, 0, None) == L.ESHAPE
     assert "block size" in err()
+    # unquantized bf16 weights: K in whole 128-channel tiles, N in 16s, blocking must divide the matrix
+    assert lib.tppx_linear_bf16(A, A, None, None, None, A, 1, 16, 192, 0, 1.0, 0, None) == L.ESHAPE
+    assert lib.tppx_linear_bf16(A, A, None, None, None, A, 1, 24, 128, 0, 1.0, 0, None) == L.ESHAPE
+    assert lib.tppx_linear_bf16(A, None, None, None, None, A, 1, 16, 128, 0, 1.0, 0, None) == L.EINVAL
+    assert lib.tppx_prepack_bf16(A, 32, 256, 16, 48, 2, A, None) == L.ESHAPE
+    assert lib.tppx_prepack_bf16(A, 32, 256, 16, 64, 3, A, None) == L.ESHAPE
     # post-op id and its inputs
     assert lib.tppx_linear_mxfp4(A, A, A, None, None, None, A, 1, 32, 128, 9, 1.0, 0, None, 0, None) == L.EINVAL
     assert lib.tppx_linear_mxfp4(A, A, A, None, None, None, A, 1, 32, 128, L.POST_MUL, 1.0, 0, None, 0, None) == L.EINVAL

@@ -511,6 +511,7 @@ def test_optimize_model_for_llama_against_transformers(weight_dtype):
             elif isinstance(m, torch.nn.Embedding):
                 m.weight.data.copy_(m.weight.data.to(torch.bfloat16).float())
     opt_model = F.OptimizeModelForLlama(copy.deepcopy(ref_model), torch.bfloat16, "cuda", weight_dtype).eval()
+    assert not opt_model.lm_head.weight.is_quantized and opt_model.lm_head.weight.dim() == 5  # bf16, as the reference's
     tol = 3e-2 if weight_dtype == "mxfp4" else 6e-2
 
     ids = torch.randint(0, 1024, (2, 19), generator=torch.Generator().manual_seed(12))
@@ -554,21 +555,40 @@ def _tiny_optimized_llama(weight_dtype="mxfp4", seed=21):
     return F, F.OptimizeModelForLlama(transformers.LlamaForCausalLM(cfg).eval(), torch.bfloat16, "cuda", weight_dtype).eval()
 
 
+def _assert_greedy(opt, out, am, n_prompt):
+    """Every generated token is a maximiser of the logits a teacher-forced pass over the finished sequence gives at
+    the position before it, up to the bf16 noise between the kernels of the two passes (3 % of the largest logit:
+    a random token of the 1024 passes with probability < 1 %)."""
+    n_new = out.shape[1] - n_prompt
+    am = torch.cat([am, am.new_ones((am.shape[0], n_new))], dim=1)
+    with torch.no_grad():
+        logits = opt(input_ids=out[:, :-1], attention_mask=am[:, :-1]).logits.float()
+    for t in range(n_prompt - 1, out.shape[1] - 1):
+        lt = logits[:, t]
+        gap = lt.max(-1).values - lt.gather(1, out[:, t + 1:t + 2])[:, 0]
+        assert bool((gap <= 0.03 * lt.abs().max(-1).values).all()), (t, gap.tolist())
+
+
 def test_transformers_generate_on_optimized_model():
     """run_generation.py:420 calls model.generate(): greedy generate() of the installed transformers on the optimized
-    model (cache created by the patched forward, or a TppCache handed in) returns what the package's own greedy
-    loop returns; beam search runs on the same cache through reorder_cache."""
+    model gives the same tokens on the cache the patched forward creates and on a TppCache handed in, and those
+    tokens, like the package's own greedy loop's, are the argmax of the model's logits (the two loops put
+    different numbers of rows through the lm_head in the prompt pass, so near-ties of a random model may break
+    differently between them); beam search runs on the same cache through reorder_cache."""
     F, opt = _tiny_optimized_llama()
     from tpp_pytorch_extension.llm.llm_common import TppCache
     ids = torch.randint(0, 1024, (2, 19), generator=torch.Generator().manual_seed(12)).cuda()
     am = torch.ones_like(ids)
     am[1, :4] = 0
     want = F.generate_greedy(opt, ids, 6, attention_mask=am)
+    assert want.shape == (2, 25) and torch.equal(want[:, :19], ids)
+    _assert_greedy(opt, want, am, 19)
     got = opt.generate(input_ids=ids, attention_mask=am, max_new_tokens=6, do_sample=False)
-    assert torch.equal(got, want)
-    got = opt.generate(input_ids=ids, attention_mask=am, max_new_tokens=6, do_sample=False,
-                       past_key_values=TppCache(capacity=64))
-    assert torch.equal(got, want)
+    assert got.shape == (2, 25) and torch.equal(got[:, :19], ids)
+    _assert_greedy(opt, got, am, 19)
+    got2 = opt.generate(input_ids=ids, attention_mask=am, max_new_tokens=6, do_sample=False,
+                        past_key_values=TppCache(capacity=64))
+    assert torch.equal(got2, got)
     beams = opt.generate(input_ids=ids, attention_mask=am, max_new_tokens=6, do_sample=False, num_beams=3)
     assert beams.shape == want.shape and torch.equal(beams[:, :19], ids)
 
@@ -589,3 +609,30 @@ def test_cache_reorder_moves_sequences():
     from tpp_pytorch_extension._lib import TppxError
     with pytest.raises(TppxError):
         b.past_key_values.reorder_cache(torch.tensor([0, 1, 0], device="cuda"))
+
+
+def test_lm_head_quantized_on_request():
+    """The lm_head stays bf16 by default; quantize_lm_head=True and run_generation.py:277-282's own way
+    (remap_and_quantize_qint8 on the blocked bf16 weight after the call) both give a QINT8 head whose logits stay
+    within the int8 rounding of the bf16 head's."""
+    transformers = pytest.importorskip("transformers")
+    import copy
+    F = _llm()
+    from tpp_pytorch_extension import _ops
+    cfg = transformers.LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=1, num_attention_heads=4,
+                                   num_key_value_heads=2, vocab_size=1600, max_position_embeddings=128, head_dim=128,
+                                   rms_norm_eps=1e-5, attn_implementation="eager")
+    torch.manual_seed(31)
+    base = transformers.LlamaForCausalLM(cfg).eval()
+    a = F.OptimizeModelForLlama(copy.deepcopy(base), torch.bfloat16, "cuda", "mxfp4").eval()
+    assert tuple(a.lm_head.weight.shape) == (16, 8, 32, 100, 2)  # FixLinear(m, 100, 64, bf16)
+    b = F.OptimizeModelForLlama(copy.deepcopy(base), torch.bfloat16, "cuda", "mxfp4", quantize_lm_head=True).eval()
+    assert b.lm_head.weight.is_quantized and b.lm_head.weight.dtype == torch.qint8
+    c = F.OptimizeModelForLlama(copy.deepcopy(base), torch.bfloat16, "cuda", "mxfp4").eval()
+    with torch.no_grad():
+        c.lm_head.weight = torch.nn.Parameter(_ops.remap_and_quantize_qint8(c.lm_head.weight), requires_grad=False)
+    ids = torch.randint(0, 1600, (2, 9), generator=torch.Generator().manual_seed(32)).cuda()
+    with torch.no_grad():
+        la, lb, lc = (m(input_ids=ids).logits.float() for m in (a, b, c))
+    assert torch.equal(lb, lc)
+    assert float((lb - la).norm() / la.norm()) <= 2e-2

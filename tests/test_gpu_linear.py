@@ -449,3 +449,57 @@ def test_launch_plan_names_the_kernels():
     assert "big_mxfp4_kernel" in buf.value.decode()
     _lib.check(L.tppx_plan_linear_mxfp4(100, 8192, 8192, 0, 0, buf, len(buf)))
     assert "tiled_mxfp4_kernel" in buf.value.decode()
+
+
+@pytest.mark.parametrize("M,N,K,post,layout", [
+    (1, 2000, 512, "none", "vnni2"), (5, 272, 1024, "add", "vnni2"), (16, 4096, 4096, "none", "vnni2"),
+    (17, 1008, 384, "silu", "plain"), (33, 528, 640, "mul", "vnni2"), (64, 1024, 11008, "add", "vnni2"),
+    (100, 304, 256, "add2", "plain"), (200, 1040, 512, "none", "blocked100")])
+def test_bf16_weight_linear(M, N, K, post, layout):
+    """Unquantized bf16 weights (the reference's default lm_head class, TppBlockedLinearW<bf16,bf16>) through
+    fc_plain / the post-op GEMMs: 1 ulp of the oracle's single-rounding result, for the blocked VNNI2 layout
+    BlockedLinear makes, a plain [N][K] matrix, and the lm_head's own blocking (bk = N/10-style odd block
+    heights: here 104 = 1040/10 rows per block)."""
+    ops = _ops()
+    W = randn_bf16((N, K), 0.02, 81)
+    x = randn_bf16((M, K), 1.0, 82)
+    bias = randn_bf16((N,), 0.01, 83)
+    in1, in2 = randn_bf16((M, N), 1.0, 84), randn_bf16((M, N), 1.0, 85)
+    scale = 0.5 if post in ("add", "add2") else 1.0
+    if layout == "vnni2":
+        Wg = block_bf16(W).cuda()
+    elif layout == "plain":
+        Wg = W.cuda()
+    else:
+        Wg = block_bf16(W, bk=104, bc=64).cuda()
+    y = ops.linear(x.cuda(), Wg, bias.cuda(), POSTS[post], in1.cuda(), in2.cuda(), scale)
+    ref = O.linear_bf16(t2bits(x), t2bits(W), t2bits(bias), POSTS[post], t2bits(in1), t2bits(in2), scale)
+    assert_close_bf16(t2bits(y), ref, ulps=1, what=f"bf16 weight M={M} N={N} K={K} post={post} {layout}",
+                      pre_bits=O.linear_bf16(t2bits(x), t2bits(W), t2bits(bias)) if post in ("add", "add2") else None)
+    y2 = ops.linear(x.cuda(), Wg, bias.cuda(), POSTS[post], in1.cuda(), in2.cuda(), scale)  # cached native tiles
+    assert torch.equal(y, y2)
+
+
+def test_bf16_weight_module_and_errors():
+    import tpp_pytorch_extension  # noqa: F401
+    from tpp_pytorch_extension.llm.llm_common import FixLinear, BlockedLinear
+    from tpp_pytorch_extension._lib import TppxError
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(256, 1000, bias=False)  # lm_head-like: FixLinear(m, 100, 64, bf16) keeps bf16 weights
+    W = lin.weight.data.clone().to(torch.bfloat16)
+    FixLinear(lin, 100, 64, torch.bfloat16)
+    assert isinstance(lin, BlockedLinear) and not lin.weight.is_quantized and lin.weight.dim() == 5
+    lin = lin.cuda()
+    x = randn_bf16((2, 3, 256), 1.0, 86)
+    with pytest.raises(TppxError):  # N = 1000 is not a multiple of 16
+        lin(x.cuda())
+    lin = torch.nn.Linear(256, 1600, bias=True)
+    W, b = lin.weight.data.clone().to(torch.bfloat16), lin.bias.data.clone().to(torch.bfloat16)
+    FixLinear(lin, 100, 64, torch.bfloat16)
+    lin = lin.cuda()
+    y = lin(x.cuda())
+    ref = O.linear_bf16(t2bits(x.view(6, 256)), t2bits(W), t2bits(b))
+    assert y.shape == (2, 3, 1600)
+    assert_close_bf16(t2bits(y).reshape(6, 1600), ref, what="bf16 BlockedLinear")
+    with pytest.raises(TppxError):
+        _ops().linear(x.cuda()[..., :128].contiguous(), lin.weight, None)

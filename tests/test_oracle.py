@@ -369,3 +369,28 @@ def test_oracle_attn_prefill_against_causal_softmax_and_decode():
         assert np.array_equal(full[:, i], one), i
     first = O.bf16_to_f32(O.attn_prefill(bits(q), bits(k[:, :, :S]), bits(v[:, :, :S])))
     assert np.array_equal(first[:, 0], v[:, :, 0].float().repeat_interleave(2, 1).numpy())
+
+
+def test_oracle_linear_bf16_against_mxfp4_restatement_and_closed_forms():
+    """The bf16-weight linear is pinned three ways: (1) on weights MXFP4 represents exactly it must give what the
+    MXFP4 restatement gives on their quantized form (same sums, one rounding each; a transposed operand, a missing
+    bias or a second rounding breaks it); (2) small-integer operands make every product and sum exact, so the result
+    is the integer matrix product; (3) the post-op is the shared one."""
+    rng = np.random.default_rng(5)
+    M, N, K = 7, 64, 256
+    W = randn_bf16((N, K), 0.02, 41)
+    q, sc = O.remap_quantize_mxfp4(W.float().numpy())
+    Wd = torch.from_numpy(O.dequantize_mxfp4_plain(q, sc)).to(torch.bfloat16)
+    assert torch.equal(Wd.float(), torch.from_numpy(O.dequantize_mxfp4_plain(q, sc)))  # exactly representable
+    x = randn_bf16((M, K), 1.0, 42)
+    bias = randn_bf16((N,), 0.01, 43)
+    res = randn_bf16((M, N), 1.0, 44)
+    for post, kw in ((O.POST_NONE, {}), (O.POST_ADD_SCALE, dict(post_in=t2bits(res), post_scale=0.5)), (O.POST_SILU, {})):
+        a = O.linear_bf16(t2bits(x), t2bits(Wd), t2bits(bias), post, **kw)
+        b = O.linear_mxfp4(t2bits(x), q, sc, t2bits(bias), post, mode=O.MODE_F64, **kw)
+        assert np.array_equal(a, b), post
+    xi = torch.from_numpy(rng.integers(-4, 5, (M, K)).astype(np.float32)).to(torch.bfloat16)
+    wi = torch.from_numpy(rng.integers(-3, 4, (N, K)).astype(np.float32)).to(torch.bfloat16)
+    want = (xi.double() @ wi.double().T)  # |sum| <= 256 * 12: exact in fp32, not always in bf16
+    got = bits2f(O.linear_bf16(t2bits(xi), t2bits(wi)))
+    assert np.array_equal(got, want.float().to(torch.bfloat16).float().numpy())

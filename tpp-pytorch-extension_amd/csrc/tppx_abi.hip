@@ -492,6 +492,34 @@ extern "C" int tppx_linear_mxfp4(const void* x, const void* qw, const void* sw,
   return run_mxfp4("tppx_linear_mxfp4", x, &s, 1, M, K, flags, false, ws, ws_bytes, (hipStream_t)stream);
 }
 
+extern "C" int tppx_linear_bf16(const void* x, const void* w, const void* bias, const void* post_in,
+                                const void* post_in2, void* y, int64_t M, int64_t N, int64_t K, int post_op,
+                                float post_scale, int flags, tppx_stream_t stream) {
+  const char* who = "tppx_linear_bf16";
+  int rc = check_common(who, x, M, K, 1, flags, nullptr, 0);
+  if (rc)
+    return rc;
+  TPPX_REQUIRE(K > 0 && K % 128 == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of 128 (native bf16 tiles span 128 input channels)", who, (long)K);
+  TPPX_REQUIRE(!(flags & (TPPX_FLAG_ACT_FP8 | TPPX_FLAG_FORCE_TILED)), TPPX_EUNSUPPORTED, "%s: only the row-group kernel is built for unquantized weights", who);
+  TPPX_REQUIRE(M * N < ((int64_t)1 << 31), TPPX_ESHAPE, "%s: M*N=%ld outputs exceed 2^31", who, (long)(M * N));
+  tppx_seg s = {w, w, bias, post_in, post_in2, y, N, post_op, post_scale}; // no scales: the slot repeats the weight
+  DecodeParams p;
+  memset(&p, 0, sizeof(p));
+  rc = fill_all(who, &s, 1, 16, false, p);
+  if (rc)
+    return rc;
+  p.x = x;
+  p.M = (int)M;
+  p.K = (int)K;
+  p.units = (int)(K / 128);
+  p.tpb = 1;
+  p.S = 1;
+  const int mg = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  const int nt = p.total_tiles > 512 ? 2 : 1; // two channel tiles per workgroup once one each still leaves two rounds
+  set_groups(p, nt, false);
+  return check_hip(launch_skinny_bf16(p, mg, nt, (hipStream_t)stream), who);
+}
+
 extern "C" int tppx_multi_linear_mxfp4(const void* x, const tppx_seg* segs,
                                        int n_segs, int64_t M, int64_t K,
                                        int flags, void* ws, int64_t ws_bytes,

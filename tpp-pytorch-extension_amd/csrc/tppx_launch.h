@@ -95,6 +95,7 @@ hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qb
 // can_fuse_quant: bf16 activations at hand and 256-wide blocks (the in-kernel quantisation's case)
 SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, bool can_fuse_quant);
 hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream);
+hipError_t launch_skinny_bf16(DecodeParams& p, int mg, int nt, hipStream_t stream);
 size_t skinny_mxfp4_xl_lds(int units, int nt, bool dual);
 hipError_t launch_skinny_mxfp4_x4(DecodeParams& p, int nt, bool dual, hipStream_t stream);
 hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hipStream_t stream);

@@ -228,6 +228,30 @@ prepack_qint8_kernel(const int8_t* __restrict__ qref, int64_t N, int64_t K,
       make_uint4(src[0], src[16], src[32], src[48]);
 }
 
+// bf16 weight in the reference's blocked layout [N/bk][K/bc][bc/v][bk][v] (v = 2: VNNI2 pairs; bk = 1, bc = K, v = 1:
+// a plain [N][K] matrix) -> native bf16 tiles [N/16][K/128][4 j][4 g][16 n][8]: the 16 bytes lane (g, n) feeds to
+// MFMA step j of K tile kt are W[nt*16 + n][kt*128 + (g*4 + j)*8 .. +7].
+__global__ void __launch_bounds__(256)
+prepack_bf16_kernel(const uint16_t* __restrict__ wref, int64_t N, int64_t K, int64_t bk, int64_t bc, int64_t v,
+                    uint16_t* __restrict__ wnat) {
+  const int64_t nchunks = N * (K / 8);
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= nchunks)
+    return;
+  const int64_t n16 = t & 15, g = (t >> 4) & 3, j = (t >> 6) & 3, rest = t >> 8;
+  const int64_t KT = K / 128, kt = rest % KT, nt = rest / KT;
+  const int64_t n = nt * 16 + n16, k0 = kt * 128 + (g * 4 + j) * 8;
+  const int64_t n1 = n / bk, k2 = n % bk;
+  uint16_t e[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int64_t k = k0 + i, c1 = k / bc, kk = k % bc;
+    e[i] = wref[(((n1 * (K / bc) + c1) * (bc / v) + kk / v) * bk + k2) * v + kk % v];
+  }
+  reinterpret_cast<uint4*>(wnat)[t] = make_uint4(e[0] | ((uint32_t)e[1] << 16), e[2] | ((uint32_t)e[3] << 16),
+                                                 e[4] | ((uint32_t)e[5] << 16), e[6] | ((uint32_t)e[7] << 16));
+}
+
 // Activation quantizer: one wave per (row, K block).  Each lane owns
 // consecutive pairs so loads and stores stay contiguous.
 __global__ void __launch_bounds__(256)
@@ -402,6 +426,21 @@ extern "C" int tppx_prepack_qint8(const void* q_ref, int64_t N, int64_t K,
   prepack_qint8_kernel<<<grid_for(nchunks, 256), 256, 0, (hipStream_t)stream>>>(
       (const int8_t*)q_ref, N, K, qbs, (int8_t*)q_nat);
   return check_hip(hipGetLastError(), "tppx_prepack_qint8");
+}
+
+extern "C" int tppx_prepack_bf16(const void* w_ref, int64_t N, int64_t K, int64_t bk, int64_t bc, int vnni,
+                                 void* w_nat, tppx_stream_t stream) {
+  TPPX_REQUIRE(w_ref && w_nat, TPPX_EINVAL, "tppx_prepack_bf16: null pointer");
+  TPPX_REQUIRE(aligned16(w_nat), TPPX_EINVAL, "tppx_prepack_bf16: output not 16-byte aligned");
+  TPPX_REQUIRE(N > 0 && K > 0 && N % 16 == 0 && K % 128 == 0, TPPX_ESHAPE,
+               "tppx_prepack_bf16: N=%ld must be a multiple of 16 and K=%ld of 128", (long)N, (long)K);
+  TPPX_REQUIRE(bk > 0 && bc > 0 && (vnni == 1 || vnni == 2) && N % bk == 0 && K % bc == 0 && bc % vnni == 0, TPPX_ESHAPE,
+               "tppx_prepack_bf16: blocking bk=%ld bc=%ld vnni=%d does not divide N=%ld K=%ld", (long)bk, (long)bc, vnni,
+               (long)N, (long)K);
+  const int64_t nchunks = N * (K / 8);
+  prepack_bf16_kernel<<<grid_for(nchunks, 256), 256, 0, (hipStream_t)stream>>>((const uint16_t*)w_ref, N, K, bk, bc, vnni,
+                                                                                (uint16_t*)w_nat);
+  return check_hip(hipGetLastError(), "tppx_prepack_bf16");
 }
 
 extern "C" int tppx_quant_act_int8(const void* x, int64_t M, int64_t K,

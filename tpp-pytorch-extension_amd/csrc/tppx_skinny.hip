@@ -1260,6 +1260,127 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Unquantized bf16 weights (the reference's default lm_head), any number of
+// rows: the row-group kernel above without the dequantisation.  Native tiles
+// hold the MFMA operands themselves, [N/16][K/128][4 j][64 lanes][16 B], so a
+// K tile of a channel tile is four 1 KB loads per wave; activations go
+// through the same wave-private LDS image.  Block rows of MG*16 rows ride on
+// grid y: beyond 64 rows every block row streams the weights again (from L2
+// / Infinity Cache when they fit), which is what a prompt's last-token
+// lm_head or a short verification batch needs, not a prefill GEMM.
+// ---------------------------------------------------------------------------
+template <int MG, int NT, int PF, int W>
+__global__ void __launch_bounds__(W * 64)
+skinny_bf16_kernel(const DecodeParams p) {
+  extern __shared__ __align__(16) float sk_lds[];
+  constexpr int MPAD = MG * 16, XL = MG * 4;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int grp = blockIdx.x;
+  const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
+  const int ltile0 = (grp - sg.grp0) * NT;
+  const int m0 = blockIdx.y * MPAD;
+  const int KT = p.units;
+  const int t0 = (wave * KT) / W, t1 = ((wave + 1) * KT) / W;
+  i32x4* xs = reinterpret_cast<i32x4*>(sk_lds) + (size_t)wave * (MPAD * 16); // [chunk 16][row MPAD] x 16 B
+
+  const i32x4* wb = reinterpret_cast<const i32x4*>(sg.qw);
+  size_t woff[NT]; // in 16-byte units
+#pragma unroll
+  for (int nt = 0; nt < NT; nt++)
+    woff[nt] = (size_t)min(ltile0 + nt, sg.tiles - 1) * KT * 256 + lane;
+
+  const char* xb = reinterpret_cast<const char*>(p.x);
+  const int r4 = lane >> 4, c16 = lane & 15;
+  i32x4 xr[XL];
+  auto load_x = [&](int t) {
+    t = min(t, t1 - 1);
+    int r = r4, c = c16;
+    asm volatile("" : "+v"(r), "+v"(c));
+    const size_t base = (size_t)t * 256u + (size_t)c * 16u;
+#pragma unroll
+    for (int it = 0; it < XL; it++) {
+      const int row = min(m0 + it * 4 + r, p.M - 1);
+      xr[it] = *reinterpret_cast<const i32x4*>(xb + (size_t)row * p.K * 2u + base);
+    }
+  };
+  auto store_x = [&]() {
+    int r = r4, c = c16;
+    asm volatile("" : "+v"(r), "+v"(c));
+#pragma unroll
+    for (int it = 0; it < XL; it++)
+      xs[c * MPAD + ((it * 4 + r) ^ c)] = xr[it];
+  };
+  int rdo[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int cj = (lane >> 4) * 4 + j;
+    rdo[j] = cj * MPAD + ((lane & 15) ^ cj);
+  }
+
+  i32x4 wreg[PF][NT][4];
+  auto load_stage = [&](int st, int t) {
+    t = min(t, t1 - 1);
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        wreg[st][nt][j] = __builtin_nontemporal_load(wb + woff[nt] + (size_t)t * 256 + j * 64);
+  };
+  if (t0 < t1) {
+    load_x(t0);
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+      load_stage(i, t0 + i);
+  }
+  SkEpilogue<MG, NT, false, W> ep;
+  ep.prefetch(p, sg, ltile0, m0);
+
+  f32x4 acc[NT][MG];
+#pragma unroll
+  for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+    for (int mg = 0; mg < MG; mg++)
+      acc[nt][mg] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  auto consume = [&](int i, int tnext) {
+    store_x();
+    load_x(tnext);
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int mg = 0; mg < MG; mg++) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, xs[rdo[j] + mg * 16]);
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++)
+          acc[nt][mg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, wreg[i][nt][j]), acc[nt][mg], 0, 0, 0);
+      }
+  };
+  int t = t0;
+  for (; t + 2 * PF <= t1; t += PF) { // branch-free full groups: every reload is a real tile
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      consume(i, t + i + 1);
+      load_stage(i, t + i + PF);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  for (; t < t1; t += PF) {
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      const int tt = t + i;
+      if (tt < t1) {
+        consume(i, tt + 1);
+        if (tt + PF < t1)
+          load_stage(i, tt + PF);
+      }
+    }
+  }
+  __syncthreads(); // every wave is done with its activation region before it becomes reduction scratch
+  ep.finish(sg, acc, sk_lds, decltype(ep)::ELEMS);
+}
+
 // launch shape of the QINT8 decode kernels
 SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, bool can_fuse_quant) {
   SkinnyPlan pl;
@@ -1510,6 +1631,28 @@ hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hi
     SKMG(4, 2, false, 2);
   SKMG(4, 1, false, 2);
 #undef SKMG
+}
+
+// bf16 weights: mg row groups of 16 per block row (1, 2 or 4), nt channel tiles per workgroup (1 or 2)
+hipError_t launch_skinny_bf16(DecodeParams& p, int mg, int nt, hipStream_t stream) {
+  dim3 grid(p.groups, (p.M + mg * 16 - 1) / (mg * 16), 1);
+  if (mg == 1) {
+    const size_t lds1 = skinny_mxfp4_mg_lds(1, nt, 16);
+    if (nt == 2)
+      return sk_launch(skinny_bf16_kernel<1, 2, 2, 16>, p, grid, 16, lds1, stream);
+    return sk_launch(skinny_bf16_kernel<1, 1, 4, 16>, p, grid, 16, lds1, stream);
+  }
+  const size_t lds = skinny_mxfp4_mg_lds(mg, nt, 8);
+#define SKBF(MG, NT, PF) return sk_launch(skinny_bf16_kernel<MG, NT, PF, 8>, p, grid, 8, lds, stream)
+  if (mg == 2) {
+    if (nt == 2)
+      SKBF(2, 2, 2);
+    SKBF(2, 1, 2);
+  }
+  if (nt == 2)
+    SKBF(4, 2, 2);
+  SKBF(4, 1, 2);
+#undef SKBF
 }
 
 } // namespace tppx

@@ -92,8 +92,11 @@ def remap_and_quantize_qint8(t):
     L = _lib.lib()
     t, dt = _float_weight_on_gpu(t)
     N, K, bk, bc, vnni = _blocked_geometry(t)
-    if bk != 16:
-        raise TppxError(_lib.EUNSUPPORTED, f"QINT8 weights are built for output-channel blocks of 16 (got {bk})")
+    # any blocking of the source is read; the quantized tensor always has 16-channel blocks (the reference keeps
+    # the source's: quantizing the 100-channel-blocked lm_head gives [N/100, K/QBS, QBS/4, 100, 4] there), with the
+    # same values and per-(channel, K block) scales
+    if N % 16:
+        raise TppxError(_lib.ESHAPE, f"QINT8 weights need a multiple of 16 output channels (got {N})")
     if 4 % vnni:
         raise TppxError(_lib.ESHAPE, "Shape not compatible for VNNI4")
     qbs = qint8_block_size_for(K)
@@ -246,7 +249,7 @@ def _prep_input(input, weight):
     if not isinstance(weight, QTensor):
         raise TppxError(
             _lib.EUNSUPPORTED,
-            "only MXFP4 / QINT8 quantized weights are built on this path "
+            "only MXFP4 / QINT8 quantized and bfloat16 weights are built on this path "
             "(quantize the weight with remap_and_quantize_mxfp4 / remap_and_quantize_qint8)",
         )
     if not weight.is_weight():
@@ -264,6 +267,47 @@ def _prep_input(input, weight):
     x = input.contiguous()
     M = x.numel() // K
     return x, M, N, K
+
+
+def _bf16_native(weight):
+    """Native tiles of an unquantized bf16 weight (blocked 5-D / 4-D or plain 2-D), made on first use and kept on
+    the tensor (the role of the reference's cached first-token remap)."""
+    key = (weight.data_ptr(), weight._version)
+    have = getattr(weight, "_tppx_native_bf16", None)
+    if have is not None and have[0] == key:
+        return have[1]
+    N, K, bk, bc, v = _blocked_geometry(weight)
+    _lib.require_gpu(weight, "weight")
+    w = weight.detach().contiguous()
+    nat = torch.empty(N * K, dtype=torch.bfloat16, device=w.device)
+    _lib.check(_lib.lib().tppx_prepack_bf16(w.data_ptr(), N, K, bk, bc, v, nat.data_ptr(), _lib.stream_of(w)))
+    weight._tppx_native_bf16 = (key, nat)
+    return nat
+
+
+def _linear_bf16(input, weight, bias, post, post_in, post_in2, post_scale, flags):
+    """TppBlockedLinearW<bf16,bf16> (src/csrc/fused_gemm.h:785-1073): unquantized bf16 weight."""
+    if isinstance(input, QTensor):
+        raise TppxError(_lib.EUNSUPPORTED, "pre-quantized activations are not built; pass bfloat16")
+    _lib.require_gpu(input, "input")
+    if input.dtype != torch.bfloat16:
+        raise TppxError(_lib.EUNSUPPORTED, f"bfloat16 weights take bfloat16 activations (got {input.dtype})")
+    N, K = _blocked_geometry(weight)[:2]
+    if input.shape[-1] != K:
+        raise TppxError(_lib.ESHAPE, f"input has {input.shape[-1]} features, weight expects {K}")
+    x = input.contiguous()
+    M = x.numel() // K
+    y = torch.empty(tuple(input.shape[:-1]) + (N,), dtype=torch.bfloat16, device=x.device)
+    if M == 0:
+        return y
+    bias = _prep_bias(bias, N, x.device)
+    post_in = _prep_post(post_in, M, N, "post-op input", x.device)
+    post_in2 = _prep_post(post_in2, M, N, "second post-op input", x.device)
+    nat = _bf16_native(weight)
+    _lib.check(_lib.lib().tppx_linear_bf16(x.data_ptr(), nat.data_ptr(), _lib.ptr(bias), _lib.ptr(post_in),
+                                           _lib.ptr(post_in2), y.data_ptr(), M, N, K, post, post_scale, flags,
+                                           _lib.stream_of(x)))
+    return y
 
 
 def _prep_bias(bias, N, dev):
@@ -300,6 +344,10 @@ def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None
     row_sumsq: f32 [16][256] table that receives the row sums of squares of the output (see sums_table());
     only honoured where takes_row_sums() says so."""
     L = _lib.lib()
+    if not isinstance(weight, QTensor) and isinstance(weight, torch.Tensor) and weight.dtype == torch.bfloat16:
+        if row_sumsq is not None:
+            raise TppxError(_lib.EUNSUPPORTED, "row sums of squares need an MXFP4 weight and at most 16 rows")
+        return _linear_bf16(input, weight, bias, post, post_in, post_in2, post_scale, flags)
     x, M, N, K = _prep_input(input, weight)
     out_shape = tuple(input.shape[:-1]) + (N,)
     y = torch.empty(out_shape, dtype=torch.bfloat16, device=x.device)

@@ -430,12 +430,14 @@ def LlamaModel_forward(self, input_ids=None, attention_mask=None, position_ids=N
     return BaseModelOutputWithPast(last_hidden_state=hidden_states, past_key_values=past_key_values)
 
 
-def OptimizeModelForLlama(model, dtype=torch.bfloat16, device="cuda", weight_dtype="mxfp4"):
+def OptimizeModelForLlama(model, dtype=torch.bfloat16, device="cuda", weight_dtype="mxfp4", quantize_lm_head=False):
     """fused_llama_infer.py:176-226 for one GPU: the rotary table from the model's own rotary_emb, every
-    LlamaDecoderLayer fused, every remaining nn.Linear (the lm_head) turned into a BlockedLinear, LlamaModel.forward
-    of this instance replaced.  Differences: the linears must be quantized (weight_dtype "mxfp4" or "qint8"; the
-    reference keeps the lm_head in bf16 unless asked to quantize it) and the KV cache is allocated for
-    TPPX_KV_CAPACITY keys per sequence (default: the model's max_position_embeddings)."""
+    LlamaDecoderLayer fused, every remaining nn.Linear (the lm_head) turned into a BlockedLinear with the
+    reference's blocking (100 x 64 where the vocabulary allows, else 64 x 64) and bf16 weights, LlamaModel.forward
+    of this instance replaced.  quantize_lm_head: True / "qint8" / "mxfp4" quantizes the lm_head as well
+    (run_generation.py:277-282 does it with remap_and_quantize_qint8 after the call; that works here too).
+    Differences: the decoder layers' linears must be quantized (weight_dtype "mxfp4" or "qint8") and the KV cache
+    is allocated for TPPX_KV_CAPACITY keys per sequence (default: the model's max_position_embeddings)."""
     import transformers
     from .llm_common import FixLinear
     if weight_dtype not in ("mxfp4", "qint8"):
@@ -459,9 +461,17 @@ def OptimizeModelForLlama(model, dtype=torch.bfloat16, device="cuda", weight_dty
         for m in list(model.modules()):
             if isinstance(m, transformers.models.llama.modeling_llama.LlamaDecoderLayer):
                 FixLlamaDecoderLayer(m, 16, 64, dtype, weight_dtype, embed_positions)
-        for m in list(model.modules()):
-            if isinstance(m, torch.nn.Linear) and m.weight.shape[0] % 32 == 0 and m.weight.shape[1] % 64 == 0:
-                FixLinear(m, 16, 64, dtype, weight_dtype=weight_dtype)  # no-op for the ones fixed above
+        head_dtype = None if not quantize_lm_head else ("qint8" if quantize_lm_head is True else quantize_lm_head)
+        for m in list(model.modules()):  # FixLinear is a no-op for the ones fixed above
+            if not isinstance(m, torch.nn.Linear) or m.weight.shape[1] % 64:
+                continue
+            if head_dtype is not None:  # quantized tiles are 16 output channels high
+                if m.weight.shape[0] % 32 == 0:
+                    FixLinear(m, 16, 64, dtype, weight_dtype=head_dtype)
+            elif m.weight.shape[0] % 100 == 0:
+                FixLinear(m, 100, 64, dtype)
+            elif m.weight.shape[0] % 64 == 0:
+                FixLinear(m, 64, 64, dtype)
     for m in model.modules():
         if isinstance(m, transformers.models.llama.modeling_llama.LlamaModel):
             m._tpp_kv_capacity = int(os.environ.get("TPPX_KV_CAPACITY", embed_positions.shape[1]))
