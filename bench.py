@@ -62,6 +62,9 @@ def main():
                          "7B-shape greedy decode; prompt = a 2048-token prompt through the same 7B-shape decoder")
     ap.add_argument("--prefill-fmt", default="mxfp4", choices=["mxfp4", "qint8"],
                     help="weight format of --workload prefill (BASELINE config 4 is MXFP4; qint8 = the same layer W8A8)")
+    ap.add_argument("--act-fp8", action="store_true",
+                    help="--workload prefill, MXFP4: quantise activations to MXFP8 and use the block-scaled MFMA "
+                         "(opt-in; not the reference's arithmetic, whose activations stay bf16)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pool", type=int, default=2, help="number of distinct weight sets cycled through")
@@ -290,6 +293,9 @@ def run_prefill(torch, _ops, args):
     g = torch.Generator(device=dev).manual_seed(1238)
 
     pfmt = args.prefill_fmt
+    fp8 = bool(args.act_fp8) and pfmt == "mxfp4"
+    _ops.ACT_FP8 = _ops.ACT_FP8 or fp8
+    fp8 = fp8 or (_ops.ACT_FP8 and pfmt == "mxfp4")
     quant = _ops.remap_and_quantize_mxfp4 if pfmt == "mxfp4" else _ops.remap_and_quantize_qint8
 
     def mk(N, K):
@@ -323,7 +329,7 @@ def run_prefill(torch, _ops, args):
 
     # roofline leg: the largest GEMM (down projection) alone, events on the launch stream
     L = _lib.lib()
-    plan = kernel_plan(L, pfmt, M, H, I, 256, 0, 0)
+    plan = kernel_plan(L, pfmt, M, H, I, 256, _lib.FLAG_ACT_FP8 if fp8 else 0, (33 * M * I) // 32 if fp8 else 0)
     inter = torch.randn((M, I), generator=g, device=dev).to(torch.bfloat16)
     for _ in range(2):
         torch.ops.tpp_llm.fc_add(inter, wd, empty, res, 1.0)
@@ -337,8 +343,9 @@ def run_prefill(torch, _ops, args):
     torch.cuda.synchronize()
     us = e0.elapsed_time(e1) * 1e3 / reps
     fl = 2.0 * M * H * I
-    peak = PEAKS_TFLOPS["bf16"] if pfmt == "mxfp4" else PEAKS_TFLOPS["int8"]
-    roof = {"bound": "mfma", "kernel": plan[-1][0] if plan else "?", "call": f"down M={M} N={H} K={I}",
+    peak = PEAKS_TFLOPS["fp8" if fp8 else "bf16"] if pfmt == "mxfp4" else PEAKS_TFLOPS["int8"]
+    roof = {"bound": "mfma", "kernel": plan[-1][0] if plan else "?",
+            "call": f"down M={M} N={H} K={I}" + (" (activation quantiser included)" if fp8 else ""),
             "achieved": round(fl / us / 1e6, 1), "peak": peak, "unit": "TFLOP/s" if pfmt == "mxfp4" else "TOP/s",
             "frac": round(fl / us / 1e6 / peak, 4), "traffic": None,
             "avg_launch_us": round(us, 1), "flops_per_launch": fl, "launches_timed": reps,
@@ -348,8 +355,10 @@ def run_prefill(torch, _ops, args):
         "metric": "quant-GEMM TFLOP/s (prefill)", "value": round(flops / (ms * 1e-3) / 1e12, 2),
         "unit": "TFLOP/s" if pfmt == "mxfp4" else "TOP/s",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if pfmt == "mxfp4" else "int8", "data": "synthetic",
-        "config": {"workload": ("cfg4: MXFP4" if pfmt == "mxfp4" else "cfg4's layer with QINT8 W8A8 (QBS=256)") +
+        "scaling": "weak", "vs_baseline": None, "dtype": ("fp8" if fp8 else "bf16") if pfmt == "mxfp4" else "int8", "data": "synthetic",
+        "config": {"workload": (("cfg4: MXFP4" + (" weights x MXFP8 activations (opt-in, not the reference's "
+                                                  "arithmetic)" if fp8 else ""))
+                                if pfmt == "mxfp4" else "cfg4's layer with QINT8 W8A8 (QBS=256)") +
                                " linears of one decoder layer (hidden 8192, intermediate 28672, kv 1024) at "
                                "M = 2048: qkv_gemm, fc_add(o), swiglu_mlp(gate, up, down)",
                    "launch": "eager op calls", "flops_per_step": flops},

@@ -159,6 +159,18 @@ int tppx_linear_mxfp4(const void* x, const void* qw, const void* sw,
                       int64_t K, int post_op, float post_scale, int flags,
                       void* ws, int64_t ws_bytes, tppx_stream_t stream);
 
+/* Activations for TPPX_FLAG_ACT_FP8 (no counterpart in the reference, whose
+ * activations stay bf16; the closest is its W4A8 USE_MXFP4_INT8 variant,
+ * src/csrc/fused_gemm.h:965-978): x bf16 [M][K] -> MXFP8, OCP E4M3 elements with
+ * one E8M0 scale per 32 input channels (exponent floor(log2 max|x|) - 8, round
+ * to nearest even, saturating at 448), in MFMA operand order:
+ * xq [ceil(M/16)][K/128][2][64][16] bytes, xs [ceil(M/16)][K/128][64] bytes
+ * (lane g*16 + m of a tile holds channels h*64 + g*16 .. +15 of row m in half h
+ * and the scale of channels g*32..g*32+31; rows past M are zeros).  K%128==0.  tppx_linear_mxfp4 and its siblings call
+ * it themselves when the flag is set (workspace: 33/32 * roundup(M,16) * K bytes). */
+int tppx_quant_act_mxfp8(const void* x, int64_t M, int64_t K, void* xq, void* xs,
+                         tppx_stream_t stream);
+
 /* Unquantized bf16 weights: TppBlockedLinearW<bf16,bf16>
  * (src/csrc/fused_gemm.h:785-1073 with the plain BRGEMM of :951-1064), the
  * class the reference's default bf16 lm_head runs through

@@ -467,6 +467,63 @@ def linear_bf16(x_bf16, w_bf16, bias=None, post=POST_NONE, post_in=None, post_in
     return post_op(y, post, post_in, post_in2, post_scale) if post != POST_NONE else y
 
 
+# ----------------------------------------------------------------------------
+# MXFP8 activations of the opt-in FP8-activation GEMM.  No reference code to follow (its activations stay bf16):
+# the OCP Microscaling v1.0 recipe -- E4M3 elements (bias 7, subnormals, maximum 448, no infinities), one E8M0
+# scale per 32 values with exponent floor(log2 max|x|) - 8, round to nearest even, saturation.
+# Pinned by known codes, the decode/encode round trip over all 254 finite codes and tie cases (tests/test_oracle.py).
+# ----------------------------------------------------------------------------
+def e4m3_decode(c):
+    c = np.asarray(c, np.uint8).astype(np.int32)
+    e, m = (c >> 3) & 15, c & 7
+    mag = np.where(e == 0, m * 2.0 ** -9, (1.0 + m / 8.0) * 2.0 ** (e - 7.0))
+    return np.where(c & 0x80, -mag, mag).astype(np.float32)
+
+
+def e4m3_encode(v):
+    v = np.asarray(v, np.float64)
+    a = np.minimum(np.abs(v), 448.0)
+    _, ex = np.frexp(a)                      # a = f * 2^ex, f in [0.5, 1)
+    e = np.maximum(ex - 1, -6)               # exponent of the value's binade, subnormals share 2^-6's
+    step = 2.0 ** (e - 3.0)
+    r = np.rint(a / step) * step             # RNE at 3 mantissa bits
+    _, ex2 = np.frexp(r)
+    e2 = ex2 - 1
+    normal = r >= 2.0 ** -6
+    code = np.where(normal, ((e2 + 7) << 3) | np.rint((r / 2.0 ** e2.astype(np.float64) - 1.0) * 8).astype(np.int64),
+                    np.rint(r * 512.0).astype(np.int64))
+    return (code | np.where(np.signbit(v), 0x80, 0)).astype(np.uint8)
+
+
+def quant_act_mxfp8(x_bf16):
+    """bf16 bits [M][K] -> (codes u8 [M][K], scale bytes u8 [M][K/32])."""
+    x = bf16_to_f32(_c(x_bf16, np.uint16))
+    M, K = x.shape
+    xb = x.reshape(M, K // 32, 32)
+    amax = np.abs(xb).max(-1)
+    E = (amax.view(np.uint32) >> 23) & 0xff
+    X = np.clip(E.astype(np.int64) - 8, 0, 254)
+    codes = e4m3_encode(xb.astype(np.float64) * 2.0 ** (127.0 - X)[..., None])
+    return codes.reshape(M, K), X.astype(np.uint8)
+
+
+def dequant_act_mxfp8(codes, scales):
+    M, K = codes.shape
+    v = e4m3_decode(codes).reshape(M, K // 32, 32).astype(np.float64) * 2.0 ** (scales.astype(np.float64) - 127.0)[..., None]
+    return v.reshape(M, K)
+
+
+def linear_mxfp4_fp8act(x_bf16, q, sc, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0):
+    """The MXFP4 linear on MXFP8-quantised activations: exact products, one rounding of bias + sum to bf16, post-op."""
+    xd = dequant_act_mxfp8(*quant_act_mxfp8(x_bf16))
+    w = dequantize_mxfp4_plain(q, sc).astype(np.float64)
+    acc = xd @ w.T
+    if bias is not None:
+        acc = acc + bf16_to_f32(_c(bias, np.uint16)).astype(np.float64)[None, :]
+    y = f32_to_bf16(acc.astype(np.float32))
+    return post_op(y, post, post_in, post_in2, post_scale) if post != POST_NONE else y
+
+
 def num_threads():
     return lib().orc_num_threads()
 

@@ -503,3 +503,77 @@ def test_bf16_weight_module_and_errors():
     assert_close_bf16(t2bits(y).reshape(6, 1600), ref, what="bf16 BlockedLinear")
     with pytest.raises(TppxError):
         _ops().linear(x.cuda()[..., :128].contiguous(), lin.weight, None)
+
+
+def _mxfp8_from_operand_order(xq, xs, M, K):
+    """GPU layout [M/16][K/128][2][64][16] / [M/16][K/128][64] -> codes [M][K], scale bytes [M][K/32]."""
+    Mt, Kt = (M + 15) // 16, K // 128
+    q = xq.view(Mt, Kt, 2, 4, 16, 16).permute(0, 4, 1, 2, 3, 5).reshape(Mt * 16, K)  # [mt][m][kt][h][g][16]
+    s = xs.view(Mt, Kt, 4, 16).permute(0, 3, 1, 2).reshape(Mt * 16, K // 32)
+    return q.cpu().numpy(), s.cpu().numpy()
+
+
+@pytest.mark.parametrize("M,K", [(1, 128), (37, 384), (128, 4096)])
+def test_mxfp8_activation_quantizer_bit_exact(M, K):
+    from tpp_pytorch_extension import _lib
+    _ops()
+    x = randn_bf16((M, K), 1.0, 91)
+    x[0, :32] = 0.0                      # an all-zero block
+    x.view(-1)[5::97] *= 37.0            # outliers that set block maxima
+    Mp = (M + 15) // 16 * 16
+    xq = torch.empty(Mp * K, dtype=torch.uint8, device="cuda")
+    xs = torch.empty(Mp * K // 32, dtype=torch.uint8, device="cuda")
+    xg = x.cuda()
+    _lib.check(_lib.lib().tppx_quant_act_mxfp8(xg.data_ptr(), M, K, xq.data_ptr(), xs.data_ptr(), _lib.stream_of(xg)))
+    q, s = _mxfp8_from_operand_order(xq, xs, M, K)
+    q_or, s_or = O.quant_act_mxfp8(t2bits(x))
+    assert np.array_equal(q[:M], q_or) and np.array_equal(s[:M], s_or)
+    assert not q[M:].any()               # padded rows are zeros
+
+
+@pytest.mark.parametrize("M,N,K,post", [(128, 256, 256, "none"), (1, 32, 128, "none"), (200, 544, 384, "add"),
+                                         (333, 4096, 1024, "silu"), (2048, 512, 4096, "none")])
+def test_mxfp4_linear_on_fp8_activations(M, N, K, post):
+    """TPPX_FLAG_ACT_FP8: MXFP4 weights on the block-scaled MFMA with MXFP8 activations.  Against the oracle of the
+    same arithmetic (exact products, fp32 sums: 1 ulp, 2 through SiLU as for the other kernels), and against the reference-arithmetic oracle (bf16
+    activations) within the rounding of E4M3: rel-L2 <= 5e-2."""
+    from tpp_pytorch_extension import _lib
+    ops = _ops()
+    qw, q_or, s_or = _make("mxfp4", N, K, 95)
+    x = randn_bf16((M, K), 1.0, 96)
+    bias = randn_bf16((N,), 0.01, 97)
+    in1 = randn_bf16((M, N), 1.0, 98)
+    scale = 0.5 if post == "add" else 1.0
+    y = ops.linear(x.cuda(), qw, bias.cuda(), POSTS[post], in1.cuda(), None, scale, flags=_lib.FLAG_ACT_FP8)
+    ref = O.linear_mxfp4_fp8act(t2bits(x), q_or, s_or, t2bits(bias), POSTS[post], t2bits(in1), None, scale)
+    pre = O.linear_mxfp4_fp8act(t2bits(x), q_or, s_or, t2bits(bias)) if post == "add" else None
+    assert_close_bf16(t2bits(y), ref, ulps=2 if post == "silu" else 1, what=f"fp8-act M={M} N={N} K={K} {post}",
+                      pre_bits=pre)
+    exact = O.linear_mxfp4(t2bits(x), q_or, s_or, t2bits(bias), POSTS[post], t2bits(in1), None, scale, O.MODE_IDEAL)
+    assert err_stats(t2bits(y), exact)["rel_l2"] <= 5e-2
+
+
+def test_fp8_activation_qkv_and_swiglu_equal_separate_calls():
+    from tpp_pytorch_extension import _lib, _ops as ops
+    _ops()
+    M, K = 160, 512
+    x = randn_bf16((M, K), 1.0, 99).cuda()
+    ws = [_make("mxfp4", n, K, 100 + i)[0] for i, n in enumerate((512, 256, 256))]
+    old = ops.ACT_FP8
+    ops.ACT_FP8 = True
+    try:
+        q, k, v = ops.qkv_gemm(x, ws, [None, None, None])
+        sw = ops.swiglu_gate_up(x, ws[1], ws[2])
+    finally:
+        ops.ACT_FP8 = old
+    for got, w in zip((q, k, v), ws):
+        assert torch.equal(got, ops.linear(x, w, None, flags=_lib.FLAG_ACT_FP8))
+    g = ops.linear(x, ws[1], None, POSTS["silu"], flags=_lib.FLAG_ACT_FP8)
+    assert torch.equal(sw, ops.linear(x, ws[2], None, POSTS["mul"], g, flags=_lib.FLAG_ACT_FP8))
+    from tpp_pytorch_extension._lib import TppxError
+    Lb = _lib.lib()
+    y = torch.empty(M, 512, dtype=torch.bfloat16, device="cuda")
+    qn, sn = ws[0].native()
+    with pytest.raises(TppxError):  # no workspace for the quantised activations
+        _lib.check(Lb.tppx_linear_mxfp4(x.data_ptr(), qn.data_ptr(), sn.data_ptr(), None, None, None, y.data_ptr(),
+                                        M, 512, K, 0, 1.0, _lib.FLAG_ACT_FP8, None, 0, _lib.stream_of(x)))

@@ -394,3 +394,26 @@ def test_oracle_linear_bf16_against_mxfp4_restatement_and_closed_forms():
     want = (xi.double() @ wi.double().T)  # |sum| <= 256 * 12: exact in fp32, not always in bf16
     got = bits2f(O.linear_bf16(t2bits(xi), t2bits(wi)))
     assert np.array_equal(got, want.float().to(torch.bfloat16).float().numpy())
+
+
+def test_oracle_mxfp8_activation_quantizer_known_answers():
+    """OCP E4M3 / MX block scale: known codes (1.0 = 0x38, 448 = 0x7E = the largest finite, saturation above it,
+    2^-9 = the smallest subnormal, ties to even on both sides of the normal boundary), decode(encode) over all 254
+    finite codes, and the block rule on hand-made blocks (max 1.0 -> scale 2^-8, so 1.0 is stored as 256 = 0x78)."""
+    c = np.arange(256, dtype=np.uint8)
+    fin = c[(c & 0x7F) != 0x7F]
+    assert np.array_equal(O.e4m3_encode(O.e4m3_decode(fin)), fin)
+    assert O.e4m3_decode([0x7E])[0] == 448.0 and O.e4m3_decode([0x01])[0] == 2.0 ** -9 and O.e4m3_decode([0x08])[0] == 2.0 ** -6
+    vals = [1.0, 448, 500, 2 ** -9, 2 ** -10, 3 * 2 ** -10, 1.0625, 1.1875, -1.0, 0.9 * 2 ** -6, 17.0, 19.0]
+    want = [0x38, 0x7E, 0x7E, 0x01, 0x00, 0x02, 0x38, 0x3A, 0xB8, 0x07, 0x58, 0x5A]  # 17 -> 16 (tie, even), 19 -> 20
+    assert O.e4m3_encode(vals).tolist() == want
+    x = np.zeros((1, 64), np.float32)
+    x[0, :4] = [1.0, -0.5, 0.75, 2.0 ** -12]          # block 0: max 1.0
+    x[0, 32:36] = [1.9, 0.001, -1.9, 100.0 * 2 ** -8]  # block 1: max 1.9 (bf16 1.8984375): 1.898 * 256 = 486 saturates
+    xb = t2bits(torch.from_numpy(x).to(torch.bfloat16))
+    codes, sc = O.quant_act_mxfp8(xb)
+    assert sc.tolist() == [[119, 119]]
+    assert codes[0, :4].tolist() == [0x78, 0xF0, 0x74, 0x18]  # 256, -128, 192, 2^-12 * 256 = 2^-4
+    assert codes[0, 32] == 0x7E and codes[0, 34] == 0xFE and codes[0, 35] == O.e4m3_encode([100.0])[0]
+    d = O.dequant_act_mxfp8(codes, sc)
+    assert d[0, 0] == 1.0 and d[0, 1] == -0.5 and d[0, 32] == 448.0 / 256

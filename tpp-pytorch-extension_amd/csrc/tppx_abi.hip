@@ -218,7 +218,6 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
   TPPX_REQUIRE(segs, TPPX_EINVAL, "%s: null segment table", who);
   TPPX_REQUIRE(K > 0 && K % 64 == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of 64", who, (long)K);
   TPPX_REQUIRE(K % 128 == 0, TPPX_EUNSUPPORTED, "%s: K=%ld is not a multiple of 128 (native MXFP4 tiles span 128 input channels)", who, (long)K);
-  TPPX_REQUIRE(!(flags & TPPX_FLAG_ACT_FP8), TPPX_EUNSUPPORTED, "%s: the FP8-activation path is not available", who);
   DecodeParams p;
   memset(&p, 0, sizeof(p));
   rc = fill_all(who, segs, n_segs, 32, dual, p);
@@ -231,6 +230,33 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
   p.tpb = 1;
   p.S = 1;
   p.sumsq_out = row_sumsq;
+  if (flags & TPPX_FLAG_ACT_FP8) {
+    // opt-in, not the reference's arithmetic: activations quantised to MXFP8 (into the workspace), then the
+    // block-scaled MFMA kernel on the weights' own codes and scales; any M, but built for prefill shapes
+    TPPX_REQUIRE(!row_sumsq, TPPX_EUNSUPPORTED, "%s: row sums of squares are not produced by the FP8-activation kernel", who);
+    const int64_t Mp = (M + 15) / 16 * 16, need = Mp * K + Mp * (K / 32);
+    TPPX_REQUIRE(ws && ws_bytes >= need, TPPX_EINVAL, "%s: the FP8-activation path needs %ld bytes of workspace for the quantised activations (got %ld)", who, (long)need, (long)ws_bytes);
+    uint8_t* xq = (uint8_t*)ws;
+    uint8_t* xs = xq + Mp * K;
+    rc = check_hip(launch_quant_act_mxfp8(x, M, K, xq, xs, stream), who);
+    if (rc)
+      return rc;
+    TiledParams t[TPPX_MAX_SEGS];
+    for (int i = 0; i < n_segs; i++) {
+      t[i] = tiled_from_seg(p, i);
+      t[i].xq = xq;
+      t[i].sa = (const float*)xs;
+    }
+    if (!dual)
+      return check_hip(launch_tiled_mxfp4_fp8_group(t, n_segs, stream), who);
+    t[0].post_op = TPPX_POST_SILU; // silu(gate), then up * that: the rounding points of the two-GEMM form
+    t[1].post_op = TPPX_POST_MUL;
+    t[1].post_in = (const uint16_t*)segs[0].y;
+    rc = check_hip(launch_tiled_mxfp4_fp8_group(&t[0], 1, stream), who);
+    if (rc)
+      return rc;
+    return check_hip(launch_tiled_mxfp4_fp8_group(&t[1], 1, stream), who);
+  }
   if (want_tiled(M, flags)) {
     TPPX_REQUIRE(!row_sumsq, TPPX_EUNSUPPORTED, "%s: row sums of squares are not produced by the large-M kernels", who);
     // prefill shapes: one LDS-tiled launch per GEMM of the group; the fused

@@ -81,6 +81,7 @@ hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream);
 bool tiled_mxfp4_takes_groups(const TiledParams& p);
 hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream);
 hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream);
+hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t stream);
 bool tiled_qint8_takes_groups(const TiledParams& p);
 hipError_t launch_tiled_qint8_group(const TiledParams* t, int n, hipStream_t stream);
 // y[i] = bf16( silu(gate[i]) * y[i] ) with the rounding points of SiluPostOp followed by MulPostOp; n % 8 == 0
@@ -91,6 +92,9 @@ int env_int(const char* name, int dflt);
 // dynamic activation quantisation; mt > 0 writes xq in MFMA operand order (see DecodeParams::mt)
 hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs, void* xq, void* sa, int mt,
                                  hipStream_t stream);
+
+// MXFP8 activations in MFMA operand order for the block-scaled prefill kernel: xq (M16*16*K bytes), xs (M16*16*K/32)
+hipError_t launch_quant_act_mxfp8(const void* x, int64_t M, int64_t K, void* xq, void* xs, hipStream_t stream);
 
 // can_fuse_quant: bf16 activations at hand and 256-wide blocks (the in-kernel quantisation's case)
 SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, bool can_fuse_quant);

@@ -252,6 +252,74 @@ prepack_bf16_kernel(const uint16_t* __restrict__ wref, int64_t N, int64_t K, int
                                                  e[4] | ((uint32_t)e[5] << 16), e[6] | ((uint32_t)e[7] << 16));
 }
 
+// Activations for the block-scaled MFMA path: bf16 [M][K] -> MXFP8 (OCP E4M3 elements, one E8M0 scale per 32
+// input channels, scale exponent = floor(log2 max|x|) - 8 as the OCP MX recipe has it), written in MFMA operand
+// order: values [M/16][K/128][2 halves][64 lanes][16 B] -- an 8-bit operand of the 16x16x128 instruction is two
+// 64-channel halves, so lane (g, m) of a 16-row x 128-channel tile holds channels g*16 .. g*16+15 of row m in half
+// 0 and 64 + g*16 .. 64 + g*16+15 in half 1 -- and scale bytes [M/16][K/128][64 lanes]: lane (b, m) holds the scale
+// of channels b*32 .. b*32+31 (the instruction scales by 32-channel block, whichever lanes hold the elements).
+// Rows past M in the last tile are zeros.  One thread per (row, 32-channel block).
+__device__ __forceinline__ uint32_t e4m3_encode_rne(float v) {
+  const uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
+  const float a = fminf(fabsf(v), 448.0f);
+  if (a < 0.015625f) // below the smallest normal 2^-6: multiples of 2^-9 (8 is the code of 2^-6 itself)
+    return sign | (uint32_t)__float2int_rn(a * 512.0f);
+  uint32_t u = __float_as_uint(a);
+  u += 0x7ffffu + ((u >> 20) & 1u); // round to nearest even at 3 mantissa bits
+  return sign | ((((u >> 23) - 120u) << 3) | ((u >> 20) & 7u));
+}
+
+__global__ void __launch_bounds__(256)
+quant_act_mxfp8_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K, uint8_t* __restrict__ xq,
+                       uint8_t* __restrict__ xs) {
+  const int64_t KB = K / 32, KT = K / 128;
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t Mp = (M + 15) / 16 * 16;
+  if (t >= Mp * KB)
+    return;
+  const int64_t m = t / KB, kb = t % KB;
+  uint32_t w[16];
+  if (m < M) {
+    const uint4* src = reinterpret_cast<const uint4*>(x + m * K + kb * 32);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint4 v = src[i];
+      w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      w[i] = 0u;
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 16; i++)
+    amax = fmaxf(amax, fmaxf(fabsf(bf16_bits_to_f32(w[i] & 0xffffu)), fabsf(bf16_bits_to_f32(w[i] >> 16))));
+  const int E = (int)((__float_as_uint(amax) >> 23) & 0xffu);
+  const int X = min(max(E - 8, 0), 254);
+  const float inv = __uint_as_float((uint32_t)(254 - X) << 23); // 2^(127 - X), X <= 246
+  uint32_t out[8];
+#pragma unroll
+  for (int d = 0; d < 8; d++) {
+    uint32_t v = 0;
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+      const uint32_t pr = w[2 * d + e];
+      v |= e4m3_encode_rne(bf16_bits_to_f32(pr & 0xffffu) * inv) << (16 * e);
+      v |= e4m3_encode_rne(bf16_bits_to_f32(pr >> 16) * inv) << (16 * e + 8);
+    }
+    out[d] = v;
+  }
+  const int64_t mt = m >> 4, kt = kb >> 2;
+  const int lane = (int)((kb & 3) * 16 + (m & 15));
+  // 16-channel chunk c = 2 * (kb & 3) + e of the tile lies in lane group c & 3 of half c >> 2
+  uint4* dst = reinterpret_cast<uint4*>(xq) + ((mt * KT + kt) * 2) * 64 + (m & 15);
+  const int c0 = (int)(kb & 3) * 2;
+  dst[(c0 >> 2) * 64 + (c0 & 3) * 16] = make_uint4(out[0], out[1], out[2], out[3]);
+  dst[((c0 + 1) >> 2) * 64 + ((c0 + 1) & 3) * 16] = make_uint4(out[4], out[5], out[6], out[7]);
+  xs[(mt * KT + kt) * 64 + lane] = (uint8_t)X;
+}
+
 // Activation quantizer: one wave per (row, K block).  Each lane owns
 // consecutive pairs so loads and stores stay contiguous.
 __global__ void __launch_bounds__(256)
@@ -320,6 +388,13 @@ hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qb
   TPPX_PLAN_ONLY(quant_act_int8_kernel, dim3(grid_for(nthreads, 256)), dim3(256), 0);
   quant_act_int8_kernel<<<grid_for(nthreads, 256), 256, 0, stream>>>((const uint16_t*)x, M, K, qbs, (int8_t*)xq,
                                                                     (float*)sa, mt);
+  return hipGetLastError();
+}
+
+hipError_t launch_quant_act_mxfp8(const void* x, int64_t M, int64_t K, void* xq, void* xs, hipStream_t stream) {
+  const int64_t nthreads = (M + 15) / 16 * 16 * (K / 32);
+  TPPX_PLAN_ONLY(quant_act_mxfp8_kernel, dim3(grid_for(nthreads, 256)), dim3(256), 0);
+  quant_act_mxfp8_kernel<<<grid_for(nthreads, 256), 256, 0, stream>>>((const uint16_t*)x, M, K, (uint8_t*)xq, (uint8_t*)xs);
   return hipGetLastError();
 }
 
@@ -441,6 +516,13 @@ extern "C" int tppx_prepack_bf16(const void* w_ref, int64_t N, int64_t K, int64_
   prepack_bf16_kernel<<<grid_for(nchunks, 256), 256, 0, (hipStream_t)stream>>>((const uint16_t*)w_ref, N, K, bk, bc, vnni,
                                                                                 (uint16_t*)w_nat);
   return check_hip(hipGetLastError(), "tppx_prepack_bf16");
+}
+
+extern "C" int tppx_quant_act_mxfp8(const void* x, int64_t M, int64_t K, void* xq, void* xs, tppx_stream_t stream) {
+  TPPX_REQUIRE(x && xq && xs, TPPX_EINVAL, "tppx_quant_act_mxfp8: null pointer");
+  TPPX_REQUIRE(aligned16(x) && aligned16(xq), TPPX_EINVAL, "tppx_quant_act_mxfp8: pointer not 16-byte aligned");
+  TPPX_REQUIRE(M > 0 && K > 0 && K % 128 == 0, TPPX_ESHAPE, "tppx_quant_act_mxfp8: bad shape M=%ld K=%ld (K in multiples of 128)", (long)M, (long)K);
+  return check_hip(launch_quant_act_mxfp8(x, M, K, xq, xs, (hipStream_t)stream), "tppx_quant_act_mxfp8");
 }
 
 extern "C" int tppx_quant_act_int8(const void* x, int64_t M, int64_t K,

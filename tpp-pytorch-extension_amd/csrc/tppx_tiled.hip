@@ -769,6 +769,128 @@ big_qint8_kernel(const BigParams P) {
 }
 
 // the large-M kernel addresses its operands with 32-bit byte offsets
+// ---------------------------------------------------------------------------
+// Large-M MXFP4 weights x MXFP8 activations on the block-scaled MFMA
+// (v_mfma_scale_f32_16x16x128_f8f6f4): the weights' E2M1 codes and E8M0 scales
+// are the instruction's operands as they lie in the native tiles -- nothing is
+// expanded -- and the activations arrive quantised in operand order
+// (quant_act_mxfp8_kernel).  Not the reference's arithmetic (its activations
+// stay bf16): an opt-in (TPPX_FLAG_ACT_FP8).
+// Workgroup tile 128 (M) x 256 (N), 8 waves (2 x 4), wave tile 64 x 64 = 16
+// MFMAs of K = 128 per step.  Both operands go from global memory straight
+// into LDS, 1 KiB per wave instruction (a native weight tile, half an
+// activation tile: lane-linear on both sides, so operand reads are
+// conflict-free 16-byte reads), a step ahead, two buffers of 32 KiB; one
+// barrier per step.  Scale bytes come from global/L2, a step ahead.
+// ---------------------------------------------------------------------------
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+__global__ void __launch_bounds__(512)
+big_fp8_kernel(const BigParams P) {
+  extern __shared__ __align__(16) uint8_t tl_lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+  const int MB = (P.seg[0].M + 127) / 128;
+  int bm, bn;
+  tile_of_block(MB, P.nb0[P.n_seg], bm, bn);
+  TiledParams p = P.seg[0];
+  int nb_first = 0;
+#pragma unroll
+  for (int i = 1; i < TPPX_MAX_SEGS; i++)
+    if (i < P.n_seg && bn >= P.nb0[i]) {
+      p = P.seg[i];
+      nb_first = P.nb0[i];
+    }
+  bn -= nb_first;
+  const int KT = p.K >> 7;
+  const int m_wg = bm * 128;
+  const int tile_base = bn * 16 + wn * 4;
+  const int MT16 = (p.M + 15) >> 4;
+
+  // this wave's share of a step's traffic: activation tile `wave` of the 8 (two halves), weight tiles 2*wave, 2*wave+1
+  const char* xqb = reinterpret_cast<const char*>(p.xq);
+  const char* qwb = reinterpret_cast<const char*>(p.qw);
+  const size_t a_src = ((size_t)min(bm * 8 + wave, MT16 - 1) * KT * 2) * 1024 + (size_t)lane * 16;
+  size_t b_src[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+    b_src[i] = ((size_t)min(bn * 16 + wave * 2 + i, p.tiles - 1) * KT) * 1024 + (size_t)lane * 16;
+  auto dma = [&](int ks, int buf) {
+    uint8_t* base = tl_lds + buf * 32768;
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xqb + a_src + ((size_t)ks * 2 + h) * 1024),
+                                       (__attribute__((address_space(3))) void*)(base + (wave * 2 + h) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(qwb + b_src[i] + (size_t)ks * 1024),
+                                       (__attribute__((address_space(3))) void*)(base + 16384 + (wave * 2 + i) * 1024), 16, 0, 0);
+  };
+  // scale bytes of this wave's 4 row tiles and 4 channel tiles
+  const uint8_t* xsb = reinterpret_cast<const uint8_t*>(p.sa);
+  const uint8_t* swb = reinterpret_cast<const uint8_t*>(p.sw);
+  size_t sa_off[4], sb_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    sa_off[i] = (size_t)min(bm * 8 + wm * 4 + i, MT16 - 1) * KT * 64 + lane;
+    sb_off[i] = (size_t)min(tile_base + i, p.tiles - 1) * KT * 64 + lane;
+  }
+  int sa_n[4], sb_n[4], sa_c[4], sb_c[4];
+  auto load_scales = [&](int ks) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      sa_n[i] = xsb[sa_off[i] + (size_t)ks * 64];
+      sb_n[i] = swb[sb_off[i] + (size_t)ks * 64];
+    }
+  };
+
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++)
+      acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  dma(0, 0);
+  load_scales(0);
+  for (int ks = 0; ks < KT; ks++) {
+    const int buf = ks & 1;
+    __syncthreads(); // step ks has landed for every wave (the barrier waits for this wave's loads first) and
+                     // nobody still reads the other buffer
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      sa_c[i] = sa_n[i];
+      sb_c[i] = sb_n[i];
+    }
+    if (ks + 1 < KT) {
+      dma(ks + 1, buf ^ 1);
+      load_scales(ks + 1);
+    }
+    const uint8_t* base = tl_lds + buf * 32768;
+    i32x8 a[4], b[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++) {
+      const i32x4 lo = *reinterpret_cast<const i32x4*>(base + ((wm * 4 + mt) * 2) * 1024 + lane * 16);
+      const i32x4 hi = *reinterpret_cast<const i32x4*>(base + ((wm * 4 + mt) * 2 + 1) * 1024 + lane * 16);
+      a[mt] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+      const i32x4 w = *reinterpret_cast<const i32x4*>(base + 16384 + (wn * 4 + nt) * 1024 + lane * 16);
+      b[nt] = i32x8{w[0], w[1], w[2], w[3], 0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+        acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[mt], b[nt], acc[mt][nt], 0 /* A: E4M3 */,
+                                                                       4 /* B: E2M1 */, 0, sa_c[mt], 0, sb_c[nt]);
+  }
+  __syncthreads(); // every wave has left the main loop: LDS is free for the epilogue staging
+  big_epilogue<4>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * 64, tile_base);
+}
+
 static bool big_fits(const TiledParams& p) {
   return (int64_t)p.M * p.K * 2 < ((int64_t)1 << 32) && (int64_t)p.tiles * 8 * p.K < ((int64_t)1 << 32);
 }
@@ -818,6 +940,34 @@ hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t str
     TPPX_PLAN_ONLY(big_mxfp4_kernel<8>, dim3(MB8 * nb), dim3(512), lds);
     big_mxfp4_kernel<8><<<dim3(MB8 * nb), dim3(512), lds, stream>>>(P);
   }
+  return hipGetLastError();
+}
+
+// MXFP4 weights x MXFP8 activations (t[i].xq = quantised activations in operand order, t[i].sa = their scale bytes)
+hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t stream) {
+  BigParams P;
+  memset(&P, 0, sizeof(P));
+  int nb = 0;
+  for (int i = 0; i < n; i++) {
+    P.seg[i] = t[i];
+    P.nb0[i] = nb;
+    nb += (t[i].tiles + 15) / 16;
+  }
+  for (int i = n; i <= TPPX_MAX_SEGS; i++)
+    P.nb0[i] = nb;
+  P.n_seg = n;
+  const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the two operand buffers
+  const int MB = (t[0].M + 127) / 128;
+  TPPX_PLAN_ONLY(big_fp8_kernel, dim3(MB * nb), dim3(512), lds);
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_fp8_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess)
+      return e;
+    attr_done = true;
+  }
+  big_fp8_kernel<<<dim3(MB * nb), dim3(512), lds, stream>>>(P);
   return hipGetLastError();
 }
 

@@ -52,6 +52,7 @@ SIGNATURES = {
     "tppx_prepack_mxfp4": [_vp, _vp, _i64, _i64, _vp, _vp, _vp],
     "tppx_prepack_qint8": [_vp, _i64, _i64, _i64, _vp, _vp],
     "tppx_quant_act_int8": [_vp, _i64, _i64, _i64, _vp, _vp, _vp],
+    "tppx_quant_act_mxfp8": [_vp, _i64, _i64, _vp, _vp, _vp],
     "tppx_prepack_bf16": [_vp, _i64, _i64, _i64, _i64, _i32, _vp, _vp],
     "tppx_linear_bf16": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _f32, _i32, _vp],
     "tppx_linear_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _f32, _i32, _vp, _i64, _vp],

@@ -337,6 +337,24 @@ def _qint8_scratch(x, M, K, qbs):
     return xq, sa
 
 
+# Opt-in (TPPX_ACT_FP8=1, or flags=FLAG_ACT_FP8 on linear()): MXFP4 GEMMs with more than 64 rows quantize their
+# activations to MXFP8 and run on the block-scaled MFMA.  Not the reference's arithmetic (its activations stay bf16).
+ACT_FP8 = os.environ.get("TPPX_ACT_FP8", "0") == "1"
+
+
+def _mxfp4_flags_ws(x, M, K, flags=0):
+    """(flags, workspace) of an MXFP4 call: the FP8-activation path keeps the quantised activations in the workspace."""
+    if ACT_FP8 and M > 64:
+        flags |= _lib.FLAG_ACT_FP8
+    ws = _lib.workspace(x)
+    if flags & _lib.FLAG_ACT_FP8:
+        Mp = (M + 15) // 16 * 16
+        need = Mp * K + Mp * (K // 32)
+        if need > ws.numel():
+            ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+    return flags, ws
+
+
 def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0, flags=0,
            row_sumsq=None):
     """One quantized GEMM with a fused post-op
@@ -367,6 +385,7 @@ def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None
                                              post, post_scale, flags, ws.data_ptr(), ws.numel(),
                                              row_sumsq.data_ptr(), st))
     elif weight._qscheme == QSCHEME_MXFP:
+        flags, ws = _mxfp4_flags_ws(x, M, K, flags)
         _lib.check(L.tppx_linear_mxfp4(x.data_ptr(), qn.data_ptr(), sn.data_ptr(), _lib.ptr(bias),
                                        _lib.ptr(post_in), _lib.ptr(post_in2), y.data_ptr(), M, N, K,
                                        post, post_scale, flags, ws.data_ptr(), ws.numel(), st))
@@ -527,7 +546,8 @@ def qkv_gemm(input, weights, biases, norm=None):
     elif scheme == QSCHEME_MXFP and norm is not None:
         _lib.check(L.tppx_norm_multi_linear_mxfp4(x.data_ptr(), norm[0].data_ptr(), float(norm[1]), segs, n, M, K, 0, st))
     elif scheme == QSCHEME_MXFP:
-        _lib.check(L.tppx_multi_linear_mxfp4(x.data_ptr(), segs, n, M, K, 0, ws.data_ptr(), ws.numel(), st))
+        fl, ws = _mxfp4_flags_ws(x, M, K)
+        _lib.check(L.tppx_multi_linear_mxfp4(x.data_ptr(), segs, n, M, K, fl, ws.data_ptr(), ws.numel(), st))
     else:
         qbs = weights[0].block_size
         xq, sa = _qint8_scratch(x, M, K, qbs)
@@ -570,12 +590,12 @@ def swiglu_gate_up(input, w_gate, w_up, b_gate=None, b_up=None, norm=None):
                                             _lib.ptr(bg), qu.data_ptr(), su.data_ptr(), _lib.ptr(bu), y.data_ptr(),
                                             M, N, K, 0, _lib.stream_of(x)))
         return y
-    ws = _lib.workspace(x)
-    if M > 64 and M * N * 2 > ws.numel():
+    fl, ws = _mxfp4_flags_ws(x, M, K)
+    if not fl and M > 64 and M * N * 2 > ws.numel():
         # prefill: room for the gate tile lets the library run gate and up as one grid (fuller last round)
         ws = torch.empty(M * N * 2, dtype=torch.uint8, device=x.device)
     _lib.check(L.tppx_swiglu_mxfp4(x.data_ptr(), qg.data_ptr(), sg.data_ptr(), _lib.ptr(bg), qu.data_ptr(),
-                                   su.data_ptr(), _lib.ptr(bu), y.data_ptr(), M, N, K, 0, ws.data_ptr(),
+                                   su.data_ptr(), _lib.ptr(bu), y.data_ptr(), M, N, K, fl, ws.data_ptr(),
                                    ws.numel(), _lib.stream_of(x)))
     return y
 
