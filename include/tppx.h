@@ -164,10 +164,12 @@ int tppx_linear_mxfp4(const void* x, const void* qw, const void* sw,
  * src/csrc/fused_gemm.h:965-978): x bf16 [M][K] -> MXFP8, OCP E4M3 elements with
  * one E8M0 scale per 32 input channels (exponent floor(log2 max|x|) - 8, round
  * to nearest even, saturating at 448), in MFMA operand order:
- * xq [ceil(M/16)][K/128][2][64][16] bytes, xs [ceil(M/16)][K/128][64] bytes
- * (lane g*16 + m of a tile holds channels h*64 + g*16 .. +15 of row m in half h
- * and the scale of channels g*32..g*32+31; rows past M are zeros).  K%128==0.  tppx_linear_mxfp4 and its siblings call
- * it themselves when the flag is set (workspace: 33/32 * roundup(M,16) * K bytes). */
+ * with Mp = roundup(M, 64): xq [Mp/16][K/128][2][64][16] bytes (lane g*16 + m
+ * of a 16-row tile holds channels h*64 + g*16 .. +15 of row m in half h) and
+ * xs [Mp/64][K/128][64][4] bytes (byte t of lane g*16 + m: the scale of
+ * channels g*32..g*32+31 of row m of the group's row tile t); rows past M are
+ * zeros.  K%128==0.  tppx_linear_mxfp4 and its siblings call it themselves
+ * when the flag is set (workspace: 33/32 * Mp * K bytes). */
 int tppx_quant_act_mxfp8(const void* x, int64_t M, int64_t K, void* xq, void* xs,
                          tppx_stream_t stream);
 

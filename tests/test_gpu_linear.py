@@ -506,10 +506,11 @@ def test_bf16_weight_module_and_errors():
 
 
 def _mxfp8_from_operand_order(xq, xs, M, K):
-    """GPU layout [M/16][K/128][2][64][16] / [M/16][K/128][64] -> codes [M][K], scale bytes [M][K/32]."""
-    Mt, Kt = (M + 15) // 16, K // 128
+    """GPU layout [Mp/16][K/128][2][64][16] / [Mp/64][K/128][64][4] (Mp = M rounded up to 64) -> codes [Mp][K],
+    scale bytes [Mp][K/32]."""
+    Mt, Kt = (M + 63) // 64 * 4, K // 128
     q = xq.view(Mt, Kt, 2, 4, 16, 16).permute(0, 4, 1, 2, 3, 5).reshape(Mt * 16, K)  # [mt][m][kt][h][g][16]
-    s = xs.view(Mt, Kt, 4, 16).permute(0, 3, 1, 2).reshape(Mt * 16, K // 32)
+    s = xs.view(Mt // 4, Kt, 4, 16, 4).permute(0, 4, 3, 1, 2).reshape(Mt * 16, K // 32)  # [q][t][m][kt][b]
     return q.cpu().numpy(), s.cpu().numpy()
 
 
@@ -520,7 +521,7 @@ def test_mxfp8_activation_quantizer_bit_exact(M, K):
     x = randn_bf16((M, K), 1.0, 91)
     x[0, :32] = 0.0                      # an all-zero block
     x.view(-1)[5::97] *= 37.0            # outliers that set block maxima
-    Mp = (M + 15) // 16 * 16
+    Mp = (M + 63) // 64 * 64
     xq = torch.empty(Mp * K, dtype=torch.uint8, device="cuda")
     xs = torch.empty(Mp * K // 32, dtype=torch.uint8, device="cuda")
     xg = x.cuda()
@@ -528,7 +529,7 @@ def test_mxfp8_activation_quantizer_bit_exact(M, K):
     q, s = _mxfp8_from_operand_order(xq, xs, M, K)
     q_or, s_or = O.quant_act_mxfp8(t2bits(x))
     assert np.array_equal(q[:M], q_or) and np.array_equal(s[:M], s_or)
-    assert not q[M:].any()               # padded rows are zeros
+    assert not q[M:].any() and not s[M:].any()  # padded rows are zeros
 
 
 @pytest.mark.parametrize("M,N,K,post", [(128, 256, 256, "none"), (1, 32, 128, "none"), (200, 544, 384, "add"),

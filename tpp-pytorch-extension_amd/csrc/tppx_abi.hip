@@ -234,7 +234,7 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     // opt-in, not the reference's arithmetic: activations quantised to MXFP8 (into the workspace), then the
     // block-scaled MFMA kernel on the weights' own codes and scales; any M, but built for prefill shapes
     TPPX_REQUIRE(!row_sumsq, TPPX_EUNSUPPORTED, "%s: row sums of squares are not produced by the FP8-activation kernel", who);
-    const int64_t Mp = (M + 15) / 16 * 16, need = Mp * K + Mp * (K / 32);
+    const int64_t Mp = (M + 63) / 64 * 64, need = Mp * K + Mp * (K / 32);
     TPPX_REQUIRE(ws && ws_bytes >= need, TPPX_EINVAL, "%s: the FP8-activation path needs %ld bytes of workspace for the quantised activations (got %ld)", who, (long)need, (long)ws_bytes);
     uint8_t* xq = (uint8_t*)ws;
     uint8_t* xs = xq + Mp * K;

@@ -93,7 +93,8 @@ int env_int(const char* name, int dflt);
 hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs, void* xq, void* sa, int mt,
                                  hipStream_t stream);
 
-// MXFP8 activations in MFMA operand order for the block-scaled prefill kernel: xq (M16*16*K bytes), xs (M16*16*K/32)
+// MXFP8 activations in MFMA operand order for the block-scaled prefill kernel: rows padded to Mp = roundup(M, 64);
+// xq Mp*K bytes, xs Mp*K/32 bytes
 hipError_t launch_quant_act_mxfp8(const void* x, int64_t M, int64_t K, void* xq, void* xs, hipStream_t stream);
 
 // can_fuse_quant: bf16 activations at hand and 256-wide blocks (the in-kernel quantisation's case)

@@ -256,9 +256,10 @@ prepack_bf16_kernel(const uint16_t* __restrict__ wref, int64_t N, int64_t K, int
 // input channels, scale exponent = floor(log2 max|x|) - 8 as the OCP MX recipe has it), written in MFMA operand
 // order: values [M/16][K/128][2 halves][64 lanes][16 B] -- an 8-bit operand of the 16x16x128 instruction is two
 // 64-channel halves, so lane (g, m) of a 16-row x 128-channel tile holds channels g*16 .. g*16+15 of row m in half
-// 0 and 64 + g*16 .. 64 + g*16+15 in half 1 -- and scale bytes [M/16][K/128][64 lanes]: lane (b, m) holds the scale
-// of channels b*32 .. b*32+31 (the instruction scales by 32-channel block, whichever lanes hold the elements).
-// Rows past M in the last tile are zeros.  One thread per (row, 32-channel block).
+// 0 and 64 + g*16 .. 64 + g*16+15 in half 1 -- and scale bytes [M/64][K/128][64 lanes][4 row tiles]: byte t of
+// lane (b, m)'s word is the scale of channels b*32 .. b*32+31 of row m of the group's row tile t (the instruction
+// scales by 32-channel block, whichever lanes hold the elements).  Rows are padded to a multiple of 64 with zeros
+// (scale byte 0).  One thread per (row, 32-channel block).
 __device__ __forceinline__ uint32_t e4m3_encode_rne(float v) {
   const uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
   const float a = fminf(fabsf(v), 448.0f);
@@ -274,7 +275,7 @@ quant_act_mxfp8_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K, uin
                        uint8_t* __restrict__ xs) {
   const int64_t KB = K / 32, KT = K / 128;
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t Mp = (M + 15) / 16 * 16;
+  const int64_t Mp = (M + 63) / 64 * 64;
   if (t >= Mp * KB)
     return;
   const int64_t m = t / KB, kb = t % KB;
@@ -317,7 +318,7 @@ quant_act_mxfp8_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K, uin
   const int c0 = (int)(kb & 3) * 2;
   dst[(c0 >> 2) * 64 + (c0 & 3) * 16] = make_uint4(out[0], out[1], out[2], out[3]);
   dst[((c0 + 1) >> 2) * 64 + ((c0 + 1) & 3) * 16] = make_uint4(out[4], out[5], out[6], out[7]);
-  xs[(mt * KT + kt) * 64 + lane] = (uint8_t)X;
+  xs[(((mt >> 2) * KT + kt) * 64 + lane) * 4 + (mt & 3)] = m < M ? (uint8_t)X : (uint8_t)0;
 }
 
 // Activation quantizer: one wave per (row, K block).  Each lane owns
@@ -392,7 +393,7 @@ hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qb
 }
 
 hipError_t launch_quant_act_mxfp8(const void* x, int64_t M, int64_t K, void* xq, void* xs, hipStream_t stream) {
-  const int64_t nthreads = (M + 15) / 16 * 16 * (K / 32);
+  const int64_t nthreads = (M + 63) / 64 * 64 * (K / 32);
   TPPX_PLAN_ONLY(quant_act_mxfp8_kernel, dim3(grid_for(nthreads, 256)), dim3(256), 0);
   quant_act_mxfp8_kernel<<<grid_for(nthreads, 256), 256, 0, stream>>>((const uint16_t*)x, M, K, (uint8_t*)xq, (uint8_t*)xs);
   return hipGetLastError();

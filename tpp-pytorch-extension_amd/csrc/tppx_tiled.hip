@@ -20,6 +20,7 @@
 // MFMA operand convention (A = activations, B = weights):
 //   lane l supplies row/col (l & 15) and K group (l >> 4);
 //   result register r of lane l is D[m = (l >> 4) * 4 + r][n = l & 15].
+#include <algorithm>
 #include <string.h>
 #include <type_traits>
 
@@ -776,22 +777,45 @@ big_qint8_kernel(const BigParams P) {
 // expanded -- and the activations arrive quantised in operand order
 // (quant_act_mxfp8_kernel).  Not the reference's arithmetic (its activations
 // stay bf16): an opt-in (TPPX_FLAG_ACT_FP8).
-// Workgroup tile 128 (M) x 256 (N), 8 waves (2 x 4), wave tile 64 x 64 = 16
-// MFMAs of K = 128 per step.  Both operands go from global memory straight
-// into LDS, 1 KiB per wave instruction (a native weight tile, half an
-// activation tile: lane-linear on both sides, so operand reads are
-// conflict-free 16-byte reads), a step ahead, two buffers of 32 KiB; one
-// barrier per step.  Scale bytes come from global/L2, a step ahead.
+// Workgroup tile (MT*32) x 256, 8 waves (2 x 4), wave tile (MT*16) x 64 =
+// 4*MT MFMAs of K = 128 per step; MT = 8 (256 rows) or 4 (128 rows).
+// Everything a step needs -- both operands AND both sets of scale bytes -- goes
+// from global memory straight into LDS (1 KiB per wave instruction for the
+// operands: a native weight tile, half an activation tile, lane-linear on both
+// sides, so operand reads are conflict-free 16-byte reads; 256 B per wave
+// instruction for scales), NB - 1 steps ahead in a ring of NB stages.  All
+// loads of the loop being of this one kind, they complete in issue order and
+// the wait at the top of a step is a partial one (the younger stages stay in
+// flight); one barrier per step.
 // ---------------------------------------------------------------------------
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
+template <int N>
+__device__ __forceinline__ void lds_wait_keep2(i32x4& a, i32x4& b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+
+template <int MT>
+struct Fp8Geom {
+  static constexpr int NB = MT == 8 ? 3 : 4;        // stages in the ring
+  static constexpr int A_BYTES = MT * 4096;         // 2*MT row tiles of 2 KiB
+  static constexpr int B_OFF = A_BYTES;             // 16 weight tiles of 1 KiB
+  static constexpr int SA_OFF = B_OFF + 16384;      // MT/2 groups of 64 rows x 256 B
+  static constexpr int SB_OFF = SA_OFF + MT * 128;  // 16 tiles x 64 B
+  static constexpr int STAGE = SB_OFF + 1024;
+  static constexpr int LPS = MT / 2 + 2 + 1;        // loads per wave and stage: A halves, weight tiles, one of scales
+};
+
+template <int MT>
 __global__ void __launch_bounds__(512)
 big_fp8_kernel(const BigParams P) {
+  using G = Fp8Geom<MT>;
+  constexpr int NB = G::NB, STAGE = G::STAGE, LPS = G::LPS;
   extern __shared__ __align__(16) uint8_t tl_lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave & 1, wn = wave >> 1;
-  const int MB = (P.seg[0].M + 127) / 128;
+  const int MB = (P.seg[0].M + MT * 32 - 1) / (MT * 32);
   int bm, bn;
   tile_of_block(MB, P.nb0[P.n_seg], bm, bn);
   TiledParams p = P.seg[0];
@@ -804,91 +828,118 @@ big_fp8_kernel(const BigParams P) {
     }
   bn -= nb_first;
   const int KT = p.K >> 7;
-  const int m_wg = bm * 128;
+  const int m_wg = bm * (MT * 32);
   const int tile_base = bn * 16 + wn * 4;
-  const int MT16 = (p.M + 15) >> 4;
+  const int Q = (p.M + 63) >> 6; // 64-row groups of the quantised activations (rows padded to 64)
 
-  // this wave's share of a step's traffic: activation tile `wave` of the 8 (two halves), weight tiles 2*wave, 2*wave+1
+  // this wave's share of a stage: MT/2 activation half tiles, 2 weight tiles, one 256-byte piece of scales
   const char* xqb = reinterpret_cast<const char*>(p.xq);
   const char* qwb = reinterpret_cast<const char*>(p.qw);
-  const size_t a_src = ((size_t)min(bm * 8 + wave, MT16 - 1) * KT * 2) * 1024 + (size_t)lane * 16;
-  size_t b_src[2];
+  const char* a_src[MT / 2];
+#pragma unroll
+  for (int i = 0; i < MT / 2; i++) {
+    const int j = wave * (MT / 2) + i; // half tile j of the 4*MT: row tile j >> 1, half j & 1
+    a_src[i] = xqb + ((size_t)min(bm * (MT * 2) + (j >> 1), Q * 4 - 1) * KT * 2 + (j & 1)) * 1024 + (size_t)lane * 16;
+  }
+  const char* b_src[2];
 #pragma unroll
   for (int i = 0; i < 2; i++)
-    b_src[i] = ((size_t)min(bn * 16 + wave * 2 + i, p.tiles - 1) * KT) * 1024 + (size_t)lane * 16;
+    b_src[i] = qwb + ((size_t)min(bn * 16 + wave * 2 + i, p.tiles - 1) * KT) * 1024 + (size_t)lane * 16;
+  const char* s_src;
+  int s_dst, s_stride;
+  if (wave < MT / 2) { // activation scales of 64-row group `wave`: [Q][KT][64 lanes][4 row tiles]
+    s_src = reinterpret_cast<const char*>(p.sa) + (size_t)min(bm * (MT / 2) + wave, Q - 1) * KT * 256 + (size_t)lane * 4;
+    s_dst = G::SA_OFF + wave * 256;
+    s_stride = 256;
+  } else { // weight scales of tiles 4i .. 4i+3: native [tile][KT][64]
+    int i = wave - MT / 2;
+    if (i >= 4)
+      i -= 2; // 128-row form: waves 6, 7 repeat what 4, 5 fetch, so that every wave issues LPS loads per stage
+    s_src = reinterpret_cast<const char*>(p.sw) + (size_t)min(bn * 16 + i * 4 + (lane >> 4), p.tiles - 1) * KT * 64 +
+            (size_t)(lane & 15) * 4;
+    s_dst = G::SB_OFF + i * 256;
+    s_stride = 64;
+  }
   auto dma = [&](int ks, int buf) {
-    uint8_t* base = tl_lds + buf * 32768;
+    uint8_t* base = tl_lds + buf * STAGE;
 #pragma unroll
-    for (int h = 0; h < 2; h++)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xqb + a_src + ((size_t)ks * 2 + h) * 1024),
-                                       (__attribute__((address_space(3))) void*)(base + (wave * 2 + h) * 1024), 16, 0, 0);
+    for (int i = 0; i < MT / 2; i++)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[i] + (size_t)ks * 2048),
+                                       (__attribute__((address_space(3))) void*)(base + (wave * (MT / 2) + i) * 1024), 16, 0, 0);
 #pragma unroll
     for (int i = 0; i < 2; i++)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(qwb + b_src[i] + (size_t)ks * 1024),
-                                       (__attribute__((address_space(3))) void*)(base + 16384 + (wave * 2 + i) * 1024), 16, 0, 0);
-  };
-  // scale bytes of this wave's 4 row tiles and 4 channel tiles
-  const uint8_t* xsb = reinterpret_cast<const uint8_t*>(p.sa);
-  const uint8_t* swb = reinterpret_cast<const uint8_t*>(p.sw);
-  size_t sa_off[4], sb_off[4];
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    sa_off[i] = (size_t)min(bm * 8 + wm * 4 + i, MT16 - 1) * KT * 64 + lane;
-    sb_off[i] = (size_t)min(tile_base + i, p.tiles - 1) * KT * 64 + lane;
-  }
-  int sa_n[4], sb_n[4], sa_c[4], sb_c[4];
-  auto load_scales = [&](int ks) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      sa_n[i] = xsb[sa_off[i] + (size_t)ks * 64];
-      sb_n[i] = swb[sb_off[i] + (size_t)ks * 64];
-    }
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[i] + (size_t)ks * 1024),
+                                       (__attribute__((address_space(3))) void*)(base + G::B_OFF + (wave * 2 + i) * 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(s_src + (size_t)ks * s_stride),
+                                     (__attribute__((address_space(3))) void*)(base + s_dst), 4, 0, 0);
   };
 
-  f32x4 acc[4][4];
+  f32x4 acc[MT][4];
 #pragma unroll
-  for (int mt = 0; mt < 4; mt++)
+  for (int mt = 0; mt < MT; mt++)
 #pragma unroll
     for (int nt = 0; nt < 4; nt++)
       acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  dma(0, 0);
-  load_scales(0);
+  const uint32_t lds0 = (uint32_t)(uintptr_t)tl_lds;
+#pragma unroll
+  for (int s = 0; s < NB - 1; s++)
+    if (s < KT)
+      dma(s, s);
+  int buf = 0;
   for (int ks = 0; ks < KT; ks++) {
-    const int buf = ks & 1;
-    __syncthreads(); // step ks has landed for every wave (the barrier waits for this wave's loads first) and
-                     // nobody still reads the other buffer
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      sa_c[i] = sa_n[i];
-      sb_c[i] = sb_n[i];
-    }
-    if (ks + 1 < KT) {
-      dma(ks + 1, buf ^ 1);
-      load_scales(ks + 1);
-    }
-    const uint8_t* base = tl_lds + buf * 32768;
-    i32x8 a[4], b[4];
-#pragma unroll
-    for (int mt = 0; mt < 4; mt++) {
-      const i32x4 lo = *reinterpret_cast<const i32x4*>(base + ((wm * 4 + mt) * 2) * 1024 + lane * 16);
-      const i32x4 hi = *reinterpret_cast<const i32x4*>(base + ((wm * 4 + mt) * 2 + 1) * 1024 + lane * 16);
-      a[mt] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    }
+    // stage ks has landed for this wave (the NB - 2 younger ones may still be in flight) ...
+    if (ks + NB - 2 < KT)
+      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(LPS * (NB - 2)) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+    // ... and for every wave; nobody still reads the stage of step ks - 1, which the next loads overwrite
+    asm volatile("s_barrier" : : : "memory");
+    if (ks + NB - 1 < KT)
+      dma(ks + NB - 1, buf == 0 ? NB - 1 : buf - 1);
+    const uint8_t* base = tl_lds + buf * STAGE;
+    i32x4 bw[4];
+    int sbv[4];
+    uint32_t sav[MT / 4];
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) {
-      const i32x4 w = *reinterpret_cast<const i32x4*>(base + 16384 + (wn * 4 + nt) * 1024 + lane * 16);
-      b[nt] = i32x8{w[0], w[1], w[2], w[3], 0, 0, 0, 0};
+      bw[nt] = *reinterpret_cast<const i32x4*>(base + G::B_OFF + (wn * 4 + nt) * 1024 + lane * 16);
+      sbv[nt] = base[G::SB_OFF + (wn * 4 + nt) * 64 + lane];
     }
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++)
+    for (int q = 0; q < MT / 4; q++)
+      sav[q] = *reinterpret_cast<const uint32_t*>(base + G::SA_OFF + (wm * (MT / 4) + q) * 256 + lane * 4);
+    // activation operands: the two halves of row tile mt, read two row tiles ahead of the MFMAs that use them
+    const uint32_t abase = lds0 + (uint32_t)(buf * STAGE + wm * MT * 2048 + lane * 16);
+    i32x4 alo[3], ahi[3];
+    static_for<0, 2>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      lds_read_b128_async<i * 2048>(alo[i], abase);
+      lds_read_b128_async<i * 2048 + 1024>(ahi[i], abase);
+    });
+    static_for<0, MT>([&](auto I) {
+      constexpr int mt = decltype(I)::value;
+      if constexpr (mt + 2 < MT) {
+        lds_read_b128_async<(mt + 2) * 2048>(alo[(mt + 2) % 3], abase);
+        lds_read_b128_async<(mt + 2) * 2048 + 1024>(ahi[(mt + 2) % 3], abase);
+        lds_wait_keep2<4>(alo[mt % 3], ahi[mt % 3]);
+      } else {
+        lds_wait_keep2<(MT - 1 - mt) * 2>(alo[mt % 3], ahi[mt % 3]);
+      }
+      const i32x4 lo = alo[mt % 3], hi = ahi[mt % 3];
+      const i32x8 a = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      const int sa = (int)((sav[mt >> 2] >> ((mt & 3) * 8)) & 0xffu);
 #pragma unroll
-      for (int nt = 0; nt < 4; nt++)
-        acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[mt], b[nt], acc[mt][nt], 0 /* A: E4M3 */,
-                                                                       4 /* B: E2M1 */, 0, sa_c[mt], 0, sb_c[nt]);
+      for (int nt = 0; nt < 4; nt++) {
+        const i32x8 b = i32x8{bw[nt][0], bw[nt][1], bw[nt][2], bw[nt][3], 0, 0, 0, 0};
+        acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[mt][nt], 0 /* A: E4M3 */,
+                                                                       4 /* B: E2M1 */, 0, sa, 0, sbv[nt]);
+      }
+    });
+    buf = buf == NB - 1 ? 0 : buf + 1;
   }
   __syncthreads(); // every wave has left the main loop: LDS is free for the epilogue staging
-  big_epilogue<4>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * 64, tile_base);
+  big_epilogue<MT>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
 }
 
 static bool big_fits(const TiledParams& p) {
@@ -956,18 +1007,35 @@ hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t
   for (int i = n; i <= TPPX_MAX_SEGS; i++)
     P.nb0[i] = nb;
   P.n_seg = n;
-  const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the two operand buffers
-  const int MB = (t[0].M + 127) / 128;
-  TPPX_PLAN_ONLY(big_fp8_kernel, dim3(MB * nb), dim3(512), lds);
+  const size_t ep = 8 * 64 * EP_LD * sizeof(float); // epilogue staging
+  const size_t lds8 = std::max(ep, (size_t)Fp8Geom<8>::NB * Fp8Geom<8>::STAGE);
+  const size_t lds4 = std::max(ep, (size_t)Fp8Geom<4>::NB * Fp8Geom<4>::STAGE);
+  // 256-row tiles unless 128-row ones fill the last round of workgroups (256 CUs, one workgroup each) better
+  const int MB8 = (t[0].M + 255) / 256, MB4 = (t[0].M + 127) / 128;
+  auto rounds = [](int wgs) { return (wgs + 255) / 256; };
+  const double cost8 = rounds(MB8 * nb), cost4 = 0.5 * 1.15 * rounds(MB4 * nb);
+  int mt = cost4 < cost8 ? 4 : 8;
+  const int env_mt = env_int("TPPX_FP8_BIG_MT", 0);
+  if (env_mt == 4 || env_mt == 8)
+    mt = env_mt;
   static bool attr_done = false;
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_fp8_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_fp8_kernel<8>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds8);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_fp8_kernel<4>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds4);
     if (e != hipSuccess)
       return e;
     attr_done = true;
   }
-  big_fp8_kernel<<<dim3(MB * nb), dim3(512), lds, stream>>>(P);
+  if (mt == 4) {
+    TPPX_PLAN_ONLY(big_fp8_kernel<4>, dim3(MB4 * nb), dim3(512), lds4);
+    big_fp8_kernel<4><<<dim3(MB4 * nb), dim3(512), lds4, stream>>>(P);
+  } else {
+    TPPX_PLAN_ONLY(big_fp8_kernel<8>, dim3(MB8 * nb), dim3(512), lds8);
+    big_fp8_kernel<8><<<dim3(MB8 * nb), dim3(512), lds8, stream>>>(P);
+  }
   return hipGetLastError();
 }
 

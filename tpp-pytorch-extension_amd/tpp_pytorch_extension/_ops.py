@@ -348,7 +348,7 @@ def _mxfp4_flags_ws(x, M, K, flags=0):
         flags |= _lib.FLAG_ACT_FP8
     ws = _lib.workspace(x)
     if flags & _lib.FLAG_ACT_FP8:
-        Mp = (M + 15) // 16 * 16
+        Mp = (M + 63) // 64 * 64
         need = Mp * K + Mp * (K // 32)
         if need > ws.numel():
             ws = torch.empty(need, dtype=torch.uint8, device=x.device)
