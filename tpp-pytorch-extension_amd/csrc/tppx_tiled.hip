@@ -860,19 +860,21 @@ big_fp8_kernel(const BigParams P) {
     s_dst = G::SB_OFF + i * 256;
     s_stride = 64;
   }
-  auto dma = [&](int ks, int buf) {
+  // load number I (of LPS) of this wave's share of a stage
+  auto dma_one = [&](auto I, int ks, int buf) {
+    constexpr int i = decltype(I)::value;
     uint8_t* base = tl_lds + buf * STAGE;
-#pragma unroll
-    for (int i = 0; i < MT / 2; i++)
+    if constexpr (i < MT / 2)
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_src[i] + (size_t)ks * 2048),
                                        (__attribute__((address_space(3))) void*)(base + (wave * (MT / 2) + i) * 1024), 16, 0, 0);
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[i] + (size_t)ks * 1024),
-                                       (__attribute__((address_space(3))) void*)(base + G::B_OFF + (wave * 2 + i) * 1024), 16, 0, 0);
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(s_src + (size_t)ks * s_stride),
-                                     (__attribute__((address_space(3))) void*)(base + s_dst), 4, 0, 0);
+    else if constexpr (i < MT / 2 + 2)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(b_src[i - MT / 2] + (size_t)ks * 1024),
+                                       (__attribute__((address_space(3))) void*)(base + G::B_OFF + (wave * 2 + i - MT / 2) * 1024), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(s_src + (size_t)ks * s_stride),
+                                       (__attribute__((address_space(3))) void*)(base + s_dst), 4, 0, 0);
   };
+  auto dma = [&](int ks, int buf) { static_for<0, LPS>([&](auto I) { dma_one(I, ks, buf); }); };
 
   f32x4 acc[MT][4];
 #pragma unroll
@@ -887,16 +889,19 @@ big_fp8_kernel(const BigParams P) {
     if (s < KT)
       dma(s, s);
   int buf = 0;
-  for (int ks = 0; ks < KT; ks++) {
+  // One K step.  DMA: the loads of stage ks + NB - 1 are issued one at a time behind the MFMA groups of the step
+  // (issued in one burst at the top, a wave stands at its load instructions while the memory pipeline's queue
+  // drains, and its MFMAs wait with it).
+  auto step = [&](auto DMA, int ks) {
+    constexpr bool with_dma = decltype(DMA)::value;
     // stage ks has landed for this wave (the NB - 2 younger ones may still be in flight) ...
-    if (ks + NB - 2 < KT)
+    if (with_dma || ks + NB - 2 < KT)
       asm volatile("s_waitcnt vmcnt(%0)" : : "n"(LPS * (NB - 2)) : "memory");
     else
       asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
     // ... and for every wave; nobody still reads the stage of step ks - 1, which the next loads overwrite
     asm volatile("s_barrier" : : : "memory");
-    if (ks + NB - 1 < KT)
-      dma(ks + NB - 1, buf == 0 ? NB - 1 : buf - 1);
+    const int nbuf = buf == 0 ? NB - 1 : buf - 1;
     const uint8_t* base = tl_lds + buf * STAGE;
     i32x4 bw[4];
     int sbv[4];
@@ -935,9 +940,21 @@ big_fp8_kernel(const BigParams P) {
         acc[mt][nt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[mt][nt], 0 /* A: E4M3 */,
                                                                        4 /* B: E2M1 */, 0, sa, 0, sbv[nt]);
       }
+      if constexpr (with_dma) {
+        // LPS loads over MT slots (LPS <= MT + 1: the last slot takes the remainder)
+        if constexpr (mt < LPS)
+          dma_one(std::integral_constant<int, mt>{}, ks + NB - 1, nbuf);
+        if constexpr (mt == MT - 1)
+          static_for<MT, (LPS > MT ? LPS : MT)>([&](auto J) { dma_one(J, ks + NB - 1, nbuf); });
+      }
     });
     buf = buf == NB - 1 ? 0 : buf + 1;
-  }
+  };
+  int ks = 0;
+  for (; ks + NB - 1 < KT; ks++)
+    step(std::true_type{}, ks);
+  for (; ks < KT; ks++)
+    step(std::false_type{}, ks);
   __syncthreads(); // every wave has left the main loop: LDS is free for the epilogue staging
   big_epilogue<MT>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
 }
