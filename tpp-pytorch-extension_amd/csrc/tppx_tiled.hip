@@ -467,22 +467,21 @@ big_mxfp4_kernel(const BigParams P) {
   const bool full = m_wg + WGM <= p.M; // uniform
   const uint32_t xrow0 = (uint32_t)((m_wg + wave * (MT * 4) + rin) * p.K) * 2u;
   const uint32_t blk_stride = (uint32_t)(4 * p.K) * 2u; // uniform
-  auto load_a = [&](int ks, int buf) {
-#pragma unroll
-    for (int i = 0; i < MT; i++) {
-      const uint32_t sw = (uint32_t)((ch ^ ((i & 3) * 4 + rin)) & 15) * 16u;
-      uint32_t off;
-      if (full) {
-        off = xrow0 + (uint32_t)i * blk_stride + sw + (uint32_t)ks * 256u;
-      } else { // past the end: re-read the last row (never stored)
-        const int row = min(m_wg + (wave * MT + i) * 4 + rin, p.M - 1);
-        off = (uint32_t)(row * p.K) * 2u + sw + (uint32_t)ks * 256u;
-      }
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xbase + (size_t)off),
-                                       (__attribute__((address_space(3))) void*)(tl_lds + buf * ABUF + (wave * MT + i) * 1024),
-                                       16, 0, 0);
+  auto load_a_one = [&](auto I, int ks, int buf) {
+    constexpr int i = decltype(I)::value;
+    const uint32_t sw = (uint32_t)((ch ^ ((i & 3) * 4 + rin)) & 15) * 16u;
+    uint32_t off;
+    if (full) {
+      off = xrow0 + (uint32_t)i * blk_stride + sw + (uint32_t)ks * 256u;
+    } else { // past the end: re-read the last row (never stored)
+      const int row = min(m_wg + (wave * MT + i) * 4 + rin, p.M - 1);
+      off = (uint32_t)(row * p.K) * 2u + sw + (uint32_t)ks * 256u;
     }
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xbase + (size_t)off),
+                                     (__attribute__((address_space(3))) void*)(tl_lds + buf * ABUF + (wave * MT + i) * 1024),
+                                     16, 0, 0);
   };
+  auto load_a = [&](int ks, int buf) { static_for<0, MT>([&](auto I) { load_a_one(I, ks, buf); }); };
   // B of one K step: 4 tiles x 4 dwords (one per step j) and the scale factors
   uint32_t bc[4][4];
   float sc[4];
@@ -516,12 +515,13 @@ big_mxfp4_kernel(const BigParams P) {
   load_a(0, 0);
   load_b(0);
   __syncthreads();
-  for (int ks = 0; ks < KT; ks++) {
+  // One K step.  MORE: the next step's A tile is requested during this one, one block behind each of the first MT
+  // MFMA groups (issued in one burst, a wave stands at its load instructions while the memory pipeline's queue
+  // drains, and its MFMAs wait with it); it lands in the other buffer.
+  auto step = [&](auto MORE, int ks) {
+    constexpr bool more = decltype(MORE)::value;
     const int buf = ks & 1;
-    const bool more = ks + 1 < KT;
     take_b();
-    if (more)
-      load_a(ks + 1, buf ^ 1); // lands in the other buffer during this step's MFMAs
     // 4*MT operand reads per K step (q = j*MT + mt), kept RD ahead of the MFMAs
     // that consume them so the LDS latency is covered by 4*RD MFMAs
     const uint32_t abase = lds0 + (uint32_t)(buf * ABUF + wm * MT * 4096);
@@ -551,13 +551,16 @@ big_mxfp4_kernel(const BigParams P) {
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
         acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[nt], acc[mt][nt], 0, 0, 0);
-      if constexpr (q == NQ / 2 - 1) {
-        if (more)
-          load_b(ks + 1); // dwords of steps 0 and 1 of the current B are dead by now
-      }
+      if constexpr (more && q < MT)
+        load_a_one(std::integral_constant<int, q>{}, ks + 1, buf ^ 1);
+      if constexpr (more && q == NQ / 2 - 1)
+        load_b(ks + 1); // dwords of steps 0 and 1 of the current B are dead by now
     });
     __syncthreads(); // waits for this wave's direct-to-LDS loads, then for everybody's
-  }
+  };
+  for (int ks = 0; ks + 1 < KT; ks++)
+    step(std::true_type{}, ks);
+  step(std::false_type{}, KT - 1);
   // every wave has left the main loop (barrier above): LDS is free for the epilogue staging
   big_epilogue<MT>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
 }
