@@ -645,37 +645,34 @@ big_qint8_kernel(const BigParams P) {
   const bool full = m_wg + WGM <= p.M;
   const uint32_t xrow0 = (uint32_t)((m_wg + wave * (MT * 4) + rin) * p.K);
   const uint32_t blk_stride = (uint32_t)(4 * p.K);
-  auto load_a = [&](int ks, int buf) {
-#pragma unroll
-    for (int i = 0; i < MT; i++) {
-      const uint32_t sw = (uint32_t)((ch ^ ((i & 3) * 4 + rin)) & 15) * 16u;
-      uint32_t off;
-      if (full) {
-        off = xrow0 + (uint32_t)i * blk_stride + sw + (uint32_t)ks * 256u;
-      } else {
-        const int row = min(m_wg + (wave * MT + i) * 4 + rin, p.M - 1);
-        off = (uint32_t)(row * p.K) + sw + (uint32_t)ks * 256u;
-      }
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xbase + (size_t)off),
-                                       (__attribute__((address_space(3))) void*)(tl_lds + buf * ABUF + (wave * MT + i) * 1024),
-                                       16, 0, 0);
+  auto load_a_one = [&](auto I, int ks, int buf) {
+    constexpr int i = decltype(I)::value;
+    const uint32_t sw = (uint32_t)((ch ^ ((i & 3) * 4 + rin)) & 15) * 16u;
+    uint32_t off;
+    if (full) {
+      off = xrow0 + (uint32_t)i * blk_stride + sw + (uint32_t)ks * 256u;
+    } else {
+      const int row = min(m_wg + (wave * MT + i) * 4 + rin, p.M - 1);
+      off = (uint32_t)(row * p.K) + sw + (uint32_t)ks * 256u;
     }
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xbase + (size_t)off),
+                                     (__attribute__((address_space(3))) void*)(tl_lds + buf * ABUF + (wave * MT + i) * 1024),
+                                     16, 0, 0);
   };
+  auto load_a = [&](int ks, int buf) { static_for<0, MT>([&](auto I) { load_a_one(I, ks, buf); }); };
   // B of step ks: this wave brings tiles 2*wave, 2*wave + 1 of the 16, all four K tiles; LDS slot (tile*4 + kt) KiB
   const char* qwb = reinterpret_cast<const char*>(p.qw);
   uint32_t bsrc[2];
 #pragma unroll
   for (int i = 0; i < 2; i++)
     bsrc[i] = (uint32_t)(min(bn * 16 + wave * 2 + i, p.tiles - 1) * KT64 * 64 + lane);
-  auto load_b = [&](int ks) {
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-      for (int kt = 0; kt < 4; kt++)
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(qwb + (size_t)((bsrc[i] + (uint32_t)(ks * 4 + kt) * 64u) * 16u)),
-            (__attribute__((address_space(3))) void*)(b_lds + ((wave * 2 + i) * 4 + kt) * 1024), 16, 0, 0);
+  auto load_b_one = [&](auto I, int ks) {
+    constexpr int i = decltype(I)::value >> 2, kt = decltype(I)::value & 3;
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void*)(qwb + (size_t)((bsrc[i] + (uint32_t)(ks * 4 + kt) * 64u) * 16u)),
+        (__attribute__((address_space(3))) void*)(b_lds + ((wave * 2 + i) * 4 + kt) * 1024), 16, 0, 0);
   };
+  auto load_b = [&](int ks) { static_for<0, 8>([&](auto I) { load_b_one(I, ks); }); };
   // activation scales: thread t < 128 carries the scale of row t for the step two ahead
   const float* sarow = p.sa + (int64_t)min(m_wg + (tid & 127), p.M - 1) * KS;
   float sareg = 0.f;
@@ -707,9 +704,11 @@ big_qint8_kernel(const BigParams P) {
   }
   __syncthreads();
   const uint32_t bwave = lds0 + (uint32_t)(2 * ABUF + wn * 16 * 1024) + (uint32_t)lane * 16u; // this wave's 4 tiles
-  for (int ks = 0; ks < KS; ks++) {
+  // One K step.  MORE: the next step's tiles are requested one wave instruction at a time behind the MFMA groups
+  // (in one burst, a wave stands at its load instructions while the memory pipeline's queue drains).
+  auto step = [&](auto MORE, int ks) {
+    constexpr bool more = decltype(MORE)::value;
     const int buf = ks & 1;
-    const bool more = ks + 1 < KS;
     // this step's weight operands: LDS -> registers, then the buffer is free for the next step's tiles
     i32x4 bq[4][4]; // [tile][MFMA step j]
     static_for<0, 16>([&](auto I) {
@@ -725,9 +724,7 @@ big_qint8_kernel(const BigParams P) {
     }
     lds_wait_keep16<0>(bq);
     __syncthreads();
-    if (more) {
-      load_b(ks + 1);
-      load_a(ks + 1, buf ^ 1);
+    if constexpr (more) {
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
         swn[nt] = swp[soff[nt] + (uint32_t)(ks + 1) * 16u];
@@ -763,12 +760,19 @@ big_qint8_kernel(const BigParams P) {
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
         iacc[mt & 1][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bq[nt][j], j == 0 ? i32x4{0, 0, 0, 0} : iacc[mt & 1][nt], 0, 0, 0);
+      if constexpr (more && q < 8)
+        load_b_one(std::integral_constant<int, q>{}, ks + 1);
+      if constexpr (more && q >= 8 && q < 8 + MT)
+        load_a_one(std::integral_constant<int, q - 8>{}, ks + 1, buf ^ 1);
       if constexpr (j == 0 && mt > 0)
         fold(std::integral_constant<int, mt - 1>{}); // the previous row tile, under this row tile's MFMAs
     });
     fold(std::integral_constant<int, MT - 1>{});
     __syncthreads();
-  }
+  };
+  for (int ks = 0; ks + 1 < KS; ks++)
+    step(std::true_type{}, ks);
+  step(std::false_type{}, KS - 1);
   big_epilogue<MT>(p, facc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
 }
 
