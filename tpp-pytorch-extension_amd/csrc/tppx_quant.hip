@@ -259,7 +259,7 @@ prepack_bf16_kernel(const uint16_t* __restrict__ wref, int64_t N, int64_t K, int
 // 0 and 64 + g*16 .. 64 + g*16+15 in half 1 -- and scale bytes [M/64][K/128][64 lanes][4 row tiles]: byte t of
 // lane (b, m)'s word is the scale of channels b*32 .. b*32+31 of row m of the group's row tile t (the instruction
 // scales by 32-channel block, whichever lanes hold the elements).  Rows are padded to a multiple of 64 with zeros
-// (scale byte 0).  One thread per (row, 32-channel block).
+// (scale byte 0).
 __device__ __forceinline__ uint32_t e4m3_encode_rne(float v) {
   const uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
   const float a = fminf(fabsf(v), 448.0f);
@@ -273,35 +273,39 @@ __device__ __forceinline__ uint32_t e4m3_encode_rne(float v) {
 __global__ void __launch_bounds__(256)
 quant_act_mxfp8_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K, uint8_t* __restrict__ xq,
                        uint8_t* __restrict__ xs) {
-  const int64_t KB = K / 32, KT = K / 128;
+  // One wave per half of a 16-row x 128-channel tile: lane (g, r) turns channels h*64 + g*16 .. +15 of row r into the
+  // 16 bytes it holds as an operand, so a wave reads 16 pieces of 128 contiguous bytes and writes 1 KiB in lane order;
+  // the two lanes that share a 32-channel block (g, g ^ 1) exchange their maxima.
+  const int64_t KT = K / 128;
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t Mp = (M + 63) / 64 * 64;
-  if (t >= Mp * KB)
+  const int64_t tile = t >> 7;
+  if (tile >= (Mp / 16) * KT) // wave-uniform
     return;
-  const int64_t m = t / KB, kb = t % KB;
-  uint32_t w[16];
+  const int lane = (int)(t & 63), h = (int)((t >> 6) & 1), g = lane >> 4, r = lane & 15;
+  const int64_t mt = tile / KT, kt = tile % KT, m = mt * 16 + r;
+  uint32_t w[8];
   if (m < M) {
-    const uint4* src = reinterpret_cast<const uint4*>(x + m * K + kb * 32);
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const uint4 v = src[i];
-      w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
-    }
+    const uint4* src = reinterpret_cast<const uint4*>(x + m * K + kt * 128 + h * 64 + g * 16);
+    const uint4 v0 = src[0], v1 = src[1];
+    w[0] = v0.x; w[1] = v0.y; w[2] = v0.z; w[3] = v0.w;
+    w[4] = v1.x; w[5] = v1.y; w[6] = v1.z; w[7] = v1.w;
   } else {
 #pragma unroll
-    for (int i = 0; i < 16; i++)
+    for (int i = 0; i < 8; i++)
       w[i] = 0u;
   }
   float amax = 0.0f;
 #pragma unroll
-  for (int i = 0; i < 16; i++)
+  for (int i = 0; i < 8; i++)
     amax = fmaxf(amax, fmaxf(fabsf(bf16_bits_to_f32(w[i] & 0xffffu)), fabsf(bf16_bits_to_f32(w[i] >> 16))));
+  amax = fmaxf(amax, __shfl_xor(amax, 16));
   const int E = (int)((__float_as_uint(amax) >> 23) & 0xffu);
   const int X = min(max(E - 8, 0), 254);
   const float inv = __uint_as_float((uint32_t)(254 - X) << 23); // 2^(127 - X), X <= 246
-  uint32_t out[8];
+  uint32_t out[4];
 #pragma unroll
-  for (int d = 0; d < 8; d++) {
+  for (int d = 0; d < 4; d++) {
     uint32_t v = 0;
 #pragma unroll
     for (int e = 0; e < 2; e++) {
@@ -311,14 +315,9 @@ quant_act_mxfp8_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K, uin
     }
     out[d] = v;
   }
-  const int64_t mt = m >> 4, kt = kb >> 2;
-  const int lane = (int)((kb & 3) * 16 + (m & 15));
-  // 16-channel chunk c = 2 * (kb & 3) + e of the tile lies in lane group c & 3 of half c >> 2
-  uint4* dst = reinterpret_cast<uint4*>(xq) + ((mt * KT + kt) * 2) * 64 + (m & 15);
-  const int c0 = (int)(kb & 3) * 2;
-  dst[(c0 >> 2) * 64 + (c0 & 3) * 16] = make_uint4(out[0], out[1], out[2], out[3]);
-  dst[((c0 + 1) >> 2) * 64 + ((c0 + 1) & 3) * 16] = make_uint4(out[4], out[5], out[6], out[7]);
-  xs[(((mt >> 2) * KT + kt) * 64 + lane) * 4 + (mt & 3)] = m < M ? (uint8_t)X : (uint8_t)0;
+  reinterpret_cast<uint4*>(xq)[((mt * KT + kt) * 2 + h) * 64 + lane] = make_uint4(out[0], out[1], out[2], out[3]);
+  if ((g & 1) == 0) // block b = h*2 + g/2 of the tile: byte (mt & 3) of lane (b, r)'s word
+    xs[(((mt >> 2) * KT + kt) * 64 + (h * 2 + (g >> 1)) * 16 + r) * 4 + (mt & 3)] = m < M ? (uint8_t)X : (uint8_t)0;
 }
 
 // Activation quantizer: one wave per (row, K block).  Each lane owns
@@ -393,7 +392,7 @@ hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qb
 }
 
 hipError_t launch_quant_act_mxfp8(const void* x, int64_t M, int64_t K, void* xq, void* xs, hipStream_t stream) {
-  const int64_t nthreads = (M + 63) / 64 * 64 * (K / 32);
+  const int64_t nthreads = (M + 63) / 64 * 4 * (K / 128) * 128; // a wave per half tile
   TPPX_PLAN_ONLY(quant_act_mxfp8_kernel, dim3(grid_for(nthreads, 256)), dim3(256), 0);
   quant_act_mxfp8_kernel<<<grid_for(nthreads, 256), 256, 0, stream>>>((const uint16_t*)x, M, K, (uint8_t*)xq, (uint8_t*)xs);
   return hipGetLastError();
