@@ -361,6 +361,25 @@ def test_qint8_fused_quant_shared_lds():
     assert_close_bf16(t2bits(y), ref, what="qint8 M=16 K=8192 N=8448")
 
 
+@pytest.mark.parametrize("M,K", [(128, 512), (200, 11008), (2048, 4096)])
+def test_qint8_activation_quantizer_many_rows_bit_exact(M, K):
+    """From 128 rows on, 256-wide blocks take the quantizer that gives 16 lanes to a (row, block); with zero rows, a
+    row of one value and a huge value in the input, bytes and scales must equal the oracle's."""
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    x = randn_bf16((M, K), 1.0, 41)
+    x[5] = 0.0
+    x[7] = -0.375
+    x[9, 300] = 3.0e38
+    x = x.cuda()
+    xq = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    sa = torch.empty((M, K // 256), dtype=torch.float32, device="cuda")
+    _lib.check(L.tppx_quant_act_int8(x.data_ptr(), M, K, 256, xq.data_ptr(), sa.data_ptr(), _lib.stream_of(x)))
+    xq_or, sa_or = O.quant_act_int8(t2bits(x.cpu()), 256)
+    assert np.array_equal(sa.cpu().numpy(), sa_or)
+    assert np.array_equal(xq.cpu().numpy(), xq_or)
+
+
 @pytest.mark.parametrize("M", [3, 24, 64])
 def test_qint8_prequantized_and_reused_activations(M):
     """x == NULL takes row-major int8 activations + scales (the reference's

@@ -378,12 +378,61 @@ quant_act_int8_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
   }
 }
 
+// Many rows, 256-wide blocks, row-major output (the large-M GEMM's input): 16 lanes per (row, block), 16 values per
+// lane -- 32-byte reads, 16-byte writes, four blocks per wave -- and the maximum taken inside the 16-lane DPP row.
+// Same arithmetic as the kernel above (the maximum does not depend on the order).
+__global__ void __launch_bounds__(256)
+quant_act_int8_rows_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K, int8_t* __restrict__ xq,
+                           float* __restrict__ sa) {
+  const int64_t nb = K >> 8;
+  const int64_t blk = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+  const int l = threadIdx.x & 15;
+  if (blk >= M * nb) // whole DPP rows leave together
+    return;
+  const uint4* src = reinterpret_cast<const uint4*>(x + blk * 256 + l * 16); // (m, b) -> m*K + b*256 = blk*256
+  const uint4 v0 = src[0], v1 = src[1];
+  const uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+  float f[16];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    f[2 * i] = bf16_bits_to_f32(w[i] & 0xffffu);
+    f[2 * i + 1] = bf16_bits_to_f32(w[i] >> 16);
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 16; i++)
+    amax = fmaxf(amax, fabsf(f[i]));
+  auto dpp = [](float v, auto CTRL) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), decltype(CTRL)::value, 0xf, 0xf, true));
+  };
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0xB1>{}));  // quad_perm [1,0,3,2]
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0x4E>{}));  // quad_perm [2,3,0,1]
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0x141>{})); // row_half_mirror
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0x140>{})); // row_mirror
+  const float s = int8_scale_of(amax);
+  const float inv = int8_inv_scale(s);
+  if (l == 0)
+    sa[blk] = s; // [M][nb]
+  uint32_t o[4];
+#pragma unroll
+  for (int d = 0; d < 4; d++)
+    o[d] = (uint32_t)(int8_q(f[4 * d], inv) & 0xff) | ((uint32_t)(int8_q(f[4 * d + 1], inv) & 0xff) << 8) |
+           ((uint32_t)(int8_q(f[4 * d + 2], inv) & 0xff) << 16) | ((uint32_t)(int8_q(f[4 * d + 3], inv) & 0xff) << 24);
+  reinterpret_cast<uint4*>(xq + blk * 256)[l] = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 static inline unsigned grid_for(int64_t n, int block) {
   return (unsigned)((n + block - 1) / block);
 }
 
 hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs, void* xq, void* sa, int mt,
                                  hipStream_t stream) {
+  if (qbs == 256 && mt == 0 && M >= 128) {
+    const int64_t nt16 = M * (K / 256) * 16;
+    TPPX_PLAN_ONLY(quant_act_int8_rows_kernel, dim3(grid_for(nt16, 256)), dim3(256), 0);
+    quant_act_int8_rows_kernel<<<grid_for(nt16, 256), 256, 0, stream>>>((const uint16_t*)x, M, K, (int8_t*)xq, (float*)sa);
+    return hipGetLastError();
+  }
   int64_t nthreads = M * (K / qbs) * 64;
   TPPX_PLAN_ONLY(quant_act_int8_kernel, dim3(grid_for(nthreads, 256)), dim3(256), 0);
   quant_act_int8_kernel<<<grid_for(nthreads, 256), 256, 0, stream>>>((const uint16_t*)x, M, K, qbs, (int8_t*)xq,
