@@ -249,6 +249,22 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     }
     if (!dual)
       return check_hip(launch_tiled_mxfp4_fp8_group(t, n_segs, stream), who);
+    {
+      // gate and up as ONE grid when that fills the last round of workgroups better than two launches and the
+      // workspace has room for the gate tile behind the quantised activations (as in the bf16-activation path below)
+      const int64_t wgs = ((M + 255) / 256) * ((t[0].tiles + 15) / 16);
+      const bool fewer_rounds = (2 * wgs + 255) / 256 < 2 * ((wgs + 255) / 256);
+      const int64_t park = (need + 255) / 256 * 256;
+      if (fewer_rounds && ws_bytes >= park + M * (int64_t)t[0].N * 2 && env_int("TPPX_TILED_DUAL_GROUP", 1) != 0) {
+        uint16_t* gate = (uint16_t*)((uint8_t*)ws + park);
+        t[0].y = gate;
+        t[0].post_op = t[1].post_op = TPPX_POST_NONE;
+        rc = check_hip(launch_tiled_mxfp4_fp8_group(t, 2, stream), who);
+        if (rc)
+          return rc;
+        return check_hip(launch_silu_mul(gate, (uint16_t*)segs[1].y, M * (int64_t)t[0].N, stream), who);
+      }
+    }
     t[0].post_op = TPPX_POST_SILU; // silu(gate), then up * that: the rounding points of the two-GEMM form
     t[1].post_op = TPPX_POST_MUL;
     t[1].post_in = (const uint16_t*)segs[0].y;

@@ -594,6 +594,12 @@ def swiglu_gate_up(input, w_gate, w_up, b_gate=None, b_up=None, norm=None):
     if not fl and M > 64 and M * N * 2 > ws.numel():
         # prefill: room for the gate tile lets the library run gate and up as one grid (fuller last round)
         ws = torch.empty(M * N * 2, dtype=torch.uint8, device=x.device)
+    elif fl & _lib.FLAG_ACT_FP8:
+        # the same behind the quantised activations
+        Mp = (M + 63) // 64 * 64
+        need = (Mp * K + Mp * (K // 32) + 255) // 256 * 256 + M * N * 2
+        if need > ws.numel():
+            ws = torch.empty(need, dtype=torch.uint8, device=x.device)
     _lib.check(L.tppx_swiglu_mxfp4(x.data_ptr(), qg.data_ptr(), sg.data_ptr(), _lib.ptr(bg), qu.data_ptr(),
                                    su.data_ptr(), _lib.ptr(bu), y.data_ptr(), M, N, K, fl, ws.data_ptr(),
                                    ws.numel(), _lib.stream_of(x)))
