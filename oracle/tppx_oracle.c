@@ -352,8 +352,10 @@ ORC_API void orc_remap_quantize_mxfp4(const float* W, int64_t N, int64_t K,
       for (int h = 0; h < 2; h++)
         for (int k2 = 0; k2 < 32; k2++) {
           const float* row = W + (nk * 32 + k2) * K + nc * 64 + h * 32;
-          float amax = 0.0f;
-          for (int j = 0; j < 32; j++) {
+          /* max = |first|, then std::max(max, |v|) (qtypes.h:156-162): a NaN in the
+           * first slot stays (byte 255), a NaN anywhere else never wins */
+          float amax = fabsf(row[0]);
+          for (int j = 1; j < 32; j++) {
             float a = fabsf(row[j]);
             amax = a > amax ? a : amax;
           }

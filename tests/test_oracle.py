@@ -158,6 +158,26 @@ def test_layout_closed_form_equals_view_permute_chain(shape):
     assert np.array_equal(q3, q4) and np.array_equal(s3, s4)
 
 
+def test_mx_block_maximum_nan_rule():
+    """PerBlockQuantizer::quantize_symetric (qtypes.h:156-162) starts its maximum at |first element| and updates with
+    std::max(max, |v|): a NaN in the first slot of a block stays (shared exponent 255 -> scale byte 255, every
+    code 0), a NaN in any other slot never wins the comparison (the block keeps the scale of its finite maximum;
+    the NaN element itself encodes as 0).  The closed-form restatement must agree with the restatement of the
+    reference's own view / permute / generic-quantizer chain on both, and Inf always wins."""
+    W = np.full((32, 64), 0.5, np.float32)
+    W[3, 0] = np.nan        # first slot of block (row 3, half 0)
+    W[4, 33] = np.nan       # second slot of block (row 4, half 1)
+    W[5, 32 + 7] = np.inf
+    W[6, 0] = -np.inf
+    q1, s1 = O.remap_and_quantize_mxfp4_blocked(O.block_weight(W, 16, 64, 1))
+    q2, s2 = O.remap_quantize_mxfp4(W)
+    assert np.array_equal(q1, q2) and np.array_equal(s1, s2)
+    sc = s2[0, 0]  # [h][k2]
+    assert sc[0, 3] == 255 and sc[1, 4] == 124 and sc[1, 5] == 255 and sc[0, 6] == 255 and sc[0, 0] == 124
+    deq = O.dequantize_mxfp4_plain(q2, s2)
+    assert deq[4, 33] == 0.0 and deq[4, 34] == 0.5 and deq[0, 0] == 0.5
+
+
 def test_layout_brute_force_index_formula():
     N, K = 32, 64
     W = np.arange(N * K, dtype=np.float32).reshape(N, K) % 13 - 6.0

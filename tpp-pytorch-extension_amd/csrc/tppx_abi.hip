@@ -6,7 +6,10 @@
 #include <string.h>
 
 #include <cxxabi.h>
+#include <map>
+#include <mutex>
 #include <string>
+#include <utility>
 
 #include "tppx_common.h"
 #include "tppx_launch.h"
@@ -54,6 +57,28 @@ void plan_note(const void* kernel_fn, dim3 grid, dim3 block, size_t lds_bytes) {
   snprintf(line, sizeof(line), "%s grid=%ux%ux%u block=%u lds=%zu\n", name.c_str(), grid.x, grid.y, grid.z, block.x,
            lds_bytes);
   *g_plan += line;
+}
+
+// Raises the dynamic-LDS limit of `kern` on the current device once per (device, kernel, size) instead of on
+// every launch; the record is per device because the attribute is.
+hipError_t allow_dynamic_lds(const void* kern, size_t lds) {
+  if (lds <= 48 * 1024)
+    return hipSuccess;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return e;
+  static std::mutex mu;
+  static std::map<std::pair<int, const void*>, size_t> allowed;
+  std::lock_guard<std::mutex> lock(mu);
+  size_t& have = allowed[{dev, kern}];
+  if (lds > have) {
+    e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess)
+      return e;
+    have = lds;
+  }
+  return hipSuccess;
 }
 
 int env_int(const char* name, int dflt) {

@@ -88,6 +88,8 @@ hipError_t launch_tiled_qint8_group(const TiledParams* t, int n, hipStream_t str
 hipError_t launch_silu_mul(const uint16_t* gate, uint16_t* y, int64_t n, hipStream_t stream);
 
 int env_int(const char* name, int dflt);
+// dynamic LDS above 48 KiB must be allowed per kernel and device before the launch
+hipError_t allow_dynamic_lds(const void* kern, size_t lds);
 
 // dynamic activation quantisation; mt > 0 writes xq in MFMA operand order (see DecodeParams::mt)
 hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs, void* xq, void* sa, int mt,

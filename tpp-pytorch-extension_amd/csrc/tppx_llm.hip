@@ -145,7 +145,7 @@ rotary_append_kernel(const RotaryParams p) {
   const int coff = p.HR >> 1;
   const int h0 = c * 8;
   const int64_t pp = p.pos[(int64_t)(p.B_pos == 1 ? 0 : b) * p.S + s];
-  if (p.emb && h0 < p.HR && pp < p.MP) {
+  if (p.emb && h0 < p.HR && pp >= 0 && pp < p.MP) { // positions outside the table are left unrotated
     // this chunk holds first halves (h0 < HR/2) or second halves of rotation pairs
     const bool first = h0 < coff;
     const int h2 = first ? h0 : h0 - coff;
@@ -236,7 +236,7 @@ attn_decode_kernel(const AttnParams p) {
     // chunk c holds first halves (c < 8) or second halves of the rotation pairs (h2, 64 + h2); partner chunk c ^ 8
     const bool first = c < 8;
     const int64_t pp = p.pos[p.B_pos == 1 ? 0 : b];
-    const bool rot = p.emb != nullptr && pp < p.MP;
+    const bool rot = p.emb != nullptr && pp >= 0 && pp < p.MP;
     float cs[8], sn[8];
 #pragma unroll
     for (int e = 0; e < 8; e++)
@@ -398,9 +398,11 @@ attn_decode_kernel(const AttnParams p) {
   if (p.splits == 1 || p.ticket0 < 0)
     return;
   // The split that arrives last merges all of them, in split order (the same sums whichever split that is).
-  // Order: the stores above are complete at the barrier (it waits for outstanding memory operations), then the
-  // ticket, then the device-scope loads of the other splits' results.  Nobody waits for anybody.
+  // Order: every thread waits until its own stores above have been acknowledged (vmcnt counts stores on this
+  // target; a workgroup barrier by itself does not wait for the global stores of the other waves), then the
+  // barrier, then the ticket, then the device-scope loads of the other splits' results.  Nobody waits for anybody.
   __shared__ int arrived_last;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (tid == 0) {
     const unsigned int last = (unsigned int)p.splits - 1;

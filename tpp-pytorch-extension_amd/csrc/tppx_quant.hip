@@ -63,10 +63,14 @@ quantize_mxfp4_kernel(const T* __restrict__ w, int64_t N, int64_t K, int64_t bk,
   int64_t nc = rest % Nc, nk = rest / Nc;
   int64_t n = nk * 32 + k2, k0 = nc * 64 + h * 32;
   float v[32];
-  float amax = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 32; j++) {
+  for (int j = 0; j < 32; j++)
     v[j] = load_as_f32<T>(w, blocked_off(n, k0 + j, K, bk, bc, vnni));
+  // max = |first|, then std::max(max, |v|) as the CPU path has it: a NaN in the first slot stays (scale byte 255),
+  // a NaN anywhere else never wins the comparison
+  float amax = fabsf(v[0]);
+#pragma unroll
+  for (int j = 1; j < 32; j++) {
     float a = fabsf(v[j]);
     amax = a > amax ? a : amax;
   }

@@ -22,7 +22,6 @@
 //   lane l supplies row/col (l & 15) and K group (l >> 4);
 //   result register r of lane l is D[m = (l >> 4) * 4 + r][n = l & 15].
 #include <mutex>
-#include <unordered_map>
 
 #include "tppx_common.h"
 #include "tppx_launch.h"
@@ -175,8 +174,11 @@ struct SkEpilogue {
     }
     // The sums travel as device-scope atomic stores and loads (written through to, and read from, the level all
     // XCDs share), so no cache write-back or invalidate is needed: a device-wide fence here costs more than the
-    // whole kernel (measured: +8 us with one fencing thread per workgroup, +40 us with all).  Order: the stores are
-    // complete at the barrier (it waits for outstanding memory operations), then the ticket, then the loads.
+    // whole kernel (measured: +8 us with one fencing thread per workgroup, +40 us with all).  Order: every thread
+    // waits until its own stores have been acknowledged (vmcnt counts stores on this target, and a workgroup
+    // barrier by itself does NOT wait for the global stores of the other waves), then the barrier, then the
+    // ticket, then the loads.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
       const unsigned int last = (unsigned int)p.S - 1;
@@ -1448,21 +1450,8 @@ int skinny_split_tickets(int n) {
 template <typename K>
 static hipError_t sk_launch(K kern, const DecodeParams& p, dim3 grid, int waves, size_t lds, hipStream_t stream) {
   TPPX_PLAN_ONLY(kern, grid, dim3(64 * waves), lds);
-  // raise the dynamic-LDS limit of a kernel once per size instead of on every launch (all kernels here share one
-  // function type, so the record is keyed by the kernel's address)
-  if (lds > 48 * 1024) {
-    static std::mutex mu;
-    static std::unordered_map<const void*, size_t> allowed;
-    std::lock_guard<std::mutex> lock(mu);
-    size_t& have = allowed[reinterpret_cast<const void*>(kern)];
-    if (lds > have) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess)
-        return e;
-      have = lds;
-    }
-  }
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds); e != hipSuccess)
+    return e;
   kern<<<grid, dim3(64 * waves), lds, stream>>>(p);
   return hipGetLastError();
 }

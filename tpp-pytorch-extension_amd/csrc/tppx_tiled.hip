@@ -997,22 +997,15 @@ hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t str
   const int env_mt = env_int("TPPX_TILED_BIG_MT", 0);
   if (env_mt == 4 || env_mt == 8)
     mt = env_mt;
-  static bool big_attr_done = false;
-  if (!big_attr_done) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_mxfp4_kernel<8>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_mxfp4_kernel<4>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess)
-      return e;
-    big_attr_done = true;
-  }
   if (mt == 4) {
     TPPX_PLAN_ONLY(big_mxfp4_kernel<4>, dim3(MB4 * nb), dim3(512), lds);
+    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_mxfp4_kernel<4>), lds); e != hipSuccess)
+      return e;
     big_mxfp4_kernel<4><<<dim3(MB4 * nb), dim3(512), lds, stream>>>(P);
   } else {
     TPPX_PLAN_ONLY(big_mxfp4_kernel<8>, dim3(MB8 * nb), dim3(512), lds);
+    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_mxfp4_kernel<8>), lds); e != hipSuccess)
+      return e;
     big_mxfp4_kernel<8><<<dim3(MB8 * nb), dim3(512), lds, stream>>>(P);
   }
   return hipGetLastError();
@@ -1042,22 +1035,15 @@ hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t
   const int env_mt = env_int("TPPX_FP8_BIG_MT", 0);
   if (env_mt == 4 || env_mt == 8)
     mt = env_mt;
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_fp8_kernel<8>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds8);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_fp8_kernel<4>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds4);
-    if (e != hipSuccess)
-      return e;
-    attr_done = true;
-  }
   if (mt == 4) {
     TPPX_PLAN_ONLY(big_fp8_kernel<4>, dim3(MB4 * nb), dim3(512), lds4);
+    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_fp8_kernel<4>), lds4); e != hipSuccess)
+      return e;
     big_fp8_kernel<4><<<dim3(MB4 * nb), dim3(512), lds4, stream>>>(P);
   } else {
     TPPX_PLAN_ONLY(big_fp8_kernel<8>, dim3(MB8 * nb), dim3(512), lds8);
+    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_fp8_kernel<8>), lds8); e != hipSuccess)
+      return e;
     big_fp8_kernel<8><<<dim3(MB8 * nb), dim3(512), lds8, stream>>>(P);
   }
   return hipGetLastError();
@@ -1069,14 +1055,8 @@ hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream) {
   const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
   const size_t lds = 2 * 2048 * 16;
   TPPX_PLAN_ONLY(tiled_mxfp4_kernel, dim3(MB * NB), dim3(256), lds);
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_mxfp4_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess)
-      return e;
-    attr_done = true;
-  }
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(tiled_mxfp4_kernel), lds); e != hipSuccess)
+    return e;
   tiled_mxfp4_kernel<<<dim3(MB * NB), dim3(256), lds, stream>>>(p);
   return hipGetLastError();
 }
@@ -1132,14 +1112,8 @@ hipError_t launch_tiled_qint8_group(const TiledParams* t, int n, hipStream_t str
     const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the A and B buffers + the scale slots
     static_assert(8 * 64 * EP_LD * sizeof(float) >= 2 * 128 * 256 + 64 * 1024 + 4 * 128 * sizeof(float), "LDS plan");
     TPPX_PLAN_ONLY(big_qint8_kernel, dim3(MB4 * NB16), dim3(512), lds);
-    static bool attr_done = false;
-    if (!attr_done) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(big_qint8_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess)
-        return e;
-      attr_done = true;
-    }
+    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_qint8_kernel), lds); e != hipSuccess)
+      return e;
     big_qint8_kernel<<<dim3(MB4 * NB16), dim3(512), lds, stream>>>(P);
     return hipGetLastError();
   }
