@@ -207,6 +207,21 @@ int tppx_linear_qint8(const void* x, void* xq, void* sa, const void* qw,
                       int flags, void* ws, int64_t ws_bytes,
                       tppx_stream_t stream);
 
+/* No counterpart in the reference.  tppx_linear_qint8 for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the quantised activations, their
+ * scales and the K-split workspace live in a static device array of the library (about 4.1 MiB per GPU, held
+ * until the process ends) instead of caller buffers.  x must be given (bf16 [M][K]); limits: M <= 64 (decode
+ * shapes), K <= 32768 -- larger sizes return TPPX_ESHAPE; flags: 0 or TPPX_FLAG_FORCE_SKINNY.  Same kernels and
+ * the same bits as tppx_linear_qint8 with a 2 MiB workspace.  The call itself allocates nothing and frees nothing.
+ * All calls on one GPU share the one array: calls that overlap on a GPU (different streams without ordering)
+ * race; order them on one stream or with events.  Nothing in the array has to start at zero (every byte read was
+ * written earlier in the same call). */
+int tppx_linear_qint8_noalloc(const void* x, const void* qw, const void* sw,
+                              const void* bias, const void* post_in,
+                              const void* post_in2, void* y, int64_t M,
+                              int64_t N, int64_t K, int64_t qbs, int post_op,
+                              float post_scale, int flags, tppx_stream_t stream);
+
 /* One GEMM of a fused group sharing the activation. */
 typedef struct tppx_seg {
   const void* qw;       /* native weight */

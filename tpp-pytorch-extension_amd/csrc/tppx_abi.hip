@@ -624,6 +624,66 @@ extern "C" int tppx_multi_linear_qint8(const void* x, void* xq, void* sa,
   return run_qint8("tppx_multi_linear_qint8", x, xq, sa, segs, n_segs, M, K, qbs, flags, ws, ws_bytes, (hipStream_t)stream);
 }
 
+// ---- the entry point that allocates nothing ----------------------------------
+// Everything tppx_linear_qint8 takes from the caller as scratch -- the quantised activations xq, their scales sa and
+// the K-split workspace -- lives in one file-scope device array instead.  The array's name is only a host-side
+// handle: its device address is looked up once per device (hipGetSymbolAddress with that device current) and only
+// that address is ever handed to kernels.
+constexpr int64_t NA_MAX_M = 64, NA_MAX_K = 32768;
+constexpr size_t NA_XQ_BYTES = (size_t)NA_MAX_M * NA_MAX_K;                        // int8 rows, 2 MiB
+constexpr size_t NA_SA_BYTES = (size_t)NA_MAX_M * (NA_MAX_K / 64) * sizeof(float); // one scale per 64 channels at most
+constexpr size_t NA_WS_BYTES = (size_t)2 * 256 * 4 * 256 * sizeof(float);          // 2 K parts x 256 tiles x 64 rows
+static __device__ __align__(256) unsigned char scratch[NA_XQ_BYTES + NA_SA_BYTES + NA_WS_BYTES];
+
+static int scratch_of_current_device(const char* who, unsigned char** out) {
+  static std::mutex mu;
+  static std::map<int, unsigned char*> per_device;
+  int dev = 0;
+  int rc = check_hip(hipGetDevice(&dev), who);
+  if (rc)
+    return rc;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = per_device.find(dev);
+  if (it == per_device.end()) {
+    void* ptr = nullptr;
+    rc = check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), who);
+    if (rc)
+      return rc;
+    TPPX_REQUIRE(ptr && (reinterpret_cast<uintptr_t>(ptr) & 255u) == 0, TPPX_EHIP, "%s: bad address of the static scratch", who);
+    it = per_device.emplace(dev, (unsigned char*)ptr).first;
+  }
+  *out = it->second;
+  return TPPX_OK;
+}
+
+extern "C" int tppx_linear_qint8_noalloc(const void* x, const void* qw, const void* sw, const void* bias,
+                                         const void* post_in, const void* post_in2, void* y, int64_t M, int64_t N,
+                                         int64_t K, int64_t qbs, int post_op, float post_scale, int flags,
+                                         tppx_stream_t stream) {
+  const char* who = "tppx_linear_qint8_noalloc";
+  TPPX_REQUIRE(x, TPPX_EINVAL, "%s: null activation pointer (pre-quantized input needs no scratch: call tppx_linear_qint8)", who);
+  TPPX_REQUIRE(M > 0 && M <= NA_MAX_M, TPPX_ESHAPE, "%s: M=%ld outside 1..%ld (the static scratch holds %ld quantised rows)", who, (long)M, (long)NA_MAX_M, (long)NA_MAX_M);
+  TPPX_REQUIRE(K > 0 && K <= NA_MAX_K, TPPX_ESHAPE, "%s: K=%ld outside 1..%ld (the static scratch holds rows of %ld channels)", who, (long)K, (long)NA_MAX_K, (long)NA_MAX_K);
+  TPPX_REQUIRE((flags & ~TPPX_FLAG_FORCE_SKINNY) == 0, TPPX_EINVAL, "%s: only TPPX_FLAG_FORCE_SKINNY is accepted here (flags 0x%x)", who, flags);
+  // the remaining checks of tppx_linear_qint8, before the first HIP call, on placeholder scratch addresses
+  void* a = reinterpret_cast<void*>(uintptr_t(1) << 20);
+  tppx_seg s = {qw, sw, bias, post_in, post_in2, y, N, post_op, post_scale};
+  {
+    std::string text;
+    g_plan = &text;
+    const int rc = run_qint8(who, x, a, a, &s, 1, M, K, qbs, flags, a, (int64_t)NA_WS_BYTES, nullptr);
+    g_plan = nullptr;
+    if (rc)
+      return rc;
+  }
+  unsigned char* base = nullptr;
+  int rc = scratch_of_current_device(who, &base);
+  if (rc)
+    return rc;
+  return run_qint8(who, x, base, base + NA_XQ_BYTES, &s, 1, M, K, qbs, flags, base + NA_XQ_BYTES + NA_SA_BYTES,
+                   (int64_t)NA_WS_BYTES, (hipStream_t)stream);
+}
+
 // ---- launch plans -----------------------------------------------------------
 static int emit_plan(const char* who, int rc, std::string& text, char* buf, int64_t buf_len) {
   g_plan = nullptr;

@@ -58,6 +58,7 @@ SIGNATURES = {
     "tppx_linear_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _f32, _i32, _vp, _i64, _vp],
     "tppx_linear_qint8": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _f32, _i32,
                           _vp, _i64, _vp],
+    "tppx_linear_qint8_noalloc": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _f32, _i32, _vp],
     "tppx_multi_linear_mxfp4": [_vp, ctypes.POINTER(Seg), _i32, _i64, _i64, _i32, _vp, _i64, _vp],
     "tppx_multi_linear_qint8": [_vp, _vp, _vp, ctypes.POINTER(Seg), _i32, _i64, _i64, _i64, _i32, _vp, _i64, _vp],
     "tppx_swiglu_mxfp4": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp],
