@@ -1,18 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the weight-quantized linear path on one MI355X.
 
-Default workload (the configuration the metric is quoted on): QINT8 W8A8
-`fc_add` at the Llama-7B MLP shapes -- up-projection 4096 -> 11008 and
-down-projection 11008 -> 4096 -- for M in {1, 8, 32, 64}; one "step" is one
-pass over those 8 fused linears.  Inputs are resident in HBM before the timed
-region; weights cycle through a pool larger than the 256 MB Infinity Cache so
-that every launch streams its weight from HBM.
-
-Prints ONE JSON line: whole-job HBM throughput (algorithmic bytes / wall time),
-the roofline of the dominant kernel (timed with events on the launch stream)
-and the CPU restatement of the reference path timed on the host cores.
+`python bench.py --gpus 1` prints ONE JSON line.  Its headline (`metric`, `value`, `roofline`, `cpu_baseline`) is the
+configuration the metric is quoted on: QINT8 W8A8 `fc_add` at the Llama-7B MLP shapes -- up-projection 4096 -> 11008
+and down-projection 11008 -> 4096 -- for M in {1, 8, 32, 64}; one "step" is one pass over those 8 fused linears.
+`config.legs` carries the other legs of the metric, each with its own roofline (kernel named by the library's launch
+plan, timed with events on the launch stream) and, where the oracle finishes a sample in seconds, its own CPU
+baseline:
+  cfg1  MXFP4 fc_plain, M = 16, 4096 x 4096, bias                              (HBM TB/s)
+  cfg3  MXFP4 SwiGLU MLP block 4096 -> 11008 -> 4096, M in {1, 4, 16, 64}      (HBM TB/s)
+  cfg4  MXFP4 linears of one 70B-shape decoder layer at M = 2048               (TFLOP/s; also the same layer in
+        QINT8 and with the opt-in MXFP8 activations, labelled)
+  cfg5  32-layer 7B-shape decoder, greedy decode, batch 1 and 16               (tokens/s)
+Inputs are resident in HBM before every timed region; weights cycle through pools larger than the 256 MB Infinity
+Cache so that every decode-shape launch streams its weight from HBM.  Every leg is timed for at least half a second
+of wall time.  `--workload` runs one leg alone (the form the profiles under profiles/ were taken in).
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -22,11 +27,15 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "tpp-pytorch-extension_amd"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E published peak
+PEAKS_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "fp4": 10100.0}
+MIN_WALL_S = 0.5       # every leg is timed for at least this long
 # BASELINE config 2 (the configuration the headline metric is quoted on); tests/ import these so that the shapes the
 # parity tests run are the shapes timed here
 CFG2_SHAPES = {"up": (11008, 4096), "down": (4096, 11008)}  # name -> (N, K)
 CFG2_MS = [1, 8, 32, 64]
-PEAKS_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "fp4": 10100.0}
+CFG3_MS = [1, 4, 16, 64]
+CFG3_DIMS = (4096, 11008)        # hidden, intermediate
+CFG4_DIMS = (2048, 8192, 28672)  # M, hidden, intermediate; q/k/v widths 8192 + 1024 + 1024
 
 
 def algorithmic_bytes(fmt, M, N, K, qbs=256, bias=False, post_in=True):
@@ -53,51 +62,124 @@ def block_bf16(W):
     return W.view(N // 16, 16, K // 64, 32, 2).permute(0, 2, 3, 1, 4).contiguous()
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--fmt", default="qint8", choices=["qint8", "mxfp4"])
-    ap.add_argument("--batch", type=int, default=1, help="sequences for --workload tokens (1 or 16 in the baseline)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "tokens", "prompt"],
-                    help="decode = the configuration the headline metric is quoted on (default); prefill = the "
-                         "MXFP4 linears of one 70B-shape decoder layer at M = 2048 (TFLOP/s, MFMA roofline); tokens = "
-                         "7B-shape greedy decode; prompt = a 2048-token prompt through the same 7B-shape decoder")
-    ap.add_argument("--prefill-fmt", default="mxfp4", choices=["mxfp4", "qint8"],
-                    help="weight format of --workload prefill (BASELINE config 4 is MXFP4; qint8 = the same layer W8A8)")
-    ap.add_argument("--act-fp8", action="store_true",
-                    help="--workload prefill, MXFP4: quantise activations to MXFP8 and use the block-scaled MFMA "
-                         "(opt-in; not the reference's arithmetic, whose activations stay bf16)")
-    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--pool", type=int, default=2, help="number of distinct weight sets cycled through")
-    ap.add_argument("--pmc-calibrate", action="store_true",
-                    help="also run three plain 256 MiB device copies, the known-size reference for scaling "
-                         "FETCH_SIZE / WRITE_SIZE counter readings")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU; --gpus must be 1 (every box has one GPU and the "
-              "path has no collectives)", file=sys.stderr)
-        sys.exit(2)
+def clone_weight(q):
+    """A second copy of a quantized weight's native tiles (so that launches stream distinct bytes)."""
+    c = q._clone_with(q.qdata, q.scales)
+    c._native = tuple(t.clone() for t in q.native())
+    return c
 
+
+def time_blocks(torch, run_step, steps, warmup, min_wall=MIN_WALL_S):
+    """`warmup` untimed steps, then blocks of EXACTLY `steps` steps, each bracketed by a synchronize on both sides,
+    until the blocks add up to `min_wall` seconds: (mean ms per step over all blocks, number of blocks)."""
+    for i in range(warmup):
+        run_step(i)
+    torch.cuda.synchronize()
+    total, blocks, i = 0.0, 0, warmup
+    while True:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            run_step(i)
+            i += 1
+        torch.cuda.synchronize()
+        total += time.perf_counter() - t0
+        blocks += 1
+        if total >= min_wall or blocks >= 20000:
+            break
+    return total * 1e3 / (steps * blocks), blocks
+
+
+def events_us(torch, fire, launches_per_fire, min_wall=0.15, use_graph=True):
+    """Mean duration (us) of one launch group: `fire(stream)` enqueues `launches_per_fire` of them on the stream it is
+    given; timed between two events on that stream around graph replays (or eager calls) for >= min_wall seconds."""
+    g = None
+    if use_graph:
+        try:
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                fire(torch.cuda.current_stream().cuda_stream)
+        except Exception:
+            g = None
+    go = (lambda: g.replay()) if g is not None else (lambda: fire(torch.cuda.current_stream().cuda_stream))
+    for _ in range(2):
+        go()
+    torch.cuda.synchronize()
+    total_ms, n = 0.0, 0
+    reps = 4
+    while total_ms < min_wall * 1e3 and n < 100000:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            go()
+        e1.record()
+        torch.cuda.synchronize()
+        total_ms += e0.elapsed_time(e1)
+        n += reps
+        reps = min(reps * 2, 256)
+    return total_ms * 1e3 / (n * launches_per_fire), n * launches_per_fire
+
+
+def plan_lines(text):
+    out = []
+    for line in text.strip().splitlines():
+        name, _, shape = line.partition(" grid=")
+        out.append((name.replace("void ", ""), "grid=" + shape))
+    return out
+
+
+def kernel_plan(L, fmt, M, N, K, qbs, flags, ws_bytes):
+    """Kernels one linear call enqueues, as the library itself reports them:
+    [(profiler name, launch shape text), ...]; the last one is the GEMM."""
+    buf = ctypes.create_string_buffer(4096)
+    if fmt == "qint8":
+        rc = L.tppx_plan_linear_qint8(M, N, K, qbs, 1, flags, ws_bytes, buf, len(buf))
+    else:
+        rc = L.tppx_plan_linear_mxfp4(M, N, K, flags, ws_bytes, buf, len(buf))
+    return plan_lines(buf.value.decode()) if rc == 0 else []
+
+
+def group_plan(L, fmt, Ns, M, K, dual, flags, ws_bytes, qbs=256):
+    """The same for a fused group (q/k/v) or, dual = 1, the gate/up pair."""
+    buf = ctypes.create_string_buffer(4096)
+    arr = (ctypes.c_int64 * len(Ns))(*Ns)
+    if fmt == "qint8":
+        rc = L.tppx_plan_multi_linear_qint8(arr, len(Ns), M, K, qbs, 1, flags, ws_bytes, buf, len(buf))
+    else:
+        rc = L.tppx_plan_multi_linear_mxfp4(arr, len(Ns), M, K, dual, flags, ws_bytes, buf, len(buf))
+    return plan_lines(buf.value.decode()) if rc == 0 else []
+
+
+def oracle_mod():
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle as O
+    cores = len(os.sched_getaffinity(0))
+    cores = min(cores, O.num_threads()) if O.num_threads() > 0 else cores
+    O.set_num_threads(cores)
+    return O, cores
+
+
+def repeat_for(fn, seconds, max_n=400):
+    fn()  # warm-up
+    n, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt > seconds or n >= max_n:
+            return n, dt
+
+
+def t_bits(t):
+    import numpy as np
     import torch
-    import tpp_pytorch_extension  # noqa: F401
-    from tpp_pytorch_extension import _ops
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(3)
+
+# ---------------------------------------------------------------------------------------------------------------
+# config 2 (headline)
+# ---------------------------------------------------------------------------------------------------------------
+def run_decode(torch, _ops, args):
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-
-    if args.workload == "prefill":
-        return run_prefill(torch, _ops, args)
-    if args.workload == "tokens":
-        return run_tokens(torch, args)
-    if args.workload == "prompt":
-        return run_prompt(torch, args)
-
     fmt = args.fmt
     shapes = dict(CFG2_SHAPES)
     Ms = list(CFG2_MS)
@@ -114,9 +196,7 @@ def main():
             base = quant(block_bf16(W[name]).to(dev))
             base.native()
             for M in Ms:
-                q = base._clone_with(base.qdata, base.scales)
-                q._native = tuple(t.clone() for t in base._native)
-                ws[(name, M)] = q
+                ws[(name, M)] = clone_weight(base)
         pool.append(ws)
     Xd = {k: v.to(dev) for k, v in X.items()}
     Rd = {k: v.to(dev) for k, v in R.items()}
@@ -165,26 +245,12 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for i in range(args.warmup):
-        run_step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        run_step(i)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ms_per_step, blocks = time_blocks(torch, run_step, args.steps, args.warmup)
     value_tbs = bytes_per_step / (ms_per_step * 1e-3) / 1e12
 
-    # ---- roofline leg: the GEMM kernel alone, events on the launch stream ----
-    roof = roofline_leg(torch, _ops, fmt, pool, Xd, Rd, Ms, shapes, qbs, args)
-
-    # ---- CPU baseline: the oracle (port of the reference recipe) -------------
-    cpu = None
-    if not args.no_cpu:
-        cpu = cpu_baseline(fmt, W, X, R, Ms, shapes, qbs, bytes_per_step)
-
-    out = {
+    roof = roofline_decode(torch, fmt, pool, Xd, Rd, Ms, shapes, qbs, args)
+    cpu = None if args.no_cpu else cpu_baseline_decode(fmt, W, X, R, Ms, shapes, qbs, bytes_per_step)
+    return {
         "metric": "quant-GEMM HBM TB/s (decode)",
         "value": round(value_tbs, 4),
         "unit": "TB/s",
@@ -201,6 +267,8 @@ def main():
             "workload": ("cfg2: QINT8 W8A8 (QBS=256) fc_add" if fmt == "qint8" else "MXFP4 fc_add")
             + ", Llama-7B MLP up 4096->11008 + down 11008->4096, M in {1,8,32,64}; one step = these 8 fused linears",
             "launch": "hipGraph replay of one step" if graphs is not None else "eager launches",
+            "timed": f"{blocks} blocks of exactly {args.steps} steps, each between two synchronizes (>= {MIN_WALL_S} s in "
+                     f"all); ms_per_step is their mean",
             "weight_pool_MB": round(len(pool) * len(Ms) * sum(algorithmic_bytes(fmt, 0, N, K, qbs, post_in=False)
                                                               for (N, K) in shapes.values()) / 1e6, 1),
             "bytes_per_step": bytes_per_step,
@@ -209,219 +277,15 @@ def main():
         "roofline": roof,
         "cpu_baseline": cpu,
     }
-    print(json.dumps(out))
 
 
-def run_tokens(torch, args):
-    """BASELINE config 5: 32-layer Llama-2-7B-shape decoder, all linears (and the lm_head) MXFP4, KV cache
-    pre-filled with 2048 positions of N(0,1), greedy decode of 128 new tokens for `--batch` sequences from
-    random token ids; the decode step is one replayed HIP graph."""
-    from tpp_pytorch_extension.llm import fused_llama_infer as F
-    dev = torch.device("cuda:0")
-    B, ctx, new = args.batch, 2048, 128
-    model = F.LlamaDecoder(hidden=4096, inter=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab=32000,
-                           max_positions=4096, weight_dtype="mxfp4", seed=1239)
-    tok = torch.randint(0, 32000, (B,), generator=torch.Generator().manual_seed(5), dtype=torch.int64).to(dev)
-    model.greedy_decode(tok, model.new_cache(B, ctx, ctx + new + 32), 8)  # warm-up run
-    cache = model.new_cache(B, ctx, ctx + new + 32)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    out = model.greedy_decode(tok, cache, new)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    # the replays alone (capture and warm-up step excluded)
-    cache2 = model.new_cache(B, ctx, ctx + new + 32)
-    steps_t = model.time_decode_steps(tok, cache2, new)
-    ms = steps_t * 1e3 / new
-    lin_bytes = 32 * (3 * 4096 * 4096 + 4096 * 4096 + 3 * 11008 * 4096) * (0.5 + 1.0 / 32) + 32000 * 4096 * (0.5 + 1.0 / 32)
-    kv_bytes = B * 32 * 2 * 32 * (ctx + new / 2) * 128 * 2
-    achieved = (lin_bytes + kv_bytes) / (ms * 1e-3) / 1e9
-    print(json.dumps({
-        "metric": "7B-shape decode tokens/s", "value": round(B * new / steps_t, 1), "unit": "tokens/s", "n_gpus": 1,
-        "steps": new, "warmup": 8, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"cfg5: 32-layer Llama-2-7B-shape decoder, MXFP4 linears and lm_head, bf16 RMSNorm / rotary / "
-                               f"KV cache, context {ctx} of N(0,1), greedy decode of {new} tokens, batch {B}",
-                   "launch": "one HIP graph per decode step, replayed", "batch": B,
-                   "wall_s_including_capture": round(dt, 4), "tokens": int(out.numel())},
-        "roofline": {"bound": "hbm", "kernel": "whole decode step (all kernels of the graph)", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "bytes_per_step": int(lin_bytes + kv_bytes)},
-        "cpu_baseline": None}))
-
-
-def run_prompt(torch, args):
-    """Prompt processing on the 7B-shape decoder of config 5: `--batch` sequences of 2048 random token ids through
-    the 32 layers in one pass (MXFP4 linears on the large-M kernels, causal attention, keys appended to an empty
-    cache), then the lm_head on the last position.  Not a BASELINE configuration; reported as prompt tokens/s."""
-    from tpp_pytorch_extension.llm import fused_llama_infer as F
-    dev = torch.device("cuda:0")
-    B, S = args.batch, 2048
-    model = F.LlamaDecoder(hidden=4096, inter=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab=32000,
-                           max_positions=4096, weight_dtype="mxfp4", seed=1239)
-    prompt = torch.randint(0, 32000, (B, S), generator=torch.Generator().manual_seed(6), dtype=torch.int64).to(dev)
-    steps, warmup = max(2, min(args.steps, 8)), max(1, min(args.warmup, 2))
-    caches = [F.TppCache(S + 32) for _ in range(steps + warmup)]
-    for c in caches[:warmup]:
-        model.prefill(prompt, c)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for c in caches[warmup:]:
-        model.prefill(prompt, c)
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / steps
-    lin_flops = 2.0 * B * S * 32 * (4 * 4096 * 4096 + 3 * 11008 * 4096) + 2.0 * B * 32000 * 4096
-    attn_flops = 32 * 4.0 * B * 32 * 128 * (S * (S + 1) / 2)
-    tf = (lin_flops + attn_flops) / (ms * 1e-3) / 1e12
-    print(json.dumps({
-        "metric": "7B-shape prompt tokens/s", "value": round(B * S / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,
-        "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"32-layer Llama-2-7B-shape decoder, MXFP4 linears, prompt of {S} tokens x batch {B} in "
-                               f"one pass onto an empty KV cache", "launch": "eager op calls", "batch": B},
-        "roofline": {"bound": "mfma", "kernel": "whole prompt pass (GEMMs + causal attention + glue)",
-                     "achieved": round(tf, 1), "peak": PEAKS_TFLOPS["bf16"], "unit": "TFLOP/s",
-                     "frac": round(tf / PEAKS_TFLOPS["bf16"], 4), "traffic": None,
-                     "flops_per_step": lin_flops + attn_flops},
-        "cpu_baseline": None}))
-
-
-def run_prefill(torch, _ops, args):
-    """BASELINE config 4: M = 2048 tokens through the MXFP4 linears of one decoder layer with hidden 8192
-    (fused qkv 8192 -> 8192+1024+1024, o 8192 -> 8192 + residual, then the MLP block gate/up 8192 -> 28672 with
-    silu * mul and down 28672 -> 8192 + residual through the package's swiglu_mlp op, whose result is bit-identical
-    to fc_silu, fc_mul, fc_add in sequence).  One step = those three op calls (seven GEMMs)."""
-    from tpp_pytorch_extension import _lib
-    dev = torch.device("cuda:0")
-    M, H, I = 2048, 8192, 28672
-    g = torch.Generator(device=dev).manual_seed(1238)
-
-    pfmt = args.prefill_fmt
-    fp8 = bool(args.act_fp8) and pfmt == "mxfp4"
-    _ops.ACT_FP8 = _ops.ACT_FP8 or fp8
-    fp8 = fp8 or (_ops.ACT_FP8 and pfmt == "mxfp4")
-    quant = _ops.remap_and_quantize_mxfp4 if pfmt == "mxfp4" else _ops.remap_and_quantize_qint8
-
-    def mk(N, K):
-        W = (torch.randn((N, K), generator=g, device=dev) * 0.02).to(torch.bfloat16)
-        q = quant(W.view(N // 16, 16, K // 64, 32, 2).permute(0, 2, 3, 1, 4).contiguous())
-        q.native()
-        return q
-
-    wq, wk, wv, wo = mk(H, H), mk(1024, H), mk(1024, H), mk(H, H)
-    wg, wu, wd = mk(I, H), mk(I, H), mk(H, I)
-    x = torch.randn((M, H), generator=g, device=dev).to(torch.bfloat16)
-    res = torch.randn((M, H), generator=g, device=dev).to(torch.bfloat16)
-    empty = torch.empty(0, dtype=torch.bfloat16, device=dev)
-
-    def step():
-        q, k, v = torch.ops.tpp_llm.qkv_gemm(x, [wq, wk, wv], [empty] * 3)
-        h = torch.ops.tpp_llm.fc_add(q, wo, empty, res, 1.0)
-        return torch.ops.tpp_llm.swiglu_mlp(h, wg, wu, wd, h, 1.0), k, v
-
-    gemms = [("qkv", 10240, H), ("o", H, H), ("gate", I, H), ("up", I, H), ("down", H, I)]
-    flops = sum(2.0 * M * N * K for _, N, K in gemms)
-    steps, warmup = max(3, min(args.steps, 20)), max(1, min(args.warmup, 3))
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / steps
-
-    # roofline leg: the largest GEMM (down projection) alone, events on the launch stream
-    L = _lib.lib()
-    plan = kernel_plan(L, pfmt, M, H, I, 256, _lib.FLAG_ACT_FP8 if fp8 else 0, (33 * M * I) // 32 if fp8 else 0)
-    inter = torch.randn((M, I), generator=g, device=dev).to(torch.bfloat16)
-    for _ in range(2):
-        torch.ops.tpp_llm.fc_add(inter, wd, empty, res, 1.0)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    reps = 10
-    e0.record()
-    for _ in range(reps):
-        torch.ops.tpp_llm.fc_add(inter, wd, empty, res, 1.0)
-    e1.record()
-    torch.cuda.synchronize()
-    us = e0.elapsed_time(e1) * 1e3 / reps
-    fl = 2.0 * M * H * I
-    peak = PEAKS_TFLOPS["fp8" if fp8 else "bf16"] if pfmt == "mxfp4" else PEAKS_TFLOPS["int8"]
-    roof = {"bound": "mfma", "kernel": plan[-1][0] if plan else "?",
-            "call": f"down M={M} N={H} K={I}" + (" (activation quantiser included)" if fp8 else ""),
-            "achieved": round(fl / us / 1e6, 1), "peak": peak, "unit": "TFLOP/s" if pfmt == "mxfp4" else "TOP/s",
-            "frac": round(fl / us / 1e6 / peak, 4), "traffic": None,
-            "avg_launch_us": round(us, 1), "flops_per_launch": fl, "launches_timed": reps,
-            "timing": "events on the launch stream around eager launches of this op alone"}
-    cpu = None if (args.no_cpu or pfmt != "mxfp4") else cpu_baseline_prefill(H)
-    print(json.dumps({
-        "metric": "quant-GEMM TFLOP/s (prefill)", "value": round(flops / (ms * 1e-3) / 1e12, 2),
-        "unit": "TFLOP/s" if pfmt == "mxfp4" else "TOP/s",
-        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": ("fp8" if fp8 else "bf16") if pfmt == "mxfp4" else "int8", "data": "synthetic",
-        "config": {"workload": (("cfg4: MXFP4" + (" weights x MXFP8 activations (opt-in, not the reference's "
-                                                  "arithmetic)" if fp8 else ""))
-                                if pfmt == "mxfp4" else "cfg4's layer with QINT8 W8A8 (QBS=256)") +
-                               " linears of one decoder layer (hidden 8192, intermediate 28672, kv 1024) at "
-                               "M = 2048: qkv_gemm, fc_add(o), swiglu_mlp(gate, up, down)",
-                   "launch": "eager op calls", "flops_per_step": flops},
-        "roofline": roof, "cpu_baseline": cpu}))
-
-
-def cpu_baseline_prefill(H):
-    """The oracle's MXFP4 linear on a bounded sample: 256 rows through an 8192 x 8192 projection, faithful mode."""
-    sys.path.insert(0, os.path.join(ROOT, "oracle"))
-    import numpy as np
-    import oracle as O
-    cores = len(os.sched_getaffinity(0))
-    cores = min(cores, O.num_threads()) if O.num_threads() > 0 else cores
-    O.set_num_threads(cores)
-    rng = np.random.default_rng(7)
-    Ms, N = 256, 2048
-    W = (rng.standard_normal((N, H), dtype=np.float32) * 0.02).astype(np.float32)
-    q, sc = O.remap_quantize_mxfp4(W)
-    xf = rng.standard_normal((Ms, H), dtype=np.float32)
-    xb = (xf.view(np.uint32) >> 16).astype(np.uint16)  # truncation is fine for a timing input
-    O.linear_mxfp4(xb, q, sc, None, O.POST_NONE, None, None, 1.0, O.MODE_FAITHFUL)
-    n, t0 = 0, time.perf_counter()
-    while True:
-        O.linear_mxfp4(xb, q, sc, None, O.POST_NONE, None, None, 1.0, O.MODE_FAITHFUL)
-        n += 1
-        dt = time.perf_counter() - t0
-        if dt > 12.0 or n >= 200:
-            break
-    fl = 2.0 * Ms * N * H
-    return {"value": round(fl * n / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"{n} passes of a {Ms} x {N} x {H} MXFP4 linear (C/OpenMP restatement of the reference recipe, "
-                      f"faithful mode; not the libxsmm JIT), {round(dt / n * 1e3, 1)} ms each"}
-
-
-def kernel_plan(L, fmt, M, N, K, qbs, flags, ws_bytes):
-    """Kernels one linear call enqueues, as the library itself reports them:
-    [(profiler name, launch shape text), ...]; the last one is the GEMM."""
-    import ctypes
-    buf = ctypes.create_string_buffer(4096)
-    if fmt == "qint8":
-        rc = L.tppx_plan_linear_qint8(M, N, K, qbs, 1, flags, ws_bytes, buf, len(buf))
-    else:
-        rc = L.tppx_plan_linear_mxfp4(M, N, K, flags, ws_bytes, buf, len(buf))
-    if rc != 0:
-        return []
-    out = []
-    for line in buf.value.decode().strip().splitlines():
-        name, _, shape = line.partition(" grid=")
-        out.append((name.replace("void ", ""), "grid=" + shape))
-    return out
-
-
-def roofline_leg(torch, _ops, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
+def roofline_decode(torch, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
     """Each GEMM kernel of the step alone, between two events on the launch
     stream.  One graph per (shape, M) holds one launch per weight copy of that
     shape in the pool (> 256 MB, so every launch streams from HBM).  For QINT8
-    with more than 4 rows the activation is quantized once beforehand and the
-    timed launches reuse it (TPPX_FLAG_XQ_REUSE), so only the GEMM kernel runs.
-    achieved = algorithmic bytes of the call / mean kernel duration."""
+    kernels that do not quantize inside the GEMM the activation is quantized once
+    beforehand and the timed launches reuse it (TPPX_FLAG_XQ_REUSE), so only the
+    GEMM kernel runs.  achieved = algorithmic bytes of the call / mean kernel duration."""
     from tpp_pytorch_extension import _lib
     L = _lib.lib()
     dev = torch.device("cuda:0")
@@ -450,7 +314,8 @@ def roofline_leg(torch, _ops, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
                                                    y.data_ptr(), M, N, K, 3, 1.0, flags, ws.data_ptr(), ws.numel(), st))
                 reuse = 0
             keep += [y]
-            plan = kernel_plan(L, fmt, M, N, K, qbs, reuse, ws.numel())
+            plan_call = kernel_plan(L, fmt, M, N, K, qbs, 0, ws.numel())       # what an op call enqueues
+            plan = kernel_plan(L, fmt, M, N, K, qbs, reuse, ws.numel())        # what is timed here
             call(copies[0][0], copies[0][1], 0, stream)  # quantizes the activation where the path keeps it
             torch.cuda.synchronize()
 
@@ -458,32 +323,13 @@ def roofline_leg(torch, _ops, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
                 for qn, sn in copies:
                     call(qn, sn, reuse, st)
 
-            g = None
-            if not args.no_graph:
-                try:
-                    g = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(g):
-                        fire(torch.cuda.current_stream().cuda_stream)
-                except Exception:
-                    g = None
-            reps = max(3, min(25, args.steps // 8))
-            for _ in range(2):
-                g.replay() if g is not None else fire(stream)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(reps):
-                g.replay() if g is not None else fire(stream)
-            e1.record()
-            torch.cuda.synchronize()
-            n_launch = reps * len(copies)
-            avg_us = e0.elapsed_time(e1) * 1e3 / n_launch
+            avg_us, n_launch = events_us(torch, fire, len(copies), use_graph=not args.no_graph)
             nbytes = algorithmic_bytes(fmt, M, N, K, qbs)
             rows.append({
                 "kernel": plan[-1][0] if plan else "?",
                 "launch": plan[-1][1] if plan else "",
                 "call": f"{name} M={M} N={N} K={K}",
-                "kernels_per_call": len(plan),
+                "kernels_per_call": len(plan_call),
                 "avg_launch_us": round(avg_us, 3),
                 "bytes_per_launch": nbytes,
                 "achieved": round(nbytes / avg_us / 1e3, 1),
@@ -526,28 +372,18 @@ def measured_traffic(kernel, call):
     return None
 
 
-def cpu_baseline(fmt, W, X, R, Ms, shapes, qbs, bytes_per_step):
+def cpu_baseline_decode(fmt, W, X, R, Ms, shapes, qbs, bytes_per_step, seconds=10.0):
     """The oracle's restatement of the reference CPU path on the host cores,
     one step's worth of linears on the same seeded inputs, repeated for about
-    12 s."""
-    sys.path.insert(0, os.path.join(ROOT, "oracle"))
-    import numpy as np
-    import torch
-    import oracle as O
-
-    def bits(t):
-        return t.contiguous().view(torch.int16).numpy().view(np.uint16)
-
-    cores = len(os.sched_getaffinity(0))
-    cores = min(cores, O.num_threads()) if O.num_threads() > 0 else cores
-    O.set_num_threads(cores)
+    10 s."""
+    O, cores = oracle_mod()
     qw = {}
     for name in shapes:
         Wf = W[name].float().numpy()
         qw[name] = O.remap_quantize_qint8(Wf)[:2] if fmt == "qint8" else O.remap_quantize_mxfp4(Wf)
     lin = O.linear_qint8 if fmt == "qint8" else O.linear_mxfp4
-    xs = {k: bits(v) for k, v in X.items()}
-    rs = {k: bits(v) for k, v in R.items()}
+    xs = {k: t_bits(v) for k, v in X.items()}
+    rs = {k: t_bits(v) for k, v in R.items()}
 
     def one_step():
         for M in Ms:
@@ -555,14 +391,7 @@ def cpu_baseline(fmt, W, X, R, Ms, shapes, qbs, bytes_per_step):
                 q, s = qw[name]
                 lin(xs[(name, M)], q, s, None, O.POST_ADD_SCALE, rs[(name, M)], None, 1.0, O.MODE_FAITHFUL)
 
-    one_step()  # warm-up
-    n, t0 = 0, time.perf_counter()
-    while True:
-        one_step()
-        n += 1
-        dt = time.perf_counter() - t0
-        if dt > 12.0 or n >= 400:
-            break
+    n, dt = repeat_for(one_step, seconds)
     sec = dt / n
     return {
         "value": round(bytes_per_step / sec / 1e12, 5),
@@ -572,6 +401,499 @@ def cpu_baseline(fmt, W, X, R, Ms, shapes, qbs, bytes_per_step):
         "sample": f"{n} passes over the same 8-linear step (C/OpenMP restatement of the reference recipe, "
                   f"faithful bf16 re-rounding; not the libxsmm JIT), {round(sec * 1e3, 1)} ms per step",
     }
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# config 1: one MXFP4 fc_plain, M = 16, 4096 x 4096, bias
+# ---------------------------------------------------------------------------------------------------------------
+def leg_cfg1(torch, _ops, args):
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    M, N, K = 16, 4096, 4096
+    g = torch.Generator(device="cpu").manual_seed(1235)
+    W = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    x = torch.randn((M, K), generator=g).to(torch.bfloat16)
+    bias = (torch.randn((N,), generator=g) * 0.01).to(torch.bfloat16)
+    base = _ops.remap_and_quantize_mxfp4(block_bf16(W).to(dev))
+    copies = [clone_weight(base) for _ in range(32)]  # 32 x 8.9 MB = 285 MB of distinct weight bytes
+    xd, bd = x.to(dev), bias.to(dev)
+
+    def fire(_st):
+        return [torch.ops.tpp_llm.fc_plain(xd, w, bd, -1, []) for w in copies]
+
+    fire(None)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        keep = fire(None)
+    ms, blocks = time_blocks(torch, lambda i: graph.replay(), 4, 2)
+    us_call = ms * 1e3 / len(copies)
+    nbytes = algorithmic_bytes("mxfp4", M, N, K, bias=True, post_in=False)
+    ev_us, n_launch = events_us(torch, lambda st: graph.replay(), len(copies), use_graph=False)
+    plan = kernel_plan(L, "mxfp4", M, N, K, 256, 0, _lib.WORKSPACE_BYTES)
+    cpu = None
+    if not args.no_cpu:
+        O, cores = oracle_mod()
+        q, sc = O.remap_quantize_mxfp4(W.float().numpy())
+        xb, bb = t_bits(x), t_bits(bias)
+        n, dt = repeat_for(lambda: O.linear_mxfp4(xb, q, sc, bb, O.POST_NONE, None, None, 1.0, O.MODE_FAITHFUL), 3.0)
+        cpu = {"value": round(nbytes * n / dt / 1e12, 5), "unit": "TB/s", "cores": cores, "kind": "port",
+               "sample": f"{n} passes of the same linear on the same inputs, {round(dt / n * 1e3, 2)} ms each"}
+    del keep
+    return {
+        "leg": "cfg1", "metric": "quant-GEMM HBM TB/s (decode)", "value": round(nbytes / us_call / 1e6, 4), "unit": "TB/s",
+        "us_per_call": round(us_call, 3), "dtype": "bf16",
+        "workload": "cfg1: MXFP4 fc_plain, M=16, K=N=4096, bf16 bias; 32 weight copies in rotation (285 MB), one HIP "
+                    "graph of 32 calls replayed",
+        "roofline": {"bound": "hbm", "kernel": plan[-1][0] if plan else "?", "launch": plan[-1][1] if plan else "",
+                     "achieved": round(nbytes / ev_us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(nbytes / ev_us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "avg_launch_us": round(ev_us, 3), "bytes_per_launch": nbytes, "launches_timed": n_launch},
+        "cpu_baseline": cpu,
+    }
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# config 3: MXFP4 SwiGLU MLP block, M in {1, 4, 16, 64}
+# ---------------------------------------------------------------------------------------------------------------
+def cfg3_bytes(M, H=4096, I=11008):
+    """weights + scales of the three projections, X, residual, out, and the intermediate written once + read once."""
+    w = 3 * (H * I // 2 + H * I // 32)
+    return w + 3 * (2 * M * H) + 2 * (2 * M * I)
+
+
+def leg_cfg3(torch, _ops, args):
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    H, I = CFG3_DIMS
+    Ms = list(CFG3_MS)
+    g = torch.Generator(device="cpu").manual_seed(1237)
+    Wg = (torch.randn((I, H), generator=g) * 0.02).to(torch.bfloat16)
+    Wu = (torch.randn((I, H), generator=g) * 0.02).to(torch.bfloat16)
+    Wd = (torch.randn((H, I), generator=g) * 0.02).to(torch.bfloat16)
+    X = {M: torch.randn((M, H), generator=g).to(torch.bfloat16) for M in Ms}
+    base = [_ops.remap_and_quantize_mxfp4(block_bf16(w).to(dev)) for w in (Wg, Wu, Wd)]
+    pool = [{M: [clone_weight(b) for b in base] for M in Ms} for _ in range(2)]  # 2 x 4 x 72 MB = 575 MB
+    Xd = {M: X[M].to(dev) for M in Ms}
+
+    def step(ws):
+        return [torch.ops.tpp_llm.swiglu_mlp(Xd[M], ws[M][0], ws[M][1], ws[M][2], Xd[M], 1.0) for M in Ms]
+
+    for ws in pool:
+        step(ws)
+    torch.cuda.synchronize()
+    graphs = []
+    for ws in pool:
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            keep = step(ws)
+        graphs.append((gr, keep))
+    ms, blocks = time_blocks(torch, lambda i: graphs[i % 2][0].replay(), 20, 5)
+    bytes_per_step = sum(cfg3_bytes(M) for M in Ms)
+
+    # each launch alone: gate/up pair, down projection
+    rows = []
+    wsb = _lib.WORKSPACE_BYTES
+    for M in Ms:
+        xin = Xd[M]
+        inter = _ops.swiglu_gate_up(xin, pool[0][M][0], pool[0][M][1])
+        sets = [p[M] for p in pool] + [[clone_weight(b) for b in base] for _ in range(10)]  # 12 x 72 MB
+
+        def fire_gu(_st):
+            return [_ops.swiglu_gate_up(xin, w[0], w[1]) for w in sets]
+
+        def fire_dn(_st):
+            return [_ops.fc_add(inter, w[2], None, xin, 1.0) for w in sets]
+
+        for nm, fire, nb, pl in (
+                ("gate/up", fire_gu, 2 * (H * I // 2 + H * I // 32) + 2 * M * H + 2 * M * I,
+                 group_plan(L, "mxfp4", [I, I], M, H, 1, 0, wsb)),
+                ("down", fire_dn, (H * I // 2 + H * I // 32) + 2 * M * I + 2 * (2 * M * H),
+                 kernel_plan(L, "mxfp4", M, H, I, 256, 0, wsb))):
+            us, n = events_us(torch, fire, len(sets), use_graph=not args.no_graph)
+            rows.append({"kernel": pl[-1][0] if pl else "?", "launch": pl[-1][1] if pl else "", "call": f"{nm} M={M}",
+                         "kernels_per_call": len(pl), "avg_launch_us": round(us, 3), "bytes_per_launch": nb,
+                         "achieved": round(nb / us / 1e3, 1), "frac": round(nb / us / 1e3 / HBM_PEAK_GBS, 4),
+                         "launches_timed": n})
+        del sets, inter
+    dom = max(rows, key=lambda r: r["avg_launch_us"])
+    cpu = None
+    if not args.no_cpu:
+        O, cores = oracle_mod()
+        qs = [O.remap_quantize_mxfp4(w.float().numpy()) for w in (Wg, Wu, Wd)]
+        xb = {M: t_bits(X[M]) for M in Ms}
+
+        def one():
+            for M in Ms:
+                gate = O.linear_mxfp4(xb[M], qs[0][0], qs[0][1], None, O.POST_SILU, None, None, 1.0, O.MODE_FAITHFUL)
+                it = O.linear_mxfp4(xb[M], qs[1][0], qs[1][1], None, O.POST_MUL, gate, None, 1.0, O.MODE_FAITHFUL)
+                O.linear_mxfp4(it, qs[2][0], qs[2][1], None, O.POST_ADD_SCALE, xb[M], None, 1.0, O.MODE_FAITHFUL)
+
+        n, dt = repeat_for(one, 6.0)
+        cpu = {"value": round(bytes_per_step * n / dt / 1e12, 5), "unit": "TB/s", "cores": cores, "kind": "port",
+               "sample": f"{n} passes over the same four MLP blocks, {round(dt / n * 1e3, 1)} ms per step"}
+    per_m = {}
+    for M in Ms:
+        us = sum(r["avg_launch_us"] for r in rows if r["call"].endswith(f"M={M}"))
+        per_m[str(M)] = {"us_per_block": round(us, 2), "TB/s": round(cfg3_bytes(M) / us / 1e6, 3)}
+    return {
+        "leg": "cfg3", "metric": "quant-GEMM HBM TB/s (decode)",
+        "value": round(bytes_per_step / (ms * 1e-3) / 1e12, 4), "unit": "TB/s", "ms_per_step": round(ms, 5), "dtype": "bf16",
+        "workload": "cfg3: MXFP4 SwiGLU MLP block (torch.ops.tpp_llm.swiglu_mlp = gate/up launch + down launch), hidden "
+                    "4096, intermediate 11008, M in {1,4,16,64}; one step = the four blocks; two weight sets of 288 MB "
+                    "alternate; HIP graph replay",
+        "bytes_per_step": bytes_per_step, "per_M": per_m,
+        "roofline": {"bound": "hbm", "kernel": dom["kernel"], "call": dom["call"], "achieved": dom["achieved"],
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"], "traffic": None,
+                     "avg_launch_us": dom["avg_launch_us"], "bytes_per_launch": dom["bytes_per_launch"],
+                     "launches_timed": dom["launches_timed"], "all_gemm_kernels": rows},
+        "cpu_baseline": cpu,
+    }
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# config 4: prefill GEMMs of one 70B-shape decoder layer at M = 2048
+# ---------------------------------------------------------------------------------------------------------------
+def leg_cfg4(torch, _ops, args, pfmt="mxfp4", fp8=False, cpu=True):
+    """M = 2048 tokens through the linears of one decoder layer with hidden 8192 (fused qkv 8192 -> 8192+1024+1024,
+    o 8192 -> 8192 + residual, then the MLP block gate/up 8192 -> 28672 with silu * mul and down 28672 -> 8192 +
+    residual through the package's swiglu_mlp op, whose result is bit-identical to fc_silu, fc_mul, fc_add in
+    sequence).  One step = those three op calls (seven GEMMs)."""
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    M, H, I = CFG4_DIMS
+    g = torch.Generator(device=dev).manual_seed(1238)
+    fp8 = bool(fp8) and pfmt == "mxfp4"
+    old_fp8 = _ops.ACT_FP8
+    _ops.ACT_FP8 = fp8
+    try:
+        quant = _ops.remap_and_quantize_mxfp4 if pfmt == "mxfp4" else _ops.remap_and_quantize_qint8
+
+        def mk(N, K):
+            W = (torch.randn((N, K), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+            q = quant(W.view(N // 16, 16, K // 64, 32, 2).permute(0, 2, 3, 1, 4).contiguous())
+            q.native()
+            return q
+
+        wq, wk, wv, wo = mk(H, H), mk(1024, H), mk(1024, H), mk(H, H)
+        wg, wu, wd = mk(I, H), mk(I, H), mk(H, I)
+        x = torch.randn((M, H), generator=g, device=dev).to(torch.bfloat16)
+        res = torch.randn((M, H), generator=g, device=dev).to(torch.bfloat16)
+        inter = torch.randn((M, I), generator=g, device=dev).to(torch.bfloat16)
+        empty = torch.empty(0, dtype=torch.bfloat16, device=dev)
+
+        def step(_i=0):
+            q, k, v = torch.ops.tpp_llm.qkv_gemm(x, [wq, wk, wv], [empty] * 3)
+            h = torch.ops.tpp_llm.fc_add(q, wo, empty, res, 1.0)
+            return torch.ops.tpp_llm.swiglu_mlp(h, wg, wu, wd, h, 1.0), k, v
+
+        gemms = [("qkv", 10240, H), ("o", H, H), ("gate", I, H), ("up", I, H), ("down", H, I)]
+        flops = sum(2.0 * M * N * K for _, N, K in gemms)
+        ms, blocks = time_blocks(torch, step, 3, 2)
+
+        peak = PEAKS_TFLOPS["fp8" if fp8 else "bf16"] if pfmt == "mxfp4" else PEAKS_TFLOPS["int8"]
+        unit = "TFLOP/s" if pfmt == "mxfp4" else "TOP/s"
+        flags = _lib.FLAG_ACT_FP8 if fp8 else 0
+        wsb = lambda K: (33 * M * K) // 32 if fp8 else _lib.WORKSPACE_BYTES  # noqa: E731
+        ops = [
+            ("qkv M=2048 N=10240 K=8192", lambda st: torch.ops.tpp_llm.qkv_gemm(x, [wq, wk, wv], [empty] * 3),
+             2.0 * M * 10240 * H, group_plan(L, pfmt, [H, 1024, 1024], M, H, 0, flags, wsb(H))),
+            ("o M=2048 N=8192 K=8192", lambda st: torch.ops.tpp_llm.fc_add(x, wo, empty, res, 1.0),
+             2.0 * M * H * H, kernel_plan(L, pfmt, M, H, H, 256, flags, wsb(H))),
+            ("gate/up M=2048 N=2x28672 K=8192 (+ silu*mul pass)", lambda st: _ops.swiglu_gate_up(x, wg, wu),
+             4.0 * M * I * H, (group_plan(L, pfmt, [I, I], M, H, 1, flags, max(wsb(H), 2 * M * I + wsb(H)))
+                               if pfmt == "mxfp4" else kernel_plan(L, pfmt, M, I, H, 256, flags, wsb(H)))),
+            ("down M=2048 N=8192 K=28672", lambda st: torch.ops.tpp_llm.fc_add(inter, wd, empty, res, 1.0),
+             2.0 * M * H * I, kernel_plan(L, pfmt, M, H, I, 256, flags, wsb(I))),
+        ]
+        rows = []
+        for name, fn, fl, pl in ops:
+            us, n = events_us(torch, fn, 1, use_graph=False)
+            gemm = [p for p in pl if "quant_act" not in p[0] and "silu_mul" not in p[0]]
+            rows.append({"kernel": gemm[-1][0] if gemm else "?", "launch": gemm[-1][1] if gemm else "", "call": name,
+                         "kernels_per_call": len(pl), "avg_launch_us": round(us, 1), "flops_per_launch": fl,
+                         "achieved": round(fl / us / 1e6, 1), "frac": round(fl / us / 1e6 / peak, 4),
+                         "launches_timed": n})
+        dom = max(rows, key=lambda r: r["avg_launch_us"] if r["call"].startswith("down") else 0)
+        cpu_b = cpu_baseline_prefill(H) if (cpu and not args.no_cpu and pfmt == "mxfp4" and not fp8) else None
+    finally:
+        _ops.ACT_FP8 = old_fp8
+    label = ("cfg4: MXFP4" + (" weights x MXFP8 activations (opt-in, NOT the reference's arithmetic)" if fp8 else
+                              " (bf16 activations, the reference's arithmetic)")) if pfmt == "mxfp4" else \
+        "cfg4's layer with QINT8 W8A8 (QBS=256; not a BASELINE configuration)"
+    return {
+        "leg": "cfg4" + ("" if pfmt == "mxfp4" and not fp8 else ("-act-fp8" if fp8 else "-qint8")),
+        "metric": "quant-GEMM TFLOP/s (prefill)", "value": round(flops / (ms * 1e-3) / 1e12, 2), "unit": unit,
+        "ms_per_step": round(ms, 4), "dtype": ("fp8" if fp8 else "bf16") if pfmt == "mxfp4" else "int8",
+        "workload": label + " linears of one decoder layer (hidden 8192, intermediate 28672, kv 1024) at M = 2048: "
+                            "qkv_gemm, fc_add(o), swiglu_mlp(gate, up, down); eager op calls",
+        "flops_per_step": flops,
+        "roofline": {"bound": "mfma", "kernel": dom["kernel"], "call": dom["call"] +
+                     (" (activation quantiser included)" if (fp8 or pfmt == "qint8") else ""),
+                     "achieved": dom["achieved"], "peak": peak, "unit": unit, "frac": dom["frac"], "traffic": None,
+                     "avg_launch_us": dom["avg_launch_us"], "flops_per_launch": dom["flops_per_launch"],
+                     "launches_timed": dom["launches_timed"],
+                     "timing": "events on the launch stream around eager launches of this op alone",
+                     "all_gemm_kernels": rows},
+        "cpu_baseline": cpu_b,
+    }
+
+
+def cpu_baseline_prefill(H, seconds=8.0):
+    """The oracle's MXFP4 linear on a bounded sample: 256 rows through an 8192 x 8192 projection, faithful mode."""
+    import numpy as np
+    O, cores = oracle_mod()
+    rng = np.random.default_rng(7)
+    Ms, N = 256, 2048
+    W = (rng.standard_normal((N, H), dtype=np.float32) * 0.02).astype(np.float32)
+    q, sc = O.remap_quantize_mxfp4(W)
+    xf = rng.standard_normal((Ms, H), dtype=np.float32)
+    xb = (xf.view(np.uint32) >> 16).astype(np.uint16)  # truncation is fine for a timing input
+    n, dt = repeat_for(lambda: O.linear_mxfp4(xb, q, sc, None, O.POST_NONE, None, None, 1.0, O.MODE_FAITHFUL), seconds, 200)
+    fl = 2.0 * Ms * N * H
+    return {"value": round(fl * n / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{n} passes of a {Ms} x {N} x {H} MXFP4 linear (C/OpenMP restatement of the reference recipe, "
+                      f"faithful mode; not the libxsmm JIT), {round(dt / n * 1e3, 1)} ms each"}
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# config 5: 32-layer 7B-shape decoder, greedy decode
+# ---------------------------------------------------------------------------------------------------------------
+_MODEL = {}
+
+
+def cfg5_model(torch):
+    if "m" not in _MODEL:
+        from tpp_pytorch_extension.llm import fused_llama_infer as F
+        _MODEL["m"] = F.LlamaDecoder(hidden=4096, inter=11008, n_layers=32, n_heads=32, n_kv_heads=32, vocab=32000,
+                                     max_positions=4096, weight_dtype="mxfp4", seed=1239)
+    return _MODEL["m"]
+
+
+def leg_cfg5(torch, args, B, cpu=True):
+    """BASELINE config 5: 32-layer Llama-2-7B-shape decoder, all linears (and the lm_head) MXFP4, KV cache
+    pre-filled with 2048 positions of N(0,1), greedy decode of 128 new tokens for B sequences from
+    random token ids; the decode step is one replayed HIP graph."""
+    dev = torch.device("cuda:0")
+    ctx, new = 2048, 128
+    model = cfg5_model(torch)
+    tok = torch.randint(0, 32000, (B,), generator=torch.Generator().manual_seed(5), dtype=torch.int64).to(dev)
+    out = model.greedy_decode(tok, model.new_cache(B, ctx, ctx + new + 32), 8)  # warm-up run
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = model.greedy_decode(tok, model.new_cache(B, ctx, ctx + new + 32), new)
+    torch.cuda.synchronize()
+    wall_with_capture = time.perf_counter() - t0
+    # the replays alone (capture and warm-up step excluded), repeated until >= MIN_WALL_S
+    total, runs = 0.0, 0
+    while total < MIN_WALL_S and runs < 50:
+        cache = model.new_cache(B, ctx, ctx + new + 32)
+        total += model.time_decode_steps(tok, cache, new)
+        runs += 1
+        del cache
+    steps_t = total / runs
+    ms = steps_t * 1e3 / new
+    lin_bytes = 32 * (3 * 4096 * 4096 + 4096 * 4096 + 3 * 11008 * 4096) * (0.5 + 1.0 / 32) + 32000 * 4096 * (0.5 + 1.0 / 32)
+    kv_bytes = B * 32 * 2 * 32 * (ctx + new / 2) * 128 * 2
+    achieved = (lin_bytes + kv_bytes) / (ms * 1e-3) / 1e9
+    cpu_b = None
+    if cpu and not args.no_cpu:
+        cpu_b = cpu_baseline_tokens(B)
+    return {
+        "leg": f"cfg5-batch{B}", "metric": "7B-shape decode tokens/s", "value": round(B * new / steps_t, 1),
+        "unit": "tokens/s", "ms_per_step": round(ms, 4), "dtype": "bf16",
+        "workload": f"cfg5: 32-layer Llama-2-7B-shape decoder, MXFP4 linears and lm_head, bf16 RMSNorm / rotary / KV cache, "
+                    f"context {ctx} of N(0,1), greedy decode of {new} tokens, batch {B}; one HIP graph per decode step, "
+                    f"replayed; {runs} runs of {new} steps timed",
+        "wall_s_one_run_including_capture": round(wall_with_capture, 4), "tokens_per_run": int(out.numel()),
+        "roofline": {"bound": "hbm", "kernel": "whole decode step (all kernels of the graph; per-kernel durations in "
+                                               f"profiles/decoder_step_kernels_cfg5_batch{B}_stats.txt)",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_step": int(lin_bytes + kv_bytes)},
+        "cpu_baseline": cpu_b,
+    }
+
+
+def cpu_baseline_tokens(B, seconds=6.0):
+    """The oracle's composition of ONE decoder layer's decode step (the reference recipe: RMSNorm, q/k/v, rotary,
+    attention over 2048 cached keys, o + residual, RMSNorm, gate/up, down + residual) on the host cores, times 32
+    layers, plus the MXFP4 lm_head: a bounded sample of the 32-layer step."""
+    import numpy as np
+    O, cores = oracle_mod()
+    rng = np.random.default_rng(11)
+    hidden, inter, Nh, H, ctx = 4096, 11008, 32, 128, 2048
+
+    def qw(N, K):
+        return O.remap_quantize_mxfp4((rng.standard_normal((N, K), dtype=np.float32) * 0.02).astype(np.float32))
+
+    def bf(a):
+        return (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+
+    Wq, Wk, Wv, Wo = qw(hidden, hidden), qw(hidden, hidden), qw(hidden, hidden), qw(hidden, hidden)
+    Wg, Wu, Wd = qw(inter, hidden), qw(inter, hidden), qw(hidden, inter)
+    Wl = qw(32000, hidden)
+    kc = bf(rng.standard_normal((B, Nh, ctx + 1, H), dtype=np.float32))
+    vc = bf(rng.standard_normal((B, Nh, ctx + 1, H), dtype=np.float32))
+    x = bf(rng.standard_normal((B, hidden), dtype=np.float32))
+    gam = np.ones(hidden, np.float32)
+    inv = 1.0 / (10000.0 ** (np.arange(0, H, 2, dtype=np.float32) / H))
+    fr = np.outer(np.arange(4096, dtype=np.float32), inv)
+    emb = np.stack([np.cos(np.concatenate([fr, fr], -1)), np.sin(np.concatenate([fr, fr], -1))]).astype(np.float32)
+    pos = np.full((B, 1), ctx, np.int64)
+
+    def mm(a, w, post=O.POST_NONE, pin=None):
+        return O.linear_mxfp4(a, w[0], w[1], None, post, pin, None, 1.0, O.MODE_FAITHFUL)
+
+    def layer():
+        h = O.rms_norm(x, gam, 1e-5)
+        q, k, v = mm(h, Wq), mm(h, Wk), mm(h, Wv)
+        q = O.rotary_llama(q.reshape(B, 1, -1), emb, pos, Nh, H).reshape(B, Nh, H)
+        k = O.rotary_llama(k.reshape(B, 1, -1), emb, pos, Nh, H).reshape(B, Nh, H)
+        kc[:, :, ctx] = k
+        vc[:, :, ctx] = v.reshape(B, Nh, H)
+        c = O.attn_decode(q, kc, vc).reshape(B, hidden)
+        so = mm(c, Wo, O.POST_ADD_SCALE, x)
+        h2 = O.rms_norm(so, gam, 1e-5)
+        g = mm(h2, Wg, O.POST_SILU)
+        return mm(mm(h2, Wu, O.POST_MUL, g), Wd, O.POST_ADD_SCALE, so)
+
+    n, dt = repeat_for(layer, seconds, 200)
+    t_layer = dt / n
+    n2, dt2 = repeat_for(lambda: mm(x, Wl), 1.0, 50)
+    t_step = 32 * t_layer + dt2 / n2
+    return {"value": round(B / t_step, 3), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"{n} passes of one decoder layer's decode step at batch {B} (oracle composition, "
+                      f"{round(t_layer * 1e3, 1)} ms each) x 32 layers + the lm_head ({round(dt2 / n2 * 1e3, 1)} ms): "
+                      f"{round(t_step * 1e3, 1)} ms per token step"}
+
+
+def run_prompt(torch, args):
+    """Prompt processing on the 7B-shape decoder of config 5: `--batch` sequences of 2048 random token ids through
+    the 32 layers in one pass (MXFP4 linears on the large-M kernels, causal attention, keys appended to an empty
+    cache), then the lm_head on the last position.  Not a BASELINE configuration; reported as prompt tokens/s."""
+    from tpp_pytorch_extension.llm import fused_llama_infer as F
+    dev = torch.device("cuda:0")
+    B, S = args.batch, 2048
+    model = cfg5_model(torch)
+    prompt = torch.randint(0, 32000, (B, S), generator=torch.Generator().manual_seed(6), dtype=torch.int64).to(dev)
+    steps, warmup = max(2, min(args.steps, 8)), max(1, min(args.warmup, 2))
+    caches = [F.TppCache(S + 32) for _ in range(steps + warmup)]
+    for c in caches[:warmup]:
+        model.prefill(prompt, c)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for c in caches[warmup:]:
+        model.prefill(prompt, c)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    lin_flops = 2.0 * B * S * 32 * (4 * 4096 * 4096 + 3 * 11008 * 4096) + 2.0 * B * 32000 * 4096
+    attn_flops = 32 * 4.0 * B * 32 * 128 * (S * (S + 1) / 2)
+    tf = (lin_flops + attn_flops) / (ms * 1e-3) / 1e12
+    return {
+        "metric": "7B-shape prompt tokens/s", "value": round(B * S / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"32-layer Llama-2-7B-shape decoder, MXFP4 linears, prompt of {S} tokens x batch {B} in "
+                               f"one pass onto an empty KV cache", "launch": "eager op calls", "batch": B},
+        "roofline": {"bound": "mfma", "kernel": "whole prompt pass (GEMMs + causal attention + glue)",
+                     "achieved": round(tf, 1), "peak": PEAKS_TFLOPS["bf16"], "unit": "TFLOP/s",
+                     "frac": round(tf / PEAKS_TFLOPS["bf16"], 4), "traffic": None,
+                     "flops_per_step": lin_flops + attn_flops},
+        "cpu_baseline": None}
+
+
+def leg_as_line(leg, args):
+    """A leg run alone (--workload ...) printed in the shape of the headline line."""
+    return {"metric": leg["metric"], "value": leg["value"], "unit": leg["unit"], "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": leg.get("ms_per_step", leg.get("us_per_call", 0.0) / 1e3),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": leg["dtype"],
+            "data": "synthetic", "config": {k: v for k, v in leg.items() if k not in ("roofline", "cpu_baseline", "metric",
+                                                                                      "value", "unit", "dtype")},
+            "roofline": leg["roofline"], "cpu_baseline": leg["cpu_baseline"]}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--fmt", default="qint8", choices=["qint8", "mxfp4"])
+    ap.add_argument("--batch", type=int, default=1, help="sequences for --workload tokens (1 or 16 in the baseline)")
+    ap.add_argument("--workload", default="all", choices=["all", "decode", "cfg1", "cfg3", "prefill", "tokens", "prompt"],
+                    help="all = the headline (config 2) plus every other leg of the metric under config.legs (default); "
+                         "decode = the headline alone; cfg1 / cfg3 / prefill (config 4) / tokens (config 5) = that leg "
+                         "alone; prompt = a 2048-token prompt through the 7B-shape decoder")
+    ap.add_argument("--prefill-fmt", default="mxfp4", choices=["mxfp4", "qint8"],
+                    help="weight format of --workload prefill (BASELINE config 4 is MXFP4; qint8 = the same layer W8A8)")
+    ap.add_argument("--act-fp8", action="store_true",
+                    help="--workload prefill, MXFP4: quantise activations to MXFP8 and use the block-scaled MFMA "
+                         "(opt-in; not the reference's arithmetic, whose activations stay bf16)")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--pool", type=int, default=2, help="number of distinct weight sets cycled through")
+    ap.add_argument("--pmc-calibrate", action="store_true",
+                    help="also run three plain 256 MiB device copies, the known-size reference for scaling "
+                         "FETCH_SIZE / WRITE_SIZE counter readings")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus must be 1 (every box has one GPU and the "
+              "path has no collectives)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import tpp_pytorch_extension  # noqa: F401
+    from tpp_pytorch_extension import _ops
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(torch.device("cuda:0"))
+
+    if args.workload == "cfg1":
+        return print(json.dumps(leg_as_line(leg_cfg1(torch, _ops, args), args)))
+    if args.workload == "cfg3":
+        return print(json.dumps(leg_as_line(leg_cfg3(torch, _ops, args), args)))
+    if args.workload == "prefill":
+        return print(json.dumps(leg_as_line(leg_cfg4(torch, _ops, args, args.prefill_fmt, args.act_fp8), args)))
+    if args.workload == "tokens":
+        return print(json.dumps(leg_as_line(leg_cfg5(torch, args, args.batch), args)))
+    if args.workload == "prompt":
+        return print(json.dumps(run_prompt(torch, args)))
+
+    t_start = time.perf_counter()
+    out = run_decode(torch, _ops, args)
+    if args.workload == "all":
+        legs = []
+        todo = [
+            ("cfg1", lambda: leg_cfg1(torch, _ops, args)),
+            ("cfg3", lambda: leg_cfg3(torch, _ops, args)),
+            ("cfg4", lambda: leg_cfg4(torch, _ops, args, "mxfp4", False)),
+            ("cfg4-qint8", lambda: leg_cfg4(torch, _ops, args, "qint8", False)),
+            ("cfg4-act-fp8", lambda: leg_cfg4(torch, _ops, args, "mxfp4", True)),
+            ("cfg5-batch1", lambda: leg_cfg5(torch, args, 1)),
+            ("cfg5-batch16", lambda: leg_cfg5(torch, args, 16)),
+        ]
+        for name, fn in todo:
+            t0 = time.perf_counter()
+            if t0 - t_start > 420.0:  # the whole run stays well inside ten minutes
+                legs.append({"leg": name, "skipped": "time budget of the run used up"})
+                continue
+            try:
+                leg = fn()
+            except Exception as e:  # a leg that fails must not take the headline with it
+                leg = {"leg": name, "error": repr(e)[:300]}
+            leg["leg_wall_s"] = round(time.perf_counter() - t0, 1)
+            legs.append(leg)
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+        _MODEL.clear()
+        out["config"]["legs"] = legs
+        out["config"]["run_wall_s"] = round(time.perf_counter() - t_start, 1)
+    print(json.dumps(out))
 
 
 if __name__ == "__main__":

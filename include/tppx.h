@@ -389,6 +389,15 @@ int tppx_plan_linear_qint8(int64_t M, int64_t N, int64_t K, int64_t qbs,
                            int x_given, int flags, int64_t ws_bytes, char* buf,
                            int64_t buf_len);
 
+/* The same for a fused group: Ns[n_segs] output widths over one activation (tppx_multi_linear_*), or, with
+ * dual = 1 and two equal widths, the gate/up pair of tppx_swiglu_mxfp4. */
+int tppx_plan_multi_linear_mxfp4(const int64_t* Ns, int n_segs, int64_t M,
+                                 int64_t K, int dual, int flags,
+                                 int64_t ws_bytes, char* buf, int64_t buf_len);
+int tppx_plan_multi_linear_qint8(const int64_t* Ns, int n_segs, int64_t M,
+                                 int64_t K, int64_t qbs, int x_given, int flags,
+                                 int64_t ws_bytes, char* buf, int64_t buf_len);
+
 #ifdef __cplusplus
 }
 #endif

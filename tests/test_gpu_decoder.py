@@ -414,6 +414,12 @@ def test_greedy_decode_graph_equals_eager():
     a = model.greedy_decode(tok, model.new_cache(3, 40, 64), 8, use_graph=False)
     b = model.greedy_decode(tok, model.new_cache(3, 40, 64), 8, use_graph=True)
     assert a.shape == (3, 8) and torch.equal(a, b)
+    # a replayed step checks nothing on the host: runs that would overrun the cache or the rotary table are refused
+    from tpp_pytorch_extension._lib import TppxError
+    with pytest.raises(TppxError):
+        model.greedy_decode(tok, model.new_cache(3, 40, 44), 8)
+    with pytest.raises(TppxError):
+        model.greedy_decode(tok, model.new_cache(3, 250, 300), 8)
 
 
 @pytest.mark.parametrize("M", [1, 5, 16])

@@ -715,3 +715,34 @@ extern "C" int tppx_plan_linear_qint8(int64_t M, int64_t N, int64_t K, int64_t q
                      ws_bytes > 0 ? a : nullptr, ws_bytes, nullptr);
   return emit_plan("tppx_plan_linear_qint8", rc, text, buf, buf_len);
 }
+
+// the same for a fused group (q/k/v: dual = 0; the gate/up pair of tppx_swiglu_mxfp4: dual = 1, two equal Ns)
+extern "C" int tppx_plan_multi_linear_mxfp4(const int64_t* Ns, int n_segs, int64_t M, int64_t K, int dual, int flags,
+                                            int64_t ws_bytes, char* buf, int64_t buf_len) {
+  const char* who = "tppx_plan_multi_linear_mxfp4";
+  TPPX_REQUIRE(Ns && n_segs >= 1 && n_segs <= TPPX_MAX_SEGS && (!dual || n_segs == 2), TPPX_EINVAL,
+               "%s: bad segment list", who);
+  void* a = reinterpret_cast<void*>(uintptr_t(1) << 20);
+  tppx_seg s[TPPX_MAX_SEGS];
+  for (int i = 0; i < n_segs; i++)
+    s[i] = {a, a, nullptr, nullptr, nullptr, a, Ns[i], TPPX_POST_NONE, 1.0f};
+  std::string text;
+  g_plan = &text;
+  int rc = run_mxfp4(who, a, s, n_segs, M, K, flags, dual != 0, ws_bytes > 0 ? a : nullptr, ws_bytes, nullptr);
+  return emit_plan(who, rc, text, buf, buf_len);
+}
+
+extern "C" int tppx_plan_multi_linear_qint8(const int64_t* Ns, int n_segs, int64_t M, int64_t K, int64_t qbs,
+                                            int x_given, int flags, int64_t ws_bytes, char* buf, int64_t buf_len) {
+  const char* who = "tppx_plan_multi_linear_qint8";
+  TPPX_REQUIRE(Ns && n_segs >= 1 && n_segs <= TPPX_MAX_SEGS, TPPX_EINVAL, "%s: bad segment list", who);
+  void* a = reinterpret_cast<void*>(uintptr_t(1) << 20);
+  tppx_seg s[TPPX_MAX_SEGS];
+  for (int i = 0; i < n_segs; i++)
+    s[i] = {a, a, nullptr, nullptr, nullptr, a, Ns[i], TPPX_POST_NONE, 1.0f};
+  std::string text;
+  g_plan = &text;
+  int rc = run_qint8(who, x_given ? a : nullptr, a, a, s, n_segs, M, K, qbs, flags, ws_bytes > 0 ? a : nullptr, ws_bytes,
+                     nullptr);
+  return emit_plan(who, rc, text, buf, buf_len);
+}

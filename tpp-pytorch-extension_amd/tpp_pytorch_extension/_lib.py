@@ -76,6 +76,9 @@ SIGNATURES = {
     "tppx_attn_prefill": [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     "tppx_plan_linear_mxfp4": [_i64, _i64, _i64, _i32, _i64, ctypes.c_char_p, _i64],
     "tppx_plan_linear_qint8": [_i64, _i64, _i64, _i64, _i32, _i32, _i64, ctypes.c_char_p, _i64],
+    "tppx_plan_multi_linear_mxfp4": [ctypes.POINTER(_i64), _i32, _i64, _i64, _i32, _i32, _i64, ctypes.c_char_p, _i64],
+    "tppx_plan_multi_linear_qint8": [ctypes.POINTER(_i64), _i32, _i64, _i64, _i64, _i32, _i32, _i64, ctypes.c_char_p,
+                                     _i64],
 }
 
 _lib = None

@@ -300,9 +300,21 @@ class LlamaDecoder:
         rest = self.greedy_decode(first, cache, n_new - 1, use_graph=use_graph)
         return torch.cat([first.view(B, 1), rest], dim=1)
 
+    def _check_room(self, cache, n_new):
+        """A replayed decode step checks nothing on the host: past the cache's capacity the kernels drop the new
+        key / value, past the rotary table they skip the rotation.  Refuse such a run up front."""
+        start = cache.get_seq_length()
+        if start + n_new > cache.get_capacity():
+            raise TppxError(_lib.ESHAPE, f"decoding {n_new} tokens from position {start} overruns the cache "
+                                         f"capacity {cache.get_capacity()}")
+        if start + n_new > self.EP.shape[1]:
+            raise TppxError(_lib.ESHAPE, f"decoding {n_new} tokens from position {start} overruns the rotary table "
+                                         f"({self.EP.shape[1]} positions)")
+
     def time_decode_steps(self, tokens, cache, n_new):
         """Seconds spent in n_new replays of the captured decode step (capture excluded)."""
         import time
+        self._check_room(cache, n_new + 1)  # one untimed eager step precedes the replays
         B = tokens.shape[0]
         cur = tokens.clone()
         pos = torch.full((B, 1), cache.get_seq_length(), dtype=torch.int64, device=self.device)
@@ -324,6 +336,7 @@ class LlamaDecoder:
 
     def greedy_decode(self, tokens, cache, n_new, use_graph=True):
         """Greedy decode of n_new tokens per sequence from the [B] start tokens; returns i64 [B][n_new]."""
+        self._check_room(cache, n_new)
         B = tokens.shape[0]
         cur = tokens.clone()
         pos = torch.full((B, 1), cache.get_seq_length(), dtype=torch.int64, device=self.device)
