@@ -116,6 +116,63 @@ int tppx_dequantize_qint8(const void* q, const void* scales, int64_t N,
                           int64_t K, int64_t qbs, void* out_f32,
                           tppx_stream_t stream);
 
+/* Per-block formats of the generic helpers below. */
+#define TPPX_Q_MXFP4 0 /* E2M1 codes, two per byte, E8M0 scale byte per block */
+#define TPPX_Q_INT8 1  /* int8, fp32 scale = max/127                          */
+#define TPPX_Q_INT4 2  /* two's complement nibbles, two per byte, fp32 scale = max/7 */
+
+/* Replace quantize_mxfp4 / quantize_int8sym / quantize_int4sym on ANY layout
+ * (src/csrc/qtypes.cpp:602-637 -> PerBlockQuantizer::quantize_symetric,
+ * src/csrc/qtypes.h:30-68,133-193) and the matching dequantize
+ * (qtypes.h:196-243).  The tensor is viewed as in[pre][bs][post][vnni] --
+ * the geometry PerBlockQuantizer derives from (sizes, block_size, axis,
+ * is_vnni): with is_vnni the last dimension is vnni and block_size / vnni
+ * consecutive indices of `axis` form a block; without it the axis is the last
+ * dimension, vnni = the format's pack size (2 for the 4-bit formats, 1 for
+ * int8) -- and one block = the bs * vnni elements sharing (pre, post).
+ * out: same order, 4-bit formats with two codes per byte (element 2*v1 in the
+ * low nibble); scales[pre][post] (u8 for MXFP4, f32 otherwise). */
+int tppx_quantize_per_block(const void* in, int in_dtype, int qfmt, int64_t pre,
+                            int64_t bs, int64_t post, int64_t vnni, void* out,
+                            void* scales, tppx_stream_t stream);
+int tppx_dequantize_per_block(const void* q, const void* scales, int qfmt,
+                              int64_t pre, int64_t bs, int64_t post,
+                              int64_t vnni, void* out_f32, tppx_stream_t stream);
+
+/* Replaces qtype.remap_and_quantize_qint2_intlv (src/csrc/qtypes.cpp:1004-1073;
+ * bound at :1092; the "qint2" choice of FixLinear, llm_common.py:506-509) for
+ * N % 32 == 0: ternary weights, scale = max(|w|, 1e-8) per (output channel,
+ * block of bs input channels), code 0 / 1 / 2 for 0 / +1 / -1, four codes per
+ * byte interleaved over output channels:
+ *   q      u8  [N/32][K/bs][bs/4][8 k2][4 c3]: bits 2*k3 hold the code of
+ *              W[n1*32 + k3*8 + k2][b*bs + c2*4 + c3]
+ *   scales f32 [N/32][K/bs][32]
+ * `w` is a blocked weight as for tppx_quantize_mxfp4.  The reference's own
+ * dequantize() of such a tensor indexes a 4-entry table with whole bytes
+ * (qtypes.h:232-239), so tppx_dequantize_qint2_intlv defines the meaningful
+ * result instead: code value * scale in the logical blocked shape
+ * [N/32][K/bs][bs/4][32][4]. */
+int tppx_quantize_qint2_intlv(const void* w, int w_dtype, int64_t N, int64_t K,
+                              int64_t bk, int64_t bc, int64_t vnni, int64_t bs,
+                              void* q, void* scales, tppx_stream_t stream);
+int tppx_dequantize_qint2_intlv(const void* q, const void* scales, int64_t N,
+                                int64_t K, int64_t bs, void* out_f32,
+                                tppx_stream_t stream);
+
+/* Low-bit affine weights run on the W8A8 kernels (TppBlockedQInt8LinearW takes
+ * kQUInt4x2 / kQUInt2x4 weights with int8 activations and int32 block sums,
+ * src/csrc/fused_gemm.h:1112-1128): a one-time expansion of the packed codes
+ * into the native int8 tiles tppx_linear_qint8 consumes (qbs = bs).
+ * tppx_prepack_qint2: the interleaved layout above -> q_nat i8 (N*K bytes) and
+ * scales_nat f32 [N/16][K/bs][16].  tppx_prepack_qint4: an INT4 weight in the
+ * VNNI2 layout [N/16][K/bs][bs/2][16] bytes (two codes each) -> q_nat; its
+ * scales [N/16][K/bs][1][16] are used unchanged. */
+int tppx_prepack_qint2(const void* q_ref, const void* scales_ref, int64_t N,
+                       int64_t K, int64_t bs, void* q_nat, void* scales_nat,
+                       tppx_stream_t stream);
+int tppx_prepack_qint4(const void* q_ref, int64_t N, int64_t K, int64_t bs,
+                       void* q_nat, tppx_stream_t stream);
+
 /* Reference layout -> native layout.  Plays the role of the reference's cached
  * first-token weight remap (wt_tensor_for_first_token,
  * src/csrc/llm/fused_llm_infer.cpp:366-420): a one-time re-layout kept next to

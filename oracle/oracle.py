@@ -322,6 +322,79 @@ def dequantize_int8sym(q, sc, block_size, axis, is_vnni):
     return out
 
 
+def quantize_int4sym(t, block_size, axis, is_vnni):
+    """quantize_int4sym (qtypes.cpp:626-637, Int4SymQuant :199-246) on an fp32 array.
+    Returns (packed uint8 with the last dim halved, fp32 scales)."""
+    t = _c(t, np.float32)
+    pre, bs, post, vnni, ssz = _per_block_geometry(t.shape, block_size, axis, is_vnni, 2)
+    out = np.empty(t.shape[:-1] + (t.shape[-1] // 2,), np.uint8)
+    sc = np.empty(ssz, np.float32)
+    lib().orc_int4_quantize_generic(_p(t), _c_i64(pre), _c_i64(bs), _c_i64(post), _c_i64(vnni), _p(out), _p(sc))
+    return out, sc
+
+
+def dequantize_int4sym(q, sc, block_size, axis, is_vnni):
+    q = _c(q, np.uint8)
+    sc = _c(sc, np.float32)
+    shape = q.shape[:-1] + (q.shape[-1] * 2,)
+    pre, bs, post, vnni, _ = _per_block_geometry(shape, block_size, axis, is_vnni, 2)
+    out = np.empty(shape, np.float32)
+    lib().orc_int4_dequantize_generic(_p(q), _p(sc), _c_i64(pre), _c_i64(bs), _c_i64(post), _c_i64(vnni), _p(out))
+    return out
+
+
+def qint2_block_size(K, env_block=256):
+    """Block rule of remap_and_quantize_qint2_intlv (qtypes.cpp:1031-1043): QINT2_BLOCK_SIZE if it divides the
+    input channels, else the largest smaller power of two >= 64 that does."""
+    return qint8_block_size(K, env_block)
+
+
+def remap_quantize_qint2_intlv(W, bs=None, env_block=256):
+    """remap_and_quantize_qint2_intlv (qtypes.cpp:1004-1073) on a plain fp32 W[N][K], N % 32 == 0:
+    -> (packed uint8 [N/32][K/bs][bs/4][8][4], fp32 scales [N/32][K/bs][32][1], bs).
+    The logical (unpacked) tensor is [N/32][K/bs][bs/4][32][4]."""
+    W = _c(W, np.float32)
+    N, K = W.shape
+    if bs is None:
+        bs = qint2_block_size(K, env_block)
+    assert N % 32 == 0 and K % bs == 0 and bs % 4 == 0
+    q = np.empty((N // 32, K // bs, bs // 4, 8, 4), np.uint8)
+    sc = np.empty((N // 32, K // bs, 32, 1), np.float32)
+    lib().orc_remap_quantize_qint2_intlv(_p(W), _c_i64(N), _c_i64(K), _c_i64(bs), _p(q), _p(sc))
+    return q, sc, bs
+
+
+def remap_quantize_qint2_intlv_chain(W, bs):
+    """The same through a restatement of the reference's own view / permute / pack chain (numpy), the check of
+    the closed form above.  W plain [N][K] fp32 (the reference first flattens its blocked input to this)."""
+    W = np.ascontiguousarray(W, np.float32)
+    N, K = W.shape
+    K1, K2, K3, C3 = N // 32, 8, 4, 4
+    C1, C2 = K // bs, bs // C3
+    t = W.reshape(K1, K2 * K3, C1, bs).transpose(0, 2, 1, 3)
+    amax = np.abs(t).max(-1, keepdims=True)
+    scales = np.maximum(amax.astype(np.float32), np.float32(1.0e-8))
+    qv = np.clip(np.rint((t / scales).astype(np.float32)), -1.0, 1.0).astype(np.int32).astype(np.uint8) & 0x3
+    qv[qv == 3] = 2
+    qv = np.ascontiguousarray(qv).reshape(K1, C1, K3, K2, C2, C3).transpose(2, 0, 1, 4, 3, 5)
+    packed = qv[0] | (qv[1] << 2) | (qv[2] << 4) | (qv[3] << 6)
+    return np.ascontiguousarray(packed).astype(np.uint8), np.ascontiguousarray(scales)
+
+
+def qint2_to_qint8_layout(q2, sc2):
+    """Ternary codes {0: 0, 1: +1, 2: -1} and scales of the interleaved 2-bit layout as an int8 weight in the QINT8
+    reference layout (q [N/16][K/bs][bs/4][16][4] i8, scales [N/16][K/bs][1][16]): the operand the W2A8 GEMM
+    (TppBlockedQInt8LinearW on a kQUInt2x4 weight, src/csrc/fused_gemm.h:1112-1128) multiplies."""
+    q2 = _c(q2, np.uint8)
+    n1, nb, c2, _, _ = q2.shape
+    codes = np.stack([(q2 >> (2 * k3)) & 3 for k3 in range(4)], axis=3)        # [n1][nb][c2][k3][k2][c3]
+    val = np.where(codes == 1, 1, np.where(codes == 2, -1, 0)).astype(np.int8)
+    val = val.reshape(n1, nb, c2, 32, 4)                                        # row r = k3*8 + k2
+    val = val.reshape(n1, nb, c2, 2, 16, 4).transpose(0, 3, 1, 2, 4, 5).reshape(n1 * 2, nb, c2, 16, 4)
+    sc = _c(sc2, np.float32).reshape(n1, nb, 2, 16).transpose(0, 2, 1, 3).reshape(n1 * 2, nb, 1, 16)
+    return np.ascontiguousarray(val), np.ascontiguousarray(sc)
+
+
 def remap_and_quantize_mxfp4_blocked(Wb):
     """Full reference entry point on a blocked fp32 array (view/permute chain
     + generic quantiser).  -> (qdata [N/32,K/64,32,32] u8, scales [N/32,K/64,2,32] u8)"""

@@ -430,6 +430,105 @@ ORC_API void orc_dequantize_qint8(const int8_t* q, const float* scales,
 }
 
 /* ------------------------------------------------------------------ */
+/* INT4 symmetric (Int4SymQuant, src/csrc/qtypes.cpp:199-246)           */
+/* ------------------------------------------------------------------ */
+/* scale = (float)(max / 7.0) (double division, narrowed), inverse in fp32,
+ * q = clamp(nearbyintf(w * iscale), -8, 7); two codes per byte, element v2
+ * of a pair in bits 4*v2 (two's complement nibble), as
+ * PerBlockQuantizer::quantize_symetric packs them (qtypes.h:166-178).
+ * Geometry as for the other generic quantisers:
+ * in[pre][bs][post][vnni] -> out[pre][bs][post][vnni/2], scales[pre][post]. */
+static const int int4_tbl[16] = {0, 1, 2, 3, 4, 5, 6, 7, -8, -7, -6, -5, -4, -3, -2, -1};
+
+ORC_API void orc_int4_quantize_generic(const float* in, int64_t pre, int64_t bs,
+                                       int64_t post, int64_t vnni, uint8_t* out,
+                                       float* scales) {
+  int64_t pv = vnni / 2;
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t i = 0; i < pre; i++)
+    for (int64_t j = 0; j < post; j++) {
+      const float* base = in + (i * bs * post + j) * vnni;
+      float amax = fabsf(base[0]);
+      for (int64_t k = 0; k < bs; k++)
+        for (int64_t v = 0; v < vnni; v++) {
+          float a = fabsf(base[k * post * vnni + v]);
+          amax = a > amax ? a : amax;
+        }
+      float s = (float)((double)amax / 7.0);
+      float inv = (s != 0.0f) ? (1.0f / s) : 0.0f;
+      scales[i * post + j] = s;
+      for (int64_t k = 0; k < bs; k++)
+        for (int64_t v1 = 0; v1 < pv; v1++) {
+          unsigned packed = 0;
+          for (int v2 = 0; v2 < 2; v2++) {
+            float r = nearbyintf(base[k * post * vnni + v1 * 2 + v2] * inv);
+            int q = r < -8.0f ? -8 : (r > 7.0f ? 7 : (int)r);
+            packed |= ((unsigned)q & 0xf) << (4 * v2);
+          }
+          out[(i * bs * post + k * post + j) * pv + v1] = (uint8_t)packed;
+        }
+    }
+}
+
+/* value = lkp_tbl[code] * scale (qtypes.cpp:241-244, qtypes.h:196-243) */
+ORC_API void orc_int4_dequantize_generic(const uint8_t* in, const float* scales,
+                                         int64_t pre, int64_t bs, int64_t post,
+                                         int64_t vnni, float* out) {
+  int64_t pv = vnni / 2;
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t i = 0; i < pre; i++)
+    for (int64_t j = 0; j < post; j++) {
+      float s = scales[i * post + j];
+      for (int64_t k = 0; k < bs; k++)
+        for (int64_t v1 = 0; v1 < pv; v1++) {
+          unsigned b = in[(i * bs * post + k * post + j) * pv + v1];
+          for (int v2 = 0; v2 < 2; v2++)
+            out[(i * bs * post + k * post + j) * vnni + v1 * 2 + v2] =
+                (float)int4_tbl[(b >> (4 * v2)) & 0xf] * s;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* QINT2 interleaved (ternary weights)                                 */
+/* ------------------------------------------------------------------ */
+/* remap_and_quantize_qint2_intlv (src/csrc/qtypes.cpp:1004-1073) for N % 32
+ * == 0 (K2 = 8, K3 = 4, C3 = 4) and a block of bs input channels:
+ *   scale[n][b] = max(|W[n][b*bs ..]|, 1e-8)           (abs max, clamp_min)
+ *   t = round_half_even(W / scale) clamped to [-1, 1]  (fp32 division)
+ *   code: 0 -> 0, +1 -> 1, -1 -> 2   (uint8(-1) & 3 = 3, then 3 -> 2)
+ *   byte[n1][b][c2][k2][c3] = code(n1*32 + 0*8 + k2) | code(.. 1*8 ..) << 2 |
+ *                             code(.. 2*8 ..) << 4 | code(.. 3*8 ..) << 6
+ *     at input channel b*bs + c2*4 + c3
+ *   scales [N/32][K/bs][32]  (row r = k3*8 + k2 of the 32-channel group) */
+ORC_API void orc_remap_quantize_qint2_intlv(const float* W, int64_t N, int64_t K,
+                                            int64_t bs, uint8_t* q, float* scales) {
+  int64_t N1 = N / 32, nb = K / bs, C2 = bs / 4;
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t n1 = 0; n1 < N1; n1++)
+    for (int64_t b = 0; b < nb; b++) {
+      uint8_t* qb = q + (n1 * nb + b) * C2 * 32;
+      memset(qb, 0, (size_t)(C2 * 32));
+      for (int r = 0; r < 32; r++) {
+        const float* row = W + (n1 * 32 + r) * K + b * bs;
+        float amax = 0.0f;
+        for (int64_t c = 0; c < bs; c++) {
+          float a = fabsf(row[c]);
+          amax = a > amax ? a : amax;
+        }
+        float s = amax < 1.0e-8f ? 1.0e-8f : amax;
+        scales[(n1 * nb + b) * 32 + r] = s;
+        int k3 = r >> 3, k2 = r & 7;
+        for (int64_t c = 0; c < bs; c++) {
+          float t = nearbyintf(row[c] / s);
+          unsigned code = t >= 1.0f ? 1u : (t <= -1.0f ? 2u : 0u);
+          qb[((c >> 2) * 8 + k2) * 4 + (c & 3)] |= (uint8_t)(code << (2 * k3));
+        }
+      }
+    }
+}
+
+/* ------------------------------------------------------------------ */
 /* Post-ops on the bf16 output tile                                    */
 /* ------------------------------------------------------------------ */
 enum {

@@ -642,3 +642,34 @@ def test_lm_head_quantized_on_request():
         la, lb, lc = (m(input_ids=ids).logits.float() for m in (a, b, c))
     assert torch.equal(lb, lc)
     assert float((lb - la).norm() / la.norm()) <= 2e-2
+
+
+def test_cache_update_appends_and_grows():
+    """TppCache.update (attn.h:198-222,258-274): append [B][Nkv][S][H] states layer by layer, per-layer lengths,
+    growth past the capacity, and attention over the updated cache equals attention over the concatenated keys."""
+    F = _llm()
+    from tpp_pytorch_extension.llm.llm_common import TppCache as HFCache
+    B, Nkv, H = 2, 2, 128
+    cache = HFCache(capacity=0)
+    k1, v1 = randn_bf16((B, Nkv, 40, H), 1.0, 901).cuda(), randn_bf16((B, Nkv, 40, H), 1.0, 902).cuda()
+    k2, v2 = randn_bf16((B, Nkv, 3, H), 1.0, 903).cuda(), randn_bf16((B, Nkv, 3, H), 1.0, 904).cuda()
+    for layer in (0, 1):
+        ks, vs = cache.update(k1, v1, layer)
+        assert ks.shape == (B, Nkv, 40, H) and torch.equal(ks, k1) and torch.equal(vs, v1)
+    assert cache.get_seq_length() == 40 and len(cache) == 2
+    cap0 = cache.get_max_length()
+    assert cap0 >= 40 + 128 and cap0 % 32 == 0          # grew by KV_CACHE_INC_SIZE beyond the need, whole blocks
+    ks, vs = cache.update(k2, v2, 0)
+    assert cache.get_seq_length(0) == 43 and cache.get_seq_length(1) == 40
+    ks1, _ = cache.update(k2, v2, 1)
+    assert torch.equal(ks, torch.cat([k1, k2], 2)) and torch.equal(ks1, ks)
+    big = randn_bf16((B, Nkv, cap0, H), 1.0, 905).cuda()
+    ks, _ = cache.update(big, big, 0)                    # past the capacity: storage is reallocated, contents kept
+    assert cache.get_max_length() >= 43 + cap0 and torch.equal(ks[:, :, :43], torch.cat([k1, k2], 2))
+    core = cache.get_cpp()
+    q = randn_bf16((B, 4, H), 1.0, 906)
+    kc, vc = core.layers[1]
+    got = _attn(F, q.cuda(), kc, vc, 43)
+    ref = O.attn_decode(t2bits(q), t2bits(torch.cat([k1, k2], 2)), t2bits(torch.cat([v1, v2], 2)))
+    g, r = bits2f(t2bits(got)).astype(np.float64), bits2f(ref).astype(np.float64)
+    assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3

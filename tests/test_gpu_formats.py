@@ -1,0 +1,152 @@
+"""The helper set on arbitrary layouts and the low-bit affine weight formats.
+
+* quantize_mxfp4 / quantize_int8sym / quantize_int4sym(t, block_size, axis, is_vnni) on layouts other than the two
+  linear-layer weight layouts, and dequantize() of every such tensor (quantized activations included): bytes, scales
+  and fp32 values equal the oracle's generic per-block functions (PerBlockQuantizer, src/csrc/qtypes.h:30-243).
+* remap_and_quantize_qint2_intlv (src/csrc/qtypes.cpp:1004-1073, the "qint2" choice of FixLinear): packed bytes and
+  scales equal the oracle (itself pinned against a restatement of the reference's view / permute / pack chain), and
+  the W2A8 linear on it equals the W8A8 oracle on the ternary weight (exact int32 block sums, same scales).
+* quantize_int4sym on the VNNI2 weight layout feeds the linears the same way.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from util import t2bits, randn_bf16, block_bf16, assert_close_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    import tpp_pytorch_extension  # noqa: F401
+    from tpp_pytorch_extension import _ops
+    return _ops
+
+
+GEOMS = [
+    # shape, block_size, axis, is_vnni
+    ((6, 96), 32, -1, False),            # plain rows, blocks along the last axis
+    ((3, 5, 128), 64, 2, False),
+    ((4, 2, 16, 8, 2), 32, 2, True),     # VNNI2 weight-like with 8-channel blocks
+    ((2, 3, 64, 10, 4), 128, 2, True),   # VNNI4, odd channel count
+    ((2, 64, 3, 2), 64, 1, True),        # blocks along axis 1, two trailing dims
+]
+
+
+@pytest.mark.parametrize("shape,bs,axis,vnni", GEOMS)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("fmt", ["mxfp4", "int8", "int4"])
+def test_generic_quantize_and_dequantize(shape, bs, axis, vnni, dtype, fmt):
+    ops = _ops()
+    g = torch.Generator().manual_seed(hash((shape, bs, fmt)) % 1000)
+    t = (torch.randn(shape, generator=g) * 0.7).to(dtype)
+    t.view(-1)[::17] = 0.0
+    t.view(-1)[3] = 5.0
+    ref_in = t.float().numpy()
+    if fmt == "mxfp4":
+        qt = ops.quantize_mxfp4(t.cuda(), bs, axis, vnni)
+        q_or, s_or = O.quantize_mxfp4(ref_in, bs, axis, vnni)
+        d_or = O.dequantize_mxfp4(q_or, s_or, bs, axis, vnni)
+        assert qt.dtype == torch.quint4x2 and ops.q_per_block_pack_size(qt) == 2
+    elif fmt == "int8":
+        qt = ops.quantize_int8sym(t.cuda(), bs, axis, vnni)
+        q_or, s_or = O.quantize_int8sym(ref_in, bs, axis, vnni)
+        d_or = O.dequantize_int8sym(q_or, s_or, bs, axis, vnni)
+        assert qt.dtype == torch.qint8 and ops.q_per_block_pack_size(qt) == 1
+    else:
+        qt = ops.quantize_int4sym(t.cuda(), bs, axis, vnni)
+        q_or, s_or = O.quantize_int4sym(ref_in, bs, axis, vnni)
+        d_or = O.dequantize_int4sym(q_or, s_or, bs, axis, vnni)
+        assert qt.dtype == torch.quint4x2
+    assert qt.is_quantized and tuple(qt.shape) == tuple(shape)
+    assert ops.q_per_block_block_size(qt) == bs and ops.q_per_block_axis(qt) == (axis % len(shape))
+    assert np.array_equal(ops.q_per_block_scales(qt).cpu().numpy().reshape(s_or.shape), s_or)
+    assert np.array_equal(qt.qdata.cpu().numpy().reshape(q_or.shape), q_or)
+    d = qt.dequantize()
+    assert d.dtype == torch.float32 and tuple(d.shape) == tuple(shape)
+    assert np.array_equal(d.cpu().numpy().view(np.uint32), d_or.view(np.uint32))
+
+
+def test_activation_qtensor_dequantizes():
+    """quantize_int8sym(x, QBS, -1, False) on bf16 activations (the call the W8A8 linear makes, fused_gemm.h:1249)
+    gives a tensor whose dequantize() is q * scale per (row, block)."""
+    ops = _ops()
+    x = randn_bf16((3, 7, 512), 1.0, 77)
+    qt = ops.quantize_int8sym(x.cuda(), 256, -1, False)
+    xq, sa = O.quant_act_int8(t2bits(x).reshape(21, 512), 256)
+    assert np.array_equal(qt.qdata.cpu().numpy().reshape(21, 512), xq)
+    want = O.dequantize_int8sym(xq, sa, 256, 1, False)
+    assert np.array_equal(qt.dequantize().cpu().numpy().reshape(21, 512), want)
+
+
+@pytest.mark.parametrize("N,K", [(64, 256), (4096, 1024), (96, 11008)])
+@pytest.mark.parametrize("src", ["bf16_5d", "f32_4d"])
+def test_qint2_quantizer_bit_exact(N, K, src):
+    ops = _ops()
+    W = randn_bf16((N, K), 0.02, 31 + N)
+    W[5, :128] = 0.0
+    W[7] = 0.0          # an all-zero (channel, block): scale clamps to 1e-8, codes 0
+    W[9, 3] = 0.5 * W[9, :256].abs().max()  # an exact tie at 0.5: rounds to even (0)
+    if src == "bf16_5d":
+        qt = ops.remap_and_quantize_qint2_intlv(block_bf16(W).cuda())
+    else:
+        Wf = W.float()
+        qt = ops.remap_and_quantize_qint2_intlv(Wf.view(N // 16, 16, K // 64, 64).permute(0, 2, 3, 1).contiguous().cuda())
+    q_or, s_or, bs = O.remap_quantize_qint2_intlv(W.float().numpy())
+    assert ops.q_per_block_block_size(qt) == bs and qt.dtype == torch.quint2x4 and ops.q_per_block_pack_size(qt) == 4
+    assert tuple(qt.shape) == (N // 32, K // bs, bs // 4, 32, 4)
+    assert np.array_equal(qt.scales.cpu().numpy(), s_or)
+    assert np.array_equal(qt.qdata.cpu().numpy(), q_or)
+    # dequantize = ternary value * scale in the logical blocked shape
+    v8, s8 = O.qint2_to_qint8_layout(q_or, s_or)
+    Wd = O.dequantize_qint8_plain(v8, s8)                                    # plain [N][K]
+    want = Wd.reshape(N // 32, 32, K // bs, bs // 4, 4).transpose(0, 2, 3, 1, 4)
+    assert np.array_equal(qt.dequantize().cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("M", [1, 8, 40, 200])
+def test_qint2_linear(M):
+    """W2A8: int8 activations per 256-block x ternary weights, exact int32 block sums, fp32 scales -- the W8A8
+    oracle on the expanded weight.  fc_add through the module API (FixLinear weight_dtype="qint2")."""
+    ops = _ops()
+    from tpp_pytorch_extension.llm.llm_common import FixLinear, BlockedLinear
+    N, K = 1024, 2048
+    torch.manual_seed(5)
+    lin = torch.nn.Linear(K, N, bias=True)
+    W = lin.weight.data.clone().to(torch.bfloat16)
+    b = lin.bias.data.clone().to(torch.bfloat16)
+    FixLinear(lin, 16, 64, torch.bfloat16, weight_dtype="qint2")
+    assert isinstance(lin, BlockedLinear) and lin.weight.is_quantized and lin.weight.dtype == torch.quint2x4
+    q_or, s_or, bs = O.remap_quantize_qint2_intlv(W.float().numpy())
+    assert np.array_equal(lin.weight.qdata.cpu().numpy(), q_or)
+    v8, s8 = O.qint2_to_qint8_layout(q_or, s_or)
+    x = randn_bf16((M, K), 1.0, 41)
+    r = randn_bf16((M, N), 1.0, 42)
+    y = torch.ops.tpp_llm.fc_add(x.cuda(), lin.weight, b.cuda(), r.cuda(), 1.0)
+    ref = O.linear_qint8(t2bits(x), v8, s8, t2bits(b), O.POST_ADD_SCALE, t2bits(r), None, 1.0)
+    assert_close_bf16(t2bits(y), ref, what=f"qint2 fc_add M={M}", pre_bits=O.linear_qint8(t2bits(x), v8, s8, t2bits(b)))
+    y2 = lin.cuda()(x.cuda())
+    assert_close_bf16(t2bits(y2), O.linear_qint8(t2bits(x), v8, s8, t2bits(b)), what=f"qint2 module M={M}")
+
+
+@pytest.mark.parametrize("M", [3, 64, 130])
+def test_qint4_vnni2_weight_linear(M):
+    """quantize_int4sym on a weight in the VNNI2 layout [N/16, K/QBS, QBS/2, 16, 2] gives a tensor the linears accept
+    (kQUInt4x2 + per-block affine -> TppBlockedQInt8LinearW, fused_gemm.h:1530-1534): W4A8 with exact int32 sums."""
+    ops = _ops()
+    N, K, qbs = 512, 1024, 256
+    W = randn_bf16((N, K), 0.02, 51)
+    t = W.view(N // 16, 16, K // qbs, qbs // 2, 2).permute(0, 2, 3, 1, 4).contiguous()
+    qt = ops.quantize_int4sym(t.cuda(), qbs, 2, True)
+    q_or, s_or = O.quantize_int4sym(t.float().numpy(), qbs, 2, True)
+    assert np.array_equal(qt.qdata.cpu().numpy().reshape(q_or.shape), q_or) and np.array_equal(qt.scales.cpu().numpy(), s_or)
+    assert qt.is_weight()
+    # the int8 weight with the same values, in the QINT8 reference layout
+    codes = np.stack([q_or[..., 0] & 0xF, q_or[..., 0] >> 4], axis=-1).astype(np.int16)
+    vals = np.where(codes >= 8, codes - 16, codes).astype(np.int8)            # [N/16][K/qbs][qbs/2][16][2]
+    v8 = vals.reshape(N // 16, K // qbs, qbs // 4, 2, 16, 2).transpose(0, 1, 2, 4, 3, 5).reshape(N // 16, K // qbs, qbs // 4, 16, 4)
+    x = randn_bf16((M, K), 1.0, 52)
+    y = ops.fc_plain(x.cuda(), qt, None)
+    ref = O.linear_qint8(t2bits(x), np.ascontiguousarray(v8), s_or)
+    assert_close_bf16(t2bits(y), ref, what=f"qint4 fc_plain M={M}")

@@ -178,6 +178,54 @@ def test_mx_block_maximum_nan_rule():
     assert deq[4, 33] == 0.0 and deq[4, 34] == 0.5 and deq[0, 0] == 0.5
 
 
+def test_int4_quantizer_closed_form_and_invariants():
+    """Int4SymQuant (qtypes.cpp:199-246): scale = max/7 (double division), codes clamp(rne(w/scale), -8, 7) as two's
+    complement nibbles, low nibble = even element; dequantize = table[code] * scale.  Known answers, the error bound
+    |w - q*s| <= s/2 and brute force against an independent numpy statement."""
+    t = np.array([[7.0, -7.0, 3.5, 2.5, 1.49, -0.5, 0.5, 0.0]], np.float32)          # max 7 -> scale 1
+    q, s = O.quantize_int4sym(t, 8, -1, False)
+    assert s.shape == (1, 1) and s[0, 0] == 1.0
+    codes = np.stack([q[0] & 0xF, q[0] >> 4], -1).reshape(-1)
+    assert codes.tolist() == [7, 9, 4, 2, 1, 0, 0, 0]                               # -7 -> 9, 3.5 -> 4, 2.5 -> 2, -0.5 -> -0
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((5, 3, 64, 6, 2)) * 0.3).astype(np.float32)
+    q, s = O.quantize_int4sym(x, 32, 2, True)
+    d = O.dequantize_int4sym(q, s, 32, 2, True)
+    # independent statement: blocks of 16 x 2 elements along axis 2 sharing (.., k2)
+    xb = x.reshape(5, 3, 4, 16, 6, 2)
+    amax = np.abs(xb).max(axis=(3, 5), keepdims=True)
+    sc = (amax.astype(np.float64) / 7.0).astype(np.float32)
+    inv = np.where(sc != 0, np.float32(1.0) / sc, np.float32(0.0)).astype(np.float32)
+    qq = np.clip(np.rint((xb * inv).astype(np.float32)), -8, 7)
+    assert np.array_equal(s.reshape(5, 3, 4, 6), sc.reshape(5, 3, 4, 6))
+    assert np.array_equal(d.reshape(xb.shape), (qq * sc).astype(np.float32))
+    assert (np.abs(d.reshape(xb.shape) - xb) <= sc / 2 + 1e-12).all()
+
+
+@pytest.mark.parametrize("N,K", [(32, 256), (96, 768), (64, 192)])
+def test_qint2_closed_form_equals_view_permute_chain(N, K):
+    """remap_and_quantize_qint2_intlv (qtypes.cpp:1004-1073): the closed-form C restatement against a numpy
+    restatement of the reference's own view / permute / bit-pack chain; ternary codes, ties to even, zero blocks."""
+    rng = np.random.default_rng(N + K)
+    W = O.bf16_round((rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+    W[1, :64] = 0.0
+    q, sc, bs = O.remap_quantize_qint2_intlv(W)
+    assert bs == O.qint2_block_size(K) and K % bs == 0
+    q2, sc2 = O.remap_quantize_qint2_intlv_chain(W, bs)
+    assert np.array_equal(q, q2) and np.array_equal(sc, sc2)
+    # brute force one element: channel n, input k
+    for n, k in ((0, 0), (13, 77), (31, K - 1), (N - 1, 5)):
+        b, c = divmod(k, bs)
+        s = max(np.abs(W[n, b * bs:(b + 1) * bs]).max(), np.float32(1e-8))
+        t = np.rint(np.float32(W[n, k]) / np.float32(s))
+        code = 1 if t >= 1 else (2 if t <= -1 else 0)
+        n1, r = divmod(n, 32)
+        byte = q[n1, b, c // 4, r % 8, c % 4]
+        assert (byte >> (2 * (r // 8))) & 3 == code and sc[n1, b, r, 0] == s
+    v8, s8 = O.qint2_to_qint8_layout(q, sc)
+    assert set(np.unique(v8).tolist()) <= {-1, 0, 1}
+
+
 def test_layout_brute_force_index_formula():
     N, K = 32, 64
     W = np.arange(N * K, dtype=np.float32).reshape(N, K) % 13 - 6.0

@@ -425,6 +425,219 @@ quant_act_int8_rows_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
   reinterpret_cast<uint4*>(xq + blk * 256)[l] = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
+// ---------------------------------------------------------------------------
+// Generic per-block quantizers: any tensor viewed as in[pre][bs][post][vnni]
+// (the geometry PerBlockQuantizer derives from sizes, block size, axis and the
+// VNNI flag), one block = the bs * vnni elements that share (pre, post).  One
+// thread per block; neighbouring threads own neighbouring `post` positions.
+// The layouts the linears consume have their own, faster kernels above; these
+// serve every other layout the helper functions accept.
+// ---------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float block_amax(const T* base, int64_t bs, int64_t post, int64_t vnni) {
+  // max = |first|, then std::max(max, |v|) as the CPU path has it
+  float amax = fabsf(load_as_f32<T>(base, 0));
+  for (int64_t k = 0; k < bs; k++)
+    for (int64_t v = 0; v < vnni; v++) {
+      const float a = fabsf(load_as_f32<T>(base, k * post * vnni + v));
+      amax = a > amax ? a : amax;
+    }
+  return amax;
+}
+
+template <typename T, int FMT>
+__global__ void __launch_bounds__(256)
+quantize_per_block_kernel(const T* __restrict__ in, int64_t pre, int64_t bs, int64_t post, int64_t vnni,
+                          uint8_t* __restrict__ out, void* __restrict__ scales) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= pre * post)
+    return;
+  const int64_t i = t / post, j = t - i * post;
+  const T* base = in + (i * bs * post + j) * vnni;
+  const float amax = block_amax<T>(base, bs, post, vnni);
+  if (FMT == TPPX_Q_MXFP4) {
+    const int e = (int)((__float_as_uint(amax) >> 23) & 0xffu);
+    const bool flush = (e == 0);
+    const int x = (e == 255) ? 255 : (e - 2 < 0 ? 0 : e - 2);
+    reinterpret_cast<uint8_t*>(scales)[t] = (uint8_t)x;
+    const int sh = 127 - x;
+    const int64_t pv = vnni / 2;
+    for (int64_t k = 0; k < bs; k++)
+      for (int64_t v1 = 0; v1 < pv; v1++) {
+        uint32_t c0 = 0, c1 = 0;
+        if (!flush && x != 255) {
+          c0 = e2m1_encode(ldexpf(load_as_f32<T>(base, k * post * vnni + 2 * v1), sh));
+          c1 = e2m1_encode(ldexpf(load_as_f32<T>(base, k * post * vnni + 2 * v1 + 1), sh));
+        }
+        out[(i * bs * post + k * post + j) * pv + v1] = (uint8_t)(c0 | (c1 << 4));
+      }
+  } else if (FMT == TPPX_Q_INT8) {
+    const float s = int8_scale_of(amax), inv = int8_inv_scale(s);
+    reinterpret_cast<float*>(scales)[t] = s;
+    for (int64_t k = 0; k < bs; k++)
+      for (int64_t v = 0; v < vnni; v++)
+        reinterpret_cast<int8_t*>(out)[(i * bs * post + k * post + j) * vnni + v] =
+            (int8_t)int8_q(load_as_f32<T>(base, k * post * vnni + v), inv);
+  } else { // INT4: scale = max / 7.0 in double, codes in [-8, 7], two per byte
+    const float s = (float)((double)amax / 7.0), inv = int8_inv_scale(s);
+    reinterpret_cast<float*>(scales)[t] = s;
+    const int64_t pv = vnni / 2;
+    for (int64_t k = 0; k < bs; k++)
+      for (int64_t v1 = 0; v1 < pv; v1++) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int v2 = 0; v2 < 2; v2++) {
+          float r = rintf(__fmul_rn(load_as_f32<T>(base, k * post * vnni + 2 * v1 + v2), inv));
+          r = fminf(fmaxf(r, -8.0f), 7.0f);
+          packed |= ((uint32_t)(int)r & 0xfu) << (4 * v2);
+        }
+        out[(i * bs * post + k * post + j) * pv + v1] = (uint8_t)packed;
+      }
+  }
+}
+
+template <int FMT>
+__global__ void __launch_bounds__(256)
+dequantize_per_block_kernel(const uint8_t* __restrict__ q, const void* __restrict__ scales, int64_t pre, int64_t bs,
+                            int64_t post, int64_t vnni, float* __restrict__ out) {
+  // one thread per stored byte
+  const int64_t pv = FMT == TPPX_Q_INT8 ? vnni : vnni / 2;
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= pre * bs * post * pv)
+    return;
+  const int64_t j = (t / pv) % post, i = t / (pv * post * bs);
+  const uint32_t b = q[t];
+  if (FMT == TPPX_Q_INT8) {
+    out[t] = (float)(int8_t)b * reinterpret_cast<const float*>(scales)[i * post + j];
+  } else if (FMT == TPPX_Q_MXFP4) {
+    const float s = e8m0_to_f32(reinterpret_cast<const uint8_t*>(scales)[i * post + j]);
+    out[2 * t] = c_e2m1_tbl[b & 0xf] * s;
+    out[2 * t + 1] = c_e2m1_tbl[b >> 4] * s;
+  } else {
+    const float s = reinterpret_cast<const float*>(scales)[i * post + j];
+    out[2 * t] = (float)(((int)(b & 0xf) ^ 8) - 8) * s; // two's complement nibbles
+    out[2 * t + 1] = (float)(((int)(b >> 4) ^ 8) - 8) * s;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// QINT2 interleaved (ternary) weights: one wave per (output channel, block of
+// bs input channels).  scale = max(|w|, 1e-8) over the block, t = rne(w / scale)
+// clamped to [-1, 1], code 0 / 1 / 2 for 0 / +1 / -1; byte [n1][b][c2][k2][c3]
+// carries the codes of channels n1*32 + k3*8 + k2 (k3 = 0..3 at bits 2*k3) at
+// input channel b*bs + c2*4 + c3.  The four channels of a byte belong to four
+// different waves, so the bytes are assembled with atomic ORs on zeroed memory.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t* __restrict__ p, int64_t n) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n)
+    p[t] = 0u;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+quantize_qint2_kernel(const T* __restrict__ w, int64_t N, int64_t K, int64_t bk, int64_t bc, int64_t vnni, int64_t bs,
+                      uint32_t* __restrict__ q32, float* __restrict__ scales) {
+  const int64_t nb = K / bs;
+  const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int lane = threadIdx.x & 63;
+  if (wave >= N * nb)
+    return;
+  const int64_t r = wave & 31, rest = wave >> 5;
+  const int64_t b = rest % nb, n1 = rest / nb;
+  const int64_t n = n1 * 32 + r;
+  float amax = 0.0f;
+  for (int64_t c = lane; c < bs; c += 64)
+    amax = fmaxf(amax, fabsf(load_as_f32<T>(w, blocked_off(n, b * bs + c, K, bk, bc, vnni))));
+  amax = wave_max(amax);
+  const float s = fmaxf(amax, 1.0e-8f);
+  if (lane == 0)
+    scales[(n1 * nb + b) * 32 + r] = s;
+  const int k3 = (int)(r >> 3), k2 = (int)(r & 7);
+  // a lane owns whole groups of 4 input channels = one byte position (c2, k2): 4 codes at bits 2*k3 of 4 bytes
+  for (int64_t c2 = lane; c2 < bs / 4; c2 += 64) {
+    uint32_t word = 0;
+#pragma unroll
+    for (int c3 = 0; c3 < 4; c3++) {
+      const float t = rintf(__fdiv_rn(load_as_f32<T>(w, blocked_off(n, b * bs + c2 * 4 + c3, K, bk, bc, vnni)), s));
+      const uint32_t code = t >= 1.0f ? 1u : (t <= -1.0f ? 2u : 0u);
+      word |= (code << (2 * k3)) << (8 * c3);
+    }
+    if (word)
+      atomicOr(&q32[((n1 * nb + b) * (bs / 4) + c2) * 8 + k2], word);
+  }
+}
+
+// packed 2-bit (interleaved) -> native int8 tiles of the W8A8 kernels + scales [N/16][K/bs][16];
+// one thread per native 16-byte chunk (nt, kt, g, n16): input channels kt*64 + g*16 .. +15 of channel nt*16 + n16
+__global__ void __launch_bounds__(256)
+prepack_qint2_kernel(const uint8_t* __restrict__ q2, const float* __restrict__ s2, int64_t N, int64_t K, int64_t bs,
+                     int8_t* __restrict__ qnat, float* __restrict__ snat) {
+  const int64_t nchunks = N * (K / 16);
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= nchunks)
+    return;
+  const int64_t n16 = t & 15, g = (t >> 4) & 3, rest = t >> 6;
+  const int64_t KT = K / 64, nb = K / bs;
+  const int64_t kt = rest % KT, nt = rest / KT;
+  const int64_t n = nt * 16 + n16, k0 = kt * 64 + g * 16;
+  const int64_t n1 = n >> 5, r = n & 31, k3 = r >> 3, k2 = r & 7;
+  const int64_t b = k0 / bs, c2 = (k0 % bs) >> 2;
+  const uint32_t* src = reinterpret_cast<const uint32_t*>(q2) + ((n1 * nb + b) * (bs / 4) + c2) * 8 + k2;
+  uint32_t o[4];
+#pragma unroll
+  for (int d = 0; d < 4; d++) {
+    const uint32_t codes = (src[d * 8] >> (2 * k3)) & 0x03030303u; // the four input channels c3 of group c2 + d
+    // 0 -> 0x00, 1 -> 0x01, 2 -> 0xff (-1) per byte
+    o[d] = __builtin_amdgcn_perm(0u, 0x00ff0100u, codes);
+  }
+  reinterpret_cast<uint4*>(qnat)[t] = make_uint4(o[0], o[1], o[2], o[3]);
+  if (g == 0 && (kt * 64) % bs == 0)
+    snat[(nt * nb + b) * 16 + n16] = s2[(n1 * nb + b) * 32 + r];
+}
+
+// packed 2-bit (interleaved) -> fp32 in the logical blocked shape [N/32][K/bs][bs/4][32][4]; one thread per output
+__global__ void __launch_bounds__(256)
+dequantize_qint2_kernel(const uint8_t* __restrict__ q2, const float* __restrict__ s2, int64_t total, int64_t bs,
+                        float* __restrict__ out) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= total)
+    return;
+  const int64_t c3 = t & 3, r = (t >> 2) & 31, rest = t >> 7; // rest = (n1*nb + b) * (bs/4) + c2
+  const int64_t blk = rest / (bs / 4);
+  const uint32_t byte = q2[(rest * 8 + (r & 7)) * 4 + c3];
+  const uint32_t code = (byte >> (2 * (r >> 3))) & 3u;
+  out[t] = (code == 1 ? 1.0f : (code == 2 ? -1.0f : 0.0f)) * s2[blk * 32 + r];
+}
+
+// INT4 weight in the VNNI2 layout [N/16][K/bs][bs/2][16][2 codes per byte] -> native int8 tiles
+__global__ void __launch_bounds__(256)
+prepack_qint4_kernel(const uint8_t* __restrict__ q4, int64_t N, int64_t K, int64_t bs, int8_t* __restrict__ qnat) {
+  const int64_t nchunks = N * (K / 16);
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= nchunks)
+    return;
+  const int64_t n16 = t & 15, g = (t >> 4) & 3, rest = t >> 6;
+  const int64_t KT = K / 64, nb = K / bs;
+  const int64_t kt = rest % KT, nt = rest / KT;
+  const int64_t k0 = kt * 64 + g * 16;
+  const int64_t b = k0 / bs, a0 = (k0 % bs) >> 1; // pair index inside the block
+  const uint8_t* src = q4 + ((nt * nb + b) * (bs / 2) + a0) * 16 + n16;
+  uint32_t o[4];
+#pragma unroll
+  for (int d = 0; d < 4; d++) {
+    uint32_t word = 0;
+#pragma unroll
+    for (int pr = 0; pr < 2; pr++) {
+      const uint32_t byte = src[(d * 2 + pr) * 16];
+      const uint32_t lo = (uint32_t)((((int)(byte & 0xf) ^ 8) - 8) & 0xff), hi = (uint32_t)((((int)(byte >> 4) ^ 8) - 8) & 0xff);
+      word |= (lo | (hi << 8)) << (16 * pr);
+    }
+    o[d] = word;
+  }
+  reinterpret_cast<uint4*>(qnat)[t] = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 static inline unsigned grid_for(int64_t n, int block) {
   return (unsigned)((n + block - 1) / block);
 }
@@ -586,4 +799,114 @@ extern "C" int tppx_quant_act_int8(const void* x, int64_t M, int64_t K,
   TPPX_REQUIRE(M > 0 && K > 0 && qbs > 0 && qbs % 64 == 0 && K % qbs == 0, TPPX_ESHAPE,
                "tppx_quant_act_int8: bad shape M=%ld K=%ld qbs=%ld", (long)M, (long)K, (long)qbs);
   return check_hip(launch_quant_act_int8(x, M, K, qbs, xq, sa, 0, (hipStream_t)stream), "tppx_quant_act_int8");
+}
+
+// ---- generic helpers ---------------------------------------------------------
+static int check_per_block(const char* who, int qfmt, int64_t pre, int64_t bs, int64_t post, int64_t vnni) {
+  TPPX_REQUIRE(qfmt == TPPX_Q_MXFP4 || qfmt == TPPX_Q_INT8 || qfmt == TPPX_Q_INT4, TPPX_EINVAL, "%s: unknown format id %d", who, qfmt);
+  TPPX_REQUIRE(pre > 0 && bs > 0 && post > 0 && vnni > 0, TPPX_ESHAPE, "%s: bad geometry pre=%ld bs=%ld post=%ld vnni=%ld", who,
+               (long)pre, (long)bs, (long)post, (long)vnni);
+  TPPX_REQUIRE(qfmt == TPPX_Q_INT8 || vnni % 2 == 0, TPPX_ESHAPE, "%s: 4-bit formats pack two codes per byte: vnni=%ld must be even", who, (long)vnni);
+  TPPX_REQUIRE(pre * bs * post * vnni < ((int64_t)1 << 40), TPPX_ESHAPE, "%s: tensor too large", who);
+  return TPPX_OK;
+}
+
+extern "C" int tppx_quantize_per_block(const void* in, int in_dtype, int qfmt, int64_t pre, int64_t bs, int64_t post,
+                                       int64_t vnni, void* out, void* scales, tppx_stream_t stream) {
+  const char* who = "tppx_quantize_per_block";
+  TPPX_REQUIRE(in && out && scales, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(in_dtype == TPPX_DT_F32 || in_dtype == TPPX_DT_BF16, TPPX_EINVAL, "%s: unknown input dtype %d", who, in_dtype);
+  if (int rc = check_per_block(who, qfmt, pre, bs, post, vnni))
+    return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned grid = grid_for(pre * post, 256);
+#define TPPX_QPB(T, F) quantize_per_block_kernel<T, F><<<grid, 256, 0, s>>>((const T*)in, pre, bs, post, vnni, (uint8_t*)out, scales)
+  if (in_dtype == TPPX_DT_F32) {
+    if (qfmt == TPPX_Q_MXFP4) TPPX_QPB(float, TPPX_Q_MXFP4);
+    else if (qfmt == TPPX_Q_INT8) TPPX_QPB(float, TPPX_Q_INT8);
+    else TPPX_QPB(float, TPPX_Q_INT4);
+  } else {
+    if (qfmt == TPPX_Q_MXFP4) TPPX_QPB(uint16_t, TPPX_Q_MXFP4);
+    else if (qfmt == TPPX_Q_INT8) TPPX_QPB(uint16_t, TPPX_Q_INT8);
+    else TPPX_QPB(uint16_t, TPPX_Q_INT4);
+  }
+#undef TPPX_QPB
+  return check_hip(hipGetLastError(), who);
+}
+
+extern "C" int tppx_dequantize_per_block(const void* q, const void* scales, int qfmt, int64_t pre, int64_t bs,
+                                         int64_t post, int64_t vnni, void* out_f32, tppx_stream_t stream) {
+  const char* who = "tppx_dequantize_per_block";
+  TPPX_REQUIRE(q && scales && out_f32, TPPX_EINVAL, "%s: null pointer", who);
+  if (int rc = check_per_block(who, qfmt, pre, bs, post, vnni))
+    return rc;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t nbytes = pre * bs * post * (qfmt == TPPX_Q_INT8 ? vnni : vnni / 2);
+  if (qfmt == TPPX_Q_MXFP4)
+    dequantize_per_block_kernel<TPPX_Q_MXFP4><<<grid_for(nbytes, 256), 256, 0, s>>>((const uint8_t*)q, scales, pre, bs, post, vnni, (float*)out_f32);
+  else if (qfmt == TPPX_Q_INT8)
+    dequantize_per_block_kernel<TPPX_Q_INT8><<<grid_for(nbytes, 256), 256, 0, s>>>((const uint8_t*)q, scales, pre, bs, post, vnni, (float*)out_f32);
+  else
+    dequantize_per_block_kernel<TPPX_Q_INT4><<<grid_for(nbytes, 256), 256, 0, s>>>((const uint8_t*)q, scales, pre, bs, post, vnni, (float*)out_f32);
+  return check_hip(hipGetLastError(), who);
+}
+
+static int check_qint2(const char* who, int64_t N, int64_t K, int64_t bs) {
+  TPPX_REQUIRE(N > 0 && K > 0 && N % 32 == 0, TPPX_ESHAPE, "%s: N=%ld must be a positive multiple of 32", who, (long)N);
+  TPPX_REQUIRE(bs > 0 && bs % 64 == 0 && K % bs == 0, TPPX_ESHAPE, "%s: block size %ld must be a multiple of 64 dividing K=%ld", who, (long)bs, (long)K);
+  return TPPX_OK;
+}
+
+extern "C" int tppx_quantize_qint2_intlv(const void* w, int w_dtype, int64_t N, int64_t K, int64_t bk, int64_t bc,
+                                         int64_t vnni, int64_t bs, void* q, void* scales, tppx_stream_t stream) {
+  const char* who = "tppx_quantize_qint2_intlv";
+  TPPX_REQUIRE(w && q && scales, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(w_dtype == TPPX_DT_F32 || w_dtype == TPPX_DT_BF16, TPPX_EINVAL, "%s: unknown weight dtype %d", who, w_dtype);
+  TPPX_REQUIRE((reinterpret_cast<uintptr_t>(q) & 3u) == 0, TPPX_EINVAL, "%s: output not 4-byte aligned", who);
+  if (int rc = check_qint2(who, N, K, bs))
+    return rc;
+  TPPX_REQUIRE(bk > 0 && bc > 0 && vnni > 0 && N % bk == 0 && K % bc == 0 && bc % vnni == 0, TPPX_ESHAPE,
+               "%s: blocking (bk=%ld, bc=%ld, vnni=%ld) does not divide [%ld,%ld]", who, (long)bk, (long)bc, (long)vnni, (long)N, (long)K);
+  hipStream_t s = (hipStream_t)stream;
+  // the bytes are assembled with ORs: start from zeros (a fill kernel, so that the call can sit in a captured graph)
+  const int64_t nwords = N * K / 16;
+  fill_zero_kernel<<<grid_for(nwords, 256), 256, 0, s>>>((uint32_t*)q, nwords);
+  const int64_t nthreads = N * (K / bs) * 64;
+  if (w_dtype == TPPX_DT_F32)
+    quantize_qint2_kernel<float><<<grid_for(nthreads, 256), 256, 0, s>>>((const float*)w, N, K, bk, bc, vnni, bs, (uint32_t*)q, (float*)scales);
+  else
+    quantize_qint2_kernel<uint16_t><<<grid_for(nthreads, 256), 256, 0, s>>>((const uint16_t*)w, N, K, bk, bc, vnni, bs, (uint32_t*)q, (float*)scales);
+  return check_hip(hipGetLastError(), who);
+}
+
+extern "C" int tppx_dequantize_qint2_intlv(const void* q, const void* scales, int64_t N, int64_t K, int64_t bs,
+                                           void* out_f32, tppx_stream_t stream) {
+  const char* who = "tppx_dequantize_qint2_intlv";
+  TPPX_REQUIRE(q && scales && out_f32, TPPX_EINVAL, "%s: null pointer", who);
+  if (int rc = check_qint2(who, N, K, bs))
+    return rc;
+  dequantize_qint2_kernel<<<grid_for(N * K, 256), 256, 0, (hipStream_t)stream>>>((const uint8_t*)q, (const float*)scales, N * K, bs, (float*)out_f32);
+  return check_hip(hipGetLastError(), who);
+}
+
+extern "C" int tppx_prepack_qint2(const void* q_ref, const void* scales_ref, int64_t N, int64_t K, int64_t bs,
+                                  void* q_nat, void* scales_nat, tppx_stream_t stream) {
+  const char* who = "tppx_prepack_qint2";
+  TPPX_REQUIRE(q_ref && scales_ref && q_nat && scales_nat, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(aligned16(q_nat) && (reinterpret_cast<uintptr_t>(q_ref) & 3u) == 0, TPPX_EINVAL, "%s: pointer not aligned", who);
+  if (int rc = check_qint2(who, N, K, bs))
+    return rc;
+  prepack_qint2_kernel<<<grid_for(N * (K / 16), 256), 256, 0, (hipStream_t)stream>>>((const uint8_t*)q_ref, (const float*)scales_ref, N, K, bs,
+                                                                                      (int8_t*)q_nat, (float*)scales_nat);
+  return check_hip(hipGetLastError(), who);
+}
+
+extern "C" int tppx_prepack_qint4(const void* q_ref, int64_t N, int64_t K, int64_t bs, void* q_nat, tppx_stream_t stream) {
+  const char* who = "tppx_prepack_qint4";
+  TPPX_REQUIRE(q_ref && q_nat, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(aligned16(q_nat), TPPX_EINVAL, "%s: output not 16-byte aligned", who);
+  TPPX_REQUIRE(N > 0 && K > 0 && N % 16 == 0 && bs > 0 && bs % 64 == 0 && K % bs == 0, TPPX_ESHAPE, "%s: bad shape N=%ld K=%ld bs=%ld", who,
+               (long)N, (long)K, (long)bs);
+  prepack_qint4_kernel<<<grid_for(N * (K / 16), 256), 256, 0, (hipStream_t)stream>>>((const uint8_t*)q_ref, N, K, bs, (int8_t*)q_nat);
+  return check_hip(hipGetLastError(), who);
 }

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libtppx_hip.so")
 OK, EINVAL, ESHAPE, EUNSUPPORTED, EHIP = 0, -1, -2, -3, -4
 POST_NONE, POST_SILU, POST_MUL, POST_ADD_SCALE, POST_ADD2_SCALE, POST_GELU, POST_RELU = range(7)
 DT_F32, DT_BF16 = 0, 1
+Q_MXFP4, Q_INT8, Q_INT4 = 0, 1, 2
 FLAG_NONE, FLAG_FORCE_SKINNY, FLAG_FORCE_TILED, FLAG_ACT_FP8, FLAG_XQ_REUSE = 0, 1, 2, 4, 8
 
 
@@ -49,6 +50,12 @@ SIGNATURES = {
     "tppx_quantize_qint8": [_vp, _i32, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp],
     "tppx_dequantize_mxfp4": [_vp, _vp, _i64, _i64, _vp, _vp],
     "tppx_dequantize_qint8": [_vp, _vp, _i64, _i64, _i64, _vp, _vp],
+    "tppx_quantize_per_block": [_vp, _i32, _i32, _i64, _i64, _i64, _i64, _vp, _vp, _vp],
+    "tppx_dequantize_per_block": [_vp, _vp, _i32, _i64, _i64, _i64, _i64, _vp, _vp],
+    "tppx_quantize_qint2_intlv": [_vp, _i32, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp],
+    "tppx_dequantize_qint2_intlv": [_vp, _vp, _i64, _i64, _i64, _vp, _vp],
+    "tppx_prepack_qint2": [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp],
+    "tppx_prepack_qint4": [_vp, _i64, _i64, _i64, _vp, _vp],
     "tppx_prepack_mxfp4": [_vp, _vp, _i64, _i64, _vp, _vp, _vp],
     "tppx_prepack_qint8": [_vp, _i64, _i64, _i64, _vp, _vp],
     "tppx_quant_act_int8": [_vp, _i64, _i64, _i64, _vp, _vp, _vp],

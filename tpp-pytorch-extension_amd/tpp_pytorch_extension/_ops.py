@@ -107,39 +107,101 @@ def remap_and_quantize_qint8(t):
     return QTensor(q, sc, tuple(q.shape), torch.qint8, QSCHEME_AFFINE, qbs, 2, True, 1)
 
 
+def _per_block_geometry(shape, block_size, axis, is_vnni, pack):
+    """(pre, bs, post, vnni, scale_sizes) as PerBlockQuantizer derives them (src/csrc/qtypes.h:30-68)."""
+    sizes = list(shape)
+    if axis < 0:
+        axis += len(sizes)
+    if is_vnni:
+        vnni = sizes.pop()
+    else:
+        if axis != len(sizes) - 1:
+            raise TppxError(_lib.EINVAL, f"Invalid axis {axis}")
+        if sizes[axis] % pack:
+            raise TppxError(_lib.ESHAPE, "Invalid dim size")
+        vnni = pack
+        sizes[axis] //= pack
+    if block_size % vnni:
+        raise TppxError(_lib.ESHAPE, "Block size must be multiple of VNNI pack size")
+    bsi = block_size // vnni
+    if not (0 <= axis < len(sizes)):
+        raise TppxError(_lib.EINVAL, "Invalid axis")
+    if sizes[axis] % bsi:
+        raise TppxError(_lib.ESHAPE, "Axis size must be multiple of block_size")
+    sizes[axis] //= bsi
+    pre = 1
+    for d in sizes[: axis + 1]:
+        pre *= d
+    post = 1
+    for d in sizes[axis + 1:]:
+        post *= d
+    return pre, bsi, post, vnni, sizes, axis
+
+
+def _quantize_generic(t, block_size, axis, is_vnni, fmt):
+    """quantize_mxfp4 / quantize_int8sym / quantize_int4sym on any layout (PerBlockQuantizer::quantize_symetric,
+    src/csrc/qtypes.h:133-193): the generic per-block kernel."""
+    L = _lib.lib()
+    if isinstance(t, QTensor):
+        raise TppxError(_lib.EINVAL, "tensor is already quantized")
+    if t.dtype not in (torch.bfloat16, torch.float32):
+        raise TppxError(_lib.EUNSUPPORTED, f"Unsupported input type for quantization: {t.dtype}")
+    _lib.require_gpu(t, "tensor to quantize")
+    t = t.detach().contiguous()
+    pack = 1 if fmt == _lib.Q_INT8 else 2
+    pre, bs, post, vnni, ssz, axis = _per_block_geometry(t.shape, block_size, axis, is_vnni, pack)
+    if pack == 2 and vnni % 2:
+        raise TppxError(_lib.ESHAPE, "4-bit formats pack two codes per byte: the packed dimension must be even")
+    qshape = tuple(t.shape[:-1]) + (t.shape[-1] // pack,)
+    q = torch.empty(qshape, dtype=torch.int8 if fmt == _lib.Q_INT8 else torch.uint8, device=t.device)
+    sc = torch.empty(tuple(ssz), dtype=torch.uint8 if fmt == _lib.Q_MXFP4 else torch.float32, device=t.device)
+    if t.numel():
+        dt = _lib.DT_BF16 if t.dtype == torch.bfloat16 else _lib.DT_F32
+        _lib.check(L.tppx_quantize_per_block(t.data_ptr(), dt, fmt, pre, bs, post, vnni, q.data_ptr(), sc.data_ptr(),
+                                             _lib.stream_of(t)))
+    if fmt == _lib.Q_MXFP4:
+        return QTensor(q, sc, tuple(t.shape), torch.quint4x2, QSCHEME_MXFP, block_size, axis, is_vnni, 2)
+    if fmt == _lib.Q_INT8:
+        return QTensor(q, sc, tuple(t.shape), torch.qint8, QSCHEME_AFFINE, block_size, axis, is_vnni, 1)
+    return QTensor(q, sc, tuple(t.shape), torch.quint4x2, QSCHEME_AFFINE, block_size, axis, is_vnni, 2)
+
+
 def quantize_mxfp4(t, block_size, axis, is_vnni):
-    """Reference: quantize_mxfp4 (qtypes.cpp:602-611).  Built for the layout
-    remap_and_quantize_mxfp4 feeds it: [N/32, K/64, 32, 32, 2], block 32, axis 2, VNNI."""
+    """Reference: quantize_mxfp4 (qtypes.cpp:602-611).  The layout remap_and_quantize_mxfp4 feeds it
+    ([N/32, K/64, 32, 32, 2], block 32, axis 2, VNNI) takes the weight kernel; any other layout the generic
+    per-block kernel (same bytes)."""
     if axis < 0:
         axis += t.dim()
-    if not (t.dim() == 5 and tuple(t.shape[2:]) == (32, 32, 2) and block_size == 32 and axis == 2 and is_vnni):
-        raise TppxError(
-            _lib.EUNSUPPORTED,
-            "quantize_mxfp4 is built for blocked weights [N/32, K/64, 32, 32, 2] with block_size=32, axis=2, is_vnni=True",
-        )
-    return remap_and_quantize_mxfp4(t)
+    if t.dim() == 5 and tuple(t.shape[2:]) == (32, 32, 2) and block_size == 32 and axis == 2 and is_vnni and t.shape[1] > 0:
+        L = _lib.lib()
+        t, dt = _float_weight_on_gpu(t)
+        N, K = t.shape[0] * 32, t.shape[1] * 64
+        q = torch.empty((N // 32, K // 64, 32, 32), dtype=torch.uint8, device=t.device)
+        sc = torch.empty((N // 32, K // 64, 2, 32), dtype=torch.uint8, device=t.device)
+        # the input is already [N/32][K/64][32][32][2]: bk=32, bc=64, vnni=2
+        _lib.check(L.tppx_quantize_mxfp4(t.data_ptr(), dt, N, K, 32, 64, 2, q.data_ptr(), sc.data_ptr(), _lib.stream_of(t)))
+        return QTensor(q, sc, (N // 32, K // 64, 32, 32, 2), torch.quint4x2, QSCHEME_MXFP, 32, 2, True, 2)
+    qt = _quantize_generic(t, block_size, axis, is_vnni, _lib.Q_MXFP4)
+    return qt
 
 
 def quantize_mxfp(t, block_size, axis, is_vnni, dtype):
-    """Reference: quantize_mxfp (qtypes.cpp:592-600); only the E2M1 element type is built."""
+    """Reference: quantize_mxfp (qtypes.cpp:592-600); only the E2M1 element type exists there too
+    (PerBlockMxFPQuantizer::quantize asserts on anything but kQUInt4x2, qtypes.cpp:430-432)."""
     if dtype != torch.quint4x2:
-        raise TppxError(_lib.EUNSUPPORTED, f"MX element type {dtype} is not built (only quint4x2 / E2M1)")
+        raise TppxError(_lib.EUNSUPPORTED, "Unsupported MXFP datatype")
     return quantize_mxfp4(t, block_size, axis, is_vnni)
 
 
 def quantize_int8sym(t, block_size, axis, is_vnni):
-    """Reference: quantize_int8sym (qtypes.cpp:613-624).  Two layouts are built:
-    the VNNI4 weight [N/16, K/QBS, QBS/4, 16, 4] (axis 2) and row-major
-    activations [..., K] quantized along the last axis (is_vnni False)."""
+    """Reference: quantize_int8sym (qtypes.cpp:613-624).  The VNNI4 weight [N/16, K/QBS, QBS/4, 16, 4] (axis 2) and
+    row-major bf16 activations quantized along the last axis take their own kernels; every other layout the generic
+    per-block kernel (same bytes)."""
     L = _lib.lib()
     if axis < 0:
         axis += t.dim()
-    if is_vnni:
-        if not (t.dim() == 5 and tuple(t.shape[3:]) == (16, 4) and axis == 2 and t.shape[2] * 4 == block_size):
-            raise TppxError(
-                _lib.EUNSUPPORTED,
-                "quantize_int8sym(is_vnni=True) is built for weights [N/16, K/QBS, QBS/4, 16, 4] with axis=2",
-            )
+    if is_vnni and t.dim() == 5 and tuple(t.shape[3:]) == (16, 4) and axis == 2 and t.shape[2] * 4 == block_size \
+            and block_size % 64 == 0:
         t, dt = _float_weight_on_gpu(t)
         N, K = t.shape[0] * 16, t.shape[1] * block_size
         q = torch.empty(tuple(t.shape), dtype=torch.int8, device=t.device)
@@ -148,21 +210,23 @@ def quantize_int8sym(t, block_size, axis, is_vnni):
         _lib.check(L.tppx_quantize_qint8(t.data_ptr(), dt, N, K, 16, block_size, 4, block_size,
                                          q.data_ptr(), sc.data_ptr(), _lib.stream_of(t)))
         return QTensor(q, sc, tuple(q.shape), torch.qint8, QSCHEME_AFFINE, block_size, 2, True, 1)
-    if axis != t.dim() - 1:
-        raise TppxError(_lib.EINVAL, f"Invalid axis {axis}")
-    _lib.require_gpu(t, "activation to quantize")
-    if t.dtype != torch.bfloat16:
-        raise TppxError(_lib.EUNSUPPORTED, f"activation quantization is built for bfloat16 (got {t.dtype})")
-    K = t.shape[-1]
-    if K % block_size:
-        raise TppxError(_lib.ESHAPE, "Axis size must be multiple of block_size")
-    t = t.contiguous()
-    M = t.numel() // K
-    xq = torch.empty(tuple(t.shape), dtype=torch.int8, device=t.device)
-    sa = torch.empty(tuple(t.shape[:-1]) + (K // block_size,), dtype=torch.float32, device=t.device)
-    _lib.check(L.tppx_quant_act_int8(t.data_ptr(), M, K, block_size, xq.data_ptr(), sa.data_ptr(),
-                                     _lib.stream_of(t)))
-    return QTensor(xq, sa, tuple(t.shape), torch.qint8, QSCHEME_AFFINE, block_size, axis, False, 1)
+    if (not is_vnni) and axis == t.dim() - 1 and t.dtype == torch.bfloat16 and t.is_cuda and block_size % 64 == 0 \
+            and t.shape[-1] % block_size == 0 and t.numel() > 0:
+        K = t.shape[-1]
+        t = t.contiguous()
+        M = t.numel() // K
+        xq = torch.empty(tuple(t.shape), dtype=torch.int8, device=t.device)
+        sa = torch.empty(tuple(t.shape[:-1]) + (K // block_size,), dtype=torch.float32, device=t.device)
+        _lib.check(L.tppx_quant_act_int8(t.data_ptr(), M, K, block_size, xq.data_ptr(), sa.data_ptr(),
+                                         _lib.stream_of(t)))
+        return QTensor(xq, sa, tuple(t.shape), torch.qint8, QSCHEME_AFFINE, block_size, axis, False, 1)
+    return _quantize_generic(t, block_size, axis, is_vnni, _lib.Q_INT8)
+
+
+def quantize_int4sym(t, block_size, axis, is_vnni):
+    """Reference: quantize_int4sym (qtypes.cpp:626-637; Int4SymQuant :199-246): scale = max/7, codes in [-8, 7],
+    two per byte.  A weight in the VNNI2 layout [N/16, K/QBS, QBS/2, 16, 2] (axis 2) is accepted by the linears."""
+    return _quantize_generic(t, block_size, axis, is_vnni, _lib.Q_INT4)
 
 
 def create_qtensor_int8sym(val, scales, block_size, axis, is_vnni):
@@ -175,16 +239,53 @@ def create_qtensor_int8sym(val, scales, block_size, axis, is_vnni):
                    block_size, axis, is_vnni, 1)
 
 
-def _unbuilt(name):
-    def f(*a, **k):
-        raise TppxError(_lib.EUNSUPPORTED, f"{name} is outside the MXFP4 / QINT8 path built here")
-    f.__name__ = name
-    return f
+def create_qtensor_int2sym(sizes, val, scales, block_size, axis, is_vnni):
+    """Reference: create_qtensor_int2sym (qtypes.cpp:686-702): wrap caller-supplied packed 2-bit codes (uint8, four
+    per byte) + fp32 scales as a kQUInt2x4 tensor of logical shape `sizes`."""
+    if val.dtype != torch.uint8 or scales.dtype != torch.float32:
+        raise TppxError(_lib.EINVAL, "create_qtensor_int2sym expects uint8 values and float32 scales")
+    sizes = tuple(int(d) for d in sizes)
+    if axis < 0:
+        axis += len(sizes)
+    return QTensor(val.contiguous(), scales.contiguous(), sizes, torch.quint2x4, QSCHEME_AFFINE, block_size, axis,
+                   is_vnni, 4)
 
 
-quantize_int4sym = _unbuilt("quantize_int4sym")
-create_qtensor_int2sym = _unbuilt("create_qtensor_int2sym")
-remap_and_quantize_qint2_intlv = _unbuilt("remap_and_quantize_qint2_intlv")
+QINT2_BLOCK_SIZE = int(os.environ.get("QINT2_BLOCK_SIZE", "256"))
+
+
+def qint2_block_size_for(K):
+    """Block-size rule of remap_and_quantize_qint2_intlv (qtypes.cpp:1031-1043)."""
+    if K % QINT2_BLOCK_SIZE == 0:
+        return QINT2_BLOCK_SIZE
+    q = 4096
+    while q >= 64:
+        if QINT2_BLOCK_SIZE > q and K % q == 0:
+            return q
+        q //= 2
+    raise TppxError(_lib.ESHAPE, f"no QINT2 block size divides K={K}")
+
+
+def remap_and_quantize_qint2_intlv(t):
+    """Reference: remap_and_quantize_qint2_intlv (src/csrc/qtypes.cpp:1004-1073), the "qint2" choice of FixLinear:
+    ternary weights, four codes per byte interleaved over output channels.
+    -> quint2x4 tensor of logical shape [N/32, K/QBS, QBS/4, 32, 4]; packed bytes [N/32, K/QBS, QBS/4, 8, 4];
+    fp32 scales [N/32, K/QBS, 32, 1].  (TPP_QINT2_AS_QINT1 is not built.)"""
+    L = _lib.lib()
+    if os.environ.get("TPP_QINT2_AS_QINT1", "0") not in ("0", ""):
+        raise TppxError(_lib.EUNSUPPORTED, "TPP_QINT2_AS_QINT1 (1-bit weights) is not built")
+    t, dt = _float_weight_on_gpu(t)
+    N, K, bk, bc, vnni = _blocked_geometry(t)
+    if N % 32:
+        raise TppxError(_lib.EUNSUPPORTED, f"QINT2 weights are built for a multiple of 32 output channels (got {N})")
+    if K % 4:
+        raise TppxError(_lib.ESHAPE, "C must be multiple of 4")
+    bs = qint2_block_size_for(K)
+    q = torch.empty((N // 32, K // bs, bs // 4, 8, 4), dtype=torch.uint8, device=t.device)
+    sc = torch.empty((N // 32, K // bs, 32, 1), dtype=torch.float32, device=t.device)
+    _lib.check(L.tppx_quantize_qint2_intlv(t.data_ptr(), dt, N, K, bk, bc, vnni, bs, q.data_ptr(), sc.data_ptr(),
+                                           _lib.stream_of(t)))
+    return create_qtensor_int2sym((N // 32, K // bs, bs // 4, 32, 4), q, sc, bs, 2, True)
 
 
 def _as_q(t):

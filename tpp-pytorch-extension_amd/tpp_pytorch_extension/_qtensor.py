@@ -54,18 +54,55 @@ class QTensor(torch.Tensor):
                     self.axis, self.is_vnni, self.pack_size)
         return q
 
+    # -- per-block geometry (PerBlockQuantizer, src/csrc/qtypes.h:30-68) ------
+    def geometry(self):
+        """(pre, bs, post, vnni) of the logical tensor viewed as [pre][bs][post][vnni]."""
+        sizes = list(self.shape)
+        axis = self.axis
+        if self.is_vnni:
+            vnni = sizes.pop()
+        else:
+            vnni = self.pack_size
+            sizes[axis] //= vnni
+        bsi = self.block_size // vnni
+        sizes[axis] //= bsi
+        pre = 1
+        for d in sizes[: axis + 1]:
+            pre *= d
+        post = 1
+        for d in sizes[axis + 1:]:
+            post *= d
+        return pre, bsi, post, vnni
+
     # -- weight geometry -----------------------------------------------------
-    def is_weight(self):
-        """True for the two weight layouts the linear kernels consume."""
+    def weight_kind(self):
+        """Which linear-layer weight layout this is: "mxfp4" [N/32, K/64, 32, 32, 2], "qint8" [N/16, K/QBS, QBS/4, 16,
+        4], "qint4" (VNNI2) [N/16, K/QBS, QBS/2, 16, 2], "qint2" (interleaved ternary) [N/32, K/QBS, QBS/4, 32, 4];
+        None for any other layout (helper-only tensors, quantized activations)."""
         s = tuple(self.shape)
+        if len(s) != 5 or not self.is_vnni or self.axis != 2:
+            return None
         if self._qscheme == QSCHEME_MXFP:
-            return len(s) == 5 and s[2:] == (32, 32, 2) and self.block_size == 32 and self.is_vnni
-        return (len(s) == 5 and s[3:] == (16, 4) and self.is_vnni and s[2] * 4 == self.block_size)
+            return "mxfp4" if s[2:] == (32, 32, 2) and self.block_size == 32 else None
+        if self.dtype == torch.qint8 and s[3:] == (16, 4) and s[2] * 4 == self.block_size:
+            return "qint8"
+        if self.dtype == torch.quint4x2 and s[3:] == (16, 2) and s[2] * 2 == self.block_size and self.block_size % 64 == 0:
+            return "qint4"
+        if self.dtype == torch.quint2x4 and s[3:] == (32, 4) and s[2] * 4 == self.block_size and self.block_size % 64 == 0:
+            return "qint2"
+        return None
+
+    def is_weight(self):
+        """True for the weight layouts the linear kernels consume."""
+        return self.weight_kind() is not None
 
     def weight_nk(self):
         s = self.shape
-        if self._qscheme == QSCHEME_MXFP:
+        kind = self.weight_kind()
+        if kind == "mxfp4":
             return s[0] * 32, s[1] * 64
+        if kind == "qint2":
+            return s[0] * 32, s[1] * self.block_size
         return s[0] * 16, s[1] * self.block_size
 
     def native(self):
@@ -77,15 +114,27 @@ class QTensor(torch.Tensor):
                 raise _lib.TppxError(_lib.EUNSUPPORTED, f"not a linear-layer weight layout: {self!r}")
             N, K = self.weight_nk()
             st = _lib.stream_of(self.qdata)
-            qn = torch.empty_like(self.qdata)
-            if self._qscheme == QSCHEME_MXFP:
+            kind = self.weight_kind()
+            if kind == "mxfp4":
+                qn = torch.empty_like(self.qdata)
                 sn = torch.empty_like(self.scales)
                 _lib.check(L.tppx_prepack_mxfp4(self.qdata.data_ptr(), self.scales.data_ptr(), N, K,
                                                 qn.data_ptr(), sn.data_ptr(), st))
-            else:
+            elif kind == "qint8":
+                qn = torch.empty_like(self.qdata)
                 sn = self.scales
                 _lib.check(L.tppx_prepack_qint8(self.qdata.data_ptr(), N, K, self.block_size,
                                                 qn.data_ptr(), st))
+            elif kind == "qint4":
+                # low-bit affine weights run on the W8A8 kernels: codes expanded once into native int8 tiles
+                qn = torch.empty(N * K, dtype=torch.int8, device=self.qdata.device)
+                sn = self.scales
+                _lib.check(L.tppx_prepack_qint4(self.qdata.data_ptr(), N, K, self.block_size, qn.data_ptr(), st))
+            else:
+                qn = torch.empty(N * K, dtype=torch.int8, device=self.qdata.device)
+                sn = torch.empty((N // 16, K // self.block_size, 1, 16), dtype=torch.float32, device=self.qdata.device)
+                _lib.check(L.tppx_prepack_qint2(self.qdata.data_ptr(), self.scales.data_ptr(), N, K, self.block_size,
+                                                qn.data_ptr(), sn.data_ptr(), st))
             self._native = (qn, sn)
         return self._native
 
@@ -95,19 +144,31 @@ class QTensor(torch.Tensor):
         L = _lib.lib()
         _lib.require_gpu(self.qdata, "quantized tensor")
         out = torch.empty(tuple(self.shape), dtype=torch.float32, device=self.device)
+        if out.numel() == 0:
+            return out
         st = _lib.stream_of(self.qdata)
-        if self._qscheme == QSCHEME_MXFP:
-            if not self.is_weight():
-                raise _lib.TppxError(_lib.EUNSUPPORTED, f"dequantize: unsupported MXFP4 layout {self!r}")
+        kind = self.weight_kind()
+        if kind == "mxfp4":
             N, K = self.weight_nk()
             _lib.check(L.tppx_dequantize_mxfp4(self.qdata.data_ptr(), self.scales.data_ptr(), N, K,
                                                out.data_ptr(), st))
-        elif self.is_weight():
+        elif kind == "qint8":
             N, K = self.weight_nk()
             _lib.check(L.tppx_dequantize_qint8(self.qdata.data_ptr(), self.scales.data_ptr(), N, K,
                                                self.block_size, out.data_ptr(), st))
-        else:
-            raise _lib.TppxError(_lib.EUNSUPPORTED, f"dequantize: unsupported QINT8 layout {self!r}")
+        elif self.dtype == torch.quint2x4:
+            if kind != "qint2":
+                raise _lib.TppxError(_lib.EUNSUPPORTED, f"dequantize: only the interleaved ternary weight layout "
+                                                        f"is defined for 2-bit tensors, got {self!r}")
+            N, K = self.weight_nk()
+            _lib.check(L.tppx_dequantize_qint2_intlv(self.qdata.data_ptr(), self.scales.data_ptr(), N, K,
+                                                     self.block_size, out.data_ptr(), st))
+        else:  # any other layout: the generic per-block kernel (quantized activations, helper-made tensors)
+            pre, bs, post, vnni = self.geometry()
+            fmt = (_lib.Q_MXFP4 if self._qscheme == QSCHEME_MXFP
+                   else (_lib.Q_INT8 if self.dtype == torch.qint8 else _lib.Q_INT4))
+            _lib.check(L.tppx_dequantize_per_block(self.qdata.data_ptr(), self.scales.data_ptr(), fmt, pre, bs, post,
+                                                   vnni, out.data_ptr(), st))
         return out
 
     @classmethod

@@ -62,6 +62,8 @@ class TppCache:
         self.layers = {}          # layer_idx -> (k, v)
         self.seq_len_dev = None   # int32 [1]: keys in the cache (same for every layer)
         self._host_len = 0
+        self._sync_len = 0        # length every layer had when the fused layers last advanced the cache
+        self._layer_len = {}      # layers that update() has moved since then
         # decode steps: row sums of squares of the residual stream, handed from the GEMM that writes it to the
         # GEMM behind the next RMSNorm (two tables: after attention, after the MLP) + the tensor the second belongs to
         self._sums = None
@@ -69,7 +71,7 @@ class TppCache:
 
     # -- reference method names -------------------------------------------------
     def get_seq_length(self, layer_idx=0):
-        return self._host_len
+        return self._layer_len.get(layer_idx, self._host_len if layer_idx == 0 else self._sync_len)
 
     def get_capacity(self):
         return self.capacity
@@ -85,6 +87,8 @@ class TppCache:
         if self._host_len > max_length:
             self._host_len = int(max_length)
             self.seq_len_dev.fill_(self._host_len)
+        self._sync_len = min(self._sync_len, int(max_length))
+        self._layer_len = {i: min(n, int(max_length)) for i, n in self._layer_len.items()}
 
     def reorder_cache(self, beam_idx):
         """attn.h:327-366 (beam search): afterwards sequence b continues the keys and values sequence beam_idx[b]
@@ -123,7 +127,8 @@ class TppCache:
         k, v = self._ensure(layer_idx, B, Nkv, H, keys.device)
         k[:, :, :S].copy_(keys)
         v[:, :, :S].copy_(values)
-        self._host_len = S
+        self._host_len = self._sync_len = S
+        self._layer_len = {}
         self.seq_len_dev.fill_(S)
         return self
 
@@ -131,6 +136,46 @@ class TppCache:
         """One decode step appended n keys to every layer (host-side bookkeeping + device counter)."""
         self._host_len += n
         self.seq_len_dev.add_(n)
+        self._sync_len = self._host_len
+        self._layer_len = {}
+
+    def update(self, key_states, value_states, layer_idx):
+        """TppCache::update / LayerCache::update (src/csrc/llm/attn.h:198-222,258-274): append key_states /
+        value_states [B][Nkv][S][H] (bf16, already rotated) to layer `layer_idx` at that layer's length and return
+        the layer's [keys, values] up to the new length.  A cache that is too small grows by KV_CACHE_INC_SIZE
+        positions beyond what is needed, as the reference's does.  The fused decoder layers do not come through
+        here (they append inside their attention launch); this is the way in for callers that hold k / v tensors.
+        Lengths are tracked per layer like the reference's offsets; the shared counter follows layer 0."""
+        B, Nkv, S, H = key_states.shape
+        if value_states.shape != key_states.shape:
+            raise TppxError(_lib.ESHAPE, "TppCache.update: keys and values differ in shape")
+        base = self._layer_len.get(layer_idx, self._sync_len)
+        if self.capacity < base + S:
+            self._grow(base + S + int(os.environ.get("KV_CACHE_INC_SIZE", "128")))
+        k, v = self._ensure(layer_idx, B, Nkv, H, key_states.device)
+        if k.shape[0] != B or k.shape[1] != Nkv or k.shape[3] != H:
+            raise TppxError(_lib.ESHAPE, f"TppCache.update: states {tuple(key_states.shape)} do not fit the cache "
+                                         f"{tuple(k.shape)}")
+        k[:, :, base:base + S].copy_(key_states)
+        v[:, :, base:base + S].copy_(value_states)
+        self._layer_len[layer_idx] = base + S
+        if layer_idx == 0:
+            self._host_len = base + S
+            self.seq_len_dev.fill_(self._host_len)
+        self._sums_of = None
+        return [k[:, :, :base + S], v[:, :, :base + S]]
+
+    def _grow(self, new_capacity):
+        """Reallocate every layer for `new_capacity` positions, rounded up to whole blocks of 32 like the
+        reference's storage (attn.h:186-194)."""
+        new_capacity = (new_capacity + self.block_size - 1) // self.block_size * self.block_size
+        for i, (k, v) in list(self.layers.items()):
+            nk = torch.zeros((k.shape[0], k.shape[1], new_capacity, k.shape[3]), dtype=k.dtype, device=k.device)
+            nv = torch.zeros_like(nk)
+            nk[:, :, :k.shape[2]].copy_(k)
+            nv[:, :, :v.shape[2]].copy_(v)
+            self.layers[i] = (nk, nv)
+        self.capacity = new_capacity
 
 
 class LlamaDecoderLayer:

@@ -118,8 +118,8 @@ def FixLinear(self, bk=None, bc=None, layer_dtype=global_layer_dtype, parallel_d
 
 class TppCache:
     """past_key_values object of the optimized models (llm_common.py:80-182): a thin wrapper around the cache the
-    fused decoder layers append to (`get_cpp()`).  Keys are appended inside the layers, so `update` is not a
-    way in."""
+    fused decoder layers append to (`get_cpp()`).  The fused layers append keys inside their attention launch;
+    `update` serves callers that hold key / value tensors themselves."""
 
     # what transformers' generate() asks of a cache object it did not create
     is_compileable = False
@@ -139,7 +139,8 @@ class TppCache:
         raise NotImplementedError
 
     def update(self, key_states, value_states, layer_idx, cache_kwargs=None):
-        raise NotImplementedError("the fused decoder layer appends keys and values itself")
+        """llm_common.py:113-124 of the reference: append to the layer and return [keys, values]."""
+        return self.tpp_cache.update(key_states, value_states, layer_idx)
 
     def get_seq_length(self, layer_idx=0):
         return self.tpp_cache.get_seq_length(layer_idx)

@@ -45,6 +45,8 @@ def _quantize_blocked(blocked, weight_dtype):
         return qtype.remap_and_quantize_mxfp4(blocked)
     if weight_dtype == "qint8":
         return qtype.remap_and_quantize_qint8(blocked)
+    if weight_dtype == "qint2":
+        return qtype.remap_and_quantize_qint2_intlv(blocked)
     raise ValueError(f"Unknown weight_dtype {weight_dtype}")
 
 
