@@ -41,7 +41,7 @@ def _make(fmt, N, K, seed):
     return qw, q_or, s_or
 
 
-def _run(fmt, M, N, K, post, with_bias, seed, ulps=1):
+def _run(fmt, M, N, K, post, with_bias, seed, ulps=1, flags=0):
     ops = _ops()
     qw, q_or, s_or = _make(fmt, N, K, seed)
     x = randn_bf16((M, K), 1.0, seed + 1)
@@ -50,7 +50,7 @@ def _run(fmt, M, N, K, post, with_bias, seed, ulps=1):
     in2 = randn_bf16((M, N), 1.0, seed + 4)
     scale = 0.5 if post in ("add", "add2") else 1.0
     y = ops.linear(x.cuda(), qw, None if bias is None else bias.cuda(), POSTS[post],
-                   in1.cuda(), in2.cuda(), scale)
+                   in1.cuda(), in2.cuda(), scale, flags=flags)
     torch.cuda.synchronize()
     lin = O.linear_mxfp4 if fmt == "mxfp4" else O.linear_qint8
     ref = lin(t2bits(x), q_or, s_or, None if bias is None else t2bits(bias), POSTS[post],
@@ -163,10 +163,22 @@ def test_module_api_and_errors():
 
 @pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])
 @pytest.mark.parametrize("M", [65, 200, 256])
-def test_prefill_tiled_small(fmt, M):
-    """More than 64 rows takes the LDS-tiled kernels; N = 384 leaves the last
-    128-wide block half empty, M = 65 / 200 leave the last row block ragged."""
-    _run(fmt, M, 384, 1024, "add", True, 500 + M)
+@pytest.mark.parametrize("family", ["tiled", "skinny", "auto"])
+def test_prefill_tiled_small(fmt, M, family):
+    """More than 64 rows: the LDS-tiled kernels (N = 384 leaves the last 128-wide block half empty, M = 65 / 200
+    leave the last row block ragged) or the decode kernels over several block rows of 64 (the library picks by a
+    cost estimate; both families forced here)."""
+    from tpp_pytorch_extension import _lib
+    flags = {"tiled": _lib.FLAG_FORCE_TILED, "skinny": _lib.FLAG_FORCE_SKINNY, "auto": 0}[family]
+    _run(fmt, M, 384, 1024, "add", True, 500 + M, flags=flags)
+
+
+@pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])
+@pytest.mark.parametrize("M,N,K", [(128, 11008, 1024), (192, 4096, 2048), (130, 512, 11008)])
+def test_mid_size_m_block_rows(fmt, M, N, K):
+    """65..256 rows at 7B-like widths: few output tiles, so the decode kernels run block rows of 64 over the full
+    grid (ragged last block row, three channel tiles per workgroup, K split over the waves)."""
+    _run(fmt, M, N, K, "add", True, 8800 + M)
 
 
 @pytest.mark.parametrize("post", ["none", "silu", "mul", "add2", "gelu"])
@@ -466,8 +478,10 @@ def test_launch_plan_names_the_kernels():
     assert buf.value.decode().count("\n") == 1 and "skinny_qint8_fq_kernel<" in buf.value.decode()
     _lib.check(L.tppx_plan_linear_mxfp4(2048, 8192, 8192, 0, 0, buf, len(buf)))
     assert "big_mxfp4_kernel" in buf.value.decode()
-    _lib.check(L.tppx_plan_linear_mxfp4(100, 8192, 8192, 0, 0, buf, len(buf)))
+    _lib.check(L.tppx_plan_linear_mxfp4(100, 8192, 8192, _lib.FLAG_FORCE_TILED, 0, buf, len(buf)))
     assert "tiled_mxfp4_kernel" in buf.value.decode()
+    _lib.check(L.tppx_plan_linear_mxfp4(128, 11008, 4096, 0, 0, buf, len(buf)))  # few tiles: block rows of 64
+    assert "skinny_mxfp4_mg_kernel" in buf.value.decode() and "x2x" in buf.value.decode()
 
 
 @pytest.mark.parametrize("M,N,K,post,layout", [

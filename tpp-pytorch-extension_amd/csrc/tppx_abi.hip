@@ -201,12 +201,30 @@ static int fill_all(const char* who, const tppx_seg* segs, int n_segs, int n_mul
 
 static const int64_t TILED_MIN_M = 65; // more rows than the decode kernels cover in one block row
 
-static bool want_tiled(int64_t M, int flags) {
+// More than 64 rows: the LDS-tiled kernels give every workgroup a whole output tile and all of K, so a launch with
+// few tiles leaves most of the 256 CUs idle (7B shapes at 256 rows: 43 workgroups), while the decode kernels run one
+// block row of 64 rows after the other over the full grid, streaming the weights once per block row.  Pick by a
+// cost estimate fitted to measurements on MI355X (us): a block row costs about 8 + weight bytes / 5.5 TB/s + 0.8 ns
+// per input channel (its activations), a round of 256 x 256 tiles about 14.5 ns per input channel (128 x 128: 20).  `wbytes` = weight bytes of the whole call, `n_tiles16` = its 16-channel
+// tiles.  TPPX_TILED_MIN_M (when set) restores a plain row threshold.
+static bool want_tiled(int64_t M, int flags, int64_t K = 0, int64_t n_tiles16 = 0, double wbytes = 0.0) {
   if (flags & TPPX_FLAG_FORCE_SKINNY)
     return false;
   if (flags & TPPX_FLAG_FORCE_TILED)
     return true;
-  return M >= env_int("TPPX_TILED_MIN_M", (int)TILED_MIN_M);
+  if (M < TILED_MIN_M)
+    return false;
+  const int env_min = env_int("TPPX_TILED_MIN_M", -1);
+  if (env_min >= 0)
+    return M >= env_min;
+  if (K <= 0 || n_tiles16 <= 0 || M > 1024)
+    return true;
+  const bool big = M >= env_int("TPPX_TILED_BIG_MIN_M", 192);
+  const int64_t rows = big ? 256 : 128, cols16 = big ? 16 : 8;
+  const int64_t wgs = ((M + rows - 1) / rows) * ((n_tiles16 + cols16 - 1) / cols16);
+  const double tiled_us = (double)((wgs + 255) / 256) * (double)K * 0.0145 * (big ? 1.0 : 1.4);
+  const double skinny_us = (double)((M + 63) / 64) * (8.0 + wbytes / 5.5e6 + (double)K * 0.0008);
+  return tiled_us <= skinny_us;
 }
 
 static TiledParams tiled_from_seg(const DecodeParams& p, int i) {
@@ -298,7 +316,8 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
       return rc;
     return check_hip(launch_tiled_mxfp4_fp8_group(&t[1], 1, stream), who);
   }
-  if (want_tiled(M, flags)) {
+  if (want_tiled(M, flags, K, dual ? 2 * p.total_tiles : p.total_tiles,
+                 (dual ? 2.0 : 1.0) * (double)p.total_tiles * 16.0 * (double)K * (0.5 + 1.0 / 32))) {
     TPPX_REQUIRE(!row_sumsq, TPPX_EUNSUPPORTED, "%s: row sums of squares are not produced by the large-M kernels", who);
     // prefill shapes: one LDS-tiled launch per GEMM of the group; the fused
     // gate/up pair becomes silu(gate) followed by up * gate (same rounding)
@@ -411,7 +430,7 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
   p.units = (int)(K / qbs);
   p.tpb = (int)(qbs / 64);
   const bool reuse = (flags & TPPX_FLAG_XQ_REUSE) != 0; // xq / sa still hold this x, quantized by an earlier call
-  if (want_tiled(M, flags) && qbs % 128 == 0) {
+  if (qbs % 128 == 0 && want_tiled(M, flags, K, p.total_tiles, (double)p.total_tiles * 16.0 * (double)K)) {
     if (x && !reuse) {
       rc = check_hip(launch_quant_act_int8(x, M, K, qbs, xq, sa, 0, stream), who);
       if (rc)
