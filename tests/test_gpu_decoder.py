@@ -72,9 +72,14 @@ def _attn(F, q, kc, vc, L, mask=None, ws=True):
     return out
 
 
+@pytest.mark.parametrize("kernel", ["auto", "rows", "wide"])
 @pytest.mark.parametrize("B,Nq,Nkv,L,Smax", [(1, 32, 32, 2048, 2304), (3, 8, 2, 77, 128), (2, 4, 4, 1, 64),
-                                             (16, 32, 32, 300, 512)])
-def test_attn_decode(B, Nq, Nkv, L, Smax):
+                                             (16, 32, 32, 300, 512), (1, 32, 32, 129, 4096), (2, 8, 8, 1000, 1000)])
+def test_attn_decode(B, Nq, Nkv, L, Smax, kernel, monkeypatch):
+    """Both single-query kernels (64 keys per trip on scalar arithmetic; 128 keys per trip on the packed bf16 dot
+    instruction) on every shape, and the launch planner's own choice."""
+    if kernel != "auto":
+        monkeypatch.setenv("TPPX_ATTN_WIDE", "1" if kernel == "wide" else "0")
     F = _llm()
     q = randn_bf16((B, Nq, 128), 1.0, 31)
     k = randn_bf16((B, Nkv, Smax, 128), 1.0, 32)
@@ -113,9 +118,11 @@ def test_attn_decode_split_merge_in_launch_equals_second_kernel(monkeypatch):
         assert torch.equal(o, two)
 
 
+@pytest.mark.parametrize("kernel", ["rows", "wide"])
 @pytest.mark.parametrize("B,Nq,Nkv,L0,Smax,B_pos", [(1, 32, 32, 2048, 2304, 1), (3, 8, 2, 300, 512, 3), (2, 4, 4, 0, 64, 1),
-                                                     (16, 32, 32, 77, 128, 16)])
-def test_attn_decode_with_rotary_and_append_in_the_launch(B, Nq, Nkv, L0, Smax, B_pos):
+                                                     (16, 32, 32, 77, 128, 16), (1, 8, 8, 255, 256, 1), (2, 4, 2, 128, 512, 2)])
+def test_attn_decode_with_rotary_and_append_in_the_launch(B, Nq, Nkv, L0, Smax, B_pos, kernel, monkeypatch):
+    monkeypatch.setenv("TPPX_ATTN_WIDE", "1" if kernel == "wide" else "0")
     """tppx_attn_decode_rotary = tppx_rotary_kv_append_llama + tppx_attn_decode(kv_len_add = 1) in one launch: same
     attention output (the rotation may contract its multiply-adds differently: bf16 tolerance), the same key / value
     row appended at position L0, nothing else in the cache touched, q / k / v inputs left as they were."""
@@ -166,12 +173,18 @@ def test_attn_decode_with_rotary_and_append_in_the_launch(B, Nq, Nkv, L0, Smax, 
     assert torch.equal(kcb[:, :, keep], kc0[:, :, keep]) and torch.isfinite(outb.float()).all()
 
 
-def test_attn_decode_mask():
+@pytest.mark.parametrize("kernel", ["rows", "wide"])
+def test_attn_decode_mask(kernel, monkeypatch):
+    """Additive mask over key positions; cache rows past the valid length hold NaN and must not reach the output
+    (the kernels read whole trips, clamped to the cache, and drop what lies past the length)."""
+    monkeypatch.setenv("TPPX_ATTN_WIDE", "1" if kernel == "wide" else "0")
     F = _llm()
     B, Nq, L, Smax = 2, 4, 100, 128
     q = randn_bf16((B, Nq, 128), 1.0, 41)
     k = randn_bf16((B, Nq, Smax, 128), 1.0, 42)
     v = randn_bf16((B, Nq, Smax, 128), 1.0, 43)
+    k[:, :, L:] = float("nan")
+    v[:, :, L:] = float("nan")
     keep = torch.ones(B, L, dtype=torch.int64)
     keep[0, :17] = 0  # left padding of sequence 0
     mask = F.TppCache(Smax).align_and_invert_mask(keep.to(torch.bfloat16))
@@ -179,6 +192,7 @@ def test_attn_decode_mask():
     got = _attn(F, q.cuda(), k.cuda(), v.cuda(), L, mask=mask.cuda())
     ref = O.attn_decode(t2bits(q), t2bits(k[:, :, :L]), t2bits(v[:, :, :L]), mask.float().numpy())
     g, r = bits2f(t2bits(got)).astype(np.float64), bits2f(ref).astype(np.float64)
+    assert np.isfinite(g).all()
     assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3
 
 

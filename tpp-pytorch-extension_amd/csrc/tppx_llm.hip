@@ -172,12 +172,20 @@ rotary_append_kernel(const RotaryParams p) {
 
 // ---------------------------------------------------------------------------
 // Decode attention (one query token per sequence), head size 128, cache
-// [B][Nkv][Smax][128] bf16.  Grid (B*Nq, splits); 4 waves; a wave instruction
-// reads 4 keys (lane = key l>>4, 16-byte chunk l&15); every 16-lane row keeps
-// its own running (max, sum, 8 output dims per lane) over its keys, merged at
-// the end through LDS.  Scores: fp32 dot * 1/sqrt(H) + mask; probabilities are
-// rounded to bf16 before they multiply V (as the CPU path stores them), sums
-// and the output accumulate in fp32.
+// [B][Nkv][Smax][128] bf16.  Grid (B*Nq, splits); split y takes the trips
+// y, y + splits, ... of the key range, whose length is a device scalar.  Two
+// kernels share the split merge (attn_finish):
+//   attn_decode_kernel       4 waves, a wave instruction reads 4 keys (lane =
+//     key l>>4, 16-byte chunk l&15), 64 keys per trip with the next trip
+//     requested ahead; every 16-lane row keeps its own running (max, sum, 8
+//     output dims per lane), merged at the end through LDS: the long loops of
+//     larger batches;
+//   attn_decode_wide_kernel  128 keys per trip on the packed bf16 dot
+//     instruction: the one- or two-trip workgroups of small batches, where
+//     the arithmetic above costs more than the cache stream.
+// Scores: fp32 dot * 1/sqrt(H) + mask; probabilities are rounded to bf16
+// before they multiply V (as the CPU path stores them), sums and the output
+// accumulate in fp32.
 // ---------------------------------------------------------------------------
 struct AttnParams {
   const uint16_t* q;    // [B][Nq][128]
@@ -201,181 +209,21 @@ struct AttnParams {
 
 // Arrival counters of the split launches, one per (sequence, head): zero between launches (the counting
 // instruction wraps on the last arrival); a launch takes a window handed out in rotation by the host.
-constexpr int ATTN_TICKETS = 16384;
-__device__ unsigned int attn_tickets[ATTN_TICKETS];
+// The counters of a launch are all hit within a microsecond or two; side by side they would queue up at the atomic
+// unit of one memory channel, so each one has 256 bytes to itself.
+constexpr int ATTN_TICKETS = 4096;
+constexpr int ATTN_TICKET_STRIDE = 64; // in counters
+__device__ unsigned int attn_tickets[ATTN_TICKETS * ATTN_TICKET_STRIDE];
 
 __device__ __forceinline__ uint4 as_uint4(const i32x4& v) {
   return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
 }
 
-// ROT: the launch also does what the rotary + append launch did before it (fused_llm_infer.cpp:1252-1253 and
-// LayerCache::update, attn.h:198-222): q and the new key arrive unrotated, every workgroup rotates its query, the
-// key / value of the new token (cache position *kv_len) are taken from registers wherever that position is read,
-// and one workgroup per KV head writes them into the cache.  Rotated values are rounded to bf16 first, as stored.
-template <bool ROT>
-__global__ void __launch_bounds__(256)
-attn_decode_kernel(const AttnParams p) {
-  __shared__ float sm[16], sl[16];
-  __shared__ float sacc[16][128];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int g = lane >> 4, c = lane & 15;
-  const int bh = blockIdx.x, b = bh / p.Nq, hq = bh - b * p.Nq;
-  const int hk = hq / (p.Nq / p.Nkv);
-  const int len0 = *p.kv_len;
-  const int L = max(0, min(len0 + p.kv_len_add, p.Smax));
-  const int nk = (ROT && len0 >= 0 && len0 < p.Smax) ? len0 : -1; // cache position of the new token
-  // this workgroup's keys: [k0, k1), split evenly in multiples of 64
-  const int per = ((L + p.splits - 1) / p.splits + 63) & ~63;
-  const int k0 = blockIdx.y * per, k1 = min(k0 + per, L);
-
-  float qf[8];
-  i32x4 knew = {0, 0, 0, 0}, vnew = {0, 0, 0, 0};
-  if (!ROT) {
-    unpack8(reinterpret_cast<const uint4*>(p.q + (int64_t)bh * 128)[c], qf);
-  } else {
-    // chunk c holds first halves (c < 8) or second halves of the rotation pairs (h2, 64 + h2); partner chunk c ^ 8
-    const bool first = c < 8;
-    const int64_t pp = p.pos[p.B_pos == 1 ? 0 : b];
-    const bool rot = p.emb != nullptr && pp >= 0 && pp < p.MP;
-    float cs[8], sn[8];
-#pragma unroll
-    for (int e = 0; e < 8; e++)
-      cs[e] = sn[e] = 0.f;
-    if (rot) {
-      const float* cp = p.emb + pp * 128 + (c & 7) * 8;
-      const float* sp = p.emb + ((int64_t)p.MP + pp) * 128 + (c & 7) * 8;
-#pragma unroll
-      for (int e = 0; e < 8; e++) {
-        cs[e] = cp[e];
-        sn[e] = sp[e];
-      }
-    }
-    auto rotate = [&](const uint16_t* row, float (&r)[8]) -> uint4 {
-      const uint4 w = reinterpret_cast<const uint4*>(row)[c];
-      if (!rot) {
-        unpack8(w, r);
-        return w;
-      }
-      const uint4 wo = reinterpret_cast<const uint4*>(row)[c ^ 8];
-      float a[8], o[8];
-      unpack8(w, a);
-      unpack8(wo, o);
-#pragma unroll
-      for (int e = 0; e < 8; e++)
-        r[e] = first ? a[e] * cs[e] - o[e] * sn[e] : a[e] * cs[e] + o[e] * sn[e];
-      const uint4 out = pack8(r);
-      unpack8(out, r); // the rotated row is a bf16 tensor
-      return out;
-    };
-    rotate(p.q + (int64_t)bh * 128, qf);
-    float kr[8];
-    const uint4 kw4 = rotate(p.k_new + ((int64_t)b * p.Nkv + hk) * 128, kr);
-    knew = i32x4{(int)kw4.x, (int)kw4.y, (int)kw4.z, (int)kw4.w};
-    vnew = *reinterpret_cast<const i32x4*>(p.v_new + ((int64_t)b * p.Nkv + hk) * 128 + c * 8);
-    // one workgroup per KV head appends: the first query head of the group, the split that owns the position
-    if (nk >= 0 && hq == hk * (p.Nq / p.Nkv) && nk >= k0 && nk < k1 && tid < 16) {
-      const int64_t o = (((int64_t)b * p.Nkv + hk) * p.Smax + nk) * 128 + c * 8;
-      *reinterpret_cast<i32x4*>(const_cast<uint16_t*>(p.kc) + o) = knew;
-      *reinterpret_cast<i32x4*>(const_cast<uint16_t*>(p.vc) + o) = vnew;
-    }
-  }
-#pragma unroll
-  for (int e = 0; e < 8; e++)
-    qf[e] *= p.scale;
-  const uint4* kb = reinterpret_cast<const uint4*>(p.kc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128) + c;
-  const uint4* vb = reinterpret_cast<const uint4*>(p.vc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128) + c;
-  const uint16_t* mrow = p.mask ? p.mask + (int64_t)b * p.mask_ld : nullptr;
-
-  float m = -3.0e38f, l = 0.f, acc[8];
-#pragma unroll
-  for (int e = 0; e < 8; e++)
-    acc[e] = 0.f;
-  constexpr int NU = 4; // keys per DPP row and trip (8 measured no better)
-  // 4 * NU keys per wave and trip (NU per DPP row); the next trip's K and V rows are requested before this trip's
-  // arithmetic so that a wave always has loads in flight (keys past the end re-read the last key, never used)
-  i32x4 kw[NU], vw[NU], kn[NU], vn[NU];
-  auto load_kv = [&](int base, i32x4 (&kd)[NU], i32x4 (&vd)[NU]) {
-#pragma unroll
-    for (int u = 0; u < NU; u++) {
-      const int kk = max(min(base + u * 4 + g, L - 1), 0);
-      kd[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(kb + (int64_t)kk * 16));
-      vd[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(vb + (int64_t)kk * 16));
-      if (ROT && kk == nk) { // not in the cache yet (or being written by another workgroup right now)
-        kd[u] = knew;
-        vd[u] = vnew;
-      }
-    }
-  };
-  load_kv(k0 + wave * (4 * NU), kw, vw);
-  for (int base = k0 + wave * (4 * NU); base < k1; base += 16 * NU) {
-    load_kv(base + 16 * NU, kn, vn);
-    int key[NU];
-#pragma unroll
-    for (int u = 0; u < NU; u++)
-      key[u] = base + u * 4 + g;
-    float sc[NU];
-#pragma unroll
-    for (int u = 0; u < NU; u++) {
-      float kf[8];
-      unpack8(as_uint4(kw[u]), kf);
-      float d = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; e++)
-        d = fmaf(qf[e], kf[e], d);
-      d = row16_sum(d);
-      if (mrow && key[u] < p.mask_ld && key[u] < k1)
-        d += bf16_bits_to_f32(mrow[key[u]]);
-      sc[u] = key[u] < k1 ? d : -3.0e38f;
-    }
-    float mn = m;
-#pragma unroll
-    for (int u = 0; u < NU; u++)
-      mn = fmaxf(mn, sc[u]);
-    const float alpha = __expf(m - mn);
-    l *= alpha;
-#pragma unroll
-    for (int e = 0; e < 8; e++)
-      acc[e] *= alpha;
-#pragma unroll
-    for (int u = 0; u < NU; u++) {
-      const float pr = key[u] < k1 ? __expf(sc[u] - mn) : 0.f;
-      l += pr;
-      const float pb = round_bf16(pr);
-      float vf[8];
-      unpack8(as_uint4(vw[u]), vf);
-#pragma unroll
-      for (int e = 0; e < 8; e++)
-        acc[e] = fmaf(pb, vf[e], acc[e]);
-    }
-    m = mn;
-#pragma unroll
-    for (int u = 0; u < NU; u++) {
-      kw[u] = kn[u];
-      vw[u] = vn[u];
-    }
-  }
-  // merge the 16 (wave, row) states
-  const int st = wave * 4 + g;
-  if (c == 0) {
-    sm[st] = m;
-    sl[st] = l;
-  }
-#pragma unroll
-  for (int e = 0; e < 8; e++)
-    sacc[st][c * 8 + e] = acc[e];
-  __syncthreads();
+// Shared end of the single-query kernels.  Threads tid < 128 hold output dimension tid of this workgroup's state: the
+// running max M, the sum Ls and the unnormalised output o.  One split: normalise and store.  Several: store the state;
+// with arrival counters the split that arrives last merges all of them inside the launch.
+__device__ __forceinline__ void attn_finish(const AttnParams& p, int bh, int tid, float M, float Ls, float o) {
   if (tid < 128) {
-    float M = sm[0];
-#pragma unroll
-    for (int i = 1; i < 16; i++)
-      M = fmaxf(M, sm[i]);
-    float Ls = 0.f, o = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-      const float w = __expf(sm[i] - M);
-      Ls = fmaf(w, sl[i], Ls);
-      o = fmaf(w, sacc[i][tid], o);
-    }
     if (p.splits == 1) {
       p.out[(int64_t)bh * 128 + tid] = (uint16_t)f32_to_bf16_bits(Ls > 0.f ? o / Ls : 0.f);
     } else if (p.ticket0 < 0) {
@@ -406,7 +254,7 @@ attn_decode_kernel(const AttnParams p) {
   __syncthreads();
   if (tid == 0) {
     const unsigned int last = (unsigned int)p.splits - 1;
-    arrived_last = atomicInc(&attn_tickets[p.ticket0 + bh], last) == last;
+    arrived_last = atomicInc(&attn_tickets[(p.ticket0 + bh) * ATTN_TICKET_STRIDE], last) == last;
   }
   __syncthreads();
   if (!arrived_last || tid >= 128)
@@ -423,12 +271,13 @@ attn_decode_kernel(const AttnParams p) {
       po[i] = __hip_atomic_load(src + i * 130 + 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
-  float M = -3.0e38f;
+  M = -3.0e38f;
 #pragma unroll
   for (int i = 0; i < 32; i++)
     if (i < p.splits)
       M = fmaxf(M, pm[i]);
-  float Ls = 0.f, o = 0.f;
+  Ls = 0.f;
+  o = 0.f;
 #pragma unroll
   for (int i = 0; i < 32; i++)
     if (i < p.splits) {
@@ -437,6 +286,433 @@ attn_decode_kernel(const AttnParams p) {
       o = fmaf(w, po[i], o);
     }
   p.out[(int64_t)bh * 128 + tid] = (uint16_t)f32_to_bf16_bits(Ls > 0.f ? o / Ls : 0.f);
+}
+
+
+// ROT: the launch also does what the rotary + append launch did before it (fused_llm_infer.cpp:1252-1253 and
+// LayerCache::update, attn.h:198-222): q and the new key arrive unrotated, every workgroup rotates its query, the
+// key / value of the new token (cache position *kv_len) are taken from registers wherever that position is read,
+// and one workgroup per KV head writes them into the cache.  Rotated values are rounded to bf16 first, as stored.
+template <bool ROT>
+__global__ void __launch_bounds__(256)
+attn_decode_kernel(const AttnParams p) {
+  __shared__ float sm[16], sl[16];
+  __shared__ float sacc[16][128];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 4, c = lane & 15;
+  const int bh = blockIdx.x, b = bh / p.Nq, hq = bh - b * p.Nq;
+  const int hk = hq / (p.Nq / p.Nkv);
+  const uint4* kb = reinterpret_cast<const uint4*>(p.kc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128) + c;
+  const uint4* vb = reinterpret_cast<const uint4*>(p.vc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128) + c;
+  constexpr int NU = 4; // keys per DPP row and trip (8 measured no better)
+  // One trip = 64 keys per workgroup, 4 * NU per wave (NU per DPP row).  Split y takes trips y, y + splits, ...: the
+  // splits differ by at most one trip whatever the length is, and the first trip's rows do not depend on the length
+  // (a device scalar), so they are requested here, before anything else is read: the cache stream starts with the
+  // launch.  Rows are clamped to the cache's last row; a trip past the end is read and never used (at most one per
+  // workgroup).  Inside the loop the next trip is requested before this trip's arithmetic.
+  i32x4 kw[NU], vw[NU], kn[NU], vn[NU];
+  auto load_kv = [&](int base, i32x4 (&kd)[NU], i32x4 (&vd)[NU]) {
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+      const int kk = min(base + u * 4 + g, p.Smax - 1);
+      kd[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(kb + (int64_t)kk * 16));
+      vd[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(vb + (int64_t)kk * 16));
+    }
+  };
+  load_kv(blockIdx.y * 64 + wave * (4 * NU), kw, vw);
+  const int len0 = *p.kv_len;
+  const int L = max(0, min(len0 + p.kv_len_add, p.Smax));
+  const int nk = (ROT && len0 >= 0 && len0 < p.Smax) ? len0 : -1; // cache position of the new token
+  const int trips = (L + 63) >> 6;
+  // the split whose trips contain the new token's position (wave-uniform)
+  const bool has_new = ROT && nk >= 0 && nk < L && ((nk >> 6) % p.splits) == (int)blockIdx.y;
+
+  float qf[8];
+  i32x4 knew = {0, 0, 0, 0}, vnew = {0, 0, 0, 0};
+  if (!ROT) {
+    unpack8(reinterpret_cast<const uint4*>(p.q + (int64_t)bh * 128)[c], qf);
+  } else {
+    // chunk c holds first halves (c < 8) or second halves of the rotation pairs (h2, 64 + h2); partner chunk c ^ 8
+    const bool first = c < 8;
+    const int64_t pp = p.pos[p.B_pos == 1 ? 0 : b];
+    const bool rot = p.emb != nullptr && pp >= 0 && pp < p.MP;
+    float cs[8], sn[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      cs[e] = sn[e] = 0.f;
+    if (rot) { // rows of 128 floats, 8 per chunk: 32-byte aligned
+      const f32x4* cp = reinterpret_cast<const f32x4*>(p.emb + pp * 128 + (c & 7) * 8);
+      const f32x4* sp = reinterpret_cast<const f32x4*>(p.emb + ((int64_t)p.MP + pp) * 128 + (c & 7) * 8);
+      const f32x4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        cs[e] = c0[e];
+        cs[4 + e] = c1[e];
+        sn[e] = s0[e];
+        sn[4 + e] = s1[e];
+      }
+    }
+    auto rotate = [&](const uint16_t* row, float (&r)[8]) -> uint4 {
+      const uint4 w = reinterpret_cast<const uint4*>(row)[c];
+      if (!rot) {
+        unpack8(w, r);
+        return w;
+      }
+      const uint4 wo = reinterpret_cast<const uint4*>(row)[c ^ 8];
+      float a[8], o[8];
+      unpack8(w, a);
+      unpack8(wo, o);
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        r[e] = first ? a[e] * cs[e] - o[e] * sn[e] : a[e] * cs[e] + o[e] * sn[e];
+      const uint4 out = pack8(r);
+      unpack8(out, r); // the rotated row is a bf16 tensor
+      return out;
+    };
+    rotate(p.q + (int64_t)bh * 128, qf);
+    if (has_new) { // only the split that reads the new token's position needs its key and value
+      float kr[8];
+      const uint4 kw4 = rotate(p.k_new + ((int64_t)b * p.Nkv + hk) * 128, kr);
+      knew = i32x4{(int)kw4.x, (int)kw4.y, (int)kw4.z, (int)kw4.w};
+      vnew = *reinterpret_cast<const i32x4*>(p.v_new + ((int64_t)b * p.Nkv + hk) * 128 + c * 8);
+      // one workgroup per KV head appends: the first query head of the group
+      if (hq == hk * (p.Nq / p.Nkv) && tid < 16) {
+        const int64_t o = (((int64_t)b * p.Nkv + hk) * p.Smax + nk) * 128 + c * 8;
+        *reinterpret_cast<i32x4*>(const_cast<uint16_t*>(p.kc) + o) = knew;
+        *reinterpret_cast<i32x4*>(const_cast<uint16_t*>(p.vc) + o) = vnew;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    qf[e] *= p.scale;
+  const uint16_t* mrow = p.mask ? p.mask + (int64_t)b * p.mask_ld : nullptr;
+
+  float m = -3.0e38f, l = 0.f, acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    acc[e] = 0.f;
+  // the new token is not in the cache yet (or is being written by another workgroup right now): wherever its
+  // position was read, the registers replace what the load returned
+  auto patch_new = [&](int base, i32x4 (&kd)[NU], i32x4 (&vd)[NU]) {
+    if (has_new) {
+#pragma unroll
+      for (int u = 0; u < NU; u++)
+        if (base + u * 4 + g == nk) {
+          kd[u] = knew;
+          vd[u] = vnew;
+        }
+    }
+  };
+  patch_new(blockIdx.y * 64 + wave * (4 * NU), kw, vw);
+  for (int t = blockIdx.y; t < trips; t += p.splits) {
+    const int base = t * 64 + wave * (4 * NU);
+    if (t + p.splits < trips) {
+      load_kv(base + p.splits * 64, kn, vn);
+      patch_new(base + p.splits * 64, kn, vn);
+    }
+    int key[NU];
+#pragma unroll
+    for (int u = 0; u < NU; u++)
+      key[u] = base + u * 4 + g;
+    float sc[NU];
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+      float kf[8];
+      unpack8(as_uint4(kw[u]), kf);
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        d = fmaf(qf[e], kf[e], d);
+      d = row16_sum(d);
+      if (mrow && key[u] < p.mask_ld && key[u] < L)
+        d += bf16_bits_to_f32(mrow[key[u]]);
+      sc[u] = key[u] < L ? d : -3.0e38f;
+    }
+    float mn = m;
+#pragma unroll
+    for (int u = 0; u < NU; u++)
+      mn = fmaxf(mn, sc[u]);
+    const float alpha = __expf(m - mn);
+    l *= alpha;
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      acc[e] *= alpha;
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+      const float pr = key[u] < L ? __expf(sc[u] - mn) : 0.f;
+      l += pr;
+      const float pb = round_bf16(pr);
+      if (t * 64 + 64 > L && key[u] >= L) // rows past the end may hold anything, NaN included
+        vw[u] = i32x4{0, 0, 0, 0};
+      float vf[8];
+      unpack8(as_uint4(vw[u]), vf);
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        acc[e] = fmaf(pb, vf[e], acc[e]);
+    }
+    m = mn;
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+      kw[u] = kn[u];
+      vw[u] = vn[u];
+    }
+  }
+  // merge the 16 (wave, row) states
+  const int st = wave * 4 + g;
+  if (c == 0) {
+    sm[st] = m;
+    sl[st] = l;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    sacc[st][c * 8 + e] = acc[e];
+  __syncthreads();
+  float M = -3.0e38f, Ls = 0.f, o = 0.f;
+  if (tid < 128) {
+    M = sm[0];
+#pragma unroll
+    for (int i = 1; i < 16; i++)
+      M = fmaxf(M, sm[i]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const float w = __expf(sm[i] - M);
+      Ls = fmaf(w, sl[i], Ls);
+      o = fmaf(w, sacc[i][tid], o);
+    }
+  }
+  attn_finish(p, bh, tid, M, Ls, o);
+}
+
+// ---------------------------------------------------------------------------
+// The same single-query attention for few trips per workgroup: at batch 1 the
+// cache of one head is a few hundred KB, every workgroup makes one or two
+// trips, and the vector arithmetic of the kernel above (bf16 unpacking, one
+// multiply-add per element, a 16-lane reduction per 4 keys) costs more than
+// the cache stream.  Here a lane owns an eighth (16 dims, chunks j*8 + q8) of
+// FOUR keys per trip -- a wave instruction reads 8 whole rows, a wave covers
+// 32 keys, the workgroup 128 -- and:
+//   * q . k runs on v_dot2c_f32_bf16 (two bf16 products per instruction, no
+//     unpacking), followed by an 8-lane reduction;
+//   * the wave shares one running max (one exp per key and lane);
+//   * p . v pairs the lane's keys: (v_a[e], v_b[e]) . (p_a, p_b), again on
+//     the dot instruction, the pair assembled by one byte permute;
+//   * the query is rotated once per workgroup (wave 0, one rotation pair per
+//     lane) and handed to the lanes through LDS; the new key only in the
+//     split that reads its position.
+// The per-lane outputs (16 dims, partial over the lane's keys) are added up
+// through LDS at the end.  The first trip's K and V rows (16 KB per wave) are
+// requested before anything else; later trips request theirs when they start
+// (the launch planner sends long loops to the kernel above).
+// ---------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_mov<0xB1>(v));
+  v = fmaxf(v, dpp_mov<0x4E>(v));
+  v = fmaxf(v, dpp_mov<0x141>(v));
+  v = fmaxf(v, dpp_mov<0x140>(v));
+  const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
+constexpr int ATTN_WIDE_KEYS = 128; // keys per workgroup and trip
+
+template <bool ROT>
+__global__ void __launch_bounds__(256, 4) // four workgroups per CU: at most 128 registers
+attn_decode_wide_kernel(const AttnParams p) {
+  __shared__ __align__(16) uint16_t q_s[128], k_s[128];
+  __shared__ float sm[4], sl[4];
+  __shared__ __align__(16) float sacc[4][8][132];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kq = lane >> 3, q8 = lane & 7;
+  const int bh = blockIdx.x, b = bh / p.Nq, hq = bh - b * p.Nq;
+  const int hk = hq / (p.Nq / p.Nkv);
+  const int S = p.splits;
+  const char* kb = reinterpret_cast<const char*>(p.kc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128) + q8 * 16;
+  const char* vb = reinterpret_cast<const char*>(p.vc + ((int64_t)b * p.Nkv + hk) * p.Smax * 128) + q8 * 16;
+  // key set s of a trip: keys base + s*8 + kq; register [s][j] holds dims (j*8 + q8)*8 .. +7 as four bf16 pairs
+  i32x4 kr[4][2], vr[4][2];
+  auto load_rows = [&](const char* src, int base, i32x4 (&dst)[4][2]) {
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const int key = min(base + s * 8 + kq, p.Smax - 1); // past the end: read, never used
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+        dst[s][j] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(src + (int64_t)key * 256 + j * 128));
+    }
+  };
+  // A wave's loads return in the order of their issue.  Wave 0 prepares the query (and the new key): it asks for
+  // those few values first, so that they do not queue behind its 16 KB of rows, and rotates them while the rows of
+  // all four waves are on their way.  Lane i owns the rotation pair (i, 64 + i).
+  i32x4 qp[2];
+  float qx1 = 0.f, qx2 = 0.f, kx1 = 0.f, kx2 = 0.f, cs = 1.f, sn = 0.f;
+  bool rot = false;
+  if (!ROT) {
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+      qp[j] = reinterpret_cast<const i32x4*>(p.q + (int64_t)bh * 128)[j * 8 + q8];
+  } else if (wave == 0) {
+    const uint16_t* qrow = p.q + (int64_t)bh * 128;
+    const uint16_t* krow = p.k_new + ((int64_t)b * p.Nkv + hk) * 128;
+    qx1 = bf16_bits_to_f32(qrow[lane]);
+    qx2 = bf16_bits_to_f32(qrow[64 + lane]);
+    kx1 = bf16_bits_to_f32(krow[lane]);
+    kx2 = bf16_bits_to_f32(krow[64 + lane]);
+    const int64_t pp = p.pos[p.B_pos == 1 ? 0 : b];
+    rot = p.emb != nullptr && pp >= 0 && pp < p.MP; // positions outside the table are left unrotated
+    if (rot) {
+      cs = p.emb[pp * 128 + lane];
+      sn = p.emb[((int64_t)p.MP + pp) * 128 + lane];
+    }
+  }
+  load_rows(kb, blockIdx.y * ATTN_WIDE_KEYS + wave * 32, kr);
+  load_rows(vb, blockIdx.y * ATTN_WIDE_KEYS + wave * 32, vr);
+  const int len0 = *p.kv_len;
+  const int L = max(0, min(len0 + p.kv_len_add, p.Smax));
+  const int nk = (ROT && len0 >= 0 && len0 < p.Smax) ? len0 : -1; // cache position of the new token
+  const int trips = (L + ATTN_WIDE_KEYS - 1) / ATTN_WIDE_KEYS;
+  // the split whose trips contain the new token's position (uniform over the workgroup)
+  const bool has_new = ROT && nk >= 0 && nk < L && ((nk / ATTN_WIDE_KEYS) % S) == (int)blockIdx.y;
+
+  if (ROT) {
+    if (wave == 0) {
+      q_s[lane] = (uint16_t)f32_to_bf16_bits(rot ? qx1 * cs - qx2 * sn : qx1);
+      q_s[64 + lane] = (uint16_t)f32_to_bf16_bits(rot ? qx2 * cs + qx1 * sn : qx2);
+      if (has_new) {
+        k_s[lane] = (uint16_t)f32_to_bf16_bits(rot ? kx1 * cs - kx2 * sn : kx1);
+        k_s[64 + lane] = (uint16_t)f32_to_bf16_bits(rot ? kx2 * cs + kx1 * sn : kx2);
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+      qp[j] = reinterpret_cast<const i32x4*>(q_s)[j * 8 + q8];
+    // one workgroup per KV head appends: the first query head of the group, in the split that reads the position
+    if (has_new && hq == hk * (p.Nq / p.Nkv) && tid < 16) {
+      const int64_t o = (((int64_t)b * p.Nkv + hk) * p.Smax + nk) * 128 + tid * 8;
+      *reinterpret_cast<i32x4*>(const_cast<uint16_t*>(p.kc) + o) = reinterpret_cast<const i32x4*>(k_s)[tid];
+      *reinterpret_cast<i32x4*>(const_cast<uint16_t*>(p.vc) + o) =
+          *reinterpret_cast<const i32x4*>(p.v_new + ((int64_t)b * p.Nkv + hk) * 128 + tid * 8);
+    }
+  }
+  const uint16_t* mrow = p.mask ? p.mask + (int64_t)b * p.mask_ld : nullptr;
+
+  float m = -3.0e38f, l = 0.f; // m is the same in every lane of the wave
+  float acc[16];
+#pragma unroll
+  for (int e = 0; e < 16; e++)
+    acc[e] = 0.f;
+  for (int t = blockIdx.y; t < trips; t += S) {
+    const int base = t * ATTN_WIDE_KEYS + wave * 32;
+    if (t != (int)blockIdx.y) { // the workgroups of this kernel make few trips: no request queue across trips
+      load_rows(kb, base, kr);
+      load_rows(vb, base, vr);
+    }
+    if (has_new && nk >= base && nk < base + 32) {
+      // the new token is not in the cache yet (or is being written right now): its lanes take the rotated key from
+      // LDS and the value from the step's input
+      const int s_new = (nk - base) >> 3;
+      if (kq == ((nk - base) & 7)) {
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+          if (s == s_new) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+              kr[s][j] = reinterpret_cast<const i32x4*>(k_s)[j * 8 + q8];
+              vr[s][j] = *reinterpret_cast<const i32x4*>(p.v_new + ((int64_t)b * p.Nkv + hk) * 128 + (j * 8 + q8) * 8);
+            }
+          }
+      }
+    }
+    float sc[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const int key = base + s * 8 + kq;
+      float d = 0.f;
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          d = dot2_bf16((uint32_t)kr[s][j][r], (uint32_t)qp[j][r], d);
+      d += dpp_mov<0xB1>(d);  // the eight parts of the key: quad_perm [1,0,3,2], [2,3,0,1], row_half_mirror
+      d += dpp_mov<0x4E>(d);
+      d += dpp_mov<0x141>(d);
+      d *= p.scale;
+      if (mrow && key < p.mask_ld && key < L)
+        d += bf16_bits_to_f32(mrow[key]);
+      sc[s] = key < L ? d : -3.0e38f;
+    }
+    const float mn = fmaxf(m, wave_max(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]))));
+    if (mn > m) { // wave-uniform; rare once the first trips have passed
+      const float alpha = __expf(m - mn);
+      l *= alpha;
+#pragma unroll
+      for (int e = 0; e < 16; e++)
+        acc[e] *= alpha;
+      m = mn;
+    }
+    uint32_t pk[2] = {0, 0}; // probabilities of the key pairs (0, 1) and (2, 3) as packed bf16
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const int key = base + s * 8 + kq;
+      const float pr = key < L ? __expf(sc[s] - m) : 0.f;
+      l += pr;
+      pk[s >> 1] |= f32_to_bf16_bits(pr) << (16 * (s & 1));
+      if (base + 32 > L && key >= L) { // rows past the end may hold anything, NaN included
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+          vr[s][j] = i32x4{0, 0, 0, 0};
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const uint32_t va = (uint32_t)vr[2 * h][j][r], vb2 = (uint32_t)vr[2 * h + 1][j][r];
+          // v_perm_b32: selector bytes 0..3 pick from the second operand, 4..7 from the first
+          const uint32_t lo = __builtin_amdgcn_perm(vb2, va, 0x05040100u); // (a.dim 2r, b.dim 2r)
+          const uint32_t hi = __builtin_amdgcn_perm(vb2, va, 0x07060302u); // (a.dim 2r+1, b.dim 2r+1)
+          acc[j * 8 + 2 * r] = dot2_bf16(lo, pk[h], acc[j * 8 + 2 * r]);
+          acc[j * 8 + 2 * r + 1] = dot2_bf16(hi, pk[h], acc[j * 8 + 2 * r + 1]);
+        }
+  }
+  // add up the lanes' partial outputs: [wave][kq][dim], rows padded against bank conflicts
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    float* dst = &sacc[wave][kq][(j * 8 + q8) * 8];
+    *reinterpret_cast<f32x4*>(dst) = f32x4{acc[j * 8], acc[j * 8 + 1], acc[j * 8 + 2], acc[j * 8 + 3]};
+    *reinterpret_cast<f32x4*>(dst + 4) = f32x4{acc[j * 8 + 4], acc[j * 8 + 5], acc[j * 8 + 6], acc[j * 8 + 7]};
+  }
+  // every key's l sits in the eight lanes of the key: the wave sum counts it eight times (exactly, a power of two)
+  const float lw = wave_sum(l) * 0.125f;
+  if (lane == 0) {
+    sm[wave] = m;
+    sl[wave] = lw;
+  }
+  __syncthreads();
+  float M = -3.0e38f, Ls = 0.f, o = 0.f;
+  if (tid < 128) {
+    M = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      float so = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+        so += sacc[w][i][tid];
+      const float wt = __expf(sm[w] - M);
+      Ls = fmaf(wt, sl[w], Ls);
+      o = fmaf(wt, so, o);
+    }
+  }
+  attn_finish(p, bh, tid, M, Ls, o);
 }
 
 __global__ void __launch_bounds__(128)
@@ -743,10 +1019,18 @@ extern "C" int tppx_rotary_kv_append_llama(void* q, void* k, const void* v, cons
 // shared tail of the two single-query entry points: split planning, counters, launch
 static int attn_decode_launch(const char* who, AttnParams& p, bool rot, int64_t B, int64_t Nq, int64_t Smax, void* ws,
                               int64_t ws_bytes, hipStream_t stream) {
-  // enough workgroups to cover the chip about twice, at least 256 keys per split
-  const int64_t target = env_int("TPPX_ATTN_TARGET_WGS", 512), min_keys = env_int("TPPX_ATTN_MIN_KEYS", 256);
-  int64_t splits = (target + B * Nq - 1) / (B * Nq);
-  const int64_t max_by_len = (Smax + min_keys - 1) / min_keys;
+  // The wide kernel (128 keys per workgroup and trip) serves launches whose workgroups make few trips; the row
+  // kernel (64 keys per trip, a deeper request queue per wave) the long loops of larger batches.  Measured at batch 1,
+  // 32 heads, 2100 keys: about one workgroup per CU is best (more splits mean more states to merge and more
+  // launches of the same few hundred KB); the row kernel wants about two per CU.  At most one split per trip and at
+  // most 32 (the merge holds every split's state in registers).
+  const int wide_env = (int)env_int("TPPX_ATTN_WIDE", -1);
+  const int64_t target_env = env_int("TPPX_ATTN_TARGET_WGS", 0);
+  const int64_t splits_wide = ((target_env > 0 ? target_env : 288) + B * Nq - 1) / (B * Nq);
+  const bool wide = wide_env >= 0 ? wide_env != 0 : (Smax + ATTN_WIDE_KEYS - 1) / ATTN_WIDE_KEYS <= 4 * splits_wide;
+  int64_t splits = wide ? splits_wide : ((target_env > 0 ? target_env : 512) + B * Nq - 1) / (B * Nq);
+  const int64_t trip_keys = wide ? ATTN_WIDE_KEYS : 64;
+  const int64_t max_by_len = (Smax + trip_keys - 1) / trip_keys;
   if (splits > max_by_len)
     splits = max_by_len;
   if (splits > 32)
@@ -769,7 +1053,11 @@ static int attn_decode_launch(const char* who, AttnParams& p, bool rot, int64_t 
     cursor += (int)(B * Nq);
   }
   const dim3 grid((unsigned)(B * Nq), (unsigned)splits);
-  if (rot)
+  if (wide && rot)
+    attn_decode_wide_kernel<true><<<grid, dim3(256), 0, stream>>>(p);
+  else if (wide)
+    attn_decode_wide_kernel<false><<<grid, dim3(256), 0, stream>>>(p);
+  else if (rot)
     attn_decode_kernel<true><<<grid, dim3(256), 0, stream>>>(p);
   else
     attn_decode_kernel<false><<<grid, dim3(256), 0, stream>>>(p);
