@@ -611,3 +611,62 @@ def test_fp8_activation_qkv_and_swiglu_equal_separate_calls():
     with pytest.raises(TppxError):  # no workspace for the quantised activations
         _lib.check(Lb.tppx_linear_mxfp4(x.data_ptr(), qn.data_ptr(), sn.data_ptr(), None, None, None, y.data_ptr(),
                                         M, 512, K, 0, 1.0, _lib.FLAG_ACT_FP8, None, 0, _lib.stream_of(x)))
+
+
+def test_split_launches_overlapping_on_two_streams():
+    """Launches that split K over workgroups (partial sums in the workspace, an arrival counter per output group, the
+    last arrival merges) and split-KV attention launches, queued on two streams so that they overlap on the card,
+    each stream with a workspace of its own (the workspace is per caller; the counters are shared and handed out in
+    rotation).  Every output must carry the bits of the same call made alone on one stream; the comparison stops
+    at the first mismatch."""
+    from tpp_pytorch_extension import _lib, _ops as ops
+    from tpp_pytorch_extension.llm import fused_llama_infer as F
+    _ops()
+    Lb = _lib.lib()
+    dev = torch.device("cuda:0")
+    cases = []
+    for fmt, M, N, K, seed in (("qint8", 64, 4096, 11008, 701), ("mxfp4", 64, 512, 4096, 702), ("mxfp4", 33, 256, 8192, 703)):
+        qw = _make(fmt, N, K, seed)[0]
+        x = randn_bf16((M, K), 1.0, seed + 1).cuda()
+        r = randn_bf16((M, N), 1.0, seed + 2).cuda()
+        cases.append(("linear", qw, x, r))
+    B, Nq, Smax, Lk = 1, 32, 2304, 2000
+    q = randn_bf16((B, Nq, 128), 1.0, 711).cuda()
+    kc = randn_bf16((B, Nq, Smax, 128), 1.0, 712).cuda()
+    vc = randn_bf16((B, Nq, Smax, 128), 1.0, 713).cuda()
+    ln = torch.tensor([Lk - 1], dtype=torch.int32, device=dev)
+    cases.append(("attn", q, kc, vc))
+
+    def call(case, ws):
+        dev_key = dev.index
+        old = _lib._workspaces.get(dev_key)
+        _lib._workspaces[dev_key] = ws  # the op picks the workspace up when it enqueues
+        try:
+            if case[0] == "linear":
+                _, qw, x, r = case
+                return ops.linear(x, qw, None, POSTS["add"], r, None, 0.5)
+            _, q, kc, vc = case
+            out = torch.empty_like(q)
+            _lib.check(Lb.tppx_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), None, 0, ln.data_ptr(), 1,
+                                           out.data_ptr(), B, Nq, Nq, 128, Smax, ws.data_ptr(), ws.numel(), _lib.stream_of(q)))
+            return out
+        finally:
+            if old is not None:
+                _lib._workspaces[dev_key] = old
+
+    ws0 = _lib.workspace(q)
+    alone = [call(c, ws0) for c in cases]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    wss = [torch.zeros_like(ws0), torch.zeros_like(ws0)]
+    torch.cuda.synchronize()
+    outs = [[], []]
+    for it in range(24):
+        for si in (0, 1):
+            with torch.cuda.stream(streams[si]):
+                ci = (it + 2 * si) % len(cases)  # the two streams run different cases side by side
+                outs[si].append((ci, call(cases[ci], wss[si])))
+    torch.cuda.synchronize()
+    for si in (0, 1):
+        for it, (ci, y) in enumerate(outs[si]):
+            assert torch.equal(y, alone[ci]), f"stream {si}, launch {it}, case {ci}: differs from the single-stream result"

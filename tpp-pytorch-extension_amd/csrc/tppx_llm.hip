@@ -215,6 +215,12 @@ constexpr int ATTN_TICKETS = 4096;
 constexpr int ATTN_TICKET_STRIDE = 64; // in counters
 __device__ unsigned int attn_tickets[ATTN_TICKETS * ATTN_TICKET_STRIDE];
 
+__global__ void attn_clear_tickets_kernel(int first, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n)
+    attn_tickets[(first + i) * ATTN_TICKET_STRIDE] = 0;
+}
+
 __device__ __forceinline__ uint4 as_uint4(const i32x4& v) {
   return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
 }
@@ -1062,6 +1068,12 @@ static int attn_decode_launch(const char* who, AttnParams& p, bool rot, int64_t 
   else
     attn_decode_kernel<false><<<grid, dim3(256), 0, stream>>>(p);
   int rc = check_hip(hipGetLastError(), who);
+  if (rc && p.ticket0 >= 0) {
+    // the refused launch leaves its counter window as it found it, but whoever gets the window next relies on zeros
+    const int n = (int)(B * Nq);
+    attn_clear_tickets_kernel<<<dim3((n + 255) / 256), dim3(256), 0, stream>>>(p.ticket0, n);
+    (void)hipGetLastError();
+  }
   if (rc || splits == 1 || p.ticket0 >= 0)
     return rc;
   attn_combine_kernel<<<dim3((unsigned)(B * Nq)), dim3(128), 0, stream>>>(p);

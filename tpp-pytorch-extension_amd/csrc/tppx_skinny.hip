@@ -1447,13 +1447,28 @@ int skinny_split_tickets(int n) {
   return first;
 }
 
+// A launch that the runtime refused leaves its counter window as it found it, but whoever gets the window next
+// relies on zeros: clear it on the way out (a fill kernel, so the call may sit inside a stream capture).
+__global__ void sk_clear_tickets_kernel(int first, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n)
+    sk_split_tickets[first + i] = 0;
+}
+
 template <typename K>
 static hipError_t sk_launch(K kern, const DecodeParams& p, dim3 grid, int waves, size_t lds, hipStream_t stream) {
   TPPX_PLAN_ONLY(kern, grid, dim3(64 * waves), lds);
-  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds); e != hipSuccess)
-    return e;
-  kern<<<grid, dim3(64 * waves), lds, stream>>>(p);
-  return hipGetLastError();
+  hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds);
+  if (e == hipSuccess) {
+    kern<<<grid, dim3(64 * waves), lds, stream>>>(p);
+    e = hipGetLastError();
+  }
+  if (e != hipSuccess && grid.z > 1 && p.ticket0 >= 0) {
+    const int n = (int)(grid.x * grid.y);
+    sk_clear_tickets_kernel<<<dim3((n + 255) / 256), dim3(256), 0, stream>>>(p.ticket0, n);
+    (void)hipGetLastError(); // the caller reports the launch's own error
+  }
+  return e;
 }
 
 // groups are counted per segment by the caller with the same ntw
