@@ -433,6 +433,21 @@ int tppx_attn_prefill(const void* q, const void* kcache, const void* vcache,
                       void* out, int64_t B, int64_t S, int64_t Nq, int64_t Nkv,
                       int64_t H, int64_t Smax, tppx_stream_t stream);
 
+/* The element-type switch of fc_plain_wrap (src/csrc/llm/fused_llm_infer.cpp:
+ * 1526-1545) for QINT8-family weights and float / half activations, or a
+ * pre-quantized qint8 input whose compute type is float
+ * (TppBlockedQInt8LinearW<float,uint8_t,float>, src/csrc/fused_gemm.h:1076-1341):
+ *   y[m][n] = bias[n] + sum_b float(sum_{k in b} xq*wq) * (sa[m][b]*sw[n][b])
+ * in fp32, one fused multiply-add per K block in ascending order, no post-op.
+ * xq i8 [M][K] row-major and sa f32 [M][K/qbs] come from
+ * tppx_quantize_per_block on the activations (quantize_int8sym,
+ * fused_gemm.h:1248); qw / sw are the native weight tiles / scales; bias f32
+ * [N] or NULL; y f32 [M][N]. */
+int tppx_linear_qint8_f32(const void* xq, const void* sa, const void* qw,
+                          const void* sw, const void* bias_f32, void* y_f32,
+                          int64_t M, int64_t N, int64_t K, int64_t qbs,
+                          tppx_stream_t stream);
+
 /* ---- launch plans ------------------------------------------------------- */
 
 /* No counterpart in the reference.  Writes into buf, one line per kernel, what

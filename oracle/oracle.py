@@ -525,6 +525,24 @@ def linear_qint8(x_bf16, q, sw, bias=None, post=POST_NONE, post_in=None, post_in
     return y
 
 
+def linear_qint8_f32(xq, sa, q, sw, bias=None):
+    """TppBlockedQInt8LinearW<float, uint8_t, float> on pre-quantized activations (fused_gemm.h:1236-1249 with a
+    quantized t_in, 1076-1341): xq int8 [M][K], sa f32 [M][K/qbs] (quantize_int8sym over the last axis), weight
+    q [N/16][K/qbs][qbs/4][16][4] + sw [N/16][K/qbs][1][16]; fp32 bias or None; returns fp32 [M][N]."""
+    xq = _c(xq, np.int8)
+    sa = _c(sa, np.float32)
+    q = _c(q, np.int8)
+    sw = _c(sw, np.float32)
+    M, K = xq.shape
+    n1, nb, a, bk, v = q.shape
+    N, qbs = n1 * 16, a * 4
+    assert nb * qbs == K and sa.shape == (M, nb)
+    bias = None if bias is None else _c(bias, np.float32)
+    y = np.empty((M, N), np.float32)
+    lib().orc_linear_qint8_f32(_p(xq), _p(sa), _c_i64(M), _c_i64(K), _p(q), _p(sw), _c_i64(N), _c_i64(qbs), _p(bias), _p(y))
+    return y
+
+
 def linear_bf16(x_bf16, w_bf16, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0):
     """Unquantized bf16 weights, TppBlockedLinearW<bf16,bf16> (src/csrc/fused_gemm.h:785-1073, non-quantized branch
     :951-1064 with one K chunk, the M <= 256 case of getBlockingParams :695-721): the bf16 output tile starts as the

@@ -20,6 +20,9 @@
  *   orc_remap_quantize_* / orc_dequantize_*  (layouts)
  *       -> pinned: closed-form index formulas vs. an independent view/permute
  *          restatement with stock torch, byte equality.
+ *   orc_linear_qint8_f32
+ *       -> pinned: its bf16 rounding equals orc_linear_qint8 (ideal); fp64
+ *          evaluation of the formula.
  *   orc_linear_mxfp4 / orc_linear_qint8 (mode ideal)
  *       -> pinned: reduces to torch.matmul in fp64 over the exactly
  *          dequantized weight; int32 partial sums bit-checked.
@@ -766,6 +769,38 @@ ORC_API void orc_linear_qint8(const uint16_t* x, int64_t M, int64_t K,
   }
   free(xq);
   free(sa);
+}
+
+/* The same GEMM on activations the caller has quantized (int8 [M][K] +
+ * f32 [M][K/qbs]) with everything after the integer sums in fp32:
+ * TppBlockedQInt8LinearW<float, uint8_t, float> (fused_gemm.h:1076-1341), the
+ * path of float / half / pre-quantized inputs (fused_llm_infer.cpp:1526-1545).
+ * y = bias + sum_b float(isum_b) * (sa*sw), one fused multiply-add per block in
+ * ascending order (mode ideal of orc_linear_qint8 without the final rounding).
+ * Pinned by: rounding y to bf16 reproduces orc_linear_qint8 (ideal) on bf16
+ * inputs; fp64 evaluation of the formula (tests/test_oracle.py). */
+ORC_API void orc_linear_qint8_f32(const int8_t* xq, const float* sa, int64_t M,
+                                  int64_t K, const int8_t* q, const float* sw,
+                                  int64_t N, int64_t qbs, const float* bias,
+                                  float* y) {
+  int64_t N1 = N / 16, nb = K / qbs;
+#pragma omp parallel for schedule(dynamic, 1)
+  for (int64_t n1 = 0; n1 < N1; n1++)
+    for (int k2 = 0; k2 < 16; k2++) {
+      int64_t n = n1 * 16 + k2;
+      for (int64_t m = 0; m < M; m++) {
+        float f = bias ? bias[n] : 0.0f;
+        for (int64_t b = 0; b < nb; b++) {
+          int32_t acc = 0;
+          for (int64_t a = 0; a < qbs / 4; a++)
+            for (int v = 0; v < 4; v++)
+              acc += (int32_t)xq[m * K + b * qbs + a * 4 + v] *
+                     (int32_t)q[(((n1 * nb + b) * (qbs / 4) + a) * 16 + k2) * 4 + v];
+          f = fmaf((float)acc, sa[m * nb + b] * sw[(n1 * nb + b) * 16 + k2], f);
+        }
+        y[m * N + n] = f;
+      }
+    }
 }
 
 ORC_API int orc_num_threads(void) {

@@ -150,3 +150,61 @@ def test_qint4_vnni2_weight_linear(M):
     y = ops.fc_plain(x.cuda(), qt, None)
     ref = O.linear_qint8(t2bits(x), np.ascontiguousarray(v8), s_or)
     assert_close_bf16(t2bits(y), ref, what=f"qint4 fc_plain M={M}")
+
+
+@pytest.mark.parametrize("M", [1, 5, 70])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_fc_plain_float_and_half_activations(M, dtype):
+    """fc_plain's element-type switch (fused_llm_infer.cpp:1526-1545) on a QINT8 weight: float / half activations are
+    quantized from their own values, the GEMM accumulates and adds the bias in fp32, the output has the activations'
+    type.  Bit-exact against the oracle's fp32 chain (half: its single rounding to half)."""
+    ops = _ops()
+    N, K = 96, 1024
+    W = randn_bf16((N, K), 0.02, 61)
+    qw = ops.remap_and_quantize_qint8(block_bf16(W).cuda())
+    q_or, s_or, qbs = O.remap_quantize_qint8(W.float().numpy())
+    g = torch.Generator().manual_seed(62 + M)
+    x = (torch.randn((M, K), generator=g) * 1.7).to(dtype)
+    bias = (torch.randn((N,), generator=g) * 0.1).to(dtype)
+    y = ops.fc_plain(x.cuda(), qw, bias.cuda())
+    assert y.dtype == dtype and tuple(y.shape) == (M, N)
+    xq, sa = O.quantize_int8sym(x.float().numpy(), qbs, -1, False)
+    ref = torch.from_numpy(O.linear_qint8_f32(xq, sa, q_or, s_or, bias.float().numpy())).to(dtype)
+    assert torch.equal(y.cpu(), ref)
+    # leading dimensions are kept, no bias
+    y3 = ops.fc_plain(x.cuda().view(1, M, K), qw, None)
+    ref3 = torch.from_numpy(O.linear_qint8_f32(xq, sa, q_or, s_or, None)).to(dtype)
+    assert tuple(y3.shape) == (1, M, N) and torch.equal(y3.cpu().view(M, N), ref3)
+    from tpp_pytorch_extension._lib import TppxError
+    with pytest.raises(TppxError):  # post-ops are a bfloat16 path
+        ops.fc_silu(x.cuda(), qw, None)
+    with pytest.raises(TppxError):  # MXFP4 weights take bfloat16 activations
+        ops.fc_plain(x.cuda(), ops.remap_and_quantize_mxfp4(block_bf16(W).cuda()), None)
+
+
+@pytest.mark.parametrize("M", [3, 40])
+def test_fc_plain_prequantized_input(M):
+    """A qint8 activation tensor (quantize_int8sym over the last axis with the weight's block size) is used as it is
+    (fused_gemm.h:1244-1246); the compute type is the bias's, float without one (fused_llm_infer.cpp:1529-1535)."""
+    ops = _ops()
+    N, K = 64, 768
+    W = randn_bf16((N, K), 0.02, 71)
+    qw = ops.remap_and_quantize_qint8(block_bf16(W).cuda())
+    q_or, s_or, qbs = O.remap_quantize_qint8(W.float().numpy())
+    x = randn_bf16((M, K), 1.0, 72)
+    bias = randn_bf16((N,), 0.1, 73)
+    xq = ops.quantize_int8sym(x.cuda(), qbs, -1, False)
+    # bfloat16 bias: the bf16 kernels on the caller's quantized rows = the call that quantizes by itself
+    yb = ops.fc_plain(xq, qw, bias.cuda())
+    assert yb.dtype == torch.bfloat16 and torch.equal(yb, ops.fc_plain(x.cuda(), qw, bias.cuda()))
+    # no bias: float
+    yf = ops.fc_plain(xq, qw, None)
+    xq_or, sa_or = O.quantize_int8sym(x.float().numpy(), qbs, -1, False)
+    assert yf.dtype == torch.float32
+    assert np.array_equal(yf.cpu().numpy(), O.linear_qint8_f32(xq_or, sa_or, q_or, s_or, None))
+    # float bias: float
+    yfb = ops.fc_plain(xq, qw, bias.float().cuda())
+    assert np.array_equal(yfb.cpu().numpy(), O.linear_qint8_f32(xq_or, sa_or, q_or, s_or, bias.float().numpy()))
+    from tpp_pytorch_extension._lib import TppxError
+    with pytest.raises(TppxError):  # quantized with another block size
+        ops.fc_plain(ops.quantize_int8sym(x.cuda(), 64, -1, False), qw, None)

@@ -485,3 +485,33 @@ def test_oracle_mxfp8_activation_quantizer_known_answers():
     assert codes[0, 32] == 0x7E and codes[0, 34] == 0xFE and codes[0, 35] == O.e4m3_encode([100.0])[0]
     d = O.dequant_act_mxfp8(codes, sc)
     assert d[0, 0] == 1.0 and d[0, 1] == -0.5 and d[0, 32] == 448.0 / 256
+
+
+def test_oracle_linear_qint8_f32_against_bf16_path_and_fp64():
+    """orc_linear_qint8_f32 (pre-quantized activations, everything after the integer sums in fp32):
+    * on bf16 activations and a bf16 bias, rounding its result to bf16 gives orc_linear_qint8 (mode ideal) bit for bit
+      (the same multiply-add chain, rounded once at the end);
+    * against the formula in fp64 from independently formed integer block sums (relative error of an fp32 chain);
+    * float activations quantize from their own values: the scale of a block is max|x| / 127 of the fp32 values."""
+    rng = np.random.default_rng(21)
+    M, N, K = 5, 48, 768
+    W = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    q, sw, qbs = O.remap_quantize_qint8(W)
+    x = randn_bf16((M, K), 1.0, 22)
+    bias = randn_bf16((N,), 0.1, 23)
+    xq, sa = O.quantize_int8sym(x.float().numpy(), qbs, -1, False)
+    y32 = O.linear_qint8_f32(xq, sa, q, sw, bias.float().numpy())
+    ybf = O.linear_qint8(t2bits(x), q, sw, t2bits(bias), O.POST_NONE, None, None, 1.0, O.MODE_IDEAL)
+    assert np.array_equal(t2bits(torch.from_numpy(y32).to(torch.bfloat16)), ybf)
+    # fp64 formula, weight un-blocked by hand: element [n1][b][a][k2][v] = Wq[n1*16 + k2][b*qbs + a*4 + v]
+    Wq = q.transpose(0, 3, 1, 2, 4).reshape(N, K).astype(np.int64)
+    swn = sw.reshape(N // 16, K // qbs, 16).transpose(0, 2, 1).reshape(N, K // qbs).astype(np.float64)
+    isum = np.einsum("mbk,nbk->mnb", xq.astype(np.int64).reshape(M, K // qbs, qbs), Wq.reshape(N, K // qbs, qbs))
+    ref = (isum * sa.astype(np.float64)[:, None, :] * swn[None, :, :]).sum(-1) + bias.float().numpy().astype(np.float64)
+    assert np.abs(y32 - ref).max() <= 1e-5 * np.abs(ref).max()
+    # fp32 activations that bf16 cannot hold
+    xf = (rng.standard_normal((M, K)) * 3.0).astype(np.float32)
+    xq2, sa2 = O.quantize_int8sym(xf, qbs, -1, False)
+    amax = np.abs(xf.reshape(M, K // qbs, qbs)).max(-1)
+    assert np.array_equal(sa2, (amax.astype(np.float64) / 127.0).astype(np.float32))
+    assert np.abs(xq2).max() == 127 and np.abs(xq2.astype(np.float64) * np.repeat(sa2, qbs, 1) - xf).max() <= sa2.max() * 0.5 * 1.0001

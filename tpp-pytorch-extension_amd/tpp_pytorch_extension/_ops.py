@@ -357,11 +357,13 @@ def _prep_input(input, weight):
         raise TppxError(_lib.EUNSUPPORTED, f"Unsupported qscheme / layout for a linear weight: {weight!r}")
     _lib.require_gpu(weight.qdata, "weight")
     if isinstance(input, QTensor):
-        raise TppxError(_lib.EUNSUPPORTED, "pre-quantized activations are not built; pass bfloat16")
+        raise TppxError(_lib.EUNSUPPORTED, "pre-quantized activations go through linear() / fc_plain() only")
     _lib.require_gpu(input, "input")
     if input.dtype != torch.bfloat16:
         raise TppxError(_lib.EUNSUPPORTED,
-                        f"quantized weights take bfloat16 activations (got {input.dtype})")
+                        f"this operator takes bfloat16 activations (got {input.dtype}); float / half activations and "
+                        f"pre-quantized qint8 activations are built for fc_plain / linear without a post-op on "
+                        f"QINT8-family weights")
     N, K = weight.weight_nk()
     if input.shape[-1] != K:
         raise TppxError(_lib.ESHAPE, f"input has {input.shape[-1]} features, weight expects {K}")
@@ -456,6 +458,65 @@ def _mxfp4_flags_ws(x, M, K, flags=0):
     return flags, ws
 
 
+def _linear_other_types(input, weight, bias, post, flags):
+    """The element-type switch of fc_plain_wrap (src/csrc/llm/fused_llm_infer.cpp:1526-1545) beyond bfloat16, for
+    QINT8-family weights (TppBlockedQInt8LinearW, src/csrc/fused_gemm.h:1236-1249):
+      float / half activations    quantized from their own values (quantize_int8sym over the last axis with the
+                                  weight's block size), fp32 accumulation and bias, output in the activations' type;
+      pre-quantized qint8 input   used as it is; the compute type is the bias's, float without a bias (:1529-1535).
+    A bfloat16 compute type runs the bf16 kernels on the quantized rows; float / half the fp32-output kernel."""
+    L = _lib.lib()
+    if not isinstance(weight, QTensor) or not weight.is_weight() or weight.weight_kind() == "mxfp4":
+        raise TppxError(_lib.EUNSUPPORTED, "float / half / pre-quantized activations need a QINT8, QINT4 or QINT2 weight "
+                                           "(MXFP4 and bf16 weights take bfloat16 activations)")
+    if post != POST_NONE:
+        raise TppxError(_lib.EUNSUPPORTED, "post-ops are built for bfloat16 activations only")
+    _lib.require_gpu(weight.qdata, "weight")
+    N, K = weight.weight_nk()
+    qbs = weight.block_size
+    if isinstance(input, QTensor):
+        if input._qscheme != QSCHEME_AFFINE or input.qdata.dtype != torch.int8 or input.is_weight() \
+                or input.block_size != qbs or input.axis != len(input.shape) - 1:
+            raise TppxError(_lib.EUNSUPPORTED, f"a pre-quantized input must be qint8, quantized over its last axis with "
+                                               f"the weight's block size {qbs}: {input!r}")
+        act = input
+        ctype = bias.dtype if bias is not None and bias.numel() else torch.float32
+    else:
+        _lib.require_gpu(input, "input")
+        ctype = input.dtype
+        if input.shape[-1] != K:
+            raise TppxError(_lib.ESHAPE, f"input has {input.shape[-1]} features, weight expects {K}")
+        act = quantize_int8sym(input.float().contiguous(), qbs, -1, False)
+    shape = tuple(act.shape)
+    if shape[-1] != K:
+        raise TppxError(_lib.ESHAPE, f"input has {shape[-1]} features, weight expects {K}")
+    xq, sa = act.qdata.contiguous(), act.scales.contiguous()
+    M = xq.numel() // K
+    qn, sn = weight.native()
+    st = _lib.stream_of(xq)
+    if ctype == torch.bfloat16:
+        y = torch.empty(shape[:-1] + (N,), dtype=torch.bfloat16, device=xq.device)
+        if M:
+            b = _prep_bias(bias, N, xq.device)
+            ws = _lib.workspace(xq)
+            _lib.check(L.tppx_linear_qint8(None, xq.data_ptr(), sa.data_ptr(), qn.data_ptr(), sn.data_ptr(), _lib.ptr(b),
+                                           None, None, y.data_ptr(), M, N, K, qbs, POST_NONE, 1.0, flags, ws.data_ptr(),
+                                           ws.numel(), st))
+        return y
+    if ctype not in (torch.float32, torch.float16):
+        raise TppxError(_lib.EUNSUPPORTED, f"compute type {ctype} is not built")
+    y = torch.empty(shape[:-1] + (N,), dtype=torch.float32, device=xq.device)
+    if M:
+        b = None
+        if bias is not None and bias.numel():
+            if bias.numel() != N:
+                raise TppxError(_lib.ESHAPE, f"bias has {bias.numel()} elements, the weight {N} channels")
+            b = bias.to(device=xq.device, dtype=torch.float32).contiguous()
+        _lib.check(L.tppx_linear_qint8_f32(xq.data_ptr(), sa.data_ptr(), qn.data_ptr(), sn.data_ptr(), _lib.ptr(b),
+                                           y.data_ptr(), M, N, K, qbs, st))
+    return y if ctype == torch.float32 else y.to(torch.float16)
+
+
 def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0, flags=0,
            row_sumsq=None):
     """One quantized GEMM with a fused post-op
@@ -467,6 +528,8 @@ def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None
         if row_sumsq is not None:
             raise TppxError(_lib.EUNSUPPORTED, "row sums of squares need an MXFP4 weight and at most 16 rows")
         return _linear_bf16(input, weight, bias, post, post_in, post_in2, post_scale, flags)
+    if isinstance(input, QTensor) or (isinstance(input, torch.Tensor) and input.dtype in (torch.float32, torch.float16)):
+        return _linear_other_types(input, weight, bias, post, flags)
     x, M, N, K = _prep_input(input, weight)
     out_shape = tuple(input.shape[:-1]) + (N,)
     y = torch.empty(out_shape, dtype=torch.bfloat16, device=x.device)
