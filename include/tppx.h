@@ -448,6 +448,27 @@ int tppx_linear_qint8_f32(const void* xq, const void* sa, const void* qw,
                           int64_t M, int64_t N, int64_t K, int64_t qbs,
                           tppx_stream_t stream);
 
+/* W4A8, the reference's USE_MXFP4_INT8 mode: TppBlockedLinearW<int8_t, uint8_t,
+ * Tout> (src/csrc/fused_gemm.h:965-978, 1523-1526) on the weight layout of
+ * remap_and_quantize_mxfp4 under that flag (src/csrc/qtypes.cpp:787-790,
+ * 840-861), read as the reference stores it:
+ *   q  u8 [N/8][K/bc][bc/8][8][4]   byte j of a group of 8 K values =
+ *                                   value j | value 4+j << 4 (E2M1 codes)
+ *   sc u8 [N/8][K/bc][bc/32][8]     E8M0 scale per 32 K values and channel
+ * xq i8 [M][K] + sa f32 [M][K/32]: activations quantized over blocks of 32
+ * (tppx_quantize_per_block), the scales already multiplied by 6/127
+ * (fused_gemm.h:975-977).
+ *   y = post( bf16( bias + sum_b float(sum_k xq*wi) * (sa[m][b] * 2^(e-127)) ) )
+ * wi = E2M1 value * 127/6 rounded to the nearest integer (0 11 21 32 42 64 85
+ * 127): the table is the reference JIT library's and is restated, so results
+ * match the reference within that rounding only.  bias / post_in / post_in2 /
+ * y bf16; N%16==0, bc%32==0, K%bc==0. */
+int tppx_linear_mxfp4_int8(const void* xq, const void* sa, const void* q,
+                           const void* sc, const void* bias, const void* post_in,
+                           const void* post_in2, void* y, int64_t M, int64_t N,
+                           int64_t K, int64_t bc, int post_op, float post_scale,
+                           tppx_stream_t stream);
+
 /* ---- launch plans ------------------------------------------------------- */
 
 /* No counterpart in the reference.  Writes into buf, one line per kernel, what

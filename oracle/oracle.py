@@ -430,6 +430,74 @@ def dequantize_mxfp4_plain(q, sc):
     return W
 
 
+def mxfp4_int8_layout(t):
+    """The VNNI8-interleaved weight layout of remap_and_quantize_mxfp4 under USE_MXFP4_INT8 (qtypes.cpp:787-790,
+    792-861) as ONE index map: blocked VNNI2 input [N/bk][K/bc][bc/2][bk][2] (bk, bc multiples of 8) ->
+    [N/8][K/bc][bc/8][8][8], element [nb][c1][g][n8][j] = W[nb*8 + n8][c1*bc + g*8 + (j % 2)*4 + j // 2]
+    (K values 0,4,1,5,2,6,3,7 of the group: a packed byte holds values i and 4 + i)."""
+    t = _c(t, np.float32)
+    K1, C1, C2, K2, C3 = t.shape
+    assert C3 == 2 and K2 % 8 == 0 and C2 % 4 == 0
+    N, bc = K1 * K2, C2 * 2
+    W = t.transpose(0, 3, 1, 2, 4).reshape(N, C1 * bc)          # plain [N][K]
+    g = W.reshape(N // 8, 8, C1, bc // 8, 2, 4)                 # [nb][n8][c1][g][i2][i4], k = i2*4 + i4
+    return np.ascontiguousarray(g.transpose(0, 2, 3, 1, 5, 4).reshape(N // 8, C1, bc // 8, 8, 8))  # j = i4*2 + i2
+
+
+def mxfp4_int8_layout_chain(t):
+    """The same layout by the reference's own sequence of views and permutes (qtypes.cpp:792-811 with desired_K2 = 8,
+    then :840-861), restated step by step: the pin of mxfp4_int8_layout()."""
+    t = _c(t, np.float32)
+    K1, C1, C2, K2, C3 = t.shape
+    if K2 < 8 and 8 % K2 == 0:
+        R = 8 // K2
+        t = t.reshape(K1 // R, R, C1, C2, K2, C3).transpose(0, 2, 3, 1, 4, 5).reshape(K1 // R, C1, C2, R * K2, C3)
+    elif K2 > 8 and K2 % 8 == 0:
+        R = K2 // 8
+        t = t.reshape(K1, C1, C2, R, 8, C3).transpose(0, 3, 1, 2, 4, 5).reshape(K1 * R, C1, C2, 8, C3)
+    K1, C1, C2, K2, C3 = t.shape
+    if C3 < 8:
+        R = 8 // C3
+        t = t.reshape(K1, C1, C2 // R, R, K2, C3).transpose(0, 1, 2, 4, 3, 5).reshape(K1, C1, C2 // R, K2, R * C3)
+    sh = t.shape
+    t = t.reshape(sh[:4] + (2, 4)).transpose(0, 1, 2, 3, 5, 4).reshape(sh)
+    return np.ascontiguousarray(t)
+
+
+def remap_quantize_mxfp4_int8(t):
+    """remap_and_quantize_mxfp4 with USE_MXFP4_INT8 = 1 on a blocked VNNI2 weight: the layout above, then
+    quantize_mxfp4(t, 32, 2, true) (qtypes.cpp:862).  -> (u8 [N/8][K/bc][bc/8][8][4], E8M0 u8 [N/8][K/bc][bc/32][8])."""
+    v = mxfp4_int8_layout(t)
+    return quantize_mxfp4(v, 32, 2, True)
+
+
+W4A8_ACT_SCALE = np.float32(6.0 / 127.0)
+
+
+def quantize_act_w4a8(x_f32):
+    """Activations of the W4A8 GEMM (fused_gemm.h:970-977): quantize_int8sym over blocks of 32 of the last axis, the
+    scales then multiplied in place by 6/127 (a float tensor times a scalar: fp32 product)."""
+    xq, sa = quantize_int8sym(_c(x_f32, np.float32), 32, -1, False)
+    return xq, (sa * W4A8_ACT_SCALE).astype(np.float32)
+
+
+def linear_w4a8(x_bf16, q, sc, bc, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0):
+    x = bf16_to_f32(_c(x_bf16, np.uint16))
+    xq, sa = quantize_act_w4a8(x)
+    q = _c(q, np.uint8)
+    sc = _c(sc, np.uint8)
+    M, K = xq.shape
+    N = q.shape[0] * 8
+    assert q.shape[1] * bc == K and q.shape[2] * 8 == bc
+    bias = None if bias is None else _c(bias, np.uint16)
+    post_in = None if post_in is None else _c(post_in, np.uint16)
+    post_in2 = None if post_in2 is None else _c(post_in2, np.uint16)
+    y = np.empty((M, N), np.uint16)
+    lib().orc_linear_w4a8(_p(xq), _p(sa), _c_i64(M), _c_i64(K), _p(q), _p(sc), _c_i64(N), _c_i64(bc), _p(bias),
+                          ctypes.c_int(post), _p(post_in), _p(post_in2), ctypes.c_float(post_scale), _p(y))
+    return y
+
+
 def remap_quantize_qint8(W, qbs=None, env_block=256):
     W = _c(W, np.float32)
     N, K = W.shape

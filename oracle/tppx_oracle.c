@@ -803,6 +803,61 @@ ORC_API void orc_linear_qint8_f32(const int8_t* xq, const float* sa, int64_t M,
     }
 }
 
+/* ------------------------------------------------------------------ */
+/* W4A8: MXFP4 weights in the VNNI8-interleaved layout of               */
+/* remap_and_quantize_mxfp4 under USE_MXFP4_INT8 (qtypes.cpp:787-790,    */
+/* 840-861) with int8 activations (TppBlockedLinearW<int8_t, uint8_t,    */
+/* Tout>, fused_gemm.h:965-978, 1523-1526).                              */
+/* q u8 [N/8][K/bc][bc/8][8][4]: byte j of the group (n8, 8 K values)    */
+/* holds K value j in its low and K value 4 + j in its high nibble;      */
+/* sc u8 [N/8][K/bc][bc/32][8] E8M0.  Activations: int8 over blocks of   */
+/* 32 along K with scale max/127 (quantize_int8sym), the scales then     */
+/* multiplied by float(6.0/127.0) (fused_gemm.h:975-977).  The consumer  */
+/* of that convention sits inside libxsmm (absent): it implies integer   */
+/* weights w_i = e2m1 * 127/6.  RESTATED HERE AS round-to-nearest-even   */
+/* of e2m1 * 127/6 -> {0, 11, 21, 32, 42, 64, 85, 127}: PARITY UNPINNED  */
+/* for that table and for the summation order; pinned are the layout     */
+/* (against the view/permute chain), the activation quantizer and the    */
+/* identity w_i * 6/127 ~ e2m1 within the table's rounding.              */
+/* y = post(bf16(bias + sum_b float(isum_b) * (sa'[m][b] * 2^(e-127)))). */
+/* ------------------------------------------------------------------ */
+static const int8_t w4a8_tbl[8] = {0, 11, 21, 32, 42, 64, 85, 127};
+ORC_API int orc_w4a8_weight_int(int code) {
+  int v = w4a8_tbl[code & 7];
+  return (code & 8) ? -v : v;
+}
+
+ORC_API void orc_linear_w4a8(const int8_t* xq, const float* sa, int64_t M,
+                             int64_t K, const uint8_t* q, const uint8_t* sc,
+                             int64_t N, int64_t bc, const uint16_t* bias,
+                             int post, const uint16_t* post_in,
+                             const uint16_t* post_in2, float post_scale,
+                             uint16_t* y) {
+  int64_t C1 = K / bc, nb = K / 32;
+#pragma omp parallel for schedule(dynamic, 8)
+  for (int64_t n = 0; n < N; n++) {
+    int64_t n8b = n / 8, n8 = n % 8;
+    for (int64_t m = 0; m < M; m++) {
+      float f = bias ? bf16_to_f32(bias[n]) : 0.0f;
+      for (int64_t b = 0; b < nb; b++) {
+        int64_t c1 = (b * 32) / bc, kb = (b * 32) % bc; /* K offset inside the bc block */
+        int32_t acc = 0;
+        for (int64_t k = 0; k < 32; k++) {
+          int64_t kk = kb + k, g = kk / 8, j = kk % 8;
+          uint8_t byte = q[(((n8b * C1 + c1) * (bc / 8) + g) * 8 + n8) * 4 + (j & 3)];
+          int code = j < 4 ? (byte & 15) : (byte >> 4);
+          acc += (int32_t)xq[m * K + b * 32 + k] * orc_w4a8_weight_int(code);
+        }
+        float ws = orc_mx_dequant_scale(sc[((n8b * C1 + c1) * (bc / 32) + kb / 32) * 8 + n8]);
+        f = fmaf((float)acc, sa[m * nb + b] * ws, f);
+      }
+      int64_t o = m * N + n;
+      y[o] = apply_post(f32_to_bf16(f), post, post_in ? post_in[o] : 0,
+                        post_in2 ? post_in2[o] : 0, post_scale);
+    }
+  }
+}
+
 ORC_API int orc_num_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();

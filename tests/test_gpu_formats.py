@@ -208,3 +208,55 @@ def test_fc_plain_prequantized_input(M):
     from tpp_pytorch_extension._lib import TppxError
     with pytest.raises(TppxError):  # quantized with another block size
         ops.fc_plain(ops.quantize_int8sym(x.cuda(), 64, -1, False), qw, None)
+
+
+@pytest.mark.parametrize("bk,bc", [(16, 64), (32, 64), (64, 128)])
+def test_w4a8_layout_and_quantizer(bk, bc):
+    """remap_and_quantize_mxfp4(t, int8_layout=True) = the reference's USE_MXFP4_INT8 branch: packed bytes and E8M0
+    scales equal the oracle's (whose layout is pinned against the reference's view / permute chain)."""
+    ops = _ops()
+    N, K = 128, 256
+    W = randn_bf16((N, K), 0.05, 81)
+    t = W.view(N // bk, bk, K // bc, bc // 2, 2).permute(0, 2, 3, 1, 4).contiguous()
+    qt = ops.remap_and_quantize_mxfp4(t.cuda(), int8_layout=True)
+    q_or, s_or = O.remap_quantize_mxfp4_int8(t.float().numpy())
+    assert tuple(qt.shape) == (N // 8, K // bc, bc // 8, 8, 8) and qt.weight_kind() == "mxfp4_int8"
+    assert qt.weight_nk() == (N, K)
+    assert np.array_equal(qt.qdata.cpu().numpy().reshape(q_or.shape), q_or)
+    assert np.array_equal(qt.scales.cpu().numpy().reshape(s_or.shape), s_or)
+    # dequantize() gives the fp32 values in the blocked shape (the generic per-block path)
+    d = qt.dequantize().cpu().numpy()
+    v = O.mxfp4_int8_layout(t.float().numpy())
+    assert d.shape == v.shape and np.abs(d - v).max() <= 0.25 * np.abs(v).max()
+
+
+@pytest.mark.parametrize("M", [1, 16, 70])
+@pytest.mark.parametrize("post", ["none", "silu", "add"])
+def test_w4a8_linear(M, post):
+    """The W4A8 GEMM (int8 activations over blocks of 32, scales times 6/127, MXFP4 weights as integers, K = 32
+    int8 MFMA) against the oracle's restatement: same integer sums, same fp32 chain -> bf16 equality up to the
+    post-op's tolerance."""
+    ops = _ops()
+    N, K, bk, bc = 96, 512, 16, 64
+    W = randn_bf16((N, K), 0.05, 82)
+    t = W.view(N // bk, bk, K // bc, bc // 2, 2).permute(0, 2, 3, 1, 4).contiguous()
+    qt = ops.remap_and_quantize_mxfp4(t.cuda(), int8_layout=True)
+    q_or, s_or = O.remap_quantize_mxfp4_int8(t.float().numpy())
+    x = randn_bf16((M, K), 1.0, 83 + M)
+    bias = randn_bf16((N,), 0.1, 84)
+    in1 = randn_bf16((M, N), 1.0, 85)
+    POSTS = {"none": O.POST_NONE, "silu": O.POST_SILU, "add": O.POST_ADD_SCALE}
+    y = ops.linear(x.cuda(), qt, bias.cuda(), POSTS[post], in1.cuda() if post == "add" else None, None, 0.5)
+    ref = O.linear_w4a8(t2bits(x), q_or, s_or, bc, t2bits(bias), POSTS[post], t2bits(in1) if post == "add" else None,
+                        None, 0.5)
+    assert_close_bf16(t2bits(y), ref, ulps=2 if post == "silu" else 1, what=f"w4a8 M={M} post={post}")
+    if post == "none":
+        # and close to the exact MXFP4 GEMM on bf16 activations (two quantization errors apart)
+        exact = ops.linear(x.cuda(), ops.remap_and_quantize_mxfp4(block_bf16(W).cuda(), int8_layout=False), bias.cuda())
+        a, b = y.double(), exact.double()
+        assert float((a - b).norm() / b.norm()) <= 3e-2
+        # the group operators fall back to one GEMM per weight
+        q1, q2 = ops.qkv_gemm(x.cuda(), [qt, qt], [bias.cuda(), None])
+        assert torch.equal(q1, y) and torch.equal(q2, ops.linear(x.cuda(), qt, None))
+        sw = ops.swiglu_gate_up(x.cuda(), qt, qt)
+        assert torch.equal(sw, ops.fc_mul(x.cuda(), qt, None, ops.fc_silu(x.cuda(), qt, None)))

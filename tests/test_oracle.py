@@ -515,3 +515,55 @@ def test_oracle_linear_qint8_f32_against_bf16_path_and_fp64():
     amax = np.abs(xf.reshape(M, K // qbs, qbs)).max(-1)
     assert np.array_equal(sa2, (amax.astype(np.float64) / 127.0).astype(np.float32))
     assert np.abs(xq2).max() == 127 and np.abs(xq2.astype(np.float64) * np.repeat(sa2, qbs, 1) - xf).max() <= sa2.max() * 0.5 * 1.0001
+
+
+def test_oracle_w4a8_layout_table_and_linear():
+    """The W4A8 restatement (USE_MXFP4_INT8):
+    * layout: the one-step index map equals the reference's sequence of views and permutes, for source channel
+      blocks below, at and above 8, and each element sits where the documented formula says;
+    * packed bytes: byte j of a group holds K value j in its low and K value 4 + j in its high nibble, and the
+      codes / scales are those of the default-layout MXFP4 quantizer on the same weight (same 32-value blocks);
+    * integer table: |w_i * 6/127 - e2m1| <= 0.5 * 6/127 for all 16 codes, sign symmetric, exact at 0 and 6;
+    * linear: equals an fp64 evaluation of its formula within fp32 chain error, and the exact-MXFP4 product on the
+      dequantized activations within the table's rounding (0.5/127 of full scale per weight)."""
+    rng = np.random.default_rng(31)
+    for N, K, bk, bc in [(32, 128, 16, 64), (64, 256, 32, 64), (16, 64, 8, 32), (64, 128, 64, 128), (32, 64, 4, 64)]:
+        W = rng.standard_normal((N, K)).astype(np.float32)
+        t = W.reshape(N // bk, bk, K // bc, bc // 2, 2).transpose(0, 2, 3, 1, 4).copy()
+        if bk >= 8:
+            a = O.mxfp4_int8_layout(t)
+            assert np.array_equal(a, O.mxfp4_int8_layout_chain(t))
+        else:
+            a = O.mxfp4_int8_layout_chain(t)
+        nb, c1, g, n8, j = N // 8 - 1, K // bc - 1, bc // 8 - 1, 5, 3
+        assert a[nb, c1, g, n8, j] == W[nb * 8 + n8, c1 * bc + g * 8 + (j % 2) * 4 + j // 2]
+    N, K, bk, bc = 64, 256, 16, 64
+    W = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+    t = W.reshape(N // bk, bk, K // bc, bc // 2, 2).transpose(0, 2, 3, 1, 4).copy()
+    q, sc = O.remap_quantize_mxfp4_int8(t)
+    assert q.shape == (N // 8, K // bc, bc // 8, 8, 4) and sc.shape == (N // 8, K // bc, bc // 32, 8)
+    q0, sc0 = O.remap_quantize_mxfp4(W)            # default layout [N/32][K/64][32][32] + [N/32][K/64][2][32]
+    Wd = O.dequantize_mxfp4_plain(q0, sc0)
+    codes = np.stack([q & 15, q >> 4], axis=-1)    # [..][n8][j][lo/hi] -> K value j + 4*hi
+    e2m1 = np.array([O.lib().orc_e2m1_decode(c) for c in range(16)], np.float32)
+    vals = e2m1[codes].transpose(0, 3, 1, 2, 5, 4).reshape(N, K // bc, bc // 8, 8)  # [n][c1][g][k = hi*4 + j]
+    scale = np.array([O.lib().orc_mx_dequant_scale(int(b)) for b in range(256)], np.float32)[sc]  # [nb][c1][sb][n8]
+    scale = np.repeat(scale.transpose(0, 3, 1, 2).reshape(N, K // 32), 32, axis=1)
+    assert np.array_equal(vals.reshape(N, K) * scale, Wd)
+    tbl = np.array([O.lib().orc_w4a8_weight_int(c) for c in range(16)], np.float64)
+    assert np.abs(tbl * 6.0 / 127.0 - e2m1.astype(np.float64)).max() <= 0.5 * 6.0 / 127.0 + 1e-12
+    assert np.array_equal(tbl[8:], -tbl[:8]) and tbl[0] == 0 and tbl[7] == 127
+    # linear
+    M = 7
+    x = randn_bf16((M, K), 1.0, 32)
+    bias = randn_bf16((N,), 0.1, 33)
+    y = bits2f(O.linear_w4a8(t2bits(x), q, sc, bc, t2bits(bias))).astype(np.float64)
+    xq, sa = O.quantize_act_w4a8(x.float().numpy())
+    wi = tbl[np.stack([q & 15, q >> 4], axis=-1)].transpose(0, 3, 1, 2, 5, 4).reshape(N, K)
+    isum = np.einsum("mbk,nbk->mnb", xq.astype(np.float64).reshape(M, K // 32, 32), wi.reshape(N, K // 32, 32))
+    wsc = scale[:, ::32].astype(np.float64)
+    ref = (isum * sa.astype(np.float64)[:, None, :] * wsc[None, :, :]).sum(-1) + bias.float().numpy().astype(np.float64)
+    assert np.abs(y - ref).max() <= 2.0 ** -8 * np.abs(ref).max()
+    exact = (xq.astype(np.float64) * np.repeat(sa / O.W4A8_ACT_SCALE, 32, axis=1)) @ Wd.astype(np.float64).T \
+        + bias.float().numpy().astype(np.float64)
+    assert np.sqrt(((ref - exact) ** 2).sum() / (exact ** 2).sum()) <= 1.5e-2

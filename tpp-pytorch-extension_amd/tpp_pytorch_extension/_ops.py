@@ -53,9 +53,38 @@ def _float_weight_on_gpu(t):
     return t.contiguous(), dt
 
 
-def remap_and_quantize_mxfp4(t):
+# USE_MXFP4_INT8 (qtypes.cpp:31): remap_and_quantize_mxfp4 produces the VNNI8-interleaved layout whose GEMM runs on
+# int8 activations (W4A8)
+USE_MXFP4_INT8 = os.environ.get("USE_MXFP4_INT8", "0") not in ("0", "")
+
+
+def _remap_mxfp4_int8(t):
+    """The USE_MXFP4_INT8 branch of remap_and_quantize_mxfp4 (qtypes.cpp:787-790, 792-861): N blocks of 8 channels,
+    K in groups of 8 ordered 0,4,1,5,2,6,3,7 (a packed byte holds values i and 4 + i), then quantize_mxfp4(t, 32,
+    2, true) -> quint4x2 [N/8, K/bc, bc/8, 8, 8] with E8M0 scales [N/8, K/bc, bc/32, 8]."""
+    t, _ = _float_weight_on_gpu(t)
+    N, K, bk, bc, vnni = _blocked_geometry(t)
+    if t.dim() == 4 and bc % 8:
+        raise TppxError(_lib.ESHAPE, "Shape not compatible for VNNI2")
+    if (bk < 8 and (8 % bk or (N // bk) % (8 // bk))) or (bk > 8 and bk % 8):
+        raise TppxError(_lib.ESHAPE, "Shape not compatible for MXFP4")
+    if bc % 32 or N % 16:
+        raise TppxError(_lib.ESHAPE, "Shape not compatible for VNNI8")
+    C1 = K // bc
+    if t.dim() == 5:
+        W = t.permute(0, 3, 1, 2, 4).reshape(N, K)   # [N/bk][K/bc][bc/vnni][bk][vnni] -> plain rows
+    else:
+        W = t.permute(0, 3, 1, 2).reshape(N, K)      # [N/bk][K/bc][bc][bk]
+    g = W.reshape(N // 8, 8, C1, bc // 8, 2, 4).permute(0, 2, 3, 1, 5, 4).reshape(N // 8, C1, bc // 8, 8, 8).contiguous()
+    return _quantize_generic(g, 32, 2, True, _lib.Q_MXFP4)
+
+
+def remap_and_quantize_mxfp4(t, int8_layout=None):
     """Reference: remap_and_quantize_mxfp4 (src/csrc/qtypes.cpp:783-864).
-    Blocked bf16 5-D / fp32 4-D weight -> quint4x2 tensor [N/32, K/64, 32, 32, 2]."""
+    Blocked bf16 5-D / fp32 4-D weight -> quint4x2 tensor [N/32, K/64, 32, 32, 2]; with int8_layout (default: the
+    USE_MXFP4_INT8 environment flag) the W4A8 layout [N/8, K/bc, bc/8, 8, 8]."""
+    if USE_MXFP4_INT8 if int8_layout is None else int8_layout:
+        return _remap_mxfp4_int8(t)
     L = _lib.lib()
     t, dt = _float_weight_on_gpu(t)
     N, K, bk, bc, vnni = _blocked_geometry(t)
@@ -466,7 +495,7 @@ def _linear_other_types(input, weight, bias, post, flags):
       pre-quantized qint8 input   used as it is; the compute type is the bias's, float without a bias (:1529-1535).
     A bfloat16 compute type runs the bf16 kernels on the quantized rows; float / half the fp32-output kernel."""
     L = _lib.lib()
-    if not isinstance(weight, QTensor) or not weight.is_weight() or weight.weight_kind() == "mxfp4":
+    if not isinstance(weight, QTensor) or not weight.is_weight() or weight.weight_kind() in ("mxfp4", "mxfp4_int8"):
         raise TppxError(_lib.EUNSUPPORTED, "float / half / pre-quantized activations need a QINT8, QINT4 or QINT2 weight "
                                            "(MXFP4 and bf16 weights take bfloat16 activations)")
     if post != POST_NONE:
@@ -517,6 +546,40 @@ def _linear_other_types(input, weight, bias, post, flags):
     return y if ctype == torch.float32 else y.to(torch.float16)
 
 
+W4A8_ACT_SCALE = 6.0 / 127.0
+
+
+def _linear_w4a8(input, weight, bias, post, post_in, post_in2, post_scale):
+    """TppBlockedLinearW<int8_t, uint8_t, Tout> (src/csrc/fused_gemm.h:965-978, 1523-1526): bf16 activations are
+    quantized to int8 over blocks of 32 (quantize_int8sym with the weight's block size), the scales multiplied by
+    6/127, and the GEMM runs on int8 against the MXFP4 weight in its VNNI8 layout."""
+    L = _lib.lib()
+    _lib.require_gpu(input, "input")
+    if input.dtype != torch.bfloat16:
+        raise TppxError(_lib.EUNSUPPORTED, f"the W4A8 path takes bfloat16 activations (got {input.dtype})")
+    N, K = weight.weight_nk()
+    if input.shape[-1] != K:
+        raise TppxError(_lib.ESHAPE, f"input has {input.shape[-1]} features, weight expects {K}")
+    x = input.contiguous()
+    M = x.numel() // K
+    y = torch.empty(tuple(input.shape[:-1]) + (N,), dtype=torch.bfloat16, device=x.device)
+    if M == 0:
+        return y
+    act = quantize_int8sym(x.view(M, K), 32, -1, False)
+    sa = act.scales.mul_(W4A8_ACT_SCALE)
+    bias = _prep_bias(bias, N, x.device)
+    post_in = _prep_post(post_in, M, N, "post-op input", x.device)
+    post_in2 = _prep_post(post_in2, M, N, "second post-op input", x.device)
+    _lib.check(L.tppx_linear_mxfp4_int8(act.qdata.data_ptr(), sa.data_ptr(), weight.qdata.data_ptr(),
+                                        weight.scales.data_ptr(), _lib.ptr(bias), _lib.ptr(post_in), _lib.ptr(post_in2),
+                                        y.data_ptr(), M, N, K, weight.shape[2] * 8, post, post_scale, _lib.stream_of(x)))
+    return y
+
+
+def _is_w4a8(w):
+    return isinstance(w, QTensor) and w.weight_kind() == "mxfp4_int8"
+
+
 def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0, flags=0,
            row_sumsq=None):
     """One quantized GEMM with a fused post-op
@@ -528,6 +591,10 @@ def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None
         if row_sumsq is not None:
             raise TppxError(_lib.EUNSUPPORTED, "row sums of squares need an MXFP4 weight and at most 16 rows")
         return _linear_bf16(input, weight, bias, post, post_in, post_in2, post_scale, flags)
+    if _is_w4a8(weight):
+        if row_sumsq is not None:
+            raise TppxError(_lib.EUNSUPPORTED, "row sums of squares need an MXFP4 weight in the default layout")
+        return _linear_w4a8(input, weight, bias, post, post_in, post_in2, post_scale)
     if isinstance(input, QTensor) or (isinstance(input, torch.Tensor) and input.dtype in (torch.float32, torch.float16)):
         return _linear_other_types(input, weight, bias, post, flags)
     x, M, N, K = _prep_input(input, weight)
@@ -637,7 +704,8 @@ def takes_row_sums(weight, M):
     """Can the GEMM with this weight leave row sums of squares of its output (MXFP4 decode kernels, <= 16 rows,
     at most 256 workgroups of up to three channel tiles: 12288 output channels)?"""
     w = _as_q(weight)
-    return NORM_FROM_SUMS and w._qscheme == QSCHEME_MXFP and 0 < M <= 16 and w.weight_nk()[0] <= 12288
+    return (NORM_FROM_SUMS and w._qscheme == QSCHEME_MXFP and w.weight_kind() == "mxfp4" and 0 < M <= 16
+            and w.weight_nk()[0] <= 12288)
 
 
 def _norm_fits(norm, scheme, M, K):
@@ -667,6 +735,14 @@ def qkv_gemm(input, weights, biases, norm=None):
     norm = (gamma, eps): llama_rms_norm is applied to the input first (inside
     the same launch for MXFP4 decode steps, as a separate launch otherwise)."""
     L = _lib.lib()
+    weights = list(weights)
+    if any(_is_w4a8(w) for w in weights):  # no fused launch for the W4A8 layout: one GEMM per weight
+        if norm is not None:
+            input = rms_norm(input, norm[0], norm[1])
+        biases = list(biases) if biases is not None else []
+        biases += [None] * (len(weights) - len(biases))
+        return [linear(input, w, b, POST_GELU if (len(weights) == 4 and i == 3) else POST_NONE)
+                for i, (w, b) in enumerate(zip(weights, biases))]
     if norm is not None:
         xin, Min, _, Kin = _prep_input(input, list(weights)[0])
         if not _norm_fusable(norm, list(weights)[0]._qscheme, Min, Kin):
@@ -725,6 +801,10 @@ def swiglu_gate_up(input, w_gate, w_up, b_gate=None, b_up=None, norm=None):
     points (fused_llm_infer.cpp:1271-1272).  norm = (gamma, eps): llama_rms_norm
     on the input first (fused_llm_infer.cpp:1269), inside the launch when possible."""
     L = _lib.lib()
+    if _is_w4a8(w_gate) or _is_w4a8(w_up):
+        if norm is not None:
+            input = rms_norm(input, norm[0], norm[1])
+        return fc_mul(input, w_up, b_up, fc_silu(input, w_gate, b_gate))
     if norm is not None:
         _, M0, _, K0 = _prep_input(input, w_gate)
         if not _norm_fusable(norm, w_gate._qscheme, M0, K0):

@@ -76,14 +76,19 @@ class QTensor(torch.Tensor):
 
     # -- weight geometry -----------------------------------------------------
     def weight_kind(self):
-        """Which linear-layer weight layout this is: "mxfp4" [N/32, K/64, 32, 32, 2], "qint8" [N/16, K/QBS, QBS/4, 16,
-        4], "qint4" (VNNI2) [N/16, K/QBS, QBS/2, 16, 2], "qint2" (interleaved ternary) [N/32, K/QBS, QBS/4, 32, 4];
-        None for any other layout (helper-only tensors, quantized activations)."""
+        """Which linear-layer weight layout this is: "mxfp4" [N/32, K/64, 32, 32, 2], "mxfp4_int8" (the VNNI8-interleaved
+        W4A8 layout) [N/8, K/bc, bc/8, 8, 8], "qint8" [N/16, K/QBS, QBS/4, 16, 4], "qint4" (VNNI2) [N/16, K/QBS, QBS/2,
+        16, 2], "qint2" (interleaved ternary) [N/32, K/QBS, QBS/4, 32, 4]; None for any other layout (helper-only
+        tensors, quantized activations)."""
         s = tuple(self.shape)
         if len(s) != 5 or not self.is_vnni or self.axis != 2:
             return None
         if self._qscheme == QSCHEME_MXFP:
-            return "mxfp4" if s[2:] == (32, 32, 2) and self.block_size == 32 else None
+            if s[2:] == (32, 32, 2) and self.block_size == 32:
+                return "mxfp4"
+            if s[3:] == (8, 8) and self.block_size == 32 and s[2] % 4 == 0 and (s[0] * 8) % 16 == 0:
+                return "mxfp4_int8"
+            return None
         if self.dtype == torch.qint8 and s[3:] == (16, 4) and s[2] * 4 == self.block_size:
             return "qint8"
         if self.dtype == torch.quint4x2 and s[3:] == (16, 2) and s[2] * 2 == self.block_size and self.block_size % 64 == 0:
@@ -101,6 +106,8 @@ class QTensor(torch.Tensor):
         kind = self.weight_kind()
         if kind == "mxfp4":
             return s[0] * 32, s[1] * 64
+        if kind == "mxfp4_int8":
+            return s[0] * 8, s[1] * s[2] * 8
         if kind == "qint2":
             return s[0] * 32, s[1] * self.block_size
         return s[0] * 16, s[1] * self.block_size
@@ -120,6 +127,8 @@ class QTensor(torch.Tensor):
                 sn = torch.empty_like(self.scales)
                 _lib.check(L.tppx_prepack_mxfp4(self.qdata.data_ptr(), self.scales.data_ptr(), N, K,
                                                 qn.data_ptr(), sn.data_ptr(), st))
+            elif kind == "mxfp4_int8":
+                qn, sn = self.qdata, self.scales  # the W4A8 kernel reads the reference layout as it is
             elif kind == "qint8":
                 qn = torch.empty_like(self.qdata)
                 sn = self.scales
