@@ -77,29 +77,45 @@ struct SkEpilogue {
   uint32_t in1[MAXE], in2[MAXE];
   uint32_t bias[MAXE], bias2[MAXE]; // bf16 bits, converted at use: a conversion here would wait for the load at once
 
+  bool has_bias, has_bias2, has_in1, has_in2; // uniform: which of the arrays below hold real inputs
+
+  // Requests the post-op inputs of this thread's outputs.  No branch around any load: an absent input is read from the
+  // output tensor instead (valid memory of the same extent; the value is dropped in settle()).  A load inside a
+  // conditional makes the compiler wait for every outstanding load at the join, which here stood between the
+  // activations and the first weight request of the kernel.
   __device__ __forceinline__ void prefetch(const DecodeParams& p, const DecodeSeg& sg, int ltile0, int m0) {
+    has_bias = sg.bias != nullptr;
+    has_bias2 = DUAL && p.seg[1].bias != nullptr;
+    has_in1 = sg.post_in != nullptr;
+    has_in2 = sg.post_in2 != nullptr;
+    const uint16_t* pb = has_bias ? sg.bias : sg.y;
+    const uint16_t* pb2 = has_bias2 ? p.seg[1].bias : sg.y;
+    const uint16_t* pi1 = has_in1 ? sg.post_in : sg.y;
+    const uint16_t* pi2 = has_in2 ? sg.post_in2 : sg.y;
 #pragma unroll
     for (int i = 0; i < MAXE; i++) {
       const int e = threadIdx.x + i * blockDim.x;
-      in1[i] = in2[i] = 0;
-      bias[i] = bias2[i] = 0;
-      off[i] = -1;
-      if (e < OUT) {
-        const int l = e & 63, r = (e >> 6) & 3, mg = (e >> 8) % MG, a = (e >> 8) / MG;
-        const int m = m0 + mg * 16 + (l >> 4) * 4 + r;
-        const int n = (ltile0 + a) * 16 + (l & 15);
-        if (m < p.M && (ltile0 + a) < sg.tiles) {
-          off[i] = m * sg.N + n;
-          if (sg.bias)
-            bias[i] = sg.bias[n];
-          if (DUAL && p.seg[1].bias)
-            bias2[i] = p.seg[1].bias[n];
-          if (sg.post_in)
-            in1[i] = sg.post_in[off[i]];
-          if (sg.post_in2)
-            in2[i] = sg.post_in2[off[i]];
-        }
-      }
+      const int l = e & 63, r = (e >> 6) & 3, mg = (e >> 8) % MG, a = (e >> 8) / MG;
+      const int m = m0 + mg * 16 + (l >> 4) * 4 + r;
+      const int n = (ltile0 + a) * 16 + (l & 15);
+      const bool valid = e < OUT && m < p.M && (ltile0 + a) < sg.tiles;
+      const int o = valid ? m * sg.N + n : 0, nn = valid ? n : 0;
+      off[i] = valid ? o : -1;
+      bias[i] = pb[nn];
+      bias2[i] = DUAL ? pb2[nn] : 0;
+      in1[i] = DUAL ? 0 : pi1[o];
+      in2[i] = DUAL ? 0 : pi2[o];
+    }
+  }
+
+  // first thing after the main loop: drop what was read in place of an absent input
+  __device__ __forceinline__ void settle() {
+#pragma unroll
+    for (int i = 0; i < MAXE; i++) {
+      bias[i] = has_bias ? bias[i] : 0;
+      bias2[i] = has_bias2 ? bias2[i] : 0;
+      in1[i] = has_in1 ? in1[i] : 0;
+      in2[i] = has_in2 ? in2[i] : 0;
     }
   }
 
@@ -107,6 +123,7 @@ struct SkEpilogue {
   // (same sums in the same order as finish()).  stride >= ELEMS / 2.
   __device__ __forceinline__ void finish_halves(const DecodeSeg& sg, f32x4 (&acc)[NACC][MG], float* red, int stride = ELEMS / 2) {
     static_assert(DUAL, "two reduction rounds are for the gate/up pair");
+    settle();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int W = blockDim.x >> 6;
     float* mine = red + wave * stride;
@@ -147,6 +164,7 @@ struct SkEpilogue {
                                                float* red, int ltile0, int stride = ELEMS) {
     static_assert(!DUAL, "the gate/up pair is not split");
     __shared__ int arrived_last;
+    settle();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int W = blockDim.x >> 6;
     float* mine = red + wave * stride;
@@ -215,6 +233,7 @@ struct SkEpilogue {
   __device__ __forceinline__ void finish(const DecodeSeg& sg, f32x4 (&acc)[NACC][MG], float* red, int stride = ELEMS,
                                          float* sumsq = nullptr, int M = 0) {
     __shared__ float sq_s[16 * NACC];
+    settle();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int W = blockDim.x >> 6;
     float* mine = red + wave * stride;
@@ -331,17 +350,17 @@ skinny_qint8_kernel(const DecodeParams p) {
   const int mtp = p.mt * 16;
   constexpr int SAB = 2 * MG; // loads per batch: 8 K blocks of this wave
   auto load_sa = [&](int i) {
-    i = min(i, nsa - 1);
+    i = max(min(i, nsa - 1), 0);
     const int ul = i / MPAD, mr = i - ul * MPAD;
     // XOP: scales transposed by the quantisation kernel, [K/qbs][mt*16]
     return XOP ? p.sa[(int64_t)(u0 + ul) * mtp + m0 + mr] : p.sa[(int64_t)min(m0 + mr, p.M - 1) * NB + u0 + ul];
   };
+  // (no branch around these first requests or the ring's: behind a conditional load the compiler can no longer count
+  // the loads in flight and waits for all of them; a wave without K blocks re-reads valid data it never uses)
   float sa0[SAB];
-  if (t0 < t1) {
 #pragma unroll
-    for (int j = 0; j < SAB; j++)
-      sa0[j] = load_sa(j * 64 + lane);
-  }
+  for (int j = 0; j < SAB; j++)
+    sa0[j] = load_sa(j * 64 + lane);
 
   // Ring of PF stages; a stage = the weight tiles, their block scale and the
   // activation operand of one k-tile.  The main loop has NO branch and NO load
@@ -351,7 +370,7 @@ skinny_qint8_kernel(const DecodeParams p) {
   i32x4 wreg[PF][NTW], xreg[PF][MG];
   float sreg[PF][NTW];
   auto load_stage = [&](int st, int t, bool fast) {
-    t = min(t, t1 - 1); // past the end: re-read the last tile (never consumed)
+    t = max(min(t, t1 - 1), 0); // past the end: re-read the last tile (never consumed)
     const int b = fast ? (t >> 2) : t / TPB;
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
@@ -362,10 +381,10 @@ skinny_qint8_kernel(const DecodeParams p) {
     for (int mg = 0; mg < MG; mg++)
       xreg[st][mg] = XOP ? xop[(int64_t)t * xstride + mg * 64] : *reinterpret_cast<const i32x4*>(xrow[mg] + t * 64);
   };
-  if (t0 < t1) {
 #pragma unroll
-    for (int i = 0; i < PF; i++)
-      load_stage(i, t0 + i, false);
+  for (int i = 0; i < PF; i++)
+    load_stage(i, t0 + i, false);
+  if (t0 < t1) {
     // the scales were requested first, so they are here long before the ring
 #pragma unroll
     for (int j = 0; j < SAB; j++)
@@ -544,18 +563,18 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
   i32x4 wreg[PF][NTW];
   float sreg[PF][NTW];
   auto load_stage = [&](int st, int t) {
-    t = min(t, t1 - 1);
+    t = max(min(t, t1 - 1), 0); // past the end (or a wave without K blocks): re-read a valid tile, never consumed
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
       wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64);
       sreg[st][nt] = ws[nt][(t >> 2) * 16];
     }
   };
-  if (t0 < t1) {
+  // No branch around the ring's first requests: with one, the compiler can no longer count the loads behind the
+  // activations and waits for the whole ring before it lets the quantisation start.
 #pragma unroll
-    for (int i = 0; i < PF; i++)
-      load_stage(i, t0 + i);
-  }
+  for (int i = 0; i < PF; i++)
+    load_stage(i, t0 + i);
 
   // wave-private LDS: xq [tile][g][M rows][16 B], then sa [unit][16]; the region of the cross-wave reduction
   // comes first unless both do not fit side by side (they overlap then, with a barrier in between)
