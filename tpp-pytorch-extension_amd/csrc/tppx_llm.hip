@@ -413,10 +413,8 @@ attn_decode_kernel(const AttnParams p) {
   patch_new(blockIdx.y * 64 + wave * (4 * NU), kw, vw);
   for (int t = blockIdx.y; t < trips; t += p.splits) {
     const int base = t * 64 + wave * (4 * NU);
-    if (t + p.splits < trips) {
-      load_kv(base + p.splits * 64, kn, vn);
-      patch_new(base + p.splits * 64, kn, vn);
-    }
+    load_kv(base + p.splits * 64, kn, vn); // unconditional (rows are clamped): a branch here would drain the queue
+    patch_new(base + p.splits * 64, kn, vn);
     int key[NU];
 #pragma unroll
     for (int u = 0; u < NU; u++)
