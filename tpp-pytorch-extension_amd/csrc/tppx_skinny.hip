@@ -758,9 +758,10 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
 
   // ---- activations of this wave's K slice -> LDS ----
   // Loads return in issue order, so the (L2-resident) activation and gamma loads go out BEFORE the weight ring and
-  // are not held up by HBM latency.  They are issued and waited for by hand ("at most the ring outstanding"): the
-  // compiler's own count is conservative across the branches around here and would wait for the ring as well, which
-  // would put everything up to the main loop behind the first HBM round trip instead of inside it.
+  // are not held up by HBM latency.  The compiler waits for exactly these ("at most the ring outstanding") as long
+  // as every load between here and their first use is unconditional: a load under a branch makes its count
+  // conservative, and it would wait for the ring as well, which would put everything up to the main loop behind the
+  // first HBM round trip instead of inside it.
   const int nch = (t1 - t0) * 16;          // 16-byte chunks per row in the slice
   const int items = p.M * nch;             // (row, chunk), chunk fastest: 16 consecutive lanes = one K tile of one row
   const int nsh = nch > 16 ? 5 : 4;        // the host admits slices of 0, 16 or 32 chunks only
@@ -775,16 +776,14 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
     const int i = min(it * 64 + lane, max(items - 1, 0));
     const int row = i >> nsh, ck = i & cmask;
     const char* src = xb + (size_t)((uint32_t)(row * p.K) * 2u + xk0 + (uint32_t)ck * 16u);
-    i32x4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(src) : "memory");
-    raw[it] = v;
+    raw[it] = *reinterpret_cast<const i32x4*>(src);
   });
   // the chunk of a lane is the same in every item when the slice is 16 or 32 chunks wide
   f32x4 gm0 = f32x4{1.f, 1.f, 1.f, 1.f}, gm1 = gm0;
   if (XMODE != 0) {
     const float* gp = p.norm_gamma + (size_t)min(t0, KT - 1) * 128 + (size_t)(lane & cmask) * 8;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(gm0) : "v"(gp) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(gm1) : "v"(gp + 4) : "memory");
+    gm0 = *reinterpret_cast<const f32x4*>(gp);
+    gm1 = *reinterpret_cast<const f32x4*>(gp + 4);
   }
   // XMODE 2: the 256 sums of squares per row left by the launch that wrote x, 4 per lane.  Up to 4 rows (XNI == 2):
   // every wave adds up all rows itself, no exchange; more rows: wave w adds up row w and the waves exchange the
@@ -795,9 +794,7 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
     static_for<0, NPQ>([&](auto R) {
       constexpr int r = decltype(R)::value;
       const float* sp = p.sumsq_in + (size_t)min(NPQ == 1 ? wave : r, p.M - 1) * 256 + (size_t)lane * 4;
-      f32x4 v;
-      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(sp) : "memory");
-      pq[r] = v;
+      pq[r] = *reinterpret_cast<const f32x4*>(sp);
     });
   }
 
@@ -805,7 +802,7 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
   i32x4 wreg[PF][NTW];
   uint32_t sreg[PF][NTW];
   auto load_stage = [&](int st, int t) {
-    t = min(t, t1 - 1);
+    t = max(min(t, t1 - 1), 0); // past the end (or a wave without K tiles): re-read a valid tile, never consumed
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
       const uint32_t slot = woff[nt % NT] + (uint32_t)t * 64u;
@@ -813,31 +810,12 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
       sreg[st][nt] = *reinterpret_cast<const uint8_t*>(swb[nt / NT] + (size_t)slot);
     }
   };
-  if (t0 < t1) {
+  // No branch around the ring's first requests and ordinary loads above: the compiler counts the ring loads behind
+  // the activations itself and waits for exactly the activations (a load under a condition, or one it cannot see,
+  // makes it wait for everything or not at all).
 #pragma unroll
-    for (int i = 0; i < PF; i++)
-      load_stage(i, t0 + i);
-  }
-  // a full ring is PF stages of distinct tiles: 2 * NTW loads each.  Shorter slices (the stages would repeat a tile
-  // and the compiler may merge the repeats) simply wait for everything.
-  if (t1 - t0 >= PF)
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PF * NTW * 2) : "memory");
-  else
-    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
-  // every use of the hand-loaded registers stays behind the wait
-  static_for<0, XNI>([&](auto IT) {
-    i32x4 v = raw[decltype(IT)::value];
-    asm volatile("" : "+v"(v));
-    raw[decltype(IT)::value] = v;
-  });
-  asm volatile("" : "+v"(gm0), "+v"(gm1));
-  if (XMODE == 2) {
-    static_for<0, NPQ>([&](auto R) {
-      f32x4 v = pq[decltype(R)::value];
-      asm volatile("" : "+v"(v));
-      pq[decltype(R)::value] = v;
-    });
-  }
+  for (int i = 0; i < PF; i++)
+    load_stage(i, t0 + i);
 
   // the slot arithmetic below starts from an opaque copy of the lane index, so that it is redone here instead of
   // being carried in registers across the loads above (where registers are scarcest)
@@ -1043,7 +1021,7 @@ skinny_mxfp4_x4_kernel(const DecodeParams p) {
   for (int nt = 0; nt < NT; nt++)
     woff[nt] = (uint32_t)(min(ltile0 + nt, sg.tiles - 1) * KT * 64 + lane);
 
-  // activations first (L2 resident), by hand, so that waiting for them does not wait for the weight ring
+  // activations first (L2 resident); no load below is conditional, so waiting for them does not wait for the weight ring
   const int nch = (t1 - t0) * 16;
   const char* xb = reinterpret_cast<const char*>(p.x);
   const uint32_t xk0 = (uint32_t)t0 * 256u;
@@ -1052,14 +1030,12 @@ skinny_mxfp4_x4_kernel(const DecodeParams p) {
     constexpr int it = decltype(IT)::value;
     const int row = min(it >> 1, p.M - 1), ck = max(min((it & 1) * 64 + lane, nch - 1), 0);
     const char* src = xb + (size_t)((uint32_t)(row * p.K) * 2u + xk0 + (uint32_t)ck * 16u);
-    i32x4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(src) : "memory");
-    raw[it] = v;
+    raw[it] = *reinterpret_cast<const i32x4*>(src);
   });
   i32x4 wreg[PF][NTW];
   uint32_t sreg[PF][NTW];
   auto load_stage = [&](int st, int t) {
-    t = min(t, t1 - 1);
+    t = max(min(t, t1 - 1), 0); // past the end (or a wave without K tiles): re-read a valid tile, never consumed
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
       const uint32_t slot = woff[nt % NT] + (uint32_t)t * 64u;
@@ -1067,21 +1043,14 @@ skinny_mxfp4_x4_kernel(const DecodeParams p) {
       sreg[st][nt] = *reinterpret_cast<const uint8_t*>(swb[nt / NT] + (size_t)slot);
     }
   };
-  if (t0 < t1) {
 #pragma unroll
-    for (int i = 0; i < PF; i++)
-      load_stage(i, t0 + i);
-  }
-  if (t1 - t0 >= PF) // a full ring: PF stages of distinct tiles, 2 * NTW loads each
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PF * NTW * 2) : "memory");
-  else
-    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+  for (int i = 0; i < PF; i++)
+    load_stage(i, t0 + i); // no branch around these: the compiler then counts them and waits for the activations only
   int lane2 = lane;
   asm volatile("" : "+v"(lane2));
   static_for<0, XNI>([&](auto IT) {
     constexpr int it = decltype(IT)::value;
-    i32x4 v = raw[it];
-    asm volatile("" : "+v"(v)); // the use stays behind the wait
+    const i32x4 v = raw[it];
     const int row = it >> 1, ck = (it & 1) * 64 + lane2;
     if (row < p.M && ck < nch)
       xs[ck * 4 + (row ^ (ck & 3))] = v;
