@@ -1162,7 +1162,7 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
   // out of the K loop.
   i32x4 xr[XL];
   auto load_x = [&](int t) {
-    t = min(t, t1 - 1);
+    t = max(min(t, t1 - 1), 0); // past the end (or a wave without K tiles): a valid tile, never consumed
     int r = r4, c = c16;
     asm volatile("" : "+v"(r), "+v"(c));
     const uint32_t base = (uint32_t)t * 256u + (uint32_t)c * 16u;
@@ -1190,7 +1190,7 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
   i32x4 wreg[PF][NTW];
   uint32_t sreg[PF][NTW];
   auto load_stage = [&](int st, int t) {
-    t = min(t, t1 - 1);
+    t = max(min(t, t1 - 1), 0); // past the end (or a wave without K tiles): a valid tile, never consumed
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
       const uint32_t slot = woff[nt % NT] + (uint32_t)t * 64u;
@@ -1198,12 +1198,12 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
       sreg[st][nt] = *reinterpret_cast<const uint8_t*>(swb[nt / NT] + (size_t)slot);
     }
   };
-  if (t0 < t1) {
-    load_x(t0); // needed first, requested first
+  // (no branch around the first requests: the compiler then counts the ring behind the activations and waits for
+  // the activations only)
+  load_x(t0); // needed first, requested first
 #pragma unroll
-    for (int i = 0; i < PF; i++)
-      load_stage(i, t0 + i);
-  }
+  for (int i = 0; i < PF; i++)
+    load_stage(i, t0 + i);
   // post-op inputs early, except where registers are scarcest (the gate/up pair has none but its biases)
   constexpr bool LATE_EP = DUAL && MG == 4;
   SkEpilogue<MG, NTW, DUAL, W> ep;
@@ -1315,7 +1315,7 @@ skinny_bf16_kernel(const DecodeParams p) {
   const int r4 = lane >> 4, c16 = lane & 15;
   i32x4 xr[XL];
   auto load_x = [&](int t) {
-    t = min(t, t1 - 1);
+    t = max(min(t, t1 - 1), 0); // past the end (or a wave without K tiles): a valid tile, never consumed
     int r = r4, c = c16;
     asm volatile("" : "+v"(r), "+v"(c));
     const size_t base = (size_t)t * 256u + (size_t)c * 16u;
@@ -1341,19 +1341,17 @@ skinny_bf16_kernel(const DecodeParams p) {
 
   i32x4 wreg[PF][NT][4];
   auto load_stage = [&](int st, int t) {
-    t = min(t, t1 - 1);
+    t = max(min(t, t1 - 1), 0); // past the end (or a wave without K tiles): a valid tile, never consumed
 #pragma unroll
     for (int nt = 0; nt < NT; nt++)
 #pragma unroll
       for (int j = 0; j < 4; j++)
         wreg[st][nt][j] = __builtin_nontemporal_load(wb + woff[nt] + (size_t)t * 256 + j * 64);
   };
-  if (t0 < t1) {
-    load_x(t0);
+  load_x(t0); // no branch around the first requests (exact wait counts)
 #pragma unroll
-    for (int i = 0; i < PF; i++)
-      load_stage(i, t0 + i);
-  }
+  for (int i = 0; i < PF; i++)
+    load_stage(i, t0 + i);
   SkEpilogue<MG, NT, false, W> ep;
   ep.prefetch(p, sg, ltile0, m0);
 
