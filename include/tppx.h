@@ -469,6 +469,26 @@ int tppx_linear_mxfp4_int8(const void* xq, const void* sa, const void* q,
                            int64_t K, int64_t bc, int post_op, float post_scale,
                            tppx_stream_t stream);
 
+/* fused_qkv_gemm (src/csrc/llm/fused_llm_infer.cpp:423-505) for decode steps
+ * (M <= 16) as ONE GEMM over the concatenated native weights of up to three
+ * projections (native tiles and scales are per 16-channel tile, so the
+ * concatenation along N is the buffers one after the other): every workgroup
+ * gets the same number of tiles whatever the projections' widths (three
+ * separate segments of 256 tiles each do not divide into 256 groups of 3).
+ * Output columns [0, n1) | [n1, n2) | [n2, N) go to three row-major bf16
+ * matrices laid one after the other in y (M x n1, M x (n2-n1), M x (N-n2)).
+ * gamma != NULL: llama_rms_norm on x inside the launch (row_sumsq != NULL: from
+ * the row sums the launch that wrote x left, as tppx_normsq_multi_linear_mxfp4;
+ * NULL: sums formed in the launch, as tppx_norm_multi_linear_mxfp4).  bias bf16
+ * [N] over the concatenated channels or NULL.  TPPX_EUNSUPPORTED when the
+ * LDS-staged kernel does not take the shape (callers fall back to
+ * tppx_*multi_linear_mxfp4). */
+int tppx_qkv_linear_mxfp4(const void* x, const void* row_sumsq, const void* gamma,
+                          float eps, const void* qw, const void* sw,
+                          const void* bias, void* y, int64_t M, int64_t N,
+                          int64_t K, int64_t n1, int64_t n2, int flags,
+                          tppx_stream_t stream);
+
 /* ---- launch plans ------------------------------------------------------- */
 
 /* No counterpart in the reference.  Writes into buf, one line per kernel, what

@@ -670,3 +670,44 @@ def test_split_launches_overlapping_on_two_streams():
     for si in (0, 1):
         for it, (ci, y) in enumerate(outs[si]):
             assert torch.equal(y, alone[ci]), f"stream {si}, launch {it}, case {ci}: differs from the single-stream result"
+
+
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("widths", [(512, 512, 512), (768, 256, 256), (512, 128)])
+def test_qkv_one_gemm_over_concatenated_weights(M, widths, monkeypatch):
+    """Decode steps run q/k/v as ONE GEMM over the concatenated native weights with three output matrices
+    (tppx_qkv_linear_mxfp4): the same bits as the segment-table launch and as separate calls, with and without the
+    RMSNorm in the launch (from handed row sums, or formed in the launch), with some biases missing; the projections'
+    own native copies become views into the concatenation and keep working on their own."""
+    from tpp_pytorch_extension import _ops as ops
+    _ops()
+    K = 2048
+    ws = [_make("mxfp4", n, K, 140 + i)[0] for i, n in enumerate(widths)]
+    bs = [randn_bf16((widths[0],), 0.01, 150).cuda()] + [None] * (len(widths) - 1)
+    x = randn_bf16((M, K), 1.0, 160 + M).cuda()
+    gamma = (torch.rand(K) + 0.5).cuda()
+    monkeypatch.setattr(ops, "QKV_ONE_GEMM", False)
+    seg = ops.qkv_gemm(x, ws, bs)
+    monkeypatch.setattr(ops, "QKV_ONE_GEMM", True)
+    one = ops.qkv_gemm(x, ws, bs)
+    assert getattr(ws[0], "_tppx_qkv_cat", None) is not None  # the one-GEMM path ran
+    for a, b, w, bias in zip(one, seg, ws, bs):
+        assert a.shape == b.shape and a.is_contiguous() and torch.equal(a, b)
+        assert torch.equal(a, ops.fc_plain(x, w, bias))  # native views into the concatenation
+    # RMSNorm inside the launch, sums formed there
+    monkeypatch.setattr(ops, "FUSE_NORM", True)
+    monkeypatch.setattr(ops, "QKV_ONE_GEMM", False)
+    seg_n = ops.qkv_gemm(x, ws, bs, norm=(gamma, 1e-5))
+    monkeypatch.setattr(ops, "QKV_ONE_GEMM", True)
+    one_n = ops.qkv_gemm(x, ws, bs, norm=(gamma, 1e-5))
+    for a, b in zip(one_n, seg_n):
+        assert torch.equal(a, b)
+    # RMSNorm from the row sums a producing GEMM left (here: formed by hand in the table's layout, slot 0 of 256)
+    table = ops.sums_table(x.device)
+    table[:M, 0] = (x.float() ** 2).sum(-1)
+    monkeypatch.setattr(ops, "QKV_ONE_GEMM", False)
+    seg_s = ops.qkv_gemm(x, ws, bs, norm=(gamma, 1e-5, table))
+    monkeypatch.setattr(ops, "QKV_ONE_GEMM", True)
+    one_s = ops.qkv_gemm(x, ws, bs, norm=(gamma, 1e-5, table))
+    for a, b in zip(one_s, seg_s):
+        assert torch.equal(a, b)

@@ -483,7 +483,7 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
 // LDS-staged MXFP4 decode kernel (M <= 16) with an optional RMSNorm in front
 static int run_mxfp4_xl(const char* who, const void* x, const void* gamma, float eps, const tppx_seg* segs,
                         int n_segs, int64_t M, int64_t K, int flags, bool dual, hipStream_t stream,
-                        const float* row_sumsq = nullptr) {
+                        const float* row_sumsq = nullptr, int64_t split1 = 0, int64_t split2 = 0) {
   int rc = check_common(who, x, M, K, n_segs, flags, nullptr, 0);
   if (rc)
     return rc;
@@ -496,6 +496,13 @@ static int run_mxfp4_xl(const char* who, const void* x, const void* gamma, float
   rc = fill_all(who, segs, n_segs, 32, dual, p);
   if (rc)
     return rc;
+  if (split1 > 0) {
+    TPPX_REQUIRE(n_segs == 1 && !dual && split1 % 16 == 0 && split2 % 16 == 0 && split1 <= split2 && split2 <= segs[0].N,
+                 TPPX_ESHAPE, "%s: output split %ld / %ld must be multiples of 16 within N=%ld", who, (long)split1, (long)split2, (long)segs[0].N);
+    TPPX_REQUIRE(M * segs[0].N < ((int64_t)1 << 31), TPPX_ESHAPE, "%s: M*N exceeds 2^31", who);
+    p.seg[0].split1 = (int)split1;
+    p.seg[0].split2 = (int)split2;
+  }
   p.x = x;
   p.M = (int)M;
   p.K = (int)K;
@@ -547,6 +554,16 @@ extern "C" int tppx_normsq_multi_linear_mxfp4(const void* x, const void* row_sum
   const char* who = "tppx_normsq_multi_linear_mxfp4";
   TPPX_REQUIRE(row_sumsq && gamma, TPPX_EINVAL, "%s: null table of row sums or gamma", who);
   return run_mxfp4_xl(who, x, gamma, eps, segs, n_segs, M, K, flags, false, (hipStream_t)stream, (const float*)row_sumsq);
+}
+
+extern "C" int tppx_qkv_linear_mxfp4(const void* x, const void* row_sumsq, const void* gamma, float eps, const void* qw,
+                                     const void* sw, const void* bias, void* y, int64_t M, int64_t N, int64_t K,
+                                     int64_t n1, int64_t n2, int flags, tppx_stream_t stream) {
+  const char* who = "tppx_qkv_linear_mxfp4";
+  TPPX_REQUIRE(n1 > 0 && n2 >= n1, TPPX_ESHAPE, "%s: output widths must be positive", who);
+  TPPX_REQUIRE(!row_sumsq || gamma, TPPX_EINVAL, "%s: row sums without gamma", who);
+  tppx_seg s = {qw, sw, bias, nullptr, nullptr, y, N, TPPX_POST_NONE, 1.0f};
+  return run_mxfp4_xl(who, x, gamma, eps, &s, 1, M, K, flags, false, (hipStream_t)stream, (const float*)row_sumsq, n1, n2);
 }
 
 extern "C" int tppx_normsq_swiglu_mxfp4(const void* x, const void* row_sumsq, const void* gamma, float eps,

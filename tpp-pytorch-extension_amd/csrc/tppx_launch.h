@@ -22,7 +22,19 @@ struct DecodeSeg {
   int grp0;                 // first workgroup (group of channel tiles) of this GEMM in the launch
   int post_op;
   float post_scale;
+  // split1 > 0: the N output channels go to up to three row-major matrices laid one after the other in y
+  // (columns [0, split1) | [split1, split2) | [split2, N): M x split1, then M x (split2 - split1), then the rest):
+  // one GEMM over concatenated weights whose results are separate tensors (q, k, v)
+  int split1, split2;
 };
+
+// element offset of output (m, n) of a segment in y (and in post_in / post_in2, which share its layout)
+__host__ __device__ inline int seg_out_offset(const DecodeSeg& sg, int M, int m, int n) {
+  if (sg.split1 <= 0)
+    return m * sg.N + n;
+  const int w0 = sg.split1, w1 = sg.split2 - sg.split1, w2 = sg.N - sg.split2;
+  return n < sg.split1 ? m * w0 + n : n < sg.split2 ? M * w0 + m * w1 + (n - sg.split1) : M * (w0 + w1) + m * w2 + (n - sg.split2);
+}
 
 struct DecodeParams {
   DecodeSeg seg[TPPX_MAX_SEGS];

@@ -99,7 +99,7 @@ struct SkEpilogue {
       const int m = m0 + mg * 16 + (l >> 4) * 4 + r;
       const int n = (ltile0 + a) * 16 + (l & 15);
       const bool valid = e < OUT && m < p.M && (ltile0 + a) < sg.tiles;
-      const int o = valid ? m * sg.N + n : 0, nn = valid ? n : 0;
+      const int o = valid ? seg_out_offset(sg, p.M, m, n) : 0, nn = valid ? n : 0;
       off[i] = valid ? o : -1;
       bias[i] = pb[nn];
       bias2[i] = DUAL ? pb2[nn] : 0;
@@ -124,7 +124,7 @@ struct SkEpilogue {
         const int m = m0 + mg * 16 + (l >> 4) * 4 + r;
         const int n = (ltile0 + a) * 16 + (l & 15);
         if (m < p.M && (ltile0 + a) < sg.tiles) {
-          off[i] = m * sg.N + n;
+          off[i] = seg_out_offset(sg, p.M, m, n);
           if (sg.bias)
             bias[i] = sg.bias[n];
           if (DUAL && p.seg[1].bias)

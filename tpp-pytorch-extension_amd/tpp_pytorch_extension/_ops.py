@@ -729,6 +729,65 @@ def _norm_table(norm):
     return norm[2] if (len(norm) > 2 and norm[2] is not None and NORM_FROM_SUMS) else None
 
 
+# Decode steps (<= 16 rows) on MXFP4 weights: q/k/v as ONE GEMM over the concatenated native weights, so that every
+# workgroup gets the same number of channel tiles (three segments of 256 tiles do not divide into 256 groups of 3:
+# 192 workgroups of 4 on 256 CUs).  TPPX_QKV_ONE_GEMM=0 keeps the segment table.
+QKV_ONE_GEMM = os.environ.get("TPPX_QKV_ONE_GEMM", "1") == "1"
+
+
+def _qkv_cat(weights):
+    """Concatenated native tiles / scales of the projections, built once and kept on the first weight; the
+    projections' own native copies become views into it (no second copy in memory)."""
+    key = tuple(id(w) for w in weights) + tuple(w.qdata.data_ptr() for w in weights)
+    have = getattr(weights[0], "_tppx_qkv_cat", None)
+    if have is not None and have[0] == key:
+        return have[1], have[2]
+    nats = [w.native() for w in weights]
+    qn = torch.cat([a.reshape(-1) for a, _ in nats])
+    sn = torch.cat([b.reshape(-1) for _, b in nats])
+    qo = so = 0
+    for w, (a, b) in zip(weights, nats):
+        w._native = (qn[qo:qo + a.numel()].view(a.shape), sn[so:so + b.numel()].view(b.shape))
+        qo += a.numel()
+        so += b.numel()
+    weights[0]._tppx_qkv_cat = (key, qn, sn)
+    return qn, sn
+
+
+def _qkv_one_gemm(L, input, x, M, K, weights, biases, norm):
+    """The fused q/k/v launch as one GEMM with three output matrices (tppx_qkv_linear_mxfp4); None when the case is
+    not its (other formats, more than 16 rows, a 4th GEMM with its GELU, a shape the LDS-staged kernel does not take)."""
+    n = len(weights)
+    if n not in (2, 3) or not (0 < M <= 16) or any(_as_q(w).weight_kind() != "mxfp4" for w in weights):
+        return None
+    widths = [w.weight_nk()[0] for w in weights]
+    if any(w.weight_nk()[1] != K for w in weights):
+        raise TppxError(_lib.ESHAPE, "Fused QKV weight block mismatch")
+    N = sum(widths)
+    qn, sn = _qkv_cat(weights)
+    bias = None
+    if any(b is not None and b.numel() for b in biases[:n]):
+        bias = torch.cat([(_prep_bias(b, w, x.device) if b is not None and b.numel()
+                           else torch.zeros(w, dtype=torch.bfloat16, device=x.device)) for b, w in zip(biases, widths)])
+    buf = torch.empty(M * N, dtype=torch.bfloat16, device=x.device)
+    gamma = sums = None
+    eps = 0.0
+    if norm is not None:  # fusable, or qkv_gemm() has applied it already
+        gamma, eps, sums = norm[0], float(norm[1]), _norm_table(norm)
+    n1 = widths[0]
+    n2 = widths[0] + widths[1]
+    rc = L.tppx_qkv_linear_mxfp4(x.data_ptr(), _lib.ptr(sums), _lib.ptr(gamma), eps, qn.data_ptr(), sn.data_ptr(),
+                                 _lib.ptr(bias), buf.data_ptr(), M, N, K, n1, n2, 0, _lib.stream_of(x))
+    if rc == _lib.EUNSUPPORTED:
+        return None
+    _lib.check(rc)
+    outs, o = [], 0
+    for w in widths:
+        outs.append(buf[o:o + M * w].view(tuple(input.shape[:-1]) + (w,)))
+        o += M * w
+    return outs
+
+
 def qkv_gemm(input, weights, biases, norm=None):
     """fused_qkv_gemm (src/csrc/llm/fused_llm_infer.cpp:423-505): several GEMMs
     over one activation in one launch; a 4th GEMM gets GELU (GPT-J fc_in).
@@ -756,6 +815,9 @@ def qkv_gemm(input, weights, biases, norm=None):
         biases.append(None)
     x, M, N0, K = _prep_input(input, weights[0])
     scheme = weights[0]._qscheme
+    outs = _qkv_one_gemm(L, input, x, M, K, weights, biases, norm) if QKV_ONE_GEMM else None
+    if outs is not None:
+        return outs
     segs = (_lib.Seg * n)()
     outs, keep = [], []
     for i, w in enumerate(weights):
