@@ -433,6 +433,12 @@ attn_decode_kernel(const AttnParams p) {
         d += bf16_bits_to_f32(mrow[key[u]]);
       sc[u] = key[u] < L ? d : -3.0e38f;
     }
+    if (t * 64 + 64 > L) { // the last trip only (wave-uniform): rows past the end may hold anything, NaN included
+#pragma unroll
+      for (int u = 0; u < NU; u++)
+        if (key[u] >= L)
+          vw[u] = i32x4{0, 0, 0, 0};
+    }
     float mn = m;
 #pragma unroll
     for (int u = 0; u < NU; u++)
@@ -447,8 +453,6 @@ attn_decode_kernel(const AttnParams p) {
       const float pr = key[u] < L ? __expf(sc[u] - mn) : 0.f;
       l += pr;
       const float pb = round_bf16(pr);
-      if (t * 64 + 64 > L && key[u] >= L) // rows past the end may hold anything, NaN included
-        vw[u] = i32x4{0, 0, 0, 0};
       float vf[8];
       unpack8(as_uint4(vw[u]), vf);
 #pragma unroll
