@@ -216,10 +216,14 @@ def test_prefill_qkv_and_swiglu_equal_composition():
     assert torch.equal(fused, ops.fc_mul(x, wu, None, ops.fc_silu(x, wg, None)))
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("bias", [False, True])
-def test_prefill_swiglu_one_grid_equals_composition(bias):
-    """Prefill rows: gate and up run as ONE grid of the large-M kernel (the gate tile parked in the workspace) and an
-    elementwise pass forms silu(gate) * up: the bits of fc_silu followed by fc_mul, ragged last row block included."""
+def test_prefill_swiglu_one_grid_equals_composition(bias, fused, monkeypatch):
+    """Prefill rows: gate and up run as ONE launch of the large-M kernel.  fused: every workgroup computes both
+    projections of its 128 output channels and forms silu(gate) * up in its epilogue; otherwise (TPPX_TILED_DUAL_FUSED=0)
+    the gate tile is parked in the workspace and an elementwise pass forms the product.  Either way the bits of
+    fc_silu followed by fc_mul, ragged last row block and ragged last channel block included."""
+    monkeypatch.setenv("TPPX_TILED_DUAL_FUSED", "1" if fused else "0")
     ops = _ops()
     K, M, N = 512, 300, 1056
     wg, qg, sg_ = _make("mxfp4", N, K, 191)

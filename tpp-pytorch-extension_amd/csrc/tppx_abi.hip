@@ -331,6 +331,16 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
       if (group) // fused q/k/v: one grid over the channel blocks of all GEMMs
         return check_hip(launch_tiled_mxfp4_group(t, n_segs, stream), who);
     }
+    if (dual && env_int("TPPX_TILED_DUAL_FUSED", 1) != 0) {
+      // Gate and up in ONE launch whose workgroups own 128 output channels each and compute both projections for
+      // them: silu(gate) * up is formed in the epilogue with the reference's rounding points and written once (no
+      // parked gate tile, no elementwise pass, no workspace).
+      TiledParams t[2] = {tiled_from_seg(p, 0), tiled_from_seg(p, 1)};
+      if (tiled_mxfp4_takes_groups(t[0])) {
+        t[0].post_op = t[1].post_op = TPPX_POST_NONE;
+        return check_hip(launch_tiled_mxfp4_group(t, 2, stream, true), who);
+      }
+    }
     if (dual) {
       // Gate and up as ONE grid when that fills the last round of workgroups better than two launches (28672
       // channels at 2048 rows: 2 x 3.5 rounds of 256 CUs become 7): the gate GEMM leaves its bf16 tile (bias + dot,

@@ -91,7 +91,8 @@ struct TiledParams {
 hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream);
 // large-M kernel: several GEMMs over one activation in one launch
 bool tiled_mxfp4_takes_groups(const TiledParams& p);
-hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream);
+// dual: the gate/up pair (t[0] = gate, t[1] = up) with silu(gate) * up formed in the launch and written to t[1].y
+hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream, bool dual = false);
 hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream);
 hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t stream);
 bool tiled_qint8_takes_groups(const TiledParams& p);

@@ -381,6 +381,60 @@ __device__ __forceinline__ void big_epilogue(const TiledParams& p, f32x4 (&acc)[
   }
 }
 
+// The gate/up pair: the wave tile's channels 0..31 are gate sums and 32..63 the up sums of the SAME 32 output
+// channels, so silu(gate) * up is formed here, with the rounding points of SiluPostOp followed by MulPostOp, and
+// only the product is written: a lane finishes 8 adjacent channels of one row (16-byte store, four lanes per row).
+template <int MT>
+__device__ __forceinline__ void big_epilogue_dual(const TiledParams& pg, const TiledParams& pu, f32x4 (&acc)[MT][4],
+                                                  float* stage, int m_base, int tile_base) {
+  const int lane = threadIdx.x & 63;
+  const int cx = (lane & 3) * 8; // first of this lane's 8 channels among the wave's 32
+  const int tile = tile_base + (cx >> 4);
+  const bool tile_ok = tile < pg.tiles;
+  const int n = min(tile, pg.tiles - 1) * 16 + (cx & 15);
+  float bg[8], bu[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    bg[e] = pg.bias ? bf16_bits_to_f32(pg.bias[n + e]) : 0.0f;
+    bu[e] = pu.bias ? bf16_bits_to_f32(pu.bias[n + e]) : 0.0f;
+  }
+#pragma unroll
+  for (int h = 0; h < MT / 4; h++) {
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          stage[(mt * 16 + (lane >> 4) * 4 + r) * EP_LD + nt * 16 + (lane & 15)] = acc[h * 4 + mt][nt][r];
+    // same wave wrote and reads: no barrier, the compiler orders the LDS accesses
+    for (int it = 0; it < 4; it++) {
+      const int row = it * 16 + (lane >> 2);
+      const int m = m_base + h * 64 + row;
+      const f32x4 g0 = *reinterpret_cast<const f32x4*>(stage + row * EP_LD + cx);
+      const f32x4 g1 = *reinterpret_cast<const f32x4*>(stage + row * EP_LD + cx + 4);
+      const f32x4 u0 = *reinterpret_cast<const f32x4*>(stage + row * EP_LD + 32 + cx);
+      const f32x4 u1 = *reinterpret_cast<const f32x4*>(stage + row * EP_LD + 32 + cx + 4);
+      if (tile_ok && m < pg.M) {
+        uint32_t out[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float glo = (e < 2 ? g0[2 * e] : g1[2 * e - 4]) + bg[2 * e];
+          const float ghi = (e < 2 ? g0[2 * e + 1] : g1[2 * e - 3]) + bg[2 * e + 1];
+          const float ulo = (e < 2 ? u0[2 * e] : u1[2 * e - 4]) + bu[2 * e];
+          const float uhi = (e < 2 ? u0[2 * e + 1] : u1[2 * e - 3]) + bu[2 * e + 1];
+          const uint32_t ga = apply_post_bits(glo, TPPX_POST_SILU, 0, 0, 1.0f);
+          const uint32_t gb = apply_post_bits(ghi, TPPX_POST_SILU, 0, 0, 1.0f);
+          const uint32_t a = apply_post_bits(ulo, TPPX_POST_MUL, ga & 0xffffu, 0, 1.0f);
+          const uint32_t b = apply_post_bits(uhi, TPPX_POST_MUL, gb & 0xffffu, 0, 1.0f);
+          out[e] = (a & 0xffffu) | (b << 16);
+        }
+        *reinterpret_cast<uint4*>(pu.y + (int64_t)m * pu.N + n) = make_uint4(out[0], out[1], out[2], out[3]);
+      }
+    }
+  }
+}
+
 // LDS operand reads issued by hand, so that they can be kept several MFMA
 // groups ahead of their use: the compiler does not track them, the waits are
 // explicit (LDS operations complete in issue order, so "at most N younger
@@ -405,7 +459,10 @@ struct BigParams {
 
 // MT = 16-row tiles per wave along M: 8 (workgroup tile 256 x 256) or 4 (128 x 256, for shapes whose 256-row tiles
 // would leave most of the last round of workgroups empty).
-template <int MT>
+// DUAL: the gate/up pair (seg[0] = gate, seg[1] = up, equal shapes).  A workgroup owns 128 output channels and
+// computes their gate AND up sums (wave tile = 2 gate tiles + the 2 up tiles of the same channels); the epilogue
+// writes silu(gate) * up once.  Channel blocks are 128 wide then.
+template <int MT, bool DUAL>
 __global__ void __launch_bounds__(512)
 big_mxfp4_kernel(const BigParams P) {
   constexpr int WGM = MT * 32;     // rows per workgroup
@@ -420,26 +477,31 @@ big_mxfp4_kernel(const BigParams P) {
   // pick this block's GEMM with uniform selects (everything stays in scalar registers)
   TiledParams p = P.seg[0];
   int nb_first = 0;
+  if (!DUAL) {
 #pragma unroll
-  for (int i = 1; i < TPPX_MAX_SEGS; i++)
-    if (i < P.n_seg && bn >= P.nb0[i]) {
-      p = P.seg[i];
-      nb_first = P.nb0[i];
-    }
+    for (int i = 1; i < TPPX_MAX_SEGS; i++)
+      if (i < P.n_seg && bn >= P.nb0[i]) {
+        p = P.seg[i];
+        nb_first = P.nb0[i];
+      }
+  }
   bn -= nb_first;
   const int KT = p.K >> 7;
   const int m_wg = bm * WGM;
-  const int tile_base = bn * 16 + wn * 4;
+  const int tile_base = DUAL ? bn * 8 + wn * 2 : bn * 16 + wn * 4;
 
   // Every global address below is a uniform base pointer plus a 32-bit byte
   // offset per lane (the launcher checks that the operands are smaller than
   // 4 GiB): one offset register instead of a 64-bit pointer pair per stream.
   const char* qwb = reinterpret_cast<const char*>(p.qw);
   const char* swb = reinterpret_cast<const char*>(p.sw);
+  // DUAL: tiles 2 and 3 of the wave are the up projection's tiles of the channels of tiles 0 and 1
+  const char* qwb2 = DUAL ? reinterpret_cast<const char*>(P.seg[1].qw) : qwb;
+  const char* swb2 = DUAL ? reinterpret_cast<const char*>(P.seg[1].sw) : swb;
   uint32_t woff[4]; // slot index of this lane in tile nt at K step 0
 #pragma unroll
   for (int nt = 0; nt < 4; nt++)
-    woff[nt] = (uint32_t)(min(tile_base + nt, p.tiles - 1) * KT * 64 + lane);
+    woff[nt] = (uint32_t)(min(tile_base + (DUAL ? (nt & 1) : nt), p.tiles - 1) * KT * 64 + lane);
 
   // A tile (256 rows x 128 K, 64 KiB): 64 blocks of 4 rows x 256 B go from
   // global memory straight into LDS, one wave instruction per block (lane =
@@ -491,8 +553,8 @@ big_mxfp4_kernel(const BigParams P) {
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) {
       const uint32_t slot = woff[nt] + (uint32_t)ks * 64u;
-      bnext[nt] = *reinterpret_cast<const i32x4*>(qwb + (size_t)(slot * 16u));
-      snext[nt] = *reinterpret_cast<const uint8_t*>(swb + (size_t)slot);
+      bnext[nt] = *reinterpret_cast<const i32x4*>((nt < 2 ? qwb : qwb2) + (size_t)(slot * 16u));
+      snext[nt] = *reinterpret_cast<const uint8_t*>((nt < 2 ? swb : swb2) + (size_t)slot);
     }
   };
   auto take_b = [&]() {
@@ -562,7 +624,11 @@ big_mxfp4_kernel(const BigParams P) {
     step(std::true_type{}, ks);
   step(std::false_type{}, KT - 1);
   // every wave has left the main loop (barrier above): LDS is free for the epilogue staging
-  big_epilogue<MT>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
+  if (DUAL)
+    big_epilogue_dual<MT>(p, P.seg[1], acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16),
+                          tile_base);
+  else
+    big_epilogue<MT>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
 }
 
 // ---------------------------------------------------------------------------
@@ -974,7 +1040,17 @@ bool tiled_mxfp4_takes_groups(const TiledParams& p) {
   return p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && big_fits(p);
 }
 
-hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream) {
+template <int MT, bool DUAL>
+static hipError_t big_launch(const BigParams& P, int wgs, size_t lds, hipStream_t stream) {
+  TPPX_PLAN_ONLY((big_mxfp4_kernel<MT, DUAL>), dim3(wgs), dim3(512), lds);
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_mxfp4_kernel<MT, DUAL>), lds); e != hipSuccess)
+    return e;
+  big_mxfp4_kernel<MT, DUAL><<<dim3(wgs), dim3(512), lds, stream>>>(P);
+  return hipGetLastError();
+}
+
+// dual: t[0] = gate, t[1] = up (equal shapes, n == 2); y[m][n] = silu(gate) * up goes to t[1].y
+hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream, bool dual) {
   BigParams P;
   memset(&P, 0, sizeof(P));
   int nb = 0;
@@ -982,6 +1058,12 @@ hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t str
     P.seg[i] = t[i];
     P.nb0[i] = nb;
     nb += (t[i].tiles + 15) / 16;
+  }
+  if (dual) {
+    if (n != 2 || t[0].tiles != t[1].tiles || t[0].K != t[1].K || t[0].M != t[1].M || t[0].x != t[1].x)
+      return hipErrorInvalidValue;
+    nb = (t[0].tiles + 7) / 8; // 128 output channels (gate and up of each) per workgroup
+    P.nb0[1] = nb;
   }
   for (int i = n; i <= TPPX_MAX_SEGS; i++)
     P.nb0[i] = nb;
@@ -997,18 +1079,9 @@ hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t str
   const int env_mt = env_int("TPPX_TILED_BIG_MT", 0);
   if (env_mt == 4 || env_mt == 8)
     mt = env_mt;
-  if (mt == 4) {
-    TPPX_PLAN_ONLY(big_mxfp4_kernel<4>, dim3(MB4 * nb), dim3(512), lds);
-    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_mxfp4_kernel<4>), lds); e != hipSuccess)
-      return e;
-    big_mxfp4_kernel<4><<<dim3(MB4 * nb), dim3(512), lds, stream>>>(P);
-  } else {
-    TPPX_PLAN_ONLY(big_mxfp4_kernel<8>, dim3(MB8 * nb), dim3(512), lds);
-    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_mxfp4_kernel<8>), lds); e != hipSuccess)
-      return e;
-    big_mxfp4_kernel<8><<<dim3(MB8 * nb), dim3(512), lds, stream>>>(P);
-  }
-  return hipGetLastError();
+  if (mt == 4)
+    return dual ? big_launch<4, true>(P, MB4 * nb, lds, stream) : big_launch<4, false>(P, MB4 * nb, lds, stream);
+  return dual ? big_launch<8, true>(P, MB8 * nb, lds, stream) : big_launch<8, false>(P, MB8 * nb, lds, stream);
 }
 
 // MXFP4 weights x MXFP8 activations (t[i].xq = quantised activations in operand order, t[i].sa = their scale bytes)
