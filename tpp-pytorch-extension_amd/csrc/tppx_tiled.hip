@@ -462,15 +462,18 @@ struct BigParams {
 // DUAL: the gate/up pair (seg[0] = gate, seg[1] = up, equal shapes).  A workgroup owns 128 output channels and
 // computes their gate AND up sums (wave tile = 2 gate tiles + the 2 up tiles of the same channels); the epilogue
 // writes silu(gate) * up once.  Channel blocks are 128 wide then.
-template <int MT, bool DUAL>
-__global__ void __launch_bounds__(512)
+// WM = rows of waves: 2 (8 waves, one workgroup per CU) or 1 (4 waves owning MT * 16 rows, TWO workgroups per CU:
+// each wave does what a wave of the 8-wave form does, but the two workgroups of a CU meet at their own barriers, so
+// while one stands at the end of a K step the matrix cores run the other's MFMAs).
+template <int MT, bool DUAL, int WM>
+__global__ void __launch_bounds__(WM * 256, WM == 1 ? 2 : 1)
 big_mxfp4_kernel(const BigParams P) {
-  constexpr int WGM = MT * 32;     // rows per workgroup
+  constexpr int WGM = MT * 16 * WM; // rows per workgroup
   constexpr int ABUF = WGM * 256;  // bytes of one A buffer (rows x 128 K bf16)
   extern __shared__ __align__(16) uint8_t tl_lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform: keeps LDS bases and block indices scalar
-  const int wm = wave & 1, wn = wave >> 1;
+  const int wm = wave % WM, wn = wave / WM;
   const int MB = (P.seg[0].M + WGM - 1) / WGM;
   int bm, bn;
   tile_of_block(MB, P.nb0[P.n_seg], bm, bn);
@@ -1040,12 +1043,15 @@ bool tiled_mxfp4_takes_groups(const TiledParams& p) {
   return p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && big_fits(p);
 }
 
-template <int MT, bool DUAL>
-static hipError_t big_launch(const BigParams& P, int wgs, size_t lds, hipStream_t stream) {
-  TPPX_PLAN_ONLY((big_mxfp4_kernel<MT, DUAL>), dim3(wgs), dim3(512), lds);
-  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_mxfp4_kernel<MT, DUAL>), lds); e != hipSuccess)
+template <int MT, bool DUAL, int WM>
+static hipError_t big_launch(const BigParams& P, int wgs, hipStream_t stream) {
+  // epilogue staging per wave; >= the two A buffers
+  const size_t lds = (size_t)WM * 4 * 64 * EP_LD * sizeof(float);
+  static_assert((size_t)WM * 4 * 64 * EP_LD * sizeof(float) >= (size_t)2 * MT * 16 * WM * 256, "LDS plan");
+  TPPX_PLAN_ONLY((big_mxfp4_kernel<MT, DUAL, WM>), dim3(wgs), dim3(WM * 256), lds);
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_mxfp4_kernel<MT, DUAL, WM>), lds); e != hipSuccess)
     return e;
-  big_mxfp4_kernel<MT, DUAL><<<dim3(wgs), dim3(512), lds, stream>>>(P);
+  big_mxfp4_kernel<MT, DUAL, WM><<<dim3(wgs), dim3(WM * 256), lds, stream>>>(P);
   return hipGetLastError();
 }
 
@@ -1068,20 +1074,22 @@ hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t str
   for (int i = n; i <= TPPX_MAX_SEGS; i++)
     P.nb0[i] = nb;
   P.n_seg = n;
-  const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the two A buffers
-  // 256-row tiles unless their last round of workgroups (256 CUs, one workgroup each) would be less than half
-  // full while 128-row tiles fill it better: then every workgroup takes half the rows
+  // 256-row workgroups of 8 waves, one per CU, or 128-row workgroups of 4 waves, two per CU (512 at a time).  The
+  // second form costs a few percent when both fill the device (measured at M = 2048: o-projection 189 -> 196 us,
+  // K = 28672 611 -> 647 us) but its workgroups are half the size, so a last partial round costs less: q/k/v with
+  // 10240 channels, 320 workgroups of 256 rows = 2 rounds, 640 of 128 rows = 1.25 (289 us with 8-wave 128-row
+  // workgroups, 259 us with these).  Costs in units of one full round of 256-row workgroups.
   const int MB8 = (t[0].M + 255) / 256, MB4 = (t[0].M + 127) / 128;
-  auto rounds = [](int wgs) { return (wgs + 255) / 256; };
-  // (measured: a 128-row workgroup needs about 0.57 of the time of a 256-row one)
-  const double cost8 = rounds(MB8 * nb), cost4 = 0.5 * 1.15 * rounds(MB4 * nb);
+  const double cost8 = (MB8 * nb + 255) / 256;
+  const int w4 = MB4 * nb;
+  const double cost4 = w4 <= 256 ? 0.6 : 1.05 * (w4 <= 512 ? 1.0 : w4 / 512.0);
   int mt = cost4 < cost8 ? 4 : 8;
   const int env_mt = env_int("TPPX_TILED_BIG_MT", 0);
   if (env_mt == 4 || env_mt == 8)
     mt = env_mt;
   if (mt == 4)
-    return dual ? big_launch<4, true>(P, MB4 * nb, lds, stream) : big_launch<4, false>(P, MB4 * nb, lds, stream);
-  return dual ? big_launch<8, true>(P, MB8 * nb, lds, stream) : big_launch<8, false>(P, MB8 * nb, lds, stream);
+    return dual ? big_launch<8, true, 1>(P, MB4 * nb, stream) : big_launch<8, false, 1>(P, MB4 * nb, stream);
+  return dual ? big_launch<8, true, 2>(P, MB8 * nb, stream) : big_launch<8, false, 2>(P, MB8 * nb, stream);
 }
 
 // MXFP4 weights x MXFP8 activations (t[i].xq = quantised activations in operand order, t[i].sa = their scale bytes)
