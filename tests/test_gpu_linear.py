@@ -189,6 +189,40 @@ def test_prefill_mxfp4_ragged_blocks_and_post_ops(post):
     _run("mxfp4", 300, 544, 384, post, post != "mul", 700, ulps=2 if post in ("silu", "gelu") else 1)
 
 
+@pytest.mark.parametrize("tile", [1, 2, 3])
+@pytest.mark.parametrize("post", ["none", "silu", "add2"])
+def test_prefill_mxfp4_every_workgroup_tile_ragged(tile, post, monkeypatch):
+    """The three workgroup tiles of the large-M MXFP4 kernel (256 x 256, 128 x 256 two per CU, 128 x 512), each
+    forced, on the ragged case above (rows, channel blocks and K steps all uneven) against the oracle."""
+    monkeypatch.setenv("TPPX_TILED_BIG_TILE", str(tile))
+    _run("mxfp4", 300, 544, 384, post, True, 705, ulps=2 if post == "silu" else 1)
+
+
+def test_prefill_mxfp4_workgroup_tiles_and_xcd_splits_agree(monkeypatch):
+    """Every workgroup tile and every split of the tile space over the XCDs computes the same sums in the same order:
+    identical bits, single GEMM, fused q/k/v and the gate/up pair."""
+    ops = _ops()
+    M, K = 1024, 512
+    w = _make("mxfp4", 4096, K, 710)[0]
+    ws = [_make("mxfp4", n, K, 711 + i)[0] for i, n in enumerate((2048, 1024, 1024))]
+    wg, wu = _make("mxfp4", 4096, K, 715)[0], _make("mxfp4", 4096, K, 716)[0]
+    x = randn_bf16((M, K), 1.0, 717).cuda()
+
+    def run():
+        return [ops.fc_plain(x, w, None)] + list(ops.qkv_gemm(x, ws, [None] * 3)) + [ops.swiglu_gate_up(x, wg, wu)]
+
+    monkeypatch.setenv("TPPX_TILED_BIG_TILE", "1")
+    monkeypatch.setenv("TPPX_TILED_XCD_M", "1")
+    want = run()
+    assert torch.equal(want[4], ops.fc_mul(x, wu, None, ops.fc_silu(x, wg, None)))
+    for tile in (1, 2, 3):
+        for xm in (1, 2, 4):
+            monkeypatch.setenv("TPPX_TILED_BIG_TILE", str(tile))
+            monkeypatch.setenv("TPPX_TILED_XCD_M", str(xm))
+            for i, (a, b) in enumerate(zip(run(), want)):
+                assert torch.equal(a, b), (tile, xm, i)
+
+
 @pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])
 def test_prefill_tiled_m2048(fmt):
     """Prefill row count of BASELINE config 4 (M = 2048) on a layer slice the

@@ -40,11 +40,23 @@ __device__ __forceinline__ bf16x8 tl_cvt_fp4x8(uint32_t codes, float scale) {
   return w;
 }
 
-// XCD-aware tile order: returns (bm, bn) of this workgroup.
-__device__ __forceinline__ void tile_of_block(int MB, int NB, int& bm, int& bn) {
+// XCD-aware tile order: returns (bm, bn) of this workgroup.  Workgroup ids go round the 8 XCDs; XCD x gets a
+// rectangle of the tile space and walks it row block fastest, so that the workgroups resident on an XCD at the same
+// time share operand tiles in its L2.  xm = how many of the 8 rectangles lie along M (1: an XCD owns NB/8 channel
+// blocks and all row blocks; 2, 4: 1/xm of the row blocks and xm/8 of the channel blocks).  Every XCD fetches
+// 1/xm of the activations and xm/8 of the weights from memory.  The host passes an xm that divides evenly.
+__device__ __forceinline__ void tile_of_block(int MB, int NB, int& bm, int& bn, int xm = 1) {
   int id = blockIdx.x;
   const int T = MB * NB;
-  if ((T & 7) == 0) {
+  if ((T & 7) == 0 && xm > 1) {
+    const int x = id & 7, r = id >> 3;
+    const int xn = 8 / xm;                // rectangles along N
+    const int mb = MB / xm, nb = NB / xn; // the rectangle of XCD x: mb x nb tiles at (x % xm, x / xm)
+    bm = (x % xm) * mb + r % mb;
+    bn = (x / xm) * nb + r / mb;
+    return;
+  }
+  if ((T & 7) == 0) { // an eighth of the tiles in column-major order, whether or not NB divides by 8
     const int per = T >> 3;
     id = (id & 7) * per + (id >> 3);
   }
@@ -455,20 +467,26 @@ struct BigParams {
   TiledParams seg[TPPX_MAX_SEGS];
   int nb0[TPPX_MAX_SEGS + 1]; // first channel block of each segment, then the total
   int n_seg;
+  int xm;                     // XCD rectangles along M (see tile_of_block)
 };
 
-// MT = 16-row tiles per wave along M: 8 (workgroup tile 256 x 256) or 4 (128 x 256, for shapes whose 256-row tiles
-// would leave most of the last round of workgroups empty).
+// MT = 16-row tiles per wave along M (8).
 // DUAL: the gate/up pair (seg[0] = gate, seg[1] = up, equal shapes).  A workgroup owns 128 output channels and
 // computes their gate AND up sums (wave tile = 2 gate tiles + the 2 up tiles of the same channels); the epilogue
 // writes silu(gate) * up once.  Channel blocks are 128 wide then.
-// WM = rows of waves: 2 (8 waves, one workgroup per CU) or 1 (4 waves owning MT * 16 rows, TWO workgroups per CU:
-// each wave does what a wave of the 8-wave form does, but the two workgroups of a CU meet at their own barriers, so
-// while one stands at the end of a K step the matrix cores run the other's MFMAs).
-template <int MT, bool DUAL, int WM>
-__global__ void __launch_bounds__(WM * 256, WM == 1 ? 2 : 1)
+// WM x WN waves, each with a wave tile of MT*16 rows x 64 channels:
+//   2 x 4  workgroup tile 256 x 256, one workgroup per CU
+//   1 x 4  128 x 256, 4 waves, TWO workgroups per CU: half-size workgroups for shapes whose last round of 256-row
+//          workgroups would be mostly empty
+//   1 x 8  128 x 512, one workgroup per CU: the same 65536 sums per CU as 2 x 4, but half the activation bytes per
+//          K step (128 rows) and every weight tile fetched by ONE wave instead of by the two of a wave column -- half
+//          the bytes moved from L2 into the CU per MFMA
+template <int MT, bool DUAL, int WM, int WN>
+__global__ void __launch_bounds__(WM * WN * 64, WM * WN == 4 ? 2 : 1)
 big_mxfp4_kernel(const BigParams P) {
   constexpr int WGM = MT * 16 * WM; // rows per workgroup
+  constexpr int NBLK = MT * 4 / WN; // blocks of 4 rows x 256 B of the A tile that a wave fetches per K step
+  static_assert(NBLK % 4 == 0, "the swizzle below takes a wave's first block to be a multiple of 4");
   constexpr int ABUF = WGM * 256;  // bytes of one A buffer (rows x 128 K bf16)
   extern __shared__ __align__(16) uint8_t tl_lds[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -476,7 +494,7 @@ big_mxfp4_kernel(const BigParams P) {
   const int wm = wave % WM, wn = wave / WM;
   const int MB = (P.seg[0].M + WGM - 1) / WGM;
   int bm, bn;
-  tile_of_block(MB, P.nb0[P.n_seg], bm, bn);
+  tile_of_block(MB, P.nb0[P.n_seg], bm, bn, P.xm);
   // pick this block's GEMM with uniform selects (everything stays in scalar registers)
   TiledParams p = P.seg[0];
   int nb_first = 0;
@@ -491,7 +509,7 @@ big_mxfp4_kernel(const BigParams P) {
   bn -= nb_first;
   const int KT = p.K >> 7;
   const int m_wg = bm * WGM;
-  const int tile_base = DUAL ? bn * 8 + wn * 2 : bn * 16 + wn * 4;
+  const int tile_base = DUAL ? bn * (WN * 2) + wn * 2 : bn * (WN * 4) + wn * 4;
 
   // Every global address below is a uniform base pointer plus a 32-bit byte
   // offset per lane (the launcher checks that the operands are smaller than
@@ -523,14 +541,14 @@ big_mxfp4_kernel(const BigParams P) {
       rdb[j] = (uint32_t)((m >> 2) * 1024 + (m & 3) * 256 + (((g * 4 + j) ^ m) & 15) * 16);
   }
   const char* xbase = reinterpret_cast<const char*>(p.x);
-  // this wave's 8 blocks: blk = wave*8 + i -> rows blk*4 + (lane>>4)
+  // this wave's NBLK blocks: blk = wave*NBLK + i -> rows blk*4 + (lane>>4)
   const int rin = (lane >> 4);          // row inside the block
   const int ch = lane & 15;             // chunk position of this lane inside the row
   // source byte offset of block i at K step ks:
   //   row(i) * K * 2 + ((ch ^ m16(i)) & 15) * 16 + ks * 256, row(i) = m_wg + (wave*8 + i)*4 + rin,
   //   m16(i) = (i & 3)*4 + rin (wave*8 is a multiple of 4)
   const bool full = m_wg + WGM <= p.M; // uniform
-  const uint32_t xrow0 = (uint32_t)((m_wg + wave * (MT * 4) + rin) * p.K) * 2u;
+  const uint32_t xrow0 = (uint32_t)((m_wg + wave * (NBLK * 4) + rin) * p.K) * 2u;
   const uint32_t blk_stride = (uint32_t)(4 * p.K) * 2u; // uniform
   auto load_a_one = [&](auto I, int ks, int buf) {
     constexpr int i = decltype(I)::value;
@@ -539,14 +557,14 @@ big_mxfp4_kernel(const BigParams P) {
     if (full) {
       off = xrow0 + (uint32_t)i * blk_stride + sw + (uint32_t)ks * 256u;
     } else { // past the end: re-read the last row (never stored)
-      const int row = min(m_wg + (wave * MT + i) * 4 + rin, p.M - 1);
+      const int row = min(m_wg + (wave * NBLK + i) * 4 + rin, p.M - 1);
       off = (uint32_t)(row * p.K) * 2u + sw + (uint32_t)ks * 256u;
     }
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xbase + (size_t)off),
-                                     (__attribute__((address_space(3))) void*)(tl_lds + buf * ABUF + (wave * MT + i) * 1024),
+                                     (__attribute__((address_space(3))) void*)(tl_lds + buf * ABUF + (wave * NBLK + i) * 1024),
                                      16, 0, 0);
   };
-  auto load_a = [&](int ks, int buf) { static_for<0, MT>([&](auto I) { load_a_one(I, ks, buf); }); };
+  auto load_a = [&](int ks, int buf) { static_for<0, NBLK>([&](auto I) { load_a_one(I, ks, buf); }); };
   // B of one K step: 4 tiles x 4 dwords (one per step j) and the scale factors
   uint32_t bc[4][4];
   float sc[4];
@@ -580,7 +598,7 @@ big_mxfp4_kernel(const BigParams P) {
   load_a(0, 0);
   load_b(0);
   __syncthreads();
-  // One K step.  MORE: the next step's A tile is requested during this one, one block behind each of the first MT
+  // One K step.  MORE: the next step's A tile is requested during this one, one block behind each of the first NBLK
   // MFMA groups (issued in one burst, a wave stands at its load instructions while the memory pipeline's queue
   // drains, and its MFMAs wait with it); it lands in the other buffer.
   auto step = [&](auto MORE, int ks) {
@@ -616,7 +634,7 @@ big_mxfp4_kernel(const BigParams P) {
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
         acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[nt], acc[mt][nt], 0, 0, 0);
-      if constexpr (more && q < MT)
+      if constexpr (more && q < NBLK)
         load_a_one(std::integral_constant<int, q>{}, ks + 1, buf ^ 1);
       if constexpr (more && q == NQ / 2 - 1)
         load_b(ks + 1); // dwords of steps 0 and 1 of the current B are dead by now
@@ -1035,6 +1053,9 @@ big_fp8_kernel(const BigParams P) {
   big_epilogue<MT>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
 }
 
+// cost of a full round of 128 x 512 workgroups relative to one of 256 x 256 (measured)
+constexpr double BIG_WIDE_COST = 0.97;
+
 static bool big_fits(const TiledParams& p) {
   return (int64_t)p.M * p.K * 2 < ((int64_t)1 << 32) && (int64_t)p.tiles * 8 * p.K < ((int64_t)1 << 32);
 }
@@ -1043,53 +1064,86 @@ bool tiled_mxfp4_takes_groups(const TiledParams& p) {
   return p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && big_fits(p);
 }
 
-template <int MT, bool DUAL, int WM>
+template <int MT, bool DUAL, int WM, int WN>
 static hipError_t big_launch(const BigParams& P, int wgs, hipStream_t stream) {
   // epilogue staging per wave; >= the two A buffers
-  const size_t lds = (size_t)WM * 4 * 64 * EP_LD * sizeof(float);
-  static_assert((size_t)WM * 4 * 64 * EP_LD * sizeof(float) >= (size_t)2 * MT * 16 * WM * 256, "LDS plan");
-  TPPX_PLAN_ONLY((big_mxfp4_kernel<MT, DUAL, WM>), dim3(wgs), dim3(WM * 256), lds);
-  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_mxfp4_kernel<MT, DUAL, WM>), lds); e != hipSuccess)
+  const size_t lds = (size_t)WM * WN * 64 * EP_LD * sizeof(float);
+  static_assert((size_t)WM * WN * 64 * EP_LD * sizeof(float) >= (size_t)2 * MT * 16 * WM * 256, "LDS plan");
+  TPPX_PLAN_ONLY((big_mxfp4_kernel<MT, DUAL, WM, WN>), dim3(wgs), dim3(WM * WN * 64), lds);
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_mxfp4_kernel<MT, DUAL, WM, WN>), lds); e != hipSuccess)
     return e;
-  big_mxfp4_kernel<MT, DUAL, WM><<<dim3(wgs), dim3(WM * 256), lds, stream>>>(P);
+  big_mxfp4_kernel<MT, DUAL, WM, WN><<<dim3(wgs), dim3(WM * WN * 64), lds, stream>>>(P);
   return hipGetLastError();
 }
 
 // dual: t[0] = gate, t[1] = up (equal shapes, n == 2); y[m][n] = silu(gate) * up goes to t[1].y
 hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream, bool dual) {
+  if (dual && (n != 2 || t[0].tiles != t[1].tiles || t[0].K != t[1].K || t[0].M != t[1].M || t[0].x != t[1].x))
+    return hipErrorInvalidValue;
+  // channel blocks of the launch when a workgroup owns `tpw` channel tiles (of each projection for the pair)
+  auto blocks = [&](int tpw) {
+    int nb = 0;
+    for (int i = 0; i < (dual ? 1 : n); i++)
+      nb += (t[i].tiles + tpw - 1) / tpw;
+    return nb;
+  };
+  const int nb4 = blocks(dual ? 8 : 16), nb8 = blocks(dual ? 16 : 32); // 4 or 8 wave columns
+  const int MB8 = (t[0].M + 255) / 256, MB4 = (t[0].M + 127) / 128;
+  // Workgroup tile.  256 x 256 (8 waves, one per CU) or 128 x 512 (8 waves, one per CU) when their rounds of 256
+  // workgroups are full; 128 x 256 (4 waves, two per CU, 512 at a time) costs a few percent more per round but its
+  // workgroups are half the size, so a last partial round costs less (q/k/v with 10240 channels at M = 2048: 320
+  // workgroups of 256 x 256 are 2 rounds, 640 of 128 x 256 are 1.25).  Costs in units of one full round of 256 x 256.
+  auto rounds = [](int wgs) { return (double)((wgs + 255) / 256); };
+  const int w4 = MB4 * nb4;
+  const double cost[3] = {rounds(MB8 * nb4), w4 <= 256 ? 0.6 : 1.05 * (w4 <= 512 ? 1.0 : w4 / 512.0),
+                          BIG_WIDE_COST * rounds(MB4 * nb8)};
+  int shape = 0;
+  for (int i = 1; i < 3; i++)
+    if (cost[i] < cost[shape])
+      shape = i;
+  const int env_shape = env_int("TPPX_TILED_BIG_TILE", 0); // 1 = 256 x 256, 2 = 128 x 256, 3 = 128 x 512
+  if (env_shape >= 1 && env_shape <= 3)
+    shape = env_shape - 1;
+  const int tpw = (shape == 2 ? 8 : 4) * (dual ? 2 : 4);
   BigParams P;
   memset(&P, 0, sizeof(P));
   int nb = 0;
   for (int i = 0; i < n; i++) {
     P.seg[i] = t[i];
     P.nb0[i] = nb;
-    nb += (t[i].tiles + 15) / 16;
+    nb += (t[i].tiles + tpw - 1) / tpw;
   }
   if (dual) {
-    if (n != 2 || t[0].tiles != t[1].tiles || t[0].K != t[1].K || t[0].M != t[1].M || t[0].x != t[1].x)
-      return hipErrorInvalidValue;
-    nb = (t[0].tiles + 7) / 8; // 128 output channels (gate and up of each) per workgroup
+    nb = (t[0].tiles + tpw - 1) / tpw;
     P.nb0[1] = nb;
   }
   for (int i = n; i <= TPPX_MAX_SEGS; i++)
     P.nb0[i] = nb;
   P.n_seg = n;
-  // 256-row workgroups of 8 waves, one per CU, or 128-row workgroups of 4 waves, two per CU (512 at a time).  The
-  // second form costs a few percent when both fill the device (measured at M = 2048: o-projection 189 -> 196 us,
-  // K = 28672 611 -> 647 us) but its workgroups are half the size, so a last partial round costs less: q/k/v with
-  // 10240 channels, 320 workgroups of 256 rows = 2 rounds, 640 of 128 rows = 1.25 (289 us with 8-wave 128-row
-  // workgroups, 259 us with these).  Costs in units of one full round of 256-row workgroups.
-  const int MB8 = (t[0].M + 255) / 256, MB4 = (t[0].M + 127) / 128;
-  const double cost8 = (MB8 * nb + 255) / 256;
-  const int w4 = MB4 * nb;
-  const double cost4 = w4 <= 256 ? 0.6 : 1.05 * (w4 <= 512 ? 1.0 : w4 / 512.0);
-  int mt = cost4 < cost8 ? 4 : 8;
-  const int env_mt = env_int("TPPX_TILED_BIG_MT", 0);
-  if (env_mt == 4 || env_mt == 8)
-    mt = env_mt;
-  if (mt == 4)
-    return dual ? big_launch<8, true, 1>(P, MB4 * nb, stream) : big_launch<8, false, 1>(P, MB4 * nb, stream);
-  return dual ? big_launch<8, true, 2>(P, MB8 * nb, stream) : big_launch<8, false, 2>(P, MB8 * nb, stream);
+  {
+    // XCD rectangles: the split that moves the fewest bytes from memory into the L2s (activations: rows x K bf16 per
+    // row block, fetched by 8 / xm XCDs... every XCD fetches 1/xm of them; weights 0.53 B per element, xm/8 each)
+    const int MBs = shape == 0 ? MB8 : MB4;
+    const double a_bytes = (double)t[0].M * t[0].K * 2.0, w_bytes = (dual ? 2.0 : 1.0) * nb * tpw * 16.0 * t[0].K * 0.53;
+    double best = 1e300;
+    P.xm = 1;
+    for (int xm = 1; xm <= 4; xm *= 2)
+      if (MBs % xm == 0 && nb % (8 / xm) == 0) {
+        const double fill = 8.0 * (a_bytes / xm + w_bytes * xm / 8.0);
+        if (fill < best) {
+          best = fill;
+          P.xm = xm;
+        }
+      }
+    const int env_xm = env_int("TPPX_TILED_XCD_M", 0);
+    if ((env_xm == 1 || env_xm == 2 || env_xm == 4) && MBs % env_xm == 0 && nb % (8 / env_xm) == 0)
+      P.xm = env_xm;
+  }
+  if (shape == 2)
+    return dual ? big_launch<8, true, 1, 8>(P, MB4 * nb, stream) : big_launch<8, false, 1, 8>(P, MB4 * nb, stream);
+  if (shape == 1)
+    return dual ? big_launch<8, true, 1, 4>(P, MB4 * nb, stream) : big_launch<8, false, 1, 4>(P, MB4 * nb, stream);
+  return dual ? big_launch<8, true, 2, 4>(P, MB8 * nb, stream) : big_launch<8, false, 2, 4>(P, MB8 * nb, stream);
 }
 
 // MXFP4 weights x MXFP8 activations (t[i].xq = quantised activations in operand order, t[i].sa = their scale bytes)
