@@ -625,12 +625,17 @@ def test_mxfp4_linear_on_fp8_activations(M, N, K, post):
     assert err_stats(t2bits(y), exact)["rel_l2"] <= 5e-2
 
 
-def test_fp8_activation_qkv_and_swiglu_equal_separate_calls():
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("M,K,widths", [(160, 512, (512, 256, 256)), (300, 384, (544, 288, 288))])
+def test_fp8_activation_qkv_and_swiglu_equal_separate_calls(M, K, widths, fused, monkeypatch):
+    """fused: the gate/up pair with both projections per workgroup and silu(gate) * up in the epilogue; otherwise
+    (TPPX_TILED_DUAL_FUSED=0) the parked gate tile and the elementwise pass.  The second shape has ragged row, channel
+    and K blocks."""
     from tpp_pytorch_extension import _lib, _ops as ops
     _ops()
-    M, K = 160, 512
+    monkeypatch.setenv("TPPX_TILED_DUAL_FUSED", "1" if fused else "0")
     x = randn_bf16((M, K), 1.0, 99).cuda()
-    ws = [_make("mxfp4", n, K, 100 + i)[0] for i, n in enumerate((512, 256, 256))]
+    ws = [_make("mxfp4", n, K, 100 + i)[0] for i, n in enumerate(widths)]
     old = ops.ACT_FP8
     ops.ACT_FP8 = True
     try:
@@ -644,11 +649,11 @@ def test_fp8_activation_qkv_and_swiglu_equal_separate_calls():
     assert torch.equal(sw, ops.linear(x, ws[2], None, POSTS["mul"], g, flags=_lib.FLAG_ACT_FP8))
     from tpp_pytorch_extension._lib import TppxError
     Lb = _lib.lib()
-    y = torch.empty(M, 512, dtype=torch.bfloat16, device="cuda")
+    y = torch.empty(M, widths[0], dtype=torch.bfloat16, device="cuda")
     qn, sn = ws[0].native()
     with pytest.raises(TppxError):  # no workspace for the quantised activations
         _lib.check(Lb.tppx_linear_mxfp4(x.data_ptr(), qn.data_ptr(), sn.data_ptr(), None, None, None, y.data_ptr(),
-                                        M, 512, K, 0, 1.0, _lib.FLAG_ACT_FP8, None, 0, _lib.stream_of(x)))
+                                        M, widths[0], K, 0, 1.0, _lib.FLAG_ACT_FP8, None, 0, _lib.stream_of(x)))
 
 
 def test_split_launches_overlapping_on_two_streams():

@@ -292,6 +292,10 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     }
     if (!dual)
       return check_hip(launch_tiled_mxfp4_fp8_group(t, n_segs, stream), who);
+    if (env_int("TPPX_TILED_DUAL_FUSED", 1) != 0) { // both projections per workgroup, silu(gate) * up in the epilogue
+      t[0].post_op = t[1].post_op = TPPX_POST_NONE;
+      return check_hip(launch_tiled_mxfp4_fp8_group(t, 2, stream, true), who);
+    }
     {
       // gate and up as ONE grid when that fills the last round of workgroups better than two launches and the
       // workspace has room for the gate tile behind the quantised activations (as in the bf16-activation path below)

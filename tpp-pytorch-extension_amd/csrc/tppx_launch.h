@@ -94,7 +94,7 @@ bool tiled_mxfp4_takes_groups(const TiledParams& p);
 // dual: the gate/up pair (t[0] = gate, t[1] = up) with silu(gate) * up formed in the launch and written to t[1].y
 hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream, bool dual = false);
 hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream);
-hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t stream);
+hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t stream, bool dual = false);
 bool tiled_qint8_takes_groups(const TiledParams& p);
 hipError_t launch_tiled_qint8_group(const TiledParams* t, int n, hipStream_t stream);
 // y[i] = bf16( silu(gate[i]) * y[i] ) with the rounding points of SiluPostOp followed by MulPostOp; n % 8 == 0

@@ -900,7 +900,9 @@ struct Fp8Geom {
   static constexpr int LPS = MT / 2 + 2 + 1;        // loads per wave and stage: A halves, weight tiles, one of scales
 };
 
-template <int MT>
+// DUAL: the gate/up pair as in big_mxfp4_kernel: 128 output channels per workgroup, the 16 weight tiles of a stage are
+// 4 x (2 gate tiles, the 2 up tiles of the same channels), one group per wave column; silu(gate) * up in the epilogue.
+template <int MT, bool DUAL>
 __global__ void __launch_bounds__(512)
 big_fp8_kernel(const BigParams P) {
   using G = Fp8Geom<MT>;
@@ -914,16 +916,21 @@ big_fp8_kernel(const BigParams P) {
   tile_of_block(MB, P.nb0[P.n_seg], bm, bn);
   TiledParams p = P.seg[0];
   int nb_first = 0;
+  if (!DUAL) {
 #pragma unroll
-  for (int i = 1; i < TPPX_MAX_SEGS; i++)
-    if (i < P.n_seg && bn >= P.nb0[i]) {
-      p = P.seg[i];
-      nb_first = P.nb0[i];
-    }
+    for (int i = 1; i < TPPX_MAX_SEGS; i++)
+      if (i < P.n_seg && bn >= P.nb0[i]) {
+        p = P.seg[i];
+        nb_first = P.nb0[i];
+      }
+  }
   bn -= nb_first;
   const int KT = p.K >> 7;
   const int m_wg = bm * (MT * 32);
-  const int tile_base = bn * 16 + wn * 4;
+  const int tile_base = DUAL ? bn * 8 + wn * 2 : bn * 16 + wn * 4;
+  // weight tile behind slot t (0..15) of a stage, and whether it is the up projection's (DUAL)
+  auto slot_tile = [&](int t) { return DUAL ? bn * 8 + (t >> 2) * 2 + (t & 1) : bn * 16 + t; };
+  auto slot_up = [&](int t) { return DUAL && (t & 2) != 0; };
   const int Q = (p.M + 63) >> 6; // 64-row groups of the quantised activations (rows padded to 64)
 
   // this wave's share of a stage: MT/2 activation half tiles, 2 weight tiles, one 256-byte piece of scales
@@ -938,7 +945,8 @@ big_fp8_kernel(const BigParams P) {
   const char* b_src[2];
 #pragma unroll
   for (int i = 0; i < 2; i++)
-    b_src[i] = qwb + ((size_t)min(bn * 16 + wave * 2 + i, p.tiles - 1) * KT) * 1024 + (size_t)lane * 16;
+    b_src[i] = (slot_up(wave * 2 + i) ? reinterpret_cast<const char*>(P.seg[1].qw) : qwb) +
+               ((size_t)min(slot_tile(wave * 2 + i), p.tiles - 1) * KT) * 1024 + (size_t)lane * 16;
   const char* s_src;
   int s_dst, s_stride;
   if (wave < MT / 2) { // activation scales of 64-row group `wave`: [Q][KT][64 lanes][4 row tiles]
@@ -949,7 +957,8 @@ big_fp8_kernel(const BigParams P) {
     int i = wave - MT / 2;
     if (i >= 4)
       i -= 2; // 128-row form: waves 6, 7 repeat what 4, 5 fetch, so that every wave issues LPS loads per stage
-    s_src = reinterpret_cast<const char*>(p.sw) + (size_t)min(bn * 16 + i * 4 + (lane >> 4), p.tiles - 1) * KT * 64 +
+    const int t = i * 4 + (lane >> 4);
+    s_src = reinterpret_cast<const char*>(slot_up(t) ? P.seg[1].sw : p.sw) + (size_t)min(slot_tile(t), p.tiles - 1) * KT * 64 +
             (size_t)(lane & 15) * 4;
     s_dst = G::SB_OFF + i * 256;
     s_stride = 64;
@@ -1050,7 +1059,11 @@ big_fp8_kernel(const BigParams P) {
   for (; ks < KT; ks++)
     step(std::false_type{}, ks);
   __syncthreads(); // every wave has left the main loop: LDS is free for the epilogue staging
-  big_epilogue<MT>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
+  if (DUAL)
+    big_epilogue_dual<MT>(p, P.seg[1], acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16),
+                          tile_base);
+  else
+    big_epilogue<MT>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
 }
 
 // cost of a full round of 128 x 512 workgroups relative to one of 256 x 256 (measured)
@@ -1147,7 +1160,21 @@ hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t str
 }
 
 // MXFP4 weights x MXFP8 activations (t[i].xq = quantised activations in operand order, t[i].sa = their scale bytes)
-hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t stream) {
+template <int MT, bool DUAL>
+static hipError_t fp8_launch(const BigParams& P, int wgs, hipStream_t stream) {
+  const size_t ep = 8 * 64 * EP_LD * sizeof(float); // epilogue staging
+  const size_t lds = std::max(ep, (size_t)Fp8Geom<MT>::NB * Fp8Geom<MT>::STAGE);
+  TPPX_PLAN_ONLY((big_fp8_kernel<MT, DUAL>), dim3(wgs), dim3(512), lds);
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_fp8_kernel<MT, DUAL>), lds); e != hipSuccess)
+    return e;
+  big_fp8_kernel<MT, DUAL><<<dim3(wgs), dim3(512), lds, stream>>>(P);
+  return hipGetLastError();
+}
+
+// dual: the gate/up pair (t[0] = gate, t[1] = up, equal shapes); silu(gate) * up goes to t[1].y
+hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t stream, bool dual) {
+  if (dual && (n != 2 || t[0].tiles != t[1].tiles || t[0].K != t[1].K || t[0].M != t[1].M || t[0].xq != t[1].xq))
+    return hipErrorInvalidValue;
   BigParams P;
   memset(&P, 0, sizeof(P));
   int nb = 0;
@@ -1156,12 +1183,13 @@ hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t
     P.nb0[i] = nb;
     nb += (t[i].tiles + 15) / 16;
   }
+  if (dual) {
+    nb = (t[0].tiles + 7) / 8; // 128 output channels (gate and up of each) per workgroup
+    P.nb0[1] = nb;
+  }
   for (int i = n; i <= TPPX_MAX_SEGS; i++)
     P.nb0[i] = nb;
   P.n_seg = n;
-  const size_t ep = 8 * 64 * EP_LD * sizeof(float); // epilogue staging
-  const size_t lds8 = std::max(ep, (size_t)Fp8Geom<8>::NB * Fp8Geom<8>::STAGE);
-  const size_t lds4 = std::max(ep, (size_t)Fp8Geom<4>::NB * Fp8Geom<4>::STAGE);
   // 256-row tiles unless 128-row ones fill the last round of workgroups (256 CUs, one workgroup each) better
   const int MB8 = (t[0].M + 255) / 256, MB4 = (t[0].M + 127) / 128;
   auto rounds = [](int wgs) { return (wgs + 255) / 256; };
@@ -1170,18 +1198,9 @@ hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t
   const int env_mt = env_int("TPPX_FP8_BIG_MT", 0);
   if (env_mt == 4 || env_mt == 8)
     mt = env_mt;
-  if (mt == 4) {
-    TPPX_PLAN_ONLY(big_fp8_kernel<4>, dim3(MB4 * nb), dim3(512), lds4);
-    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_fp8_kernel<4>), lds4); e != hipSuccess)
-      return e;
-    big_fp8_kernel<4><<<dim3(MB4 * nb), dim3(512), lds4, stream>>>(P);
-  } else {
-    TPPX_PLAN_ONLY(big_fp8_kernel<8>, dim3(MB8 * nb), dim3(512), lds8);
-    if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_fp8_kernel<8>), lds8); e != hipSuccess)
-      return e;
-    big_fp8_kernel<8><<<dim3(MB8 * nb), dim3(512), lds8, stream>>>(P);
-  }
-  return hipGetLastError();
+  if (mt == 4)
+    return dual ? fp8_launch<4, true>(P, MB4 * nb, stream) : fp8_launch<4, false>(P, MB4 * nb, stream);
+  return dual ? fp8_launch<8, true>(P, MB8 * nb, stream) : fp8_launch<8, false>(P, MB8 * nb, stream);
 }
 
 hipError_t launch_tiled_mxfp4(const TiledParams& p, hipStream_t stream) {
