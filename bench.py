@@ -603,7 +603,7 @@ def leg_cfg4(torch, _ops, args, pfmt="mxfp4", fp8=False, cpu=True):
              2.0 * M * 10240 * H, group_plan(L, pfmt, [H, 1024, 1024], M, H, 0, flags, wsb(H))),
             ("o M=2048 N=8192 K=8192", lambda st: torch.ops.tpp_llm.fc_add(x, wo, empty, res, 1.0),
              2.0 * M * H * H, kernel_plan(L, pfmt, M, H, H, 256, flags, wsb(H))),
-            ("gate/up M=2048 N=2x28672 K=8192 " + ("(silu*mul in the epilogue)" if pfmt == "mxfp4" and not fp8 else "(+ silu*mul pass)" if fp8 else "(fc_silu, then fc_mul)"), lambda st: _ops.swiglu_gate_up(x, wg, wu),
+            ("gate/up M=2048 N=2x28672 K=8192 " + ("(silu*mul in the epilogue)" if pfmt == "mxfp4" else "(fc_silu, then fc_mul)"), lambda st: _ops.swiglu_gate_up(x, wg, wu),
              4.0 * M * I * H, (group_plan(L, pfmt, [I, I], M, H, 1, flags, max(wsb(H), 2 * M * I + wsb(H)))
                                if pfmt == "mxfp4" else kernel_plan(L, pfmt, M, I, H, 256, flags, wsb(H)))),
             ("down M=2048 N=8192 K=28672", lambda st: torch.ops.tpp_llm.fc_add(inter, wd, empty, res, 1.0),
