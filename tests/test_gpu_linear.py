@@ -351,6 +351,29 @@ def test_k_split_across_workgroups(fmt, M, N):
         assert torch.equal(o, first)
 
 
+@pytest.mark.parametrize("split", [True, False])
+@pytest.mark.parametrize("M,N,K", [(5, 4096, 11008), (16, 4096, 11008), (9, 2048, 16384), (16, 4096, 8192)])
+def test_mxfp4_few_rows_long_k_split_across_workgroups(M, N, K, split, monkeypatch):
+    """5..16 rows, at most 256 channel tiles and a K too long for one workgroup's staging: the LDS-staged kernel with
+    K in 4 parts across workgroups of 4 channel tiles (21/22 K tiles per part at K = 11008, 1 or 2 per wave), partial
+    sums through the workspace, the last workgroup to arrive finishes -- or (TPPX_MXFP4_XL_SPLIT=0) the tile-by-tile
+    kernel.  Against the oracle; the row sums of squares the finishing workgroup leaves equal the sums over the output
+    bits; repeated launches give the same bits."""
+    monkeypatch.setenv("TPPX_MXFP4_XL_SPLIT", "1" if split else "0")
+    ops = _ops()
+    y, ref, s, ctx = _run("mxfp4", M, N, K, "add", True, 7500 + M)
+    qw, q_or, s_or, x, bias, in1, in2, scale = ctx
+    xs, b, r = x.cuda(), bias.cuda(), in1.cuda()
+    tab = torch.full((16, 256), 3.0, dtype=torch.float32, device="cuda")  # stale contents must not survive
+    outs = [ops.fc_add(xs, qw, b, r, scale, row_sumsq=tab) for _ in range(20)]
+    torch.cuda.synchronize()
+    for o in outs:
+        assert torch.equal(o, y)
+    want = (y.double() ** 2).sum(-1).cpu().numpy()
+    got = tab[:M].double().sum(-1).cpu().numpy()
+    assert np.allclose(got, want, rtol=1e-5), (got, want)
+
+
 def test_prefill_qint8_qkv_one_launch_equals_separate():
     """QINT8, enough rows for the large-M kernel: fused q/k/v share one launch (ragged channel blocks: 544, 128 and
     256 channels) and give the bits of the single-GEMM calls, which match the oracle."""

@@ -385,6 +385,17 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     // the 4 rows kept; otherwise the tile-by-tile kernel with one row group (measured at K = 11008, N = 4096:
     // 1 row 8.8 -> 7.7 us, 16 rows 14.7 -> 11.7 us against operands read straight from global memory).
     const bool x4 = M <= 4 && p.units <= 128;
+    // 5..16 rows, few channel tiles (N = 4096 at K = 11008, the Llama down-projection): the LDS-staged kernel with K
+    // in 4 parts across workgroups that own 4 channel tiles each -- the same number of workgroups, every part short
+    // enough for the staging, 16 KiB of partial sums per workgroup through the workspace.
+    if (!x4 && !dual && n_segs == 1 && env_int("TPPX_MXFP4_XL_SPLIT", 1) == 1 && p.total_tiles % 4 == 0 &&
+        p.total_tiles <= 256 && (p.units + 3) / 4 <= 32 && p.units >= 64 &&
+        ws && ws_bytes >= (int64_t)4 * p.total_tiles * 256 * (int64_t)sizeof(float)) {
+      set_groups(p, 4, false);
+      p.S = 4;
+      p.part = (float*)ws;
+      return check_hip(launch_skinny_mxfp4_xl(p, 4, false, stream), who);
+    }
     int nt = 1;
     for (; nt < 3; nt++) {
       set_groups(p, nt, dual);

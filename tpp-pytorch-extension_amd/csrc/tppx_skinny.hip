@@ -187,11 +187,48 @@ struct SkEpilogue {
       }
   }
 
+  // Row sums of squares of this workgroup's outputs (MG == 1): ov[i] = the rounded output of slot i as a float, 0
+  // where nothing was stored.  Called by every thread of the workgroup; entry [row][blockIdx.x] of the [16][256]
+  // table gets the sum over this workgroup's channel tiles in a fixed order, and workgroup 0 zeroes the slots past
+  // the grid.
+  __device__ __forceinline__ void leave_row_sums(const float (&ov)[MAXE], float* sumsq, int M) {
+    __shared__ float sq_s[16 * NACC];
+#pragma unroll
+    for (int i = 0; i < MAXE; i++) {
+      const int e = threadIdx.x + i * blockDim.x;
+      if (e < OUT) { // wave-uniform: e < OUT holds for whole waves
+        float sq = ov[i] * ov[i];
+        // the 16 lanes of a DPP row hold the 16 channels of one (row, tile) pair
+        sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0xB1, 0xf, 0xf, true));
+        sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0x4E, 0xf, 0xf, true));
+        sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0x141, 0xf, 0xf, true));
+        sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0x140, 0xf, 0xf, true));
+        if ((e & 15) == 0)
+          sq_s[(((e & 63) >> 4) * 4 + ((e >> 6) & 3)) * NACC + (e >> 8)] = sq; // [row][tile]
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < 16 && (int)threadIdx.x < M) {
+      float tot = 0.f;
+#pragma unroll
+      for (int a = 0; a < NACC; a++)
+        tot += sq_s[threadIdx.x * NACC + a];
+      sumsq[threadIdx.x * 256 + blockIdx.x] = tot;
+    }
+    if (blockIdx.x == 0)
+      for (int j = (int)gridDim.x + (int)threadIdx.x; j < 256 * min(M, 16); j += (int)blockDim.x) {
+        const int row = j >> 8, part = j & 255; // slots gridDim.x .. 255 of every row (j walks a superset)
+        if (part >= (int)gridDim.x)
+          sumsq[row * 256 + part] = 0.f;
+      }
+  }
+
   // K split across workgroups (blockIdx.z = part).  Every workgroup leaves its sums in the workspace,
   // [part][block row][tile][row group][r * 64 + lane] floats, and takes a ticket; the workgroup that arrives last
   // adds the parts in part order (the same sums whichever workgroup that is) and runs the epilogue.  Nobody waits.
+  // sumsq (MG == 1): the finishing workgroup also leaves the row sums of squares, see leave_row_sums().
   __device__ __forceinline__ void finish_split(const DecodeParams& p, const DecodeSeg& sg, f32x4 (&acc)[NACC][MG],
-                                               float* red, int ltile0, int stride = ELEMS) {
+                                               float* red, int ltile0, int stride = ELEMS, float* sumsq = nullptr) {
     static_assert(!DUAL, "the gate/up pair is not split");
     __shared__ int arrived_last;
     settle();
@@ -245,16 +282,23 @@ struct SkEpilogue {
           pv[i][k] = __hip_atomic_load(part + k * part_stride + threadIdx.x + i * blockDim.x, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
       }
+    float ov[MAXE];
 #pragma unroll
-    for (int i = 0; i < MAXE; i++)
+    for (int i = 0; i < MAXE; i++) {
+      ov[i] = 0.f;
       if (off[i] >= 0) {
         float v = 0.f;
 #pragma unroll
         for (int k = 0; k < 4; k++)
           if (k < p.S)
             v += k == (int)blockIdx.z ? own[i] : pv[i][k];
-        sg.y[off[i]] = (uint16_t)apply_post_bits(v + bf16_bits_to_f32(bias[i]), sg.post_op, in1[i], in2[i], sg.post_scale);
+        const uint32_t out = apply_post_bits(v + bf16_bits_to_f32(bias[i]), sg.post_op, in1[i], in2[i], sg.post_scale);
+        sg.y[off[i]] = (uint16_t)out;
+        ov[i] = bf16_bits_to_f32(out & 0xffffu);
       }
+    }
+    if (MG == 1 && sumsq) // uniform
+      leave_row_sums(ov, sumsq, p.M);
   }
 
   // stride = floats between the regions of two waves (>= ELEMS).  sumsq (MG == 1, not the gate/up pair): also
@@ -262,7 +306,6 @@ struct SkEpilogue {
   // [16][256] table (workgroup 0 zeroes the slots past the grid), added in a fixed order.
   __device__ __forceinline__ void finish(const DecodeSeg& sg, f32x4 (&acc)[NACC][MG], float* red, int stride = ELEMS,
                                          float* sumsq = nullptr, int M = 0) {
-    __shared__ float sq_s[16 * NACC];
     settle();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int W = blockDim.x >> 6;
@@ -275,9 +318,11 @@ struct SkEpilogue {
         for (int r = 0; r < 4; r++)
           mine[(a * MG + mg) * 256 + r * 64 + lane] = acc[a][mg][r];
     __syncthreads();
+    float ov[MAXE];
 #pragma unroll
     for (int i = 0; i < MAXE; i++) {
       const int e = threadIdx.x + i * blockDim.x;
+      ov[i] = 0.f;
       if (e < OUT) {
         float v = 0.f, v2 = 0.f;
         for (int w = 0; w < W; w++)
@@ -294,36 +339,12 @@ struct SkEpilogue {
             out = apply_post_bits(v + bf16_bits_to_f32(bias[i]), sg.post_op, in1[i], in2[i], sg.post_scale);
           }
           sg.y[off[i]] = (uint16_t)out;
-        }
-        if (!DUAL && MG == 1 && sumsq) { // wave-uniform: e < OUT holds for whole waves
-          const float ov = off[i] >= 0 ? bf16_bits_to_f32(out & 0xffffu) : 0.f;
-          float sq = ov * ov;
-          // the 16 lanes of a DPP row hold the 16 channels of one (row, tile) pair
-          sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0xB1, 0xf, 0xf, true));
-          sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0x4E, 0xf, 0xf, true));
-          sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0x141, 0xf, 0xf, true));
-          sq += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sq), 0x140, 0xf, 0xf, true));
-          if ((e & 15) == 0)
-            sq_s[(((e & 63) >> 4) * 4 + ((e >> 6) & 3)) * NACC + (e >> 8)] = sq; // [row][tile]
+          ov[i] = bf16_bits_to_f32(out & 0xffffu);
         }
       }
     }
-    if (!DUAL && MG == 1 && sumsq) {
-      __syncthreads();
-      if (threadIdx.x < 16 && (int)threadIdx.x < M) {
-        float tot = 0.f;
-#pragma unroll
-        for (int a = 0; a < NACC; a++)
-          tot += sq_s[threadIdx.x * NACC + a];
-        sumsq[threadIdx.x * 256 + blockIdx.x] = tot;
-      }
-      if (blockIdx.x == 0)
-        for (int j = (int)gridDim.x + (int)threadIdx.x; j < 256 * min(M, 16); j += (int)blockDim.x) {
-          const int row = j >> 8, part = j & 255; // slots gridDim.x .. 255 of every row (j walks a superset)
-          if (part >= (int)gridDim.x)
-            sumsq[row * 256 + part] = 0.f;
-        }
-    }
+    if (!DUAL && MG == 1 && sumsq) // uniform
+      leave_row_sums(ov, sumsq, M);
   }
 };
 
@@ -736,7 +757,12 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
   const DecodeSeg& sg = p.seg[seg_id];
   const int ltile0 = (grp - sg.grp0) * NT;
   const int KT = p.units;
-  const int t0 = (wave * KT) / W, t1 = ((wave + 1) * KT) / W;
+  // K parts across workgroups (blockIdx.z of p.S, finished by finish_split): only the form that takes a K too long
+  // for one workgroup's staging carries it -- a single GEMM, four channel tiles per workgroup, x as it is
+  constexpr bool KSPLIT = NT == 4 && !DUAL && XMODE == 0;
+  const int kt0 = KSPLIT ? ((int)blockIdx.z * KT) / p.S : 0;
+  const int ktn = KSPLIT ? (((int)blockIdx.z + 1) * KT) / p.S - kt0 : KT; // K tiles of this workgroup
+  const int t0 = kt0 + (wave * ktn) / W, t1 = kt0 + ((wave + 1) * ktn) / W;
   const int cht = p.cht;                       // K tiles per wave, at most
   const int wstride = max(cht * 1024, NTW * 256); // floats per wave region (x slice, later the reduction scratch)
   uint4* xs = reinterpret_cast<uint4*>(sk_lds + (size_t)wave * wstride);
@@ -978,6 +1004,12 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
     }
   }
   __syncthreads(); // every wave is done with its x region before it becomes reduction scratch
+  if constexpr (KSPLIT) {
+    if (p.S > 1) {
+      ep.finish_split(p, sg, acc, sk_lds, ltile0, wstride, p.sumsq_out);
+      return;
+    }
+  }
   ep.finish(sg, acc, sk_lds, wstride, p.sumsq_out, p.M);
 }
 
@@ -1539,9 +1571,15 @@ size_t skinny_mxfp4_xl_lds(int units, int nt, bool dual) {
 }
 
 hipError_t launch_skinny_mxfp4_xl(DecodeParams& p, int nt, bool dual, hipStream_t stream) {
-  p.cht = (p.units + 15) / 16;
-  const size_t lds = skinny_mxfp4_xl_lds(p.units, nt, dual);
-  dim3 grid(p.groups, 1);
+  // p.S > 1 (nt == 4, single GEMM, no normalisation; the caller checks): K parts across workgroups, every part staged
+  // like a whole K of its length
+  const int S = p.S > 1 ? p.S : 1;
+  const int units = (p.units + S - 1) / S;
+  p.cht = (units + 15) / 16;
+  const size_t lds = skinny_mxfp4_xl_lds(units, nt, dual);
+  dim3 grid(p.groups, 1, S);
+  if (S > 1 && (S > 4 || nt != 4 || dual || p.norm_gamma || (p.ticket0 = skinny_split_tickets((int)grid.x)) < 0))
+    return hipErrorInvalidValue;
   const bool norm = p.norm_gamma != nullptr;
   const bool few = p.M <= 4; // 4 rows x 32 chunks fit two items per lane
   const bool handed = norm && p.sumsq_in != nullptr; // row sums of squares come from the launch that wrote x
