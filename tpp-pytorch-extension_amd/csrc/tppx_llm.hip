@@ -1027,16 +1027,25 @@ extern "C" int tppx_rotary_kv_append_llama(void* q, void* k, const void* v, cons
 // shared tail of the two single-query entry points: split planning, counters, launch
 static int attn_decode_launch(const char* who, AttnParams& p, bool rot, int64_t B, int64_t Nq, int64_t Smax, void* ws,
                               int64_t ws_bytes, hipStream_t stream) {
-  // The wide kernel (128 keys per workgroup and trip) serves launches whose workgroups make few trips; the row
-  // kernel (64 keys per trip, a deeper request queue per wave) the long loops of larger batches.  Measured at batch 1,
-  // 32 heads, 2100 keys: about one workgroup per CU is best (more splits mean more states to merge and more
-  // launches of the same few hundred KB); the row kernel wants about two per CU.  At most one split per trip and at
-  // most 32 (the merge holds every split's state in registers).
+  // The wide kernel (128 keys per workgroup and trip) is the default: measured against the row kernel (64 keys per
+  // trip) over 32 heads, it is faster at every batch size from 1 to 64 and context from 100 to 8000 keys once its
+  // workgroups make about two trips each (batch 16, 2048 keys: 3660 -> 3739 tokens/s for the whole decode step;
+  // batch 1, 8000 keys: 29.1 us with the row kernel, 32.1 with 9 wide splits per head, 27.0 with 16).  Splits per
+  // head: two trips per workgroup, but no fewer workgroups than 288 (about one per CU: fewer leave CUs idle) and no
+  // more than 512 (more splits mean more states to merge); the row kernel (TPPX_ATTN_WIDE=0) wants about two
+  // workgroups per CU.  At most one split per trip and at most 32 (the merge holds every split's state in registers).
   const int wide_env = (int)env_int("TPPX_ATTN_WIDE", -1);
   const int64_t target_env = env_int("TPPX_ATTN_TARGET_WGS", 0);
-  const int64_t splits_wide = ((target_env > 0 ? target_env : 288) + B * Nq - 1) / (B * Nq);
-  const bool wide = wide_env >= 0 ? wide_env != 0 : (Smax + ATTN_WIDE_KEYS - 1) / ATTN_WIDE_KEYS <= 4 * splits_wide;
-  int64_t splits = wide ? splits_wide : ((target_env > 0 ? target_env : 512) + B * Nq - 1) / (B * Nq);
+  const bool wide = wide_env != 0;
+  const int64_t heads = B * Nq;
+  int64_t splits;
+  if (target_env > 0 || !wide) {
+    splits = ((target_env > 0 ? target_env : 512) + heads - 1) / heads;
+  } else {
+    const int64_t lo = (288 + heads - 1) / heads, hi = (512 + heads - 1) / heads;
+    splits = ((Smax + ATTN_WIDE_KEYS - 1) / ATTN_WIDE_KEYS + 1) / 2;
+    splits = splits < lo ? lo : splits > hi ? hi : splits;
+  }
   const int64_t trip_keys = wide ? ATTN_WIDE_KEYS : 64;
   const int64_t max_by_len = (Smax + trip_keys - 1) / trip_keys;
   if (splits > max_by_len)
