@@ -489,6 +489,21 @@ int tppx_qkv_linear_mxfp4(const void* x, const void* row_sumsq, const void* gamm
                           int64_t K, int64_t n1, int64_t n2, int flags,
                           tppx_stream_t stream);
 
+/* Greedy step of a generation loop (what transformers' generate() does between
+ * two forward passes when examples/llm/run_generation.py:420 runs with
+ * --greedy: torch.argmax over the logits, the embedding lookup of the chosen
+ * token) as one launch, so that a decode step replayed as a graph ends in a
+ * single small kernel:
+ *   tokens[b] (int64) = the first maximal index of logits[b][0..V) (bf16; a NaN
+ *                       counts as maximal, like torch.argmax)
+ *   pos[b] (int64)   += 1                       (pos != NULL)
+ *   seq_len[0] (i32) += 1                       (seq_len != NULL)
+ *   h_next[b][:]      = embed[tokens[b]][:]     (h_next != NULL; bf16 [*][hidden])
+ * V % 8 == 0, hidden % 8 == 0. */
+int tppx_greedy_next(const void* logits, int64_t B, int64_t V, const void* embed,
+                     int64_t hidden, void* tokens, void* pos, void* seq_len,
+                     void* h_next, tppx_stream_t stream);
+
 /* ---- launch plans ------------------------------------------------------- */
 
 /* No counterpart in the reference.  Writes into buf, one line per kernel, what

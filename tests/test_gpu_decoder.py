@@ -436,6 +436,38 @@ def test_greedy_decode_graph_equals_eager():
         model.greedy_decode(tok, model.new_cache(3, 250, 300), 8)
 
 
+@pytest.mark.parametrize("B,V,hidden", [(1, 32000, 4096), (3, 1024, 512), (16, 32000, 4096), (2, 8, 8)])
+def test_greedy_next_token_step(B, V, hidden):
+    """tppx_greedy_next against torch: argmax (first maximal index, ties and a NaN row included), the embedding row of
+    the chosen token, position and cache-length counters moved on by one."""
+    _llm()
+    from tpp_pytorch_extension import _lib
+    g = torch.Generator().manual_seed(40 + B)
+    logits = torch.randn((B, V), generator=g).to(torch.bfloat16)
+    logits[0, V // 2] = logits[0].max()          # a tie: the earlier index wins
+    logits[0, 3] = logits[0].max()
+    if B > 1:
+        logits[1, V - 1] = float("nan")          # torch.argmax takes a NaN for the maximum
+    embed = torch.randn((V, hidden), generator=g).to(torch.bfloat16).cuda()
+    lg = logits.cuda()
+    tokens = torch.full((B,), -1, dtype=torch.int64, device="cuda")
+    pos = torch.arange(B, dtype=torch.int64, device="cuda").view(B, 1) + 7
+    seq = torch.tensor([41], dtype=torch.int32, device="cuda")
+    h = torch.zeros((B, 1, hidden), dtype=torch.bfloat16, device="cuda")
+    L = _lib.lib()
+    _lib.check(L.tppx_greedy_next(lg.data_ptr(), B, V, embed.data_ptr(), hidden, tokens.data_ptr(), pos.data_ptr(),
+                                  seq.data_ptr(), h.data_ptr(), _lib.stream_of(lg)))
+    want = lg.argmax(dim=-1)
+    assert torch.equal(tokens, want), (tokens, want)
+    assert torch.equal(h.view(B, hidden), embed.index_select(0, want))
+    assert torch.equal(pos.view(-1).cpu(), torch.arange(B) + 8) and seq.item() == 42
+    # only the tokens when the other outputs are not asked for
+    t2 = torch.empty_like(tokens)
+    _lib.check(L.tppx_greedy_next(lg.data_ptr(), B, V, None, 0, t2.data_ptr(), None, None, None, _lib.stream_of(lg)))
+    assert torch.equal(t2, want) and seq.item() == 42
+    assert L.tppx_greedy_next(lg.data_ptr(), B, V + 1, None, 0, t2.data_ptr(), None, None, None, None) == _lib.ESHAPE
+
+
 @pytest.mark.parametrize("M", [1, 5, 16])
 @pytest.mark.parametrize("K", [512, 4096])
 def test_rms_norm_fused_into_gemms(M, K, monkeypatch):

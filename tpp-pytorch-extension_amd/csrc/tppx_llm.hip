@@ -957,9 +957,89 @@ attn_prefill_kernel(const AttnPrefillParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Greedy step of a generation loop: next token = argmax of the row's logits (the first maximal index; a NaN counts
+// as maximal, as torch.argmax has it), stored as int64; the position of the row moves on by one; the token's
+// embedding row becomes the row of the next step's hidden states; workgroup 0 moves the cache length on by one.
+// One workgroup of 1024 threads per row: 16-byte loads, (value, index) maxima through DPP-free LDS steps.
+// ---------------------------------------------------------------------------
+struct GreedyKey {
+  float v;
+  int i;
+};
+__device__ __forceinline__ bool greedy_before(float v, int i, float bv, int bi) {
+  // total order: NaN above everything, then larger value, then smaller index
+  const bool vn = v != v, bn = bv != bv;
+  if (vn != bn)
+    return vn;
+  if (!vn && v != bv)
+    return v > bv;
+  return i < bi;
+}
+
+__global__ void __launch_bounds__(1024)
+greedy_next_kernel(const uint16_t* __restrict__ logits, int V, const uint16_t* __restrict__ embed, int hidden,
+                   int64_t* __restrict__ tokens, int64_t* __restrict__ pos, int32_t* __restrict__ seq_len,
+                   uint16_t* __restrict__ h_next) {
+  __shared__ float sv[1024];
+  __shared__ int si[1024];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const uint16_t* row = logits + (size_t)b * V;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int c = tid * 8; c < V; c += 1024 * 8) { // V % 8 == 0
+    const uint4 raw = *reinterpret_cast<const uint4*>(row + c);
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float v = bf16_bits_to_f32((w[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+      if (greedy_before(v, c + e, bv, bi)) {
+        bv = v;
+        bi = c + e;
+      }
+    }
+  }
+  sv[tid] = bv;
+  si[tid] = bi;
+  __syncthreads();
+  for (int step = 512; step > 0; step >>= 1) {
+    if (tid < step && greedy_before(sv[tid + step], si[tid + step], sv[tid], si[tid])) {
+      sv[tid] = sv[tid + step];
+      si[tid] = si[tid + step];
+    }
+    __syncthreads();
+  }
+  const int tok = si[0];
+  if (tid == 0) {
+    tokens[b] = tok;
+    if (pos)
+      pos[b] += 1;
+    if (seq_len && b == 0)
+      seq_len[0] += 1;
+  }
+  if (h_next)
+    for (int c = tid * 8; c < hidden; c += 1024 * 8) // hidden % 8 == 0
+      *reinterpret_cast<uint4*>(h_next + (size_t)b * hidden + c) = *reinterpret_cast<const uint4*>(embed + (size_t)tok * hidden + c);
+}
+
 } // namespace tppx
 
 using namespace tppx;
+
+extern "C" int tppx_greedy_next(const void* logits, int64_t B, int64_t V, const void* embed, int64_t hidden, void* tokens,
+                                void* pos, void* seq_len, void* h_next, tppx_stream_t stream) {
+  const char* who = "tppx_greedy_next";
+  TPPX_REQUIRE(logits && tokens, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(aligned16(logits), TPPX_EINVAL, "%s: logits not 16-byte aligned", who);
+  TPPX_REQUIRE(B > 0 && B < (1 << 16) && V > 0 && V % 8 == 0 && V < ((int64_t)1 << 31), TPPX_ESHAPE,
+               "%s: bad shape B=%ld V=%ld (V must be a multiple of 8)", who, (long)B, (long)V);
+  TPPX_REQUIRE(!h_next || (embed && aligned16(embed) && aligned16(h_next) && hidden > 0 && hidden % 8 == 0), TPPX_EINVAL,
+               "%s: the next hidden states need a 16-byte aligned embedding table and output with hidden %% 8 == 0", who);
+  greedy_next_kernel<<<dim3((unsigned)B), dim3(1024), 0, (hipStream_t)stream>>>(
+      (const uint16_t*)logits, (int)V, (const uint16_t*)embed, (int)hidden, (int64_t*)tokens, (int64_t*)pos, (int32_t*)seq_len,
+      (uint16_t*)h_next);
+  return check_hip(hipGetLastError(), who);
+}
 
 extern "C" int tppx_rms_norm(const void* x, const void* gamma, int gamma_dtype, void* y, int64_t rows, int64_t K,
                              float eps, tppx_stream_t stream) {

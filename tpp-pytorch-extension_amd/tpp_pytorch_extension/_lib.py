@@ -80,6 +80,7 @@ SIGNATURES = {
                                     _i64, _i64, _vp],
     "tppx_linear_qint8_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "tppx_linear_mxfp4_int8": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _f32, _vp],
+    "tppx_greedy_next": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp],
     "tppx_qkv_linear_mxfp4": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _vp],
     "tppx_attn_decode": [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp],
     "tppx_attn_decode_rotary": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp],

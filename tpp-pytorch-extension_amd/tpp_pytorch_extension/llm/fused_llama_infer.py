@@ -36,6 +36,9 @@ rms_norm = _ops.rms_norm  # llama_rms_norm (fused_llm_infer.cpp:337-363)
 
 # decode steps: rotary embedding + cache append inside the attention launch (TPPX_FUSE_ROTARY=0: separate launch)
 FUSE_ROTARY = os.environ.get("TPPX_FUSE_ROTARY", "1") == "1"
+# Greedy decoding: argmax, the counters and the next token's embedding row in one launch at the end of a decode step
+# (tppx_greedy_next) instead of torch's argmax / copy / add / index_select kernels.  TPPX_FUSE_GREEDY=0 keeps those.
+FUSE_GREEDY = os.environ.get("TPPX_FUSE_GREEDY", "1") == "1"
 
 
 def apply_rotary_pos_emb_llama(t_in, t_emb_pos, t_pos, N, H):
@@ -320,6 +323,28 @@ class LlamaDecoder:
         logits = _ops.fc_plain(h, self.lm_head, None)
         return logits.view(logits.shape[0], -1).argmax(dim=-1)
 
+    def _step_greedy(self, h, cur, pos, cache, advance=True):
+        """One decode step that ends in tppx_greedy_next: h bf16 [B][1][hidden] holds the embeddings of the current
+        tokens; afterwards cur (i64 [B]) holds the next tokens and, with advance, pos (i64 [B][1]) and the cache's
+        device counter have moved on by one and h holds the next tokens' embeddings -- everything a replayed graph
+        needs for its next step.  Without advance nothing but cur changes (the warm-up in front of a capture)."""
+        x = h
+        for layer in self.layers:
+            x = layer.forward([x, None, pos], cache)[0]
+        x = rms_norm(x, self.norm_w, self.eps)
+        logits = _ops.fc_plain(x, self.lm_head, None)
+        B = logits.shape[0]
+        logits = logits.view(B, -1)
+        _lib.check(_lib.lib().tppx_greedy_next(
+            logits.data_ptr(), B, logits.shape[1], self.embed.data_ptr(), self.hidden, cur.data_ptr(),
+            pos.data_ptr() if advance else None, cache.seq_len_dev.data_ptr() if advance else None,
+            h.data_ptr() if advance else None, _lib.stream_of(logits)))
+        return cur
+
+    def _greedy_fusable(self, B):
+        return (FUSE_GREEDY and self.vocab % 8 == 0 and self.hidden % 8 == 0 and self.embed.is_contiguous()
+                and self.embed.dtype == torch.bfloat16 and B < 65536)
+
     def prefill(self, prompt, cache, mask=None):
         """prompt i64 [B][S] (device) on top of whatever the cache holds -> next tokens i64 [B]; advances the cache
         by S.  mask: additive bf16 [B][keys] over cache positions (TppCache.align_and_invert_mask) or None."""
@@ -363,14 +388,22 @@ class LlamaDecoder:
         B = tokens.shape[0]
         cur = tokens.clone()
         pos = torch.full((B, 1), cache.get_seq_length(), dtype=torch.int64, device=self.device)
-        self.step(cur, pos, cache)
+        fused = self._greedy_fusable(B)
+        if fused:
+            h = self.embed.index_select(0, cur).unsqueeze(1).contiguous()
+            self._step_greedy(h, cur.clone(), pos, cache, advance=False)
+        else:
+            self.step(cur, pos, cache)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            nxt = self.step(cur, pos, cache)
-            cur.copy_(nxt)
-            pos.add_(1)
-            cache.seq_len_dev.add_(1)
+            if fused:
+                self._step_greedy(h, cur, pos, cache)
+            else:
+                nxt = self.step(cur, pos, cache)
+                cur.copy_(nxt)
+                pos.add_(1)
+                cache.seq_len_dev.add_(1)
         graph.replay()  # one untimed replay
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -387,14 +420,23 @@ class LlamaDecoder:
         pos = torch.full((B, 1), cache.get_seq_length(), dtype=torch.int64, device=self.device)
         out = torch.empty((B, n_new), dtype=torch.int64, device=self.device)
         if use_graph:
-            nxt = self.step(cur, pos, cache)  # warm-up outside capture (allocations, lazy module loads)
+            fused = self._greedy_fusable(B)
+            # warm-up outside capture (allocations, lazy module loads); it leaves the counters where they are
+            if fused:
+                h = self.embed.index_select(0, cur).unsqueeze(1).contiguous()
+                self._step_greedy(h, cur.clone(), pos, cache, advance=False)
+            else:
+                nxt = self.step(cur, pos, cache)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                nxt = self.step(cur, pos, cache)
-                cur.copy_(nxt)
-                pos.add_(1)
-                cache.seq_len_dev.add_(1)
+                if fused:
+                    self._step_greedy(h, cur, pos, cache)
+                else:
+                    nxt = self.step(cur, pos, cache)
+                    cur.copy_(nxt)
+                    pos.add_(1)
+                    cache.seq_len_dev.add_(1)
             for t in range(n_new):
                 graph.replay()
                 out[:, t].copy_(cur)
