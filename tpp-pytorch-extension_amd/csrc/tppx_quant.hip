@@ -1,6 +1,7 @@
 // Quantize / de-quantize / re-layout kernels (HBM-bound byte work, one-time per
 // weight except for the activation quantizer which runs on every QINT8 call).
 #include "tppx_common.h"
+#include "tppx_launch.h"
 
 namespace tppx {
 
@@ -387,7 +388,7 @@ quant_act_int8_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
 // Same arithmetic as the kernel above (the maximum does not depend on the order).
 __global__ void __launch_bounds__(256)
 quant_act_int8_rows_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K, int8_t* __restrict__ xq,
-                           float* __restrict__ sa) {
+                           float* __restrict__ sa, int mt) {
   const int64_t nb = K >> 8;
   const int64_t blk = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
   const int l = threadIdx.x & 15;
@@ -415,14 +416,23 @@ quant_act_int8_rows_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
   amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0x140>{})); // row_mirror
   const float s = int8_scale_of(amax);
   const float inv = int8_inv_scale(s);
+  const int64_t m = blk / nb, b = blk - m * nb;
   if (l == 0)
-    sa[blk] = s; // [M][nb]
+    sa[mt > 0 ? b * (int64_t)mt * 16 + m : blk] = s; // [M][nb], or [nb][mt * 16] beside operand-order values
   uint32_t o[4];
 #pragma unroll
   for (int d = 0; d < 4; d++)
     o[d] = (uint32_t)(int8_q(f[4 * d], inv) & 0xff) | ((uint32_t)(int8_q(f[4 * d + 1], inv) & 0xff) << 8) |
            ((uint32_t)(int8_q(f[4 * d + 2], inv) & 0xff) << 16) | ((uint32_t)(int8_q(f[4 * d + 3], inv) & 0xff) << 24);
-  reinterpret_cast<uint4*>(xq + blk * 256)[l] = make_uint4(o[0], o[1], o[2], o[3]);
+  if (mt > 0) {
+    // operand order: the lane's 16 values are K group l % 4 of tile b * 4 + l / 4 (64 K each), row m % 16 of row
+    // tile m / 16: [tile][mt row tiles][4 K groups][16 rows][16 B]
+    const int64_t t = b * 4 + (l >> 2);
+    const int64_t slot = (t * mt + (m >> 4)) * 64 + (l & 3) * 16 + (m & 15);
+    reinterpret_cast<uint4*>(xq)[slot] = make_uint4(o[0], o[1], o[2], o[3]);
+  } else {
+    reinterpret_cast<uint4*>(xq + blk * 256)[l] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -644,10 +654,12 @@ static inline unsigned grid_for(int64_t n, int block) {
 
 hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qbs, void* xq, void* sa, int mt,
                                  hipStream_t stream) {
-  if (qbs == 256 && mt == 0 && M >= 128) {
+  // 16 lanes per (row, block) -- 32-byte reads, one 16-byte write per lane -- from 128 rows on, and for the operand-
+  // order output of the decode kernels (17..64 rows) whatever the row count; a whole wave per (row, block) otherwise
+  if (qbs == 256 && (M >= 128 || mt > 0) && env_int("TPPX_QUANT_ROWS16", 1) != 0) {
     const int64_t nt16 = M * (K / 256) * 16;
     TPPX_PLAN_ONLY(quant_act_int8_rows_kernel, dim3(grid_for(nt16, 256)), dim3(256), 0);
-    quant_act_int8_rows_kernel<<<grid_for(nt16, 256), 256, 0, stream>>>((const uint16_t*)x, M, K, (int8_t*)xq, (float*)sa);
+    quant_act_int8_rows_kernel<<<grid_for(nt16, 256), 256, 0, stream>>>((const uint16_t*)x, M, K, (int8_t*)xq, (float*)sa, mt);
     return hipGetLastError();
   }
   int64_t nthreads = M * (K / qbs) * 64;
