@@ -534,7 +534,7 @@ def test_launch_plan_names_the_kernels():
     buf = ctypes.create_string_buffer(2048)
     _lib.check(L.tppx_plan_linear_qint8(64, 11008, 4096, 256, 1, 0, 1 << 25, buf, len(buf)))
     lines = buf.value.decode().strip().splitlines()
-    assert len(lines) == 2 and "quant_act_int8_kernel" in lines[0] and "skinny_qint8_kernel<" in lines[1]
+    assert len(lines) == 2 and "quant_act_int8_rows_kernel" in lines[0] and "skinny_qint8_kernel<" in lines[1]
     _lib.check(L.tppx_plan_linear_qint8(1, 11008, 4096, 256, 1, 0, 1 << 25, buf, len(buf)))
     assert buf.value.decode().count("\n") == 1 and "skinny_qint8_fq_kernel<" in buf.value.decode()
     _lib.check(L.tppx_plan_linear_mxfp4(2048, 8192, 8192, 0, 0, buf, len(buf)))
