@@ -190,3 +190,43 @@ def test_fix_vnni_and_block_size_rule():
     assert v2[1, 0, 5, 2, 1] == t[1, 0, 2, 2, 3]  # c2'=5 -> c2=2, half 1 -> c3 = 2 + 1
     assert _ops.qint8_block_size_for(4096) == 256 and _ops.qint8_block_size_for(11008) == 256
     assert _ops.qint8_block_size_for(192) == 64 and _ops.qint8_block_size_for(384) == 128
+
+
+def test_launch_plans_of_the_baseline_shapes():
+    """Host-side planning (no GPU work): which kernel and grid the library would launch for the BASELINE shapes --
+    decode GEMMs fill one round of 256 workgroups, the prefill GEMMs get the workgroup tile whose rounds are full, the
+    q/k/v GEMM the half-size workgroups that shorten its last round."""
+    import ctypes
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    buf = ctypes.create_string_buffer(4096)
+
+    def plan(fn, *args):
+        _lib.check(fn(*args, buf, len(buf)))
+        return buf.value.decode().strip().splitlines()
+
+    ws = 1 << 25
+    # config 2: QINT8 MLP linears
+    assert "skinny_qint8_fq_kernel<3," in plan(L.tppx_plan_linear_qint8, 1, 11008, 4096, 256, 1, 0, ws)[0]
+    lines = plan(L.tppx_plan_linear_qint8, 64, 4096, 11008, 256, 1, 0, ws)
+    assert len(lines) == 2 and "quant_act_int8_rows_kernel" in lines[0]
+    assert "skinny_qint8_kernel<4, 2, 4, 8, 8, true>" in lines[1] and "grid=128x1x2" in lines[1]  # K in two parts
+    assert len(plan(L.tppx_plan_linear_qint8, 64, 4096, 11008, 256, 0, 0, ws)) == 1             # pre-quantized input
+    # config 3 / 5: MXFP4 decode
+    assert "skinny_mxfp4_x4_kernel<1, 4, false> grid=256x1x1" in plan(L.tppx_plan_linear_mxfp4, 1, 4096, 11008, 0, ws)[0]
+    assert "skinny_mxfp4_xl_kernel<4, 2, false, 0, 8> grid=64x1x4" in plan(L.tppx_plan_linear_mxfp4, 16, 4096, 11008, 0, ws)[0]
+    assert "skinny_mxfp4_mg_kernel<1, 1, false, 4, 16>" in plan(L.tppx_plan_linear_mxfp4, 16, 4096, 11008, 0, 0)[0]  # no workspace
+    assert "skinny_mxfp4_xl_kernel<1, 2, false, 0, 8> grid=256x1x1" in plan(L.tppx_plan_linear_mxfp4, 16, 4096, 4096, 0, ws)[0]
+    gate_up = (ctypes.c_int64 * 2)(11008, 11008)
+    assert "skinny_mxfp4_xl_kernel<3, 2, true, 0, 2> grid=230x1x1" in plan(L.tppx_plan_multi_linear_mxfp4, gate_up, 2, 1, 4096, 1, 0, ws)[0]
+    assert "skinny_mxfp4_mg_kernel<4, 3, true, 1, 8> grid=230x1x1" in plan(L.tppx_plan_multi_linear_mxfp4, gate_up, 2, 64, 4096, 1, 0, ws)[0]
+    # config 4: prefill at 2048 rows
+    assert "big_mxfp4_kernel<8, false, 1, 8> grid=256x1x1 block=512" in plan(L.tppx_plan_linear_mxfp4, 2048, 8192, 8192, 0, 0)[0]
+    assert "big_mxfp4_kernel<8, false, 1, 8> grid=256x1x1" in plan(L.tppx_plan_linear_mxfp4, 2048, 8192, 28672, 0, 0)[0]
+    qkv = (ctypes.c_int64 * 3)(8192, 1024, 1024)
+    assert "big_mxfp4_kernel<8, false, 1, 4> grid=640x1x1 block=256" in plan(L.tppx_plan_multi_linear_mxfp4, qkv, 3, 2048, 8192, 0, 0, 0)[0]
+    pair = (ctypes.c_int64 * 2)(28672, 28672)
+    lines = plan(L.tppx_plan_multi_linear_mxfp4, pair, 2, 2048, 8192, 1, 0, 0)
+    assert len(lines) == 1 and "big_mxfp4_kernel<8, true, 1, 8> grid=1792x1x1" in lines[0]       # silu*mul in the epilogue
+    lines = plan(L.tppx_plan_multi_linear_mxfp4, pair, 2, 2048, 8192, 1, _lib.FLAG_ACT_FP8, 1 << 28)
+    assert any("big_fp8_kernel<8, true> grid=1792x1x1" in l for l in lines), lines
