@@ -679,14 +679,14 @@ def test_fp8_activation_qkv_and_swiglu_equal_separate_calls(M, K, widths, fused,
                                         M, widths[0], K, 0, 1.0, _lib.FLAG_ACT_FP8, None, 0, _lib.stream_of(x)))
 
 
-def test_split_launches_overlapping_on_two_streams():
+def test_split_launches_from_two_threads_on_two_streams():
     """Launches that split K over workgroups (partial sums in the workspace, an arrival counter per output group, the
-    last arrival merges) and split-KV attention launches, queued on two streams so that they overlap on the card,
-    each stream with a workspace of its own (the workspace is per caller; the counters are shared and handed out in
-    rotation).  Every output must carry the bits of the same call made alone on one stream; the comparison stops
-    at the first mismatch."""
+    last arrival merges) and split-KV attention launches, issued by two Python threads, each on a stream of its own, so
+    that they overlap on the card.  The ops take their workspace per (device, stream) and the library hands the
+    arrival counters out in rotation, so the threads need no ordering between them.  Every output must carry the bits
+    of the same call made alone on one stream; the comparison stops at the first mismatch."""
+    import threading
     from tpp_pytorch_extension import _lib, _ops as ops
-    from tpp_pytorch_extension.llm import fused_llama_infer as F
     _ops()
     Lb = _lib.lib()
     dev = torch.device("cuda:0")
@@ -703,39 +703,46 @@ def test_split_launches_overlapping_on_two_streams():
     ln = torch.tensor([Lk - 1], dtype=torch.int32, device=dev)
     cases.append(("attn", q, kc, vc))
 
-    def call(case, ws):
-        dev_key = dev.index
-        old = _lib._workspaces.get(dev_key)
-        _lib._workspaces[dev_key] = ws  # the op picks the workspace up when it enqueues
-        try:
-            if case[0] == "linear":
-                _, qw, x, r = case
-                return ops.linear(x, qw, None, POSTS["add"], r, None, 0.5)
-            _, q, kc, vc = case
-            out = torch.empty_like(q)
-            _lib.check(Lb.tppx_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), None, 0, ln.data_ptr(), 1,
-                                           out.data_ptr(), B, Nq, Nq, 128, Smax, ws.data_ptr(), ws.numel(), _lib.stream_of(q)))
-            return out
-        finally:
-            if old is not None:
-                _lib._workspaces[dev_key] = old
+    def call(case):
+        if case[0] == "linear":
+            _, qw, x, r = case
+            return ops.linear(x, qw, None, POSTS["add"], r, None, 0.5)
+        _, q, kc, vc = case
+        ws = _lib.workspace(q)
+        out = torch.empty_like(q)
+        _lib.check(Lb.tppx_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), None, 0, ln.data_ptr(), 1,
+                                       out.data_ptr(), B, Nq, Nq, 128, Smax, ws.data_ptr(), ws.numel(), _lib.stream_of(q)))
+        return out
 
-    ws0 = _lib.workspace(q)
-    alone = [call(c, ws0) for c in cases]
+    alone = [call(c) for c in cases]
     torch.cuda.synchronize()
     streams = [torch.cuda.Stream(), torch.cuda.Stream()]
-    wss = [torch.zeros_like(ws0), torch.zeros_like(ws0)]
-    torch.cuda.synchronize()
     outs = [[], []]
-    for it in range(24):
-        for si in (0, 1):
+    seen_ws = [None, None]
+    errors = []
+
+    def worker(si):
+        try:
             with torch.cuda.stream(streams[si]):
-                ci = (it + 2 * si) % len(cases)  # the two streams run different cases side by side
-                outs[si].append((ci, call(cases[ci], wss[si])))
+                seen_ws[si] = _lib.workspace(q).data_ptr()
+                for it in range(24):
+                    ci = (it + 2 * si) % len(cases)  # the two threads run different cases side by side
+                    outs[si].append((ci, call(cases[ci])))
+        except Exception as e:  # reported by the main thread
+            errors.append((si, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(si,)) for si in (0, 1)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
     torch.cuda.synchronize()
+    assert not errors, errors
+    assert len({seen_ws[0], seen_ws[1], _lib.workspace(q).data_ptr()}) == 3, "each stream works in a workspace of its own"
     for si in (0, 1):
+        assert len(outs[si]) == 24
         for it, (ci, y) in enumerate(outs[si]):
-            assert torch.equal(y, alone[ci]), f"stream {si}, launch {it}, case {ci}: differs from the single-stream result"
+            assert torch.equal(y, alone[ci]), f"thread {si}, launch {it}, case {ci}: differs from the single-stream result"
 
 
 @pytest.mark.parametrize("M", [1, 5, 16])

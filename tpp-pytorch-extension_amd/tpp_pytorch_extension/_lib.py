@@ -4,6 +4,7 @@ The HIP library is the only compute backend of this package: if it is missing
 the import of any op fails loudly; there is no CPU or eager fallback.
 """
 import ctypes
+import threading
 import os
 
 import torch
@@ -132,21 +133,37 @@ def stream_of(t):
 
 WORKSPACE_BYTES = 32 << 20
 _workspaces = {}
+_workspaces_lock = threading.Lock()
 
 
 def workspace(t):
-    """Zero-initialised split-K scratch of `t`'s device (see include/tppx.h).
-    One buffer per device: ops that use it must be ordered with respect to
-    each other (same stream, or streams ordered by events / graph replay),
-    which is how the single-caller reference behaves as well."""
-    key = t.device.index
-    ws = _workspaces.get(key)
-    if ws is None:
-        if torch.cuda.is_current_stream_capturing():
+    """Split-K / staging scratch for an op on `t`'s device (see include/tppx.h).
+    One zero-initialised buffer per (device, stream): every op orders itself on
+    the caller's current stream, so threads that work on streams of their own
+    never share scratch and need no ordering between them. Work recorded under
+    stream capture uses one more buffer per device, created together with the
+    device's first eager one (a capture cannot allocate it): run the op once
+    eagerly before capturing, and order replays of different graphs that use
+    these ops with respect to each other."""
+    dev = t.device.index
+    if torch.cuda.is_current_stream_capturing():
+        ws = _workspaces.get((dev, "capture"))
+        if ws is None:
             raise TppxError(EINVAL, "first call on this device happens inside graph capture: run the op once "
                                     "eagerly before capturing so that its workspace exists")
-        ws = torch.zeros(WORKSPACE_BYTES, dtype=torch.uint8, device=t.device)
-        _workspaces[key] = ws
+        return ws
+    key = (dev, stream_of(t))
+    ws = _workspaces.get(key)
+    if ws is None:
+        with _workspaces_lock:
+            ws = _workspaces.get(key)
+            if ws is None:
+                if (dev, "capture") not in _workspaces:
+                    cap = torch.zeros(WORKSPACE_BYTES, dtype=torch.uint8, device=t.device)
+                    torch.cuda.current_stream(t.device).synchronize()  # zeroed before any capture stream sees it
+                    _workspaces[(dev, "capture")] = cap
+                ws = torch.zeros(WORKSPACE_BYTES, dtype=torch.uint8, device=t.device)
+                _workspaces[key] = ws
     return ws
 
 
