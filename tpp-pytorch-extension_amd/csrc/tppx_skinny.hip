@@ -1533,6 +1533,16 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
       return sk_launch(skinny_qint8_fq_kernel<3, 4, 16, 16, 2>, p, grid, 16, lds, stream);
     if (pl.ntw == 2)
       return sk_launch(skinny_qint8_fq_kernel<2, 4, 16, 16, 4>, p, grid, 16, lds, stream);
+    // Up to three K blocks (12 weight tiles) per wave: a ring of four tiles; one of eight would hold most of the
+    // wave's K range and only delays its first MFMA (4096 x 4096 at one row 6.9 -> 5.9 us).  With more than 16
+    // (row, block) items per wave, six quantisation passes are in flight, so that up to 24 items (8 rows x 3 blocks
+    // of the K = 11008 down-projection) are requested before the weight ring and none queues behind it
+    // (14.0 -> 12.2 us).  From four blocks per wave on the ring of eight wins.
+    if (pl.max_units <= 3) {
+      if ((int64_t)p.M * pl.max_units > 16)
+        return sk_launch(skinny_qint8_fq_kernel<1, 4, 16, 16, 6>, p, grid, 16, lds, stream);
+      return sk_launch(skinny_qint8_fq_kernel<1, 4, 16, 16, 4>, p, grid, 16, lds, stream);
+    }
     return sk_launch(skinny_qint8_fq_kernel<1, 8, 16, 16, 4>, p, grid, 16, lds, stream);
   }
   size_t lds = ((size_t)pl.waves * pl.ntw * pl.mg * 256 + (size_t)pl.waves * pl.max_units * pl.mg * 16) * sizeof(float);
