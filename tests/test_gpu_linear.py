@@ -77,6 +77,14 @@ def test_no_bias_ragged_k(fmt):
     _run(fmt, 8, 64, 11008, "none", False, 300)
 
 
+@pytest.mark.parametrize("M,N,K", [(12, 64, 11008), (13, 64, 11008), (9, 64, 14336), (4, 32, 16384), (1, 64, 4096)])
+def test_qint8_few_rows_quantised_in_the_gemm_ring_forms(M, N, K):
+    """QINT8 with the activation quantisation inside the GEMM kernel, one channel tile per workgroup: up to three
+    K blocks per wave run a ring of four weight tiles (six quantisation passes in flight once a wave has more than 16
+    (row, block) items: 36 and 39 items here, two rounds), four blocks per wave (K >= 14336) the ring of eight."""
+    _run("qint8", M, N, K, "add", True, 9100 + M + K)
+
+
 def test_cfg1_mxfp4_fc_plain():
     """BASELINE config 1: M=16, K=N=4096, MXFP4, bias."""
     _run("mxfp4", 16, 4096, 4096, "none", True, 1235)
