@@ -85,6 +85,13 @@ typedef void* tppx_stream_t;
 
 int tppx_version(void);
 const char* tppx_last_error(void);
+/* The library reads its TPPX_* environment switches once per process, the
+ * first time a launch asks for one, and keeps the answer (no getenv() per
+ * launch; a kernel choice recorded in a captured graph cannot drift from the
+ * eager one).  This drops what was kept, so the next launch reads the
+ * environment again.  No counterpart in the reference (its switches are read
+ * at static-initialisation time, e.g. src/csrc/fused_gemm.h:26-37). */
+void tppx_reload_env(void);
 
 /* ---- quantize / remap -------------------------------------------------- */
 

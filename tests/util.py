@@ -43,10 +43,17 @@ def err_stats(got_bits, ref_bits):
     }
 
 
-def assert_close_bf16(got_bits, ref_bits, ulps=1, rel_l2=4e-3, what="", pre_bits=None):
+def assert_close_bf16(got_bits, ref_bits, ulps=1, rel_l2=4e-3, what="", pre_bits=None, max_mismatch="auto"):
     """Tolerance of the parity tests: every element within `ulps` bf16 ulps of
     the oracle (|d| <= ulps * (2^-7 |ref| + 2^-8 rms(ref)), the second term
     covering outputs that cancel to near zero) and relative L2 error <= rel_l2.
+    `max_mismatch` bounds how many elements may differ from the oracle's bits AT
+    ALL: a different fp32 summation order moves 5-100 elements per million
+    across a rounding boundary, so a kernel that is one ulp off everywhere is an
+    error even though each element is within the bound.  "auto" = 1e-3 of the
+    elements (at least 3) for the 1-ulp comparisons, no count for the 2-ulp ones
+    (SiLU / GELU go through the hardware's exp2 and reciprocal, whose results
+    differ from libm's in more places).
     `pre_bits` = the oracle's bf16 GEMM(+bias) tile before an additive post-op.
     A different fp32 summation order moves a few elements per million of that
     tile by one bf16 ulp (the no-post tests accept exactly that); the post-op
@@ -66,4 +73,10 @@ def assert_close_bf16(got_bits, ref_bits, ulps=1, rel_l2=4e-3, what="", pre_bits
         f"rel_l2={s['rel_l2']:.3g} first={np.argwhere(bad)[:4].tolist()}"
     )
     assert s["rel_l2"] <= rel_l2, f"{what}: rel_l2={s['rel_l2']:.3g} > {rel_l2}"
+    if max_mismatch == "auto":
+        max_mismatch = 1e-3 if ulps == 1 else None
+    if max_mismatch is not None:
+        n_diff = int(np.count_nonzero(np.asarray(got_bits) != np.asarray(ref_bits)))
+        allowed = max(3, int(np.ceil(max_mismatch * np.asarray(ref_bits).size)))
+        assert n_diff <= allowed, f"{what}: {n_diff} of {np.asarray(ref_bits).size} elements differ from the oracle (allowed {allowed})"
     return s

@@ -81,9 +81,22 @@ hipError_t allow_dynamic_lds(const void* kern, size_t lds) {
   return hipSuccess;
 }
 
+// TPPX_* switches are read from the environment ONCE per process (the first time a launch site asks) and kept, so
+// that a launch costs no getenv() and a kernel choice recorded in a captured graph cannot drift from the eager
+// one.  tppx_reload_env() drops what was kept (tests that flip a switch call it).  Keyed by the address of the
+// name literal: every call site passes its own.
+static std::mutex g_env_mu;
+static std::map<const char*, std::pair<bool, int>> g_env_kept; // name -> (set in the environment, its value)
+
 int env_int(const char* name, int dflt) {
-  const char* v = getenv(name);
-  return (v && *v) ? atoi(v) : dflt;
+  std::lock_guard<std::mutex> lock(g_env_mu);
+  auto it = g_env_kept.find(name);
+  if (it == g_env_kept.end()) {
+    const char* v = getenv(name);
+    const bool set = v && *v;
+    it = g_env_kept.emplace(name, std::make_pair(set, set ? atoi(v) : 0)).first;
+  }
+  return it->second.first ? it->second.second : dflt;
 }
 
 static bool valid_post(int post) {
@@ -452,8 +465,13 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
   p.sa = (const float*)sa;
   p.M = (int)M;
   p.K = (int)K;
-  p.units = (int)(K / qbs);
   p.tpb = (int)(qbs / 64);
+  p.nblk = (int)(K / qbs);
+  // what is dealt to waves and K parts: runs of 256 input channels inside larger blocks (per-output-channel scales,
+  // qbs = K, keep every wave busy that way), whole blocks below 256, single tiles for other block sizes
+  p.deal = p.tpb % 4 == 0 ? 4 : (p.tpb < 4 ? p.tpb : 1);
+  p.units = (int)(K / (64 * p.deal));
+  p.spb_magic = (p.deal == 4 && p.tpb > 4) ? (unsigned int)((((uint64_t)1 << 32) + (uint64_t)(p.tpb / 4) - 1) / (uint64_t)(p.tpb / 4)) : 0u;
   const bool reuse = (flags & TPPX_FLAG_XQ_REUSE) != 0; // xq / sa still hold this x, quantized by an earlier call
   if (qbs % 128 == 0 && want_tiled(M, flags, K, p.total_tiles, (double)p.total_tiles * 16.0 * (double)K)) {
     if (x && !reuse) {
@@ -482,7 +500,7 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
     return TPPX_OK;
   }
   p.S = 1;
-  SkinnyPlan sp = plan_skinny(M, p.total_tiles, p.units, x != nullptr && qbs == 256);
+  SkinnyPlan sp = plan_skinny(M, p.total_tiles, p.units, p.tpb, p.deal, x != nullptr && qbs % 256 == 0);
   // 33..64 rows, few channel tiles and a long K: every workgroup would pull all of the int8 activations (M x K)
   // through its CU.  Two K parts of two channel tiles each halve that (measured at N = 4096, 64 rows: K = 11008
   // 20.4 -> 18.5 us, K = 14336 25.1 -> 21.6 us; K = 8192 and shorter lose to the extra pass over the partial sums).
@@ -491,7 +509,7 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
     p.part = (float*)ws;
     sp.ntw = 2;
     sp.waves = 8;
-    sp.max_units = (p.units + 7) / 8;
+    sp.max_units = skinny_qint8_blocks_per_wave(((p.units + 1) / 2 + 7) / 8, p.tpb, p.deal, p.nblk);
   }
   if (x && !sp.fused_quant) {
     // quantise straight into MFMA operand order: the GEMM then reads one
@@ -743,6 +761,11 @@ extern "C" int tppx_linear_qint8_noalloc(const void* x, const void* qw, const vo
     return rc;
   return run_qint8(who, x, base, base + NA_XQ_BYTES, &s, 1, M, K, qbs, flags, base + NA_XQ_BYTES + NA_SA_BYTES,
                    (int64_t)NA_WS_BYTES, (hipStream_t)stream);
+}
+
+extern "C" void tppx_reload_env(void) {
+  std::lock_guard<std::mutex> lock(g_env_mu);
+  g_env_kept.clear();
 }
 
 // ---- launch plans -----------------------------------------------------------

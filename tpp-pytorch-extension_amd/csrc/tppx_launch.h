@@ -46,8 +46,16 @@ struct DecodeParams {
   const float* sa; // f32  [M][K/qbs] (QINT8, unless quantised in-kernel)
   int M, K;
   int mt;    // > 0: xq is [K/64][mt][4 g][16 m][16 B] (operand tiles of 16 rows x 64 K); 0: row-major
-  int units; // K/128 (MXFP4 tiles) or K/qbs (QINT8 blocks)
-  int tpb;   // native tiles per unit (1 for MXFP4, qbs/64 for QINT8)
+  int units; // what is dealt to waves (and K parts): K/128 (MXFP4 tiles); QINT8: K / (64 * deal)
+  int tpb;   // native tiles per scale block (1 for MXFP4, qbs/64 for QINT8)
+  // QINT8: K is dealt in runs of `deal` 64-wide tiles: 4 (256 input channels) when a scale block is a whole number of
+  // such runs, whole blocks when a block has fewer than 4 tiles, single tiles otherwise.  A run that ends inside a
+  // scale block folds its exact int32 sums with the block's scales like a block of its own.
+  int deal;
+  int nblk;  // QINT8: K / qbs scale blocks
+  // deal == 4: scale block of run u = spb_magic ? mulhi(u, spb_magic) : u   (spb_magic = ceil(2^32 / (tpb / 4)),
+  // exact for u * (tpb / 4) < 2^32; 0 when a block is one run)
+  unsigned int spb_magic;
   int S;     // K parts across workgroups (grid z, at most 4); > 1: partial sums go to `part`, the workgroup that
              // arrives last at its ticket adds them and runs the epilogue
   int ticket0; // first arrival counter of this launch (S > 1), see skinny_split_tickets()
@@ -112,8 +120,11 @@ hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qb
 // xq Mp*K bytes, xs Mp*K/32 bytes
 hipError_t launch_quant_act_mxfp8(const void* x, int64_t M, int64_t K, void* xq, void* xs, hipStream_t stream);
 
-// can_fuse_quant: bf16 activations at hand and 256-wide blocks (the in-kernel quantisation's case)
-SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, bool can_fuse_quant);
+// units = runs of K dealt to waves (DecodeParams::units), tpb / deal as in DecodeParams;
+// can_fuse_quant: bf16 activations at hand and blocks of a multiple of 256 (the in-kernel quantisation's case)
+SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, int tpb, int deal, bool can_fuse_quant);
+// scale blocks a wave that owns `runs` consecutive runs of K can touch
+int skinny_qint8_blocks_per_wave(int runs, int tpb, int deal, int nblk);
 hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream);
 hipError_t launch_skinny_bf16(DecodeParams& p, int mg, int nt, hipStream_t stream);
 size_t skinny_mxfp4_xl_lds(int units, int nt, bool dual);

@@ -435,6 +435,87 @@ quant_act_int8_rows_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
   }
 }
 
+// Scale blocks of several 256-wide runs (per-output-channel weights: one block = all of K): one workgroup per
+// (row, block), 16 lanes per run as above; the runs' maxima meet in LDS.  A lane group's first run stays in registers
+// between the two steps, further runs (blocks beyond 16 Ki channels) are read a second time.
+__global__ void __launch_bounds__(1024)
+quant_act_int8_bigblk_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K, int64_t qbs, int8_t* __restrict__ xq,
+                             float* __restrict__ sa, int mt) {
+  __shared__ float gmax[64];
+  const int64_t nb = K / qbs, m = blockIdx.x / nb, b = blockIdx.x - m * nb;
+  const int spb = (int)(qbs >> 8), groups = blockDim.x >> 4;
+  const int l = threadIdx.x & 15, grp = threadIdx.x >> 4;
+  const uint16_t* row = x + m * K + b * qbs;
+  auto dpp = [](float v, auto CTRL) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), decltype(CTRL)::value, 0xf, 0xf, true));
+  };
+  auto load_run = [&](int r, uint32_t (&w)[8]) {
+    const uint4* src = reinterpret_cast<const uint4*>(row + (int64_t)r * 256 + l * 16);
+    const uint4 v0 = src[0], v1 = src[1];
+    w[0] = v0.x; w[1] = v0.y; w[2] = v0.z; w[3] = v0.w;
+    w[4] = v1.x; w[5] = v1.y; w[6] = v1.z; w[7] = v1.w;
+  };
+  auto amax_of = [&](const uint32_t (&w)[8]) {
+    float a = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      a = fmaxf(a, fmaxf(fabsf(bf16_bits_to_f32(w[i] & 0xffffu)), fabsf(bf16_bits_to_f32(w[i] >> 16))));
+    return a;
+  };
+  uint32_t first[8] = {0, 0, 0, 0, 0, 0, 0, 0}, w[8];
+  float amax = 0.0f;
+  if (grp < spb) {
+    load_run(grp, first);
+    amax = amax_of(first);
+  }
+  for (int r = grp + groups; r < spb; r += groups) {
+    load_run(r, w);
+    amax = fmaxf(amax, amax_of(w));
+  }
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0xB1>{}));
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0x4E>{}));
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0x141>{}));
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0x140>{}));
+  if (l == 0)
+    gmax[grp] = amax;
+  __syncthreads();
+  amax = 0.0f;
+  for (int j = l; j < groups; j += 16)
+    amax = fmaxf(amax, gmax[j]);
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0xB1>{}));
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0x4E>{}));
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0x141>{}));
+  amax = fmaxf(amax, dpp(amax, std::integral_constant<int, 0x140>{}));
+  const float s = int8_scale_of(amax);
+  const float inv = int8_inv_scale(s);
+  if (threadIdx.x == 0)
+    sa[mt > 0 ? b * (int64_t)mt * 16 + m : m * nb + b] = s;
+  auto emit = [&](int r, const uint32_t (&src)[8]) {
+    uint32_t o[4];
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+      const float f0 = bf16_bits_to_f32(src[2 * d] & 0xffffu), f1 = bf16_bits_to_f32(src[2 * d] >> 16);
+      const float f2 = bf16_bits_to_f32(src[2 * d + 1] & 0xffffu), f3 = bf16_bits_to_f32(src[2 * d + 1] >> 16);
+      o[d] = (uint32_t)(int8_q(f0, inv) & 0xff) | ((uint32_t)(int8_q(f1, inv) & 0xff) << 8) |
+             ((uint32_t)(int8_q(f2, inv) & 0xff) << 16) | ((uint32_t)(int8_q(f3, inv) & 0xff) << 24);
+    }
+    const int64_t k0 = b * qbs + (int64_t)r * 256; // first channel of the run
+    if (mt > 0) {
+      const int64_t t = (k0 >> 6) + (l >> 2);
+      const int64_t slot = (t * mt + (m >> 4)) * 64 + (l & 3) * 16 + (m & 15);
+      reinterpret_cast<uint4*>(xq)[slot] = make_uint4(o[0], o[1], o[2], o[3]);
+    } else {
+      reinterpret_cast<uint4*>(xq + m * K + k0)[l] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+  };
+  if (grp < spb)
+    emit(grp, first);
+  for (int r = grp + groups; r < spb; r += groups) {
+    load_run(r, w);
+    emit(r, w);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Generic per-block quantizers: any tensor viewed as in[pre][bs][post][vnni]
 // (the geometry PerBlockQuantizer derives from sizes, block size, axis and the
@@ -660,6 +741,14 @@ hipError_t launch_quant_act_int8(const void* x, int64_t M, int64_t K, int64_t qb
     const int64_t nt16 = M * (K / 256) * 16;
     TPPX_PLAN_ONLY(quant_act_int8_rows_kernel, dim3(grid_for(nt16, 256)), dim3(256), 0);
     quant_act_int8_rows_kernel<<<grid_for(nt16, 256), 256, 0, stream>>>((const uint16_t*)x, M, K, (int8_t*)xq, (float*)sa, mt);
+    return hipGetLastError();
+  }
+  if (qbs > 256 && qbs % 256 == 0 && M * (K / qbs) < (1 << 30)) {
+    const int64_t lanes = (qbs >> 8) * 16;
+    const unsigned block = (unsigned)(lanes >= 1024 ? 1024 : (lanes + 63) / 64 * 64);
+    const dim3 grid((unsigned)(M * (K / qbs)));
+    TPPX_PLAN_ONLY(quant_act_int8_bigblk_kernel, grid, dim3(block), 0);
+    quant_act_int8_bigblk_kernel<<<grid, block, 0, stream>>>((const uint16_t*)x, M, K, qbs, (int8_t*)xq, (float*)sa, mt);
     return hipGetLastError();
   }
   int64_t nthreads = M * (K / qbs) * 64;

@@ -362,13 +362,20 @@ skinny_qint8_kernel(const DecodeParams p) {
   const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
   const int ltile0 = (grp - sg.grp0) * NTW;
   const int m0 = blockIdx.y * MPAD;
-  const int NB = p.units, TPB = p.tpb, KT = NB * TPB;
-  const bool TPB4 = TPB == 4; // 256-wide K blocks: the default
+  const int NB = p.nblk, TPB = p.tpb, KT = NB * TPB, G = p.deal;
+  // K is dealt in runs of G tiles.  G == 4 (a scale block is a whole number of 256-wide runs; one run by default):
+  // static ring slots, the int32 sums are folded after every run with the scales of the run's block.
+  const bool FAST = G == 4;
   constexpr int UN = (PF % 4 == 0) ? PF : (PF % 2 == 0 ? 2 * PF : 4 * PF); // lcm(PF, 4) tiles per unrolled trip
-  // K blocks of this workgroup (all of them unless K is split across workgroups), then of this wave
-  const int ub = (int)(((int64_t)blockIdx.z * NB) / p.S), ue = (int)(((int64_t)(blockIdx.z + 1) * NB) / p.S);
+  // runs of this workgroup (all of them unless K is split across workgroups), then of this wave
+  const int ub = (int)(((int64_t)blockIdx.z * p.units) / p.S), ue = (int)(((int64_t)(blockIdx.z + 1) * p.units) / p.S);
   const int u0 = ub + (int)(((int64_t)wave * (ue - ub)) / W), u1 = ub + (int)(((int64_t)(wave + 1) * (ue - ub)) / W);
-  const int t0 = u0 * TPB, t1 = u1 * TPB;
+  const int t0 = u0 * G, t1 = u1 * G;
+  const unsigned int magic = p.spb_magic;
+  auto blk_of = [&](int t, bool fast) { // scale block of tile t (uniform)
+    return fast ? (magic ? (int)__umulhi((unsigned int)(t >> 2), magic) : (t >> 2)) : t / TPB;
+  };
+  const int b0 = blk_of(max(min(t0, KT - 1), 0), FAST); // first scale block of this wave
 
   const i32x4* wq[NTW];
   const float* ws[NTW];
@@ -397,14 +404,14 @@ skinny_qint8_kernel(const DecodeParams p) {
   // activation scales of this wave's K blocks, transposed in LDS: [u - u0][MPAD]
   float* red = sk_lds;
   float* sa_s = sk_lds + (size_t)W * NTW * MG * 256 + (size_t)wave * p.cht * MPAD;
-  const int nsa = (u1 - u0) * MPAD;
+  const int nsa = t0 < t1 ? (blk_of(t1 - 1, FAST) - b0 + 1) * MPAD : 0;
   const int mtp = p.mt * 16;
   constexpr int SAB = 2 * MG; // loads per batch: 8 K blocks of this wave
   auto load_sa = [&](int i) {
     i = max(min(i, nsa - 1), 0);
     const int ul = i / MPAD, mr = i - ul * MPAD;
     // XOP: scales transposed by the quantisation kernel, [K/qbs][mt*16]
-    return XOP ? p.sa[(int64_t)(u0 + ul) * mtp + m0 + mr] : p.sa[(int64_t)min(m0 + mr, p.M - 1) * NB + u0 + ul];
+    return XOP ? p.sa[(int64_t)(b0 + ul) * mtp + m0 + mr] : p.sa[(int64_t)min(m0 + mr, p.M - 1) * NB + b0 + ul];
   };
   // (no branch around these first requests or the ring's: behind a conditional load the compiler can no longer count
   // the loads in flight and waits for all of them; a wave without K blocks re-reads valid data it never uses)
@@ -422,7 +429,7 @@ skinny_qint8_kernel(const DecodeParams p) {
   float sreg[PF][NTW];
   auto load_stage = [&](int st, int t, bool fast) {
     t = max(min(t, t1 - 1), 0); // past the end: re-read the last tile (never consumed)
-    const int b = fast ? (t >> 2) : t / TPB;
+    const int b = blk_of(t, fast);
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
       wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64);
@@ -463,7 +470,7 @@ skinny_qint8_kernel(const DecodeParams p) {
       iacc[nt][mg] = i32x4{0, 0, 0, 0};
     }
 
-  // multiply stage i (tile tt); `last` = tt closes a K block: fold into fp32
+  // multiply stage i (tile tt); `last` = tt closes a K block or this wave's part of one: fold into fp32
   auto consume = [&](int i, int tt, bool last, bool fast) {
     float swv[NTW];
 #pragma unroll
@@ -474,10 +481,10 @@ skinny_qint8_kernel(const DecodeParams p) {
         iacc[nt][mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xreg[i][mg], wreg[i][nt], iacc[nt][mg], 0, 0, 0);
     }
     if (last) {
-      const int b = fast ? (tt >> 2) : tt / TPB;
+      const int b = blk_of(tt, fast);
 #pragma unroll
       for (int mg = 0; mg < MG; mg++) {
-        const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + (b - u0) * MPAD + mg * 16 + (lane >> 4) * 4);
+        const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + (b - b0) * MPAD + mg * 16 + (lane >> 4) * 4);
 #pragma unroll
         for (int nt = 0; nt < NTW; nt++)
 #pragma unroll
@@ -490,8 +497,8 @@ skinny_qint8_kernel(const DecodeParams p) {
   };
 
   int t = t0;
-  if (TPB4) {
-    // full trips of UN tiles: static ring slots and block boundaries (t0 is a
+  if (FAST) {
+    // full trips of UN tiles: static ring slots and fold points (t0 is a
     // multiple of 4), every reload a real tile
     for (; t + UN + PF <= t1; t += UN) {
 #pragma unroll
@@ -502,14 +509,14 @@ skinny_qint8_kernel(const DecodeParams p) {
       }
     }
   }
-  // remaining tiles (and every tile when the K block is not 256 wide); the
-  // ring slot of tile tt is (tt - t0) % PF
+  // remaining tiles (and every tile when K is not dealt in runs of 4 tiles);
+  // the ring slot of tile tt is (tt - t0) % PF
   for (int tb = t; tb < t1; tb += PF) {
 #pragma unroll
     for (int i = 0; i < PF; i++) {
       const int tt = tb + i;
       if (tt < t1) {
-        consume(i, tt, (tt + 1) % TPB == 0, false);
+        consume(i, tt, FAST ? (tt & 3) == 3 : ((tt + 1) % TPB == 0 || tt + 1 == t1), FAST);
         if (tt + PF < t1)
           load_stage(i, tt + PF, false);
       }
@@ -566,7 +573,10 @@ __device__ __forceinline__ uint32_t sk_int8x4_rne(float a, float b, float c, flo
   return __builtin_amdgcn_perm(ub, ua, 0x0c0c0400u) | __builtin_amdgcn_perm(ud, uc, 0x04000c0cu);
 }
 
-template <int NTW, int PF, int MAXW, int MINW, int XB>
+// BIGB: scale blocks of several 256-wide runs.  Every wave takes the maxima of its own (row, run) items, the waves
+// exchange them through LDS (one barrier), and an item is quantised with the maximum over the runs of its block; all
+// of a wave's items stay in registers meanwhile (the launcher checks that there are at most 4 * XB).
+template <int NTW, int PF, int MAXW, int MINW, int XB, bool BIGB>
 __global__ void __launch_bounds__(MAXW * 64)
 skinny_qint8_fq_kernel(const DecodeParams p) {
   extern __shared__ __align__(16) float sk_lds[];
@@ -576,9 +586,11 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
   const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
   const int ltile0 = (grp - sg.grp0) * NTW;
   const int M = p.M; // <= 16, one block row
-  const int NB = p.units, KT = NB * 4;
-  const int u0 = (int)(((int64_t)wave * NB) / W), u1 = (int)(((int64_t)(wave + 1) * NB) / W);
+  const int NR = p.units, KT = NR * 4, NB = p.nblk; // 256-wide runs of K, tiles, scale blocks
+  const int u0 = (int)(((int64_t)wave * NR) / W), u1 = (int)(((int64_t)(wave + 1) * NR) / W);
   const int t0 = u0 * 4, t1 = u1 * 4;
+  const unsigned int magic = p.spb_magic;
+  auto blk_of_run = [&](int u) { return BIGB ? (int)__umulhi((unsigned int)u, magic) : u; };
 
   const i32x4* wq[NTW];
   const float* ws[NTW];
@@ -618,7 +630,7 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
       wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64);
-      sreg[st][nt] = ws[nt][(t >> 2) * 16];
+      sreg[st][nt] = ws[nt][blk_of_run(t >> 2) * 16];
     }
   };
   // No branch around the ring's first requests: with one, the compiler can no longer count the loads behind the
@@ -633,6 +645,42 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
   uint8_t* mine = reinterpret_cast<uint8_t*>(sk_lds + (p.lds_overlap ? 0 : (size_t)W * NTW * 256)) + (size_t)wave * p.cht * (256 * M + 64);
   uint32_t* xq_s = reinterpret_cast<uint32_t*>(mine);
   float* sa_s = reinterpret_cast<float*>(mine + (size_t)p.cht * 256 * M);
+  // maximum of |x| over the 256 values of the pass's item, in every lane of its DPP row
+  auto item_amax = [&](auto PS) {
+    constexpr int ps = decltype(PS)::value;
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const uint32_t wd = (uint32_t)raw[ps][j >> 2][j & 3];
+      amax = fmaxf(amax, fmaxf(fabsf(bf16_bits_to_f32(wd & 0xffffu)), fabsf(bf16_bits_to_f32(wd >> 16))));
+    }
+    amax = sk_dpp_max<0xB1>(amax);  // quad_perm [1,0,3,2]
+    amax = sk_dpp_max<0x4E>(amax);  // quad_perm [2,3,0,1]
+    amax = sk_dpp_max<0x141>(amax); // row_half_mirror
+    return sk_dpp_max<0x140>(amax); // row_mirror: every lane of the row holds the max
+  };
+  // BIGB: [row][run] maxima of all waves, behind every wave's private region
+  float* amax_s = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(sk_lds + (p.lds_overlap ? 0 : (size_t)W * NTW * 256)) +
+                                           (size_t)W * p.cht * (256 * M + 64));
+  if (BIGB) {
+    static_for<0, XB>([&](auto PS) {
+      constexpr int ps = decltype(PS)::value;
+      if (ps * 4 < nitems) { // wave-uniform
+        const int it = ps * 4 + (lane >> 4);
+        const uint32_t itc = (uint32_t)min(it, nitems - 1);
+        const uint32_t ul = itc / Mu, mr = itc - ul * Mu;
+        const float am = item_amax(PS);
+        if (it < nitems && (lane & 15) == 0)
+          amax_s[mr * NR + u0 + ul] = am;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    __syncthreads();
+    // the values are unpacked again behind the barrier: kept across it, the floats of all passes would spill
+#pragma unroll
+    for (int ps = 0; ps < XB; ps++)
+      asm volatile("" : "+v"(raw[ps][0]), "+v"(raw[ps][1]));
+  }
   auto quant_pass = [&](auto PS, int base) {
     constexpr int ps = decltype(PS)::value;
     if ((base + ps) * 4 < nitems) { // wave-uniform
@@ -640,18 +688,26 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
       const uint32_t itc = (uint32_t)min(it, nitems - 1);
       const uint32_t ul = itc / Mu, mr = itc - ul * Mu;
       float v[16];
-      float amax = 0.0f;
 #pragma unroll
       for (int j = 0; j < 8; j++) {
         const uint32_t wd = (uint32_t)raw[ps][j >> 2][j & 3];
         v[2 * j] = bf16_bits_to_f32(wd & 0xffffu);
         v[2 * j + 1] = bf16_bits_to_f32(wd >> 16);
-        amax = fmaxf(amax, fmaxf(fabsf(v[2 * j]), fabsf(v[2 * j + 1])));
       }
-      amax = sk_dpp_max<0xB1>(amax);  // quad_perm [1,0,3,2]
-      amax = sk_dpp_max<0x4E>(amax);  // quad_perm [2,3,0,1]
-      amax = sk_dpp_max<0x141>(amax); // row_half_mirror
-      amax = sk_dpp_max<0x140>(amax); // row_mirror: every lane of the row holds the max
+      float amax;
+      if (BIGB) {
+        // the item's block = runs [blk * spb, (blk + 1) * spb): the 16 lanes of the DPP row share them out
+        const int spb = p.tpb >> 2, r0 = blk_of_run(u0 + (int)ul) * spb;
+        amax = 0.0f;
+        for (int j = lane & 15; j < spb; j += 16)
+          amax = fmaxf(amax, amax_s[mr * NR + r0 + j]);
+        amax = sk_dpp_max<0xB1>(amax);
+        amax = sk_dpp_max<0x4E>(amax);
+        amax = sk_dpp_max<0x141>(amax);
+        amax = sk_dpp_max<0x140>(amax);
+      } else {
+        amax = item_amax(PS);
+      }
       // == float(double(amax) / 127.0): amax is a bf16 value, so the
       // quotient cannot sit on a double-rounding boundary
       const float sc = __fdiv_rn(amax, 127.0f);
@@ -661,19 +717,22 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
       for (int d = 0; d < 4; d++)
         pk[d] = sk_int8x4_rne(v[4 * d], v[4 * d + 1], v[4 * d + 2], v[4 * d + 3], inv);
       if (it < nitems) {
-        // values k = (lane&15)*16.. of the block: tile (lane&15)/4, K group (lane&15)%4
+        // values k = (lane&15)*16.. of the run: tile (lane&15)/4, K group (lane&15)%4
         const int tl = (int)ul * 4 + ((lane & 15) >> 2), g = lane & 3;
         reinterpret_cast<uint4*>(xq_s)[(tl * 4 + g) * M + (int)mr] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
         if ((lane & 15) == 0)
-          sa_s[ul * 16 + mr] = sc;
+          sa_s[ul * 16 + mr] = sc; // per run: the runs of one block hold the same scale
       }
     }
+    if (BIGB)
+      __builtin_amdgcn_sched_barrier(0); // one pass after the other: interleaved, their temporaries spill
   };
   static_for<0, XB>([&](auto PS) { quant_pass(PS, 0); });
-  for (int base = XB; base * 4 < nitems; base += XB) { // more than 16 items per wave
-    static_for<0, XB>([&](auto PS) { load_pass(PS, base); });
-    static_for<0, XB>([&](auto PS) { quant_pass(PS, base); });
-  }
+  if (!BIGB)
+    for (int base = XB; base * 4 < nitems; base += XB) { // more than 4 * XB items per wave
+      static_for<0, XB>([&](auto PS) { load_pass(PS, base); });
+      static_for<0, XB>([&](auto PS) { quant_pass(PS, base); });
+    }
   const int xoff = ((lane >> 4) * M + min(lane & 15, M - 1)) * 4; // dword offset inside a tile
 
   f32x4 facc[NTW][1];
@@ -693,7 +752,7 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
     }
     if (last) { // K block complete
       // result rows (lane>>4)*4 + r; scales of rows >= M are whatever the LDS held: those rows are not stored
-      const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + ((tt >> 2) - u0) * 16 + (lane >> 4) * 4);
+      const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + ((tt >> 2) - u0) * 16 + (lane >> 4) * 4); // by run
 #pragma unroll
       for (int nt = 0; nt < NTW; nt++)
 #pragma unroll
@@ -1431,16 +1490,27 @@ skinny_bf16_kernel(const DecodeParams p) {
   ep.finish(sg, acc, sk_lds, decltype(ep)::ELEMS);
 }
 
+// Scale blocks that `runs` consecutive runs of `deal` tiles can touch (slots of activation scales a wave keeps in LDS).
+int skinny_qint8_blocks_per_wave(int runs, int tpb, int deal, int nblk) {
+  const int tiles = runs * deal;
+  int n = (deal % tpb == 0) ? tiles / tpb : (tiles + tpb - 1) / tpb + 1; // whole blocks : a range that starts anywhere
+  if (n > nblk)
+    n = nblk;
+  return n < 1 ? 1 : n;
+}
+
 // launch shape of the QINT8 decode kernels
-SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, bool can_fuse_quant) {
+SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, int tpb, int deal, bool can_fuse_quant) {
+  const int env_ntw = env_int("TPPX_SKINNY_NTW", 0), env_waves = env_int("TPPX_SKINNY_WAVES", 0),
+            env_fusedq = env_int("TPPX_SKINNY_FUSEDQ", 1);
   SkinnyPlan pl;
+  const int nblk = (int)((int64_t)units * deal / tpb);
   const int mrows = (int)(M < 64 ? M : 64);
   pl.mg = mrows <= 16 ? 1 : (mrows <= 32 ? 2 : 4);
   pl.grid_y = (int)((M + 16 * pl.mg - 1) / (16 * pl.mg));
   // two channel tiles per wave once there are plenty of tiles: halves the
   // activation-operand traffic per weight byte
   pl.ntw = total_tiles >= 512 ? 2 : 1;
-  const int env_ntw = env_int("TPPX_SKINNY_NTW", 0);
   if (env_ntw == 1 || env_ntw == 2)
     pl.ntw = env_ntw;
   // more than 16 rows: these kernels run one workgroup per CU, so prefer a grid
@@ -1449,12 +1519,12 @@ SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, bool can_fuse_quan
     pl.ntw = 3;
   // Wave-count window of the kernel instantiation that will run (register
   // budget: 16 waves leave 128 VGPRs per lane, 8 leave 256; the epilogue's
-  // outputs-per-thread bound sets the minimum).  Waves beyond the number of K
-  // units simply get an empty range.
+  // outputs-per-thread bound sets the minimum).  Waves beyond the number of
+  // runs of K simply get an empty range.
   const bool wide = pl.mg == 4 || (pl.mg == 2 && pl.ntw >= 2);
   const int max_w = wide ? 8 : 16, min_w = wide ? 8 : 4;
   // few tiles: one 16-wave workgroup per CU keeps the whole weight in flight
-  int w = env_int("TPPX_SKINNY_WAVES", (total_tiles / pl.ntw <= 320) ? 16 : 8);
+  int w = env_waves > 0 ? env_waves : ((total_tiles / pl.ntw <= 320) ? 16 : 8);
   if (w > units)
     w = units;
   if (w > max_w)
@@ -1462,16 +1532,19 @@ SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, bool can_fuse_quan
   if (w < min_w)
     w = min_w;
   pl.waves = w;
-  pl.max_units = (units + w - 1) / w;
+  pl.max_units = skinny_qint8_blocks_per_wave((units + w - 1) / w, tpb, deal, nblk);
   pl.fused_quant = false;
   pl.lds_overlap = false;
-  if (M <= 16 && can_fuse_quant && env_int("TPPX_SKINNY_FUSEDQ", 1) != 0) {
+  if (M <= 16 && can_fuse_quant && env_fusedq != 0) {
     // quantisation inside the GEMM kernel: 16 waves, the fewest channel tiles per workgroup that keep the grid
     // within one round of 256 workgroups, as long as the quantised rows of all waves fit the LDS
     const int ntw = total_tiles <= 256 ? 1 : (total_tiles <= 512 ? 2 : 3);
-    const int cht = (units + 15) / 16;
-    const size_t xbytes = (size_t)16 * cht * (256 * (size_t)M + 64), rbytes = (size_t)16 * ntw * 1024;
-    if (xbytes <= 160 * 1024 && rbytes <= 160 * 1024) {
+    const int cht = (units + 15) / 16; // runs of 256 input channels per wave
+    const bool bigb = tpb > 4;         // blocks of several runs: maxima exchanged between the waves, items in registers
+    const size_t abytes = bigb ? (size_t)M * units * sizeof(float) : 0;
+    const size_t xbytes = (size_t)16 * cht * (256 * (size_t)M + 64) + abytes, rbytes = (size_t)16 * ntw * 1024;
+    const int xb = bigb ? (ntw == 1 ? 6 : 4) : 0;
+    if (xbytes <= 160 * 1024 && rbytes <= 160 * 1024 && (!bigb || M * (int64_t)cht <= 4 * xb)) {
       pl.fused_quant = true;
       pl.lds_overlap = xbytes + rbytes > 160 * 1024;
       pl.ntw = ntw;
@@ -1526,13 +1599,24 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
   if (grid.z > 1 && (p.S > 4 || (p.ticket0 = skinny_split_tickets((int)(grid.x * grid.y))) < 0))
     return hipErrorInvalidValue;
   if (pl.fused_quant) {
-    const size_t xbytes = (size_t)16 * pl.max_units * (256 * (size_t)p.M + 64), rbytes = (size_t)16 * pl.ntw * 1024;
+    const bool bigb = p.tpb > 4;
+    const size_t abytes = bigb ? (size_t)p.M * p.units * sizeof(float) : 0;
+    const size_t xbytes = (size_t)16 * pl.max_units * (256 * (size_t)p.M + 64) + abytes, rbytes = (size_t)16 * pl.ntw * 1024;
     const size_t lds = pl.lds_overlap ? (xbytes > rbytes ? xbytes : rbytes) : xbytes + rbytes;
     p.lds_overlap = pl.lds_overlap ? 1 : 0;
+    if (bigb) { // all (row, run) items of a wave stay in registers: M * runs per wave <= 4 * XB (plan_skinny checked)
+      if (pl.ntw == 3)
+        return sk_launch(skinny_qint8_fq_kernel<3, 4, 16, 16, 4, true>, p, grid, 16, lds, stream);
+      if (pl.ntw == 2)
+        return sk_launch(skinny_qint8_fq_kernel<2, 4, 16, 16, 4, true>, p, grid, 16, lds, stream);
+      if (pl.max_units <= 3)
+        return sk_launch(skinny_qint8_fq_kernel<1, 4, 16, 16, 6, true>, p, grid, 16, lds, stream);
+      return sk_launch(skinny_qint8_fq_kernel<1, 8, 16, 16, 6, true>, p, grid, 16, lds, stream);
+    }
     if (pl.ntw == 3)
-      return sk_launch(skinny_qint8_fq_kernel<3, 4, 16, 16, 2>, p, grid, 16, lds, stream);
+      return sk_launch(skinny_qint8_fq_kernel<3, 4, 16, 16, 2, false>, p, grid, 16, lds, stream);
     if (pl.ntw == 2)
-      return sk_launch(skinny_qint8_fq_kernel<2, 4, 16, 16, 4>, p, grid, 16, lds, stream);
+      return sk_launch(skinny_qint8_fq_kernel<2, 4, 16, 16, 4, false>, p, grid, 16, lds, stream);
     // Up to three K blocks (12 weight tiles) per wave: a ring of four tiles; one of eight would hold most of the
     // wave's K range and only delays its first MFMA (4096 x 4096 at one row 6.9 -> 5.9 us).  With more than 16
     // (row, block) items per wave, six quantisation passes are in flight, so that up to 24 items (8 rows x 3 blocks
@@ -1540,10 +1624,10 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
     // (14.0 -> 12.2 us).  From four blocks per wave on the ring of eight wins.
     if (pl.max_units <= 3) {
       if ((int64_t)p.M * pl.max_units > 16)
-        return sk_launch(skinny_qint8_fq_kernel<1, 4, 16, 16, 6>, p, grid, 16, lds, stream);
-      return sk_launch(skinny_qint8_fq_kernel<1, 4, 16, 16, 4>, p, grid, 16, lds, stream);
+        return sk_launch(skinny_qint8_fq_kernel<1, 4, 16, 16, 6, false>, p, grid, 16, lds, stream);
+      return sk_launch(skinny_qint8_fq_kernel<1, 4, 16, 16, 4, false>, p, grid, 16, lds, stream);
     }
-    return sk_launch(skinny_qint8_fq_kernel<1, 8, 16, 16, 4>, p, grid, 16, lds, stream);
+    return sk_launch(skinny_qint8_fq_kernel<1, 8, 16, 16, 4, false>, p, grid, 16, lds, stream);
   }
   size_t lds = ((size_t)pl.waves * pl.ntw * pl.mg * 256 + (size_t)pl.waves * pl.max_units * pl.mg * 16) * sizeof(float);
 #define SKQ(MG, NTW, PF, MAXW, MINW)                                                                   \

@@ -47,6 +47,7 @@ _vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_
 SIGNATURES = {
     "tppx_version": [],
     "tppx_last_error": [],
+    "tppx_reload_env": [],
     "tppx_quantize_mxfp4": [_vp, _i32, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp],
     "tppx_quantize_qint8": [_vp, _i32, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp],
     "tppx_dequantize_mxfp4": [_vp, _vp, _i64, _i64, _vp, _vp],
@@ -132,8 +133,11 @@ def stream_of(t):
 
 
 WORKSPACE_BYTES = 32 << 20
+MAX_STREAM_WORKSPACES = 8  # per device; the least recently used one beyond that is released
 _workspaces = {}
 _workspaces_lock = threading.Lock()
+_workspace_use = {}  # (device, stream) -> tick of its last use
+_tick = 0
 
 
 def workspace(t):
@@ -144,7 +148,11 @@ def workspace(t):
     stream capture uses one more buffer per device, created together with the
     device's first eager one (a capture cannot allocate it): run the op once
     eagerly before capturing, and order replays of different graphs that use
-    these ops with respect to each other."""
+    these ops with respect to each other.  A device keeps at most
+    MAX_STREAM_WORKSPACES per-stream buffers: beyond that the least recently
+    used one goes back to torch's allocator (it was allocated on its own stream,
+    so work still queued there keeps it valid)."""
+    global _tick
     dev = t.device.index
     if torch.cuda.is_current_stream_capturing():
         ws = _workspaces.get((dev, "capture"))
@@ -162,8 +170,15 @@ def workspace(t):
                     cap = torch.zeros(WORKSPACE_BYTES, dtype=torch.uint8, device=t.device)
                     torch.cuda.current_stream(t.device).synchronize()  # zeroed before any capture stream sees it
                     _workspaces[(dev, "capture")] = cap
+                mine = [k for k in _workspace_use if k[0] == dev]
+                if len(mine) >= MAX_STREAM_WORKSPACES:
+                    old = min(mine, key=_workspace_use.get)
+                    _workspace_use.pop(old)
+                    _workspaces.pop(old, None)
                 ws = torch.zeros(WORKSPACE_BYTES, dtype=torch.uint8, device=t.device)
                 _workspaces[key] = ws
+    _tick += 1
+    _workspace_use[key] = _tick
     return ws
 
 
