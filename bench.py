@@ -178,14 +178,25 @@ def t_bits(t):
 # ---------------------------------------------------------------------------------------------------------------
 # config 2 (headline)
 # ---------------------------------------------------------------------------------------------------------------
-def run_decode(torch, _ops, args):
+def run_decode(torch, _ops, args, per_channel=False):
+    """per_channel: one scale per output channel (QINT8_BLOCK_SIZE = K for each weight: 4096 on the up-projection,
+    11008 on the down-projection) instead of the reference default of 256-wide blocks."""
     dev = torch.device("cuda:0")
     fmt = args.fmt
     shapes = dict(CFG2_SHAPES)
     Ms = list(CFG2_MS)
-    qbs = 256
+    qbs = {name: (K if per_channel else 256) for name, (N, K) in shapes.items()}
     W, X, R = make_inputs(torch, shapes, Ms, 1236)
-    quant = _ops.remap_and_quantize_qint8 if fmt == "qint8" else _ops.remap_and_quantize_mxfp4
+
+    def quant(t):
+        if fmt != "qint8":
+            return _ops.remap_and_quantize_mxfp4(t)
+        old = _ops.QINT8_BLOCK_SIZE
+        _ops.QINT8_BLOCK_SIZE = t.shape[1] * t.shape[2] * t.shape[4] if per_channel else 256
+        try:
+            return _ops.remap_and_quantize_qint8(t)
+        finally:
+            _ops.QINT8_BLOCK_SIZE = old
 
     # pool of weight sets: every (set, shape, M) gets its own copy so a step
     # touches len(Ms) * (45+45) MB = 360 MB of distinct weight bytes (QINT8)
@@ -209,7 +220,7 @@ def run_decode(torch, _ops, args):
                 outs.append(torch.ops.tpp_llm.fc_add(Xd[(name, M)], ws[(name, M)], empty, Rd[(name, M)], 1.0))
         return outs
 
-    bytes_per_step = sum(algorithmic_bytes(fmt, M, N, K, qbs) for (N, K) in shapes.values() for M in Ms)
+    bytes_per_step = sum(algorithmic_bytes(fmt, M, N, K, qbs[name]) for name, (N, K) in shapes.items() for M in Ms)
     flops_per_step = sum(2 * M * N * K for (N, K) in shapes.values() for M in Ms)
 
     graphs = None
@@ -264,13 +275,14 @@ def run_decode(torch, _ops, args):
         "dtype": "int8" if fmt == "qint8" else "bf16",
         "data": "synthetic",
         "config": {
-            "workload": ("cfg2: QINT8 W8A8 (QBS=256) fc_add" if fmt == "qint8" else "MXFP4 fc_add")
+            "workload": (("cfg2: QINT8 W8A8 (per-output-channel scales, QBS=K) fc_add" if per_channel else
+                          "cfg2: QINT8 W8A8 (QBS=256) fc_add") if fmt == "qint8" else "MXFP4 fc_add")
             + ", Llama-7B MLP up 4096->11008 + down 11008->4096, M in {1,8,32,64}; one step = these 8 fused linears",
             "launch": "hipGraph replay of one step" if graphs is not None else "eager launches",
             "timed": f"{blocks} blocks of exactly {args.steps} steps, each between two synchronizes (>= {MIN_WALL_S} s in "
                      f"all); ms_per_step is their mean",
-            "weight_pool_MB": round(len(pool) * len(Ms) * sum(algorithmic_bytes(fmt, 0, N, K, qbs, post_in=False)
-                                                              for (N, K) in shapes.values()) / 1e6, 1),
+            "weight_pool_MB": round(len(pool) * len(Ms) * sum(algorithmic_bytes(fmt, 0, N, K, qbs[name], post_in=False)
+                                                              for name, (N, K) in shapes.items()) / 1e6, 1),
             "bytes_per_step": bytes_per_step,
             "tflops": round(flops_per_step / (ms_per_step * 1e-3) / 1e12, 2),
         },
@@ -279,7 +291,7 @@ def run_decode(torch, _ops, args):
     }
 
 
-def roofline_decode(torch, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
+def roofline_decode(torch, fmt, pool, Xd, Rd, Ms, shapes, qbs_by_shape, args):
     """Each GEMM kernel of the step alone, between two events on the launch
     stream.  One graph per (shape, M) holds one launch per weight copy of that
     shape in the pool (> 256 MB, so every launch streams from HBM).  For QINT8
@@ -298,14 +310,15 @@ def roofline_decode(torch, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
             x, r = Xd[(name, M)], Rd[(name, M)]
             y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
             copies = [w.native() for wset in pool for (nm, _m), w in wset.items() if nm == name]
+            qb = qbs_by_shape[name]
             if fmt == "qint8":
                 xq = torch.empty(((M + 63) // 64 * 64, K), dtype=torch.int8, device=dev)
-                sa = torch.empty(((M + 63) // 64 * 64, K // qbs), dtype=torch.float32, device=dev)
+                sa = torch.empty(((M + 63) // 64 * 64, K // qb), dtype=torch.float32, device=dev)
                 keep += [xq, sa]
 
-                def call(qn, sn, flags, st):
+                def call(qn, sn, flags, st, qb=qb):
                     _lib.check(L.tppx_linear_qint8(x.data_ptr(), xq.data_ptr(), sa.data_ptr(), qn.data_ptr(),
-                                                   sn.data_ptr(), None, r.data_ptr(), None, y.data_ptr(), M, N, K, qbs,
+                                                   sn.data_ptr(), None, r.data_ptr(), None, y.data_ptr(), M, N, K, qb,
                                                    3, 1.0, flags, ws.data_ptr(), ws.numel(), st))
                 reuse = _lib.FLAG_XQ_REUSE
             else:
@@ -314,8 +327,8 @@ def roofline_decode(torch, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
                                                    y.data_ptr(), M, N, K, 3, 1.0, flags, ws.data_ptr(), ws.numel(), st))
                 reuse = 0
             keep += [y]
-            plan_call = kernel_plan(L, fmt, M, N, K, qbs, 0, ws.numel())       # what an op call enqueues
-            plan = kernel_plan(L, fmt, M, N, K, qbs, reuse, ws.numel())        # what is timed here
+            plan_call = kernel_plan(L, fmt, M, N, K, qb, 0, ws.numel())       # what an op call enqueues
+            plan = kernel_plan(L, fmt, M, N, K, qb, reuse, ws.numel())        # what is timed here
             call(copies[0][0], copies[0][1], 0, stream)  # quantizes the activation where the path keeps it
             torch.cuda.synchronize()
 
@@ -324,16 +337,26 @@ def roofline_decode(torch, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
                     call(qn, sn, reuse, st)
 
             avg_us, n_launch = events_us(torch, fire, len(copies), use_graph=not args.no_graph)
-            nbytes = algorithmic_bytes(fmt, M, N, K, qbs)
+            call_us = avg_us
+            if len(plan_call) > len(plan):  # the whole call: activation quantizer + GEMM
+
+                def fire_call(st):
+                    for qn, sn in copies:
+                        call(qn, sn, 0, st)
+
+                call_us, _ = events_us(torch, fire_call, len(copies), use_graph=not args.no_graph)
+            nbytes = algorithmic_bytes(fmt, M, N, K, qb)
             rows.append({
                 "kernel": plan[-1][0] if plan else "?",
                 "launch": plan[-1][1] if plan else "",
                 "call": f"{name} M={M} N={N} K={K}",
                 "kernels_per_call": len(plan_call),
                 "avg_launch_us": round(avg_us, 3),
+                "call_us": round(call_us, 3),
                 "bytes_per_launch": nbytes,
                 "achieved": round(nbytes / avg_us / 1e3, 1),
                 "frac": round(nbytes / avg_us / 1e3 / HBM_PEAK_GBS, 4),
+                "call_frac": round(nbytes / call_us / 1e3 / HBM_PEAK_GBS, 4),
                 "launches_timed": n_launch,
             })
     # the dominant kernel = the one a step spends most time in (each runs once per step)
@@ -351,7 +374,8 @@ def roofline_decode(torch, fmt, pool, Xd, Rd, Ms, shapes, qbs, args):
         "avg_launch_us": dom["avg_launch_us"],
         "bytes_per_launch": dom["bytes_per_launch"],
         "launches_timed": dom["launches_timed"],
-        "timing": "events on the launch stream around graph replays of this kernel alone",
+        "timing": "events on the launch stream around graph replays of this kernel alone; frac = the call's algorithmic "
+                  "bytes / the GEMM kernel's time, call_frac = the same bytes / (activation quantizer + GEMM)",
         "all_gemm_kernels": rows,
     }
 
@@ -380,7 +404,7 @@ def cpu_baseline_decode(fmt, W, X, R, Ms, shapes, qbs, bytes_per_step, seconds=1
     qw = {}
     for name in shapes:
         Wf = W[name].float().numpy()
-        qw[name] = O.remap_quantize_qint8(Wf)[:2] if fmt == "qint8" else O.remap_quantize_mxfp4(Wf)
+        qw[name] = O.remap_quantize_qint8(Wf, env_block=qbs[name])[:2] if fmt == "qint8" else O.remap_quantize_mxfp4(Wf)
     lin = O.linear_qint8 if fmt == "qint8" else O.linear_mxfp4
     xs = {k: t_bits(v) for k, v in X.items()}
     rs = {k: t_bits(v) for k, v in R.items()}
@@ -546,7 +570,8 @@ def leg_cfg3(torch, _ops, args):
                     "alternate; HIP graph replay",
         "bytes_per_step": bytes_per_step, "per_M": per_m,
         "roofline": {"bound": "hbm", "kernel": dom["kernel"], "call": dom["call"], "achieved": dom["achieved"],
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"], "traffic": None,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"],
+                     "traffic": measured_traffic(dom["kernel"], dom["call"]),
                      "avg_launch_us": dom["avg_launch_us"], "bytes_per_launch": dom["bytes_per_launch"],
                      "launches_timed": dom["launches_timed"], "all_gemm_kernels": rows},
         "cpu_baseline": cpu,
@@ -618,7 +643,7 @@ def leg_cfg4(torch, _ops, args, pfmt="mxfp4", fp8=False, cpu=True):
                          "achieved": round(fl / us / 1e6, 1), "frac": round(fl / us / 1e6 / peak, 4),
                          "launches_timed": n})
         dom = max(rows, key=lambda r: r["avg_launch_us"] if r["call"].startswith("down") else 0)
-        cpu_b = cpu_baseline_prefill(H) if (cpu and not args.no_cpu and pfmt == "mxfp4" and not fp8) else None
+        cpu_b = cpu_baseline_prefill(H, pfmt) if (cpu and not args.no_cpu and not fp8) else None
     finally:
         _ops.ACT_FP8 = old_fp8
     label = ("cfg4: MXFP4" + (" weights x MXFP8 activations (opt-in, NOT the reference's arithmetic)" if fp8 else
@@ -633,7 +658,8 @@ def leg_cfg4(torch, _ops, args, pfmt="mxfp4", fp8=False, cpu=True):
         "flops_per_step": flops,
         "roofline": {"bound": "mfma", "kernel": dom["kernel"], "call": dom["call"] +
                      (" (activation quantiser included)" if (fp8 or pfmt == "qint8") else ""),
-                     "achieved": dom["achieved"], "peak": peak, "unit": unit, "frac": dom["frac"], "traffic": None,
+                     "achieved": dom["achieved"], "peak": peak, "unit": unit, "frac": dom["frac"],
+                     "traffic": measured_traffic(dom["kernel"], dom["call"]),
                      "avg_launch_us": dom["avg_launch_us"], "flops_per_launch": dom["flops_per_launch"],
                      "launches_timed": dom["launches_timed"],
                      "timing": "events on the launch stream around eager launches of this op alone",
@@ -642,21 +668,28 @@ def leg_cfg4(torch, _ops, args, pfmt="mxfp4", fp8=False, cpu=True):
     }
 
 
-def cpu_baseline_prefill(H, seconds=8.0):
-    """The oracle's MXFP4 linear on a bounded sample: 256 rows through an 8192 x 8192 projection, faithful mode."""
+def cpu_baseline_prefill(H, pfmt="mxfp4", seconds=8.0):
+    """The oracle's MXFP4 (or QINT8) linear on a bounded sample: 256 rows through a 2048 x 8192 slice of a
+    projection, faithful mode."""
     import numpy as np
     O, cores = oracle_mod()
     rng = np.random.default_rng(7)
     Ms, N = 256, 2048
     W = (rng.standard_normal((N, H), dtype=np.float32) * 0.02).astype(np.float32)
-    q, sc = O.remap_quantize_mxfp4(W)
     xf = rng.standard_normal((Ms, H), dtype=np.float32)
     xb = (xf.view(np.uint32) >> 16).astype(np.uint16)  # truncation is fine for a timing input
-    n, dt = repeat_for(lambda: O.linear_mxfp4(xb, q, sc, None, O.POST_NONE, None, None, 1.0, O.MODE_FAITHFUL), seconds, 200)
+    if pfmt == "mxfp4":
+        q, sc = O.remap_quantize_mxfp4(W)
+        lin = O.linear_mxfp4
+    else:
+        q, sc, _ = O.remap_quantize_qint8(W)
+        lin = O.linear_qint8
+    n, dt = repeat_for(lambda: lin(xb, q, sc, None, O.POST_NONE, None, None, 1.0, O.MODE_FAITHFUL), seconds, 200)
     fl = 2.0 * Ms * N * H
-    return {"value": round(fl * n / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"{n} passes of a {Ms} x {N} x {H} MXFP4 linear (C/OpenMP restatement of the reference recipe, "
-                      f"faithful mode; not the libxsmm JIT), {round(dt / n * 1e3, 1)} ms each"}
+    return {"value": round(fl * n / dt / 1e12, 4), "unit": "TFLOP/s" if pfmt == "mxfp4" else "TOP/s", "cores": cores,
+            "kind": "port",
+            "sample": f"{n} passes of a {Ms} x {N} x {H} {pfmt.upper()} linear (C/OpenMP restatement of the reference "
+                      f"recipe, faithful mode; not the libxsmm JIT), {round(dt / n * 1e3, 1)} ms each"}
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -709,10 +742,11 @@ def leg_cfg5(torch, args, B, cpu=True):
                     f"context {ctx} of N(0,1), greedy decode of {new} tokens, batch {B}; one HIP graph per decode step, "
                     f"replayed; {runs} runs of {new} steps timed",
         "wall_s_one_run_including_capture": round(wall_with_capture, 4), "tokens_per_run": int(out.numel()),
-        "roofline": {"bound": "hbm", "kernel": "whole decode step (all kernels of the graph; per-kernel durations in "
-                                               f"profiles/decoder_step_kernels_cfg5_batch{B}_stats.txt)",
+        "roofline": {"bound": "hbm", "kernel": "whole decode step (one graph)",
+                     "per_kernel": f"profiles/decoder_step_kernels_cfg5_batch{B}_stats.txt",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": measured_traffic("whole decode step", f"cfg5 batch {B}"),
                      "bytes_per_step": int(lin_bytes + kv_bytes)},
         "cpu_baseline": cpu_b,
     }
@@ -806,6 +840,77 @@ def run_prompt(torch, args):
         "cpu_baseline": None}
 
 
+def short_kernel(name):
+    return name.replace("tppx::", "").replace("_kernel", "").replace(" ", "")
+
+
+def compact_rows(rows):
+    """[kernel, call, GEMM-kernel us, frac of peak, kernels per call, whole-call us] per GEMM of a leg."""
+    out = []
+    for r in rows:
+        row = [short_kernel(r["kernel"]), r["call"].split(" N=")[0].split(" (")[0], round(r["avg_launch_us"], 2),
+               round(r["frac"], 3)]
+        if r["kernels_per_call"] > 1:  # a quantizer launch in front: kernels per call, whole-call us
+            row += [r["kernels_per_call"], round(r.get("call_us", r["avg_launch_us"]), 2)]
+        out.append(row)
+    return out
+
+
+def compact_roofline(r, leg=False):
+    if not r:
+        return r
+    keep = ("bound", "kernel", "call", "achieved", "peak", "unit", "frac", "traffic", "avg_launch_us") + \
+        (() if leg else ("bytes_per_launch", "flops_per_launch", "bytes_per_step"))
+    out = {k: r[k] for k in keep if k in r}
+    out["kernel"] = short_kernel(out.get("kernel", ""))[:40]
+    if "call" in out:
+        out["call"] = out["call"].split(" (")[0]
+    return out
+
+
+def compact_cpu(c, leg=False):
+    if not c:
+        return c
+    out = dict(c)
+    out["sample"] = out.get("sample", "").split(" (")[0][:70 if leg else 110]
+    return out
+
+
+def compact_leg(leg):
+    """What the one-line record keeps of a leg (the verbose form goes to stderr)."""
+    if "roofline" not in leg:
+        return leg
+    # value, unit, ms_per_step, the dominant kernel, its duration and fraction are in the line's `summary` row of the leg
+    roof = compact_roofline(leg["roofline"], True)
+    for k in ("kernel", "avg_launch_us", "frac"):
+        roof.pop(k, None)
+    out = {"leg": leg["leg"], "dtype": leg["dtype"],
+           "workload": leg["workload"].split(";")[0].split(" linears of")[0][:72], "roofline": roof,
+           "cpu_baseline": compact_cpu(leg["cpu_baseline"], True)}
+    rows = leg["roofline"].get("all_gemm_kernels")
+    if rows:
+        out["gemm_kernels"] = compact_rows(rows)
+    return out
+
+
+def summary_of(headline, legs):
+    """One row per leg, the headline first: [leg, value, unit, ms_per_step, dominant kernel, its us, its fraction of
+    the roofline, HBM traffic / algorithmic bytes (or None), CPU value].  The LAST key of the line."""
+    rows = []
+    for name, d in [("cfg2", headline)] + [(l.get("leg"), l) for l in legs]:
+        r = d.get("roofline")
+        if not r:
+            rows.append([name, d.get("error") or d.get("skipped")])
+            continue
+        tr = r.get("traffic")
+        ratio = round(tr / r["bytes_per_launch"], 3) if tr and r.get("bytes_per_launch") else None
+        cpu = d.get("cpu_baseline") or {}
+        rows.append([name, d["value"], d["unit"], d.get("ms_per_step", round(d.get("us_per_call", 0.0) / 1e3, 6)),
+                     short_kernel(r.get("kernel", ""))[:40],
+                     r.get("avg_launch_us"), r.get("frac"), ratio, cpu.get("value")])
+    return rows
+
+
 def leg_as_line(leg, args):
     """A leg run alone (--workload ...) printed in the shape of the headline line."""
     return {"metric": leg["metric"], "value": leg["value"], "unit": leg["unit"], "n_gpus": 1, "steps": args.steps,
@@ -868,7 +973,15 @@ def main():
     out = run_decode(torch, _ops, args)
     if args.workload == "all":
         legs = []
+
+        def per_channel_leg():
+            d = run_decode(torch, _ops, args, per_channel=True)
+            return {"leg": "cfg2-per-channel", "metric": d["metric"], "value": d["value"], "unit": d["unit"],
+                    "ms_per_step": d["ms_per_step"], "dtype": d["dtype"], "workload": d["config"]["workload"],
+                    "roofline": d["roofline"], "cpu_baseline": d["cpu_baseline"]}
+
         todo = [
+            ("cfg2-per-channel", per_channel_leg),
             ("cfg1", lambda: leg_cfg1(torch, _ops, args)),
             ("cfg3", lambda: leg_cfg3(torch, _ops, args)),
             ("cfg4", lambda: leg_cfg4(torch, _ops, args, "mxfp4", False)),
@@ -891,9 +1004,22 @@ def main():
             torch.cuda.synchronize()
             torch.cuda.empty_cache()
         _MODEL.clear()
-        out["config"]["legs"] = legs
+        # the verbose record (launch shapes, launch counts, full kernel names) goes to stderr, one line per leg; the
+        # one line on stdout keeps every leg in a compact form and ends with a summary row per leg
+        print("bench.py verbose: " + json.dumps({"leg": "cfg2", "roofline": out["roofline"], "config": out["config"]}),
+              file=sys.stderr)
+        for leg in legs:
+            print("bench.py verbose: " + json.dumps(leg), file=sys.stderr)
+        out["config"]["legs"] = [compact_leg(l) for l in legs]
         out["config"]["run_wall_s"] = round(time.perf_counter() - t_start, 1)
-    print(json.dumps(out))
+        out["config"]["gemm_kernels_columns"] = "kernel, call, GEMM kernel us, frac of peak[, kernels per call, whole-call us]"
+        out["config"].pop("timed", None)
+        out["config"]["gemm_kernels"] = compact_rows(out["roofline"].pop("all_gemm_kernels"))
+        out["roofline"] = compact_roofline(out["roofline"])
+        out["cpu_baseline"] = compact_cpu(out["cpu_baseline"])
+        out["summary_columns"] = "leg, value, unit, ms_per_step, dominant kernel, its us, frac of roofline, HBM traffic / algorithmic bytes, cpu value"
+        out["summary"] = summary_of(out, legs)
+    print(json.dumps(out, separators=(",", ":")))
 
 
 if __name__ == "__main__":
