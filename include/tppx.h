@@ -278,8 +278,11 @@ int tppx_linear_qint8(const void* x, void* xq, void* sa, const void* qw,
  * shapes), K <= 32768 -- larger sizes return TPPX_ESHAPE; flags: 0 or TPPX_FLAG_FORCE_SKINNY.  Same kernels and
  * the same bits as tppx_linear_qint8 with a 2 MiB workspace.  The call itself allocates nothing and frees nothing.
  * All calls on one GPU share the one array: calls that overlap on a GPU (different streams without ordering)
- * race; order them on one stream or with events.  Nothing in the array has to start at zero (every byte read was
- * written earlier in the same call). */
+ * race; order them on one stream or with events.  Nothing in the array has to start at zero: every value that reaches
+ * an output was written earlier in the same call (the padding rows of the last 16-row tile of quantised
+ * activations are read as they lie, but the results of those rows are never stored).  The first call on a device
+ * looks up the array's address (hipGetSymbolAddress, which may load the code object): make one eager call per
+ * device before recording the entry point into a graph. */
 int tppx_linear_qint8_noalloc(const void* x, const void* qw, const void* sw,
                               const void* bias, const void* post_in,
                               const void* post_in2, void* y, int64_t M,

@@ -230,3 +230,73 @@ def test_launch_plans_of_the_baseline_shapes():
     assert len(lines) == 1 and "big_mxfp4_kernel<8, true, 1, 8> grid=1792x1x1" in lines[0]       # silu*mul in the epilogue
     lines = plan(L.tppx_plan_multi_linear_mxfp4, pair, 2, 2048, 8192, 1, _lib.FLAG_ACT_FP8, 1 << 28)
     assert any("big_fp8_kernel<8, true> grid=1792x1x1" in l for l in lines), lines
+
+
+def test_launch_plans_of_per_output_channel_qint8():
+    """QINT8 with one scale block = all of K (and other multiples of 256): up to 16 rows the quantisation stays inside
+    the GEMM launch (maxima exchanged between the waves), above that the big-block quantizer runs in front; all 8 or
+    16 waves of a workgroup get a share of K (the grid and block are those of the 256-wide default)."""
+    import ctypes
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    buf = ctypes.create_string_buffer(4096)
+
+    def plan(*args):
+        _lib.check(L.tppx_plan_linear_qint8(*args, buf, len(buf)))
+        return buf.value.decode().strip().splitlines()
+
+    ws = 1 << 25
+    for M in (1, 8):
+        one = plan(M, 11008, 4096, 4096, 1, 0, ws)
+        assert len(one) == 1 and "skinny_qint8_fq_kernel<3, 4, 16, 16, 4, true> grid=230x1x1 block=1024" in one[0], one
+        one = plan(M, 4096, 11008, 11008, 1, 0, ws)
+        assert len(one) == 1 and "skinny_qint8_fq_kernel<1, 4, 16, 16, 6, true> grid=256x1x1 block=1024" in one[0], one
+    two = plan(64, 11008, 4096, 4096, 1, 0, ws)
+    assert len(two) == 2 and "quant_act_int8_bigblk_kernel grid=64x1x1 block=256" in two[0], two
+    assert "skinny_qint8_kernel<4, 3, 2, 8, 8, true> grid=230x1x1 block=512" in two[1], two
+    two = plan(64, 4096, 11008, 11008, 1, 0, ws)
+    assert "quant_act_int8_bigblk_kernel grid=64x1x1 block=704" in two[0] and "grid=128x1x2" in two[1], two
+    # a block that is not a whole number of 256-wide runs is dealt tile by tile: still one GEMM launch, quantizer in front
+    odd = plan(5, 512, 1280, 320, 1, 0, ws)
+    assert len(odd) == 2 and "quant_act_int8_kernel" in odd[0] and "skinny_qint8_kernel<1, 1, 4, 16, 4, true>" in odd[1], odd
+
+
+def test_environment_switches_are_read_once(monkeypatch):
+    """The library keeps a TPPX_* switch after its first read (no getenv per launch, and a captured graph's kernel
+    choice cannot drift); tppx_reload_env() makes it read again."""
+    import ctypes
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    buf = ctypes.create_string_buffer(4096)
+
+    def plan():
+        _lib.check(L.tppx_plan_linear_qint8(1, 4096, 4096, 256, 1, 0, 0, buf, len(buf)))
+        return buf.value.decode()
+
+    L.tppx_reload_env()
+    assert "skinny_qint8_fq_kernel" in plan()
+    os.environ["TPPX_SKINNY_FUSEDQ"] = "0"
+    try:
+        assert "skinny_qint8_fq_kernel" in plan(), "the switch was read again without a reload"
+        L.tppx_reload_env()
+        assert "skinny_qint8_fq_kernel" not in plan() and "quant_act_int8" in plan()
+    finally:
+        del os.environ["TPPX_SKINNY_FUSEDQ"]
+        L.tppx_reload_env()
+    assert "skinny_qint8_fq_kernel" in plan()
+
+
+def test_cache_lengths_after_graph_replayed_steps():
+    """Steps replayed from a graph move the device counter themselves; the host bookkeeping that follows them must
+    move every layer's length, so that get_seq_length(layer) and a later update() on any layer see the new keys."""
+    from tpp_pytorch_extension.llm.fused_llama_infer import TppCache
+    cache = TppCache(64)
+    kv = torch.zeros((1, 2, 5, 8), dtype=torch.bfloat16)
+    for i in range(3):
+        cache.fill_(i, kv, kv)
+    cache._advance_host(4)  # what greedy_decode / time_decode_steps do per replay
+    assert [cache.get_seq_length(i) for i in range(3)] == [9, 9, 9]
+    one = torch.ones((1, 2, 1, 8), dtype=torch.bfloat16)
+    k, v = cache.update(one, one, 2)
+    assert k.shape[2] == 10 and cache.get_seq_length(2) == 10 and cache.get_seq_length(1) == 9
+    assert float(k[0, 0, 9, 0]) == 1.0 and float(k[0, 0, 8, 0]) == 0.0

@@ -255,3 +255,35 @@ def test_cfg5_full_size_layer_step(B):
     assert_close_bf16(t2bits(kc[:, :, ctx]), k.reshape(B, Nh, H), what="cached key")
     assert_close_bf16(t2bits(vc[:, :, ctx]), v.reshape(B, Nh, H), what="cached value")
     assert torch.equal(kc[:, :, :ctx].cpu(), k0)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# config 5 as bench.py runs it: the 32-layer 7B-shape decoder, 2048-token context, 128 greedy tokens from one
+# replayed graph.  No oracle finishes 32 layers x 128 steps in seconds, so the chain is held by properties: the
+# replayed steps give the tokens of eager launches of the same kernels (first 8 steps), every token is a vocabulary
+# id, the counters end at 2048 + 128 in every layer, and the appended keys are there (non-zero) and nothing beyond.
+# ---------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("B", [1, 16])
+def test_cfg5_full_size_greedy_chain(B):
+    import bench
+    model = bench.cfg5_model(torch)
+    assert model.n_layers == 32 and model.hidden == 4096 and model.vocab == 32000
+    ctx, new = 2048, 128
+    tok = torch.randint(0, 32000, (B,), generator=torch.Generator().manual_seed(5), dtype=torch.int64).cuda()
+    cache = model.new_cache(B, ctx, ctx + new + 32)
+    out = model.greedy_decode(tok, cache, new)  # one graph, 128 replays
+    torch.cuda.synchronize()
+    assert out.shape == (B, new) and int(out.min()) >= 0 and int(out.max()) < 32000
+    assert int(cache.seq_len_dev.item()) == ctx + new
+    assert [cache.get_seq_length(i) for i in (0, 15, 31)] == [ctx + new] * 3
+    for i in (0, 31):
+        k, v = cache.layers[i]
+        assert bool((k[:, :, ctx:ctx + new].float().abs().amax(dim=-1) > 0).all()), "a replayed step left no key"
+        assert float(k[:, :, ctx + new:].float().abs().max()) == 0.0 and float(v[:, :, ctx + new:].float().abs().max()) == 0.0
+    del cache
+    eager_cache = model.new_cache(B, ctx, ctx + new + 32)  # same seed: the same context
+    eager = model.greedy_decode(tok, eager_cache, 8, use_graph=False)
+    assert torch.equal(out[:, :8], eager), "replayed steps and eager steps give different tokens"
+    del eager_cache
+    bench._MODEL.clear()
+    torch.cuda.empty_cache()

@@ -51,3 +51,40 @@ def test_noalloc_entry_point_equals_caller_scratch_entry_point():
     assert L.tppx_linear_qint8_noalloc(A, A, A, None, None, None, A, 1, 16, 32768 + 256, 256, 0, 1.0, 0, None) == _lib.ESHAPE
     assert L.tppx_linear_qint8_noalloc(None, A, A, None, None, None, A, 1, 16, 256, 256, 0, 1.0, 0, None) == _lib.EINVAL
     assert L.tppx_linear_qint8_noalloc(A, A, A, None, None, None, A, 1, 16, 256, 256, 0, 1.0, _lib.FLAG_XQ_REUSE, None) == _lib.EINVAL
+
+
+def test_noalloc_entry_point_inside_graph_capture():
+    """After one eager call on the device (which takes the static array's address), the entry point can be recorded
+    into a HIP graph -- it allocates nothing -- and every replay gives the bits of the eager call, on the fused-
+    quantisation path (8 rows), the quantizer + GEMM path (40 rows) and the K-split path (64 rows, long K)."""
+    import tpp_pytorch_extension  # noqa: F401
+    from tpp_pytorch_extension import _lib, _ops
+    L = _lib.lib()
+    for i, (M, N, K) in enumerate([(8, 512, 1024), (40, 256, 2048), (64, 4096, 11008)]):
+        W = randn_bf16((N, K), 0.02, 9950 + i)
+        qw = _ops.remap_and_quantize_qint8(block_bf16(W).cuda())
+        qn, sn = qw.native()
+        x = randn_bf16((M, K), 1.0, 9960 + i).cuda()
+        r = randn_bf16((M, N), 1.0, 9970 + i).cuda()
+        y_eager = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+        y_graph = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+
+        def call(y):
+            _lib.check(L.tppx_linear_qint8_noalloc(x.data_ptr(), qn.data_ptr(), sn.data_ptr(), None, r.data_ptr(), None,
+                                                   y.data_ptr(), M, N, K, 256, _lib.POST_ADD_SCALE, 1.0, 0,
+                                                   _lib.stream_of(x)))
+
+        call(y_eager)
+        torch.cuda.synchronize()
+        # capture_error_mode="global" (torch's default, spelled out): a hipMalloc / hipFree or any other call that is
+        # illegal under capture, from any thread, fails the capture -- so a capture that succeeds allocated nothing
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, capture_error_mode="global"):
+            call(y_graph)
+        for rep in range(3):
+            y_graph.zero_()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y_graph, y_eager), f"case {i}: replay {rep} differs from the eager call"
+            call(y_eager)  # eager work of the same entry point between the replays
+            torch.cuda.synchronize()

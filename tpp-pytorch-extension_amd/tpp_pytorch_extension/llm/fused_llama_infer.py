@@ -142,6 +142,13 @@ class TppCache:
         self._sync_len = self._host_len
         self._layer_len = {}
 
+    def _advance_host(self, n=1):
+        """Host-side bookkeeping alone, for steps whose device counter moved inside a replayed graph: every layer
+        holds n more keys."""
+        self._host_len += n
+        self._sync_len = self._host_len
+        self._layer_len = {}
+
     def update(self, key_states, value_states, layer_idx):
         """TppCache::update / LayerCache::update (src/csrc/llm/attn.h:198-222,258-274): append key_states /
         value_states [B][Nkv][S][H] (bf16, already rotated) to layer `layer_idx` at that layer's length and return
@@ -410,7 +417,9 @@ class LlamaDecoder:
         for _ in range(n_new - 1):
             graph.replay()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * n_new / (n_new - 1)
+        dt = time.perf_counter() - t0
+        cache._advance_host(n_new)  # every replay moved the device counter
+        return dt * n_new / (n_new - 1)
 
     def greedy_decode(self, tokens, cache, n_new, use_graph=True):
         """Greedy decode of n_new tokens per sequence from the [B] start tokens; returns i64 [B][n_new]."""
@@ -440,7 +449,7 @@ class LlamaDecoder:
             for t in range(n_new):
                 graph.replay()
                 out[:, t].copy_(cur)
-                cache._host_len += 1
+                cache._advance_host(1)
         else:
             for t in range(n_new):
                 nxt = self.step(cur, pos, cache)
