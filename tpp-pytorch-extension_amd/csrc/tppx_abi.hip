@@ -220,7 +220,8 @@ static const int64_t TILED_MIN_M = 65; // more rows than the decode kernels cove
 // cost estimate fitted to measurements on MI355X (us): a block row costs about 8 + weight bytes / 5.5 TB/s + 0.8 ns
 // per input channel (its activations), a round of 256 x 256 tiles about 14.5 ns per input channel (128 x 128: 20).  `wbytes` = weight bytes of the whole call, `n_tiles16` = its 16-channel
 // tiles.  TPPX_TILED_MIN_M (when set) restores a plain row threshold.
-static bool want_tiled(int64_t M, int flags, int64_t K = 0, int64_t n_tiles16 = 0, double wbytes = 0.0) {
+static bool want_tiled(int64_t M, int flags, int64_t K = 0, int64_t n_tiles16 = 0, double wbytes = 0.0,
+                       bool small_tiles_only = false) {
   if (flags & TPPX_FLAG_FORCE_SKINNY)
     return false;
   if (flags & TPPX_FLAG_FORCE_TILED)
@@ -232,7 +233,7 @@ static bool want_tiled(int64_t M, int flags, int64_t K = 0, int64_t n_tiles16 = 
     return M >= env_min;
   if (K <= 0 || n_tiles16 <= 0 || M > 1024)
     return true;
-  const bool big = M >= env_int("TPPX_TILED_BIG_MIN_M", 192);
+  const bool big = !small_tiles_only && M >= env_int("TPPX_TILED_BIG_MIN_M", 192);
   const int64_t rows = big ? 256 : 128, cols16 = big ? 16 : 8;
   const int64_t wgs = ((M + rows - 1) / rows) * ((n_tiles16 + cols16 - 1) / cols16);
   const double tiled_us = (double)((wgs + 255) / 256) * (double)K * 0.0145 * (big ? 1.0 : 1.4);
@@ -646,7 +647,7 @@ extern "C" int tppx_linear_bf16(const void* x, const void* w, const void* bias, 
   if (rc)
     return rc;
   TPPX_REQUIRE(K > 0 && K % 128 == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of 128 (native bf16 tiles span 128 input channels)", who, (long)K);
-  TPPX_REQUIRE(!(flags & (TPPX_FLAG_ACT_FP8 | TPPX_FLAG_FORCE_TILED)), TPPX_EUNSUPPORTED, "%s: only the row-group kernel is built for unquantized weights", who);
+  TPPX_REQUIRE(!(flags & TPPX_FLAG_ACT_FP8), TPPX_EUNSUPPORTED, "%s: FP8 activations are built for MXFP4 weights only", who);
   TPPX_REQUIRE(M * N < ((int64_t)1 << 31), TPPX_ESHAPE, "%s: M*N=%ld outputs exceed 2^31", who, (long)(M * N));
   tppx_seg s = {w, w, bias, post_in, post_in2, y, N, post_op, post_scale}; // no scales: the slot repeats the weight
   DecodeParams p;
@@ -660,6 +661,12 @@ extern "C" int tppx_linear_bf16(const void* x, const void* w, const void* bias, 
   p.units = (int)(K / 128);
   p.tpb = 1;
   p.S = 1;
+  // more than 64 rows: the LDS-tiled kernel once it is the cheaper one (the estimate of the quantized formats with the
+  // weight's real bytes: the row-group kernel streams the whole weight once per 64 rows)
+  if (want_tiled(M, flags, K, p.total_tiles, (double)N * (double)K * 2.0, true)) {
+    TPPX_REQUIRE(aligned16(w), TPPX_EINVAL, "%s: weight not 16-byte aligned", who);
+    return check_hip(launch_tiled_bf16(tiled_from_seg(p, 0), (hipStream_t)stream), who);
+  }
   const int mg = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   const int nt = p.total_tiles > 512 ? 2 : 1; // two channel tiles per workgroup once one each still leaves two rounds
   set_groups(p, nt, false);

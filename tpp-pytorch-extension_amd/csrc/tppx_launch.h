@@ -102,6 +102,8 @@ bool tiled_mxfp4_takes_groups(const TiledParams& p);
 // dual: the gate/up pair (t[0] = gate, t[1] = up) with silu(gate) * up formed in the launch and written to t[1].y
 hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream, bool dual = false);
 hipError_t launch_tiled_qint8(const TiledParams& p, hipStream_t stream);
+// unquantized bf16 weights (native bf16 tiles in p.qw), more than 64 rows
+hipError_t launch_tiled_bf16(const TiledParams& p, hipStream_t stream);
 hipError_t launch_tiled_mxfp4_fp8_group(const TiledParams* t, int n, hipStream_t stream, bool dual = false);
 bool tiled_qint8_takes_groups(const TiledParams& p);
 hipError_t launch_tiled_qint8_group(const TiledParams* t, int n, hipStream_t stream);

@@ -192,6 +192,100 @@ tiled_mxfp4_kernel(const TiledParams p) {
 }
 
 // ---------------------------------------------------------------------------
+// Unquantized bf16 weights at prefill shapes (the prompt pass of a model whose
+// first-token weights stay bf16): the kernel above without the expansion.  The
+// native bf16 tiles [N/16][K/128][4 j][64 lanes][16 B] hold the MFMA operands
+// themselves, 4 KiB per (channel tile, K step) -- eight times the bytes of the
+// packed codes -- so B runs as a ring of the four steps j of a K step: the
+// operand of (ks, j) is requested right behind the MFMAs that consumed
+// (ks - 1, j), a whole K step ahead, and no second register set is needed.
+// All loads are ordinary register loads, so the compiler's partial waits hold.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+tiled_bf16_kernel(const TiledParams p) {
+  extern __shared__ __align__(16) uint8_t tl_lds[];
+  bf16x8* As = reinterpret_cast<bf16x8*>(tl_lds); // 2 buffers x 2048 slots
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int MB = (p.M + 127) >> 7, NB = (p.tiles + 7) >> 3;
+  int bm, bn;
+  tile_of_block(MB, NB, bm, bn);
+  const int KT = p.K >> 7;
+  const int m_wg = bm * 128;
+  const int tile_base = bn * 8 + wn * 4;
+
+  const i32x4* wq[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; nt++) {
+    const int64_t t = min(tile_base + nt, p.tiles - 1);
+    wq[nt] = reinterpret_cast<const i32x4*>(p.qw) + t * KT * 256 + lane;
+  }
+  const uint16_t* xb = reinterpret_cast<const uint16_t*>(p.x);
+  const uint16_t* arow[8];
+#pragma unroll
+  for (int q = 0; q < 8; q++) {
+    const int m = min(m_wg + q * 16 + (tid & 15), p.M - 1);
+    arow[q] = xb + (int64_t)m * p.K + ((tid >> 4) & 3) * 32 + wave * 8;
+  }
+  bf16x8 areg[8];
+  i32x4 bring[4][4]; // [j][nt]
+  auto load_a = [&](int ks) {
+#pragma unroll
+    for (int q = 0; q < 8; q++)
+      areg[q] = *reinterpret_cast<const bf16x8*>(arow[q] + ks * 128);
+  };
+  auto load_b = [&](int ks, int j) {
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++)
+      bring[j][nt] = wq[nt][(int64_t)ks * 256 + j * 64];
+  };
+  auto store_a = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < 8; q++)
+      As[buf * 2048 + q * 256 + tid] = areg[q];
+  };
+
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++)
+      acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  load_a(0);
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+    load_b(0, j);
+  store_a(0);
+  __syncthreads();
+  for (int ks = 0; ks < KT; ks++) {
+    const int buf = ks & 1;
+    const bool more = ks + 1 < KT;
+    if (more)
+      load_a(ks + 1);
+    const bf16x8* Ab = As + buf * 2048 + (wm * 4) * 256 + lane;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      bf16x8 a[4];
+#pragma unroll
+      for (int mt = 0; mt < 4; mt++)
+        a[mt] = Ab[mt * 256 + j * 64];
+#pragma unroll
+      for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[mt], __builtin_bit_cast(bf16x8, bring[j][nt]), acc[mt][nt], 0, 0, 0);
+      if (more)
+        load_b(ks + 1, j);
+    }
+    if (more)
+      store_a(buf ^ 1);
+    __syncthreads();
+  }
+  tiled_epilogue(p, acc, m_wg + wm * 64, tile_base);
+}
+
+// ---------------------------------------------------------------------------
 // QINT8 (W8A8): activations pre-quantised (int8 [M][K], f32 [M][K/qbs]).
 // K step = 128 = two native tiles; LDS A layout per buffer:
 // [mt 8][t 2][lane 64] x 16 B (16 KiB) + the activation scales of the step's
@@ -1233,6 +1327,18 @@ silu_mul_kernel(const uint16_t* __restrict__ gate, uint16_t* __restrict__ y, int
     }
     reinterpret_cast<uint4*>(y)[i] = make_uint4(o[0], o[1], o[2], o[3]);
   }
+}
+
+hipError_t launch_tiled_bf16(const TiledParams& p, hipStream_t stream) {
+  const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
+  const dim3 grid((unsigned)(MB * NB));
+  const size_t lds = 2 * 2048 * 16;
+  TPPX_PLAN_ONLY(tiled_bf16_kernel, grid, dim3(256), lds);
+  hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(tiled_bf16_kernel), lds);
+  if (e != hipSuccess)
+    return e;
+  tiled_bf16_kernel<<<grid, 256, lds, stream>>>(p);
+  return hipGetLastError();
 }
 
 hipError_t launch_silu_mul(const uint16_t* gate, uint16_t* y, int64_t n, hipStream_t stream) {

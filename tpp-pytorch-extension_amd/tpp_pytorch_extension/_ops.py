@@ -580,6 +580,25 @@ def _is_w4a8(w):
     return isinstance(w, QTensor) and w.weight_kind() == "mxfp4_int8"
 
 
+def _is_plain(w):
+    """An unquantized (bf16 / fp32, blocked or flat) weight tensor."""
+    return isinstance(w, torch.Tensor) and not isinstance(w, QTensor)
+
+
+def weight_nk(w):
+    """(output channels, input channels) of a quantized or an unquantized blocked weight."""
+    return tuple(w.weight_nk()) if isinstance(w, QTensor) else tuple(_blocked_geometry(w)[:2])
+
+
+def _one_launch_group(weights):
+    """Do these weights share a fused launch (one quantized format in the default layout)?  Unquantized weights,
+    the W4A8 layout and mixed formats run one GEMM per weight."""
+    if any(_is_plain(w) or _is_w4a8(w) for w in weights):
+        return False
+    return all(w._qscheme == weights[0]._qscheme and w.block_size == weights[0].block_size and
+               w.weight_kind() == weights[0].weight_kind() for w in weights)
+
+
 def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0, flags=0,
            row_sumsq=None):
     """One quantized GEMM with a fused post-op
@@ -703,7 +722,9 @@ def sums_table(device):
 def takes_row_sums(weight, M):
     """Can the GEMM with this weight leave row sums of squares of its output (MXFP4 decode kernels, <= 16 rows,
     at most 256 workgroups of up to three channel tiles: 12288 output channels)?"""
-    w = _as_q(weight)
+    if not isinstance(weight, QTensor):
+        return False
+    w = weight
     return (NORM_FROM_SUMS and w._qscheme == QSCHEME_MXFP and w.weight_kind() == "mxfp4" and 0 < M <= 16
             and w.weight_nk()[0] <= 12288)
 
@@ -795,7 +816,7 @@ def qkv_gemm(input, weights, biases, norm=None):
     the same launch for MXFP4 decode steps, as a separate launch otherwise)."""
     L = _lib.lib()
     weights = list(weights)
-    if any(_is_w4a8(w) for w in weights):  # no fused launch for the W4A8 layout: one GEMM per weight
+    if not _one_launch_group(weights):  # unquantized weights, the W4A8 layout, mixed formats: one GEMM per weight
         if norm is not None:
             input = rms_norm(input, norm[0], norm[1])
         biases = list(biases) if biases is not None else []
@@ -863,7 +884,7 @@ def swiglu_gate_up(input, w_gate, w_up, b_gate=None, b_up=None, norm=None):
     points (fused_llm_infer.cpp:1271-1272).  norm = (gamma, eps): llama_rms_norm
     on the input first (fused_llm_infer.cpp:1269), inside the launch when possible."""
     L = _lib.lib()
-    if _is_w4a8(w_gate) or _is_w4a8(w_up):
+    if not _one_launch_group([w_gate, w_up]):
         if norm is not None:
             input = rms_norm(input, norm[0], norm[1])
         return fc_mul(input, w_up, b_up, fc_silu(input, w_gate, b_gate))

@@ -41,6 +41,40 @@ FUSE_ROTARY = os.environ.get("TPPX_FUSE_ROTARY", "1") == "1"
 FUSE_GREEDY = os.environ.get("TPPX_FUSE_GREEDY", "1") == "1"
 
 
+# Weight-format switches of the decoder layers, read once at import like the reference's file-statics
+# (src/csrc/llm/fused_llm_infer.cpp:35-45).  A layer built from UNQUANTIZED blocked weights quantizes them itself
+# under USE_MXFP4 / USE_QINT8 / USE_QINT2 (the decode-step copy); passes of FT_OPT_SIZE or more tokens run on the
+# first-token copy instead, which stays unquantized unless USE_*_FT picks a format for it, and is only used when
+# TPP_CACHE_REMAPPED_WEIGHTS is on.
+def _env_int(name, default):
+    v = os.environ.get(name, "")
+    return int(v) if v.strip() else default
+
+
+TPP_CACHE_REMAPPED_WEIGHTS = _env_int("TPP_CACHE_REMAPPED_WEIGHTS", 1)
+FT_OPT_SIZE = _env_int("FT_OPT_SIZE", 256)
+USE_MXFP4 = _env_int("USE_MXFP4", 0)
+USE_MXFP4_FT = _env_int("USE_MXFP4_FT", 0)
+USE_QINT8 = _env_int("USE_QINT8", 0)
+USE_QINT8_FT = _env_int("USE_QINT8_FT", 0)
+USE_QINT2 = _env_int("USE_QINT2", 0)
+USE_QINT2_FT = _env_int("USE_QINT2_FT", 0)
+
+
+def wt_tensor_for_first_token(t):
+    """wt_tensor_for_first_token (fused_llm_infer.cpp:365-420): the copy of an unquantized weight that passes of
+    FT_OPT_SIZE or more tokens run on.  The reference re-blocks it to 64 output channels per block for its CPU
+    GEMM; the kernels here read any blocking through the native tiles made on first use, so unquantized stays as
+    it is -- and USE_QINT8_FT / USE_MXFP4_FT / USE_QINT2_FT (in the reference's order) quantize it."""
+    if USE_QINT8_FT == 1:
+        return _ops.remap_and_quantize_qint8(t)
+    if USE_MXFP4_FT == 1:
+        return _ops.remap_and_quantize_mxfp4(t)
+    if USE_QINT2_FT == 1:
+        return _ops.remap_and_quantize_qint2_intlv(t)
+    return t
+
+
 def apply_rotary_pos_emb_llama(t_in, t_emb_pos, t_pos, N, H):
     """In place on t_in [B][S][N*H] (fused_llm_infer.cpp:207-253); t_emb_pos f32 [2][MP][HR]; t_pos i64 [B_pos][S]."""
     L = _lib.lib()
@@ -198,8 +232,37 @@ class LlamaDecoderLayer:
          self.t_Wg, self.t_Wu, self.t_Wd, self.t_EP) = params
         self.layer_idx, self.eps, self.H = int(layer_idx), float(eps), int(H)
         self.max_positions, self.rotary_dim = int(max_positions), int(rotary_dim)
-        self.Nq = _ops._as_q(self.t_Wq).weight_nk()[0] // self.H
-        self.Nkv = _ops._as_q(self.t_Wk).weight_nk()[0] // self.H
+        # fused_llm_infer.cpp:1112-1162: quantized weights serve every pass; unquantized ones are quantized here
+        # for the decode steps under USE_MXFP4 / USE_QINT8 / USE_QINT2, after the first-token copies were taken
+        self.first_token_remapped = False
+        self._first = None
+        names = ("t_Wq", "t_Wk", "t_Wv", "t_Wp", "t_Wg", "t_Wu", "t_Wd")
+        if isinstance(self.t_Wq, _ops.QTensor):
+            self._first = tuple(getattr(self, n) for n in names)
+            self.first_token_remapped = True
+        else:
+            quant = (_ops.remap_and_quantize_mxfp4 if USE_MXFP4 else _ops.remap_and_quantize_qint8 if USE_QINT8
+                     else _ops.remap_and_quantize_qint2_intlv if USE_QINT2 else None)
+            if quant is not None:
+                self.remap_for_first_token()
+                for n in names:
+                    setattr(self, n, quant(getattr(self, n)))
+        self.Nq = _ops.weight_nk(self.t_Wq)[0] // self.H
+        self.Nkv = _ops.weight_nk(self.t_Wk)[0] // self.H
+
+    def remap_for_first_token(self):
+        """LlamaDecoderLayer::remap_for_first_token (fused_llm_infer.cpp:1164-1175)."""
+        self._first = tuple(wt_tensor_for_first_token(w) for w in
+                            (self.t_Wq, self.t_Wk, self.t_Wv, self.t_Wp, self.t_Wg, self.t_Wu, self.t_Wd))
+        self.first_token_remapped = True
+
+    def _weights_for(self, rows):
+        """check_weight_reuse + the switch to the first-token copies (fused_llm_infer.cpp:518-524, 1216-1227)."""
+        if rows >= FT_OPT_SIZE and TPP_CACHE_REMAPPED_WEIGHTS:
+            if not self.first_token_remapped:
+                self.remap_for_first_token()
+            return self._first
+        return (self.t_Wq, self.t_Wk, self.t_Wv, self.t_Wp, self.t_Wg, self.t_Wu, self.t_Wd)
 
     def forward(self, inputs, cache, use_cache=True):
         """inputs = [hidden [B][S][hidden], additive mask [B][keys] or empty, position_ids i64 [B or 1][S]].
@@ -217,18 +280,18 @@ class LlamaDecoderLayer:
                                          f"{tuple(t_pid.shape)} {t_pid.dtype}")
         st = _lib.stream_of(t_HS)
         empty = torch.empty(0, dtype=torch.bfloat16, device=t_HS.device)
+        Wq, Wk, Wv, Wp, Wg, Wu, Wd = self._weights_for(B * S)
         t_res = t_HS
         # Decode steps on MXFP4 weights: the o- and down-projection launches leave the row sums of squares of the
         # residual stream, so the RMSNorm behind them is a scale applied while the next GEMM stages its input.
         M = B * S
         if cache._sums is None:
             cache._sums = (_ops.sums_table(t_HS.device), _ops.sums_table(t_HS.device))
-        sums_attn = cache._sums[0] if _ops.takes_row_sums(self.t_Wp, M) else None
-        sums_out = cache._sums[1] if _ops.takes_row_sums(self.t_Wd, M) else None
+        sums_attn = cache._sums[0] if _ops.takes_row_sums(Wp, M) else None
+        sums_out = cache._sums[1] if _ops.takes_row_sums(Wd, M) else None
         sums_in = cache._sums[1] if cache._sums_of is t_HS else None
         # input RMSNorm + q/k/v GEMMs
-        q, k, v = _ops.qkv_gemm(t_HS, [self.t_Wq, self.t_Wk, self.t_Wv], [empty] * 3,
-                                norm=(self.t_Gi, self.eps, sums_in))
+        q, k, v = _ops.qkv_gemm(t_HS, [Wq, Wk, Wv], [empty] * 3, norm=(self.t_Gi, self.eps, sums_in))
         kc, vc = cache._ensure(self.layer_idx, B, self.Nkv, self.H, t_HS.device)
         ws = _lib.workspace(t_HS)
         mask_ptr = t_am.data_ptr() if t_am is not None and t_am.numel() else None
@@ -241,7 +304,7 @@ class LlamaDecoderLayer:
                 self.t_EP.shape[1], self.t_EP.shape[2], kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
                 cache.seq_len_dev.data_ptr(), ctx.data_ptr(), B, self.Nq, self.Nkv, self.H, cache.capacity,
                 ws.data_ptr(), ws.numel(), st))
-            return self._after_attention(ctx, t_res, empty, cache, sums_attn, sums_out)
+            return self._after_attention(ctx, t_res, empty, cache, sums_attn, sums_out, Wp, Wg, Wu, Wd)
         # rotary on q and k + append of k, v at position seq_len (device counter), one launch
         _lib.check(L.tppx_rotary_kv_append_llama(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), self.t_EP.data_ptr(), t_pid.data_ptr(), kc.data_ptr(),
@@ -257,13 +320,13 @@ class LlamaDecoderLayer:
             _lib.check(L.tppx_attn_prefill(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
                                            cache.get_seq_length(), ctx.data_ptr(), B, S, self.Nq, self.Nkv, self.H,
                                            cache.capacity, st))
-        return self._after_attention(ctx, t_res, empty, cache, sums_attn, sums_out)
+        return self._after_attention(ctx, t_res, empty, cache, sums_attn, sums_out, Wp, Wg, Wu, Wd)
 
-    def _after_attention(self, ctx, t_res, empty, cache, sums_attn, sums_out):
-        t_SO = _ops.fc_add(ctx, self.t_Wp, empty, t_res, 1.0, row_sumsq=sums_attn)
+    def _after_attention(self, ctx, t_res, empty, cache, sums_attn, sums_out, Wp, Wg, Wu, Wd):
+        t_SO = _ops.fc_add(ctx, Wp, empty, t_res, 1.0, row_sumsq=sums_attn)
         # post-attention RMSNorm + gate/up GEMMs + silu*mul
-        t_I = _ops.swiglu_gate_up(t_SO, self.t_Wg, self.t_Wu, norm=(self.t_Gpa, self.eps, sums_attn))
-        t_Out = _ops.fc_add(t_I, self.t_Wd, empty, t_SO, 1.0, row_sumsq=sums_out)
+        t_I = _ops.swiglu_gate_up(t_SO, Wg, Wu, norm=(self.t_Gpa, self.eps, sums_attn))
+        t_Out = _ops.fc_add(t_I, Wd, empty, t_SO, 1.0, row_sumsq=sums_out)
         cache._sums_of = t_Out if sums_out is not None else None
         return [t_Out]
 
