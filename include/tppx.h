@@ -68,6 +68,11 @@ extern "C" {
 /* Element type of a floating-point weight handed to the quantizers. */
 #define TPPX_DT_F32 0
 #define TPPX_DT_BF16 1
+#define TPPX_DT_F16 2
+
+/* Weight kinds of tppx_linear_wide. */
+#define TPPX_W_MXFP4 0 /* native tiles + scale bytes of tppx_prepack_mxfp4 */
+#define TPPX_W_BF16 1  /* native tiles of tppx_prepack_bf16 */
 
 /* flags for the linear entry points */
 #define TPPX_FLAG_NONE 0
@@ -457,6 +462,30 @@ int tppx_linear_qint8_f32(const void* xq, const void* sa, const void* qw,
                           const void* sw, const void* bias_f32, void* y_f32,
                           int64_t M, int64_t N, int64_t K, int64_t qbs,
                           tppx_stream_t stream);
+
+/* The same switch for MXFP4 and unquantized bf16 weights:
+ * TppBlockedLinearW<Tin, uint8_t, Tout> / <Tin, bfloat16, Tout> with Tin =
+ * float or half (src/csrc/fused_gemm.h:1519-1523, 1541-1550; 785-1073).  The
+ * activations keep their own precision; every weight value is exact in fp32;
+ *   y[m][n] = bias[n] + sum_k x[m][k] * w[n][k]      in fp32.
+ * x fp32 or fp16 [M][K] (x_dtype = TPPX_DT_F32 / TPPX_DT_F16); w / sw native
+ * tiles (w_kind = TPPX_W_MXFP4: tppx_prepack_mxfp4's tiles and scale bytes;
+ * TPPX_W_BF16: tppx_prepack_bf16's tiles, sw ignored); bias f32 [N] or NULL;
+ * y f32 [M][N].  K % 128 == 0.  The caller rounds to the activations' type
+ * and applies the post-op with tppx_post_op_wide. */
+int tppx_linear_wide(const void* x, int x_dtype, const void* w, const void* sw,
+                     int w_kind, const void* bias_f32, void* y_f32, int64_t M,
+                     int64_t N, int64_t K, tppx_stream_t stream);
+
+/* Post-ops of call_gemm_with_post_op on a float or half output tile
+ * (src/csrc/fused_gemm.h:1343-1488 with Tout = float / half): out[i] =
+ * post(round_T(acc[i])) with a rounding to T (T = half; none for float) where
+ * the CPU path stores its tile.  acc f32 [count] (bias + dot product);
+ * post_in / post_in2 and out in T (out_dtype = TPPX_DT_F32 / TPPX_DT_F16). */
+int tppx_post_op_wide(const void* acc_f32, int out_dtype, int post_op,
+                      const void* post_in, const void* post_in2,
+                      float post_scale, void* out, int64_t count,
+                      tppx_stream_t stream);
 
 /* W4A8, the reference's USE_MXFP4_INT8 mode: TppBlockedLinearW<int8_t, uint8_t,
  * Tout> (src/csrc/fused_gemm.h:965-978, 1523-1526) on the weight layout of

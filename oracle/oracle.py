@@ -627,6 +627,65 @@ def linear_bf16(x_bf16, w_bf16, bias=None, post=POST_NONE, post_in=None, post_in
 
 
 # ----------------------------------------------------------------------------
+# float / half activations on MXFP4 or unquantized bf16 weights: TppBlockedLinearW<Tin, uint8_t, Tout> and
+# <Tin, bfloat16, Tout> with Tin = Tout = float or half (src/csrc/fused_gemm.h:1519-1523, 1541-1550, 785-1073; the
+# element-type switch of fc_plain_wrap, src/csrc/llm/fused_llm_infer.cpp:1526-1545).  The activations keep their own
+# precision and every weight value is exact in fp32, so the GEMM tile is the exact dot product (evaluated in fp64
+# here) plus the bias, rounded once to T; post-ops then work on T, re-rounding to T where the CPU path stores its
+# tile (src/csrc/fused_gemm.h:1343-1488).  Pinned by: fp64 matmul of the dequantized weight is the definition; on
+# bf16-representable activations the T = float tile rounded to bf16 equals linear_mxfp4 / linear_bf16 (ideal mode)
+# up to their fp32 summation order (tests/test_oracle.py).  libxsmm's own summation order and its sigmoid / GELU
+# polynomials are not in the tree: parity unpinned for those, covered by the stated tolerance.
+# ----------------------------------------------------------------------------
+def post_op_wide(y, post, in1=None, in2=None, scale=1.0):
+    """y, in1, in2: numpy float32 or float16 arrays of one shape; arithmetic in fp32, stores in y's dtype."""
+    T = y.dtype.type
+    rt = lambda a: np.asarray(a, np.float32).astype(T).astype(np.float32)  # noqa: E731
+    yf = y.astype(np.float32)
+    a = None if in1 is None else np.asarray(in1).astype(np.float32)
+    b = None if in2 is None else np.asarray(in2).astype(np.float32)
+    sc = np.float32(scale)
+    if post == POST_SILU:
+        out = yf * rt(np.float32(1.0) / (np.float32(1.0) + np.exp(-yf.astype(np.float64)).astype(np.float32)))
+    elif post == POST_MUL:
+        out = a * yf
+    elif post == POST_ADD_SCALE:
+        out = (a.astype(np.float64) * np.float64(sc) + yf.astype(np.float64)).astype(np.float32)  # one fused multiply-add
+    elif post == POST_ADD2_SCALE:
+        t = rt(yf + a)
+        out = (b.astype(np.float64) * np.float64(sc) + t.astype(np.float64)).astype(np.float32)
+    elif post == POST_GELU:
+        from math import erf
+        e = np.vectorize(erf)(yf.astype(np.float64) * 0.70710678118654752)
+        out = (0.5 * yf.astype(np.float64) * (1.0 + e)).astype(np.float32)
+    elif post == POST_RELU:
+        out = np.where(yf < 0, np.float32(0), yf)
+    else:
+        out = yf
+    return out.astype(T)
+
+
+def _linear_wide(x, W_f32, bias, post, post_in, post_in2, post_scale):
+    x = np.asarray(x)
+    assert x.dtype in (np.float32, np.float16)
+    acc = x.astype(np.float64) @ np.asarray(W_f32, np.float64).T
+    if bias is not None:
+        acc = acc + np.asarray(bias).astype(np.float64)[None, :]
+    y = acc.astype(np.float32).astype(x.dtype)
+    return post_op_wide(y, post, post_in, post_in2, post_scale)
+
+
+def linear_mxfp4_wide(x, q, sc, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0):
+    """x float32 / float16 [M][K]; q, sc the reference-layout MXFP4 weight; bias / post inputs in x's dtype."""
+    return _linear_wide(x, dequantize_mxfp4_plain(q, sc), bias, post, post_in, post_in2, post_scale)
+
+
+def linear_bf16_wide(x, w_bf16, bias=None, post=POST_NONE, post_in=None, post_in2=None, post_scale=1.0):
+    """x float32 / float16 [M][K]; w bits [N][K] (plain layout)."""
+    return _linear_wide(x, bf16_to_f32(_c(w_bf16, np.uint16)), bias, post, post_in, post_in2, post_scale)
+
+
+# ----------------------------------------------------------------------------
 # MXFP8 activations of the opt-in FP8-activation GEMM.  No reference code to follow (its activations stay bf16):
 # the OCP Microscaling v1.0 recipe -- E4M3 elements (bias 7, subnormals, maximum 448, no infinities), one E8M0
 # scale per 32 values with exponent floor(log2 max|x|) - 8, round to nearest even, saturation.

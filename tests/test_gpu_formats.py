@@ -175,11 +175,73 @@ def test_fc_plain_float_and_half_activations(M, dtype):
     y3 = ops.fc_plain(x.cuda().view(1, M, K), qw, None)
     ref3 = torch.from_numpy(O.linear_qint8_f32(xq, sa, q_or, s_or, None)).to(dtype)
     assert tuple(y3.shape) == (1, M, N) and torch.equal(y3.cpu().view(M, N), ref3)
-    from tpp_pytorch_extension._lib import TppxError
-    with pytest.raises(TppxError):  # post-ops are a bfloat16 path
-        ops.fc_silu(x.cuda(), qw, None)
-    with pytest.raises(TppxError):  # MXFP4 weights take bfloat16 activations
-        ops.fc_plain(x.cuda(), ops.remap_and_quantize_mxfp4(block_bf16(W).cuda()), None)
+    # post-ops work on the output type (fused_gemm.h:1343-1488 with Tout = float / half)
+    acc = torch.from_numpy(O.linear_qint8_f32(xq, sa, q_or, s_or, None)).to(dtype)
+    res = (torch.randn((M, N), generator=g) * 0.5).to(dtype)
+    for post, fn, args in ((O.POST_SILU, ops.fc_silu, ()), (O.POST_ADD_SCALE, ops.fc_add, (res.cuda(), 0.5)),
+                           (O.POST_MUL, ops.fc_mul, (res.cuda(),))):
+        got = fn(x.cuda(), qw, None, *args)
+        want = O.post_op_wide(acc.numpy(), post, res.numpy(), None, 0.5)
+        assert got.dtype == dtype
+        tol = 2e-3 if dtype == torch.float16 else 2e-6
+        assert np.allclose(got.cpu().float().numpy(), want.astype(np.float32), rtol=tol, atol=tol), post
+
+
+@pytest.mark.parametrize("M", [1, 7, 70])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("wkind", ["mxfp4", "bf16"])
+def test_float_and_half_activations_on_mxfp4_and_bf16_weights(M, dtype, wkind):
+    """TppBlockedLinearW<Tin, uint8_t, Tout> / <Tin, bfloat16, Tout> with Tin = float or half
+    (src/csrc/fused_gemm.h:1519-1523, 1541-1550): the activations keep their own precision (a bf16-rounded input would
+    miss the bound below by two orders of magnitude), fp32 sums, output and post-ops in the activations' type.
+    Against the oracle's exact (fp64) dot product: float within 4 fp32 ulps of sum |x||w| (the fp32 accumulation over
+    K), half within one half ulp of it; then every post-op."""
+    ops = _ops()
+    N, K = 96, 1024
+    W = randn_bf16((N, K), 0.05, 161)
+    g = torch.Generator().manual_seed(162 + M)
+    x = (torch.randn((M, K), generator=g) * 1.3).to(dtype)
+    bias = (torch.randn((N,), generator=g) * 0.1).to(dtype)
+    if wkind == "mxfp4":
+        w = ops.remap_and_quantize_mxfp4(block_bf16(W).cuda())
+        q_or, s_or = O.remap_quantize_mxfp4(W.float().numpy())
+        Wd = O.dequantize_mxfp4_plain(q_or, s_or)
+        lin = lambda *a: O.linear_mxfp4_wide(x.numpy(), q_or, s_or, *a)  # noqa: E731
+    else:
+        w = block_bf16(W).cuda()
+        Wd = W.float().numpy()
+        lin = lambda *a: O.linear_bf16_wide(x.numpy(), t2bits(W), *a)  # noqa: E731
+    y = ops.fc_plain(x.cuda(), w, bias.cuda())
+    assert y.dtype == dtype and tuple(y.shape) == (M, N)
+    ref = lin(bias.numpy())
+    mag = np.abs(x.float().numpy()).astype(np.float64) @ np.abs(Wd).astype(np.float64).T + np.abs(bias.float().numpy())
+    d = np.abs(y.cpu().float().numpy().astype(np.float64) - ref.astype(np.float64))
+    if dtype == torch.float32:
+        assert (d <= 4 * 2.0 ** -23 * mag).all(), float((d / mag).max())
+        # the input was NOT rounded to bf16 on the way in
+        y_bf = ops.fc_plain(x.to(torch.bfloat16).float().cuda(), w, bias.cuda()).cpu().numpy().astype(np.float64)
+        assert np.abs(y_bf - ref).max() > 50 * d.max()
+    else:
+        ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref.astype(np.float64)), 2.0 ** -14))) - 10)
+        assert (d <= ulp + 4 * 2.0 ** -23 * mag).all()
+        assert np.mean(y.cpu().numpy() != ref) <= 1e-2  # fp32 sums of 1024 products land across a half rounding boundary now and then
+    # leading dimensions kept, no bias
+    y3 = ops.fc_plain(x.cuda().view(1, M, K), w, None)
+    assert tuple(y3.shape) == (1, M, N)
+    # post-ops on the output type
+    res = (torch.randn((M, N), generator=g) * 0.5).to(dtype)
+    res2 = (torch.randn((M, N), generator=g) * 0.5).to(dtype)
+    tol = 2e-3 if dtype == torch.float16 else 1e-5
+    for post, call in ((O.POST_SILU, lambda: ops.fc_silu(x.cuda(), w, bias.cuda())),
+                       (O.POST_MUL, lambda: ops.fc_mul(x.cuda(), w, bias.cuda(), res.cuda())),
+                       (O.POST_ADD_SCALE, lambda: ops.fc_add(x.cuda(), w, bias.cuda(), res.cuda(), 0.5)),
+                       (O.POST_ADD2_SCALE, lambda: ops.fc_add2(x.cuda(), w, bias.cuda(), res.cuda(), res2.cuda(), 0.5)),
+                       (O.POST_GELU, lambda: ops.fc_gelu(x.cuda(), w, bias.cuda())),
+                       (O.POST_RELU, lambda: ops.fc_relu(x.cuda(), w, bias.cuda()))):
+        got = call()
+        want = lin(bias.numpy(), post, res.numpy(), res2.numpy(), 0.5)
+        assert got.dtype == dtype
+        assert np.allclose(got.cpu().float().numpy(), want.astype(np.float32), rtol=tol, atol=tol * 4), post
 
 
 @pytest.mark.parametrize("M", [3, 40])

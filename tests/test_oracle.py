@@ -567,3 +567,62 @@ def test_oracle_w4a8_layout_table_and_linear():
     exact = (xq.astype(np.float64) * np.repeat(sa / O.W4A8_ACT_SCALE, 32, axis=1)) @ Wd.astype(np.float64).T \
         + bias.float().numpy().astype(np.float64)
     assert np.sqrt(((ref - exact) ** 2).sum() / (exact ** 2).sum()) <= 1.5e-2
+
+
+def test_wide_activation_linears_pinned_on_bf16_inputs():
+    """linear_mxfp4_wide / linear_bf16_wide (float / half activations, fp64 dot product) against the pinned bf16
+    restatements: on activations that ARE bf16 values the float tile, rounded to bf16, is the ideal-mode tile of
+    linear_mxfp4 / linear_bf16 except where the fp32 summation order crosses a rounding boundary (a few elements per
+    thousand at K = 512, one bf16 ulp each); the post-ops on float match the bf16 ones within bf16 resolution."""
+    rng = np.random.default_rng(5)
+    M, N, K = 24, 64, 512
+    W = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+    wb = O.f32_to_bf16(W)
+    xb = O.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    xf = O.bf16_to_f32(xb)
+    bias_b = O.f32_to_bf16((rng.standard_normal(N) * 0.1).astype(np.float32))
+    q, sc = O.remap_quantize_mxfp4(O.bf16_to_f32(wb))
+    for wide, narrow in ((O.linear_mxfp4_wide(xf, q, sc, O.bf16_to_f32(bias_b)), O.linear_mxfp4(xb, q, sc, bias_b)),
+                         (O.linear_bf16_wide(xf, wb, O.bf16_to_f32(bias_b)), O.linear_bf16(xb, wb, bias_b))):
+        assert wide.dtype == np.float32
+        as_bf16 = O.f32_to_bf16(wide)
+        diff = as_bf16 != narrow
+        assert diff.mean() <= 5e-3
+        assert np.abs(O.bf16_to_f32(as_bf16) - O.bf16_to_f32(narrow)).max() <= 2.0 ** -7 * np.abs(O.bf16_to_f32(narrow)).max()
+    # half: one rounding of the same exact sum
+    xh = xf.astype(np.float16)
+    wide_h = O.linear_mxfp4_wide(xh, q, sc, None)
+    exact = xh.astype(np.float64) @ O.dequantize_mxfp4_plain(q, sc).astype(np.float64).T
+    assert wide_h.dtype == np.float16 and np.array_equal(wide_h, exact.astype(np.float32).astype(np.float16))
+    # post-ops on float: the textbook formulas
+    y = (rng.standard_normal((M, N))).astype(np.float32)
+    a = (rng.standard_normal((M, N))).astype(np.float32)
+    b = (rng.standard_normal((M, N))).astype(np.float32)
+    assert np.allclose(O.post_op_wide(y, O.POST_SILU), y / (1 + np.exp(-y.astype(np.float64))), rtol=1e-6, atol=1e-7)
+    assert np.array_equal(O.post_op_wide(y, O.POST_MUL, a), a * y)
+    assert np.allclose(O.post_op_wide(y, O.POST_ADD_SCALE, a, None, 0.25), y + 0.25 * a.astype(np.float64), rtol=1e-7, atol=1e-7)
+    assert np.allclose(O.post_op_wide(y, O.POST_ADD2_SCALE, a, b, 0.25), y.astype(np.float64) + a + 0.25 * b, rtol=1e-6, atol=1e-6)
+    assert np.array_equal(O.post_op_wide(y, O.POST_RELU), np.maximum(y, 0))
+    import math
+    assert np.allclose(O.post_op_wide(y[:2], O.POST_GELU), [[0.5 * v * (1 + math.erf(v / math.sqrt(2))) for v in r] for r in y[:2]], rtol=1e-6, atol=1e-7)
+    # half post-ops store half after every step
+    yh, ah = y.astype(np.float16), a.astype(np.float16)
+    assert np.array_equal(O.post_op_wide(yh, O.POST_MUL, ah), (ah.astype(np.float32) * yh.astype(np.float32)).astype(np.float16))
+
+
+def test_w4a8_integer_table_is_bounded_the_reference_table_is_unreadable_here():
+    """The integers the reference multiplies for MXFP4 weights in the W4A8 mode (USE_MXFP4_INT8,
+    src/csrc/fused_gemm.h:965-978) come out of its JIT library, whose sources are not in the tree: the table cannot be
+    read here, so it is restated as round-to-nearest of E2M1 x 127/6 and BOUNDED instead of pinned -- for every one of
+    the 16 codes table[c] x 6/127 lies within half an int8 step (0.5 x 6/127) of the E2M1 value, the table is odd,
+    monotone in the code's magnitude, exact at 0 and at the format's maximum 6 (= 127), and no other integer is closer
+    to any code.  Parity of this one table stays unpinned."""
+    e2m1 = np.array([O.lib().orc_e2m1_decode(c) for c in range(16)], np.float64)
+    tbl = np.array([O.lib().orc_w4a8_weight_int(c) for c in range(16)], np.float64)
+    step = 6.0 / 127.0
+    assert np.abs(tbl * step - e2m1).max() <= 0.5 * step + 1e-12
+    assert np.array_equal(tbl[8:], -tbl[:8]) and tbl[0] == 0 and tbl[7] == 127 and tbl[15] == -127
+    assert np.all(np.diff(tbl[:8]) > 0) and np.all(np.abs(tbl) <= 127) and np.array_equal(tbl, np.rint(tbl))
+    for c in range(16):
+        for other in (tbl[c] - 1, tbl[c] + 1):
+            assert abs(other * step - e2m1[c]) >= abs(tbl[c] * step - e2m1[c])

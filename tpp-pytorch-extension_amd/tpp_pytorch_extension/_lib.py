@@ -14,7 +14,8 @@ LIB_PATH = os.path.join(_HERE, "libtppx_hip.so")
 
 OK, EINVAL, ESHAPE, EUNSUPPORTED, EHIP = 0, -1, -2, -3, -4
 POST_NONE, POST_SILU, POST_MUL, POST_ADD_SCALE, POST_ADD2_SCALE, POST_GELU, POST_RELU = range(7)
-DT_F32, DT_BF16 = 0, 1
+DT_F32, DT_BF16, DT_F16 = 0, 1, 2
+W_MXFP4, W_BF16 = 0, 1
 Q_MXFP4, Q_INT8, Q_INT4 = 0, 1, 2
 FLAG_NONE, FLAG_FORCE_SKINNY, FLAG_FORCE_TILED, FLAG_ACT_FP8, FLAG_XQ_REUSE = 0, 1, 2, 4, 8
 
@@ -81,6 +82,8 @@ SIGNATURES = {
     "tppx_rotary_kv_append_llama": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                     _i64, _i64, _vp],
     "tppx_linear_qint8_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
+    "tppx_linear_wide": [_vp, _i32, _vp, _vp, _i32, _vp, _vp, _i64, _i64, _i64, _vp],
+    "tppx_post_op_wide": [_vp, _i32, _i32, _vp, _vp, _f32, _vp, _i64, _vp],
     "tppx_linear_mxfp4_int8": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _f32, _vp],
     "tppx_greedy_next": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp],
     "tppx_qkv_linear_mxfp4": [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _vp],

@@ -487,19 +487,75 @@ def _mxfp4_flags_ws(x, M, K, flags=0):
     return flags, ws
 
 
-def _linear_other_types(input, weight, bias, post, flags):
-    """The element-type switch of fc_plain_wrap (src/csrc/llm/fused_llm_infer.cpp:1526-1545) beyond bfloat16, for
+def _wide_post(acc, ctype, post, post_in, post_in2, post_scale, shape):
+    """fp32 GEMM tile (bias + dot) -> the activations' type with the post-op applied there (tppx_post_op_wide)."""
+    L = _lib.lib()
+    if ctype == torch.float32 and post == POST_NONE:
+        return acc.view(shape)
+    out = torch.empty(shape, dtype=ctype, device=acc.device)
+    ins = []
+    for t, need in ((post_in, post in (POST_MUL, POST_ADD_SCALE, POST_ADD2_SCALE)), (post_in2, post == POST_ADD2_SCALE)):
+        if not need:
+            ins.append(None)
+            continue
+        if t is None or tuple(t.shape) != tuple(shape) or t.device != acc.device:
+            raise TppxError(_lib.ESHAPE, f"post-op {post} needs an input of the output's shape {tuple(shape)} on {acc.device}")
+        ins.append(t.to(ctype).contiguous())
+    if out.numel():
+        _lib.check(L.tppx_post_op_wide(acc.data_ptr(), _lib.DT_F16 if ctype == torch.float16 else _lib.DT_F32, post,
+                                       _lib.ptr(ins[0]), _lib.ptr(ins[1]), float(post_scale), out.data_ptr(),
+                                       out.numel(), _lib.stream_of(acc)))
+    return out
+
+
+def _linear_wide(input, weight, bias, post, post_in, post_in2, post_scale):
+    """float / half activations on an MXFP4 or an unquantized bf16 weight: TppBlockedLinearW<Tin, uint8_t, Tout> /
+    <Tin, bfloat16, Tout> with Tin = float or half (src/csrc/fused_gemm.h:1519-1523, 1541-1550).  The activations are
+    NOT rounded to bf16: fp32 products and sums (every weight value is exact in fp32), output and post-op in the
+    activations' type."""
+    L = _lib.lib()
+    _lib.require_gpu(input, "input")
+    ctype = input.dtype
+    if isinstance(weight, QTensor):
+        N, K = weight.weight_nk()
+        qn, sn = weight.native()
+        kind = _lib.W_MXFP4
+    else:
+        N, K = _blocked_geometry(weight)[:2]
+        qn, sn, kind = _bf16_native(weight), None, _lib.W_BF16
+    if input.shape[-1] != K:
+        raise TppxError(_lib.ESHAPE, f"input has {input.shape[-1]} features, weight expects {K}")
+    x = input.contiguous()
+    M = x.numel() // K
+    shape = tuple(input.shape[:-1]) + (N,)
+    acc = torch.empty((M, N), dtype=torch.float32, device=x.device)
+    if M:
+        b = None
+        if bias is not None and bias.numel():
+            if bias.numel() != N:
+                raise TppxError(_lib.ESHAPE, f"bias has {bias.numel()} elements, the weight {N} channels")
+            b = bias.to(device=x.device, dtype=torch.float32).contiguous()
+        _lib.check(L.tppx_linear_wide(x.data_ptr(), _lib.DT_F16 if ctype == torch.float16 else _lib.DT_F32, qn.data_ptr(),
+                                      _lib.ptr(sn), kind, _lib.ptr(b), acc.data_ptr(), M, N, K, _lib.stream_of(x)))
+    return _wide_post(acc, ctype, post, post_in, post_in2, post_scale, shape)
+
+
+def _linear_other_types(input, weight, bias, post, flags, post_in=None, post_in2=None, post_scale=1.0):
+    """The element-type switch of fc_plain_wrap (src/csrc/llm/fused_llm_infer.cpp:1526-1545) beyond bfloat16.
     QINT8-family weights (TppBlockedQInt8LinearW, src/csrc/fused_gemm.h:1236-1249):
       float / half activations    quantized from their own values (quantize_int8sym over the last axis with the
                                   weight's block size), fp32 accumulation and bias, output in the activations' type;
       pre-quantized qint8 input   used as it is; the compute type is the bias's, float without a bias (:1529-1535).
-    A bfloat16 compute type runs the bf16 kernels on the quantized rows; float / half the fp32-output kernel."""
+    A bfloat16 compute type runs the bf16 kernels on the quantized rows; float / half the fp32-output kernel.
+    MXFP4 and unquantized bf16 weights take float / half activations as they are (_linear_wide)."""
     L = _lib.lib()
+    wide_weight = (isinstance(weight, QTensor) and weight.is_weight() and weight.weight_kind() == "mxfp4") or \
+        (_is_plain(weight) and weight.dtype == torch.bfloat16)
+    if wide_weight and not isinstance(input, QTensor):
+        return _linear_wide(input, weight, bias, post, post_in, post_in2, post_scale)
     if not isinstance(weight, QTensor) or not weight.is_weight() or weight.weight_kind() in ("mxfp4", "mxfp4_int8"):
-        raise TppxError(_lib.EUNSUPPORTED, "float / half / pre-quantized activations need a QINT8, QINT4 or QINT2 weight "
-                                           "(MXFP4 and bf16 weights take bfloat16 activations)")
-    if post != POST_NONE:
-        raise TppxError(_lib.EUNSUPPORTED, "post-ops are built for bfloat16 activations only")
+        raise TppxError(_lib.EUNSUPPORTED, "pre-quantized activations need a QINT8, QINT4 or QINT2 weight; float / half "
+                                           "activations any weight but the W4A8 layout")
     _lib.require_gpu(weight.qdata, "weight")
     N, K = weight.weight_nk()
     qbs = weight.block_size
@@ -527,14 +583,16 @@ def _linear_other_types(input, weight, bias, post, flags):
         y = torch.empty(shape[:-1] + (N,), dtype=torch.bfloat16, device=xq.device)
         if M:
             b = _prep_bias(bias, N, xq.device)
+            p1 = _prep_post(post_in, M, N, "post-op input", xq.device) if post in (POST_MUL, POST_ADD_SCALE, POST_ADD2_SCALE) else None
+            p2 = _prep_post(post_in2, M, N, "second post-op input", xq.device) if post == POST_ADD2_SCALE else None
             ws = _lib.workspace(xq)
             _lib.check(L.tppx_linear_qint8(None, xq.data_ptr(), sa.data_ptr(), qn.data_ptr(), sn.data_ptr(), _lib.ptr(b),
-                                           None, None, y.data_ptr(), M, N, K, qbs, POST_NONE, 1.0, flags, ws.data_ptr(),
-                                           ws.numel(), st))
+                                           _lib.ptr(p1), _lib.ptr(p2), y.data_ptr(), M, N, K, qbs, post, float(post_scale),
+                                           flags, ws.data_ptr(), ws.numel(), st))
         return y
     if ctype not in (torch.float32, torch.float16):
         raise TppxError(_lib.EUNSUPPORTED, f"compute type {ctype} is not built")
-    y = torch.empty(shape[:-1] + (N,), dtype=torch.float32, device=xq.device)
+    y = torch.empty((M, N), dtype=torch.float32, device=xq.device)
     if M:
         b = None
         if bias is not None and bias.numel():
@@ -543,7 +601,7 @@ def _linear_other_types(input, weight, bias, post, flags):
             b = bias.to(device=xq.device, dtype=torch.float32).contiguous()
         _lib.check(L.tppx_linear_qint8_f32(xq.data_ptr(), sa.data_ptr(), qn.data_ptr(), sn.data_ptr(), _lib.ptr(b),
                                            y.data_ptr(), M, N, K, qbs, st))
-    return y if ctype == torch.float32 else y.to(torch.float16)
+    return _wide_post(y, ctype, post, post_in, post_in2, post_scale, shape[:-1] + (N,))
 
 
 W4A8_ACT_SCALE = 6.0 / 127.0
@@ -606,6 +664,11 @@ def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None
     row_sumsq: f32 [16][256] table that receives the row sums of squares of the output (see sums_table());
     only honoured where takes_row_sums() says so."""
     L = _lib.lib()
+    other_type = isinstance(input, QTensor) or (isinstance(input, torch.Tensor) and input.dtype in (torch.float32, torch.float16))
+    if other_type and not _is_w4a8(weight):
+        if row_sumsq is not None:
+            raise TppxError(_lib.EUNSUPPORTED, "row sums of squares need bfloat16 activations")
+        return _linear_other_types(input, weight, bias, post, flags, post_in, post_in2, post_scale)
     if not isinstance(weight, QTensor) and isinstance(weight, torch.Tensor) and weight.dtype == torch.bfloat16:
         if row_sumsq is not None:
             raise TppxError(_lib.EUNSUPPORTED, "row sums of squares need an MXFP4 weight and at most 16 rows")
@@ -614,8 +677,6 @@ def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None
         if row_sumsq is not None:
             raise TppxError(_lib.EUNSUPPORTED, "row sums of squares need an MXFP4 weight in the default layout")
         return _linear_w4a8(input, weight, bias, post, post_in, post_in2, post_scale)
-    if isinstance(input, QTensor) or (isinstance(input, torch.Tensor) and input.dtype in (torch.float32, torch.float16)):
-        return _linear_other_types(input, weight, bias, post, flags)
     x, M, N, K = _prep_input(input, weight)
     out_shape = tuple(input.shape[:-1]) + (N,)
     y = torch.empty(out_shape, dtype=torch.bfloat16, device=x.device)
