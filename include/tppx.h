@@ -278,10 +278,10 @@ int tppx_linear_qint8(const void* x, void* xq, void* sa, const void* qw,
 
 /* No counterpart in the reference.  tppx_linear_qint8 for callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the quantised activations, their
- * scales and the K-split workspace live in a static device array of the library (about 4.1 MiB per GPU, held
+ * scales and the K-split workspace live in a static device array of the library (about 6.1 MiB per GPU, held
  * until the process ends) instead of caller buffers.  x must be given (bf16 [M][K]); limits: M <= 64 (decode
  * shapes), K <= 32768 -- larger sizes return TPPX_ESHAPE; flags: 0 or TPPX_FLAG_FORCE_SKINNY.  Same kernels and
- * the same bits as tppx_linear_qint8 with a 2 MiB workspace.  The call itself allocates nothing and frees nothing.
+ * the same bits as tppx_linear_qint8 with a 4 MiB workspace.  The call itself allocates nothing and frees nothing.
  * All calls on one GPU share the one array: calls that overlap on a GPU (different streams without ordering)
  * race; order them on one stream or with events.  Nothing in the array has to start at zero: every value that reaches
  * an output was written earlier in the same call (the padding rows of the last 16-row tile of quantised

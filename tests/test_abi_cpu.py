@@ -210,7 +210,12 @@ def test_launch_plans_of_the_baseline_shapes():
     assert "skinny_qint8_fq_kernel<3," in plan(L.tppx_plan_linear_qint8, 1, 11008, 4096, 256, 1, 0, ws)[0]
     lines = plan(L.tppx_plan_linear_qint8, 64, 4096, 11008, 256, 1, 0, ws)
     assert len(lines) == 2 and "quant_act_int8_rows_kernel" in lines[0]
-    assert "skinny_qint8_kernel<4, 2, 4, 8, 8, true>" in lines[1] and "grid=128x1x2" in lines[1]  # K in two parts
+    # four channel tiles x four K parts per workgroup, K in four slices across workgroups (64 groups x 4)
+    assert "skinny_qint8_nk_kernel<4, 4, 4, 3, 1, 8> grid=256x1x1 block=1024" in lines[1], lines
+    lines = plan(L.tppx_plan_linear_qint8, 32, 4096, 11008, 256, 1, 0, ws)
+    assert "skinny_qint8_nk_kernel<2, 4, 4, 3, 1, 8> grid=256x1x1" in lines[1], lines
+    lines = plan(L.tppx_plan_linear_qint8, 64, 4096, 11008, 256, 1, 0, 0)  # no workspace: no K split
+    assert "skinny_qint8_kernel<4, 1, 8, 8, 8, true> grid=256x1x1" in lines[1], lines
     assert len(plan(L.tppx_plan_linear_qint8, 64, 4096, 11008, 256, 0, 0, ws)) == 1             # pre-quantized input
     # config 3 / 5: MXFP4 decode
     assert "skinny_mxfp4_x4_kernel<1, 4, false> grid=256x1x1" in plan(L.tppx_plan_linear_mxfp4, 1, 4096, 11008, 0, ws)[0]
@@ -255,7 +260,7 @@ def test_launch_plans_of_per_output_channel_qint8():
     assert len(two) == 2 and "quant_act_int8_bigblk_kernel grid=64x1x1 block=256" in two[0], two
     assert "skinny_qint8_kernel<4, 3, 2, 8, 8, true> grid=230x1x1 block=512" in two[1], two
     two = plan(64, 4096, 11008, 11008, 1, 0, ws)
-    assert "quant_act_int8_bigblk_kernel grid=64x1x1 block=704" in two[0] and "grid=128x1x2" in two[1], two
+    assert "quant_act_int8_bigblk_kernel grid=64x1x1 block=704" in two[0] and "skinny_qint8_nk_kernel<4," in two[1], two
     # a block that is not a whole number of 256-wide runs is dealt tile by tile: still one GEMM launch, quantizer in front
     odd = plan(5, 512, 1280, 320, 1, 0, ws)
     assert len(odd) == 2 and "quant_act_int8_kernel" in odd[0] and "skinny_qint8_kernel<1, 1, 4, 16, 4, true>" in odd[1], odd

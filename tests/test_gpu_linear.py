@@ -163,8 +163,10 @@ def test_module_api_and_errors():
     assert_close_bf16(t2bits(y).reshape(15, 128), ref, what="BlockedLinear")
     with pytest.raises(TppxError):
         torch.ops.tpp_llm.fc_plain(x.to(torch.bfloat16)[..., :128].contiguous(), lin.weight, torch.Tensor(), -1, [])
+    yf = torch.ops.tpp_llm.fc_plain(x, lin.weight, torch.Tensor(), -1, [])  # fp32 activations: fp32 result
+    assert yf.dtype == torch.float32 and yf.shape == (3, 5, 128)
     with pytest.raises(TppxError):
-        torch.ops.tpp_llm.fc_plain(x, lin.weight, torch.Tensor(), -1, [])  # fp32 activations
+        torch.ops.tpp_llm.fc_plain(x.to(torch.float64), lin.weight, torch.Tensor(), -1, [])
     e = torch.ops.tpp_llm.fc_plain(torch.empty(0, 256, dtype=torch.bfloat16).cuda(), lin.weight, torch.Tensor(), -1, [])
     assert e.shape == (0, 128)
 
@@ -357,6 +359,32 @@ def test_k_split_across_workgroups(fmt, M, N):
     assert torch.equal(first, y)
     for o in outs:
         assert torch.equal(o, first)
+
+
+@pytest.mark.parametrize("M,N,K,post", [(64, 4096, 8192, "add"), (33, 4080, 14336, "add2"), (50, 2048, 16384, "none"),
+                                        (17, 4096, 11008, "mul"), (32, 4064, 14336, "silu"), (64, 1600, 32768, "add"),
+                                        (20, 4096, 12288, "gelu")])
+def test_qint8_tile_by_k_part_kernel(M, N, K, post, monkeypatch):
+    """QINT8, 17..64 rows, up to 256 channel tiles and a long K: four channel tiles x four K parts per workgroup with
+    the activation operands shared through LDS, K in four slices across workgroups, partial tiles exchanged as
+    128-bit device-scope stores / loads (2..8 steps per wave, ragged last channel group, partly filled row groups,
+    every post-op).  Against the oracle; twenty launches give the same bits; the kernel it replaces
+    (TPPX_QINT8_NK=0) is within one ulp of it as well (another summation order, so not bit-identical)."""
+    import ctypes
+    from tpp_pytorch_extension import _lib
+    buf = ctypes.create_string_buffer(2048)
+    _lib.check(_lib.lib().tppx_plan_linear_qint8(M, N, K, 256, 1, 0, _lib.WORKSPACE_BYTES, buf, len(buf)))
+    assert "skinny_qint8_nk_kernel" in buf.value.decode(), buf.value.decode()
+    y, ref, st, ctx = _run("qint8", M, N, K, post, True, 7700 + M, ulps=2 if post in ("silu", "gelu") else 1)
+    qw, q_or, s_or, x, bias, in1, in2, scale = ctx
+    ops = _ops()
+    again = [ops.linear(x.cuda(), qw, bias.cuda(), POSTS[post], in1.cuda(), in2.cuda(), scale) for _ in range(20)]
+    torch.cuda.synchronize()
+    for o in again:
+        assert torch.equal(o, y)
+    monkeypatch.setenv("TPPX_QINT8_NK", "0")
+    old = ops.linear(x.cuda(), qw, bias.cuda(), POSTS[post], in1.cuda(), in2.cuda(), scale)
+    assert_close_bf16(t2bits(old), ref, ulps=2 if post in ("silu", "gelu") else 1, what="kernel without the tile x K-part grid")
 
 
 @pytest.mark.parametrize("split", [True, False])

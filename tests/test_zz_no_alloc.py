@@ -12,7 +12,7 @@ from util import t2bits, randn_bf16, block_bf16, assert_close_bf16
 pytestmark = pytest.mark.gpu
 
 
-def _both(L, _lib, qw, x, res, M, N, K, qbs, post, ws_bytes=2 * 256 * 4 * 256 * 4):
+def _both(L, _lib, qw, x, res, M, N, K, qbs, post, ws_bytes=4 * 256 * 4 * 256 * 4):
     qn, sn = qw.native()
     st = _lib.stream_of(x)
     y0 = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")

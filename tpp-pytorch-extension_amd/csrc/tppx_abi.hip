@@ -505,6 +505,28 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
   // 33..64 rows, few channel tiles and a long K: every workgroup would pull all of the int8 activations (M x K)
   // through its CU.  Two K parts of two channel tiles each halve that (measured at N = 4096, 64 rows: K = 11008
   // 20.4 -> 18.5 us, K = 14336 25.1 -> 21.6 us; K = 8192 and shorter lose to the extra pass over the partial sums).
+  // The same shapes with bf16 activations at hand (so that they are quantised into operand order): four channel
+  // tiles x four K parts per workgroup with the operands shared through LDS, K in 4 (or 2) slices across workgroups.
+  // (measured at N = 4096: 64 rows K = 8192 19.2 -> 14.6 us, K = 11008 18.9 -> 17.1, K = 14336 21.7 -> 20.9; 32 rows
+  // K = 11008 15.3 -> 14.1 and no gain at K = 8192, so 17..32 rows take it from K = 10240 on)
+  if (x && sp.mg >= env_int("TPPX_QINT8_NK_MIN_MG", 2) && (sp.mg == 4 || p.units >= 40) && !sp.fused_quant && p.n_seg == 1 &&
+      p.deal == 4 && M <= 64 && env_int("TPPX_QINT8_NK", 1) != 0) {
+    const int groups = (p.total_tiles + 3) / 4;
+    // four slices or nothing: with two, half the chip streams the weights (measured 25.8 us against 18.9 unsplit)
+    int S = 0;
+    if (groups * 4 <= 256 && groups * 4 >= 96 && p.units >= 32 && (p.units + 3) / 4 <= 32 &&
+        (int64_t)4 * groups * 4 * sp.mg * 256 * (int64_t)sizeof(float) * sp.grid_y <= ws_bytes)
+      S = 4;
+    if (S > 0) {
+      p.S = S;
+      p.part = (float*)ws;
+      p.mt = sp.grid_y * sp.mg;
+      rc = reuse ? TPPX_OK : check_hip(launch_quant_act_int8(x, M, K, qbs, xq, sa, p.mt, stream), who);
+      if (rc)
+        return rc;
+      return check_hip(launch_skinny_qint8_nk(p, sp.mg, stream), who);
+    }
+  }
   if (sp.mg == 4 && !sp.fused_quant && pick_split(p, M, K, sp.mg, 2, 5504, ws_bytes) == 2) {
     p.S = 2;
     p.part = (float*)ws;
@@ -718,7 +740,7 @@ extern "C" int tppx_multi_linear_qint8(const void* x, void* xq, void* sa,
 constexpr int64_t NA_MAX_M = 64, NA_MAX_K = 32768;
 constexpr size_t NA_XQ_BYTES = (size_t)NA_MAX_M * NA_MAX_K;                        // int8 rows, 2 MiB
 constexpr size_t NA_SA_BYTES = (size_t)NA_MAX_M * (NA_MAX_K / 64) * sizeof(float); // one scale per 64 channels at most
-constexpr size_t NA_WS_BYTES = (size_t)2 * 256 * 4 * 256 * sizeof(float);          // 2 K parts x 256 tiles x 64 rows
+constexpr size_t NA_WS_BYTES = (size_t)4 * 256 * 4 * 256 * sizeof(float);          // 4 K slices x 256 tiles x 64 rows
 static __device__ __align__(256) unsigned char scratch[NA_XQ_BYTES + NA_SA_BYTES + NA_WS_BYTES];
 
 static int scratch_of_current_device(const char* who, unsigned char** out) {

@@ -529,6 +529,232 @@ skinny_qint8_kernel(const DecodeParams p) {
 }
 
 // ---------------------------------------------------------------------------
+// QINT8, 17..64 rows, few channel tiles and a long K (the Llama down-projection): in the kernel above every wave
+// pulls its own activation operands, so a workgroup drags M x K bytes of int8 activations through its CU beside
+// 1-2 tiles' worth of weights, and the CU's load path, not HBM, sets the pace.  Here the sixteen waves form a
+// TW x KPW grid: wave (tw, kp) owns channel tile tw over K part kp of the workgroup's K slice, and the TW waves of a
+// K part share the activation operands of each 256-wide run through LDS (each fetches 1 / TW of the run's 4 x MG
+// operand tiles; one barrier per run).  With K split over S workgroups that own TW tiles each, the grid still fills
+// the chip and a workgroup reads 1 / (TW * S) of the activations per weight tile it streams.
+// Workgroup id -> (channel group id / S, K slice id % S): the workgroups of one XCD (ids equal mod 8) then share ONE
+// K slice when S divides 8, so every XCD's L2 fetches only that slice of the activations from memory.
+// The K slices' partial tiles travel as 128-bit device-scope stores and loads (16 bytes per lane instruction; as
+// dwords the exchange cost more than the split saved), merged by the last workgroup to arrive, in slice order.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void sk_store_x4_device(float* dst, f32x4 v) {
+  // device scope: performed where every XCD observes it (the 128-bit form of the atomic stores of finish_split)
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
+}
+__device__ __forceinline__ f32x4 sk_load_x4_device(const float* src) {
+  f32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(src) : "memory");
+  return v;
+}
+
+template <int MG, int TW, int KPW, int WPF, int XPF, int MAXSTEPS>
+__global__ void __launch_bounds__(TW * KPW * 64)
+skinny_qint8_nk_kernel(const DecodeParams p) {
+  extern __shared__ __align__(16) float sk_lds[];
+  constexpr int W = TW * KPW;
+  constexpr int XT = 4 * MG;              // operand tiles per run: tile j = k-tile j / MG, row group j % MG
+  constexpr int XPW = (XT + TW - 1) / TW; // fetched by one wave: j = tw + TW * i
+  constexpr int OUT = TW * MG * 256;      // outputs of the workgroup, element e = ((tw * MG + mg) * 4 + r) * 64 + lane
+  static_assert(XPF <= WPF, "the weights (HBM) are requested at least as far ahead as the activations (L2)");
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int tw = wave % TW, kp = wave / TW;
+  const int S = p.S;
+  const int grp = (int)blockIdx.x / S, z = (int)blockIdx.x % S;
+  const DecodeSeg& sg = p.seg[0];
+  const int ltile0 = grp * TW;
+  const int m0 = blockIdx.y * (MG * 16);
+  const int NR = p.units, NB = p.nblk; // 256-wide runs of K, scale blocks
+  const unsigned int magic = p.spb_magic;
+  auto blk_of_run = [&](int u) { return magic ? (int)__umulhi((unsigned int)u, magic) : u; };
+  // runs of this workgroup's K slice, then of this wave's K part; every wave makes the same number of steps
+  const int ub = (int)(((int64_t)z * NR) / S), ue = (int)(((int64_t)(z + 1) * NR) / S);
+  const int u0 = ub + (kp * (ue - ub)) / KPW, u1 = ub + ((kp + 1) * (ue - ub)) / KPW;
+  const int nsteps = (ue - ub + KPW - 1) / KPW; // <= MAXSTEPS (the launcher checks)
+
+  const int64_t lt = min(ltile0 + tw, sg.tiles - 1); // ragged last group: duplicate, not stored
+  const i32x4* wq = reinterpret_cast<const i32x4*>(sg.qw) + lt * ((int64_t)NR * 4) * 64 + lane;
+  const float* ws = reinterpret_cast<const float*>(sg.sw) + lt * NB * 16 + (lane & 15);
+  const i32x4* xop = reinterpret_cast<const i32x4*>(p.xq) + (int64_t)blockIdx.y * MG * 64 + lane;
+  const int xstride = p.mt * 64, mtp = p.mt * 16;
+
+  // Two rings: weights (from HBM) WPF steps ahead, the wave's share of the activation operands and the scales
+  // (L2-resident) XPF steps ahead.  Loads return in issue order, so a step's activations are requested BEFORE
+  // weights of later steps wherever both are issued together.
+  i32x4 wreg[WPF][4], xreg[XPF][XPW];
+  float sreg[XPF], sareg[XPF];
+  auto run_of = [&](int s) { return min(min(u0 + s, max(u1 - 1, u0)), NR - 1); }; // past the part's end: re-read (never used)
+  auto load_w = [&](int st, int s) {
+    const int u = run_of(s);
+#pragma unroll
+    for (int kt = 0; kt < 4; kt++)
+      wreg[st][kt] = __builtin_nontemporal_load(wq + (int64_t)(u * 4 + kt) * 64);
+  };
+  auto load_x = [&](int st, int s) {
+    const int u = run_of(s), b = blk_of_run(u);
+#pragma unroll
+    for (int i = 0; i < XPW; i++) {
+      const int j = min(tw + TW * i, XT - 1);
+      xreg[st][i] = xop[(int64_t)(u * 4 + j / MG) * xstride + (j % MG) * 64];
+    }
+    sreg[st] = ws[b * 16];
+    // activation scales of the run's block, transposed by the quantisation kernel: [K block][mt * 16 rows]
+    sareg[st] = p.sa[(int64_t)b * mtp + m0 + min(lane, MG * 16 - 1)];
+  };
+  static_for<0, WPF>([&](auto I) {
+    constexpr int i = decltype(I)::value;
+    if constexpr (i < XPF)
+      load_x(i, i);
+    load_w(i, i);
+  });
+
+  // LDS: operand stage [buffer][K part][tile j][lane] x 16 B, then scales [buffer][K part][64]; the reduction of the
+  // epilogue reuses the space
+  i32x4* xs = reinterpret_cast<i32x4*>(sk_lds);
+  float* sas = sk_lds + (size_t)2 * KPW * XT * 256;
+  f32x4 facc[MG];
+  i32x4 iacc[MG];
+#pragma unroll
+  for (int mg = 0; mg < MG; mg++) {
+    facc[mg] = f32x4{0.f, 0.f, 0.f, 0.f};
+    iacc[mg] = i32x4{0, 0, 0, 0};
+  }
+  static_for<0, MAXSTEPS>([&](auto SS) {
+    constexpr int s = decltype(SS)::value;
+    constexpr int wi = s % WPF, xi = s % XPF;
+    if (s < nsteps) { // uniform over the workgroup
+      i32x4* xb = xs + (size_t)(((s & 1) * KPW + kp) * XT) * 64 + lane;
+      float* sb = sas + ((s & 1) * KPW + kp) * 64;
+#pragma unroll
+      for (int ii = 0; ii < XPW; ii++)
+        if (tw + TW * ii < XT)
+          xb[(tw + TW * ii) * 64] = xreg[xi][ii];
+      if (tw == 0)
+        sb[lane] = sareg[xi];
+      const float swv = sreg[xi];
+      if (s + XPF < nsteps)
+        load_x(xi, s + XPF);
+      // one barrier per step: a wave that reaches the barrier of step s + 1 has finished reading the stage of
+      // step s, so that buffer may be overwritten for step s + 2
+      __syncthreads();
+      if (u0 + s < u1) {
+#pragma unroll
+        for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+          for (int mg = 0; mg < MG; mg++)
+            iacc[mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xb[(kt * MG + mg) * 64], wreg[wi][kt], iacc[mg], 0, 0, 0);
+#pragma unroll
+        for (int mg = 0; mg < MG; mg++) {
+          const f32x4 sav = *reinterpret_cast<const f32x4*>(sb + mg * 16 + (lane >> 4) * 4);
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            facc[mg][r] = fmaf((float)iacc[mg][r], sav[r] * swv, facc[mg][r]);
+            iacc[mg][r] = 0;
+          }
+        }
+      }
+      if (s + WPF < nsteps)
+        load_w(wi, s + WPF);
+    }
+  });
+
+  // ---- epilogue: a thread finishes Q quads of four adjacent channels of one row, e = (q * W * 64 + t) * 4 ..
+  constexpr int Q = (OUT + W * 256 - 1) / (W * 256);
+  int64_t o[Q];
+  bool valid[Q];
+  uint2 bias2[Q], in1[Q], in2[Q];
+#pragma unroll
+  for (int q = 0; q < Q; q++) {
+    const int e0 = (q * W * 64 + (int)threadIdx.x) * 4;
+    const int el = e0 & 63, er = (e0 >> 6) & 3, emg = (e0 >> 8) % MG, etw = (e0 >> 8) / MG;
+    const int m = m0 + emg * 16 + (el >> 4) * 4 + er;
+    const int n = (ltile0 + etw) * 16 + (el & 15);
+    valid[q] = e0 < OUT && m < p.M && (ltile0 + etw) < sg.tiles;
+    o[q] = (int64_t)m * sg.N + n;
+    bias2[q] = in1[q] = in2[q] = make_uint2(0, 0);
+    if (valid[q]) { // requested now, used after the reduction (and, with a K split, after the arrival counter)
+      if (sg.bias)
+        bias2[q] = *reinterpret_cast<const uint2*>(sg.bias + n);
+      if (sg.post_in)
+        in1[q] = *reinterpret_cast<const uint2*>(sg.post_in + o[q]);
+      if (sg.post_in2)
+        in2[q] = *reinterpret_cast<const uint2*>(sg.post_in2 + o[q]);
+    }
+  }
+  __syncthreads(); // everybody has read the last operands: the scratch takes their place
+  float* red = sk_lds; // [kp][OUT]
+#pragma unroll
+  for (int mg = 0; mg < MG; mg++)
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+      red[(size_t)kp * OUT + ((tw * MG + mg) * 4 + r) * 64 + lane] = facc[mg][r];
+  __syncthreads();
+  f32x4 own[Q], tot[Q];
+#pragma unroll
+  for (int q = 0; q < Q; q++) {
+    const int e0 = min((q * W * 64 + (int)threadIdx.x) * 4, OUT - 4); // threads past the outputs repeat the last quad
+    own[q] = *reinterpret_cast<const f32x4*>(red + e0);
+#pragma unroll
+    for (int k = 1; k < KPW; k++)
+      own[q] += *reinterpret_cast<const f32x4*>(red + (size_t)k * OUT + e0);
+    tot[q] = own[q];
+  }
+  if (S > 1) {
+    __shared__ int arrived_last;
+    // partial tiles [slice][block row][channel group][OUT]: whole groups, so a ragged last group stays inside its slot
+    const size_t slice_stride = (size_t)gridDim.y * (gridDim.x / S) * OUT;
+    // (threads past the outputs write and read the last quad again: the same values)
+    float* mine = p.part + ((size_t)blockIdx.y * (gridDim.x / S) + grp) * OUT +
+                  (size_t)min((int)threadIdx.x * 4, OUT - 4 - (Q - 1) * W * 256);
+#pragma unroll
+    for (int q = 0; q < Q; q++)
+      sk_store_x4_device(mine + (size_t)z * slice_stride + q * W * 256, own[q]);
+    // every thread's stores acknowledged at device scope, then the barrier, then the ticket, then the loads (see
+    // SkEpilogue::finish_split)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const unsigned int last = (unsigned int)S - 1;
+      arrived_last = atomicInc(&sk_split_tickets[p.ticket0 + blockIdx.y * (gridDim.x / S) + grp], last) == last;
+    }
+    __syncthreads();
+    if (!arrived_last)
+      return;
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+      f32x4 other[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++)
+        other[k] = (k < S && k != z) ? sk_load_x4_device(mine + (size_t)k * slice_stride + q * W * 256) : f32x4{0.f, 0.f, 0.f, 0.f};
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(other[0]), "+v"(other[1]), "+v"(other[2]), "+v"(other[3])::"memory");
+      tot[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < 4; k++)
+        if (k < S)
+          tot[q] += (k == z) ? own[q] : other[k]; // slice order: the same sums whichever workgroup arrives last
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < Q; q++)
+    if (valid[q]) {
+      const uint32_t bw[2] = {bias2[q].x, bias2[q].y}, w1[2] = {in1[q].x, in1[q].y}, w2[2] = {in2[q].x, in2[q].y};
+      uint32_t out[2];
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const uint32_t a = apply_post_bits(tot[q][2 * h] + bf16_bits_to_f32(bw[h] & 0xffffu), sg.post_op, w1[h] & 0xffffu,
+                                           w2[h] & 0xffffu, sg.post_scale);
+        const uint32_t b = apply_post_bits(tot[q][2 * h + 1] + bf16_bits_to_f32(bw[h] >> 16), sg.post_op, w1[h] >> 16,
+                                           w2[h] >> 16, sg.post_scale);
+        out[h] = (a & 0xffffu) | (b << 16);
+      }
+      *reinterpret_cast<uint2*>(sg.y + o[q]) = make_uint2(out[0], out[1]);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // QINT8 with the activation quantisation fused in, for M <= 16 (qbs == 256).
 // Every wave quantises the rows of its own K range (one (row, block) item =
 // 16 lanes x 16 values, DPP max reduction) into a wave-private LDS region that
@@ -1654,6 +1880,48 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
       return sk_launch(skinny_qint8_kernel<4, 1, 4, 8, 8, false>, p, grid, pl.waves, lds, stream); // row-major rows: shorter ring, no spills
   }
 #undef SKQ
+}
+
+// 17..32 (mg = 2) or 33..64 (mg = 4) rows per block row, four channel tiles x four K parts per workgroup, K in p.S slices across workgroups
+// (grid x = channel groups * S); p.units = 256-wide runs of K, activations in operand order (p.mt > 0)
+template <int MG, int TW, int KPW, int WPF, int XPF, int MAXSTEPS>
+static hipError_t sk_launch_nk(const DecodeParams& p, dim3 grid, hipStream_t stream) {
+  const size_t stage = ((size_t)2 * KPW * 4 * MG * 256 + 2 * KPW * 64) * sizeof(float);
+  const size_t redb = (size_t)KPW * TW * MG * 256 * sizeof(float);
+  const size_t lds = stage > redb ? stage : redb;
+  const auto kern = skinny_qint8_nk_kernel<MG, TW, KPW, WPF, XPF, MAXSTEPS>;
+  TPPX_PLAN_ONLY(kern, grid, dim3(TW * KPW * 64), lds);
+  hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds);
+  if (e == hipSuccess) {
+    kern<<<grid, dim3(TW * KPW * 64), lds, stream>>>(p);
+    e = hipGetLastError();
+  }
+  return e;
+}
+
+hipError_t launch_skinny_qint8_nk(DecodeParams& p, int mg, hipStream_t stream) {
+  const int groups = (p.total_tiles + 3) / 4, grid_y = (p.M + mg * 16 - 1) / (mg * 16);
+  dim3 grid(groups * p.S, grid_y, 1);
+  if (p.S > 4 || p.n_seg != 1 || p.mt <= 0 || p.deal != 4)
+    return hipErrorInvalidValue;
+  if (p.S > 1 && (p.ticket0 = skinny_split_tickets(groups * grid_y)) < 0)
+    return hipErrorInvalidValue;
+  // steps of a wave: runs of a K slice over the four K parts
+  const int nsteps = ((p.units + p.S - 1) / p.S + 3) / 4;
+  if (nsteps > 8)
+    return hipErrorInvalidValue;
+  const int form = env_int("TPPX_QINT8_NK_FORM", 0);
+  hipError_t e = mg == 2     ? sk_launch_nk<2, 4, 4, 3, 1, 8>(p, grid, stream)
+                 : form == 1   ? sk_launch_nk<4, 4, 4, 2, 2, 8>(p, grid, stream)
+                 : form == 2 ? sk_launch_nk<4, 4, 4, 4, 1, 8>(p, grid, stream)
+                 : form == 3 ? sk_launch_nk<4, 4, 4, 3, 2, 8>(p, grid, stream)
+                             : sk_launch_nk<4, 4, 4, 3, 1, 8>(p, grid, stream);
+  if (e != hipSuccess && p.S > 1 && p.ticket0 >= 0 && !plan_recording()) {
+    const int n = groups * grid_y;
+    sk_clear_tickets_kernel<<<dim3((n + 255) / 256), dim3(256), 0, stream>>>(p.ticket0, n);
+    (void)hipGetLastError();
+  }
+  return e;
 }
 
 // x staged in LDS, optional fused RMSNorm; 16 waves; nt = channel tiles per workgroup (of each GEMM when dual)
