@@ -387,6 +387,34 @@ def test_qint8_tile_by_k_part_kernel(M, N, K, post, monkeypatch):
     assert_close_bf16(t2bits(old), ref, ulps=2 if post in ("silu", "gelu") else 1, what="kernel without the tile x K-part grid")
 
 
+@pytest.mark.parametrize("form", [0, 1])
+@pytest.mark.parametrize("M,N,K,post", [(64, 4096, 8192, "add"), (33, 4064, 14336, "add2"), (50, 2048, 16384, "none"),
+                                        (64, 1632, 12288, "silu"), (47, 4096, 11008, "mul")])
+def test_mxfp4_tile_by_k_part_kernel(M, N, K, post, form, monkeypatch):
+    """MXFP4, 33..64 rows, up to 256 channel tiles and a long K: four channel tiles x four K parts per workgroup (two
+    tiles per wave and eight waves, or one and sixteen: TPPX_MXFP4_NK_FORM), a K tile's activations staged once per
+    workgroup, K in four slices across workgroups, workgroups walking their K part from rotated starting tiles.
+    Against the oracle; twenty launches give the same bits; the kernel it replaces (TPPX_MXFP4_NK=0) meets the oracle
+    too."""
+    import ctypes
+    from tpp_pytorch_extension import _lib
+    monkeypatch.setenv("TPPX_MXFP4_NK_FORM", str(form))
+    buf = ctypes.create_string_buffer(2048)
+    _lib.check(_lib.lib().tppx_plan_linear_mxfp4(M, N, K, 0, _lib.WORKSPACE_BYTES, buf, len(buf)))
+    assert "skinny_mxfp4_nk_kernel<4, 4, %d," % (2 - form) in buf.value.decode(), buf.value.decode()
+    y, ref, st, ctx = _run("mxfp4", M, N, K, post, True, 7800 + M, ulps=2 if post == "silu" else 1)
+    qw, q_or, s_or, x, bias, in1, in2, scale = ctx
+    ops = _ops()
+    again = [ops.linear(x.cuda(), qw, bias.cuda(), POSTS[post], in1.cuda(), in2.cuda(), scale) for _ in range(20)]
+    torch.cuda.synchronize()
+    for o in again:
+        assert torch.equal(o, y)
+    if form == 0:
+        monkeypatch.setenv("TPPX_MXFP4_NK", "0")
+        old = ops.linear(x.cuda(), qw, bias.cuda(), POSTS[post], in1.cuda(), in2.cuda(), scale)
+        assert_close_bf16(t2bits(old), ref, ulps=2 if post == "silu" else 1, what="kernel without the tile x K-part grid")
+
+
 @pytest.mark.parametrize("split", [True, False])
 @pytest.mark.parametrize("M,N,K", [(5, 4096, 11008), (16, 4096, 11008), (9, 2048, 16384), (16, 4096, 8192)])
 def test_mxfp4_few_rows_long_k_split_across_workgroups(M, N, K, split, monkeypatch):

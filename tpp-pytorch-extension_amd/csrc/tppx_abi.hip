@@ -427,6 +427,17 @@ static int run_mxfp4(const char* who, const void* x, const tppx_seg* segs, int n
     // Split K across S workgroups that own S times the channel tiles each: the same number of workgroups, 1/S of
     // the activations per CU, fp32 partial tiles through the workspace, summed by whichever of the S workgroups
     // finishes last (measured: 26 -> 21 us for 64 rows at K = 11008 / N = 4096; no gain for 32 rows).
+    // 33..64 rows, a single GEMM with few channel tiles and a long K: four tiles x four K parts per workgroup with
+    // the activations of a K tile staged ONCE per workgroup, K in four slices across workgroups
+    if (!dual && mg == 4 && n_segs == 1 && !row_sumsq && env_int("TPPX_MXFP4_NK", 1) != 0) {
+      const int groups = (p.total_tiles + 3) / 4;
+      if (groups * 4 <= 256 && groups * 4 >= 96 && p.units >= 64 && (p.units + 3) / 4 <= 32 &&
+          (int64_t)4 * groups * 4 * mg * 256 * (int64_t)sizeof(float) * ((M + 63) / 64) <= ws_bytes) {
+        p.S = 4;
+        p.part = (float*)ws;
+        return check_hip(launch_skinny_mxfp4_nk(p, stream), who);
+      }
+    }
     const int S = (dual || mg != 4) ? 1 : pick_split(p, M, K, mg, 4, 2048, ws_bytes);
     int nt = S;
     if (S == 1) {

@@ -129,6 +129,7 @@ SkinnyPlan plan_skinny(int64_t M, int total_tiles, int units, int tpb, int deal,
 int skinny_qint8_blocks_per_wave(int runs, int tpb, int deal, int nblk);
 hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_t stream);
 hipError_t launch_skinny_qint8_nk(DecodeParams& p, int mg, hipStream_t stream);
+hipError_t launch_skinny_mxfp4_nk(DecodeParams& p, hipStream_t stream);
 hipError_t launch_skinny_bf16(DecodeParams& p, int mg, int nt, hipStream_t stream);
 size_t skinny_mxfp4_xl_lds(int units, int nt, bool dual);
 hipError_t launch_skinny_mxfp4_x4(DecodeParams& p, int nt, bool dual, hipStream_t stream);

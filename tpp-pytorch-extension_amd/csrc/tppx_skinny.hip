@@ -551,6 +551,112 @@ __device__ __forceinline__ f32x4 sk_load_x4_device(const float* src) {
   return v;
 }
 
+// Epilogue of the TW x KPW kernels: the K parts' sums meet in LDS, the K slices' partial tiles in the workspace
+// (128-bit device-scope stores / loads, arrival counter as in SkEpilogue::finish_split), then bias, rounding and
+// post-op.  Thread t finishes Q quads of four adjacent channels of one row, e = (q * W * 64 + t) * 4 .., of the
+// workgroup's outputs e = ((tw * MG + mg) * 4 + r) * 64 + lane.  Called by every thread, after the main loop.
+// TPW = channel tiles per wave (tw = the wave's first tile); the workgroup has (TW / TPW) * KPW waves.
+template <int MG, int TW, int KPW, int TPW = 1>
+__device__ __forceinline__ void sk_nk_finish(const DecodeParams& p, const DecodeSeg& sg, f32x4 (&facc)[TPW][MG], float* sk_lds,
+                                             int grp, int z, int tw, int kp, int ltile0, int m0) {
+  constexpr int W = (TW / TPW) * KPW;
+  constexpr int OUT = TW * MG * 256;
+  const int lane = threadIdx.x & 63;
+  const int S = p.S;
+  constexpr int Q = (OUT + W * 256 - 1) / (W * 256);
+  int64_t o[Q];
+  bool valid[Q];
+  uint2 bias2[Q], in1[Q], in2[Q];
+#pragma unroll
+  for (int q = 0; q < Q; q++) {
+    const int e0 = (q * W * 64 + (int)threadIdx.x) * 4;
+    const int el = e0 & 63, er = (e0 >> 6) & 3, emg = (e0 >> 8) % MG, etw = (e0 >> 8) / MG;
+    const int m = m0 + emg * 16 + (el >> 4) * 4 + er;
+    const int n = (ltile0 + etw) * 16 + (el & 15);
+    valid[q] = e0 < OUT && m < p.M && (ltile0 + etw) < sg.tiles;
+    o[q] = (int64_t)m * sg.N + n;
+    bias2[q] = in1[q] = in2[q] = make_uint2(0, 0);
+    if (valid[q]) { // requested now, used after the reduction (and, with a K split, after the arrival counter)
+      if (sg.bias)
+        bias2[q] = *reinterpret_cast<const uint2*>(sg.bias + n);
+      if (sg.post_in)
+        in1[q] = *reinterpret_cast<const uint2*>(sg.post_in + o[q]);
+      if (sg.post_in2)
+        in2[q] = *reinterpret_cast<const uint2*>(sg.post_in2 + o[q]);
+    }
+  }
+  __syncthreads(); // everybody has read the last operands: the scratch takes their place
+  float* red = sk_lds; // [kp][OUT]
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+#pragma unroll
+    for (int mg = 0; mg < MG; mg++)
+#pragma unroll
+      for (int r = 0; r < 4; r++)
+        red[(size_t)kp * OUT + (((tw + t) * MG + mg) * 4 + r) * 64 + lane] = facc[t][mg][r];
+  __syncthreads();
+  f32x4 own[Q], tot[Q];
+#pragma unroll
+  for (int q = 0; q < Q; q++) {
+    const int e0 = min((q * W * 64 + (int)threadIdx.x) * 4, OUT - 4); // threads past the outputs repeat the last quad
+    own[q] = *reinterpret_cast<const f32x4*>(red + e0);
+#pragma unroll
+    for (int k = 1; k < KPW; k++)
+      own[q] += *reinterpret_cast<const f32x4*>(red + (size_t)k * OUT + e0);
+    tot[q] = own[q];
+  }
+  if (S > 1) {
+    __shared__ int arrived_last;
+    // partial tiles [slice][block row][channel group][OUT]: whole groups, so a ragged last group stays inside its slot
+    const size_t slice_stride = (size_t)gridDim.y * (gridDim.x / S) * OUT;
+    // (threads past the outputs write and read the last quad again: the same values)
+    float* mine = p.part + ((size_t)blockIdx.y * (gridDim.x / S) + grp) * OUT +
+                  (size_t)min((int)threadIdx.x * 4, OUT - 4 - (Q - 1) * W * 256);
+#pragma unroll
+    for (int q = 0; q < Q; q++)
+      sk_store_x4_device(mine + (size_t)z * slice_stride + q * W * 256, own[q]);
+    // every thread's stores acknowledged at device scope, then the barrier, then the ticket, then the loads (see
+    // SkEpilogue::finish_split)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const unsigned int last = (unsigned int)S - 1;
+      arrived_last = atomicInc(&sk_split_tickets[p.ticket0 + blockIdx.y * (gridDim.x / S) + grp], last) == last;
+    }
+    __syncthreads();
+    if (!arrived_last)
+      return;
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+      f32x4 other[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++)
+        other[k] = (k < S && k != z) ? sk_load_x4_device(mine + (size_t)k * slice_stride + q * W * 256) : f32x4{0.f, 0.f, 0.f, 0.f};
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(other[0]), "+v"(other[1]), "+v"(other[2]), "+v"(other[3])::"memory");
+      tot[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < 4; k++)
+        if (k < S)
+          tot[q] += (k == z) ? own[q] : other[k]; // slice order: the same sums whichever workgroup arrives last
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < Q; q++)
+    if (valid[q]) {
+      const uint32_t bw[2] = {bias2[q].x, bias2[q].y}, w1[2] = {in1[q].x, in1[q].y}, w2[2] = {in2[q].x, in2[q].y};
+      uint32_t out[2];
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const uint32_t a = apply_post_bits(tot[q][2 * h] + bf16_bits_to_f32(bw[h] & 0xffffu), sg.post_op, w1[h] & 0xffffu,
+                                           w2[h] & 0xffffu, sg.post_scale);
+        const uint32_t b = apply_post_bits(tot[q][2 * h + 1] + bf16_bits_to_f32(bw[h] >> 16), sg.post_op, w1[h] >> 16,
+                                           w2[h] >> 16, sg.post_scale);
+        out[h] = (a & 0xffffu) | (b << 16);
+      }
+      *reinterpret_cast<uint2*>(sg.y + o[q]) = make_uint2(out[0], out[1]);
+    }
+}
+
 template <int MG, int TW, int KPW, int WPF, int XPF, int MAXSTEPS>
 __global__ void __launch_bounds__(TW * KPW * 64)
 skinny_qint8_nk_kernel(const DecodeParams p) {
@@ -615,11 +721,11 @@ skinny_qint8_nk_kernel(const DecodeParams p) {
   // epilogue reuses the space
   i32x4* xs = reinterpret_cast<i32x4*>(sk_lds);
   float* sas = sk_lds + (size_t)2 * KPW * XT * 256;
-  f32x4 facc[MG];
+  f32x4 facc[1][MG];
   i32x4 iacc[MG];
 #pragma unroll
   for (int mg = 0; mg < MG; mg++) {
-    facc[mg] = f32x4{0.f, 0.f, 0.f, 0.f};
+    facc[0][mg] = f32x4{0.f, 0.f, 0.f, 0.f};
     iacc[mg] = i32x4{0, 0, 0, 0};
   }
   static_for<0, MAXSTEPS>([&](auto SS) {
@@ -651,7 +757,7 @@ skinny_qint8_nk_kernel(const DecodeParams p) {
           const f32x4 sav = *reinterpret_cast<const f32x4*>(sb + mg * 16 + (lane >> 4) * 4);
 #pragma unroll
           for (int r = 0; r < 4; r++) {
-            facc[mg][r] = fmaf((float)iacc[mg][r], sav[r] * swv, facc[mg][r]);
+            facc[0][mg][r] = fmaf((float)iacc[mg][r], sav[r] * swv, facc[0][mg][r]);
             iacc[mg][r] = 0;
           }
         }
@@ -661,97 +767,136 @@ skinny_qint8_nk_kernel(const DecodeParams p) {
     }
   });
 
-  // ---- epilogue: a thread finishes Q quads of four adjacent channels of one row, e = (q * W * 64 + t) * 4 ..
-  constexpr int Q = (OUT + W * 256 - 1) / (W * 256);
-  int64_t o[Q];
-  bool valid[Q];
-  uint2 bias2[Q], in1[Q], in2[Q];
+  sk_nk_finish<MG, TW, KPW, 1>(p, sg, facc, sk_lds, grp, z, tw, kp, ltile0, m0);
+}
+
+// ---------------------------------------------------------------------------
+// MXFP4, 33..64 rows, few channel tiles and a long K: the same TW x KPW grid of waves.  Wave (tw, kp) owns channel
+// tile tw over K part kp of the workgroup's K slice; per K tile (128 channels) the TW = MG waves of a K part stage
+// the 64 x 128 bf16 activations in LDS once -- wave tw fetches row group tw with row-contiguous 16-byte loads and
+// writes it in the swizzled operand-order image of skinny_mxfp4_mg_kernel -- and every wave reads all of it as MFMA
+// operands.  Against that kernel, where each wave stages the whole tile for itself, a workgroup moves a quarter of
+// the activation bytes per weight tile, and a wave's whole weight range (one 1 KiB tile per step) is in flight from
+// the first instruction.  K slices across workgroups and the merge as in skinny_qint8_nk_kernel.
+// ---------------------------------------------------------------------------
+template <int MG, int TW, int TPW, int KPW, int WPF, int XPF, int MAXSTEPS>
+__global__ void __launch_bounds__((TW / TPW) * KPW * 64)
+skinny_mxfp4_nk_kernel(const DecodeParams p) {
+  constexpr int WC = TW / TPW;  // wave columns: wave (wc, kp) owns channel tiles wc*TPW .. of K part kp
+  constexpr int RGW = MG / WC;  // row groups of a K tile's activations that one wave stages
+  static_assert(WC * TPW == TW && RGW * WC == MG, "tiles and row groups divide among the wave columns");
+  extern __shared__ __align__(16) float sk_lds[];
+  constexpr int MPAD = MG * 16, XI = RGW * 4; // items (4 rows x 256 B) a wave stages per K tile
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wc = wave % WC, kp = wave / WC;
+  const int S = p.S;
+  const int grp = (int)blockIdx.x / S, z = (int)blockIdx.x % S;
+  const DecodeSeg& sg = p.seg[0];
+  const int ltile0 = grp * TW;
+  const int m0 = blockIdx.y * MPAD;
+  const int KT = p.units; // K tiles of 128
+  const int tb = (int)(((int64_t)z * KT) / S), te = (int)(((int64_t)(z + 1) * KT) / S);
+  const int t0 = tb + (kp * (te - tb)) / KPW, t1 = tb + ((kp + 1) * (te - tb)) / KPW;
+  const int nsteps = (te - tb + KPW - 1) / KPW; // <= MAXSTEPS (the launcher checks)
+
+  uint32_t woff[TPW];
 #pragma unroll
-  for (int q = 0; q < Q; q++) {
-    const int e0 = (q * W * 64 + (int)threadIdx.x) * 4;
-    const int el = e0 & 63, er = (e0 >> 6) & 3, emg = (e0 >> 8) % MG, etw = (e0 >> 8) / MG;
-    const int m = m0 + emg * 16 + (el >> 4) * 4 + er;
-    const int n = (ltile0 + etw) * 16 + (el & 15);
-    valid[q] = e0 < OUT && m < p.M && (ltile0 + etw) < sg.tiles;
-    o[q] = (int64_t)m * sg.N + n;
-    bias2[q] = in1[q] = in2[q] = make_uint2(0, 0);
-    if (valid[q]) { // requested now, used after the reduction (and, with a K split, after the arrival counter)
-      if (sg.bias)
-        bias2[q] = *reinterpret_cast<const uint2*>(sg.bias + n);
-      if (sg.post_in)
-        in1[q] = *reinterpret_cast<const uint2*>(sg.post_in + o[q]);
-      if (sg.post_in2)
-        in2[q] = *reinterpret_cast<const uint2*>(sg.post_in2 + o[q]);
+  for (int t = 0; t < TPW; t++)
+    woff[t] = (uint32_t)(min(ltile0 + wc * TPW + t, sg.tiles - 1) * KT * 64 + lane);
+  const char* qwb = reinterpret_cast<const char*>(sg.qw);
+  const char* swb = reinterpret_cast<const char*>(sg.sw);
+  const char* xb = reinterpret_cast<const char*>(p.x);
+  const int r4 = lane >> 4, c16 = lane & 15;
+  // Every workgroup of a K slice reads the same activation tiles; walking them in the same order, all of them ask
+  // the same L2 channels for the same lines at the same moment.  Workgroup `grp` starts `grp` tiles into its part
+  // and wraps round: the sums are added in a rotated (fixed) order.
+  const int len = t1 - t0, rot = len > 0 ? grp % len : 0;
+  auto tile_of = [&](int s) { // past the part's end: a valid tile, never consumed
+    const int i = s + rot;
+    return max(min(t0 + (i >= len ? i - len : i), t1 - 1), 0);
+  };
+
+  i32x4 wreg[WPF][TPW], xr[XPF][XI];
+  uint32_t sreg[WPF][TPW];
+  auto load_w = [&](int st, int s) {
+#pragma unroll
+    for (int t = 0; t < TPW; t++) {
+      const uint32_t slot = woff[t] + (uint32_t)tile_of(s) * 64u;
+      wreg[st][t] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(qwb + (size_t)(slot * 16u)));
+      sreg[st][t] = *reinterpret_cast<const uint8_t*>(swb + (size_t)slot);
     }
-  }
-  __syncthreads(); // everybody has read the last operands: the scratch takes their place
-  float* red = sk_lds; // [kp][OUT]
+  };
+  // this wave's share of a K tile's activations: rows wc*RGW*16 + it*4 + lane/16, chunk lane%16 of the tile's 256
+  // bytes; rows past M re-read row M-1 (their results are not stored)
+  auto load_x = [&](int st, int s) {
+    const uint32_t base = (uint32_t)tile_of(s) * 256u + (uint32_t)c16 * 16u;
 #pragma unroll
-  for (int mg = 0; mg < MG; mg++)
-#pragma unroll
-    for (int r = 0; r < 4; r++)
-      red[(size_t)kp * OUT + ((tw * MG + mg) * 4 + r) * 64 + lane] = facc[mg][r];
-  __syncthreads();
-  f32x4 own[Q], tot[Q];
-#pragma unroll
-  for (int q = 0; q < Q; q++) {
-    const int e0 = min((q * W * 64 + (int)threadIdx.x) * 4, OUT - 4); // threads past the outputs repeat the last quad
-    own[q] = *reinterpret_cast<const f32x4*>(red + e0);
-#pragma unroll
-    for (int k = 1; k < KPW; k++)
-      own[q] += *reinterpret_cast<const f32x4*>(red + (size_t)k * OUT + e0);
-    tot[q] = own[q];
-  }
-  if (S > 1) {
-    __shared__ int arrived_last;
-    // partial tiles [slice][block row][channel group][OUT]: whole groups, so a ragged last group stays inside its slot
-    const size_t slice_stride = (size_t)gridDim.y * (gridDim.x / S) * OUT;
-    // (threads past the outputs write and read the last quad again: the same values)
-    float* mine = p.part + ((size_t)blockIdx.y * (gridDim.x / S) + grp) * OUT +
-                  (size_t)min((int)threadIdx.x * 4, OUT - 4 - (Q - 1) * W * 256);
-#pragma unroll
-    for (int q = 0; q < Q; q++)
-      sk_store_x4_device(mine + (size_t)z * slice_stride + q * W * 256, own[q]);
-    // every thread's stores acknowledged at device scope, then the barrier, then the ticket, then the loads (see
-    // SkEpilogue::finish_split)
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      const unsigned int last = (unsigned int)S - 1;
-      arrived_last = atomicInc(&sk_split_tickets[p.ticket0 + blockIdx.y * (gridDim.x / S) + grp], last) == last;
+    for (int it = 0; it < XI; it++) {
+      const int row = min(m0 + wc * (RGW * 16) + it * 4 + r4, p.M - 1);
+      xr[st][it] = *reinterpret_cast<const i32x4*>(xb + (size_t)((uint32_t)(row * p.K) * 2u + base));
     }
-    __syncthreads();
-    if (!arrived_last)
-      return;
+  };
+  // a step's activations are requested before weights of later steps (loads return in issue order)
+  static_for<0, WPF>([&](auto I) {
+    constexpr int i = decltype(I)::value;
+    if constexpr (i < XPF)
+      load_x(i, i);
+    load_w(i, i);
+  });
+
+  // LDS: [buffer][K part][chunk 16][row MPAD] x 16 B; the reduction of the epilogue reuses the space
+  i32x4* xs = reinterpret_cast<i32x4*>(sk_lds);
+  int rdo[4]; // operand slot of this lane for step j: chunk g*4 + j, row m of row group mg (+ mg*16)
 #pragma unroll
-    for (int q = 0; q < Q; q++) {
-      f32x4 other[4];
-#pragma unroll
-      for (int k = 0; k < 4; k++)
-        other[k] = (k < S && k != z) ? sk_load_x4_device(mine + (size_t)k * slice_stride + q * W * 256) : f32x4{0.f, 0.f, 0.f, 0.f};
-      asm volatile("s_waitcnt vmcnt(0)" : "+v"(other[0]), "+v"(other[1]), "+v"(other[2]), "+v"(other[3])::"memory");
-      tot[q] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int k = 0; k < 4; k++)
-        if (k < S)
-          tot[q] += (k == z) ? own[q] : other[k]; // slice order: the same sums whichever workgroup arrives last
-    }
+  for (int j = 0; j < 4; j++) {
+    const int cj = (lane >> 4) * 4 + j;
+    rdo[j] = cj * MPAD + ((lane & 15) ^ cj);
   }
+  f32x4 acc[TPW][MG];
 #pragma unroll
-  for (int q = 0; q < Q; q++)
-    if (valid[q]) {
-      const uint32_t bw[2] = {bias2[q].x, bias2[q].y}, w1[2] = {in1[q].x, in1[q].y}, w2[2] = {in2[q].x, in2[q].y};
-      uint32_t out[2];
+  for (int t = 0; t < TPW; t++)
 #pragma unroll
-      for (int h = 0; h < 2; h++) {
-        const uint32_t a = apply_post_bits(tot[q][2 * h] + bf16_bits_to_f32(bw[h] & 0xffffu), sg.post_op, w1[h] & 0xffffu,
-                                           w2[h] & 0xffffu, sg.post_scale);
-        const uint32_t b = apply_post_bits(tot[q][2 * h + 1] + bf16_bits_to_f32(bw[h] >> 16), sg.post_op, w1[h] >> 16,
-                                           w2[h] >> 16, sg.post_scale);
-        out[h] = (a & 0xffffu) | (b << 16);
+    for (int mg = 0; mg < MG; mg++)
+      acc[t][mg] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  static_for<0, MAXSTEPS>([&](auto SS) {
+    constexpr int s = decltype(SS)::value;
+    constexpr int wi = s % WPF, xi = s % XPF;
+    if (s < nsteps) { // uniform over the workgroup
+      i32x4* stage = xs + (size_t)((s & 1) * KPW + kp) * (MPAD * 16);
+#pragma unroll
+      for (int it = 0; it < XI; it++)
+        stage[c16 * MPAD + ((wc * (RGW * 16) + it * 4 + r4) ^ c16)] = xr[xi][it];
+      if (s + XPF < nsteps)
+        load_x(xi, s + XPF);
+      // one barrier per step: a wave that reaches the barrier of step s + 1 has finished reading the stage of
+      // step s, so that buffer may be overwritten for step s + 2
+      __syncthreads();
+      if (t0 + s < t1) {
+        float sc[TPW];
+#pragma unroll
+        for (int t = 0; t < TPW; t++)
+          sc[t] = e8m0_to_f32(sreg[wi][t]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          bf16x8 b[TPW];
+#pragma unroll
+          for (int t = 0; t < TPW; t++)
+            b[t] = sk_cvt_fp4x8((uint32_t)wreg[wi][t][j], sc[t]);
+#pragma unroll
+          for (int mg = 0; mg < MG; mg++) {
+            const bf16x8 a = __builtin_bit_cast(bf16x8, stage[rdo[j] + mg * 16]);
+#pragma unroll
+            for (int t = 0; t < TPW; t++)
+              acc[t][mg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[t], acc[t][mg], 0, 0, 0);
+          }
+        }
       }
-      *reinterpret_cast<uint2*>(sg.y + o[q]) = make_uint2(out[0], out[1]);
+      if (s + WPF < nsteps)
+        load_w(wi, s + WPF);
     }
+  });
+  sk_nk_finish<MG, TW, KPW, TPW>(p, sg, acc, sk_lds, grp, z, wc * TPW, kp, ltile0, m0);
 }
 
 // ---------------------------------------------------------------------------
@@ -1910,13 +2055,46 @@ hipError_t launch_skinny_qint8_nk(DecodeParams& p, int mg, hipStream_t stream) {
   const int nsteps = ((p.units + p.S - 1) / p.S + 3) / 4;
   if (nsteps > 8)
     return hipErrorInvalidValue;
-  const int form = env_int("TPPX_QINT8_NK_FORM", 0);
-  hipError_t e = mg == 2     ? sk_launch_nk<2, 4, 4, 3, 1, 8>(p, grid, stream)
-                 : form == 1   ? sk_launch_nk<4, 4, 4, 2, 2, 8>(p, grid, stream)
-                 : form == 2 ? sk_launch_nk<4, 4, 4, 4, 1, 8>(p, grid, stream)
-                 : form == 3 ? sk_launch_nk<4, 4, 4, 3, 2, 8>(p, grid, stream)
-                             : sk_launch_nk<4, 4, 4, 3, 1, 8>(p, grid, stream);
+  // weights three steps ahead, activations one: deeper rings spill at 128 registers (+4 us), two and two is level
+  hipError_t e = mg == 2 ? sk_launch_nk<2, 4, 4, 3, 1, 8>(p, grid, stream) : sk_launch_nk<4, 4, 4, 3, 1, 8>(p, grid, stream);
   if (e != hipSuccess && p.S > 1 && p.ticket0 >= 0 && !plan_recording()) {
+    const int n = groups * grid_y;
+    sk_clear_tickets_kernel<<<dim3((n + 255) / 256), dim3(256), 0, stream>>>(p.ticket0, n);
+    (void)hipGetLastError();
+  }
+  return e;
+}
+
+// MXFP4, 33..64 rows per block row: four channel tiles x four K parts per workgroup, K in p.S slices across workgroups
+hipError_t launch_skinny_mxfp4_nk(DecodeParams& p, hipStream_t stream) {
+  const int groups = (p.total_tiles + 3) / 4, grid_y = (p.M + 63) / 64;
+  dim3 grid(groups * p.S, grid_y, 1);
+  const int nsteps = ((p.units + p.S - 1) / p.S + 3) / 4;
+  if (p.S > 4 || p.n_seg != 1 || nsteps > 8)
+    return hipErrorInvalidValue;
+  if (p.S > 1 && (p.ticket0 = skinny_split_tickets(groups * grid_y)) < 0)
+    return hipErrorInvalidValue;
+  const size_t lds = (size_t)2 * 4 * 64 * 16 * 16; // two stages x four K parts x 64 rows x 256 B (> the reduction's 64 KiB)
+  const int form = env_int("TPPX_MXFP4_NK_FORM", 0);
+  hipError_t e;
+  if (form == 1) { // one tile per wave, sixteen waves
+    const auto kern = skinny_mxfp4_nk_kernel<4, 4, 1, 4, 6, 2, 8>;
+    TPPX_PLAN_ONLY(kern, grid, dim3(1024), lds);
+    e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds);
+    if (e == hipSuccess) {
+      kern<<<grid, dim3(1024), lds, stream>>>(p);
+      e = hipGetLastError();
+    }
+  } else { // two tiles per wave, eight waves: half the operand reads from LDS per MFMA
+    const auto kern = skinny_mxfp4_nk_kernel<4, 4, 2, 4, 6, 2, 8>;
+    TPPX_PLAN_ONLY(kern, grid, dim3(512), lds);
+    e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds);
+    if (e == hipSuccess) {
+      kern<<<grid, dim3(512), lds, stream>>>(p);
+      e = hipGetLastError();
+    }
+  }
+  if (e != hipSuccess && p.S > 1 && p.ticket0 >= 0) {
     const int n = groups * grid_y;
     sk_clear_tickets_kernel<<<dim3((n + 255) / 256), dim3(256), 0, stream>>>(p.ticket0, n);
     (void)hipGetLastError();
