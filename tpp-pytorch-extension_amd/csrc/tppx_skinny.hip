@@ -47,6 +47,13 @@ __device__ __forceinline__ uint32_t sk_pack_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
+// floor(a * b / c) for the K-range splits: a * b stays far below 2^31 (at most 2^18 tiles times 16 waves or 4 parts),
+// so one 32-bit unsigned division does (the 64-bit form is a hundred instructions and four branches per use, and stood
+// in front of every kernel's first weight request).
+__device__ __forceinline__ int sk_share(int a, int b, int c) {
+  return (int)(((unsigned int)a * (unsigned int)b) / (unsigned int)c);
+}
+
 __device__ __forceinline__ int sk_find_seg(const DecodeParams& p, int grp) {
   int s = 0;
 #pragma unroll
@@ -84,6 +91,11 @@ struct SkEpilogue {
   // conditional makes the compiler wait for every outstanding load at the join, which here stood between the
   // activations and the first weight request of the kernel.
   __device__ __forceinline__ void prefetch_flat(const DecodeParams& p, const DecodeSeg& sg, int ltile0, int m0) {
+    // Everything the loop needs of the descriptors is read ONCE into scalars here: left to the use sites, every
+    // element's offset arithmetic fetched its fields again behind branches of its own (in the 64-row kernels 43 scalar
+    // loads, 29 waits and 45 branches stood in front of the first weight request).  The QINT8 kernels never split
+    // their output over several matrices (DecodeSeg::split1 is the MXFP4 q/k/v launch's), so the offset is m * N + n.
+    const int M = p.M, N = sg.N, tiles = sg.tiles;
     has_bias = sg.bias != nullptr;
     has_bias2 = DUAL && p.seg[1].bias != nullptr;
     has_in1 = sg.post_in != nullptr;
@@ -98,8 +110,8 @@ struct SkEpilogue {
       const int l = e & 63, r = (e >> 6) & 3, mg = (e >> 8) % MG, a = (e >> 8) / MG;
       const int m = m0 + mg * 16 + (l >> 4) * 4 + r;
       const int n = (ltile0 + a) * 16 + (l & 15);
-      const bool valid = e < OUT && m < p.M && (ltile0 + a) < sg.tiles;
-      const int o = valid ? seg_out_offset(sg, p.M, m, n) : 0, nn = valid ? n : 0;
+      const bool valid = e < OUT && m < M && (ltile0 + a) < tiles;
+      const int o = valid ? m * N + n : 0, nn = valid ? n : 0;
       off[i] = valid ? o : -1;
       bias[i] = pb[nn];
       bias2[i] = DUAL ? pb2[nn] : 0;
@@ -368,8 +380,8 @@ skinny_qint8_kernel(const DecodeParams p) {
   const bool FAST = G == 4;
   constexpr int UN = (PF % 4 == 0) ? PF : (PF % 2 == 0 ? 2 * PF : 4 * PF); // lcm(PF, 4) tiles per unrolled trip
   // runs of this workgroup (all of them unless K is split across workgroups), then of this wave
-  const int ub = (int)(((int64_t)blockIdx.z * p.units) / p.S), ue = (int)(((int64_t)(blockIdx.z + 1) * p.units) / p.S);
-  const int u0 = ub + (int)(((int64_t)wave * (ue - ub)) / W), u1 = ub + (int)(((int64_t)(wave + 1) * (ue - ub)) / W);
+  const int ub = sk_share(blockIdx.z, p.units, p.S), ue = sk_share(blockIdx.z + 1, p.units, p.S);
+  const int u0 = ub + sk_share(wave, ue - ub, W), u1 = ub + sk_share(wave + 1, ue - ub, W);
   const int t0 = u0 * G, t1 = u1 * G;
   const unsigned int magic = p.spb_magic;
   auto blk_of = [&](int t, bool fast) { // scale block of tile t (uniform)
@@ -401,6 +413,7 @@ skinny_qint8_kernel(const DecodeParams p) {
   // them does not wait for HBM.
   SkEpilogue<MG, NTW, false, MINW> ep;
   ep.prefetch_flat(p, sg, ltile0, m0);
+  __builtin_amdgcn_sched_barrier(0); // keep the issue order of independent loads (see skinny_qint8_fq_kernel)
   // activation scales of this wave's K blocks, transposed in LDS: [u - u0][MPAD]
   float* red = sk_lds;
   float* sa_s = sk_lds + (size_t)W * NTW * MG * 256 + (size_t)wave * p.cht * MPAD;
@@ -419,6 +432,7 @@ skinny_qint8_kernel(const DecodeParams p) {
 #pragma unroll
   for (int j = 0; j < SAB; j++)
     sa0[j] = load_sa(j * 64 + lane);
+  __builtin_amdgcn_sched_barrier(0);
 
   // Ring of PF stages; a stage = the weight tiles, their block scale and the
   // activation operand of one k-tile.  The main loop has NO branch and NO load
@@ -677,7 +691,7 @@ skinny_qint8_nk_kernel(const DecodeParams p) {
   const unsigned int magic = p.spb_magic;
   auto blk_of_run = [&](int u) { return magic ? (int)__umulhi((unsigned int)u, magic) : u; };
   // runs of this workgroup's K slice, then of this wave's K part; every wave makes the same number of steps
-  const int ub = (int)(((int64_t)z * NR) / S), ue = (int)(((int64_t)(z + 1) * NR) / S);
+  const int ub = sk_share(z, NR, S), ue = sk_share(z + 1, NR, S);
   const int u0 = ub + (kp * (ue - ub)) / KPW, u1 = ub + ((kp + 1) * (ue - ub)) / KPW;
   const int nsteps = (ue - ub + KPW - 1) / KPW; // <= MAXSTEPS (the launcher checks)
 
@@ -795,7 +809,7 @@ skinny_mxfp4_nk_kernel(const DecodeParams p) {
   const int ltile0 = grp * TW;
   const int m0 = blockIdx.y * MPAD;
   const int KT = p.units; // K tiles of 128
-  const int tb = (int)(((int64_t)z * KT) / S), te = (int)(((int64_t)(z + 1) * KT) / S);
+  const int tb = sk_share(z, KT, S), te = sk_share(z + 1, KT, S);
   const int t0 = tb + (kp * (te - tb)) / KPW, t1 = tb + ((kp + 1) * (te - tb)) / KPW;
   const int nsteps = (te - tb + KPW - 1) / KPW; // <= MAXSTEPS (the launcher checks)
 
@@ -958,7 +972,7 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
   const int ltile0 = (grp - sg.grp0) * NTW;
   const int M = p.M; // <= 16, one block row
   const int NR = p.units, KT = NR * 4, NB = p.nblk; // 256-wide runs of K, tiles, scale blocks
-  const int u0 = (int)(((int64_t)wave * NR) / W), u1 = (int)(((int64_t)(wave + 1) * NR) / W);
+  const int u0 = sk_share(wave, NR, W), u1 = sk_share(wave + 1, NR, W);
   const int t0 = u0 * 4, t1 = u1 * 4;
   const unsigned int magic = p.spb_magic;
   auto blk_of_run = [&](int u) { return BIGB ? (int)__umulhi((unsigned int)u, magic) : u; };
@@ -990,8 +1004,12 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
     raw[ps][1] = src[1];
   };
   static_for<0, XB>([&](auto PS) { load_pass(PS, 0); });
+  // (the scheduler is free to move independent loads past one another: pinned, or it puts some of the activation
+  // requests behind the weight ring and the quantisation waits for HBM)
+  __builtin_amdgcn_sched_barrier(0);
   SkEpilogue<1, NTW, false, MINW> ep;
   ep.prefetch_flat(p, sg, ltile0, 0);
+  __builtin_amdgcn_sched_barrier(0);
 
   // ring stage = weight tiles + their block scale (see skinny_qint8_kernel)
   i32x4 wreg[PF][NTW];
@@ -1009,6 +1027,7 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
 #pragma unroll
   for (int i = 0; i < PF; i++)
     load_stage(i, t0 + i);
+  __builtin_amdgcn_sched_barrier(0);
 
   // wave-private LDS: xq [tile][g][M rows][16 B], then sa [unit][16]; the region of the cross-wave reduction
   // comes first unless both do not fit side by side (they overlap then, with a barrier in between)
@@ -1597,7 +1616,7 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
   const int m0 = blockIdx.y * MPAD;
   const int KT = p.units;
   // K tiles of this workgroup (all of them unless K is split across workgroups), then of this wave
-  const int tb = (int)(((int64_t)blockIdx.z * KT) / p.S), te = (int)(((int64_t)(blockIdx.z + 1) * KT) / p.S);
+  const int tb = sk_share(blockIdx.z, KT, p.S), te = sk_share(blockIdx.z + 1, KT, p.S);
   const int t0 = tb + (wave * (te - tb)) / W, t1 = tb + ((wave + 1) * (te - tb)) / W;
   i32x4* xs = reinterpret_cast<i32x4*>(sk_lds) + (size_t)wave * (MPAD * 16); // [chunk 16][row MPAD] x 16 B
 
