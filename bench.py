@@ -428,6 +428,62 @@ def cpu_baseline_decode(fmt, W, X, R, Ms, shapes, qbs, bytes_per_step, seconds=1
 
 
 # ---------------------------------------------------------------------------------------------------------------
+# config 2's shapes with QINT4 and ternary QINT2 weights (the other members of the reference's W8A8 class): decode
+# steps stream the codes at their own width
+# ---------------------------------------------------------------------------------------------------------------
+def leg_low_bit(torch, _ops, args):
+    from tpp_pytorch_extension import _lib
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(1240)
+    rows, total_bytes, total_us = [], 0.0, 0.0
+    for kind, bits in (("qint4", 4), ("qint2", 2)):
+        for name, (N, K) in CFG2_SHAPES.items():
+            nc = 16  # 16 copies x 11..22 MB per shape: beyond the 256 MB Infinity Cache together with the other shape
+
+            def mk():
+                W = (torch.randn((N, K), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+                if kind == "qint4":
+                    t = W.view(N // 16, 16, K // 256, 128, 2).permute(0, 2, 3, 1, 4).contiguous()
+                    w = _ops.quantize_int4sym(t, 256, 2, True)
+                else:
+                    w = _ops.remap_and_quantize_qint2_intlv(block_bf16(W))
+                w.native_packed()
+                w._native = None  # the decode step needs the packed codes only
+                return w
+
+            ws = [mk() for _ in range(nc)]
+            for M in (1, 8):
+                x = torch.randn((M, K), generator=g, device=dev).to(torch.bfloat16)
+                r = torch.randn((M, N), generator=g, device=dev).to(torch.bfloat16)
+
+                def fire(_st):
+                    return [_ops.fc_add(x, w, None, r, 1.0) for w in ws]
+
+                fire(None)
+                us, n = events_us(torch, fire, nc, use_graph=not args.no_graph)
+                nbytes = N * K * bits // 8 + 4 * N * (K // 256) + 2 * M * K + 4 * M * N
+                rows.append({"kernel": kind, "call": f"{name} M={M}", "kernels_per_call": 1, "avg_launch_us": round(us, 3),
+                             "bytes_per_launch": nbytes, "achieved": round(nbytes / us / 1e3, 1),
+                             "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "launches_timed": n})
+                total_bytes += nbytes
+                total_us += us
+            del ws
+    dom = max(rows, key=lambda r: r["avg_launch_us"])
+    buf = ctypes.create_string_buffer(1024)
+    return {
+        "leg": "cfg2-qint4-qint2", "metric": "quant-GEMM HBM TB/s (decode)", "value": round(total_bytes / total_us / 1e6, 4),
+        "unit": "TB/s", "ms_per_step": round(total_us / 1e3, 5), "dtype": "int8",
+        "workload": "cfg2 shapes, QINT4 and ternary QINT2 weights (codes streamed at 4 / 2 bits), fc_add, M in {1,8}",
+        "roofline": {"bound": "hbm", "kernel": "skinny_qint8_fq_kernel<.., 4 | 2> (" + dom["kernel"] + ")", "call": dom["call"],
+                     "achieved": dom["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"], "traffic": None,
+                     "avg_launch_us": dom["avg_launch_us"], "bytes_per_launch": dom["bytes_per_launch"],
+                     "all_gemm_kernels": rows},
+        "cpu_baseline": None,
+    }
+
+
+# ---------------------------------------------------------------------------------------------------------------
 # config 1: one MXFP4 fc_plain, M = 16, 4096 x 4096, bias
 # ---------------------------------------------------------------------------------------------------------------
 def leg_cfg1(torch, _ops, args):
@@ -841,7 +897,7 @@ def run_prompt(torch, args):
 
 
 def short_kernel(name):
-    return name.replace("tppx::", "").replace("_kernel", "").replace(" ", "")
+    return name.replace("tppx::", "").replace("_kernel", "").replace("skinny_", "sk_").replace(" ", "")
 
 
 def compact_rows(rows):
@@ -872,7 +928,10 @@ def compact_cpu(c, leg=False):
     if not c:
         return c
     out = dict(c)
-    out["sample"] = out.get("sample", "").split(" (")[0][:70 if leg else 110]
+    out["sample"] = out.get("sample", "").split(" (")[0][:40 if leg else 110]
+    if leg:  # same host, same threads and the same kind of baseline as the headline's
+        out.pop("cores", None)
+        out.pop("kind", None)
     return out
 
 
@@ -882,10 +941,10 @@ def compact_leg(leg):
         return leg
     # value, unit, ms_per_step, the dominant kernel, its duration and fraction are in the line's `summary` row of the leg
     roof = compact_roofline(leg["roofline"], True)
-    for k in ("kernel", "avg_launch_us", "frac"):
+    for k in ("kernel", "avg_launch_us", "frac", "unit", "peak"):
         roof.pop(k, None)
     out = {"leg": leg["leg"], "dtype": leg["dtype"],
-           "workload": leg["workload"].split(";")[0].split(" linears of")[0][:72], "roofline": roof,
+           "workload": leg["workload"].split(";")[0].split(" linears of")[0].split(", Llama")[0][:60], "roofline": roof,
            "cpu_baseline": compact_cpu(leg["cpu_baseline"], True)}
     rows = leg["roofline"].get("all_gemm_kernels")
     if rows:
@@ -906,7 +965,7 @@ def summary_of(headline, legs):
         ratio = round(tr / r["bytes_per_launch"], 3) if tr and r.get("bytes_per_launch") else None
         cpu = d.get("cpu_baseline") or {}
         rows.append([name, d["value"], d["unit"], d.get("ms_per_step", round(d.get("us_per_call", 0.0) / 1e3, 6)),
-                     short_kernel(r.get("kernel", ""))[:40],
+                     short_kernel(r.get("kernel", ""))[:32],
                      r.get("avg_launch_us"), r.get("frac"), ratio, cpu.get("value")])
     return rows
 
@@ -982,6 +1041,7 @@ def main():
 
         todo = [
             ("cfg2-per-channel", per_channel_leg),
+            ("cfg2-qint4-qint2", lambda: leg_low_bit(torch, _ops, args)),
             ("cfg1", lambda: leg_cfg1(torch, _ops, args)),
             ("cfg3", lambda: leg_cfg3(torch, _ops, args)),
             ("cfg4", lambda: leg_cfg4(torch, _ops, args, "mxfp4", False)),
@@ -1012,12 +1072,12 @@ def main():
             print("bench.py verbose: " + json.dumps(leg), file=sys.stderr)
         out["config"]["legs"] = [compact_leg(l) for l in legs]
         out["config"]["run_wall_s"] = round(time.perf_counter() - t_start, 1)
-        out["config"]["gemm_kernels_columns"] = "kernel, call, GEMM kernel us, frac of peak[, kernels per call, whole-call us]"
+        out["config"]["gemm_kernels_columns"] = "kernel, call, kernel us, frac[, kernels per call, call us]"
         out["config"].pop("timed", None)
         out["config"]["gemm_kernels"] = compact_rows(out["roofline"].pop("all_gemm_kernels"))
         out["roofline"] = compact_roofline(out["roofline"])
         out["cpu_baseline"] = compact_cpu(out["cpu_baseline"])
-        out["summary_columns"] = "leg, value, unit, ms_per_step, dominant kernel, its us, frac of roofline, HBM traffic / algorithmic bytes, cpu value"
+        out["summary_columns"] = "leg, value, unit, ms_per_step, dominant kernel, its us, roofline frac, HBM traffic / algorithmic bytes, cpu value"
         out["summary"] = summary_of(out, legs)
     print(json.dumps(out, separators=(",", ":")))
 

@@ -253,9 +253,9 @@ def test_launch_plans_of_per_output_channel_qint8():
     ws = 1 << 25
     for M in (1, 8):
         one = plan(M, 11008, 4096, 4096, 1, 0, ws)
-        assert len(one) == 1 and "skinny_qint8_fq_kernel<3, 4, 16, 16, 4, true> grid=230x1x1 block=1024" in one[0], one
+        assert len(one) == 1 and "skinny_qint8_fq_kernel<3, 4, 16, 16, 4, true, 8> grid=230x1x1 block=1024" in one[0], one
         one = plan(M, 4096, 11008, 11008, 1, 0, ws)
-        assert len(one) == 1 and "skinny_qint8_fq_kernel<1, 4, 16, 16, 6, true> grid=256x1x1 block=1024" in one[0], one
+        assert len(one) == 1 and "skinny_qint8_fq_kernel<1, 4, 16, 16, 6, true, 8> grid=256x1x1 block=1024" in one[0], one
     two = plan(64, 11008, 4096, 4096, 1, 0, ws)
     assert len(two) == 2 and "quant_act_int8_bigblk_kernel grid=64x1x1 block=256" in two[0], two
     assert "skinny_qint8_kernel<4, 3, 2, 8, 8, true> grid=230x1x1 block=512" in two[1], two

@@ -322,3 +322,37 @@ def test_w4a8_linear(M, post):
         assert torch.equal(q1, y) and torch.equal(q2, ops.linear(x.cuda(), qt, None))
         sw = ops.swiglu_gate_up(x.cuda(), qt, qt)
         assert torch.equal(sw, ops.fc_mul(x.cuda(), qt, None, ops.fc_silu(x.cuda(), qt, None)))
+
+
+@pytest.mark.parametrize("kind", ["qint4", "qint2"])
+@pytest.mark.parametrize("M,N,K,post", [(1, 11008, 4096, "none"), (8, 4096, 11008, "add"), (16, 4096, 4096, "silu"),
+                                        (5, 96, 1024, "mul"), (3, 8448, 14336, "add")])
+def test_packed_code_decode_kernel_equals_expanded_weight(kind, M, N, K, post, monkeypatch):
+    """QINT4 / ternary QINT2 weights at their own width (src/csrc/fused_gemm.h:1110-1126 multiplies the packed codes as
+    they lie): up to 16 rows the decode kernel streams N*K/2 or N*K/4 bytes of codes and expands them in registers in
+    front of the int8 MFMA.  Same integer sums, scales and rounding as the expanded int8 tiles, so the SAME BITS as
+    that path (TPPX_PACKED_CODES=0), and within 1 ulp (2 through SiLU) of the oracle on the expanded weight."""
+    ops = _ops()
+    from tpp_pytorch_extension import _lib
+    posts = {"none": O.POST_NONE, "add": O.POST_ADD_SCALE, "silu": O.POST_SILU, "mul": O.POST_MUL}
+    W = randn_bf16((N, K), 0.02, 2600 + M)
+    if kind == "qint4":
+        t = W.view(N // 16, 16, K // 256, 128, 2).permute(0, 2, 3, 1, 4).contiguous()  # VNNI2 [N/16][K/256][128][16][2]
+        qt = ops.quantize_int4sym(t.cuda(), 256, 2, True)
+    else:
+        qt = ops.remap_and_quantize_qint2_intlv(block_bf16(W).cuda())
+    assert qt.weight_kind() == kind and qt.block_size == 256
+    x = randn_bf16((M, K), 1.0, 2610 + M).cuda()
+    b = randn_bf16((N,), 0.01, 2620).cuda()
+    r = randn_bf16((M, N), 1.0, 2630).cuda()
+    y = ops.linear(x, qt, b, posts[post], r, None, 0.5)
+    packed, sn, bits = qt.native_packed()
+    assert packed.numel() == N * K * bits // 8
+    monkeypatch.setattr(ops, "PACKED_CODES", False)
+    y_expanded = ops.linear(x, qt, b, posts[post], r, None, 0.5)
+    assert torch.equal(y, y_expanded), "packed codes and expanded int8 tiles give different bits"
+    # the packed path really ran: the entry point accepts the call (no fall-through)
+    y2 = torch.empty_like(y)
+    _lib.check(_lib.lib().tppx_linear_qintx(x.data_ptr(), packed.data_ptr(), sn.data_ptr(), b.data_ptr(), r.data_ptr(), None,
+                                            y2.data_ptr(), M, N, K, bits, posts[post], 0.5, _lib.stream_of(x)))
+    assert torch.equal(y2, y)

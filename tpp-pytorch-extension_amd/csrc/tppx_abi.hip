@@ -803,6 +803,38 @@ extern "C" int tppx_linear_qint8_noalloc(const void* x, const void* qw, const vo
                    (int64_t)NA_WS_BYTES, (hipStream_t)stream);
 }
 
+extern "C" int tppx_linear_qintx(const void* x, const void* qw_packed, const void* sw, const void* bias,
+                                 const void* post_in, const void* post_in2, void* y, int64_t M, int64_t N, int64_t K,
+                                 int bits, int post_op, float post_scale, tppx_stream_t stream) {
+  const char* who = "tppx_linear_qintx";
+  int rc = check_common(who, x, M, K, 1, 0, nullptr, 0);
+  if (rc)
+    return rc;
+  TPPX_REQUIRE(bits == 4 || bits == 2, TPPX_EINVAL, "%s: %d-bit codes are not built (4 or 2)", who, bits);
+  TPPX_REQUIRE(M <= 16, TPPX_EUNSUPPORTED, "%s: the packed-code kernel takes at most 16 rows (M=%ld); larger calls run on the expanded int8 tiles", who, (long)M);
+  TPPX_REQUIRE(K > 0 && K % 256 == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of the 256-wide scale block", who, (long)K);
+  tppx_seg s = {qw_packed, sw, bias, post_in, post_in2, y, N, post_op, post_scale};
+  DecodeParams p;
+  memset(&p, 0, sizeof(p));
+  rc = fill_all(who, &s, 1, 16, false, p);
+  if (rc)
+    return rc;
+  p.x = x;
+  p.M = (int)M;
+  p.K = (int)K;
+  p.tpb = 4;
+  p.nblk = (int)(K / 256);
+  p.deal = 4;
+  p.units = p.nblk;
+  p.spb_magic = 0;
+  p.S = 1;
+  p.wbits = bits;
+  SkinnyPlan sp = plan_skinny(M, p.total_tiles, p.units, p.tpb, p.deal, true);
+  TPPX_REQUIRE(sp.fused_quant, TPPX_EUNSUPPORTED, "%s: M=%ld rows of K=%ld channels do not fit the in-kernel quantisation's LDS; run the call on the expanded int8 tiles", who, (long)M, (long)K);
+  set_groups(p, sp.ntw, false);
+  return check_hip(launch_skinny_qint8(p, sp, (hipStream_t)stream), who);
+}
+
 extern "C" void tppx_reload_env(void) {
   std::lock_guard<std::mutex> lock(g_env_mu);
   g_env_kept.clear();

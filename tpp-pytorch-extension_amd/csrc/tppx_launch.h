@@ -53,6 +53,7 @@ struct DecodeParams {
   // scale block folds its exact int32 sums with the block's scales like a block of its own.
   int deal;
   int nblk;  // QINT8: K / qbs scale blocks
+  int wbits; // QINT8 family, fused-quantisation kernel: 4 or 2 = seg[].qw holds packed codes (tppx_pack_qint_tiles); else int8 tiles
   // deal == 4: scale block of run u = spb_magic ? mulhi(u, spb_magic) : u   (spb_magic = ceil(2^32 / (tpb / 4)),
   // exact for u * (tpb / 4) < 2^32; 0 when a block is one run)
   unsigned int spb_magic;

@@ -729,6 +729,44 @@ prepack_qint4_kernel(const uint8_t* __restrict__ q4, int64_t N, int64_t K, int64
   reinterpret_cast<uint4*>(qnat)[t] = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
+// Native int8 tiles [N/16][K/64][64 lanes][16 B] of a QINT4 / QINT2 weight -> the codes at their own width, for the
+// decode kernel that expands them in registers: [N/16][K/(64 G)][64 lanes][16 B], G = 8 / BITS tiles per 16 bytes.
+//   BITS 4: byte b of dword d = (tile 0's byte d*4+b & 15) | (tile 1's byte d*4+b << 4)        (values -8..7)
+//   BITS 2: byte i of dword kt = two's-complement 2-bit codes (0, 1, 3 = -1) of tile kt's bytes i, 4+i, 8+i, 12+i
+//           (byte i of its four operand dwords) in bits 0-1, 2-3, 4-5, 6-7
+template <int BITS>
+__global__ void __launch_bounds__(256)
+pack_qint_tiles_kernel(const int8_t* __restrict__ nat, int64_t groups, uint8_t* __restrict__ out) {
+  constexpr int G = 8 / BITS;
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; // (tile group, lane)
+  if (t >= groups * 64)
+    return;
+  const int64_t grp = t >> 6;
+  const int lane = (int)(t & 63);
+  int8_t v[G][16];
+#pragma unroll
+  for (int g = 0; g < G; g++) {
+    const uint4 w = reinterpret_cast<const uint4*>(nat)[(grp * G + g) * 64 + lane];
+    const uint32_t d[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      v[g][i] = (int8_t)((d[i >> 2] >> (8 * (i & 3))) & 0xffu);
+  }
+  uint32_t o[4] = {0, 0, 0, 0};
+  if (BITS == 4) {
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      o[i >> 2] |= (((uint32_t)v[0][i] & 15u) | (((uint32_t)v[G - 1][i] & 15u) << 4)) << (8 * (i & 3));
+  } else {
+#pragma unroll
+    for (int kt = 0; kt < G; kt++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) // value i = byte i & 3 of operand dword i >> 2
+        o[kt & 3] |= ((uint32_t)v[kt][i] & 3u) << (8 * (i & 3) + 2 * (i >> 2));
+  }
+  reinterpret_cast<uint4*>(out)[t] = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 static inline unsigned grid_for(int64_t n, int block) {
   return (unsigned)((n + block - 1) / block);
 }
@@ -868,6 +906,21 @@ extern "C" int tppx_prepack_qint8(const void* q_ref, int64_t N, int64_t K,
   prepack_qint8_kernel<<<grid_for(nchunks, 256), 256, 0, (hipStream_t)stream>>>(
       (const int8_t*)q_ref, N, K, qbs, (int8_t*)q_nat);
   return check_hip(hipGetLastError(), "tppx_prepack_qint8");
+}
+
+extern "C" int tppx_pack_qint_tiles(const void* native_i8, int64_t N, int64_t K, int bits, void* packed,
+                                    tppx_stream_t stream) {
+  const char* who = "tppx_pack_qint_tiles";
+  TPPX_REQUIRE(native_i8 && packed, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(aligned16(native_i8) && aligned16(packed), TPPX_EINVAL, "%s: pointer not 16-byte aligned", who);
+  TPPX_REQUIRE(bits == 4 || bits == 2, TPPX_EINVAL, "%s: %d-bit codes are not built (4 or 2)", who, bits);
+  TPPX_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 256 == 0, TPPX_ESHAPE, "%s: N=%ld must be a multiple of 16 and K=%ld of 256", who, (long)N, (long)K);
+  const int64_t groups = (N / 16) * (K / 64) / (8 / bits);
+  if (bits == 4)
+    pack_qint_tiles_kernel<4><<<grid_for(groups * 64, 256), 256, 0, (hipStream_t)stream>>>((const int8_t*)native_i8, groups, (uint8_t*)packed);
+  else
+    pack_qint_tiles_kernel<2><<<grid_for(groups * 64, 256), 256, 0, (hipStream_t)stream>>>((const int8_t*)native_i8, groups, (uint8_t*)packed);
+  return check_hip(hipGetLastError(), who);
 }
 
 extern "C" int tppx_prepack_bf16(const void* w_ref, int64_t N, int64_t K, int64_t bk, int64_t bc, int vnni,

@@ -961,9 +961,33 @@ __device__ __forceinline__ uint32_t sk_int8x4_rne(float a, float b, float c, flo
 // BIGB: scale blocks of several 256-wide runs.  Every wave takes the maxima of its own (row, run) items, the waves
 // exchange them through LDS (one barrier), and an item is quantised with the maximum over the runs of its block; all
 // of a wave's items stay in registers meanwhile (the launcher checks that there are at most 4 * XB).
-template <int NTW, int PF, int MAXW, int MINW, int XB, bool BIGB>
+// WBITS = 4 / 2: QINT4 / ternary QINT2 weights streamed at their own width.  A 16-byte load per lane then holds the
+// lane's operands of G = 8 / WBITS consecutive K tiles (tppx_pack_qint_tiles), expanded in registers right in front
+// of the MFMA, two instructions per operand dword: 4-bit codes as 16 x value (the nibble moved to the top of its
+// byte), ternary codes as 64 x value (two's complement in two bits -- 0, 1, 3 = -1 -- moved to the top of their
+// byte); the fold divides by 16 or 64, which is exact.  The ring's stages are such loads (PF of them).
+template <int WBITS>
+__device__ __forceinline__ i32x4 sk_expand_codes(i32x4 w, int g) {
+  i32x4 o;
+  if constexpr (WBITS == 4) {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      o[j] = (int)((g == 0 ? ((uint32_t)w[j] << 4) : (uint32_t)w[j]) & 0xF0F0F0F0u);
+  } else {
+    // dword g = K tile g; its byte i holds the codes of byte i of the four operand dwords j, two bits each
+    const uint32_t pw = (uint32_t)(g == 0 ? w[0] : g == 1 ? w[1] : g == 2 ? w[2] : w[3]);
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      o[j] = (int)((j == 3 ? pw : (pw << (6 - 2 * j))) & 0xC0C0C0C0u);
+  }
+  return o;
+}
+
+template <int NTW, int PF, int MAXW, int MINW, int XB, bool BIGB, int WBITS = 8>
 __global__ void __launch_bounds__(MAXW * 64)
 skinny_qint8_fq_kernel(const DecodeParams p) {
+  constexpr int G = 8 / WBITS; // K tiles per 16-byte weight load of a lane
+  static_assert(WBITS == 8 || !BIGB, "the packed formats run 256-wide blocks");
   extern __shared__ __align__(16) float sk_lds[];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int W = blockDim.x >> 6;
@@ -982,7 +1006,7 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
 #pragma unroll
   for (int nt = 0; nt < NTW; nt++) {
     const int64_t lt = min(ltile0 + nt, sg.tiles - 1);
-    wq[nt] = reinterpret_cast<const i32x4*>(sg.qw) + lt * KT * 64 + lane;
+    wq[nt] = reinterpret_cast<const i32x4*>(sg.qw) + lt * (KT / G) * 64 + lane;
     ws[nt] = reinterpret_cast<const float*>(sg.sw) + lt * NB * 16 + (lane & 15);
   }
   // Loads return in issue order, so everything small and L2-resident that the
@@ -1014,19 +1038,20 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
   // ring stage = weight tiles + their block scale (see skinny_qint8_kernel)
   i32x4 wreg[PF][NTW];
   float sreg[PF][NTW];
+  // (WBITS < 8: `t` counts 16-byte loads = groups of G tiles; t0, t1 are multiples of 4, so of G)
   auto load_stage = [&](int st, int t) {
-    t = max(min(t, t1 - 1), 0); // past the end (or a wave without K blocks): re-read a valid tile, never consumed
+    t = max(min(t, t1 / G - 1), 0); // past the end (or a wave without K blocks): re-read a valid tile, never consumed
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
       wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64);
-      sreg[st][nt] = ws[nt][blk_of_run(t >> 2) * 16];
+      sreg[st][nt] = ws[nt][blk_of_run((t * G) >> 2) * 16];
     }
   };
   // No branch around the ring's first requests: with one, the compiler can no longer count the loads behind the
   // activations and waits for the whole ring before it lets the quantisation start.
 #pragma unroll
   for (int i = 0; i < PF; i++)
-    load_stage(i, t0 + i);
+    load_stage(i, t0 / G + i);
   __builtin_amdgcn_sched_barrier(0);
 
   // wave-private LDS: xq [tile][g][M rows][16 B], then sa [unit][16]; the region of the cross-wave reduction
@@ -1152,24 +1177,69 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
         }
     }
   };
-  int t = t0;
-  for (; t + 2 * PF <= t1; t += PF) { // branch-free full groups (PF is a multiple of 4): every reload is a real tile
+  if constexpr (WBITS == 8) {
+    int t = t0;
+    for (; t + 2 * PF <= t1; t += PF) { // branch-free full groups (PF is a multiple of 4): every reload is a real tile
 #pragma unroll
-    for (int i = 0; i < PF; i++) {
-      consume(i, t + i, (i & 3) == 3);
-      load_stage(i, t + i + PF);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  }
-  for (; t < t1; t += PF) {
-#pragma unroll
-    for (int i = 0; i < PF; i++) {
-      const int tt = t + i;
-      if (tt < t1) {
-        consume(i, tt, (i & 3) == 3);
-        if (tt + PF < t1)
-          load_stage(i, tt + PF);
+      for (int i = 0; i < PF; i++) {
+        consume(i, t + i, (i & 3) == 3);
+        load_stage(i, t + i + PF);
+        __builtin_amdgcn_sched_barrier(0);
       }
+    }
+    for (; t < t1; t += PF) {
+#pragma unroll
+      for (int i = 0; i < PF; i++) {
+        const int tt = t + i;
+        if (tt < t1) {
+          consume(i, tt, (i & 3) == 3);
+          if (tt + PF < t1)
+            load_stage(i, tt + PF);
+        }
+      }
+    }
+  } else {
+    // one stage = G tiles; a run of 256 channels (4 tiles) closes every 4 / G stages
+    auto consume_packed = [&](int i, int s) {
+#pragma unroll
+      for (int g = 0; g < G; g++) {
+        const int tt = s * G + g;
+        const i32x4 xa = *reinterpret_cast<const i32x4*>(xq_s + (tt - t0) * 16 * M + xoff);
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++)
+          iacc[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa, sk_expand_codes<WBITS>(wreg[i][nt], g), iacc[nt], 0, 0, 0);
+        if ((tt & 3) == 3) {
+          const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + ((tt >> 2) - u0) * 16 + (lane >> 4) * 4);
+#pragma unroll
+          for (int nt = 0; nt < NTW; nt++) {
+            const float swv = sreg[i][nt] * (WBITS == 4 ? 0.0625f : 0.015625f); // operands are 16 x / 64 x the value
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              facc[nt][0][r] = fmaf((float)iacc[nt][r], sav[r] * swv, facc[nt][0][r]);
+              iacc[nt][r] = 0;
+            }
+          }
+        }
+      }
+    };
+    const int s1 = t1 / G;
+    int s = t0 / G;
+    for (; s + 2 * PF <= s1; s += PF) { // branch-free full groups
+#pragma unroll
+      for (int i = 0; i < PF; i++) {
+        consume_packed(i, s + i);
+        load_stage(i, s + i + PF);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    for (; s < s1; s += PF) {
+#pragma unroll
+      for (int i = 0; i < PF; i++)
+        if (s + i < s1) {
+          consume_packed(i, s + i);
+          if (s + i + PF < s1)
+            load_stage(i, s + i + PF);
+        }
     }
   }
   if (p.lds_overlap)
@@ -1994,6 +2064,19 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
     const size_t xbytes = (size_t)16 * pl.max_units * (256 * (size_t)p.M + 64) + abytes, rbytes = (size_t)16 * pl.ntw * 1024;
     const size_t lds = pl.lds_overlap ? (xbytes > rbytes ? xbytes : rbytes) : xbytes + rbytes;
     p.lds_overlap = pl.lds_overlap ? 1 : 0;
+    if (p.wbits == 4 || p.wbits == 2) { // packed codes (256-wide blocks; the caller checks)
+#define SKQX(NTW, XB)                                                                                           \
+  return p.wbits == 4 ? sk_launch(skinny_qint8_fq_kernel<NTW, 4, 16, 16, XB, false, 4>, p, grid, 16, lds, stream) \
+                      : sk_launch(skinny_qint8_fq_kernel<NTW, (NTW == 3 ? 2 : 4), 16, 16, XB, false, 2>, p, grid, 16, lds, stream)
+      if (pl.ntw == 3)
+        SKQX(3, 2);
+      if (pl.ntw == 2)
+        SKQX(2, 4);
+      if ((int64_t)p.M * pl.max_units > 16)
+        SKQX(1, 6);
+      SKQX(1, 4);
+#undef SKQX
+    }
     if (bigb) { // all (row, run) items of a wave stay in registers: M * runs per wave <= 4 * XB (plan_skinny checked)
       if (pl.ntw == 3)
         return sk_launch(skinny_qint8_fq_kernel<3, 4, 16, 16, 4, true>, p, grid, 16, lds, stream);

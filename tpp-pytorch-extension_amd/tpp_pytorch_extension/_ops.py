@@ -604,6 +604,7 @@ def _linear_other_types(input, weight, bias, post, flags, post_in=None, post_in2
     return _wide_post(y, ctype, post, post_in, post_in2, post_scale, shape[:-1] + (N,))
 
 
+PACKED_CODES = os.environ.get("TPPX_PACKED_CODES", "1") == "1"
 W4A8_ACT_SCALE = 6.0 / 127.0
 
 
@@ -685,6 +686,16 @@ def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None
     bias = _prep_bias(bias, N, x.device)
     post_in = _prep_post(post_in, M, N, "post-op input", x.device)
     post_in2 = _prep_post(post_in2, M, N, "second post-op input", x.device)
+    # QINT4 / QINT2 decode steps: the codes streamed at their own width and expanded in registers (same bits as the
+    # expanded int8 tiles).  TPPX_PACKED_CODES=0 keeps the expanded tiles.
+    if PACKED_CODES and M <= 16 and weight.weight_kind() in ("qint4", "qint2") and weight.block_size == 256 \
+            and row_sumsq is None and not flags:
+        qp, sp, bits = weight.native_packed()
+        rc = L.tppx_linear_qintx(x.data_ptr(), qp.data_ptr(), sp.data_ptr(), _lib.ptr(bias), _lib.ptr(post_in),
+                                 _lib.ptr(post_in2), y.data_ptr(), M, N, K, bits, post, post_scale, _lib.stream_of(x))
+        if rc != _lib.EUNSUPPORTED:  # rows that do not fit the in-kernel quantisation fall through to the int8 tiles
+            _lib.check(rc)
+            return y
     qn, sn = weight.native()
     st = _lib.stream_of(x)
     ws = _lib.workspace(x)

@@ -147,6 +147,22 @@ class QTensor(torch.Tensor):
             self._native = (qn, sn)
         return self._native
 
+    def native_packed(self):
+        """QINT4 / QINT2 weights: (codes at their own width in the decode kernel's order, scales, bits) --
+        N*K*bits/8 bytes made once from the native int8 tiles (tppx_pack_qint_tiles)."""
+        have = getattr(self, "_native_packed", None)
+        if have is None:
+            kind = self.weight_kind()
+            if kind not in ("qint4", "qint2"):
+                raise _lib.TppxError(_lib.EUNSUPPORTED, f"only QINT4 / QINT2 weights have a packed native form: {self!r}")
+            bits = 4 if kind == "qint4" else 2
+            qn, sn = self.native()
+            N, K = self.weight_nk()
+            packed = torch.empty(N * K * bits // 8, dtype=torch.uint8, device=qn.device)
+            _lib.check(_lib.lib().tppx_pack_qint_tiles(qn.data_ptr(), N, K, bits, packed.data_ptr(), _lib.stream_of(qn)))
+            have = self._native_packed = (packed, sn, bits)
+        return have
+
     def dequantize(self):
         """fp32 tensor in the blocked shape (PerBlock*Quantizer::dequantize,
         src/csrc/qtypes.cpp:438-473,521-577)."""
