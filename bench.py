@@ -249,13 +249,6 @@ def run_decode(torch, _ops, args, per_channel=False):
         else:
             step(pool[i % len(pool)])
 
-    if args.pmc_calibrate:
-        src = torch.ones(64 * 1024 * 1024, dtype=torch.int32, device=dev)  # 256 MiB read + 256 MiB written
-        for _ in range(3):
-            dst = src.clone()
-        torch.cuda.synchronize()
-        del src, dst
-
     ms_per_step, blocks = time_blocks(torch, run_step, args.steps, args.warmup)
     value_tbs = bytes_per_step / (ms_per_step * 1e-3) / 1e12
 
@@ -690,13 +683,18 @@ def leg_cfg4(torch, _ops, args, pfmt="mxfp4", fp8=False, cpu=True):
             ("down M=2048 N=8192 K=28672", lambda st: torch.ops.tpp_llm.fc_add(inter, wd, empty, res, 1.0),
              2.0 * M * H * I, kernel_plan(L, pfmt, M, H, I, 256, flags, wsb(I))),
         ]
+        wb = (lambda N, K: N * K // 2 + N * K // 32) if pfmt == "mxfp4" else (lambda N, K: N * K + 4 * N * (K // 256))
+        # algorithmic bytes per call: weights + scales, activations in, outputs (and the residual) -- what an ideal
+        # single pass would move; the kernels are MFMA-bound, the measured HBM traffic is reported beside it
+        algo = [wb(10240, H) + 2 * M * H + 2 * M * 10240, wb(H, H) + 2 * M * H + 4 * M * H,
+                2 * wb(I, H) + 2 * M * H + 2 * M * I, wb(H, I) + 2 * M * I + 4 * M * H]
         rows = []
-        for name, fn, fl, pl in ops:
+        for (name, fn, fl, pl), nb in zip(ops, algo):
             us, n = events_us(torch, fn, 1, use_graph=False)
             gemm = [p for p in pl if "quant_act" not in p[0] and "silu_mul" not in p[0]]
             rows.append({"kernel": gemm[-1][0] if gemm else "?", "launch": gemm[-1][1] if gemm else "", "call": name,
                          "kernels_per_call": len(pl), "avg_launch_us": round(us, 1), "flops_per_launch": fl,
-                         "achieved": round(fl / us / 1e6, 1), "frac": round(fl / us / 1e6 / peak, 4),
+                         "bytes_per_launch": nb, "achieved": round(fl / us / 1e6, 1), "frac": round(fl / us / 1e6 / peak, 4),
                          "launches_timed": n})
         dom = max(rows, key=lambda r: r["avg_launch_us"] if r["call"].startswith("down") else 0)
         cpu_b = cpu_baseline_prefill(H, pfmt) if (cpu and not args.no_cpu and not fp8) else None
@@ -717,7 +715,7 @@ def leg_cfg4(torch, _ops, args, pfmt="mxfp4", fp8=False, cpu=True):
                      "achieved": dom["achieved"], "peak": peak, "unit": unit, "frac": dom["frac"],
                      "traffic": measured_traffic(dom["kernel"], dom["call"]),
                      "avg_launch_us": dom["avg_launch_us"], "flops_per_launch": dom["flops_per_launch"],
-                     "launches_timed": dom["launches_timed"],
+                     "bytes_per_launch": dom["bytes_per_launch"], "launches_timed": dom["launches_timed"],
                      "timing": "events on the launch stream around eager launches of this op alone",
                      "all_gemm_kernels": rows},
         "cpu_baseline": cpu_b,
@@ -1016,6 +1014,14 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
     torch.cuda.set_device(torch.device("cuda:0"))
+
+    if args.pmc_calibrate:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.int32, device="cuda:0")  # 256 MiB read + 256 MiB written
+        for _ in range(3):
+            dst = src.clone()
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     if args.workload == "cfg1":
         return print(json.dumps(leg_as_line(leg_cfg1(torch, _ops, args), args)))
