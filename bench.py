@@ -904,7 +904,7 @@ def compact_rows(rows):
     for r in rows:
         row = [short_kernel(r["kernel"]), r["call"].split(" N=")[0].split(" (")[0], round(r["avg_launch_us"], 2),
                round(r["frac"], 3)]
-        if r["kernels_per_call"] > 1:  # a quantizer launch in front: kernels per call, whole-call us
+        if r["kernels_per_call"] > 1 and "call_us" in r:  # a quantizer launch in front: kernels per call, whole-call us
             row += [r["kernels_per_call"], round(r.get("call_us", r["avg_launch_us"]), 2)]
         out.append(row)
     return out
