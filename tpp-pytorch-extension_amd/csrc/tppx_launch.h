@@ -57,6 +57,11 @@ struct DecodeParams {
   // deal == 4: scale block of run u = spb_magic ? mulhi(u, spb_magic) : u   (spb_magic = ceil(2^32 / (tpb / 4)),
   // exact for u * (tpb / 4) < 2^32; 0 when a block is one run)
   unsigned int spb_magic;
+  // fused-quantisation kernel: (row, run) item i -> run i / M as mulhi(i, m_magic), m_magic = ceil(2^32 / M) (exact
+  // for i < 2^17, M <= 16); 0 when M == 1
+  unsigned int m_magic;
+  // 17..64-row kernel: scale block of tile t = tpb_magic ? mulhi(t, tpb_magic) : t   (ceil(2^32 / tpb); 0 when tpb == 1)
+  unsigned int tpb_magic;
   int S;     // K parts across workgroups (grid z, at most 4); > 1: partial sums go to `part`, the workgroup that
              // arrives last at its ticket adds them and runs the epilogue
   int ticket0; // first arrival counter of this launch (S > 1), see skinny_split_tickets()

@@ -54,6 +54,11 @@ __device__ __forceinline__ int sk_share(int a, int b, int c) {
   return (int)(((unsigned int)a * (unsigned int)b) / (unsigned int)c);
 }
 
+// the same for the K slices across workgroups: their number is 1, 2 or 4 (the launchers check), so a shift does
+__device__ __forceinline__ int sk_share_pow2(int a, int b, int c) {
+  return (int)(((unsigned int)a * (unsigned int)b) >> __builtin_ctz((unsigned int)c));
+}
+
 __device__ __forceinline__ int sk_find_seg(const DecodeParams& p, int grp) {
   int s = 0;
 #pragma unroll
@@ -369,7 +374,7 @@ skinny_qint8_kernel(const DecodeParams p) {
   extern __shared__ __align__(16) float sk_lds[];
   constexpr int MPAD = MG * 16;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int W = blockDim.x >> 6;
+  const int W = MAXW == MINW ? MAXW : (int)(blockDim.x >> 6); // (a constant where it can be: divisions become shifts)
   const int grp = blockIdx.x;
   const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
   const int ltile0 = (grp - sg.grp0) * NTW;
@@ -380,12 +385,12 @@ skinny_qint8_kernel(const DecodeParams p) {
   const bool FAST = G == 4;
   constexpr int UN = (PF % 4 == 0) ? PF : (PF % 2 == 0 ? 2 * PF : 4 * PF); // lcm(PF, 4) tiles per unrolled trip
   // runs of this workgroup (all of them unless K is split across workgroups), then of this wave
-  const int ub = sk_share(blockIdx.z, p.units, p.S), ue = sk_share(blockIdx.z + 1, p.units, p.S);
+  const int ub = sk_share_pow2(blockIdx.z, p.units, p.S), ue = sk_share_pow2(blockIdx.z + 1, p.units, p.S);
   const int u0 = ub + sk_share(wave, ue - ub, W), u1 = ub + sk_share(wave + 1, ue - ub, W);
   const int t0 = u0 * G, t1 = u1 * G;
-  const unsigned int magic = p.spb_magic;
-  auto blk_of = [&](int t, bool fast) { // scale block of tile t (uniform)
-    return fast ? (magic ? (int)__umulhi((unsigned int)(t >> 2), magic) : (t >> 2)) : t / TPB;
+  const unsigned int magic = p.tpb_magic;
+  auto blk_of = [&](int t, bool) { // scale block of tile t (uniform): t / TPB without the division
+    return magic ? (int)__umulhi((unsigned int)t, magic) : t;
   };
   const int b0 = blk_of(max(min(t0, KT - 1), 0), FAST); // first scale block of this wave
 
@@ -408,13 +413,6 @@ skinny_qint8_kernel(const DecodeParams p) {
     xrow[mg] = reinterpret_cast<const int8_t*>(p.xq) + (int64_t)m * p.K + (lane >> 4) * 16;
   }
 
-  // Loads return in issue order: the small L2-resident ones (activation
-  // scales, post-op inputs) go out BEFORE the weight ring so that waiting for
-  // them does not wait for HBM.
-  SkEpilogue<MG, NTW, false, MINW> ep;
-  ep.prefetch_flat(p, sg, ltile0, m0);
-  __builtin_amdgcn_sched_barrier(0); // keep the issue order of independent loads (see skinny_qint8_fq_kernel)
-  // activation scales of this wave's K blocks, transposed in LDS: [u - u0][MPAD]
   float* red = sk_lds;
   float* sa_s = sk_lds + (size_t)W * NTW * MG * 256 + (size_t)wave * p.cht * MPAD;
   const int nsa = t0 < t1 ? (blk_of(t1 - 1, FAST) - b0 + 1) * MPAD : 0;
@@ -426,13 +424,6 @@ skinny_qint8_kernel(const DecodeParams p) {
     // XOP: scales transposed by the quantisation kernel, [K/qbs][mt*16]
     return XOP ? p.sa[(int64_t)(b0 + ul) * mtp + m0 + mr] : p.sa[(int64_t)min(m0 + mr, p.M - 1) * NB + b0 + ul];
   };
-  // (no branch around these first requests or the ring's: behind a conditional load the compiler can no longer count
-  // the loads in flight and waits for all of them; a wave without K blocks re-reads valid data it never uses)
-  float sa0[SAB];
-#pragma unroll
-  for (int j = 0; j < SAB; j++)
-    sa0[j] = load_sa(j * 64 + lane);
-  __builtin_amdgcn_sched_barrier(0);
 
   // Ring of PF stages; a stage = the weight tiles, their block scale and the
   // activation operand of one k-tile.  The main loop has NO branch and NO load
@@ -453,9 +444,27 @@ skinny_qint8_kernel(const DecodeParams p) {
     for (int mg = 0; mg < MG; mg++)
       xreg[st][mg] = XOP ? xop[(int64_t)t * xstride + mg * 64] : *reinterpret_cast<const i32x4*>(xrow[mg] + t * 64);
   };
+  // The ring's first requests are the kernel's first vector loads: the set-up of the epilogue (offsets and post-op
+  // inputs of up to six outputs per thread) is several hundred instructions, which two waves per SIMD take 2 us to
+  // get through.  (Timestamps: with the ring in front, a wave's first request goes out 0.8 instead of 2.1 us after
+  // the first wave's start -- and its first tile still arrives about 4 us after the start: the memory system's own
+  // start-up, not the request time, sets the beginning of the stream, so the kernel's time did not change.)  Loads
+  // return in issue order, so the activation scales (L2) wait for the first stages; they are needed after four tiles.
+  // (no branch around these first requests: behind a conditional load the compiler can no longer count the loads
+  // in flight and waits for all of them; a wave without K blocks re-reads valid data it never uses)
 #pragma unroll
   for (int i = 0; i < PF; i++)
     load_stage(i, t0 + i, false);
+  __builtin_amdgcn_sched_barrier(0); // keep the issue order of independent loads (see skinny_qint8_fq_kernel)
+  // activation scales of this wave's K blocks, transposed in LDS: [u - u0][MPAD]
+  float sa0[SAB];
+#pragma unroll
+  for (int j = 0; j < SAB; j++)
+    sa0[j] = load_sa(j * 64 + lane);
+  __builtin_amdgcn_sched_barrier(0);
+  SkEpilogue<MG, NTW, false, MINW> ep;
+  ep.prefetch_flat(p, sg, ltile0, m0);
+  __builtin_amdgcn_sched_barrier(0);
   if (t0 < t1) {
     // the scales were requested first, so they are here long before the ring
 #pragma unroll
@@ -691,7 +700,7 @@ skinny_qint8_nk_kernel(const DecodeParams p) {
   const unsigned int magic = p.spb_magic;
   auto blk_of_run = [&](int u) { return magic ? (int)__umulhi((unsigned int)u, magic) : u; };
   // runs of this workgroup's K slice, then of this wave's K part; every wave makes the same number of steps
-  const int ub = sk_share(z, NR, S), ue = sk_share(z + 1, NR, S);
+  const int ub = sk_share_pow2(z, NR, S), ue = sk_share_pow2(z + 1, NR, S);
   const int u0 = ub + (kp * (ue - ub)) / KPW, u1 = ub + ((kp + 1) * (ue - ub)) / KPW;
   const int nsteps = (ue - ub + KPW - 1) / KPW; // <= MAXSTEPS (the launcher checks)
 
@@ -990,7 +999,7 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
   static_assert(WBITS == 8 || !BIGB, "the packed formats run 256-wide blocks");
   extern __shared__ __align__(16) float sk_lds[];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int W = blockDim.x >> 6;
+  const int W = MAXW == MINW ? MAXW : (int)(blockDim.x >> 6);
   const int grp = blockIdx.x;
   const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
   const int ltile0 = (grp - sg.grp0) * NTW;
@@ -1017,12 +1026,13 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
   // row.  Items are numbered row-fastest; XB passes are in flight at a time.
   const uint16_t* xb = reinterpret_cast<const uint16_t*>(p.x);
   const int nitems = M * (u1 - u0);
-  const uint32_t Mu = (uint32_t)M;
+  const uint32_t Mu = (uint32_t)M, mmagic = p.m_magic;
+  auto run_of_item = [&](uint32_t it) { return mmagic ? __umulhi(it, mmagic) : it; }; // it / M without the division
   i32x4 raw[XB][2]; // first-class vectors: copies of the HIP struct type would keep the array in scratch
   auto load_pass = [&](auto PS, int base) {
     constexpr int ps = decltype(PS)::value;
     const uint32_t it = (uint32_t)min((base + ps) * 4 + (lane >> 4), max(nitems - 1, 0));
-    const uint32_t ul = it / Mu, mr = it - ul * Mu;
+    const uint32_t ul = run_of_item(it), mr = it - ul * Mu;
     const i32x4* src = reinterpret_cast<const i32x4*>(xb + (int64_t)mr * p.K + (int64_t)(u0 + (int)ul) * 256 + (lane & 15) * 16);
     raw[ps][0] = src[0];
     raw[ps][1] = src[1];
@@ -1083,7 +1093,7 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
       if (ps * 4 < nitems) { // wave-uniform
         const int it = ps * 4 + (lane >> 4);
         const uint32_t itc = (uint32_t)min(it, nitems - 1);
-        const uint32_t ul = itc / Mu, mr = itc - ul * Mu;
+        const uint32_t ul = run_of_item(itc), mr = itc - ul * Mu;
         const float am = item_amax(PS);
         if (it < nitems && (lane & 15) == 0)
           amax_s[mr * NR + u0 + ul] = am;
@@ -1101,7 +1111,7 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
     if ((base + ps) * 4 < nitems) { // wave-uniform
       const int it = (base + ps) * 4 + (lane >> 4);
       const uint32_t itc = (uint32_t)min(it, nitems - 1);
-      const uint32_t ul = itc / Mu, mr = itc - ul * Mu;
+      const uint32_t ul = run_of_item(itc), mr = itc - ul * Mu;
       float v[16];
 #pragma unroll
       for (int j = 0; j < 8; j++) {
@@ -2058,7 +2068,9 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
   dim3 grid(p.groups, pl.grid_y, pl.fused_quant ? 1 : p.S);
   if (grid.z > 1 && (p.S > 4 || (p.ticket0 = skinny_split_tickets((int)(grid.x * grid.y))) < 0))
     return hipErrorInvalidValue;
+  p.tpb_magic = p.tpb > 1 ? (unsigned int)(((1ull << 32) + (unsigned int)p.tpb - 1) / (unsigned int)p.tpb) : 0u;
   if (pl.fused_quant) {
+    p.m_magic = p.M > 1 ? (unsigned int)(((1ull << 32) + (unsigned int)p.M - 1) / (unsigned int)p.M) : 0u;
     const bool bigb = p.tpb > 4;
     const size_t abytes = bigb ? (size_t)p.M * p.units * sizeof(float) : 0;
     const size_t xbytes = (size_t)16 * pl.max_units * (256 * (size_t)p.M + 64) + abytes, rbytes = (size_t)16 * pl.ntw * 1024;
