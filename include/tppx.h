@@ -280,16 +280,19 @@ int tppx_linear_qint8(const void* x, void* xq, void* sa, const void* qw,
  * they lie (TppBlockedQInt8LinearW on kQUInt4x2 / kQUInt2x4 weights, src/csrc/fused_gemm.h:1110-1126; BRGEMM with
  * b_vnni, src/csrc/xsmm_functors.h:2640-2666).  tppx_pack_qint_tiles turns the native int8 tiles of such a weight
  * (tppx_prepack_qint4 / tppx_prepack_qint2) into 4- or 2-bit codes in the kernel's order, N*K*bits/8 bytes;
- * tppx_linear_qintx is tppx_linear_qint8 on them for M <= 16 rows and 256-wide scale blocks: bf16 activations
- * quantized inside the launch, the codes expanded in registers in front of the int8 MFMA -- the same integer sums,
- * scales and rounding as the expanded weight, so the same bits.  sw: the f32 scales tppx_linear_qint8 takes.
- * TPPX_EUNSUPPORTED when the rows do not fit the in-kernel quantisation (run the expanded tiles then). */
+ * tppx_linear_qintx is tppx_linear_qint8 on them for decode shapes and 256-wide scale blocks, the codes expanded
+ * in registers in front of the int8 MFMA -- the same integer sums, scales and rounding as the expanded weight, so
+ * the same bits.  Up to 16 rows the bf16 activations are quantized inside the launch (xq, sa may be NULL); more rows
+ * run block rows of 32 / 64 behind the activation quantizer and need the xq / sa scratch of tppx_linear_qint8
+ * (flags: 0 or TPPX_FLAG_XQ_REUSE).  sw: the f32 scales tppx_linear_qint8 takes.  TPPX_EUNSUPPORTED when at most
+ * 16 rows do not fit the in-kernel quantisation (run the expanded tiles then). */
 int tppx_pack_qint_tiles(const void* native_i8, int64_t N, int64_t K, int bits,
                          void* packed, tppx_stream_t stream);
-int tppx_linear_qintx(const void* x, const void* qw_packed, const void* sw,
-                      const void* bias, const void* post_in, const void* post_in2,
-                      void* y, int64_t M, int64_t N, int64_t K, int bits,
-                      int post_op, float post_scale, tppx_stream_t stream);
+int tppx_linear_qintx(const void* x, void* xq, void* sa, const void* qw_packed,
+                      const void* sw, const void* bias, const void* post_in,
+                      const void* post_in2, void* y, int64_t M, int64_t N,
+                      int64_t K, int bits, int post_op, float post_scale,
+                      int flags, tppx_stream_t stream);
 
 /* No counterpart in the reference.  tppx_linear_qint8 for callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the quantised activations, their

@@ -326,12 +326,15 @@ def test_w4a8_linear(M, post):
 
 @pytest.mark.parametrize("kind", ["qint4", "qint2"])
 @pytest.mark.parametrize("M,N,K,post", [(1, 11008, 4096, "none"), (8, 4096, 11008, "add"), (16, 4096, 4096, "silu"),
-                                        (5, 96, 1024, "mul"), (3, 8448, 14336, "add")])
+                                        (5, 96, 1024, "mul"), (3, 8448, 14336, "add"),
+                                        (32, 11008, 4096, "add"), (64, 4096, 11008, "add"), (40, 96, 1024, "mul"),
+                                        (17, 544, 2048, "silu"), (64, 8448, 1536, "none"), (33, 4064, 2816, "add")])
 def test_packed_code_decode_kernel_equals_expanded_weight(kind, M, N, K, post, monkeypatch):
     """QINT4 / ternary QINT2 weights at their own width (src/csrc/fused_gemm.h:1110-1126 multiplies the packed codes as
-    they lie): up to 16 rows the decode kernel streams N*K/2 or N*K/4 bytes of codes and expands them in registers in
-    front of the int8 MFMA.  Same integer sums, scales and rounding as the expanded int8 tiles, so the SAME BITS as
-    that path (TPPX_PACKED_CODES=0), and within 1 ulp (2 through SiLU) of the oracle on the expanded weight."""
+    they lie): up to 64 rows the decode kernels stream N*K/2 or N*K/4 bytes of codes and expand them in registers in
+    front of the int8 MFMA.  Same integer sums, scales and rounding as the expanded int8 tiles: within 1 ulp (2 through
+    SiLU) of the oracle on the expanded weight, and the SAME BITS as the int8-tile kernel that sums K in the same order
+    (TPPX_PACKED_CODES=0; above 16 rows that is the eight-wave kernel without a K split across workgroups)."""
     ops = _ops()
     from tpp_pytorch_extension import _lib
     posts = {"none": O.POST_NONE, "add": O.POST_ADD_SCALE, "silu": O.POST_SILU, "mul": O.POST_MUL}
@@ -348,11 +351,30 @@ def test_packed_code_decode_kernel_equals_expanded_weight(kind, M, N, K, post, m
     y = ops.linear(x, qt, b, posts[post], r, None, 0.5)
     packed, sn, bits = qt.native_packed()
     assert packed.numel() == N * K * bits // 8
+    # the packed path really ran: the entry point accepts the call (no fall-through) and gives the op's bits
+    y2 = torch.empty_like(y)
+    xq, sa = ops._qint8_scratch(x, M, K, 256)
+    _lib.check(_lib.lib().tppx_linear_qintx(x.data_ptr(), xq.data_ptr(), sa.data_ptr(), packed.data_ptr(), sn.data_ptr(),
+                                            b.data_ptr(), r.data_ptr(), None, y2.data_ptr(), M, N, K, bits, posts[post], 0.5,
+                                            0, _lib.stream_of(x)))
+    assert torch.equal(y2, y)
+    if M > 16:  # the quantised rows are still in xq / sa: the GEMM alone
+        y3 = torch.empty_like(y)
+        _lib.check(_lib.lib().tppx_linear_qintx(x.data_ptr(), xq.data_ptr(), sa.data_ptr(), packed.data_ptr(), sn.data_ptr(),
+                                                b.data_ptr(), r.data_ptr(), None, y3.data_ptr(), M, N, K, bits, posts[post],
+                                                0.5, _lib.FLAG_XQ_REUSE, _lib.stream_of(x)))
+        assert torch.equal(y3, y)
+    # against the default path on the expanded int8 tiles (itself tested against the oracle above): another fp32
+    # summation order above 16 rows, so one ulp apart at most
     monkeypatch.setattr(ops, "PACKED_CODES", False)
+    y_default = ops.linear(x, qt, b, posts[post], r, None, 0.5)
+    assert_close_bf16(t2bits(y), t2bits(y_default), ulps=2 if post == "silu" else 1, what=f"{kind} packed vs expanded tiles M={M}")
+    # eight waves, no K split across workgroups: the packed kernels' summation order
+    monkeypatch.setenv("TPPX_QINT8_NK", "0")
+    monkeypatch.setenv("TPPX_SKINNY_SPLITK", "0")
+    if M > 16:
+        monkeypatch.setenv("TPPX_SKINNY_WAVES", "8")
+    _lib.lib().tppx_reload_env()
     y_expanded = ops.linear(x, qt, b, posts[post], r, None, 0.5)
     assert torch.equal(y, y_expanded), "packed codes and expanded int8 tiles give different bits"
-    # the packed path really ran: the entry point accepts the call (no fall-through)
-    y2 = torch.empty_like(y)
-    _lib.check(_lib.lib().tppx_linear_qintx(x.data_ptr(), packed.data_ptr(), sn.data_ptr(), b.data_ptr(), r.data_ptr(), None,
-                                            y2.data_ptr(), M, N, K, bits, posts[post], 0.5, _lib.stream_of(x)))
-    assert torch.equal(y2, y)
+

@@ -803,15 +803,16 @@ extern "C" int tppx_linear_qint8_noalloc(const void* x, const void* qw, const vo
                    (int64_t)NA_WS_BYTES, (hipStream_t)stream);
 }
 
-extern "C" int tppx_linear_qintx(const void* x, const void* qw_packed, const void* sw, const void* bias,
-                                 const void* post_in, const void* post_in2, void* y, int64_t M, int64_t N, int64_t K,
-                                 int bits, int post_op, float post_scale, tppx_stream_t stream) {
+extern "C" int tppx_linear_qintx(const void* x, void* xq, void* sa, const void* qw_packed, const void* sw,
+                                 const void* bias, const void* post_in, const void* post_in2, void* y, int64_t M,
+                                 int64_t N, int64_t K, int bits, int post_op, float post_scale, int flags,
+                                 tppx_stream_t stream) {
   const char* who = "tppx_linear_qintx";
   int rc = check_common(who, x, M, K, 1, 0, nullptr, 0);
   if (rc)
     return rc;
   TPPX_REQUIRE(bits == 4 || bits == 2, TPPX_EINVAL, "%s: %d-bit codes are not built (4 or 2)", who, bits);
-  TPPX_REQUIRE(M <= 16, TPPX_EUNSUPPORTED, "%s: the packed-code kernel takes at most 16 rows (M=%ld); larger calls run on the expanded int8 tiles", who, (long)M);
+  TPPX_REQUIRE((flags & ~TPPX_FLAG_XQ_REUSE) == 0, TPPX_EINVAL, "%s: flags 0x%x not taken here (TPPX_FLAG_XQ_REUSE only)", who, flags);
   TPPX_REQUIRE(K > 0 && K % 256 == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of the 256-wide scale block", who, (long)K);
   tppx_seg s = {qw_packed, sw, bias, post_in, post_in2, y, N, post_op, post_scale};
   DecodeParams p;
@@ -830,9 +831,29 @@ extern "C" int tppx_linear_qintx(const void* x, const void* qw_packed, const voi
   p.S = 1;
   p.wbits = bits;
   SkinnyPlan sp = plan_skinny(M, p.total_tiles, p.units, p.tpb, p.deal, true);
-  TPPX_REQUIRE(sp.fused_quant, TPPX_EUNSUPPORTED, "%s: M=%ld rows of K=%ld channels do not fit the in-kernel quantisation's LDS; run the call on the expanded int8 tiles", who, (long)M, (long)K);
-  set_groups(p, sp.ntw, false);
-  return check_hip(launch_skinny_qint8(p, sp, (hipStream_t)stream), who);
+  if (sp.fused_quant) { // up to 16 rows whose quantised form fits the LDS: one launch
+    set_groups(p, sp.ntw, false);
+    return check_hip(launch_skinny_qint8(p, sp, (hipStream_t)stream), who);
+  }
+  // more rows: the activation quantiser in front (operand-order int8 rows), then the 17..64-row kernel on block
+  // rows of 32 or 64
+  TPPX_REQUIRE(M > 16, TPPX_EUNSUPPORTED, "%s: M=%ld rows of K=%ld channels do not fit the in-kernel quantisation's LDS; run the call on the expanded int8 tiles", who, (long)M, (long)K);
+  TPPX_REQUIRE(xq && sa, TPPX_EINVAL, "%s: more than 16 rows need the xq / sa scratch of tppx_linear_qint8", who);
+  TPPX_REQUIRE(aligned16(xq) && aligned16(sa), TPPX_EINVAL, "%s: scratch not 16-byte aligned", who);
+  int ntw = 1;
+  for (; ntw < 3; ntw++)
+    if ((p.total_tiles + ntw - 1) / ntw <= 256)
+      break;
+  set_groups(p, ntw, false);
+  p.xq = xq;
+  p.sa = (const float*)sa;
+  p.mt = sp.grid_y * sp.mg;
+  if (!(flags & TPPX_FLAG_XQ_REUSE)) {
+    rc = check_hip(launch_quant_act_int8(x, M, K, 256, xq, sa, p.mt, (hipStream_t)stream), who);
+    if (rc)
+      return rc;
+  }
+  return check_hip(launch_skinny_qintx(p, sp.mg, ntw, (hipStream_t)stream), who);
 }
 
 extern "C" void tppx_reload_env(void) {

@@ -1258,6 +1258,156 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
 }
 
 // ---------------------------------------------------------------------------
+// QINT4 / ternary QINT2 weights at their own width, 17..64 rows per block row (256-wide scale blocks): the
+// activations arrive quantised in operand order (quant_act_int8_rows_kernel, as for skinny_qint8_kernel), a ring
+// stage of activations is one K tile, a ring stage of weights one 16-byte load per lane and channel tile that
+// holds G = 8 / WBITS consecutive K tiles (tppx_pack_qint_tiles), expanded in registers in front of the MFMA as in
+// skinny_qint8_fq_kernel.  Eight waves split K in runs of 256 channels; same int32 sums, scales and fp32
+// operations as skinny_qint8_kernel on the expanded tiles, so the same bits.
+// ---------------------------------------------------------------------------
+template <int MG, int NTW, int PF, int WBITS>
+__global__ void __launch_bounds__(512)
+skinny_qintx_kernel(const DecodeParams p) {
+  extern __shared__ __align__(16) float sk_lds[];
+  constexpr int G = 8 / WBITS, WS = 2, W = 8, MPAD = MG * 16;
+  constexpr int UN = G * WS; // tiles per unrolled trip: 4 or 8 (a multiple of PF and of a 4-tile run)
+  static_assert(UN % PF == 0 && UN % 4 == 0, "ring slots are static inside a trip");
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int grp = blockIdx.x;
+  const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
+  const int ltile0 = (grp - sg.grp0) * NTW;
+  const int m0 = blockIdx.y * MPAD;
+  const int NR = p.units, KT = NR * 4; // 256-wide runs (= scale blocks), K tiles
+  const int u0 = (wave * NR) / W, u1 = ((wave + 1) * NR) / W;
+  const int t0 = u0 * 4, t1 = u1 * 4;
+
+  const i32x4* wq[NTW];
+  const float* ws[NTW];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++) {
+    const int64_t lt = min(ltile0 + nt, sg.tiles - 1); // ragged last group: duplicate, not stored
+    wq[nt] = reinterpret_cast<const i32x4*>(sg.qw) + lt * (KT / G) * 64 + lane;
+    ws[nt] = reinterpret_cast<const float*>(sg.sw) + lt * NR * 16 + (lane & 15);
+  }
+  const i32x4* xop = reinterpret_cast<const i32x4*>(p.xq) + (int64_t)blockIdx.y * MG * 64 + lane;
+  const int xstride = p.mt * 64, mtp = p.mt * 16;
+
+  i32x4 wreg[WS][NTW], xreg[PF][MG];
+  float sreg[WS][NTW];
+  // (past the end, or a wave without runs: re-read valid data that is never consumed -- no branch around a load)
+  auto load_w = [&](int st, int gi) {
+    gi = max(min(gi, t1 / G - 1), 0);
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++) {
+      wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)gi * 64);
+      sreg[st][nt] = ws[nt][((gi * G) >> 2) * 16];
+    }
+  };
+  auto load_x = [&](int st, int t) {
+    t = max(min(t, t1 - 1), 0);
+#pragma unroll
+    for (int mg = 0; mg < MG; mg++)
+      xreg[st][mg] = xop[(int64_t)t * xstride + mg * 64];
+  };
+#pragma unroll
+  for (int i = 0; i < WS; i++)
+    load_w(i, t0 / G + i);
+#pragma unroll
+  for (int i = 0; i < PF; i++)
+    load_x(i, t0 + i);
+  __builtin_amdgcn_sched_barrier(0);
+  // activation scales of this wave's runs, transposed in LDS: [u - u0][MPAD]
+  float* red = sk_lds;
+  float* sa_s = sk_lds + (size_t)W * NTW * MG * 256 + (size_t)wave * p.cht * MPAD;
+  const int nsa = (u1 - u0) * MPAD;
+  constexpr int SAB = 2 * MG;
+  auto load_sa = [&](int i) {
+    i = max(min(i, nsa - 1), 0);
+    const int ul = i / MPAD, mr = i - ul * MPAD;
+    return p.sa[(int64_t)(u0 + ul) * mtp + m0 + mr]; // [K / 256][mt * 16], written by the quantisation kernel
+  };
+  float sa0[SAB];
+#pragma unroll
+  for (int j = 0; j < SAB; j++)
+    sa0[j] = load_sa(j * 64 + lane);
+  __builtin_amdgcn_sched_barrier(0);
+  SkEpilogue<MG, NTW, false, 8> ep;
+  ep.prefetch_flat(p, sg, ltile0, m0);
+  __builtin_amdgcn_sched_barrier(0);
+  if (t0 < t1) {
+#pragma unroll
+    for (int j = 0; j < SAB; j++)
+      if (j * 64 + lane < nsa)
+        sa_s[j * 64 + lane] = sa0[j];
+    for (int i0 = SAB * 64; i0 < nsa; i0 += SAB * 64) { // more than 8 runs per wave
+      float v[SAB];
+#pragma unroll
+      for (int j = 0; j < SAB; j++)
+        v[j] = load_sa(i0 + j * 64 + lane);
+#pragma unroll
+      for (int j = 0; j < SAB; j++)
+        if (i0 + j * 64 + lane < nsa)
+          sa_s[i0 + j * 64 + lane] = v[j];
+    }
+  }
+
+  f32x4 facc[NTW][MG];
+  i32x4 iacc[NTW][MG];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++)
+#pragma unroll
+    for (int mg = 0; mg < MG; mg++) {
+      facc[nt][mg] = f32x4{0.f, 0.f, 0.f, 0.f};
+      iacc[nt][mg] = i32x4{0, 0, 0, 0};
+    }
+  // tile tt: activations in stage xs, weights = part g of stage wst; a run closes every fourth tile
+  auto consume = [&](int xs, int wst, int g, int tt) {
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++) {
+      const i32x4 wop = sk_expand_codes<WBITS>(wreg[wst][nt], g);
+#pragma unroll
+      for (int mg = 0; mg < MG; mg++)
+        iacc[nt][mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xreg[xs][mg], wop, iacc[nt][mg], 0, 0, 0);
+    }
+    if ((tt & 3) == 3) {
+#pragma unroll
+      for (int mg = 0; mg < MG; mg++) {
+        const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + ((tt >> 2) - u0) * MPAD + mg * 16 + (lane >> 4) * 4);
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++) {
+          const float swv = sreg[wst][nt] * (WBITS == 4 ? 0.0625f : 0.015625f); // operands are 16 x / 64 x the value
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            facc[nt][mg][r] = fmaf((float)iacc[nt][mg][r], sav[r] * swv, facc[nt][mg][r]);
+            iacc[nt][mg][r] = 0;
+          }
+        }
+      }
+    }
+  };
+  int t = t0;
+  for (; t + UN <= t1; t += UN) { // branch-free full trips (reloads past the end are clamped re-reads)
+#pragma unroll
+    for (int i = 0; i < UN; i++) {
+      consume(i % PF, (i / G) % WS, i % G, t + i);
+      load_x(i % PF, t + i + PF);
+      if (i % G == G - 1)
+        load_w((i / G) % WS, (t + i) / G + WS);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  if (t < t1) { // one run left (UN == 8): its tiles are in the stages a trip would use
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      consume(i % PF, (i / G) % WS, i % G, t + i);
+      if (i + PF < 4)
+        load_x(i % PF, t + i + PF);
+    }
+  }
+  ep.finish(sg, facc, red);
+}
+
+// ---------------------------------------------------------------------------
 // MXFP4, M <= 16, activations staged in LDS by the wave that consumes them,
 // with an optional transform on the way in:
 //   XMODE 0  x as it is
@@ -2121,7 +2271,7 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
   if (pl.ntw == 3) {
     if (pl.mg == 2)
       SKQ(2, 3, 4, 8, 8);
-    SKQ(4, 3, 2, 8, 8);
+    SKQ(4, 3, 2, 8, 8); // (225 registers; a ring of three or four stages spills 620 / 164 bytes per lane)
   }
   if (pl.ntw == 2) {
     switch (pl.mg) {
@@ -2177,6 +2327,24 @@ hipError_t launch_skinny_qint8_nk(DecodeParams& p, int mg, hipStream_t stream) {
     (void)hipGetLastError();
   }
   return e;
+}
+
+// QINT4 / QINT2 codes at their own width, 17..64 rows per block row (p.wbits, p.mt set; 256-wide blocks, one K part)
+hipError_t launch_skinny_qintx(DecodeParams& p, int mg, int ntw, hipStream_t stream) {
+  if ((p.wbits != 4 && p.wbits != 2) || p.S != 1 || p.mt <= 0 || p.deal != 4 || p.tpb != 4 || (mg != 2 && mg != 4) ||
+      ntw < 1 || ntw > 3)
+    return hipErrorInvalidValue;
+  p.cht = (p.units + 7) / 8; // runs of a wave: slots of activation scales in LDS
+  dim3 grid(p.groups, (p.M + mg * 16 - 1) / (mg * 16), 1);
+  const size_t lds = ((size_t)8 * ntw * mg * 256 + (size_t)8 * p.cht * mg * 16) * sizeof(float);
+  // activations two tiles ahead at four row groups, four at two (the register budget of eight waves per workgroup)
+#define SKQR(MG, NTW)                                                                                            \
+  if (mg == MG && ntw == NTW)                                                                                    \
+    return p.wbits == 4 ? sk_launch(skinny_qintx_kernel<MG, NTW, (MG == 4 ? 2 : 4), 4>, p, grid, 8, lds, stream) \
+                        : sk_launch(skinny_qintx_kernel<MG, NTW, (MG == 4 ? 2 : 4), 2>, p, grid, 8, lds, stream);
+  SKQR(2, 1) SKQR(2, 2) SKQR(2, 3) SKQR(4, 1) SKQR(4, 2) SKQR(4, 3)
+#undef SKQR
+  return hipErrorInvalidValue;
 }
 
 // MXFP4, 33..64 rows per block row: four channel tiles x four K parts per workgroup, K in p.S slices across workgroups

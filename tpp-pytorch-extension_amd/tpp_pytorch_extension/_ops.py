@@ -686,13 +686,15 @@ def linear(input, weight, bias=None, post=POST_NONE, post_in=None, post_in2=None
     bias = _prep_bias(bias, N, x.device)
     post_in = _prep_post(post_in, M, N, "post-op input", x.device)
     post_in2 = _prep_post(post_in2, M, N, "second post-op input", x.device)
-    # QINT4 / QINT2 decode steps: the codes streamed at their own width and expanded in registers (same bits as the
-    # expanded int8 tiles).  TPPX_PACKED_CODES=0 keeps the expanded tiles.
-    if PACKED_CODES and M <= 16 and weight.weight_kind() in ("qint4", "qint2") and weight.block_size == 256 \
-            and row_sumsq is None and not flags:
+    # QINT4 / QINT2 decode steps (up to 64 rows): the codes streamed at their own width and expanded in registers
+    # (same bits as the expanded int8 tiles).  TPPX_PACKED_CODES=0 keeps the expanded tiles.
+    if PACKED_CODES and M <= 64 and weight.weight_kind() in ("qint4", "qint2") and weight.block_size == 256 \
+            and row_sumsq is None and not (flags & ~_lib.FLAG_XQ_REUSE):
         qp, sp, bits = weight.native_packed()
-        rc = L.tppx_linear_qintx(x.data_ptr(), qp.data_ptr(), sp.data_ptr(), _lib.ptr(bias), _lib.ptr(post_in),
-                                 _lib.ptr(post_in2), y.data_ptr(), M, N, K, bits, post, post_scale, _lib.stream_of(x))
+        xq, sa = _qint8_scratch(x, M, K, 256) if M > 16 else (None, None)
+        rc = L.tppx_linear_qintx(x.data_ptr(), _lib.ptr(xq), _lib.ptr(sa), qp.data_ptr(), sp.data_ptr(), _lib.ptr(bias),
+                                 _lib.ptr(post_in), _lib.ptr(post_in2), y.data_ptr(), M, N, K, bits, post, post_scale,
+                                 flags, _lib.stream_of(x))
         if rc != _lib.EUNSUPPORTED:  # rows that do not fit the in-kernel quantisation fall through to the int8 tiles
             _lib.check(rc)
             return y
