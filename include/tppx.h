@@ -276,6 +276,25 @@ int tppx_linear_qint8(const void* x, void* xq, void* sa, const void* qw,
                       int flags, void* ws, int64_t ws_bytes,
                       tppx_stream_t stream);
 
+/* W4A8 decode calls (M <= 16) in one launch.  tppx_prepack_mxfp4_int8 turns the USE_MXFP4_INT8 weight
+ * (src/csrc/qtypes.cpp:787-790, 840-861: q u8 [N/8][K/bc][bc/8][8][4], scales u8 [N/8][K/bc][bc/32][8]) into
+ * tiles in MFMA operand order (q_nat N*K/2 bytes, s_nat N*K/32 bytes; N % 16 == 0, K % 128 == 0), once per weight;
+ * tppx_linear_mxfp4_int8_rows is TppBlockedLinearW<int8_t, uint8_t, Tout> (src/csrc/fused_gemm.h:965-978) on them
+ * for bf16 activations x [M][K]: the rows are quantized to int8 over blocks of 32 inside the launch
+ * (quantize_int8sym, scales times 6/127), K is split over the waves of a workgroup.  Same arithmetic as
+ * tppx_linear_mxfp4_int8 (exact int32 block sums, one fp32 multiply-add per block) in another summation order.
+ * TPPX_EUNSUPPORTED for more than 16 rows or rows that do not fit the LDS: quantize the activations and call
+ * tppx_linear_mxfp4_int8 then. */
+int tppx_prepack_mxfp4_int8(const void* q_ref, const void* sc_ref, int64_t N,
+                            int64_t K, int64_t bc, void* q_nat, void* s_nat,
+                            tppx_stream_t stream);
+int tppx_linear_mxfp4_int8_rows(const void* x, const void* q_nat,
+                                const void* s_nat, const void* bias,
+                                const void* post_in, const void* post_in2,
+                                void* y, int64_t M, int64_t N, int64_t K,
+                                int post_op, float post_scale,
+                                tppx_stream_t stream);
+
 /* QINT4 / ternary QINT2 weights at their own width for decode shapes.  The reference multiplies the packed codes as
  * they lie (TppBlockedQInt8LinearW on kQUInt4x2 / kQUInt2x4 weights, src/csrc/fused_gemm.h:1110-1126; BRGEMM with
  * b_vnni, src/csrc/xsmm_functors.h:2640-2666).  tppx_pack_qint_tiles turns the native int8 tiles of such a weight

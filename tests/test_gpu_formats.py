@@ -324,6 +324,47 @@ def test_w4a8_linear(M, post):
         assert torch.equal(sw, ops.fc_mul(x.cuda(), qt, None, ops.fc_silu(x.cuda(), qt, None)))
 
 
+@pytest.mark.parametrize("M,N,K,bc,post", [(1, 4096, 4096, 64, "none"), (8, 11008, 4096, 64, "add"), (16, 512, 2048, 128, "silu"),
+                                           (5, 96, 1280, 32, "mul"), (8, 4096, 11008, 64, "add"), (3, 8448, 1536, 64, "none"),
+                                           (16, 4096, 11008, 64, "add")])
+def test_w4a8_decode_kernel(M, N, K, bc, post, monkeypatch):
+    """W4A8 decode calls (TppBlockedLinearW<int8_t, uint8_t, Tout>, src/csrc/fused_gemm.h:965-978, at most 16 rows) in
+    one launch: rows quantized to int8 over blocks of 32 inside the kernel, K split over the waves of a workgroup,
+    weights from tiles made once by tppx_prepack_mxfp4_int8.  Within 1 bf16 ulp (2 through SiLU) of the oracle's
+    restatement and of the two-step path (the same integer sums and per-block fp32 multiply-adds in another order);
+    16 rows x 11008 do not fit the kernel's LDS and take the two-step path by themselves."""
+    ops = _ops()
+    from tpp_pytorch_extension import _lib
+    posts = {"none": O.POST_NONE, "add": O.POST_ADD_SCALE, "silu": O.POST_SILU, "mul": O.POST_MUL}
+    W = randn_bf16((N, K), 0.05, 2700 + M)
+    t = W.view(N // 16, 16, K // bc, bc // 2, 2).permute(0, 2, 3, 1, 4).contiguous()
+    qt = ops.remap_and_quantize_mxfp4(t.cuda(), int8_layout=True)
+    q_or, s_or = O.remap_quantize_mxfp4_int8(t.float().numpy())
+    assert np.array_equal(qt.qdata.cpu().numpy().reshape(q_or.shape), q_or)
+    x = randn_bf16((M, K), 1.0, 2710 + M)
+    x[0, 5] = 0.0
+    if M > 2:
+        x[2, :64] = 0.0  # two all-zero blocks: scale 0, codes 0
+    b = randn_bf16((N,), 0.01, 2720)
+    r = randn_bf16((M, N), 1.0, 2730)
+    y = ops.linear(x.cuda(), qt, b.cuda(), posts[post], r.cuda(), None, 0.5)
+    fits = not (M == 16 and K == 11008)
+    rc = _lib.lib().tppx_linear_mxfp4_int8_rows(x.cuda().data_ptr(), *[a.data_ptr() for a in qt.native_w4a8()], None, None, None,
+                                                torch.empty((M, N), dtype=torch.bfloat16, device="cuda").data_ptr(), M, N, K,
+                                                0, 1.0, None)
+    assert (rc == _lib.OK) == fits and (fits or rc == _lib.EUNSUPPORTED)
+    ref = O.linear_w4a8(t2bits(x), q_or, s_or, bc, t2bits(b), posts[post], t2bits(r), None, 0.5)
+    # (the GEMM tile before an additive / multiplicative post-op may itself be one ulp from the oracle's: its ulp
+    # is added to the bound)
+    pre = O.linear_w4a8(t2bits(x), q_or, s_or, bc, t2bits(b)) if post in ("add", "mul") else None
+    assert_close_bf16(t2bits(y), ref, ulps=2 if post == "silu" else 1, what=f"w4a8 decode M={M} N={N} K={K} {post}", pre_bits=pre)
+    monkeypatch.setattr(ops, "W4A8_DECODE", False)
+    y2 = ops.linear(x.cuda(), qt, b.cuda(), posts[post], r.cuda(), None, 0.5)
+    assert_close_bf16(t2bits(y), t2bits(y2), ulps=2 if post == "silu" else 1, what="one launch vs quantizer + GEMM", pre_bits=pre)
+    if not fits:
+        assert torch.equal(y, y2)
+
+
 @pytest.mark.parametrize("kind", ["qint4", "qint2"])
 @pytest.mark.parametrize("M,N,K,post", [(1, 11008, 4096, "none"), (8, 4096, 11008, "add"), (16, 4096, 4096, "silu"),
                                         (5, 96, 1024, "mul"), (3, 8448, 14336, "add"),

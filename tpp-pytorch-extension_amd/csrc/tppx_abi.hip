@@ -856,6 +856,33 @@ extern "C" int tppx_linear_qintx(const void* x, void* xq, void* sa, const void* 
   return check_hip(launch_skinny_qintx(p, sp.mg, ntw, (hipStream_t)stream), who);
 }
 
+extern "C" int tppx_linear_mxfp4_int8_rows(const void* x, const void* q_nat, const void* s_nat, const void* bias,
+                                           const void* post_in, const void* post_in2, void* y, int64_t M, int64_t N,
+                                           int64_t K, int post_op, float post_scale, tppx_stream_t stream) {
+  const char* who = "tppx_linear_mxfp4_int8_rows";
+  int rc = check_common(who, x, M, K, 1, 0, nullptr, 0);
+  if (rc)
+    return rc;
+  TPPX_REQUIRE(K > 0 && K % 128 == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of 128", who, (long)K);
+  tppx_seg s = {q_nat, s_nat, bias, post_in, post_in2, y, N, post_op, post_scale};
+  DecodeParams p;
+  memset(&p, 0, sizeof(p));
+  rc = fill_all(who, &s, 1, 16, false, p);
+  if (rc)
+    return rc;
+  int ntw = 1;
+  TPPX_REQUIRE(skinny_w4a8_fits(M, p.total_tiles, (int)(K / 128), &ntw), TPPX_EUNSUPPORTED,
+               "%s: M=%ld rows of K=%ld channels are not a decode shape of this kernel (at most 16 rows whose int8 form fits the LDS); quantize the activations and call tppx_linear_mxfp4_int8", who, (long)M, (long)K);
+  p.x = x;
+  p.M = (int)M;
+  p.K = (int)K;
+  p.units = (int)(K / 128);
+  p.tpb = 1;
+  p.S = 1;
+  set_groups(p, ntw, false);
+  return check_hip(launch_skinny_w4a8(p, ntw, (hipStream_t)stream), who);
+}
+
 extern "C" void tppx_reload_env(void) {
   std::lock_guard<std::mutex> lock(g_env_mu);
   g_env_kept.clear();

@@ -108,4 +108,15 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
+// W4A8 (USE_MXFP4_INT8): the integer the reference multiplies for an E2M1 code = its value times 127 / 6, rounded
+// four 4-bit E2M1 codes (one per byte, bits 0..3) -> four int8 values
+__device__ __forceinline__ uint32_t w4a8_expand(uint32_t codes) {
+  const uint32_t sel = codes & 0x07070707u;
+  // v_perm_b32: selector bytes 0..3 pick from the second operand, 4..7 from the first
+  const uint32_t pos = __builtin_amdgcn_perm(0x7F55402Au, 0x20150B00u, sel); // 0 11 21 32 | 42 64 85 127
+  const uint32_t neg = __builtin_amdgcn_perm(0x81ABC0D6u, 0xE0EBF500u, sel); // the same, negated
+  const uint32_t m = ((codes >> 3) & 0x01010101u) * 0xFFu;                   // 0xFF in the bytes with the sign bit
+  return (neg & m) | (pos & ~m);
+}
+
 } // namespace tppx

@@ -138,6 +138,9 @@ hipError_t launch_skinny_qint8_nk(DecodeParams& p, int mg, hipStream_t stream);
 // QINT4 / QINT2 codes at their own width, 17..64 rows per block row: mg = 2 / 4 row groups, ntw = 1..3 channel tiles
 // per workgroup; p.wbits, p.mt (operand-order activations) and p.groups set by the caller
 hipError_t launch_skinny_qintx(DecodeParams& p, int mg, int ntw, hipStream_t stream);
+// W4A8 decode kernel (M <= 16): does it fit (LDS), and with how many channel tiles per workgroup; p.units = K / 128
+bool skinny_w4a8_fits(int64_t M, int total_tiles, int ktiles, int* ntw_out);
+hipError_t launch_skinny_w4a8(DecodeParams& p, int ntw, hipStream_t stream);
 hipError_t launch_skinny_mxfp4_nk(DecodeParams& p, hipStream_t stream);
 hipError_t launch_skinny_bf16(DecodeParams& p, int mg, int nt, hipStream_t stream);
 size_t skinny_mxfp4_xl_lds(int units, int nt, bool dual);

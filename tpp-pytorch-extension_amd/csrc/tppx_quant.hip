@@ -729,6 +729,34 @@ prepack_qint4_kernel(const uint8_t* __restrict__ q4, int64_t N, int64_t K, int64
   reinterpret_cast<uint4*>(qnat)[t] = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
+// W4A8 weight (remap_and_quantize_mxfp4 under USE_MXFP4_INT8: q u8 [N/8][K/bc][bc/8][8][4], byte i of a group of 8
+// K values = value i | value 4 + i << 4; scales u8 [N/8][K/bc][bc/32][8]) -> the decode kernel's tiles:
+// q [N/16][K/128][64 lanes][4 dwords], lane = (channel c = lane & 15, K group kg = lane >> 4), dword j = the
+// reference's dword of K group kg of MX block j of the tile; scales [N/16][K/128][16 c] dwords of the tile's four
+// E8M0 bytes.  One thread per (tile, lane).
+__global__ void __launch_bounds__(256)
+prepack_w4a8_kernel(const uint32_t* __restrict__ qref, const uint8_t* __restrict__ sref, int64_t N, int64_t K, int64_t bc,
+                    uint32_t* __restrict__ qnat, uint32_t* __restrict__ snat) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t KT = K / 128;
+  if (t >= (N / 16) * KT * 64)
+    return;
+  const int lane = (int)(t & 63), c = lane & 15, kg = lane >> 4;
+  const int64_t tile = t >> 6, kt = tile % KT, ntile = tile / KT;
+  const int64_t n = ntile * 16 + c, n8b = n >> 3, n8 = n & 7;
+  const int64_t C1 = K / bc, G = bc / 8, SB = bc / 32;
+  uint32_t w[4], sc = 0;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int64_t k0 = (kt * 4 + j) * 32, c1 = k0 / bc, kb = k0 % bc;
+    w[j] = qref[(((n8b * C1 + c1) * G + (kb >> 3) + kg) * 8 + n8)];
+    sc |= (uint32_t)sref[((n8b * C1 + c1) * SB + (kb >> 5)) * 8 + n8] << (8 * j);
+  }
+  reinterpret_cast<uint4*>(qnat)[t] = make_uint4(w[0], w[1], w[2], w[3]);
+  if (kg == 0)
+    snat[tile * 16 + c] = sc;
+}
+
 // Native int8 tiles [N/16][K/64][64 lanes][16 B] of a QINT4 / QINT2 weight -> the codes at their own width, for the
 // decode kernel that expands them in registers: [N/16][K/(64 G)][64 lanes][16 B], G = 8 / BITS tiles per 16 bytes.
 //   BITS 4: byte b of dword d = (tile 0's byte d*4+b & 15) | (tile 1's byte d*4+b << 4)        (values -8..7)
@@ -906,6 +934,19 @@ extern "C" int tppx_prepack_qint8(const void* q_ref, int64_t N, int64_t K,
   prepack_qint8_kernel<<<grid_for(nchunks, 256), 256, 0, (hipStream_t)stream>>>(
       (const int8_t*)q_ref, N, K, qbs, (int8_t*)q_nat);
   return check_hip(hipGetLastError(), "tppx_prepack_qint8");
+}
+
+extern "C" int tppx_prepack_mxfp4_int8(const void* q_ref, const void* sc_ref, int64_t N, int64_t K, int64_t bc,
+                                       void* q_nat, void* s_nat, tppx_stream_t stream) {
+  const char* who = "tppx_prepack_mxfp4_int8";
+  TPPX_REQUIRE(q_ref && sc_ref && q_nat && s_nat, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(aligned16(q_nat) && ((uintptr_t)q_ref & 3) == 0 && ((uintptr_t)s_nat & 3) == 0, TPPX_EINVAL, "%s: pointer misaligned", who);
+  TPPX_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 128 == 0 && bc >= 32 && bc % 32 == 0 && K % bc == 0, TPPX_ESHAPE,
+               "%s: N=%ld must be a multiple of 16, K=%ld of 128 and of the block %ld (a multiple of 32)", who, (long)N, (long)K, (long)bc);
+  const int64_t threads = (N / 16) * (K / 128) * 64;
+  prepack_w4a8_kernel<<<grid_for(threads, 256), 256, 0, (hipStream_t)stream>>>((const uint32_t*)q_ref, (const uint8_t*)sc_ref,
+                                                                              N, K, bc, (uint32_t*)q_nat, (uint32_t*)s_nat);
+  return check_hip(hipGetLastError(), who);
 }
 
 extern "C" int tppx_pack_qint_tiles(const void* native_i8, int64_t N, int64_t K, int bits, void* packed,

@@ -1408,6 +1408,167 @@ skinny_qintx_kernel(const DecodeParams p) {
 }
 
 // ---------------------------------------------------------------------------
+// W4A8 (USE_MXFP4_INT8: MXFP4 weights x int8 activations over blocks of 32, src/csrc/fused_gemm.h:965-978), M <= 16.
+// The shape of skinny_qint8_fq_kernel: W waves (sixteen; eight with three channel tiles per workgroup, whose
+// registers sixteen cannot hold) split K in tiles of 128 channels; a wave quantises its K
+// range of the bf16 rows itself -- one (row, tile) item = 8 lanes x 16 values, the two lanes of a 32-wide block
+// exchange their maxima, scale = max / 127 as quantize_int8sym, times 6 / 127 as the reference scales it -- into
+// wave-private LDS in MFMA operand order, and streams the weights through a register ring.  Weight tiles are
+// tppx_prepack_mxfp4_int8's: lane (channel c = lane & 15, K group kg = lane >> 4) holds four dwords, dword j = the
+// eight codes of K group kg of MX block j of the tile as the reference packs them (byte i = value i | value 4 + i
+// << 4), so each dword expands to the lane's operand of one K = 32 int8 MFMA = one MX block, whose exact int32 sums
+// are folded into fp32 with sa[row][block] * 2^(e - 127); scales [tile][16 c] dwords of four E8M0 bytes.
+// ---------------------------------------------------------------------------
+template <int NTW, int PF, int XB, int W>
+__global__ void __launch_bounds__(W * 64)
+skinny_w4a8_kernel(const DecodeParams p) {
+  extern __shared__ __align__(16) float sk_lds[];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int grp = blockIdx.x;
+  const DecodeSeg& sg = p.seg[sk_find_seg(p, grp)];
+  const int ltile0 = (grp - sg.grp0) * NTW;
+  const int M = p.M; // <= 16
+  const int KT = p.units; // K tiles of 128 channels
+  const int t0 = (wave * KT) / W, t1 = ((wave + 1) * KT) / W;
+
+  const i32x4* wq[NTW];
+  const uint32_t* ws[NTW];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++) {
+    const int64_t lt = min(ltile0 + nt, sg.tiles - 1);
+    // (uniform bases: the lane's part stays a 32-bit offset, so the loads take scalar base + vector offset and the
+    // six pointers cost no vector registers)
+    wq[nt] = reinterpret_cast<const i32x4*>(sg.qw) + lt * KT * 64;
+    ws[nt] = reinterpret_cast<const uint32_t*>(sg.sw) + lt * KT * 16;
+  }
+  // activation rows first (L2), then the post-op inputs, then the weight ring (loads return in issue order)
+  const uint16_t* xb = reinterpret_cast<const uint16_t*>(p.x);
+  const int nitems = M * (t1 - t0);
+  const uint32_t Mu = (uint32_t)M, mmagic = p.m_magic;
+  auto tile_of_item = [&](uint32_t it) { return mmagic ? __umulhi(it, mmagic) : it; }; // it / M
+  i32x4 raw[XB][2];
+  auto load_pass = [&](auto PS, int base) {
+    constexpr int ps = decltype(PS)::value;
+    const uint32_t it = (uint32_t)min((base + ps) * 8 + (lane >> 3), max(nitems - 1, 0));
+    const uint32_t ul = tile_of_item(it), mr = it - ul * Mu;
+    const i32x4* src = reinterpret_cast<const i32x4*>(xb + (int64_t)mr * p.K + (int64_t)(t0 + (int)ul) * 128 + (lane & 7) * 16);
+    raw[ps][0] = src[0];
+    raw[ps][1] = src[1];
+  };
+  static_for<0, XB>([&](auto PS) { load_pass(PS, 0); });
+  __builtin_amdgcn_sched_barrier(0);
+  SkEpilogue<1, NTW, false, W> ep;
+  ep.prefetch_flat(p, sg, ltile0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+  i32x4 wreg[PF][NTW];
+  uint32_t sreg[PF][NTW];
+  auto load_stage = [&](int st, int t) {
+    t = max(min(t, t1 - 1), 0); // past the end (or a wave without tiles): re-read a valid tile, never consumed
+#pragma unroll
+    for (int nt = 0; nt < NTW; nt++) {
+      wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64 + lane);
+      sreg[st][nt] = (ws[nt] + (int64_t)t * 16)[lane & 15];
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < PF; i++)
+    load_stage(i, t0 + i);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // wave-private LDS behind the reduction region: xq [tile][block j][K group][M rows] x 8 B, then sa [tile][j][16]
+  float* red = sk_lds;
+  uint8_t* mine = reinterpret_cast<uint8_t*>(sk_lds + (size_t)W * NTW * 256) + (size_t)wave * p.cht * (128 * M + 256);
+  uint2* xq_s = reinterpret_cast<uint2*>(mine);
+  float* sa_s = reinterpret_cast<float*>(mine + (size_t)p.cht * 128 * M);
+  auto quant_pass = [&](auto PS, int base) {
+    constexpr int ps = decltype(PS)::value;
+    if ((base + ps) * 8 < nitems) { // wave-uniform
+      const int it = (base + ps) * 8 + (lane >> 3);
+      const uint32_t itc = (uint32_t)min(it, nitems - 1);
+      const uint32_t ul = tile_of_item(itc), mr = itc - ul * Mu;
+      float v[16];
+      float amax = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const uint32_t wd = (uint32_t)raw[ps][j >> 2][j & 3];
+        v[2 * j] = bf16_bits_to_f32(wd & 0xffffu);
+        v[2 * j + 1] = bf16_bits_to_f32(wd >> 16);
+        amax = fmaxf(amax, fmaxf(fabsf(v[2 * j]), fabsf(v[2 * j + 1])));
+      }
+      amax = sk_dpp_max<0xB1>(amax); // quad_perm [1,0,3,2]: the other half of the 32-wide block
+      const float sc = __fdiv_rn(amax, 127.0f);
+      const float inv = sc != 0.0f ? __frcp_rn(sc) : 0.0f;
+      uint32_t pk[4];
+#pragma unroll
+      for (int d = 0; d < 4; d++)
+        pk[d] = sk_int8x4_rne(v[4 * d], v[4 * d + 1], v[4 * d + 2], v[4 * d + 3], inv);
+      if (it < nitems) {
+        const int s = lane & 7, j = s >> 1, kg0 = (s & 1) * 2; // values s*16 .. of the tile: block j, K groups kg0, kg0 + 1
+        uint2* dst = xq_s + (((int)ul * 4 + j) * 4 + kg0) * M + (int)mr;
+        dst[0] = make_uint2(pk[0], pk[1]);
+        dst[M] = make_uint2(pk[2], pk[3]);
+        if ((s & 1) == 0)
+          sa_s[((int)ul * 4 + j) * 16 + (int)mr] = __fmul_rn(sc, (float)(6.0 / 127.0));
+      }
+    }
+  };
+  static_for<0, XB>([&](auto PS) { quant_pass(PS, 0); });
+  for (int base = XB; base * 8 < nitems; base += XB) {
+    static_for<0, XB>([&](auto PS) { load_pass(PS, base); });
+    static_for<0, XB>([&](auto PS) { quant_pass(PS, base); });
+  }
+  const int xoff = (lane >> 4) * M + min(lane & 15, M - 1); // (K group, row) inside a block's operand image
+
+  f32x4 facc[NTW][1];
+#pragma unroll
+  for (int nt = 0; nt < NTW; nt++)
+    facc[nt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto consume = [&](int i, int tt) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const uint2 xa2 = xq_s[((tt - t0) * 4 + j) * 4 * M + xoff];
+      const long xa = (long)(((uint64_t)xa2.y << 32) | xa2.x);
+      // result rows (lane >> 4) * 4 + r; scales of rows >= M are whatever the LDS held: those rows are not stored
+      const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + ((tt - t0) * 4 + j) * 16 + (lane >> 4) * 4);
+#pragma unroll
+      for (int nt = 0; nt < NTW; nt++) {
+        const uint32_t codes = (uint32_t)wreg[i][nt][j];
+        const uint32_t lo = w4a8_expand(codes & 0x0F0F0F0Fu), hi = w4a8_expand((codes >> 4) & 0x0F0F0F0Fu);
+        const long wb = (long)(((uint64_t)hi << 32) | lo);
+        const i32x4 acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, wb, i32x4{0, 0, 0, 0}, 0, 0, 0);
+        const float wsc = e8m0_to_f32(sreg[i][nt] >> (8 * j));
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          facc[nt][0][r] = fmaf((float)acc[r], sav[r] * wsc, facc[nt][0][r]);
+      }
+      if (NTW > 2)
+        __builtin_amdgcn_sched_barrier(0); // one block after the other: interleaved, their temporaries spill
+    }
+  };
+  int t = t0;
+  for (; t + 2 * PF <= t1; t += PF) { // branch-free full groups: every reload is a real tile
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      consume(i, t + i);
+      load_stage(i, t + i + PF);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  for (; t < t1; t += PF) {
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+      const int tt = t + i;
+      if (tt < t1) {
+        consume(i, tt);
+        if (tt + PF < t1)
+          load_stage(i, tt + PF);
+      }
+    }
+  }
+  ep.finish(sg, facc, red);
+}
+
+// ---------------------------------------------------------------------------
 // MXFP4, M <= 16, activations staged in LDS by the wave that consumes them,
 // with an optional transform on the way in:
 //   XMODE 0  x as it is
@@ -2345,6 +2506,30 @@ hipError_t launch_skinny_qintx(DecodeParams& p, int mg, int ntw, hipStream_t str
   SKQR(2, 1) SKQR(2, 2) SKQR(2, 3) SKQR(4, 1) SKQR(4, 2) SKQR(4, 3)
 #undef SKQR
   return hipErrorInvalidValue;
+}
+
+// W4A8, M <= 16, weights prepacked by tppx_prepack_mxfp4_int8; false when the quantised rows do not fit the LDS
+bool skinny_w4a8_fits(int64_t M, int total_tiles, int ktiles, int* ntw_out) {
+  const int ntw = total_tiles <= 256 ? 1 : (total_tiles <= 512 ? 2 : 3);
+  const int w = ntw == 3 ? 8 : 16;
+  const int cht = (ktiles + w - 1) / w;
+  const size_t xbytes = (size_t)w * cht * (128 * (size_t)M + 256), rbytes = (size_t)w * ntw * 1024;
+  *ntw_out = ntw;
+  return M >= 1 && M <= 16 && xbytes + rbytes <= 160 * 1024;
+}
+
+hipError_t launch_skinny_w4a8(DecodeParams& p, int ntw, hipStream_t stream) {
+  const int w = ntw == 3 ? 8 : 16;
+  p.cht = (p.units + w - 1) / w;
+  p.m_magic = p.M > 1 ? (unsigned int)(((1ull << 32) + (unsigned int)p.M - 1) / (unsigned int)p.M) : 0u;
+  dim3 grid(p.groups, 1, 1);
+  const size_t lds = (size_t)w * p.cht * (128 * (size_t)p.M + 256) + (size_t)w * ntw * 1024;
+  // a wave holds at most four K tiles at the 7B shapes: a ring of four (two with two channel tiles: registers)
+  switch (ntw) {
+    case 1: return sk_launch(skinny_w4a8_kernel<1, 4, 4, 16>, p, grid, 16, lds, stream);
+    case 2: return sk_launch(skinny_w4a8_kernel<2, 2, 4, 16>, p, grid, 16, lds, stream);
+    default: return sk_launch(skinny_w4a8_kernel<3, 4, 4, 8>, p, grid, 8, lds, stream);
+  }
 }
 
 // MXFP4, 33..64 rows per block row: four channel tiles x four K parts per workgroup, K in p.S slices across workgroups

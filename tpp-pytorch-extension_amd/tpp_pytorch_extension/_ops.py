@@ -606,6 +606,7 @@ def _linear_other_types(input, weight, bias, post, flags, post_in=None, post_in2
 
 PACKED_CODES = os.environ.get("TPPX_PACKED_CODES", "1") == "1"
 W4A8_ACT_SCALE = 6.0 / 127.0
+W4A8_DECODE = os.environ.get("TPPX_W4A8_DECODE", "1") == "1"
 
 
 def _linear_w4a8(input, weight, bias, post, post_in, post_in2, post_scale):
@@ -624,11 +625,21 @@ def _linear_w4a8(input, weight, bias, post, post_in, post_in2, post_scale):
     y = torch.empty(tuple(input.shape[:-1]) + (N,), dtype=torch.bfloat16, device=x.device)
     if M == 0:
         return y
-    act = quantize_int8sym(x.view(M, K), 32, -1, False)
-    sa = act.scales.mul_(W4A8_ACT_SCALE)
     bias = _prep_bias(bias, N, x.device)
     post_in = _prep_post(post_in, M, N, "post-op input", x.device)
     post_in2 = _prep_post(post_in2, M, N, "second post-op input", x.device)
+    # decode steps: one launch that quantizes its rows itself and splits K over the waves of a workgroup
+    # (TPPX_W4A8_DECODE=0 keeps the two-step path)
+    nat = weight.native_w4a8() if (M <= 16 and W4A8_DECODE) else None
+    if nat is not None:
+        rc = L.tppx_linear_mxfp4_int8_rows(x.data_ptr(), nat[0].data_ptr(), nat[1].data_ptr(), _lib.ptr(bias),
+                                           _lib.ptr(post_in), _lib.ptr(post_in2), y.data_ptr(), M, N, K, post, post_scale,
+                                           _lib.stream_of(x))
+        if rc != _lib.EUNSUPPORTED:  # rows that do not fit the kernel's LDS take the two-step path
+            _lib.check(rc)
+            return y
+    act = quantize_int8sym(x.view(M, K), 32, -1, False)
+    sa = act.scales.mul_(W4A8_ACT_SCALE)
     _lib.check(L.tppx_linear_mxfp4_int8(act.qdata.data_ptr(), sa.data_ptr(), weight.qdata.data_ptr(),
                                         weight.scales.data_ptr(), _lib.ptr(bias), _lib.ptr(post_in), _lib.ptr(post_in2),
                                         y.data_ptr(), M, N, K, weight.shape[2] * 8, post, post_scale, _lib.stream_of(x)))

@@ -163,6 +163,26 @@ class QTensor(torch.Tensor):
             have = self._native_packed = (packed, sn, bits)
         return have
 
+    def native_w4a8(self):
+        """W4A8 (USE_MXFP4_INT8) weights: (codes in MFMA operand order, E8M0 scales per tile and channel) for the
+        decode kernel, made once from the reference layout (tppx_prepack_mxfp4_int8); None when K is not a multiple
+        of 128 or N of 16."""
+        have = getattr(self, "_native_w4a8", None)
+        if have is None:
+            if self.weight_kind() != "mxfp4_int8":
+                raise _lib.TppxError(_lib.EUNSUPPORTED, f"not a W4A8 weight: {self!r}")
+            N, K = self.weight_nk()
+            if N % 16 or K % 128:
+                have = self._native_w4a8 = ()
+            else:
+                qn = torch.empty(N * K // 2, dtype=torch.uint8, device=self.qdata.device)
+                sn = torch.empty(N * K // 32, dtype=torch.uint8, device=self.qdata.device)
+                _lib.check(_lib.lib().tppx_prepack_mxfp4_int8(self.qdata.data_ptr(), self.scales.data_ptr(), N, K,
+                                                              self.shape[2] * 8, qn.data_ptr(), sn.data_ptr(),
+                                                              _lib.stream_of(self.qdata)))
+                have = self._native_w4a8 = (qn, sn)
+        return have or None
+
     def dequantize(self):
         """fp32 tensor in the blocked shape (PerBlock*Quantizer::dequantize,
         src/csrc/qtypes.cpp:438-473,521-577)."""
