@@ -450,7 +450,9 @@ int tppx_rotary_kv_append_llama(void* q, void* k, const void* v,
  * sequence: q bf16 [B][Nq][128], cache bf16 [B][Nkv][Smax][128], additive mask
  * bf16 [B][mask_ld] or NULL; valid keys = *kv_len_dev (device i32) + kv_len_add
  * (the counter may still hold the length before this step's append); out bf16
- * [B][Nq][128].  ws: optional scratch for split-KV partial results. */
+ * [B][Nq][128].  ws: optional scratch for split-KV partial results.  Head sizes
+ * H other than 128 (multiples of 8 up to 256, tensors [..][H]) run a plain,
+ * untuned kernel; anything else returns TPPX_EUNSUPPORTED. */
 int tppx_attn_decode(const void* q, const void* kcache, const void* vcache,
                      const void* mask, int64_t mask_ld, const void* kv_len_dev,
                      int64_t kv_len_add, void* out, int64_t B, int64_t Nq,
@@ -479,7 +481,7 @@ int tppx_attn_decode_rotary(const void* q, const void* k, const void* v,
  * q / out bf16 [B][S][Nq][128]; the cache already holds the S new keys at
  * positions past_len .. past_len+S-1 (tppx_rotary_kv_append_llama before this
  * call); query i sees keys 0 .. past_len+i; additive mask bf16 [B][mask_ld]
- * over key positions or NULL. */
+ * over key positions or NULL.  Head sizes other than 128: as tppx_attn_decode. */
 int tppx_attn_prefill(const void* q, const void* kcache, const void* vcache,
                       const void* mask, int64_t mask_ld, int64_t past_len,
                       void* out, int64_t B, int64_t S, int64_t Nq, int64_t Nkv,

@@ -1171,6 +1171,107 @@ static int attn_decode_launch(const char* who, AttnParams& p, bool rot, int64_t 
   return check_hip(hipGetLastError(), who);
 }
 
+// ---------------------------------------------------------------------------
+// Attention for head sizes other than 128 (attn<T>, src/csrc/llm/attn.cpp:781-955, is generic in the head size; the
+// kernels above are built for 128): one kernel for the single-query step and for prompt passes, H a multiple of 8
+// up to 256.  One wave per (sequence, query token, query head), four per workgroup, no barrier: 64 keys per trip,
+// a lane takes the whole dot product of its key (16-byte loads along its row, the query as fp32 in wave-private
+// LDS, read as broadcasts), online softmax over the trip with the probabilities rounded to bf16 before they multiply
+// V and the normaliser summing the unrounded ones, then lanes turn to output dimensions (lane, lane + 64, ...) and
+// walk the trip's value rows.  A plain kernel for the shapes the tuned ones do not take, not a tuned one.
+// ---------------------------------------------------------------------------
+struct AttnGenParams {
+  const uint16_t* q;   // [B][S][Nq][H]
+  const uint16_t* kc;  // [B][Nkv][Smax][H]
+  const uint16_t* vc;
+  const uint16_t* mask; // bf16 [B][mask_ld] additive, or null
+  const int32_t* kv_len; // single-query step: device scalar, valid keys = *kv_len + kv_len_add; null: prompt pass
+  int kv_len_add;
+  uint16_t* out;       // [B][S][Nq][H]
+  int B, S, Nq, Nkv, H, Smax, mask_ld, past; // prompt pass: query i sees keys 0 .. past + i
+  float scale;
+};
+
+__global__ void __launch_bounds__(256)
+attn_generic_kernel(const AttnGenParams p) {
+  __shared__ __align__(16) float q_s[4][256];
+  __shared__ float p_s[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t qi = (int64_t)blockIdx.x * 4 + wave;
+  if (qi >= (int64_t)p.B * p.S * p.Nq) // whole waves; nothing below synchronises across waves
+    return;
+  const int h = (int)(qi % p.Nq), sq = (int)((qi / p.Nq) % p.S), b = (int)(qi / ((int64_t)p.Nq * p.S));
+  const int hk = h / (p.Nq / p.Nkv), H = p.H;
+  int L = p.kv_len ? p.kv_len[0] + p.kv_len_add : p.past + sq + 1;
+  L = max(min(L, p.Smax), 0);
+  const uint16_t* qrow = p.q + qi * H;
+  for (int d = lane; d < H; d += 64)
+    q_s[wave][d] = bf16_bits_to_f32(qrow[d]);
+  // the lanes of a wave hand values to one another through LDS: the LDS serves a wave's accesses in order; the
+  // fence and the wave barrier keep the compiler from moving the reads above the writes
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  const uint16_t* kb = p.kc + ((int64_t)b * p.Nkv + hk) * (int64_t)p.Smax * H;
+  const uint16_t* vb = p.vc + ((int64_t)b * p.Nkv + hk) * (int64_t)p.Smax * H;
+  const uint16_t* mrow = p.mask ? p.mask + (int64_t)b * p.mask_ld : nullptr;
+  float m = -3.0e38f, l = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int c0 = 0; c0 < L; c0 += 64) {
+    const int key = c0 + lane;
+    const uint16_t* krow = kb + (int64_t)min(key, L - 1) * H;
+    float d = 0.f;
+    for (int e = 0; e < H; e += 8) {
+      const i32x4 kv = *reinterpret_cast<const i32x4*>(krow + e);
+      const f32x4 qa = *reinterpret_cast<const f32x4*>(&q_s[wave][e]), qb = *reinterpret_cast<const f32x4*>(&q_s[wave][e + 4]);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const uint32_t w = (uint32_t)kv[j];
+        const float q0 = j < 2 ? qa[2 * j] : qb[2 * j - 4], q1 = j < 2 ? qa[2 * j + 1] : qb[2 * j - 3];
+        d = fmaf(bf16_bits_to_f32(w & 0xffffu), q0, d);
+        d = fmaf(bf16_bits_to_f32(w >> 16), q1, d);
+      }
+    }
+    d *= p.scale;
+    if (mrow && key < p.mask_ld && key < L)
+      d += bf16_bits_to_f32(mrow[key]);
+    const float sc = key < L ? d : -3.0e38f;
+    const float mn = fmaxf(m, wave_max(sc));
+    const float alpha = __expf(m - mn); // 1 when the maximum stays
+    m = mn;
+    const float pr = key < L ? __expf(sc - m) : 0.f;
+    l = l * alpha + wave_sum(pr);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      acc[i] *= alpha;
+    __builtin_amdgcn_wave_barrier(); // (the previous trip's reads of p_s are done)
+    p_s[wave][lane] = round_bf16(pr);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const int nk = min(64, L - c0);
+    for (int j = 0; j < nk; j++) {
+      const float pj = p_s[wave][j];
+      const uint16_t* vrow = vb + (int64_t)(c0 + j) * H;
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        if (lane + 64 * i < H)
+          acc[i] = fmaf(pj, bf16_bits_to_f32(vrow[lane + 64 * i]), acc[i]);
+    }
+  }
+  uint16_t* orow = p.out + qi * H;
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+    if (lane + 64 * i < H)
+      orow[lane + 64 * i] = (uint16_t)f32_to_bf16_bits(l > 0.f ? acc[i] / l : 0.f);
+}
+
+static int attn_generic_launch(const char* who, AttnGenParams& p, hipStream_t stream) {
+  TPPX_REQUIRE(p.H >= 8 && p.H <= 256 && p.H % 8 == 0, TPPX_EUNSUPPORTED,
+               "%s: head size %d (128 on the tuned kernels, other multiples of 8 up to 256 on the plain one)", who, p.H);
+  const int64_t waves = (int64_t)p.B * p.S * p.Nq;
+  TPPX_REQUIRE(waves > 0 && (waves + 3) / 4 < ((int64_t)1 << 31), TPPX_ESHAPE, "%s: problem too large", who);
+  attn_generic_kernel<<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(p);
+  return check_hip(hipGetLastError(), who);
+}
+
 extern "C" int tppx_attn_decode(const void* q, const void* kcache, const void* vcache, const void* mask,
                                 int64_t mask_ld, const void* kv_len_dev, int64_t kv_len_add, void* out, int64_t B, int64_t Nq,
                                 int64_t Nkv, int64_t H, int64_t Smax, void* ws, int64_t ws_bytes,
@@ -1179,10 +1280,18 @@ extern "C" int tppx_attn_decode(const void* q, const void* kcache, const void* v
   TPPX_REQUIRE(q && kcache && vcache && kv_len_dev && out, TPPX_EINVAL, "%s: null pointer", who);
   TPPX_REQUIRE(aligned16(q) && aligned16(kcache) && aligned16(vcache) && aligned16(out), TPPX_EINVAL,
                "%s: pointer not 16-byte aligned", who);
-  TPPX_REQUIRE(H == 128, TPPX_EUNSUPPORTED, "%s: head size %ld (only 128 is built)", who, (long)H);
   TPPX_REQUIRE(B > 0 && Nq > 0 && Nkv > 0 && Nq % Nkv == 0 && Smax > 0 && B * Nq < (1 << 30), TPPX_ESHAPE,
                "%s: bad shape B=%ld Nq=%ld Nkv=%ld Smax=%ld", who, (long)B, (long)Nq, (long)Nkv, (long)Smax);
   TPPX_REQUIRE(ws_bytes >= 0 && (ws_bytes == 0 || ws), TPPX_EINVAL, "%s: workspace size given with a null workspace", who);
+  if (H != 128) { // other head sizes: the plain kernel
+    AttnGenParams g;
+    memset(&g, 0, sizeof(g));
+    g.q = (const uint16_t*)q; g.kc = (const uint16_t*)kcache; g.vc = (const uint16_t*)vcache; g.mask = (const uint16_t*)mask;
+    g.kv_len = (const int32_t*)kv_len_dev; g.kv_len_add = (int)kv_len_add; g.out = (uint16_t*)out;
+    g.B = (int)B; g.S = 1; g.Nq = (int)Nq; g.Nkv = (int)Nkv; g.H = (int)H; g.Smax = (int)Smax; g.mask_ld = (int)mask_ld;
+    g.scale = 1.0f / sqrtf((float)H);
+    return attn_generic_launch(who, g, (hipStream_t)stream);
+  }
   AttnParams p;
   memset(&p, 0, sizeof(p));
   p.q = (const uint16_t*)q; p.kc = (const uint16_t*)kcache; p.vc = (const uint16_t*)vcache;
@@ -1227,7 +1336,6 @@ extern "C" int tppx_attn_prefill(const void* q, const void* kcache, const void* 
   TPPX_REQUIRE(q && kcache && vcache && out, TPPX_EINVAL, "%s: null pointer", who);
   TPPX_REQUIRE(aligned16(q) && aligned16(kcache) && aligned16(vcache) && aligned16(out), TPPX_EINVAL,
                "%s: pointer not 16-byte aligned", who);
-  TPPX_REQUIRE(H == 128, TPPX_EUNSUPPORTED, "%s: head size %ld (only 128 is built)", who, (long)H);
   TPPX_REQUIRE(B > 0 && S > 0 && Nq > 0 && Nkv > 0 && Nq % Nkv == 0 && Smax > 0 && B * Nq < 65536 &&
                    S < ((int64_t)1 << 24) && Smax < ((int64_t)1 << 30),
                TPPX_ESHAPE, "%s: bad shape B=%ld S=%ld Nq=%ld Nkv=%ld Smax=%ld", who, (long)B, (long)S, (long)Nq,
@@ -1235,6 +1343,16 @@ extern "C" int tppx_attn_prefill(const void* q, const void* kcache, const void* 
   TPPX_REQUIRE(past_len >= 0 && past_len + S <= Smax, TPPX_ESHAPE,
                "%s: %ld cached + %ld new keys exceed the cache capacity %ld", who, (long)past_len, (long)S, (long)Smax);
   TPPX_REQUIRE(!mask || mask_ld > 0, TPPX_EINVAL, "%s: mask given with mask_ld=%ld", who, (long)mask_ld);
+  if (H != 128) { // other head sizes: the plain kernel
+    AttnGenParams g;
+    memset(&g, 0, sizeof(g));
+    g.q = (const uint16_t*)q; g.kc = (const uint16_t*)kcache; g.vc = (const uint16_t*)vcache; g.mask = (const uint16_t*)mask;
+    g.out = (uint16_t*)out;
+    g.B = (int)B; g.S = (int)S; g.Nq = (int)Nq; g.Nkv = (int)Nkv; g.H = (int)H; g.Smax = (int)Smax; g.mask_ld = (int)mask_ld;
+    g.past = (int)past_len;
+    g.scale = 1.0f / sqrtf((float)H);
+    return attn_generic_launch(who, g, (hipStream_t)stream);
+  }
   AttnPrefillParams p;
   memset(&p, 0, sizeof(p));
   p.q = (const uint16_t*)q; p.kc = (const uint16_t*)kcache; p.vc = (const uint16_t*)vcache;
