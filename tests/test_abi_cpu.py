@@ -215,7 +215,7 @@ def test_launch_plans_of_the_baseline_shapes():
     lines = plan(L.tppx_plan_linear_qint8, 32, 4096, 11008, 256, 1, 0, ws)
     assert "skinny_qint8_nk_kernel<2, 4, 4, 3, 1, 8> grid=256x1x1" in lines[1], lines
     lines = plan(L.tppx_plan_linear_qint8, 64, 4096, 11008, 256, 1, 0, 0)  # no workspace: no K split
-    assert "skinny_qint8_kernel<4, 1, 8, 8, 8, true> grid=256x1x1" in lines[1], lines
+    assert "skinny_qint8_kernel<4, 1, 4, 8, 8, true> grid=256x1x1" in lines[1], lines
     assert len(plan(L.tppx_plan_linear_qint8, 64, 4096, 11008, 256, 0, 0, ws)) == 1             # pre-quantized input
     # config 3 / 5: MXFP4 decode
     assert "skinny_mxfp4_x4_kernel<1, 4, false> grid=256x1x1" in plan(L.tppx_plan_linear_mxfp4, 1, 4096, 11008, 0, ws)[0]

@@ -79,8 +79,14 @@ __device__ unsigned int sk_split_tickets[SK_TICKETS];
 // red layout: [wave][(a*MG + mg)*256 + r*64 + lane]; every thread finishes
 // EPT = NACC_OUT*MG*256 / blockDim outputs whose post-op inputs it fetched
 // before the main loop.
-template <int MG, int NACC, bool DUAL, int MINW>
+// FIXW: the number of waves of the workgroup where the kernel knows it at compile time (0: read from the launch).  The
+// cross-wave sums then unroll completely and all of a thread's LDS reads are issued before the first wait; with a
+// run-time count the compiler waited for the LDS once per output and batch of eight (36 waits of an LDS round trip
+// each in the 64-row gate/up epilogue: 1.3 us per half).
+template <int MG, int NACC, bool DUAL, int MINW, int FIXW = 0>
 struct SkEpilogue {
+  static __device__ __forceinline__ int nthreads() { return FIXW ? FIXW * 64 : (int)blockDim.x; }
+  static __device__ __forceinline__ int nwaves() { return FIXW ? FIXW : (int)(blockDim.x >> 6); }
   static constexpr int ELEMS = NACC * MG * 256;
   static constexpr int OUT = DUAL ? ELEMS / 2 : ELEMS;
   // outputs per thread; the launcher never uses fewer than MINW waves
@@ -111,7 +117,7 @@ struct SkEpilogue {
     const uint16_t* pi2 = has_in2 ? sg.post_in2 : sg.y;
 #pragma unroll
     for (int i = 0; i < MAXE; i++) {
-      const int e = threadIdx.x + i * blockDim.x;
+      const int e = threadIdx.x + i * nthreads();
       const int l = e & 63, r = (e >> 6) & 3, mg = (e >> 8) % MG, a = (e >> 8) / MG;
       const int m = m0 + mg * 16 + (l >> 4) * 4 + r;
       const int n = (ltile0 + a) * 16 + (l & 15);
@@ -132,7 +138,7 @@ struct SkEpilogue {
     has_bias = has_bias2 = has_in1 = has_in2 = true; // absent inputs are zeros already
 #pragma unroll
     for (int i = 0; i < MAXE; i++) {
-      const int e = threadIdx.x + i * blockDim.x;
+      const int e = threadIdx.x + i * nthreads();
       in1[i] = in2[i] = 0;
       bias[i] = bias2[i] = 0;
       off[i] = -1;
@@ -172,7 +178,7 @@ struct SkEpilogue {
     static_assert(DUAL, "two reduction rounds are for the gate/up pair");
     settle();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int W = blockDim.x >> 6;
+    const int W = nwaves();
     float* mine = red + wave * stride;
     float v[2][MAXE];
 #pragma unroll
@@ -189,10 +195,11 @@ struct SkEpilogue {
       __syncthreads();
 #pragma unroll
       for (int i = 0; i < MAXE; i++) {
-        const int e = threadIdx.x + i * blockDim.x;
+        const int e = threadIdx.x + i * nthreads();
         v[h][i] = 0.f;
         if (e < OUT)
-          for (int w = 0; w < W; w++)
+#pragma unroll
+          for (int w = 0; w < (FIXW ? FIXW : W); w++)
             v[h][i] += red[w * stride + e];
       }
     }
@@ -212,7 +219,7 @@ struct SkEpilogue {
     __shared__ float sq_s[16 * NACC];
 #pragma unroll
     for (int i = 0; i < MAXE; i++) {
-      const int e = threadIdx.x + i * blockDim.x;
+      const int e = threadIdx.x + i * nthreads();
       if (e < OUT) { // wave-uniform: e < OUT holds for whole waves
         float sq = ov[i] * ov[i];
         // the 16 lanes of a DPP row hold the 16 channels of one (row, tile) pair
@@ -250,7 +257,7 @@ struct SkEpilogue {
     __shared__ int arrived_last;
     settle();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int W = blockDim.x >> 6;
+    const int W = nwaves();
     float* mine = red + wave * stride;
 #pragma unroll
     for (int a = 0; a < NACC; a++)
@@ -265,10 +272,11 @@ struct SkEpilogue {
     float own[MAXE];
 #pragma unroll
     for (int i = 0; i < MAXE; i++) {
-      const int e = threadIdx.x + i * blockDim.x;
+      const int e = threadIdx.x + i * nthreads();
       own[i] = 0.f;
       if (e < OUT) {
-        for (int w = 0; w < W; w++)
+#pragma unroll
+        for (int w = 0; w < (FIXW ? FIXW : W); w++)
           own[i] += red[w * stride + e];
         if (ltile0 + e / (MG * 256) < sg.tiles)
           __hip_atomic_store(part + blockIdx.z * part_stride + e, own[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -296,7 +304,7 @@ struct SkEpilogue {
       for (int k = 0; k < 4; k++) {
         pv[i][k] = 0.f;
         if (off[i] >= 0 && k < p.S && k != (int)blockIdx.z)
-          pv[i][k] = __hip_atomic_load(part + k * part_stride + threadIdx.x + i * blockDim.x, __ATOMIC_RELAXED,
+          pv[i][k] = __hip_atomic_load(part + k * part_stride + threadIdx.x + i * nthreads(), __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
       }
     float ov[MAXE];
@@ -325,7 +333,7 @@ struct SkEpilogue {
                                          float* sumsq = nullptr, int M = 0) {
     settle();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int W = blockDim.x >> 6;
+    const int W = nwaves();
     float* mine = red + wave * stride;
 #pragma unroll
     for (int a = 0; a < NACC; a++)
@@ -338,15 +346,18 @@ struct SkEpilogue {
     float ov[MAXE];
 #pragma unroll
     for (int i = 0; i < MAXE; i++) {
-      const int e = threadIdx.x + i * blockDim.x;
+      const int e = threadIdx.x + i * nthreads();
       ov[i] = 0.f;
       if (e < OUT) {
         float v = 0.f, v2 = 0.f;
-        for (int w = 0; w < W; w++)
+#pragma unroll
+        for (int w = 0; w < (FIXW ? FIXW : W); w++)
           v += red[w * stride + e];
-        if (DUAL)
-          for (int w = 0; w < W; w++)
+        if (DUAL) {
+#pragma unroll
+          for (int w = 0; w < (FIXW ? FIXW : W); w++)
             v2 += red[w * stride + e + ELEMS / 2];
+        }
         uint32_t out = 0;
         if (off[i] >= 0) {
           if (DUAL) {
@@ -462,7 +473,7 @@ skinny_qint8_kernel(const DecodeParams p) {
   for (int j = 0; j < SAB; j++)
     sa0[j] = load_sa(j * 64 + lane);
   __builtin_amdgcn_sched_barrier(0);
-  SkEpilogue<MG, NTW, false, MINW> ep;
+  SkEpilogue<MG, NTW, false, MINW, (MAXW == MINW ? MAXW : 0)> ep;
   ep.prefetch_flat(p, sg, ltile0, m0);
   __builtin_amdgcn_sched_barrier(0);
   if (t0 < t1) {
@@ -1041,7 +1052,7 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
   // (the scheduler is free to move independent loads past one another: pinned, or it puts some of the activation
   // requests behind the weight ring and the quantisation waits for HBM)
   __builtin_amdgcn_sched_barrier(0);
-  SkEpilogue<1, NTW, false, MINW> ep;
+  SkEpilogue<1, NTW, false, MINW, (MAXW == MINW ? MAXW : 0)> ep;
   ep.prefetch_flat(p, sg, ltile0, 0);
   __builtin_amdgcn_sched_barrier(0);
 
@@ -1230,6 +1241,8 @@ skinny_qint8_fq_kernel(const DecodeParams p) {
             }
           }
         }
+        if (NTW > 2)
+          __builtin_amdgcn_sched_barrier(0); // one tile after the other: interleaved, the expanded operands spill
       }
     };
     const int s1 = t1 / G;
@@ -1331,7 +1344,7 @@ skinny_qintx_kernel(const DecodeParams p) {
   for (int j = 0; j < SAB; j++)
     sa0[j] = load_sa(j * 64 + lane);
   __builtin_amdgcn_sched_barrier(0);
-  SkEpilogue<MG, NTW, false, 8> ep;
+  SkEpilogue<MG, NTW, false, 8, 8> ep;
   ep.prefetch_flat(p, sg, ltile0, m0);
   __builtin_amdgcn_sched_barrier(0);
   if (t0 < t1) {
@@ -1457,7 +1470,7 @@ skinny_w4a8_kernel(const DecodeParams p) {
   };
   static_for<0, XB>([&](auto PS) { load_pass(PS, 0); });
   __builtin_amdgcn_sched_barrier(0);
-  SkEpilogue<1, NTW, false, W> ep;
+  SkEpilogue<1, NTW, false, W, W> ep;
   ep.prefetch_flat(p, sg, ltile0, 0);
   __builtin_amdgcn_sched_barrier(0);
   i32x4 wreg[PF][NTW];
@@ -1804,7 +1817,7 @@ skinny_mxfp4_xl_kernel(const DecodeParams p) {
   __builtin_amdgcn_sched_barrier(0);
 
   // post-op inputs: requested here so that their registers are not live while the activations are in flight
-  SkEpilogue<1, NTW, DUAL, 16> ep;
+  SkEpilogue<1, NTW, DUAL, 16, 16> ep;
   ep.prefetch(p, sg, ltile0, 0);
 
   f32x4 acc[NTW][1];
@@ -1929,7 +1942,7 @@ skinny_mxfp4_x4_kernel(const DecodeParams p) {
   });
   // the wave reads only what it wrote itself: program order is enough
 
-  SkEpilogue<1, NTW, DUAL, 16> ep;
+  SkEpilogue<1, NTW, DUAL, 16, 16> ep;
   ep.prefetch(p, sg, ltile0, 0);
   f32x4 acc[NTW][1];
 #pragma unroll
@@ -1992,7 +2005,7 @@ skinny_mxfp4_x4_kernel(const DecodeParams p) {
 // second kernel.  The epilogue's reduction scratch reuses the activation
 // regions.
 // ---------------------------------------------------------------------------
-template <int MG, int NT, bool DUAL, int PF, int W = 8>
+template <int MG, int NT, bool DUAL, int PF, int W = 8, bool XLATE = false>
 __global__ void __launch_bounds__(W * 64)
 skinny_mxfp4_mg_kernel(const DecodeParams p) {
   extern __shared__ __align__(16) float sk_lds[];
@@ -2078,7 +2091,7 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
     load_stage(i, t0 + i);
   // post-op inputs early, except where registers are scarcest (the gate/up pair has none but its biases)
   constexpr bool LATE_EP = DUAL && MG == 4;
-  SkEpilogue<MG, NTW, DUAL, W> ep;
+  SkEpilogue<MG, NTW, DUAL, W, W> ep;
   if (!LATE_EP)
     ep.prefetch(p, sg, ltile0, m0);
 
@@ -2090,9 +2103,15 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
       acc[nt][mg] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // one K tile: activations of the tile into LDS, the next tile's requested, then 4 steps x MG x NT MFMAs
+  // XLATE (the widest variants, 96 accumulators): the next tile's activations are requested BEHIND the tile's MFMAs,
+  // where the 64 staging registers are free, instead of in front of them -- that is what makes room for a second
+  // stage of the weight ring.  With one stage the next tile's weights could only be requested after the tile's last
+  // MFMA and were needed right away: every K tile waited a whole HBM round trip (4 x 2.3 us per wave at K = 4096);
+  // now it waits the L2 round trip of its activations.
   auto consume = [&](int i, int tnext) {
     store_x();
-    load_x(tnext);
+    if (!XLATE)
+      load_x(tnext);
     float sc[NTW];
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++)
@@ -2124,6 +2143,10 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
 #pragma unroll
     for (int i = 0; i < PF; i++) {
       consume(i, t + i + 1);
+      if (XLATE) {
+        __builtin_amdgcn_sched_barrier(0);
+        load_x(t + i + 1); // in front of the weights: loads return in issue order
+      }
       load_stage(i, t + i + PF);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -2134,6 +2157,10 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
       const int tt = t + i;
       if (tt < t1) {
         consume(i, tt + 1);
+        if (XLATE) {
+          __builtin_amdgcn_sched_barrier(0);
+          load_x(tt + 1);
+        }
         if (tt + PF < t1)
           load_stage(i, tt + PF);
       }
@@ -2224,7 +2251,7 @@ skinny_bf16_kernel(const DecodeParams p) {
 #pragma unroll
   for (int i = 0; i < PF; i++)
     load_stage(i, t0 + i);
-  SkEpilogue<MG, NT, false, W> ep;
+  SkEpilogue<MG, NT, false, W, W> ep;
   ep.prefetch(p, sg, ltile0, m0);
 
   f32x4 acc[NT][MG];
@@ -2445,9 +2472,11 @@ hipError_t launch_skinny_qint8(DecodeParams& p, const SkinnyPlan& pl, hipStream_
     case 1: SKQ(1, 1, 4, 16, 4);
     case 2: SKQ(2, 1, 4, 16, 4);
     default:
+      // a ring of four: one of eight spills 36 bytes per lane, and scratch costs far more than the deeper ring gains
+      // (4096 x 4096 at 64 rows: 11.9 us with it, 9.8 us without)
       if (p.mt > 0)
-        return sk_launch(skinny_qint8_kernel<4, 1, 8, 8, 8, true>, p, grid, pl.waves, lds, stream);
-      return sk_launch(skinny_qint8_kernel<4, 1, 4, 8, 8, false>, p, grid, pl.waves, lds, stream); // row-major rows: shorter ring, no spills
+        return sk_launch(skinny_qint8_kernel<4, 1, 4, 8, 8, true>, p, grid, pl.waves, lds, stream);
+      return sk_launch(skinny_qint8_kernel<4, 1, 4, 8, 8, false>, p, grid, pl.waves, lds, stream);
   }
 #undef SKQ
 }
@@ -2665,6 +2694,7 @@ hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hi
   }
   const size_t lds = skinny_mxfp4_mg_lds(mg, nt, 8); // the gate/up pair is reduced one half at a time
 #define SKMG(MG, NT, DUAL, PF) return sk_launch(skinny_mxfp4_mg_kernel<MG, NT, DUAL, PF>, p, grid, 8, lds, stream)
+#define SKMGL(MG, NT, DUAL, PF) return sk_launch(skinny_mxfp4_mg_kernel<MG, NT, DUAL, PF, 8, true>, p, grid, 8, lds, stream)
   if (dual) {
     if (mg == 2) {
       if (nt == 3)
@@ -2673,8 +2703,11 @@ hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hi
         SKMG(2, 2, true, 2);
       SKMG(2, 1, true, 2);
     }
-    if (nt == 3)
-      SKMG(4, 3, true, 1); // 96 accumulators + 64 staging registers: one ring stage
+    if (nt == 3) {
+      if (env_int("TPPX_MXFP4_MG_LATE", 1) != 0)
+        SKMGL(4, 3, true, 2); // 96 accumulators: two ring stages with the activations requested behind the MFMAs
+      SKMG(4, 3, true, 1);    // ... or one stage with them requested in front (64 staging registers live)
+    }
     if (nt == 2)
       SKMG(4, 2, true, 2);
     SKMG(4, 1, true, 2);
@@ -2688,14 +2721,18 @@ hipError_t launch_skinny_mxfp4_mg(DecodeParams& p, int mg, int nt, bool dual, hi
       SKMG(2, 2, false, 2);
     SKMG(2, 1, false, 2);
   }
-  if (nt == 4)
+  if (nt == 4) {
+    if (env_int("TPPX_MXFP4_MG_LATE", 1) != 0)
+      SKMGL(4, 4, false, 2);
     SKMG(4, 4, false, 1);
+  }
   if (nt == 3)
     SKMG(4, 3, false, 2);
   if (nt == 2)
     SKMG(4, 2, false, 2);
   SKMG(4, 1, false, 2);
 #undef SKMG
+#undef SKMGL
 }
 
 // bf16 weights: mg row groups of 16 per block row (1, 2 or 4), nt channel tiles per workgroup (1 or 2)
