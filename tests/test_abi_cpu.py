@@ -220,11 +220,11 @@ def test_launch_plans_of_the_baseline_shapes():
     # config 3 / 5: MXFP4 decode
     assert "skinny_mxfp4_x4_kernel<1, 4, false> grid=256x1x1" in plan(L.tppx_plan_linear_mxfp4, 1, 4096, 11008, 0, ws)[0]
     assert "skinny_mxfp4_xl_kernel<4, 2, false, 0, 8> grid=64x1x4" in plan(L.tppx_plan_linear_mxfp4, 16, 4096, 11008, 0, ws)[0]
-    assert "skinny_mxfp4_mg_kernel<1, 1, false, 4, 16>" in plan(L.tppx_plan_linear_mxfp4, 16, 4096, 11008, 0, 0)[0]  # no workspace
+    assert "skinny_mxfp4_mg_kernel<1, 1, false, 4, 16, false>" in plan(L.tppx_plan_linear_mxfp4, 16, 4096, 11008, 0, 0)[0]  # no workspace
     assert "skinny_mxfp4_xl_kernel<1, 2, false, 0, 8> grid=256x1x1" in plan(L.tppx_plan_linear_mxfp4, 16, 4096, 4096, 0, ws)[0]
     gate_up = (ctypes.c_int64 * 2)(11008, 11008)
     assert "skinny_mxfp4_xl_kernel<3, 2, true, 0, 2> grid=230x1x1" in plan(L.tppx_plan_multi_linear_mxfp4, gate_up, 2, 1, 4096, 1, 0, ws)[0]
-    assert "skinny_mxfp4_mg_kernel<4, 3, true, 1, 8> grid=230x1x1" in plan(L.tppx_plan_multi_linear_mxfp4, gate_up, 2, 64, 4096, 1, 0, ws)[0]
+    assert "skinny_mxfp4_mg_kernel<4, 3, true, 2, 8, true> grid=230x1x1" in plan(L.tppx_plan_multi_linear_mxfp4, gate_up, 2, 64, 4096, 1, 0, ws)[0]
     # config 4: prefill at 2048 rows
     assert "big_mxfp4_kernel<8, false, 1, 8> grid=256x1x1 block=512" in plan(L.tppx_plan_linear_mxfp4, 2048, 8192, 8192, 0, 0)[0]
     assert "big_mxfp4_kernel<8, false, 1, 8> grid=256x1x1" in plan(L.tppx_plan_linear_mxfp4, 2048, 8192, 28672, 0, 0)[0]
