@@ -193,22 +193,27 @@ struct SkEpilogue {
           for (int r = 0; r < 4; r++)
             mine[(a * MG + mg) * 256 + r * 64 + lane] = acc[h * (NACC / 2) + a][mg][r];
       __syncthreads();
+      // (no branch per output here or below: slots past the outputs repeat the last one and are not stored, so the
+      // outputs' LDS reads and their SiLU / multiply chains interleave instead of running one after the other)
 #pragma unroll
       for (int i = 0; i < MAXE; i++) {
-        const int e = threadIdx.x + i * nthreads();
+        const int e = min((int)threadIdx.x + i * nthreads(), OUT - 1);
         v[h][i] = 0.f;
-        if (e < OUT)
 #pragma unroll
-          for (int w = 0; w < (FIXW ? FIXW : W); w++)
-            v[h][i] += red[w * stride + e];
+        for (int w = 0; w < (FIXW ? FIXW : W); w++)
+          v[h][i] += red[w * stride + e];
       }
+    }
+    uint32_t out[MAXE];
+#pragma unroll
+    for (int i = 0; i < MAXE; i++) {
+      const uint32_t gact = apply_post_bits(v[0][i] + bf16_bits_to_f32(bias[i]), TPPX_POST_SILU, 0, 0, 1.0f);
+      out[i] = apply_post_bits(v[1][i] + bf16_bits_to_f32(bias2[i]), TPPX_POST_MUL, gact, 0, 1.0f);
     }
 #pragma unroll
     for (int i = 0; i < MAXE; i++)
-      if (off[i] >= 0) {
-        const uint32_t gact = apply_post_bits(v[0][i] + bf16_bits_to_f32(bias[i]), TPPX_POST_SILU, 0, 0, 1.0f);
-        sg.y[off[i]] = (uint16_t)apply_post_bits(v[1][i] + bf16_bits_to_f32(bias2[i]), TPPX_POST_MUL, gact, 0, 1.0f);
-      }
+      if (off[i] >= 0)
+        sg.y[off[i]] = (uint16_t)out[i];
   }
 
   // Row sums of squares of this workgroup's outputs (MG == 1): ov[i] = the rounded output of slot i as a float, 0
@@ -343,32 +348,39 @@ struct SkEpilogue {
         for (int r = 0; r < 4; r++)
           mine[(a * MG + mg) * 256 + r * 64 + lane] = acc[a][mg][r];
     __syncthreads();
+    // (no branch per output: slots past the outputs repeat the last one and are not stored, so the outputs' LDS reads
+    // and post-op chains interleave)
+    float v[MAXE], v2[MAXE];
+#pragma unroll
+    for (int i = 0; i < MAXE; i++) {
+      const int e = min((int)threadIdx.x + i * nthreads(), OUT - 1);
+      v[i] = v2[i] = 0.f;
+#pragma unroll
+      for (int w = 0; w < (FIXW ? FIXW : W); w++)
+        v[i] += red[w * stride + e];
+      if (DUAL) {
+#pragma unroll
+        for (int w = 0; w < (FIXW ? FIXW : W); w++)
+          v2[i] += red[w * stride + e + ELEMS / 2];
+      }
+    }
+    uint32_t out[MAXE];
+#pragma unroll
+    for (int i = 0; i < MAXE; i++) {
+      if (DUAL) {
+        const uint32_t gact = apply_post_bits(v[i] + bf16_bits_to_f32(bias[i]), TPPX_POST_SILU, 0, 0, 1.0f);
+        out[i] = apply_post_bits(v2[i] + bf16_bits_to_f32(bias2[i]), TPPX_POST_MUL, gact, 0, 1.0f);
+      } else {
+        out[i] = apply_post_bits(v[i] + bf16_bits_to_f32(bias[i]), sg.post_op, in1[i], in2[i], sg.post_scale);
+      }
+    }
     float ov[MAXE];
 #pragma unroll
     for (int i = 0; i < MAXE; i++) {
-      const int e = threadIdx.x + i * nthreads();
       ov[i] = 0.f;
-      if (e < OUT) {
-        float v = 0.f, v2 = 0.f;
-#pragma unroll
-        for (int w = 0; w < (FIXW ? FIXW : W); w++)
-          v += red[w * stride + e];
-        if (DUAL) {
-#pragma unroll
-          for (int w = 0; w < (FIXW ? FIXW : W); w++)
-            v2 += red[w * stride + e + ELEMS / 2];
-        }
-        uint32_t out = 0;
-        if (off[i] >= 0) {
-          if (DUAL) {
-            uint32_t gact = apply_post_bits(v + bf16_bits_to_f32(bias[i]), TPPX_POST_SILU, 0, 0, 1.0f);
-            out = apply_post_bits(v2 + bf16_bits_to_f32(bias2[i]), TPPX_POST_MUL, gact, 0, 1.0f);
-          } else {
-            out = apply_post_bits(v + bf16_bits_to_f32(bias[i]), sg.post_op, in1[i], in2[i], sg.post_scale);
-          }
-          sg.y[off[i]] = (uint16_t)out;
-          ov[i] = bf16_bits_to_f32(out & 0xffffu);
-        }
+      if (off[i] >= 0) {
+        sg.y[off[i]] = (uint16_t)out[i];
+        ov[i] = bf16_bits_to_f32(out[i] & 0xffffu);
       }
     }
     if (!DUAL && MG == 1 && sumsq) // uniform
@@ -674,21 +686,24 @@ __device__ __forceinline__ void sk_nk_finish(const DecodeParams& p, const Decode
           tot[q] += (k == z) ? own[q] : other[k]; // slice order: the same sums whichever workgroup arrives last
     }
   }
+  // (no branch per quad around the arithmetic: the quads' post-op chains interleave; only the store is conditional)
+  uint32_t out[Q][2];
+#pragma unroll
+  for (int q = 0; q < Q; q++) {
+    const uint32_t bw[2] = {bias2[q].x, bias2[q].y}, w1[2] = {in1[q].x, in1[q].y}, w2[2] = {in2[q].x, in2[q].y};
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const uint32_t a = apply_post_bits(tot[q][2 * h] + bf16_bits_to_f32(bw[h] & 0xffffu), sg.post_op, w1[h] & 0xffffu,
+                                         w2[h] & 0xffffu, sg.post_scale);
+      const uint32_t b = apply_post_bits(tot[q][2 * h + 1] + bf16_bits_to_f32(bw[h] >> 16), sg.post_op, w1[h] >> 16,
+                                         w2[h] >> 16, sg.post_scale);
+      out[q][h] = (a & 0xffffu) | (b << 16);
+    }
+  }
 #pragma unroll
   for (int q = 0; q < Q; q++)
-    if (valid[q]) {
-      const uint32_t bw[2] = {bias2[q].x, bias2[q].y}, w1[2] = {in1[q].x, in1[q].y}, w2[2] = {in2[q].x, in2[q].y};
-      uint32_t out[2];
-#pragma unroll
-      for (int h = 0; h < 2; h++) {
-        const uint32_t a = apply_post_bits(tot[q][2 * h] + bf16_bits_to_f32(bw[h] & 0xffffu), sg.post_op, w1[h] & 0xffffu,
-                                           w2[h] & 0xffffu, sg.post_scale);
-        const uint32_t b = apply_post_bits(tot[q][2 * h + 1] + bf16_bits_to_f32(bw[h] >> 16), sg.post_op, w1[h] >> 16,
-                                           w2[h] >> 16, sg.post_scale);
-        out[h] = (a & 0xffffu) | (b << 16);
-      }
-      *reinterpret_cast<uint2*>(sg.y + o[q]) = make_uint2(out[0], out[1]);
-    }
+    if (valid[q])
+      *reinterpret_cast<uint2*>(sg.y + o[q]) = make_uint2(out[q][0], out[q][1]);
 }
 
 template <int MG, int TW, int KPW, int WPF, int XPF, int MAXSTEPS>
