@@ -324,6 +324,34 @@ def test_w4a8_linear(M, post):
         assert torch.equal(sw, ops.fc_mul(x.cuda(), qt, None, ops.fc_silu(x.cuda(), qt, None)))
 
 
+@pytest.mark.parametrize("kind", ["qint4", "qint2"])
+@pytest.mark.parametrize("M", [100, 130])
+def test_packed_code_kernel_block_rows(kind, M):
+    """tppx_linear_qintx beyond 64 rows (the Python op keeps such calls on the expanded tiles): block rows of 64 on the
+    grid's second axis, the last one ragged; against the op on the expanded int8 tiles (another kernel family, so
+    another fp32 summation order: one ulp, plus the pre-op tile's ulp through the residual add)."""
+    ops = _ops()
+    from tpp_pytorch_extension import _lib
+    N, K = 1056 if kind == "qint4" else 1088, 2048
+    W = randn_bf16((N, K), 0.02, 2800 + M)
+    if kind == "qint4":
+        qt = ops.quantize_int4sym(W.view(N // 16, 16, K // 256, 128, 2).permute(0, 2, 3, 1, 4).contiguous().cuda(), 256, 2, True)
+    else:
+        qt = ops.remap_and_quantize_qint2_intlv(block_bf16(W).cuda())
+    x = randn_bf16((M, K), 1.0, 2810 + M).cuda()
+    r = randn_bf16((M, N), 1.0, 2830).cuda()
+    packed, sn, bits = qt.native_packed()
+    xq, sa = ops._qint8_scratch(x, M, K, 256)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    _lib.check(_lib.lib().tppx_linear_qintx(x.data_ptr(), xq.data_ptr(), sa.data_ptr(), packed.data_ptr(), sn.data_ptr(), None,
+                                            r.data_ptr(), None, y.data_ptr(), M, N, K, bits, O.POST_ADD_SCALE, 1.0, 0,
+                                            _lib.stream_of(x)))
+    assert M > 64  # the op itself does not take the packed kernel here
+    ref = ops.linear(x, qt, None, O.POST_ADD_SCALE, r, None, 1.0)
+    pre = ops.linear(x, qt, None)
+    assert_close_bf16(t2bits(y), t2bits(ref), what=f"{kind} packed block rows M={M}", pre_bits=t2bits(pre))
+
+
 @pytest.mark.parametrize("M,N,K,bc,post", [(1, 4096, 4096, 64, "none"), (8, 11008, 4096, 64, "add"), (16, 512, 2048, 128, "silu"),
                                            (5, 96, 1280, 32, "mul"), (8, 4096, 11008, 64, "add"), (3, 8448, 1536, 64, "none"),
                                            (16, 4096, 11008, 64, "add")])

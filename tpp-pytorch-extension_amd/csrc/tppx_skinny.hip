@@ -412,10 +412,10 @@ skinny_qint8_kernel(const DecodeParams p) {
   const int u0 = ub + sk_share(wave, ue - ub, W), u1 = ub + sk_share(wave + 1, ue - ub, W);
   const int t0 = u0 * G, t1 = u1 * G;
   const unsigned int magic = p.tpb_magic;
-  auto blk_of = [&](int t, bool) { // scale block of tile t (uniform): t / TPB without the division
+  auto blk_of = [&](int t) { // scale block of tile t (uniform): t / TPB without the division
     return magic ? (int)__umulhi((unsigned int)t, magic) : t;
   };
-  const int b0 = blk_of(max(min(t0, KT - 1), 0), FAST); // first scale block of this wave
+  const int b0 = blk_of(max(min(t0, KT - 1), 0)); // first scale block of this wave
 
   const i32x4* wq[NTW];
   const float* ws[NTW];
@@ -438,7 +438,7 @@ skinny_qint8_kernel(const DecodeParams p) {
 
   float* red = sk_lds;
   float* sa_s = sk_lds + (size_t)W * NTW * MG * 256 + (size_t)wave * p.cht * MPAD;
-  const int nsa = t0 < t1 ? (blk_of(t1 - 1, FAST) - b0 + 1) * MPAD : 0;
+  const int nsa = t0 < t1 ? (blk_of(t1 - 1) - b0 + 1) * MPAD : 0;
   const int mtp = p.mt * 16;
   constexpr int SAB = 2 * MG; // loads per batch: 8 K blocks of this wave
   auto load_sa = [&](int i) {
@@ -455,9 +455,9 @@ skinny_qint8_kernel(const DecodeParams p) {
   // order, or a branch inside the loop, drains the whole ring).
   i32x4 wreg[PF][NTW], xreg[PF][MG];
   float sreg[PF][NTW];
-  auto load_stage = [&](int st, int t, bool fast) {
+  auto load_stage = [&](int st, int t) {
     t = max(min(t, t1 - 1), 0); // past the end: re-read the last tile (never consumed)
-    const int b = blk_of(t, fast);
+    const int b = blk_of(t);
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
       wreg[st][nt] = __builtin_nontemporal_load(wq[nt] + (int64_t)t * 64);
@@ -477,7 +477,7 @@ skinny_qint8_kernel(const DecodeParams p) {
   // in flight and waits for all of them; a wave without K blocks re-reads valid data it never uses)
 #pragma unroll
   for (int i = 0; i < PF; i++)
-    load_stage(i, t0 + i, false);
+    load_stage(i, t0 + i);
   __builtin_amdgcn_sched_barrier(0); // keep the issue order of independent loads (see skinny_qint8_fq_kernel)
   // activation scales of this wave's K blocks, transposed in LDS: [u - u0][MPAD]
   float sa0[SAB];
@@ -517,7 +517,7 @@ skinny_qint8_kernel(const DecodeParams p) {
     }
 
   // multiply stage i (tile tt); `last` = tt closes a K block or this wave's part of one: fold into fp32
-  auto consume = [&](int i, int tt, bool last, bool fast) {
+  auto consume = [&](int i, int tt, bool last) {
     float swv[NTW];
 #pragma unroll
     for (int nt = 0; nt < NTW; nt++) {
@@ -527,7 +527,7 @@ skinny_qint8_kernel(const DecodeParams p) {
         iacc[nt][mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xreg[i][mg], wreg[i][nt], iacc[nt][mg], 0, 0, 0);
     }
     if (last) {
-      const int b = blk_of(tt, fast);
+      const int b = blk_of(tt);
 #pragma unroll
       for (int mg = 0; mg < MG; mg++) {
         const f32x4 sav = *reinterpret_cast<const f32x4*>(sa_s + (b - b0) * MPAD + mg * 16 + (lane >> 4) * 4);
@@ -549,8 +549,8 @@ skinny_qint8_kernel(const DecodeParams p) {
     for (; t + UN + PF <= t1; t += UN) {
 #pragma unroll
       for (int i = 0; i < UN; i++) {
-        consume(i % PF, t + i, (i & 3) == 3, true);
-        load_stage(i % PF, t + i + PF, true);
+        consume(i % PF, t + i, (i & 3) == 3);
+        load_stage(i % PF, t + i + PF);
         __builtin_amdgcn_sched_barrier(0); // keep the reload right behind its stage: the ring stays PF deep
       }
     }
@@ -562,9 +562,9 @@ skinny_qint8_kernel(const DecodeParams p) {
     for (int i = 0; i < PF; i++) {
       const int tt = tb + i;
       if (tt < t1) {
-        consume(i, tt, FAST ? (tt & 3) == 3 : ((tt + 1) % TPB == 0 || tt + 1 == t1), FAST);
+        consume(i, tt, FAST ? (tt & 3) == 3 : ((tt + 1) % TPB == 0 || tt + 1 == t1));
         if (tt + PF < t1)
-          load_stage(i, tt + PF, false);
+          load_stage(i, tt + PF);
       }
     }
   }
