@@ -8,8 +8,8 @@
 // Weight bytes are read where the reference keeps them, no repacking: q u8 [N/8][K/bc][bc/8][8][4], byte j of a
 // group (channel n8, 8 K values) = K value j | K value 4 + j << 4 -- the low nibbles of a lane's four bytes are the
 // first four of its eight MFMA operand bytes, the high nibbles the last four; scales u8 [N/8][K/bc][bc/32][8].
-// One wave owns a 16 x 16 output tile over the whole K (blocks in ascending order), four waves = 64 rows per
-// workgroup: the simple shape of a seldom-used path, not a tuned kernel.
+// A workgroup owns a 16 x 16 output tile; its four waves split the MX blocks of K and add their partial sums in
+// wave order: the simple shape of the calls the decode kernel (skinny_w4a8_kernel) does not take, not a tuned kernel.
 #include <hip/hip_runtime.h>
 
 #include "tppx.h"
@@ -32,22 +32,21 @@ struct W4A8Params {
 
 __global__ void __launch_bounds__(256)
 linear_w4a8_kernel(const W4A8Params p) {
+  __shared__ float part[4][64][4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int m0 = (blockIdx.y * 4 + wave) * 16;
-  if (m0 >= p.M) // whole waves only; no barrier below
-    return;
+  const int m0 = blockIdx.y * 16;
   const int n = blockIdx.x * 16 + (lane & 15), kg = lane >> 4;
   const int n8b = n >> 3, n8 = n & 7;
   const int C1 = p.K / p.bc, G = p.bc / 8, SB = p.bc / 32, NB = p.K / 32;
   const int8_t* xr = p.xq + (int64_t)min(m0 + (lane & 15), p.M - 1) * p.K + kg * 8;
-  float f[4];
+  float f[4] = {0.f, 0.f, 0.f, 0.f};
   const float* sar[4];
 #pragma unroll
-  for (int r = 0; r < 4; r++) {
-    f[r] = p.bias ? bf16_bits_to_f32(p.bias[n]) : 0.f;
+  for (int r = 0; r < 4; r++)
     sar[r] = p.sa + (int64_t)min(m0 + kg * 4 + r, p.M - 1) * NB;
-  }
-  for (int b = 0; b < NB; b++) {
+  // the four waves split the MX blocks of K (ascending ranges), their partial sums meet in LDS in wave order
+  const int b0 = (wave * NB) / 4, b1 = ((wave + 1) * NB) / 4;
+  for (int b = b0; b < b1; b++) {
     const int c1 = (b * 32) / p.bc, kb = (b * 32) % p.bc;
     const int64_t blk = (int64_t)n8b * C1 + c1;
     const uint32_t codes = *reinterpret_cast<const uint32_t*>(p.q + ((blk * G + (kb >> 3) + kg) * 8 + n8) * 4);
@@ -61,11 +60,19 @@ linear_w4a8_kernel(const W4A8Params p) {
       f[r] = fmaf((float)acc[r], sar[r][b] * wsc, f[r]);
   }
 #pragma unroll
+  for (int r = 0; r < 4; r++)
+    part[wave][lane][r] = f[r];
+  __syncthreads();
+  if (wave != 0)
+    return;
+  const float bias = p.bias ? bf16_bits_to_f32(p.bias[n]) : 0.f;
+#pragma unroll
   for (int r = 0; r < 4; r++) {
     const int m = m0 + kg * 4 + r;
+    const float v = bias + (((part[0][lane][r] + part[1][lane][r]) + part[2][lane][r]) + part[3][lane][r]);
     if (m < p.M) {
       const int64_t o = (int64_t)m * p.N + n;
-      p.y[o] = (uint16_t)apply_post_bits(f[r], p.post_op, p.post_in ? p.post_in[o] : 0, p.post_in2 ? p.post_in2[o] : 0,
+      p.y[o] = (uint16_t)apply_post_bits(v, p.post_op, p.post_in ? p.post_in[o] : 0, p.post_in2 ? p.post_in2[o] : 0,
                                          p.post_scale);
     }
   }
@@ -86,7 +93,7 @@ extern "C" int tppx_linear_mxfp4_int8(const void* xq, const void* sa, const void
   TPPX_REQUIRE(N > 0 && N % 16 == 0, TPPX_ESHAPE, "%s: N=%ld must be a positive multiple of 16", who, (long)N);
   TPPX_REQUIRE(bc >= 32 && bc % 32 == 0, TPPX_ESHAPE, "%s: input-channel block %ld must be a multiple of 32", who, (long)bc);
   TPPX_REQUIRE(K > 0 && K % bc == 0, TPPX_ESHAPE, "%s: K=%ld must be a positive multiple of the block %ld", who, (long)K, (long)bc);
-  const int64_t by = (M + 63) / 64;
+  const int64_t by = (M + 15) / 16;
   TPPX_REQUIRE(by <= 65535 && M * N < ((int64_t)1 << 40), TPPX_ESHAPE, "%s: problem too large", who);
   if (M == 0)
     return TPPX_OK;
