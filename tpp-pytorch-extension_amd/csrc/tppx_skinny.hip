@@ -2119,10 +2119,11 @@ skinny_mxfp4_mg_kernel(const DecodeParams p) {
 
   // one K tile: activations of the tile into LDS, the next tile's requested, then 4 steps x MG x NT MFMAs
   // XLATE (the widest variants, 96 accumulators): the next tile's activations are requested BEHIND the tile's MFMAs,
-  // where the 64 staging registers are free, instead of in front of them -- that is what makes room for a second
-  // stage of the weight ring.  With one stage the next tile's weights could only be requested after the tile's last
-  // MFMA and were needed right away: every K tile waited a whole HBM round trip (4 x 2.3 us per wave at K = 4096);
-  // now it waits the L2 round trip of its activations.
+  // where the 64 staging registers are free, instead of in front of them -- that makes room for a second stage of
+  // the weight ring (with one stage the next tile's weights can only be requested after the tile's last MFMA and are
+  // needed right away).  Measured level with the one-stage form (64-row gate/up pair 24.4 against 24.6 us): a wave
+  // waits a memory round trip per K tile either way, for its weights there and for its activations here; both
+  // prefetches together need 188 bytes of scratch per lane.
   auto consume = [&](int i, int tnext) {
     store_x();
     if (!XLATE)
