@@ -752,8 +752,12 @@ big_mxfp4_kernel(const BigParams P) {
 // What bounds int8 at this size is operand delivery and the fold, not the
 // MFMA: weights are 4x the bytes of MXFP4 per MAC, the MFMA runs at twice the
 // bf16 rate, and every block's int32 sums have to be converted, scaled by
-// sa[m] * sw[n] and added to the fp32 sums (3 vector instructions per output
-// and block, 3/4 of the MFMA time).  So:
+// sa[m] * sw[n] and added to the fp32 sums: 3 vector instructions per output
+// and block, 3 per MFMA.  Measured on this part, an int8 MFMA holds its SIMD's
+// vector issue for about 8 cycles and any other vector instruction for 4,
+// whichever wave they come from (16.5 / 17.5 / 18 / 21.5 / 25.5 cycles per MFMA
+// with 0 / 1 / 2 / 3 / 4 independent fp32 instructions behind each), so the
+// fold alone caps the MFMA busy fraction near 0.73.  So:
 //   * BOTH operands go from global memory straight into LDS (no staging
 //     registers, nothing for the compiler to wait on before the barrier) and
 //     every weight tile is fetched once per workgroup instead of once per wave
