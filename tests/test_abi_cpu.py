@@ -305,3 +305,16 @@ def test_cache_lengths_after_graph_replayed_steps():
     k, v = cache.update(one, one, 2)
     assert k.shape[2] == 10 and cache.get_seq_length(2) == 10 and cache.get_seq_length(1) == 9
     assert float(k[0, 0, 9, 0]) == 1.0 and float(k[0, 0, 8, 0]) == 0.0
+
+
+def test_qwen2_front_end_surface():
+    """The Qwen2 front-end mirrors the reference module's names (fused_qwen2_infer.py:45-238) and checks its
+    parameter list without touching a GPU."""
+    from tpp_pytorch_extension.llm import fused_qwen2_infer as Q
+    from tpp_pytorch_extension.llm import fused_llama_infer as F
+    from tpp_pytorch_extension._lib import TppxError
+    for name in ("Qwen2DecoderLayer", "FixQwen2DecoderLayer", "OptimizeModelForQwen2", "Qwen2Model_forward", "TppCache"):
+        assert hasattr(Q, name), name
+    assert issubclass(Q.Qwen2DecoderLayer, F.LlamaDecoderLayer)
+    with pytest.raises(TppxError):
+        Q.Qwen2DecoderLayer([None] * 10, 0, 1e-6, 128, 64, 128)  # the Llama list: three biases short

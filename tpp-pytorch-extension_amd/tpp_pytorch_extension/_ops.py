@@ -873,8 +873,15 @@ def _qkv_one_gemm(L, input, x, M, K, weights, biases, norm):
     qn, sn = _qkv_cat(weights)
     bias = None
     if any(b is not None and b.numel() for b in biases[:n]):
-        bias = torch.cat([(_prep_bias(b, w, x.device) if b is not None and b.numel()
-                           else torch.zeros(w, dtype=torch.bfloat16, device=x.device)) for b, w in zip(biases, widths)])
+        # the projections' biases side by side, built once per set of bias tensors and kept on the first weight
+        key = tuple((id(b), b.data_ptr(), b._version) if b is not None and b.numel() else None for b in biases[:n])
+        have = getattr(weights[0], "_tppx_qkv_bias", None)
+        if have is None or have[0] != key:
+            have = (key, torch.cat([(_prep_bias(b, w, x.device) if b is not None and b.numel()
+                                     else torch.zeros(w, dtype=torch.bfloat16, device=x.device))
+                                    for b, w in zip(biases, widths)]))
+            weights[0]._tppx_qkv_bias = have
+        bias = have[1]
     buf = torch.empty(M * N, dtype=torch.bfloat16, device=x.device)
     gamma = sums = None
     eps = 0.0

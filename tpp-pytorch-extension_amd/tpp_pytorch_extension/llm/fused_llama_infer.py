@@ -227,9 +227,13 @@ class LlamaDecoderLayer:
     with params = [ln_in gamma, Wq, Wk, Wv, Wo, ln_post gamma, Wg, Wu, Wd, embed_positions]
     (fused_llm_infer.cpp:1096-1110); the linears are quantized tensors of this package."""
 
-    def __init__(self, params, layer_idx, eps, H, max_positions, rotary_dim):
+    def _take_params(self, params):
         (self.t_Gi, self.t_Wq, self.t_Wk, self.t_Wv, self.t_Wp, self.t_Gpa,
          self.t_Wg, self.t_Wu, self.t_Wd, self.t_EP) = params
+        self.t_Bq = self.t_Bk = self.t_Bv = None
+
+    def __init__(self, params, layer_idx, eps, H, max_positions, rotary_dim):
+        self._take_params(params)
         self.layer_idx, self.eps, self.H = int(layer_idx), float(eps), int(H)
         self.max_positions, self.rotary_dim = int(max_positions), int(rotary_dim)
         # fused_llm_infer.cpp:1112-1162: quantized weights serve every pass; unquantized ones are quantized here
@@ -291,7 +295,8 @@ class LlamaDecoderLayer:
         sums_out = cache._sums[1] if _ops.takes_row_sums(Wd, M) else None
         sums_in = cache._sums[1] if cache._sums_of is t_HS else None
         # input RMSNorm + q/k/v GEMMs
-        q, k, v = _ops.qkv_gemm(t_HS, [Wq, Wk, Wv], [empty] * 3, norm=(self.t_Gi, self.eps, sums_in))
+        q, k, v = _ops.qkv_gemm(t_HS, [Wq, Wk, Wv], [self.t_Bq, self.t_Bk, self.t_Bv],
+                                norm=(self.t_Gi, self.eps, sums_in))
         kc, vc = cache._ensure(self.layer_idx, B, self.Nkv, self.H, t_HS.device)
         ws = _lib.workspace(t_HS)
         mask_ptr = t_am.data_ptr() if t_am is not None and t_am.numel() else None
