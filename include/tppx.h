@@ -446,6 +446,34 @@ int tppx_rotary_kv_append_llama(void* q, void* k, const void* v,
                                 int64_t HR, int64_t B_pos, int64_t Smax,
                                 tppx_stream_t stream);
 
+/* Replaces lyr_norm / LayerNormFwdTPP (src/csrc/llm/fused_llm_infer.cpp:254-306,
+ * src/csrc/xsmm_functors.h:4749-4786), the normalisation of GPTJBlock and
+ * OPTDecoderLayer: m = mean(x), v = max(mean(x^2) - m^2, 0), s = 1/sqrt(v + eps),
+ * y = bf16((x * s - s * m) * gamma + beta); x, y bf16 [rows][K] (K % 8 == 0),
+ * gamma and beta both f32 or both bf16 [K] (TPPX_DT_*). */
+int tppx_layer_norm(const void* x, const void* gamma, const void* beta,
+                    int param_dtype, void* y, int64_t rows, int64_t K, float eps,
+                    tppx_stream_t stream);
+
+/* Replaces apply_rotary_pos_emb_gptj (src/csrc/llm/fused_llm_infer.cpp:150-205):
+ * in place on t bf16 [B][S][N][H], pairs (h, h + 1) for h < HR; emb_pos f32
+ * [MP][HR] = sin | cos (sin of pair h/2 at [p][h/2], cos at [p][HR/2 + h/2]);
+ * pos i64 [B_pos][S]; positions >= MP are left untouched. */
+int tppx_rotary_gptj(void* t, const void* emb_pos, const void* pos, int64_t B,
+                     int64_t S, int64_t N, int64_t H, int64_t MP, int64_t HR,
+                     int64_t B_pos, tppx_stream_t stream);
+
+/* The two rotary calls of GPTJBlock::_forward (fused_llm_infer.cpp:784-785) and
+ * LayerCache::update (src/csrc/llm/attn.h:198-222) in one launch: as
+ * tppx_rotary_kv_append_llama with the GPT-J pairing and table. */
+int tppx_rotary_kv_append_gptj(void* q, void* k, const void* v,
+                               const void* emb_pos, const void* pos,
+                               void* kcache, void* vcache,
+                               const void* offset_dev, int64_t B, int64_t S,
+                               int64_t Nq, int64_t Nkv, int64_t H, int64_t MP,
+                               int64_t HR, int64_t B_pos, int64_t Smax,
+                               tppx_stream_t stream);
+
 /* Replaces attn<T> (src/csrc/llm/attn.cpp:781-955) for one query token per
  * sequence: q bf16 [B][Nq][128], cache bf16 [B][Nkv][Smax][128], additive mask
  * bf16 [B][mask_ld] or NULL; valid keys = *kv_len_dev (device i32) + kv_len_add

@@ -772,6 +772,45 @@ def rms_norm(x_bf16, gamma_f32, eps):
     return f32_to_bf16(out.astype(np.float32))
 
 
+def layer_norm(x_bf16, gamma_f32, beta_f32, eps):
+    """LayerNormFwdTPP::ref (src/csrc/xsmm_functors.h:4786-4819, called per row by lyr_norm,
+    src/csrc/llm/fused_llm_infer.cpp:254-282): m = mean(x); v = max(mean(x^2) - m^2, 0); s = 1/sqrt(v + eps);
+    b = -s*m; out = bf16((x*s + b)*gamma + beta), all in fp32.  Returns bf16 bit patterns."""
+    x = bf16_to_f32(_c(x_bf16, np.uint16)).astype(np.float32)
+    g = np.asarray(gamma_f32, np.float32)
+    bt = np.asarray(beta_f32, np.float32)
+    c = np.float32(1.0 / x.shape[-1])
+    m = x.sum(-1, dtype=np.float32) * c
+    v = (x * x).sum(-1, dtype=np.float32) * c
+    v = np.maximum(v - m * m, np.float32(0.0)).astype(np.float32)
+    s = (np.float32(1.0) / np.sqrt(v + np.float32(eps), dtype=np.float32)).astype(np.float32)
+    b = (np.float32(-1.0) * s * m).astype(np.float32)
+    out = ((x * s[..., None] + b[..., None]).astype(np.float32) * g).astype(np.float32) + bt
+    return f32_to_bf16(out.astype(np.float32))
+
+
+def rotary_gptj(t_bf16, emb_pos, pos, N, H):
+    """apply_rotary_pos_emb_gptj (src/csrc/llm/fused_llm_infer.cpp:150-205): t [B][S][N*H] bf16 bits, emb_pos f32
+    [MP][HR] = sin | cos, pos i64 [B_pos][S]; pairs (h, h+1) for h < HR with sin = emb[p][h/2], cos = emb[p][HR/2 + h/2];
+    out0 = in0*cos - in1*sin, out1 = in1*cos + in0*sin; positions >= MP untouched."""
+    t = bf16_to_f32(_c(t_bf16, np.uint16)).copy()
+    B, S = t.shape[0], t.shape[1]
+    t = t.reshape(B, S, N, H)
+    emb_pos = np.asarray(emb_pos, np.float32)
+    MP, HR = emb_pos.shape
+    coff = HR // 2
+    for b in range(B):
+        for s in range(S):
+            p = int(pos[0 if pos.shape[0] == 1 else b][s])
+            if p >= MP:
+                continue
+            sin, cos = emb_pos[p][:coff], emb_pos[p][coff:HR]
+            in0, in1 = t[b, s, :, 0:HR:2].copy(), t[b, s, :, 1:HR:2].copy()
+            t[b, s, :, 0:HR:2] = _bf16_round_f32(in0 * cos - in1 * sin)
+            t[b, s, :, 1:HR:2] = _bf16_round_f32(in1 * cos + in0 * sin)
+    return f32_to_bf16(t.reshape(B, S, N * H))
+
+
 def rotary_llama(t_bf16, emb_pos, pos, N, H):
     """apply_rotary_pos_emb_llama (src/csrc/llm/fused_llm_infer.cpp:207-253): t [B][S][N*H] bf16 bits,
     emb_pos f32 [2][MP][HR] (cos, sin), pos i64 [B_pos][S]; pairs (h2, HR/2 + h2); positions >= MP untouched."""

@@ -318,3 +318,22 @@ def test_qwen2_front_end_surface():
     assert issubclass(Q.Qwen2DecoderLayer, F.LlamaDecoderLayer)
     with pytest.raises(TppxError):
         Q.Qwen2DecoderLayer([None] * 10, 0, 1e-6, 128, 64, 128)  # the Llama list: three biases short
+
+
+def test_gptj_and_opt_front_end_surface():
+    """The GPT-J and OPT front-ends mirror the reference modules' names (fused_gptj_infer.py:46-193,
+    fused_opt_infer.py:45-203) and check their parameter lists without touching a GPU."""
+    from tpp_pytorch_extension.llm import fused_gptj_infer as G
+    from tpp_pytorch_extension.llm import fused_opt_infer as P
+    from tpp_pytorch_extension._lib import TppxError
+    for name in ("GPTJBlock", "FixGPTJBlock", "OptimizeModelForGPTJ", "GPTJModel_forward", "create_sinusoidal_positions"):
+        assert hasattr(G, name), name
+    for name in ("OPTDecoderLayer", "FixOPTDecoderLayer", "OptimizeModelForOPT", "OPTDecoder_forward"):
+        assert hasattr(P, name), name
+    with pytest.raises(TppxError):
+        G.GPTJBlock([None] * 10, 0, 1e-5, 256, 2048, 64)
+    with pytest.raises(TppxError):
+        P.OPTDecoderLayer([None] * 11, 0, 1e-5, 1e-5, 64, True)
+    t = G.create_sinusoidal_positions(8, 4)  # sin | cos of position * 10000^(-2i/dim)
+    assert t.shape == (8, 4) and torch.allclose(t[0], torch.tensor([0.0, 0.0, 1.0, 1.0]))
+    assert torch.allclose(t[3, :2], torch.sin(torch.tensor([3.0, 0.03]))) and torch.allclose(t[3, 2:], torch.cos(torch.tensor([3.0, 0.03])))

@@ -380,6 +380,73 @@ def test_oracle_rotary_is_a_rotation_and_matches_rotate_half():
     assert np.allclose((a ** 2).sum(3), (b ** 2).sum(3), rtol=2e-2, atol=1e-3)
 
 
+def test_oracle_layer_norm_against_torch_and_closed_forms():
+    """The LayerNorm restatement against torch's own layer_norm (an independent library routine, evaluated in
+    fp64) and against what the formula fixes: a constant row gives beta exactly (v = 0, x*s + b = 0), a row of
+    +-a has mean 0 and variance a^2, and swapping gamma with beta or dropping the mean changes the result."""
+    import torch
+    g = torch.Generator().manual_seed(13)
+    x = (torch.randn(5, 384, generator=g) * 2 + 0.7).to(torch.bfloat16)
+    w = torch.rand(384, generator=g) + 0.5
+    b = torch.randn(384, generator=g) * 0.3
+    got = O.bf16_to_f32(O.layer_norm(x.view(torch.int16).numpy().view(np.uint16), w.numpy(), b.numpy(), 1e-5))
+    ref64 = torch.nn.functional.layer_norm(x.double(), (384,), w.double(), b.double(), 1e-5)
+    ref = ref64.float().to(torch.bfloat16).float().numpy()
+    assert np.abs(got - ref).max() <= 2.0 ** -7 * np.abs(ref).max()
+    assert (got != ref).mean() < 0.02  # E[x^2] - m^2 in fp32 against the two-pass fp64 variance: last-bit differences
+    # without the mean (RMSNorm) or with gamma and beta swapped the answer is far off
+    nomean = ((x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + 1e-5)) * w + b).float().numpy()
+    assert np.abs(got - nomean).max() > 0.1
+    swapped = torch.nn.functional.layer_norm(x.double(), (384,), b.double(), w.double(), 1e-5).float().numpy()
+    assert np.abs(got - swapped).max() > 0.1
+    # closed forms
+    c = np.full((1, 64), 3.0, np.float32)
+    beta = np.linspace(-1, 1, 64).astype(np.float32)
+    const = O.bf16_to_f32(O.layer_norm(O.f32_to_bf16(c), np.full(64, 7.0, np.float32), beta, 1e-5))
+    assert np.array_equal(const[0], O.bf16_to_f32(O.f32_to_bf16(beta)))
+    pm = np.tile(np.array([2.0, -2.0], np.float32), 32)[None]
+    out = O.bf16_to_f32(O.layer_norm(O.f32_to_bf16(pm), np.ones(64, np.float32), np.zeros(64, np.float32), 1e-12))
+    assert np.allclose(out, np.sign(pm), atol=2.0 ** -8)
+
+
+def test_oracle_rotary_gptj_is_a_rotation_of_adjacent_pairs():
+    """The GPT-J rotary restatement against the Hugging Face formulation (x*cos + rotate_every_two(x)*sin with the
+    sin | cos table of create_sinusoidal_positions, written out here in torch) and against closed forms: position 0
+    is the identity, dims >= rotary_dim are untouched, adjacent pairs keep their norm, and (x, 0) at angle theta
+    becomes (x cos theta, x sin theta) -- a swapped table half or a wrong sign fails one of them."""
+    import torch
+    B, S, N, H, HR, MP = 2, 3, 2, 32, 16, 16
+    g = torch.Generator().manual_seed(14)
+    t = torch.randn(B, S, N * H, generator=g).to(torch.bfloat16)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, HR, 2).float() / HR))
+    fr = torch.outer(torch.arange(MP).float(), inv)
+    emb = torch.cat((fr.sin(), fr.cos()), dim=1)  # [MP][HR]
+    pos = torch.tensor([[0, 5, 15], [7, 16, 2]])  # 16 is out of range
+    got = O.bf16_to_f32(O.rotary_gptj(t.view(torch.int16).numpy().view(np.uint16), emb.numpy(), pos.numpy(), N, H))
+    x = t.float().view(B, S, N, H)
+    p = pos.clamp(max=MP - 1)
+    sin = torch.repeat_interleave(emb[p][:, :, None, :HR // 2], 2, dim=-1)
+    cos = torch.repeat_interleave(emb[p][:, :, None, HR // 2:], 2, dim=-1)
+    xr = x[..., :HR]
+    r2 = torch.stack((-xr[..., 1::2], xr[..., ::2]), dim=-1).flatten(-2)  # rotate_every_two
+    ref = x.clone()
+    ref[..., :HR] = xr * cos + r2 * sin
+    ref[1, 1] = x[1, 1]
+    ref = ref.to(torch.bfloat16).float().view(B, S, N * H).numpy()
+    assert np.abs(got - ref).max() <= 2.0 ** -7 * np.abs(ref).max()
+    tf = t.float().numpy()
+    assert np.array_equal(got[0, 0], tf[0, 0])                                     # position 0
+    assert np.array_equal(got.reshape(B, S, N, H)[..., HR:], tf.reshape(B, S, N, H)[..., HR:])  # pass-through dims
+    a = tf.reshape(B, S, N, H)[..., :HR].reshape(B, S, N, HR // 2, 2)
+    b = got.reshape(B, S, N, H)[..., :HR].reshape(B, S, N, HR // 2, 2)
+    assert np.allclose((a ** 2).sum(-1), (b ** 2).sum(-1), rtol=2e-2, atol=1e-3)
+    one = np.zeros((1, 1, H), np.float32)
+    one[0, 0, 0] = 1.0                                                             # pair 0 = (1, 0)
+    e = O.bf16_to_f32(O.rotary_gptj(O.f32_to_bf16(one), emb.numpy(), np.array([[3]]), 1, H))
+    theta = 3.0 * float(inv[0])
+    assert abs(e[0, 0, 0] - np.cos(theta)) < 2.0 ** -8 and abs(e[0, 0, 1] - np.sin(theta)) < 2.0 ** -8
+
+
 def test_oracle_attn_decode_against_softmax_and_special_cases():
     import torch
     B, Nq, Nkv, L, H = 2, 4, 2, 19, 16

@@ -96,6 +96,68 @@ rms_norm_kernel(const uint16_t* __restrict__ x, const void* __restrict__ gamma, 
 }
 
 // ---------------------------------------------------------------------------
+// LayerNorm (lyr_norm, fused_llm_infer.cpp:254-306; LayerNormFwdTPP,
+// xsmm_functors.h:4749-4786): m = mean(x), v = max(mean(x^2) - m^2, 0),
+// s = 1 / sqrt(v + eps), y = bf16( (x * s - s * m) * gamma + beta ), fp32 inside.
+// One workgroup of 256 threads per row; K a multiple of 8.
+// ---------------------------------------------------------------------------
+template <bool PARAMS_F32>
+__device__ __forceinline__ void load8_param(const void* p, int i, float (&g)[8]) {
+  if (PARAMS_F32) {
+    const float4* gp = reinterpret_cast<const float4*>(p) + 2 * i;
+    const float4 g0 = gp[0], g1 = gp[1];
+    g[0] = g0.x; g[1] = g0.y; g[2] = g0.z; g[3] = g0.w;
+    g[4] = g1.x; g[5] = g1.y; g[6] = g1.z; g[7] = g1.w;
+  } else {
+    unpack8(reinterpret_cast<const uint4*>(p)[i], g);
+  }
+}
+
+template <bool PARAMS_F32>
+__global__ void __launch_bounds__(256)
+layer_norm_kernel(const uint16_t* __restrict__ x, const void* __restrict__ gamma, const void* __restrict__ beta,
+                  uint16_t* __restrict__ y, int K, float eps) {
+  __shared__ float red[2][4];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const uint4* xr = reinterpret_cast<const uint4*>(x + (int64_t)row * K);
+  uint4* yr = reinterpret_cast<uint4*>(y + (int64_t)row * K);
+  const int nchunk = K >> 3;
+  float sm = 0.f, ss = 0.f;
+  for (int i = tid; i < nchunk; i += 256) {
+    float f[8];
+    unpack8(xr[i], f);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      sm += f[e];
+      ss = fmaf(f[e], f[e], ss);
+    }
+  }
+  sm = wave_sum(sm);
+  ss = wave_sum(ss);
+  if ((tid & 63) == 0) {
+    red[0][tid >> 6] = sm;
+    red[1][tid >> 6] = ss;
+  }
+  __syncthreads();
+  const float c = 1.0f / (float)K;
+  const float m = ((red[0][0] + red[0][1]) + (red[0][2] + red[0][3])) * c;
+  float v = ((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) * c;
+  v = fmaxf(v - m * m, 0.0f);
+  const float s = 1.0f / sqrtf(v + eps);
+  const float b = -1.0f * s * m;
+  for (int i = tid; i < nchunk; i += 256) {
+    float f[8], g[8], bt[8];
+    unpack8(xr[i], f); // second read hits L2/L1
+    load8_param<PARAMS_F32>(gamma, i, g);
+    load8_param<PARAMS_F32>(beta, i, bt);
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      f[e] = (f[e] * s + b) * g[e] + bt[e];
+    yr[i] = pack8(f);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Llama rotary embedding, in place on t [B][S][N][H] (rotate-half pairs
 // (h2, HR/2 + h2)), cos/sin table f32 [2][MP][HR], positions i64 [B_pos][S].
 // Optionally the rotated key rows and the value rows are also written into
@@ -113,6 +175,7 @@ struct RotaryParams {
   const int64_t* pos;  // [B_pos][S]
   const int32_t* offset; // device scalar: cache length before this append
   int B, S, Nq, Nkv, H, MP, HR, B_pos, Smax;
+  int gptj;            // 1: GPT-J pairs (h, h + 1) and a sin | cos table f32 [MP][HR] (fused_llm_infer.cpp:150-205)
 };
 
 __global__ void __launch_bounds__(256)
@@ -145,7 +208,21 @@ rotary_append_kernel(const RotaryParams p) {
   const int coff = p.HR >> 1;
   const int h0 = c * 8;
   const int64_t pp = p.pos[(int64_t)(p.B_pos == 1 ? 0 : b) * p.S + s];
-  if (p.emb && h0 < p.HR && pp >= 0 && pp < p.MP) { // positions outside the table are left unrotated
+  if (p.gptj) {
+    if (p.emb && h0 < p.HR && pp >= 0 && pp < p.MP) {
+      // a chunk of 8 holds four whole pairs (h, h + 1); sin at [p][h / 2], cos at [p][HR / 2 + h / 2]
+      float a[8], r[8];
+      unpack8(w, a);
+      const float* sn = p.emb + pp * p.HR + (h0 >> 1);
+      const float* cs = sn + coff;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        r[2 * e] = a[2 * e] * cs[e] - a[2 * e + 1] * sn[e];
+        r[2 * e + 1] = a[2 * e + 1] * cs[e] + a[2 * e] * sn[e];
+      }
+      w = pack8(r);
+    }
+  } else if (p.emb && h0 < p.HR && pp >= 0 && pp < p.MP) { // positions outside the table are left unrotated
     // this chunk holds first halves (h0 < HR/2) or second halves of rotation pairs
     const bool first = h0 < coff;
     const int h2 = first ? h0 : h0 - coff;
@@ -1057,6 +1134,24 @@ extern "C" int tppx_rms_norm(const void* x, const void* gamma, int gamma_dtype, 
   return check_hip(hipGetLastError(), "tppx_rms_norm");
 }
 
+extern "C" int tppx_layer_norm(const void* x, const void* gamma, const void* beta, int param_dtype, void* y,
+                               int64_t rows, int64_t K, float eps, tppx_stream_t stream) {
+  TPPX_REQUIRE(x && gamma && beta && y, TPPX_EINVAL, "tppx_layer_norm: null pointer");
+  TPPX_REQUIRE(aligned16(x) && aligned16(gamma) && aligned16(beta) && aligned16(y), TPPX_EINVAL,
+               "tppx_layer_norm: pointer not 16-byte aligned");
+  TPPX_REQUIRE(param_dtype == TPPX_DT_F32 || param_dtype == TPPX_DT_BF16, TPPX_EINVAL,
+               "tppx_layer_norm: unknown gamma / beta dtype %d", param_dtype);
+  TPPX_REQUIRE(rows > 0 && rows < ((int64_t)1 << 31) && K > 0 && K % 8 == 0 && K < (1 << 24), TPPX_ESHAPE,
+               "tppx_layer_norm: bad shape rows=%ld K=%ld (K must be a multiple of 8)", (long)rows, (long)K);
+  if (param_dtype == TPPX_DT_F32)
+    layer_norm_kernel<true><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
+        (const uint16_t*)x, gamma, beta, (uint16_t*)y, (int)K, eps);
+  else
+    layer_norm_kernel<false><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
+        (const uint16_t*)x, gamma, beta, (uint16_t*)y, (int)K, eps);
+  return check_hip(hipGetLastError(), "tppx_layer_norm");
+}
+
 static int rotary_common(const char* who, RotaryParams& p, hipStream_t stream) {
   TPPX_REQUIRE(p.B > 0 && p.S > 0 && p.H >= 16 && p.H <= 512 && (p.H & (p.H - 1)) == 0, TPPX_ESHAPE,
                "%s: bad shape B=%d S=%d H=%d (head size must be a power of two in 16..512)", who, p.B, p.S, p.H);
@@ -1101,6 +1196,41 @@ extern "C" int tppx_rotary_kv_append_llama(void* q, void* k, const void* v, cons
   p.emb = (const float*)emb_pos; p.pos = (const int64_t*)pos; p.offset = (const int32_t*)offset_dev;
   p.B = (int)B; p.S = (int)S; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.H = (int)H; p.MP = (int)MP; p.HR = (int)HR;
   p.B_pos = (int)B_pos; p.Smax = (int)Smax;
+  return rotary_common(who, p, (hipStream_t)stream);
+}
+
+extern "C" int tppx_rotary_gptj(void* t, const void* emb_pos, const void* pos, int64_t B, int64_t S, int64_t N,
+                                int64_t H, int64_t MP, int64_t HR, int64_t B_pos, tppx_stream_t stream) {
+  TPPX_REQUIRE(t && emb_pos && pos, TPPX_EINVAL, "tppx_rotary_gptj: null pointer");
+  TPPX_REQUIRE(aligned16(t), TPPX_EINVAL, "tppx_rotary_gptj: pointer not 16-byte aligned");
+  TPPX_REQUIRE(N > 0, TPPX_ESHAPE, "tppx_rotary_gptj: N=%ld", (long)N);
+  RotaryParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = (uint16_t*)t;
+  p.emb = (const float*)emb_pos;
+  p.pos = (const int64_t*)pos;
+  p.B = (int)B; p.S = (int)S; p.Nq = (int)N; p.H = (int)H; p.MP = (int)MP; p.HR = (int)HR; p.B_pos = (int)B_pos;
+  p.gptj = 1;
+  return rotary_common("tppx_rotary_gptj", p, (hipStream_t)stream);
+}
+
+extern "C" int tppx_rotary_kv_append_gptj(void* q, void* k, const void* v, const void* emb_pos, const void* pos,
+                                          void* kcache, void* vcache, const void* offset_dev, int64_t B, int64_t S,
+                                          int64_t Nq, int64_t Nkv, int64_t H, int64_t MP, int64_t HR, int64_t B_pos,
+                                          int64_t Smax, tppx_stream_t stream) {
+  const char* who = "tppx_rotary_kv_append_gptj";
+  TPPX_REQUIRE(k && v && kcache && vcache && offset_dev && pos && emb_pos, TPPX_EINVAL, "%s: null pointer", who);
+  TPPX_REQUIRE(aligned16(k) && aligned16(v) && aligned16(kcache) && aligned16(vcache) && (!q || aligned16(q)),
+               TPPX_EINVAL, "%s: pointer not 16-byte aligned", who);
+  TPPX_REQUIRE(Nkv > 0 && Smax > 0 && (!q || Nq > 0), TPPX_ESHAPE, "%s: bad head counts / capacity", who);
+  RotaryParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = (uint16_t*)q; p.k = (uint16_t*)k; p.v = (const uint16_t*)v;
+  p.kc = (uint16_t*)kcache; p.vc = (uint16_t*)vcache;
+  p.emb = (const float*)emb_pos; p.pos = (const int64_t*)pos; p.offset = (const int32_t*)offset_dev;
+  p.B = (int)B; p.S = (int)S; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.H = (int)H; p.MP = (int)MP; p.HR = (int)HR;
+  p.B_pos = (int)B_pos; p.Smax = (int)Smax;
+  p.gptj = 1;
   return rotary_common(who, p, (hipStream_t)stream);
 }
 

@@ -78,6 +78,10 @@ SIGNATURES = {
     "tppx_normsq_multi_linear_mxfp4": [_vp, _vp, _vp, ctypes.c_float, ctypes.POINTER(Seg), _i32, _i64, _i64, _i32, _vp],
     "tppx_normsq_swiglu_mxfp4": [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
     "tppx_rms_norm": [_vp, _vp, _i32, _vp, _i64, _i64, ctypes.c_float, _vp],
+    "tppx_layer_norm": [_vp, _vp, _vp, _i32, _vp, _i64, _i64, ctypes.c_float, _vp],
+    "tppx_rotary_gptj": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
+    "tppx_rotary_kv_append_gptj": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                   _i64, _i64, _vp],
     "tppx_rotary_llama": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     "tppx_rotary_kv_append_llama": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                     _i64, _i64, _vp],

@@ -787,6 +787,26 @@ def rms_norm(t_in, t_wt, eps):
     return y
 
 
+def layer_norm(t_in, t_gamma, t_beta, eps):
+    """lyr_norm (src/csrc/llm/fused_llm_infer.cpp:254-306): bf16 in/out, gamma and beta both fp32 or both bf16."""
+    L = _lib.lib()
+    if not t_in.is_cuda or t_in.dtype != torch.bfloat16:
+        raise TppxError(_lib.EINVAL, "lyr_norm: input must be a bfloat16 tensor on the GPU")
+    x = t_in.contiguous()
+    K = x.shape[-1]
+    if t_gamma.dtype not in (torch.float32, torch.bfloat16) or t_gamma.numel() != K or not t_gamma.is_cuda:
+        raise TppxError(_lib.EINVAL, "lyr_norm: gamma must be fp32 or bf16 [K] on the GPU")
+    if t_beta.dtype != t_gamma.dtype or t_beta.numel() != K or not t_beta.is_cuda:
+        raise TppxError(_lib.EINVAL, "lyr_norm: beta must have gamma's dtype and size")
+    y = torch.empty_like(x)
+    rows = x.numel() // K
+    if rows:
+        _lib.check(L.tppx_layer_norm(x.data_ptr(), t_gamma.contiguous().data_ptr(), t_beta.contiguous().data_ptr(),
+                                     0 if t_gamma.dtype == torch.float32 else 1, y.data_ptr(), rows, K, float(eps),
+                                     _lib.stream_of(x)))
+    return y
+
+
 # RMSNorm inside the GEMM launch (tppx_norm_multi_linear_mxfp4 / tppx_norm_swiglu_mxfp4).  Off by default: on MI355X
 # the fused launch measured slower than the normalisation kernel followed by the plain launch (every workgroup
 # repeats the row reduction behind a barrier, and the extra registers spill); TPPX_FUSE_NORM=1 turns it on.

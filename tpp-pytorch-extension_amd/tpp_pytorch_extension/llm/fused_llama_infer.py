@@ -222,10 +222,95 @@ class TppCache:
         self.capacity = new_capacity
 
 
-class LlamaDecoderLayer:
+def rotate_append_attend(q, k, v, t_am, t_pid, cache, layer_idx, B, S, Nq, Nkv, H, t_EP, style):
+    """What every decoder block of the reference does between its q/k/v GEMMs and its output projection
+    (fused_llm_infer.cpp:784-789, 1025-1027, 1252-1257): rotary embedding on q and k in place (style "llama":
+    rotate-half with a [2][MP][HR] cos / sin table; "gptj": adjacent pairs with a [MP][HR] sin | cos table; None:
+    no rotation, OPT), append of the S new keys and values at the cache length (LayerCache::update, attn.h:198-222),
+    attention over the cached and the new keys (attn<T>, attn.cpp:781-955).  Returns the context [B][S][Nq*H]."""
+    L = _lib.lib()
+    st = _lib.stream_of(q)
+    kc, vc = cache._ensure(layer_idx, B, Nkv, H, q.device)
+    ws = _lib.workspace(q)
+    mask_ptr = t_am.data_ptr() if t_am is not None and t_am.numel() else None
+    mask_ld = t_am.shape[-1] if mask_ptr else 0
+    if style == "gptj":
+        _lib.check(L.tppx_rotary_kv_append_gptj(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), t_EP.data_ptr(), t_pid.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+            cache.seq_len_dev.data_ptr(), B, S, Nq, Nkv, H, t_EP.shape[0], t_EP.shape[1], t_pid.shape[0],
+            cache.capacity, st))
+    else:
+        emb = t_EP.data_ptr() if style == "llama" else None  # no table: append only, q is not touched
+        _lib.check(L.tppx_rotary_kv_append_llama(
+            q.data_ptr() if emb else None, k.data_ptr(), v.data_ptr(), emb, t_pid.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+            cache.seq_len_dev.data_ptr(), B, S, Nq, Nkv, H, t_EP.shape[1] if emb else 1, t_EP.shape[2] if emb else H,
+            t_pid.shape[0], cache.capacity, st))
+    ctx = torch.empty_like(q)
+    if S == 1:
+        _lib.check(L.tppx_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
+                                      cache.seq_len_dev.data_ptr(), 1, ctx.data_ptr(), B, Nq, Nkv, H, cache.capacity,
+                                      ws.data_ptr(), ws.numel(), st))
+    else:
+        _lib.check(L.tppx_attn_prefill(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
+                                       cache.get_seq_length(), ctx.data_ptr(), B, S, Nq, Nkv, H, cache.capacity, st))
+    return ctx
+
+
+def check_layer_inputs(who, t_HS, t_pid, cache):
+    """Shape checks shared by the decoder blocks: room in the cache for the S new keys, int64 positions [B or 1][S]."""
+    B, S, _ = t_HS.shape
+    if cache.get_seq_length() + S > cache.capacity:
+        raise TppxError(_lib.ESHAPE, f"{who}: {cache.get_seq_length()} cached + {S} new keys exceed "
+                                     f"the cache capacity {cache.capacity}")
+    if t_pid.dim() != 2 or t_pid.shape[1] != S or t_pid.shape[0] not in (1, B) or t_pid.dtype != torch.int64:
+        raise TppxError(_lib.ESHAPE, f"{who}: position_ids must be int64 [B or 1][S={S}], got "
+                                     f"{tuple(t_pid.shape)} {t_pid.dtype}")
+
+
+class FormatSwitches:
+    """The weight-format handling every decoder block of the reference repeats in its constructor and at the top of
+    its forward (e.g. fused_llm_infer.cpp:650-738, 741-758 for GPT-J): quantized weights serve every pass;
+    unquantized ones are quantized for the decode steps under USE_MXFP4 / USE_QINT8 / USE_QINT2 after the
+    first-token copies were taken; passes of FT_OPT_SIZE or more tokens run on those copies when
+    TPP_CACHE_REMAPPED_WEIGHTS is on.  `_weight_names` lists the attributes holding the linears' weights."""
+
+    _weight_names = ()
+
+    def _setup_formats(self):
+        self.first_token_remapped = False
+        self._first = None
+        names = self._weight_names
+        if isinstance(getattr(self, names[0]), _ops.QTensor):
+            self._first = tuple(getattr(self, n) for n in names)
+            self.first_token_remapped = True
+        else:
+            quant = (_ops.remap_and_quantize_mxfp4 if USE_MXFP4 else _ops.remap_and_quantize_qint8 if USE_QINT8
+                     else _ops.remap_and_quantize_qint2_intlv if USE_QINT2 else None)
+            if quant is not None:
+                self.remap_for_first_token()
+                for n in names:
+                    setattr(self, n, quant(getattr(self, n)))
+
+    def remap_for_first_token(self):
+        """remap_for_first_token of the reference's blocks (fused_llm_infer.cpp:726-738, 972-983, 1164-1175)."""
+        self._first = tuple(wt_tensor_for_first_token(getattr(self, n)) for n in self._weight_names)
+        self.first_token_remapped = True
+
+    def _weights_for(self, rows):
+        """check_weight_reuse + the switch to the first-token copies (fused_llm_infer.cpp:518-524, 1216-1227)."""
+        if rows >= FT_OPT_SIZE and TPP_CACHE_REMAPPED_WEIGHTS:
+            if not self.first_token_remapped:
+                self.remap_for_first_token()
+            return self._first
+        return tuple(getattr(self, n) for n in self._weight_names)
+
+
+class LlamaDecoderLayer(FormatSwitches):
     """torch.classes.tpp_llm.LlamaDecoderLayer(params, layer_idx, eps, H, max_positions, rotary_dim)
     with params = [ln_in gamma, Wq, Wk, Wv, Wo, ln_post gamma, Wg, Wu, Wd, embed_positions]
     (fused_llm_infer.cpp:1096-1110); the linears are quantized tensors of this package."""
+
+    _weight_names = ("t_Wq", "t_Wk", "t_Wv", "t_Wp", "t_Wg", "t_Wu", "t_Wd")
 
     def _take_params(self, params):
         (self.t_Gi, self.t_Wq, self.t_Wk, self.t_Wv, self.t_Wp, self.t_Gpa,
@@ -238,35 +323,9 @@ class LlamaDecoderLayer:
         self.max_positions, self.rotary_dim = int(max_positions), int(rotary_dim)
         # fused_llm_infer.cpp:1112-1162: quantized weights serve every pass; unquantized ones are quantized here
         # for the decode steps under USE_MXFP4 / USE_QINT8 / USE_QINT2, after the first-token copies were taken
-        self.first_token_remapped = False
-        self._first = None
-        names = ("t_Wq", "t_Wk", "t_Wv", "t_Wp", "t_Wg", "t_Wu", "t_Wd")
-        if isinstance(self.t_Wq, _ops.QTensor):
-            self._first = tuple(getattr(self, n) for n in names)
-            self.first_token_remapped = True
-        else:
-            quant = (_ops.remap_and_quantize_mxfp4 if USE_MXFP4 else _ops.remap_and_quantize_qint8 if USE_QINT8
-                     else _ops.remap_and_quantize_qint2_intlv if USE_QINT2 else None)
-            if quant is not None:
-                self.remap_for_first_token()
-                for n in names:
-                    setattr(self, n, quant(getattr(self, n)))
+        self._setup_formats()
         self.Nq = _ops.weight_nk(self.t_Wq)[0] // self.H
         self.Nkv = _ops.weight_nk(self.t_Wk)[0] // self.H
-
-    def remap_for_first_token(self):
-        """LlamaDecoderLayer::remap_for_first_token (fused_llm_infer.cpp:1164-1175)."""
-        self._first = tuple(wt_tensor_for_first_token(w) for w in
-                            (self.t_Wq, self.t_Wk, self.t_Wv, self.t_Wp, self.t_Wg, self.t_Wu, self.t_Wd))
-        self.first_token_remapped = True
-
-    def _weights_for(self, rows):
-        """check_weight_reuse + the switch to the first-token copies (fused_llm_infer.cpp:518-524, 1216-1227)."""
-        if rows >= FT_OPT_SIZE and TPP_CACHE_REMAPPED_WEIGHTS:
-            if not self.first_token_remapped:
-                self.remap_for_first_token()
-            return self._first
-        return (self.t_Wq, self.t_Wk, self.t_Wv, self.t_Wp, self.t_Wg, self.t_Wu, self.t_Wd)
 
     def forward(self, inputs, cache, use_cache=True):
         """inputs = [hidden [B][S][hidden], additive mask [B][keys] or empty, position_ids i64 [B or 1][S]].
@@ -276,12 +335,7 @@ class LlamaDecoderLayer:
         L = _lib.lib()
         t_HS, t_am, t_pid = inputs[0], inputs[1], inputs[2]
         B, S, hidden = t_HS.shape
-        if cache.get_seq_length() + S > cache.capacity:
-            raise TppxError(_lib.ESHAPE, f"LlamaDecoderLayer: {cache.get_seq_length()} cached + {S} new keys exceed "
-                                         f"the cache capacity {cache.capacity}")
-        if t_pid.dim() != 2 or t_pid.shape[1] != S or t_pid.shape[0] not in (1, B) or t_pid.dtype != torch.int64:
-            raise TppxError(_lib.ESHAPE, f"LlamaDecoderLayer: position_ids must be int64 [B or 1][S={S}], got "
-                                         f"{tuple(t_pid.shape)} {t_pid.dtype}")
+        check_layer_inputs(type(self).__name__, t_HS, t_pid, cache)
         st = _lib.stream_of(t_HS)
         empty = torch.empty(0, dtype=torch.bfloat16, device=t_HS.device)
         Wq, Wk, Wv, Wp, Wg, Wu, Wd = self._weights_for(B * S)
@@ -310,21 +364,8 @@ class LlamaDecoderLayer:
                 cache.seq_len_dev.data_ptr(), ctx.data_ptr(), B, self.Nq, self.Nkv, self.H, cache.capacity,
                 ws.data_ptr(), ws.numel(), st))
             return self._after_attention(ctx, t_res, empty, cache, sums_attn, sums_out, Wp, Wg, Wu, Wd)
-        # rotary on q and k + append of k, v at position seq_len (device counter), one launch
-        _lib.check(L.tppx_rotary_kv_append_llama(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), self.t_EP.data_ptr(), t_pid.data_ptr(), kc.data_ptr(),
-            vc.data_ptr(), cache.seq_len_dev.data_ptr(), B, S, self.Nq, self.Nkv, self.H, self.t_EP.shape[1],
-            self.t_EP.shape[2], t_pid.shape[0], cache.capacity, st))
-        # attention over the cached keys + the new ones
-        ctx = torch.empty_like(q)
-        if S == 1:
-            _lib.check(L.tppx_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
-                                          cache.seq_len_dev.data_ptr(), 1, ctx.data_ptr(), B, self.Nq, self.Nkv, self.H,
-                                          cache.capacity, ws.data_ptr(), ws.numel(), st))
-        else:
-            _lib.check(L.tppx_attn_prefill(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld,
-                                           cache.get_seq_length(), ctx.data_ptr(), B, S, self.Nq, self.Nkv, self.H,
-                                           cache.capacity, st))
+        ctx = rotate_append_attend(q, k, v, t_am, t_pid, cache, self.layer_idx, B, S, self.Nq, self.Nkv, self.H,
+                                   self.t_EP, "llama")
         return self._after_attention(ctx, t_res, empty, cache, sums_attn, sums_out, Wp, Wg, Wu, Wd)
 
     def _after_attention(self, ctx, t_res, empty, cache, sums_attn, sums_out, Wp, Wg, Wu, Wd):
