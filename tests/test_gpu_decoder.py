@@ -719,3 +719,35 @@ def test_cache_update_appends_and_grows():
     ref = O.attn_decode(t2bits(q), t2bits(torch.cat([k1, k2], 2)), t2bits(torch.cat([v1, v2], 2)))
     g, r = bits2f(t2bits(got)).astype(np.float64), bits2f(ref).astype(np.float64)
     assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3
+
+
+@pytest.mark.parametrize("Sq,past", [(1, 37), (9, 21), (40, 0)])
+def test_attn_entry_point_of_the_cache_module(Sq, past):
+    """_C._tpp_attn.attn (attn_wrapper, attn.cpp:957-1043): keys / values appended to a layer of the cache, then
+    attention of q [B][Nkv][Sq][R][H] over everything cached, against the oracle's functions on the same tensors."""
+    _llm()
+    from tpp_pytorch_extension._C import _tpp_attn
+    from tpp_pytorch_extension._lib import TppxError
+    B, Nkv, R, H = 2, 2, 2, 128
+    cache = _tpp_attn.TppCache(64)
+    k0, v0 = randn_bf16((B, Nkv, past, H), 1.0, 81), randn_bf16((B, Nkv, past, H), 1.0, 82)
+    if past:
+        cache.update(k0.cuda(), v0.cuda(), 3)
+    q = randn_bf16((B, Nkv, Sq, R, H), 1.0, 83)
+    k, v = randn_bf16((B, Nkv, Sq, H), 1.0, 84), randn_bf16((B, Nkv, Sq, H), 1.0, 85)
+    got = _tpp_attn.attn(q.cuda(), k.cuda(), v.cuda(), torch.Tensor(), cache, 3, True).cpu()
+    assert got.shape == q.shape and cache.get_seq_length(3) == past + Sq
+    kall = np.concatenate([t2bits(k0), t2bits(k)], axis=2)
+    vall = np.concatenate([t2bits(v0), t2bits(v)], axis=2)
+    qo = q.permute(0, 2, 1, 3, 4).reshape(B, Sq, Nkv * R, H)  # the oracle's head order: key head * R + r
+    if Sq == 1:
+        ref = O.attn_decode(t2bits(qo[:, 0]), kall, vall).reshape(B, 1, Nkv, R, H)
+    else:
+        ref = O.attn_prefill(t2bits(qo), kall, vall).reshape(B, Sq, Nkv, R, H)
+    ref = ref.transpose(0, 2, 1, 3, 4)
+    g, r = bits2f(t2bits(got)).astype(np.float64), bits2f(np.ascontiguousarray(ref)).astype(np.float64)
+    assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3
+    assert np.abs(g - r).max() <= 2.0 ** -7 * np.abs(r).max()
+    if Sq > 1:
+        with pytest.raises(TppxError):
+            _tpp_attn.attn(q.cuda(), k.cuda(), v.cuda(), torch.Tensor(), cache, 3, False)

@@ -256,6 +256,40 @@ def rotate_append_attend(q, k, v, t_am, t_pid, cache, layer_idx, B, S, Nq, Nkv, 
     return ctx
 
 
+def attn(t_QL, t_KL, t_VL, t_AM, cache, layer_idx, isCausal=True):
+    """_C._tpp_attn.attn (attn_wrapper, src/csrc/llm/attn.cpp:957-1043): append t_KL / t_VL [B][Nkv][Sq][H] to layer
+    `layer_idx` of the cache, then attention of t_QL [B][Nkv][Sq][R][H] (R = query heads per key head) over all
+    cached keys; additive mask t_AM [B][keys] or empty; returns the context in t_QL's layout.  The new tokens see
+    the older keys and, causally, each other; isCausal = False is only taken for one query token per sequence,
+    where it means the same (the prompt kernel here is causal)."""
+    L = _lib.lib()
+    if t_QL.dim() != 5 or not t_QL.is_cuda or t_QL.dtype != torch.bfloat16:
+        raise TppxError(_lib.EINVAL, "attn: t_QL must be a bfloat16 tensor [B][Nkv][Sq][R][H] on the GPU")
+    B, Nkv, Sq, R, H = t_QL.shape
+    if not isCausal and Sq != 1:
+        raise TppxError(_lib.EUNSUPPORTED, "attn: non-causal attention over several query tokens is not built")
+    if tuple(t_KL.shape) != (B, Nkv, Sq, H) or tuple(t_VL.shape) != (B, Nkv, Sq, H):
+        raise TppxError(_lib.ESHAPE, f"attn: keys / values must be [B][Nkv][Sq][H] = {(B, Nkv, Sq, H)}")
+    core = cache.get_cpp() if hasattr(cache, "get_cpp") else cache
+    core.update(_bf16_cuda(t_KL, "t_KL"), _bf16_cuda(t_VL, "t_VL"), layer_idx)
+    key_len = core.get_seq_length(layer_idx)
+    kc, vc = core.layers[layer_idx]
+    q = t_QL.permute(0, 2, 1, 3, 4).reshape(B, Sq, Nkv * R, H).contiguous()  # head index = key head * R + r
+    out = torch.empty_like(q)
+    st = _lib.stream_of(q)
+    ws = _lib.workspace(q)
+    mask = t_AM.to(torch.bfloat16).contiguous() if t_AM is not None and t_AM.numel() else None
+    mask_ptr, mask_ld = (mask.data_ptr(), mask.shape[-1]) if mask is not None else (None, 0)
+    klen = torch.full((1,), key_len, dtype=torch.int32, device=q.device)
+    if Sq == 1:
+        _lib.check(L.tppx_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld, klen.data_ptr(), 0,
+                                      out.data_ptr(), B, Nkv * R, Nkv, H, core.capacity, ws.data_ptr(), ws.numel(), st))
+    else:
+        _lib.check(L.tppx_attn_prefill(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), mask_ptr, mask_ld, key_len - Sq,
+                                       out.data_ptr(), B, Sq, Nkv * R, Nkv, H, core.capacity, st))
+    return out.view(B, Sq, Nkv, R, H).permute(0, 2, 1, 3, 4).contiguous()
+
+
 def check_layer_inputs(who, t_HS, t_pid, cache):
     """Shape checks shared by the decoder blocks: room in the cache for the S new keys, int64 positions [B or 1][S]."""
     B, S, _ = t_HS.shape
