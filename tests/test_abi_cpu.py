@@ -337,3 +337,37 @@ def test_gptj_and_opt_front_end_surface():
     t = G.create_sinusoidal_positions(8, 4)  # sin | cos of position * 10000^(-2i/dim)
     assert t.shape == (8, 4) and torch.allclose(t[0], torch.tensor([0.0, 0.0, 1.0, 1.0]))
     assert torch.allclose(t[3, :2], torch.sin(torch.tensor([3.0, 0.03]))) and torch.allclose(t[3, 2:], torch.cos(torch.tensor([3.0, 0.03])))
+
+
+def test_common_module_helpers_one_process():
+    """llm_common's process-group helpers in their one-process form, ShardLinear as pure slicing (the shards of all
+    ranks tile the weight; a row-parallel split sums back to the whole linear), BlockedLayerNorm on the CPU."""
+    import copy
+    from tpp_pytorch_extension.llm import llm_common as C
+    assert C.get_rank() == 0 and C.get_size() == 1
+    C.set_pg()
+    t = torch.arange(4.0)
+    assert C.all_reduce(t) is t and C.shm_allreduce(t) is t
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(96, 160)
+    x = torch.randn(5, 96)
+    full = lin(x)
+    def shard(dim, r, size, bs):
+        m = copy.deepcopy(lin)
+        C.ShardLinear(m, dim, r, size, bs)  # in place, like the reference's
+        return m
+
+    cols = [shard(0, r, 3, 32) for r in range(3)]
+    assert cols[0].split_sizes == [32, 64, 64] and [c.weight.shape[0] for c in cols] == [32, 64, 64]
+    assert torch.equal(torch.cat([c.weight.data for c in cols]), lin.weight.data)
+    assert torch.allclose(torch.cat([torch.nn.functional.linear(x, c.weight, c.bias) for c in cols], -1), full, atol=1e-6)
+    rows = [shard(1, r, 3, 32) for r in range(3)]
+    assert rows[0].split_sizes == [32, 32, 32]
+    parts = [torch.nn.functional.linear(x[:, 32 * r:32 * r + 32], m.weight, m.bias) for r, m in enumerate(rows)]
+    assert torch.allclose(sum(parts), full, atol=1e-5)  # the bias was divided by the number of ranks
+    with pytest.raises(ValueError):
+        shard(0, 0, 2, 64)  # 160 is not a multiple of 64
+    ln = C.BlockedLayerNorm(64)
+    y = ln(torch.randn(3, 64))
+    assert torch.allclose(y.mean(-1), torch.zeros(3), atol=1e-5)
+    assert C.compare(t, t.clone(), "same") is True and C.compare(t, t + 1, "shifted") is False

@@ -2,10 +2,16 @@
 
 Reference: ``src/tpp_pytorch_extension/llm/llm_common.py`` -- ``fc_plain``
 (:379), ``BlockedLinear`` (:383-434), ``FixLinear`` (:437-515) and the
-``TppCache`` wrapper handed around as ``past_key_values`` (:80-182).  The
-generation wrapper and tensor-parallel sharding of that file are outside the
-path built here.
+``TppCache`` wrapper handed around as ``past_key_values`` (:80-182), and the
+small helpers callers of that module import next to them (``compare``,
+``print_line_info``, ``BlockedLayerNorm``, and the process-group helpers in
+their one-process form: ``get_rank`` / ``get_size`` / ``set_pg`` /
+``all_reduce`` / ``ShardLinear``, :47-77, :429-434, :517-578).  The torch.jit
+tracing wrapper of that file has no counterpart: decode steps are replayed
+as HIP graphs instead.
 """
+import inspect
+
 import torch
 
 from ..utils.blocked_layout import BlockedParameter, BlockedModule
@@ -63,6 +69,105 @@ class BlockedLinear(BlockedModule, torch.nn.Linear):
     def forward_mul(self, input, mul_in):
         bias = self.bias if self.bias is not None else torch.Tensor()
         return torch.ops.tpp_llm.fc_mul(input.to(self._io_dtype()), self.weight, bias, mul_in)
+
+
+class BlockedLayerNorm(BlockedModule, torch.nn.LayerNorm):
+    """llm_common.py:429-434: a LayerNorm whose parameters may be blocked.  bf16 inputs on the GPU run the
+    lyr_norm kernel of the decoder blocks; anything else takes torch's own."""
+
+    def maybe_block_params(self):
+        if self.elementwise_affine:
+            if hasattr(self.weight, "block"):
+                self.weight.block()
+            if self.bias is not None and hasattr(self.bias, "block"):
+                self.bias.block()
+
+    def forward(self, input):
+        from .. import _ops
+        if (input.is_cuda and input.dtype == torch.bfloat16 and self.elementwise_affine and self.bias is not None
+                and len(self.normalized_shape) == 1 and self.normalized_shape[0] % 8 == 0
+                and self.weight.dtype in (torch.float32, torch.bfloat16) and self.bias.dtype == self.weight.dtype):
+            return _ops.layer_norm(input, self.weight.data, self.bias.data, self.eps)
+        return super().forward(input)
+
+
+def compare(ref, opt, name=""):
+    """llm_common.py:47-63: print where `opt` leaves `ref` (relative to the mean magnitude), worst first."""
+    ref, opt = ref.detach().float().cpu(), opt.detach().float().cpu()
+    if ref.allclose(opt, atol=1e-6, rtol=1e-6):
+        return True
+    print(f"{name}: ref = {ref.reshape(-1)[:8]}, opt = {opt.reshape(-1)[:8]}")
+    adiff = (ref - opt).abs()
+    rdiff = adiff / ref.abs().mean()
+    worst = torch.argsort(rdiff.reshape(-1), descending=True)[:8]
+    for i in worst.tolist():
+        print(f"{i}: ref: {ref.reshape(-1)[i].item():.7g} opt: {opt.reshape(-1)[i].item():.7g} "
+              f"diff: {adiff.reshape(-1)[i].item():.7g}  rdiff: {rdiff.reshape(-1)[i].item():.7g}")
+    return False
+
+
+def print_line_info():
+    """llm_common.py:70-77: where the caller is running and who called it."""
+    cf = inspect.currentframe().f_back
+    up = cf.f_back
+    where = f"{up.f_code.co_filename}:{up.f_lineno}:{up.f_code.co_name}()" if up is not None else "<top>"
+    print(f"Running At {cf.f_code.co_name}():{cf.f_lineno}  from {where}")
+
+
+# Process-group helpers (llm_common.py:517-578).  This build runs one process on one GPU: rank 0 of 1, collectives
+# are the identity; with an initialised torch.distributed group of more than one rank they refuse, because the
+# tensor-parallel exchange steps of the decoder blocks are not built.
+def get_rank():
+    if torch.distributed.is_available() and torch.distributed.is_initialized():
+        return torch.distributed.get_rank()
+    return 0
+
+
+def get_size():
+    if torch.distributed.is_available() and torch.distributed.is_initialized():
+        return torch.distributed.get_world_size()
+    return 1
+
+
+def _one_process(what):
+    if get_size() > 1:
+        raise NotImplementedError(f"{what}: tensor parallelism over {get_size()} ranks is not built (one GPU per model)")
+
+
+def set_pg():
+    _one_process("set_pg")
+
+
+def all_reduce(t):
+    _one_process("all_reduce")
+    return t
+
+
+def shm_allreduce(t):
+    _one_process("shm_allreduce")
+    return t
+
+
+def ShardLinear(m, dim, rank, size, block_size=1):
+    """llm_common.py:517-546: keep rank's share of an nn.Linear, split along the output (dim 0) or input (dim 1)
+    features in whole blocks of block_size, and record every rank's share in m.split_sizes.  Pure slicing: it is
+    what a tensor-parallel caller does before FixLinear; the exchange steps it implies are not built."""
+    total = m.weight.shape[dim]
+    if total % block_size:
+        raise ValueError(f"dim_size ({total}) is not multiple of block_size ({block_size})")
+    blocks = total // block_size
+    cuts = [0] + [((blocks * (i + 1)) // size) * block_size for i in range(size)]
+    lo, hi = cuts[rank], cuts[rank + 1]
+    m.split_sizes = [cuts[i + 1] - cuts[i] for i in range(size)]
+    with torch.no_grad():
+        if dim == 0:
+            m.weight.data = m.weight.data[lo:hi, :].contiguous()
+            if m.bias is not None:
+                m.bias.data = m.bias.data[lo:hi].contiguous()
+        else:
+            m.weight.data = m.weight.data[:, lo:hi].contiguous()
+            if m.bias is not None:
+                m.bias.data = m.bias.data / size
 
 
 def _resolve_weight_dtype(weight_dtype, layer_dtype):
