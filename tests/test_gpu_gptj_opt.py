@@ -293,3 +293,41 @@ def test_optimize_model_for_opt_against_transformers(weight_dtype, before, proj)
     opt_model = F.OptimizeModelForOPT(copy.deepcopy(ref_model), torch.bfloat16, "cuda", weight_dtype).eval()
     assert type(opt_model.model.decoder.layers[0].cpp_block).__name__ == "OPTDecoderLayer"
     _compare_with_stock(ref_model, opt_model, 3e-2 if weight_dtype == "mxfp4" else 6e-2, 1024, F.generate_greedy)
+
+
+@pytest.mark.parametrize("family", ["llama", "qwen2", "gptj", "opt"])
+def test_transformers_generate_on_optimized_models(family):
+    """transformers' own generate() (greedy, left-padded batch) runs on the optimized model of every family and
+    returns the tokens of this package's plain greedy loop."""
+    T = pytest.importorskip("transformers")
+    import tpp_pytorch_extension  # noqa: F401
+    from tpp_pytorch_extension.llm import fused_llama_infer as FL, fused_qwen2_infer as FQ
+    torch.manual_seed(7)
+    if family == "llama":
+        model = T.LlamaForCausalLM(T.LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=2,
+                                                 num_attention_heads=4, num_key_value_heads=2, vocab_size=1024,
+                                                 max_position_embeddings=256, head_dim=128))
+        opt, F = FL.OptimizeModelForLlama(model.eval(), torch.bfloat16, "cuda", "mxfp4"), FL
+    elif family == "qwen2":
+        model = T.Qwen2ForCausalLM(T.Qwen2Config(hidden_size=512, intermediate_size=1024, num_hidden_layers=2,
+                                                 num_attention_heads=4, num_key_value_heads=2, vocab_size=1024,
+                                                 max_position_embeddings=256, use_sliding_window=False,
+                                                 tie_word_embeddings=False))
+        opt, F = FQ.OptimizeModelForQwen2(model.eval(), torch.bfloat16, "cuda", "mxfp4"), FQ
+    elif family == "gptj":
+        model = T.GPTJForCausalLM(T.GPTJConfig(n_embd=512, n_head=4, n_layer=2, n_positions=256, rotary_dim=64,
+                                               vocab_size=1600, bos_token_id=1, eos_token_id=2))
+        opt, F = _gj().OptimizeModelForGPTJ(model.eval(), torch.bfloat16, "cuda", "mxfp4"), _gj()
+    else:
+        model = T.OPTForCausalLM(T.OPTConfig(hidden_size=512, ffn_dim=1024, num_hidden_layers=2, num_attention_heads=8,
+                                             vocab_size=1024, max_position_embeddings=256, bos_token_id=1,
+                                             eos_token_id=2, pad_token_id=0))
+        opt, F = _opt().OptimizeModelForOPT(model.eval(), torch.bfloat16, "cuda", "mxfp4"), _opt()
+    opt = opt.eval()
+    ids = torch.randint(3, 1000, (2, 11), generator=torch.Generator().manual_seed(8)).cuda()
+    am = torch.ones_like(ids)
+    am[1, :3] = 0
+    out = opt.generate(input_ids=ids, attention_mask=am, max_new_tokens=4, do_sample=False, pad_token_id=0)
+    assert out.shape == (2, 15) and torch.equal(out[:, :11], ids)
+    ref = F.generate_greedy(opt, ids, 4, attention_mask=am)
+    assert torch.equal(out, ref)

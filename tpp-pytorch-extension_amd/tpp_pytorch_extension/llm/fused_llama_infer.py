@@ -744,8 +744,13 @@ def generate_greedy(model, input_ids, max_new_tokens, attention_mask=None):
     cache = None
     cur = input_ids
     for _ in range(max_new_tokens):
-        out = model(input_ids=cur, attention_mask=attention_mask, past_key_values=cache, use_cache=True,
-                    logits_to_keep=1)
+        pos = None
+        if attention_mask is not None:
+            # positions count the real tokens, as generate() derives them from the mask (padding gets position 1)
+            pos = attention_mask.long().cumsum(-1) - 1
+            pos = pos.masked_fill(attention_mask == 0, 1)[:, -cur.shape[1]:]
+        out = model(input_ids=cur, attention_mask=attention_mask, position_ids=pos, past_key_values=cache,
+                    use_cache=True, logits_to_keep=1)
         cache = out.past_key_values
         cur = out.logits[:, -1].argmax(dim=-1, keepdim=True)
         ids = torch.cat([ids, cur], dim=1)
