@@ -56,6 +56,10 @@ class GPTJBlock(FormatSwitches):
          self.t_EP) = params
         self.layer_idx, self.eps, self.H = int(layer_idx), float(eps), int(H)
         self.max_positions, self.rotary_dim = int(max_positions), int(rotary_dim)
+        if self.t_EP.dim() != 2 or self.t_EP.shape[1] % 16 or self.t_EP.shape[1] > self.H:
+            raise TppxError(_lib.ESHAPE, f"GPTJBlock: embed_positions must be [max_positions][rotary_dim] with rotary_dim a "
+                                         f"multiple of 16 and at most H = {self.H}, got {tuple(self.t_EP.shape)}")
+        self.t_EP = self.t_EP.to(torch.float32).contiguous()  # the kernel reads an fp32 sin | cos table
         self._setup_formats()
         self.N = _ops.weight_nk(self.t_Wq)[0] // self.H
 

@@ -38,6 +38,7 @@ class OPTDecoderLayer(FormatSwitches):
          self.t_Wp, self.t_Bp, self.t_Wi, self.t_Bi, self.t_Wo, self.t_Bo) = params
         self.layer_idx, self.eps1, self.eps2, self.H = int(layer_idx), float(eps1), float(eps2), int(H)
         self.do_layer_norm_before = bool(do_layer_norm_before)
+        self._pos = {}
         self._setup_formats()
         self.N = _ops.weight_nk(self.t_Wq)[0] // self.H
 
@@ -45,7 +46,9 @@ class OPTDecoderLayer(FormatSwitches):
         t_HS = inputs[0]
         t_am = inputs[1] if len(inputs) > 1 else None
         B, S, _ = t_HS.shape
-        pos = torch.zeros((1, S), dtype=torch.int64, device=t_HS.device)  # unused: nothing is rotated
+        pos = self._pos.get((t_HS.device, S))  # never read (nothing is rotated), but the append launch takes one
+        if pos is None:
+            pos = self._pos[(t_HS.device, S)] = torch.zeros((1, S), dtype=torch.int64, device=t_HS.device)
         check_layer_inputs("OPTDecoderLayer", t_HS, pos, cache)
         Wq, Wk, Wv, Wp, Wi, Wo = self._weights_for(B * S)
         t_res = t_HS
