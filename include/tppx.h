@@ -479,8 +479,9 @@ int tppx_rotary_kv_append_gptj(void* q, void* k, const void* v,
  * bf16 [B][mask_ld] or NULL; valid keys = *kv_len_dev (device i32) + kv_len_add
  * (the counter may still hold the length before this step's append); out bf16
  * [B][Nq][128].  ws: optional scratch for split-KV partial results.  Head sizes
- * H other than 128 (multiples of 8 up to 256, tensors [..][H]) run a plain,
- * untuned kernel; anything else returns TPPX_EUNSUPPORTED. */
+ * H other than 128 (multiples of 8 up to 256, tensors [..][H]) run a kernel of
+ * the same layout with 8, 16 or 32 lanes per key (not the rotary-fused form);
+ * anything else returns TPPX_EUNSUPPORTED. */
 int tppx_attn_decode(const void* q, const void* kcache, const void* vcache,
                      const void* mask, int64_t mask_ld, const void* kv_len_dev,
                      int64_t kv_len_add, void* out, int64_t B, int64_t Nq,

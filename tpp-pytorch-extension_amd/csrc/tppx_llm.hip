@@ -1304,7 +1304,8 @@ static int attn_decode_launch(const char* who, AttnParams& p, bool rot, int64_t 
 // ---------------------------------------------------------------------------
 // Attention for head sizes other than 128 (attn<T>, src/csrc/llm/attn.cpp:781-955, is generic in the head size; the
 // kernels above are built for 128): one kernel for the single-query step and for prompt passes, H a multiple of 8
-// up to 256.  One wave per (sequence, query token, query head), four per workgroup, no barrier: 64 keys per trip,
+// up to 256, and a second kernel for the single-query step (below).  The first: one wave per (sequence, query token,
+// query head), four per workgroup, no barrier: 64 keys per trip,
 // a lane takes the whole dot product of its key (16-byte loads along its row, the query as fp32 in wave-private
 // LDS, read as broadcasts), online softmax over the trip with the probabilities rounded to bf16 before they multiply
 // V and the normaliser summing the unrounded ones, then lanes turn to output dimensions (lane, lane + 64, ...) and
@@ -1320,6 +1321,8 @@ struct AttnGenParams {
   uint16_t* out;       // [B][S][Nq][H]
   int B, S, Nq, Nkv, H, Smax, mask_ld, past; // prompt pass: query i sees keys 0 .. past + i
   float scale;
+  int splits;          // single-query step (attn_generic_rows_kernel): workgroups per query, see there
+  float* part;         // splits > 1: [query][split][2 + H] floats (running maximum, sum, unnormalised output)
 };
 
 __global__ void __launch_bounds__(256)
@@ -1393,10 +1396,212 @@ attn_generic_kernel(const AttnGenParams p) {
       orow[lane + 64 * i] = (uint16_t)f32_to_bf16_bits(l > 0.f ? acc[i] / l : 0.f);
 }
 
-static int attn_generic_launch(const char* who, AttnGenParams& p, hipStream_t stream) {
+// The single-query step at those head sizes, laid out like attn_decode_kernel: G = 8, 16 or 32 lanes share a key
+// (lane = key slot l / G, 16-byte chunk l % G; chunks past H / 8 idle), so a wave instruction reads 64 / G whole
+// rows; NU instructions per wave and trip with the next trip requested ahead; every lane group keeps its own
+// running (maximum, sum, 8 output dims per lane), merged at the end through LDS.  Grid (B * Nq, splits): split y
+// takes the trips y, y + splits, ...; several splits leave their states for attn_generic_merge_kernel.
+template <int G>
+__global__ void __launch_bounds__(256)
+attn_generic_rows_kernel(const AttnGenParams p) {
+  constexpr int KPI = 64 / G;            // keys per wave instruction
+  constexpr int NU = G == 8 ? 2 : 4;     // instructions per wave and trip
+  constexpr int WK = NU * KPI;           // keys per wave and trip
+  constexpr int TRIP = 4 * WK;           // keys per workgroup and trip
+  constexpr int NG = 4 * KPI;            // lane groups per workgroup
+  __shared__ float sm[NG], sl[NG];
+  __shared__ float sacc[NG * G * 8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int grp = lane / G, c = lane % G;
+  const int H = p.H, C = H >> 3;
+  const bool live = c < C;               // this lane's chunk exists
+  const int cc = min(c, C - 1);
+  const int bh = blockIdx.x, b = bh / p.Nq, hq = bh - b * p.Nq;
+  const int hk = hq / (p.Nq / p.Nkv);
+  const uint16_t* kb = p.kc + ((int64_t)b * p.Nkv + hk) * (int64_t)p.Smax * H + cc * 8;
+  const uint16_t* vb = p.vc + ((int64_t)b * p.Nkv + hk) * (int64_t)p.Smax * H + cc * 8;
+  i32x4 kw[NU], vw[NU], kn[NU], vn[NU];
+  auto load_kv = [&](int base, i32x4 (&kd)[NU], i32x4 (&vd)[NU]) {
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+      const int kk = min(base + u * KPI + grp, p.Smax - 1);
+      kd[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(kb + (int64_t)kk * H));
+      vd[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(vb + (int64_t)kk * H));
+    }
+  };
+  load_kv(blockIdx.y * TRIP + wave * WK, kw, vw); // the first trip does not depend on the length (a device scalar)
+  const int L = max(0, min(p.kv_len[0] + p.kv_len_add, p.Smax));
+  const int trips = (L + TRIP - 1) / TRIP;
+  float qf[8];
+  unpack8(*reinterpret_cast<const uint4*>(p.q + (int64_t)bh * H + cc * 8), qf);
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    qf[e] = live ? qf[e] * p.scale : 0.f;
+  const uint16_t* mrow = p.mask ? p.mask + (int64_t)b * p.mask_ld : nullptr;
+  float m = -3.0e38f, l = 0.f, acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    acc[e] = 0.f;
+  for (int t = blockIdx.y; t < trips; t += p.splits) {
+    const int base = t * TRIP + wave * WK;
+    load_kv(base + p.splits * TRIP, kn, vn); // unconditional (rows are clamped): a branch here would drain the queue
+    float sc[NU];
+    int key[NU];
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+      key[u] = base + u * KPI + grp;
+      float kf[8];
+      unpack8(as_uint4(kw[u]), kf);
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        d = fmaf(qf[e], kf[e], d);
+      // sum over the G lanes of the key: DPP steps inside a row of 16, then the other half of a 32-lane group
+      d += dpp_mov<0xB1>(d);
+      d += dpp_mov<0x4E>(d);
+      d += dpp_mov<0x141>(d);
+      if (G >= 16)
+        d += dpp_mov<0x140>(d);
+      if (G == 32)
+        d += __shfl_xor(d, 16);
+      if (mrow && key[u] < p.mask_ld && key[u] < L)
+        d += bf16_bits_to_f32(mrow[key[u]]);
+      sc[u] = key[u] < L ? d : -3.0e38f;
+    }
+    if (t * TRIP + TRIP > L) { // the last trip only (wave-uniform): rows past the end may hold anything, NaN included
+#pragma unroll
+      for (int u = 0; u < NU; u++)
+        if (key[u] >= L)
+          vw[u] = i32x4{0, 0, 0, 0};
+    }
+    float mn = m;
+#pragma unroll
+    for (int u = 0; u < NU; u++)
+      mn = fmaxf(mn, sc[u]);
+    const float alpha = __expf(m - mn);
+    l *= alpha;
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      acc[e] *= alpha;
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+      const float pr = key[u] < L ? __expf(sc[u] - mn) : 0.f;
+      l += pr;
+      const float pb = round_bf16(pr); // the probabilities that multiply V are bf16, the normaliser sums the unrounded
+      float vf[8];
+      unpack8(as_uint4(vw[u]), vf);
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        acc[e] = fmaf(pb, vf[e], acc[e]);
+    }
+    m = mn;
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+      kw[u] = kn[u];
+      vw[u] = vn[u];
+    }
+  }
+  // merge the lane groups of the workgroup
+  const int gi = wave * KPI + grp;
+  if (c == 0) {
+    sm[gi] = m;
+    sl[gi] = l;
+  }
+  if (live) {
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      sacc[gi * (G * 8) + c * 8 + e] = acc[e];
+  }
+  __syncthreads();
+  if (tid < H) {
+    float M = -3.0e38f;
+#pragma unroll
+    for (int g = 0; g < NG; g++)
+      M = fmaxf(M, sm[g]);
+    float Ls = 0.f, o = 0.f;
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+      const float w = __expf(sm[g] - M);
+      Ls = fmaf(w, sl[g], Ls);
+      o = fmaf(w, sacc[g * (G * 8) + tid], o);
+    }
+    if (p.splits == 1) {
+      p.out[(int64_t)bh * H + tid] = (uint16_t)f32_to_bf16_bits(Ls > 0.f ? o / Ls : 0.f);
+    } else {
+      float* st = p.part + ((int64_t)bh * p.splits + blockIdx.y) * (int64_t)(H + 2);
+      st[2 + tid] = o;
+      if (tid == 0) {
+        st[0] = M;
+        st[1] = Ls;
+      }
+    }
+  }
+}
+
+// one wave per query: the splits' (maximum, sum, output) states, in split order, become the normalised output
+__global__ void __launch_bounds__(64)
+attn_generic_merge_kernel(const AttnGenParams p) {
+  const int lane = threadIdx.x;
+  const int64_t qi = blockIdx.x;
+  const int H = p.H;
+  const float* st = p.part + qi * p.splits * (int64_t)(H + 2);
+  float M = -3.0e38f;
+  for (int i = 0; i < p.splits; i++)
+    M = fmaxf(M, st[i * (H + 2)]);
+  float Ls = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < p.splits; i++) {
+    const float* si = st + i * (int64_t)(H + 2);
+    const float w = __expf(si[0] - M); // a split without keys carries sum 0 and output 0
+    Ls = fmaf(w, si[1], Ls);
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (lane + 64 * j < H)
+        o[j] = fmaf(w, si[2 + lane + 64 * j], o[j]);
+  }
+  uint16_t* orow = p.out + qi * H;
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+    if (lane + 64 * j < H)
+      orow[lane + 64 * j] = (uint16_t)f32_to_bf16_bits(Ls > 0.f ? o[j] / Ls : 0.f);
+}
+
+static int attn_generic_launch(const char* who, AttnGenParams& p, hipStream_t stream, void* ws = nullptr,
+                               int64_t ws_bytes = 0) {
   TPPX_REQUIRE(p.H >= 8 && p.H <= 256 && p.H % 8 == 0, TPPX_EUNSUPPORTED,
                "%s: head size %d (128 on the tuned kernels, other multiples of 8 up to 256 on the plain one)", who, p.H);
-  const int64_t waves = (int64_t)p.B * p.S * p.Nq;
+  const int64_t queries = (int64_t)p.B * p.S * p.Nq;
+  p.splits = 1;
+  if (p.kv_len && p.S == 1 && env_int("TPPX_ATTN_GENERIC_ROWS", 1) != 0) {
+    // Single-query steps: a workgroup per (query, split of the key range).  Up to 384 workgroups in all (measured at
+    // 2048 keys: 16 heads of 256 59.9 -> 21.1 us with 24 splits, 64 queries 57.8 -> 27.6 us with 6, 256 queries
+    // better unsplit), at least two trips each at the cache's capacity (the length itself is a device scalar: splits
+    // whose trips lie past the keys leave empty states), at most 32; one split for caches under 512 keys (the merge
+    // launch costs more than it saves) and when the caller's workspace cannot hold the states.
+    const int G = p.H <= 64 ? 8 : p.H <= 128 ? 16 : 32;
+    const int trip = G == 32 ? 32 : 64;
+    int64_t want = env_int("TPPX_ATTN_GENERIC_SPLITS", 0);
+    if (want <= 0)
+      want = p.Smax < 512 ? 1 : 384 / queries;
+    want = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, 32), ((int64_t)p.Smax + 2 * trip - 1) / (2 * trip)));
+    if (want > 1 && ws && queries * want * (p.H + 2) * (int64_t)sizeof(float) <= ws_bytes) {
+      p.splits = (int)want;
+      p.part = (float*)ws;
+    }
+    TPPX_REQUIRE(queries < ((int64_t)1 << 31), TPPX_ESHAPE, "%s: problem too large", who);
+    const dim3 grid((unsigned)queries, (unsigned)p.splits);
+    if (G == 8)
+      attn_generic_rows_kernel<8><<<grid, dim3(256), 0, stream>>>(p);
+    else if (G == 16)
+      attn_generic_rows_kernel<16><<<grid, dim3(256), 0, stream>>>(p);
+    else
+      attn_generic_rows_kernel<32><<<grid, dim3(256), 0, stream>>>(p);
+    int rc = check_hip(hipGetLastError(), who);
+    if (rc || p.splits == 1)
+      return rc;
+    attn_generic_merge_kernel<<<dim3((unsigned)queries), dim3(64), 0, stream>>>(p);
+    return check_hip(hipGetLastError(), who);
+  }
+  const int64_t waves = queries;
   TPPX_REQUIRE(waves > 0 && (waves + 3) / 4 < ((int64_t)1 << 31), TPPX_ESHAPE, "%s: problem too large", who);
   attn_generic_kernel<<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(p);
   return check_hip(hipGetLastError(), who);
@@ -1420,7 +1625,7 @@ extern "C" int tppx_attn_decode(const void* q, const void* kcache, const void* v
     g.kv_len = (const int32_t*)kv_len_dev; g.kv_len_add = (int)kv_len_add; g.out = (uint16_t*)out;
     g.B = (int)B; g.S = 1; g.Nq = (int)Nq; g.Nkv = (int)Nkv; g.H = (int)H; g.Smax = (int)Smax; g.mask_ld = (int)mask_ld;
     g.scale = 1.0f / sqrtf((float)H);
-    return attn_generic_launch(who, g, (hipStream_t)stream);
+    return attn_generic_launch(who, g, (hipStream_t)stream, ws, ws_bytes);
   }
   AttnParams p;
   memset(&p, 0, sizeof(p));
