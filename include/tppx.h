@@ -510,7 +510,8 @@ int tppx_attn_decode_rotary(const void* q, const void* k, const void* v,
  * q / out bf16 [B][S][Nq][128]; the cache already holds the S new keys at
  * positions past_len .. past_len+S-1 (tppx_rotary_kv_append_llama before this
  * call); query i sees keys 0 .. past_len+i; additive mask bf16 [B][mask_ld]
- * over key positions or NULL.  Head sizes other than 128: as tppx_attn_decode. */
+ * over key positions or NULL.  Head sizes other than 128 (multiples of 8 up to
+ * 256) run the same kernel over a head size padded to 64, 128 or 256. */
 int tppx_attn_prefill(const void* q, const void* kcache, const void* vcache,
                       const void* mask, int64_t mask_ld, int64_t past_len,
                       void* out, int64_t B, int64_t S, int64_t Nq, int64_t Nkv,

@@ -1,5 +1,5 @@
 """Attention for head sizes other than 128 (attn<T>, src/csrc/llm/attn.cpp:781-955, is generic in the head size):
-the plain kernel behind tppx_attn_decode / tppx_attn_prefill, against the oracle (tolerance as for the 128-wide
+the kernels behind tppx_attn_decode / tppx_attn_prefill for those sizes, against the oracle (tolerance as for the 128-wide
 kernels: rel-L2 5e-3, max-abs 2^-7 of the largest output) and plain PyTorch fp32 softmax attention (1e-2), and a
 decoder layer with 64-wide heads against the oracle composition."""
 import numpy as np
@@ -55,7 +55,36 @@ def test_attn_decode_other_head_size_with_mask():
     assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3
 
 
-@pytest.mark.parametrize("H", [64, 96, 256])
+@pytest.mark.parametrize("H", [64, 80, 256, 8, 200])
+@pytest.mark.parametrize("B,Nq,Nkv,L,Smax", [(1, 4, 2, 700, 1024), (2, 8, 8, 100, 1024), (1, 2, 1, 1000, 1000)])
+def test_attn_decode_other_head_sizes_split_key_range(H, B, Nq, Nkv, L, Smax, monkeypatch):
+    """Caches of 512 keys and more: the key range is dealt to several workgroups per query (some of them past the
+    valid length, leaving empty states) and merged by a second launch; one split gives the same answer up to the
+    order of the sums."""
+    F = _llm()
+    q = randn_bf16((B, Nq, H), 1.0, 131 + H)
+    k = randn_bf16((B, Nkv, Smax, H), 1.0, 132 + H)
+    v = randn_bf16((B, Nkv, Smax, H), 1.0, 133 + H)
+    k[:, :, L:] = float("nan")
+    v[:, :, L:] = float("nan")
+    got = _attn(F, q.cuda(), k.cuda(), v.cuda(), L)
+    ref = O.attn_decode(t2bits(q), t2bits(k[:, :, :L]), t2bits(v[:, :, :L]))
+    kk = k[:, :, :L].float().repeat_interleave(Nq // Nkv, dim=1)
+    vv = v[:, :, :L].float().repeat_interleave(Nq // Nkv, dim=1)
+    s = torch.einsum("bnh,bnlh->bnl", q.float(), kk) / np.sqrt(float(H))
+    t = torch.einsum("bnl,bnlh->bnh", torch.softmax(s, -1), vv).numpy().astype(np.float64)
+    _close(got, ref, t)
+    monkeypatch.setenv("TPPX_ATTN_GENERIC_SPLITS", "1")
+    one = _attn(F, q.cuda(), k.cuda(), v.cuda(), L)
+    _close(one, ref, t)
+    monkeypatch.setenv("TPPX_ATTN_GENERIC_SPLITS", "5")
+    five = _attn(F, q.cuda(), k.cuda(), v.cuda(), L)
+    _close(five, ref, t)
+    none = _attn(F, q.cuda(), k.cuda(), v.cuda(), L, ws=False)  # no workspace: one split
+    assert torch.equal(none, one)
+
+
+@pytest.mark.parametrize("H", [64, 80, 96, 256, 8, 200])
 @pytest.mark.parametrize("B,S,Nq,Nkv,past,Smax", [(1, 130, 4, 4, 0, 256), (2, 77, 8, 2, 0, 128), (2, 5, 4, 4, 100, 128), (3, 1, 4, 2, 40, 64)])
 def test_attn_prefill_other_head_sizes(H, B, S, Nq, Nkv, past, Smax):
     _llm()
@@ -134,3 +163,41 @@ def test_decoder_layer_with_64_wide_heads(S, past):
     kc, vc = cache.get(0)
     assert_close_bf16(t2bits(kc[:, :, past:]), np.ascontiguousarray(k), what="cached keys")
     assert_close_bf16(t2bits(vc[:, :, past:]), np.ascontiguousarray(v), what="cached values")
+
+
+@pytest.mark.parametrize("H", [64, 256])
+def test_attn_prefill_other_head_sizes_full_prompt_and_plain_kernel(H, monkeypatch):
+    """A prompt long enough for 32 queries per wave (head size 64) and many key tiles: sampled rows against the
+    oracle's single-query function, and the MFMA kernel against the plain one-wave-per-query kernel it replaced."""
+    _llm()
+    B, S, Nq = 1, 600, 16
+    q = randn_bf16((B, S, Nq, H), 1.0, 171 + H)
+    k = randn_bf16((B, Nq, S, H), 1.0, 172 + H)
+    v = randn_bf16((B, Nq, S, H), 1.0, 173 + H)
+    got = _attn_prefill(q.cuda(), k.cuda(), v.cuda(), 0).cpu()
+    for i in (0, 1, 63, 64, 65, 511, 599):
+        ref = O.attn_decode(t2bits(q[:, i]), t2bits(k[:, :, :i + 1]), t2bits(v[:, :, :i + 1]))
+        g, r = bits2f(t2bits(got[:, i])).astype(np.float64), bits2f(ref).astype(np.float64)
+        assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3, i
+        assert np.abs(g - r).max() <= 2.0 ** -7 * np.abs(r).max(), i
+    monkeypatch.setenv("TPPX_ATTN_PREFILL_MFMA", "0")
+    plain = _attn_prefill(q.cuda(), k.cuda(), v.cuda(), 0).cpu()
+    d = (plain.float() - got.float()).double()
+    assert float(d.norm() / plain.double().norm()) <= 5e-3
+
+
+@pytest.mark.parametrize("H", [64, 200])
+def test_attn_prefill_other_head_size_with_mask(H):
+    F = _llm()
+    B, S, Nq, Smax = 2, 70, 4, 128
+    q = randn_bf16((B, S, Nq, H), 1.0, 181 + H)
+    k = randn_bf16((B, Nq, Smax, H), 1.0, 182 + H)
+    v = randn_bf16((B, Nq, Smax, H), 1.0, 183 + H)
+    keep = torch.ones(B, S, dtype=torch.int64)
+    keep[0, :9] = 0  # left padding of sequence 0
+    mask = F.TppCache(Smax).align_and_invert_mask(keep.to(torch.bfloat16))
+    got = _attn_prefill(q.cuda(), k.cuda(), v.cuda(), 0, mask=mask.cuda())
+    ref = O.attn_prefill(t2bits(q), t2bits(k[:, :, :S]), t2bits(v[:, :, :S]), mask.float().numpy())
+    g, r = bits2f(t2bits(got)).astype(np.float64), bits2f(ref).astype(np.float64)
+    assert np.isfinite(g).all()
+    assert np.sqrt(((g - r) ** 2).sum() / (r ** 2).sum()) <= 5e-3

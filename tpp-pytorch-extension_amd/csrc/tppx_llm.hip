@@ -840,6 +840,7 @@ struct AttnPrefillParams {
   uint16_t* out;        // [B][S][Nq][128]
   int B, S, Nq, Nkv, Smax, mask_ld, past;
   float scale;
+  int H;                // head size (attn_prefill_hd_kernel; the kernel for 128 does not read it)
 };
 
 constexpr int AP_KP = 136; // LDS row pitch of the K tile, bf16 elements (128 + 8: rows 16-byte aligned, banks spread)
@@ -1029,6 +1030,211 @@ attn_prefill_kernel(const AttnPrefillParams p) {
           w[h] = f32_to_bf16_bits(ls > 0.f ? acc[qg][dt][2 * h] / ls : 0.f) |
                  (f32_to_bf16_bits(ls > 0.f ? acc[qg][dt][2 * h + 1] / ls : 0.f) << 16);
         *reinterpret_cast<uint2*>(orow + dt * 16 + g * 4) = make_uint2(w[0], w[1]);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Prompt attention at head sizes other than 128: attn_prefill_kernel with the head size padded to HD = 64, 128 or
+// 256 (H a multiple of 8, H <= HD; dims past H are staged as zeros and not stored), the K tile 64 x (HD + 8) and the
+// V^T tile HD x 68 in dynamic LDS, HD / 32 MFMAs per 16 keys for the scores and HD / 16 output tiles per query group.
+// Same arithmetic and rounding points as the kernel for 128.
+// ---------------------------------------------------------------------------
+template <int QG, int HD>
+__global__ void __launch_bounds__(256)
+attn_prefill_hd_kernel(const AttnPrefillParams p) {
+  extern __shared__ __align__(16) uint16_t ap_lds[];
+  constexpr int KP = HD + 8, VP = AP_VP, NJ = HD / 32, NDT = HD / 16, CH = HD / 8;
+  constexpr int VI = (CH + 15) / 16; // value chunks per thread: 16 threads (key quads) x 16 chunks per pass
+  uint16_t* ks = ap_lds;           // [64 keys][KP]
+  uint16_t* vt = ap_lds + 64 * KP; // [HD dims][VP]
+  constexpr int QB = 64 * QG;
+  const int H = p.H, HC = H >> 3;  // real 8-dim chunks per row
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 4, c = lane & 15;
+  const int bh = blockIdx.y, b = bh / p.Nq, hq = bh - b * p.Nq;
+  const int hk = hq / (p.Nq / p.Nkv);
+  const int qblk = (int)gridDim.x - 1 - (int)blockIdx.x; // the last query blocks see the most keys: start them first
+  const int q0 = qblk * QB + wave * (16 * QG);
+  const int last_key = p.past + p.S - 1;
+  const i32x4 zero4 = {0, 0, 0, 0};
+
+  int qpos[QG];
+  bf16x8 qreg[QG][NJ];
+#pragma unroll
+  for (int qg = 0; qg < QG; qg++) {
+    const int qi = min(q0 + qg * 16 + c, p.S - 1);
+    qpos[qg] = p.past + qi;
+    const uint16_t* qrow = p.q + (((int64_t)b * p.S + qi) * p.Nq + hq) * H;
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+      const int ch = j * 4 + g;
+      qreg[qg][j] = __builtin_bit_cast(bf16x8, ch < HC ? *reinterpret_cast<const i32x4*>(qrow + ch * 8) : zero4);
+    }
+  }
+  const uint16_t* kbase = p.kc + ((int64_t)b * p.Nkv + hk) * (int64_t)p.Smax * H;
+  const uint16_t* vbase = p.vc + ((int64_t)b * p.Nkv + hk) * (int64_t)p.Smax * H;
+  const uint16_t* mrow = p.mask ? p.mask + (int64_t)b * p.mask_ld : nullptr;
+
+  // staging registers: K rows chunk-fastest; V: a thread takes one chunk of FOUR consecutive keys per pass
+  i32x4 kst[NJ], vst[VI][4];
+  const int vq = tid & 15;
+  auto load_tile = [&](int kb) {
+#pragma unroll
+    for (int i = 0; i < NJ; i++) {
+      const int idx = tid + i * 256;
+      const int key = idx / CH, ch = idx % CH;
+      const int kk = min(kb * 64 + key, last_key);
+      kst[i] = ch < HC ? *reinterpret_cast<const i32x4*>(kbase + (int64_t)kk * H + ch * 8) : zero4;
+    }
+#pragma unroll
+    for (int it = 0; it < VI; it++) {
+      const int vch = (tid >> 4) + it * 16;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int kv = min(kb * 64 + vq * 4 + i, last_key);
+        vst[it][i] = vch < HC ? *reinterpret_cast<const i32x4*>(vbase + (int64_t)kv * H + vch * 8) : zero4;
+      }
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < NJ; i++) {
+      const int idx = tid + i * 256;
+      *reinterpret_cast<i32x4*>(ks + (idx / CH) * KP + (idx % CH) * 8) = kst[i];
+    }
+#pragma unroll
+    for (int it = 0; it < VI; it++) {
+      const int vch = (tid >> 4) + it * 16;
+      if (vch < CH) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+          const uint32_t lo = __builtin_amdgcn_perm((uint32_t)vst[it][1][e >> 1], (uint32_t)vst[it][0][e >> 1], sel);
+          const uint32_t hi = __builtin_amdgcn_perm((uint32_t)vst[it][3][e >> 1], (uint32_t)vst[it][2][e >> 1], sel);
+          *reinterpret_cast<uint2*>(vt + (vch * 8 + e) * VP + vq * 4) = make_uint2(lo, hi);
+        }
+      }
+    }
+  };
+
+  const float scale2 = p.scale * 1.44269504f;
+  float m[QG], l[QG];
+  f32x4 acc[QG][NDT];
+#pragma unroll
+  for (int qg = 0; qg < QG; qg++) {
+    m[qg] = -3.0e38f;
+    l[qg] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++)
+      acc[qg][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int nkb = (p.past + min(qblk * QB + QB - 1, p.S - 1)) / 64 + 1;
+  load_tile(0);
+  for (int kb = 0; kb < nkb; kb++) {
+    __syncthreads(); // the previous tile has been read by every wave
+    store_tile();
+    __syncthreads();
+    if (kb + 1 < nkb)
+      load_tile(kb + 1); // in flight during the arithmetic below
+
+    f32x4 sc[QG][4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+#pragma unroll
+      for (int qg = 0; qg < QG; qg++)
+        sc[qg][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < NJ; j++) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks + (t * 16 + c) * KP + j * 32 + g * 8);
+#pragma unroll
+        for (int qg = 0; qg < QG; qg++)
+          sc[qg][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[qg][j], sc[qg][t], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int qg = 0; qg < QG; qg++)
+#pragma unroll
+      for (int t = 0; t < 4; t++)
+        sc[qg][t] *= scale2;
+    if (mrow) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int key = kb * 64 + (i >> 2) * 16 + g * 4 + (i & 3);
+        const float mk = key < p.mask_ld ? bf16_bits_to_f32(mrow[key]) * 1.44269504f : 0.f;
+#pragma unroll
+        for (int qg = 0; qg < QG; qg++)
+          sc[qg][i >> 2][i & 3] += mk;
+      }
+    }
+    bf16x8 pb[QG][2];
+    const bool edge = kb * 64 + 63 > p.past + q0;
+#pragma unroll
+    for (int qg = 0; qg < QG; qg++) {
+      if (edge) {
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const int key = kb * 64 + t * 16 + g * 4 + r;
+            sc[qg][t][r] = key <= qpos[qg] ? sc[qg][t][r] : -INFINITY;
+          }
+      }
+      float mx = -3.0e38f;
+#pragma unroll
+      for (int t = 0; t < 4; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          mx = fmaxf(mx, sc[qg][t][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float mn = fmaxf(m[qg], mx);
+      const float alpha = __builtin_amdgcn_exp2f(m[qg] - mn);
+      l[qg] *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++)
+        acc[qg][dt] *= alpha;
+#pragma unroll
+      for (int u = 0; u < 2; u++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const float pr = __builtin_amdgcn_exp2f(sc[qg][2 * u + (j >> 2)][j & 3] - mn);
+          l[qg] += pr;
+          pb[qg][u][j] = (__bf16)pr;
+        }
+      m[qg] = mn;
+    }
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+      for (int u = 0; u < 2; u++) {
+        const uint16_t* vrow = vt + (dt * 16 + c) * VP + u * 32 + g * 4;
+        const uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 16);
+        const i32x4 av = {(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
+#pragma unroll
+        for (int qg = 0; qg < QG; qg++)
+          acc[qg][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), pb[qg][u], acc[qg][dt], 0, 0, 0);
+      }
+  }
+#pragma unroll
+  for (int qg = 0; qg < QG; qg++) {
+    float ls = l[qg];
+    ls += __shfl_xor(ls, 16);
+    ls += __shfl_xor(ls, 32);
+    const int qi = q0 + qg * 16 + c;
+    if (qi < p.S) {
+      uint16_t* orow = p.out + (((int64_t)b * p.S + qi) * p.Nq + hq) * H;
+#pragma unroll
+      for (int dt = 0; dt < NDT; dt++) {
+        if (dt * 16 + g * 4 < H) { // H is a multiple of 8: the four dims of this lane exist together
+          uint32_t w[2];
+#pragma unroll
+          for (int h = 0; h < 2; h++)
+            w[h] = f32_to_bf16_bits(ls > 0.f ? acc[qg][dt][2 * h] / ls : 0.f) |
+                   (f32_to_bf16_bits(ls > 0.f ? acc[qg][dt][2 * h + 1] / ls : 0.f) << 16);
+          *reinterpret_cast<uint2*>(orow + dt * 16 + g * 4) = make_uint2(w[0], w[1]);
+        }
       }
     }
   }
@@ -1303,9 +1509,10 @@ static int attn_decode_launch(const char* who, AttnParams& p, bool rot, int64_t 
 
 // ---------------------------------------------------------------------------
 // Attention for head sizes other than 128 (attn<T>, src/csrc/llm/attn.cpp:781-955, is generic in the head size; the
-// kernels above are built for 128): one kernel for the single-query step and for prompt passes, H a multiple of 8
-// up to 256, and a second kernel for the single-query step (below).  The first: one wave per (sequence, query token,
-// query head), four per workgroup, no barrier: 64 keys per trip,
+// kernels above are built for 128), H a multiple of 8 up to 256.  The single-query step runs on
+// attn_generic_rows_kernel below, prompt passes on attn_prefill_hd_kernel above; this first, plain kernel serves
+// both when those are switched off (TPPX_ATTN_GENERIC_ROWS=0, TPPX_ATTN_PREFILL_MFMA=0).  One wave per (sequence,
+// query token, query head), four per workgroup, no barrier: 64 keys per trip,
 // a lane takes the whole dot product of its key (16-byte loads along its row, the query as fp32 in wave-private
 // LDS, read as broadcasts), online softmax over the trip with the probabilities rounded to bf16 before they multiply
 // V and the normaliser summing the unrounded ones, then lanes turn to output dimensions (lane, lane + 64, ...) and
@@ -1678,7 +1885,7 @@ extern "C" int tppx_attn_prefill(const void* q, const void* kcache, const void* 
   TPPX_REQUIRE(past_len >= 0 && past_len + S <= Smax, TPPX_ESHAPE,
                "%s: %ld cached + %ld new keys exceed the cache capacity %ld", who, (long)past_len, (long)S, (long)Smax);
   TPPX_REQUIRE(!mask || mask_ld > 0, TPPX_EINVAL, "%s: mask given with mask_ld=%ld", who, (long)mask_ld);
-  if (H != 128) { // other head sizes: the plain kernel
+  if (H != 128 && env_int("TPPX_ATTN_PREFILL_MFMA", 1) == 0) { // other head sizes on the plain kernel
     AttnGenParams g;
     memset(&g, 0, sizeof(g));
     g.q = (const uint16_t*)q; g.kc = (const uint16_t*)kcache; g.vc = (const uint16_t*)vcache; g.mask = (const uint16_t*)mask;
@@ -1695,6 +1902,37 @@ extern "C" int tppx_attn_prefill(const void* q, const void* kcache, const void* 
   p.B = (int)B; p.S = (int)S; p.Nq = (int)Nq; p.Nkv = (int)Nkv; p.Smax = (int)Smax; p.mask_ld = (int)mask_ld;
   p.past = (int)past_len;
   p.scale = 1.0f / sqrtf((float)H);
+  p.H = (int)H;
+  if (H != 128) { // other head sizes: the same kernel over a padded head size
+    TPPX_REQUIRE(H >= 8 && H <= 256 && H % 8 == 0, TPPX_EUNSUPPORTED,
+                 "%s: head size %ld (multiples of 8 up to 256)", who, (long)H);
+    const int hd = H <= 64 ? 64 : H <= 128 ? 128 : 256;
+    const long wgs2h = ((S + 127) / 128) * B * Nq;
+    const bool two = hd != 256 && S > 64 && env_int("TPPX_ATTN_QG", wgs2h >= 512 ? 2 : 1) == 2;
+    const size_t lds = (size_t)(64 * (hd + 8) + hd * AP_VP) * sizeof(uint16_t);
+    const dim3 grid((unsigned)((S + (two ? 127 : 63)) / (two ? 128 : 64)), (unsigned)(B * Nq));
+    hipError_t e = hipSuccess;
+#define TPPX_AP_HD(QG_, HD_)                                                                                          \
+  do {                                                                                                               \
+    e = allow_dynamic_lds(reinterpret_cast<const void*>(attn_prefill_hd_kernel<QG_, HD_>), lds);                     \
+    if (e == hipSuccess)                                                                                             \
+      attn_prefill_hd_kernel<QG_, HD_><<<grid, dim3(256), lds, (hipStream_t)stream>>>(p);                            \
+  } while (0)
+    if (hd == 64 && two)
+      TPPX_AP_HD(2, 64);
+    else if (hd == 64)
+      TPPX_AP_HD(1, 64);
+    else if (hd == 128 && two)
+      TPPX_AP_HD(2, 128);
+    else if (hd == 128)
+      TPPX_AP_HD(1, 128);
+    else
+      TPPX_AP_HD(1, 256);
+#undef TPPX_AP_HD
+    if (e != hipSuccess)
+      return check_hip(e, who);
+    return check_hip(hipGetLastError(), who);
+  }
   // 32 queries per wave (QG = 2) halve the LDS reads per MFMA at 226 registers, still two waves per SIMD; they win
   // when the launch still has two workgroups per CU (S = 2048, 32 heads: 97 us against 117 us; 16 x 128 queries
   // behind 1024 cached keys: 69 against 96 us) and lose below that (S = 512, 32 heads: 22.5 against 17 us)
