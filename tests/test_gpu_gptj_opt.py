@@ -49,7 +49,7 @@ def test_layer_norm(K, pdt):
         F.lyr_norm(x.cuda(), g.cuda(), b.float().cuda() if pdt == torch.bfloat16 else b.bfloat16().cuda(), 1e-5)
 
 
-@pytest.mark.parametrize("H,HR", [(128, 64), (256, 64), (64, 64), (32, 16)])
+@pytest.mark.parametrize("H,HR", [(128, 64), (256, 64), (64, 64), (32, 16), (80, 32), (200, 64)])
 def test_rotary_gptj(H, HR):
     F = _gj()
     B, S, N, MP = 2, 5, 3, 64
@@ -203,7 +203,7 @@ def _dequantized_copy(ref_model, weight_dtype):
         for m in ref_model.modules():
             if isinstance(m, torch.nn.Linear):
                 w = m.weight.data.to(torch.bfloat16).float()
-                if w.shape[0] % 32 == 0 and w.shape[1] % 256 == 0 and getattr(m, "_quantize_me", True):
+                if w.shape[0] % 32 == 0 and w.shape[1] % 128 == 0 and getattr(m, "_quantize_me", True):
                     if weight_dtype == "mxfp4":
                         q, sc = O.remap_quantize_mxfp4(w.numpy())
                         w = torch.from_numpy(O.dequantize_mxfp4_plain(q, sc))
@@ -271,14 +271,14 @@ def test_optimize_model_for_gptj_against_transformers(weight_dtype):
 
 
 @pytest.mark.parametrize("weight_dtype", ["mxfp4", "qint8"])
-@pytest.mark.parametrize("before,proj", [(True, 512), (False, 512), (True, 256)])
-def test_optimize_model_for_opt_against_transformers(weight_dtype, before, proj):
-    """OptimizeModelForOPT on a random-initialised transformers OPTForCausalLM (2 layers, 8 heads of 64; LayerNorm
-    before or after each half; with and without the project_in / project_out linears) against the stock model in
-    fp32 on the CPU holding the dequantized weights."""
+@pytest.mark.parametrize("before,proj,hidden", [(True, 512, 512), (False, 512, 512), (True, 256, 512), (True, 640, 640)])
+def test_optimize_model_for_opt_against_transformers(weight_dtype, before, proj, hidden):
+    """OptimizeModelForOPT on a random-initialised transformers OPTForCausalLM (2 layers, 8 heads of 64 -- or of 80,
+    a head size that is no power of two, as OPT-2.7B has; LayerNorm before or after each half; with and without the
+    project_in / project_out linears) against the stock model in fp32 on the CPU holding the dequantized weights."""
     transformers = pytest.importorskip("transformers")
     F = _opt()
-    cfg = transformers.OPTConfig(hidden_size=512, ffn_dim=1024, num_hidden_layers=2, num_attention_heads=8,
+    cfg = transformers.OPTConfig(hidden_size=hidden, ffn_dim=2 * hidden, num_hidden_layers=2, num_attention_heads=8,
                                  vocab_size=1024, max_position_embeddings=256, do_layer_norm_before=before,
                                  word_embed_proj_dim=proj, dropout=0.0, attention_dropout=0.0, layerdrop=0.0,
                                  bos_token_id=1, eos_token_id=2, pad_token_id=0, attn_implementation="eager",
@@ -331,3 +331,11 @@ def test_transformers_generate_on_optimized_models(family):
     assert out.shape == (2, 15) and torch.equal(out[:, :11], ids)
     ref = F.generate_greedy(opt, ids, 4, attention_mask=am)
     assert torch.equal(out, ref)
+    # the same tokens with the decode steps replayed from one graph (longer, so that the cache crosses a block of 32)
+    long_ref = F.generate_greedy(opt, ids, 30, attention_mask=am)
+    long_graph = F.generate_greedy_graph(opt, ids, 30, attention_mask=am)
+    assert long_graph.shape == (2, 41) and torch.equal(long_graph, long_ref)
+    assert torch.equal(F.generate_greedy_graph(opt, ids[:1], 1), F.generate_greedy(opt, ids[:1], 1))
+    from tpp_pytorch_extension._lib import TppxError
+    with pytest.raises(TppxError):
+        F.generate_greedy_graph(opt, ids, 400, attention_mask=am)  # 11 + 400 keys do not fit the cache of 256

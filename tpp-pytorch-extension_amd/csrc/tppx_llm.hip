@@ -1359,8 +1359,14 @@ extern "C" int tppx_layer_norm(const void* x, const void* gamma, const void* bet
 }
 
 static int rotary_common(const char* who, RotaryParams& p, hipStream_t stream) {
-  TPPX_REQUIRE(p.B > 0 && p.S > 0 && p.H >= 16 && p.H <= 512 && (p.H & (p.H - 1)) == 0, TPPX_ESHAPE,
-               "%s: bad shape B=%d S=%d H=%d (head size must be a power of two in 16..512)", who, p.B, p.S, p.H);
+  // Rotate-half pairs are two chunks of a head apart, read by one thread and written by another: both sit in one wave
+  // only when a head's chunks are a power of two (work items are numbered chunk-fastest).  GPT-J pairs lie inside a
+  // chunk and a plain append touches nothing twice, so those take any multiple of 8.
+  if (p.emb && !p.gptj)
+    TPPX_REQUIRE(p.H >= 16 && p.H <= 512 && (p.H & (p.H - 1)) == 0, TPPX_ESHAPE,
+                 "%s: head size %d (rotate-half rotation takes a power of two in 16..512)", who, p.H);
+  TPPX_REQUIRE(p.B > 0 && p.S > 0 && p.H >= 8 && p.H <= 512 && p.H % 8 == 0, TPPX_ESHAPE,
+               "%s: bad shape B=%d S=%d H=%d (head size must be a multiple of 8 up to 512)", who, p.B, p.S, p.H);
   if (p.emb)
     TPPX_REQUIRE(p.HR > 0 && p.HR <= p.H && p.HR % 16 == 0 && p.MP > 0, TPPX_ESHAPE,
                  "%s: rotary_dim=%d must be a multiple of 16 and <= H=%d", who, p.HR, p.H);

@@ -15,10 +15,10 @@ import torch
 from .. import _lib, _ops
 from .._lib import TppxError
 from .fused_llama_infer import (FormatSwitches, TppCache, check_layer_inputs, generate_greedy,  # noqa: F401
-                                rotate_append_attend)
+                                generate_greedy_graph, rotate_append_attend)
 
 __all__ = ["GPTJBlock", "FixGPTJBlock", "OptimizeModelForGPTJ", "GPTJModel_forward", "create_sinusoidal_positions",
-           "apply_rotary_pos_emb_gptj", "lyr_norm", "TppCache", "generate_greedy"]
+           "apply_rotary_pos_emb_gptj", "lyr_norm", "TppCache", "generate_greedy", "generate_greedy_graph"]
 
 lyr_norm = _ops.layer_norm  # lyr_norm (fused_llm_infer.cpp:254-306)
 
@@ -198,4 +198,5 @@ def OptimizeModelForGPTJ(model, dtype=torch.bfloat16, device="cuda", weight_dtyp
             m._tpp_ln_f = (m.ln_f.weight.data.to(torch.bfloat16).contiguous(),
                            m.ln_f.bias.data.to(torch.bfloat16).contiguous(), m.ln_f.eps)
             m.forward = types.MethodType(GPTJModel_forward, m)
+            m._tpp_core_model = True
     return model

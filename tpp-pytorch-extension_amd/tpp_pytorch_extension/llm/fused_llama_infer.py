@@ -734,6 +734,7 @@ def OptimizeModelForLlama(model, dtype=torch.bfloat16, device="cuda", weight_dty
             m._tpp_norm_weight = m.norm.weight.data.float().contiguous()
             m._tpp_norm_eps = m.norm.variance_epsilon
             m.forward = types.MethodType(LlamaModel_forward, m)
+            m._tpp_core_model = True
     return model
 
 
@@ -757,3 +758,71 @@ def generate_greedy(model, input_ids, max_new_tokens, attention_mask=None):
         if attention_mask is not None:
             attention_mask = torch.cat([attention_mask, attention_mask.new_ones((ids.shape[0], 1))], dim=1)
     return ids
+
+
+def generate_greedy_graph(model, input_ids, max_new_tokens, attention_mask=None):
+    """generate_greedy with the decode steps replayed from one HIP graph: the prompt runs as usual, then a single
+    step of the patched inner model (embedding, layers, final norm), the lm_head and the argmax is captured and
+    replayed max_new_tokens - 1 times.  What changes from step to step lives on the device: the current tokens, their
+    positions (counted over real tokens, as generate() derives them from the mask), the cache length, and an additive
+    key mask over the cache's whole capacity (0 everywhere but at the prompt's padding), so that no kernel argument
+    depends on the step.  Works on every model an OptimizeModelFor* of this package has patched; returns i64
+    [B][S + max_new_tokens], the same tokens as generate_greedy."""
+    from .llm_common import TppCache as HFTppCache
+    core = next((m for m in model.modules() if getattr(m, "_tpp_core_model", False)), None)
+    if core is None:
+        raise TppxError(_lib.EINVAL, "generate_greedy_graph: the model was not optimized by this package")
+    B, S = input_ids.shape
+    dev = input_ids.device
+    if attention_mask is None:
+        attention_mask = torch.ones_like(input_ids)
+    cap = core._tpp_kv_capacity
+    if S + max_new_tokens > cap:
+        raise TppxError(_lib.ESHAPE, f"generate_greedy_graph: {S} prompt + {max_new_tokens} new tokens exceed the "
+                                     f"cache capacity {cap}")
+    cache = HFTppCache(capacity=cap)
+    pos0 = attention_mask.long().cumsum(-1) - 1
+    pos0 = pos0.masked_fill(attention_mask == 0, 1)
+    out = model(input_ids=input_ids, attention_mask=attention_mask, position_ids=pos0, past_key_values=cache,
+                use_cache=True, logits_to_keep=1)
+    cur = out.logits[:, -1].argmax(dim=-1, keepdim=True)
+    ids = [input_ids, cur]
+    if max_new_tokens <= 1:
+        return torch.cat(ids[:1 + max_new_tokens], dim=1)
+    inner = cache.get_cpp()
+    # additive mask over the whole capacity: the lowest bf16 at the prompt's padding, 0 elsewhere (keys past the
+    # cache length are never read)
+    width = (inner.capacity + inner.block_size - 1) // inner.block_size * inner.block_size
+    smask = torch.zeros((B, width), dtype=torch.bfloat16, device=dev)
+    smask[:, :S].masked_fill_(attention_mask == 0, torch.finfo(torch.bfloat16).min)
+    cache.static_mask = smask
+    cur = cur.clone()
+    pos = (pos0[:, -1:] + 1).contiguous()
+    ones = torch.ones((B, 1), dtype=attention_mask.dtype, device=dev)
+
+    def step():
+        h = core(input_ids=cur, attention_mask=ones, position_ids=pos, past_key_values=cache, use_cache=True)
+        logits = model.lm_head(h.last_hidden_state[:, -1:])
+        return logits[:, -1].argmax(dim=-1, keepdim=True)
+
+    try:
+        # warm-up outside capture (allocations, lazy module loads), then the counters go back: the key it wrote at the
+        # cache's end is written again by the first replay
+        host_len = inner.get_seq_length()
+        step()
+        inner.seq_len_dev.sub_(1)
+        inner._advance_host(host_len - inner.get_seq_length())
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            nxt = step()  # (the patched forward moves the device counter itself)
+            cur.copy_(nxt)
+            pos.add_(1)
+        inner._advance_host(host_len - inner.get_seq_length())  # capture ran the host bookkeeping once, no kernels
+        for _ in range(max_new_tokens - 1):
+            graph.replay()
+            inner._advance_host(1)
+            ids.append(cur.clone())
+    finally:
+        cache.static_mask = None
+    return torch.cat(ids, dim=1)

@@ -15,10 +15,10 @@ import torch
 from .. import _lib, _ops
 from .._lib import TppxError
 from .fused_llama_infer import (FormatSwitches, TppCache, check_layer_inputs, generate_greedy,  # noqa: F401
-                                rotate_append_attend)
+                                generate_greedy_graph, rotate_append_attend)
 
 __all__ = ["OPTDecoderLayer", "FixOPTDecoderLayer", "OptimizeModelForOPT", "OPTDecoder_forward", "lyr_norm",
-           "TppCache", "generate_greedy"]
+           "TppCache", "generate_greedy", "generate_greedy_graph"]
 
 lyr_norm = _ops.layer_norm  # lyr_norm (fused_llm_infer.cpp:254-306)
 
@@ -186,4 +186,5 @@ def OptimizeModelForOPT(model, dtype=torch.bfloat16, device="cuda", weight_dtype
                 m._tpp_ln_f = (m.final_layer_norm.weight.data.to(torch.bfloat16).contiguous(),
                                m.final_layer_norm.bias.data.to(torch.bfloat16).contiguous(), m.final_layer_norm.eps)
             m.forward = types.MethodType(OPTDecoder_forward, m)
+            m._tpp_core_model = True
     return model

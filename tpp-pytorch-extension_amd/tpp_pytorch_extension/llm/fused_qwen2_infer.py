@@ -15,10 +15,11 @@ import torch
 from .. import _lib
 from .._lib import TppxError
 from . import fused_llama_infer as _llama
-from .fused_llama_infer import LlamaDecoderLayer, LlamaDecoderLayerModule, LlamaModel_forward, TppCache, generate_greedy  # noqa: F401
+from .fused_llama_infer import (LlamaDecoderLayer, LlamaDecoderLayerModule, LlamaModel_forward, TppCache,  # noqa: F401
+                                generate_greedy, generate_greedy_graph)
 
 __all__ = ["Qwen2DecoderLayer", "FixQwen2DecoderLayer", "OptimizeModelForQwen2", "Qwen2Model_forward", "TppCache",
-           "generate_greedy"]
+           "generate_greedy", "generate_greedy_graph"]
 
 
 class Qwen2DecoderLayer(LlamaDecoderLayer):
@@ -123,4 +124,5 @@ def OptimizeModelForQwen2(model, dtype=torch.bfloat16, device="cuda", weight_dty
             m._tpp_norm_weight = m.norm.weight.data.float().contiguous()
             m._tpp_norm_eps = m.norm.variance_epsilon
             m.forward = types.MethodType(Qwen2Model_forward, m)
+            m._tpp_core_model = True
     return model

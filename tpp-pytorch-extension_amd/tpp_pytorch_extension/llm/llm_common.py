@@ -233,6 +233,7 @@ class TppCache:
     def __init__(self, capacity=0, **kwargs):
         from .fused_llama_infer import TppCache as _CoreCache
         self.tpp_cache = _CoreCache(capacity)
+        self.static_mask = None  # an additive mask over the whole capacity that replaces the aligned one (graph replay)
 
     def __len__(self):
         return self.tpp_cache.size()
@@ -261,6 +262,8 @@ class TppCache:
             self.tpp_cache.crop(max_length)
 
     def align_and_invert_mask(self, mask, inputs_embeds):
+        if self.static_mask is not None:
+            return self.static_mask
         if mask is None:
             mask = torch.ones((inputs_embeds.shape[0], inputs_embeds.shape[1]), device=inputs_embeds.device,
                               dtype=torch.bfloat16)
