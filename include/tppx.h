@@ -427,7 +427,8 @@ int tppx_rms_norm(const void* x, const void* gamma, int gamma_dtype, void* y,
 
 /* Replaces apply_rotary_pos_emb_llama (src/csrc/llm/fused_llm_infer.cpp:207-253):
  * in place on t bf16 [B][S][N][H]; emb_pos f32 [2][MP][HR] (cos, sin); pos i64
- * [B_pos][S] with B_pos 1 or B; positions >= MP are left untouched. */
+ * [B_pos][S] with B_pos 1 or B; positions >= MP are left untouched.  H a
+ * multiple of 8 up to 512, HR a multiple of 16. */
 int tppx_rotary_llama(void* t, const void* emb_pos, const void* pos, int64_t B,
                       int64_t S, int64_t N, int64_t H, int64_t MP, int64_t HR,
                       int64_t B_pos, tppx_stream_t stream);

@@ -39,10 +39,10 @@ def test_rms_norm(K, gdt):
     assert_close_bf16(t2bits(y).reshape(-1, K), t2bits(t.to(torch.bfloat16)).reshape(-1, K), what="rms_norm vs torch")
 
 
-@pytest.mark.parametrize("HR", [128, 64])
-def test_rotary_llama(HR):
+@pytest.mark.parametrize("H,HR", [(128, 128), (128, 64), (96, 96), (80, 32), (200, 80)])
+def test_rotary_llama(H, HR):
     F = _llm()
-    B, S, N, H, MP = 2, 5, 6, 128, 64
+    B, S, N, MP = 2, 5, 6, 64
     t = randn_bf16((B, S, N * H), 1.0, 21)
     emb = F.llama_rotary_table(MP, HR, device="cpu")
     pos = torch.tensor([[3, 9, 63, 64, 0], [1, 2, 3, 4, 70]], dtype=torch.int64)  # 64 and 70 are out of range: untouched

@@ -113,15 +113,17 @@ def test_unsupported_head_sizes_are_rejected():
         assert L.tppx_attn_prefill(A, A, A, None, 0, 0, A, 1, 8, 4, 4, H, 64, None) == _lib.EUNSUPPORTED
 
 
+@pytest.mark.parametrize("H", [64, 96])
 @pytest.mark.parametrize("S,past", [(1, 21), (40, 0), (7, 30)])
-def test_decoder_layer_with_64_wide_heads(S, past):
-    """LlamaDecoderLayer (src/csrc/llm/fused_llm_infer.cpp:1229-1275) with head size 64: rotary + cache append as
-    their own launch, attention on the plain kernel, MXFP4 linears; against the composition of the oracle
+def test_decoder_layer_with_64_wide_heads(S, past, H):
+    """LlamaDecoderLayer (src/csrc/llm/fused_llm_infer.cpp:1229-1275) with head size 64, and 96 (no power of two: the
+    rotate-half pairs of a head can straddle two waves of the rotary launch): rotary + cache append as their own
+    launch, attention on the kernels for other head sizes, MXFP4 linears; against the composition of the oracle
     functions (rel-L2 <= 2e-2 for the layer output, cached keys / values within 1 bf16 ulp)."""
     import tpp_pytorch_extension  # noqa: F401
     from tpp_pytorch_extension import _ops
     F = _llm()
-    HID, INTER, NQ, NKV, H, MP = 256, 512, 4, 2, 64, 256
+    HID, INTER, NQ, NKV, MP = 256, 512, 4, 2, 256
     shapes = [(NQ * H, HID), (NKV * H, HID), (NKV * H, HID), (HID, NQ * H), (INTER, HID), (INTER, HID), (HID, INTER)]
     Ws = [randn_bf16(s, 0.05, 910 + i) for i, s in enumerate(shapes)]
     rng = torch.Generator().manual_seed(91)

@@ -226,16 +226,35 @@ rotary_append_kernel(const RotaryParams p) {
     // this chunk holds first halves (h0 < HR/2) or second halves of rotation pairs
     const bool first = h0 < coff;
     const int h2 = first ? h0 : h0 - coff;
-    const uint4 wo = reinterpret_cast<const uint4*>(row)[first ? c + (coff >> 3) : c - (coff >> 3)];
+    const int cp = first ? c + (coff >> 3) : c - (coff >> 3); // the partner chunk
+    const uint4 wo = reinterpret_cast<const uint4*>(row)[cp];
     float a[8], o[8], r[8];
     unpack8(w, a);
     unpack8(wo, o);
     const float* cs = p.emb + pp * p.HR + h2;
     const float* sn = p.emb + ((int64_t)p.MP + pp) * p.HR + h2;
+    if ((CH & (CH - 1)) != 0) {
+      // A head of a number of chunks that is no power of two can straddle two waves, and the partner thread in the
+      // other wave might read this chunk after it has been rewritten: the thread of the first half writes both
+      // chunks here, the thread of the second half writes nothing.
+      if (!first)
+        return;
+      float r2[8];
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-      // first half: in0*cos - in1*sin ; second half: in1*cos + in0*sin
-      r[e] = first ? a[e] * cs[e] - o[e] * sn[e] : a[e] * cs[e] + o[e] * sn[e];
+      for (int e = 0; e < 8; e++) {
+        r[e] = a[e] * cs[e] - o[e] * sn[e];
+        r2[e] = o[e] * cs[e] + a[e] * sn[e];
+      }
+      const uint4 w2 = pack8(r2);
+      reinterpret_cast<uint4*>(row)[cp] = w2;
+      if (is_k && p.kc && off + s < p.Smax)
+        reinterpret_cast<uint4*>(p.kc + (((int64_t)b * p.Nkv + n) * p.Smax + off + s) * p.H)[cp] = w2;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        // first half: in0*cos - in1*sin ; second half: in1*cos + in0*sin
+        r[e] = first ? a[e] * cs[e] - o[e] * sn[e] : a[e] * cs[e] + o[e] * sn[e];
+      }
     }
     w = pack8(r);
   }
@@ -1359,12 +1378,6 @@ extern "C" int tppx_layer_norm(const void* x, const void* gamma, const void* bet
 }
 
 static int rotary_common(const char* who, RotaryParams& p, hipStream_t stream) {
-  // Rotate-half pairs are two chunks of a head apart, read by one thread and written by another: both sit in one wave
-  // only when a head's chunks are a power of two (work items are numbered chunk-fastest).  GPT-J pairs lie inside a
-  // chunk and a plain append touches nothing twice, so those take any multiple of 8.
-  if (p.emb && !p.gptj)
-    TPPX_REQUIRE(p.H >= 16 && p.H <= 512 && (p.H & (p.H - 1)) == 0, TPPX_ESHAPE,
-                 "%s: head size %d (rotate-half rotation takes a power of two in 16..512)", who, p.H);
   TPPX_REQUIRE(p.B > 0 && p.S > 0 && p.H >= 8 && p.H <= 512 && p.H % 8 == 0, TPPX_ESHAPE,
                "%s: bad shape B=%d S=%d H=%d (head size must be a multiple of 8 up to 512)", who, p.B, p.S, p.H);
   if (p.emb)
