@@ -535,7 +535,7 @@ def test_rms_norm_from_row_sums(M, Kprod, N):
     assert_close_bf16(t2bits(fz), t2bits(_ops.swiglu_gate_up(hn, ws[1], ws[2])), ulps=2, what=f"norm from row sums, swiglu M={M}")
 
 
-@pytest.mark.parametrize("weight_dtype", ["mxfp4", "qint8"])
+@pytest.mark.parametrize("weight_dtype", ["mxfp4", "qint8", "bf16"])
 def test_optimize_model_for_llama_against_transformers(weight_dtype):
     """OptimizeModelForLlama on a random-initialised transformers LlamaForCausalLM (2 layers, GQA 4/2 heads of
     128): the logits of the prompt pass and of two decode steps against the stock transformers model in fp32 on
@@ -557,12 +557,15 @@ def test_optimize_model_for_llama_against_transformers(weight_dtype):
                 if weight_dtype == "mxfp4":
                     q, sc = O.remap_quantize_mxfp4(w.numpy())
                     m.weight.data.copy_(torch.from_numpy(O.dequantize_mxfp4_plain(q, sc)))
-                else:
+                elif weight_dtype == "qint8":
                     q, sc, _ = O.remap_quantize_qint8(w.numpy())
                     m.weight.data.copy_(torch.from_numpy(O.dequantize_qint8_plain(q, sc)))
+                else:
+                    m.weight.data.copy_(w)
             elif isinstance(m, torch.nn.Embedding):
                 m.weight.data.copy_(m.weight.data.to(torch.bfloat16).float())
-    opt_model = F.OptimizeModelForLlama(copy.deepcopy(ref_model), torch.bfloat16, "cuda", weight_dtype).eval()
+    opt_model = F.OptimizeModelForLlama(copy.deepcopy(ref_model), torch.bfloat16, "cuda",
+                                        None if weight_dtype == "bf16" else weight_dtype).eval()
     assert not opt_model.lm_head.weight.is_quantized and opt_model.lm_head.weight.dim() == 5  # bf16, as the reference's
     tol = 3e-2 if weight_dtype == "mxfp4" else 6e-2
 

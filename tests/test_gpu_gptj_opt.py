@@ -203,7 +203,7 @@ def _dequantized_copy(ref_model, weight_dtype):
         for m in ref_model.modules():
             if isinstance(m, torch.nn.Linear):
                 w = m.weight.data.to(torch.bfloat16).float()
-                if w.shape[0] % 32 == 0 and w.shape[1] % 128 == 0 and getattr(m, "_quantize_me", True):
+                if w.shape[0] % 32 == 0 and w.shape[1] % 128 == 0 and getattr(m, "_quantize_me", True) and weight_dtype != "bf16":
                     if weight_dtype == "mxfp4":
                         q, sc = O.remap_quantize_mxfp4(w.numpy())
                         w = torch.from_numpy(O.dequantize_mxfp4_plain(q, sc))
@@ -251,7 +251,7 @@ def _compare_with_stock(ref_model, opt_model, tol, vocab, generate):
     assert out.shape == (1, 24) and torch.equal(out[:, :19].cpu(), ids[:1])
 
 
-@pytest.mark.parametrize("weight_dtype", ["mxfp4", "qint8"])
+@pytest.mark.parametrize("weight_dtype", ["mxfp4", "qint8", "bf16"])
 def test_optimize_model_for_gptj_against_transformers(weight_dtype):
     """OptimizeModelForGPTJ on a random-initialised transformers GPTJForCausalLM (2 blocks, 4 heads of 128, rotary
     on 64 dims) against the stock model in fp32 on the CPU holding the dequantized weights.  The stock model is
@@ -265,12 +265,13 @@ def test_optimize_model_for_gptj_against_transformers(weight_dtype):
     ref_model = transformers.GPTJForCausalLM(cfg).eval()
     ref_model.lm_head._quantize_me = False
     _dequantized_copy(ref_model, weight_dtype)
-    opt_model = F.OptimizeModelForGPTJ(copy.deepcopy(ref_model), torch.bfloat16, "cuda", weight_dtype).eval()
+    opt_model = F.OptimizeModelForGPTJ(copy.deepcopy(ref_model), torch.bfloat16, "cuda",
+                                       None if weight_dtype == "bf16" else weight_dtype).eval()
     assert type(opt_model.transformer.h[0].cpp_block).__name__ == "GPTJBlock"
     _compare_with_stock(ref_model, opt_model, 3e-2 if weight_dtype == "mxfp4" else 6e-2, 1600, F.generate_greedy)
 
 
-@pytest.mark.parametrize("weight_dtype", ["mxfp4", "qint8"])
+@pytest.mark.parametrize("weight_dtype", ["mxfp4", "qint8", "bf16"])
 @pytest.mark.parametrize("before,proj,hidden", [(True, 512, 512), (False, 512, 512), (True, 256, 512), (True, 640, 640)])
 def test_optimize_model_for_opt_against_transformers(weight_dtype, before, proj, hidden):
     """OptimizeModelForOPT on a random-initialised transformers OPTForCausalLM (2 layers, 8 heads of 64 -- or of 80,
@@ -290,7 +291,8 @@ def test_optimize_model_for_opt_against_transformers(weight_dtype, before, proj,
         ref_model.model.decoder.project_in._quantize_me = False
         ref_model.model.decoder.project_out._quantize_me = False
     _dequantized_copy(ref_model, weight_dtype)
-    opt_model = F.OptimizeModelForOPT(copy.deepcopy(ref_model), torch.bfloat16, "cuda", weight_dtype).eval()
+    opt_model = F.OptimizeModelForOPT(copy.deepcopy(ref_model), torch.bfloat16, "cuda",
+                                      None if weight_dtype == "bf16" else weight_dtype).eval()
     assert type(opt_model.model.decoder.layers[0].cpp_block).__name__ == "OPTDecoderLayer"
     _compare_with_stock(ref_model, opt_model, 3e-2 if weight_dtype == "mxfp4" else 6e-2, 1024, F.generate_greedy)
 

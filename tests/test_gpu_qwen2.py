@@ -110,7 +110,7 @@ def test_qwen2_decoder_layer_parameter_list():
         F.Qwen2DecoderLayer([None] * 10, 0, 1e-5, 128, 256, 128)
 
 
-@pytest.mark.parametrize("weight_dtype", ["mxfp4", "qint8"])
+@pytest.mark.parametrize("weight_dtype", ["mxfp4", "qint8", "bf16"])
 def test_optimize_model_for_qwen2_against_transformers(weight_dtype):
     """OptimizeModelForQwen2 on a random-initialised transformers Qwen2ForCausalLM (2 layers, GQA 4/2 heads of 128,
     q/k/v biases drawn at N(0, 0.5) so that they matter): logits of the prompt pass and of two decode steps against
@@ -131,15 +131,18 @@ def test_optimize_model_for_qwen2_against_transformers(weight_dtype):
                 if weight_dtype == "mxfp4":
                     q, sc = O.remap_quantize_mxfp4(w.numpy())
                     m.weight.data.copy_(torch.from_numpy(O.dequantize_mxfp4_plain(q, sc)))
-                else:
+                elif weight_dtype == "qint8":
                     q, sc, _ = O.remap_quantize_qint8(w.numpy())
                     m.weight.data.copy_(torch.from_numpy(O.dequantize_qint8_plain(q, sc)))
+                else:
+                    m.weight.data.copy_(w)
                 if m.bias is not None:
                     m.bias.data.copy_((torch.randn_like(m.bias) * 0.5).to(torch.bfloat16).float())
             elif isinstance(m, torch.nn.Embedding):
                 m.weight.data.copy_(m.weight.data.to(torch.bfloat16).float())
     assert ref_model.model.layers[0].self_attn.q_proj.bias is not None
-    opt_model = F.OptimizeModelForQwen2(copy.deepcopy(ref_model), torch.bfloat16, "cuda", weight_dtype).eval()
+    opt_model = F.OptimizeModelForQwen2(copy.deepcopy(ref_model), torch.bfloat16, "cuda",
+                                        None if weight_dtype == "bf16" else weight_dtype).eval()
     assert type(opt_model.model.layers[0].cpp_block).__name__ == "Qwen2DecoderLayer"
     tol = 3e-2 if weight_dtype == "mxfp4" else 6e-2
 
@@ -175,4 +178,9 @@ def test_optimize_model_for_qwen2_against_transformers(weight_dtype):
     cfg_sw = copy.deepcopy(cfg)
     cfg_sw.use_sliding_window = True
     with pytest.raises(NotImplementedError):
-        F.OptimizeModelForQwen2(transformers.Qwen2ForCausalLM(cfg_sw), torch.bfloat16, "cuda", weight_dtype)
+        F.OptimizeModelForQwen2(transformers.Qwen2ForCausalLM(cfg_sw), torch.bfloat16, "cuda",
+                                "bfloat16" if weight_dtype == "bf16" else weight_dtype)
+    # an unquantized format that the bf16 blocks cannot hold is refused by name
+    from tpp_pytorch_extension._lib import TppxError
+    with pytest.raises(TppxError):
+        F.OptimizeModelForQwen2(transformers.Qwen2ForCausalLM(cfg), torch.bfloat16, "cuda", "float32")

@@ -163,16 +163,16 @@ def GPTJModel_forward(self, input_ids=None, past_key_values=None, attention_mask
     return BaseModelOutputWithPast(last_hidden_state=hidden_states, past_key_values=past_key_values)
 
 
-def OptimizeModelForGPTJ(model, dtype=torch.bfloat16, device="cuda", weight_dtype="mxfp4"):
+def OptimizeModelForGPTJ(model, dtype=torch.bfloat16, device="cuda", weight_dtype=None):
     """fused_gptj_infer.py:175-193 for one GPU: every GPTJBlock fused, the lm_head turned into a BlockedLinear with
     the reference's 100 x 64 blocking (64 x 64 when the vocabulary does not divide), GPTJModel.forward of this
-    instance replaced.  As for Llama, the blocks' linears must be quantized (weight_dtype "mxfp4" or "qint8") and the
-    KV cache holds TPPX_KV_CAPACITY keys per sequence (default: the model's n_positions)."""
+    instance replaced.  weight_dtype as for Llama (None = bf16 weights, "mxfp4", "qint8", "qint2"); the KV cache
+    holds TPPX_KV_CAPACITY keys per sequence (default: the model's n_positions)."""
     import transformers
     from .llm_common import FixLinear
     gj = transformers.models.gptj.modeling_gptj
-    if weight_dtype not in ("mxfp4", "qint8"):
-        raise TppxError(_lib.EUNSUPPORTED, f"OptimizeModelForGPTJ: weight_dtype {weight_dtype!r} (only quantized linears are built)")
+    from .fused_llama_infer import layer_weight_dtype
+    weight_dtype = layer_weight_dtype("OptimizeModelForGPTJ", weight_dtype, dtype)
     tables = {}
     for name, m in model.named_modules():  # before the cast: the sin | cos tables are fp32 buffers
         if isinstance(m, gj.GPTJAttention):

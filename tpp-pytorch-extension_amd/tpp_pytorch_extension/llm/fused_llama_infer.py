@@ -343,7 +343,7 @@ class FormatSwitches:
 class LlamaDecoderLayer(FormatSwitches):
     """torch.classes.tpp_llm.LlamaDecoderLayer(params, layer_idx, eps, H, max_positions, rotary_dim)
     with params = [ln_in gamma, Wq, Wk, Wv, Wo, ln_post gamma, Wg, Wu, Wd, embed_positions]
-    (fused_llm_infer.cpp:1096-1110); the linears are quantized tensors of this package."""
+    (fused_llm_infer.cpp:1096-1110); the linears are quantized tensors of this package or blocked bf16 weights."""
 
     _weight_names = ("t_Wq", "t_Wk", "t_Wv", "t_Wp", "t_Wg", "t_Wu", "t_Wd")
 
@@ -686,18 +686,31 @@ def LlamaModel_forward(self, input_ids=None, attention_mask=None, position_ids=N
     return BaseModelOutputWithPast(last_hidden_state=hidden_states, past_key_values=past_key_values)
 
 
-def OptimizeModelForLlama(model, dtype=torch.bfloat16, device="cuda", weight_dtype="mxfp4", quantize_lm_head=False):
+def layer_weight_dtype(who, weight_dtype, dtype):
+    """The weight_dtype argument of the reference's OptimizeModelFor* (None = the layer dtype; a torch dtype or its
+    name; "mxfp4" / "qint8" / "qint2", run_generation.py:68-75) as FixLinear takes it.  The fused blocks compute in
+    bf16, so an unquantized format other than bf16 is refused."""
+    if weight_dtype is None:
+        weight_dtype = dtype
+    if isinstance(weight_dtype, str) and weight_dtype not in ("mxfp4", "qint8", "qint2"):
+        weight_dtype = getattr(torch, weight_dtype, weight_dtype)
+    if weight_dtype in ("mxfp4", "qint8", "qint2") or weight_dtype == torch.bfloat16:
+        return weight_dtype
+    raise TppxError(_lib.EUNSUPPORTED, f"{who}: weight_dtype {weight_dtype!r} (bfloat16, mxfp4, qint8 or qint2)")
+
+
+def OptimizeModelForLlama(model, dtype=torch.bfloat16, device="cuda", weight_dtype=None, quantize_lm_head=False):
     """fused_llama_infer.py:176-226 for one GPU: the rotary table from the model's own rotary_emb, every
     LlamaDecoderLayer fused, every remaining nn.Linear (the lm_head) turned into a BlockedLinear with the
     reference's blocking (100 x 64 where the vocabulary allows, else 64 x 64) and bf16 weights, LlamaModel.forward
     of this instance replaced.  quantize_lm_head: True / "qint8" / "mxfp4" quantizes the lm_head as well
     (run_generation.py:277-282 does it with remap_and_quantize_qint8 after the call; that works here too).
-    Differences: the decoder layers' linears must be quantized (weight_dtype "mxfp4" or "qint8") and the KV cache
-    is allocated for TPPX_KV_CAPACITY keys per sequence (default: the model's max_position_embeddings)."""
+    weight_dtype as in the reference: None = the layers keep bf16 weights (and quantize them themselves under
+    USE_MXFP4 / USE_QINT8 / USE_QINT2), or "mxfp4" / "qint8" / "qint2".  Difference: the KV cache is allocated for
+    TPPX_KV_CAPACITY keys per sequence (default: the model's max_position_embeddings)."""
     import transformers
     from .llm_common import FixLinear
-    if weight_dtype not in ("mxfp4", "qint8"):
-        raise TppxError(_lib.EUNSUPPORTED, f"OptimizeModelForLlama: weight_dtype {weight_dtype!r} (only quantized linears are built)")
+    weight_dtype = layer_weight_dtype("OptimizeModelForLlama", weight_dtype, dtype)
     if getattr(model.config, "attention_bias", False):
         raise NotImplementedError("attention_bias is not supported for Llama yet!")
     model.config._attn_implementation = "tpp"

@@ -158,16 +158,16 @@ def OPTDecoder_forward(self, input_ids=None, attention_mask=None, past_key_value
     return BaseModelOutputWithPast(last_hidden_state=hidden_states, past_key_values=past_key_values)
 
 
-def OptimizeModelForOPT(model, dtype=torch.bfloat16, device="cuda", weight_dtype="mxfp4"):
+def OptimizeModelForOPT(model, dtype=torch.bfloat16, device="cuda", weight_dtype=None):
     """fused_opt_infer.py:175-203 for one GPU: every OPTDecoderLayer fused, every remaining nn.Linear (lm_head,
     project_in / project_out) turned into a bf16 BlockedLinear with 16 x 64 blocking as the reference does,
-    OPTDecoder.forward of this instance replaced.  The layers' linears must be quantized (weight_dtype "mxfp4" or
-    "qint8"); the KV cache holds TPPX_KV_CAPACITY keys per sequence (default: max_position_embeddings)."""
+    OPTDecoder.forward of this instance replaced.  weight_dtype as for Llama (None = bf16 weights, "mxfp4", "qint8",
+    "qint2"); the KV cache holds TPPX_KV_CAPACITY keys per sequence (default: max_position_embeddings)."""
     import transformers
     from .llm_common import FixLinear
     op = transformers.models.opt.modeling_opt
-    if weight_dtype not in ("mxfp4", "qint8"):
-        raise TppxError(_lib.EUNSUPPORTED, f"OptimizeModelForOPT: weight_dtype {weight_dtype!r} (only quantized linears are built)")
+    from .fused_llama_infer import layer_weight_dtype
+    weight_dtype = layer_weight_dtype("OptimizeModelForOPT", weight_dtype, dtype)
     for i, l in enumerate(model.model.decoder.layers):
         if not hasattr(l.self_attn, "layer_idx") or l.self_attn.layer_idx is None:
             l.self_attn.layer_idx = i

@@ -78,17 +78,17 @@ def FixQwen2DecoderLayer(self, bk=None, bc=None, layer_dtype=torch.bfloat16, wei
 Qwen2Model_forward = LlamaModel_forward  # fused_qwen2_infer.py:240-340: the same walk over the layers on a TppCache
 
 
-def OptimizeModelForQwen2(model, dtype=torch.bfloat16, device="cuda", weight_dtype="mxfp4", quantize_lm_head=False):
+def OptimizeModelForQwen2(model, dtype=torch.bfloat16, device="cuda", weight_dtype=None, quantize_lm_head=False):
     """fused_qwen2_infer.py:180-238 for one GPU: the rotary table from the model's own rotary_emb, every
     Qwen2DecoderLayer fused, the remaining nn.Linear (the lm_head) turned into a BlockedLinear, Qwen2Model.forward of
-    this instance replaced.  Sliding-window attention is refused as in the reference (:184-187).  As for Llama, the
-    decoder layers' linears must be quantized (weight_dtype "mxfp4" or "qint8") and the KV cache holds
-    TPPX_KV_CAPACITY keys per sequence (default: the model's max_position_embeddings)."""
+    this instance replaced.  Sliding-window attention is refused as in the reference (:184-187).  weight_dtype as for
+    Llama (None = bf16 weights, "mxfp4", "qint8", "qint2"); the KV cache holds TPPX_KV_CAPACITY keys per sequence
+    (default: the model's max_position_embeddings)."""
     import transformers
     from .llm_common import FixLinear
     q2 = transformers.models.qwen2.modeling_qwen2
-    if weight_dtype not in ("mxfp4", "qint8"):
-        raise TppxError(_lib.EUNSUPPORTED, f"OptimizeModelForQwen2: weight_dtype {weight_dtype!r} (only quantized linears are built)")
+    from .fused_llama_infer import layer_weight_dtype
+    weight_dtype = layer_weight_dtype("OptimizeModelForQwen2", weight_dtype, dtype)
     if getattr(model.config, "use_sliding_window", False):
         raise NotImplementedError("use_sliding_window is not supported for Qwen2 yet!")
     model.config._attn_implementation = "tpp"
