@@ -722,6 +722,65 @@ def leg_cfg4(torch, _ops, args, pfmt="mxfp4", fp8=False, cpu=True):
     }
 
 
+def leg_w4a8(torch, _ops, args):
+    """The reference's USE_MXFP4_INT8 mode (W4A8: MXFP4 weights as integers x int8 activations over blocks of 32,
+    src/csrc/fused_gemm.h:965-978) on the linears of config 4's layer at M = 2048, one fc_plain / fc_add call per
+    weight (the mode has no fused q/k/v or gate/up launch).  Not a BASELINE configuration; run alone with
+    --workload w4a8."""
+    dev = torch.device("cuda:0")
+    M, H, I = CFG4_DIMS
+    g = torch.Generator(device=dev).manual_seed(1239)
+
+    def mk(N, K):
+        W = (torch.randn((N, K), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        q = _ops.remap_and_quantize_mxfp4(W.view(N // 16, 16, K // 64, 32, 2).permute(0, 2, 3, 1, 4).contiguous(),
+                                          int8_layout=True)
+        q.native_w4a8_wide()
+        return q
+
+    shapes = [("qkv", 10240, H), ("o", H, H), ("gate", I, H), ("up", I, H), ("down", H, I)]
+    ws = {name: mk(N, K) for name, N, K in shapes}
+    xs = {H: torch.randn((M, H), generator=g, device=dev).to(torch.bfloat16),
+          I: torch.randn((M, I), generator=g, device=dev).to(torch.bfloat16)}
+    res = torch.randn((M, H), generator=g, device=dev).to(torch.bfloat16)
+    empty = torch.empty(0, dtype=torch.bfloat16, device=dev)
+
+    def call(name, K):
+        if name in ("o", "down"):
+            return torch.ops.tpp_llm.fc_add(xs[K], ws[name], empty, res, 1.0)
+        return torch.ops.tpp_llm.fc_plain(xs[K], ws[name], empty, -1, [])
+
+    def step(_i=0):
+        return [call(name, K) for name, _, K in shapes]
+
+    flops = sum(2.0 * M * N * K for _, N, K in shapes)
+    ms, blocks = time_blocks(torch, step, 3, 2)
+    peak = PEAKS_TFLOPS["bf16"]  # the block sums run on the bf16 MFMA
+    rows = []
+    for name, N, K in shapes:
+        us, n = events_us(torch, lambda st, name=name, K=K: call(name, K), 1, use_graph=False)
+        fl = 2.0 * M * N * K
+        rows.append({"kernel": "tppx::linear_w4a8_wide_kernel", "call": f"{name} M={M} N={N} K={K} (row quantizer included)",
+                     "kernels_per_call": 2, "avg_launch_us": round(us, 1), "flops_per_launch": fl,
+                     "bytes_per_launch": 2 * N * K + 2 * M * K + 2 * M * N, "achieved": round(fl / us / 1e6, 1),
+                     "frac": round(fl / us / 1e6 / peak, 4), "launches_timed": n})
+    dom = max(rows, key=lambda r: r["avg_launch_us"])
+    return {
+        "leg": "w4a8", "metric": "quant-GEMM TFLOP/s (prefill)", "value": round(flops / (ms * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s", "ms_per_step": round(ms, 4), "dtype": "int8 activations x 4-bit weights (exact block sums on the bf16 MFMA)",
+        "workload": "config 4's layer under the reference's USE_MXFP4_INT8 mode (W4A8), M = 2048: one call per weight "
+                    "(q/k/v as one 10240-channel weight, o, gate, up, down); eager op calls; not a BASELINE configuration",
+        "flops_per_step": flops,
+        "roofline": {"bound": "mfma", "kernel": dom["kernel"], "call": dom["call"], "achieved": dom["achieved"],
+                     "peak": peak, "unit": "TFLOP/s", "frac": dom["frac"], "traffic": None,
+                     "avg_launch_us": dom["avg_launch_us"], "flops_per_launch": dom["flops_per_launch"],
+                     "bytes_per_launch": dom["bytes_per_launch"], "launches_timed": dom["launches_timed"],
+                     "timing": "events on the launch stream around eager launches of this op alone",
+                     "all_gemm_kernels": rows},
+        "cpu_baseline": None,
+    }
+
+
 def cpu_baseline_prefill(H, pfmt="mxfp4", seconds=8.0):
     """The oracle's MXFP4 (or QINT8) linear on a bounded sample: 256 rows through a 2048 x 8192 slice of a
     projection, faithful mode."""
@@ -985,10 +1044,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--fmt", default="qint8", choices=["qint8", "mxfp4"])
     ap.add_argument("--batch", type=int, default=1, help="sequences for --workload tokens (1 or 16 in the baseline)")
-    ap.add_argument("--workload", default="all", choices=["all", "decode", "cfg1", "cfg3", "prefill", "tokens", "prompt"],
+    ap.add_argument("--workload", default="all", choices=["all", "decode", "cfg1", "cfg3", "prefill", "tokens", "prompt", "w4a8"],
                     help="all = the headline (config 2) plus every other leg of the metric under config.legs (default); "
                          "decode = the headline alone; cfg1 / cfg3 / prefill (config 4) / tokens (config 5) = that leg "
-                         "alone; prompt = a 2048-token prompt through the 7B-shape decoder")
+                         "alone; prompt = a 2048-token prompt through the 7B-shape decoder; w4a8 = config 4's layer under the "
+                         "reference's USE_MXFP4_INT8 mode (never part of the default run)")
     ap.add_argument("--prefill-fmt", default="mxfp4", choices=["mxfp4", "qint8"],
                     help="weight format of --workload prefill (BASELINE config 4 is MXFP4; qint8 = the same layer W8A8)")
     ap.add_argument("--act-fp8", action="store_true",
@@ -1033,6 +1093,8 @@ def main():
         return print(json.dumps(leg_as_line(leg_cfg5(torch, args, args.batch), args)))
     if args.workload == "prompt":
         return print(json.dumps(run_prompt(torch, args)))
+    if args.workload == "w4a8":
+        return print(json.dumps(leg_as_line(leg_w4a8(torch, _ops, args), args)))
 
     t_start = time.perf_counter()
     out = run_decode(torch, _ops, args)

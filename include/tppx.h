@@ -295,6 +295,25 @@ int tppx_linear_mxfp4_int8_rows(const void* x, const void* q_nat,
                                 int post_op, float post_scale,
                                 tppx_stream_t stream);
 
+/* W4A8 with many rows (prompt passes): the same arithmetic on the bf16 MFMA.  An int8 activation and a weight
+ * integer times its block's power of two are exact in bf16 and so is the fp32 sum of one MX block's 32 products, so
+ * one K = 32 MFMA per block gives float(int32 block sum) * 2^(e - 127) and the fold is one fp32 multiply-add with
+ * sa[row][block] per output and block, in ascending block order from the bias: the same bits as
+ * tppx_linear_mxfp4_int8's formula (src/csrc/fused_gemm.h:965-978).  tppx_prepack_mxfp4_int8_wide turns the
+ * USE_MXFP4_INT8 weight (layout as for tppx_prepack_mxfp4_int8) into bf16 operand tiles, w_nat N*K*2 bytes,
+ * N % 16 == 0, K % 128 == 0, once per weight.  tppx_linear_mxfp4_int8_wide takes bf16 rows x [M][K], quantizes
+ * them over blocks of 32 (quantize_int8sym, scales times 6/127) into the workspace and runs the GEMM; ws must hold
+ * Mp*K*2 + Mp*(K/32)*4 bytes with Mp = M rounded up to a multiple of 128, 16-byte aligned. */
+int tppx_prepack_mxfp4_int8_wide(const void* q_ref, const void* sc_ref,
+                                 int64_t N, int64_t K, int64_t bc, void* w_nat,
+                                 tppx_stream_t stream);
+int tppx_linear_mxfp4_int8_wide(const void* x, const void* w_nat,
+                                const void* bias, const void* post_in,
+                                const void* post_in2, void* y, int64_t M,
+                                int64_t N, int64_t K, int post_op,
+                                float post_scale, void* ws, int64_t ws_bytes,
+                                tppx_stream_t stream);
+
 /* QINT4 / ternary QINT2 weights at their own width for decode shapes.  The reference multiplies the packed codes as
  * they lie (TppBlockedQInt8LinearW on kQUInt4x2 / kQUInt2x4 weights, src/csrc/fused_gemm.h:1110-1126; BRGEMM with
  * b_vnni, src/csrc/xsmm_functors.h:2640-2666).  tppx_pack_qint_tiles turns the native int8 tiles of such a weight

@@ -352,6 +352,67 @@ def test_packed_code_kernel_block_rows(kind, M):
     assert_close_bf16(t2bits(y), t2bits(ref), what=f"{kind} packed block rows M={M}", pre_bits=t2bits(pre))
 
 
+@pytest.mark.parametrize("M,N,K,bc,post", [(130, 96, 512, 64, "none"), (200, 272, 1024, 128, "add"), (129, 128, 256, 32, "silu"),
+                                           (300, 1040, 1280, 64, "mul"), (257, 16, 128, 32, "add2"), (640, 512, 2048, 64, "relu")])
+def test_w4a8_wide_kernel(M, N, K, bc, post, monkeypatch):
+    """W4A8 passes of many rows (tppx_linear_mxfp4_int8_wide): the int8 rows and the weight integers times their
+    block's power of two as bf16 MFMA operands, one K = 32 MFMA per MX block, one fp32 multiply-add with
+    sa[row][block] per output and block in ascending order from the bias -- the oracle's loop
+    (src/csrc/fused_gemm.h:965-978 restated) term for term, so the GEMM result is EQUAL to the oracle's, bit for
+    bit; post-ops keep their usual bound.  Ragged row and channel counts, blocks of all-zero rows, every post-op
+    family, and the row threshold that picks the kernel."""
+    ops = _ops()
+    from tpp_pytorch_extension import _lib
+    posts = {"none": O.POST_NONE, "add": O.POST_ADD_SCALE, "silu": O.POST_SILU, "mul": O.POST_MUL,
+             "add2": O.POST_ADD2_SCALE, "relu": O.POST_RELU}
+    W = randn_bf16((N, K), 0.05, 2800 + M)
+    t = W.view(N // 16, 16, K // bc, bc // 2, 2).permute(0, 2, 3, 1, 4).contiguous()
+    qt = ops.remap_and_quantize_mxfp4(t.cuda(), int8_layout=True)
+    q_or, s_or = O.remap_quantize_mxfp4_int8(t.float().numpy())
+    x = randn_bf16((M, K), 1.0, 2810 + M)
+    x[0, 5] = 0.0
+    x[2, :64] = 0.0  # two all-zero blocks: scale 0, codes 0
+    x[M - 1] = 0.0
+    b = randn_bf16((N,), 0.01, 2820)
+    r = randn_bf16((M, N), 1.0, 2830)
+    r2 = randn_bf16((M, N), 1.0, 2840) if post == "add2" else None
+    assert M >= ops.W4A8_WIDE_ROWS and qt.native_w4a8_wide() is not None
+    # the GEMM alone: equal to the oracle
+    y0 = ops.linear(x.cuda(), qt, b.cuda(), O.POST_NONE, None, None, 1.0)
+    pre = O.linear_w4a8(t2bits(x), q_or, s_or, bc, t2bits(b))
+    assert np.array_equal(t2bits(y0), pre), f"w4a8 wide M={M} N={N} K={K}: {(t2bits(y0) != pre).sum()} of {pre.size} differ"
+    y = ops.linear(x.cuda(), qt, b.cuda(), posts[post], r.cuda(), None if r2 is None else r2.cuda(), 0.5)
+    ref = O.linear_w4a8(t2bits(x), q_or, s_or, bc, t2bits(b), posts[post], t2bits(r), None if r2 is None else t2bits(r2), 0.5)
+    assert_close_bf16(t2bits(y), ref, ulps=2 if post == "silu" else 1, what=f"w4a8 wide M={M} N={N} K={K} {post}")
+    # without a bias, and against the simple kernel below the threshold (the same sums in another order)
+    y1 = ops.linear(x.cuda(), qt, None, O.POST_NONE, None, None, 1.0)
+    assert np.array_equal(t2bits(y1), O.linear_w4a8(t2bits(x), q_or, s_or, bc, None))
+    monkeypatch.setattr(ops, "W4A8_WIDE_ROWS", 1 << 30)
+    y2 = ops.linear(x.cuda(), qt, b.cuda(), O.POST_NONE, None, None, 1.0)
+    assert_close_bf16(t2bits(y2), pre, ulps=1, what="simple kernel")
+    # the entry point rejects a workspace that is too small, and misaligned outputs
+    L = _lib.lib()
+    out = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    small = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    rc = L.tppx_linear_mxfp4_int8_wide(x.cuda().data_ptr(), qt.native_w4a8_wide().data_ptr(), None, None, None, out.data_ptr(),
+                                       M, N, K, 0, 1.0, small.data_ptr(), small.numel(), None)
+    assert rc == _lib.EINVAL and b"workspace" in L.tppx_last_error()
+
+
+def test_w4a8_wide_kernel_at_a_layer_shape():
+    """One 7B-shape projection (11008 x 4096) at 512 rows: the many-row W4A8 kernel equal to the oracle."""
+    ops = _ops()
+    M, N, K, bc = 512, 11008, 4096, 64
+    W = randn_bf16((N, K), 0.02, 2900)
+    t = W.view(N // 16, 16, K // bc, bc // 2, 2).permute(0, 2, 3, 1, 4).contiguous()
+    qt = ops.remap_and_quantize_mxfp4(t.cuda(), int8_layout=True)
+    q_or, s_or = O.remap_quantize_mxfp4_int8(t.float().numpy())
+    x = randn_bf16((M, K), 1.0, 2901)
+    y = ops.linear(x.cuda(), qt, None, O.POST_NONE, None, None, 1.0)
+    ref = O.linear_w4a8(t2bits(x), q_or, s_or, bc, None)
+    assert np.array_equal(t2bits(y), ref)
+
+
 @pytest.mark.parametrize("M,N,K,bc,post", [(1, 4096, 4096, 64, "none"), (8, 11008, 4096, 64, "add"), (16, 512, 2048, 128, "silu"),
                                            (5, 96, 1280, 32, "mul"), (8, 4096, 11008, 64, "add"), (3, 8448, 1536, 64, "none"),
                                            (16, 4096, 11008, 64, "add")])

@@ -89,6 +89,8 @@ SIGNATURES = {
     "tppx_pack_qint_tiles": [_vp, _i64, _i64, _i32, _vp, _vp],
     "tppx_prepack_mxfp4_int8": [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp],
     "tppx_linear_mxfp4_int8_rows": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _f32, _vp],
+    "tppx_prepack_mxfp4_int8_wide": [_vp, _vp, _i64, _i64, _i64, _vp, _vp],
+    "tppx_linear_mxfp4_int8_wide": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _f32, _vp, _i64, _vp],
     "tppx_linear_qintx": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _f32, _i32, _vp],
     "tppx_linear_wide": [_vp, _i32, _vp, _vp, _i32, _vp, _vp, _i64, _i64, _i64, _vp],
     "tppx_post_op_wide": [_vp, _i32, _i32, _vp, _vp, _f32, _vp, _i64, _vp],

@@ -607,6 +607,7 @@ def _linear_other_types(input, weight, bias, post, flags, post_in=None, post_in2
 PACKED_CODES = os.environ.get("TPPX_PACKED_CODES", "1") == "1"
 W4A8_ACT_SCALE = 6.0 / 127.0
 W4A8_DECODE = os.environ.get("TPPX_W4A8_DECODE", "1") == "1"
+W4A8_WIDE_ROWS = int(os.environ.get("TPPX_W4A8_WIDE_ROWS", "129"))
 
 
 def _linear_w4a8(input, weight, bias, post, post_in, post_in2, post_scale):
@@ -638,6 +639,16 @@ def _linear_w4a8(input, weight, bias, post, post_in, post_in2, post_scale):
         if rc != _lib.EUNSUPPORTED:  # rows that do not fit the kernel's LDS take the two-step path
             _lib.check(rc)
             return y
+    # prompt passes: rows and weights as bf16-coded integers on the bf16 MFMA, one fp32 multiply-add per block
+    # (TPPX_W4A8_WIDE_ROWS: from how many rows; the weight keeps a second, 2-byte-per-value copy for it)
+    wide = weight.native_w4a8_wide() if M >= W4A8_WIDE_ROWS else None
+    if wide is not None:
+        mp = (M + 127) // 128 * 128
+        ws = torch.empty(mp * K * 2 + mp * (K // 32) * 4, dtype=torch.uint8, device=x.device)
+        _lib.check(L.tppx_linear_mxfp4_int8_wide(x.data_ptr(), wide.data_ptr(), _lib.ptr(bias), _lib.ptr(post_in),
+                                                 _lib.ptr(post_in2), y.data_ptr(), M, N, K, post, post_scale,
+                                                 ws.data_ptr(), ws.numel(), _lib.stream_of(x)))
+        return y
     act = quantize_int8sym(x.view(M, K), 32, -1, False)
     sa = act.scales.mul_(W4A8_ACT_SCALE)
     _lib.check(L.tppx_linear_mxfp4_int8(act.qdata.data_ptr(), sa.data_ptr(), weight.qdata.data_ptr(),

@@ -183,6 +183,25 @@ class QTensor(torch.Tensor):
                 have = self._native_w4a8 = (qn, sn)
         return have or None
 
+    def native_w4a8_wide(self):
+        """W4A8 (USE_MXFP4_INT8) weights for passes of many rows: bf16 operand tiles holding integer * 2^(e - 127),
+        2 bytes per weight, made once (tppx_prepack_mxfp4_int8_wide); None when K is not a multiple of 128 or N of
+        16."""
+        have = getattr(self, "_native_w4a8_wide", None)
+        if have is None:
+            if self.weight_kind() != "mxfp4_int8":
+                raise _lib.TppxError(_lib.EUNSUPPORTED, f"not a W4A8 weight: {self!r}")
+            N, K = self.weight_nk()
+            if N % 16 or K % 128:
+                have = self._native_w4a8_wide = ()
+            else:
+                wn = torch.empty(N * K, dtype=torch.bfloat16, device=self.qdata.device)
+                _lib.check(_lib.lib().tppx_prepack_mxfp4_int8_wide(self.qdata.data_ptr(), self.scales.data_ptr(), N, K,
+                                                                   self.shape[2] * 8, wn.data_ptr(),
+                                                                   _lib.stream_of(self.qdata)))
+                have = self._native_w4a8_wide = (wn,)
+        return have[0] if have else None
+
     def dequantize(self):
         """fp32 tensor in the blocked shape (PerBlock*Quantizer::dequantize,
         src/csrc/qtypes.cpp:438-473,521-577)."""
