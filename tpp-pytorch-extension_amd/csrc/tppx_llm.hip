@@ -877,8 +877,11 @@ attn_prefill_kernel(const AttnPrefillParams p) {
   const int g = lane >> 4, c = lane & 15;
   const int bh = blockIdx.y, b = bh / p.Nq, hq = bh - b * p.Nq;
   const int hk = hq / (p.Nq / p.Nkv);
-  // the last query blocks see the most keys: start them first
-  const int qblk = (int)gridDim.x - 1 - (int)blockIdx.x;
+  // The last query blocks see the most keys: start them first.  Two workgroups share a CU, and the dispatcher puts
+  // workgroup i + 256 beside workgroup i: every other run of 256 workgroups walks its query blocks the other way
+  // round, so that a long block meets a short one instead of its twin of another head.
+  const int wg = (int)(blockIdx.y * gridDim.x + blockIdx.x);
+  const int qblk = ((wg >> 8) & 1) ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;
   const int q0 = qblk * QB + wave * (16 * QG);
   const int last_key = p.past + p.S - 1;
 
@@ -1074,7 +1077,10 @@ attn_prefill_hd_kernel(const AttnPrefillParams p) {
   const int g = lane >> 4, c = lane & 15;
   const int bh = blockIdx.y, b = bh / p.Nq, hq = bh - b * p.Nq;
   const int hk = hq / (p.Nq / p.Nkv);
-  const int qblk = (int)gridDim.x - 1 - (int)blockIdx.x; // the last query blocks see the most keys: start them first
+  // the last query blocks see the most keys: start them first; every other run of 256 workgroups the other way
+  // round, so that the workgroups that share a CU (i, i + 256, ...) are a long one and a short one
+  const int wg = (int)(blockIdx.y * gridDim.x + blockIdx.x);
+  const int qblk = ((wg >> 8) & 1) ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;
   const int q0 = qblk * QB + wave * (16 * QG);
   const int last_key = p.past + p.S - 1;
   const i32x4 zero4 = {0, 0, 0, 0};
