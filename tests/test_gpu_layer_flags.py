@@ -127,10 +127,13 @@ def test_layer_weight_format_flags(flags, cache_remapped, fmts, monkeypatch):
 
 
 @pytest.mark.parametrize("M,N,K,post", [(128, 256, 512, "none"), (300, 1056, 1024, "add"), (2048, 4096, 4096, "silu"),
-                                        (65, 48, 128, "mul"), (1000, 11008, 4096, "none")])
-def test_unquantized_bf16_weight_gemm_at_prompt_shapes(M, N, K, post):
+                                        (65, 48, 128, "mul"), (1000, 11008, 4096, "none"), (193, 16, 128, "add"),
+                                        (257, 4112, 256, "mul")])
+def test_unquantized_bf16_weight_gemm_at_prompt_shapes(M, N, K, post, monkeypatch):
     """TppBlockedLinearW<bf16, bf16> (src/csrc/fused_gemm.h:785-1073, non-quantized branch) above 64 rows: the
-    LDS-tiled bf16 kernel (ragged rows, ragged channel tiles) and the row-group kernel give the oracle's tile."""
+    LDS-tiled bf16 kernels (ragged rows, ragged channel tiles: from 192 rows the 128 x 256 form of the large prefill
+    kernel with hand-counted weight loads, below that and under TPPX_BF16_BIG=0 the 128 x 128 one) and the
+    row-group kernel give the oracle's tile."""
     import ctypes
     import tpp_pytorch_extension  # noqa: F401
     from tpp_pytorch_extension import _ops, _lib
@@ -146,3 +149,7 @@ def test_unquantized_bf16_weight_gemm_at_prompt_shapes(M, N, K, post):
         y = _ops.linear(x.cuda(), wb, b.cuda(), posts[post], pin.cuda(), None, 0.5, flags=flags)
         assert_close_bf16(t2bits(y), ref, ulps=2 if post == "silu" else 1, what=f"bf16 weight M={M} N={N} K={K} {post} flags={flags}",
                           pre_bits=pre)
+    monkeypatch.setenv("TPPX_BF16_BIG", "0")
+    y = _ops.linear(x.cuda(), wb, b.cuda(), posts[post], pin.cuda(), None, 0.5, flags=_lib.FLAG_FORCE_TILED)
+    assert_close_bf16(t2bits(y), ref, ulps=2 if post == "silu" else 1, what=f"bf16 weight M={M} N={N} K={K} {post} 128 x 128 kernel",
+                      pre_bits=pre)

@@ -575,9 +575,15 @@ struct BigParams {
 //   1 x 8  128 x 512, one workgroup per CU: the same 65536 sums per CU as 2 x 4, but half the activation bytes per
 //          K step (128 rows) and every weight tile fetched by ONE wave instead of by the two of a wave column -- half
 //          the bytes moved from L2 into the CU per MFMA
-template <int MT, bool DUAL, int WM, int WN>
-__global__ void __launch_bounds__(WM * WN * 64, WM * WN == 4 ? 2 : 1)
-big_mxfp4_kernel(const BigParams P) {
+// WBF16: unquantized bf16 weights in their native tiles ([N/16][K/128][4 j][64 lanes][16 B], the MFMA operands
+// themselves) instead of packed codes + scales: 16 bytes per lane, tile and MFMA step, so they run as a ring of the
+// four steps j of a K step -- (ks + 1, j) is requested right behind the last MFMA group of (ks, j), a whole K step
+// ahead -- and no second register set is needed.  These loads are issued and waited for by hand (they complete in
+// issue order, so "at most N younger loads outstanding" is the wait): with loads into LDS pending the compiler
+// answers the first use of any loaded register, and the fence of __syncthreads(), with a wait for ALL loads.
+template <int MT, bool DUAL, int WM, int WN, bool WBF16>
+__device__ __forceinline__ void big_gemm_body(const BigParams& P) {
+  static_assert(!WBF16 || (!DUAL && MT * 4 / WN == 8), "the bf16-weight form: single GEMMs, 8 blocks of A per wave and K step");
   constexpr int WGM = MT * 16 * WM; // rows per workgroup
   constexpr int NBLK = MT * 4 / WN; // blocks of 4 rows x 256 B of the A tile that a wave fetches per K step
   static_assert(NBLK % 4 == 0, "the swizzle below takes a wave's first block to be a multiple of 4");
@@ -681,6 +687,15 @@ big_mxfp4_kernel(const BigParams P) {
       sc[nt] = e8m0_to_f32(snext[nt]);
     }
   };
+  i32x4 bw[4][4]; // WBF16: [j][nt]
+  auto load_bw = [&](int ks, int j) {
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+      // native bf16 tiles: slot ((tile * KT + ks) * 4 + j) * 64 + lane, 16 bytes each
+      const char* src = qwb + (size_t)(((woff[nt] - (uint32_t)lane) * 4u + (uint32_t)(ks * 4 + j) * 64u + (uint32_t)lane) * 16u);
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(bw[j][nt]) : "v"(src));
+    }
+  };
 
   f32x4 acc[MT][4];
 #pragma unroll
@@ -690,7 +705,13 @@ big_mxfp4_kernel(const BigParams P) {
       acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   load_a(0, 0);
-  load_b(0);
+  if constexpr (WBF16) {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      load_bw(0, j);
+  } else {
+    load_b(0);
+  }
   __syncthreads();
   // One K step.  MORE: the next step's A tile is requested during this one, one block behind each of the first NBLK
   // MFMA groups (issued in one burst, a wave stands at its load instructions while the memory pipeline's queue
@@ -698,7 +719,8 @@ big_mxfp4_kernel(const BigParams P) {
   auto step = [&](auto MORE, int ks) {
     constexpr bool more = decltype(MORE)::value;
     const int buf = ks & 1;
-    take_b();
+    if constexpr (!WBF16)
+      take_b();
     // 4*MT operand reads per K step (q = j*MT + mt), kept RD ahead of the MFMAs
     // that consume them so the LDS latency is covered by 4*RD MFMAs
     const uint32_t abase = lds0 + (uint32_t)(buf * ABUF + wm * MT * 4096);
@@ -713,7 +735,17 @@ big_mxfp4_kernel(const BigParams P) {
     static_for<0, NQ>([&](auto Q) {
       constexpr int q = decltype(Q)::value;
       constexpr int j = q / MT, mt = q % MT;
-      if constexpr (mt == 0) {
+      if constexpr (mt == 0 && WBF16) {
+        // Step j's weights were requested a K step ago.  Behind them then: the later steps' (4 each); in this K
+        // step, when it requests anything: its 8 blocks of A (behind the first 8 groups) and the next K step's
+        // weights of the steps before j.
+        constexpr int younger = (3 - j) * 4 + (more ? (j >= 1 ? 8 : 0) + j * 4 : 0);
+        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(bw[j][0]), "+v"(bw[j][1]), "+v"(bw[j][2]), "+v"(bw[j][3]) : "n"(younger));
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++)
+          b[nt] = __builtin_bit_cast(bf16x8, bw[j][nt]);
+      }
+      if constexpr (mt == 0 && !WBF16) {
 #pragma unroll
         for (int nt = 0; nt < 4; nt++)
           b[nt] = tl_cvt_fp4x8(bc[nt][j], sc[nt]);
@@ -730,10 +762,21 @@ big_mxfp4_kernel(const BigParams P) {
         acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[nt], acc[mt][nt], 0, 0, 0);
       if constexpr (more && q < NBLK)
         load_a_one(std::integral_constant<int, q>{}, ks + 1, buf ^ 1);
-      if constexpr (more && q == NQ / 2 - 1)
-        load_b(ks + 1); // dwords of steps 0 and 1 of the current B are dead by now
+      if constexpr (WBF16) {
+        if constexpr (more && mt == MT - 1)
+          load_bw(ks + 1, j); // the MFMAs that read step j's registers have been issued
+      } else {
+        if constexpr (more && q == NQ / 2 - 1)
+          load_b(ks + 1); // dwords of steps 0 and 1 of the current B are dead by now
+      }
     });
-    __syncthreads(); // waits for this wave's direct-to-LDS loads, then for everybody's
+    if constexpr (WBF16 && more) {
+      // this wave's loads into LDS have landed (the 16 weight loads of the next K step went out behind them), then
+      // everybody's; a bare barrier, see above
+      asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" : : : "memory");
+    } else {
+      __syncthreads(); // waits for this wave's direct-to-LDS loads, then for everybody's
+    }
   };
   for (int ks = 0; ks + 1 < KT; ks++)
     step(std::true_type{}, ks);
@@ -744,6 +787,18 @@ big_mxfp4_kernel(const BigParams P) {
                           tile_base);
   else
     big_epilogue<MT>(p, acc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
+}
+
+template <int MT, bool DUAL, int WM, int WN>
+__global__ void __launch_bounds__(WM * WN * 64, WM * WN == 4 ? 2 : 1)
+big_mxfp4_kernel(const BigParams P) {
+  big_gemm_body<MT, DUAL, WM, WN, false>(P);
+}
+
+template <int MT, int WM, int WN>
+__global__ void __launch_bounds__(WM * WN * 64, WM * WN == 4 ? 2 : 1)
+big_bf16_kernel(const BigParams P) {
+  big_gemm_body<MT, false, WM, WN, true>(P);
 }
 
 // ---------------------------------------------------------------------------
@@ -1187,6 +1242,17 @@ static hipError_t big_launch(const BigParams& P, int wgs, hipStream_t stream) {
   return hipGetLastError();
 }
 
+template <int MT, int WM, int WN>
+static hipError_t big_bf16_launch(const BigParams& P, int wgs, hipStream_t stream) {
+  const size_t lds = (size_t)WM * WN * 64 * EP_LD * sizeof(float);
+  static_assert((size_t)WM * WN * 64 * EP_LD * sizeof(float) >= (size_t)2 * MT * 16 * WM * 256, "LDS plan");
+  TPPX_PLAN_ONLY((big_bf16_kernel<MT, WM, WN>), dim3(wgs), dim3(WM * WN * 64), lds);
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_bf16_kernel<MT, WM, WN>), lds); e != hipSuccess)
+    return e;
+  big_bf16_kernel<MT, WM, WN><<<dim3(wgs), dim3(WM * WN * 64), lds, stream>>>(P);
+  return hipGetLastError();
+}
+
 // dual: t[0] = gate, t[1] = up (equal shapes, n == 2); y[m][n] = silu(gate) * up goes to t[1].y
 hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t stream, bool dual) {
   if (dual && (n != 2 || t[0].tiles != t[1].tiles || t[0].K != t[1].K || t[0].M != t[1].M || t[0].x != t[1].x))
@@ -1334,6 +1400,20 @@ silu_mul_kernel(const uint16_t* __restrict__ gate, uint16_t* __restrict__ y, int
 }
 
 hipError_t launch_tiled_bf16(const TiledParams& p, hipStream_t stream) {
+  // prompt-sized passes: the 128 x 256 form of the large MXFP4 kernel with the weights read as they are (two
+  // workgroups of four waves per CU); its 32-bit offsets want operands below 4 GiB
+  if (p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && env_int("TPPX_BF16_BIG", 1) != 0 &&
+      (int64_t)p.M * p.K * 2 < ((int64_t)1 << 32) && (int64_t)p.tiles * 32 * p.K < ((int64_t)1 << 32)) {
+    BigParams P;
+    memset(&P, 0, sizeof(P));
+    P.seg[0] = p;
+    const int nb = (p.tiles + 15) / 16;
+    for (int i = 1; i <= TPPX_MAX_SEGS; i++)
+      P.nb0[i] = nb;
+    P.n_seg = 1;
+    P.xm = 1;
+    return big_bf16_launch<8, 1, 4>(P, ((p.M + 127) / 128) * nb, stream);
+  }
   const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
   const dim3 grid((unsigned)(MB * NB));
   const size_t lds = 2 * 2048 * 16;
