@@ -583,7 +583,8 @@ struct BigParams {
 // answers the first use of any loaded register, and the fence of __syncthreads(), with a wait for ALL loads.
 template <int MT, bool DUAL, int WM, int WN, bool WBF16>
 __device__ __forceinline__ void big_gemm_body(const BigParams& P) {
-  static_assert(!WBF16 || (!DUAL && MT * 4 / WN == 8), "the bf16-weight form: single GEMMs, 8 blocks of A per wave and K step");
+  static_assert(!WBF16 || (!DUAL && MT * 4 / WN <= MT), "the bf16-weight form: single GEMMs; the wait counts below take a wave's "
+                                                       "blocks of A to be requested behind the first MT groups");
   constexpr int WGM = MT * 16 * WM; // rows per workgroup
   constexpr int NBLK = MT * 4 / WN; // blocks of 4 rows x 256 B of the A tile that a wave fetches per K step
   static_assert(NBLK % 4 == 0, "the swizzle below takes a wave's first block to be a multiple of 4");
@@ -737,9 +738,9 @@ __device__ __forceinline__ void big_gemm_body(const BigParams& P) {
       constexpr int j = q / MT, mt = q % MT;
       if constexpr (mt == 0 && WBF16) {
         // Step j's weights were requested a K step ago.  Behind them then: the later steps' (4 each); in this K
-        // step, when it requests anything: its 8 blocks of A (behind the first 8 groups) and the next K step's
-        // weights of the steps before j.
-        constexpr int younger = (3 - j) * 4 + (more ? (j >= 1 ? 8 : 0) + j * 4 : 0);
+        // step, when it requests anything: its NBLK blocks of A (behind the first NBLK groups, all of step 0) and
+        // the next K step's weights of the steps before j.
+        constexpr int younger = (3 - j) * 4 + (more ? (j >= 1 ? NBLK : 0) + j * 4 : 0);
         asm volatile("s_waitcnt vmcnt(%4)" : "+v"(bw[j][0]), "+v"(bw[j][1]), "+v"(bw[j][2]), "+v"(bw[j][3]) : "n"(younger));
 #pragma unroll
         for (int nt = 0; nt < 4; nt++)
@@ -1407,6 +1408,8 @@ hipError_t launch_tiled_bf16(const TiledParams& p, hipStream_t stream) {
     BigParams P;
     memset(&P, 0, sizeof(P));
     P.seg[0] = p;
+    // (the 256 x 256 and 128 x 512 forms of eight waves were measured too: equal at 28672 x 8192, 20-30 % slower
+    // at the 7B shapes)
     const int nb = (p.tiles + 15) / 16;
     for (int i = 1; i <= TPPX_MAX_SEGS; i++)
       P.nb0[i] = nb;
