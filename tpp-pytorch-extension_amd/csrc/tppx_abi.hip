@@ -6,6 +6,7 @@
 #include <string.h>
 
 #include <cxxabi.h>
+#include <algorithm>
 #include <map>
 #include <mutex>
 #include <string>
@@ -217,11 +218,14 @@ static const int64_t TILED_MIN_M = 65; // more rows than the decode kernels cove
 // More than 64 rows: the LDS-tiled kernels give every workgroup a whole output tile and all of K, so a launch with
 // few tiles leaves most of the 256 CUs idle (7B shapes at 256 rows: 43 workgroups), while the decode kernels run one
 // block row of 64 rows after the other over the full grid, streaming the weights once per block row.  Pick by a
-// cost estimate fitted to measurements on MI355X (us): a block row costs about 8 + weight bytes / 5.5 TB/s + 0.8 ns
-// per input channel (its activations), a round of 256 x 256 tiles about 14.5 ns per input channel (128 x 128: 20).  `wbytes` = weight bytes of the whole call, `n_tiles16` = its 16-channel
-// tiles.  TPPX_TILED_MIN_M (when set) restores a plain row threshold.
+// cost estimates fitted to measurements on MI355X (us).  MXFP4: a block row of 64 costs about 8 + weight bytes /
+// 5.5 TB/s + 0.8 ns per input channel (its activations), a round of 256 x 256 tiles about 14.5 ns per input channel
+// (128 x 128: 20).  QINT8 (128 x 256 tiles, one workgroup per CU) and unquantized bf16 weights (from 192 rows 128 x 256
+// tiles, two workgroups per CU; below that the 128 x 128 kernel): their own fits below.  `wbytes` = weight bytes of
+// the whole call, `n_tiles16` = its 16-channel tiles.  TPPX_TILED_MIN_M (when set) restores a plain row threshold.
+enum { COST_MXFP4 = 0, COST_QINT8 = 1, COST_BF16 = 2 };
 static bool want_tiled(int64_t M, int flags, int64_t K = 0, int64_t n_tiles16 = 0, double wbytes = 0.0,
-                       bool small_tiles_only = false) {
+                       int kind = COST_MXFP4) {
   if (flags & TPPX_FLAG_FORCE_SKINNY)
     return false;
   if (flags & TPPX_FLAG_FORCE_TILED)
@@ -233,11 +237,24 @@ static bool want_tiled(int64_t M, int flags, int64_t K = 0, int64_t n_tiles16 = 
     return M >= env_min;
   if (K <= 0 || n_tiles16 <= 0 || M > 1024)
     return true;
-  const bool big = !small_tiles_only && M >= env_int("TPPX_TILED_BIG_MIN_M", 192);
+  const double rows64 = (double)((M + 63) / 64);
+  if (kind == COST_QINT8) {
+    const int64_t wgs = ((M + 127) / 128) * ((n_tiles16 + 15) / 16);
+    const double tiled_us = (double)((wgs + 255) / 256) * (10.0 + (double)K * 0.0075);
+    const double skinny_us = rows64 * (5.0 + wbytes / 5.5e6 + (double)K * 0.0004);
+    return tiled_us <= skinny_us;
+  }
+  if (kind == COST_BF16 && M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && env_int("TPPX_BF16_BIG", 1) != 0) {
+    const int64_t wgs = ((M + 127) / 128) * ((n_tiles16 + 15) / 16);
+    const double tiled_us = (17.0 + (double)K * 0.009) * std::max(1.0, (double)wgs / 200.0);
+    const double skinny_us = rows64 * (6.5 + wbytes / 5.5e6 + (double)K * 0.0006);
+    return tiled_us <= skinny_us;
+  }
+  const bool big = kind == COST_MXFP4 && M >= env_int("TPPX_TILED_BIG_MIN_M", 192);
   const int64_t rows = big ? 256 : 128, cols16 = big ? 16 : 8;
   const int64_t wgs = ((M + rows - 1) / rows) * ((n_tiles16 + cols16 - 1) / cols16);
   const double tiled_us = (double)((wgs + 255) / 256) * (double)K * 0.0145 * (big ? 1.0 : 1.4);
-  const double skinny_us = (double)((M + 63) / 64) * (8.0 + wbytes / 5.5e6 + (double)K * 0.0008);
+  const double skinny_us = rows64 * (8.0 + wbytes / 5.5e6 + (double)K * 0.0008);
   return tiled_us <= skinny_us;
 }
 
@@ -485,7 +502,7 @@ static int run_qint8(const char* who, const void* x, void* xq, void* sa, const t
   p.units = (int)(K / (64 * p.deal));
   p.spb_magic = (p.deal == 4 && p.tpb > 4) ? (unsigned int)((((uint64_t)1 << 32) + (uint64_t)(p.tpb / 4) - 1) / (uint64_t)(p.tpb / 4)) : 0u;
   const bool reuse = (flags & TPPX_FLAG_XQ_REUSE) != 0; // xq / sa still hold this x, quantized by an earlier call
-  if (qbs % 128 == 0 && want_tiled(M, flags, K, p.total_tiles, (double)p.total_tiles * 16.0 * (double)K)) {
+  if (qbs % 128 == 0 && want_tiled(M, flags, K, p.total_tiles, (double)p.total_tiles * 16.0 * (double)K, COST_QINT8)) {
     if (x && !reuse) {
       rc = check_hip(launch_quant_act_int8(x, M, K, qbs, xq, sa, 0, stream), who);
       if (rc)
@@ -696,7 +713,7 @@ extern "C" int tppx_linear_bf16(const void* x, const void* w, const void* bias, 
   p.S = 1;
   // more than 64 rows: the LDS-tiled kernel once it is the cheaper one (the estimate of the quantized formats with the
   // weight's real bytes: the row-group kernel streams the whole weight once per 64 rows)
-  if (want_tiled(M, flags, K, p.total_tiles, (double)N * (double)K * 2.0, true)) {
+  if (want_tiled(M, flags, K, p.total_tiles, (double)N * (double)K * 2.0, COST_BF16)) {
     TPPX_REQUIRE(aligned16(w), TPPX_EINVAL, "%s: weight not 16-byte aligned", who);
     return check_hip(launch_tiled_bf16(tiled_from_seg(p, 0), (hipStream_t)stream), who);
   }
