@@ -257,6 +257,25 @@ def test_attn_prefill_full_size_rows_equal_single_query_problem():
         assert np.abs(g - r).max() <= 2.0 ** -7 * np.abs(r).max(), i
 
 
+@pytest.mark.parametrize("S,Nq,queries_per_wave", [(600, 32, 16), (1100, 32, 32), (700, 48, 16)])
+def test_attn_prefill_more_than_256_workgroups(S, Nq, queries_per_wave, monkeypatch):
+    """Launches of more than 256 workgroups whose query blocks per head do not divide 256 (the heads of every other
+    run of 256 workgroups walk their blocks in the other order; a run boundary inside a head must not change that
+    head's order): EVERY row against plain PyTorch fp32 causal attention."""
+    _llm()
+    monkeypatch.setenv("TPPX_ATTN_QG", str(queries_per_wave // 16))
+    q = randn_bf16((1, S, Nq, 128), 1.0, 61)
+    k = randn_bf16((1, Nq, S, 128), 1.0, 62)
+    v = randn_bf16((1, Nq, S, 128), 1.0, 63)
+    got = _attn_prefill(q.cuda(), k.cuda(), v.cuda(), 0).float()
+    s = torch.einsum("bsnh,bnlh->bnsl", q.cuda().float(), k.cuda().float()) / np.sqrt(128.0)
+    causal = torch.arange(S, device="cuda")[None, :] > torch.arange(S, device="cuda")[:, None]
+    s = s.masked_fill(causal[None, None], float("-inf"))
+    ref = torch.einsum("bnsl,bnlh->bsnh", torch.softmax(s, -1), v.cuda().float())
+    err = (got - ref).flatten(2).norm(dim=-1) / ref.flatten(2).norm(dim=-1)  # per (batch, row)
+    assert float(err.max()) <= 2e-2, (int(err.argmax()), float(err.max()))
+
+
 @pytest.mark.parametrize("queries_per_wave", [16, 32])
 def test_attn_prefill_mask_and_errors(queries_per_wave, monkeypatch):
     F = _llm()

@@ -169,10 +169,11 @@ def test_decoder_layer_with_64_wide_heads(S, past, H):
 
 @pytest.mark.parametrize("H", [64, 256])
 def test_attn_prefill_other_head_sizes_full_prompt_and_plain_kernel(H, monkeypatch):
-    """A prompt long enough for 32 queries per wave (head size 64) and many key tiles: sampled rows against the
-    oracle's single-query function, and the MFMA kernel against the plain one-wave-per-query kernel it replaced."""
+    """A prompt long enough for many key tiles and for more than 256 workgroups (the ones past 256 walk their query
+    blocks in the other order): sampled rows against the oracle's single-query function, and the MFMA kernel
+    against the plain one-wave-per-query kernel it replaced, over every row."""
     _llm()
-    B, S, Nq = 1, 600, 16
+    B, S, Nq = 2, 600, 16
     q = randn_bf16((B, S, Nq, H), 1.0, 171 + H)
     k = randn_bf16((B, Nq, S, H), 1.0, 172 + H)
     v = randn_bf16((B, Nq, S, H), 1.0, 173 + H)

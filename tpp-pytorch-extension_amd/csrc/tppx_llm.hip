@@ -878,10 +878,12 @@ attn_prefill_kernel(const AttnPrefillParams p) {
   const int bh = blockIdx.y, b = bh / p.Nq, hq = bh - b * p.Nq;
   const int hk = hq / (p.Nq / p.Nkv);
   // The last query blocks see the most keys: start them first.  Two workgroups share a CU, and the dispatcher puts
-  // workgroup i + 256 beside workgroup i: every other run of 256 workgroups walks its query blocks the other way
-  // round, so that a long block meets a short one instead of its twin of another head.
-  const int wg = (int)(blockIdx.y * gridDim.x + blockIdx.x);
-  const int qblk = ((wg >> 8) & 1) ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;
+  // workgroup i + 256 beside workgroup i: the heads of every other run of 256 workgroups walk their query blocks
+  // the other way round, so that a long block meets a short one instead of its twin of another head.  (One order
+  // per head -- taken from the head's first workgroup -- or a run boundary inside a head would visit some blocks
+  // twice and others never.)
+  const int wg0 = (int)(blockIdx.y * gridDim.x);
+  const int qblk = ((wg0 >> 8) & 1) ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;
   const int q0 = qblk * QB + wave * (16 * QG);
   const int last_key = p.past + p.S - 1;
 
@@ -1077,10 +1079,11 @@ attn_prefill_hd_kernel(const AttnPrefillParams p) {
   const int g = lane >> 4, c = lane & 15;
   const int bh = blockIdx.y, b = bh / p.Nq, hq = bh - b * p.Nq;
   const int hk = hq / (p.Nq / p.Nkv);
-  // the last query blocks see the most keys: start them first; every other run of 256 workgroups the other way
-  // round, so that the workgroups that share a CU (i, i + 256, ...) are a long one and a short one
-  const int wg = (int)(blockIdx.y * gridDim.x + blockIdx.x);
-  const int qblk = ((wg >> 8) & 1) ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;
+  // the last query blocks see the most keys: start them first; the heads of every other run of 256 workgroups the
+  // other way round, so that the workgroups that share a CU (i, i + 256, ...) are a long one and a short one (one
+  // order per head, taken from the head's first workgroup)
+  const int wg0 = (int)(blockIdx.y * gridDim.x);
+  const int qblk = ((wg0 >> 8) & 1) ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;
   const int q0 = qblk * QB + wave * (16 * QG);
   const int last_key = p.past + p.S - 1;
   const i32x4 zero4 = {0, 0, 0, 0};
