@@ -1319,6 +1319,11 @@ hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t str
   }
   if (shape == 2)
     return dual ? big_launch<8, true, 1, 8>(P, MB4 * nb, stream) : big_launch<8, false, 1, 8>(P, MB4 * nb, stream);
+  // 128 x 256 workgroups that do not fill the CUs (at most one each): eight waves of 64 x 64 instead of four of
+  // 128 x 64 -- two waves per SIMD, so that one wave's waits are another's issue slots (the same sums in the same
+  // order: the same bits; 4096 x 4096 at 192-1024 rows 63-70 -> 49-57 us)
+  if (shape == 1 && MB4 * nb <= 256 && env_int("TPPX_TILED_W8", 1) != 0)
+    return dual ? big_launch<4, true, 2, 4>(P, MB4 * nb, stream) : big_launch<4, false, 2, 4>(P, MB4 * nb, stream);
   if (shape == 1)
     return dual ? big_launch<8, true, 1, 4>(P, MB4 * nb, stream) : big_launch<8, false, 1, 4>(P, MB4 * nb, stream);
   return dual ? big_launch<8, true, 2, 4>(P, MB8 * nb, stream) : big_launch<8, false, 2, 4>(P, MB8 * nb, stream);
@@ -1415,6 +1420,8 @@ hipError_t launch_tiled_bf16(const TiledParams& p, hipStream_t stream) {
       P.nb0[i] = nb;
     P.n_seg = 1;
     P.xm = 1;
+    if (((p.M + 127) / 128) * nb <= 256 && env_int("TPPX_TILED_W8", 1) != 0) // at most one workgroup per CU: eight waves, as for MXFP4
+      return big_bf16_launch<4, 2, 4>(P, ((p.M + 127) / 128) * nb, stream);
     return big_bf16_launch<8, 1, 4>(P, ((p.M + 127) / 128) * nb, stream);
   }
   const int MB = (p.M + 127) / 128, NB = (p.tiles + 7) / 8;
