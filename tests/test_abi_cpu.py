@@ -235,11 +235,18 @@ def test_launch_plans_of_the_baseline_shapes():
     assert len(lines) == 1 and "big_mxfp4_kernel<8, true, 1, 8> grid=1792x1x1" in lines[0]       # silu*mul in the epilogue
     lines = plan(L.tppx_plan_multi_linear_mxfp4, pair, 2, 2048, 8192, 1, _lib.FLAG_ACT_FP8, 1 << 28)
     assert any("big_fp8_kernel<8, true> grid=1792x1x1" in l for l in lines), lines
-    # prompts of a few hundred tokens: launches of at most 256 workgroups run eight waves per 128 x 256 workgroup
-    assert "big_mxfp4_kernel<4, false, 2, 4> grid=64x1x1 block=512" in plan(L.tppx_plan_linear_mxfp4, 512, 4096, 4096,
-                                                                            _lib.FLAG_FORCE_TILED, 0)[0]
+    # prompts of a few hundred tokens: launches of at most 128 workgroups of 128 x 256 run as four times as many of
+    # 64 x 128; up to 256 of them, as eight waves per workgroup
+    assert "big_mxfp4_kernel<2, false, 2, 2> grid=256x1x1 block=256" in plan(L.tppx_plan_linear_mxfp4, 512, 4096, 4096,
+                                                                             _lib.FLAG_FORCE_TILED, 0)[0]
+    assert "big_mxfp4_kernel<2, false, 2, 2>" in plan(L.tppx_plan_linear_mxfp4, 512, 4096, 4096, 0, 0)[0]   # and it is the choice
+    assert "big_mxfp4_kernel<4, false, 2, 4> grid=172x1x1 block=512" in plan(L.tppx_plan_linear_mxfp4, 512, 11008, 4096,
+                                                                             _lib.FLAG_FORCE_TILED, 0)[0]
     pair7 = (ctypes.c_int64 * 2)(11008, 11008)
     assert "big_mxfp4_kernel<4, true, 2, 4> grid=172x1x1 block=512" in plan(L.tppx_plan_multi_linear_mxfp4, pair7, 2, 256, 4096, 1,
+                                                                           _lib.FLAG_FORCE_TILED, 0)[0]
+    pair1 = (ctypes.c_int64 * 2)(4096, 4096)
+    assert "big_mxfp4_kernel<2, true, 2, 2> grid=256x1x1 block=256" in plan(L.tppx_plan_multi_linear_mxfp4, pair1, 2, 256, 4096, 1,
                                                                            _lib.FLAG_FORCE_TILED, 0)[0]
     assert "big_mxfp4_kernel<8, false, 1, 8> grid=176x1x1 block=512" in plan(L.tppx_plan_linear_mxfp4, 1024, 11008, 4096,
                                                                              _lib.FLAG_FORCE_TILED, 0)[0]  # 128 x 512: eight waves anyway

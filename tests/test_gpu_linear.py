@@ -19,6 +19,12 @@ POSTS = {"none": O.POST_NONE, "silu": O.POST_SILU, "mul": O.POST_MUL, "add": O.P
          "add2": O.POST_ADD2_SCALE, "gelu": O.POST_GELU, "relu": O.POST_RELU}
 
 
+def _lib_mod():
+    import tpp_pytorch_extension  # noqa: F401
+    from tpp_pytorch_extension import _lib
+    return _lib
+
+
 def _ops():
     import tpp_pytorch_extension  # noqa: F401
     from tpp_pytorch_extension import _ops
@@ -231,6 +237,38 @@ def test_prefill_mxfp4_workgroup_tiles_and_xcd_splits_agree(monkeypatch):
             monkeypatch.setenv("TPPX_TILED_XCD_M", str(xm))
             for i, (a, b) in enumerate(zip(run(), want)):
                 assert torch.equal(a, b), (tile, xm, i)
+
+
+@pytest.mark.parametrize("M", [200, 500])
+def test_prefill_forms_for_small_launches_agree(M, monkeypatch):
+    """Launches that leave CUs empty run other forms of the large-M kernel's body -- 64 x 128 workgroups of four waves
+    up to 128 workgroups of 128 x 256, eight waves per 128 x 256 workgroup up to 256 -- with the same sums in the
+    same order: identical bits to the four-wave 128 x 256 form, for a single GEMM (ragged rows and channel blocks),
+    fused q/k/v, the gate/up pair and unquantized bf16 weights; and the single GEMM against the oracle."""
+    ops = _ops()
+    K = 640
+    w, q_or, s_or = _make("mxfp4", 1056, K, 720)[:3]
+    ws = [_make("mxfp4", n, K, 721 + i)[0] for i, n in enumerate((1024, 256, 256))]
+    wg, wu = _make("mxfp4", 1120, K, 725)[0], _make("mxfp4", 1120, K, 726)[0]
+    Wb = randn_bf16((1056, K), 0.05, 727)
+    wb = block_bf16(Wb).cuda()
+    x = randn_bf16((M, K), 1.0, 728)
+    xg = x.cuda()
+
+    def run():
+        return [ops.fc_plain(xg, w, None)] + list(ops.qkv_gemm(xg, ws, [None] * 3)) + [ops.swiglu_gate_up(xg, wg, wu)] + \
+            [ops.linear(xg, wb, None, O.POST_NONE, None, None, 1.0, flags=_lib_mod().FLAG_FORCE_TILED)]
+
+    monkeypatch.setenv("TPPX_TILED_MIN_M", "0")  # the LDS-tiled family whatever the cost estimate says
+    got = run()
+    ref = O.linear_mxfp4(t2bits(x), q_or, s_or, None, O.POST_NONE, None, None, 1.0, O.MODE_IDEAL)
+    assert_close_bf16(t2bits(got[0]), ref, ulps=1, what=f"64 x 128 workgroups M={M}")
+    monkeypatch.setenv("TPPX_TILED_SMALL", "0")
+    mid = run()
+    monkeypatch.setenv("TPPX_TILED_W8", "0")
+    base = run()
+    for i, (a, b, c) in enumerate(zip(got, mid, base)):
+        assert torch.equal(a, c) and torch.equal(b, c), i
 
 
 @pytest.mark.parametrize("fmt", ["mxfp4", "qint8"])

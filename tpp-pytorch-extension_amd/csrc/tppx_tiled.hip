@@ -449,19 +449,20 @@ __device__ __forceinline__ void big_epilogue(const TiledParams& p, f32x4 (&acc)[
 #pragma unroll
   for (int e = 0; e < 8; e++)
     bias[e] = p.bias ? bf16_bits_to_f32(p.bias[n + e]) : 0.0f;
+  constexpr int MH = MT < 4 ? MT : 4; // row tiles staged at a time (64 rows, or the whole wave tile when it has fewer)
 #pragma unroll
-  for (int h = 0; h < MT / 4; h++) {
+  for (int h = 0; h < MT / MH; h++) {
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++)
+    for (int mt = 0; mt < MH; mt++)
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
 #pragma unroll
         for (int r = 0; r < 4; r++)
-          stage[(mt * 16 + (lane >> 4) * 4 + r) * EP_LD + nt * 16 + (lane & 15)] = acc[h * 4 + mt][nt][r];
+          stage[(mt * 16 + (lane >> 4) * 4 + r) * EP_LD + nt * 16 + (lane & 15)] = acc[h * MH + mt][nt][r];
     // same wave wrote and reads: no barrier, the compiler orders the LDS accesses
-    for (int it = 0; it < 8; it++) {
+    for (int it = 0; it < MH * 2; it++) {
       const int row = it * 8 + (lane >> 3);
-      const int m = m_base + h * 64 + row;
+      const int m = m_base + h * (MH * 16) + row;
       const f32x4 v0 = *reinterpret_cast<const f32x4*>(stage + row * EP_LD + cx);
       const f32x4 v1 = *reinterpret_cast<const f32x4*>(stage + row * EP_LD + cx + 4);
       if (tile_ok && m < p.M) {
@@ -504,19 +505,20 @@ __device__ __forceinline__ void big_epilogue_dual(const TiledParams& pg, const T
     bg[e] = pg.bias ? bf16_bits_to_f32(pg.bias[n + e]) : 0.0f;
     bu[e] = pu.bias ? bf16_bits_to_f32(pu.bias[n + e]) : 0.0f;
   }
+  constexpr int MH = MT < 4 ? MT : 4; // row tiles staged at a time
 #pragma unroll
-  for (int h = 0; h < MT / 4; h++) {
+  for (int h = 0; h < MT / MH; h++) {
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++)
+    for (int mt = 0; mt < MH; mt++)
 #pragma unroll
       for (int nt = 0; nt < 4; nt++)
 #pragma unroll
         for (int r = 0; r < 4; r++)
-          stage[(mt * 16 + (lane >> 4) * 4 + r) * EP_LD + nt * 16 + (lane & 15)] = acc[h * 4 + mt][nt][r];
+          stage[(mt * 16 + (lane >> 4) * 4 + r) * EP_LD + nt * 16 + (lane & 15)] = acc[h * MH + mt][nt][r];
     // same wave wrote and reads: no barrier, the compiler orders the LDS accesses
-    for (int it = 0; it < 4; it++) {
+    for (int it = 0; it < MH; it++) {
       const int row = it * 16 + (lane >> 2);
-      const int m = m_base + h * 64 + row;
+      const int m = m_base + h * (MH * 16) + row;
       const f32x4 g0 = *reinterpret_cast<const f32x4*>(stage + row * EP_LD + cx);
       const f32x4 g1 = *reinterpret_cast<const f32x4*>(stage + row * EP_LD + cx + 4);
       const f32x4 u0 = *reinterpret_cast<const f32x4*>(stage + row * EP_LD + 32 + cx);
@@ -1282,7 +1284,11 @@ hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t str
   const int env_shape = env_int("TPPX_TILED_BIG_TILE", 0); // 1 = 256 x 256, 2 = 128 x 256, 3 = 128 x 512
   if (env_shape >= 1 && env_shape <= 3)
     shape = env_shape - 1;
-  const int tpw = (shape == 2 ? 8 : 4) * (dual ? 2 : 4);
+  // Launches that would leave half the CUs empty with 128 x 256 workgroups: 64 x 128 workgroups of four waves (32 x 64
+  // each) instead, four times as many (the same sums in the same order: the same bits; 4096 x 4096 at 256 rows
+  // 50 -> 28 us, 4096 x 11008 at 512 rows 124 -> 79 us; beyond 128 such workgroups the small ones lose)
+  const bool small = shape == 1 && MB4 * nb4 <= 128 && env_int("TPPX_TILED_SMALL", 1) != 0 && env_shape == 0;
+  const int tpw = small ? (dual ? 4 : 8) : (shape == 2 ? 8 : 4) * (dual ? 2 : 4);
   BigParams P;
   memset(&P, 0, sizeof(P));
   int nb = 0;
@@ -1301,7 +1307,7 @@ hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t str
   {
     // XCD rectangles: the split that moves the fewest bytes from memory into the L2s (activations: rows x K bf16 per
     // row block, fetched by 8 / xm XCDs... every XCD fetches 1/xm of them; weights 0.53 B per element, xm/8 each)
-    const int MBs = shape == 0 ? MB8 : MB4;
+    const int MBs = small ? (t[0].M + 63) / 64 : shape == 0 ? MB8 : MB4;
     const double a_bytes = (double)t[0].M * t[0].K * 2.0, w_bytes = (dual ? 2.0 : 1.0) * nb * tpw * 16.0 * t[0].K * 0.53;
     double best = 1e300;
     P.xm = 1;
@@ -1322,6 +1328,9 @@ hipError_t launch_tiled_mxfp4_group(const TiledParams* t, int n, hipStream_t str
   // 128 x 256 workgroups that do not fill the CUs (at most one each): eight waves of 64 x 64 instead of four of
   // 128 x 64 -- two waves per SIMD, so that one wave's waits are another's issue slots (the same sums in the same
   // order: the same bits; 4096 x 4096 at 192-1024 rows 63-70 -> 49-57 us)
+  if (small)
+    return dual ? big_launch<2, true, 2, 2>(P, ((t[0].M + 63) / 64) * nb, stream)
+                : big_launch<2, false, 2, 2>(P, ((t[0].M + 63) / 64) * nb, stream);
   if (shape == 1 && MB4 * nb <= 256 && env_int("TPPX_TILED_W8", 1) != 0)
     return dual ? big_launch<4, true, 2, 4>(P, MB4 * nb, stream) : big_launch<4, false, 2, 4>(P, MB4 * nb, stream);
   if (shape == 1)
