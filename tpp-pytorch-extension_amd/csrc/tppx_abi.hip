@@ -246,7 +246,9 @@ static bool want_tiled(int64_t M, int flags, int64_t K = 0, int64_t n_tiles16 = 
   }
   if (kind == COST_BF16 && M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && env_int("TPPX_BF16_BIG", 1) != 0) {
     const int64_t wgs = ((M + 127) / 128) * ((n_tiles16 + 15) / 16);
-    const double tiled_us = (17.0 + (double)K * 0.009) * std::max(1.0, (double)wgs / 200.0);
+    const int64_t wgs2 = ((M + 63) / 64) * ((n_tiles16 + 7) / 8); // as 64 x 128 workgroups: the form up to 256 of them
+    const bool small = wgs2 <= 256 && env_int("TPPX_TILED_SMALL", 1) != 0;
+    const double tiled_us = small ? 12.0 + (double)K * 0.0045 : (17.0 + (double)K * 0.009) * std::max(1.0, (double)wgs / 200.0);
     const double skinny_us = rows64 * (6.5 + wbytes / 5.5e6 + (double)K * 0.0006);
     return tiled_us <= skinny_us;
   }

@@ -585,8 +585,7 @@ struct BigParams {
 // answers the first use of any loaded register, and the fence of __syncthreads(), with a wait for ALL loads.
 template <int MT, bool DUAL, int WM, int WN, bool WBF16>
 __device__ __forceinline__ void big_gemm_body(const BigParams& P) {
-  static_assert(!WBF16 || (!DUAL && MT * 4 / WN <= MT), "the bf16-weight form: single GEMMs; the wait counts below take a wave's "
-                                                       "blocks of A to be requested behind the first MT groups");
+  static_assert(!WBF16 || !DUAL, "the bf16-weight form: single GEMMs");
   constexpr int WGM = MT * 16 * WM; // rows per workgroup
   constexpr int NBLK = MT * 4 / WN; // blocks of 4 rows x 256 B of the A tile that a wave fetches per K step
   static_assert(NBLK % 4 == 0, "the swizzle below takes a wave's first block to be a multiple of 4");
@@ -739,10 +738,13 @@ __device__ __forceinline__ void big_gemm_body(const BigParams& P) {
       constexpr int q = decltype(Q)::value;
       constexpr int j = q / MT, mt = q % MT;
       if constexpr (mt == 0 && WBF16) {
-        // Step j's weights were requested a K step ago.  Behind them then: the later steps' (4 each); in this K
-        // step, when it requests anything: its NBLK blocks of A (behind the first NBLK groups, all of step 0) and
-        // the next K step's weights of the steps before j.
-        constexpr int younger = (3 - j) * 4 + (more ? (j >= 1 ? NBLK : 0) + j * 4 : 0);
+        // Step j's weights were requested a K step ago, behind group j * MT + MT - 1.  Behind them then: the later
+        // steps' (4 each) and the blocks of A that K step still had to request (block d goes out behind group d);
+        // in this K step, when it requests anything: the blocks of A behind the groups before this one and the
+        // next K step's weights of the steps before j.
+        constexpr int qj = j * MT + MT - 1;
+        constexpr int younger = (3 - j) * 4 + (NBLK - 1 - qj > 0 ? NBLK - 1 - qj : 0) +
+                                (more ? (j * MT < NBLK ? j * MT : NBLK) + j * 4 : 0);
         asm volatile("s_waitcnt vmcnt(%4)" : "+v"(bw[j][0]), "+v"(bw[j][1]), "+v"(bw[j][2]), "+v"(bw[j][3]) : "n"(younger));
 #pragma unroll
         for (int nt = 0; nt < 4; nt++)
@@ -774,9 +776,10 @@ __device__ __forceinline__ void big_gemm_body(const BigParams& P) {
       }
     });
     if constexpr (WBF16 && more) {
-      // this wave's loads into LDS have landed (the 16 weight loads of the next K step went out behind them), then
-      // everybody's; a bare barrier, see above
-      asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" : : : "memory");
+      // this wave's loads into LDS have landed -- behind the last of them went out the next K step's weights of
+      // every step j whose last group is not before that block's -- then everybody's; a bare barrier, see above
+      constexpr int after = 4 * ((MT - 1 >= NBLK - 1) + (2 * MT - 1 >= NBLK - 1) + (3 * MT - 1 >= NBLK - 1) + (4 * MT - 1 >= NBLK - 1));
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(after) : "memory");
     } else {
       __syncthreads(); // waits for this wave's direct-to-LDS loads, then for everybody's
     }
@@ -1429,6 +1432,14 @@ hipError_t launch_tiled_bf16(const TiledParams& p, hipStream_t stream) {
       P.nb0[i] = nb;
     P.n_seg = 1;
     P.xm = 1;
+    // 64 x 128 workgroups, as for MXFP4, while there are at most 256 of them (with 2-byte weights they lose earlier:
+    // 11008 x 4096 at 192 rows, 258 workgroups: 62 us against 52)
+    if (((p.M + 63) / 64) * ((p.tiles + 7) / 8) <= 256 && env_int("TPPX_TILED_SMALL", 1) != 0) {
+      const int nbs = (p.tiles + 7) / 8;
+      for (int i = 1; i <= TPPX_MAX_SEGS; i++)
+        P.nb0[i] = nbs;
+      return big_bf16_launch<2, 2, 2>(P, ((p.M + 63) / 64) * nbs, stream);
+    }
     if (((p.M + 127) / 128) * nb <= 256 && env_int("TPPX_TILED_W8", 1) != 0) // at most one workgroup per CU: eight waves, as for MXFP4
       return big_bf16_launch<4, 2, 4>(P, ((p.M + 127) / 128) * nb, stream);
     return big_bf16_launch<8, 1, 4>(P, ((p.M + 127) / 128) * nb, stream);
