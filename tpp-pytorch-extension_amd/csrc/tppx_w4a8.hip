@@ -176,15 +176,20 @@ prepack_w4a8_wide_kernel(const uint32_t* __restrict__ qref, const uint8_t* __res
 // matrix pipe: 64 multiply-adds per lane and block beside 16 MFMAs.  (Tried and dropped: 256 x 128 workgroups of
 // eight waves with every operand through LDS, by loads into registers or straight into LDS -- those take about
 // 2.5 us to land on this part whatever they hit -- were 5-15 % slower: half the work per barrier.)
+// MTW = row tiles of 16 per wave: 4 (workgroup 128 x 128) or 2 (64 x 128: twice as many workgroups for launches that
+// would leave CUs empty or at one wave per SIMD).
+template <int MTW>
 __global__ void __launch_bounds__(256, 2)
 linear_w4a8_wide_kernel(const W4A8WideParams p) {
+  constexpr int WMT = MTW * 2; // row tiles per workgroup
   extern __shared__ __align__(16) uint8_t w4_lds[];
-  // LDS: rows 2 buffers x [8 mt][4 b][64 lanes] x 16 B, then scales 2 buffers x [2 groups of 64 rows][4 b][16 m] x 16 B
+  // LDS: rows 2 buffers x [WMT mt][4 b][64 lanes] x 16 B (32 KiB each at most), then scales 2 buffers x
+  // [groups of 64 rows][4 b][16 m] x 16 B
   i32x4* As = reinterpret_cast<i32x4*>(w4_lds);
   i32x4* Ss = reinterpret_cast<i32x4*>(w4_lds + 2 * 32768);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave & 1, wn = wave >> 1, g = lane >> 4;
-  const int MB = p.MT16 >> 3, NB = (p.tiles + 7) >> 3;
+  const int MB = p.MT16 / WMT, NB = (p.tiles + 7) >> 3;
   int id = blockIdx.x;
   const int T = MB * NB;
   if ((T & 7) == 0) // workgroup ids go round the 8 XCDs: give each an eighth of the tiles, row blocks fastest
@@ -199,17 +204,17 @@ linear_w4a8_wide_kernel(const W4A8WideParams p) {
     const int64_t t = min(tile_base + nt, p.tiles - 1);
     wq[nt] = reinterpret_cast<const i32x4*>(p.wn) + t * KT * 256 + lane;
   }
-  const i32x4* xa = reinterpret_cast<const i32x4*>(p.xa) + (int64_t)bm * 8 * 256 + tid;
-  const i32x4* sa = reinterpret_cast<const i32x4*>(p.sa) + (int64_t)bm * 8 * 16 + (tid & 127);
+  const i32x4* xa = reinterpret_cast<const i32x4*>(p.xa) + (int64_t)bm * WMT * 256 + tid;
+  const i32x4* sa = reinterpret_cast<const i32x4*>(p.sa) + (int64_t)bm * WMT * 16 + (tid & (WMT * 16 - 1));
   const int64_t xa_kt = (int64_t)p.MT16 * 256, sa_kt = (int64_t)p.MT16 * 16;
 
-  i32x4 areg[8], sreg;
+  i32x4 areg[WMT], sreg;
   i32x4 bring[4][4]; // [b][nt]
   auto load_a = [&](int ks) {
 #pragma unroll
-    for (int q = 0; q < 8; q++)
+    for (int q = 0; q < WMT; q++)
       areg[q] = xa[ks * xa_kt + q * 256];
-    sreg = sa[ks * sa_kt]; // 2 KiB of scales: waves 2 and 3 fetch and store what waves 0 and 1 do
+    sreg = sa[ks * sa_kt]; // WMT * 256 bytes of scales: the other waves fetch and store the same values again
   };
   auto load_b = [&](int ks, int b) {
 #pragma unroll
@@ -218,12 +223,12 @@ linear_w4a8_wide_kernel(const W4A8WideParams p) {
   };
   auto store_a = [&](int buf) {
 #pragma unroll
-    for (int q = 0; q < 8; q++)
+    for (int q = 0; q < WMT; q++)
       As[buf * 2048 + q * 256 + tid] = areg[q];
-    Ss[buf * 128 + (tid & 127)] = sreg;
+    Ss[buf * 128 + (tid & (WMT * 16 - 1))] = sreg;
   };
 
-  f32x4 f[4][4]; // [mt][nt][r]: row mt*16 + (lane & 15), channel nt*16 + g*4 + r
+  f32x4 f[MTW][4]; // [mt][nt][r]: row mt*16 + (lane & 15), channel nt*16 + g*4 + r
 #pragma unroll
   for (int nt = 0; nt < 4; nt++) {
     const int n = min(tile_base + nt, p.tiles - 1) * 16 + g * 4;
@@ -234,7 +239,7 @@ linear_w4a8_wide_kernel(const W4A8WideParams p) {
                  bf16_bits_to_f32(bb.y >> 16)};
     }
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++)
+    for (int mt = 0; mt < MTW; mt++)
       f[mt][nt] = bv;
   }
 
@@ -250,18 +255,20 @@ linear_w4a8_wide_kernel(const W4A8WideParams p) {
     // the compiler sinks every fold below the last one, behind all 64 MFMAs.
     const int kn = min(ks + 1, KT - 1);
     load_a(kn);
-    const i32x4* Ab = As + buf * 2048 + (wm * 4) * 256 + lane;
-    const i32x4* Sb = Ss + buf * 128 + wm * 64 + (lane & 15);
-    // 16 groups (block b, row tile mt) of four MFMAs, fenced: left alone the compiler issues all 64 MFMAs of the K
+    const i32x4* Ab = As + buf * 2048 + (wm * MTW) * 256 + lane;
+    // a group of 64 rows has its four row tiles' scales side by side: a wave of two row tiles reads its half of them
+    const i32x4* Sb = Ss + buf * 128 + (MTW == 4 ? wm * 64 : 0) + (lane & 15);
+    constexpr int NG = 4 * MTW; // groups (block b, row tile mt) of four MFMAs
+    // NG groups of four MFMAs, fenced: left alone the compiler issues all 64 MFMAs of the K
     // tile first (none depends on another) and needs a register for every result.
     // The fold of a group runs under the MFMAs of the next one (results by the parity of the group).
     i32x4 sv[2];
     sv[0] = Sb[0];
     f32x4 t[2][4];
-    static_for<0, 17>([&](auto GI) {
+    static_for<0, NG + 1>([&](auto GI) {
       constexpr int gi = decltype(GI)::value;
-      if constexpr (gi < 16) {
-        constexpr int b = gi >> 2, mt = gi & 3;
+      if constexpr (gi < NG) {
+        constexpr int b = gi / MTW, mt = gi % MTW;
         const bf16x8 a = __builtin_bit_cast(bf16x8, Ab[mt * 256 + b * 64]);
         if constexpr (mt == 1 && b < 3) // (not at mt == 0: block b - 1's last fold, below, still reads that register)
           sv[(b + 1) & 1] = Sb[(b + 1) * 16];
@@ -272,14 +279,15 @@ linear_w4a8_wide_kernel(const W4A8WideParams p) {
                                                                   f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
       }
       if constexpr (gi > 0) {
-        constexpr int pb = (gi - 1) >> 2, pmt = (gi - 1) & 3;
-        const float sc = __builtin_bit_cast(f32x4, sv[pb & 1])[pmt];
+        constexpr int pb = (gi - 1) / MTW, pmt = (gi - 1) % MTW;
+        const f32x4 sq = __builtin_bit_cast(f32x4, sv[pb & 1]);
+        const float sc = MTW == 4 ? sq[pmt] : (wm ? sq[2 + pmt] : sq[pmt]);
 #pragma unroll
         for (int nt = 0; nt < 4; nt++)
 #pragma unroll
           for (int r = 0; r < 4; r++)
             f[pmt][nt][r] = fmaf(t[(gi - 1) & 1][nt][r], sc, f[pmt][nt][r]);
-        if constexpr (pmt == 3)
+        if constexpr (pmt == MTW - 1)
           load_b(kn, pb);
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -288,7 +296,7 @@ linear_w4a8_wide_kernel(const W4A8WideParams p) {
     __syncthreads();
   }
 
-  const int m_base = bm * 128 + wm * 64 + (lane & 15);
+  const int m_base = bm * (WMT * 16) + wm * (MTW * 16) + (lane & 15);
 #pragma unroll
   for (int nt = 0; nt < 4; nt++) {
     const int tile = tile_base + nt;
@@ -296,7 +304,7 @@ linear_w4a8_wide_kernel(const W4A8WideParams p) {
       continue;
     const int n = tile * 16 + g * 4;
 #pragma unroll
-    for (int mt = 0; mt < 4; mt++) {
+    for (int mt = 0; mt < MTW; mt++) {
       const int m = m_base + mt * 16;
       if (m >= p.M)
         continue;
@@ -416,9 +424,17 @@ extern "C" int tppx_linear_mxfp4_int8_wide(const void* x, const void* w_nat, con
   if (rc != TPPX_OK)
     return rc;
   const size_t lds = 2 * 32768 + 2 * 2048;
-  rc = check_hip(allow_dynamic_lds(reinterpret_cast<const void*>(linear_w4a8_wide_kernel), lds), who);
+  // launches of at most 256 workgroups of 128 x 128 (at most one per CU: one wave per SIMD): 64 x 128 ones, twice as many
+  if (mb * nb <= 256) {
+    rc = check_hip(allow_dynamic_lds(reinterpret_cast<const void*>(linear_w4a8_wide_kernel<2>), lds), who);
+    if (rc != TPPX_OK)
+      return rc;
+    linear_w4a8_wide_kernel<2><<<dim3((unsigned)(mb * 2 * nb)), dim3(256), lds, (hipStream_t)stream>>>(p);
+    return check_hip(hipGetLastError(), who);
+  }
+  rc = check_hip(allow_dynamic_lds(reinterpret_cast<const void*>(linear_w4a8_wide_kernel<4>), lds), who);
   if (rc != TPPX_OK)
     return rc;
-  linear_w4a8_wide_kernel<<<dim3((unsigned)(mb * nb)), dim3(256), lds, (hipStream_t)stream>>>(p);
+  linear_w4a8_wide_kernel<4><<<dim3((unsigned)(mb * nb)), dim3(256), lds, (hipStream_t)stream>>>(p);
   return check_hip(hipGetLastError(), who);
 }

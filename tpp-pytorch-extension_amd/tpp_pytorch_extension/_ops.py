@@ -607,7 +607,7 @@ def _linear_other_types(input, weight, bias, post, flags, post_in=None, post_in2
 PACKED_CODES = os.environ.get("TPPX_PACKED_CODES", "1") == "1"
 W4A8_ACT_SCALE = 6.0 / 127.0
 W4A8_DECODE = os.environ.get("TPPX_W4A8_DECODE", "1") == "1"
-W4A8_WIDE_ROWS = int(os.environ.get("TPPX_W4A8_WIDE_ROWS", "129"))
+W4A8_WIDE_ROWS = int(os.environ.get("TPPX_W4A8_WIDE_ROWS", "64"))
 
 
 def _linear_w4a8(input, weight, bias, post, post_in, post_in2, post_scale):
