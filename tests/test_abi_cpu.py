@@ -245,6 +245,10 @@ def test_launch_plans_of_the_baseline_shapes():
     pair7 = (ctypes.c_int64 * 2)(11008, 11008)
     assert "big_mxfp4_kernel<4, true, 2, 4> grid=172x1x1 block=512" in plan(L.tppx_plan_multi_linear_mxfp4, pair7, 2, 256, 4096, 1,
                                                                            _lib.FLAG_FORCE_TILED, 0)[0]
+    assert "big_qint8_small_kernel grid=128x1x1 block=512" in plan(L.tppx_plan_linear_qint8, 512, 4096, 4096, 256, 1,
+                                                                    _lib.FLAG_FORCE_TILED, 1 << 25)[-1]
+    assert "big_qint8_kernel grid=172x1x1 block=512" in plan(L.tppx_plan_linear_qint8, 512, 11008, 4096, 256, 1,
+                                                              _lib.FLAG_FORCE_TILED, 1 << 25)[-1]
     pair1 = (ctypes.c_int64 * 2)(4096, 4096)
     assert "big_mxfp4_kernel<2, true, 2, 2> grid=256x1x1 block=256" in plan(L.tppx_plan_multi_linear_mxfp4, pair1, 2, 256, 4096, 1,
                                                                            _lib.FLAG_FORCE_TILED, 0)[0]

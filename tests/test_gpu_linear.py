@@ -244,7 +244,8 @@ def test_prefill_forms_for_small_launches_agree(M, monkeypatch):
     """Launches that leave CUs empty run other forms of the large-M kernel's body -- 64 x 128 workgroups of four waves
     up to 128 workgroups of 128 x 256, eight waves per 128 x 256 workgroup up to 256 -- with the same sums in the
     same order: identical bits to the four-wave 128 x 256 form, for a single GEMM (ragged rows and channel blocks),
-    fused q/k/v, the gate/up pair and unquantized bf16 weights; and the single GEMM against the oracle."""
+    fused q/k/v, the gate/up pair and unquantized bf16 weights; the same for the QINT8 kernel's 64 x 256 form (single
+    GEMM and fused q/k/v); and the single MXFP4 GEMM against the oracle."""
     ops = _ops()
     K = 640
     w, q_or, s_or = _make("mxfp4", 1056, K, 720)[:3]
@@ -252,12 +253,16 @@ def test_prefill_forms_for_small_launches_agree(M, monkeypatch):
     wg, wu = _make("mxfp4", 1120, K, 725)[0], _make("mxfp4", 1120, K, 726)[0]
     Wb = randn_bf16((1056, K), 0.05, 727)
     wb = block_bf16(Wb).cuda()
+    w8 = _make("qint8", 1056, 768, 729)[0]
+    w8s = [_make("qint8", n, 768, 730 + i)[0] for i, n in enumerate((1024, 256, 256))]
+    x8 = randn_bf16((M, 768), 1.0, 733).cuda()
     x = randn_bf16((M, K), 1.0, 728)
     xg = x.cuda()
 
     def run():
         return [ops.fc_plain(xg, w, None)] + list(ops.qkv_gemm(xg, ws, [None] * 3)) + [ops.swiglu_gate_up(xg, wg, wu)] + \
-            [ops.linear(xg, wb, None, O.POST_NONE, None, None, 1.0, flags=_lib_mod().FLAG_FORCE_TILED)]
+            [ops.linear(xg, wb, None, O.POST_NONE, None, None, 1.0, flags=_lib_mod().FLAG_FORCE_TILED)] + \
+            [ops.fc_plain(x8, w8, None)] + list(ops.qkv_gemm(x8, w8s, [None] * 3))
 
     monkeypatch.setenv("TPPX_TILED_MIN_M", "0")  # the LDS-tiled family whatever the cost estimate says
     got = run()

@@ -240,7 +240,9 @@ static bool want_tiled(int64_t M, int flags, int64_t K = 0, int64_t n_tiles16 = 
   const double rows64 = (double)((M + 63) / 64);
   if (kind == COST_QINT8) {
     const int64_t wgs = ((M + 127) / 128) * ((n_tiles16 + 15) / 16);
-    const double tiled_us = (double)((wgs + 255) / 256) * (10.0 + (double)K * 0.0075);
+    // (launches of at most 128 such workgroups run as twice as many of 64 x 256)
+    const bool small = wgs <= 128 && env_int("TPPX_TILED_SMALL", 1) != 0;
+    const double tiled_us = small ? 8.0 + (double)K * 0.006 : (double)((wgs + 255) / 256) * (10.0 + (double)K * 0.0075);
     const double skinny_us = rows64 * (5.0 + wbytes / 5.5e6 + (double)K * 0.0004);
     return tiled_us <= skinny_us;
   }

@@ -846,9 +846,10 @@ __device__ __forceinline__ void lds_wait_keep16(i32x4 (&b)[4][4]) {
                : "n"(N));
 }
 
-__global__ void __launch_bounds__(512)
-big_qint8_kernel(const BigParams P) {
-  constexpr int MT = 4, WGM = 128, ABUF = WGM * 256, BBUF = 64 * 1024;
+// MT = row tiles of 16 per wave: 4 (workgroup 128 x 256) or 2 (64 x 256, for launches that leave CUs empty).
+template <int MT>
+__device__ __forceinline__ void big_qint8_body(const BigParams& P) {
+  constexpr int WGM = MT * 32, ABUF = WGM * 256, BBUF = 64 * 1024;
   extern __shared__ __align__(16) uint8_t tl_lds[];
   uint8_t* b_lds = tl_lds + 2 * ABUF;
   float* sa_s = reinterpret_cast<float*>(tl_lds + 2 * ABUF + BBUF); // [4][128]: scales of steps ks .. ks+2 (mod 4)
@@ -893,7 +894,8 @@ big_qint8_kernel(const BigParams P) {
   const uint32_t blk_stride = (uint32_t)(4 * p.K);
   auto load_a_one = [&](auto I, int ks, int buf) {
     constexpr int i = decltype(I)::value;
-    const uint32_t sw = (uint32_t)((ch ^ ((i & 3) * 4 + rin)) & 15) * 16u;
+    // row of this block inside its 16-row tile: the wave's first block is a multiple of 4 only with four row tiles
+    const uint32_t sw = (uint32_t)((ch ^ (((wave * MT + i) & 3) * 4 + rin)) & 15) * 16u;
     uint32_t off;
     if (full) {
       off = xrow0 + (uint32_t)i * blk_stride + sw + (uint32_t)ks * 256u;
@@ -942,7 +944,7 @@ big_qint8_kernel(const BigParams P) {
 #pragma unroll
   for (int nt = 0; nt < 4; nt++)
     swn[nt] = swp[soff[nt]];
-  if (tid < 128) {
+  if (tid < WGM) {
     sa_s[tid] = sarow[0];
     if (KS > 1)
       sa_s[128 + tid] = sarow[1];
@@ -964,7 +966,7 @@ big_qint8_kernel(const BigParams P) {
 #pragma unroll
     for (int nt = 0; nt < 4; nt++)
       swv[nt] = swn[nt];
-    if (tid < 128 && ks + 2 < KS) {
+    if (tid < WGM && ks + 2 < KS) {
       sa_s[((ks + 2) & 3) * 128 + tid] = sareg; // loaded two steps ago
       sareg = ks + 3 < KS ? sarow[ks + 3] : 0.f;
     }
@@ -976,7 +978,7 @@ big_qint8_kernel(const BigParams P) {
         swn[nt] = swp[soff[nt] + (uint32_t)(ks + 1) * 16u];
     }
     const uint32_t abase = lds0 + (uint32_t)(buf * ABUF + wm * MT * 4096);
-    const float* sab = sa_s + (ks & 3) * 128 + wm * 64 + (lane >> 4) * 4;
+    const float* sab = sa_s + (ks & 3) * 128 + wm * (MT * 16) + (lane >> 4) * 4;
     auto fold = [&](auto MTI) { // facc += int32 sum * (sa[row] * sw[channel]) for row tile mt
       constexpr int mt = decltype(MTI)::value;
       const f32x4 sav = *reinterpret_cast<const f32x4*>(sab + mt * 16);
@@ -1008,8 +1010,10 @@ big_qint8_kernel(const BigParams P) {
         iacc[mt & 1][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bq[nt][j], j == 0 ? i32x4{0, 0, 0, 0} : iacc[mt & 1][nt], 0, 0, 0);
       if constexpr (more && q < 8)
         load_b_one(std::integral_constant<int, q>{}, ks + 1);
-      if constexpr (more && q >= 8 && q < 8 + MT)
-        load_a_one(std::integral_constant<int, q - 8>{}, ks + 1, buf ^ 1);
+      // the MT blocks of A behind the groups after the weight tiles' (with two row tiles there are only 8 groups: behind the last MT of them)
+      constexpr int qa = NQ >= 8 + MT ? 8 : NQ - MT;
+      if constexpr (more && q >= qa && q < qa + MT)
+        load_a_one(std::integral_constant<int, q - qa>{}, ks + 1, buf ^ 1);
       if constexpr (j == 0 && mt > 0)
         fold(std::integral_constant<int, mt - 1>{}); // the previous row tile, under this row tile's MFMAs
     });
@@ -1020,6 +1024,16 @@ big_qint8_kernel(const BigParams P) {
     step(std::true_type{}, ks);
   step(std::false_type{}, KS - 1);
   big_epilogue<MT>(p, facc, reinterpret_cast<float*>(tl_lds) + wave * 64 * EP_LD, m_wg + wm * (MT * 16), tile_base);
+}
+
+__global__ void __launch_bounds__(512)
+big_qint8_kernel(const BigParams P) {
+  big_qint8_body<4>(P);
+}
+
+__global__ void __launch_bounds__(512)
+big_qint8_small_kernel(const BigParams P) {
+  big_qint8_body<2>(P);
 }
 
 // the large-M kernel addresses its operands with 32-bit byte offsets
@@ -1485,6 +1499,15 @@ hipError_t launch_tiled_qint8_group(const TiledParams* t, int n, hipStream_t str
     const int MB4 = (t[0].M + 127) / 128, NB16 = nb;
     const size_t lds = 8 * 64 * EP_LD * sizeof(float); // epilogue staging; >= the A and B buffers + the scale slots
     static_assert(8 * 64 * EP_LD * sizeof(float) >= 2 * 128 * 256 + 64 * 1024 + 4 * 128 * sizeof(float), "LDS plan");
+    // launches of at most 128 workgroups of 128 x 256: twice as many of 64 x 256, so that fewer CUs stay empty
+    if (MB4 * NB16 <= 128 && env_int("TPPX_TILED_SMALL", 1) != 0) {
+      const int MB2 = (t[0].M + 63) / 64;
+      TPPX_PLAN_ONLY(big_qint8_small_kernel, dim3(MB2 * NB16), dim3(512), lds);
+      if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_qint8_small_kernel), lds); e != hipSuccess)
+        return e;
+      big_qint8_small_kernel<<<dim3(MB2 * NB16), dim3(512), lds, stream>>>(P);
+      return hipGetLastError();
+    }
     TPPX_PLAN_ONLY(big_qint8_kernel, dim3(MB4 * NB16), dim3(512), lds);
     if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(big_qint8_kernel), lds); e != hipSuccess)
       return e;
