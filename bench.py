@@ -919,12 +919,13 @@ def cpu_baseline_tokens(B, seconds=6.0):
 
 
 def run_prompt(torch, args):
-    """Prompt processing on the 7B-shape decoder of config 5: `--batch` sequences of 2048 random token ids through
-    the 32 layers in one pass (MXFP4 linears on the large-M kernels, causal attention, keys appended to an empty
-    cache), then the lm_head on the last position.  Not a BASELINE configuration; reported as prompt tokens/s."""
+    """Prompt processing on the 7B-shape decoder of config 5: `--batch` sequences of `--prompt-len` (2048) random
+    token ids through the 32 layers in one pass (MXFP4 linears on the large-M kernels, causal attention, keys
+    appended to an empty cache), then the lm_head on the last position.  Not a BASELINE configuration; reported as
+    prompt tokens/s."""
     from tpp_pytorch_extension.llm import fused_llama_infer as F
     dev = torch.device("cuda:0")
-    B, S = args.batch, 2048
+    B, S = args.batch, args.prompt_len
     model = cfg5_model(torch)
     prompt = torch.randint(0, 32000, (B, S), generator=torch.Generator().manual_seed(6), dtype=torch.int64).to(dev)
     steps, warmup = max(2, min(args.steps, 8)), max(1, min(args.warmup, 2))
@@ -1044,6 +1045,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--fmt", default="qint8", choices=["qint8", "mxfp4"])
     ap.add_argument("--batch", type=int, default=1, help="sequences for --workload tokens (1 or 16 in the baseline)")
+    ap.add_argument("--prompt-len", type=int, default=2048, help="tokens per sequence for --workload prompt")
     ap.add_argument("--workload", default="all", choices=["all", "decode", "cfg1", "cfg3", "prefill", "tokens", "prompt", "w4a8"],
                     help="all = the headline (config 2) plus every other leg of the metric under config.legs (default); "
                          "decode = the headline alone; cfg1 / cfg3 / prefill (config 4) / tokens (config 5) = that leg "
