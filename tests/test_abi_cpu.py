@@ -254,6 +254,11 @@ def test_launch_plans_of_the_baseline_shapes():
                                                                            _lib.FLAG_FORCE_TILED, 0)[0]
     assert "big_mxfp4_kernel<8, false, 1, 8> grid=176x1x1 block=512" in plan(L.tppx_plan_linear_mxfp4, 1024, 11008, 4096,
                                                                              _lib.FLAG_FORCE_TILED, 0)[0]  # 128 x 512: eight waves anyway
+    # from 65 rows on the 64-row forms take what the planner hands to a tiled kernel
+    assert "big_mxfp4_kernel<2, false, 2, 2> grid=96x1x1 block=256" in plan(L.tppx_plan_linear_mxfp4, 160, 4096, 4096, 0, 0)[0]
+    assert "skinny_mxfp4" in plan(L.tppx_plan_linear_mxfp4, 128, 4096, 4096, 0, ws)[0]
+    assert "big_qint8_small_kernel grid=129x1x1 block=512" in plan(L.tppx_plan_linear_qint8, 160, 11008, 4096, 256, 1, 0, ws)[-1]
+    assert "big_mxfp4_kernel<2, false, 2, 2>" in plan(L.tppx_plan_linear_mxfp4, 100, 4096, 4096, _lib.FLAG_FORCE_TILED, 0)[0]
 
 
 def test_launch_plans_of_per_output_channel_qint8():

@@ -239,7 +239,7 @@ def test_prefill_mxfp4_workgroup_tiles_and_xcd_splits_agree(monkeypatch):
                 assert torch.equal(a, b), (tile, xm, i)
 
 
-@pytest.mark.parametrize("M", [200, 500])
+@pytest.mark.parametrize("M", [70, 150, 200, 500])
 def test_prefill_forms_for_small_launches_agree(M, monkeypatch):
     """Launches that leave CUs empty run other forms of the large-M kernel's body -- 64 x 128 workgroups of four waves
     up to 128 workgroups of 128 x 256, eight waves per 128 x 256 workgroup up to 256 -- with the same sums in the
@@ -647,7 +647,7 @@ def test_launch_plan_names_the_kernels():
     _lib.check(L.tppx_plan_linear_mxfp4(2048, 8192, 8192, 0, 0, buf, len(buf)))
     assert "big_mxfp4_kernel" in buf.value.decode()
     _lib.check(L.tppx_plan_linear_mxfp4(100, 8192, 8192, _lib.FLAG_FORCE_TILED, 0, buf, len(buf)))
-    assert "tiled_mxfp4_kernel" in buf.value.decode()
+    assert "big_mxfp4_kernel<2, false, 2, 2>" in buf.value.decode()  # 64 x 128 workgroups from 65 rows on
     _lib.check(L.tppx_plan_linear_mxfp4(128, 11008, 4096, 0, 0, buf, len(buf)))  # few tiles: block rows of 64
     assert "skinny_mxfp4_mg_kernel" in buf.value.decode() and "x2x" in buf.value.decode()
 

@@ -220,8 +220,9 @@ static const int64_t TILED_MIN_M = 65; // more rows than the decode kernels cove
 // block row of 64 rows after the other over the full grid, streaming the weights once per block row.  Pick by a
 // cost estimates fitted to measurements on MI355X (us).  MXFP4: a block row of 64 costs about 8 + weight bytes /
 // 5.5 TB/s + 0.8 ns per input channel (its activations), a round of 256 x 256 tiles about 14.5 ns per input channel
-// (128 x 128: 20; launches small enough for 64 x 128 workgroups: 10 us + 6 ns per input channel).  QINT8 (128 x 256 tiles, one workgroup per CU) and unquantized bf16 weights (from 192 rows 128 x 256
-// tiles, two workgroups per CU; below that the 128 x 128 kernel): their own fits below.  `wbytes` = weight bytes of
+// (128 x 128: 20; launches small enough for 64 x 128 workgroups: 10 us + 6 ns per input channel).  QINT8 (128 x 256
+// tiles, one workgroup per CU) and unquantized bf16 weights (128 x 256 tiles, two workgroups per CU): their own fits
+// below.  `wbytes` = weight bytes of
 // the whole call, `n_tiles16` = its 16-channel tiles.  TPPX_TILED_MIN_M (when set) restores a plain row threshold.
 enum { COST_MXFP4 = 0, COST_QINT8 = 1, COST_BF16 = 2 };
 static bool want_tiled(int64_t M, int flags, int64_t K = 0, int64_t n_tiles16 = 0, double wbytes = 0.0,
@@ -246,7 +247,7 @@ static bool want_tiled(int64_t M, int flags, int64_t K = 0, int64_t n_tiles16 = 
     const double skinny_us = rows64 * (5.0 + wbytes / 5.5e6 + (double)K * 0.0004);
     return tiled_us <= skinny_us;
   }
-  if (kind == COST_BF16 && M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && env_int("TPPX_BF16_BIG", 1) != 0) {
+  if (kind == COST_BF16 && M >= big_min_rows() && env_int("TPPX_BF16_BIG", 1) != 0) {
     const int64_t wgs = ((M + 127) / 128) * ((n_tiles16 + 15) / 16);
     const int64_t wgs2 = ((M + 63) / 64) * ((n_tiles16 + 7) / 8); // as 64 x 128 workgroups: the form up to 256 of them
     const bool small = wgs2 <= 256 && env_int("TPPX_TILED_SMALL", 1) != 0;
@@ -254,13 +255,15 @@ static bool want_tiled(int64_t M, int flags, int64_t K = 0, int64_t n_tiles16 = 
     const double skinny_us = rows64 * (6.5 + wbytes / 5.5e6 + (double)K * 0.0006);
     return tiled_us <= skinny_us;
   }
-  const bool big = kind == COST_MXFP4 && M >= env_int("TPPX_TILED_BIG_MIN_M", 192);
+  const bool big = kind == COST_MXFP4 && M >= big_min_rows();
   if (big && env_int("TPPX_TILED_SMALL", 1) != 0) {
     // launches of at most 128 workgroups of 128 x 256 run as four times as many of 64 x 128
     const int64_t wgs1 = ((M + 127) / 128) * ((n_tiles16 + 15) / 16);
     if (wgs1 <= 128) {
       const int64_t wgs2 = ((M + 63) / 64) * ((n_tiles16 + 7) / 8);
-      const double tiled_us = 10.0 + (double)K * 0.006 * (wgs2 <= 128 ? 1.0 : wgs2 <= 384 ? 1.05 : 1.25);
+      // (up to 128 of them: 26 us at K = 4096, 74 at K = 11008 whatever the rows)
+      const double tiled_us = wgs2 <= 128 ? std::max(12.0, (double)K * 0.007 - 2.0)
+                                          : 10.0 + (double)K * 0.006 * (wgs2 <= 384 ? 1.05 : 1.25);
       const double skinny_us = rows64 * (6.0 + wbytes / 5.5e6 + (double)K * 0.0007);
       return tiled_us <= skinny_us;
     }

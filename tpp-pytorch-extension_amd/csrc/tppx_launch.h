@@ -117,6 +117,10 @@ hipError_t launch_tiled_qint8_group(const TiledParams* t, int n, hipStream_t str
 hipError_t launch_silu_mul(const uint16_t* gate, uint16_t* y, int64_t n, hipStream_t stream);
 
 int env_int(const char* name, int dflt);
+// rows from which the prefill kernels of 128-row workgroups (and their 64-row forms for small launches) take a
+// GEMM; below it the older 128 x 128 kernels run.  (It was 192 before the 64-row forms existed: at 4096 x 4096 and
+// 160 rows they take 26 us where the old kernels took 62-88; TPPX_TILED_BIG_MIN_M overrides.)
+inline int big_min_rows() { return env_int("TPPX_TILED_BIG_MIN_M", 65); }
 // dynamic LDS above 48 KiB must be allowed per kernel and device before the launch
 hipError_t allow_dynamic_lds(const void* kern, size_t lds);
 

@@ -1247,7 +1247,7 @@ static bool big_fits(const TiledParams& p) {
 }
 
 bool tiled_mxfp4_takes_groups(const TiledParams& p) {
-  return p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && big_fits(p);
+  return p.M >= big_min_rows() && big_fits(p);
 }
 
 template <int MT, bool DUAL, int WM, int WN>
@@ -1434,7 +1434,7 @@ silu_mul_kernel(const uint16_t* __restrict__ gate, uint16_t* __restrict__ y, int
 hipError_t launch_tiled_bf16(const TiledParams& p, hipStream_t stream) {
   // prompt-sized passes: the 128 x 256 form of the large MXFP4 kernel with the weights read as they are (two
   // workgroups of four waves per CU); its 32-bit offsets want operands below 4 GiB
-  if (p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && env_int("TPPX_BF16_BIG", 1) != 0 &&
+  if (p.M >= big_min_rows() && env_int("TPPX_BF16_BIG", 1) != 0 &&
       (int64_t)p.M * p.K * 2 < ((int64_t)1 << 32) && (int64_t)p.tiles * 32 * p.K < ((int64_t)1 << 32)) {
     BigParams P;
     memset(&P, 0, sizeof(P));
@@ -1478,7 +1478,7 @@ hipError_t launch_silu_mul(const uint16_t* gate, uint16_t* y, int64_t n, hipStre
 }
 
 bool tiled_qint8_takes_groups(const TiledParams& p) {
-  return p.qbs == 256 && p.M >= env_int("TPPX_TILED_BIG_MIN_M", 192) && env_int("TPPX_TILED_BIG_QINT8", 1) != 0 &&
+  return p.qbs == 256 && p.M >= big_min_rows() && env_int("TPPX_TILED_BIG_QINT8", 1) != 0 &&
          (int64_t)p.M * p.K < ((int64_t)1 << 32) && (int64_t)p.tiles * 16 * p.K < ((int64_t)1 << 32);
 }
 
