@@ -395,3 +395,27 @@ def test_common_module_helpers_one_process():
     y = ln(torch.randn(3, 64))
     assert torch.allclose(y.mean(-1), torch.zeros(3), atol=1e-5)
     assert C.compare(t, t.clone(), "same") is True and C.compare(t, t + 1, "shifted") is False
+
+
+def test_cache_allocates_small_layers_together():
+    """Layers of a small KV cache share one zeroed allocation (up to eight layers, keys and values), handed out as
+    the layers ask for storage; a layer of another shape, or a cache whose layers are large, allocates on its own."""
+    import torch
+    from tpp_pytorch_extension.llm.fused_llama_infer import TppCache
+    c = TppCache(48)
+    got = [c._ensure(i, 2, 4, 16, "cpu") for i in range(10)]
+    base = got[0][0].untyped_storage().data_ptr()
+    assert all(k.untyped_storage().data_ptr() == base and v.untyped_storage().data_ptr() == base for k, v in got[:8])
+    assert got[8][0].untyped_storage().data_ptr() != base           # ninth layer: the next group
+    ptrs = {t.data_ptr() for kv in got for t in kv}
+    assert len(ptrs) == 20                                          # no two layers share memory
+    for k, v in got:
+        assert k.shape == (2, 4, 48, 16) and k.is_contiguous() and v.is_contiguous()
+        assert not k.any() and not v.any()
+    assert c._ensure(3, 2, 4, 16, "cpu")[0].data_ptr() == got[3][0].data_ptr()   # a layer keeps its storage
+    k, _ = c._ensure(10, 1, 4, 16, "cpu")                            # another shape: not the waiting storage
+    assert k.shape == (1, 4, 48, 16) and not k.any()
+    big = TppCache(48)
+    big.SLAB_BYTES = 4 * 2 * 4 * 48 * 16                            # room for one layer only
+    a, b = big._ensure(0, 2, 4, 16, "cpu"), big._ensure(1, 2, 4, 16, "cpu")
+    assert a[0].untyped_storage().data_ptr() != b[0].untyped_storage().data_ptr() and not big._spare

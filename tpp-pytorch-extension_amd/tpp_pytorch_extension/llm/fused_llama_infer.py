@@ -94,10 +94,12 @@ class TppCache:
     The sequence length lives in a device int32 so that a decode step can be replayed as a graph."""
 
     block_size = 32  # LayerCache::block_size, used by align_and_invert_mask
+    SLAB_BYTES = 64 << 20  # layers are allocated together while a group stays under this
 
     def __init__(self, capacity=0):
         self.capacity = int(capacity)
         self.layers = {}          # layer_idx -> (k, v)
+        self._spare = {}          # layer_idx -> [2][B][Nkv][capacity][H], zeroed storage waiting for that layer
         self.seq_len_dev = None   # int32 [1]: keys in the cache (same for every layer)
         self._host_len = 0
         self._sync_len = 0        # length every layer had when the fused layers last advanced the cache
@@ -153,8 +155,18 @@ class TppCache:
         if self.capacity <= 0:
             raise TppxError(_lib.EINVAL, "TppCache: give the cache a capacity (keys per sequence) before use")
         if layer_idx not in self.layers:
-            k = torch.zeros((B, Nkv, self.capacity, H), dtype=torch.bfloat16, device=device)
-            self.layers[layer_idx] = (k, torch.zeros_like(k))
+            # Small caches come several layers to an allocation (the layers of a pass ask in ascending order): one
+            # allocator call and one fill for up to eight layers' keys and values instead of two per layer, which
+            # at prompts of a hundred tokens were a device allocation per layer on every fresh cache.
+            shape = (B, Nkv, self.capacity, H)
+            spare = self._spare.pop(layer_idx, None)
+            if spare is None or tuple(spare.shape[1:]) != shape or spare.device != torch.device(device):
+                per_layer = 4 * B * Nkv * self.capacity * H
+                group = max(1, min(8, self.SLAB_BYTES // max(per_layer, 1)))
+                slab = torch.zeros((group, 2) + shape, dtype=torch.bfloat16, device=device)
+                self._spare = {layer_idx + j: slab[j] for j in range(1, group) if layer_idx + j not in self.layers}
+                spare = slab[0]
+            self.layers[layer_idx] = (spare[0], spare[1])
         if self.seq_len_dev is None:
             self.seq_len_dev = torch.zeros(1, dtype=torch.int32, device=device)
         return self.layers[layer_idx]
